@@ -1,0 +1,180 @@
+/*
+ * taac_hip.h - C ABI of libtaac_hip.so: the gfx950 (MI355X) kernel path of the TAAC-2026 unified
+ * pCVR token backbone.
+ *
+ * Conventions shared by every entry point
+ *   - All data pointers are DEVICE pointers owned by the caller; nothing is allocated or freed here.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream). Work is enqueued
+ *     asynchronously on it; the call returns as soon as the launches are queued.
+ *   - Return value: TAAC_OK (0) or a negative TAAC_ERR_* code. After a failure taac_last_error()
+ *     returns a human-readable message (thread-local storage, valid until the next call on that thread).
+ *   - Arguments are validated on the host before any kernel is launched; a rejected call launches nothing.
+ *   - `dtype` is a taac_dtype value.
+ *   - No global mutable state besides the thread-local error string: calls from different host threads
+ *     and on different streams are independent.
+ *
+ * Each declaration cites the reference interface it replaces (path:line under the reference tree,
+ * Puiching-Memory/TAAC_2026). The reference has no C ABI on this path: its operators are Python
+ * functions that dispatch to torch / Triton / TileLang; the entry points here are what a
+ * `register_*_kernel` hook or a drop-in Python operator binds with ctypes.
+ */
+#ifndef TAAC_HIP_H
+#define TAAC_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TAAC_ABI_VERSION 1
+
+enum taac_status {
+  TAAC_OK = 0,
+  TAAC_ERR_INVALID_VALUE = -1, /* bad shape / size / enum: the Python layer raises ValueError */
+  TAAC_ERR_UNSUPPORTED = -2,   /* valid request outside the kernels' envelope: RuntimeError   */
+  TAAC_ERR_LAUNCH = -3         /* HIP reported an error at launch: RuntimeError                */
+};
+
+enum taac_dtype { TAAC_F32 = 0, TAAC_BF16 = 1, TAAC_F16 = 2 };
+
+/* Epilogues of the dense-layer entry points (taac_linear_*). */
+enum taac_epilogue {
+  TAAC_EPI_NONE = 0,   /* out = a @ w^T (+ bias)                                              */
+  TAAC_EPI_RESIDUAL = 1, /* out = residual + a @ w^T (+ bias); out may alias residual          */
+  TAAC_EPI_SWIGLU = 2  /* w is [2F, K]; out[M, F] = silu(g) * u (gate_first) or g * silu(u)    */
+};
+
+int taac_abi_version(void);
+const char* taac_last_error(void);
+
+/*
+ * RMSNorm forward: y[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * w, fp32 accumulation, one rounding
+ * to the storage dtype. x, y: [rows, cols] contiguous; w: [cols] in the same dtype as x.
+ * Replaces: rms_norm / _torch_rms_norm (src/taac2026/infrastructure/accelerators/normalization/rms_norm.py:377-401,
+ * 71-73) and the Triton forward kernel (normalization/kernels/triton.py:30-50). Matches the signature
+ * a kernel registered through register_rms_norm_kernel receives (rms_norm.py:31,66-68).
+ */
+int taac_rmsnorm_fwd(const void* x, const void* w, void* y, int64_t rows, int32_t cols, float eps, int dtype,
+                     void* stream);
+
+/*
+ * LayerNorm forward: y = (x - mean) * rsqrt(var + eps) * w + b, biased variance computed from centred
+ * values, fp32 accumulation. Shapes as taac_rmsnorm_fwd, b: [cols].
+ * Replaces: layer_norm / _torch_layer_norm (normalization/layer_norm.py:261-280, 65-66) and the Triton
+ * inference kernel (normalization/kernels/triton.py:224-247); hook signature of register_layer_norm_kernel
+ * (layer_norm.py:24,60-62).
+ */
+int taac_layernorm_fwd(const void* x, const void* w, const void* b, void* y, int64_t rows, int32_t cols, float eps,
+                       int dtype, void* stream);
+
+/*
+ * Key-padding-masked attention forward: o = softmax(q k^T / sqrt(d) + mask) v per (batch, head), softmax in
+ * fp32, bf16/fp16 MFMA operands. Key j of batch b is visible iff j < key_lengths[b] (and j <= query index when
+ * is_causal). key_lengths == NULL means every key is visible. Rows with no visible key produce zeros.
+ * q/o: logical shape (B, H, Tq, d); k/v: (B, H, Tk, d). *_strides are ELEMENT strides of the four logical
+ * dimensions, so (B,H,T,d)-contiguous and (B,T,H,d)-contiguous tensors are both read in place; the last
+ * stride must be 1, the others multiples of 8, and base pointers 16-byte aligned. d must be a multiple of 8, <= 128.
+ * zero_padded_queries != 0 (requires Tq == Tk): query rows t >= key_lengths[b] are written as zeros instead
+ * of being computed over the visible keys.
+ * dtype: TAAC_BF16 or TAAC_F16.
+ * Replaces: flash_attention's kernel call `_flash_attention_kernel(q, k, v, key_lengths)`
+ * (accelerators/attention/flash_attention.py:338-367, hook at :26,102-104) and the TileLang inference kernel
+ * (accelerators/attention/kernels/tilelang.py:36-138); the strided form also replaces the four layout copies of
+ * scaled_dot_product_attention (infrastructure/modeling/sequence.py:81-116).
+ */
+int taac_flash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths, void* o, int32_t B,
+                        int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
+                        const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4],
+                        int is_causal, int zero_padded_queries, int dtype, void* stream);
+
+/*
+ * Dense layer, bf16 storage / bf16 MFMA / fp32 accumulation: out = epilogue(a @ w^T + bias).
+ * a: [M, K] with row stride lda (elements); w: [N, K] contiguous (torch nn.Linear layout, [out, in]);
+ * bias: [N] bf16 or NULL; residual: [M, N_out] with row stride ldo or NULL; out: [M, N_out] with row stride ldo,
+ * where N_out = N, or N / 2 for TAAC_EPI_SWIGLU. K must be a multiple of 8, lda/ldo multiples of 8.
+ * TAAC_EPI_SWIGLU: rows [0, N/2) of w produce g, rows [N/2, N) produce u (torch .chunk(2, -1) order);
+ * gate_first != 0 gives silu(g) * u (experiments/symbiosis/backbone.py:19-21), gate_first == 0 gives g * silu(u)
+ * (experiments/baseline/model.py:108-113).
+ * Replaces: the nn.Linear calls of UnifiedSelfAttention / SwiGLUFeedForward (experiments/symbiosis/backbone.py:
+ * 11-47) together with the elementwise SiLU-gate and the residual adds of UnifiedInteractionBlock (:58-68).
+ */
+int taac_linear_bf16(const void* a, int64_t lda, const void* w, const void* bias, const void* residual, void* out,
+                     int64_t ldo, int64_t M, int32_t N, int32_t K, int epilogue, int gate_first, void* stream);
+
+/*
+ * Per-tensor absolute maximum, for the FP8 scale (scale = amax / 448). Writes max(|x|) over n elements to
+ * *amax_out (device float). The kernel clears *amax_out itself before reducing.
+ * No counterpart in the reference (it has no FP8 code); defined by the FP8 configuration of this path.
+ */
+int taac_amax(const void* x, int64_t n, int dtype, float* amax_out, void* stream);
+
+/*
+ * Quantise to OCP e4m3fn with a per-tensor scale: q = sat(x / scale) where scale = max(*amax, tiny) / 448.
+ * x: n elements of `dtype`; q: n bytes; amax: device float. Round-to-nearest-even, saturating at +-448.
+ */
+int taac_quantize_fp8(const void* x, int64_t n, int dtype, const float* amax, void* q, void* stream);
+
+/*
+ * Dense layer with FP8 (e4m3fn) MFMA operands and per-tensor scales:
+ *   out = epilogue( (qa @ qw^T) * (amax_a / 448) * (amax_w / 448) + bias )
+ * a: [M, K] bf16 activations, quantised on load with scale amax_a / 448 (a_is_fp8 == 0), or already e4m3
+ * bytes (a_is_fp8 != 0). w: [N, K] e4m3 bytes. amax_a / amax_w: device floats. bias / residual / out are bf16
+ * with the same meaning as in taac_linear_bf16. K must be a multiple of 16.
+ * No counterpart in the reference; semantics follow the quantize -> matmul -> dequantize emulation
+ * q = (t / s).to(float8_e4m3fn), y = (qa.float() @ qw.float().T) * s_a * s_w.
+ */
+int taac_linear_fp8(const void* a, int a_is_fp8, int64_t lda, const void* w, const float* amax_a, const float* amax_w,
+                    const void* bias, const void* residual, void* out, int64_t ldo, int64_t M, int32_t N, int32_t K,
+                    int epilogue, int gate_first, void* stream);
+
+/*
+ * Readout of the backbone: p[b] = sigmoid( masked_mean(x[b, :L_b, :]) . w_head + b_head ), with
+ * L_b = clamp(lengths[b], 0, T) and the mean's divisor clamped to >= 1.
+ * x: [B, T, D] bf16 contiguous; lengths: int32 [B]; w_head: [D] bf16; b_head: [1] bf16 or NULL; p: float [B].
+ * Replaces: masked_mean (infrastructure/modeling/sequence.py:54-60) followed by Linear(D, 1) and sigmoid.
+ */
+int taac_masked_mean_head(const void* x, const int32_t* lengths, const void* w_head, const void* b_head, float* p,
+                          int32_t B, int32_t T, int32_t D, void* stream);
+
+/*
+ * Weights of one backbone block; every pointer is a device pointer to bf16 data in torch nn.Linear layout.
+ * Field names follow the reference's parameter names (experiments/symbiosis/backbone.py:24-56).
+ * Biases may be NULL (treated as zero).
+ */
+typedef struct taac_block_weights {
+  const void* attn_norm_weight; /* [D]                                   */
+  const void* qkv_weight;       /* [3D, D], rows ordered q, k, v         */
+  const void* qkv_bias;         /* [3D]                                  */
+  const void* out_weight;       /* [D, D]                                */
+  const void* out_bias;         /* [D]                                   */
+  const void* ffn_norm_weight;  /* [D]                                   */
+  const void* up_weight;        /* [2F, D], rows ordered gate, value     */
+  const void* up_bias;          /* [2F]                                  */
+  const void* down_weight;      /* [D, F]                                */
+  const void* down_bias;        /* [D]                                   */
+} taac_block_weights;
+
+/* Bytes of workspace taac_backbone_fwd needs for the given shape (device memory, 256-byte aligned). */
+int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D, int32_t F);
+
+/*
+ * Forward of n_blocks pre-norm blocks plus the pCVR readout:
+ *   for each block: h = rmsnorm(x); q,k,v = chunk3(h Wqkv^T + b); a = attention(q,k,v, key_lengths)
+ *                   (padded query rows -> 0); x = x + a Wo^T + b; h2 = rmsnorm(x);
+ *                   g,u = chunk2(h2 Wup^T + b); x = x + (silu(g) * u) Wdown^T + b
+ *   p = sigmoid(masked_mean(x, lengths) . w_head + b_head)
+ * emb: [B, T, D] bf16 (not modified); key_lengths: int32 [B] valid-prefix lengths; hidden_out: [B, T, D] bf16
+ * final hidden state or NULL; p: float [B]. heads divides D and D / heads is a multiple of 8.
+ * Rows at or beyond key_lengths[b] of hidden_out hold unspecified finite values (they are never read by the readout).
+ * Replaces: the block loop _run_backbone (experiments/symbiosis/model.py:283-292) over UnifiedInteractionBlock
+ * (experiments/symbiosis/backbone.py:50-68) in its canonical pre-norm form, plus masked_mean + Linear + sigmoid.
+ */
+int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, const taac_block_weights* blocks, int32_t n_blocks,
+                      const void* w_head, const void* b_head, int32_t B, int32_t T, int32_t D, int32_t heads, int32_t F,
+                      float eps, void* workspace, int64_t workspace_bytes, void* hidden_out, float* p, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TAAC_HIP_H */

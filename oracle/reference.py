@@ -1,0 +1,253 @@
+"""CPU oracle: a restatement of the reference's torch implementation of the backbone kernel path.
+
+TEST INFRASTRUCTURE ONLY. Nothing under ``taac_2026_amd/`` imports this module; it is used by ``tests/``, by
+``__graft_entry__.smoke()`` as the checker, and by ``bench.py``'s ``cpu_baseline`` leg as the thing timed on the host.
+Everything here runs on CPU tensors with plain torch / numpy; it never touches the HIP library.
+
+Each function cites the reference source it restates (paths relative to the reference tree,
+Puiching-Memory/TAAC_2026). How each function is pinned, independently of its own formula (tests/test_oracle.py):
+
+  rms_norm            closed form restated by the reference's own test (tests/unit/infrastructure/accelerators/
+                      test_tilelang_ops.py:533-540); float64 loop brute force, scale equivariance, row independence,
+                      the identity sum((y/w)^2)/D = 1 - eps*s^2.
+  layer_norm          torch.nn.functional.layer_norm (library routine, test_tilelang_ops.py:543-551); float64 brute
+                      force; zero mean / unit variance of the normalised rows; shift invariance.
+  attention           F.scaled_dot_product_attention with a bool mask (test_tilelang_ops.py:305-313); float64 loop
+                      brute force; len == T reduces to unmasked SDPA; len == 1 returns v[0]; identical keys return the
+                      mean of the valid values; committed golden vector tests/golden/attention_small.json.
+  make_padding_mask / safe_key_padding_mask / plan of structured masks
+                      literal known answers held by the reference's tests (tests/unit/infrastructure/modeling/
+                      test_primitives.py:36-39, tests/contract/experiments/test_packages.py:597-617,
+                      test_tilelang_ops.py:361-428), committed as tests/golden/mask_vectors.json.
+  masked_mean         float64 brute force; all-padded rows give zeros (divisor clamp).
+  swiglu_ffn / linear / block / backbone
+                      compositions of library routines F.linear, F.silu, the functions above; float64 loop brute
+                      force on tiny shapes for swiglu_ffn; the reference holds no numeric test for these
+                      (tests/contract/experiments/test_packages.py:170-192 checks shapes and finiteness only).
+  fp8 emulation       PARITY UNPINNED by the reference (it has no FP8 code). Defined by the configuration text:
+                      s = amax/448, q = (t/s).to(float8_e4m3fn), y = (qa.float() @ qw.float().T) * s_a * s_w.
+                      The e4m3 rounding itself is pinned against an exhaustive decode table of all 256 codes and
+                      nearest-even brute force (tests/test_oracle.py).
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+FP8_MAX = 448.0
+
+
+# ---- normalisation ---------------------------------------------------------------------------------------------------
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """``_torch_rms_norm`` (src/taac2026/infrastructure/accelerators/normalization/rms_norm.py:71-73), computed in
+    x's dtype exactly as the reference's torch backend does (bf16 inputs round x^2 to bf16 before the mean)."""
+    weight = weight.to(dtype=x.dtype)  # rms_norm.py:85
+    scale = torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + eps)
+    return x * scale * weight
+
+
+def rms_norm_fp32(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """Same closed form with fp32 statistics and a single rounding to x's dtype - what the reference's Triton and
+    TileLang kernels compute (normalization/kernels/triton.py:30-50). This is the parity target for 16-bit inputs."""
+    xf = x.float()
+    wf = weight.to(dtype=x.dtype).float()
+    scale = torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps)
+    return (xf * scale * wf).to(x.dtype)
+
+
+def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float = 1e-5) -> torch.Tensor:
+    """``_torch_layer_norm`` (normalization/layer_norm.py:65-66)."""
+    return F.layer_norm(x, (x.shape[-1],), weight.to(x.dtype), bias.to(x.dtype), eps)
+
+
+def layer_norm_fp32(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float = 1e-5) -> torch.Tensor:
+    """fp32 statistics, one rounding (normalization/kernels/triton.py:224-247)."""
+    out = F.layer_norm(x.float(), (x.shape[-1],), weight.to(x.dtype).float(), bias.to(x.dtype).float(), eps)
+    return out.to(x.dtype)
+
+
+# ---- masks and pooling -----------------------------------------------------------------------------------------------
+
+
+def make_padding_mask(lengths: torch.Tensor, max_len: int) -> torch.Tensor:
+    """modeling/sequence.py:32-34: True = padding."""
+    positions = torch.arange(max_len, device=lengths.device).unsqueeze(0)
+    return positions >= lengths.unsqueeze(1)
+
+
+def safe_key_padding_mask(mask: torch.Tensor) -> torch.Tensor:
+    """modeling/sequence.py:37-45."""
+    if mask.numel() == 0 or mask.shape[1] == 0:
+        return mask
+    all_masked = mask.all(dim=1, keepdim=True)
+    first_column = torch.zeros_like(mask)
+    first_column[:, :1] = True
+    return torch.where(all_masked, mask & ~first_column, mask)
+
+
+def masked_mean(tokens: torch.Tensor, padding_mask: torch.Tensor | None = None) -> torch.Tensor:
+    """modeling/sequence.py:54-60."""
+    if tokens.shape[1] == 0:
+        return tokens.new_zeros(tokens.shape[0], tokens.shape[-1])
+    if padding_mask is None:
+        return tokens.mean(dim=1)
+    valid = (~padding_mask).to(tokens.dtype).unsqueeze(-1)
+    return (tokens * valid).sum(dim=1) / valid.sum(dim=1).clamp_min(1.0)
+
+
+def key_length_mask(key_lengths: torch.Tensor, heads: int, query_len: int, kv_len: int) -> torch.Tensor:
+    """(B, H, Tq, Tk) bool mask, True = attend, for per-sample valid key prefixes - the mask family the reference's
+    planner reduces to ``key_lengths`` (attention/flash_attention.py:172-181)."""
+    key_valid = torch.arange(kv_len).unsqueeze(0) < key_lengths.unsqueeze(1).to(torch.int64)
+    return key_valid[:, None, None, :].expand(key_lengths.shape[0], heads, query_len, kv_len)
+
+
+def causal_valid_attention_mask(padding_mask: torch.Tensor, num_heads: int) -> torch.Tensor:
+    """modeling/sequence.py:119-127."""
+    batch_size, token_count = padding_mask.shape
+    causal = torch.ones(token_count, token_count, dtype=torch.bool).tril()
+    mask = causal.unsqueeze(0) & (~padding_mask).unsqueeze(1)
+    fallback = torch.eye(token_count, dtype=torch.bool).unsqueeze(0)
+    mask = torch.where(padding_mask.unsqueeze(-1), fallback, mask)
+    return mask.unsqueeze(1).expand(batch_size, num_heads, token_count, token_count)
+
+
+# ---- attention -------------------------------------------------------------------------------------------------------
+
+
+def sdpa(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, attn_mask: torch.Tensor | None = None,
+         is_causal: bool = False) -> torch.Tensor:
+    """``_torch_flash_attention`` in eval mode (attention/flash_attention.py:552-570)."""
+    return F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, dropout_p=0.0,
+                                          is_causal=is_causal if attn_mask is None else False)
+
+
+def attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    key_lengths: torch.Tensor | None = None,
+    *,
+    is_causal: bool = False,
+    zero_padded_queries: bool = False,
+) -> torch.Tensor:
+    """fp32 ``softmax(q k^T / sqrt(d) masked_fill -inf) v`` on (B, H, T, d) inputs, result in v's dtype.
+
+    The explicit form the reference's GPU tests compare against
+    (tests/gpu/infrastructure/accelerators/test_tilelang_ops_cuda.py:37-57). Rows whose visible key set is empty
+    give 0, as the reference kernel does (attention/kernels/tilelang.py:127-133). With ``zero_padded_queries`` rows
+    ``t >= key_lengths[b]`` are set to 0 (the benchmark configuration's definition of padded query rows).
+    """
+    batch, heads, query_len, head_dim = q.shape
+    kv_len = k.shape[2]
+    scores = torch.matmul(q.float(), k.float().transpose(-1, -2)) * (1.0 / math.sqrt(head_dim))
+    visible = torch.ones(batch, 1, query_len, kv_len, dtype=torch.bool)
+    if key_lengths is not None:
+        visible = visible & (torch.arange(kv_len)[None, None, None, :] < key_lengths.to(torch.int64)[:, None, None, None])
+    if is_causal:
+        visible = visible & (torch.arange(query_len)[:, None] >= torch.arange(kv_len)[None, :])[None, None]
+    scores = scores.masked_fill(~visible, float("-inf"))
+    row_max = scores.amax(dim=-1, keepdim=True)
+    row_max = torch.where(torch.isinf(row_max), torch.zeros_like(row_max), row_max)
+    weights = torch.exp(scores - row_max)
+    denom = weights.sum(dim=-1, keepdim=True)
+    probs = torch.where(denom > 0, weights / denom.clamp_min(1e-38), torch.zeros_like(weights))
+    out = torch.matmul(probs, v.float())
+    if zero_padded_queries and key_lengths is not None:
+        keep = torch.arange(query_len)[None, :] < key_lengths.to(torch.int64)[:, None]
+        out = out * keep[:, None, :, None].to(out.dtype)
+    return out.to(v.dtype)
+
+
+def scaled_dot_product_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, num_heads: int,
+                                 key_lengths: torch.Tensor | None = None, zero_padded_queries: bool = False) -> torch.Tensor:
+    """modeling/sequence.py:81-116 on (B, T, D) projections, with the key-length mask."""
+    batch, query_len, d_model = q.shape
+    head_dim = d_model // num_heads
+    q4 = q.view(batch, query_len, num_heads, head_dim).transpose(1, 2)
+    k4 = k.view(batch, k.shape[1], num_heads, head_dim).transpose(1, 2)
+    v4 = v.view(batch, v.shape[1], num_heads, head_dim).transpose(1, 2)
+    out = attention(q4, k4, v4, key_lengths, zero_padded_queries=zero_padded_queries)
+    return out.transpose(1, 2).contiguous().view(batch, query_len, d_model)
+
+
+# ---- dense layers ----------------------------------------------------------------------------------------------------
+
+
+def swiglu_ffn(x: torch.Tensor, up_weight: torch.Tensor, up_bias: torch.Tensor | None, down_weight: torch.Tensor,
+               down_bias: torch.Tensor | None, *, gate_first: bool = True) -> torch.Tensor:
+    """``SwiGLUFeedForward.forward`` in eval mode (experiments/symbiosis/backbone.py:19-21); ``gate_first=False`` is
+    the Baseline convention ``x1 * silu(x2)`` (experiments/baseline/model.py:108-113)."""
+    gate, value = F.linear(x, up_weight, up_bias).chunk(2, dim=-1)
+    hidden = F.silu(gate) * value if gate_first else gate * F.silu(value)
+    return F.linear(hidden, down_weight, down_bias)
+
+
+def swiglu_hidden(x: torch.Tensor, up_weight: torch.Tensor, up_bias: torch.Tensor | None, *, gate_first: bool = True) -> torch.Tensor:
+    gate, value = F.linear(x, up_weight, up_bias).chunk(2, dim=-1)
+    return F.silu(gate) * value if gate_first else gate * F.silu(value)
+
+
+def block(x: torch.Tensor, key_lengths: torch.Tensor, w: dict[str, torch.Tensor], *, num_heads: int, eps: float = 1e-6) -> torch.Tensor:
+    """One canonical pre-norm block: the recipe of ``UnifiedInteractionBlock.forward``
+    (experiments/symbiosis/backbone.py:58-68) without QK-norm and without the padding multiply on the updates
+    (padded rows are don't-care), attention over the valid key prefix with padded query rows set to 0."""
+    h = rms_norm(x, w["attn_norm.weight"], eps)
+    q, k, v = F.linear(h, w["qkv.weight"], w.get("qkv.bias")).chunk(3, dim=-1)
+    a = scaled_dot_product_attention(q, k, v, num_heads=num_heads, key_lengths=key_lengths, zero_padded_queries=True)
+    x = x + F.linear(a, w["out.weight"], w.get("out.bias"))
+    h2 = rms_norm(x, w["ffn_norm.weight"], eps)
+    return x + swiglu_ffn(h2, w["up.weight"], w.get("up.bias"), w["down.weight"], w.get("down.bias"))
+
+
+def backbone(emb: torch.Tensor, key_lengths: torch.Tensor, blocks: list[dict[str, torch.Tensor]],
+             head_weight: torch.Tensor, head_bias: torch.Tensor | None, *, num_heads: int, eps: float = 1e-6,
+             return_hidden: bool = False):
+    """n pre-norm blocks (``_run_backbone``, experiments/symbiosis/model.py:283-292) + masked mean-pool
+    (modeling/sequence.py:54-60) -> Linear(D, 1) -> sigmoid. Returns float32 probabilities [B]."""
+    x = emb
+    for w in blocks:
+        x = block(x, key_lengths, w, num_heads=num_heads, eps=eps)
+    padding = make_padding_mask(key_lengths.to(torch.int64), x.shape[1])
+    pooled = masked_mean(x, padding)
+    logits = F.linear(pooled, head_weight.reshape(1, -1), head_bias).squeeze(-1)
+    probs = torch.sigmoid(logits.float())
+    return (probs, x) if return_hidden else probs
+
+
+# ---- FP8 emulation (no reference counterpart; parity unpinned, see the module docstring) -------------------------------
+
+
+def fp8_scale(t: torch.Tensor) -> torch.Tensor:
+    return t.float().abs().max().clamp_min(1e-12) / FP8_MAX
+
+
+def fp8_quantize(t: torch.Tensor, scale: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """``q = (t / s).to(float8_e4m3fn)`` with ``s = amax / 448``. Returns (q, s)."""
+    if scale is None:
+        scale = fp8_scale(t)
+    q = (t.float() / scale).clamp(-FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn)
+    return q, scale
+
+
+def linear_fp8(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *,
+               residual: torch.Tensor | None = None, swiglu: bool = False, gate_first: bool = True,
+               x_scale: torch.Tensor | None = None, w_scale: torch.Tensor | None = None) -> torch.Tensor:
+    """quantize -> matmul -> dequantize emulation: ``y = (qx.float() @ qw.float().T) * s_x * s_w`` (+ bias), then the
+    fp32 epilogue (SiLU-gate or residual) and one rounding to bf16."""
+    qx, sx = fp8_quantize(x, x_scale)
+    qw, sw = fp8_quantize(weight, w_scale)
+    y = torch.matmul(qx.float(), qw.float().t()) * (sx * sw)
+    if bias is not None:
+        y = y + bias.float()
+    if swiglu:
+        gate, value = y.chunk(2, dim=-1)
+        y = F.silu(gate) * value if gate_first else gate * F.silu(value)
+    if residual is not None:
+        y = y + residual.float()
+    return y.to(torch.bfloat16)

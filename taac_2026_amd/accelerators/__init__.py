@@ -1,0 +1,51 @@
+"""Operator boundary of the HIP kernel path: flat re-exports in the style of the reference's
+``taac2026.infrastructure.accelerators`` package (accelerators/__init__.py:83-138)."""
+
+from taac_2026_amd.accelerators.attention import (
+    FlashAttentionMaskPlan,
+    _plan_tilelang_flash_attention_mask,
+    flash_attention,
+    hip_flash_attention_kernel,
+    plan_flash_attention_mask,
+    resolved_flash_attention_backend,
+)
+from taac_2026_amd.accelerators.linear import amax, linear, linear_fp8, quantize_fp8, swiglu_ffn, swiglu_linear
+from taac_2026_amd.accelerators.normalization import (
+    hip_layer_norm_kernel,
+    hip_rms_norm_kernel,
+    layer_norm,
+    resolved_layer_norm_backend,
+    resolved_rms_norm_backend,
+    rms_norm,
+)
+from taac_2026_amd.accelerators.tensor_validation import (
+    concrete_tensors,
+    require_cuda_tensors,
+    require_same_device,
+    require_same_dtype,
+)
+
+__all__ = [
+    "FlashAttentionMaskPlan",
+    "_plan_tilelang_flash_attention_mask",
+    "amax",
+    "concrete_tensors",
+    "flash_attention",
+    "hip_flash_attention_kernel",
+    "hip_layer_norm_kernel",
+    "hip_rms_norm_kernel",
+    "layer_norm",
+    "linear",
+    "linear_fp8",
+    "plan_flash_attention_mask",
+    "quantize_fp8",
+    "require_cuda_tensors",
+    "require_same_device",
+    "require_same_dtype",
+    "resolved_flash_attention_backend",
+    "resolved_layer_norm_backend",
+    "resolved_rms_norm_backend",
+    "rms_norm",
+    "swiglu_ffn",
+    "swiglu_linear",
+]

@@ -1,0 +1,278 @@
+"""Flash-attention operator boundary backed by the gfx950 key-length kernel.
+
+Mirrors ``flash_attention`` and its mask planner
+(src/taac2026/infrastructure/accelerators/attention/flash_attention.py:107-209, 871-919). The kernel understands one
+mask family: a per-sample valid key prefix (``key_lengths``), optionally combined with a causal triangle. A 4-D bool
+``attn_mask`` is reduced to that form by :func:`plan_flash_attention_mask`, which accepts the same structured masks
+as the reference planner and rejects the rest with the reference's messages; callers that already know the lengths
+pass ``key_lengths=`` and skip the planning (and its device-to-host synchronisation) entirely.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from taac_2026_amd import _native
+from taac_2026_amd.accelerators.tensor_validation import (
+    require_cuda_tensors,
+    require_inference,
+    require_same_dtype,
+)
+
+FLASH_ATTENTION_BACKENDS = ("hip", "torch", "tilelang")
+
+
+@dataclass(frozen=True)
+class FlashAttentionMaskPlan:
+    """What the kernel needs to know about a mask (flash_attention.py:60-64)."""
+
+    key_lengths: torch.Tensor
+    query_self_mask: torch.Tensor | None
+    is_causal: bool
+
+
+def _normalize_flash_attention_inputs(
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Shape / dtype checks of flash_attention.py:107-123; layout is left alone (the kernel reads strides)."""
+    if q.ndim != 4 or k.ndim != 4 or v.ndim != 4:
+        raise ValueError("flash_attention expects q, k, and v with shape (batch, heads, seq_len, head_dim)")
+    if q.shape[0] != k.shape[0] or q.shape[0] != v.shape[0]:
+        raise ValueError("flash_attention requires matching batch dimensions")
+    if q.shape[1] != k.shape[1] or q.shape[1] != v.shape[1]:
+        raise ValueError("flash_attention requires matching head counts")
+    if k.shape[2] != v.shape[2]:
+        raise ValueError("flash_attention requires matching key and value sequence lengths")
+    if q.shape[3] != k.shape[3] or q.shape[3] != v.shape[3]:
+        raise ValueError("flash_attention requires matching head dimensions")
+    require_same_dtype("flash_attention", q, k, v)
+    return q, k, v
+
+
+def _full_key_lengths(q: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
+    return torch.full((q.shape[0],), k.shape[2], dtype=torch.int32, device=q.device)
+
+
+def _is_prefix_valid_mask(valid: torch.Tensor) -> bool:
+    """True iff every row of the (B, Tk) bool matrix is ``True`` on a prefix and ``False`` after it."""
+    lengths = valid.sum(dim=1, dtype=torch.int32).unsqueeze(1)
+    expected = torch.arange(valid.shape[1], device=valid.device).unsqueeze(0) < lengths
+    return bool(torch.equal(valid, expected))
+
+
+def _causal_valid_mask_from_lengths(lengths: torch.Tensor, token_count: int, num_heads: int) -> torch.Tensor:
+    """The mask ``causal_valid_attention_mask`` builds for prefix lengths (modeling/sequence.py:119-127)."""
+    positions = torch.arange(token_count, device=lengths.device)
+    padded = positions.unsqueeze(0) >= lengths.unsqueeze(1)  # (B, T)
+    lower = positions.unsqueeze(1) >= positions.unsqueeze(0)  # (T, T), query >= key
+    visible = lower.unsqueeze(0) & ~padded.unsqueeze(1)
+    diagonal = torch.eye(token_count, dtype=torch.bool, device=lengths.device).unsqueeze(0)
+    mask = torch.where(padded.unsqueeze(-1), diagonal, visible)
+    return mask.unsqueeze(1).expand(lengths.shape[0], num_heads, token_count, token_count)
+
+
+def plan_flash_attention_mask(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    attn_mask: torch.Tensor | None,
+    *,
+    is_causal: bool,
+) -> FlashAttentionMaskPlan:
+    """Reduce a bool mask to ``key_lengths`` (+ optional padded-query fallback), like flash_attention.py:149-198.
+
+    Accepted: ``None``; a (B, H, Tq, Tk) bool mask that is head-shared, query-broadcast and prefix-valid on keys;
+    a ``causal_valid_attention_mask``-style (B, H, T, T) mask. In addition to the reference, the broadcastable
+    key-padding forms (B, Tk) and (B, 1, 1, Tk) (True = attend) are accepted without expanding them.
+    """
+    if attn_mask is None:
+        return FlashAttentionMaskPlan(_full_key_lengths(q, k), None, is_causal)
+    if attn_mask.dtype is not torch.bool:
+        raise RuntimeError("hip flash_attention only supports structured bool attention masks")
+
+    batch, heads, query_len, kv_len = q.shape[0], q.shape[1], q.shape[2], k.shape[2]
+    key_valid: torch.Tensor | None = None
+    if attn_mask.ndim == 2 and attn_mask.shape == (batch, kv_len):
+        key_valid = attn_mask
+    elif attn_mask.ndim == 4 and attn_mask.shape == (batch, 1, 1, kv_len):
+        key_valid = attn_mask[:, 0, 0, :]
+    if key_valid is not None:
+        if not _is_prefix_valid_mask(key_valid):
+            raise RuntimeError("hip flash_attention requires bool key masks to be prefix-valid")
+        return FlashAttentionMaskPlan(key_valid.sum(dim=1, dtype=torch.int32), None, is_causal)
+
+    if attn_mask.ndim != 4 or attn_mask.shape != (batch, heads, query_len, kv_len):
+        raise RuntimeError(
+            "hip flash_attention only supports 4D bool masks matching (batch, heads, query_len, kv_len)"
+        )
+    first_head = attn_mask[:, :1]
+    if not torch.equal(attn_mask, first_head.expand_as(attn_mask)):
+        raise RuntimeError("hip flash_attention requires the bool attention mask to be shared across heads")
+
+    per_query = first_head[:, 0]  # (B, Tq, Tk)
+    if torch.equal(per_query, per_query[:, :1, :].expand_as(per_query)):
+        key_valid = per_query[:, 0, :]
+        if not _is_prefix_valid_mask(key_valid):
+            raise RuntimeError("hip flash_attention requires bool key masks to be prefix-valid")
+        return FlashAttentionMaskPlan(key_valid.sum(dim=1, dtype=torch.int32), None, is_causal)
+
+    if query_len != kv_len:
+        raise RuntimeError(
+            "hip flash_attention only supports non-broadcast bool masks when query and key lengths match"
+        )
+    query_lengths = per_query[:, :, 0].sum(dim=1, dtype=torch.int32)
+    if not torch.equal(attn_mask, _causal_valid_mask_from_lengths(query_lengths, query_len, heads)):
+        raise RuntimeError(
+            "hip flash_attention only supports prefix key masks or causal_valid_attention_mask-style bool masks"
+        )
+    positions = torch.arange(query_len, device=q.device).unsqueeze(0)
+    return FlashAttentionMaskPlan(query_lengths, positions >= query_lengths.unsqueeze(1), True)
+
+
+# Name under which the reference exports its planner (accelerators/__init__.py:83-138).
+_plan_tilelang_flash_attention_mask = plan_flash_attention_mask
+
+
+def _apply_query_self_mask_fallback(
+    output: torch.Tensor, value: torch.Tensor, query_self_mask: torch.Tensor | None
+) -> torch.Tensor:
+    """Padded query rows of a causal-valid mask attend only to themselves: their output is their value row."""
+    if query_self_mask is None:
+        return output
+    return torch.where(query_self_mask[:, None, :, None], value, output)
+
+
+def _resolve_flash_attention_backend(q: torch.Tensor, backend: str, *, dropout_p: float, training: bool) -> str:
+    if backend not in FLASH_ATTENTION_BACKENDS:
+        raise ValueError(f"unsupported flash attention backend: {backend}")
+    if dropout_p < 0.0 or dropout_p >= 1.0:
+        raise RuntimeError("hip flash_attention requires dropout_p to be in [0, 1)")
+    if training and dropout_p != 0.0:
+        raise RuntimeError("hip flash_attention is forward-only inference and does not apply dropout")
+    require_cuda_tensors("hip flash_attention", q)
+    return "hip"
+
+
+def resolved_flash_attention_backend(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    backend: str = "hip",
+    *,
+    attn_mask: torch.Tensor | None = None,
+    dropout_p: float = 0.0,
+    training: bool = False,
+    is_causal: bool = False,
+) -> str:
+    _normalize_flash_attention_inputs(q, k, v)
+    plan_flash_attention_mask(q, k, attn_mask, is_causal=is_causal)
+    return _resolve_flash_attention_backend(q, backend, dropout_p=dropout_p, training=training)
+
+
+def _kernel_view(t: torch.Tensor) -> torch.Tensor:
+    """Return ``t`` if the kernel can read it in place (unit last stride, other strides multiples of 8 elements,
+    16-byte aligned base), else a contiguous copy."""
+    strides = t.stride()
+    if strides[-1] == 1 and all(s % 8 == 0 and s >= 0 for s in strides[:-1]) and t.data_ptr() % 16 == 0:
+        return t
+    return t.contiguous()
+
+
+def hip_flash_attention_kernel(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    key_lengths: torch.Tensor | None,
+    *,
+    is_causal: bool = False,
+    zero_padded_queries: bool = False,
+) -> torch.Tensor:
+    """``(q, k, v: (B, H, T, d) bf16/fp16, key_lengths: int32[B]) -> (B, H, Tq, d)``.
+
+    Same contract as a kernel handed to the reference's ``register_flash_attention_kernel``
+    (flash_attention.py:26,102-104, called at :351-352), extended by the two keyword flags. The output keeps
+    q's memory layout, so (B, T, H, d)-strided views stay copy-free in both directions.
+    """
+    library = _native.load_library()
+    require_cuda_tensors("hip flash_attention", q, k, v, key_lengths)
+    if q.dtype not in (torch.bfloat16, torch.float16):
+        raise RuntimeError(f"hip flash_attention kernel does not support dtype {q.dtype}")
+    q, k, v = _kernel_view(q), _kernel_view(k), _kernel_view(v)
+    out = torch.empty_like(q)  # keeps q's dimension order in memory, without q's gaps
+    if out.stride(-1) != 1 or any(s % 8 for s in out.stride()[:-1]):
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    if key_lengths is not None:
+        if key_lengths.ndim != 1 or key_lengths.shape[0] != q.shape[0]:
+            raise ValueError("flash_attention key_lengths must have shape (batch,)")
+        if key_lengths.dtype != torch.int32 or not key_lengths.is_contiguous():
+            key_lengths = key_lengths.to(torch.int32).contiguous()
+    batch, heads, query_len, head_dim = q.shape
+    status = library.taac_flash_attn_fwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), out.data_ptr(),
+        batch, heads, query_len, k.shape[2], head_dim,
+        _native.Int64x4(*q.stride()), _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()),
+        _native.Int64x4(*out.stride()),
+        int(bool(is_causal)), int(bool(zero_padded_queries)), _native.dtype_code(q.dtype),
+        _native.current_stream(q.device),
+    )
+    _native.check(status, "flash_attention")
+    return out
+
+
+def flash_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    *,
+    backend: str = "hip",
+    attn_mask: torch.Tensor | None = None,
+    dropout_p: float = 0.0,
+    training: bool = False,
+    is_causal: bool = False,
+    block_m: int = 64,
+    block_n: int = 64,
+    num_stages: int = 1,
+    threads: int = 128,
+    key_lengths: torch.Tensor | None = None,
+    zero_padded_queries: bool = False,
+) -> torch.Tensor:
+    """``softmax(q k^T / sqrt(d) + mask) v`` for (B, H, T, d) tensors.
+
+    ``attn_mask`` is a bool mask with True = attend (structured as described in :func:`plan_flash_attention_mask`);
+    ``key_lengths`` (int32 [B]) states the valid key prefix directly and excludes ``attn_mask``.
+    fp32 inputs are computed in bf16 and returned as fp32, as the reference's accelerated path does
+    (flash_attention.py:249-252, 300-309). ``block_m`` .. ``threads`` are TileLang launch hints, accepted and ignored.
+    With ``zero_padded_queries`` the query rows at or beyond ``key_lengths[b]`` are returned as zeros; otherwise they
+    attend to the valid keys like every other row (the behaviour of the reference's torch and TileLang paths).
+    """
+    del block_m, block_n, num_stages, threads
+    q, k, v = _normalize_flash_attention_inputs(q, k, v)
+    _resolve_flash_attention_backend(q, backend, dropout_p=dropout_p, training=training)
+    require_inference("hip flash_attention", q, k, v)
+    if key_lengths is not None:
+        if attn_mask is not None:
+            raise ValueError("flash_attention takes either attn_mask or key_lengths, not both")
+        plan = FlashAttentionMaskPlan(key_lengths, None, is_causal)
+    else:
+        plan = plan_flash_attention_mask(q, k, attn_mask, is_causal=is_causal)
+    output_dtype = v.dtype
+    if q.dtype == torch.float32:
+        q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
+    lengths = plan.key_lengths if (attn_mask is not None or key_lengths is not None) else None
+    output = hip_flash_attention_kernel(
+        q, k, v, lengths, is_causal=plan.is_causal, zero_padded_queries=zero_padded_queries
+    )
+    output = _apply_query_self_mask_fallback(output, v, plan.query_self_mask)
+    return output if output.dtype == output_dtype else output.to(output_dtype)
+
+
+__all__ = [
+    "FLASH_ATTENTION_BACKENDS",
+    "FlashAttentionMaskPlan",
+    "_plan_tilelang_flash_attention_mask",
+    "flash_attention",
+    "hip_flash_attention_kernel",
+    "plan_flash_attention_mask",
+    "resolved_flash_attention_backend",
+]

@@ -1,0 +1,212 @@
+"""Dense-layer operators of the backbone block on gfx950 MFMA (bf16 and FP8 e4m3 operands).
+
+These replace the ``nn.Linear`` + elementwise sequences of the reference's block
+(experiments/symbiosis/backbone.py:11-68): ``linear`` covers QKV / output / down projections with an optional
+fused residual add, ``swiglu_linear`` is the up projection with ``silu(gate) * value`` fused into its epilogue, and
+the ``*_fp8`` functions are the per-tensor-scaled e4m3 variants (scale = amax / 448, fp32 accumulation, bf16 out).
+Weights use the torch ``nn.Linear`` layout ``[out_features, in_features]``.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from taac_2026_amd import _native
+from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference
+
+FP8_MAX = 448.0
+
+
+def _as_rows(x: torch.Tensor) -> tuple[torch.Tensor, torch.Size]:
+    if x.ndim < 2:
+        raise ValueError("linear expects input with at least 2 dimensions")
+    rows = x.reshape(-1, x.shape[-1])
+    if rows.stride(-1) != 1 or rows.stride(0) % 8 != 0 or rows.data_ptr() % 16 != 0:
+        rows = rows.contiguous()
+    return rows, x.shape
+
+
+def _check_bf16(operator_name: str, *tensors: torch.Tensor | None) -> None:
+    for t in tensors:
+        if t is not None and t.dtype != torch.bfloat16:
+            raise RuntimeError(f"{operator_name} expects bfloat16 tensors, got {t.dtype}")
+
+
+def _check_weight(operator_name: str, rows: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None) -> None:
+    if weight.ndim != 2:
+        raise ValueError(f"{operator_name} weight must be a 2D tensor [out_features, in_features]")
+    if rows.shape[-1] != weight.shape[1]:
+        raise ValueError(f"last dimension {rows.shape[-1]} does not match weight in_features {weight.shape[1]}")
+    if bias is not None and (bias.ndim != 1 or bias.shape[0] != weight.shape[0]):
+        raise ValueError(f"{operator_name} bias must have shape ({weight.shape[0]},)")
+
+
+def linear(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None = None,
+    *,
+    residual: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """``F.linear(x, weight, bias)`` (+ ``residual``) in bf16 with fp32 accumulation."""
+    name = "hip linear"
+    require_cuda_tensors(name, x, weight, bias, residual)
+    require_inference(name, x, weight, bias, residual)
+    _check_bf16(name, x, weight, bias, residual)
+    rows, shape = _as_rows(x)
+    _check_weight(name, rows, weight, bias)
+    weight = weight.contiguous()
+    out_features = weight.shape[0]
+    out = torch.empty((rows.shape[0], out_features), dtype=x.dtype, device=x.device)
+    res_rows = None
+    if residual is not None:
+        if residual.shape != (*shape[:-1], out_features):
+            raise ValueError("linear residual must have the shape of the output")
+        res_rows = residual.reshape(-1, out_features).contiguous()
+    library = _native.load_library()
+    status = library.taac_linear_bf16(
+        rows.data_ptr(), rows.stride(0), weight.data_ptr(), _native.ptr(bias), _native.ptr(res_rows), out.data_ptr(),
+        out_features, rows.shape[0], out_features, weight.shape[1],
+        _native.EPI_RESIDUAL if res_rows is not None else _native.EPI_NONE, 1, _native.current_stream(x.device),
+    )
+    _native.check(status, "linear")
+    return out.reshape(*shape[:-1], out_features)
+
+
+def swiglu_linear(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None = None,
+    *,
+    gate_first: bool = True,
+) -> torch.Tensor:
+    """``g, u = F.linear(x, weight, bias).chunk(2, -1); silu(g) * u`` (``g * silu(u)`` if not ``gate_first``)."""
+    name = "hip swiglu_linear"
+    require_cuda_tensors(name, x, weight, bias)
+    require_inference(name, x, weight, bias)
+    _check_bf16(name, x, weight, bias)
+    rows, shape = _as_rows(x)
+    _check_weight(name, rows, weight, bias)
+    if weight.shape[0] % 2 != 0:
+        raise ValueError("swiglu_linear weight must have an even number of output features")
+    weight = weight.contiguous()
+    hidden = weight.shape[0] // 2
+    out = torch.empty((rows.shape[0], hidden), dtype=x.dtype, device=x.device)
+    library = _native.load_library()
+    status = library.taac_linear_bf16(
+        rows.data_ptr(), rows.stride(0), weight.data_ptr(), _native.ptr(bias), None, out.data_ptr(), hidden,
+        rows.shape[0], weight.shape[0], weight.shape[1], _native.EPI_SWIGLU, int(bool(gate_first)),
+        _native.current_stream(x.device),
+    )
+    _native.check(status, "swiglu_linear")
+    return out.reshape(*shape[:-1], hidden)
+
+
+def swiglu_ffn(
+    x: torch.Tensor,
+    up_weight: torch.Tensor,
+    up_bias: torch.Tensor | None,
+    down_weight: torch.Tensor,
+    down_bias: torch.Tensor | None,
+    *,
+    residual: torch.Tensor | None = None,
+    gate_first: bool = True,
+) -> torch.Tensor:
+    """``down(silu(gate) * value)`` with ``gate, value = up(x).chunk(2, -1)``; optional fused ``+ residual``."""
+    hidden = swiglu_linear(x, up_weight, up_bias, gate_first=gate_first)
+    return linear(hidden, down_weight, down_bias, residual=residual)
+
+
+# ---- FP8 (OCP e4m3fn, per-tensor scale = amax / 448) ---------------------------------------------------------------
+
+
+def amax(x: torch.Tensor) -> torch.Tensor:
+    """``x.abs().max()`` as a float32 scalar tensor on x's device."""
+    name = "hip amax"
+    require_cuda_tensors(name, x)
+    x = x.contiguous()
+    out = torch.empty((), dtype=torch.float32, device=x.device)
+    library = _native.load_library()
+    status = library.taac_amax(x.data_ptr(), x.numel(), _native.dtype_code(x.dtype), out.data_ptr(),
+                               _native.current_stream(x.device))
+    _native.check(status, "amax")
+    return out
+
+
+def quantize_fp8(x: torch.Tensor, amax_value: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """Quantise to e4m3fn with scale ``amax / 448``. Returns ``(q as torch.float8_e4m3fn, amax float32 scalar)``."""
+    name = "hip quantize_fp8"
+    require_cuda_tensors(name, x, amax_value)
+    x = x.contiguous()
+    if amax_value is None:
+        amax_value = amax(x)
+    if amax_value.dtype != torch.float32 or amax_value.numel() != 1:
+        raise ValueError("quantize_fp8 amax must be a float32 scalar tensor")
+    q = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    library = _native.load_library()
+    status = library.taac_quantize_fp8(x.data_ptr(), x.numel(), _native.dtype_code(x.dtype), amax_value.data_ptr(),
+                                       q.data_ptr(), _native.current_stream(x.device))
+    _native.check(status, "quantize_fp8")
+    return q.view(torch.float8_e4m3fn), amax_value
+
+
+def linear_fp8(
+    x: torch.Tensor,
+    weight_fp8: torch.Tensor,
+    amax_x: torch.Tensor,
+    amax_w: torch.Tensor,
+    bias: torch.Tensor | None = None,
+    *,
+    residual: torch.Tensor | None = None,
+    swiglu: bool = False,
+    gate_first: bool = True,
+) -> torch.Tensor:
+    """``epilogue((q_x @ q_w^T) * s_x * s_w + bias)`` with e4m3 MFMA operands, bf16 result.
+
+    ``x`` is bf16 (quantised on load with scale ``amax_x / 448``) or already ``float8_e4m3fn``;
+    ``weight_fp8`` is ``float8_e4m3fn`` ``[out, in]`` quantised with scale ``amax_w / 448``.
+    ``swiglu`` selects the ``silu(gate) * value`` epilogue (output has ``out / 2`` features), ``residual`` the
+    fused residual add; they are exclusive.
+    """
+    name = "hip linear_fp8"
+    require_cuda_tensors(name, x, weight_fp8, amax_x, amax_w, bias, residual)
+    require_inference(name, x, bias, residual)
+    _check_bf16(name, bias, residual)
+    if weight_fp8.dtype != torch.float8_e4m3fn:
+        raise RuntimeError("linear_fp8 weight must be float8_e4m3fn")
+    if x.dtype not in (torch.bfloat16, torch.float8_e4m3fn):
+        raise RuntimeError(f"linear_fp8 activations must be bfloat16 or float8_e4m3fn, got {x.dtype}")
+    if swiglu and residual is not None:
+        raise ValueError("linear_fp8 cannot combine the swiglu and residual epilogues")
+    if x.ndim < 2:
+        raise ValueError("linear expects input with at least 2 dimensions")
+    shape = x.shape
+    rows = x.reshape(-1, shape[-1]).contiguous()
+    _check_weight(name, rows, weight_fp8, bias)
+    weight_fp8 = weight_fp8.contiguous()
+    n = weight_fp8.shape[0]
+    if swiglu and n % 2 != 0:
+        raise ValueError("swiglu weight must have an even number of output features")
+    out_features = n // 2 if swiglu else n
+    out = torch.empty((rows.shape[0], out_features), dtype=torch.bfloat16, device=x.device)
+    res_rows = residual.reshape(-1, out_features).contiguous() if residual is not None else None
+    epilogue = _native.EPI_SWIGLU if swiglu else (_native.EPI_RESIDUAL if res_rows is not None else _native.EPI_NONE)
+    library = _native.load_library()
+    status = library.taac_linear_fp8(
+        rows.data_ptr(), int(x.dtype == torch.float8_e4m3fn), rows.stride(0), weight_fp8.data_ptr(),
+        amax_x.data_ptr(), amax_w.data_ptr(), _native.ptr(bias), _native.ptr(res_rows), out.data_ptr(), out_features,
+        rows.shape[0], n, weight_fp8.shape[1], epilogue, int(bool(gate_first)), _native.current_stream(x.device),
+    )
+    _native.check(status, "linear_fp8")
+    return out.reshape(*shape[:-1], out_features)
+
+
+__all__ = [
+    "FP8_MAX",
+    "amax",
+    "linear",
+    "linear_fp8",
+    "quantize_fp8",
+    "swiglu_ffn",
+    "swiglu_linear",
+]

@@ -1,0 +1,346 @@
+// Key-padding-masked attention forward for gfx950.
+//
+// Work decomposition
+//   One workgroup (4 wavefronts) owns 128 query rows of one (batch, head); each wavefront owns 32 of them for the
+//   whole kernel, with its Q fragment, running max / sum and output accumulator in registers. Keys and values
+//   are streamed through LDS in chunks of 64 keys shared by the four wavefronts. Only key chunks below the
+//   sample's valid length are visited; query blocks entirely in the padding are either zero-filled or skipped.
+//   Sibling workgroups of the same (batch, head) get adjacent logical ids on the same accelerator die so that their
+//   K/V re-reads hit that die's L2.
+//
+// MFMA formulation (v_mfma_f32_32x32x16, 64-wide wavefront)
+//   Scores are computed transposed, S^T[key, query] = K Q^T, so that in the accumulator layout every lane owns ONE
+//   query column (lane % 32) and 16 of the tile's 32 keys: the softmax row reductions are in-register plus one
+//   exchange with lane ^ 32. The probabilities are then already in the B-operand layout of the second product
+//   O^T[d, query] = V^T P^T, so P never leaves registers. The accumulator's key order (4-key runs interleaved
+//   between the two lane halves) is matched by storing V^T in LDS with the same key permutation.
+//
+// Semantics follow the reference's inference kernel (accelerators/attention/kernels/tilelang.py:36-138): base-2
+// online softmax with scale log2(e)/sqrt(d), key j visible iff j < key_lengths[b] (and j <= i when causal),
+// P rounded to the storage dtype before the second product, rows with an empty visible set produce 0.
+#include <math.h>
+
+#include "common.h"
+
+namespace taac {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kQB = 128;  // query rows per workgroup
+constexpr int kKC = 64;   // keys per LDS chunk
+
+struct AttnParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;
+  const int32_t* key_lengths;
+  int32_t B, H, Tq, Tk, d;
+  int64_t qs[4], ks[4], vs[4], os[4];
+  float scale_log2;  // log2(e) / sqrt(d)
+  int32_t zero_pad;
+  uint32_t nqc;    // query chunks per (batch, head)
+  uint32_t total;  // workgroups
+};
+
+template <typename T>
+struct Mfma32;
+template <>
+struct Mfma32<bf16_t> {
+  static __device__ __forceinline__ f32x16 run(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma32<f16_t> {
+  static __device__ __forceinline__ f32x16 run(f16x8 a, f16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(T lo, T hi) {
+  return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, lo)) |
+         (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, hi)) << 16);
+}
+
+// Position of key k (0..15 inside a 16-key group) in the permuted V^T row: the accumulator layout gives lane half
+// hh = (k / 4) % 2 the keys {hh*4 .. hh*4+3} and {8 + hh*4 .. 8 + hh*4+3}; they become 8 consecutive elements.
+__device__ __forceinline__ int vt_pos16(int k) { return ((k >> 2) & 1) * 8 + (k >> 3) * 4 + (k & 3); }
+
+template <typename T, int DP, bool CAUSAL>
+__global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnParams p) {
+  typedef typename Vec8<T>::type vec_t;
+  typedef typename Vec8<T>::half_type vec4_t;
+  constexpr int KSTEPS = DP / 16;  // MFMA k-steps of the score product
+  constexpr int MB = DP / 32;      // 32-row blocks of O^T
+  constexpr int C8 = DP / 8;       // 128-bit column chunks per row
+  constexpr int KSTR = DP + 8;     // LDS row strides in elements (+16 bytes against bank conflicts)
+  constexpr int VSTR = kKC + 8;
+  __shared__ __attribute__((aligned(16))) T sK[kKC * KSTR];
+  __shared__ __attribute__((aligned(16))) T sVt[DP * VSTR];
+
+  const uint32_t logical = xcd_remap(blockIdx.x, p.total);
+  const int qc = static_cast<int>(logical % p.nqc);
+  const int bh = static_cast<int>(logical / p.nqc);
+  const int h = bh % p.H;
+  const int b = bh / p.H;
+
+  const int tid = threadIdx.x;
+  const int wave = tid / kWave;
+  const int lane = tid % kWave;
+  const int l32 = lane % 32;
+  const int hh = lane / 32;
+
+  const T* qb = static_cast<const T*>(p.q) + b * p.qs[0] + h * p.qs[1];
+  const T* kb = static_cast<const T*>(p.k) + b * p.ks[0] + h * p.ks[1];
+  const T* vb = static_cast<const T*>(p.v) + b * p.vs[0] + h * p.vs[1];
+  T* ob = static_cast<T*>(p.o) + b * p.os[0] + h * p.os[1];
+
+  int len = p.Tk;
+  if (p.key_lengths != nullptr) {
+    len = p.key_lengths[b];
+    len = len < 0 ? 0 : (len > p.Tk ? p.Tk : len);
+  }
+  const int q_begin = qc * kQB;
+  const int q_valid = p.zero_pad ? (len < p.Tq ? len : p.Tq) : p.Tq;  // rows at or beyond are written as zeros
+
+  vec_t zero_vec;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) zero_vec[e] = static_cast<T>(0.f);
+
+  if (q_begin >= q_valid) {
+    // Whole block lies in the padding: zero-fill its rows.
+    const int c8n = p.d / 8;
+    for (int idx = tid; idx < kQB * c8n; idx += kThreads) {
+      const int row = q_begin + idx / c8n;
+      const int c8 = idx % c8n;
+      if (row < p.Tq) *reinterpret_cast<vec_t*>(ob + row * p.os[2] + c8 * 8) = zero_vec;
+    }
+    return;
+  }
+
+  int kv_end = len;
+  if (CAUSAL) kv_end = kv_end < q_begin + kQB ? kv_end : q_begin + kQB;
+
+  // Q fragments: B operand of S^T = K Q^T; lane holds query row l32, features 16*s + 8*hh .. +7.
+  const int qi = q_begin + wave * 32 + l32;
+  vec_t qf[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    const int col = 16 * s + 8 * hh;
+    qf[s] = (qi < p.Tq && col < p.d) ? *reinterpret_cast<const vec_t*>(qb + qi * p.qs[2] + col) : zero_vec;
+  }
+
+  f32x16 oacc[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) oacc[mb][j] = 0.f;
+  float m_run = -INFINITY;
+  float l_run = 0.f;
+  const float c = p.scale_log2;
+
+  int wave_kv_end = kv_end;
+  if (CAUSAL) {
+    const int wlim = q_begin + wave * 32 + 32;
+    wave_kv_end = wave_kv_end < wlim ? wave_kv_end : wlim;
+  }
+
+  for (int kc0 = 0; kc0 < kv_end; kc0 += kKC) {
+    if (kc0 > 0) __syncthreads();
+    // ---- stage K chunk: sK[key][feature] ------------------------------------------------------------------
+    for (int idx = tid; idx < kKC * C8; idx += kThreads) {
+      const int key = idx / C8;
+      const int c8 = idx % C8;
+      const int kidx = kc0 + key;
+      vec_t val = zero_vec;
+      if (kidx < kv_end && c8 * 8 < p.d) val = *reinterpret_cast<const vec_t*>(kb + kidx * p.ks[2] + c8 * 8);
+      *reinterpret_cast<vec_t*>(&sK[key * KSTR + c8 * 8]) = val;
+    }
+    // ---- stage V chunk transposed and key-permuted: sVt[feature][pos(key)] ---------------------------------
+    for (int idx = tid; idx < (kKC / 2) * C8; idx += kThreads) {
+      const int pair = idx / C8;
+      const int c8 = idx % C8;
+      const int key0 = 2 * pair;
+      const int kidx = kc0 + key0;
+      vec_t v0 = zero_vec, v1 = zero_vec;
+      if (c8 * 8 < p.d) {
+        if (kidx < kv_end) v0 = *reinterpret_cast<const vec_t*>(vb + kidx * p.vs[2] + c8 * 8);
+        if (kidx + 1 < kv_end) v1 = *reinterpret_cast<const vec_t*>(vb + (kidx + 1) * p.vs[2] + c8 * 8);
+      }
+      const int pos = (key0 & ~15) + vt_pos16(key0 & 15);  // even; key0 + 1 lands at pos + 1
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        *reinterpret_cast<uint32_t*>(&sVt[(c8 * 8 + i) * VSTR + pos]) = pack2<T>(v0[i], v1[i]);
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int kt = 0; kt < kKC / 32; ++kt) {
+      const int k0 = kc0 + kt * 32;
+      if (k0 >= wave_kv_end) break;  // wavefront-uniform
+
+      // ---- S^T tile: 32 keys x 32 queries ---------------------------------------------------------------
+      f32x16 sacc;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) sacc[j] = 0.f;
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) {
+        const vec_t a = *reinterpret_cast<const vec_t*>(&sK[(kt * 32 + l32) * KSTR + 16 * s + 8 * hh]);
+        sacc = Mfma32<T>::run(a, qf[s], sacc);
+      }
+      const bool tail = (k0 + 32 > kv_end) || (CAUSAL && (k0 + 31 > q_begin + wave * 32));
+      if (tail) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const int key = k0 + (j / 4) * 8 + hh * 4 + (j % 4);
+          const bool masked = key >= kv_end || (CAUSAL && key > qi);
+          if (masked) sacc[j] = -INFINITY;
+        }
+      }
+      // ---- online softmax, one query per lane (pair of lanes l, l ^ 32) ------------------------------------
+      float mx = sacc[0];
+#pragma unroll
+      for (int j = 1; j < 16; ++j) mx = fmaxf(mx, sacc[j]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
+      const float mc = -m_use * c;
+      float pr[16];
+      float rs = 0.f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        pr[j] = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, mc));
+        rs += pr[j];
+      }
+      rs += __shfl_xor(rs, 32, kWave);
+      l_run = l_run * alpha + rs;
+      m_run = m_new;
+      vec_t pb[2];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        pb[0][e] = static_cast<T>(pr[e]);
+        pb[1][e] = static_cast<T>(pr[8 + e]);
+      }
+      // ---- O^T += V^T P^T --------------------------------------------------------------------------------
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const vec_t a =
+              *reinterpret_cast<const vec_t*>(&sVt[(mb * 32 + l32) * VSTR + kt * 32 + s2 * 16 + hh * 8]);
+          oacc[mb] = Mfma32<T>::run(a, pb[s2], oacc[mb]);
+        }
+      }
+    }
+  }
+
+  // ---- finalise: O / l, zero rows in the padding, store 4 consecutive features per register group -------------
+  const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+  const float fin = (qi < q_valid) ? inv : 0.f;
+  if (qi < p.Tq) {
+    T* orow = ob + qi * p.os[2];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+      for (int jq = 0; jq < 4; ++jq) {
+        const int col = mb * 32 + jq * 8 + hh * 4;
+        if (col < p.d) {
+          vec4_t ov;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) ov[e] = static_cast<T>(oacc[mb][jq * 4 + e] * fin);
+          *reinterpret_cast<vec4_t*>(orow + col) = ov;
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int DP>
+void launch(const AttnParams& p, bool causal, hipStream_t s) {
+  if (causal)
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  else
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+}
+
+template <typename T>
+void launch_dp(const AttnParams& p, bool causal, hipStream_t s) {
+  if (p.d <= 32)
+    launch<T, 32>(p, causal, s);
+  else if (p.d <= 64)
+    launch<T, 64>(p, causal, s);
+  else
+    launch<T, 128>(p, causal, s);
+}
+
+bool strides_ok(const int64_t* st) {
+  if (st[3] != 1) return false;
+  for (int i = 0; i < 3; ++i)
+    if (st[i] % 8 != 0 || st[i] < 0) return false;
+  return true;
+}
+
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_flash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths, void* o,
+                                   int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                                   const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
+                                   const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype,
+                                   void* stream) {
+  using namespace taac;
+  const char* name = "taac_flash_attn_fwd";
+  if (B < 0 || H < 0 || Tq < 0 || Tk < 0 || d <= 0)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: negative dimension or non-positive head_dim", name);
+  if (dtype != TAAC_BF16 && dtype != TAAC_F16)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: dtype must be bf16 or fp16 (got %d)", name, dtype);
+  if (d % 8 != 0 || d > 128)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: head_dim %d unsupported (multiple of 8, at most 128)", name, d);
+  if (!q_strides || !k_strides || !v_strides || !o_strides)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: null stride array", name);
+  if (B == 0 || H == 0 || Tq == 0) return TAAC_OK;
+  if (!q || !o || (Tk > 0 && (!k || !v))) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
+  if (!strides_ok(q_strides) || !strides_ok(k_strides) || !strides_ok(v_strides) || !strides_ok(o_strides))
+    return set_error(TAAC_ERR_UNSUPPORTED,
+                     "%s: strides must be non-negative multiples of 8 elements with a unit last stride", name);
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
+  if (zero_padded_queries && Tq != Tk)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: zero_padded_queries requires Tq == Tk", name);
+
+  AttnParams p;
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.o = o;
+  p.key_lengths = key_lengths;
+  p.B = B;
+  p.H = H;
+  p.Tq = Tq;
+  p.Tk = Tk;
+  p.d = d;
+  for (int i = 0; i < 4; ++i) {
+    p.qs[i] = q_strides[i];
+    p.ks[i] = k_strides[i];
+    p.vs[i] = v_strides[i];
+    p.os[i] = o_strides[i];
+  }
+  p.scale_log2 = 1.4426950408889634f / sqrtf(static_cast<float>(d));
+  p.zero_pad = zero_padded_queries ? 1 : 0;
+  p.nqc = static_cast<uint32_t>((Tq + kQB - 1) / kQB);
+  const int64_t total = static_cast<int64_t>(p.nqc) * B * H;
+  if (total > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many workgroups (%lld)", name, (long long)total);
+  p.total = static_cast<uint32_t>(total);
+
+  hipStream_t s = as_stream(stream);
+  if (dtype == TAAC_BF16)
+    launch_dp<bf16_t>(p, is_causal != 0, s);
+  else
+    launch_dp<f16_t>(p, is_causal != 0, s);
+  return check_launch(name);
+}

@@ -1,0 +1,159 @@
+// Forward driver of the unified token backbone (pre-norm blocks + pCVR readout) and the readout kernel.
+// The driver only sequences the library's own entry points on one stream over a caller-provided workspace.
+#include "common.h"
+
+namespace taac {
+namespace {
+
+constexpr int kBlock = 256;
+
+inline int64_t align256(int64_t v) { return (v + 255) & ~static_cast<int64_t>(255); }
+
+// One workgroup per sample: fp32 sum over the valid prefix of the sample's tokens, mean, dot with the head weight,
+// sigmoid. Thread layout: chunk = tid % (D/8) picks 8 features, group = tid / (D/8) strides over tokens.
+__global__ __launch_bounds__(kBlock) void masked_mean_head_kernel(const bf16_t* __restrict__ x,
+                                                                  const int32_t* __restrict__ lengths,
+                                                                  const bf16_t* __restrict__ w_head,
+                                                                  const bf16_t* __restrict__ b_head,
+                                                                  float* __restrict__ p, int T, int D) {
+  __shared__ float s_acc[kBlock][8];
+  __shared__ float s_dot[kBlock];
+  const int b = blockIdx.x;
+  const int c8n = D / 8;
+  const int groups = kBlock / c8n;
+  const int chunk = threadIdx.x % c8n;
+  const int group = threadIdx.x / c8n;
+  int len = lengths[b];
+  len = len < 0 ? 0 : (len > T ? T : len);
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  if (group < groups) {
+    const bf16_t* xb = x + static_cast<int64_t>(b) * T * D + chunk * 8;
+    for (int t = group; t < len; t += groups) {
+      const bf16x8 v = *reinterpret_cast<const bf16x8*>(xb + static_cast<int64_t>(t) * D);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += static_cast<float>(v[e]);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) s_acc[threadIdx.x][e] = acc[e];
+  __syncthreads();
+  float dot = 0.f;
+  if (threadIdx.x < c8n) {
+    const float denom = static_cast<float>(len < 1 ? 1 : len);
+    const bf16x8 wv = *reinterpret_cast<const bf16x8*>(w_head + threadIdx.x * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float s = 0.f;
+      for (int g = 0; g < groups; ++g) s += s_acc[g * c8n + threadIdx.x][e];
+      dot += (s / denom) * static_cast<float>(wv[e]);
+    }
+  }
+  s_dot[threadIdx.x] = dot;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float z = b_head != nullptr ? static_cast<float>(b_head[0]) : 0.f;
+    for (int i = 0; i < c8n; ++i) z += s_dot[i];
+    p[b] = 1.0f / (1.0f + expf(-z));
+  }
+}
+
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_masked_mean_head(const void* x, const int32_t* lengths, const void* w_head, const void* b_head,
+                                     float* p, int32_t B, int32_t T, int32_t D, void* stream) {
+  using namespace taac;
+  const char* name = "taac_masked_mean_head";
+  if (B < 0 || T < 0 || D <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: bad dimensions", name);
+  if (D % 8 != 0 || D > 8 * kBlock)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: D=%d must be a multiple of 8 and at most %d", name, D, 8 * kBlock);
+  if (B == 0) return TAAC_OK;
+  if (!x || !lengths || !w_head || !p) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  if (!aligned16(x) || !aligned16(w_head))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: x and w_head must be 16-byte aligned", name);
+  hipLaunchKernelGGL(masked_mean_head_kernel, dim3(B), dim3(kBlock), 0, as_stream(stream),
+                     static_cast<const bf16_t*>(x), lengths, static_cast<const bf16_t*>(w_head),
+                     static_cast<const bf16_t*>(b_head), p, T, D);
+  return check_launch(name);
+}
+
+extern "C" int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D, int32_t F) {
+  using namespace taac;
+  if (B < 0 || T < 0 || D <= 0 || F <= 0) return -1;
+  const int64_t M = static_cast<int64_t>(B) * T;
+  // x, h (shared with the attention output), qkv, gated hidden
+  return align256(M * D * 2) * 2 + align256(M * 3 * D * 2) + align256(M * F * 2);
+}
+
+extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, const taac_block_weights* blocks,
+                                 int32_t n_blocks, const void* w_head, const void* b_head, int32_t B, int32_t T,
+                                 int32_t D, int32_t heads, int32_t F, float eps, void* workspace,
+                                 int64_t workspace_bytes, void* hidden_out, float* p, void* stream) {
+  using namespace taac;
+  const char* name = "taac_backbone_fwd";
+  if (B < 0 || T < 0 || D <= 0 || F <= 0 || heads <= 0 || n_blocks < 0)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: bad dimensions", name);
+  if (D % heads != 0 || (D / heads) % 8 != 0 || D / heads > 128)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: D=%d heads=%d: head_dim must be a multiple of 8, at most 128", name, D,
+                     heads);
+  if (D % 8 != 0 || F % 8 != 0) return set_error(TAAC_ERR_UNSUPPORTED, "%s: D and F must be multiples of 8", name);
+  if (B == 0 || T == 0) return TAAC_OK;
+  if (!emb || !key_lengths || !p || !w_head || (n_blocks > 0 && !blocks))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  const int64_t need = taac_backbone_workspace_bytes(B, T, D, F);
+  if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: workspace must be 256-byte aligned and hold %lld bytes", name,
+                     (long long)need);
+
+  const int64_t M = static_cast<int64_t>(B) * T;
+  char* ws = static_cast<char*>(workspace);
+  bf16_t* x = reinterpret_cast<bf16_t*>(ws);
+  ws += align256(M * D * 2);
+  bf16_t* h = reinterpret_cast<bf16_t*>(ws);
+  ws += align256(M * D * 2);
+  bf16_t* qkv = reinterpret_cast<bf16_t*>(ws);
+  ws += align256(M * 3 * D * 2);
+  bf16_t* g = reinterpret_cast<bf16_t*>(ws);
+
+  const int dh = D / heads;
+  const int64_t qkv_strides[4] = {static_cast<int64_t>(T) * 3 * D, dh, 3 * static_cast<int64_t>(D), 1};
+  const int64_t o_strides[4] = {static_cast<int64_t>(T) * D, dh, D, 1};
+
+  const bf16_t* cur = static_cast<const bf16_t*>(emb);
+  int rc;
+  for (int i = 0; i < n_blocks; ++i) {
+    const taac_block_weights& w = blocks[i];
+    if (!w.attn_norm_weight || !w.qkv_weight || !w.out_weight || !w.ffn_norm_weight || !w.up_weight || !w.down_weight)
+      return set_error(TAAC_ERR_INVALID_VALUE, "%s: block %d has a null weight", name, i);
+    const bool last = (i == n_blocks - 1);
+    bf16_t* x_out = (last && hidden_out != nullptr) ? static_cast<bf16_t*>(hidden_out) : x;
+    // attention half
+    if ((rc = taac_rmsnorm_fwd(cur, w.attn_norm_weight, h, M, D, eps, TAAC_BF16, stream)) != TAAC_OK) return rc;
+    if ((rc = taac_linear_bf16(h, D, w.qkv_weight, w.qkv_bias, nullptr, qkv, 3 * D, M, 3 * D, D, TAAC_EPI_NONE, 1,
+                               stream)) != TAAC_OK)
+      return rc;
+    if ((rc = taac_flash_attn_fwd(qkv, qkv + D, qkv + 2 * D, key_lengths, h, B, heads, T, T, dh, qkv_strides,
+                                  qkv_strides, qkv_strides, o_strides, 0, 1, TAAC_BF16, stream)) != TAAC_OK)
+      return rc;
+    if ((rc = taac_linear_bf16(h, D, w.out_weight, w.out_bias, cur, x, D, M, D, D, TAAC_EPI_RESIDUAL, 1, stream)) !=
+        TAAC_OK)
+      return rc;
+    // feed-forward half
+    if ((rc = taac_rmsnorm_fwd(x, w.ffn_norm_weight, h, M, D, eps, TAAC_BF16, stream)) != TAAC_OK) return rc;
+    if ((rc = taac_linear_bf16(h, D, w.up_weight, w.up_bias, nullptr, g, F, M, 2 * F, D, TAAC_EPI_SWIGLU, 1, stream)) !=
+        TAAC_OK)
+      return rc;
+    if ((rc = taac_linear_bf16(g, F, w.down_weight, w.down_bias, x, x_out, D, M, D, F, TAAC_EPI_RESIDUAL, 1, stream)) !=
+        TAAC_OK)
+      return rc;
+    cur = x_out;
+  }
+  if (n_blocks == 0 && hidden_out != nullptr) {
+    if (hipMemcpyAsync(hidden_out, emb, static_cast<size_t>(M) * D * 2, hipMemcpyDeviceToDevice, as_stream(stream)) !=
+        hipSuccess)
+      return set_error(TAAC_ERR_LAUNCH, "%s: copy of the embeddings failed", name);
+  }
+  return taac_masked_mean_head(cur, key_lengths, w_head, b_head, p, B, T, D, stream);
+}

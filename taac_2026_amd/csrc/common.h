@@ -1,0 +1,76 @@
+// Shared device/host helpers for the gfx950 kernels of libtaac_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/taac_hip.h"
+
+namespace taac {
+
+// ---- vector / element types -------------------------------------------------------------------------------------
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(_Float16)))) _Float16 f16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2;
+typedef __attribute__((__vector_size__(8 * sizeof(int)))) int i32x8;
+
+constexpr int kWave = 64;     // CDNA wavefront width
+constexpr int kNumXcd = 8;    // MI355X: 8 accelerator dies, workgroup i is dispatched to die i % 8
+
+// ---- host-side error plumbing -----------------------------------------------------------------------------------
+int set_error(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+__host__ __device__ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- device helpers ---------------------------------------------------------------------------------------------
+template <typename T>
+struct Vec8;  // eight 16-bit elements = one 128-bit access
+template <>
+struct Vec8<bf16_t> {
+  typedef bf16x8 type;
+  typedef bf16x4 half_type;
+};
+template <>
+struct Vec8<f16_t> {
+  typedef f16x8 type;
+  typedef f16x4 half_type;
+};
+
+__device__ __forceinline__ float wave_shfl_xor(float v, int mask) { return __shfl_xor(v, mask, kWave); }
+
+// Sum / max over groups of G consecutive lanes (G a power of two <= 64). Every lane of a group gets the result.
+template <int G>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int off = G / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+template <int G>
+__device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+  for (int off = G / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+// Logical -> physical workgroup id so that consecutive logical ids run on the same accelerator die (and share its
+// L2). Hardware sends physical id p to die p % 8; die x is given the contiguous logical range starting at
+// x * (total / 8) + min(x, total % 8).
+__device__ __forceinline__ uint32_t xcd_remap(uint32_t pid, uint32_t total) {
+  const uint32_t xcd = pid % kNumXcd;
+  const uint32_t local = pid / kNumXcd;
+  const uint32_t base = total / kNumXcd;
+  const uint32_t rem = total % kNumXcd;
+  const uint32_t start = xcd * base + (xcd < rem ? xcd : rem);
+  return start + local;
+}
+
+}  // namespace taac

@@ -1,0 +1,279 @@
+// RMSNorm / LayerNorm forward for gfx950: single-pass row kernels.
+//
+// A row is owned by a group of G consecutive lanes of one wavefront (G = 1..64, a power of two). Each lane keeps
+// NV 128-bit vectors of the row in registers, so x is read from HBM exactly once and y written exactly once;
+// the reductions are wavefront shuffles inside the lane group and all arithmetic is fp32. Consecutive groups own
+// consecutive rows, so a wavefront's loads and stores cover one contiguous span of memory.
+//
+// Arithmetic follows the reference's closed forms
+//   RMSNorm:   y = x * rsqrt(mean(x^2) + eps) * w      (accelerators/normalization/rms_norm.py:71-73)
+//   LayerNorm: y = (x - mean) * rsqrt(var + eps) * w + b, var from centred values
+//                                                      (normalization/kernels/triton.py:224-247)
+#include "common.h"
+
+namespace taac {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kMaxNV = 8;
+
+template <typename T>
+struct Pack;
+template <>
+struct Pack<float> {
+  static constexpr int VEC = 4;
+  typedef f32x4 vec;
+  static __device__ __forceinline__ void unpack(const vec& v, float* f) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) f[i] = v[i];
+  }
+  static __device__ __forceinline__ vec pack(const float* f) {
+    vec v;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = f[i];
+    return v;
+  }
+};
+template <>
+struct Pack<bf16_t> {
+  static constexpr int VEC = 8;
+  typedef bf16x8 vec;
+  static __device__ __forceinline__ void unpack(const vec& v, float* f) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) f[i] = static_cast<float>(v[i]);
+  }
+  static __device__ __forceinline__ vec pack(const float* f) {
+    vec v;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = static_cast<bf16_t>(f[i]);
+    return v;
+  }
+};
+template <>
+struct Pack<f16_t> {
+  static constexpr int VEC = 8;
+  typedef f16x8 vec;
+  static __device__ __forceinline__ void unpack(const vec& v, float* f) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) f[i] = static_cast<float>(v[i]);
+  }
+  static __device__ __forceinline__ vec pack(const float* f) {
+    vec v;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = static_cast<f16_t>(f[i]);
+    return v;
+  }
+};
+
+// One block = 256 / G lane groups, each group normalises R rows per launch slot.
+template <typename T, int G, int NV, int R, bool LN>
+__global__ __launch_bounds__(kBlock) void norm_rows_vec_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                               const T* __restrict__ b, T* __restrict__ y,
+                                                               int64_t rows, int cols, int nvec, float eps) {
+  typedef Pack<T> P;
+  typedef typename P::vec vec_t;
+  constexpr int VEC = P::VEC;
+  constexpr int GPB = kBlock / G;  // lane groups (rows in flight) per block
+  const int lane = threadIdx.x % G;
+  const int gid = threadIdx.x / G;
+
+  // Issue every load of this thread before touching the data: R * NV independent 128-bit loads in flight.
+  vec_t raw[R][NV];
+  bool row_ok[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t row = (static_cast<int64_t>(blockIdx.x) * R + r) * GPB + gid;
+    row_ok[r] = row < rows;
+    const vec_t* xr = reinterpret_cast<const vec_t*>(x + row * cols);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = lane + i * G;
+      if (row_ok[r] && v < nvec) {
+        raw[r][i] = __builtin_nontemporal_load(xr + v);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) raw[r][i][e] = 0;
+      }
+    }
+  }
+
+  float wf[NV][VEC];
+  float bf[LN ? NV : 1][VEC];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = lane + i * G;
+    if (v < nvec) {
+      P::unpack(reinterpret_cast<const vec_t*>(w)[v], wf[i]);
+      if (LN) P::unpack(reinterpret_cast<const vec_t*>(b)[v], bf[LN ? i : 0]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        wf[i][e] = 0.f;
+        if (LN) bf[LN ? i : 0][e] = 0.f;
+      }
+    }
+  }
+
+  const float inv_cols = 1.0f / static_cast<float>(cols);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float xf[NV][VEC];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) P::unpack(raw[r][i], xf[i]);
+
+    float mean = 0.f;
+    if (LN) {
+      float s = 0.f;
+#pragma unroll
+      for (int i = 0; i < NV; ++i)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) s += xf[i][e];
+      mean = group_sum<G>(s) * inv_cols;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const bool live = (lane + i * G) < nvec;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float c = LN ? (live ? xf[i][e] - mean : 0.f) : xf[i][e];
+        ss += c * c;
+      }
+    }
+    ss = group_sum<G>(ss);
+    const float scale = rsqrtf(ss * inv_cols + eps);
+
+    if (row_ok[r]) {
+      const int64_t row = (static_cast<int64_t>(blockIdx.x) * R + r) * GPB + gid;
+      vec_t* yr = reinterpret_cast<vec_t*>(y + row * cols);
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int v = lane + i * G;
+        if (v < nvec) {
+          float of[VEC];
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            if (LN)
+              of[e] = (xf[i][e] - mean) * scale * wf[i][e] + bf[LN ? i : 0][e];
+            else
+              of[e] = xf[i][e] * scale * wf[i][e];
+          }
+          __builtin_nontemporal_store(P::pack(of), yr + v);
+        }
+      }
+    }
+  }
+}
+
+// Fallback for column counts that are not a whole number of 128-bit vectors, unaligned bases, or very long rows:
+// one wavefront per row, element-wise loads; the second and third sweep of a row come from cache.
+template <typename T, bool LN>
+__global__ __launch_bounds__(kBlock) void norm_rows_generic_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                   const T* __restrict__ b, T* __restrict__ y,
+                                                                   int64_t rows, int cols, float eps) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + threadIdx.x / kWave;
+  if (row >= rows) return;
+  const T* xr = x + row * cols;
+  T* yr = y + row * cols;
+  const float inv_cols = 1.0f / static_cast<float>(cols);
+  float mean = 0.f;
+  if (LN) {
+    float s = 0.f;
+    for (int c = lane; c < cols; c += kWave) s += static_cast<float>(xr[c]);
+    mean = group_sum<kWave>(s) * inv_cols;
+  }
+  float ss = 0.f;
+  for (int c = lane; c < cols; c += kWave) {
+    const float d = static_cast<float>(xr[c]) - mean;
+    ss += d * d;
+  }
+  ss = group_sum<kWave>(ss);
+  const float scale = rsqrtf(ss * inv_cols + eps);
+  for (int c = lane; c < cols; c += kWave) {
+    const float xv = static_cast<float>(xr[c]);
+    float o;
+    if (LN)
+      o = (xv - mean) * scale * static_cast<float>(w[c]) + static_cast<float>(b[c]);
+    else
+      o = xv * scale * static_cast<float>(w[c]);
+    yr[c] = static_cast<T>(o);
+  }
+}
+
+template <typename T, int G, int NV, bool LN>
+void launch_vec(const T* x, const T* w, const T* b, T* y, int64_t rows, int cols, int nvec, float eps,
+                hipStream_t s) {
+  constexpr int R = (NV <= 2) ? 2 : 1;
+  constexpr int GPB = kBlock / G;
+  const int64_t rows_per_block = static_cast<int64_t>(GPB) * R;
+  const int64_t grid = (rows + rows_per_block - 1) / rows_per_block;
+  hipLaunchKernelGGL((norm_rows_vec_kernel<T, G, NV, R, LN>), dim3(static_cast<uint32_t>(grid)), dim3(kBlock), 0, s,
+                     x, w, b, y, rows, cols, nvec, eps);
+}
+
+template <typename T, bool LN>
+int dispatch(const void* xv, const void* wv, const void* bv, void* yv, int64_t rows, int cols, float eps,
+             hipStream_t s) {
+  const T* x = static_cast<const T*>(xv);
+  const T* w = static_cast<const T*>(wv);
+  const T* b = static_cast<const T*>(bv);
+  T* y = static_cast<T*>(yv);
+  constexpr int VEC = Pack<T>::VEC;
+  const bool vec_ok = (cols % VEC == 0) && aligned16(x) && aligned16(y) && aligned16(w) && (!LN || aligned16(b)) &&
+                      (cols / VEC) <= kWave * kMaxNV;
+  if (!vec_ok) {
+    const int64_t grid = (rows + (kBlock / kWave) - 1) / (kBlock / kWave);
+    hipLaunchKernelGGL((norm_rows_generic_kernel<T, LN>), dim3(static_cast<uint32_t>(grid)), dim3(kBlock), 0, s, x, w,
+                       b, y, rows, cols, eps);
+    return TAAC_OK;
+  }
+  const int nvec = cols / VEC;
+#define TAAC_NORM_CASE(G, NV)                                          \
+  launch_vec<T, G, NV, LN>(x, w, b, y, rows, cols, nvec, eps, s);      \
+  return TAAC_OK;
+  if (nvec <= 1) { TAAC_NORM_CASE(1, 1) }
+  if (nvec <= 2) { TAAC_NORM_CASE(2, 1) }
+  if (nvec <= 4) { TAAC_NORM_CASE(4, 1) }
+  if (nvec <= 8) { TAAC_NORM_CASE(8, 1) }
+  if (nvec <= 16) { TAAC_NORM_CASE(16, 1) }
+  if (nvec <= 32) { TAAC_NORM_CASE(32, 1) }
+  if (nvec <= 64) { TAAC_NORM_CASE(64, 1) }
+  if (nvec <= 128) { TAAC_NORM_CASE(64, 2) }
+  if (nvec <= 256) { TAAC_NORM_CASE(64, 4) }
+  TAAC_NORM_CASE(64, 8)
+#undef TAAC_NORM_CASE
+}
+
+template <bool LN>
+int norm_entry(const char* name, const void* x, const void* w, const void* b, void* y, int64_t rows, int32_t cols,
+               float eps, int dtype, void* stream) {
+  if (rows < 0 || cols <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows must be >= 0 and cols > 0", name);
+  if (rows == 0) return TAAC_OK;
+  if (!x || !w || !y || (LN && !b)) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
+  const int64_t max_rows = static_cast<int64_t>(0x7fffffff) * 1;  // grid.x limit with >= 1 row per block
+  if (rows > max_rows) return set_error(TAAC_ERR_UNSUPPORTED, "%s: more than 2^31-1 rows", name);
+  hipStream_t s = as_stream(stream);
+  int rc;
+  switch (dtype) {
+    case TAAC_F32: rc = dispatch<float, LN>(x, w, b, y, rows, cols, eps, s); break;
+    case TAAC_BF16: rc = dispatch<bf16_t, LN>(x, w, b, y, rows, cols, eps, s); break;
+    case TAAC_F16: rc = dispatch<f16_t, LN>(x, w, b, y, rows, cols, eps, s); break;
+    default: return set_error(TAAC_ERR_INVALID_VALUE, "%s: unknown dtype %d", name, dtype);
+  }
+  if (rc != TAAC_OK) return rc;
+  return check_launch(name);
+}
+
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_rmsnorm_fwd(const void* x, const void* w, void* y, int64_t rows, int32_t cols, float eps,
+                                int dtype, void* stream) {
+  return taac::norm_entry<false>("taac_rmsnorm_fwd", x, w, nullptr, y, rows, cols, eps, dtype, stream);
+}
+
+extern "C" int taac_layernorm_fwd(const void* x, const void* w, const void* b, void* y, int64_t rows, int32_t cols,
+                                  float eps, int dtype, void* stream) {
+  return taac::norm_entry<true>("taac_layernorm_fwd", x, w, b, y, rows, cols, eps, dtype, stream);
+}

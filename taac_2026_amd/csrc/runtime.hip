@@ -1,0 +1,28 @@
+// Error reporting and ABI version of libtaac_hip.so.
+#include <cstdarg>
+#include <cstdio>
+
+#include "common.h"
+
+namespace taac {
+
+static thread_local char g_last_error[512] = "";
+
+int set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return set_error(TAAC_ERR_LAUNCH, "%s: HIP launch failed: %s", what, hipGetErrorString(e));
+  return TAAC_OK;
+}
+
+}  // namespace taac
+
+extern "C" int taac_abi_version(void) { return TAAC_ABI_VERSION; }
+extern "C" const char* taac_last_error(void) { return taac::g_last_error; }

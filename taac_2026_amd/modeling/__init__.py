@@ -1,0 +1,41 @@
+"""Model-level primitives built on the HIP operators."""
+
+from taac_2026_amd.modeling.backbone import (
+    PCVRBackbone,
+    SwiGLUFeedForward,
+    UnifiedInteractionBlock,
+    UnifiedSelfAttention,
+)
+from taac_2026_amd.modeling.normalization import (
+    LayerNorm,
+    RMSNorm,
+    configure_rms_norm_runtime,
+    rms_norm_runtime_state,
+)
+from taac_2026_amd.modeling.sequence import (
+    causal_valid_attention_mask,
+    configure_flash_attention_runtime,
+    flash_attention_runtime_state,
+    make_padding_mask,
+    masked_mean,
+    safe_key_padding_mask,
+    scaled_dot_product_attention,
+)
+
+__all__ = [
+    "LayerNorm",
+    "PCVRBackbone",
+    "RMSNorm",
+    "SwiGLUFeedForward",
+    "UnifiedInteractionBlock",
+    "UnifiedSelfAttention",
+    "causal_valid_attention_mask",
+    "configure_flash_attention_runtime",
+    "configure_rms_norm_runtime",
+    "flash_attention_runtime_state",
+    "make_padding_mask",
+    "masked_mean",
+    "rms_norm_runtime_state",
+    "safe_key_padding_mask",
+    "scaled_dot_product_attention",
+]

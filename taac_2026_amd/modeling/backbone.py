@@ -1,0 +1,224 @@
+"""Unified token backbone blocks on the HIP kernels.
+
+``SwiGLUFeedForward`` / ``UnifiedSelfAttention`` / ``UnifiedInteractionBlock`` keep the constructor signatures,
+parameter names (``up``, ``down``, ``qkv``, ``out``, ``attn_norm`` ...) and forward semantics of
+experiments/symbiosis/backbone.py:11-68 (TokenFormer's feed-forward, experiments/tokenformer/model.py:118-128, is the
+same module), with every dense layer, norm and attention call routed to libtaac_hip.so. They are inference modules:
+dropout probabilities are stored but only the eval-mode behaviour (identity) exists.
+
+``PCVRBackbone`` is the canonical pre-norm stack + pCVR readout (mean-pool over valid tokens -> Linear(D, 1) ->
+sigmoid) executed by a single ``taac_backbone_fwd`` call.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+import torch.nn as nn
+
+from taac_2026_amd import _native
+from taac_2026_amd.accelerators.linear import linear, swiglu_linear
+from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference
+from taac_2026_amd.modeling.normalization import RMSNorm
+from taac_2026_amd.modeling.sequence import scaled_dot_product_attention
+
+
+def _bf16(parameter: torch.Tensor | None) -> torch.Tensor | None:
+    if parameter is None:
+        return None
+    return parameter if parameter.dtype == torch.bfloat16 else parameter.to(torch.bfloat16)
+
+
+def _dense(layer: nn.Linear, x: torch.Tensor, *, residual: torch.Tensor | None = None) -> torch.Tensor:
+    return linear(x, _bf16(layer.weight), _bf16(layer.bias), residual=residual)
+
+
+class SwiGLUFeedForward(nn.Module):
+    """``down(silu(gate) * value)``, ``gate, value = up(x).chunk(2, -1)``; SiLU-gate fused into the up projection."""
+
+    def __init__(self, d_model: int, hidden_mult: int, dropout: float = 0.0, *, gate_first: bool = True) -> None:
+        super().__init__()
+        hidden_dim = int(d_model) * int(hidden_mult)
+        self.up = nn.Linear(d_model, hidden_dim * 2)
+        self.dropout = nn.Dropout(dropout)
+        self.down = nn.Linear(hidden_dim, d_model)
+        self.gate_first = bool(gate_first)
+
+    def forward(self, tokens: torch.Tensor, *, residual: torch.Tensor | None = None) -> torch.Tensor:
+        if self.training and self.dropout.p > 0.0:
+            raise RuntimeError("hip SwiGLUFeedForward is forward-only inference and does not apply dropout")
+        output_dtype = tokens.dtype
+        x = tokens if tokens.dtype == torch.bfloat16 else tokens.to(torch.bfloat16)
+        hidden = swiglu_linear(x, _bf16(self.up.weight), _bf16(self.up.bias), gate_first=self.gate_first)
+        out = _dense(self.down, hidden, residual=_bf16(residual))
+        return out if out.dtype == output_dtype else out.to(output_dtype)
+
+
+class UnifiedSelfAttention(nn.Module):
+    def __init__(self, d_model: int, num_heads: int, dropout: float = 0.0, *, qk_norm: bool = True) -> None:
+        super().__init__()
+        self.num_heads = int(num_heads)
+        self.dropout = float(dropout)
+        self.qkv = nn.Linear(d_model, d_model * 3)
+        self.query_norm = RMSNorm(d_model) if qk_norm else None
+        self.key_norm = RMSNorm(d_model) if qk_norm else None
+        self.out = nn.Linear(d_model, d_model)
+
+    def forward(
+        self,
+        tokens: torch.Tensor,
+        attention_mask: torch.Tensor | None = None,
+        *,
+        key_lengths: torch.Tensor | None = None,
+        zero_padded_queries: bool = False,
+        residual: torch.Tensor | None = None,
+    ) -> torch.Tensor:
+        output_dtype = tokens.dtype
+        x = tokens if tokens.dtype == torch.bfloat16 else tokens.to(torch.bfloat16)
+        query, key, value = _dense(self.qkv, x).chunk(3, dim=-1)
+        if self.query_norm is not None:
+            query = self.query_norm(query)
+            key = self.key_norm(key)
+        attended = scaled_dot_product_attention(
+            query,
+            key,
+            value,
+            num_heads=self.num_heads,
+            attn_mask=attention_mask,
+            dropout_p=self.dropout,
+            training=self.training,
+            key_lengths=key_lengths,
+            zero_padded_queries=zero_padded_queries,
+        )
+        out = _dense(self.out, attended, residual=_bf16(residual))
+        return out if out.dtype == output_dtype else out.to(output_dtype)
+
+
+class UnifiedInteractionBlock(nn.Module):
+    """Pre-RMSNorm self-attention and SwiGLU feed-forward with residuals masked at padded positions."""
+
+    def __init__(self, d_model: int, num_heads: int, hidden_mult: int, dropout: float = 0.0, *, qk_norm: bool = True) -> None:
+        super().__init__()
+        self.attn_norm = RMSNorm(d_model)
+        self.attention = UnifiedSelfAttention(d_model, num_heads, dropout, qk_norm=qk_norm)
+        self.ffn_norm = RMSNorm(d_model)
+        self.ffn = SwiGLUFeedForward(d_model, hidden_mult, dropout)
+
+    def forward(
+        self,
+        tokens: torch.Tensor,
+        padding_mask: torch.Tensor,
+        attention_mask: torch.Tensor | None,
+        *,
+        key_lengths: torch.Tensor | None = None,
+    ) -> tuple[torch.Tensor, torch.Tensor]:
+        keep = (~padding_mask).unsqueeze(-1)
+        attn_update = self.attention(self.attn_norm(tokens), attention_mask, key_lengths=key_lengths)
+        attn_tokens = tokens + attn_update * keep.to(attn_update.dtype)
+        ffn_update = self.ffn(self.ffn_norm(attn_tokens))
+        output = attn_tokens + ffn_update * keep.to(ffn_update.dtype)
+        return output, attn_tokens
+
+
+class _PlainBlock(nn.Module):
+    """Parameter container of one canonical block: RMSNorm -> MHA -> +res -> RMSNorm -> SwiGLU -> +res."""
+
+    def __init__(self, d_model: int, num_heads: int, d_ff: int) -> None:
+        super().__init__()
+        self.attn_norm = RMSNorm(d_model)
+        self.qkv = nn.Linear(d_model, 3 * d_model)
+        self.out = nn.Linear(d_model, d_model)
+        self.ffn_norm = RMSNorm(d_model)
+        self.up = nn.Linear(d_model, 2 * d_ff)
+        self.down = nn.Linear(d_ff, d_model)
+        self.num_heads = num_heads
+
+
+class PCVRBackbone(nn.Module):
+    """n_blocks pre-norm blocks + masked mean-pool -> Linear(D, 1) -> sigmoid, run by one ``taac_backbone_fwd`` call.
+
+    Initialisation: Xavier-uniform weights, zero biases, unit norm weights.
+    ``forward(emb[B, T, D] bf16, key_lengths[B] int32) -> p[B] float32``; ``return_hidden=True`` also returns the
+    final hidden state (rows at or beyond ``key_lengths[b]`` are unspecified).
+    """
+
+    def __init__(self, d_model: int = 256, num_heads: int = 8, d_ff: int = 1024, n_blocks: int = 4, eps: float = 1e-6) -> None:
+        super().__init__()
+        if d_model % num_heads != 0:
+            raise ValueError("d_model must be divisible by num_heads")
+        self.d_model, self.num_heads, self.d_ff, self.eps = int(d_model), int(num_heads), int(d_ff), float(eps)
+        self.blocks = nn.ModuleList(_PlainBlock(d_model, num_heads, d_ff) for _ in range(n_blocks))
+        self.head = nn.Linear(d_model, 1)
+        self.reset_parameters()
+        self._workspace: torch.Tensor | None = None
+
+    def reset_parameters(self) -> None:
+        for module in self.modules():
+            if isinstance(module, nn.Linear):
+                nn.init.xavier_uniform_(module.weight)
+                nn.init.zeros_(module.bias)
+
+    def _get_workspace(self, nbytes: int, device: torch.device) -> torch.Tensor:
+        ws = self._workspace
+        if ws is None or ws.numel() < nbytes or ws.device != device:
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            self._workspace = ws
+        return ws
+
+    def forward(self, emb: torch.Tensor, key_lengths: torch.Tensor, *, return_hidden: bool = False):
+        name = "hip PCVRBackbone"
+        require_cuda_tensors(name, emb, key_lengths)
+        require_inference(name, emb)
+        if emb.ndim != 3 or emb.shape[-1] != self.d_model:
+            raise ValueError(f"PCVRBackbone expects embeddings of shape (batch, tokens, {self.d_model})")
+        if emb.dtype != torch.bfloat16:
+            raise RuntimeError(f"{name} expects bfloat16 embeddings, got {emb.dtype}")
+        if key_lengths.shape != (emb.shape[0],):
+            raise ValueError("key_lengths must have shape (batch,)")
+        emb = emb.contiguous()
+        key_lengths = key_lengths.to(torch.int32).contiguous()
+        batch, tokens, _ = emb.shape
+        library = _native.load_library()
+
+        keep_alive: list[torch.Tensor] = []
+
+        def dev(parameter: torch.Tensor | None) -> int | None:
+            tensor = _bf16(parameter)
+            if tensor is None:
+                return None
+            tensor = tensor.detach().contiguous()
+            keep_alive.append(tensor)
+            return tensor.data_ptr()
+
+        packed = (_native.BlockWeights * len(self.blocks))()
+        for slot, block in zip(packed, self.blocks):
+            slot.attn_norm_weight = dev(block.attn_norm.weight)
+            slot.qkv_weight, slot.qkv_bias = dev(block.qkv.weight), dev(block.qkv.bias)
+            slot.out_weight, slot.out_bias = dev(block.out.weight), dev(block.out.bias)
+            slot.ffn_norm_weight = dev(block.ffn_norm.weight)
+            slot.up_weight, slot.up_bias = dev(block.up.weight), dev(block.up.bias)
+            slot.down_weight, slot.down_bias = dev(block.down.weight), dev(block.down.bias)
+
+        nbytes = library.taac_backbone_workspace_bytes(batch, tokens, self.d_model, self.d_ff)
+        workspace = self._get_workspace(int(nbytes), emb.device)
+        hidden = torch.empty_like(emb) if return_hidden else None
+        probabilities = torch.empty(batch, dtype=torch.float32, device=emb.device)
+        status = library.taac_backbone_fwd(
+            emb.data_ptr(), key_lengths.data_ptr(), packed, len(self.blocks), dev(self.head.weight.reshape(-1)),
+            dev(self.head.bias), batch, tokens, self.d_model, self.num_heads, self.d_ff, ctypes.c_float(self.eps),
+            workspace.data_ptr(), workspace.numel(), _native.ptr(hidden), probabilities.data_ptr(),
+            _native.current_stream(emb.device),
+        )
+        _native.check(status, "backbone_fwd")
+        if return_hidden:
+            return probabilities, hidden
+        return probabilities
+
+
+__all__ = [
+    "PCVRBackbone",
+    "SwiGLUFeedForward",
+    "UnifiedInteractionBlock",
+    "UnifiedSelfAttention",
+]

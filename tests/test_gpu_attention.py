@@ -1,0 +1,152 @@
+"""GPU parity: key-padding-masked attention HIP kernel (through the C ABI) against the CPU oracle."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import reference as oracle
+from taac_2026_amd import workloads
+from taac_2026_amd.api import causal_valid_attention_mask, flash_attention, scaled_dot_product_attention
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = dict(rtol=2e-2, atol=2e-2)
+
+
+def _qkv(batch, heads, tq, tk, dim, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(batch, heads, tq, dim, generator=g).to(dtype)
+    k = torch.randn(batch, heads, tk, dim, generator=g).to(dtype)
+    v = torch.randn(batch, heads, tk, dim, generator=g).to(dtype)
+    return q, k, v
+
+
+def _run(q, k, v, device, **kwargs):
+    with torch.no_grad():
+        return flash_attention(q.to(device), k.to(device), v.to(device), **kwargs).cpu()
+
+
+def test_unmasked_fp16_small_matches_sdpa(device):
+    # shape and tolerance of the reference's GPU test (test_tilelang_ops_cuda.py:61-73)
+    q, k, v = _qkv(2, 4, 32, 32, 16, torch.float16, 0)
+    got = _run(q, k, v, device)
+    expected = F.scaled_dot_product_attention(q.float(), k.float(), v.float())
+    torch.testing.assert_close(got.float(), expected, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dim", [8, 16, 32, 64, 96, 128])
+@pytest.mark.parametrize("tokens", [1, 31, 32, 33, 64, 100, 128, 129, 300])
+def test_key_lengths_bf16(device, dim, tokens):
+    batch, heads = 5, 3
+    q, k, v = _qkv(batch, heads, tokens, tokens, dim, torch.bfloat16, dim * 1000 + tokens)
+    lengths = torch.tensor([tokens, 1, max(1, tokens // 2), 0, max(1, tokens - 1)], dtype=torch.int32)
+    expected = oracle.attention(q, k, v, lengths)
+    got = _run(q, k, v, device, key_lengths=lengths.to(device))
+    torch.testing.assert_close(got.float(), expected.float(), **BF16_TOL)
+    expected_zero = oracle.attention(q, k, v, lengths, zero_padded_queries=True)
+    got_zero = _run(q, k, v, device, key_lengths=lengths.to(device), zero_padded_queries=True)
+    torch.testing.assert_close(got_zero.float(), expected_zero.float(), **BF16_TOL)
+    # padded query rows are exactly zero
+    for b in range(batch):
+        assert got_zero[b, :, int(lengths[b]):].abs().max().item() == 0.0 if lengths[b] < tokens else True
+
+
+def test_cross_attention_lengths_differ(device):
+    q, k, v = _qkv(2, 3, 5, 7, 8, torch.bfloat16, 11)
+    got = _run(q, k, v, device)
+    torch.testing.assert_close(got.float(), oracle.attention(q, k, v).float(), **BF16_TOL)
+    q, k, v = _qkv(3, 2, 150, 77, 64, torch.bfloat16, 12)
+    lengths = torch.tensor([77, 40, 3], dtype=torch.int32)
+    got = _run(q, k, v, device, key_lengths=lengths.to(device))
+    torch.testing.assert_close(got.float(), oracle.attention(q, k, v, lengths).float(), **BF16_TOL)
+
+
+def test_bool_mask_forms(device):
+    q, k, v = _qkv(2, 3, 4, 6, 8, torch.bfloat16, 5)
+    key_valid = torch.tensor([[True, True, True, True, False, False], [True, True, False, False, False, False]])
+    mask4 = key_valid[:, None, None, :].expand(2, 3, 4, 6)
+    expected = oracle.sdpa(q.float(), k.float(), v.float(), attn_mask=mask4)
+    for mask in (mask4, key_valid, key_valid[:, None, None, :]):
+        got = _run(q, k, v, device, attn_mask=mask.to(device))
+        torch.testing.assert_close(got.float(), expected, **BF16_TOL)
+
+
+@pytest.mark.parametrize("tokens,dim", [(5, 8), (64, 32), (130, 64), (257, 32)])
+def test_causal_valid_mask(device, tokens, dim):
+    batch, heads = 3, 2
+    q, k, v = _qkv(batch, heads, tokens, tokens, dim, torch.bfloat16, tokens)
+    lengths = torch.tensor([tokens, max(1, tokens // 3), 1])
+    padding = oracle.make_padding_mask(lengths, tokens)
+    mask = oracle.causal_valid_attention_mask(padding, heads)
+    expected = oracle.sdpa(q.float(), k.float(), v.float(), attn_mask=mask)
+    got = _run(q, k, v, device, attn_mask=causal_valid_attention_mask(padding.to(device), heads))
+    torch.testing.assert_close(got.float(), expected, **BF16_TOL)
+    # plain causal without lengths
+    got = _run(q, k, v, device, is_causal=True)
+    torch.testing.assert_close(got.float(), oracle.attention(q, k, v, is_causal=True).float(), **BF16_TOL)
+
+
+def test_float32_callers_are_computed_in_bf16(device):
+    q, k, v = _qkv(2, 4, 32, 32, 16, torch.float32, 3)
+    got = _run(q, k, v, device)
+    assert got.dtype == torch.float32
+    torch.testing.assert_close(got, F.scaled_dot_product_attention(q, k, v), rtol=1.5e-2, atol=1.5e-2)
+
+
+def test_projection_layout_is_read_in_place(device):
+    """(B, T, 3D) fused projection -> strided (B, H, T, dh) views, no copies, result (B, T, D)."""
+    batch, tokens, heads, dh = 3, 70, 8, 32
+    g = torch.Generator().manual_seed(9)
+    qkv = torch.randn(batch, tokens, 3 * heads * dh, generator=g).to(torch.bfloat16)
+    lengths = torch.tensor([70, 33, 1], dtype=torch.int32)
+    q, k, v = qkv.chunk(3, dim=-1)
+    expected = oracle.scaled_dot_product_attention(q, k, v, num_heads=heads, key_lengths=lengths, zero_padded_queries=True)
+    dq, dk, dv = qkv.to(device).chunk(3, dim=-1)
+    with torch.no_grad():
+        got = scaled_dot_product_attention(dq, dk, dv, num_heads=heads, attn_mask=None, dropout_p=0.0, training=False,
+                                           key_lengths=lengths.to(device), zero_padded_queries=True)
+    assert got.shape == (batch, tokens, heads * dh)
+    torch.testing.assert_close(got.cpu().float(), expected.float(), **BF16_TOL)
+
+
+def test_special_cases(device):
+    # identical keys -> uniform softmax -> mean of the valid values; len == 1 -> v[0]
+    batch, heads, tokens, dim = 2, 2, 96, 64
+    q, k, v = _qkv(batch, heads, tokens, tokens, dim, torch.bfloat16, 21)
+    k = k[:, :, :1].expand(-1, -1, tokens, -1).contiguous()
+    lengths = torch.tensor([50, 1], dtype=torch.int32)
+    got = _run(q, k, v, device, key_lengths=lengths.to(device)).float()
+    torch.testing.assert_close(got[0], v[0, :, :50].float().mean(dim=1, keepdim=True).expand(-1, tokens, -1), **BF16_TOL)
+    torch.testing.assert_close(got[1], v[1, :, :1].float().expand(-1, tokens, -1), **BF16_TOL)
+
+
+def test_config3_full_size(device):
+    """Config 3 (B=2048, H=4, T=256, d=64, lengths ~ U{16..256}) at full size: a slice of samples against the oracle,
+    padded rows exactly zero, everything finite."""
+    q, k, v, lengths = workloads.attention_inputs()
+    with torch.no_grad():
+        got = flash_attention(q.to(device), k.to(device), v.to(device), key_lengths=lengths.to(device),
+                              zero_padded_queries=True)
+        assert torch.isfinite(got).all()
+        positions = torch.arange(256, device=device)[None, :] >= lengths.to(device)[:, None]
+        assert got.float().abs().amax(dim=(1, 3))[positions].max().item() == 0.0
+    got = got.cpu()
+    pick = torch.arange(0, 2048, 53)
+    expected = oracle.attention(q[pick], k[pick], v[pick], lengths[pick], zero_padded_queries=True)
+    torch.testing.assert_close(got[pick].float(), expected.float(), **BF16_TOL)
+
+
+def test_errors(device):
+    q, k, v = _qkv(2, 3, 5, 5, 8, torch.bfloat16, 1)
+    with pytest.raises(ValueError, match="matching head dimensions"):
+        flash_attention(q.to(device), k.to(device), v[..., :4].to(device))
+    bad = torch.tensor([[True, False, True, False, False]]).expand(2, 5)[:, None, None, :].expand(2, 3, 5, 5)
+    with pytest.raises(RuntimeError, match="prefix-valid"):
+        flash_attention(q.to(device), k.to(device), v.to(device), attn_mask=bad.to(device))
+    with pytest.raises(RuntimeError, match="requires CUDA tensors"):
+        flash_attention(q, k, v)
+    q7 = torch.randn(1, 1, 4, 12, dtype=torch.bfloat16, device=device)
+    with pytest.raises(RuntimeError, match="head_dim"):
+        flash_attention(q7, q7, q7)

@@ -1,0 +1,140 @@
+"""GPU parity: dense-layer HIP kernels (bf16 and FP8 MFMA, fused epilogues) against the CPU oracle."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import reference as oracle
+from taac_2026_amd.api import (
+    SwiGLUFeedForward,
+    amax,
+    linear,
+    linear_fp8,
+    quantize_fp8,
+    swiglu_ffn,
+    swiglu_linear,
+)
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = dict(rtol=2e-2, atol=2e-2)
+
+
+def _draw(m, n, k, seed, *, x_scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    x = (x_scale * torch.randn(m, k, generator=g)).to(torch.bfloat16)
+    bound = (6.0 / (n + k)) ** 0.5
+    w = ((torch.rand(n, k, generator=g) * 2 - 1) * bound).to(torch.bfloat16)
+    b = (0.1 * torch.randn(n, generator=g)).to(torch.bfloat16)
+    return x, w, b
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 8, 8), (127, 768, 256), (128, 256, 256), (300, 256, 1024), (513, 264, 72),
+                                   (1000, 768, 256), (64, 2048, 256)])
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_linear_matches_oracle(device, m, n, k, use_bias):
+    x, w, b = _draw(m, n, k, seed=m + n + k)
+    bias = b if use_bias else None
+    expected = F.linear(x.float(), w.float(), None if bias is None else bias.float())
+    with torch.no_grad():
+        got = linear(x.to(device), w.to(device), None if bias is None else bias.to(device))
+    assert got.dtype == torch.bfloat16 and got.shape == (m, n)
+    torch.testing.assert_close(got.cpu().float(), expected, **BF16_TOL)
+    # the reference's bf16 torch path is inside the same tolerance
+    torch.testing.assert_close(got.cpu().float(), F.linear(x, w, bias).float(), **BF16_TOL)
+
+
+def test_linear_residual_and_batch_dims(device):
+    x, w, b = _draw(6 * 50, 256, 256, seed=4)
+    x3 = x.view(6, 50, 256)
+    g = torch.Generator().manual_seed(5)
+    res = torch.randn(6, 50, 256, generator=g).to(torch.bfloat16)
+    expected = res.float() + F.linear(x3.float(), w.float(), b.float())
+    with torch.no_grad():
+        got = linear(x3.to(device), w.to(device), b.to(device), residual=res.to(device))
+    assert got.shape == (6, 50, 256)
+    torch.testing.assert_close(got.cpu().float(), expected, **BF16_TOL)
+
+
+@pytest.mark.parametrize("m,f,k", [(1, 8, 8), (200, 1024, 256), (129, 72, 64), (512, 64, 256)])
+@pytest.mark.parametrize("gate_first", [True, False])
+def test_swiglu_linear(device, m, f, k, gate_first):
+    x, w, b = _draw(m, 2 * f, k, seed=m + f)
+    expected = oracle.swiglu_hidden(x.float(), w.float(), b.float(), gate_first=gate_first)
+    with torch.no_grad():
+        got = swiglu_linear(x.to(device), w.to(device), b.to(device), gate_first=gate_first)
+    assert got.shape == (m, f)
+    torch.testing.assert_close(got.cpu().float(), expected, **BF16_TOL)
+
+
+def test_swiglu_ffn_module_matches_reference_formula(device):
+    torch.manual_seed(0)
+    module = SwiGLUFeedForward(256, 4, 0.0).eval()
+    x = (torch.randn(3, 40, 256)).to(torch.bfloat16)
+    weights = {name: p.detach().to(torch.bfloat16) for name, p in module.named_parameters()}
+    expected = oracle.swiglu_ffn(x, weights["up.weight"], weights["up.bias"], weights["down.weight"], weights["down.bias"])
+    module = module.to(device)
+    with torch.no_grad():
+        got = module(x.to(device))
+        got_fn = swiglu_ffn(x.to(device), weights["up.weight"].to(device), weights["up.bias"].to(device),
+                            weights["down.weight"].to(device), weights["down.bias"].to(device))
+    torch.testing.assert_close(got.cpu().float(), expected.float(), **BF16_TOL)
+    torch.testing.assert_close(got_fn.cpu().float(), expected.float(), **BF16_TOL)
+
+
+# ---- FP8 ---------------------------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("n", [1, 7, 8, 1000, 65536 + 3])
+def test_amax_and_quantize_fp8(device, dtype, n):
+    g = torch.Generator().manual_seed(n)
+    x = (3.0 * torch.randn(n, generator=g)).to(dtype)
+    with torch.no_grad():
+        a = amax(x.to(device))
+        q, a2 = quantize_fp8(x.to(device))
+    assert a.item() == x.float().abs().max().item() == a2.item()
+    expected_q, _ = oracle.fp8_quantize(x)
+    assert torch.equal(q.cpu().view(torch.uint8), expected_q.view(torch.uint8))
+
+
+def _rel_err(got, expected):
+    return ((got.float() - expected.float()).abs().max() / expected.float().abs().max()).item()
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 768, 256), (130, 256, 256), (77, 256, 1024), (64, 64, 16)])
+def test_linear_fp8_matches_emulation(device, m, n, k):
+    x, w, b = _draw(m, n, k, seed=m * 3 + n)
+    expected = oracle.linear_fp8(x, w, b)
+    with torch.no_grad():
+        wq, wa = quantize_fp8(w.to(device))
+        xa = amax(x.to(device))
+        got = linear_fp8(x.to(device), wq, xa, wa, b.to(device))
+        # pre-quantised activations take the same path
+        xq, _ = quantize_fp8(x.to(device), xa)
+        got_q = linear_fp8(xq, wq, xa, wa, b.to(device))
+    assert _rel_err(got.cpu(), expected) <= 5e-2
+    assert _rel_err(got_q.cpu(), expected) <= 5e-2
+    torch.testing.assert_close(got.cpu().float(), expected.float(), rtol=0, atol=5e-2 * expected.float().abs().max().item())
+
+
+def test_linear_fp8_epilogues(device):
+    m, f, k = 200, 1024, 256
+    x, w, b = _draw(m, 2 * f, k, seed=77)
+    expected = oracle.linear_fp8(x, w, b, swiglu=True)
+    with torch.no_grad():
+        wq, wa = quantize_fp8(w.to(device))
+        xa = amax(x.to(device))
+        got = linear_fp8(x.to(device), wq, xa, wa, b.to(device), swiglu=True)
+    assert got.shape == (m, f)
+    assert _rel_err(got.cpu(), expected) <= 5e-2
+    x2, w2, b2 = _draw(m, 256, 1024, seed=78)
+    res = torch.randn(m, 256, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    expected = oracle.linear_fp8(x2, w2, b2, residual=res)
+    with torch.no_grad():
+        wq, wa = quantize_fp8(w2.to(device))
+        xa = amax(x2.to(device))
+        got = linear_fp8(x2.to(device), wq, xa, wa, b2.to(device), residual=res.to(device))
+    assert _rel_err(got.cpu(), expected) <= 5e-2
