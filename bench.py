@@ -1,0 +1,282 @@
+#!/usr/bin/env python3
+"""Benchmark of the unified pCVR token backbone's kernel path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one 4-block backbone forward (one ``taac_backbone_fwd`` call) over one batch of synthetic input at the
+headline configuration: B=1024, T=32+480, d_model=256, 8 heads x 32, SwiGLU d_ff=1024, bf16, inputs and weights
+resident in HBM. One JSON line is printed: whole-job throughput in pCVR samples/s, the roofline position of the
+kernel that takes the largest share of the step (duration measured here with HIP events on the launch stream), the
+stand-alone operator figures the metric also names (attention TFLOP/s, norm HBM GB/s), and the reference's torch
+formulas timed on the host CPU over a bounded sample of the same workload.
+
+No time is reported unless the accuracy gate passed in the same process (the rule of the reference's operator
+benchmark, src/taac2026/application/benchmarking/pcvr_tilelang_ops_benchmark.py:201-215).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+REPO_ROOT = Path(__file__).resolve().parent
+if str(REPO_ROOT) not in sys.path:
+    sys.path.insert(0, str(REPO_ROOT))
+
+import torch  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
+
+
+def _event_ms(fn, iters: int, warmup: int) -> float:
+    """Average duration of ``fn`` in ms, HIP events on the current stream (the stream the kernels are launched on)."""
+    for _ in range(warmup):
+        fn()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def _accuracy_gate(model, inputs, device) -> dict:
+    """Probabilities of a slice of the batch against the CPU oracle (2e-2 absolute)."""
+    from oracle import reference as oracle
+
+    pick = torch.tensor([0, 341, 682, 1023]) % inputs.emb.shape[0]
+    with torch.no_grad():
+        p = model(inputs.emb.to(device), inputs.key_lengths.to(device)).cpu()
+    expected = oracle.backbone(inputs.emb[pick], inputs.key_lengths[pick], inputs.blocks, inputs.head_weight,
+                               inputs.head_bias, num_heads=inputs.num_heads)
+    err = (p[pick] - expected).abs().max().item()
+    if not (torch.isfinite(p).all() and err <= 2e-2):
+        raise SystemExit(f"accuracy gate failed: max |p - oracle| = {err}")
+    return {"checked_samples": int(pick.numel()), "max_abs_err": err, "atol": 2e-2}
+
+
+def _kernel_breakdown(inputs, device, iters: int) -> dict:
+    """Stand-alone timing of each kernel of one block at the step's shapes (HIP events on the launch stream)."""
+    from taac_2026_amd.api import linear, rms_norm, scaled_dot_product_attention, swiglu_linear
+
+    B, T, D = inputs.emb.shape
+    M, F, H = B * T, inputs.d_ff, inputs.num_heads
+    w = {k: v.to(device) for k, v in inputs.blocks[0].items()}
+    x = inputs.emb.to(device)
+    lengths = inputs.key_lengths.to(device)
+    out: dict[str, dict] = {}
+    with torch.no_grad():
+        h = rms_norm(x, w["attn_norm.weight"])
+        qkv = linear(h, w["qkv.weight"], w["qkv.bias"])
+        q, k, v = qkv.chunk(3, dim=-1)
+        attn = lambda: scaled_dot_product_attention(q, k, v, num_heads=H, attn_mask=None, dropout_p=0.0,  # noqa: E731
+                                                    training=False, key_lengths=lengths, zero_padded_queries=True)
+        a = attn()
+        g = swiglu_linear(h, w["up.weight"], w["up.bias"])
+        valid_tokens = float(lengths.sum().item())
+        sum_sq = float((lengths.double() ** 2).sum().item())
+        dh = D // H
+        cases = {
+            "rmsnorm": (lambda: rms_norm(x, w["attn_norm.weight"]), 0.0, 2.0 * M * D * 2 + 2 * D),
+            "linear_qkv": (lambda: linear(h, w["qkv.weight"], w["qkv.bias"]), 2.0 * M * 3 * D * D,
+                           2.0 * (M * D + 3 * D * D + M * 3 * D)),
+            # useful work only: visible (query, key) pairs; Q/K/V valid rows read, O written in full
+            "attention": (attn, 4.0 * H * dh * sum_sq, 2.0 * (3 * D * valid_tokens + M * D)),
+            "linear_out_residual": (lambda: linear(a, w["out.weight"], w["out.bias"], residual=x), 2.0 * M * D * D,
+                                    2.0 * (3 * M * D + D * D)),
+            "linear_up_swiglu": (lambda: swiglu_linear(h, w["up.weight"], w["up.bias"]), 2.0 * M * 2 * F * D,
+                                 2.0 * (M * D + 2 * F * D + M * F)),
+            "linear_down_residual": (lambda: linear(g, w["down.weight"], w["down.bias"], residual=x),
+                                     2.0 * M * D * F, 2.0 * (M * F + D * F + 2 * M * D)),
+        }
+        for name, (fn, flops, nbytes) in cases.items():
+            ms = _event_ms(fn, iters, 3)
+            out[name] = {
+                "ms": ms,
+                "algorithmic_flops": flops,
+                "algorithmic_bytes": nbytes,
+                "tflops": flops / ms / 1e9,
+                "gbs": nbytes / ms / 1e6,
+                "frac_mfma": flops / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS,
+                "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS,
+            }
+    return out
+
+
+def _operator_figures(device, iters: int) -> dict:
+    """Stand-alone operators at configurations 2 and 3: norm HBM GB/s and masked-attention TFLOP/s."""
+    from oracle import reference as oracle
+    from taac_2026_amd import workloads
+    from taac_2026_amd.api import flash_attention, layer_norm, rms_norm
+
+    figures: dict[str, dict] = {}
+    with torch.no_grad():
+        x, gamma, beta = workloads.norm_bf16_inputs()
+        xd, gd, bd = x.to(device), gamma.to(device), beta.to(device)
+        got = rms_norm(xd[:16], gd).cpu().float()
+        torch.testing.assert_close(got, oracle.rms_norm_fp32(x[:16], gamma).float(), rtol=2e-2, atol=2e-2)
+        got = layer_norm(xd[:16], gd, bd).cpu().float()
+        torch.testing.assert_close(got, oracle.layer_norm_fp32(x[:16], gamma, beta).float(), rtol=2e-2, atol=2e-2)
+        nbytes = 2.0 * x.numel() * 2 + 2 * 256
+        ms = _event_ms(lambda: rms_norm(xd, gd), iters, 5)
+        figures["rmsnorm_bf16_1048576x256"] = {"ms": ms, "gbs": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS}
+        ms = _event_ms(lambda: layer_norm(xd, gd, bd), iters, 5)
+        figures["layernorm_bf16_1048576x256"] = {"ms": ms, "gbs": (nbytes + 512) / ms / 1e6,
+                                                 "frac_hbm": (nbytes + 512) / ms / 1e6 / HBM_PEAK_GBS}
+        del xd
+
+        q, k, v, lengths = workloads.attention_inputs()
+        qd, kd, vd, ld = q.to(device), k.to(device), v.to(device), lengths.to(device)
+        pick = torch.arange(0, q.shape[0], 257)
+        got = flash_attention(qd, kd, vd, key_lengths=ld, zero_padded_queries=True).cpu()[pick].float()
+        expected = oracle.attention(q[pick], k[pick], v[pick], lengths[pick], zero_padded_queries=True).float()
+        torch.testing.assert_close(got, expected, rtol=2e-2, atol=2e-2)
+        B, H, T, d = q.shape
+        sum_sq = float((lengths.double() ** 2).sum().item())
+        useful = 4.0 * H * d * sum_sq
+        nbytes = 3.0 * H * d * 2 * float(lengths.sum().item()) + B * H * T * d * 2
+        ms = _event_ms(lambda: flash_attention(qd, kd, vd, key_lengths=ld, zero_padded_queries=True), iters, 5)
+        figures["attention_bf16_B2048_H4_T256_d64"] = {
+            "ms": ms,
+            "useful_tflops": useful / ms / 1e9,
+            "dense_equivalent_tflops": 4.0 * B * H * T * T * d / ms / 1e9,
+            "gbs": nbytes / ms / 1e6,
+            "frac_mfma": useful / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS,
+            "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS,
+        }
+    return figures
+
+
+def _cpu_baseline(inputs, budget_s: float = 20.0) -> dict:
+    """The oracle's backbone forward (the reference's torch formulas) on the host cores, on a bounded sample."""
+    from oracle import reference as oracle
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    results = {}
+    for label, cast in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
+        blocks = [{k: v.to(cast) for k, v in w.items()} for w in inputs.blocks]
+        hw, hb = inputs.head_weight.to(cast), inputs.head_bias.to(cast)
+
+        def run(n, blocks=blocks, hw=hw, hb=hb, cast=cast):
+            with torch.no_grad():
+                t0 = time.perf_counter()
+                oracle.backbone(inputs.emb[:n].to(cast), inputs.key_lengths[:n], blocks, hw, hb, num_heads=inputs.num_heads)
+                return time.perf_counter() - t0
+
+        run(2)  # warm-up
+        probe = run(4)
+        n = int(max(4, min(inputs.emb.shape[0], (budget_s / 2) / max(probe / 4, 1e-6))))
+        n = min(n, 256)
+        elapsed = run(n)
+        results[label] = {"samples": n, "seconds": elapsed, "samples_per_s": n / elapsed}
+    best = max(results, key=lambda name: results[name]["samples_per_s"])
+    return {
+        "value": results[best]["samples_per_s"],
+        "unit": "samples/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"first {results[best]['samples']} samples of the same batch, torch CPU {best}, "
+                  f"{torch.get_num_threads()} threads, one forward",
+        "detail": results,
+    }
+
+
+def main() -> None:
+    parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=5)
+    parser.add_argument("--batch", type=int, default=1024, help="samples per step (headline: 1024)")
+    parser.add_argument("--skip-cpu-baseline", action="store_true")
+    parser.add_argument("--skip-operators", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs on ONE GPU (the path has no cross-GPU stage); use --gpus 1")
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+
+    from taac_2026_amd import workloads
+    from taac_2026_amd.api import PCVRBackbone
+
+    device = torch.device("cuda:0")
+    inputs = workloads.backbone_inputs(batch=args.batch)
+    B, T, D = inputs.emb.shape
+    model = PCVRBackbone(d_model=D, num_heads=inputs.num_heads, d_ff=inputs.d_ff, n_blocks=len(inputs.blocks))
+    workloads.load_backbone_state(model, inputs)
+    model = model.to(device=device, dtype=torch.bfloat16).eval()
+
+    accuracy = _accuracy_gate(model, inputs, device)
+
+    emb = inputs.emb.to(device)
+    lengths = inputs.key_lengths.to(device)
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            model(emb, lengths)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            model(emb, lengths)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = B / (elapsed / args.steps)
+
+    kernels = _kernel_breakdown(inputs, device, iters=10)
+    dominant = max(kernels, key=lambda name: kernels[name]["ms"])
+    dom = kernels[dominant]
+    bound = "mfma" if dom["frac_mfma"] >= dom["frac_hbm"] else "hbm"
+    roofline = {
+        "kernel": dominant,
+        "bound": bound,
+        "achieved": dom["tflops"] if bound == "mfma" else dom["gbs"],
+        "peak": MFMA_BF16_PEAK_TFLOPS if bound == "mfma" else HBM_PEAK_GBS,
+        "unit": "TFLOP/s" if bound == "mfma" else "GB/s",
+        "frac": dom["frac_mfma"] if bound == "mfma" else dom["frac_hbm"],
+        "traffic": None,
+        "launch_ms": dom["ms"],
+    }
+
+    dense_flops = len(inputs.blocks) * (2.0 * B * T * (3 * D * D + D * D + 3 * D * inputs.d_ff) + 4.0 * B * T * T * D)
+    line = {
+        "metric": "pCVR samples/s (4-block fwd, B=1024,T=512); attn TFLOP/s; norm HBM GB/s",
+        "value": value,
+        "unit": "samples/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"4-block unified token backbone forward, B={B}, T=32+{T - 32}, d_model={D}, "
+                        f"{inputs.num_heads} heads x {D // inputs.num_heads}, SwiGLU d_ff={inputs.d_ff}, "
+                        "valid length ~ U{64..512}, masked mean-pool -> Linear -> sigmoid",
+            "batch": B,
+            "tokens": T,
+        },
+        "dense_equivalent_tflops": dense_flops / (elapsed / args.steps) / 1e12,
+        "roofline": roofline,
+        "accuracy": accuracy,
+        "kernels": kernels,
+    }
+    if not args.skip_operators:
+        line["operators"] = _operator_figures(device, iters=20)
+    if not args.skip_cpu_baseline:
+        line["cpu_baseline"] = _cpu_baseline(inputs)
+        line["gpu_over_cpu"] = value / line["cpu_baseline"]["value"]
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
