@@ -1,0 +1,289 @@
+"""Pins the CPU oracle (oracle/reference.py) independently of its own formulas: golden vectors the reference's tests
+hold, library routines, float64 loop brute force, closed-form special cases and invariants."""
+
+from __future__ import annotations
+
+import json
+import math
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import reference as oracle
+
+GOLDEN = Path(__file__).resolve().parent / "golden"
+MASKS = json.loads((GOLDEN / "mask_vectors.json").read_text())
+
+
+# ---- normalisation ---------------------------------------------------------------------------------------------------
+
+
+def _rms_loop(x: np.ndarray, w: np.ndarray, eps: float) -> np.ndarray:
+    out = np.zeros_like(x, dtype=np.float64)
+    for r in range(x.shape[0]):
+        acc = 0.0
+        for c in range(x.shape[1]):
+            acc += float(x[r, c]) ** 2
+        s = 1.0 / math.sqrt(acc / x.shape[1] + eps)
+        for c in range(x.shape[1]):
+            out[r, c] = float(x[r, c]) * s * float(w[c])
+    return out
+
+
+def _ln_loop(x: np.ndarray, w: np.ndarray, b: np.ndarray, eps: float) -> np.ndarray:
+    out = np.zeros_like(x, dtype=np.float64)
+    for r in range(x.shape[0]):
+        mean = sum(float(v) for v in x[r]) / x.shape[1]
+        var = sum((float(v) - mean) ** 2 for v in x[r]) / x.shape[1]
+        for c in range(x.shape[1]):
+            out[r, c] = (float(x[r, c]) - mean) / math.sqrt(var + eps) * float(w[c]) + float(b[c])
+    return out
+
+
+def test_rms_norm_brute_force_and_reference_test_formula():
+    torch.manual_seed(0)
+    x = torch.randn(8, 4, 16)
+    w = torch.randn(16)
+    got = oracle.rms_norm(x, w)
+    # the closed form as the reference's own unit test writes it (test_tilelang_ops.py:533-540)
+    torch.testing.assert_close(got, x * torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + 1e-6) * w)
+    loop = _rms_loop(x.reshape(-1, 16).numpy(), w.numpy(), 1e-6)
+    np.testing.assert_allclose(got.reshape(-1, 16).numpy(), loop, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(oracle.rms_norm_fp32(x, w).reshape(-1, 16).numpy(), loop, rtol=1e-5, atol=1e-6)
+
+
+def test_rms_norm_invariants():
+    torch.manual_seed(1)
+    x = torch.randn(32, 64, dtype=torch.float64)
+    w = torch.rand(64, dtype=torch.float64) + 0.5
+    eps = 1e-6
+    y = oracle.rms_norm(x, w, eps)
+    # scale equivariance: rms(c x; c^2 eps) == rms(x; eps); sign flip
+    torch.testing.assert_close(oracle.rms_norm(8.0 * x, w, eps * 64.0), y)
+    torch.testing.assert_close(oracle.rms_norm(-x, w, eps), -y)
+    # sum((y/w)^2)/D = 1 - eps * s^2 with s = rsqrt(mean(x^2) + eps)
+    s2 = 1.0 / (x.pow(2).mean(dim=-1) + eps)
+    torch.testing.assert_close((y / w).pow(2).mean(dim=-1), 1.0 - eps * s2)
+    # rows are independent
+    x2 = x.clone()
+    x2[5] = 100.0
+    y2 = oracle.rms_norm(x2, w, eps)
+    assert torch.equal(torch.cat([y2[:5], y2[6:]]), torch.cat([y[:5], y[6:]]))
+
+
+def test_layer_norm_library_brute_force_and_invariants():
+    torch.manual_seed(2)
+    x = torch.randn(8, 4, 16) * 3 + 2
+    w, b = torch.randn(16), torch.randn(16)
+    got = oracle.layer_norm(x, w, b)
+    torch.testing.assert_close(got, F.layer_norm(x, (16,), w, b, 1e-5))
+    loop = _ln_loop(x.reshape(-1, 16).numpy(), w.numpy(), b.numpy(), 1e-5)
+    np.testing.assert_allclose(got.reshape(-1, 16).numpy(), loop, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(oracle.layer_norm_fp32(x, w, b).reshape(-1, 16).numpy(), loop, rtol=1e-4, atol=1e-5)
+    unit = oracle.layer_norm(x.double(), torch.ones(16, dtype=torch.float64), torch.zeros(16, dtype=torch.float64))
+    torch.testing.assert_close(unit.mean(dim=-1), torch.zeros(8, 4, dtype=torch.float64), atol=1e-12, rtol=0)
+    var = x.double().var(dim=-1, unbiased=False)
+    torch.testing.assert_close(unit.var(dim=-1, unbiased=False), var / (var + 1e-5))
+    torch.testing.assert_close(oracle.layer_norm(x.double() + 7.0, w.double(), b.double()),
+                               oracle.layer_norm(x.double(), w.double(), b.double()))
+
+
+def test_bf16_variants_stay_close_to_fp32_statistics():
+    torch.manual_seed(3)
+    x = torch.randn(64, 256).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(256)).to(torch.bfloat16)
+    torch.testing.assert_close(oracle.rms_norm(x, w).float(), oracle.rms_norm_fp32(x, w).float(), rtol=2e-2, atol=2e-2)
+
+
+# ---- masks and pooling -----------------------------------------------------------------------------------------------
+
+
+def test_mask_helpers_match_reference_known_answers():
+    case = MASKS["make_padding_mask"]
+    assert oracle.make_padding_mask(torch.tensor(case["lengths"]), case["max_len"]).tolist() == case["expected"]
+    case = MASKS["safe_key_padding_mask"]
+    assert oracle.safe_key_padding_mask(torch.tensor(case["mask"])).tolist() == case["expected"]
+
+
+def test_masked_mean_brute_force_and_empty_rows():
+    torch.manual_seed(4)
+    tokens = torch.randn(3, 5, 4, dtype=torch.float64)
+    padding = torch.tensor([[False, False, True, True, True], [False] * 5, [True] * 5])
+    got = oracle.masked_mean(tokens, padding)
+    for b in range(3):
+        keep = [t for t in range(5) if not padding[b, t]]
+        expected = sum(tokens[b, t] for t in keep) / max(1, len(keep)) if keep else torch.zeros(4, dtype=torch.float64)
+        torch.testing.assert_close(got[b], expected)
+    torch.testing.assert_close(oracle.masked_mean(tokens, None), tokens.mean(dim=1))
+
+
+def test_causal_valid_mask_known_answer():
+    case = MASKS["plan_causal_valid_mask"]
+    padding = torch.tensor(case["padding_mask"])
+    mask = oracle.causal_valid_attention_mask(padding, 3)
+    assert mask.shape == (2, 3, 5, 5)
+    # sample 0: length 3 -> causal over keys 0..2; padded queries 3, 4 see only themselves
+    assert mask[0, 0].tolist() == [
+        [True, False, False, False, False],
+        [True, True, False, False, False],
+        [True, True, True, False, False],
+        [False, False, False, True, False],
+        [False, False, False, False, True],
+    ]
+
+
+# ---- attention -------------------------------------------------------------------------------------------------------
+
+
+def test_attention_golden_vector():
+    data = json.loads((GOLDEN / "attention_small.json").read_text())
+    q, k, v = (torch.tensor(data[name], dtype=torch.float64) for name in ("q", "k", "v"))
+    lengths = torch.tensor(data["key_lengths"], dtype=torch.int32)
+    expected = {name: torch.tensor(value, dtype=torch.float64) for name, value in data["expected"].items()}
+    torch.testing.assert_close(oracle.attention(q, k, v, lengths).double(), expected["plain"], rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(oracle.attention(q, k, v, lengths, zero_padded_queries=True).double(),
+                               expected["zero_padded"], rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(oracle.attention(q, k, v, lengths, is_causal=True).double(), expected["causal"],
+                               rtol=1e-5, atol=1e-6)
+
+
+def test_attention_reduces_to_library_sdpa():
+    torch.manual_seed(5)
+    q, k, v = torch.randn(2, 3, 5, 8), torch.randn(2, 3, 7, 8), torch.randn(2, 3, 7, 8)
+    torch.testing.assert_close(oracle.attention(q, k, v), F.scaled_dot_product_attention(q, k, v))
+    torch.testing.assert_close(oracle.sdpa(q, k, v), F.scaled_dot_product_attention(q, k, v))
+    lengths = torch.tensor([7, 4], dtype=torch.int32)
+    mask = oracle.key_length_mask(lengths, 3, 5, 7)
+    torch.testing.assert_close(oracle.attention(q, k, v, lengths), F.scaled_dot_product_attention(q, k, v, attn_mask=mask))
+    qs, ks, vs = torch.randn(2, 2, 6, 8), torch.randn(2, 2, 6, 8), torch.randn(2, 2, 6, 8)
+    torch.testing.assert_close(oracle.attention(qs, ks, vs, is_causal=True),
+                               F.scaled_dot_product_attention(qs, ks, vs, is_causal=True))
+
+
+def test_attention_special_cases():
+    torch.manual_seed(6)
+    q, k, v = torch.randn(2, 2, 9, 8), torch.randn(2, 2, 9, 8), torch.randn(2, 2, 9, 8)
+    # a single visible key returns its value row for every query
+    out = oracle.attention(q, k, v, torch.tensor([1, 1], dtype=torch.int32))
+    torch.testing.assert_close(out, v[:, :, :1].expand_as(out))
+    # identical keys -> uniform weights -> mean of the visible values
+    same = k[:, :, :1].expand(-1, -1, 9, -1)
+    out = oracle.attention(q, same, v, torch.tensor([9, 4], dtype=torch.int32))
+    torch.testing.assert_close(out[0], v[0].mean(dim=1, keepdim=True).expand_as(out[0]))
+    torch.testing.assert_close(out[1], v[1, :, :4].mean(dim=1, keepdim=True).expand_as(out[1]))
+    # no visible key -> zeros, never NaN; zero_padded_queries zeroes rows at or beyond the length
+    out = oracle.attention(q, k, v, torch.tensor([0, 5], dtype=torch.int32), zero_padded_queries=True)
+    assert torch.equal(out[0], torch.zeros_like(out[0])) and torch.isfinite(out).all()
+    assert torch.equal(out[1, :, 5:], torch.zeros_like(out[1, :, 5:])) and out[1, :, :5].abs().min() > 0
+
+
+# ---- dense layers ----------------------------------------------------------------------------------------------------
+
+
+def test_swiglu_ffn_brute_force_and_chunk_order():
+    torch.manual_seed(7)
+    d, f, m = 4, 6, 3
+    x = torch.randn(m, d, dtype=torch.float64)
+    wu, bu = torch.randn(2 * f, d, dtype=torch.float64), torch.randn(2 * f, dtype=torch.float64)
+    wd, bd = torch.randn(d, f, dtype=torch.float64), torch.randn(d, dtype=torch.float64)
+    for gate_first in (True, False):
+        expected = torch.zeros(m, d, dtype=torch.float64)
+        for r in range(m):
+            hidden = []
+            for j in range(f):
+                g = sum(float(x[r, c]) * float(wu[j, c]) for c in range(d)) + float(bu[j])
+                u = sum(float(x[r, c]) * float(wu[f + j, c]) for c in range(d)) + float(bu[f + j])
+                silu = lambda t: t / (1.0 + math.exp(-t))  # noqa: E731
+                hidden.append(silu(g) * u if gate_first else g * silu(u))
+            for o in range(d):
+                expected[r, o] = sum(hidden[j] * float(wd[o, j]) for j in range(f)) + float(bd[o])
+        torch.testing.assert_close(oracle.swiglu_ffn(x, wu, bu, wd, bd, gate_first=gate_first), expected)
+        torch.testing.assert_close(F.linear(oracle.swiglu_hidden(x, wu, bu, gate_first=gate_first), wd, bd), expected)
+
+
+def test_block_and_backbone_compose_the_pinned_pieces():
+    from taac_2026_amd import workloads
+
+    inputs = workloads.backbone_inputs(batch=2, n_feature_tokens=4, n_sequence_tokens=12, d_model=32, num_heads=4,
+                                       d_ff=64, n_blocks=2, min_sequence_len=3)
+    w = {k: v.float() for k, v in inputs.blocks[0].items()}
+    x = inputs.emb.float()
+    lengths = inputs.key_lengths
+    h = oracle.rms_norm(x, w["attn_norm.weight"])
+    q, k, v = F.linear(h, w["qkv.weight"], w["qkv.bias"]).chunk(3, -1)
+    split = lambda t: t.view(2, 16, 4, 8).transpose(1, 2)  # noqa: E731
+    mask = oracle.key_length_mask(lengths, 4, 16, 16)
+    a = F.scaled_dot_product_attention(split(q), split(k), split(v), attn_mask=mask).transpose(1, 2).reshape(2, 16, 32)
+    a = a * (~oracle.make_padding_mask(lengths.long(), 16)).unsqueeze(-1)
+    x1 = x + F.linear(a, w["out.weight"], w["out.bias"])
+    expected = x1 + oracle.swiglu_ffn(oracle.rms_norm(x1, w["ffn_norm.weight"]), w["up.weight"], w["up.bias"],
+                                      w["down.weight"], w["down.bias"])
+    torch.testing.assert_close(oracle.block(x, lengths, w, num_heads=4), expected, rtol=1e-5, atol=1e-6)
+
+    blocks = [{k: v.float() for k, v in b.items()} for b in inputs.blocks]
+    p, hidden = oracle.backbone(x, lengths, blocks, inputs.head_weight.float(), inputs.head_bias.float(), num_heads=4,
+                                return_hidden=True)
+    y = x
+    for b in blocks:
+        y = oracle.block(y, lengths, b, num_heads=4)
+    torch.testing.assert_close(hidden, y)
+    for i in range(2):
+        pooled = y[i, : int(lengths[i])].mean(dim=0)
+        z = float(pooled @ inputs.head_weight.float().reshape(-1))
+        assert abs(float(p[i]) - 1.0 / (1.0 + math.exp(-z))) < 1e-6
+    # batch rows are independent
+    p0 = oracle.backbone(x[:1], lengths[:1], blocks, inputs.head_weight.float(), inputs.head_bias.float(), num_heads=4)
+    torch.testing.assert_close(p0, p[:1])
+
+
+# ---- FP8 (no reference counterpart; the rounding itself is pinned, the layer is defined by its formula) ----------------
+
+
+def _e4m3_value(code: int) -> float:
+    sign, exp, man = code >> 7, (code >> 3) & 15, code & 7
+    if exp == 15 and man == 7:
+        return math.nan
+    mag = man / 8.0 * 2.0 ** -6 if exp == 0 else (1.0 + man / 8.0) * 2.0 ** (exp - 7)
+    return -mag if sign else mag
+
+
+def test_e4m3_decode_table_and_nearest_even_rounding():
+    codes = torch.arange(256, dtype=torch.uint8)
+    decoded = codes.view(torch.float8_e4m3fn).float()
+    table = [_e4m3_value(c) for c in range(256)]
+    for c in range(256):
+        assert (math.isnan(table[c]) and math.isnan(decoded[c].item())) or decoded[c].item() == table[c]
+    assert max(v for v in table if not math.isnan(v)) == oracle.FP8_MAX
+    # brute-force nearest-even rounding of arbitrary values onto the finite grid
+    grid = sorted(set(v for v in table if not math.isnan(v)))
+    torch.manual_seed(8)
+    values = torch.cat([torch.randn(2000) * 100, torch.randn(2000), torch.tensor([448.0, -448.0, 0.0, 447.9, 1e-4])])
+    values = values.clamp(-448, 448)
+    q, scale = oracle.fp8_quantize(values, torch.tensor(1.0))
+    assert scale.item() == 1.0
+    for val, got in zip(values.tolist(), q.float().tolist()):
+        best = min(grid, key=lambda g: (abs(g - val), abs(int(torch.tensor(g).to(torch.float8_e4m3fn).view(torch.uint8)) & 1)))
+        assert got == best, (val, got, best)
+
+
+def test_fp8_linear_definition():
+    torch.manual_seed(9)
+    x = torch.randn(16, 32).to(torch.bfloat16)
+    w = (0.1 * torch.randn(24, 32)).to(torch.bfloat16)
+    sx, sw = x.float().abs().max() / 448.0, w.float().abs().max() / 448.0
+    qx = (x.float() / sx).to(torch.float8_e4m3fn)
+    qw = (w.float() / sw).to(torch.float8_e4m3fn)
+    expected = ((qx.float() @ qw.float().T) * sx * sw).to(torch.bfloat16)
+    assert torch.equal(oracle.linear_fp8(x, w), expected)
+    assert oracle.fp8_quantize(x)[0].float().abs().max().item() == 448.0
+    # quantisation error of the layer stays inside the configuration's 5e-2 relative bound
+    exact = x.float() @ w.float().T
+    rel = ((expected.float() - exact).abs().max() / exact.abs().max()).item()
+    assert rel < 5e-2
+    # epilogues
+    gate_value = oracle.linear_fp8(x, w, swiglu=True)
+    y = (qx.float() @ qw.float().T) * sx * sw
+    torch.testing.assert_close(gate_value.float(), (F.silu(y[:, :12]) * y[:, 12:]).to(torch.bfloat16).float())
