@@ -64,7 +64,7 @@ def _accuracy_gate(model, inputs, device) -> dict:
 
 def _kernel_breakdown(inputs, device, iters: int) -> dict:
     """Stand-alone timing of each kernel of one block at the step's shapes (HIP events on the launch stream)."""
-    from taac_2026_amd.api import linear, rms_norm, scaled_dot_product_attention, swiglu_linear
+    from taac_2026_amd.api import norm_linear, scaled_dot_product_attention, swiglu_ffn
 
     B, T, D = inputs.emb.shape
     M, F, H = B * T, inputs.d_ff, inputs.num_heads
@@ -73,28 +73,26 @@ def _kernel_breakdown(inputs, device, iters: int) -> dict:
     lengths = inputs.key_lengths.to(device)
     out: dict[str, dict] = {}
     with torch.no_grad():
-        h = rms_norm(x, w["attn_norm.weight"])
-        qkv = linear(h, w["qkv.weight"], w["qkv.bias"])
+        qkv = norm_linear(x, w["qkv.weight"], w["qkv.bias"], norm_weight=w["attn_norm.weight"])
         q, k, v = qkv.chunk(3, dim=-1)
         attn = lambda: scaled_dot_product_attention(q, k, v, num_heads=H, attn_mask=None, dropout_p=0.0,  # noqa: E731
                                                     training=False, key_lengths=lengths, zero_padded_queries=True)
         a = attn()
-        g = swiglu_linear(h, w["up.weight"], w["up.bias"])
         valid_tokens = float(lengths.sum().item())
         sum_sq = float((lengths.double() ** 2).sum().item())
         dh = D // H
+        # (callable, algorithmic flops, algorithmic HBM bytes) per launch; bf16 = 2 bytes per element
         cases = {
-            "rmsnorm": (lambda: rms_norm(x, w["attn_norm.weight"]), 0.0, 2.0 * M * D * 2 + 2 * D),
-            "linear_qkv": (lambda: linear(h, w["qkv.weight"], w["qkv.bias"]), 2.0 * M * 3 * D * D,
-                           2.0 * (M * D + 3 * D * D + M * 3 * D)),
+            "rmsnorm_qkv": (lambda: norm_linear(x, w["qkv.weight"], w["qkv.bias"], norm_weight=w["attn_norm.weight"]),
+                            2.0 * M * 3 * D * D, 2.0 * (M * D + 3 * D * D + M * 3 * D)),
             # useful work only: visible (query, key) pairs; Q/K/V valid rows read, O written in full
             "attention": (attn, 4.0 * H * dh * sum_sq, 2.0 * (3 * D * valid_tokens + M * D)),
-            "linear_out_residual": (lambda: linear(a, w["out.weight"], w["out.bias"], residual=x), 2.0 * M * D * D,
-                                    2.0 * (3 * M * D + D * D)),
-            "linear_up_swiglu": (lambda: swiglu_linear(h, w["up.weight"], w["up.bias"]), 2.0 * M * 2 * F * D,
-                                 2.0 * (M * D + 2 * F * D + M * F)),
-            "linear_down_residual": (lambda: linear(g, w["down.weight"], w["down.bias"], residual=x),
-                                     2.0 * M * D * F, 2.0 * (M * F + D * F + 2 * M * D)),
+            "out_residual": (lambda: norm_linear(a, w["out.weight"], w["out.bias"], residual=x), 2.0 * M * D * D,
+                             2.0 * (3 * M * D + D * D)),
+            "rmsnorm_swiglu_ffn_residual": (
+                lambda: swiglu_ffn(x, w["up.weight"], w["up.bias"], w["down.weight"], w["down.bias"], residual=x,
+                                   norm_weight=w["ffn_norm.weight"]),
+                2.0 * M * 3 * D * F, 2.0 * (2 * M * D + 3 * D * F)),
         }
         for name, (fn, flops, nbytes) in cases.items():
             ms = _event_ms(fn, iters, 3)

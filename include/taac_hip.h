@@ -103,6 +103,31 @@ int taac_linear_bf16(const void* a, int64_t lda, const void* w, const void* bias
                      int64_t ldo, int64_t M, int32_t N, int32_t K, int epilogue, int gate_first, void* stream);
 
 /*
+ * Fused feed-forward half of a block, one kernel:
+ *   out = residual + down( silu(g) * u ),   g, u = chunk2( up( norm_weight ? rmsnorm(x, norm_weight, eps) : x ) )
+ * x: [M, D] bf16 (row stride ldx); w_up: [2F, D]; b_up: [2F] or NULL; w_down: [D, F]; b_down: [D] or NULL;
+ * residual: [M, D] (row stride ldr) or NULL; out: [M, D] (row stride ldo), may alias residual and x.
+ * D must be 128 or 256, F a multiple of 32. The [M, 2F] projection and the [M, F] gated hidden state are never
+ * written to memory. gate_first as in taac_linear_bf16.
+ * Replaces: ffn_norm + SwiGLUFeedForward.forward + residual add of UnifiedInteractionBlock.forward
+ * (experiments/symbiosis/backbone.py:19-21, 66-67).
+ */
+int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w_up,
+                        const void* b_up, const void* w_down, const void* b_down, const void* residual, int64_t ldr,
+                        void* out, int64_t ldo, int64_t M, int32_t D, int32_t F, int gate_first, void* stream);
+
+/*
+ * Fused [RMSNorm ->] dense layer [-> + residual] with the token rows held in registers:
+ *   out = (residual ? residual : 0) + (norm_weight ? rmsnorm(x, norm_weight, eps) : x) @ w^T + bias
+ * x: [M, K] bf16; w: [N, K]; bias: [N] or NULL; residual / out: [M, N]. K must be 128 or 256, N a multiple of 64.
+ * Replaces: attn_norm + the qkv projection, and the out projection + residual add, of UnifiedInteractionBlock /
+ * UnifiedSelfAttention (experiments/symbiosis/backbone.py:34-35, 47, 64-65).
+ */
+int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
+                         const void* bias, const void* residual, int64_t ldr, void* out, int64_t ldo, int64_t M,
+                         int32_t N, int32_t K, void* stream);
+
+/*
  * Per-tensor absolute maximum, for the FP8 scale (scale = amax / 448). Writes max(|x|) over n elements to
  * *amax_out (device float). The kernel clears *amax_out itself before reducing.
  * No counterpart in the reference (it has no FP8 code); defined by the FP8 configuration of this path.

@@ -9,7 +9,7 @@ from taac_2026_amd.accelerators.attention import (
     plan_flash_attention_mask,
     resolved_flash_attention_backend,
 )
-from taac_2026_amd.accelerators.linear import amax, linear, linear_fp8, quantize_fp8, swiglu_ffn, swiglu_linear
+from taac_2026_amd.accelerators.linear import amax, linear, linear_fp8, norm_linear, quantize_fp8, swiglu_ffn, swiglu_linear
 from taac_2026_amd.accelerators.normalization import (
     hip_layer_norm_kernel,
     hip_rms_norm_kernel,
@@ -37,6 +37,7 @@ __all__ = [
     "layer_norm",
     "linear",
     "linear_fp8",
+    "norm_linear",
     "plan_flash_attention_mask",
     "quantize_fp8",
     "require_cuda_tensors",

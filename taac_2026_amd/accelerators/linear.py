@@ -102,6 +102,10 @@ def swiglu_linear(
     return out.reshape(*shape[:-1], hidden)
 
 
+def _fused_width(d: int) -> bool:
+    return d in (128, 256)
+
+
 def swiglu_ffn(
     x: torch.Tensor,
     up_weight: torch.Tensor,
@@ -111,10 +115,98 @@ def swiglu_ffn(
     *,
     residual: torch.Tensor | None = None,
     gate_first: bool = True,
+    norm_weight: torch.Tensor | None = None,
+    eps: float = 1e-6,
 ) -> torch.Tensor:
-    """``down(silu(gate) * value)`` with ``gate, value = up(x).chunk(2, -1)``; optional fused ``+ residual``."""
-    hidden = swiglu_linear(x, up_weight, up_bias, gate_first=gate_first)
-    return linear(hidden, down_weight, down_bias, residual=residual)
+    """``residual + down(silu(gate) * value)`` with ``gate, value = up(rmsnorm(x)).chunk(2, -1)``.
+
+    ``norm_weight`` (optional) fuses the pre-FFN RMSNorm; ``residual`` (optional) the residual add. For model widths
+    128 / 256 with a hidden size that is a multiple of 32 the whole expression is ONE kernel
+    (``taac_swiglu_ffn_fwd``: the projection and the gated hidden state stay in registers); other shapes run
+    norm -> up(+SiLU-gate) -> down(+residual) as separate kernels.
+    """
+    name = "hip swiglu_ffn"
+    require_cuda_tensors(name, x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight)
+    require_inference(name, x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight)
+    _check_bf16(name, x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight)
+    rows, shape = _as_rows(x)
+    _check_weight(name, rows, up_weight, up_bias)
+    d_model, hidden = rows.shape[1], up_weight.shape[0] // 2
+    if up_weight.shape[0] % 2 != 0 or down_weight.shape != (d_model, hidden):
+        raise ValueError("swiglu_ffn expects up_weight [2F, D] and down_weight [D, F]")
+    if residual is not None and residual.shape != shape:
+        raise ValueError("swiglu_ffn residual must have the shape of the input")
+    if not (_fused_width(d_model) and hidden % 32 == 0):
+        h = rows
+        if norm_weight is not None:
+            from taac_2026_amd.accelerators.normalization import rms_norm
+
+            h = rms_norm(rows, norm_weight, eps)
+        gated = swiglu_linear(h, up_weight, up_bias, gate_first=gate_first)
+        res_rows = residual.reshape(-1, d_model) if residual is not None else None
+        return linear(gated, down_weight, down_bias, residual=res_rows).reshape(shape)
+    up_weight, down_weight = up_weight.contiguous(), down_weight.contiguous()
+    res_rows = None
+    if residual is not None:
+        res_rows = residual.reshape(-1, d_model)
+        if res_rows.stride(-1) != 1 or res_rows.stride(0) % 8 != 0:
+            res_rows = res_rows.contiguous()
+    out = torch.empty((rows.shape[0], d_model), dtype=x.dtype, device=x.device)
+    library = _native.load_library()
+    status = library.taac_swiglu_ffn_fwd(
+        rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), up_weight.data_ptr(),
+        _native.ptr(up_bias), down_weight.data_ptr(), _native.ptr(down_bias), _native.ptr(res_rows),
+        res_rows.stride(0) if res_rows is not None else d_model, out.data_ptr(), d_model, rows.shape[0], d_model,
+        hidden, int(bool(gate_first)), _native.current_stream(x.device),
+    )
+    _native.check(status, "swiglu_ffn")
+    return out.reshape(shape)
+
+
+def norm_linear(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None = None,
+    *,
+    norm_weight: torch.Tensor | None = None,
+    eps: float = 1e-6,
+    residual: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """``residual + F.linear(rmsnorm(x, norm_weight, eps), weight, bias)`` (norm and residual optional) as one
+    kernel when ``in_features`` is 128 / 256 and ``out_features`` a multiple of 64; otherwise composed from the
+    stand-alone kernels."""
+    name = "hip norm_linear"
+    require_cuda_tensors(name, x, weight, bias, residual, norm_weight)
+    require_inference(name, x, weight, bias, residual, norm_weight)
+    _check_bf16(name, x, weight, bias, residual, norm_weight)
+    rows, shape = _as_rows(x)
+    _check_weight(name, rows, weight, bias)
+    in_features, out_features = weight.shape[1], weight.shape[0]
+    if not (_fused_width(in_features) and out_features % 64 == 0):
+        h = rows
+        if norm_weight is not None:
+            from taac_2026_amd.accelerators.normalization import rms_norm
+
+            h = rms_norm(rows, norm_weight, eps)
+        res = residual.reshape(-1, out_features) if residual is not None else None
+        return linear(h, weight, bias, residual=res).reshape(*shape[:-1], out_features)
+    weight = weight.contiguous()
+    res_rows = None
+    if residual is not None:
+        if residual.shape != (*shape[:-1], out_features):
+            raise ValueError("norm_linear residual must have the shape of the output")
+        res_rows = residual.reshape(-1, out_features)
+        if res_rows.stride(-1) != 1 or res_rows.stride(0) % 8 != 0:
+            res_rows = res_rows.contiguous()
+    out = torch.empty((rows.shape[0], out_features), dtype=x.dtype, device=x.device)
+    library = _native.load_library()
+    status = library.taac_norm_linear_fwd(
+        rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), weight.data_ptr(), _native.ptr(bias),
+        _native.ptr(res_rows), res_rows.stride(0) if res_rows is not None else out_features, out.data_ptr(),
+        out_features, rows.shape[0], out_features, in_features, _native.current_stream(x.device),
+    )
+    _native.check(status, "norm_linear")
+    return out.reshape(*shape[:-1], out_features)
 
 
 # ---- FP8 (OCP e4m3fn, per-tensor scale = amax / 448) ---------------------------------------------------------------
@@ -206,6 +298,7 @@ __all__ = [
     "amax",
     "linear",
     "linear_fp8",
+    "norm_linear",
     "quantize_fp8",
     "swiglu_ffn",
     "swiglu_linear",

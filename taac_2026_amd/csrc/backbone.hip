@@ -129,25 +129,41 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
       return set_error(TAAC_ERR_INVALID_VALUE, "%s: block %d has a null weight", name, i);
     const bool last = (i == n_blocks - 1);
     bf16_t* x_out = (last && hidden_out != nullptr) ? static_cast<bf16_t*>(hidden_out) : x;
+    const bool fused = (D == 128 || D == 256) && F % 32 == 0;  // token-stationary kernels: norms and residuals fused
     // attention half
-    if ((rc = taac_rmsnorm_fwd(cur, w.attn_norm_weight, h, M, D, eps, TAAC_BF16, stream)) != TAAC_OK) return rc;
-    if ((rc = taac_linear_bf16(h, D, w.qkv_weight, w.qkv_bias, nullptr, qkv, 3 * D, M, 3 * D, D, TAAC_EPI_NONE, 1,
-                               stream)) != TAAC_OK)
-      return rc;
+    if (fused) {
+      if ((rc = taac_norm_linear_fwd(cur, D, w.attn_norm_weight, eps, w.qkv_weight, w.qkv_bias, nullptr, 0, qkv, 3 * D,
+                                     M, 3 * D, D, stream)) != TAAC_OK)
+        return rc;
+    } else {
+      if ((rc = taac_rmsnorm_fwd(cur, w.attn_norm_weight, h, M, D, eps, TAAC_BF16, stream)) != TAAC_OK) return rc;
+      if ((rc = taac_linear_bf16(h, D, w.qkv_weight, w.qkv_bias, nullptr, qkv, 3 * D, M, 3 * D, D, TAAC_EPI_NONE, 1,
+                                 stream)) != TAAC_OK)
+        return rc;
+    }
     if ((rc = taac_flash_attn_fwd(qkv, qkv + D, qkv + 2 * D, key_lengths, h, B, heads, T, T, dh, qkv_strides,
                                   qkv_strides, qkv_strides, o_strides, 0, 1, TAAC_BF16, stream)) != TAAC_OK)
       return rc;
-    if ((rc = taac_linear_bf16(h, D, w.out_weight, w.out_bias, cur, x, D, M, D, D, TAAC_EPI_RESIDUAL, 1, stream)) !=
-        TAAC_OK)
-      return rc;
-    // feed-forward half
-    if ((rc = taac_rmsnorm_fwd(x, w.ffn_norm_weight, h, M, D, eps, TAAC_BF16, stream)) != TAAC_OK) return rc;
-    if ((rc = taac_linear_bf16(h, D, w.up_weight, w.up_bias, nullptr, g, F, M, 2 * F, D, TAAC_EPI_SWIGLU, 1, stream)) !=
-        TAAC_OK)
-      return rc;
-    if ((rc = taac_linear_bf16(g, F, w.down_weight, w.down_bias, x, x_out, D, M, D, F, TAAC_EPI_RESIDUAL, 1, stream)) !=
-        TAAC_OK)
-      return rc;
+    if (fused) {
+      if ((rc = taac_norm_linear_fwd(h, D, nullptr, eps, w.out_weight, w.out_bias, cur, D, x, D, M, D, D, stream)) !=
+          TAAC_OK)
+        return rc;
+      // feed-forward half: RMSNorm -> up -> SiLU-gate -> down -> + residual in one kernel
+      if ((rc = taac_swiglu_ffn_fwd(x, D, w.ffn_norm_weight, eps, w.up_weight, w.up_bias, w.down_weight, w.down_bias, x,
+                                    D, x_out, D, M, D, F, 1, stream)) != TAAC_OK)
+        return rc;
+    } else {
+      if ((rc = taac_linear_bf16(h, D, w.out_weight, w.out_bias, cur, x, D, M, D, D, TAAC_EPI_RESIDUAL, 1, stream)) !=
+          TAAC_OK)
+        return rc;
+      if ((rc = taac_rmsnorm_fwd(x, w.ffn_norm_weight, h, M, D, eps, TAAC_BF16, stream)) != TAAC_OK) return rc;
+      if ((rc = taac_linear_bf16(h, D, w.up_weight, w.up_bias, nullptr, g, F, M, 2 * F, D, TAAC_EPI_SWIGLU, 1,
+                                 stream)) != TAAC_OK)
+        return rc;
+      if ((rc = taac_linear_bf16(g, F, w.down_weight, w.down_bias, x, x_out, D, M, D, F, TAAC_EPI_RESIDUAL, 1,
+                                 stream)) != TAAC_OK)
+        return rc;
+    }
     cur = x_out;
   }
   if (n_blocks == 0 && hidden_out != nullptr) {

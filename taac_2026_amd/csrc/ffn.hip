@@ -1,0 +1,503 @@
+// Token-stationary fused dense kernels for gfx950 (model width D = 256 or 128):
+//   taac_swiglu_ffn_fwd : out = residual + down( silu(gate) * value ),  gate, value = up( rmsnorm(x) ).chunk(2)
+//   taac_norm_linear_fwd: out = [residual +] linear( [rmsnorm](x) )
+//
+// Why token-stationary. With D = 256 the whole reduction axis of a token fits in registers: a wavefront keeps the
+// (optionally RMS-normalised) rows of its 64 tokens as MFMA B-operand fragments for the entire kernel
+// (16 k-steps x 2 token tiles x 4 VGPRs) and only the WEIGHTS stream past it. The weights are staged through LDS
+// in fragment order by direct global->LDS loads (no register staging, one 1 KB fragment per wavefront-wide
+// instruction), double-buffered, one workgroup barrier per chunk of ~3 000 MFMA cycles. Every weight fragment read
+// from LDS feeds two MFMAs (the two token tiles), so the LDS read traffic is half a fragment per MFMA, and the token
+// matrix is read from HBM exactly once and never written back between the fused stages.
+//
+// Fused SwiGLU FFN. The products are formed transposed: H^T[hidden, token] = W_up X^T, so a lane owns one token and
+// eight hidden units of a 16-unit chunk; silu(g) * u is formed in registers and is already the B operand of the
+// second product O^T[feature, token] += W_down[:, chunk] H^T. The row order in which a chunk's W_up rows are loaded
+// is chosen so that the accumulator's register order of hidden units equals the natural k order of W_down's
+// fragments. The [M, 2F] projection and the [M, F] gated hidden state never exist in memory.
+// Replaces SwiGLUFeedForward.forward + the ffn_norm and residual of UnifiedInteractionBlock.forward
+// (experiments/symbiosis/backbone.py:19-21, 66-67).
+#include <cstdlib>
+
+#include "common.h"
+
+namespace taac {
+namespace {
+
+constexpr int kTokPerWg = 256;
+constexpr int kFrag = 1024;       // bytes of one 32 x 16 bf16 MFMA operand fragment
+constexpr int kNC = 64;           // output features per chunk of the plain linear kernel
+
+struct TsParams {
+  const bf16_t* x;          // [M, D] row stride ldx
+  const bf16_t* norm_w;     // [D] or null (no normalisation)
+  const bf16_t* w1;         // FFN: w_up [2F, D];  linear: w [N, D]
+  const bf16_t* b1;         // FFN: b_up [2F] or null; linear: bias [N] or null
+  const bf16_t* w2;         // FFN: w_down [D, F]
+  const bf16_t* b2;         // FFN: b_down [D] or null
+  const bf16_t* residual;   // [M, D or N] row stride ldr, or null
+  bf16_t* out;              // [M, D or N] row stride ldo
+  int64_t M, ldx, ldr, ldo;
+  int32_t F;                // FFN hidden size
+  int32_t N;                // linear output features
+  float eps;
+  int32_t gate_first;
+};
+
+__device__ __forceinline__ float silu_f(float v) {
+  return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * v));
+}
+
+__device__ __forceinline__ void lds_dma16(const void* gsrc, void* lds_wave_base) {
+  // 16 bytes per lane, lane l lands at lds_wave_base + 16 * l
+  __builtin_amdgcn_global_load_lds(gsrc, lds_wave_base, 16, 0, 0);
+}
+
+// Loads the wavefront's 64 token rows as B-operand fragments and, if norm_w is given, RMS-normalises them in place:
+// y = bf16( x * rsqrt(mean(x^2) + eps) * w ). Lane (l32, hh) holds features 16*ks + 8*hh .. +7 of token l32.
+template <int D, int TT>
+__device__ __forceinline__ void load_tokens(const TsParams& p, int64_t tok0, int l32, int hh,
+                                            bf16x8 (&xf)[TT][D / 16]) {
+  constexpr int KS = D / 16;
+#pragma unroll
+  for (int t = 0; t < TT; ++t) {
+    // Rows beyond M are clamped to the last row: their results are computed but never stored.
+    int64_t tok = tok0 + t * 32 + l32;
+    tok = tok < p.M ? tok : p.M - 1;
+    const bf16_t* row = p.x + tok * p.ldx + hh * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) xf[t][ks] = *reinterpret_cast<const bf16x8*>(row + ks * 16);
+  }
+  if (p.norm_w == nullptr) return;
+  float scale[TT];
+#pragma unroll
+  for (int t = 0; t < TT; ++t) {
+    float ss = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float v = static_cast<float>(xf[t][ks][e]);
+        ss += v * v;
+      }
+    ss += __shfl_xor(ss, 32, kWave);
+    scale[t] = rsqrtf(ss * (1.0f / D) + p.eps);
+  }
+  // Make the packed rows opaque here: otherwise the compiler keeps all D fp32 copies from the first sweep alive for
+  // the second one, which does not fit the register file next to the accumulators.
+#pragma unroll
+  for (int t = 0; t < TT; ++t)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(xf[t][ks]));
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const bf16x8 wv = *reinterpret_cast<const bf16x8*>(p.norm_w + ks * 16 + hh * 8);
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        xf[t][ks][e] = static_cast<bf16_t>(static_cast<float>(xf[t][ks][e]) * scale[t] * static_cast<float>(wv[e]));
+      asm volatile("" : "+v"(xf[t][ks]));
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// Fused RMSNorm -> up -> SiLU-gate -> down -> + residual
+//
+// A chunk is 16 hidden units. Its up-projection fragment has 32 rows: 16 gate rows on top of the 16 matching value
+// rows, so ONE accumulator (16 registers per lane) holds g in registers 0..7 and u in registers 8..15 for the same
+// eight hidden units of the lane's token. silu(g) * u of those eight is exactly one B-operand fragment (k = 16) of
+// the down projection. Two chunks are staged and consumed per barrier.
+// ------------------------------------------------------------------------------------------------------------------
+constexpr int kHU = 16;  // hidden units per chunk
+constexpr int kCPB = 2;  // chunks per barrier
+
+// Hidden unit (0..15) loaded into row slot m16 of the gate (or value) half of an up fragment: chosen so that
+// accumulator register j < 8 of lane half hh holds hidden unit 8*hh + j, the k order of a W_down fragment.
+__device__ __forceinline__ int up_unit_of_slot(int m16) { return 8 * ((m16 >> 2) & 1) + 4 * (m16 >> 3) + (m16 & 3); }
+
+template <int D, int TT>
+__global__ __launch_bounds__(kTokPerWg / (32 * TT) * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_kernel(const TsParams p) {
+  constexpr int NWAVES = kTokPerWg / (32 * TT);  // 4 wavefronts of 64 tokens, or 8 of 32
+  constexpr int KS = D / 16;             // k-steps of the up projection = up fragments per chunk
+  constexpr int MB = D / 32;             // 32-feature row blocks of the down projection = down fragments per chunk
+  constexpr int CFRAG = KS + MB;         // fragments per chunk
+  constexpr int NFRAG = kCPB * CFRAG;    // fragments per barrier step
+  constexpr int FPW = NFRAG / NWAVES;    // fragments staged per wavefront
+  static_assert(NFRAG % NWAVES == 0, "fragments must divide over the wavefronts");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // 2 buffers x NFRAG KB
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // wavefront-uniform, kept in a scalar register
+  const int lane = tid % kWave;
+  const int l32 = lane % 32;
+  const int hh = lane / 32;
+  const int64_t tok0 = static_cast<int64_t>(blockIdx.x) * kTokPerWg + wave * (32 * TT);
+  const int F = p.F;
+  const int nsteps = F / (kHU * kCPB);
+
+  // Source address of a staged fragment = wavefront-uniform base (scalar registers) + a 32-bit per-lane byte offset:
+  //   up fragment (chunk q, k-step ks): row slot l32 -> W_up row [value ? F : 0] + q*16 + unit(l32 % 16), cols ks*16 + hh*8
+  //   down fragment (chunk q, block mb): W_down row mb*32 + l32, cols q*16 + hh*8
+  const char* w_up_bytes = reinterpret_cast<const char*>(p.w1);
+  const char* w_down_bytes = reinterpret_cast<const char*>(p.w2);
+  auto stage = [&](int step, int buf) {
+    // The two lane offsets are recomputed from an opaque copy of the lane id on every call: as loop invariants they
+    // would be kept live (and spilled) across the whole main loop.
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const int s32 = ln & 31, shh = ln >> 5;
+    const uint32_t up_lane_off =
+        static_cast<uint32_t>((((s32 >= 16 ? F : 0) + up_unit_of_slot(s32 & 15)) * D + shh * 8) * 2);
+    const uint32_t down_lane_off = static_cast<uint32_t>((s32 * F + shh * 8) * 2);
+    uint8_t* base = smem + buf * (NFRAG * kFrag) + wave * (FPW * kFrag);
+#pragma unroll
+    for (int i = 0; i < FPW; ++i) {
+      const int f = wave * FPW + i;       // wavefront-uniform
+      const int q = f / CFRAG;            // chunk inside the step
+      const int r = f % CFRAG;
+      const int64_t unit0 = static_cast<int64_t>(step * kCPB + q) * kHU;
+      if (r < KS)
+        lds_dma16(w_up_bytes + (unit0 * D + r * 16) * 2 + up_lane_off, base + i * kFrag);
+      else
+        lds_dma16(w_down_bytes + (static_cast<int64_t>(r - KS) * 32 * F + unit0) * 2 + down_lane_off, base + i * kFrag);
+    }
+  };
+
+  stage(0, 0);
+
+  bf16x8 xf[TT][KS];
+  load_tokens<D, TT>(p, tok0, l32, hh, xf);
+
+  f32x16 oacc[TT][MB];
+#pragma unroll
+  for (int t = 0; t < TT; ++t)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) oacc[t][mb][j] = 0.f;
+
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  for (int step = 0; step < nsteps; ++step) {
+    const int buf = step & 1;
+    if (step + 1 < nsteps) stage(step + 1, buf ^ 1);
+#pragma unroll
+    for (int q = 0; q < kCPB; ++q) {
+      const uint8_t* wb = smem + buf * (NFRAG * kFrag) + q * (CFRAG * kFrag) + lane * 16;
+      const int unit0 = (step * kCPB + q) * kHU;
+      // ---- up projection: rows 0..15 gate, rows 16..31 value, both token tiles ------------------------------------
+      f32x16 gu[TT];
+#pragma unroll
+      for (int t = 0; t < TT; ++t)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) gu[t][j] = 0.f;
+      // Fragment reads run kPre fragments ahead of their MFMAs; the scheduling fences keep the compiler from hoisting
+      // every read of the chunk to the top (which would not fit the register file).
+      constexpr int kPre = 3;
+      bf16x8 apipe[kPre + 1];
+#pragma unroll
+      for (int i = 0; i < kPre; ++i) apipe[i] = *reinterpret_cast<const bf16x8*>(wb + i * kFrag);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks + kPre < KS + MB)
+          apipe[(ks + kPre) % (kPre + 1)] = *reinterpret_cast<const bf16x8*>(wb + (ks + kPre) * kFrag);
+        const bf16x8 a = apipe[ks % (kPre + 1)];
+#pragma unroll
+        for (int t = 0; t < TT; ++t) gu[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, xf[t][ks], gu[t], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // ---- bias + SiLU gate: register j < 8 is g, register 8 + j is u of hidden unit unit0 + 8*hh + j --------------
+      float bg[8], bu[8];
+      if (p.b1 != nullptr) {
+        const bf16x8 vg = *reinterpret_cast<const bf16x8*>(p.b1 + unit0 + 8 * hh);
+        const bf16x8 vu = *reinterpret_cast<const bf16x8*>(p.b1 + F + unit0 + 8 * hh);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          bg[e] = static_cast<float>(vg[e]);
+          bu[e] = static_cast<float>(vu[e]);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          bg[e] = 0.f;
+          bu[e] = 0.f;
+        }
+      }
+      bf16x8 hb[TT];
+#pragma unroll
+      for (int t = 0; t < TT; ++t)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float g = gu[t][e] + bg[e];
+          const float u = gu[t][8 + e] + bu[e];
+          hb[t][e] = static_cast<bf16_t>(p.gate_first ? silu_f(g) * u : g * silu_f(u));
+        }
+      // ---- down projection: O^T[feature, token] += W_down[feature, chunk] H^T --------------------------------------
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const int f = KS + mb;  // fragment index inside the chunk; the first kPre down fragments are already in flight
+        if (f + kPre < KS + MB)
+          apipe[(f + kPre) % (kPre + 1)] = *reinterpret_cast<const bf16x8*>(wb + (f + kPre) * kFrag);
+        const bf16x8 ad = apipe[f % (kPre + 1)];
+#pragma unroll
+        for (int t = 0; t < TT; ++t)
+          oacc[t][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ad, hb[t], oacc[t][mb], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+
+  // ---- epilogue: + b_down + residual, bf16 store; lane owns token l32 and 4-feature runs ---------------------------
+#pragma unroll
+  for (int t = 0; t < TT; ++t) {
+    const int64_t tok = tok0 + t * 32 + l32;
+    if (tok >= p.M) continue;
+    bf16_t* orow = p.out + tok * p.ldo;
+    const bf16_t* rrow = p.residual != nullptr ? p.residual + tok * p.ldr : nullptr;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+      for (int jq = 0; jq < 4; ++jq) {
+        const int col = mb * 32 + jq * 8 + hh * 4;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = oacc[t][mb][jq * 4 + e];
+        if (p.b2 != nullptr) {
+          const bf16x4 bv = *reinterpret_cast<const bf16x4*>(p.b2 + col);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] += static_cast<float>(bv[e]);
+        }
+        if (rrow != nullptr) {
+          const bf16x4 rv = *reinterpret_cast<const bf16x4*>(rrow + col);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] += static_cast<float>(rv[e]);
+        }
+        bf16x4 ov;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ov[e] = static_cast<bf16_t>(v[e]);
+        *reinterpret_cast<bf16x4*>(orow + col) = ov;
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keep the residual loads of later blocks from being hoisted up here
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// [RMSNorm ->] linear [-> + residual], K = D, N a multiple of 64
+// ------------------------------------------------------------------------------------------------------------------
+template <int D, int TT>
+__global__ __launch_bounds__(kTokPerWg / (32 * TT) * kWave, TT == 1 ? 2 : 1) void norm_linear_kernel(const TsParams p) {
+  constexpr int NWAVES = kTokPerWg / (32 * TT);
+  constexpr int KS = D / 16;
+  constexpr int NFRAG = 2 * KS;    // two 32-feature row blocks per chunk
+  constexpr int FPW = NFRAG / NWAVES;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // wavefront-uniform, kept in a scalar register
+  const int lane = tid % kWave;
+  const int l32 = lane % 32;
+  const int hh = lane / 32;
+  const int64_t tok0 = static_cast<int64_t>(blockIdx.x) * kTokPerWg + wave * (32 * TT);
+  const int nchunks = p.N / kNC;
+
+  // fragment f of a chunk = (row block f / KS, k-step f % KS); source = uniform base + 32-bit per-lane byte offset
+  const char* w_bytes = reinterpret_cast<const char*>(p.w1);
+  auto stage = [&](int chunk, int buf) {
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const uint32_t lane_off = static_cast<uint32_t>(((ln & 31) * D + (ln >> 5) * 8) * 2);
+    uint8_t* base = smem + buf * (NFRAG * kFrag) + wave * (FPW * kFrag);
+#pragma unroll
+    for (int i = 0; i < FPW; ++i) {
+      const int f = wave * FPW + i;  // wavefront-uniform
+      const int64_t row0 = static_cast<int64_t>(chunk) * kNC + (f / KS) * 32;
+      lds_dma16(w_bytes + (row0 * D + (f % KS) * 16) * 2 + lane_off, base + i * kFrag);
+    }
+  };
+
+  stage(0, 0);
+  bf16x8 xf[TT][KS];
+  load_tokens<D, TT>(p, tok0, l32, hh, xf);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  for (int c = 0; c < nchunks; ++c) {
+    const int buf = c & 1;
+    if (c + 1 < nchunks) stage(c + 1, buf ^ 1);
+    const uint8_t* wb = smem + buf * (NFRAG * kFrag) + lane * 16;
+    f32x16 acc[2][TT];  // [row block][token tile]
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int t = 0; t < TT; ++t)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[rb][t][j] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(wb + ks * kFrag);
+      const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(wb + (KS + ks) * kFrag);
+#pragma unroll
+      for (int t = 0; t < TT; ++t) {
+        acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, xf[t][ks], acc[0][t], 0, 0, 0);
+        acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, xf[t][ks], acc[1][t], 0, 0, 0);
+      }
+    }
+    // epilogue of this chunk: features c*64 + rb*32 + jq*8 + hh*4 .. +3 of token l32
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+      const int64_t tok = tok0 + t * 32 + l32;
+      if (tok < p.M) {
+        bf16_t* orow = p.out + tok * p.ldo;
+        const bf16_t* rrow = p.residual != nullptr ? p.residual + tok * p.ldr : nullptr;
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+          for (int jq = 0; jq < 4; ++jq) {
+            const int col = c * kNC + rb * 32 + jq * 8 + hh * 4;
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[rb][t][jq * 4 + e];
+            if (p.b1 != nullptr) {
+              const bf16x4 bv = *reinterpret_cast<const bf16x4*>(p.b1 + col);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[e] += static_cast<float>(bv[e]);
+            }
+            if (rrow != nullptr) {
+              const bf16x4 rv = *reinterpret_cast<const bf16x4*>(rrow + col);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[e] += static_cast<float>(rv[e]);
+            }
+            bf16x4 ov;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ov[e] = static_cast<bf16_t>(v[e]);
+            *reinterpret_cast<bf16x4*>(orow + col) = ov;
+          }
+        }
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+}
+
+// The kernels use more than the default 64 KB of dynamic LDS; the opt-in is idempotent and cheap, so it is simply
+// repeated before every launch (no cached per-process state to go stale across devices).
+template <typename K>
+int launch_ts(K kernel, const TsParams& p, int threads, size_t lds_bytes, hipStream_t s, const char* name) {
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          static_cast<int>(lds_bytes)) != hipSuccess)
+    return set_error(TAAC_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", name, lds_bytes);
+  const int64_t grid = (p.M + kTokPerWg - 1) / kTokPerWg;
+  if (grid > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many workgroups", name);
+  hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(grid)), dim3(threads), lds_bytes, s, p);
+  return check_launch(name);
+}
+
+// Token tiles per wavefront: 1 = 8 wavefronts x 32 tokens (two per SIMD), 2 = 4 wavefronts x 64 tokens.
+int ts_token_tiles() {
+  static const int tiles = [] {
+    const char* env = getenv("TAAC_TS_TOKEN_TILES");
+    return (env != nullptr && env[0] == '2') ? 2 : 1;
+  }();
+  return tiles;
+}
+
+bool ptr_ok(const void* p, uintptr_t mask) { return (reinterpret_cast<uintptr_t>(p) & mask) == 0; }
+
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w_up,
+                                   const void* b_up, const void* w_down, const void* b_down, const void* residual,
+                                   int64_t ldr, void* out, int64_t ldo, int64_t M, int32_t D, int32_t F, int gate_first,
+                                   void* stream) {
+  using namespace taac;
+  const char* name = "taac_swiglu_ffn_fwd";
+  if (M < 0 || D <= 0 || F <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, D and F > 0", name);
+  if (D != 256 && D != 128)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: fused kernel is built for D = 128 or 256 (got %d)", name, D);
+  if (F % (kHU * kCPB) != 0)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: F=%d must be a multiple of %d", name, F, kHU * kCPB);
+  if (ldx < D || ldo < D || (residual && ldr < D) || ldx % 8 || ldo % 8 || (residual && ldr % 8))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: row strides must cover a row and be multiples of 8", name);
+  if (M == 0) return TAAC_OK;
+  if (!x || !w_up || !w_down || !out) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
+  if (!ptr_ok(x, 15) || !ptr_ok(w_up, 15) || !ptr_ok(w_down, 15) || !ptr_ok(out, 15) || !ptr_ok(residual, 15) ||
+      !ptr_ok(norm_weight, 15) || !ptr_ok(b_up, 15) || !ptr_ok(b_down, 15))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
+  TsParams p{};
+  p.x = static_cast<const bf16_t*>(x);
+  p.norm_w = static_cast<const bf16_t*>(norm_weight);
+  p.w1 = static_cast<const bf16_t*>(w_up);
+  p.b1 = static_cast<const bf16_t*>(b_up);
+  p.w2 = static_cast<const bf16_t*>(w_down);
+  p.b2 = static_cast<const bf16_t*>(b_down);
+  p.residual = static_cast<const bf16_t*>(residual);
+  p.out = static_cast<bf16_t*>(out);
+  p.M = M;
+  p.ldx = ldx;
+  p.ldr = ldr;
+  p.ldo = ldo;
+  p.F = F;
+  p.eps = eps;
+  p.gate_first = gate_first ? 1 : 0;
+  hipStream_t s = as_stream(stream);
+  const int tt = ts_token_tiles();
+  const int threads = kTokPerWg / (32 * tt) * kWave;
+  if (D == 256) {
+    const size_t lds = 2 * kCPB * (16 + 8) * kFrag;
+    return tt == 1 ? launch_ts(swiglu_ffn_kernel<256, 1>, p, threads, lds, s, name)
+                   : launch_ts(swiglu_ffn_kernel<256, 2>, p, threads, lds, s, name);
+  }
+  const size_t lds = 2 * kCPB * (8 + 4) * kFrag;
+  return tt == 1 ? launch_ts(swiglu_ffn_kernel<128, 1>, p, threads, lds, s, name)
+                 : launch_ts(swiglu_ffn_kernel<128, 2>, p, threads, lds, s, name);
+}
+
+extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
+                                    const void* bias, const void* residual, int64_t ldr, void* out, int64_t ldo,
+                                    int64_t M, int32_t N, int32_t K, void* stream) {
+  using namespace taac;
+  const char* name = "taac_norm_linear_fwd";
+  if (M < 0 || N <= 0 || K <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, N and K > 0", name);
+  if (K != 256 && K != 128)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: token-stationary kernel is built for K = 128 or 256 (got %d)", name, K);
+  if (N % kNC != 0) return set_error(TAAC_ERR_UNSUPPORTED, "%s: N=%d must be a multiple of %d", name, N, kNC);
+  if (ldx < K || ldo < N || (residual && ldr < N) || ldx % 8 || ldo % 8 || (residual && ldr % 8))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: row strides must cover a row and be multiples of 8", name);
+  if (M == 0) return TAAC_OK;
+  if (!x || !w || !out) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
+  if (!ptr_ok(x, 15) || !ptr_ok(w, 15) || !ptr_ok(out, 15) || !ptr_ok(residual, 15) || !ptr_ok(norm_weight, 15) ||
+      !ptr_ok(bias, 7))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
+  TsParams p{};
+  p.x = static_cast<const bf16_t*>(x);
+  p.norm_w = static_cast<const bf16_t*>(norm_weight);
+  p.w1 = static_cast<const bf16_t*>(w);
+  p.b1 = static_cast<const bf16_t*>(bias);
+  p.residual = static_cast<const bf16_t*>(residual);
+  p.out = static_cast<bf16_t*>(out);
+  p.M = M;
+  p.ldx = ldx;
+  p.ldr = ldr;
+  p.ldo = ldo;
+  p.N = N;
+  p.eps = eps;
+  hipStream_t s = as_stream(stream);
+  const int tt = ts_token_tiles();
+  const int threads = kTokPerWg / (32 * tt) * kWave;
+  if (K == 256) {
+    const size_t lds = 2 * (2 * 16) * kFrag;
+    return tt == 1 ? launch_ts(norm_linear_kernel<256, 1>, p, threads, lds, s, name)
+                   : launch_ts(norm_linear_kernel<256, 2>, p, threads, lds, s, name);
+  }
+  const size_t lds = 2 * (2 * 8) * kFrag;
+  return tt == 1 ? launch_ts(norm_linear_kernel<128, 1>, p, threads, lds, s, name)
+                 : launch_ts(norm_linear_kernel<128, 2>, p, threads, lds, s, name);
+}

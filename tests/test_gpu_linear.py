@@ -138,3 +138,63 @@ def test_linear_fp8_epilogues(device):
         xa = amax(x2.to(device))
         got = linear_fp8(x2.to(device), wq, xa, wa, b2.to(device), residual=res.to(device))
     assert _rel_err(got.cpu(), expected) <= 5e-2
+
+
+# ---- token-stationary fused kernels --------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("m,d,f", [(1, 256, 32), (300, 256, 1024), (64, 128, 64), (1000, 256, 96), (257, 128, 256)])
+@pytest.mark.parametrize("gate_first", [True, False])
+def test_fused_swiglu_ffn(device, m, d, f, gate_first):
+    """RMSNorm -> up -> SiLU-gate -> down -> + residual in one kernel against the oracle's pieces evaluated in fp32."""
+    from taac_2026_amd.api import swiglu_ffn
+
+    g = torch.Generator().manual_seed(m + d + f)
+    x = torch.randn(m, d, generator=g).to(torch.bfloat16)
+    nw = (1 + 0.1 * torch.randn(d, generator=g)).to(torch.bfloat16)
+    wu = (torch.randn(2 * f, d, generator=g) * (2.0 / (d + 2 * f)) ** 0.5).to(torch.bfloat16)
+    bu = (0.1 * torch.randn(2 * f, generator=g)).to(torch.bfloat16)
+    wd = (torch.randn(d, f, generator=g) * (2.0 / (d + f)) ** 0.5).to(torch.bfloat16)
+    bd = (0.1 * torch.randn(d, generator=g)).to(torch.bfloat16)
+    h = oracle.rms_norm_fp32(x, nw)
+    expected = x.float() + oracle.swiglu_ffn(h.float(), wu.float(), bu.float(), wd.float(), bd.float(), gate_first=gate_first)
+    with torch.no_grad():
+        got = swiglu_ffn(x.to(device), wu.to(device), bu.to(device), wd.to(device), bd.to(device), residual=x.to(device),
+                         norm_weight=nw.to(device), gate_first=gate_first)
+        plain = swiglu_ffn(x.to(device), wu.to(device), None, wd.to(device), None)
+    torch.testing.assert_close(got.cpu().float(), expected, **BF16_TOL)
+    torch.testing.assert_close(plain.cpu().float(), oracle.swiglu_ffn(x.float(), wu.float(), None, wd.float(), None), **BF16_TOL)
+    # the reference's bf16 evaluation of the same expression stays inside the same tolerance
+    ref_bf16 = x + oracle.swiglu_ffn(oracle.rms_norm(x, nw), wu, bu, wd, bd, gate_first=gate_first)
+    torch.testing.assert_close(got.cpu().float(), ref_bf16.float(), rtol=4e-2, atol=4e-2)
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 256, 64), (300, 256, 768), (64, 128, 256), (1000, 256, 256), (513, 128, 768)])
+def test_fused_norm_linear(device, m, k, n):
+    from taac_2026_amd.api import norm_linear
+
+    x, w, b = _draw(m, n, k, seed=m + n)
+    g = torch.Generator().manual_seed(7)
+    nw = (1 + 0.1 * torch.randn(k, generator=g)).to(torch.bfloat16)
+    res = torch.randn(m, n, generator=g).to(torch.bfloat16)
+    expected = res.float() + F.linear(oracle.rms_norm_fp32(x, nw).float(), w.float(), b.float())
+    with torch.no_grad():
+        got = norm_linear(x.to(device), w.to(device), b.to(device), norm_weight=nw.to(device), residual=res.to(device))
+        plain = norm_linear(x.to(device), w.to(device))
+    torch.testing.assert_close(got.cpu().float(), expected, **BF16_TOL)
+    torch.testing.assert_close(plain.cpu().float(), F.linear(x.float(), w.float()), **BF16_TOL)
+
+
+def test_fused_paths_fall_back_for_other_widths(device):
+    from taac_2026_amd.api import norm_linear, swiglu_ffn
+
+    x, w, b = _draw(100, 72, 96, seed=3)  # K = 96, N = 72: not a token-stationary shape
+    with torch.no_grad():
+        got = norm_linear(x.to(device), w.to(device), b.to(device))
+    torch.testing.assert_close(got.cpu().float(), F.linear(x.float(), w.float(), b.float()), **BF16_TOL)
+    _, wu, _ = _draw(1, 2 * 40, 96, seed=4)
+    _, wd, _ = _draw(1, 96, 40, seed=5)
+    with torch.no_grad():
+        got = swiglu_ffn(x.to(device), wu.to(device), None, wd.to(device), None, residual=x.to(device))
+    expected = x.float() + oracle.swiglu_ffn(x.float(), wu.float(), None, wd.float(), None)
+    torch.testing.assert_close(got.cpu().float(), expected, **BF16_TOL)
