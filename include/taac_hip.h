@@ -107,25 +107,40 @@ int taac_linear_bf16(const void* a, int64_t lda, const void* w, const void* bias
  *   out = residual + down( silu(g) * u ),   g, u = chunk2( up( norm_weight ? rmsnorm(x, norm_weight, eps) : x ) )
  * x: [M, D] bf16 (row stride ldx); w_up: [2F, D]; b_up: [2F] or NULL; w_down: [D, F]; b_down: [D] or NULL;
  * residual: [M, D] (row stride ldr) or NULL; out: [M, D] (row stride ldo), may alias residual and x.
+ * packed_weights: NULL, or the blob written by taac_ffn_pack_weights for the same (w_up, w_down); when given,
+ * w_up / w_down are not read (they may be NULL) and weight staging reads contiguous memory.
  * D must be 128 or 256, F a multiple of 32. The [M, 2F] projection and the [M, F] gated hidden state are never
  * written to memory. gate_first as in taac_linear_bf16.
  * Replaces: ffn_norm + SwiGLUFeedForward.forward + residual add of UnifiedInteractionBlock.forward
  * (experiments/symbiosis/backbone.py:19-21, 66-67).
  */
 int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w_up,
-                        const void* b_up, const void* w_down, const void* b_down, const void* residual, int64_t ldr,
-                        void* out, int64_t ldo, int64_t M, int32_t D, int32_t F, int gate_first, void* stream);
+                        const void* b_up, const void* w_down, const void* b_down, const void* packed_weights,
+                        const void* residual, int64_t ldr, void* out, int64_t ldo, int64_t M, int32_t D, int32_t F,
+                        int gate_first, void* stream);
 
 /*
  * Fused [RMSNorm ->] dense layer [-> + residual] with the token rows held in registers:
  *   out = (residual ? residual : 0) + (norm_weight ? rmsnorm(x, norm_weight, eps) : x) @ w^T + bias
- * x: [M, K] bf16; w: [N, K]; bias: [N] or NULL; residual / out: [M, N]. K must be 128 or 256, N a multiple of 64.
+ * x: [M, K] bf16; w: [N, K]; bias: [N] or NULL; residual / out: [M, N]; packed_weights: NULL or the blob written by
+ * taac_linear_pack_weights for w. K must be 128 or 256, N a multiple of 64.
  * Replaces: attn_norm + the qkv projection, and the out projection + residual add, of UnifiedInteractionBlock /
  * UnifiedSelfAttention (experiments/symbiosis/backbone.py:34-35, 47, 64-65).
  */
 int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
-                         const void* bias, const void* residual, int64_t ldr, void* out, int64_t ldo, int64_t M,
-                         int32_t N, int32_t K, void* stream);
+                         const void* bias, const void* packed_weights, const void* residual, int64_t ldr, void* out,
+                         int64_t ldo, int64_t M, int32_t N, int32_t K, void* stream);
+
+/*
+ * Weight packing for the two fused kernels above: copies the weights into MFMA-fragment order (the order in which
+ * the kernels stage them into LDS). Pack once per weight set; the blob has the size of the weights themselves.
+ * taac_*_packed_bytes return the blob size, or -1 for shapes the fused kernels do not take.
+ * No counterpart in the reference (its dense layers are library GEMMs on nn.Linear weights).
+ */
+int64_t taac_ffn_packed_bytes(int32_t D, int32_t F);
+int taac_ffn_pack_weights(const void* w_up, const void* w_down, void* packed, int32_t D, int32_t F, void* stream);
+int64_t taac_linear_packed_bytes(int32_t N, int32_t K);
+int taac_linear_pack_weights(const void* w, void* packed, int32_t N, int32_t K, void* stream);
 
 /*
  * Per-tensor absolute maximum, for the FP8 scale (scale = amax / 448). Writes max(|x|) over n elements to
@@ -180,8 +195,9 @@ typedef struct taac_block_weights {
   const void* down_bias;        /* [D]                                   */
 } taac_block_weights;
 
-/* Bytes of workspace taac_backbone_fwd needs for the given shape (device memory, 256-byte aligned). */
-int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D, int32_t F);
+/* Bytes of workspace taac_backbone_fwd needs for the given shape (device memory, 256-byte aligned): activations
+ * plus, for the fused path, one fragment-ordered copy of every block's weights (repacked on each call). */
+int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D, int32_t F, int32_t n_blocks);
 
 /*
  * Forward of n_blocks pre-norm blocks plus the pCVR readout:

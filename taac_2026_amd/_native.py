@@ -73,14 +73,18 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "taac_swiglu_ffn_fwd": (
         c_int,
-        [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
-         c_int64, c_int64, c_int32, c_int32, c_int, c_void_p],
+        [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+         c_void_p, c_int64, c_int64, c_int32, c_int32, c_int, c_void_p],
     ),
     "taac_norm_linear_fwd": (
         c_int,
-        [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int64,
-         c_int32, c_int32, c_void_p],
+        [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
+         c_int64, c_int32, c_int32, c_void_p],
     ),
+    "taac_ffn_packed_bytes": (c_int64, [c_int32, c_int32]),
+    "taac_ffn_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
+    "taac_linear_packed_bytes": (c_int64, [c_int32, c_int32]),
+    "taac_linear_pack_weights": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
     "taac_amax": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p]),
     "taac_quantize_fp8": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p]),
     "taac_linear_fp8": (
@@ -92,7 +96,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p],
     ),
-    "taac_backbone_workspace_bytes": (c_int64, [c_int32, c_int32, c_int32, c_int32]),
+    "taac_backbone_workspace_bytes": (c_int64, [c_int32, c_int32, c_int32, c_int32, c_int32]),
     "taac_backbone_fwd": (
         c_int,
         [c_void_p, c_void_p, ctypes.POINTER(BlockWeights), c_int32, c_void_p, c_void_p, c_int32, c_int32, c_int32,

@@ -9,6 +9,8 @@ Weights use the torch ``nn.Linear`` layout ``[out_features, in_features]``.
 
 from __future__ import annotations
 
+import weakref
+
 import torch
 
 from taac_2026_amd import _native
@@ -106,6 +108,69 @@ def _fused_width(d: int) -> bool:
     return d in (128, 256)
 
 
+class _PackedWeightCache:
+    """Fragment-ordered copies of weight tensors for the token-stationary kernels, keyed by tensor identity and
+    version counter so that an in-place update of a weight is repacked. Bounded; oldest entries are dropped."""
+
+    def __init__(self, capacity: int = 128) -> None:
+        self._entries: dict[tuple, tuple[tuple, torch.Tensor]] = {}
+        self._capacity = capacity
+
+    def get(self, tensors: tuple[torch.Tensor, ...], pack) -> torch.Tensor:
+        key = tuple(id(t) for t in tensors)
+        stamp = tuple((weakref.ref(t), t._version, t.data_ptr()) for t in tensors)
+        hit = self._entries.get(key)
+        if hit is not None:
+            old_stamp, packed = hit
+            if all(o[0]() is t and o[1] == t._version and o[2] == t.data_ptr() for o, t in zip(old_stamp, tensors)):
+                return packed
+        packed = pack()
+        if len(self._entries) >= self._capacity:
+            self._entries.pop(next(iter(self._entries)))
+        self._entries[key] = (stamp, packed)
+        return packed
+
+    def clear(self) -> None:
+        self._entries.clear()
+
+
+_packed_cache = _PackedWeightCache()
+
+
+def clear_packed_weight_cache() -> None:
+    _packed_cache.clear()
+
+
+def pack_ffn_weights(up_weight: torch.Tensor, down_weight: torch.Tensor) -> torch.Tensor:
+    """Fragment-ordered blob of ``(up_weight [2F, D], down_weight [D, F])`` for ``swiglu_ffn`` (uint8 tensor)."""
+    library = _native.load_library()
+    d_model, hidden = down_weight.shape
+    nbytes = library.taac_ffn_packed_bytes(d_model, hidden)
+    if nbytes < 0:
+        raise RuntimeError(f"pack_ffn_weights: unsupported shape D={d_model}, F={hidden}")
+    up_weight, down_weight = up_weight.contiguous(), down_weight.contiguous()
+    packed = torch.empty(nbytes, dtype=torch.uint8, device=up_weight.device)
+    status = library.taac_ffn_pack_weights(up_weight.data_ptr(), down_weight.data_ptr(), packed.data_ptr(), d_model,
+                                           hidden, _native.current_stream(up_weight.device))
+    _native.check(status, "pack_ffn_weights")
+    return packed
+
+
+def pack_linear_weight(weight: torch.Tensor) -> torch.Tensor:
+    """Fragment-ordered blob of ``weight [N, K]`` for ``norm_linear`` (uint8 tensor)."""
+    library = _native.load_library()
+    out_features, in_features = weight.shape
+    nbytes = library.taac_linear_packed_bytes(out_features, in_features)
+    if nbytes < 0:
+        raise RuntimeError(f"pack_linear_weight: unsupported shape N={out_features}, K={in_features}")
+    weight = weight.contiguous()
+    packed = torch.empty(nbytes, dtype=torch.uint8, device=weight.device)
+    status = library.taac_linear_pack_weights(weight.data_ptr(), packed.data_ptr(), out_features, in_features,
+                                              _native.current_stream(weight.device))
+    _native.check(status, "pack_linear_weight")
+    return packed
+
+
 def swiglu_ffn(
     x: torch.Tensor,
     up_weight: torch.Tensor,
@@ -145,7 +210,7 @@ def swiglu_ffn(
         gated = swiglu_linear(h, up_weight, up_bias, gate_first=gate_first)
         res_rows = residual.reshape(-1, d_model) if residual is not None else None
         return linear(gated, down_weight, down_bias, residual=res_rows).reshape(shape)
-    up_weight, down_weight = up_weight.contiguous(), down_weight.contiguous()
+    packed = _packed_cache.get((up_weight, down_weight), lambda: pack_ffn_weights(up_weight, down_weight))
     res_rows = None
     if residual is not None:
         res_rows = residual.reshape(-1, d_model)
@@ -154,8 +219,8 @@ def swiglu_ffn(
     out = torch.empty((rows.shape[0], d_model), dtype=x.dtype, device=x.device)
     library = _native.load_library()
     status = library.taac_swiglu_ffn_fwd(
-        rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), up_weight.data_ptr(),
-        _native.ptr(up_bias), down_weight.data_ptr(), _native.ptr(down_bias), _native.ptr(res_rows),
+        rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), None,
+        _native.ptr(up_bias), None, _native.ptr(down_bias), packed.data_ptr(), _native.ptr(res_rows),
         res_rows.stride(0) if res_rows is not None else d_model, out.data_ptr(), d_model, rows.shape[0], d_model,
         hidden, int(bool(gate_first)), _native.current_stream(x.device),
     )
@@ -190,7 +255,7 @@ def norm_linear(
             h = rms_norm(rows, norm_weight, eps)
         res = residual.reshape(-1, out_features) if residual is not None else None
         return linear(h, weight, bias, residual=res).reshape(*shape[:-1], out_features)
-    weight = weight.contiguous()
+    packed = _packed_cache.get((weight,), lambda: pack_linear_weight(weight))
     res_rows = None
     if residual is not None:
         if residual.shape != (*shape[:-1], out_features):
@@ -201,8 +266,8 @@ def norm_linear(
     out = torch.empty((rows.shape[0], out_features), dtype=x.dtype, device=x.device)
     library = _native.load_library()
     status = library.taac_norm_linear_fwd(
-        rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), weight.data_ptr(), _native.ptr(bias),
-        _native.ptr(res_rows), res_rows.stride(0) if res_rows is not None else out_features, out.data_ptr(),
+        rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), None, _native.ptr(bias),
+        packed.data_ptr(), _native.ptr(res_rows), res_rows.stride(0) if res_rows is not None else out_features, out.data_ptr(),
         out_features, rows.shape[0], out_features, in_features, _native.current_stream(x.device),
     )
     _native.check(status, "norm_linear")
@@ -296,9 +361,12 @@ def linear_fp8(
 __all__ = [
     "FP8_MAX",
     "amax",
+    "clear_packed_weight_cache",
     "linear",
     "linear_fp8",
     "norm_linear",
+    "pack_ffn_weights",
+    "pack_linear_weight",
     "quantize_fp8",
     "swiglu_ffn",
     "swiglu_linear",

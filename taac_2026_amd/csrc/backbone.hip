@@ -79,12 +79,25 @@ extern "C" int taac_masked_mean_head(const void* x, const int32_t* lengths, cons
   return check_launch(name);
 }
 
-extern "C" int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D, int32_t F) {
+namespace taac {
+namespace {
+// Fused (token-stationary) path: model widths 128 / 256, hidden size a multiple of 32.
+inline bool fused_shape(int32_t D, int32_t F) { return (D == 128 || D == 256) && F % 32 == 0; }
+// Fragment-ordered weights of one block: qkv, out, feed-forward.
+inline int64_t packed_block_bytes(int32_t D, int32_t F) {
+  return align256(static_cast<int64_t>(3) * D * D * 2) + align256(static_cast<int64_t>(D) * D * 2) +
+         align256(static_cast<int64_t>(3) * D * F * 2);
+}
+}  // namespace
+}  // namespace taac
+
+extern "C" int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D, int32_t F, int32_t n_blocks) {
   using namespace taac;
-  if (B < 0 || T < 0 || D <= 0 || F <= 0) return -1;
+  if (B < 0 || T < 0 || D <= 0 || F <= 0 || n_blocks < 0) return -1;
   const int64_t M = static_cast<int64_t>(B) * T;
-  // x, h (shared with the attention output), qkv, gated hidden
-  return align256(M * D * 2) * 2 + align256(M * 3 * D * 2) + align256(M * F * 2);
+  // x, h (shared with the attention output), qkv, then either the packed weights or the gated hidden state
+  const int64_t acts = align256(M * D * 2) * 2 + align256(M * 3 * D * 2);
+  return acts + (fused_shape(D, F) ? n_blocks * packed_block_bytes(D, F) : align256(M * F * 2));
 }
 
 extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, const taac_block_weights* blocks,
@@ -102,7 +115,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
   if (B == 0 || T == 0) return TAAC_OK;
   if (!emb || !key_lengths || !p || !w_head || (n_blocks > 0 && !blocks))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
-  const int64_t need = taac_backbone_workspace_bytes(B, T, D, F);
+  const int64_t need = taac_backbone_workspace_bytes(B, T, D, F, n_blocks);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: workspace must be 256-byte aligned and hold %lld bytes", name,
                      (long long)need);
@@ -115,7 +128,9 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
   ws += align256(M * D * 2);
   bf16_t* qkv = reinterpret_cast<bf16_t*>(ws);
   ws += align256(M * 3 * D * 2);
-  bf16_t* g = reinterpret_cast<bf16_t*>(ws);
+  bf16_t* g = reinterpret_cast<bf16_t*>(ws);  // unfused path: gated hidden state; fused path: packed weights
+  char* packed = ws;
+  const bool fused = fused_shape(D, F);
 
   const int dh = D / heads;
   const int64_t qkv_strides[4] = {static_cast<int64_t>(T) * 3 * D, dh, 3 * static_cast<int64_t>(D), 1};
@@ -129,11 +144,17 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
       return set_error(TAAC_ERR_INVALID_VALUE, "%s: block %d has a null weight", name, i);
     const bool last = (i == n_blocks - 1);
     bf16_t* x_out = (last && hidden_out != nullptr) ? static_cast<bf16_t*>(hidden_out) : x;
-    const bool fused = (D == 128 || D == 256) && F % 32 == 0;  // token-stationary kernels: norms and residuals fused
+    // Fused path: token-stationary kernels with norms and residuals fused, weights repacked into fragment order.
+    char* pk_qkv = packed + static_cast<int64_t>(i) * packed_block_bytes(D, F);
+    char* pk_out = pk_qkv + align256(static_cast<int64_t>(3) * D * D * 2);
+    char* pk_ffn = pk_out + align256(static_cast<int64_t>(D) * D * 2);
     // attention half
     if (fused) {
-      if ((rc = taac_norm_linear_fwd(cur, D, w.attn_norm_weight, eps, w.qkv_weight, w.qkv_bias, nullptr, 0, qkv, 3 * D,
-                                     M, 3 * D, D, stream)) != TAAC_OK)
+      if ((rc = taac_linear_pack_weights(w.qkv_weight, pk_qkv, 3 * D, D, stream)) != TAAC_OK) return rc;
+      if ((rc = taac_linear_pack_weights(w.out_weight, pk_out, D, D, stream)) != TAAC_OK) return rc;
+      if ((rc = taac_ffn_pack_weights(w.up_weight, w.down_weight, pk_ffn, D, F, stream)) != TAAC_OK) return rc;
+      if ((rc = taac_norm_linear_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, nullptr, 0, qkv,
+                                     3 * D, M, 3 * D, D, stream)) != TAAC_OK)
         return rc;
     } else {
       if ((rc = taac_rmsnorm_fwd(cur, w.attn_norm_weight, h, M, D, eps, TAAC_BF16, stream)) != TAAC_OK) return rc;
@@ -145,11 +166,11 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
                                   qkv_strides, qkv_strides, o_strides, 0, 1, TAAC_BF16, stream)) != TAAC_OK)
       return rc;
     if (fused) {
-      if ((rc = taac_norm_linear_fwd(h, D, nullptr, eps, w.out_weight, w.out_bias, cur, D, x, D, M, D, D, stream)) !=
-          TAAC_OK)
+      if ((rc = taac_norm_linear_fwd(h, D, nullptr, eps, nullptr, w.out_bias, pk_out, cur, D, x, D, M, D, D,
+                                     stream)) != TAAC_OK)
         return rc;
       // feed-forward half: RMSNorm -> up -> SiLU-gate -> down -> + residual in one kernel
-      if ((rc = taac_swiglu_ffn_fwd(x, D, w.ffn_norm_weight, eps, w.up_weight, w.up_bias, w.down_weight, w.down_bias, x,
+      if ((rc = taac_swiglu_ffn_fwd(x, D, w.ffn_norm_weight, eps, nullptr, w.up_bias, nullptr, w.down_bias, pk_ffn, x,
                                     D, x_out, D, M, D, F, 1, stream)) != TAAC_OK)
         return rc;
     } else {

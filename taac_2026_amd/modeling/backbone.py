@@ -200,7 +200,7 @@ class PCVRBackbone(nn.Module):
             slot.up_weight, slot.up_bias = dev(block.up.weight), dev(block.up.bias)
             slot.down_weight, slot.down_bias = dev(block.down.weight), dev(block.down.bias)
 
-        nbytes = library.taac_backbone_workspace_bytes(batch, tokens, self.d_model, self.d_ff)
+        nbytes = library.taac_backbone_workspace_bytes(batch, tokens, self.d_model, self.d_ff, len(self.blocks))
         workspace = self._get_workspace(int(nbytes), emb.device)
         hidden = torch.empty_like(emb) if return_hidden else None
         probabilities = torch.empty(batch, dtype=torch.float32, device=emb.device)

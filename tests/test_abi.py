@@ -64,7 +64,9 @@ def test_host_side_argument_validation_without_gpu():
     assert library.taac_linear_bf16(fake, 16, fake, None, None, fake, 16, 0, 16, 16, _native.EPI_NONE, 1, None) == _native.TAAC_OK
     assert library.taac_linear_bf16(fake, 16, fake, None, None, fake, 16, 4, 16, 16, 7, 1, None) == _native.TAAC_ERR_INVALID_VALUE
     # backbone: workspace too small
-    assert library.taac_backbone_workspace_bytes(2, 16, 32, 64) == 2 * (2 * 16 * 32 * 2) + 2 * 16 * 96 * 2 + 2 * 16 * 64 * 2
+    assert library.taac_backbone_workspace_bytes(2, 16, 32, 64, 1) == 2 * (2 * 16 * 32 * 2) + 2 * 16 * 96 * 2 + 2 * 16 * 64 * 2
+    assert library.taac_ffn_packed_bytes(256, 1024) == 3 * 256 * 1024 * 2 and library.taac_ffn_packed_bytes(96, 64) == -1
+    assert library.taac_linear_packed_bytes(768, 256) == 768 * 256 * 2 and library.taac_linear_packed_bytes(72, 256) == -1
     weights = (_native.BlockWeights * 1)()
     status = library.taac_backbone_fwd(fake, fake, weights, 1, fake, None, 2, 16, 32, 4, 64, 1e-6, fake, 16, None, fake, None)
     assert status == _native.TAAC_ERR_INVALID_VALUE and b"workspace" in library.taac_last_error()
