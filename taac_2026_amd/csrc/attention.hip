@@ -58,6 +58,18 @@ struct Mfma32<f16_t> {
   }
 };
 
+// Combine a value with the one held by lane ^ 32 (both lanes of a pair own the same query column).
+__device__ __forceinline__ float pair_max(float v) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // r[0] = lower half's, r[1] = upper half's
+  return fmaxf(__builtin_bit_cast(float, static_cast<uint32_t>(r[0])), __builtin_bit_cast(float, static_cast<uint32_t>(r[1])));
+}
+__device__ __forceinline__ float pair_sum(float v) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, static_cast<uint32_t>(r[0])) + __builtin_bit_cast(float, static_cast<uint32_t>(r[1]));
+}
+
 template <typename T>
 __device__ __forceinline__ uint32_t pack2(T lo, T hi) {
   return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, lo)) |
@@ -77,8 +89,12 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   constexpr int C8 = DP / 8;       // 128-bit column chunks per row
   constexpr int KSTR = DP + 8;     // LDS row strides in elements (+16 bytes against bank conflicts)
   constexpr int VSTR = kKC + 8;
-  __shared__ __attribute__((aligned(16))) T sK[kKC * KSTR];
-  __shared__ __attribute__((aligned(16))) T sVt[DP * VSTR];
+  constexpr int OROW = DP * 2 + 16;                 // bytes per row of a wavefront's output tile
+  constexpr int KV_BYTES = (kKC * KSTR + DP * VSTR) * 2;
+  constexpr int OT_BYTES = (kThreads / kWave) * 32 * OROW;
+  __shared__ __attribute__((aligned(16))) uint8_t smem[KV_BYTES > OT_BYTES ? KV_BYTES : OT_BYTES];
+  T* sK = reinterpret_cast<T*>(smem);               // [kKC][KSTR]
+  T* sVt = sK + kKC * KSTR;                         // [DP][VSTR]
 
   const uint32_t logical = xcd_remap(blockIdx.x, p.total);
   const int qc = static_cast<int>(logical % p.nqc);
@@ -146,6 +162,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
     const int wlim = q_begin + wave * 32 + 32;
     wave_kv_end = wave_kv_end < wlim ? wave_kv_end : wlim;
   }
+  // A wavefront whose 32 query rows all lie in the padding (or beyond Tq) only helps staging; its output is zeros.
+  if (q_begin + wave * 32 >= q_valid) wave_kv_end = 0;
 
   for (int kc0 = 0; kc0 < kv_end; kc0 += kKC) {
     if (kc0 > 0) __syncthreads();
@@ -203,7 +221,7 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
       float mx = sacc[0];
 #pragma unroll
       for (int j = 1; j < 16; ++j) mx = fmaxf(mx, sacc[j]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      mx = pair_max(mx);
       const float m_new = fmaxf(m_run, mx);
       const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
       const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
@@ -215,7 +233,7 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
         pr[j] = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, mc));
         rs += pr[j];
       }
-      rs += __shfl_xor(rs, 32, kWave);
+      rs = pair_sum(rs);
       l_run = l_run * alpha + rs;
       m_run = m_new;
       vec_t pb[2];
@@ -225,10 +243,13 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
         pb[1][e] = static_cast<T>(pr[8 + e]);
       }
       // ---- O^T += V^T P^T --------------------------------------------------------------------------------
+      const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0;  // wavefront-uniform
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
+        if (rescale) {
 #pragma unroll
-        for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;
+          for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;
+        }
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
           const vec_t a =
@@ -239,24 +260,30 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
     }
   }
 
-  // ---- finalise: O / l, zero rows in the padding, store 4 consecutive features per register group -------------
+  // ---- finalise: O / l (0 for rows in the padding), transpose through a wavefront-private LDS tile, 16-byte stores --
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
   const float fin = (qi < q_valid) ? inv : 0.f;
-  if (qi < p.Tq) {
-    T* orow = ob + qi * p.os[2];
+  __syncthreads();  // every wavefront is done with sK / sVt: the buffer now holds the output tiles
+  uint8_t* tile = smem + wave * (32 * OROW);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
+  for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
-      for (int jq = 0; jq < 4; ++jq) {
-        const int col = mb * 32 + jq * 8 + hh * 4;
-        if (col < p.d) {
-          vec4_t ov;
+    for (int jq = 0; jq < 4; ++jq) {
+      vec4_t ov;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) ov[e] = static_cast<T>(oacc[mb][jq * 4 + e] * fin);
-          *reinterpret_cast<vec4_t*>(orow + col) = ov;
-        }
-      }
+      for (int e = 0; e < 4; ++e) ov[e] = static_cast<T>(oacc[mb][jq * 4 + e] * fin);
+      *reinterpret_cast<vec4_t*>(tile + l32 * OROW + (mb * 32 + jq * 8 + hh * 4) * 2) = ov;
     }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  constexpr int RPP = kWave / C8;  // rows per pass: C8 lanes cover one row
+  const int c8 = lane % C8;
+#pragma unroll
+  for (int pass = 0; pass < 32 / RPP; ++pass) {
+    const int row = pass * RPP + lane / C8;
+    const int q_row = q_begin + wave * 32 + row;
+    const vec_t v = *reinterpret_cast<const vec_t*>(tile + row * OROW + c8 * 16);
+    if (q_row < p.Tq && c8 * 8 < p.d) *reinterpret_cast<vec_t*>(ob + q_row * p.os[2] + c8 * 8) = v;
   }
 }
 

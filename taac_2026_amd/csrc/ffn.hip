@@ -29,7 +29,6 @@
 namespace taac {
 namespace {
 
-constexpr int kTokPerWg = 256;
 constexpr int kFrag = 1024;  // bytes of one 32 x 16 bf16 MFMA operand fragment
 constexpr int kNC = 64;      // output features per chunk of the plain linear kernel
 constexpr int kHU = 16;      // hidden units per FFN chunk
@@ -228,13 +227,13 @@ __device__ __forceinline__ void load_residual(const bf16_t* residual, int64_t ld
 // the down projection. Two chunks are staged and consumed per barrier.
 // LDS: [2 weight buffers][b_up (2F) | b_down (D)]; after the main loop the weight buffers hold the epilogue tiles.
 // ------------------------------------------------------------------------------------------------------------------
-template <int D, int TT>
-__global__ __launch_bounds__(kTokPerWg / (32 * TT) * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_kernel(const TsParams p) {
-  constexpr int NWAVES = kTokPerWg / (32 * TT);  // 4 wavefronts of 64 tokens, or 8 of 32
+template <int D, int TT, int NWAVES, int CPB>
+__global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_kernel(const TsParams p) {
+  constexpr int kTokPerWg = NWAVES * 32 * TT;  // TT token tiles of 32 per wavefront
   constexpr int KS = D / 16;             // k-steps of the up projection = up fragments per chunk
   constexpr int MB = D / 32;             // 32-feature row blocks of the down projection = down fragments per chunk
   constexpr int CFRAG = KS + MB;         // fragments per chunk
-  constexpr int NFRAG = kCPB * CFRAG;    // fragments per barrier step
+  constexpr int NFRAG = CPB * CFRAG;     // fragments per barrier step
   constexpr int FPW = NFRAG / NWAVES;    // fragments staged per wavefront
   static_assert(NFRAG % NWAVES == 0, "fragments must divide over the wavefronts");
   static_assert(2 * NFRAG * kFrag >= NWAVES * kStageWave, "epilogue tiles must fit in the weight buffers");
@@ -248,7 +247,7 @@ __global__ __launch_bounds__(kTokPerWg / (32 * TT) * kWave, TT == 1 ? 2 : 1) voi
   const int hh = lane / 32;
   const int64_t tok0 = static_cast<int64_t>(blockIdx.x) * kTokPerWg + wave * (32 * TT);
   const int F = p.F;
-  const int nsteps = F / (kHU * kCPB);
+  const int nsteps = F / (kHU * CPB);
 
   // Source address of a staged fragment = wavefront-uniform base (scalar registers) + a 32-bit per-lane byte offset.
   //   packed:   blob + (step * NFRAG + f) KB + 16 * lane
@@ -277,7 +276,7 @@ __global__ __launch_bounds__(kTokPerWg / (32 * TT) * kWave, TT == 1 ? 2 : 1) voi
       const int f = wave * FPW + i;  // wavefront-uniform
       const int q = f / CFRAG;       // chunk inside the step
       const int r = f % CFRAG;
-      const int64_t unit0 = static_cast<int64_t>(step * kCPB + q) * kHU;
+      const int64_t unit0 = static_cast<int64_t>(step * CPB + q) * kHU;
       if (r < KS)
         lds_dma16(w_up_bytes + (unit0 * D + r * 16) * 2 + up_lane_off, base + i * kFrag);
       else
@@ -307,9 +306,9 @@ __global__ __launch_bounds__(kTokPerWg / (32 * TT) * kWave, TT == 1 ? 2 : 1) voi
     const int buf = step & 1;
     if (step + 1 < nsteps) stage(step + 1, buf ^ 1);
 #pragma unroll
-    for (int q = 0; q < kCPB; ++q) {
+    for (int q = 0; q < CPB; ++q) {
       const uint8_t* wb = smem + buf * (NFRAG * kFrag) + q * (CFRAG * kFrag) + lane * 16;
-      const int unit0 = (step * kCPB + q) * kHU;
+      const int unit0 = (step * CPB + q) * kHU;
       // ---- up projection: rows 0..15 gate, rows 16..31 value, every token tile -------------------------------------
       f32x16 gu[TT];
 #pragma unroll
@@ -386,9 +385,9 @@ __global__ __launch_bounds__(kTokPerWg / (32 * TT) * kWave, TT == 1 ? 2 : 1) voi
 // [RMSNorm ->] linear [-> + residual], K = D, N a multiple of 64
 // LDS: [2 weight buffers of 2*KS fragments][NWAVES epilogue tiles][bias (N)]
 // ------------------------------------------------------------------------------------------------------------------
-template <int D, int TT>
-__global__ __launch_bounds__(kTokPerWg / (32 * TT) * kWave, TT == 1 ? 2 : 1) void norm_linear_kernel(const TsParams p) {
-  constexpr int NWAVES = kTokPerWg / (32 * TT);
+template <int D, int TT, int NWAVES>
+__global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void norm_linear_kernel(const TsParams p) {
+  constexpr int kTokPerWg = NWAVES * 32 * TT;
   constexpr int KS = D / 16;
   constexpr int NFRAG = 2 * KS;    // two 32-feature row blocks per chunk
   constexpr int FPW = NFRAG / NWAVES;
@@ -479,23 +478,28 @@ __global__ __launch_bounds__(kTokPerWg / (32 * TT) * kWave, TT == 1 ? 2 : 1) voi
 // The kernels use more than the default 64 KB of dynamic LDS; the opt-in is idempotent and cheap, so it is simply
 // repeated before every launch (no cached per-process state to go stale across devices).
 template <typename K>
-int launch_ts(K kernel, const TsParams& p, int threads, size_t lds_bytes, hipStream_t s, const char* name) {
+int launch_ts(K kernel, const TsParams& p, int threads, int tokens_per_wg, size_t lds_bytes, hipStream_t s,
+              const char* name) {
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                           static_cast<int>(lds_bytes)) != hipSuccess)
     return set_error(TAAC_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", name, lds_bytes);
-  const int64_t grid = (p.M + kTokPerWg - 1) / kTokPerWg;
+  const int64_t grid = (p.M + tokens_per_wg - 1) / tokens_per_wg;
   if (grid > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many workgroups", name);
   hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(grid)), dim3(threads), lds_bytes, s, p);
   return check_launch(name);
 }
 
-// Token tiles per wavefront: 1 = 8 wavefronts x 32 tokens (two per SIMD), 2 = 4 wavefronts x 64 tokens.
-int ts_token_tiles() {
-  static const int tiles = [] {
-    const char* env = getenv("TAAC_TS_TOKEN_TILES");
-    return (env != nullptr && env[0] == '2') ? 2 : 1;
+// Workgroup shape of the token-stationary kernels (tuning knob, read once from TAAC_TS_CONFIG; default 1, the
+// fastest of the three on MI355X at D = 256):
+//   0 = 4 wavefronts x 32 tokens, one FFN chunk per barrier  -> two workgroups per CU run independently
+//   1 = 8 wavefronts x 32 tokens, two FFN chunks per barrier -> one workgroup per CU, two wavefronts per SIMD
+//   2 = 4 wavefronts x 64 tokens, two FFN chunks per barrier -> one workgroup per CU, one wavefront per SIMD
+int ts_config() {
+  static const int config = [] {
+    const char* env = getenv("TAAC_TS_CONFIG");
+    return (env != nullptr && env[0] >= '0' && env[0] <= '2') ? env[0] - '0' : 1;
   }();
-  return tiles;
+  return config;
 }
 
 bool ptr_ok(const void* p, uintptr_t mask) { return (reinterpret_cast<uintptr_t>(p) & mask) == 0; }
@@ -564,10 +568,8 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
   if (!ptr_ok(x, 15) || !ptr_ok(w_up, 15) || !ptr_ok(w_down, 15) || !ptr_ok(out, 15) || !ptr_ok(residual, 15) ||
       !ptr_ok(norm_weight, 15) || !ptr_ok(b_up, 15) || !ptr_ok(b_down, 15) || !ptr_ok(packed_weights, 15))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
-  const int KS = D / 16, MB = D / 32;
-  const size_t lds = static_cast<size_t>(2 * kCPB * (KS + MB)) * kFrag + static_cast<size_t>(2 * F + D) * 2;
-  if (lds > kMaxLdsBytes)
-    return set_error(TAAC_ERR_UNSUPPORTED, "%s: F=%d needs %zu bytes of LDS (limit %d)", name, F, lds, kMaxLdsBytes);
+  if (static_cast<size_t>(2 * kCPB * (D / 16 + D / 32)) * kFrag + static_cast<size_t>(2 * F + D) * 2 > kMaxLdsBytes)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: F=%d does not fit the LDS (limit %d bytes)", name, F, kMaxLdsBytes);
   TsParams p{};
   p.x = static_cast<const bf16_t*>(x);
   p.norm_w = static_cast<const bf16_t*>(norm_weight);
@@ -586,13 +588,21 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
   p.gate_first = gate_first ? 1 : 0;
   p.packed = packed_weights ? 1 : 0;
   hipStream_t s = as_stream(stream);
-  const int tt = ts_token_tiles();
-  const int threads = kTokPerWg / (32 * tt) * kWave;
-  if (D == 256)
-    return tt == 1 ? launch_ts(swiglu_ffn_kernel<256, 1>, p, threads, lds, s, name)
-                   : launch_ts(swiglu_ffn_kernel<256, 2>, p, threads, lds, s, name);
-  return tt == 1 ? launch_ts(swiglu_ffn_kernel<128, 1>, p, threads, lds, s, name)
-                 : launch_ts(swiglu_ffn_kernel<128, 2>, p, threads, lds, s, name);
+  const int KS = D / 16, MB = D / 32;
+  const size_t bias_bytes = static_cast<size_t>(2 * F + D) * 2;
+#define TAAC_FFN_LAUNCH(DD, TT, NW, CPB)                                                                      \
+  return launch_ts(swiglu_ffn_kernel<DD, TT, NW, CPB>, p, NW * kWave, NW * 32 * TT,                          \
+                   static_cast<size_t>(2 * CPB * (KS + MB)) * kFrag + bias_bytes, s, name)
+  const int cfg = ts_config();
+  if (D == 256) {
+    if (cfg == 0) TAAC_FFN_LAUNCH(256, 1, 4, 1);
+    if (cfg == 1) TAAC_FFN_LAUNCH(256, 1, 8, 2);
+    TAAC_FFN_LAUNCH(256, 2, 4, 2);
+  }
+  if (cfg == 0) TAAC_FFN_LAUNCH(128, 1, 4, 1);
+  if (cfg == 1) TAAC_FFN_LAUNCH(128, 1, 8, 2);
+  TAAC_FFN_LAUNCH(128, 2, 4, 2);
+#undef TAAC_FFN_LAUNCH
 }
 
 extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
@@ -611,12 +621,9 @@ extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm
   if (!ptr_ok(x, 15) || !ptr_ok(w, 15) || !ptr_ok(out, 15) || !ptr_ok(residual, 15) || !ptr_ok(norm_weight, 15) ||
       !ptr_ok(bias, 15) || !ptr_ok(packed_weights, 15))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
-  const int tt = ts_token_tiles();
-  const int nwaves = kTokPerWg / (32 * tt);
-  const size_t lds = static_cast<size_t>(2 * 2 * (K / 16)) * kFrag + static_cast<size_t>(nwaves) * kStageWave +
-                     static_cast<size_t>(N) * 2;
-  if (lds > kMaxLdsBytes)
-    return set_error(TAAC_ERR_UNSUPPORTED, "%s: N=%d needs %zu bytes of LDS (limit %d)", name, N, lds, kMaxLdsBytes);
+  if (static_cast<size_t>(2 * 2 * (K / 16)) * kFrag + 8 * static_cast<size_t>(kStageWave) + static_cast<size_t>(N) * 2 >
+      kMaxLdsBytes)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: N=%d does not fit the LDS (limit %d bytes)", name, N, kMaxLdsBytes);
   TsParams p{};
   p.x = static_cast<const bf16_t*>(x);
   p.norm_w = static_cast<const bf16_t*>(norm_weight);
@@ -632,10 +639,19 @@ extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm
   p.eps = eps;
   p.packed = packed_weights ? 1 : 0;
   hipStream_t s = as_stream(stream);
-  const int threads = nwaves * kWave;
-  if (K == 256)
-    return tt == 1 ? launch_ts(norm_linear_kernel<256, 1>, p, threads, lds, s, name)
-                   : launch_ts(norm_linear_kernel<256, 2>, p, threads, lds, s, name);
-  return tt == 1 ? launch_ts(norm_linear_kernel<128, 1>, p, threads, lds, s, name)
-                 : launch_ts(norm_linear_kernel<128, 2>, p, threads, lds, s, name);
+#define TAAC_LIN_LAUNCH(KK, TT, NW)                                                                            \
+  return launch_ts(norm_linear_kernel<KK, TT, NW>, p, NW * kWave, NW * 32 * TT,                               \
+                   static_cast<size_t>(2 * 2 * (KK / 16)) * kFrag + static_cast<size_t>(NW) * kStageWave +    \
+                       static_cast<size_t>(N) * 2,                                                             \
+                   s, name)
+  const int cfg = ts_config();
+  if (K == 256) {
+    if (cfg == 0) TAAC_LIN_LAUNCH(256, 1, 4);
+    if (cfg == 1) TAAC_LIN_LAUNCH(256, 1, 8);
+    TAAC_LIN_LAUNCH(256, 2, 4);
+  }
+  if (cfg == 0) TAAC_LIN_LAUNCH(128, 1, 4);
+  if (cfg == 1) TAAC_LIN_LAUNCH(128, 1, 8);
+  TAAC_LIN_LAUNCH(128, 2, 4);
+#undef TAAC_LIN_LAUNCH
 }

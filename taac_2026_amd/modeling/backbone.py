@@ -18,7 +18,7 @@ import torch
 import torch.nn as nn
 
 from taac_2026_amd import _native
-from taac_2026_amd.accelerators.linear import linear, swiglu_linear
+from taac_2026_amd.accelerators.linear import norm_linear, swiglu_ffn
 from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference
 from taac_2026_amd.modeling.normalization import RMSNorm
 from taac_2026_amd.modeling.sequence import scaled_dot_product_attention
@@ -31,11 +31,12 @@ def _bf16(parameter: torch.Tensor | None) -> torch.Tensor | None:
 
 
 def _dense(layer: nn.Linear, x: torch.Tensor, *, residual: torch.Tensor | None = None) -> torch.Tensor:
-    return linear(x, _bf16(layer.weight), _bf16(layer.bias), residual=residual)
+    return norm_linear(x, _bf16(layer.weight), _bf16(layer.bias), residual=residual)
 
 
 class SwiGLUFeedForward(nn.Module):
-    """``down(silu(gate) * value)``, ``gate, value = up(x).chunk(2, -1)``; SiLU-gate fused into the up projection."""
+    """``down(silu(gate) * value)``, ``gate, value = up(x).chunk(2, -1)``: one fused kernel for model widths 128 / 256
+    (the projection and the gated hidden state stay in registers), up(+SiLU-gate) and down kernels otherwise."""
 
     def __init__(self, d_model: int, hidden_mult: int, dropout: float = 0.0, *, gate_first: bool = True) -> None:
         super().__init__()
@@ -50,8 +51,8 @@ class SwiGLUFeedForward(nn.Module):
             raise RuntimeError("hip SwiGLUFeedForward is forward-only inference and does not apply dropout")
         output_dtype = tokens.dtype
         x = tokens if tokens.dtype == torch.bfloat16 else tokens.to(torch.bfloat16)
-        hidden = swiglu_linear(x, _bf16(self.up.weight), _bf16(self.up.bias), gate_first=self.gate_first)
-        out = _dense(self.down, hidden, residual=_bf16(residual))
+        out = swiglu_ffn(x, _bf16(self.up.weight), _bf16(self.up.bias), _bf16(self.down.weight), _bf16(self.down.bias),
+                         residual=_bf16(residual), gate_first=self.gate_first)
         return out if out.dtype == output_dtype else out.to(output_dtype)
 
 
