@@ -165,34 +165,59 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   // A wavefront whose 32 query rows all lie in the padding (or beyond Tq) only helps staging; its output is zeros.
   if (q_begin + wave * 32 >= q_valid) wave_kv_end = 0;
 
-  for (int kc0 = 0; kc0 < kv_end; kc0 += kKC) {
-    if (kc0 > 0) __syncthreads();
-    // ---- stage K chunk: sK[key][feature] ------------------------------------------------------------------
-    for (int idx = tid; idx < kKC * C8; idx += kThreads) {
-      const int key = idx / C8;
-      const int c8 = idx % C8;
-      const int kidx = kc0 + key;
-      vec_t val = zero_vec;
-      if (kidx < kv_end && c8 * 8 < p.d) val = *reinterpret_cast<const vec_t*>(kb + kidx * p.ks[2] + c8 * 8);
-      *reinterpret_cast<vec_t*>(&sK[key * KSTR + c8 * 8]) = val;
-    }
-    // ---- stage V chunk transposed and key-permuted: sVt[feature][pos(key)] ---------------------------------
-    for (int idx = tid; idx < (kKC / 2) * C8; idx += kThreads) {
-      const int pair = idx / C8;
-      const int c8 = idx % C8;
-      const int key0 = 2 * pair;
-      const int kidx = kc0 + key0;
-      vec_t v0 = zero_vec, v1 = zero_vec;
-      if (c8 * 8 < p.d) {
-        if (kidx < kv_end) v0 = *reinterpret_cast<const vec_t*>(vb + kidx * p.vs[2] + c8 * 8);
-        if (kidx + 1 < kv_end) v1 = *reinterpret_cast<const vec_t*>(vb + (kidx + 1) * p.vs[2] + c8 * 8);
-      }
-      const int pos = (key0 & ~15) + vt_pos16(key0 & 15);  // even; key0 + 1 lands at pos + 1
+  // K / V staging is split into a register fetch and an LDS commit so that the global loads of chunk c + 1 are in
+  // flight while chunk c is being consumed. Piece idx of a chunk: K -> (key idx / C8, 8 features idx % C8);
+  // V -> (key pair idx / C8, 8 features idx % C8), written transposed and key-permuted as sVt[feature][pos(key)].
+  constexpr int KLD = (kKC * C8 + kThreads - 1) / kThreads;
+  constexpr int VLD = ((kKC / 2) * C8 + kThreads - 1) / kThreads;
+  vec_t kreg[KLD], vreg[VLD][2];
+  auto fetch = [&](int kc0) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        *reinterpret_cast<uint32_t*>(&sVt[(c8 * 8 + i) * VSTR + pos]) = pack2<T>(v0[i], v1[i]);
+    for (int i = 0; i < KLD; ++i) {
+      const int idx = tid + i * kThreads;
+      const int kidx = kc0 + idx / C8;
+      const int c8 = idx % C8;
+      kreg[i] = (idx < kKC * C8 && kidx < kv_end && c8 * 8 < p.d)
+                    ? *reinterpret_cast<const vec_t*>(kb + kidx * p.ks[2] + c8 * 8)
+                    : zero_vec;
     }
+#pragma unroll
+    for (int i = 0; i < VLD; ++i) {
+      const int idx = tid + i * kThreads;
+      const int kidx = kc0 + 2 * (idx / C8);
+      const int c8 = idx % C8;
+      const bool ok = idx < (kKC / 2) * C8 && c8 * 8 < p.d;
+      vreg[i][0] = (ok && kidx < kv_end) ? *reinterpret_cast<const vec_t*>(vb + kidx * p.vs[2] + c8 * 8) : zero_vec;
+      vreg[i][1] =
+          (ok && kidx + 1 < kv_end) ? *reinterpret_cast<const vec_t*>(vb + (kidx + 1) * p.vs[2] + c8 * 8) : zero_vec;
+    }
+  };
+  auto commit = [&]() {
+#pragma unroll
+    for (int i = 0; i < KLD; ++i) {
+      const int idx = tid + i * kThreads;
+      if (idx < kKC * C8) *reinterpret_cast<vec_t*>(&sK[(idx / C8) * KSTR + (idx % C8) * 8]) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VLD; ++i) {
+      const int idx = tid + i * kThreads;
+      if (idx < (kKC / 2) * C8) {
+        const int key0 = 2 * (idx / C8);
+        const int c8 = idx % C8;
+        const int pos = (key0 & ~15) + vt_pos16(key0 & 15);  // even; key0 + 1 lands at pos + 1
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          *reinterpret_cast<uint32_t*>(&sVt[(c8 * 8 + e) * VSTR + pos]) = pack2<T>(vreg[i][0][e], vreg[i][1][e]);
+      }
+    }
+  };
+
+  if (kv_end > 0) fetch(0);
+  for (int kc0 = 0; kc0 < kv_end; kc0 += kKC) {
+    if (kc0 > 0) __syncthreads();  // every wavefront is done reading the previous chunk
+    commit();
     __syncthreads();
+    if (kc0 + kKC < kv_end) fetch(kc0 + kKC);
 
 #pragma unroll
     for (int kt = 0; kt < kKC / 32; ++kt) {
@@ -243,13 +268,12 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
         pb[1][e] = static_cast<T>(pr[8 + e]);
       }
       // ---- O^T += V^T P^T --------------------------------------------------------------------------------
-      const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0;  // wavefront-uniform
+      // The rescale is unconditional on purpose: a wavefront-uniform branch around it placed the accumulator read-back
+      // of the preceding MFMA on a path without the required wait states (wrong values in the last accumulator register).
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        if (rescale) {
 #pragma unroll
-          for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;
-        }
+        for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
           const vec_t a =
