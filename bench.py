@@ -47,6 +47,18 @@ def _event_ms(fn, iters: int, warmup: int) -> float:
     return start.elapsed_time(stop) / iters
 
 
+def _measured_traffic(kernel_name: str) -> int | None:
+    """HBM bytes per launch of ``kernel_name`` as measured with the FETCH_SIZE / WRITE_SIZE counters (scaled by a kernel
+    of known traffic); read from the committed counter summary, None if the kernel is not listed there."""
+    summary = REPO_ROOT / "profiles" / "pmc_traffic_backbone_c4.txt"
+    if not summary.exists():
+        return None
+    for line in summary.read_text().splitlines():
+        if line.startswith(kernel_name + ":") and "traffic_bytes=" in line:
+            return int(line.split("traffic_bytes=")[1].split()[0])
+    return None
+
+
 def _accuracy_gate(model, inputs, device) -> dict:
     """Probabilities of a slice of the batch against the CPU oracle (2e-2 absolute)."""
     from oracle import reference as oracle
@@ -152,6 +164,59 @@ def _operator_figures(device, iters: int) -> dict:
     return figures
 
 
+def _fp8_figures(inputs, device, iters: int) -> dict:
+    """Configuration 5: the block's four dense layers with e4m3 operands (per-tensor scale amax / 448) over all
+    M = B * T tokens, each checked on a slice of rows against the quantize -> matmul -> dequantize emulation."""
+    from oracle import reference as oracle
+    from taac_2026_amd.api import (amax, flash_attention, linear_fp8, norm_linear, quantize_fp8, rms_norm,
+                                   scaled_dot_product_attention, swiglu_linear)
+
+    del flash_attention
+    B, T, D = inputs.emb.shape
+    M, F, H = B * T, inputs.d_ff, inputs.num_heads
+    w = {k: v.to(device) for k, v in inputs.blocks[0].items()}
+    x = inputs.emb.to(device)
+    lengths = inputs.key_lengths.to(device)
+    figures: dict[str, dict] = {}
+    with torch.no_grad():
+        h = rms_norm(x, w["attn_norm.weight"])
+        q, k, v = norm_linear(h, w["qkv.weight"], w["qkv.bias"]).chunk(3, dim=-1)
+        a = scaled_dot_product_attention(q, k, v, num_heads=H, attn_mask=None, dropout_p=0.0, training=False,
+                                         key_lengths=lengths, zero_padded_queries=True)
+        x1 = norm_linear(a, w["out.weight"], w["out.bias"], residual=x)
+        h2 = rms_norm(x1, w["ffn_norm.weight"])
+        g = swiglu_linear(h2, w["up.weight"], w["up.bias"])
+        layers = {
+            "qkv": (h.view(M, D), "qkv", False, None),
+            "out": (a.view(M, D), "out", False, x.view(M, D)),
+            "up_swiglu": (h2.view(M, D), "up", True, None),
+            "down": (g.view(M, F), "down", False, x1.view(M, D)),
+        }
+        total_flops, total_ms = 0.0, 0.0
+        for name, (act, key, swiglu, residual) in layers.items():
+            weight, bias = w[f"{key}.weight"], w[f"{key}.bias"]
+            wq, wa = quantize_fp8(weight)
+            xa = amax(act)
+            run = lambda act=act, wq=wq, xa=xa, wa=wa, bias=bias, residual=residual, swiglu=swiglu: linear_fp8(  # noqa: E731
+                act, wq, xa, wa, bias, residual=residual, swiglu=swiglu)
+            got = run()[:512].cpu().float()
+            expected = oracle.linear_fp8(act[:512].cpu(), weight.cpu(), bias.cpu(),
+                                         residual=None if residual is None else residual[:512].cpu(), swiglu=swiglu,
+                                         x_scale=(xa.cpu() / 448.0), w_scale=(wa.cpu() / 448.0)).float()
+            rel = ((got - expected).abs().max() / expected.abs().max()).item()
+            if rel > 5e-2:
+                raise SystemExit(f"fp8 accuracy gate failed for {name}: relative error {rel}")
+            flops = 2.0 * M * weight.shape[0] * weight.shape[1]
+            ms = _event_ms(run, iters, 3)
+            ms_amax = _event_ms(lambda act=act: amax(act), iters, 3)
+            figures[name] = {"ms": ms, "amax_ms": ms_amax, "tflops": flops / ms / 1e9,
+                             "frac_mfma_fp8": flops / ms / 1e9 / 5000.0, "rel_err": rel}
+            total_flops += flops
+            total_ms += ms + ms_amax
+        figures["block_set"] = {"ms_including_amax": total_ms, "tflops": total_flops / total_ms / 1e9}
+    return figures
+
+
 def _cpu_baseline(inputs, budget_s: float = 20.0) -> dict:
     """The oracle's backbone forward (the reference's torch formulas) on the host cores, on a bounded sample."""
     from oracle import reference as oracle
@@ -238,7 +303,7 @@ def main() -> None:
         "peak": MFMA_BF16_PEAK_TFLOPS if bound == "mfma" else HBM_PEAK_GBS,
         "unit": "TFLOP/s" if bound == "mfma" else "GB/s",
         "frac": dom["frac_mfma"] if bound == "mfma" else dom["frac_hbm"],
-        "traffic": None,
+        "traffic": _measured_traffic(dominant),
         "launch_ms": dom["ms"],
     }
 
@@ -270,6 +335,7 @@ def main() -> None:
     }
     if not args.skip_operators:
         line["operators"] = _operator_figures(device, iters=20)
+        line["fp8_dense_layers"] = _fp8_figures(inputs, device, iters=10)
     if not args.skip_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(inputs)
         line["gpu_over_cpu"] = value / line["cpu_baseline"]["value"]
