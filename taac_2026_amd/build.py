@@ -34,6 +34,12 @@ HIPCC_FLAGS = (
     "-Wno-unused-value",
 )
 
+# Per-source extras. -amdgpu-mfma-vgpr-form: keep MFMA accumulators in ordinary VGPRs where the kernel interleaves
+# MFMAs with VALU work on the same values (softmax), instead of copying them to and from the accumulator registers.
+EXTRA_FLAGS = {
+    "attention.hip": ("-mllvm", "-amdgpu-mfma-vgpr-form=1"),
+}
+
 
 def find_hipcc() -> str:
     candidate = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
@@ -57,7 +63,7 @@ def build_library(*, verbose: bool = False, jobs: int | None = None) -> Path:
     for source in SOURCES:
         obj = BUILD_DIR / (Path(source).stem + ".o")
         objects.append(str(obj))
-        commands.append([hipcc, *HIPCC_FLAGS, "-c", str(CSRC_DIR / source), "-o", str(obj)])
+        commands.append([hipcc, *HIPCC_FLAGS, *EXTRA_FLAGS.get(source, ()), "-c", str(CSRC_DIR / source), "-o", str(obj)])
     workers = jobs or min(len(commands), max(1, (os.cpu_count() or 2) // 2), 8)
     with ThreadPoolExecutor(max_workers=workers) as pool:
         for cmd, _ in zip(commands, pool.map(_run, commands)):
