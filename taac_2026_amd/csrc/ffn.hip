@@ -460,6 +460,9 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void norm_linear_k
         acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, xf[t][ks], acc[1][t], 0, 0, 0);
       }
     }
+    // Wait for the next chunk's weights (and this chunk's residual pieces) BEFORE the output stores are issued: the
+    // memory counter also counts stores, and waiting on it after them would expose the full write latency per chunk.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
       tile_to_lds(tile, acc[0][t], acc[1][t], bias_lds + c * kNC, l32, hh);
@@ -470,7 +473,6 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void norm_linear_k
         tile_to_global<false>(tile, p.out, p.ldo, tok0 + t * 32, p.M, c * kNC, res[t], lane);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
 }
