@@ -134,11 +134,13 @@ int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, fl
 /*
  * Weight packing for the two fused kernels above: copies the weights into MFMA-fragment order (the order in which
  * the kernels stage them into LDS). Pack once per weight set; the blob has the size of the weights themselves.
+ * The FFN blob depends on gate_first (which half of w_up is gated): taac_swiglu_ffn_fwd must be given the same value.
  * taac_*_packed_bytes return the blob size, or -1 for shapes the fused kernels do not take.
  * No counterpart in the reference (its dense layers are library GEMMs on nn.Linear weights).
  */
 int64_t taac_ffn_packed_bytes(int32_t D, int32_t F);
-int taac_ffn_pack_weights(const void* w_up, const void* w_down, void* packed, int32_t D, int32_t F, void* stream);
+int taac_ffn_pack_weights(const void* w_up, const void* w_down, void* packed, int32_t D, int32_t F, int gate_first,
+                          void* stream);
 int64_t taac_linear_packed_bytes(int32_t N, int32_t K);
 int taac_linear_pack_weights(const void* w, void* packed, int32_t N, int32_t K, void* stream);
 

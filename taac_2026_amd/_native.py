@@ -82,7 +82,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
          c_int64, c_int32, c_int32, c_void_p],
     ),
     "taac_ffn_packed_bytes": (c_int64, [c_int32, c_int32]),
-    "taac_ffn_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
+    "taac_ffn_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int, c_void_p]),
     "taac_linear_packed_bytes": (c_int64, [c_int32, c_int32]),
     "taac_linear_pack_weights": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
     "taac_amax": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p]),

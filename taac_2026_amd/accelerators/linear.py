@@ -116,8 +116,8 @@ class _PackedWeightCache:
         self._entries: dict[tuple, tuple[tuple, torch.Tensor]] = {}
         self._capacity = capacity
 
-    def get(self, tensors: tuple[torch.Tensor, ...], pack) -> torch.Tensor:
-        key = tuple(id(t) for t in tensors)
+    def get(self, tensors: tuple[torch.Tensor, ...], pack, variant: int = 0) -> torch.Tensor:
+        key = tuple(id(t) for t in tensors) + (variant,)
         stamp = tuple((weakref.ref(t), t._version, t.data_ptr()) for t in tensors)
         hit = self._entries.get(key)
         if hit is not None:
@@ -141,8 +141,11 @@ def clear_packed_weight_cache() -> None:
     _packed_cache.clear()
 
 
-def pack_ffn_weights(up_weight: torch.Tensor, down_weight: torch.Tensor) -> torch.Tensor:
-    """Fragment-ordered blob of ``(up_weight [2F, D], down_weight [D, F])`` for ``swiglu_ffn`` (uint8 tensor)."""
+def pack_ffn_weights(up_weight: torch.Tensor, down_weight: torch.Tensor, *, gate_first: bool = True) -> torch.Tensor:
+    """Fragment-ordered blob of ``(up_weight [2F, D], down_weight [D, F])`` for ``swiglu_ffn`` (uint8 tensor).
+
+    The blob depends on ``gate_first`` (which half of ``up_weight`` goes through SiLU): pass the same value to
+    ``swiglu_ffn``."""
     library = _native.load_library()
     d_model, hidden = down_weight.shape
     nbytes = library.taac_ffn_packed_bytes(d_model, hidden)
@@ -151,7 +154,8 @@ def pack_ffn_weights(up_weight: torch.Tensor, down_weight: torch.Tensor) -> torc
     up_weight, down_weight = up_weight.contiguous(), down_weight.contiguous()
     packed = torch.empty(nbytes, dtype=torch.uint8, device=up_weight.device)
     status = library.taac_ffn_pack_weights(up_weight.data_ptr(), down_weight.data_ptr(), packed.data_ptr(), d_model,
-                                           hidden, _native.current_stream(up_weight.device))
+                                           hidden, int(bool(gate_first)),
+                                           _native.current_stream(up_weight.device))
     _native.check(status, "pack_ffn_weights")
     return packed
 
@@ -210,7 +214,9 @@ def swiglu_ffn(
         gated = swiglu_linear(h, up_weight, up_bias, gate_first=gate_first)
         res_rows = residual.reshape(-1, d_model) if residual is not None else None
         return linear(gated, down_weight, down_bias, residual=res_rows).reshape(shape)
-    packed = _packed_cache.get((up_weight, down_weight), lambda: pack_ffn_weights(up_weight, down_weight))
+    packed = _packed_cache.get((up_weight, down_weight),
+                               lambda: pack_ffn_weights(up_weight, down_weight, gate_first=gate_first),
+                               variant=int(bool(gate_first)))
     res_rows = None
     if residual is not None:
         res_rows = residual.reshape(-1, d_model)

@@ -152,7 +152,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
     if (fused) {
       if ((rc = taac_linear_pack_weights(w.qkv_weight, pk_qkv, 3 * D, D, stream)) != TAAC_OK) return rc;
       if ((rc = taac_linear_pack_weights(w.out_weight, pk_out, D, D, stream)) != TAAC_OK) return rc;
-      if ((rc = taac_ffn_pack_weights(w.up_weight, w.down_weight, pk_ffn, D, F, stream)) != TAAC_OK) return rc;
+      if ((rc = taac_ffn_pack_weights(w.up_weight, w.down_weight, pk_ffn, D, F, 1, stream)) != TAAC_OK) return rc;
       if ((rc = taac_norm_linear_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, nullptr, 0, qkv,
                                      3 * D, M, 3 * D, D, stream)) != TAAC_OK)
         return rc;

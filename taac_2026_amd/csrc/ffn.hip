@@ -23,6 +23,8 @@
 // segment; the residual is read the same way and added after the rounding of the layer output, which is the order
 // of roundings of the reference's bf16 evaluation (linear output rounded, then the residual add rounded).
 #include <cstdlib>
+#include <type_traits>
+#include <utility>
 
 #include "common.h"
 
@@ -51,6 +53,7 @@ struct TsParams {
   float eps;
   int32_t gate_first;
   int32_t packed;           // weights are in fragment order
+  int32_t stagger;          // linear: wavefront groups may change token tiles out of phase (x does not alias out)
 };
 
 __device__ __forceinline__ float silu_f(float v) {
@@ -72,7 +75,7 @@ __host__ __device__ __forceinline__ int up_unit_of_slot(int m16) {
 // FFN blob: step s (32 hidden units) holds, for chunk q = 0, 1: KS up fragments (k-step r) then MB down fragments
 // (row block r - KS); exactly the image one barrier step needs in LDS. A fragment is 64 lanes x 16 bytes.
 __global__ void ffn_pack_kernel(const bf16_t* __restrict__ w_up, const bf16_t* __restrict__ w_down,
-                                bf16x8* __restrict__ packed, int D, int F) {
+                                bf16x8* __restrict__ packed, int D, int F, int gate_first) {
   const int KS = D / 16, MB = D / 32, CFRAG = KS + MB, NFRAG = kCPB * CFRAG;
   const int64_t total = static_cast<int64_t>(F / (kHU * kCPB)) * NFRAG * 64;
   const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -85,7 +88,7 @@ __global__ void ffn_pack_kernel(const bf16_t* __restrict__ w_up, const bf16_t* _
   const int l32 = lane % 32, hh = lane / 32;
   const bf16_t* src;
   if (r < KS)
-    src = w_up + ((l32 >= 16 ? F : 0) + unit0 + up_unit_of_slot(l32 & 15)) * D + r * 16 + hh * 8;
+    src = w_up + (((l32 < 16) == (gate_first != 0) ? 0 : F) + unit0 + up_unit_of_slot(l32 & 15)) * D + r * 16 + hh * 8;
   else
     src = w_down + static_cast<int64_t>((r - KS) * 32 + l32) * F + unit0 + hh * 8;
   packed[gid] = *reinterpret_cast<const bf16x8*>(src);
@@ -107,22 +110,27 @@ __global__ void linear_pack_kernel(const bf16_t* __restrict__ w, bf16x8* __restr
 
 // ---- shared pieces ---------------------------------------------------------------------------------------------------
 
-// Loads the wavefront's token rows as B-operand fragments and, if norm_w is given, RMS-normalises them in place:
-// y = bf16( x * rsqrt(mean(x^2) + eps) * w ). Lane (l32, hh) holds features 16*ks + 8*hh .. +7 of token l32.
+// Loads the wavefront's token rows as B-operand fragments: lane (l32, hh) holds features 16*ks + 8*hh .. +7 of token
+// l32 of each 32-token tile.
 template <int D, int TT>
-__device__ __forceinline__ void load_tokens(const TsParams& p, int64_t tok0, int l32, int hh,
-                                            bf16x8 (&xf)[TT][D / 16]) {
+__device__ __forceinline__ void load_token_rows(const TsParams& p, int64_t tok0, int l32, int hh,
+                                                bf16x8 (&xf)[TT][D / 16]) {
   constexpr int KS = D / 16;
 #pragma unroll
   for (int t = 0; t < TT; ++t) {
-    // Rows beyond M are clamped to the last row: their results are computed but never stored.
+    // Rows beyond M are clamped to the last row: their results are bit-identical to that row's.
     int64_t tok = tok0 + t * 32 + l32;
     tok = tok < p.M ? tok : p.M - 1;
     const bf16_t* row = p.x + tok * p.ldx + hh * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) xf[t][ks] = *reinterpret_cast<const bf16x8*>(row + ks * 16);
   }
-  if (p.norm_w == nullptr) return;
+}
+
+// RMS-normalises the loaded rows in place: y = bf16( x * rsqrt(mean(x^2) + eps) * w ), w read from its LDS copy.
+template <int D, int TT>
+__device__ __forceinline__ void normalize_tokens(float eps, const bf16_t* norm_w_lds, int hh, bf16x8 (&xf)[TT][D / 16]) {
+  constexpr int KS = D / 16;
   float scale[TT];
 #pragma unroll
   for (int t = 0; t < TT; ++t) {
@@ -135,7 +143,7 @@ __device__ __forceinline__ void load_tokens(const TsParams& p, int64_t tok0, int
         ss += v * v;
       }
     ss += __shfl_xor(ss, 32, kWave);
-    scale[t] = rsqrtf(ss * (1.0f / D) + p.eps);
+    scale[t] = rsqrtf(ss * (1.0f / D) + eps);
   }
   // Make the packed rows opaque here: otherwise the compiler keeps all D fp32 copies from the first sweep alive for
   // the second one, which does not fit the register file next to the accumulators.
@@ -145,7 +153,7 @@ __device__ __forceinline__ void load_tokens(const TsParams& p, int64_t tok0, int
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(xf[t][ks]));
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
-    const bf16x8 wv = *reinterpret_cast<const bf16x8*>(p.norm_w + ks * 16 + hh * 8);
+    const bf16x8 wv = *reinterpret_cast<const bf16x8*>(norm_w_lds + ks * 16 + hh * 8);
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
 #pragma unroll
@@ -170,20 +178,37 @@ __device__ __forceinline__ void stage_bias(const bf16_t* src, bf16_t* dst, int n
   }
 }
 
+// Up-projection bias in fragment row order: entry chunk * 32 + m belongs to row slot m of the chunk's up fragment
+// (slots 0..15 the gated half, 16..31 the other half), so lane l32 of a wavefront finds the bias of its fragment row at
+// chunk * 32 + l32. Zeros when there is no bias.
+__device__ __forceinline__ void stage_up_bias(const bf16_t* b_up, bf16_t* dst, int F, int gate_first, int tid,
+                                              int nthreads) {
+  for (int i = tid; i < 2 * F; i += nthreads) {
+    const int m = i % 32;
+    const int src = ((m < 16) == (gate_first != 0) ? 0 : F) + (i / 32) * kHU + up_unit_of_slot(m % 16);
+    dst[i] = b_up != nullptr ? b_up[src] : static_cast<bf16_t>(0.f);
+  }
+}
+
+// Bias values of a 64-feature chunk in accumulator order: piece rb*4 + jq holds features rb*32 + jq*8 + hh*4 .. +3.
+__device__ __forceinline__ void read_chunk_bias(const bf16_t* bias_lds, int hh, bf16x4 (&bv)[8]) {
+#pragma unroll
+  for (int q = 0; q < 8; ++q) bv[q] = *reinterpret_cast<const bf16x4*>(bias_lds + (q / 4) * 32 + (q % 4) * 8 + hh * 4);
+}
+
 // Writes two 32-feature accumulator blocks (64 features) of one 32-token tile into the wavefront's epilogue tile,
 // adding the bias and rounding to bf16. Accumulator register jq*4 + e of lane (l32, hh) is feature jq*8 + hh*4 + e.
-__device__ __forceinline__ void tile_to_lds(uint8_t* tile, const f32x16& a0, const f32x16& a1, const bf16_t* bias_lds,
+__device__ __forceinline__ void tile_to_lds(uint8_t* tile, const f32x16& a0, const f32x16& a1, const bf16x4 (&bv)[8],
                                             int l32, int hh) {
 #pragma unroll
   for (int rb = 0; rb < 2; ++rb) {
 #pragma unroll
     for (int jq = 0; jq < 4; ++jq) {
       const int col = rb * 32 + jq * 8 + hh * 4;
-      const bf16x4 bv = *reinterpret_cast<const bf16x4*>(bias_lds + col);
       bf16x4 ov;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        ov[e] = static_cast<bf16_t>((rb == 0 ? a0[jq * 4 + e] : a1[jq * 4 + e]) + static_cast<float>(bv[e]));
+        ov[e] = static_cast<bf16_t>((rb == 0 ? a0[jq * 4 + e] : a1[jq * 4 + e]) + static_cast<float>(bv[rb * 4 + jq][e]));
       *reinterpret_cast<bf16x4*>(tile + l32 * kStageRow + col * 2) = ov;
     }
   }
@@ -218,6 +243,75 @@ __device__ __forceinline__ void load_residual(const bf16_t* residual, int64_t ld
   }
 }
 
+// ---- hand-issued LDS / global operations ---------------------------------------------------------------------------
+// The compiler treats every global->LDS load as a "flat" access and, while one is in flight, turns each of its own
+// waits into a wait for EVERYTHING (vmcnt(0) / lgkmcnt(0)). Operations whose latency must stay hidden are therefore
+// issued and awaited by hand with exact counts, which is sound because the operations of one counter complete in
+// issue order; a hand-written count may be too small (waits longer), never too large.
+__device__ __forceinline__ uint32_t lds_offset(const void* lds_ptr) {
+  // The low 32 bits of a generic pointer into LDS are the LDS byte offset.
+  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_ptr));
+}
+
+template <int OFFSET>
+__device__ __forceinline__ void lds_read_frag(bf16x8& dst, uint32_t addr) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFFSET) : "memory");
+}
+
+// Waits until at most N of this wavefront's LDS operations are outstanding; the two fragments are tied to the wait so
+// that their consumers cannot be scheduled above it.
+template <int N>
+__device__ __forceinline__ void lds_wait_pair(bf16x8& a, bf16x8& b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
+}
+
+__device__ __forceinline__ void global_load16_async(bf16x8& dst, const void* src) {
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(src) : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void vm_wait() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void vm_wait_res(bf16x8 (&res)[4]) {
+  asm volatile("s_waitcnt vmcnt(%4)" : "+v"(res[0]), "+v"(res[1]), "+v"(res[2]), "+v"(res[3]) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void vm_wait_res(bf16x8 (&res)[8]) {
+  asm volatile("s_waitcnt vmcnt(%8)"
+               : "+v"(res[0]), "+v"(res[1]), "+v"(res[2]), "+v"(res[3]), "+v"(res[4]), "+v"(res[5]), "+v"(res[6]),
+                 "+v"(res[7])
+               : "n"(N)
+               : "memory");
+}
+
+template <int OFFSET>
+__device__ __forceinline__ void lds_read_u16(uint32_t& dst, uint32_t addr) {
+  asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFFSET) : "memory");
+}
+
+// Same for a single fragment, optionally tying one more value (read earlier than the fragment) to the wait.
+template <int N>
+__device__ __forceinline__ void lds_wait_frag(bf16x8& a) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_frag(bf16x8& a, uint32_t& b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
+}
+
+// Calls f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}) in order.
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
+
 // ------------------------------------------------------------------------------------------------------------------
 // Fused RMSNorm -> up -> SiLU-gate -> down -> + residual
 //
@@ -225,9 +319,9 @@ __device__ __forceinline__ void load_residual(const bf16_t* residual, int64_t ld
 // rows, so ONE accumulator (16 registers per lane) holds g in registers 0..7 and u in registers 8..15 for the same
 // eight hidden units of the lane's token. silu(g) * u of those eight is exactly one B-operand fragment (k = 16) of
 // the down projection. Two chunks are staged and consumed per barrier.
-// LDS: [2 weight buffers][b_up (2F) | b_down (D)]; after the main loop the weight buffers hold the epilogue tiles.
+// LDS: [2 weight buffers][b_up (2F) | b_down (D) | norm weight (D)]; after the main loop the weight buffers hold the epilogue tiles.
 // ------------------------------------------------------------------------------------------------------------------
-template <int D, int TT, int NWAVES, int CPB>
+template <int D, int TT, int NWAVES, int CPB, bool DEFER>
 __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_kernel(const TsParams p) {
   constexpr int kTokPerWg = NWAVES * 32 * TT;  // TT token tiles of 32 per wavefront
   constexpr int KS = D / 16;             // k-steps of the up projection = up fragments per chunk
@@ -236,9 +330,11 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
   constexpr int NFRAG = CPB * CFRAG;     // fragments per barrier step
   constexpr int FPW = NFRAG / NWAVES;    // fragments staged per wavefront
   static_assert(NFRAG % NWAVES == 0, "fragments must divide over the wavefronts");
-  static_assert(2 * NFRAG * kFrag >= NWAVES * kStageWave, "epilogue tiles must fit in the weight buffers");
+  constexpr int NBUF = DEFER ? 3 : 2;    // weight buffers in LDS
+  static_assert(MB == 4 || MB == 8, "the activation pairs are spread over the down-projection MFMAs");
+  static_assert(NBUF * NFRAG * kFrag >= NWAVES * kStageWave, "epilogue tiles must fit in the weight buffers");
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  bf16_t* bias_lds = reinterpret_cast<bf16_t*>(smem + 2 * NFRAG * kFrag);
+  bf16_t* bias_lds = reinterpret_cast<bf16_t*>(smem + NBUF * NFRAG * kFrag);
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // wavefront-uniform, kept in a scalar register
@@ -269,7 +365,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
     }
     const int s32 = ln & 31, shh = ln >> 5;
     const uint32_t up_lane_off =
-        static_cast<uint32_t>((((s32 >= 16 ? F : 0) + up_unit_of_slot(s32 & 15)) * D + shh * 8) * 2);
+        static_cast<uint32_t>(((((s32 < 16) == (p.gate_first != 0) ? 0 : F) + up_unit_of_slot(s32 & 15)) * D + shh * 8) * 2);
     const uint32_t down_lane_off = static_cast<uint32_t>((s32 * F + shh * 8) * 2);
 #pragma unroll
     for (int i = 0; i < FPW; ++i) {
@@ -285,11 +381,12 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
   };
 
   stage(0, 0);
-  stage_bias(p.b1, bias_lds, 2 * F, tid, NWAVES * kWave);
+  stage_up_bias(p.b1, bias_lds, F, p.gate_first, tid, NWAVES * kWave);
   stage_bias(p.b2, bias_lds + 2 * F, D, tid, NWAVES * kWave);
+  if (p.norm_w != nullptr) stage_bias(p.norm_w, bias_lds + 2 * F + D, D, tid, NWAVES * kWave);
 
   bf16x8 xf[TT][KS];
-  load_tokens<D, TT>(p, tok0, l32, hh, xf);
+  load_token_rows<D, TT>(p, tok0, l32, hh, xf);
 
   f32x16 oacc[TT][MB];
 #pragma unroll
@@ -301,62 +398,138 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
+  if (p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + 2 * F + D, hh, xf);
 
+  // One barrier step = CPB chunks = NFRAG fragments, consumed in their LDS order: per chunk KS up fragments, then MB
+  // down fragments. Fragment reads run P fragments ahead of their MFMAs through a ring of P registers sets; the two
+  // bias vectors of a chunk are read just before the chunk's first fragment, so they have landed (operations
+  // complete in order) whenever a later fragment has.
+  constexpr int P = 4;
+  const uint32_t smem_off = lds_offset(smem) + lane * 16;
+  const uint32_t bias_off = lds_offset(bias_lds) + l32 * 2;
+  // The up-projection bias enters through the matrix unit: one extra MFMA per chunk whose A operand carries the bias of
+  // fragment row l32 at k = 0 and whose B operand is 1 at k = 0 and 0 elsewhere (k = 0..7 live in lanes 0..31).
+  u32x4 ones_bits = {hh == 0 ? 0x3f80u : 0u, 0u, 0u, 0u};
+  asm volatile("" : "+v"(ones_bits));
+  const bf16x8 ones = __builtin_bit_cast(bf16x8, ones_bits);
+  // DEFER: the down projection of a chunk is issued one chunk late, interleaved with the SiLU arithmetic of the next
+  // chunk (MFMA j of the old chunk, then two gated values of the new one), so the matrix unit has work while the
+  // wavefront evaluates the activation. hb is the gated hidden state whose down projection is pending; before the
+  // first chunk it is zero and the (finite) fragments it is multiplied with do not matter.
+  bf16x8 hb[TT];
+#pragma unroll
+  for (int t = 0; t < TT; ++t)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) hb[t][e] = static_cast<bf16_t>(0.f);
+  int buf = 0;
+  uint32_t wb_prev = smem_off;
   for (int step = 0; step < nsteps; ++step) {
-    const int buf = step & 1;
-    if (step + 1 < nsteps) stage(step + 1, buf ^ 1);
+    // The target buffer was last read before the barrier that ended the previous step (with DEFER: its down
+    // fragments at the start of the previous step, hence three buffers).
+    if (step + 1 < nsteps) stage(step + 1, buf == NBUF - 1 ? 0 : buf + 1);
+    const uint32_t wb = smem_off + buf * (NFRAG * kFrag);
+    const uint32_t bias_step = bias_off + step * (CPB * 32 * 2);
+    bf16x8 ring[P];
+    uint32_t brow[CPB];  // bias of this lane's fragment row, one per chunk, zero-extended bf16
+    f32x16 gu[TT];
+    bf16x8 hb_new[TT];
+    // Fragment i of the step's stream: chunk q = i / CFRAG; r < KS is up fragment r of chunk q, r >= KS is down
+    // fragment r - KS of chunk q (of the chunk before q with DEFER, which for q = 0 lives in the previous buffer).
+    auto read_stream = [&](auto ic, bf16x8& dst) {
+      constexpr int i = decltype(ic)::value;
+      constexpr int q = i / CFRAG, r = i % CFRAG;
+      if constexpr (!DEFER || r < KS)
+        lds_read_frag<i * kFrag>(dst, wb);
+      else if constexpr (q == 0)
+        lds_read_frag<((CPB - 1) * CFRAG + r) * kFrag>(dst, wb_prev);
+      else
+        lds_read_frag<((q - 1) * CFRAG + r) * kFrag>(dst, wb);
+    };
+    lds_read_u16<0>(brow[0], bias_step);
+    static_for<P>([&](auto ic) { read_stream(ic, ring[decltype(ic)::value]); });
+    static_for<NFRAG>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      constexpr int q = i / CFRAG;  // chunk inside the step
+      constexpr int r = i % CFRAG;  // fragment inside the chunk
+      // Operations issued after the read of fragment i: the next P - 1 fragments (fewer at the end of the step) and
+      // the bias read of the following chunk if it was issued among them.
+      constexpr int after = (P - 1 < NFRAG - 1 - i ? P - 1 : NFRAG - 1 - i) +
+                            ((i / CFRAG != (i + P - 1) / CFRAG && (i + P - 1) < NFRAG) ? 1 : 0);
+      if constexpr (r == 0)
+        lds_wait_frag<after>(ring[i % P], brow[q]);  // the bias read is older than the chunk's first fragment
+      else
+        lds_wait_frag<after>(ring[i % P]);
+      if constexpr (r < KS) {
+        // ---- up projection: rows 0..15 gated half, rows 16..31 the other half ------------------------------------------
+        if constexpr (r == 0) {
+          const u32x4 bias_bits = {brow[q], 0u, 0u, 0u};
+          const bf16x8 bias_frag = __builtin_bit_cast(bf16x8, bias_bits);
+          const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          f32x16 binit = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bias_frag, ones, zero, 0, 0, 0);
 #pragma unroll
-    for (int q = 0; q < CPB; ++q) {
-      const uint8_t* wb = smem + buf * (NFRAG * kFrag) + q * (CFRAG * kFrag) + lane * 16;
-      const int unit0 = (step * CPB + q) * kHU;
-      // ---- up projection: rows 0..15 gate, rows 16..31 value, every token tile -------------------------------------
-      f32x16 gu[TT];
+          for (int t = 0; t < TT; ++t)
+            gu[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % P], xf[t][r], binit, 0, 0, 0);
+        } else {
 #pragma unroll
-      for (int t = 0; t < TT; ++t)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) gu[t][j] = 0.f;
-      // Fragment reads run kPre fragments ahead of their MFMAs; the scheduling fences keep the compiler from hoisting
-      // every read of the chunk to the top (which would not fit the register file).
-      constexpr int kPre = 3;
-      bf16x8 apipe[kPre + 1];
-#pragma unroll
-      for (int i = 0; i < kPre; ++i) apipe[i] = *reinterpret_cast<const bf16x8*>(wb + i * kFrag);
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        if (ks + kPre < KS + MB)
-          apipe[(ks + kPre) % (kPre + 1)] = *reinterpret_cast<const bf16x8*>(wb + (ks + kPre) * kFrag);
-        const bf16x8 a = apipe[ks % (kPre + 1)];
-#pragma unroll
-        for (int t = 0; t < TT; ++t) gu[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, xf[t][ks], gu[t], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      // ---- bias + SiLU gate: register j < 8 is g, register 8 + j is u of hidden unit unit0 + 8*hh + j --------------
-      const bf16x8 vg = *reinterpret_cast<const bf16x8*>(bias_lds + unit0 + 8 * hh);
-      const bf16x8 vu = *reinterpret_cast<const bf16x8*>(bias_lds + F + unit0 + 8 * hh);
-      bf16x8 hb[TT];
-#pragma unroll
-      for (int t = 0; t < TT; ++t)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float g = gu[t][e] + static_cast<float>(vg[e]);
-          const float u = gu[t][8 + e] + static_cast<float>(vu[e]);
-          hb[t][e] = static_cast<bf16_t>(p.gate_first ? silu_f(g) * u : g * silu_f(u));
+          for (int t = 0; t < TT; ++t)
+            gu[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % P], xf[t][r], gu[t], 0, 0, 0);
         }
-      // ---- down projection: O^T[feature, token] += W_down[feature, chunk] H^T --------------------------------------
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        const int f = KS + mb;  // fragment index inside the chunk; the first kPre down fragments are already in flight
-        if (f + kPre < KS + MB)
-          apipe[(f + kPre) % (kPre + 1)] = *reinterpret_cast<const bf16x8*>(wb + (f + kPre) * kFrag);
-        const bf16x8 ad = apipe[f % (kPre + 1)];
+      } else {
+        // ---- down projection: O^T[feature, token] += W_down[feature, chunk] H^T --------------------------------------
 #pragma unroll
         for (int t = 0; t < TT; ++t)
-          oacc[t][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ad, hb[t], oacc[t][mb], 0, 0, 0);
+          oacc[t][r - KS] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % P], hb[t], oacc[t][r - KS], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (i + P < NFRAG) {
+        if constexpr ((i + P) % CFRAG == 0) lds_read_u16<((i + P) / CFRAG) * 64>(brow[(i + P) / CFRAG], bias_step);
+        read_stream(std::integral_constant<int, i + P>{}, ring[i % P]);
+      }
+      // ---- SiLU gate: register e < 8 is the gated value, register 8 + e its partner, hidden unit unit0 + 8*hh + e -----
+      if constexpr (!DEFER && r == KS - 1) {
+#pragma unroll
+        for (int t = 0; t < TT; ++t)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) hb[t][e] = static_cast<bf16_t>(silu_f(gu[t][e]) * gu[t][8 + e]);
         __builtin_amdgcn_sched_barrier(0);
       }
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if constexpr (DEFER && r >= KS) {
+        constexpr int j = r - KS;  // down MFMA just issued; the 4 pairs of gated values are spread over the MB MFMAs
+#pragma unroll
+        for (int t = 0; t < TT; ++t)
+#pragma unroll
+          for (int g = (j * 4) / MB; g < ((j + 1) * 4) / MB; ++g)
+#pragma unroll
+            for (int e = 2 * g; e < 2 * g + 2; ++e)
+              hb_new[t][e] = static_cast<bf16_t>(silu_f(gu[t][e]) * gu[t][8 + e]);
+        if constexpr (r == CFRAG - 1) {
+#pragma unroll
+          for (int t = 0; t < TT; ++t) hb[t] = hb_new[t];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    });
+    // The next step's weights must have landed (the only vector-memory operations of this loop).
+    vm_wait<0>();
     __syncthreads();
+    wb_prev = wb;
+    buf = buf == NBUF - 1 ? 0 : buf + 1;
+  }
+  if constexpr (DEFER) {
+    // The down projection of the last chunk is still pending; its fragments are in the last step's buffer.
+    bf16x8 tail[MB];
+    static_for<MB>([&](auto ic) {
+      constexpr int j = decltype(ic)::value;
+      lds_read_frag<((CPB - 1) * CFRAG + KS + j) * kFrag>(tail[j], wb_prev);
+    });
+    static_for<MB>([&](auto ic) {
+      constexpr int j = decltype(ic)::value;
+      lds_wait_frag<MB - 1 - j>(tail[j]);
+#pragma unroll
+      for (int t = 0; t < TT; ++t)
+        oacc[t][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tail[j], hb[t], oacc[t][j], 0, 0, 0);
+    });
+    __syncthreads();  // the epilogue tiles below overwrite the weight buffers
   }
 
   // ---- epilogue: + b_down, round, transpose through the wavefront's LDS tile, + residual, coalesced bf16 stores ----
@@ -369,7 +542,9 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
     for (int pr = 0; pr < MB / 2; ++pr) {  // 64 features at a time
       bf16x8 res[4];
       if (p.residual != nullptr) load_residual(p.residual, p.ldr, tok_base, p.M, pr * 64, res, lane);
-      tile_to_lds(tile, oacc[t][2 * pr], oacc[t][2 * pr + 1], bdown_lds + pr * 64, l32, hh);
+      bf16x4 bv[8];
+      read_chunk_bias(bdown_lds + pr * 64, hh, bv);
+      tile_to_lds(tile, oacc[t][2 * pr], oacc[t][2 * pr + 1], bv, l32, hh);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       if (p.residual != nullptr)
         tile_to_global<true>(tile, p.out, p.ldo, tok_base, p.M, pr * 64, res, lane);
@@ -383,16 +558,37 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 
 // ------------------------------------------------------------------------------------------------------------------
 // [RMSNorm ->] linear [-> + residual], K = D, N a multiple of 64
-// LDS: [2 weight buffers of 2*KS fragments][NWAVES epilogue tiles][bias (N)]
+//
+// Persistent: a workgroup (8 wavefronts x TT tiles of 32 tokens) walks token tiles blockIdx.x, blockIdx.x + gridDim.x, ...; for
+// each tile it walks the N / 64 output chunks. The weight chunks form one endless stream over the global step number
+// s = tile_index * nchunks + chunk, staged by DMA into a ring of three LDS buffers two steps ahead of their use, so
+// the stream never drains at a tile boundary.
+//
+// Memory-counter discipline. The compiler treats every global->LDS load as a "flat" access and, while one is in
+// flight, turns each of its own waits into a wait for EVERYTHING (vmcnt(0) / lgkmcnt(0)). The operations whose latency
+// must stay hidden are therefore issued and awaited by hand with exact counts, which is sound because operations of
+// one counter complete in issue order:
+//   * weight fragments are read from LDS with ds_read_b128 four (row block 0, row block 1) pairs ahead of their MFMAs;
+//   * per step and wavefront the vector-memory operations are issued in this order:
+//       [RES: NST residual loads of step s+1] [FPW weight DMAs of step s+2] ... [NST output stores of step s]
+//     (NST = 4 per 32-token tile) and the step ends with vmcnt(FPW + NST) (vmcnt(NST) when no DMA was issued): the residual pieces of step s+1 and
+//     the weights of step s+1 have landed, the weights of step s+2 and the stores of step s stay in flight.
+//   Every wavefront issues exactly these counts: rows beyond M are clamped to row M-1 for loads AND stores (the
+//   clamped rows compute bit-identical values, so the duplicate stores are benign).
+// LDS: [3 weight buffers of 2*KS fragments][8 epilogue tiles][bias (N) | norm weight (D)]
 // ------------------------------------------------------------------------------------------------------------------
-template <int D, int TT, int NWAVES>
-__global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void norm_linear_kernel(const TsParams p) {
-  constexpr int kTokPerWg = NWAVES * 32 * TT;
+template <int D, int TT, bool RES>
+__global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParams p, const int num_tiles) {
+  constexpr int NWAVES = 8;
+  constexpr int kTokPerWg = NWAVES * 32 * TT;  // TT token tiles of 32 per wavefront
   constexpr int KS = D / 16;
-  constexpr int NFRAG = 2 * KS;    // two 32-feature row blocks per chunk
+  constexpr int NFRAG = 2 * KS;  // two 32-feature row blocks per chunk
   constexpr int FPW = NFRAG / NWAVES;
+  constexpr int kBuf = NFRAG * kFrag;
+  constexpr int PRE = 4;  // fragment pairs in flight
+  constexpr int NST = 4 * TT;  // output stores (and residual pieces) per wavefront and step
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  uint8_t* tiles = smem + 2 * NFRAG * kFrag;
+  uint8_t* tiles = smem + 3 * kBuf;
   bf16_t* bias_lds = reinterpret_cast<bf16_t*>(tiles + NWAVES * kStageWave);
 
   const int tid = threadIdx.x;
@@ -400,15 +596,17 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void norm_linear_k
   const int lane = tid % kWave;
   const int l32 = lane % 32;
   const int hh = lane / 32;
-  const int64_t tok0 = static_cast<int64_t>(blockIdx.x) * kTokPerWg + wave * (32 * TT);
   const int nchunks = p.N / kNC;
+  const int my_tiles = (num_tiles - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) /
+                       static_cast<int>(gridDim.x);
+  const int total = my_tiles * nchunks;
 
   // fragment f of a chunk = (row block f / KS, k-step f % KS); source = uniform base + 32-bit per-lane byte offset
   const char* w_bytes = reinterpret_cast<const char*>(p.w1);
   auto stage = [&](int chunk, int buf) {
     int ln = lane;
     asm volatile("" : "+v"(ln));
-    uint8_t* base = smem + buf * (NFRAG * kFrag) + wave * (FPW * kFrag);
+    uint8_t* base = smem + buf * kBuf + wave * (FPW * kFrag);
     if (p.packed) {
       const char* src = w_bytes + (static_cast<int64_t>(chunk) * NFRAG + wave * FPW) * kFrag + ln * 16;
 #pragma unroll
@@ -423,57 +621,155 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void norm_linear_k
       lds_dma16(w_bytes + (row0 * D + (f % KS) * 16) * 2 + lane_off, base + i * kFrag);
     }
   };
-
-  stage(0, 0);
-  stage_bias(p.b1, bias_lds, p.N, tid, NWAVES * kWave);
+  // Two phase groups. Wavefronts 4..7 change token tiles half a tile (nchunks / 2 steps) later than wavefronts 0..3:
+  // the output chunks of a tile are independent, so a wavefront may walk them in any cyclic order, and with the two
+  // groups out of phase the token loads and the RMSNorm arithmetic of one group run under the MFMAs of the other
+  // (one wavefront of each group per SIMD). A wavefront of the late group sees the token tiles as slots
+  // 0, 1, ..., my_tiles - 1, 0: chunks [0, nchunks/2) of its first tile at the start, the rest of them at the end
+  // (it loads that tile's rows twice, so the host switches this off when the output overwrites the input).
+  const bool late = p.stagger && (nchunks % 2 == 0) && wave >= NWAVES / 2;
+  const int switch_chunk = late ? nchunks / 2 : 0;
+  auto rows_of_slot = [&](int slot) -> int64_t {
+    const int idx = slot < my_tiles ? slot : 0;
+    return (static_cast<int64_t>(blockIdx.x) + static_cast<int64_t>(idx) * gridDim.x) * kTokPerWg + wave * (32 * TT);
+  };
+  // Residual pieces of (rows, chunk) in the layout of the epilogue stores: piece i = token 8*i + lane/8, 16 bytes.
+  auto request_residual = [&](int64_t tok_base, int chunk, bf16x8 (&res)[NST]) {
+#pragma unroll
+    for (int i = 0; i < NST; ++i) {
+      int64_t tok = tok_base + i * 8 + lane / 8;
+      tok = tok < p.M ? tok : p.M - 1;
+      global_load16_async(res[i], p.residual + tok * p.ldr + chunk * kNC + (lane % 8) * 8);
+    }
+  };
   bf16x8 xf[TT][KS];
-  load_tokens<D, TT>(p, tok0, l32, hh, xf);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
+  auto load_slot = [&](int64_t tok_base) {
+    load_token_rows<D, TT>(p, tok_base, l32, hh, xf);
+    // Consume the rows right here: otherwise the compiler's wait for them lands in front of the first MFMA of EVERY
+    // step, where it also waits for the weights and stores that are meant to stay in flight.
+#pragma unroll
+    for (int t = 0; t < TT; ++t)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(xf[t][ks]));
+  };
 
-  uint8_t* tile = tiles + wave * kStageWave;
-  for (int c = 0; c < nchunks; ++c) {
-    const int buf = c & 1;
-    // Residual pieces of this chunk are requested BEFORE the next chunk's weights, so that waiting for them does not
-    // also wait for the weight transfer (memory operations complete in issue order).
-    bf16x8 res[TT][4];
-    if (p.residual != nullptr) {
-#pragma unroll
-      for (int t = 0; t < TT; ++t) load_residual(p.residual, p.ldr, tok0 + t * 32, p.M, c * kNC, res[t], lane);
+  bf16x8 res_cur[NST], res_next[NST];
+  int slot = 0;
+  int64_t tok_wave = rows_of_slot(0);                 // first token row of this wavefront's current tile
+  stage(0, 0);
+  if (total > 1) stage(nchunks > 1 ? 1 : 0, 1);
+  if (RES) request_residual(tok_wave, 0, res_cur);
+  stage_bias(p.b1, bias_lds, p.N, tid, NWAVES * kWave);
+  if (p.norm_w != nullptr) stage_bias(p.norm_w, bias_lds + p.N, D, tid, NWAVES * kWave);
+  load_slot(tok_wave);
+  if (RES) vm_wait_res<0>(res_cur); else vm_wait<0>();
+  __syncthreads();
+  if (p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + p.N, hh, xf);
+
+  uint8_t* tile_lds = tiles + wave * kStageWave;
+  int chunk = 0;                                      // chunk of step s
+  int buf = 0;                                        // ring slot of step s
+  int chunk2 = 2 % nchunks;                           // chunk of step s + 2
+  for (int s = 0; s < total; ++s) {
+    // ---- requests for later steps ------------------------------------------------------------------------------------
+    const bool has_next = s + 1 < total;
+    const bool stage_ahead = s + 2 < total;
+    const bool new_tile = s > 0 && chunk == switch_chunk;  // this wavefront moves to its next token tile in this step
+    if (new_tile) tok_wave = rows_of_slot(++slot);
+    if (RES && has_next) {
+      const int next_chunk = chunk + 1 == nchunks ? 0 : chunk + 1;
+      request_residual(next_chunk == switch_chunk ? rows_of_slot(slot + 1) : tok_wave, next_chunk, res_next);
     }
-    if (c + 1 < nchunks) stage(c + 1, buf ^ 1);
-    const uint8_t* wb = smem + buf * (NFRAG * kFrag) + lane * 16;
-    f32x16 acc[2][TT];  // [row block][token tile]
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-      for (int t = 0; t < TT; ++t)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) acc[rb][t][j] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(wb + ks * kFrag);
-      const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(wb + (KS + ks) * kFrag);
-#pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, xf[t][ks], acc[0][t], 0, 0, 0);
-        acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, xf[t][ks], acc[1][t], 0, 0, 0);
-      }
+    if (stage_ahead) stage(chunk2, buf == 0 ? 2 : buf - 1);  // slot (s + 2) % 3, last read in step s - 1
+    if (new_tile) {
+      // The rows are requested after the weights and residual pieces of the later steps, so that those are not held
+      // back by the wait for the rows (the compiler's wait for these loads is a full vmcnt(0), once per tile).
+      load_slot(tok_wave);
+      if (p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + p.N, hh, xf);
     }
-    // Wait for the next chunk's weights (and this chunk's residual pieces) BEFORE the output stores are issued: the
-    // memory counter also counts stores, and waiting on it after them would expose the full write latency per chunk.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    // ---- the products of this chunk ------------------------------------------------------------------------------------
+    const uint32_t wb = lds_offset(smem) + buf * kBuf + lane * 16;
+    f32x16 acc0[TT], acc1[TT];
+#pragma unroll
+    for (int t = 0; t < TT; ++t)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc0[t][j] = acc1[t][j] = 0.f;
+    bf16x8 fa[PRE], fb[PRE];
+#define TAAC_READ_PAIR(K_)                                  \
+  lds_read_frag<(K_) * kFrag>(fa[(K_) % PRE], wb);          \
+  lds_read_frag<(KS + (K_)) * kFrag>(fb[(K_) % PRE], wb)
+    static_assert(PRE == 4 && KS % 4 == 0, "the read schedule below is written for four pairs in flight");
+    TAAC_READ_PAIR(0);
+    TAAC_READ_PAIR(1);
+    TAAC_READ_PAIR(2);
+    TAAC_READ_PAIR(3);
+#pragma unroll
+    for (int k4 = 0; k4 < KS; k4 += 4) {
+      const bool last = k4 + 4 >= KS;
+      // pair k4 + i: pairs up to k4 + i + 3 (or KS - 1) have been requested after it
+#define TAAC_STEP(I_)                                                                                   \
+  if (last)                                                                                             \
+    lds_wait_pair<2 * (3 - (I_))>(fa[I_], fb[I_]);                                                       \
+  else                                                                                                  \
+    lds_wait_pair<6>(fa[I_], fb[I_]);                                                                    \
+  _Pragma("unroll") for (int t = 0; t < TT; ++t) {                                                      \
+    acc0[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[I_], xf[t][k4 + (I_)], acc0[t], 0, 0, 0);      \
+    acc1[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[I_], xf[t][k4 + (I_)], acc1[t], 0, 0, 0);      \
+  }                                                                                                     \
+  __builtin_amdgcn_sched_barrier(0)
+      // The read of pair k4 + 4 + i reuses the registers of pair k4 + i right after its two MFMAs were issued.
+      TAAC_STEP(0);
+      if (!last) { lds_read_frag<0>(fa[0], wb + (k4 + 4) * kFrag); lds_read_frag<0>(fb[0], wb + (KS + k4 + 4) * kFrag); }
+      TAAC_STEP(1);
+      if (!last) { lds_read_frag<0>(fa[1], wb + (k4 + 5) * kFrag); lds_read_frag<0>(fb[1], wb + (KS + k4 + 5) * kFrag); }
+      TAAC_STEP(2);
+      if (!last) { lds_read_frag<0>(fa[2], wb + (k4 + 6) * kFrag); lds_read_frag<0>(fb[2], wb + (KS + k4 + 6) * kFrag); }
+      TAAC_STEP(3);
+      if (!last) { lds_read_frag<0>(fa[3], wb + (k4 + 7) * kFrag); lds_read_frag<0>(fb[3], wb + (KS + k4 + 7) * kFrag); }
+#undef TAAC_STEP
+    }
+#undef TAAC_READ_PAIR
+
+    // ---- epilogue of this chunk: bias, rounding, transpose through LDS, residual, 4 stores ---------------------------
+    bf16x4 bv[8];
+    read_chunk_bias(bias_lds + chunk * kNC, hh, bv);
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
-      tile_to_lds(tile, acc[0][t], acc[1][t], bias_lds + c * kNC, l32, hh);
+      tile_to_lds(tile_lds, acc0[t], acc1[t], bv, l32, hh);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      if (p.residual != nullptr)
-        tile_to_global<true>(tile, p.out, p.ldo, tok0 + t * 32, p.M, c * kNC, res[t], lane);
-      else
-        tile_to_global<false>(tile, p.out, p.ldo, tok0 + t * 32, p.M, c * kNC, res[t], lane);
+      const int64_t tok_base = tok_wave + t * 32;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = i * 8 + lane / 8;
+        int64_t tok = tok_base + row;
+        tok = tok < p.M ? tok : p.M - 1;
+        bf16x8 v = *reinterpret_cast<const bf16x8*>(tile_lds + row * kStageRow + (lane % 8) * 16);
+        if (RES) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            v[e] = static_cast<bf16_t>(static_cast<float>(v[e]) + static_cast<float>(res_cur[t * 4 + i][e]));
+        }
+        *reinterpret_cast<bf16x8*>(p.out + tok * p.ldo + chunk * kNC + (lane % 8) * 8) = v;
+      }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
-    __syncthreads();
+    // ---- close the step ------------------------------------------------------------------------------------------------
+    if (has_next) {
+      if (stage_ahead) {
+        if (RES) vm_wait_res<FPW + NST>(res_next); else vm_wait<FPW + NST>();
+      } else {
+        if (RES) vm_wait_res<NST>(res_next); else vm_wait<NST>();
+      }
+      __syncthreads();
+      if (RES) {
+#pragma unroll
+        for (int i = 0; i < NST; ++i) res_cur[i] = res_next[i];
+      }
+    }
+    buf = buf == 2 ? 0 : buf + 1;
+    if (++chunk == nchunks) chunk = 0;
+    if (++chunk2 == nchunks) chunk2 = 0;
   }
 }
 
@@ -491,17 +787,27 @@ int launch_ts(K kernel, const TsParams& p, int threads, int tokens_per_wg, size_
   return check_launch(name);
 }
 
-// Workgroup shape of the token-stationary kernels (tuning knob, read once from TAAC_TS_CONFIG; default 1, the
-// fastest of the three on MI355X at D = 256):
-//   0 = 4 wavefronts x 32 tokens, one FFN chunk per barrier  -> two workgroups per CU run independently
-//   1 = 8 wavefronts x 32 tokens, two FFN chunks per barrier -> one workgroup per CU, two wavefronts per SIMD
-//   2 = 4 wavefronts x 64 tokens, two FFN chunks per barrier -> one workgroup per CU, one wavefront per SIMD
+// Schedule of the fused FFN kernel (tuning knob, read once from TAAC_TS_CONFIG; default 1):
+//   0 = down projection of a chunk right after its activation, two weight buffers
+//   1 = down projection deferred by one chunk and interleaved with the next activation, three weight buffers
 int ts_config() {
   static const int config = [] {
     const char* env = getenv("TAAC_TS_CONFIG");
-    return (env != nullptr && env[0] >= '0' && env[0] <= '2') ? env[0] - '0' : 1;
+    return (env != nullptr && env[0] >= '0' && env[0] <= '1') ? env[0] - '0' : 1;
   }();
   return config;
+}
+
+// Compute units of the current device (the persistent kernels launch one workgroup per unit), cached per device.
+int compute_units() {
+  static int cached[64] = {};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return -1;
+  if (cached[device] > 0) return cached[device];
+  int count = 0;
+  if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0) return -1;
+  cached[device] = count;
+  return count;
 }
 
 bool ptr_ok(const void* p, uintptr_t mask) { return (reinterpret_cast<uintptr_t>(p) & mask) == 0; }
@@ -517,7 +823,7 @@ extern "C" int64_t taac_ffn_packed_bytes(int32_t D, int32_t F) {
 }
 
 extern "C" int taac_ffn_pack_weights(const void* w_up, const void* w_down, void* packed, int32_t D, int32_t F,
-                                     void* stream) {
+                                     int gate_first, void* stream) {
   using namespace taac;
   const char* name = "taac_ffn_pack_weights";
   if (taac_ffn_packed_bytes(D, F) < 0)
@@ -528,7 +834,7 @@ extern "C" int taac_ffn_pack_weights(const void* w_up, const void* w_down, void*
   const int64_t pieces = static_cast<int64_t>(3) * D * F / 8;
   hipLaunchKernelGGL(ffn_pack_kernel, dim3(static_cast<uint32_t>((pieces + 255) / 256)), dim3(256), 0,
                      as_stream(stream), static_cast<const bf16_t*>(w_up), static_cast<const bf16_t*>(w_down),
-                     static_cast<bf16x8*>(packed), D, F);
+                     static_cast<bf16x8*>(packed), D, F, gate_first ? 1 : 0);
   return check_launch(name);
 }
 
@@ -570,7 +876,7 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
   if (!ptr_ok(x, 15) || !ptr_ok(w_up, 15) || !ptr_ok(w_down, 15) || !ptr_ok(out, 15) || !ptr_ok(residual, 15) ||
       !ptr_ok(norm_weight, 15) || !ptr_ok(b_up, 15) || !ptr_ok(b_down, 15) || !ptr_ok(packed_weights, 15))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
-  if (static_cast<size_t>(2 * kCPB * (D / 16 + D / 32)) * kFrag + static_cast<size_t>(2 * F + D) * 2 > kMaxLdsBytes)
+  if (static_cast<size_t>(2 * kCPB * (D / 16 + D / 32)) * kFrag + static_cast<size_t>(2 * F + 2 * D) * 2 > kMaxLdsBytes)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: F=%d does not fit the LDS (limit %d bytes)", name, F, kMaxLdsBytes);
   TsParams p{};
   p.x = static_cast<const bf16_t*>(x);
@@ -591,19 +897,19 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
   p.packed = packed_weights ? 1 : 0;
   hipStream_t s = as_stream(stream);
   const int KS = D / 16, MB = D / 32;
-  const size_t bias_bytes = static_cast<size_t>(2 * F + D) * 2;
-#define TAAC_FFN_LAUNCH(DD, TT, NW, CPB)                                                                      \
-  return launch_ts(swiglu_ffn_kernel<DD, TT, NW, CPB>, p, NW * kWave, NW * 32 * TT,                          \
-                   static_cast<size_t>(2 * CPB * (KS + MB)) * kFrag + bias_bytes, s, name)
-  const int cfg = ts_config();
+  const size_t bias_bytes = static_cast<size_t>(2 * F + 2 * D) * 2;
+#define TAAC_FFN_LAUNCH(DD, TT, NW, CPB, DEFER)                                                               \
+  return launch_ts(swiglu_ffn_kernel<DD, TT, NW, CPB, DEFER>, p, NW * kWave, NW * 32 * TT,                   \
+                   static_cast<size_t>((DEFER ? 3 : 2) * CPB * (KS + MB)) * kFrag + bias_bytes, s, name)
+  int cfg = ts_config();
+  // the deferred schedule needs a third weight buffer: fall back when a large F leaves no room for it next to the biases
+  if (cfg >= 1 && static_cast<size_t>(3 * kCPB * (KS + MB)) * kFrag + bias_bytes > kMaxLdsBytes) cfg = 0;
   if (D == 256) {
-    if (cfg == 0) TAAC_FFN_LAUNCH(256, 1, 4, 1);
-    if (cfg == 1) TAAC_FFN_LAUNCH(256, 1, 8, 2);
-    TAAC_FFN_LAUNCH(256, 2, 4, 2);
+    if (cfg == 1) TAAC_FFN_LAUNCH(256, 1, 8, 2, true);
+    TAAC_FFN_LAUNCH(256, 1, 8, 2, false);
   }
-  if (cfg == 0) TAAC_FFN_LAUNCH(128, 1, 4, 1);
-  if (cfg == 1) TAAC_FFN_LAUNCH(128, 1, 8, 2);
-  TAAC_FFN_LAUNCH(128, 2, 4, 2);
+  if (cfg == 1) TAAC_FFN_LAUNCH(128, 1, 8, 2, true);
+  TAAC_FFN_LAUNCH(128, 1, 8, 2, false);
 #undef TAAC_FFN_LAUNCH
 }
 
@@ -623,7 +929,7 @@ extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm
   if (!ptr_ok(x, 15) || !ptr_ok(w, 15) || !ptr_ok(out, 15) || !ptr_ok(residual, 15) || !ptr_ok(norm_weight, 15) ||
       !ptr_ok(bias, 15) || !ptr_ok(packed_weights, 15))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
-  if (static_cast<size_t>(2 * 2 * (K / 16)) * kFrag + 8 * static_cast<size_t>(kStageWave) + static_cast<size_t>(N) * 2 >
+  if (static_cast<size_t>(3 * 2 * (K / 16)) * kFrag + 8 * static_cast<size_t>(kStageWave) + static_cast<size_t>(N + K) * 2 >
       kMaxLdsBytes)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: N=%d does not fit the LDS (limit %d bytes)", name, N, kMaxLdsBytes);
   TsParams p{};
@@ -640,20 +946,43 @@ extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm
   p.N = N;
   p.eps = eps;
   p.packed = packed_weights ? 1 : 0;
-  hipStream_t s = as_stream(stream);
-#define TAAC_LIN_LAUNCH(KK, TT, NW)                                                                            \
-  return launch_ts(norm_linear_kernel<KK, TT, NW>, p, NW * kWave, NW * 32 * TT,                               \
-                   static_cast<size_t>(2 * 2 * (KK / 16)) * kFrag + static_cast<size_t>(NW) * kStageWave +    \
-                       static_cast<size_t>(N) * 2,                                                             \
-                   s, name)
-  const int cfg = ts_config();
-  if (K == 256) {
-    if (cfg == 0) TAAC_LIN_LAUNCH(256, 1, 4);
-    if (cfg == 1) TAAC_LIN_LAUNCH(256, 1, 8);
-    TAAC_LIN_LAUNCH(256, 2, 4);
+  {
+    const char* x_lo = static_cast<const char*>(x);
+    const char* x_hi = x_lo + ((M - 1) * ldx + K) * 2;
+    const char* o_lo = static_cast<const char*>(out);
+    const char* o_hi = o_lo + ((M - 1) * ldo + N) * 2;
+    p.stagger = (o_hi <= x_lo || x_hi <= o_lo) ? 1 : 0;
   }
-  if (cfg == 0) TAAC_LIN_LAUNCH(128, 1, 4);
-  if (cfg == 1) TAAC_LIN_LAUNCH(128, 1, 8);
-  TAAC_LIN_LAUNCH(128, 2, 4);
+  hipStream_t s = as_stream(stream);
+  // Without a residual two token tiles per wavefront fit the register file: every weight fragment read from LDS then
+  // feeds two MFMAs, which halves the LDS traffic that otherwise caps the kernel.
+  const int tt = residual ? 1 : 2;
+  const int64_t tiles64 = (M + 256 * tt - 1) / (256 * tt);
+  if (tiles64 > 0x3fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many token tiles", name);
+  const int num_tiles = static_cast<int>(tiles64);
+  const int cus = compute_units();
+  if (cus <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
+  int grid = num_tiles < cus ? num_tiles : cus;
+  // Test hook: cap the number of persistent workgroups so that small inputs exercise the multi-tile path.
+  if (const char* cap = getenv("TAAC_TS_MAX_WORKGROUPS")) {
+    const int limit = atoi(cap);
+    if (limit > 0 && limit < grid) grid = limit;
+  }
+  const size_t lds_bytes =
+      static_cast<size_t>(3 * 2 * (K / 16)) * kFrag + 8 * static_cast<size_t>(kStageWave) + static_cast<size_t>(N + K) * 2;
+#define TAAC_LIN_LAUNCH(KK, TT, RR)                                                                                  \
+  do {                                                                                                            \
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(norm_linear_kernel<KK, TT, RR>),                            \
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)) != hipSuccess) \
+      return set_error(TAAC_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", name, lds_bytes);                  \
+    hipLaunchKernelGGL((norm_linear_kernel<KK, TT, RR>), dim3(grid), dim3(8 * kWave), lds_bytes, s, p, num_tiles);    \
+    return check_launch(name);                                                                                    \
+  } while (0)
+  if (K == 256) {
+    if (residual) TAAC_LIN_LAUNCH(256, 1, true);
+    TAAC_LIN_LAUNCH(256, 2, false);
+  }
+  if (residual) TAAC_LIN_LAUNCH(128, 1, true);
+  TAAC_LIN_LAUNCH(128, 2, false);
 #undef TAAC_LIN_LAUNCH
 }

@@ -185,6 +185,27 @@ def test_fused_norm_linear(device, m, k, n):
     torch.testing.assert_close(plain.cpu().float(), F.linear(x.float(), w.float()), **BF16_TOL)
 
 
+@pytest.mark.parametrize("workgroups", [1, 2, 3])
+@pytest.mark.parametrize("m,k,n", [(3000, 256, 768), (2049, 128, 256), (1500, 256, 64)])
+def test_fused_norm_linear_walks_several_token_tiles(device, monkeypatch, workgroups, m, k, n):
+    """The linear kernel is persistent: with few workgroups each one walks several token tiles (what happens at full
+    size on 256 compute units), including the out-of-phase tile changes of its two wavefront groups and the residual
+    pieces requested one step ahead across a tile boundary."""
+    from taac_2026_amd.api import norm_linear
+
+    monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+    x, w, b = _draw(m, n, k, seed=m + n + workgroups)
+    g = torch.Generator().manual_seed(11)
+    nw = (1 + 0.1 * torch.randn(k, generator=g)).to(torch.bfloat16)
+    res = torch.randn(m, n, generator=g).to(torch.bfloat16)
+    expected = res.float() + F.linear(oracle.rms_norm_fp32(x, nw).float(), w.float(), b.float())
+    with torch.no_grad():
+        got = norm_linear(x.to(device), w.to(device), b.to(device), norm_weight=nw.to(device), residual=res.to(device))
+        plain = norm_linear(x.to(device), w.to(device))
+    torch.testing.assert_close(got.cpu().float(), expected, **BF16_TOL)
+    torch.testing.assert_close(plain.cpu().float(), F.linear(x.float(), w.float()), **BF16_TOL)
+
+
 def test_fused_paths_fall_back_for_other_widths(device):
     from taac_2026_amd.api import norm_linear, swiglu_ffn
 
