@@ -27,6 +27,14 @@ constexpr int kNumXcd = 8;    // MI355X: 8 accelerator dies, workgroup i is disp
 // ---- host-side error plumbing -----------------------------------------------------------------------------------
 int set_error(int code, const char* fmt, ...);
 int check_launch(const char* what);
+// Compute units of the current device, cached per device; -1 when the query fails.
+int compute_units();
+// Token-stationary e4m3 dense layer (fp8_ts.hip): TAAC_OK after a launch, a negative status on an error, 1 when the shape
+// is not covered and the caller must use the tiled kernel.
+int launch_linear_fp8_ts(const void* a, int a_is_fp8, int64_t lda, const void* w, const float* amax_a,
+                         const float* amax_w, const void* bias, const void* residual, void* out, int64_t ldo,
+                         int64_t M, int32_t N, int32_t K, int epilogue, int gate_first, hipStream_t s,
+                         const char* name);
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 __host__ __device__ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -23,10 +23,9 @@
 // segment; the residual is read the same way and added after the rounding of the layer output, which is the order
 // of roundings of the reference's bf16 evaluation (linear output rounded, then the residual add rounded).
 #include <cstdlib>
-#include <type_traits>
-#include <utility>
 
 #include "common.h"
+#include "ts_common.h"
 
 namespace taac {
 namespace {
@@ -58,11 +57,6 @@ struct TsParams {
 
 __device__ __forceinline__ float silu_f(float v) {
   return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * v));
-}
-
-// 16 bytes per lane from global memory straight into LDS; lane l lands at lds_wave_base + 16 * l.
-__device__ __forceinline__ void lds_dma16(const void* gsrc, void* lds_wave_base) {
-  __builtin_amdgcn_global_load_lds(gsrc, lds_wave_base, 16, 0, 0);
 }
 
 // Hidden unit (0..15) loaded into row slot m16 of the gate (or value) half of an up fragment: chosen so that
@@ -164,20 +158,6 @@ __device__ __forceinline__ void normalize_tokens(float eps, const bf16_t* norm_w
   }
 }
 
-// Copies n bf16 values (or zeros when src is null) into LDS with the whole workgroup; n is a multiple of 8.
-__device__ __forceinline__ void stage_bias(const bf16_t* src, bf16_t* dst, int n, int tid, int nthreads) {
-  for (int i = tid * 8; i < n; i += nthreads * 8) {
-    bf16x8 v;
-    if (src != nullptr) {
-      v = *reinterpret_cast<const bf16x8*>(src + i);
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = static_cast<bf16_t>(0.f);
-    }
-    *reinterpret_cast<bf16x8*>(dst + i) = v;
-  }
-}
-
 // Up-projection bias in fragment row order: entry chunk * 32 + m belongs to row slot m of the chunk's up fragment
 // (slots 0..15 the gated half, 16..31 the other half), so lane l32 of a wavefront finds the bias of its fragment row at
 // chunk * 32 + l32. Zeros when there is no bias.
@@ -241,75 +221,6 @@ __device__ __forceinline__ void load_residual(const bf16_t* residual, int64_t ld
     tok = tok < M ? tok : M - 1;
     res[i] = *reinterpret_cast<const bf16x8*>(residual + tok * ldr + col0 + (lane % 8) * 8);
   }
-}
-
-// ---- hand-issued LDS / global operations ---------------------------------------------------------------------------
-// The compiler treats every global->LDS load as a "flat" access and, while one is in flight, turns each of its own
-// waits into a wait for EVERYTHING (vmcnt(0) / lgkmcnt(0)). Operations whose latency must stay hidden are therefore
-// issued and awaited by hand with exact counts, which is sound because the operations of one counter complete in
-// issue order; a hand-written count may be too small (waits longer), never too large.
-__device__ __forceinline__ uint32_t lds_offset(const void* lds_ptr) {
-  // The low 32 bits of a generic pointer into LDS are the LDS byte offset.
-  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_ptr));
-}
-
-template <int OFFSET>
-__device__ __forceinline__ void lds_read_frag(bf16x8& dst, uint32_t addr) {
-  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFFSET) : "memory");
-}
-
-// Waits until at most N of this wavefront's LDS operations are outstanding; the two fragments are tied to the wait so
-// that their consumers cannot be scheduled above it.
-template <int N>
-__device__ __forceinline__ void lds_wait_pair(bf16x8& a, bf16x8& b) {
-  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
-}
-
-__device__ __forceinline__ void global_load16_async(bf16x8& dst, const void* src) {
-  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(src) : "memory");
-}
-
-template <int N>
-__device__ __forceinline__ void vm_wait() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
-template <int N>
-__device__ __forceinline__ void vm_wait_res(bf16x8 (&res)[4]) {
-  asm volatile("s_waitcnt vmcnt(%4)" : "+v"(res[0]), "+v"(res[1]), "+v"(res[2]), "+v"(res[3]) : "n"(N) : "memory");
-}
-template <int N>
-__device__ __forceinline__ void vm_wait_res(bf16x8 (&res)[8]) {
-  asm volatile("s_waitcnt vmcnt(%8)"
-               : "+v"(res[0]), "+v"(res[1]), "+v"(res[2]), "+v"(res[3]), "+v"(res[4]), "+v"(res[5]), "+v"(res[6]),
-                 "+v"(res[7])
-               : "n"(N)
-               : "memory");
-}
-
-template <int OFFSET>
-__device__ __forceinline__ void lds_read_u16(uint32_t& dst, uint32_t addr) {
-  asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFFSET) : "memory");
-}
-
-// Same for a single fragment, optionally tying one more value (read earlier than the fragment) to the wait.
-template <int N>
-__device__ __forceinline__ void lds_wait_frag(bf16x8& a) {
-  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a) : "n"(N) : "memory");
-}
-template <int N>
-__device__ __forceinline__ void lds_wait_frag(bf16x8& a, uint32_t& b) {
-  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
-}
-
-// Calls f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}) in order.
-template <class F, int... I>
-__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-  static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
 }
 
 // ------------------------------------------------------------------------------------------------------------------
@@ -564,17 +475,17 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 // s = tile_index * nchunks + chunk, staged by DMA into a ring of three LDS buffers two steps ahead of their use, so
 // the stream never drains at a tile boundary.
 //
-// Memory-counter discipline. The compiler treats every global->LDS load as a "flat" access and, while one is in
-// flight, turns each of its own waits into a wait for EVERYTHING (vmcnt(0) / lgkmcnt(0)). The operations whose latency
-// must stay hidden are therefore issued and awaited by hand with exact counts, which is sound because operations of
-// one counter complete in issue order:
+// Memory-counter discipline. The weight transfers are issued by hand (lds_dma16) and are invisible to the compiler,
+// so their completion is awaited by hand; everything else (token rows, residual pieces, output stores) is ordinary
+// code whose waits the compiler inserts with its own - hence conservative - counts.
 //   * weight fragments are read from LDS with ds_read_b128 four (row block 0, row block 1) pairs ahead of their MFMAs;
 //   * per step and wavefront the vector-memory operations are issued in this order:
 //       [RES: NST residual loads of step s+1] [FPW weight DMAs of step s+2] ... [NST output stores of step s]
-//     (NST = 4 per 32-token tile) and the step ends with vmcnt(FPW + NST) (vmcnt(NST) when no DMA was issued): the residual pieces of step s+1 and
-//     the weights of step s+1 have landed, the weights of step s+2 and the stores of step s stay in flight.
-//   Every wavefront issues exactly these counts: rows beyond M are clamped to row M-1 for loads AND stores (the
-//   clamped rows compute bit-identical values, so the duplicate stores are benign).
+//     (NST = 4 per 32-token tile) and the step ends with vmcnt(FPW + NST) (vmcnt(NST) when no DMA was issued): the
+//     weights of step s+1 have landed, the weights of step s+2 and the stores of step s may stay in flight.
+//   Every wavefront issues at least these counts after the transfer it waits for: rows beyond M are clamped to row
+//   M-1 for loads AND stores (the clamped rows compute bit-identical values, so the duplicate stores are benign),
+//   and the "memory" clobbers of the hand-written statements keep loads and stores on their side of them.
 // LDS: [3 weight buffers of 2*KS fragments][8 epilogue tiles][bias (N) | norm weight (D)]
 // ------------------------------------------------------------------------------------------------------------------
 template <int D, int TT, bool RES>
@@ -639,7 +550,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     for (int i = 0; i < NST; ++i) {
       int64_t tok = tok_base + i * 8 + lane / 8;
       tok = tok < p.M ? tok : p.M - 1;
-      global_load16_async(res[i], p.residual + tok * p.ldr + chunk * kNC + (lane % 8) * 8);
+      res[i] = *reinterpret_cast<const bf16x8*>(p.residual + tok * p.ldr + chunk * kNC + (lane % 8) * 8);
     }
   };
   bf16x8 xf[TT][KS];
@@ -662,7 +573,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
   stage_bias(p.b1, bias_lds, p.N, tid, NWAVES * kWave);
   if (p.norm_w != nullptr) stage_bias(p.norm_w, bias_lds + p.N, D, tid, NWAVES * kWave);
   load_slot(tok_wave);
-  if (RES) vm_wait_res<0>(res_cur); else vm_wait<0>();
+  vm_wait<0>();
   __syncthreads();
   if (p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + p.N, hh, xf);
 
@@ -757,9 +668,9 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     // ---- close the step ------------------------------------------------------------------------------------------------
     if (has_next) {
       if (stage_ahead) {
-        if (RES) vm_wait_res<FPW + NST>(res_next); else vm_wait<FPW + NST>();
+        vm_wait<FPW + NST>();
       } else {
-        if (RES) vm_wait_res<NST>(res_next); else vm_wait<NST>();
+        vm_wait<NST>();
       }
       __syncthreads();
       if (RES) {
@@ -796,18 +707,6 @@ int ts_config() {
     return (env != nullptr && env[0] >= '0' && env[0] <= '1') ? env[0] - '0' : 1;
   }();
   return config;
-}
-
-// Compute units of the current device (the persistent kernels launch one workgroup per unit), cached per device.
-int compute_units() {
-  static int cached[64] = {};
-  int device = 0;
-  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return -1;
-  if (cached[device] > 0) return cached[device];
-  int count = 0;
-  if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0) return -1;
-  cached[device] = count;
-  return count;
 }
 
 bool ptr_ok(const void* p, uintptr_t mask) { return (reinterpret_cast<uintptr_t>(p) & mask) == 0; }

@@ -485,6 +485,9 @@ extern "C" int taac_linear_fp8(const void* a, int a_is_fp8, int64_t lda, const v
   rc = fill_params(name, p, M, N, epilogue);
   if (rc != TAAC_OK) return rc;
   hipStream_t s = as_stream(stream);
+  rc = launch_linear_fp8_ts(a, a_is_fp8, lda, w, amax_a, amax_w, bias, residual, out, ldo, M, N, K, epilogue, gate_first,
+                            s, name);
+  if (rc <= 0) return rc;  // launched (or failed) on the token-stationary path
 #define TAAC_FP8_LAUNCH(EPI)                                                                                   \
   if (a_is_fp8)                                                                                                \
     hipLaunchKernelGGL((linear_fp8_kernel<EPI, true>), dim3(p.total), dim3(kThreads), 0, s, p);               \

@@ -22,6 +22,18 @@ int check_launch(const char* what) {
   return TAAC_OK;
 }
 
+// Compute units of the current device (the persistent kernels launch one workgroup per unit), cached per device.
+int compute_units() {
+  static int cached[64] = {};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return -1;
+  if (cached[device] > 0) return cached[device];
+  int count = 0;
+  if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0) return -1;
+  cached[device] = count;
+  return count;
+}
+
 }  // namespace taac
 
 extern "C" int taac_abi_version(void) { return TAAC_ABI_VERSION; }

@@ -140,6 +140,40 @@ def test_linear_fp8_epilogues(device):
     assert _rel_err(got.cpu(), expected) <= 5e-2
 
 
+@pytest.mark.parametrize("workgroups", [None, 1, 2])
+@pytest.mark.parametrize("epilogue", ["none", "residual", "swiglu", "swiglu_value_first"])
+def test_linear_fp8_token_stationary_path(device, monkeypatch, epilogue, workgroups):
+    """K = 256 layers run on the token-stationary e4m3 kernel: every epilogue, bf16 and pre-quantised activations,
+    ragged M, one and several token tiles per workgroup; and the tiled kernel (forced) gives the same numbers up to the
+    rounding of the output."""
+    if workgroups is not None:
+        monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+    m, k = 1333, 256
+    swiglu = epilogue.startswith("swiglu")
+    gate_first = epilogue != "swiglu_value_first"
+    n = 512 if swiglu else 320
+    x, w, b = _draw(m, n, k, seed=len(epilogue) + (workgroups or 0))
+    res = torch.randn(m, n, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16) if epilogue == "residual" else None
+    expected = oracle.linear_fp8(x, w, b, residual=res, swiglu=swiglu, gate_first=gate_first)
+    kwargs = dict(swiglu=swiglu, gate_first=gate_first, residual=None if res is None else res.to(device))
+    with torch.no_grad():
+        wq, wa = quantize_fp8(w.to(device))
+        xa = amax(x.to(device))
+        got = linear_fp8(x.to(device), wq, xa, wa, b.to(device), **kwargs)
+        xq, _ = quantize_fp8(x.to(device), xa)
+        got_q = linear_fp8(xq, wq, xa, wa, b.to(device), **kwargs)
+        no_bias = linear_fp8(x.to(device), wq, xa, wa, None, **kwargs)
+        monkeypatch.setenv("TAAC_FP8_TILED", "1")
+        tiled = linear_fp8(x.to(device), wq, xa, wa, b.to(device), **kwargs)
+        tiled_no_bias = linear_fp8(x.to(device), wq, xa, wa, None, **kwargs)
+    assert got.shape == expected.shape
+    assert _rel_err(got.cpu(), expected) <= 5e-2
+    assert _rel_err(got_q.cpu(), expected) <= 5e-2
+    scale = expected.float().abs().max().item()
+    torch.testing.assert_close(got.cpu().float(), tiled.cpu().float(), rtol=0, atol=2.0 ** -7 * scale)
+    torch.testing.assert_close(no_bias.cpu().float(), tiled_no_bias.cpu().float(), rtol=0, atol=2.0 ** -7 * scale)
+
+
 # ---- token-stationary fused kernels --------------------------------------------------------------------------------
 
 
