@@ -75,8 +75,9 @@ def _accuracy_gate(model, inputs, device) -> dict:
 
 
 def _kernel_breakdown(inputs, device, iters: int) -> dict:
-    """Stand-alone timing of each kernel of one block at the step's shapes (HIP events on the launch stream)."""
-    from taac_2026_amd.api import norm_linear, scaled_dot_product_attention, swiglu_ffn
+    """Stand-alone timing of each kernel of one block at the step's shapes (HIP events on the launch stream). The dense
+    layers walk the valid tokens only, as they do inside the step; their algorithmic work counts those tokens."""
+    from taac_2026_amd.api import norm_linear, scaled_dot_product_attention, swiglu_ffn, valid_rows
 
     B, T, D = inputs.emb.shape
     M, F, H = B * T, inputs.d_ff, inputs.num_heads
@@ -85,31 +86,36 @@ def _kernel_breakdown(inputs, device, iters: int) -> dict:
     lengths = inputs.key_lengths.to(device)
     out: dict[str, dict] = {}
     with torch.no_grad():
-        qkv = norm_linear(x, w["qkv.weight"], w["qkv.bias"], norm_weight=w["attn_norm.weight"])
+        index = valid_rows(lengths, T)
+        qkv = norm_linear(x, w["qkv.weight"], w["qkv.bias"], norm_weight=w["attn_norm.weight"], token_rows=index)
+        buf = torch.zeros_like(x)  # output buffer of the [M, D] layers (rows outside the index are never touched)
         q, k, v = qkv.chunk(3, dim=-1)
         attn = lambda: scaled_dot_product_attention(q, k, v, num_heads=H, attn_mask=None, dropout_p=0.0,  # noqa: E731
                                                     training=False, key_lengths=lengths, zero_padded_queries=True)
         a = attn()
         valid_tokens = float(lengths.sum().item())
+        Mv = valid_tokens
         sum_sq = float((lengths.double() ** 2).sum().item())
         dh = D // H
         # (callable, algorithmic flops, algorithmic HBM bytes) per launch; bf16 = 2 bytes per element
         cases = {
-            "rmsnorm_qkv": (lambda: norm_linear(x, w["qkv.weight"], w["qkv.bias"], norm_weight=w["attn_norm.weight"]),
-                            2.0 * M * 3 * D * D, 2.0 * (M * D + 3 * D * D + M * 3 * D)),
+            "rmsnorm_qkv": (lambda: norm_linear(x, w["qkv.weight"], w["qkv.bias"], norm_weight=w["attn_norm.weight"],
+                                                token_rows=index, out=qkv),
+                            2.0 * Mv * 3 * D * D, 2.0 * (Mv * D + 3 * D * D + Mv * 3 * D)),
             # useful work only: visible (query, key) pairs; Q/K/V valid rows read, O written in full
             "attention": (attn, 4.0 * H * dh * sum_sq, 2.0 * (3 * D * valid_tokens + M * D)),
-            "out_residual": (lambda: norm_linear(a, w["out.weight"], w["out.bias"], residual=x), 2.0 * M * D * D,
-                             2.0 * (3 * M * D + D * D)),
+            "out_residual": (lambda: norm_linear(a, w["out.weight"], w["out.bias"], residual=x, token_rows=index, out=buf),
+                             2.0 * Mv * D * D, 2.0 * (3 * Mv * D + D * D)),
             "rmsnorm_swiglu_ffn_residual": (
                 lambda: swiglu_ffn(x, w["up.weight"], w["up.bias"], w["down.weight"], w["down.bias"], residual=x,
-                                   norm_weight=w["ffn_norm.weight"]),
-                2.0 * M * 3 * D * F, 2.0 * (2 * M * D + 3 * D * F)),
+                                   norm_weight=w["ffn_norm.weight"], token_rows=index, out=buf),
+                2.0 * Mv * 3 * D * F, 2.0 * (2 * Mv * D + 3 * D * F)),
         }
         for name, (fn, flops, nbytes) in cases.items():
             ms = _event_ms(fn, iters, 3)
             out[name] = {
                 "ms": ms,
+                "tokens": int(Mv) if name != "attention" else int(M),
                 "algorithmic_flops": flops,
                 "algorithmic_bytes": nbytes,
                 "tflops": flops / ms / 1e9,
@@ -292,6 +298,16 @@ def main() -> None:
     ms_per_step = elapsed * 1e3 / args.steps
     value = B / (elapsed / args.steps)
 
+    # The same step with the dense layers run over all B*T positions, padding included (what the reference's dense
+    # [B, T, D] formulation does): reported next to the headline figure, never as the value.
+    os.environ["TAAC_DENSE_TOKENS"] = "1"
+    try:
+        with torch.no_grad():
+            dense_ms = _event_ms(lambda: model(emb, lengths), max(args.steps // 2, 1), 2)
+    finally:
+        del os.environ["TAAC_DENSE_TOKENS"]
+    valid_fraction = float(inputs.key_lengths.clamp(0, T).sum().item()) / (B * T)
+
     kernels = _kernel_breakdown(inputs, device, iters=10)
     dominant = max(kernels, key=lambda name: kernels[name]["ms"])
     dom = kernels[dominant]
@@ -324,11 +340,15 @@ def main() -> None:
         "config": {
             "workload": f"4-block unified token backbone forward, B={B}, T=32+{T - 32}, d_model={D}, "
                         f"{inputs.num_heads} heads x {D // inputs.num_heads}, SwiGLU d_ff={inputs.d_ff}, "
-                        "valid length ~ U{64..512}, masked mean-pool -> Linear -> sigmoid",
+                        "valid length ~ U{64..512}, masked mean-pool -> Linear -> sigmoid; dense layers and attention "
+                        "skip the padded positions",
             "batch": B,
             "tokens": T,
         },
         "dense_equivalent_tflops": dense_flops / (elapsed / args.steps) / 1e12,
+        "valid_token_fraction": valid_fraction,
+        "all_positions": {"ms_per_step": dense_ms, "samples_per_s": B / (dense_ms * 1e-3),
+                          "note": "dense layers run over the padded positions too (TAAC_DENSE_TOKENS=1)"},
         "roofline": roofline,
         "accuracy": accuracy,
         "kernels": kernels,

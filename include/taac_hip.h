@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define TAAC_ABI_VERSION 1
+#define TAAC_ABI_VERSION 2
 
 enum taac_status {
   TAAC_OK = 0,
@@ -75,8 +75,8 @@ int taac_layernorm_fwd(const void* x, const void* w, const void* b, void* y, int
  * q/o: logical shape (B, H, Tq, d); k/v: (B, H, Tk, d). *_strides are ELEMENT strides of the four logical
  * dimensions, so (B,H,T,d)-contiguous and (B,T,H,d)-contiguous tensors are both read in place; the last
  * stride must be 1, the others multiples of 8, and base pointers 16-byte aligned. d must be a multiple of 8, <= 128.
- * zero_padded_queries != 0 (requires Tq == Tk): query rows t >= key_lengths[b] are written as zeros instead
- * of being computed over the visible keys.
+ * zero_padded_queries != 0 (requires Tq == Tk): query rows t >= key_lengths[b] are not read and not computed; they are
+ * written as zeros (1) or left untouched (2).
  * dtype: TAAC_BF16 or TAAC_F16.
  * Replaces: flash_attention's kernel call `_flash_attention_kernel(q, k, v, key_lengths)`
  * (accelerators/attention/flash_attention.py:338-367, hook at :26,102-104) and the TileLang inference kernel
@@ -111,25 +111,40 @@ int taac_linear_bf16(const void* a, int64_t lda, const void* w, const void* bias
  * w_up / w_down are not read (they may be NULL) and weight staging reads contiguous memory.
  * D must be 128 or 256, F a multiple of 32. The [M, 2F] projection and the [M, F] gated hidden state are never
  * written to memory. gate_first as in taac_linear_bf16.
+ * rows / n_rows: both NULL (every row 0..M-1 is a token), or a row index as written by taac_valid_rows: the tokens are
+ * rows[0 .. *n_rows) of x / residual / out (*n_rows <= M, read on the device), all other rows are neither read nor
+ * written - this is how the layers skip the padded positions of a padded [B, T, D] batch.
  * Replaces: ffn_norm + SwiGLUFeedForward.forward + residual add of UnifiedInteractionBlock.forward
  * (experiments/symbiosis/backbone.py:19-21, 66-67).
  */
 int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w_up,
                         const void* b_up, const void* w_down, const void* b_down, const void* packed_weights,
                         const void* residual, int64_t ldr, void* out, int64_t ldo, int64_t M, int32_t D, int32_t F,
-                        int gate_first, void* stream);
+                        int gate_first, const int32_t* rows, const int32_t* n_rows, void* stream);
 
 /*
  * Fused [RMSNorm ->] dense layer [-> + residual] with the token rows held in registers:
  *   out = (residual ? residual : 0) + (norm_weight ? rmsnorm(x, norm_weight, eps) : x) @ w^T + bias
  * x: [M, K] bf16; w: [N, K]; bias: [N] or NULL; residual / out: [M, N]; packed_weights: NULL or the blob written by
- * taac_linear_pack_weights for w. K must be 128 or 256, N a multiple of 64.
+ * taac_linear_pack_weights for w. K must be 128 or 256, N a multiple of 64. out may alias residual, not x.
+ * rows / n_rows: as in taac_swiglu_ffn_fwd.
  * Replaces: attn_norm + the qkv projection, and the out projection + residual add, of UnifiedInteractionBlock /
  * UnifiedSelfAttention (experiments/symbiosis/backbone.py:34-35, 47, 64-65).
  */
 int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
                          const void* bias, const void* packed_weights, const void* residual, int64_t ldr, void* out,
-                         int64_t ldo, int64_t M, int32_t N, int32_t K, void* stream);
+                         int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows, const int32_t* n_rows,
+                         void* stream);
+
+/*
+ * Row index of the valid tokens of a padded batch: token t of sample b is valid iff t < key_lengths[b] (clamped to
+ * [0, T]). Writes rows[i] = b * T + t for the valid tokens in increasing order, *n_rows = their number, and the
+ * per-sample offsets (exclusive prefix sums of the lengths, B + 1 values, the last one equal to *n_rows) to
+ * rows[B * T .. B * T + B]. rows must hold B * T + B + 1 values. Everything stays on the device.
+ * No counterpart in the reference, which runs its dense layers over the padded positions as well
+ * (experiments/symbiosis/backbone.py:58-68 masks their updates afterwards).
+ */
+int taac_valid_rows(const int32_t* key_lengths, int32_t B, int32_t T, int32_t* rows, int32_t* n_rows, void* stream);
 
 /*
  * Weight packing for the two fused kernels above: copies the weights into MFMA-fragment order (the order in which

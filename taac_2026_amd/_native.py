@@ -22,7 +22,7 @@ TAAC_ERR_LAUNCH = -3
 TAAC_F32, TAAC_BF16, TAAC_F16 = 0, 1, 2
 EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _DTYPE_CODES = {torch.float32: TAAC_F32, torch.bfloat16: TAAC_BF16, torch.float16: TAAC_F16}
 
@@ -74,13 +74,14 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "taac_swiglu_ffn_fwd": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
-         c_void_p, c_int64, c_int64, c_int32, c_int32, c_int, c_void_p],
+         c_void_p, c_int64, c_int64, c_int32, c_int32, c_int, c_void_p, c_void_p, c_void_p],
     ),
     "taac_norm_linear_fwd": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
-         c_int64, c_int32, c_int32, c_void_p],
+         c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p],
     ),
+    "taac_valid_rows": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p]),
     "taac_ffn_packed_bytes": (c_int64, [c_int32, c_int32]),
     "taac_ffn_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int, c_void_p]),
     "taac_linear_packed_bytes": (c_int64, [c_int32, c_int32]),

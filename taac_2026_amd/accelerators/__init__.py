@@ -9,7 +9,16 @@ from taac_2026_amd.accelerators.attention import (
     plan_flash_attention_mask,
     resolved_flash_attention_backend,
 )
-from taac_2026_amd.accelerators.linear import amax, linear, linear_fp8, norm_linear, quantize_fp8, swiglu_ffn, swiglu_linear
+from taac_2026_amd.accelerators.linear import (
+    amax,
+    linear,
+    linear_fp8,
+    norm_linear,
+    quantize_fp8,
+    swiglu_ffn,
+    swiglu_linear,
+    valid_rows,
+)
 from taac_2026_amd.accelerators.normalization import (
     hip_layer_norm_kernel,
     hip_rms_norm_kernel,
@@ -49,4 +58,5 @@ __all__ = [
     "rms_norm",
     "swiglu_ffn",
     "swiglu_linear",
+    "valid_rows",
 ]

@@ -175,6 +175,45 @@ def pack_linear_weight(weight: torch.Tensor) -> torch.Tensor:
     return packed
 
 
+def valid_rows(key_lengths: torch.Tensor, tokens: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Row index of the valid tokens of a padded ``[B, tokens, ...]`` batch (token ``t`` of sample ``b`` is valid iff
+    ``t < key_lengths[b]``): ``(rows, n_rows)`` with ``rows[:n_rows] = b * tokens + t`` in increasing order, both int32
+    on the device (no host synchronisation). ``rows[B * tokens : B * tokens + B + 1]`` holds the per-sample offsets.
+    Pass the pair as ``token_rows=`` to :func:`norm_linear` / :func:`swiglu_ffn` to skip the padded positions."""
+    name = "hip valid_rows"
+    require_cuda_tensors(name, key_lengths)
+    lengths = key_lengths.to(torch.int32).contiguous()
+    batch = lengths.numel()
+    rows = torch.empty(batch * int(tokens) + batch + 1, dtype=torch.int32, device=lengths.device)
+    count = torch.empty(1, dtype=torch.int32, device=lengths.device)
+    library = _native.load_library()
+    status = library.taac_valid_rows(lengths.data_ptr(), batch, int(tokens), rows.data_ptr(), count.data_ptr(),
+                                     _native.current_stream(lengths.device))
+    _native.check(status, "valid_rows")
+    return rows, count
+
+
+def _output_rows(name: str, out: torch.Tensor | None, shape: tuple[int, int], sparse: bool, like: torch.Tensor):
+    if out is None:
+        return (torch.zeros if sparse else torch.empty)(shape, dtype=like.dtype, device=like.device)
+    require_cuda_tensors(name, like, out)
+    if out.dtype != like.dtype or out.numel() != shape[0] * shape[1] or out.shape[-1] != shape[1] or not out.is_contiguous():
+        raise ValueError(f"{name}: out must be a contiguous {like.dtype} tensor with {shape[0]} rows of {shape[1]}")
+    return out.view(shape)
+
+
+def _token_rows(name: str, token_rows, rows: torch.Tensor):
+    if token_rows is None:
+        return None, None
+    index, count = token_rows
+    require_cuda_tensors(name, index, count)
+    if index.dtype != torch.int32 or count.dtype != torch.int32 or count.numel() != 1 or not index.is_contiguous():
+        raise ValueError(f"{name}: token_rows must be (int32 row index, int32 scalar count) as returned by valid_rows")
+    if index.numel() < rows.shape[0]:
+        raise ValueError(f"{name}: the row index must cover the {rows.shape[0]} rows of the input")
+    return index, count
+
+
 def swiglu_ffn(
     x: torch.Tensor,
     up_weight: torch.Tensor,
@@ -186,6 +225,8 @@ def swiglu_ffn(
     gate_first: bool = True,
     norm_weight: torch.Tensor | None = None,
     eps: float = 1e-6,
+    token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
+    out: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """``residual + down(silu(gate) * value)`` with ``gate, value = up(rmsnorm(x)).chunk(2, -1)``.
 
@@ -193,6 +234,10 @@ def swiglu_ffn(
     128 / 256 with a hidden size that is a multiple of 32 the whole expression is ONE kernel
     (``taac_swiglu_ffn_fwd``: the projection and the gated hidden state stay in registers); other shapes run
     norm -> up(+SiLU-gate) -> down(+residual) as separate kernels.
+
+    ``token_rows`` (fused shapes only): ``(rows, n_rows)`` from :func:`valid_rows`; only those rows of the flattened
+    input are processed, the other rows of the result are zeros. ``out`` (fused shapes only): a contiguous bf16 tensor
+    of the result's shape to write into (rows outside ``token_rows`` keep their content); it may be ``residual``.
     """
     name = "hip swiglu_ffn"
     require_cuda_tensors(name, x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight)
@@ -206,6 +251,8 @@ def swiglu_ffn(
     if residual is not None and residual.shape != shape:
         raise ValueError("swiglu_ffn residual must have the shape of the input")
     if not (_fused_width(d_model) and hidden % 32 == 0):
+        if token_rows is not None or out is not None:
+            raise RuntimeError("swiglu_ffn: token_rows / out need a fused shape (width 128 / 256, hidden size a multiple of 32)")
         h = rows
         if norm_weight is not None:
             from taac_2026_amd.accelerators.normalization import rms_norm
@@ -222,13 +269,14 @@ def swiglu_ffn(
         res_rows = residual.reshape(-1, d_model)
         if res_rows.stride(-1) != 1 or res_rows.stride(0) % 8 != 0:
             res_rows = res_rows.contiguous()
-    out = torch.empty((rows.shape[0], d_model), dtype=x.dtype, device=x.device)
+    index, count = _token_rows(name, token_rows, rows)
+    out = _output_rows(name, out, (rows.shape[0], d_model), index is not None, x)
     library = _native.load_library()
     status = library.taac_swiglu_ffn_fwd(
         rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), None,
         _native.ptr(up_bias), None, _native.ptr(down_bias), packed.data_ptr(), _native.ptr(res_rows),
         res_rows.stride(0) if res_rows is not None else d_model, out.data_ptr(), d_model, rows.shape[0], d_model,
-        hidden, int(bool(gate_first)), _native.current_stream(x.device),
+        hidden, int(bool(gate_first)), _native.ptr(index), _native.ptr(count), _native.current_stream(x.device),
     )
     _native.check(status, "swiglu_ffn")
     return out.reshape(shape)
@@ -242,6 +290,8 @@ def norm_linear(
     norm_weight: torch.Tensor | None = None,
     eps: float = 1e-6,
     residual: torch.Tensor | None = None,
+    token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
+    out: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """``residual + F.linear(rmsnorm(x, norm_weight, eps), weight, bias)`` (norm and residual optional) as one
     kernel when ``in_features`` is 128 / 256 and ``out_features`` a multiple of 64; otherwise composed from the
@@ -254,6 +304,8 @@ def norm_linear(
     _check_weight(name, rows, weight, bias)
     in_features, out_features = weight.shape[1], weight.shape[0]
     if not (_fused_width(in_features) and out_features % 64 == 0):
+        if token_rows is not None or out is not None:
+            raise RuntimeError("norm_linear: token_rows / out need a fused shape (K 128 / 256, N a multiple of 64)")
         h = rows
         if norm_weight is not None:
             from taac_2026_amd.accelerators.normalization import rms_norm
@@ -269,12 +321,14 @@ def norm_linear(
         res_rows = residual.reshape(-1, out_features)
         if res_rows.stride(-1) != 1 or res_rows.stride(0) % 8 != 0:
             res_rows = res_rows.contiguous()
-    out = torch.empty((rows.shape[0], out_features), dtype=x.dtype, device=x.device)
+    index, count = _token_rows(name, token_rows, rows)
+    out = _output_rows(name, out, (rows.shape[0], out_features), index is not None, x)
     library = _native.load_library()
     status = library.taac_norm_linear_fwd(
         rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), None, _native.ptr(bias),
         packed.data_ptr(), _native.ptr(res_rows), res_rows.stride(0) if res_rows is not None else out_features, out.data_ptr(),
-        out_features, rows.shape[0], out_features, in_features, _native.current_stream(x.device),
+        out_features, rows.shape[0], out_features, in_features, _native.ptr(index), _native.ptr(count),
+        _native.current_stream(x.device),
     )
     _native.check(status, "norm_linear")
     return out.reshape(*shape[:-1], out_features)
@@ -372,6 +426,7 @@ __all__ = [
     "linear_fp8",
     "norm_linear",
     "pack_ffn_weights",
+    "valid_rows",
     "pack_linear_weight",
     "quantize_fp8",
     "swiglu_ffn",

@@ -126,7 +126,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   for (int e = 0; e < 8; ++e) zero_vec[e] = static_cast<T>(0.f);
 
   if (q_begin >= q_valid) {
-    // Whole block lies in the padding: zero-fill its rows.
+    // Whole block lies in the padding: zero-fill its rows, or leave them alone.
+    if (p.zero_pad == 2) return;
     const int c8n = p.d / 8;
     for (int idx = tid; idx < kQB * c8n; idx += kThreads) {
       const int row = q_begin + idx / c8n;
@@ -145,7 +146,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 #pragma unroll
   for (int s = 0; s < KSTEPS; ++s) {
     const int col = 16 * s + 8 * hh;
-    qf[s] = (qi < p.Tq && col < p.d) ? *reinterpret_cast<const vec_t*>(qb + qi * p.qs[2] + col) : zero_vec;
+    // Query rows in the padding are not read (they may be uninitialised memory): a zero query keeps the arithmetic finite.
+    qf[s] = (qi < q_valid && col < p.d) ? *reinterpret_cast<const vec_t*>(qb + qi * p.qs[2] + col) : zero_vec;
   }
 
   f32x16 oacc[MB];
@@ -307,7 +309,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
     const int row = pass * RPP + lane / C8;
     const int q_row = q_begin + wave * 32 + row;
     const vec_t v = *reinterpret_cast<const vec_t*>(tile + row * OROW + c8 * 16);
-    if (q_row < p.Tq && c8 * 8 < p.d) *reinterpret_cast<vec_t*>(ob + q_row * p.os[2] + c8 * 8) = v;
+    const int q_store_end = p.zero_pad == 2 ? q_valid : p.Tq;  // mode 2: rows in the padding are left untouched
+    if (q_row < q_store_end && c8 * 8 < p.d) *reinterpret_cast<vec_t*>(ob + q_row * p.os[2] + c8 * 8) = v;
   }
 }
 
@@ -382,7 +385,7 @@ extern "C" int taac_flash_attn_fwd(const void* q, const void* k, const void* v, 
     p.os[i] = o_strides[i];
   }
   p.scale_log2 = 1.4426950408889634f / sqrtf(static_cast<float>(d));
-  p.zero_pad = zero_padded_queries ? 1 : 0;
+  p.zero_pad = zero_padded_queries == 2 ? 2 : (zero_padded_queries ? 1 : 0);
   p.nqc = static_cast<uint32_t>((Tq + kQB - 1) / kQB);
   const int64_t total = static_cast<int64_t>(p.nqc) * B * H;
   if (total > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many workgroups (%lld)", name, (long long)total);

@@ -1,5 +1,7 @@
 // Forward driver of the unified token backbone (pre-norm blocks + pCVR readout) and the readout kernel.
 // The driver only sequences the library's own entry points on one stream over a caller-provided workspace.
+#include <cstdlib>
+
 #include "common.h"
 
 namespace taac {
@@ -59,8 +61,80 @@ __global__ __launch_bounds__(kBlock) void masked_mean_head_kernel(const bf16_t* 
   }
 }
 
+// Exclusive prefix sums of the clamped lengths (one workgroup; B is walked in slabs of kBlock with a running carry).
+__global__ __launch_bounds__(kBlock) void length_offsets_kernel(const int32_t* __restrict__ lengths, int B, int T,
+                                                                int32_t* __restrict__ offsets,
+                                                                int32_t* __restrict__ n_rows) {
+  __shared__ int32_t s_scan[kBlock];
+  int32_t carry = 0;
+  for (int base = 0; base < B; base += kBlock) {
+    const int b = base + threadIdx.x;
+    int32_t len = b < B ? lengths[b] : 0;
+    len = len < 0 ? 0 : (len > T ? T : len);
+    s_scan[threadIdx.x] = len;
+    __syncthreads();
+    for (int step = 1; step < kBlock; step <<= 1) {  // inclusive scan, Hillis-Steele
+      const int32_t add = threadIdx.x >= step ? s_scan[threadIdx.x - step] : 0;
+      __syncthreads();
+      s_scan[threadIdx.x] += add;
+      __syncthreads();
+    }
+    if (b < B) offsets[b] = carry + s_scan[threadIdx.x] - len;
+    carry += s_scan[kBlock - 1];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    offsets[B] = carry;
+    *n_rows = carry;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void valid_rows_kernel(const int32_t* __restrict__ lengths,
+                                                            const int32_t* __restrict__ offsets, int T,
+                                                            int32_t* __restrict__ rows) {
+  const int b = blockIdx.y;
+  int32_t len = lengths[b];
+  len = len < 0 ? 0 : (len > T ? T : len);
+  const int t = blockIdx.x * kBlock + threadIdx.x;
+  if (t < len) rows[offsets[b] + t] = b * T + t;
+}
+
+// Zero-fills the rows of the padded positions of x [B, T, D] (16 bytes per thread).
+__global__ __launch_bounds__(kBlock) void zero_padded_rows_kernel(bf16_t* __restrict__ x,
+                                                                  const int32_t* __restrict__ lengths, int T, int D) {
+  const int b = blockIdx.y;
+  int32_t len = lengths[b];
+  len = len < 0 ? 0 : (len > T ? T : len);
+  const int c8n = D / 8;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  const int64_t t = len + idx / c8n;
+  if (t >= T) return;
+  bf16x8 z;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) z[e] = static_cast<bf16_t>(0.f);
+  *reinterpret_cast<bf16x8*>(x + (static_cast<int64_t>(b) * T + t) * D + (idx % c8n) * 8) = z;
+}
+
 }  // namespace
 }  // namespace taac
+
+extern "C" int taac_valid_rows(const int32_t* key_lengths, int32_t B, int32_t T, int32_t* rows, int32_t* n_rows,
+                               void* stream) {
+  using namespace taac;
+  const char* name = "taac_valid_rows";
+  if (B < 0 || T < 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: bad dimensions", name);
+  if (static_cast<int64_t>(B) * T > 0x7fffffffLL - B - 1)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: B * T must fit 32-bit row numbers", name);
+  if (!rows || !n_rows || (B > 0 && !key_lengths)) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  if (B > 65535) return set_error(TAAC_ERR_UNSUPPORTED, "%s: at most 65535 samples", name);
+  int32_t* offsets = rows + static_cast<int64_t>(B) * T;
+  hipLaunchKernelGGL(length_offsets_kernel, dim3(1), dim3(kBlock), 0, as_stream(stream), key_lengths, B, T, offsets,
+                     n_rows);
+  if (B > 0 && T > 0)
+    hipLaunchKernelGGL(valid_rows_kernel, dim3((T + kBlock - 1) / kBlock, B), dim3(kBlock), 0, as_stream(stream),
+                       key_lengths, offsets, T, rows);
+  return check_launch(name);
+}
 
 extern "C" int taac_masked_mean_head(const void* x, const int32_t* lengths, const void* w_head, const void* b_head,
                                      float* p, int32_t B, int32_t T, int32_t D, void* stream) {
@@ -84,6 +158,8 @@ namespace {
 // Fused (token-stationary) path: model widths 128 / 256, hidden size a multiple of 32.
 inline bool fused_shape(int32_t D, int32_t F) { return (D == 128 || D == 256) && F % 32 == 0; }
 // Fragment-ordered weights of one block: qkv, out, feed-forward.
+// Row index of the valid tokens: B*T rows + B+1 offsets + the count.
+inline int64_t row_index_bytes(int32_t B, int32_t T) { return align256((static_cast<int64_t>(B) * T + B + 2) * 4); }
 inline int64_t packed_block_bytes(int32_t D, int32_t F) {
   return align256(static_cast<int64_t>(3) * D * D * 2) + align256(static_cast<int64_t>(D) * D * 2) +
          align256(static_cast<int64_t>(3) * D * F * 2);
@@ -95,9 +171,10 @@ extern "C" int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D
   using namespace taac;
   if (B < 0 || T < 0 || D <= 0 || F <= 0 || n_blocks < 0) return -1;
   const int64_t M = static_cast<int64_t>(B) * T;
-  // x, h (shared with the attention output), qkv, then either the packed weights or the gated hidden state
+  // x, h (shared with the attention output), qkv, then either the packed weights + the valid-row index (fused path)
+  // or the gated hidden state
   const int64_t acts = align256(M * D * 2) * 2 + align256(M * 3 * D * 2);
-  return acts + (fused_shape(D, F) ? n_blocks * packed_block_bytes(D, F) : align256(M * F * 2));
+  return acts + (fused_shape(D, F) ? n_blocks * packed_block_bytes(D, F) + row_index_bytes(B, T) : align256(M * F * 2));
 }
 
 extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, const taac_block_weights* blocks,
@@ -131,6 +208,16 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
   bf16_t* g = reinterpret_cast<bf16_t*>(ws);  // unfused path: gated hidden state; fused path: packed weights
   char* packed = ws;
   const bool fused = fused_shape(D, F);
+  // Fused path: the dense layers walk the valid tokens only (row index built from key_lengths on the device); the
+  // padded positions of the residual stream are never read or written. TAAC_DENSE_TOKENS switches this off.
+  int32_t* rows = nullptr;
+  int32_t* n_rows = nullptr;
+  if (fused && n_blocks > 0 && getenv("TAAC_DENSE_TOKENS") == nullptr) {
+    rows = reinterpret_cast<int32_t*>(packed + static_cast<int64_t>(n_blocks) * packed_block_bytes(D, F));
+    n_rows = rows + M + B + 1;
+    const int rc_rows = taac_valid_rows(key_lengths, B, T, rows, n_rows, stream);
+    if (rc_rows != TAAC_OK) return rc_rows;
+  }
 
   const int dh = D / heads;
   const int64_t qkv_strides[4] = {static_cast<int64_t>(T) * 3 * D, dh, 3 * static_cast<int64_t>(D), 1};
@@ -154,7 +241,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
       if ((rc = taac_linear_pack_weights(w.out_weight, pk_out, D, D, stream)) != TAAC_OK) return rc;
       if ((rc = taac_ffn_pack_weights(w.up_weight, w.down_weight, pk_ffn, D, F, 1, stream)) != TAAC_OK) return rc;
       if ((rc = taac_norm_linear_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, nullptr, 0, qkv,
-                                     3 * D, M, 3 * D, D, stream)) != TAAC_OK)
+                                     3 * D, M, 3 * D, D, rows, n_rows, stream)) != TAAC_OK)
         return rc;
     } else {
       if ((rc = taac_rmsnorm_fwd(cur, w.attn_norm_weight, h, M, D, eps, TAAC_BF16, stream)) != TAAC_OK) return rc;
@@ -163,15 +250,15 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
         return rc;
     }
     if ((rc = taac_flash_attn_fwd(qkv, qkv + D, qkv + 2 * D, key_lengths, h, B, heads, T, T, dh, qkv_strides,
-                                  qkv_strides, qkv_strides, o_strides, 0, 1, TAAC_BF16, stream)) != TAAC_OK)
+                                  qkv_strides, qkv_strides, o_strides, 0, rows ? 2 : 1, TAAC_BF16, stream)) != TAAC_OK)
       return rc;
     if (fused) {
-      if ((rc = taac_norm_linear_fwd(h, D, nullptr, eps, nullptr, w.out_bias, pk_out, cur, D, x, D, M, D, D,
-                                     stream)) != TAAC_OK)
+      if ((rc = taac_norm_linear_fwd(h, D, nullptr, eps, nullptr, w.out_bias, pk_out, cur, D, x, D, M, D, D, rows,
+                                     n_rows, stream)) != TAAC_OK)
         return rc;
       // feed-forward half: RMSNorm -> up -> SiLU-gate -> down -> + residual in one kernel
       if ((rc = taac_swiglu_ffn_fwd(x, D, w.ffn_norm_weight, eps, nullptr, w.up_bias, nullptr, w.down_bias, pk_ffn, x,
-                                    D, x_out, D, M, D, F, 1, stream)) != TAAC_OK)
+                                    D, x_out, D, M, D, F, 1, rows, n_rows, stream)) != TAAC_OK)
         return rc;
     } else {
       if ((rc = taac_linear_bf16(h, D, w.out_weight, w.out_bias, cur, x, D, M, D, D, TAAC_EPI_RESIDUAL, 1, stream)) !=
@@ -186,6 +273,13 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
         return rc;
     }
     cur = x_out;
+  }
+  if (rows != nullptr && hidden_out != nullptr) {
+    // The padded positions of the returned hidden state were never written: define them as zeros.
+    const int64_t pieces = static_cast<int64_t>(T) * (D / 8);
+    hipLaunchKernelGGL(zero_padded_rows_kernel, dim3(static_cast<uint32_t>((pieces + kBlock - 1) / kBlock), B),
+                       dim3(kBlock), 0, as_stream(stream), static_cast<bf16_t*>(hidden_out), key_lengths, T, D);
+    if ((rc = check_launch(name)) != TAAC_OK) return rc;
   }
   if (n_blocks == 0 && hidden_out != nullptr) {
     if (hipMemcpyAsync(hidden_out, emb, static_cast<size_t>(M) * D * 2, hipMemcpyDeviceToDevice, as_stream(stream)) !=

@@ -52,7 +52,8 @@ struct TsParams {
   float eps;
   int32_t gate_first;
   int32_t packed;           // weights are in fragment order
-  int32_t stagger;          // linear: wavefront groups may change token tiles out of phase (x does not alias out)
+  const int32_t* rows;      // optional row index: token i lives in row rows[i] of x / residual / out
+  const int32_t* n_rows;    // with rows: device pointer to the number of tokens (at most M)
 };
 
 __device__ __forceinline__ float silu_f(float v) {
@@ -104,18 +105,30 @@ __global__ void linear_pack_kernel(const bf16_t* __restrict__ w, bf16x8* __restr
 
 // ---- shared pieces ---------------------------------------------------------------------------------------------------
 
+// Number of tokens to process: M, or *n_rows (clamped to M) when a row index is given.
+__device__ __forceinline__ int64_t token_count(const TsParams& p) {
+  if (p.rows == nullptr) return p.M;
+  const int64_t n = *p.n_rows;
+  return n < p.M ? n : p.M;
+}
+
+// Row of x / residual / out that holds token `tok`. Tokens at or beyond the count are mapped to the last token: they
+// compute bit-identical values, so loading and storing them again is benign and every wavefront issues the same
+// number of memory operations.
+__device__ __forceinline__ int64_t token_row(const TsParams& p, int64_t count, int64_t tok) {
+  tok = tok < count ? tok : count - 1;
+  return p.rows != nullptr ? static_cast<int64_t>(p.rows[tok]) : tok;
+}
+
 // Loads the wavefront's token rows as B-operand fragments: lane (l32, hh) holds features 16*ks + 8*hh .. +7 of token
 // l32 of each 32-token tile.
 template <int D, int TT>
-__device__ __forceinline__ void load_token_rows(const TsParams& p, int64_t tok0, int l32, int hh,
+__device__ __forceinline__ void load_token_rows(const TsParams& p, int64_t count, int64_t tok0, int l32, int hh,
                                                 bf16x8 (&xf)[TT][D / 16]) {
   constexpr int KS = D / 16;
 #pragma unroll
   for (int t = 0; t < TT; ++t) {
-    // Rows beyond M are clamped to the last row: their results are bit-identical to that row's.
-    int64_t tok = tok0 + t * 32 + l32;
-    tok = tok < p.M ? tok : p.M - 1;
-    const bf16_t* row = p.x + tok * p.ldx + hh * 8;
+    const bf16_t* row = p.x + token_row(p, count, tok0 + t * 32 + l32) * p.ldx + hh * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) xf[t][ks] = *reinterpret_cast<const bf16x8*>(row + ks * 16);
   }
@@ -196,31 +209,28 @@ __device__ __forceinline__ void tile_to_lds(uint8_t* tile, const f32x16& a0, con
 
 // Reads the epilogue tile back row-wise (lane -> token 8*i + lane/8, features 8*(lane%8) .. +7), adds the residual
 // pieces loaded earlier and stores 16 bytes per lane: every 128-byte row segment is written by 8 consecutive lanes.
+// prow[i] is the memory row of token 8*i + lane/8 of the tile, live[i] whether that token exists.
 template <bool RES>
-__device__ __forceinline__ void tile_to_global(const uint8_t* tile, bf16_t* out, int64_t ldo, int64_t tok_base,
-                                               int64_t M, int col0, const bf16x8 (&res)[4], int lane) {
+__device__ __forceinline__ void tile_to_global(const uint8_t* tile, bf16_t* out, int64_t ldo, const int64_t (&prow)[4],
+                                               const bool (&live)[4], int col0, const bf16x8 (&res)[4], int lane) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int row = i * 8 + lane / 8;
-    const int64_t tok = tok_base + row;
     bf16x8 v = *reinterpret_cast<const bf16x8*>(tile + row * kStageRow + (lane % 8) * 16);
     if (RES) {
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         v[e] = static_cast<bf16_t>(static_cast<float>(v[e]) + static_cast<float>(res[i][e]));
     }
-    if (tok < M) *reinterpret_cast<bf16x8*>(out + tok * ldo + col0 + (lane % 8) * 8) = v;
+    if (live[i]) *reinterpret_cast<bf16x8*>(out + prow[i] * ldo + col0 + (lane % 8) * 8) = v;
   }
 }
 
-__device__ __forceinline__ void load_residual(const bf16_t* residual, int64_t ldr, int64_t tok_base, int64_t M,
-                                              int col0, bf16x8 (&res)[4], int lane) {
+__device__ __forceinline__ void load_residual(const bf16_t* residual, int64_t ldr, const int64_t (&prow)[4], int col0,
+                                              bf16x8 (&res)[4], int lane) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int64_t tok = tok_base + i * 8 + lane / 8;
-    tok = tok < M ? tok : M - 1;
-    res[i] = *reinterpret_cast<const bf16x8*>(residual + tok * ldr + col0 + (lane % 8) * 8);
-  }
+  for (int i = 0; i < 4; ++i)
+    res[i] = *reinterpret_cast<const bf16x8*>(residual + prow[i] * ldr + col0 + (lane % 8) * 8);
 }
 
 // ------------------------------------------------------------------------------------------------------------------
@@ -252,6 +262,8 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
   const int lane = tid % kWave;
   const int l32 = lane % 32;
   const int hh = lane / 32;
+  const int64_t count = token_count(p);
+  if (static_cast<int64_t>(blockIdx.x) * kTokPerWg >= count) return;  // whole workgroup: no tokens left for it
   const int64_t tok0 = static_cast<int64_t>(blockIdx.x) * kTokPerWg + wave * (32 * TT);
   const int F = p.F;
   const int nsteps = F / (kHU * CPB);
@@ -297,7 +309,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
   if (p.norm_w != nullptr) stage_bias(p.norm_w, bias_lds + 2 * F + D, D, tid, NWAVES * kWave);
 
   bf16x8 xf[TT][KS];
-  load_token_rows<D, TT>(p, tok0, l32, hh, xf);
+  load_token_rows<D, TT>(p, count, tok0, l32, hh, xf);
 
   f32x16 oacc[TT][MB];
 #pragma unroll
@@ -449,18 +461,25 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 #pragma unroll
   for (int t = 0; t < TT; ++t) {
     const int64_t tok_base = tok0 + t * 32;
+    int64_t prow[4];
+    bool live[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      prow[i] = token_row(p, count, tok_base + i * 8 + lane / 8);
+      live[i] = tok_base + i * 8 + lane / 8 < count;
+    }
 #pragma unroll
     for (int pr = 0; pr < MB / 2; ++pr) {  // 64 features at a time
       bf16x8 res[4];
-      if (p.residual != nullptr) load_residual(p.residual, p.ldr, tok_base, p.M, pr * 64, res, lane);
+      if (p.residual != nullptr) load_residual(p.residual, p.ldr, prow, pr * 64, res, lane);
       bf16x4 bv[8];
       read_chunk_bias(bdown_lds + pr * 64, hh, bv);
       tile_to_lds(tile, oacc[t][2 * pr], oacc[t][2 * pr + 1], bv, l32, hh);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       if (p.residual != nullptr)
-        tile_to_global<true>(tile, p.out, p.ldo, tok_base, p.M, pr * 64, res, lane);
+        tile_to_global<true>(tile, p.out, p.ldo, prow, live, pr * 64, res, lane);
       else
-        tile_to_global<false>(tile, p.out, p.ldo, tok_base, p.M, pr * 64, res, lane);
+        tile_to_global<false>(tile, p.out, p.ldo, prow, live, pr * 64, res, lane);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -483,13 +502,13 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 //       [RES: NST residual loads of step s+1] [FPW weight DMAs of step s+2] ... [NST output stores of step s]
 //     (NST = 4 per 32-token tile) and the step ends with vmcnt(FPW + NST) (vmcnt(NST) when no DMA was issued): the
 //     weights of step s+1 have landed, the weights of step s+2 and the stores of step s may stay in flight.
-//   Every wavefront issues at least these counts after the transfer it waits for: rows beyond M are clamped to row
-//   M-1 for loads AND stores (the clamped rows compute bit-identical values, so the duplicate stores are benign),
+//   Every wavefront issues at least these counts after the transfer it waits for: tokens beyond the count are mapped
+//   to the last token for loads AND stores (they compute bit-identical values, so the duplicate stores are benign),
 //   and the "memory" clobbers of the hand-written statements keep loads and stores on their side of them.
 // LDS: [3 weight buffers of 2*KS fragments][8 epilogue tiles][bias (N) | norm weight (D)]
 // ------------------------------------------------------------------------------------------------------------------
 template <int D, int TT, bool RES>
-__global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParams p, const int num_tiles) {
+__global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParams p) {
   constexpr int NWAVES = 8;
   constexpr int kTokPerWg = NWAVES * 32 * TT;  // TT token tiles of 32 per wavefront
   constexpr int KS = D / 16;
@@ -508,6 +527,9 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
   const int l32 = lane % 32;
   const int hh = lane / 32;
   const int nchunks = p.N / kNC;
+  const int64_t count = token_count(p);
+  const int num_tiles = static_cast<int>((count + kTokPerWg - 1) / kTokPerWg);
+  if (static_cast<int>(blockIdx.x) >= num_tiles) return;  // whole workgroup: no token tile for it
   const int my_tiles = (num_tiles - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) /
                        static_cast<int>(gridDim.x);
   const int total = my_tiles * nchunks;
@@ -532,30 +554,25 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
       lds_dma16(w_bytes + (row0 * D + (f % KS) * 16) * 2 + lane_off, base + i * kFrag);
     }
   };
-  // Two phase groups. Wavefronts 4..7 change token tiles half a tile (nchunks / 2 steps) later than wavefronts 0..3:
-  // the output chunks of a tile are independent, so a wavefront may walk them in any cyclic order, and with the two
-  // groups out of phase the token loads and the RMSNorm arithmetic of one group run under the MFMAs of the other
-  // (one wavefront of each group per SIMD). A wavefront of the late group sees the token tiles as slots
-  // 0, 1, ..., my_tiles - 1, 0: chunks [0, nchunks/2) of its first tile at the start, the rest of them at the end
-  // (it loads that tile's rows twice, so the host switches this off when the output overwrites the input).
-  const bool late = p.stagger && (nchunks % 2 == 0) && wave >= NWAVES / 2;
-  const int switch_chunk = late ? nchunks / 2 : 0;
-  auto rows_of_slot = [&](int slot) -> int64_t {
-    const int idx = slot < my_tiles ? slot : 0;
+  // First token of this wavefront in the workgroup's idx-th tile.
+  auto tokens_of_tile = [&](int idx) -> int64_t {
     return (static_cast<int64_t>(blockIdx.x) + static_cast<int64_t>(idx) * gridDim.x) * kTokPerWg + wave * (32 * TT);
   };
-  // Residual pieces of (rows, chunk) in the layout of the epilogue stores: piece i = token 8*i + lane/8, 16 bytes.
-  auto request_residual = [&](int64_t tok_base, int chunk, bf16x8 (&res)[NST]) {
+  // Memory rows of a tile in the layout of the epilogue stores: piece i = token (i / 4) * 32 + 8 * (i % 4) + lane / 8.
+  auto rows_of_tile = [&](int64_t tok_base, int32_t (&prow)[NST]) {
 #pragma unroll
-    for (int i = 0; i < NST; ++i) {
-      int64_t tok = tok_base + i * 8 + lane / 8;
-      tok = tok < p.M ? tok : p.M - 1;
-      res[i] = *reinterpret_cast<const bf16x8*>(p.residual + tok * p.ldr + chunk * kNC + (lane % 8) * 8);
-    }
+    for (int i = 0; i < NST; ++i)
+      prow[i] = static_cast<int32_t>(token_row(p, count, tok_base + (i / 4) * 32 + (i % 4) * 8 + lane / 8));
+  };
+  auto request_residual = [&](const int32_t (&prow)[NST], int chunk, bf16x8 (&res)[NST]) {
+#pragma unroll
+    for (int i = 0; i < NST; ++i)
+      res[i] = *reinterpret_cast<const bf16x8*>(p.residual + static_cast<int64_t>(prow[i]) * p.ldr + chunk * kNC +
+                                                (lane % 8) * 8);
   };
   bf16x8 xf[TT][KS];
-  auto load_slot = [&](int64_t tok_base) {
-    load_token_rows<D, TT>(p, tok_base, l32, hh, xf);
+  auto load_tile = [&](int64_t tok_base) {
+    load_token_rows<D, TT>(p, count, tok_base, l32, hh, xf);
     // Consume the rows right here: otherwise the compiler's wait for them lands in front of the first MFMA of EVERY
     // step, where it also waits for the weights and stores that are meant to stay in flight.
 #pragma unroll
@@ -565,14 +582,16 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
   };
 
   bf16x8 res_cur[NST], res_next[NST];
-  int slot = 0;
-  int64_t tok_wave = rows_of_slot(0);                 // first token row of this wavefront's current tile
+  int32_t prow[NST], prow_next[NST];  // rows of the current tile / of the tile the next step belongs to
+  int tile_idx = 0;
+  int64_t tok_wave = tokens_of_tile(0);
+  rows_of_tile(tok_wave, prow);
   stage(0, 0);
   if (total > 1) stage(nchunks > 1 ? 1 : 0, 1);
-  if (RES) request_residual(tok_wave, 0, res_cur);
+  if (RES) request_residual(prow, 0, res_cur);
   stage_bias(p.b1, bias_lds, p.N, tid, NWAVES * kWave);
   if (p.norm_w != nullptr) stage_bias(p.norm_w, bias_lds + p.N, D, tid, NWAVES * kWave);
-  load_slot(tok_wave);
+  load_tile(tok_wave);
   vm_wait<0>();
   __syncthreads();
   if (p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + p.N, hh, xf);
@@ -585,17 +604,29 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     // ---- requests for later steps ------------------------------------------------------------------------------------
     const bool has_next = s + 1 < total;
     const bool stage_ahead = s + 2 < total;
-    const bool new_tile = s > 0 && chunk == switch_chunk;  // this wavefront moves to its next token tile in this step
-    if (new_tile) tok_wave = rows_of_slot(++slot);
+    const bool new_tile = s > 0 && chunk == 0;  // the workgroup moves to its next token tile in this step
+    if (new_tile) {
+      tok_wave = tokens_of_tile(++tile_idx);
+      if (RES) {
+#pragma unroll
+        for (int i = 0; i < NST; ++i) prow[i] = prow_next[i];
+      } else {
+        rows_of_tile(tok_wave, prow);
+      }
+    }
     if (RES && has_next) {
-      const int next_chunk = chunk + 1 == nchunks ? 0 : chunk + 1;
-      request_residual(next_chunk == switch_chunk ? rows_of_slot(slot + 1) : tok_wave, next_chunk, res_next);
+      if (chunk + 1 == nchunks) {  // the next step opens the next tile
+        rows_of_tile(tokens_of_tile(tile_idx + 1), prow_next);
+        request_residual(prow_next, 0, res_next);
+      } else {
+        request_residual(prow, chunk + 1, res_next);
+      }
     }
     if (stage_ahead) stage(chunk2, buf == 0 ? 2 : buf - 1);  // slot (s + 2) % 3, last read in step s - 1
     if (new_tile) {
       // The rows are requested after the weights and residual pieces of the later steps, so that those are not held
-      // back by the wait for the rows (the compiler's wait for these loads is a full vmcnt(0), once per tile).
-      load_slot(tok_wave);
+      // back by the wait for the rows.
+      load_tile(tok_wave);
       if (p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + p.N, hh, xf);
     }
 
@@ -649,19 +680,17 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     for (int t = 0; t < TT; ++t) {
       tile_to_lds(tile_lds, acc0[t], acc1[t], bv, l32, hh);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      const int64_t tok_base = tok_wave + t * 32;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int row = i * 8 + lane / 8;
-        int64_t tok = tok_base + row;
-        tok = tok < p.M ? tok : p.M - 1;
         bf16x8 v = *reinterpret_cast<const bf16x8*>(tile_lds + row * kStageRow + (lane % 8) * 16);
         if (RES) {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
             v[e] = static_cast<bf16_t>(static_cast<float>(v[e]) + static_cast<float>(res_cur[t * 4 + i][e]));
         }
-        *reinterpret_cast<bf16x8*>(p.out + tok * p.ldo + chunk * kNC + (lane % 8) * 8) = v;
+        *reinterpret_cast<bf16x8*>(p.out + static_cast<int64_t>(prow[t * 4 + i]) * p.ldo + chunk * kNC +
+                                   (lane % 8) * 8) = v;
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
@@ -759,7 +788,8 @@ extern "C" int taac_linear_pack_weights(const void* w, void* packed, int32_t N, 
 extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w_up,
                                    const void* b_up, const void* w_down, const void* b_down, const void* packed_weights,
                                    const void* residual, int64_t ldr, void* out, int64_t ldo, int64_t M, int32_t D,
-                                   int32_t F, int gate_first, void* stream) {
+                                   int32_t F, int gate_first, const int32_t* rows, const int32_t* n_rows,
+                                   void* stream) {
   using namespace taac;
   const char* name = "taac_swiglu_ffn_fwd";
   if (M < 0 || D <= 0 || F <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, D and F > 0", name);
@@ -772,6 +802,9 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
   if (M == 0) return TAAC_OK;
   if (!x || !out || (!packed_weights && (!w_up || !w_down)))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
+  if ((rows == nullptr) != (n_rows == nullptr))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows and n_rows must be given together", name);
+  if (rows && M > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: a row index covers at most 2^31 rows", name);
   if (!ptr_ok(x, 15) || !ptr_ok(w_up, 15) || !ptr_ok(w_down, 15) || !ptr_ok(out, 15) || !ptr_ok(residual, 15) ||
       !ptr_ok(norm_weight, 15) || !ptr_ok(b_up, 15) || !ptr_ok(b_down, 15) || !ptr_ok(packed_weights, 15))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
@@ -794,6 +827,8 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
   p.eps = eps;
   p.gate_first = gate_first ? 1 : 0;
   p.packed = packed_weights ? 1 : 0;
+  p.rows = rows;
+  p.n_rows = n_rows;
   hipStream_t s = as_stream(stream);
   const int KS = D / 16, MB = D / 32;
   const size_t bias_bytes = static_cast<size_t>(2 * F + 2 * D) * 2;
@@ -814,7 +849,8 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
 
 extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
                                     const void* bias, const void* packed_weights, const void* residual, int64_t ldr,
-                                    void* out, int64_t ldo, int64_t M, int32_t N, int32_t K, void* stream) {
+                                    void* out, int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows,
+                                    const int32_t* n_rows, void* stream) {
   using namespace taac;
   const char* name = "taac_norm_linear_fwd";
   if (M < 0 || N <= 0 || K <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, N and K > 0", name);
@@ -825,6 +861,9 @@ extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: row strides must cover a row and be multiples of 8", name);
   if (M == 0) return TAAC_OK;
   if (!x || !out || (!packed_weights && !w)) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
+  if ((rows == nullptr) != (n_rows == nullptr))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows and n_rows must be given together", name);
+  if (M > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: at most 2^31 rows", name);
   if (!ptr_ok(x, 15) || !ptr_ok(w, 15) || !ptr_ok(out, 15) || !ptr_ok(residual, 15) || !ptr_ok(norm_weight, 15) ||
       !ptr_ok(bias, 15) || !ptr_ok(packed_weights, 15))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
@@ -845,20 +884,15 @@ extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm
   p.N = N;
   p.eps = eps;
   p.packed = packed_weights ? 1 : 0;
-  {
-    const char* x_lo = static_cast<const char*>(x);
-    const char* x_hi = x_lo + ((M - 1) * ldx + K) * 2;
-    const char* o_lo = static_cast<const char*>(out);
-    const char* o_hi = o_lo + ((M - 1) * ldo + N) * 2;
-    p.stagger = (o_hi <= x_lo || x_hi <= o_lo) ? 1 : 0;
-  }
+  p.rows = rows;
+  p.n_rows = n_rows;
   hipStream_t s = as_stream(stream);
   // Without a residual two token tiles per wavefront fit the register file: every weight fragment read from LDS then
   // feeds two MFMAs, which halves the LDS traffic that otherwise caps the kernel.
   const int tt = residual ? 1 : 2;
   const int64_t tiles64 = (M + 256 * tt - 1) / (256 * tt);
   if (tiles64 > 0x3fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many token tiles", name);
-  const int num_tiles = static_cast<int>(tiles64);
+  const int num_tiles = static_cast<int>(tiles64);  // upper bound: with a row index the kernel derives its own
   const int cus = compute_units();
   if (cus <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
   int grid = num_tiles < cus ? num_tiles : cus;
@@ -874,7 +908,7 @@ extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(norm_linear_kernel<KK, TT, RR>),                            \
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)) != hipSuccess) \
       return set_error(TAAC_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", name, lds_bytes);                  \
-    hipLaunchKernelGGL((norm_linear_kernel<KK, TT, RR>), dim3(grid), dim3(8 * kWave), lds_bytes, s, p, num_tiles);    \
+    hipLaunchKernelGGL((norm_linear_kernel<KK, TT, RR>), dim3(grid), dim3(8 * kWave), lds_bytes, s, p);               \
     return check_launch(name);                                                                                    \
   } while (0)
   if (K == 256) {

@@ -57,6 +57,26 @@ def test_backbone_matches_oracle(device, batch, n_feature, n_sequence):
     assert torch.isfinite(hidden).all()
 
 
+def test_backbone_skips_padded_positions(device, monkeypatch):
+    """The fused forward walks the valid tokens only: garbage (NaN) at the padded positions of the embeddings changes
+    nothing, the valid rows of the hidden state are bit-identical to the run over all B*T positions
+    (TAAC_DENSE_TOKENS), and the padded rows of the returned hidden state are zeros."""
+    inputs = workloads.backbone_inputs(batch=7, n_feature_tokens=32, n_sequence_tokens=224, min_sequence_len=16, seed=3)
+    tokens = inputs.emb.shape[1]
+    valid = torch.arange(tokens)[None, :] < inputs.key_lengths[:, None]
+    p_ref, h_ref = _run(inputs, device)
+    poisoned = workloads.BackboneInputs(inputs.emb.clone(), inputs.key_lengths, inputs.blocks, inputs.head_weight,
+                                        inputs.head_bias, inputs.num_heads, inputs.d_ff)
+    poisoned.emb[~valid] = float("nan")
+    p_poisoned, h_poisoned = _run(poisoned, device)
+    assert torch.equal(p_poisoned, p_ref) and torch.equal(h_poisoned, h_ref)
+    assert (h_ref.cpu()[~valid] == 0).all()
+    monkeypatch.setenv("TAAC_DENSE_TOKENS", "1")
+    p_dense, h_dense = _run(inputs, device)
+    assert torch.equal(p_dense, p_ref)
+    assert torch.equal(h_dense.cpu()[valid], h_ref.cpu()[valid])
+
+
 def test_backbone_config4_full_size(device):
     """Config 4 at full size (B=1024, T=512): a slice of samples against the oracle; all outputs finite; batch rows
     independent (a sample gives the same probability alone and inside the batch)."""

@@ -240,6 +240,66 @@ def test_fused_norm_linear_walks_several_token_tiles(device, monkeypatch, workgr
     torch.testing.assert_close(plain.cpu().float(), F.linear(x.float(), w.float()), **BF16_TOL)
 
 
+def test_valid_rows_index(device):
+    """Row index of a padded batch: valid rows in increasing order, count, per-sample offsets; lengths are clamped to
+    [0, T]."""
+    from taac_2026_amd.api import valid_rows
+
+    tokens = 37
+    lengths = torch.tensor([5, 0, 37, 12, 99, -3, 1], dtype=torch.int32)
+    rows, count = valid_rows(lengths.to(device), tokens)
+    clamped = lengths.clamp(0, tokens)
+    expected = torch.cat([b * tokens + torch.arange(int(n)) for b, n in enumerate(clamped)]).to(torch.int32)
+    n = int(count.item())
+    assert n == int(clamped.sum())
+    assert torch.equal(rows[:n].cpu(), expected)
+    offsets = rows[len(lengths) * tokens:len(lengths) * tokens + len(lengths) + 1].cpu()
+    assert torch.equal(offsets, torch.cat([torch.zeros(1, dtype=torch.int64), clamped.cumsum(0)]).to(torch.int32))
+    big = torch.randint(0, 513, (3000,), dtype=torch.int32, generator=torch.Generator().manual_seed(0))
+    rows, count = valid_rows(big.to(device), 512)
+    assert int(count.item()) == int(big.sum())
+    mask = torch.arange(512)[None, :] < big[:, None]
+    assert torch.equal(rows[:int(count.item())].cpu().long(), mask.flatten().nonzero().flatten())
+
+
+@pytest.mark.parametrize("workgroups", [None, 2])
+def test_fused_layers_skip_padded_rows(device, monkeypatch, workgroups):
+    """With a row index the fused layers process exactly the valid rows of a padded batch: those rows are bit-identical
+    to the dense run, all other rows are neither read (they hold NaN here) nor written."""
+    from taac_2026_amd.api import norm_linear, swiglu_ffn, valid_rows
+
+    if workgroups is not None:
+        monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+    g = torch.Generator().manual_seed(21)
+    batch, tokens, d, f = 9, 200, 256, 96
+    lengths = torch.tensor([200, 1, 0, 77, 128, 199, 33, 64, 160], dtype=torch.int32)
+    valid = (torch.arange(tokens)[None, :] < lengths[:, None]).flatten()
+    x = torch.randn(batch * tokens, d, generator=g).to(torch.bfloat16)
+    res = torch.randn(batch * tokens, d, generator=g).to(torch.bfloat16)
+    nw = (1 + 0.1 * torch.randn(d, generator=g)).to(torch.bfloat16)
+    _, w, b = _draw(1, 768, d, seed=1)
+    _, wo, bo = _draw(1, d, d, seed=2)
+    _, wu, bu = _draw(1, 2 * f, d, seed=3)
+    _, wd, bd = _draw(1, d, f, seed=4)
+    poisoned = x.clone()
+    poisoned[~valid] = float("nan")
+    res_poisoned = res.clone()
+    res_poisoned[~valid] = float("nan")
+    to = lambda t: t.to(device)
+    with torch.no_grad():
+        index = valid_rows(to(lengths), tokens)
+        dense_qkv = norm_linear(to(x), to(w), to(b), norm_weight=to(nw))
+        skip_qkv = norm_linear(to(poisoned), to(w), to(b), norm_weight=to(nw), token_rows=index)
+        dense_out = norm_linear(to(x), to(wo), to(bo), residual=to(res))
+        skip_out = norm_linear(to(poisoned), to(wo), to(bo), residual=to(res_poisoned), token_rows=index)
+        dense_ffn = swiglu_ffn(to(x), to(wu), to(bu), to(wd), to(bd), residual=to(res), norm_weight=to(nw))
+        skip_ffn = swiglu_ffn(to(poisoned), to(wu), to(bu), to(wd), to(bd), residual=to(res_poisoned), norm_weight=to(nw),
+                              token_rows=index)
+    for dense, skipped in ((dense_qkv, skip_qkv), (dense_out, skip_out), (dense_ffn, skip_ffn)):
+        assert torch.equal(skipped.cpu()[valid], dense.cpu()[valid])
+        assert (skipped.cpu()[~valid] == 0).all()
+
+
 def test_fused_paths_fall_back_for_other_widths(device):
     from taac_2026_amd.api import norm_linear, swiglu_ffn
 
