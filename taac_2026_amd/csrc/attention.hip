@@ -20,6 +20,8 @@
 // P rounded to the storage dtype before the second product, rows with an empty visible set produce 0.
 #include <math.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace taac {
@@ -221,54 +223,65 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
     __syncthreads();
     if (kc0 + kKC < kv_end) fetch(kc0 + kKC);
 
+    // One softmax update per chunk: both 32-key tiles when the second one has a visible key for this wavefront
+    // (NT = 2), the first tile alone otherwise (NT = 1). Per update: scores S^T (NT tiles of 32 keys x 32 queries),
+    // running max / sum of one query per lane pair, P rounded to the storage type, one rescale of O^T, O^T += V^T P^T.
+    if (kc0 >= wave_kv_end) continue;  // wavefront-uniform: nothing visible in this chunk (padding / causal bound)
+    auto update = [&](auto nt_tag) {
+      constexpr int NT = decltype(nt_tag)::value;
+      f32x16 sacc[NT];
 #pragma unroll
-    for (int kt = 0; kt < kKC / 32; ++kt) {
-      const int k0 = kc0 + kt * 32;
-      if (k0 >= wave_kv_end) break;  // wavefront-uniform
-
-      // ---- S^T tile: 32 keys x 32 queries ---------------------------------------------------------------
-      f32x16 sacc;
+      for (int kt = 0; kt < NT; ++kt) {
 #pragma unroll
-      for (int j = 0; j < 16; ++j) sacc[j] = 0.f;
+        for (int j = 0; j < 16; ++j) sacc[kt][j] = 0.f;
 #pragma unroll
-      for (int s = 0; s < KSTEPS; ++s) {
-        const vec_t a = *reinterpret_cast<const vec_t*>(&sK[(kt * 32 + l32) * KSTR + 16 * s + 8 * hh]);
-        sacc = Mfma32<T>::run(a, qf[s], sacc);
-      }
-      const bool tail = (k0 + 32 > kv_end) || (CAUSAL && (k0 + 31 > q_begin + wave * 32));
-      if (tail) {
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          const int key = k0 + (j / 4) * 8 + hh * 4 + (j % 4);
-          const bool masked = key >= kv_end || (CAUSAL && key > qi);
-          if (masked) sacc[j] = -INFINITY;
+        for (int s = 0; s < KSTEPS; ++s) {
+          const vec_t a = *reinterpret_cast<const vec_t*>(&sK[(kt * 32 + l32) * KSTR + 16 * s + 8 * hh]);
+          sacc[kt] = Mfma32<T>::run(a, qf[s], sacc[kt]);
         }
       }
-      // ---- online softmax, one query per lane (pair of lanes l, l ^ 32) ------------------------------------
-      float mx = sacc[0];
+      const int k_last = kc0 + NT * 32;  // one past the last key of this update
+      const bool tail = (k_last > kv_end) || (CAUSAL && (k_last - 1 > q_begin + wave * 32));
+      if (tail) {
 #pragma unroll
-      for (int j = 1; j < 16; ++j) mx = fmaxf(mx, sacc[j]);
+        for (int kt = 0; kt < NT; ++kt)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) {
+            const int key = kc0 + kt * 32 + (j / 4) * 8 + hh * 4 + (j % 4);
+            const bool masked = key >= kv_end || (CAUSAL && key > qi);
+            if (masked) sacc[kt][j] = -INFINITY;
+          }
+      }
+      // ---- online softmax, one query per lane (pair of lanes l, l ^ 32) ------------------------------------
+      float mx = sacc[0][0];
+#pragma unroll
+      for (int kt = 0; kt < NT; ++kt)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) mx = fmaxf(mx, sacc[kt][j]);
       mx = pair_max(mx);
       const float m_new = fmaxf(m_run, mx);
       const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
       const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
       const float mc = -m_use * c;
-      float pr[16];
       float rs = 0.f;
+      vec_t pb[NT][2];
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        pr[j] = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, mc));
-        rs += pr[j];
+      for (int kt = 0; kt < NT; ++kt) {
+        float pr[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          pr[j] = __builtin_amdgcn_exp2f(fmaf(sacc[kt][j], c, mc));
+          rs += pr[j];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          pb[kt][0][e] = static_cast<T>(pr[e]);
+          pb[kt][1][e] = static_cast<T>(pr[8 + e]);
+        }
       }
       rs = pair_sum(rs);
       l_run = l_run * alpha + rs;
       m_run = m_new;
-      vec_t pb[2];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        pb[0][e] = static_cast<T>(pr[e]);
-        pb[1][e] = static_cast<T>(pr[8 + e]);
-      }
       // ---- O^T += V^T P^T --------------------------------------------------------------------------------
       // The rescale is unconditional on purpose: a wavefront-uniform branch around it placed the accumulator read-back
       // of the preceding MFMA on a path without the required wait states (wrong values in the last accumulator register).
@@ -277,13 +290,19 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 #pragma unroll
         for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          const vec_t a =
-              *reinterpret_cast<const vec_t*>(&sVt[(mb * 32 + l32) * VSTR + kt * 32 + s2 * 16 + hh * 8]);
-          oacc[mb] = Mfma32<T>::run(a, pb[s2], oacc[mb]);
-        }
+        for (int kt = 0; kt < NT; ++kt)
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            const vec_t a =
+                *reinterpret_cast<const vec_t*>(&sVt[(mb * 32 + l32) * VSTR + kt * 32 + s2 * 16 + hh * 8]);
+            oacc[mb] = Mfma32<T>::run(a, pb[kt][s2], oacc[mb]);
+          }
       }
-    }
+    };
+    if (kc0 + 32 < wave_kv_end)
+      update(std::integral_constant<int, 2>{});
+    else
+      update(std::integral_constant<int, 1>{});
   }
 
   // ---- finalise: O / l (0 for rows in the padding), transpose through a wavefront-private LDS tile, 16-byte stores --

@@ -490,8 +490,8 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 // [RMSNorm ->] linear [-> + residual], K = D, N a multiple of 64
 //
 // Persistent: a workgroup (8 wavefronts x TT tiles of 32 tokens) walks token tiles blockIdx.x, blockIdx.x + gridDim.x, ...; for
-// each tile it walks the N / 64 output chunks. The weight chunks form one endless stream over the global step number
-// s = tile_index * nchunks + chunk, staged by DMA into a ring of three LDS buffers two steps ahead of their use, so
+// each tile it walks the N / 64 output chunks (the tiles of the last, partial round are split by chunks over several
+// workgroups). The weight chunks form one endless stream over the workgroup's step number, staged by DMA into a ring of three LDS buffers two steps ahead of their use, so
 // the stream never drains at a tile boundary.
 //
 // Memory-counter discipline. The weight transfers are issued by hand (lds_dma16) and are invisible to the compiler,
@@ -529,10 +529,27 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
   const int nchunks = p.N / kNC;
   const int64_t count = token_count(p);
   const int num_tiles = static_cast<int>((count + kTokPerWg - 1) / kTokPerWg);
-  if (static_cast<int>(blockIdx.x) >= num_tiles) return;  // whole workgroup: no token tile for it
-  const int my_tiles = (num_tiles - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) /
-                       static_cast<int>(gridDim.x);
-  const int total = my_tiles * nchunks;
+  // Work split. The first full_rounds * gridDim.x tiles go round-robin to the workgroups, every one with all of its
+  // output chunks. The R = num_tiles % gridDim.x tiles that remain would keep R workgroups busy for a whole tile
+  // while the others idle, so each of them is split by output chunks (they are independent) into S = gridDim.x / R
+  // segments handled by different workgroups, which all load the tile's rows.
+  const int G = static_cast<int>(gridDim.x);
+  const int wg = static_cast<int>(blockIdx.x);
+  const int full_rounds = num_tiles / G;
+  const int R = num_tiles % G;
+  int S = R > 0 ? G / R : 1;
+  S = S < nchunks ? S : nchunks;
+  const bool has_tail = R > 0 && wg < R * S;
+  const int tail_tile = full_rounds * G + wg / S;
+  const int tail_begin = has_tail ? ((wg % S) * nchunks) / S : 0;
+  const int tail_len = has_tail ? (((wg % S) + 1) * nchunks) / S - tail_begin : 0;
+  const int full_total = full_rounds * nchunks;
+  const int total = full_total + tail_len;
+  if (total == 0) return;  // whole workgroup: nothing assigned to it
+  // Step s of this workgroup works on chunk_of(s) of tile tile_of(s); first_of_tile(s) opens a new tile.
+  auto chunk_of = [&](int step) -> int { return step < full_total ? step % nchunks : tail_begin + (step - full_total); };
+  auto tile_of = [&](int step) -> int { return step < full_total ? wg + (step / nchunks) * G : tail_tile; };
+  auto first_of_tile = [&](int step) -> bool { return step < full_total ? step % nchunks == 0 : step == full_total; };
 
   // fragment f of a chunk = (row block f / KS, k-step f % KS); source = uniform base + 32-bit per-lane byte offset
   const char* w_bytes = reinterpret_cast<const char*>(p.w1);
@@ -554,10 +571,8 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
       lds_dma16(w_bytes + (row0 * D + (f % KS) * 16) * 2 + lane_off, base + i * kFrag);
     }
   };
-  // First token of this wavefront in the workgroup's idx-th tile.
-  auto tokens_of_tile = [&](int idx) -> int64_t {
-    return (static_cast<int64_t>(blockIdx.x) + static_cast<int64_t>(idx) * gridDim.x) * kTokPerWg + wave * (32 * TT);
-  };
+  // First token of this wavefront in token tile `tile`.
+  auto tokens_of_tile = [&](int tile) -> int64_t { return static_cast<int64_t>(tile) * kTokPerWg + wave * (32 * TT); };
   // Memory rows of a tile in the layout of the epilogue stores: piece i = token (i / 4) * 32 + 8 * (i % 4) + lane / 8.
   auto rows_of_tile = [&](int64_t tok_base, int32_t (&prow)[NST]) {
 #pragma unroll
@@ -583,12 +598,11 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
 
   bf16x8 res_cur[NST], res_next[NST];
   int32_t prow[NST], prow_next[NST];  // rows of the current tile / of the tile the next step belongs to
-  int tile_idx = 0;
-  int64_t tok_wave = tokens_of_tile(0);
+  int64_t tok_wave = tokens_of_tile(tile_of(0));
   rows_of_tile(tok_wave, prow);
-  stage(0, 0);
-  if (total > 1) stage(nchunks > 1 ? 1 : 0, 1);
-  if (RES) request_residual(prow, 0, res_cur);
+  stage(chunk_of(0), 0);
+  if (total > 1) stage(chunk_of(1), 1);
+  if (RES) request_residual(prow, chunk_of(0), res_cur);
   stage_bias(p.b1, bias_lds, p.N, tid, NWAVES * kWave);
   if (p.norm_w != nullptr) stage_bias(p.norm_w, bias_lds + p.N, D, tid, NWAVES * kWave);
   load_tile(tok_wave);
@@ -597,16 +611,15 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
   if (p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + p.N, hh, xf);
 
   uint8_t* tile_lds = tiles + wave * kStageWave;
-  int chunk = 0;                                      // chunk of step s
   int buf = 0;                                        // ring slot of step s
-  int chunk2 = 2 % nchunks;                           // chunk of step s + 2
   for (int s = 0; s < total; ++s) {
+    const int chunk = chunk_of(s);
     // ---- requests for later steps ------------------------------------------------------------------------------------
     const bool has_next = s + 1 < total;
     const bool stage_ahead = s + 2 < total;
-    const bool new_tile = s > 0 && chunk == 0;  // the workgroup moves to its next token tile in this step
+    const bool new_tile = s > 0 && first_of_tile(s);  // the workgroup moves to its next token tile in this step
     if (new_tile) {
-      tok_wave = tokens_of_tile(++tile_idx);
+      tok_wave = tokens_of_tile(tile_of(s));
       if (RES) {
 #pragma unroll
         for (int i = 0; i < NST; ++i) prow[i] = prow_next[i];
@@ -615,14 +628,14 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
       }
     }
     if (RES && has_next) {
-      if (chunk + 1 == nchunks) {  // the next step opens the next tile
-        rows_of_tile(tokens_of_tile(tile_idx + 1), prow_next);
-        request_residual(prow_next, 0, res_next);
+      if (first_of_tile(s + 1)) {  // the next step opens the next tile
+        rows_of_tile(tokens_of_tile(tile_of(s + 1)), prow_next);
+        request_residual(prow_next, chunk_of(s + 1), res_next);
       } else {
-        request_residual(prow, chunk + 1, res_next);
+        request_residual(prow, chunk_of(s + 1), res_next);
       }
     }
-    if (stage_ahead) stage(chunk2, buf == 0 ? 2 : buf - 1);  // slot (s + 2) % 3, last read in step s - 1
+    if (stage_ahead) stage(chunk_of(s + 2), buf == 0 ? 2 : buf - 1);  // slot (s + 2) % 3, last read in step s - 1
     if (new_tile) {
       // The rows are requested after the weights and residual pieces of the later steps, so that those are not held
       // back by the wait for the rows.
@@ -708,8 +721,6 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
       }
     }
     buf = buf == 2 ? 0 : buf + 1;
-    if (++chunk == nchunks) chunk = 0;
-    if (++chunk2 == nchunks) chunk2 = 0;
   }
 }
 
