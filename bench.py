@@ -266,6 +266,8 @@ def main() -> None:
     parser.add_argument("--batch", type=int, default=1024, help="samples per step (headline: 1024)")
     parser.add_argument("--skip-cpu-baseline", action="store_true")
     parser.add_argument("--skip-operators", action="store_true")
+    parser.add_argument("--skip-all-positions", action="store_true",
+                        help="do not time the comparison run over the padded positions (keeps kernel traces to one mode)")
     args = parser.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU (the path has no cross-GPU stage); use --gpus 1")
@@ -300,12 +302,14 @@ def main() -> None:
 
     # The same step with the dense layers run over all B*T positions, padding included (what the reference's dense
     # [B, T, D] formulation does): reported next to the headline figure, never as the value.
-    os.environ["TAAC_DENSE_TOKENS"] = "1"
-    try:
-        with torch.no_grad():
-            dense_ms = _event_ms(lambda: model(emb, lengths), max(args.steps // 2, 1), 2)
-    finally:
-        del os.environ["TAAC_DENSE_TOKENS"]
+    dense_ms = None
+    if not args.skip_all_positions:
+        os.environ["TAAC_DENSE_TOKENS"] = "1"
+        try:
+            with torch.no_grad():
+                dense_ms = _event_ms(lambda: model(emb, lengths), max(args.steps // 2, 1), 2)
+        finally:
+            del os.environ["TAAC_DENSE_TOKENS"]
     valid_fraction = float(inputs.key_lengths.clamp(0, T).sum().item()) / (B * T)
 
     kernels = _kernel_breakdown(inputs, device, iters=10)
@@ -347,8 +351,9 @@ def main() -> None:
         },
         "dense_equivalent_tflops": dense_flops / (elapsed / args.steps) / 1e12,
         "valid_token_fraction": valid_fraction,
-        "all_positions": {"ms_per_step": dense_ms, "samples_per_s": B / (dense_ms * 1e-3),
-                          "note": "dense layers run over the padded positions too (TAAC_DENSE_TOKENS=1)"},
+        "all_positions": None if dense_ms is None else {
+            "ms_per_step": dense_ms, "samples_per_s": B / (dense_ms * 1e-3),
+            "note": "dense layers run over the padded positions too (TAAC_DENSE_TOKENS=1)"},
         "roofline": roofline,
         "accuracy": accuracy,
         "kernels": kernels,
