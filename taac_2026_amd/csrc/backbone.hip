@@ -1,6 +1,7 @@
 // Forward driver of the unified token backbone (pre-norm blocks + pCVR readout) and the readout kernel.
 // The driver only sequences the library's own entry points on one stream over a caller-provided workspace.
 #include <cstdlib>
+#include <vector>
 
 #include "common.h"
 
@@ -225,6 +226,22 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
 
   const bf16_t* cur = static_cast<const bf16_t*>(emb);
   int rc;
+  if (fused && n_blocks > 0) {
+    // One launch re-lays the weights of all blocks into fragment order.
+    std::vector<void*> pk(3 * static_cast<size_t>(n_blocks));
+    for (int i = 0; i < n_blocks; ++i) {
+      const taac_block_weights& w = blocks[i];
+      if (!w.qkv_weight || !w.out_weight || !w.up_weight || !w.down_weight)
+        return set_error(TAAC_ERR_INVALID_VALUE, "%s: block %d has a null weight", name, i);
+      char* base = packed + static_cast<int64_t>(i) * packed_block_bytes(D, F);
+      pk[i] = base;
+      pk[n_blocks + i] = base + align256(static_cast<int64_t>(3) * D * D * 2);
+      pk[2 * n_blocks + i] = base + align256(static_cast<int64_t>(3) * D * D * 2) + align256(static_cast<int64_t>(D) * D * 2);
+    }
+    if ((rc = pack_backbone_blocks(blocks, n_blocks, D, F, pk.data(), pk.data() + n_blocks, pk.data() + 2 * n_blocks,
+                                   as_stream(stream), name)) != TAAC_OK)
+      return rc;
+  }
   for (int i = 0; i < n_blocks; ++i) {
     const taac_block_weights& w = blocks[i];
     if (!w.attn_norm_weight || !w.qkv_weight || !w.out_weight || !w.ffn_norm_weight || !w.up_weight || !w.down_weight)
@@ -237,9 +254,6 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
     char* pk_ffn = pk_out + align256(static_cast<int64_t>(D) * D * 2);
     // attention half
     if (fused) {
-      if ((rc = taac_linear_pack_weights(w.qkv_weight, pk_qkv, 3 * D, D, stream)) != TAAC_OK) return rc;
-      if ((rc = taac_linear_pack_weights(w.out_weight, pk_out, D, D, stream)) != TAAC_OK) return rc;
-      if ((rc = taac_ffn_pack_weights(w.up_weight, w.down_weight, pk_ffn, D, F, 1, stream)) != TAAC_OK) return rc;
       if ((rc = taac_norm_linear_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, nullptr, 0, qkv,
                                      3 * D, M, 3 * D, D, rows, n_rows, stream)) != TAAC_OK)
         return rc;

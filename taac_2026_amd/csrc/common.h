@@ -29,6 +29,9 @@ int set_error(int code, const char* fmt, ...);
 int check_launch(const char* what);
 // Compute units of the current device, cached per device; -1 when the query fails.
 int compute_units();
+// Packs the qkv / out / feed-forward weights (gate first) of n backbone blocks into fragment order (ffn.hip).
+int pack_backbone_blocks(const taac_block_weights* blocks, int n, int32_t D, int32_t F, void* const* packed_qkv,
+                         void* const* packed_out, void* const* packed_ffn, hipStream_t s, const char* name);
 // Token-stationary e4m3 dense layer (fp8_ts.hip): TAAC_OK after a launch, a negative status on an error, 1 when the shape
 // is not covered and the caller must use the tiled kernel.
 int launch_linear_fp8_ts(const void* a, int a_is_fp8, int64_t lda, const void* w, const float* amax_a,

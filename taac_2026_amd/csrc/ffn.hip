@@ -69,12 +69,9 @@ __host__ __device__ __forceinline__ int up_unit_of_slot(int m16) {
 // ---- fragment-order packing ------------------------------------------------------------------------------------------
 // FFN blob: step s (32 hidden units) holds, for chunk q = 0, 1: KS up fragments (k-step r) then MB down fragments
 // (row block r - KS); exactly the image one barrier step needs in LDS. A fragment is 64 lanes x 16 bytes.
-__global__ void ffn_pack_kernel(const bf16_t* __restrict__ w_up, const bf16_t* __restrict__ w_down,
-                                bf16x8* __restrict__ packed, int D, int F, int gate_first) {
+__device__ __forceinline__ void ffn_pack_piece(const bf16_t* __restrict__ w_up, const bf16_t* __restrict__ w_down,
+                                               bf16x8* __restrict__ packed, int D, int F, int gate_first, int64_t gid) {
   const int KS = D / 16, MB = D / 32, CFRAG = KS + MB, NFRAG = kCPB * CFRAG;
-  const int64_t total = static_cast<int64_t>(F / (kHU * kCPB)) * NFRAG * 64;
-  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (gid >= total) return;
   const int lane = static_cast<int>(gid % 64);
   const int f = static_cast<int>((gid / 64) % NFRAG);
   const int64_t step = gid / 64 / NFRAG;
@@ -89,18 +86,53 @@ __global__ void ffn_pack_kernel(const bf16_t* __restrict__ w_up, const bf16_t* _
   packed[gid] = *reinterpret_cast<const bf16x8*>(src);
 }
 
-// Linear blob: chunk c (64 output features) holds fragments (row block rb, k-step ks) at index rb * KS + ks.
-__global__ void linear_pack_kernel(const bf16_t* __restrict__ w, bf16x8* __restrict__ packed, int N, int K) {
-  const int KS = K / 16, NFRAG = 2 * KS;
-  const int64_t total = static_cast<int64_t>(N / kNC) * NFRAG * 64;
+__global__ void ffn_pack_kernel(const bf16_t* __restrict__ w_up, const bf16_t* __restrict__ w_down,
+                                bf16x8* __restrict__ packed, int D, int F, int gate_first) {
+  const int64_t total = static_cast<int64_t>(3) * D * F / 8;
   const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (gid >= total) return;
+  if (gid < total) ffn_pack_piece(w_up, w_down, packed, D, F, gate_first, gid);
+}
+
+// Linear blob: chunk c (64 output features) holds fragments (row block rb, k-step ks) at index rb * KS + ks.
+__device__ __forceinline__ void linear_pack_piece(const bf16_t* __restrict__ w, bf16x8* __restrict__ packed, int K,
+                                                  int64_t gid) {
+  const int KS = K / 16, NFRAG = 2 * KS;
   const int lane = static_cast<int>(gid % 64);
   const int f = static_cast<int>((gid / 64) % NFRAG);
   const int64_t chunk = gid / 64 / NFRAG;
   const int l32 = lane % 32, hh = lane / 32;
   const bf16_t* src = w + (chunk * kNC + (f / KS) * 32 + l32) * K + (f % KS) * 16 + hh * 8;
   packed[gid] = *reinterpret_cast<const bf16x8*>(src);
+}
+
+__global__ void linear_pack_kernel(const bf16_t* __restrict__ w, bf16x8* __restrict__ packed, int N, int K) {
+  const int64_t total = static_cast<int64_t>(N) * K / 8;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (gid < total) linear_pack_piece(w, packed, K, gid);
+}
+
+// All weights of up to kPackBatch backbone blocks in one launch: blockIdx.y = block, blockIdx.x walks the 16-byte
+// pieces of its qkv, out and feed-forward blobs in that order.
+constexpr int kPackBatch = 16;
+struct PackBatch {
+  const bf16_t* qkv[kPackBatch];
+  const bf16_t* out[kPackBatch];
+  const bf16_t* up[kPackBatch];
+  const bf16_t* down[kPackBatch];
+  bf16x8* packed_qkv[kPackBatch];
+  bf16x8* packed_out[kPackBatch];
+  bf16x8* packed_ffn[kPackBatch];
+};
+__global__ void pack_blocks_kernel(const PackBatch batch, int D, int F) {
+  const int blk = blockIdx.y;
+  const int64_t n_qkv = static_cast<int64_t>(3) * D * D / 8, n_out = static_cast<int64_t>(D) * D / 8;
+  const int64_t n_ffn = static_cast<int64_t>(3) * D * F / 8;
+  int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (gid < n_qkv) return linear_pack_piece(batch.qkv[blk], batch.packed_qkv[blk], D, gid);
+  gid -= n_qkv;
+  if (gid < n_out) return linear_pack_piece(batch.out[blk], batch.packed_out[blk], D, gid);
+  gid -= n_out;
+  if (gid < n_ffn) ffn_pack_piece(batch.up[blk], batch.down[blk], batch.packed_ffn[blk], D, F, 1, gid);
 }
 
 // ---- shared pieces ---------------------------------------------------------------------------------------------------
@@ -754,6 +786,36 @@ bool ptr_ok(const void* p, uintptr_t mask) { return (reinterpret_cast<uintptr_t>
 constexpr int kMaxLdsBytes = 160 * 1024;
 
 }  // namespace
+}  // namespace taac
+
+namespace taac {
+// Packs the qkv / out / feed-forward weights (gate first) of n backbone blocks with as few launches as possible.
+int pack_backbone_blocks(const taac_block_weights* blocks, int n, int32_t D, int32_t F, void* const* packed_qkv,
+                         void* const* packed_out, void* const* packed_ffn, hipStream_t s, const char* name) {
+  for (int base = 0; base < n; base += kPackBatch) {
+    PackBatch batch{};
+    const int m = n - base < kPackBatch ? n - base : kPackBatch;
+    for (int i = 0; i < m; ++i) {
+      const taac_block_weights& w = blocks[base + i];
+      if (!ptr_ok(w.qkv_weight, 15) || !ptr_ok(w.out_weight, 15) || !ptr_ok(w.up_weight, 15) ||
+          !ptr_ok(w.down_weight, 15))
+        return set_error(TAAC_ERR_UNSUPPORTED, "%s: weights must be 16-byte aligned", name);
+      batch.qkv[i] = static_cast<const bf16_t*>(w.qkv_weight);
+      batch.out[i] = static_cast<const bf16_t*>(w.out_weight);
+      batch.up[i] = static_cast<const bf16_t*>(w.up_weight);
+      batch.down[i] = static_cast<const bf16_t*>(w.down_weight);
+      batch.packed_qkv[i] = static_cast<bf16x8*>(packed_qkv[base + i]);
+      batch.packed_out[i] = static_cast<bf16x8*>(packed_out[base + i]);
+      batch.packed_ffn[i] = static_cast<bf16x8*>(packed_ffn[base + i]);
+    }
+    const int64_t pieces = (static_cast<int64_t>(4) * D * D + static_cast<int64_t>(3) * D * F) / 8;
+    hipLaunchKernelGGL(pack_blocks_kernel, dim3(static_cast<uint32_t>((pieces + 255) / 256), m), dim3(256), 0, s, batch,
+                       D, F);
+    const int rc = check_launch(name);
+    if (rc != TAAC_OK) return rc;
+  }
+  return TAAC_OK;
+}
 }  // namespace taac
 
 extern "C" int64_t taac_ffn_packed_bytes(int32_t D, int32_t F) {
