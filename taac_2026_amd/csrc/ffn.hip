@@ -54,6 +54,7 @@ struct TsParams {
   int32_t packed;           // weights are in fragment order
   const int32_t* rows;      // optional row index: token i lives in row rows[i] of x / residual / out
   const int32_t* n_rows;    // with rows: device pointer to the number of tokens (at most M)
+  int32_t units;            // FFN: compute units the last, partial round of workgroups is spread over
 };
 
 __device__ __forceinline__ float silu_f(float v) {
@@ -294,9 +295,29 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
   const int lane = tid % kWave;
   const int l32 = lane % 32;
   const int hh = lane / 32;
+  // Work split: workgroups [0, base) take one full tile of kTokPerWg tokens each, base = the largest multiple of
+  // p.units not above the number of complete tiles; the tokens that remain (fewer than p.units tiles) are spread
+  // evenly over the next p.units workgroups in slices of whole 32-token wavefront tiles, so that the last round keeps
+  // every compute unit busy for a fraction of a tile instead of some of them for a whole one.
   const int64_t count = token_count(p);
-  if (static_cast<int64_t>(blockIdx.x) * kTokPerWg >= count) return;  // whole workgroup: no tokens left for it
-  const int64_t tok0 = static_cast<int64_t>(blockIdx.x) * kTokPerWg + wave * (32 * TT);
+  const int64_t base = count / kTokPerWg / p.units * p.units;
+  int64_t wg_tok0;
+  int wg_ntok;
+  if (static_cast<int64_t>(blockIdx.x) < base) {
+    wg_tok0 = static_cast<int64_t>(blockIdx.x) * kTokPerWg;
+    wg_ntok = kTokPerWg;
+  } else {
+    const int64_t rest = count - base * kTokPerWg;  // < p.units * kTokPerWg
+    const int64_t per = ((rest + p.units - 1) / p.units + 32 * TT - 1) / (32 * TT) * (32 * TT);
+    const int64_t j = static_cast<int64_t>(blockIdx.x) - base;
+    wg_tok0 = base * kTokPerWg + j * per;
+    const int64_t left = count - wg_tok0;
+    wg_ntok = static_cast<int>(left < per ? left : per);
+    if (j >= p.units || wg_ntok <= 0) return;  // whole workgroup: no tokens left for it
+  }
+  // A wavefront whose tile lies beyond the workgroup's slice only helps staging the weights.
+  const bool active = wave * (32 * TT) < wg_ntok;
+  const int64_t tok0 = wg_tok0 + wave * (32 * TT);
   const int F = p.F;
   const int nsteps = F / (kHU * CPB);
 
@@ -341,7 +362,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
   if (p.norm_w != nullptr) stage_bias(p.norm_w, bias_lds + 2 * F + D, D, tid, NWAVES * kWave);
 
   bf16x8 xf[TT][KS];
-  load_token_rows<D, TT>(p, count, tok0, l32, hh, xf);
+  if (active) load_token_rows<D, TT>(p, count, tok0, l32, hh, xf);
 
   f32x16 oacc[TT][MB];
 #pragma unroll
@@ -353,7 +374,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  if (p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + 2 * F + D, hh, xf);
+  if (active && p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + 2 * F + D, hh, xf);
 
   // One barrier step = CPB chunks = NFRAG fragments, consumed in their LDS order: per chunk KS up fragments, then MB
   // down fragments. Fragment reads run P fragments ahead of their MFMAs through a ring of P registers sets; the two
@@ -384,6 +405,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
     if (step + 1 < nsteps) stage(step + 1, buf == NBUF - 1 ? 0 : buf + 1);
     const uint32_t wb = smem_off + buf * (NFRAG * kFrag);
     const uint32_t bias_step = bias_off + step * (CPB * 32 * 2);
+    if (active) {
     bf16x8 ring[P];
     uint32_t brow[CPB];  // bias of this lane's fragment row, one per chunk, zero-extended bf16
     f32x16 gu[TT];
@@ -464,6 +486,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
         __builtin_amdgcn_sched_barrier(0);
       }
     });
+    }  // active
     // The next step's weights must have landed (the only vector-memory operations of this loop).
     vm_wait<0>();
     __syncthreads();
@@ -472,6 +495,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
   }
   if constexpr (DEFER) {
     // The down projection of the last chunk is still pending; its fragments are in the last step's buffer.
+    if (active) {
     bf16x8 tail[MB];
     static_for<MB>([&](auto ic) {
       constexpr int j = decltype(ic)::value;
@@ -484,10 +508,12 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
       for (int t = 0; t < TT; ++t)
         oacc[t][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tail[j], hb[t], oacc[t][j], 0, 0, 0);
     });
+    }
     __syncthreads();  // the epilogue tiles below overwrite the weight buffers
   }
 
   // ---- epilogue: + b_down, round, transpose through the wavefront's LDS tile, + residual, coalesced bf16 stores ----
+  if (!active) return;  // no barrier below
   uint8_t* tile = smem + wave * kStageWave;  // the weight buffers are free after the last barrier
   const bf16_t* bdown_lds = bias_lds + 2 * F;
 #pragma unroll
@@ -498,7 +524,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       prow[i] = token_row(p, count, tok_base + i * 8 + lane / 8);
-      live[i] = tok_base + i * 8 + lane / 8 < count;
+      live[i] = tok_base + i * 8 + lane / 8 < wg_tok0 + wg_ntok;
     }
 #pragma unroll
     for (int pr = 0; pr < MB / 2; ++pr) {  // 64 features at a time
@@ -764,7 +790,8 @@ int launch_ts(K kernel, const TsParams& p, int threads, int tokens_per_wg, size_
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                           static_cast<int>(lds_bytes)) != hipSuccess)
     return set_error(TAAC_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", name, lds_bytes);
-  const int64_t grid = (p.M + tokens_per_wg - 1) / tokens_per_wg;
+  // upper bound of the kernel's own split: one workgroup per complete tile plus one per unit for the rest
+  const int64_t grid = p.M / tokens_per_wg + p.units;
   if (grid > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many workgroups", name);
   hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(grid)), dim3(threads), lds_bytes, s, p);
   return check_launch(name);
@@ -902,6 +929,12 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
   p.packed = packed_weights ? 1 : 0;
   p.rows = rows;
   p.n_rows = n_rows;
+  p.units = compute_units();
+  if (p.units <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
+  if (const char* cap = getenv("TAAC_TS_MAX_WORKGROUPS")) {  // test hook, as in the linear kernel
+    const int limit = atoi(cap);
+    if (limit > 0 && limit < p.units) p.units = limit;
+  }
   hipStream_t s = as_stream(stream);
   const int KS = D / 16, MB = D / 32;
   const size_t bias_bytes = static_cast<size_t>(2 * F + 2 * D) * 2;
