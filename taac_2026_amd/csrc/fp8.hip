@@ -20,7 +20,18 @@ __global__ __launch_bounds__(kBlock) void amax_kernel(const T* __restrict__ x, i
   const int64_t nvec = aligned16(x) ? n / VEC : 0;
   typedef T vec_t __attribute__((ext_vector_type(VEC)));
   const vec_t* xv = reinterpret_cast<const vec_t*>(x);
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < nvec; i += stride) {
+  // Four independent 16-byte loads per thread and trip keep enough bytes in flight to stream from HBM.
+  int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  for (; i + 3 * stride < nvec; i += 4 * stride) {
+    vec_t v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(xv + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) m = fmaxf(m, fabsf(static_cast<float>(v[u][e])));
+  }
+  for (; i < nvec; i += stride) {
     const vec_t v = xv[i];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) m = fmaxf(m, fabsf(static_cast<float>(v[e])));

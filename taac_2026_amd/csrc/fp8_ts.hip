@@ -27,20 +27,19 @@
 namespace taac {
 namespace {
 
-constexpr int kK = 256;                  // reduction length this kernel is built for
-constexpr int kKS = kK / 64;             // k-steps of the fp8 MFMA
-constexpr int kRows = 64;                // weight rows per step: two 32-row blocks
 constexpr int kFrag8 = 2048;             // bytes of one 32 x 64 e4m3 fragment
-constexpr int kNFrag = 2 * kKS;          // fragments per step
-constexpr int kBuf8 = kNFrag * kFrag8;   // 16 KB
-constexpr int kTileRow = 64 * 4 + 16;    // bytes per token row of the fp32 epilogue tile (64 features + pad)
-constexpr int kTileWave = 32 * kTileRow; // one 32-token tile
 constexpr int kWaves = 8;
+// Per reduction length K: 32-row weight blocks per step (two for K = 256, one for K = 1024, whose fragments are four
+// times as many), and the epilogue tile of a wavefront (fp32, 32 tokens x 32 features per row block + 16 bytes pad).
+constexpr int row_blocks(int K) { return K <= 256 ? 2 : 1; }
+constexpr int tile_row_bytes(int K) { return row_blocks(K) * 32 * 4 + 16; }
+constexpr int step_bytes(int K) { return row_blocks(K) * (K / 64) * kFrag8; }
 constexpr int kScaleOne = 127;           // E8M0 exponent of 1.0 for the block-scale operands of the f8f6f4 MFMA
 
-// 32-token tiles per wavefront: two (every weight fragment read from LDS feeds two MFMAs), one with the residual
-// epilogue, whose double-buffered residual pieces would not fit the register file next to two tiles.
-constexpr int tiles_per_wave(int epilogue) { return epilogue == TAAC_EPI_RESIDUAL ? 1 : 2; }
+// 32-token tiles per wavefront: two (every weight fragment read from LDS feeds two MFMAs) for K = 256 without a
+// residual; one with the residual epilogue, whose double-buffered residual pieces would not fit the register file next
+// to two tiles, and for K = 1024, where one tile's fragments already take 128 registers.
+constexpr int tiles_per_wave(int K, int epilogue) { return (epilogue == TAAC_EPI_RESIDUAL || K > 256) ? 1 : 2; }
 
 struct Fp8TsParams {
   const void* a;            // [M, K] bf16 or e4m3, row stride lda (elements)
@@ -81,18 +80,28 @@ __device__ __forceinline__ void lds_wait_halves(u32x4& a, u32x4& b) {
   asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
 }
 
-template <int EPI, bool A_FP8>
+template <int kK, int EPI, bool A_FP8>
 __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const Fp8TsParams p, const int num_tiles) {
   constexpr bool RES = EPI == TAAC_EPI_RESIDUAL;
-  constexpr int kTT = tiles_per_wave(EPI);
+  constexpr int kTT = tiles_per_wave(kK, EPI);
   constexpr int kTokPerWg = kWaves * 32 * kTT;
   constexpr bool GLU = EPI == TAAC_EPI_SWIGLU;
-  constexpr int OUTC = GLU ? 32 : 64;             // output features per step
+  constexpr int kKS = kK / 64;                    // k-steps of the fp8 MFMA
+  constexpr int RB = row_blocks(kK);              // 32-row weight blocks per step
+  constexpr int kRows = RB * 32;                  // weight rows per step
+  constexpr int kNFrag = RB * kKS;                // fragments per step
+  constexpr int kBuf8 = step_bytes(kK);
+  constexpr int FPW = kNFrag * 2 / kWaves;        // DMA instructions per wavefront and step
+  constexpr int kTileRow = tile_row_bytes(kK);
+  constexpr int kTileWave = 32 * kTileRow;
+  static_assert(!GLU || RB == 2, "the SiLU-gate epilogue pairs two row blocks");
+  static_assert(kNFrag * 2 % kWaves == 0, "the DMA instructions of a step divide over the wavefronts");
+  constexpr int OUTC = GLU ? 32 : kRows;          // output features per step
   constexpr int PIECES = OUTC / 8;                // 16-byte output pieces per token row
   constexpr int ROWS_PER_STORE = kWave / PIECES;  // token rows covered by one store instruction
   constexpr int NSTT = 32 / ROWS_PER_STORE;       // stores per 32-token tile
   constexpr int NST = NSTT * kTT;                 // stores (and residual pieces) per wavefront and step
-  constexpr int P = 4;                            // fragments in flight
+  constexpr int P = 4;             // fragments in flight
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   uint8_t* tiles = smem + 3 * kBuf8;
   bf16_t* bias_lds = reinterpret_cast<bf16_t*>(tiles + kWaves * kTileWave);
@@ -119,16 +128,19 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
     if (GLU) return ((rb == 0) == (p.gate_first != 0) ? 0 : F) + chunk * 32;
     return chunk * kRows + rb * 32;
   };
-  // Wavefront w stages fragment w of the step (row block w / KS, k-step w % KS): two DMA instructions.
+  // DMA instruction d of a step (two per fragment) moves half d % 2 of fragment d / 2 = (row block f / KS, k-step
+  // f % KS); wavefront w issues instructions w * FPW .. + FPW - 1.
   auto stage = [&](int chunk, int buf) {
     int ln = lane;
     asm volatile("" : "+v"(ln));
-    const int rb = wave / kKS, ks = wave % kKS;
-    const uint8_t* src = p.w + static_cast<int64_t>(block_row0(chunk, rb)) * kK + ks * 64 +
-                         static_cast<uint32_t>((ln & 31) * kK + (ln >> 5) * 32);
-    uint8_t* dst = smem + buf * kBuf8 + wave * kFrag8;
-    lds_dma16(src, dst);
-    lds_dma16(src + 16, dst + 1024);
+    const uint32_t lane_off = static_cast<uint32_t>((ln & 31) * kK + (ln >> 5) * 32);
+#pragma unroll
+    for (int i = 0; i < FPW; ++i) {
+      const int d = wave * FPW + i;  // wavefront-uniform
+      const int f = d / 2, half = d % 2;
+      const uint8_t* src = p.w + static_cast<int64_t>(block_row0(chunk, f / kKS)) * kK + (f % kKS) * 64 + half * 16 + lane_off;
+      lds_dma16(src, smem + buf * kBuf8 + f * kFrag8 + half * 1024);
+    }
   };
   auto rows_of_tile = [&](int idx) -> int64_t {
     return (static_cast<int64_t>(blockIdx.x) + static_cast<int64_t>(idx) * gridDim.x) * kTokPerWg + wave * (32 * kTT);
@@ -160,17 +172,22 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
         }
       } else {
         const bf16_t* row = static_cast<const bf16_t*>(p.a) + tok * p.lda + hh * 32;
-        bf16x8 raw[kKS][4];
+        // Four k-steps (16 loads, 64 registers) at a time: load, then quantise.
 #pragma unroll
-        for (int ks = 0; ks < kKS; ++ks)
+        for (int k4 = 0; k4 < kKS; k4 += 4) {
+          bf16x8 raw[4][4];
 #pragma unroll
-          for (int c = 0; c < 4; ++c) raw[ks][c] = *reinterpret_cast<const bf16x8*>(row + ks * 64 + c * 8);
+          for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-        for (int ks = 0; ks < kKS; ++ks) {
-          int q[8];
+            for (int c = 0; c < 4; ++c) raw[ks][c] = *reinterpret_cast<const bf16x8*>(row + (k4 + ks) * 64 + c * 8);
 #pragma unroll
-          for (int c = 0; c < 4; ++c) quant8(raw[ks][c], inv_scale_a, q[2 * c], q[2 * c + 1]);
-          xq[t][ks] = i32x8{q[0], q[1], q[2], q[3], q[4], q[5], q[6], q[7]};
+          for (int ks = 0; ks < 4; ++ks) {
+            int q[8];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) quant8(raw[ks][c], inv_scale_a, q[2 * c], q[2 * c + 1]);
+            xq[t][k4 + ks] = i32x8{q[0], q[1], q[2], q[3], q[4], q[5], q[6], q[7]};
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
@@ -209,20 +226,20 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
     if (stage_ahead) stage(chunk2, buf == 0 ? 2 : buf - 1);  // slot (s + 2) % 3, last read in step s - 1
     if (new_tile) load_tile(tok_wave);
 
-    // ---- the products of this step: fragment stream (ks, rb) = (i / 2, i % 2), LDS fragment index rb * KS + ks -------
+    // ---- the products of this step: fragment stream (ks, rb) = (i / RB, i % RB), LDS fragment index rb * KS + ks -----
     const uint32_t wb = lds_offset(smem) + buf * kBuf8 + lane * 16;
-    f32x16 acc[2][kTT];
+    f32x16 acc[RB][kTT];
     u32x4 rlo[P], rhi[P];
     auto read_frag = [&](auto ic, int slot) {
       constexpr int i = decltype(ic)::value;
-      constexpr int f = (i % 2) * kKS + i / 2;
+      constexpr int f = (i % RB) * kKS + i / RB;
       lds_read16<f * kFrag8>(rlo[slot], wb);
       lds_read16<f * kFrag8 + 1024>(rhi[slot], wb);
     };
     static_for<P>([&](auto ic) { read_frag(ic, decltype(ic)::value); });
     static_for<kNFrag>([&](auto ic) {
       constexpr int i = decltype(ic)::value;
-      constexpr int ks = i / 2, rb = i % 2;
+      constexpr int ks = i / RB, rb = i % RB;
       constexpr int after = 2 * (P - 1 < kNFrag - 1 - i ? P - 1 : kNFrag - 1 - i);
       lds_wait_halves<after>(rlo[i % P], rhi[i % P]);
       const u32x4 lo = rlo[i % P], hi = rhi[i % P];
@@ -236,6 +253,9 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
           acc[rb][t] =
               __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf, xq[t][ks], acc[rb][t], 0, 0, 0, kScaleOne, 0, kScaleOne);
         }
+        // The product has no side effect, so instruction selection may sink a whole accumulation chain below the LDS reads
+        // that follow it and keep every fragment of the step live at once; this empty statement keeps it in place.
+        asm volatile("" : "+v"(acc[rb][t]));
       }
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (i + P < kNFrag) read_frag(std::integral_constant<int, i + P>{}, i % P);
@@ -243,27 +263,27 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
 
     // ---- epilogue: dequantise, bias, gate; fp32 tile transpose; residual; one rounding; NST stores -------------------
     // Accumulator register jq*4 + e of lane (l32, hh) is row jq*8 + hh*4 + e of its 32-row block, token l32.
-    bf16x4 bv[8];
+    bf16x4 bv[4 * RB];
 #pragma unroll
-    for (int q = 0; q < 8; ++q)
+    for (int q = 0; q < 4 * RB; ++q)
       bv[q] = *reinterpret_cast<const bf16x4*>(bias_lds + block_row0(chunk, q / 4) + (q % 4) * 8 + hh * 4);
 #pragma unroll
     for (int t = 0; t < kTT; ++t) {
 #pragma unroll
       for (int jq = 0; jq < 4; ++jq) {
-        f32x4 v0, v1;
+        f32x4 v[RB];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          v0[e] = acc[0][t][jq * 4 + e] * dq + static_cast<float>(bv[jq][e]);
-          v1[e] = acc[1][t][jq * 4 + e] * dq + static_cast<float>(bv[4 + jq][e]);
-        }
-        if (GLU) {
+        for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v0[e] = silu_f(v0[e]) * v1[e];
-          *reinterpret_cast<f32x4*>(tile_lds + l32 * kTileRow + (jq * 8 + hh * 4) * 4) = v0;
+          for (int e = 0; e < 4; ++e) v[rb][e] = acc[rb][t][jq * 4 + e] * dq + static_cast<float>(bv[rb * 4 + jq][e]);
+        if constexpr (GLU) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[0][e] = silu_f(v[0][e]) * v[1][e];
+          *reinterpret_cast<f32x4*>(tile_lds + l32 * kTileRow + (jq * 8 + hh * 4) * 4) = v[0];
         } else {
-          *reinterpret_cast<f32x4*>(tile_lds + l32 * kTileRow + (jq * 8 + hh * 4) * 4) = v0;
-          *reinterpret_cast<f32x4*>(tile_lds + l32 * kTileRow + (32 + jq * 8 + hh * 4) * 4) = v1;
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb)
+            *reinterpret_cast<f32x4*>(tile_lds + l32 * kTileRow + (rb * 32 + jq * 8 + hh * 4) * 4) = v[rb];
         }
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -292,7 +312,7 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
     // ---- close the step ------------------------------------------------------------------------------------------------
     if (has_next) {
       if (stage_ahead) {
-        vm_wait<2 + NST>();
+        vm_wait<FPW + NST>();
       } else {
         vm_wait<NST>();
       }
@@ -308,24 +328,61 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
   }
 }
 
+// Launches the token-stationary kernel when the shape fits it: K = 256 (any epilogue, weight rows a multiple of 64) or
+// K = 1024 (no SiLU-gate, weight rows a multiple of 32), 16-byte aligned rows. Returns TAAC_OK after a launch, a negative
+// status on a launch error and 1 when the shape is not covered (the caller then uses the tiled kernel).
+template <int K>
+int launch_fp8_ts_for_k(const Fp8TsParams& p, int a_is_fp8, int epilogue, hipStream_t s, const char* name) {
+  const size_t lds_bytes = static_cast<size_t>(3 * step_bytes(K)) + static_cast<size_t>(kWaves) * 32 * tile_row_bytes(K) +
+                           static_cast<size_t>(p.N) * 2;
+  if (lds_bytes > 160 * 1024) return 1;
+  const int tok_per_wg = kWaves * 32 * tiles_per_wave(K, epilogue);
+  const int64_t tiles64 = (p.M + tok_per_wg - 1) / tok_per_wg;
+  if (tiles64 > 0x3fffffffLL) return 1;
+  const int num_tiles = static_cast<int>(tiles64);
+  const int cus = compute_units();
+  if (cus <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
+  int grid = num_tiles < cus ? num_tiles : cus;
+  if (const char* cap = getenv("TAAC_TS_MAX_WORKGROUPS")) {  // test hook, as in the bf16 kernel
+    const int limit = atoi(cap);
+    if (limit > 0 && limit < grid) grid = limit;
+  }
+#define TAAC_FP8_TS_LAUNCH(EPI, AF8)                                                                                \
+  do {                                                                                                              \
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(linear_fp8_ts_kernel<K, EPI, AF8>),                       \
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)) != hipSuccess) \
+      return set_error(TAAC_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", name, lds_bytes);                    \
+    hipLaunchKernelGGL((linear_fp8_ts_kernel<K, EPI, AF8>), dim3(grid), dim3(kWaves * kWave), lds_bytes, s, p,      \
+                       num_tiles);                                                                                  \
+    return check_launch(name);                                                                                      \
+  } while (0)
+  if (epilogue == TAAC_EPI_NONE) {
+    if (a_is_fp8) TAAC_FP8_TS_LAUNCH(TAAC_EPI_NONE, true);
+    TAAC_FP8_TS_LAUNCH(TAAC_EPI_NONE, false);
+  }
+  if (epilogue == TAAC_EPI_RESIDUAL) {
+    if (a_is_fp8) TAAC_FP8_TS_LAUNCH(TAAC_EPI_RESIDUAL, true);
+    TAAC_FP8_TS_LAUNCH(TAAC_EPI_RESIDUAL, false);
+  }
+  if constexpr (row_blocks(K) == 2) {
+    if (a_is_fp8) TAAC_FP8_TS_LAUNCH(TAAC_EPI_SWIGLU, true);
+    TAAC_FP8_TS_LAUNCH(TAAC_EPI_SWIGLU, false);
+  }
+  return 1;
+#undef TAAC_FP8_TS_LAUNCH
+}
+
 }  // namespace
 
-// Launches the token-stationary kernel when the shape fits it: K = 256, weight rows a multiple of 64, 16-byte aligned
-// rows. Returns TAAC_OK after a launch, a negative status on a launch error and 1 when the shape is not covered (the
-// caller then uses the tiled kernel).
 int launch_linear_fp8_ts(const void* a, int a_is_fp8, int64_t lda, const void* w, const float* amax_a,
                          const float* amax_w, const void* bias, const void* residual, void* out, int64_t ldo,
                          int64_t M, int32_t N, int32_t K, int epilogue, int gate_first, hipStream_t s,
                          const char* name) {
-  if (K != kK || N % kRows != 0 || M <= 0) return 1;
+  if ((K != 256 && K != 1024) || M <= 0) return 1;
+  if (N % (row_blocks(K) * 32) != 0) return 1;
+  if (K == 1024 && epilogue == TAAC_EPI_SWIGLU) return 1;
   if (lda % (a_is_fp8 ? 16 : 8) != 0 || ldo % 8 != 0 || (reinterpret_cast<uintptr_t>(bias) & 15u)) return 1;
   if (getenv("TAAC_FP8_TILED") != nullptr) return 1;  // tuning / test hook: force the tiled kernel
-  const size_t lds_bytes = static_cast<size_t>(3 * kBuf8) + static_cast<size_t>(kWaves) * kTileWave +
-                           static_cast<size_t>(N) * 2;
-  if (lds_bytes > 160 * 1024) return 1;
-  const int tok_per_wg = kWaves * 32 * tiles_per_wave(epilogue);
-  const int64_t tiles64 = (M + tok_per_wg - 1) / tok_per_wg;
-  if (tiles64 > 0x3fffffffLL) return 1;
   Fp8TsParams p{};
   p.a = a;
   p.w = static_cast<const uint8_t*>(w);
@@ -339,34 +396,8 @@ int launch_linear_fp8_ts(const void* a, int a_is_fp8, int64_t lda, const void* w
   p.ldo = ldo;
   p.N = N;
   p.gate_first = gate_first ? 1 : 0;
-  const int num_tiles = static_cast<int>(tiles64);
-  const int cus = compute_units();
-  if (cus <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
-  int grid = num_tiles < cus ? num_tiles : cus;
-  if (const char* cap = getenv("TAAC_TS_MAX_WORKGROUPS")) {  // test hook, as in the bf16 kernel
-    const int limit = atoi(cap);
-    if (limit > 0 && limit < grid) grid = limit;
-  }
-#define TAAC_FP8_TS_LAUNCH(EPI, AF8)                                                                                \
-  do {                                                                                                              \
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(linear_fp8_ts_kernel<EPI, AF8>),                          \
-                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)) != hipSuccess) \
-      return set_error(TAAC_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", name, lds_bytes);                    \
-    hipLaunchKernelGGL((linear_fp8_ts_kernel<EPI, AF8>), dim3(grid), dim3(kWaves * kWave), lds_bytes, s, p,         \
-                       num_tiles);                                                                                  \
-    return check_launch(name);                                                                                      \
-  } while (0)
-  if (epilogue == TAAC_EPI_NONE) {
-    if (a_is_fp8) TAAC_FP8_TS_LAUNCH(TAAC_EPI_NONE, true);
-    TAAC_FP8_TS_LAUNCH(TAAC_EPI_NONE, false);
-  }
-  if (epilogue == TAAC_EPI_RESIDUAL) {
-    if (a_is_fp8) TAAC_FP8_TS_LAUNCH(TAAC_EPI_RESIDUAL, true);
-    TAAC_FP8_TS_LAUNCH(TAAC_EPI_RESIDUAL, false);
-  }
-  if (a_is_fp8) TAAC_FP8_TS_LAUNCH(TAAC_EPI_SWIGLU, true);
-  TAAC_FP8_TS_LAUNCH(TAAC_EPI_SWIGLU, false);
-#undef TAAC_FP8_TS_LAUNCH
+  if (K == 256) return launch_fp8_ts_for_k<256>(p, a_is_fp8, epilogue, s, name);
+  return launch_fp8_ts_for_k<1024>(p, a_is_fp8, epilogue, s, name);
 }
 
 }  // namespace taac

@@ -174,6 +174,33 @@ def test_linear_fp8_token_stationary_path(device, monkeypatch, epilogue, workgro
     torch.testing.assert_close(no_bias.cpu().float(), tiled_no_bias.cpu().float(), rtol=0, atol=2.0 ** -7 * scale)
 
 
+@pytest.mark.parametrize("epilogue", ["none", "residual"])
+@pytest.mark.parametrize("workgroups", [None, 2])
+def test_linear_fp8_token_stationary_long_reduction(device, monkeypatch, epilogue, workgroups):
+    """K = 1024 (the FFN down projection) on the token-stationary e4m3 kernel: one 32-row weight block per step, ragged
+    M, several token tiles per workgroup, bf16 and pre-quantised activations, against the oracle and the tiled kernel."""
+    if workgroups is not None:
+        monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+    m, n, k = 1111, 96, 1024
+    x, w, b = _draw(m, n, k, seed=17 + (workgroups or 0))
+    res = torch.randn(m, n, generator=torch.Generator().manual_seed(6)).to(torch.bfloat16) if epilogue == "residual" else None
+    expected = oracle.linear_fp8(x, w, b, residual=res)
+    kwargs = dict(residual=None if res is None else res.to(device))
+    with torch.no_grad():
+        wq, wa = quantize_fp8(w.to(device))
+        xa = amax(x.to(device))
+        got = linear_fp8(x.to(device), wq, xa, wa, b.to(device), **kwargs)
+        xq, _ = quantize_fp8(x.to(device), xa)
+        got_q = linear_fp8(xq, wq, xa, wa, b.to(device), **kwargs)
+        monkeypatch.setenv("TAAC_FP8_TILED", "1")
+        tiled = linear_fp8(x.to(device), wq, xa, wa, b.to(device), **kwargs)
+    assert _rel_err(got.cpu(), expected) <= 5e-2
+    assert _rel_err(got_q.cpu(), expected) <= 5e-2
+    scale = expected.float().abs().max().item()
+    torch.testing.assert_close(got.cpu().float(), tiled.cpu().float(), rtol=0, atol=2.0 ** -7 * scale)
+    torch.testing.assert_close(got_q.cpu().float(), got.cpu().float(), rtol=0, atol=2.0 ** -7 * scale)
+
+
 # ---- token-stationary fused kernels --------------------------------------------------------------------------------
 
 
