@@ -137,6 +137,28 @@ int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, fl
                          void* stream);
 
 /*
+ * Query / key preparation of the attention layers, one pass over q and k (each read once, written once; in place when
+ * q_out == q and k_out == k):
+ *   x_hat = x * rsqrt(mean(x^2 over all d_model features) + eps) * weight      (when q_weight / k_weight are given)
+ *   per head, feature pair (2i, 2i+1) at sequence position t:                    (when cos_sin is given)
+ *     out[2i]   = x_hat[2i] * cos(t, i) - x_hat[2i+1] * sin(t, i)
+ *     out[2i+1] = x_hat[2i] * sin(t, i) + x_hat[2i+1] * cos(t, i)
+ * fp32 arithmetic, one rounding to the storage dtype. q, k: [rows, d_model] with row stride ld_in (elements), row r is
+ * the token at position r % tokens_per_sample of sample r / tokens_per_sample; q_out, k_out likewise with ld_out.
+ * q_weight, k_weight: [d_model] in the storage dtype, both or neither. cos_sin: [tokens_per_sample, head_dim / 2, 2] =
+ * (cos, sin) of position * rope_base^(-2i / head_dim), in the storage dtype, or null. row_index / n_rows: optional
+ * device-side list of the rows to process (taac_valid_rows), both or neither; other rows are left untouched.
+ * d_model, the strides and (with a table) head_dim must be multiples of the 16-byte vector (8 elements, 4 for fp32).
+ * Replaces: query_norm / key_norm (RMSNorm(d_model)) of UnifiedSelfAttention.forward
+ * (experiments/symbiosis/backbone.py:33-36) and BFTSAttention.forward + _apply_rope + _rotate_half_pairs
+ * (experiments/tokenformer/model.py:131-136, 149-154, 165-192), i.e. two norm passes and the elementwise rotary passes.
+ */
+int taac_qk_norm_rope_fwd(const void* q, const void* k, int64_t ld_in, void* q_out, void* k_out, int64_t ld_out,
+                          int64_t rows, int32_t tokens_per_sample, int32_t d_model, int32_t num_heads,
+                          const void* q_weight, const void* k_weight, float eps, const void* cos_sin,
+                          const int32_t* row_index, const int32_t* n_rows, int dtype, void* stream);
+
+/*
  * Row index of the valid tokens of a padded batch: token t of sample b is valid iff t < key_lengths[b] (clamped to
  * [0, T]). Writes rows[i] = b * T + t for the valid tokens in increasing order, *n_rows = their number, and the
  * per-sample offsets (exclusive prefix sums of the lengths, B + 1 values, the last one equal to *n_rows) to

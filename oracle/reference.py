@@ -20,6 +20,11 @@ Puiching-Memory/TAAC_2026). How each function is pinned, independently of its ow
                       test_primitives.py:36-39, tests/contract/experiments/test_packages.py:597-617,
                       test_tilelang_ops.py:361-428), committed as tests/golden/mask_vectors.json.
   masked_mean         float64 brute force; all-padded rows give zeros (divisor clamp).
+  rotate_half_pairs / rope_tables / apply_rope / qk_norm_rope
+                      the reference holds no numeric test for them; pinned by what a rotation fixes: multiplication of
+                      even + i*odd by exp(i*angle) (numpy complex128), position 0 is the identity, pair norms are
+                      kept, the score of a rotated query and key depends only on the position difference, angles
+                      against a float64 loop; the norm part reduces to rms_norm over the model width.
   swiglu_ffn / linear / block / backbone
                       compositions of library routines F.linear, F.silu, the functions above; float64 loop brute
                       force on tiny shapes for swiglu_ffn; the reference holds no numeric test for these
@@ -174,6 +179,86 @@ def scaled_dot_product_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tens
     v4 = v.view(batch, v.shape[1], num_heads, head_dim).transpose(1, 2)
     out = attention(q4, k4, v4, key_lengths, zero_padded_queries=zero_padded_queries)
     return out.transpose(1, 2).contiguous().view(batch, query_len, d_model)
+
+
+# ---- query / key normalisation and rotary embedding ------------------------------------------------------------------
+
+
+def rotate_half_pairs(values: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """``_rotate_half_pairs`` (experiments/tokenformer/model.py:131-136): features (2i, 2i + 1) are one plane, rotated
+    by the angle of frequency i; evaluated in the dtype of ``values`` as the reference does."""
+    even = values[..., 0::2]
+    odd = values[..., 1::2]
+    return torch.stack((even * cos - odd * sin, even * sin + odd * cos), dim=-1).flatten(-2)
+
+
+def rope_tables(token_count: int, head_dim: int, rope_base: float, dtype: torch.dtype) -> tuple[torch.Tensor, torch.Tensor]:
+    """cos / sin of ``position * rope_base ** (-2i / rotary_dim)`` rounded to the activation dtype
+    (experiments/tokenformer/model.py:174-179): shape (tokens, rotary_dim / 2), rotary_dim = 2 * (head_dim // 2)."""
+    rotary_dim = (head_dim // 2) * 2
+    positions = torch.arange(token_count, dtype=torch.float32)
+    frequencies = torch.arange(0, rotary_dim, 2, dtype=torch.float32)
+    inv_freq = torch.pow(torch.tensor(float(rope_base)), -frequencies / max(1, rotary_dim))
+    angles = positions[:, None] * inv_freq[None, :]
+    return angles.cos().to(dtype), angles.sin().to(dtype)
+
+
+def apply_rope(query: torch.Tensor, key: torch.Tensor, *, num_heads: int, rope_base: float) -> tuple[torch.Tensor, torch.Tensor]:
+    """``BFTSAttention._apply_rope`` (experiments/tokenformer/model.py:165-192) on (B, T, D) projections: positions
+    are the token indices 0..T-1, each head rotates its first rotary_dim features and keeps an odd last one."""
+    batch, token_count, d_model = query.shape
+    head_dim = d_model // num_heads
+    rotary_dim = (head_dim // 2) * 2
+    if rotary_dim <= 0:
+        return query, key
+    cos, sin = rope_tables(token_count, head_dim, rope_base, query.dtype)
+    cos = cos.view(1, token_count, 1, -1)
+    sin = sin.view(1, token_count, 1, -1)
+
+    def rotate(values: torch.Tensor) -> torch.Tensor:
+        heads = values.reshape(batch, token_count, num_heads, head_dim)
+        rotated = rotate_half_pairs(heads[..., :rotary_dim], cos, sin)
+        if rotary_dim != head_dim:
+            rotated = torch.cat([rotated, heads[..., rotary_dim:]], dim=-1)
+        return rotated.reshape(batch, token_count, d_model)
+
+    return rotate(query), rotate(key)
+
+
+def qk_norm_rope(query: torch.Tensor, key: torch.Tensor, query_weight: torch.Tensor | None,
+                 key_weight: torch.Tensor | None, *, num_heads: int, eps: float = 1e-6, rope_base: float | None = None,
+                 fp32: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
+    """What ``UnifiedSelfAttention.forward`` (experiments/symbiosis/backbone.py:33-36) and ``BFTSAttention.forward``
+    (experiments/tokenformer/model.py:149-154) do to the query and key projections before attention: RMSNorm over the
+    whole model width (not per head), then the rotary embedding when ``rope_base`` is given. ``fp32=True`` evaluates
+    the same expressions in float32 from the stored inputs (tables still rounded to the storage dtype) and rounds once:
+    the parity target of a fused kernel, as ``rms_norm_fp32`` is for the norm alone."""
+    dtype = query.dtype
+    if fp32:
+        query, key = query.float(), key.float()
+    if query_weight is not None:
+        query = rms_norm(query, query_weight.to(dtype).to(query.dtype), eps)
+        key = rms_norm(key, key_weight.to(dtype).to(key.dtype), eps)
+    if rope_base is not None:
+        if fp32:
+            batch, token_count, d_model = query.shape
+            head_dim = d_model // num_heads
+            cos, sin = rope_tables(token_count, head_dim, rope_base, dtype)
+            cos = cos.float().view(1, token_count, 1, -1)
+            sin = sin.float().view(1, token_count, 1, -1)
+            rotary_dim = (head_dim // 2) * 2
+
+            def rotate(values: torch.Tensor) -> torch.Tensor:
+                heads = values.reshape(batch, token_count, num_heads, head_dim)
+                rotated = rotate_half_pairs(heads[..., :rotary_dim], cos, sin)
+                if rotary_dim != head_dim:
+                    rotated = torch.cat([rotated, heads[..., rotary_dim:]], dim=-1)
+                return rotated.reshape(batch, token_count, d_model)
+
+            query, key = rotate(query), rotate(key)
+        else:
+            query, key = apply_rope(query, key, num_heads=num_heads, rope_base=rope_base)
+    return query.to(dtype), key.to(dtype)
 
 
 # ---- dense layers ----------------------------------------------------------------------------------------------------

@@ -82,6 +82,11 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
          c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p],
     ),
     "taac_valid_rows": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p]),
+    "taac_qk_norm_rope_fwd": (
+        c_int,
+        [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p,
+         c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
+    ),
     "taac_ffn_packed_bytes": (c_int64, [c_int32, c_int32]),
     "taac_ffn_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int, c_void_p]),
     "taac_linear_packed_bytes": (c_int64, [c_int32, c_int32]),

@@ -7,7 +7,9 @@ from taac_2026_amd.accelerators.attention import (
     flash_attention,
     hip_flash_attention_kernel,
     plan_flash_attention_mask,
+    qk_norm_rope,
     resolved_flash_attention_backend,
+    rope_table,
 )
 from taac_2026_amd.accelerators.linear import (
     amax,
@@ -48,6 +50,7 @@ __all__ = [
     "linear_fp8",
     "norm_linear",
     "plan_flash_attention_mask",
+    "qk_norm_rope",
     "quantize_fp8",
     "require_cuda_tensors",
     "require_same_device",
@@ -56,6 +59,7 @@ __all__ = [
     "resolved_layer_norm_backend",
     "resolved_rms_norm_backend",
     "rms_norm",
+    "rope_table",
     "swiglu_ffn",
     "swiglu_linear",
     "valid_rows",

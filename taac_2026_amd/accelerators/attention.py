@@ -267,6 +267,111 @@ def flash_attention(
     return output if output.dtype == output_dtype else output.to(output_dtype)
 
 
+# ---- query / key preparation: RMSNorm over the model width + rotary embedding ----------------------------------------
+
+_ROPE_TABLES: dict[tuple, torch.Tensor] = {}
+
+
+def rope_table(token_count: int, head_dim: int, rope_base: float, dtype: torch.dtype, device: torch.device) -> torch.Tensor:
+    """``[tokens, head_dim / 2, 2]`` table of (cos, sin) of ``position * rope_base ** (-2i / head_dim)``, computed in
+    float32 and rounded to the activation dtype as ``BFTSAttention._apply_rope`` does
+    (experiments/tokenformer/model.py:174-179); cached per shape, base, dtype and device."""
+    if head_dim % 2 != 0:
+        raise ValueError("hip qk_norm_rope rotates whole heads: head_dim must be even")
+    key = (int(token_count), int(head_dim), float(rope_base), dtype, str(device))
+    table = _ROPE_TABLES.get(key)
+    if table is None:
+        positions = torch.arange(token_count, dtype=torch.float32)
+        frequencies = torch.arange(0, head_dim, 2, dtype=torch.float32)
+        inv_freq = torch.pow(torch.tensor(float(rope_base)), -frequencies / max(1, head_dim))
+        angles = positions[:, None] * inv_freq[None, :]
+        table = torch.stack((angles.cos().to(dtype), angles.sin().to(dtype)), dim=-1).contiguous().to(device)
+        _ROPE_TABLES[key] = table
+    return table
+
+
+def _row_stride(name: str, t: torch.Tensor) -> int | None:
+    """Row stride (elements) when the (..., D) tensor is a uniform stack of contiguous rows, else None."""
+    if t.stride(-1) != 1:
+        return None
+    for dim in range(t.ndim - 2):
+        if t.shape[dim] != 1 and t.stride(dim) != t.stride(dim + 1) * t.shape[dim + 1]:
+            return None
+    return int(t.stride(-2))
+
+
+def qk_norm_rope(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    query_weight: torch.Tensor | None,
+    key_weight: torch.Tensor | None,
+    *,
+    num_heads: int,
+    eps: float = 1e-6,
+    rope_base: float | None = None,
+    token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
+    inplace: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """What the reference's attention layers do to the query and key projections before attention, in one pass:
+    ``RMSNorm(d_model)`` of each (experiments/symbiosis/backbone.py:33-36) and, with ``rope_base``, the rotary embedding
+    over the token positions (experiments/tokenformer/model.py:165-192). ``query`` / ``key``: (batch, tokens, d_model),
+    possibly the ``chunk(3, -1)`` views of a packed projection (rows are read with their stride). ``inplace`` writes the
+    result over the inputs. ``token_rows`` (:func:`valid_rows`) restricts the pass to the valid tokens; the other rows
+    of the result are then zero (new tensors) or untouched (in place)."""
+    name = "hip qk_norm_rope"
+    if query.ndim != 3 or key.shape != query.shape:
+        raise ValueError("qk_norm_rope expects query and key of the same shape (batch, tokens, d_model)")
+    require_same_dtype("qk_norm_rope", query, key)
+    require_cuda_tensors(name, query, key)
+    require_inference(name, query, key)
+    batch, tokens, d_model = query.shape
+    if d_model % int(num_heads) != 0:
+        raise ValueError("d_model must be divisible by num_heads")
+    if (query_weight is None) != (key_weight is None):
+        raise ValueError("qk_norm_rope takes both norm weights or neither")
+    if query_weight is None and rope_base is None:
+        raise ValueError("qk_norm_rope needs norm weights, a rope_base, or both")
+    weights = []
+    for weight in (query_weight, key_weight):
+        if weight is None:
+            weights.append(None)
+            continue
+        if weight.ndim != 1 or weight.shape[0] != d_model:
+            raise ValueError("rms_norm weight must be 1D and match the normalized dimension")
+        require_cuda_tensors(name, weight)
+        weights.append(weight.detach().to(dtype=query.dtype).contiguous())
+    table = None
+    if rope_base is not None:
+        table = rope_table(tokens, d_model // int(num_heads), rope_base, query.dtype, query.device)
+    strides = (_row_stride(name, query), _row_stride(name, key))
+    if strides[0] is None or strides[0] != strides[1]:
+        if inplace:
+            raise ValueError(f"{name}: in-place operation needs query and key with one common uniform row stride")
+        query, key = query.contiguous(), key.contiguous()
+        strides = (d_model, d_model)
+    index, count = (None, None)
+    if token_rows is not None:
+        index, count = token_rows
+        require_cuda_tensors(name, index, count)
+        if index.dtype != torch.int32 or count.dtype != torch.int32 or count.numel() != 1 or index.numel() < batch * tokens:
+            raise ValueError(f"{name}: token_rows must be (int32 row index, int32 scalar count) as returned by valid_rows")
+    if inplace:
+        query_out, key_out, ld_out = query, key, strides[0]
+    else:
+        make = torch.zeros if token_rows is not None else torch.empty
+        query_out = make((batch, tokens, d_model), dtype=query.dtype, device=query.device)
+        key_out = make((batch, tokens, d_model), dtype=query.dtype, device=query.device)
+        ld_out = d_model
+    library = _native.load_library()
+    status = library.taac_qk_norm_rope_fwd(
+        query.data_ptr(), key.data_ptr(), strides[0], query_out.data_ptr(), key_out.data_ptr(), ld_out, batch * tokens,
+        tokens, d_model, int(num_heads), _native.ptr(weights[0]), _native.ptr(weights[1]), float(eps), _native.ptr(table),
+        _native.ptr(index), _native.ptr(count), _native.dtype_code(query.dtype), _native.current_stream(query.device),
+    )
+    _native.check(status, "qk_norm_rope")
+    return query_out, key_out
+
+
 __all__ = [
     "FLASH_ATTENTION_BACKENDS",
     "FlashAttentionMaskPlan",
@@ -274,5 +379,7 @@ __all__ = [
     "flash_attention",
     "hip_flash_attention_kernel",
     "plan_flash_attention_mask",
+    "qk_norm_rope",
     "resolved_flash_attention_backend",
+    "rope_table",
 ]

@@ -265,6 +265,161 @@ int norm_entry(const char* name, const void* x, const void* w, const void* b, vo
   return check_launch(name);
 }
 
+
+// ---- query / key RMSNorm + rotary embedding ---------------------------------------------------------------------------
+//
+// Work unit u = (token slot u / 2, which = u % 2): the query (0) or key (1) row of one token; the two rows of a token
+// go to neighbouring lane groups, so with the packed [q | k | v] layout a wavefront reads one contiguous span. A row is
+// held in registers between the statistic and the scaling, so q and k are read once and written once. The rotary
+// table holds (cos, sin) of feature pair i of a head at [position][2i], [position][2i + 1] in the storage dtype, i.e.
+// a lane that owns features d .. d + VEC - 1 of a head reads the VEC table entries at [position][d ..].
+struct QkParams {
+  const void* q;
+  const void* k;
+  void* q_out;
+  void* k_out;
+  const void* q_weight;
+  const void* k_weight;
+  const void* cos_sin;
+  const int32_t* row_index;
+  const int32_t* n_rows;
+  int64_t ld_in, ld_out, rows;
+  int32_t tokens_per_sample, d_model, head_dim, nvec;
+  float eps;
+};
+
+template <typename T, int G, int NV, int R, bool NORM, bool ROPE>
+__global__ __launch_bounds__(kBlock) void qk_norm_rope_kernel(const QkParams p) {
+  typedef Pack<T> P;
+  typedef typename P::vec vec_t;
+  constexpr int VEC = P::VEC;
+  constexpr int GPB = kBlock / G;
+  const int lane = threadIdx.x % G;
+  const int gid = threadIdx.x / G;
+  const int64_t count = p.n_rows ? static_cast<int64_t>(*p.n_rows) : p.rows;
+
+  vec_t raw[R][NV];
+  vec_t table[ROPE ? R : 1][ROPE ? NV : 1];
+  bool live[R];
+  int64_t row[R];
+  int which[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t unit = (static_cast<int64_t>(blockIdx.x) * R + r) * GPB + gid;
+    const int64_t slot = unit >> 1;
+    which[r] = static_cast<int>(unit & 1);
+    live[r] = slot < count;
+    row[r] = live[r] ? (p.row_index ? static_cast<int64_t>(p.row_index[slot]) : slot) : 0;
+    const T* src = static_cast<const T*>(which[r] ? p.k : p.q) + row[r] * p.ld_in;
+    const int pos = static_cast<int>(row[r] % p.tokens_per_sample);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = lane + i * G;
+      if (live[r] && v < p.nvec) {
+        raw[r][i] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(src + v * VEC));
+        if (ROPE) {
+          const int d = (v * VEC) % p.head_dim;
+          table[ROPE ? r : 0][ROPE ? i : 0] = *reinterpret_cast<const vec_t*>(
+              static_cast<const T*>(p.cos_sin) + static_cast<int64_t>(pos) * p.head_dim + d);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) raw[r][i][e] = 0;
+      }
+    }
+  }
+
+  const float inv_cols = 1.0f / static_cast<float>(p.d_model);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float xf[NV][VEC];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) P::unpack(raw[r][i], xf[i]);
+    float scale = 1.0f;
+    if (NORM) {
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < NV; ++i)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) ss += xf[i][e] * xf[i][e];
+      ss = group_sum<G>(ss);
+      scale = rsqrtf(ss * inv_cols + p.eps);
+    }
+    if (!live[r]) continue;
+    T* dst = static_cast<T*>(which[r] ? p.k_out : p.q_out) + row[r] * p.ld_out;
+    const T* w = static_cast<const T*>(which[r] ? p.k_weight : p.q_weight);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = lane + i * G;
+      if (v >= p.nvec) continue;
+      float of[VEC];
+      if (NORM) {
+        float wf[VEC];
+        P::unpack(*reinterpret_cast<const vec_t*>(w + v * VEC), wf);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) of[e] = xf[i][e] * scale * wf[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) of[e] = xf[i][e];
+      }
+      if (ROPE) {
+        float cs[VEC];
+        P::unpack(table[ROPE ? r : 0][ROPE ? i : 0], cs);
+#pragma unroll
+        for (int e = 0; e < VEC; e += 2) {
+          const float even = of[e], odd = of[e + 1];
+          of[e] = even * cs[e] - odd * cs[e + 1];
+          of[e + 1] = even * cs[e + 1] + odd * cs[e];
+        }
+      }
+      __builtin_nontemporal_store(P::pack(of), reinterpret_cast<vec_t*>(dst + v * VEC));
+    }
+  }
+}
+
+template <typename T, int G, int NV>
+void launch_qk(const QkParams& p, bool norm, bool rope, hipStream_t s) {
+  constexpr int R = NV <= 2 ? 4 : 2;
+  constexpr int GPB = kBlock / G;
+  const int64_t units = 2 * p.rows;
+  const int64_t per_block = static_cast<int64_t>(GPB) * R;
+  const dim3 grid(static_cast<uint32_t>((units + per_block - 1) / per_block));
+  if (norm && rope)
+    hipLaunchKernelGGL((qk_norm_rope_kernel<T, G, NV, R, true, true>), grid, dim3(kBlock), 0, s, p);
+  else if (norm)
+    hipLaunchKernelGGL((qk_norm_rope_kernel<T, G, NV, R, true, false>), grid, dim3(kBlock), 0, s, p);
+  else
+    hipLaunchKernelGGL((qk_norm_rope_kernel<T, G, NV, R, false, true>), grid, dim3(kBlock), 0, s, p);
+}
+
+template <typename T>
+int dispatch_qk(QkParams p, bool norm, bool rope, hipStream_t s, const char* name) {
+  constexpr int VEC = Pack<T>::VEC;
+  const bool ok = p.d_model % VEC == 0 && p.ld_in % VEC == 0 && p.ld_out % VEC == 0 && aligned16(p.q) &&
+                  aligned16(p.k) && aligned16(p.q_out) && aligned16(p.k_out) &&
+                  (!norm || (aligned16(p.q_weight) && aligned16(p.k_weight))) &&
+                  (!rope || (p.head_dim % VEC == 0 && aligned16(p.cos_sin)));
+  if (!ok)
+    return set_error(TAAC_ERR_UNSUPPORTED,
+                     "%s: d_model, head_dim (with a rotary table) and the row strides must be multiples of %d elements "
+                     "and every pointer 16-byte aligned",
+                     name, VEC);
+  p.nvec = p.d_model / VEC;
+  if (p.nvec > kWave * kMaxNV) return set_error(TAAC_ERR_UNSUPPORTED, "%s: d_model above %d", name, kWave * kMaxNV * VEC);
+#define TAAC_QK_CASE(G, NV)               \
+  launch_qk<T, G, NV>(p, norm, rope, s);  \
+  return TAAC_OK;
+  if (p.nvec <= 4) { TAAC_QK_CASE(4, 1) }
+  if (p.nvec <= 8) { TAAC_QK_CASE(8, 1) }
+  if (p.nvec <= 16) { TAAC_QK_CASE(16, 1) }
+  if (p.nvec <= 32) { TAAC_QK_CASE(32, 1) }
+  if (p.nvec <= 64) { TAAC_QK_CASE(64, 1) }
+  if (p.nvec <= 128) { TAAC_QK_CASE(64, 2) }
+  if (p.nvec <= 256) { TAAC_QK_CASE(64, 4) }
+  TAAC_QK_CASE(64, 8)
+#undef TAAC_QK_CASE
+}
+
 }  // namespace
 }  // namespace taac
 
@@ -276,4 +431,53 @@ extern "C" int taac_rmsnorm_fwd(const void* x, const void* w, void* y, int64_t r
 extern "C" int taac_layernorm_fwd(const void* x, const void* w, const void* b, void* y, int64_t rows, int32_t cols,
                                   float eps, int dtype, void* stream) {
   return taac::norm_entry<true>("taac_layernorm_fwd", x, w, b, y, rows, cols, eps, dtype, stream);
+}
+
+extern "C" int taac_qk_norm_rope_fwd(const void* q, const void* k, int64_t ld_in, void* q_out, void* k_out,
+                                     int64_t ld_out, int64_t rows, int32_t tokens_per_sample, int32_t d_model,
+                                     int32_t num_heads, const void* q_weight, const void* k_weight, float eps,
+                                     const void* cos_sin, const int32_t* row_index, const int32_t* n_rows, int dtype,
+                                     void* stream) {
+  using namespace taac;
+  const char* name = "taac_qk_norm_rope_fwd";
+  if (rows < 0 || d_model <= 0 || num_heads <= 0 || tokens_per_sample <= 0)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows >= 0 and d_model, num_heads, tokens_per_sample > 0 required", name);
+  if (d_model % num_heads != 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: d_model must be divisible by num_heads", name);
+  if (rows == 0) return TAAC_OK;
+  if (!q || !k || !q_out || !k_out) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
+  if ((q_weight == nullptr) != (k_weight == nullptr))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: query and key norm weights come together", name);
+  if (!q_weight && !cos_sin) return set_error(TAAC_ERR_INVALID_VALUE, "%s: neither norm weights nor a rotary table", name);
+  if (ld_in < d_model || ld_out < d_model) return set_error(TAAC_ERR_INVALID_VALUE, "%s: row stride below d_model", name);
+  if ((row_index == nullptr) != (n_rows == nullptr))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: row_index and n_rows come together", name);
+  if (rows > 0x3fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: more than 2^30-1 rows", name);
+  QkParams p{};
+  p.q = q;
+  p.k = k;
+  p.q_out = q_out;
+  p.k_out = k_out;
+  p.q_weight = q_weight;
+  p.k_weight = k_weight;
+  p.cos_sin = cos_sin;
+  p.row_index = row_index;
+  p.n_rows = n_rows;
+  p.ld_in = ld_in;
+  p.ld_out = ld_out;
+  p.rows = rows;
+  p.tokens_per_sample = tokens_per_sample;
+  p.d_model = d_model;
+  p.head_dim = d_model / num_heads;
+  p.eps = eps;
+  hipStream_t s = as_stream(stream);
+  const bool norm = q_weight != nullptr, rope = cos_sin != nullptr;
+  int rc;
+  switch (dtype) {
+    case TAAC_F32: rc = dispatch_qk<float>(p, norm, rope, s, name); break;
+    case TAAC_BF16: rc = dispatch_qk<bf16_t>(p, norm, rope, s, name); break;
+    case TAAC_F16: rc = dispatch_qk<f16_t>(p, norm, rope, s, name); break;
+    default: return set_error(TAAC_ERR_INVALID_VALUE, "%s: unknown dtype %d", name, dtype);
+  }
+  if (rc != TAAC_OK) return rc;
+  return check_launch(name);
 }

@@ -1,6 +1,7 @@
 """Model-level primitives built on the HIP operators."""
 
 from taac_2026_amd.modeling.backbone import (
+    BFTSAttention,
     PCVRBackbone,
     SwiGLUFeedForward,
     UnifiedInteractionBlock,
@@ -23,6 +24,7 @@ from taac_2026_amd.modeling.sequence import (
 )
 
 __all__ = [
+    "BFTSAttention",
     "LayerNorm",
     "PCVRBackbone",
     "RMSNorm",

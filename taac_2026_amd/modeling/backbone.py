@@ -1,6 +1,6 @@
 """Unified token backbone blocks on the HIP kernels.
 
-``SwiGLUFeedForward`` / ``UnifiedSelfAttention`` / ``UnifiedInteractionBlock`` keep the constructor signatures,
+``SwiGLUFeedForward`` / ``UnifiedSelfAttention`` / ``BFTSAttention`` / ``UnifiedInteractionBlock`` keep the constructor signatures,
 parameter names (``up``, ``down``, ``qkv``, ``out``, ``attn_norm`` ...) and forward semantics of
 experiments/symbiosis/backbone.py:11-68 (TokenFormer's feed-forward, experiments/tokenformer/model.py:118-128, is the
 same module), with every dense layer, norm and attention call routed to libtaac_hip.so. They are inference modules:
@@ -18,6 +18,7 @@ import torch
 import torch.nn as nn
 
 from taac_2026_amd import _native
+from taac_2026_amd.accelerators.attention import qk_norm_rope
 from taac_2026_amd.accelerators.linear import norm_linear, swiglu_ffn
 from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference
 from taac_2026_amd.modeling.normalization import RMSNorm
@@ -57,6 +58,12 @@ class SwiGLUFeedForward(nn.Module):
 
 
 class UnifiedSelfAttention(nn.Module):
+    """qkv projection -> RMSNorm(d_model) of the query and of the key -> attention -> out projection
+    (experiments/symbiosis/backbone.py:24-48). The two norms (and the rotary embedding of the subclass) run as one
+    in-place pass over the packed projection."""
+
+    rope_base: float | None = None
+
     def __init__(self, d_model: int, num_heads: int, dropout: float = 0.0, *, qk_norm: bool = True) -> None:
         super().__init__()
         self.num_heads = int(num_heads)
@@ -78,9 +85,15 @@ class UnifiedSelfAttention(nn.Module):
         output_dtype = tokens.dtype
         x = tokens if tokens.dtype == torch.bfloat16 else tokens.to(torch.bfloat16)
         query, key, value = _dense(self.qkv, x).chunk(3, dim=-1)
-        if self.query_norm is not None:
-            query = self.query_norm(query)
-            key = self.key_norm(key)
+        if self.query_norm is not None or self.rope_base is not None:
+            # one pass over the q and k columns of the packed projection, in place
+            qk_norm_rope(
+                query, key,
+                None if self.query_norm is None else _bf16(self.query_norm.weight),
+                None if self.key_norm is None else _bf16(self.key_norm.weight),
+                num_heads=self.num_heads, eps=1e-6 if self.query_norm is None else self.query_norm.eps,
+                rope_base=self.rope_base, inplace=True,
+            )
         attended = scaled_dot_product_attention(
             query,
             key,
@@ -94,6 +107,18 @@ class UnifiedSelfAttention(nn.Module):
         )
         out = _dense(self.out, attended, residual=_bf16(residual))
         return out if out.dtype == output_dtype else out.to(output_dtype)
+
+
+class BFTSAttention(UnifiedSelfAttention):
+    """TokenFormer's attention layer (experiments/tokenformer/model.py:139-163): the same layer with an optional
+    rotary embedding of the normalised query and key over the token positions (``_apply_rope``, :165-192)."""
+
+    def __init__(self, d_model: int, num_heads: int, dropout: float = 0.0, *, use_rope: bool, rope_base: float) -> None:
+        super().__init__(d_model, num_heads, dropout, qk_norm=True)
+        if (int(d_model) // int(num_heads)) % 2 != 0 and use_rope:
+            raise ValueError("hip BFTSAttention rotates whole heads: head_dim must be even")
+        self.use_rope = bool(use_rope)
+        self.rope_base = float(rope_base) if use_rope else None
 
 
 class UnifiedInteractionBlock(nn.Module):
@@ -218,6 +243,7 @@ class PCVRBackbone(nn.Module):
 
 
 __all__ = [
+    "BFTSAttention",
     "PCVRBackbone",
     "SwiGLUFeedForward",
     "UnifiedInteractionBlock",

@@ -1,0 +1,152 @@
+"""GPU parity: the one-pass query / key RMSNorm + rotary embedding (through the C ABI) against the CPU oracle, and the
+attention layers that use it."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import reference as oracle
+from taac_2026_amd.api import BFTSAttention, UnifiedSelfAttention, qk_norm_rope, valid_rows
+
+pytestmark = pytest.mark.gpu
+
+# fp32 1e-5 and bf16 2e-2 are the benchmark configuration's tolerances for the norms; fp16 5e-3 is the reference's GPU
+# test tolerance (tests/gpu/infrastructure/accelerators/test_tilelang_ops_cuda.py:205). The rotary table is rounded to
+# the storage dtype on both sides.
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 5e-3}
+
+
+def _draw(batch, tokens, d_model, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    q = (1.5 * torch.randn(batch, tokens, d_model, generator=g)).to(dtype)
+    k = (0.7 * torch.randn(batch, tokens, d_model, generator=g)).to(dtype)
+    wq = (1.0 + 0.1 * torch.randn(d_model, generator=g)).to(dtype)
+    wk = (1.0 + 0.1 * torch.randn(d_model, generator=g)).to(dtype)
+    return q, k, wq, wk
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(2, 7, 256, 8), (3, 5, 64, 2), (1, 33, 1024, 8), (2, 9, 32, 4), (1, 3, 2048, 16),
+                                   (5, 130, 128, 4), (1, 6, 1536, 12)])
+@pytest.mark.parametrize("mode", ["norm", "rope", "norm+rope"])
+def test_qk_norm_rope_matches_oracle(device, dtype, shape, mode):
+    batch, tokens, d_model, heads = shape
+    q, k, wq, wk = _draw(batch, tokens, d_model, dtype, seed=d_model + tokens)
+    weights = (wq, wk) if "norm" in mode else (None, None)
+    base = 10000.0 if "rope" in mode else None
+    expected_q, expected_k = oracle.qk_norm_rope(q, k, *weights, num_heads=heads, eps=1e-6, rope_base=base, fp32=True)
+    with torch.no_grad():
+        got_q, got_k = qk_norm_rope(q.to(device), k.to(device), *(None if w is None else w.to(device) for w in weights),
+                                    num_heads=heads, eps=1e-6, rope_base=base)
+    assert got_q.shape == q.shape and got_q.dtype == dtype and got_q.is_contiguous()
+    torch.testing.assert_close(got_q.cpu().float(), expected_q.float(), rtol=TOL[dtype], atol=TOL[dtype])
+    torch.testing.assert_close(got_k.cpu().float(), expected_k.float(), rtol=TOL[dtype], atol=TOL[dtype])
+    if dtype == torch.bfloat16:
+        # the reference's own evaluation order (every intermediate rounded to bf16) stays within twice the tolerance
+        ref_q, ref_k = oracle.qk_norm_rope(q, k, *weights, num_heads=heads, eps=1e-6, rope_base=base)
+        torch.testing.assert_close(got_q.cpu().float(), ref_q.float(), rtol=4e-2, atol=4e-2)
+        torch.testing.assert_close(got_k.cpu().float(), ref_k.float(), rtol=4e-2, atol=4e-2)
+
+
+def test_qk_norm_rope_in_place_on_a_packed_projection(device):
+    """q and k are the chunk views of a [B, T, 3D] projection: the pass runs in place with the packed row stride, equals
+    the out-of-place result bit for bit and leaves the value columns alone."""
+    batch, tokens, d_model, heads = 3, 50, 256, 8
+    g = torch.Generator().manual_seed(11)
+    packed = torch.randn(batch, tokens, 3 * d_model, generator=g).to(torch.bfloat16)
+    wq = (1.0 + 0.1 * torch.randn(d_model, generator=g)).to(torch.bfloat16)
+    wk = (1.0 + 0.1 * torch.randn(d_model, generator=g)).to(torch.bfloat16)
+    q, k, v = packed.chunk(3, dim=-1)
+    expected_q, expected_k = oracle.qk_norm_rope(q, k, wq, wk, num_heads=heads, rope_base=10000.0, fp32=True)
+    with torch.no_grad():
+        dev = packed.to(device)
+        dq, dk, dv = dev.chunk(3, dim=-1)
+        fresh_q, fresh_k = qk_norm_rope(dq, dk, wq.to(device), wk.to(device), num_heads=heads, rope_base=10000.0)
+        out_q, out_k = qk_norm_rope(dq, dk, wq.to(device), wk.to(device), num_heads=heads, rope_base=10000.0, inplace=True)
+    assert out_q.data_ptr() == dq.data_ptr() and out_k.data_ptr() == dk.data_ptr()
+    assert torch.equal(dq, fresh_q) and torch.equal(dk, fresh_k)
+    assert torch.equal(dv.cpu(), v)
+    torch.testing.assert_close(dq.cpu().float(), expected_q.float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(dk.cpu().float(), expected_k.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_qk_norm_rope_skips_padded_rows(device):
+    """With a row index only the valid tokens are read and written: NaNs at the padded positions change nothing, the
+    valid rows equal the run over all rows bit for bit (positions included: the rotary angle follows the token's place
+    in its sample, not its place in the index), padded rows come back zero (new tensors) or untouched (in place)."""
+    batch, tokens, d_model, heads = 6, 40, 128, 4
+    q, k, wq, wk = _draw(batch, tokens, d_model, torch.bfloat16, seed=3)
+    lengths = torch.tensor([40, 1, 17, 0, 33, 8], dtype=torch.int32)
+    valid = torch.arange(tokens)[None, :] < lengths[:, None]
+    with torch.no_grad():
+        full_q, full_k = qk_norm_rope(q.to(device), k.to(device), wq.to(device), wk.to(device), num_heads=heads,
+                                      rope_base=100.0)
+        index = valid_rows(lengths.to(device), tokens)
+        qn = torch.where(valid[..., None], q, torch.full_like(q, float("nan"))).to(device)
+        kn = torch.where(valid[..., None], k, torch.full_like(k, float("nan"))).to(device)
+        got_q, got_k = qk_norm_rope(qn, kn, wq.to(device), wk.to(device), num_heads=heads, rope_base=100.0,
+                                    token_rows=index)
+        before = qn.clone()
+        qk_norm_rope(qn, kn, wq.to(device), wk.to(device), num_heads=heads, rope_base=100.0, token_rows=index, inplace=True)
+    mask = valid.to(device)
+    assert torch.equal(got_q[mask], full_q[mask]) and torch.equal(got_k[mask], full_k[mask])
+    assert torch.count_nonzero(got_q[~mask]) == 0 and torch.count_nonzero(got_k[~mask]) == 0
+    assert torch.equal(qn[mask], full_q[mask])
+    assert torch.isnan(qn[~mask]).all() and torch.isnan(before[~mask]).all()
+
+
+def test_qk_norm_rope_argument_errors(device):
+    q, k, wq, wk = _draw(2, 4, 64, torch.bfloat16, seed=1)
+    q, k, wq, wk = q.to(device), k.to(device), wq.to(device), wk.to(device)
+    with pytest.raises(ValueError, match="same shape"):
+        qk_norm_rope(q, k[:, :3], wq, wk, num_heads=2)
+    with pytest.raises(ValueError, match="divisible"):
+        qk_norm_rope(q, k, wq, wk, num_heads=3)
+    with pytest.raises(ValueError, match="both norm weights or neither"):
+        qk_norm_rope(q, k, wq, None, num_heads=2)
+    with pytest.raises(ValueError, match="norm weights, a rope_base, or both"):
+        qk_norm_rope(q, k, None, None, num_heads=2)
+    with pytest.raises(ValueError, match="1D and match"):
+        qk_norm_rope(q, k, wq[:32], wk[:32], num_heads=2)
+    with pytest.raises(RuntimeError, match="multiples of 8"):  # head_dim 4: a 16-byte vector would straddle heads
+        qk_norm_rope(q, k, wq, wk, num_heads=16, rope_base=10000.0)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        qk_norm_rope(q.cpu(), k.cpu(), wq.cpu(), wk.cpu(), num_heads=2)
+
+
+@pytest.mark.parametrize("layer", ["symbiosis", "tokenformer", "tokenformer_no_rope"])
+def test_attention_layers_with_normalised_queries_and_keys(device, layer):
+    """``UnifiedSelfAttention`` (experiments/symbiosis/backbone.py:24-48) and ``BFTSAttention``
+    (experiments/tokenformer/model.py:139-163) against the oracle's composition of the same steps."""
+    batch, tokens, d_model, heads = 4, 48, 256, 8
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16)
+    lengths = torch.tensor([48, 5, 31, 16], dtype=torch.int32)
+    if layer == "symbiosis":
+        module = UnifiedSelfAttention(d_model, heads, 0.0)
+        base = None
+    else:
+        base = 10000.0 if layer == "tokenformer" else None
+        module = BFTSAttention(d_model, heads, 0.0, use_rope=base is not None, rope_base=10000.0)
+    with torch.no_grad():
+        module.query_norm.weight.copy_(1.0 + 0.1 * torch.randn(d_model, generator=g))
+        module.key_norm.weight.copy_(1.0 + 0.1 * torch.randn(d_model, generator=g))
+        module.qkv.bias.copy_(0.05 * torch.randn(3 * d_model, generator=g))
+    module = module.eval()
+    bf = lambda t: t.detach().to(torch.bfloat16)
+    q, k, v = F.linear(x, bf(module.qkv.weight), bf(module.qkv.bias)).chunk(3, dim=-1)
+    q, k = oracle.qk_norm_rope(q, k, bf(module.query_norm.weight), bf(module.key_norm.weight), num_heads=heads,
+                               eps=module.query_norm.eps, rope_base=base)
+    attended = oracle.scaled_dot_product_attention(q, k, v, num_heads=heads, key_lengths=lengths, zero_padded_queries=True)
+    expected = F.linear(attended, bf(module.out.weight), bf(module.out.bias))
+    with torch.no_grad():
+        got = module.to(device)(x.to(device), key_lengths=lengths.to(device), zero_padded_queries=True)
+    torch.testing.assert_close(got.cpu().float(), expected.float(), rtol=2e-2, atol=2e-2)
+    if base is not None:  # the rotation matters: without it the result is measurably different
+        plain = UnifiedSelfAttention(d_model, heads, 0.0).eval()
+        plain.load_state_dict(module.state_dict())
+        with torch.no_grad():
+            other = plain.to(device)(x.to(device), key_lengths=lengths.to(device), zero_padded_queries=True)
+        assert (other.float() - got.float()).abs().max().item() > 5e-2

@@ -287,3 +287,83 @@ def test_fp8_linear_definition():
     gate_value = oracle.linear_fp8(x, w, swiglu=True)
     y = (qx.float() @ qw.float().T) * sx * sw
     torch.testing.assert_close(gate_value.float(), (F.silu(y[:, :12]) * y[:, 12:]).to(torch.bfloat16).float())
+
+
+# ---- query / key normalisation and rotary embedding ------------------------------------------------------------------
+
+
+def test_rope_is_a_complex_rotation_of_feature_pairs():
+    """(even + i*odd) * exp(i*angle) in numpy complex128, angle = position * base^(-2i / rotary_dim) from a float64
+    loop: catches a wrong sign, swapped cos / sin, half-split instead of interleaved pairs, a wrong exponent."""
+    batch, tokens, heads, head_dim, base = 2, 7, 3, 8, 100.0
+    q = torch.randn(batch, tokens, heads * head_dim, dtype=torch.float64, generator=torch.Generator().manual_seed(0))
+    k = torch.randn(batch, tokens, heads * head_dim, dtype=torch.float64, generator=torch.Generator().manual_seed(1))
+    got_q, got_k = oracle.apply_rope(q, k, num_heads=heads, rope_base=base)
+    for values, got in ((q, got_q), (k, got_k)):
+        expected = np.zeros_like(values.numpy())
+        for t in range(tokens):
+            for h in range(heads):
+                for i in range(head_dim // 2):
+                    angle = t * base ** (-(2.0 * i) / head_dim)
+                    c = h * head_dim + 2 * i
+                    z = (values[:, t, c].numpy() + 1j * values[:, t, c + 1].numpy()) * np.exp(1j * angle)
+                    expected[:, t, c], expected[:, t, c + 1] = z.real, z.imag
+        # the oracle's angle table is float32 like the reference's
+        np.testing.assert_allclose(got.numpy(), expected, rtol=0, atol=5e-6)
+
+
+def test_rope_invariants():
+    batch, tokens, heads, head_dim = 1, 9, 2, 6
+    q = torch.randn(batch, tokens, heads * head_dim, dtype=torch.float64, generator=torch.Generator().manual_seed(2))
+    k = torch.randn(batch, tokens, heads * head_dim, dtype=torch.float64, generator=torch.Generator().manual_seed(3))
+    rq, rk = oracle.apply_rope(q, k, num_heads=heads, rope_base=10000.0)
+    # position 0 is not rotated; every pair keeps its length
+    torch.testing.assert_close(rq[:, 0], q[:, 0], rtol=0, atol=0)
+    pairs = lambda t: t.reshape(batch, tokens, heads, head_dim // 2, 2).pow(2).sum(-1)
+    torch.testing.assert_close(pairs(rq), pairs(q), rtol=1e-6, atol=1e-6)
+    # the score of a rotated query and key depends only on their distance: same vectors placed at (m, n) and
+    # (m + 3, n + 3) give the same per-head dot product
+    same_q = q[:, :1].expand(-1, tokens, -1).contiguous()
+    same_k = k[:, :1].expand(-1, tokens, -1).contiguous()
+    sq, sk = oracle.apply_rope(same_q, same_k, num_heads=heads, rope_base=10000.0)
+    score = lambda m, n: (sq[0, m].view(heads, head_dim) * sk[0, n].view(heads, head_dim)).sum(-1)
+    torch.testing.assert_close(score(1, 4), score(4, 7), rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(score(5, 2), score(8, 5), rtol=1e-5, atol=1e-5)
+    assert not torch.allclose(score(1, 4), score(1, 5))
+
+
+def test_rope_keeps_an_odd_last_feature_and_tables_round_to_the_activation_dtype():
+    q = torch.randn(1, 4, 10, generator=torch.Generator().manual_seed(4))
+    rq, _ = oracle.apply_rope(q, q.clone(), num_heads=2, rope_base=50.0)  # head_dim 5: rotary_dim 4
+    torch.testing.assert_close(rq.view(1, 4, 2, 5)[..., 4], q.view(1, 4, 2, 5)[..., 4], rtol=0, atol=0)
+    assert not torch.equal(rq.view(1, 4, 2, 5)[:, 1:, :, :4], q.view(1, 4, 2, 5)[:, 1:, :, :4])
+    cos, sin = oracle.rope_tables(6, 8, 10000.0, torch.bfloat16)
+    assert cos.dtype == torch.bfloat16 and cos.shape == (6, 4) and sin.shape == (6, 4)
+    assert float(cos[0, 0]) == 1.0 and float(sin[0, 0]) == 0.0
+    assert abs(float(cos[1, 0]) - math.cos(1.0)) < 2e-3 and abs(float(sin[3, 1]) - math.sin(3 * 10000.0 ** -0.25)) < 2e-3
+
+
+def test_qk_norm_rope_normalises_over_the_model_width_then_rotates():
+    batch, tokens, heads, head_dim = 2, 5, 2, 4
+    d_model = heads * head_dim
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(batch, tokens, d_model, dtype=torch.float64, generator=g)
+    k = torch.randn(batch, tokens, d_model, dtype=torch.float64, generator=g)
+    wq = 1 + 0.1 * torch.randn(d_model, dtype=torch.float64, generator=g)
+    wk = 1 + 0.1 * torch.randn(d_model, dtype=torch.float64, generator=g)
+    nq, nk = oracle.qk_norm_rope(q, k, wq, wk, num_heads=heads, eps=1e-6)
+    # the statistic is the mean square of all d_model features of a token (float64 loop), not of one head
+    np.testing.assert_allclose(nq.numpy().reshape(-1, d_model), _rms_loop(q.numpy().reshape(-1, d_model), wq.numpy(), 1e-6), rtol=1e-12)
+    np.testing.assert_allclose(nk.numpy().reshape(-1, d_model), _rms_loop(k.numpy().reshape(-1, d_model), wk.numpy(), 1e-6), rtol=1e-12)
+    rq, rk = oracle.qk_norm_rope(q, k, wq, wk, num_heads=heads, eps=1e-6, rope_base=10000.0)
+    eq, ek = oracle.apply_rope(nq, nk, num_heads=heads, rope_base=10000.0)
+    torch.testing.assert_close(rq, eq, rtol=0, atol=0)
+    torch.testing.assert_close(rk, ek, rtol=0, atol=0)
+    # rope alone, and the float32 evaluation used as the target of the fused kernel
+    pq, _ = oracle.qk_norm_rope(q, k, None, None, num_heads=heads, rope_base=10000.0)
+    torch.testing.assert_close(pq, oracle.apply_rope(q, k, num_heads=heads, rope_base=10000.0)[0], rtol=0, atol=0)
+    qb, kb = q.to(torch.bfloat16), k.to(torch.bfloat16)
+    f32q, _ = oracle.qk_norm_rope(qb, kb, wq, wk, num_heads=heads, rope_base=10000.0, fp32=True)
+    b16q, _ = oracle.qk_norm_rope(qb, kb, wq, wk, num_heads=heads, rope_base=10000.0)
+    assert f32q.dtype == torch.bfloat16
+    torch.testing.assert_close(f32q.float(), b16q.float(), rtol=2e-2, atol=2e-2)
