@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define TAAC_ABI_VERSION 2
+#define TAAC_ABI_VERSION 3
 
 enum taac_status {
   TAAC_OK = 0,
@@ -87,6 +87,23 @@ int taac_flash_attn_fwd(const void* q, const void* k, const void* v, const int32
                         int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
                         const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4],
                         int is_causal, int zero_padded_queries, int dtype, void* stream);
+
+/*
+ * taac_flash_attn_fwd with one positive factor per query row and per key row, shared by the heads:
+ * scores = (q_row_scale[b, i] * q[b, h, i, :]) . (k_row_scale[b, j] * k[b, h, j, :]) / sqrt(d). q_row_scale: fp32
+ * [B, Tq] contiguous or NULL (all ones); k_row_scale: fp32 [B, Tk] or NULL. The query factor joins the softmax scale
+ * (no rounding); the key rows are multiplied in fp32 and rounded once to the storage dtype on their way to the MFMA.
+ * Factors of rows in the padding are not read. Everything else as taac_flash_attn_fwd.
+ * Use: a per-token normalisation statistic that is only known after the projection that produced q and k has
+ * finished (RMSNorm over the model width: the factor is rsqrt(mean(x^2) + eps), taac_norm_linear_qk_fwd +
+ * taac_row_rstd), so that the normalisation costs no pass over q and k. Replaces, together with those, query_norm /
+ * key_norm of UnifiedSelfAttention.forward (experiments/symbiosis/backbone.py:33-36).
+ */
+int taac_flash_attn_scaled_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
+                               const float* q_row_scale, const float* k_row_scale, void* o, int32_t B, int32_t H,
+                               int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
+                               const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4],
+                               int is_causal, int zero_padded_queries, int dtype, void* stream);
 
 /*
  * Dense layer, bf16 storage / bf16 MFMA / fp32 accumulation: out = epilogue(a @ w^T + bias).
@@ -159,6 +176,35 @@ int taac_qk_norm_rope_fwd(const void* q, const void* k, int64_t ld_in, void* q_o
                           const int32_t* row_index, const int32_t* n_rows, int dtype, void* stream);
 
 /*
+ * taac_norm_linear_fwd for the packed [q | k | v] projection of an attention layer (N = 3 * d_model, K = d_model, no
+ * residual) with the query / key preparation folded into the epilogue. For the 2 * d_model query and key features:
+ *   qk_sumsq[c, r] = sum of squares of the 64 rounded projection values of chunk c (features 64c .. 64c+63) of row r
+ *                    (fp32 [2 * d_model / 64, M]; the statistic of RMSNorm(d_model) is the sum over a projection's
+ *                    chunks, see taac_row_rstd), when qk_sumsq is given;
+ *   out = rotate(projection * qk_weight) with qk_weight [2 * d_model] = query | key norm weights (NULL: ones) and the
+ *         rotation of taac_qk_norm_rope_fwd over cos_sin [tokens_per_sample, head_dim / 2, 2] (NULL: none); row r is
+ *         the token at position r % tokens_per_sample.
+ * The value features are stored unchanged. The per-token factor rsqrt(mean + eps) of the norm commutes with the weight
+ * and the rotation and is left to the attention kernel (taac_flash_attn_scaled_fwd). d_model: 128 or 256; head_dim a
+ * multiple of 8 with a table. Other arguments as taac_norm_linear_fwd.
+ * Replaces: qkv + query_norm + key_norm of UnifiedSelfAttention.forward (experiments/symbiosis/backbone.py:33-36)
+ * and BFTSAttention._apply_rope (experiments/tokenformer/model.py:165-192) without a pass of their own over q and k.
+ */
+int taac_norm_linear_qk_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
+                            const void* bias, const void* packed_weights, void* out, int64_t ldo, int64_t M,
+                            int32_t d_model, int32_t num_heads, int32_t tokens_per_sample, const void* qk_weight,
+                            const void* cos_sin, float* qk_sumsq, const int32_t* rows, const int32_t* n_rows,
+                            void* stream);
+
+/*
+ * rstd[0, r] = rsqrt(sum_c qk_sumsq[c, r] / d_model + eps) over the d_model / 64 chunks of the query projection,
+ * rstd[1, r] likewise over the key projection's chunks: fp32 [2, M], the q_row_scale / k_row_scale of
+ * taac_flash_attn_scaled_fwd. With rows / n_rows only the listed rows are written.
+ */
+int taac_row_rstd(const float* qk_sumsq, int64_t M, int32_t d_model, float eps, float* rstd, const int32_t* rows,
+                  const int32_t* n_rows, void* stream);
+
+/*
  * Row index of the valid tokens of a padded batch: token t of sample b is valid iff t < key_lengths[b] (clamped to
  * [0, T]). Writes rows[i] = b * T + t for the valid tokens in increasing order, *n_rows = their number, and the
  * per-sample offsets (exclusive prefix sums of the lengths, B + 1 values, the last one equal to *n_rows) to
@@ -219,7 +265,8 @@ int taac_masked_mean_head(const void* x, const int32_t* lengths, const void* w_h
 /*
  * Weights of one backbone block; every pointer is a device pointer to bf16 data in torch nn.Linear layout.
  * Field names follow the reference's parameter names (experiments/symbiosis/backbone.py:24-56).
- * Biases may be NULL (treated as zero).
+ * Biases may be NULL (treated as zero). query_norm_weight / key_norm_weight are the attention layer's
+ * RMSNorm(d_model) of its query and key (backbone.py:30-36); NULL gives the plain layer of the benchmark recipe.
  */
 typedef struct taac_block_weights {
   const void* attn_norm_weight; /* [D]                                   */
@@ -232,6 +279,8 @@ typedef struct taac_block_weights {
   const void* up_bias;          /* [2F]                                  */
   const void* down_weight;      /* [D, F]                                */
   const void* down_bias;        /* [D]                                   */
+  const void* query_norm_weight; /* [D] RMSNorm(d_model) of the query projection, or NULL: no query / key norm */
+  const void* key_norm_weight;   /* [D] likewise for the key projection (both or neither)                       */
 } taac_block_weights;
 
 /* Bytes of workspace taac_backbone_fwd needs for the given shape (device memory, 256-byte aligned): activations
@@ -240,19 +289,27 @@ int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D, int32_t F
 
 /*
  * Forward of n_blocks pre-norm blocks plus the pCVR readout:
- *   for each block: h = rmsnorm(x); q,k,v = chunk3(h Wqkv^T + b); a = attention(q,k,v, key_lengths)
+ *   for each block: h = rmsnorm(x); q,k,v = chunk3(h Wqkv^T + b);
+ *                   [q = rmsnorm(q, query_norm_weight); k = rmsnorm(k, key_norm_weight) over all D features]
+ *                   [q, k = rotary embedding over the token positions, table rope_cos_sin]
+ *                   a = attention(q,k,v, key_lengths)
  *                   (padded query rows -> 0); x = x + a Wo^T + b; h2 = rmsnorm(x);
  *                   g,u = chunk2(h2 Wup^T + b); x = x + (silu(g) * u) Wdown^T + b
  *   p = sigmoid(masked_mean(x, lengths) . w_head + b_head)
  * emb: [B, T, D] bf16 (not modified); key_lengths: int32 [B] valid-prefix lengths; hidden_out: [B, T, D] bf16
  * final hidden state or NULL; p: float [B]. heads divides D and D / heads is a multiple of 8.
- * Rows at or beyond key_lengths[b] of hidden_out hold unspecified finite values (they are never read by the readout).
+ * rope_cos_sin: [T, D / heads / 2, 2] bf16 table of (cos, sin) as in taac_qk_norm_rope_fwd, or NULL (no rotation);
+ * the same eps serves every norm. Rows at or beyond key_lengths[b] of hidden_out hold unspecified finite values (they
+ * are never read by the readout).
  * Replaces: the block loop _run_backbone (experiments/symbiosis/model.py:283-292) over UnifiedInteractionBlock
- * (experiments/symbiosis/backbone.py:50-68) in its canonical pre-norm form, plus masked_mean + Linear + sigmoid.
+ * (experiments/symbiosis/backbone.py:50-68) in its canonical pre-norm form, plus masked_mean + Linear + sigmoid; with
+ * the query / key norm weights UnifiedSelfAttention as the reference runs it (backbone.py:24-48), with the table
+ * TokenFormer's BFTSAttention (experiments/tokenformer/model.py:139-192).
  */
 int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, const taac_block_weights* blocks, int32_t n_blocks,
                       const void* w_head, const void* b_head, int32_t B, int32_t T, int32_t D, int32_t heads, int32_t F,
-                      float eps, void* workspace, int64_t workspace_bytes, void* hidden_out, float* p, void* stream);
+                      float eps, const void* rope_cos_sin, void* workspace, int64_t workspace_bytes, void* hidden_out,
+                      float* p, void* stream);
 
 #ifdef __cplusplus
 }

@@ -278,12 +278,19 @@ def swiglu_hidden(x: torch.Tensor, up_weight: torch.Tensor, up_bias: torch.Tenso
     return F.silu(gate) * value if gate_first else gate * F.silu(value)
 
 
-def block(x: torch.Tensor, key_lengths: torch.Tensor, w: dict[str, torch.Tensor], *, num_heads: int, eps: float = 1e-6) -> torch.Tensor:
+def block(x: torch.Tensor, key_lengths: torch.Tensor, w: dict[str, torch.Tensor], *, num_heads: int, eps: float = 1e-6,
+          rope_base: float | None = None) -> torch.Tensor:
     """One canonical pre-norm block: the recipe of ``UnifiedInteractionBlock.forward``
-    (experiments/symbiosis/backbone.py:58-68) without QK-norm and without the padding multiply on the updates
-    (padded rows are don't-care), attention over the valid key prefix with padded query rows set to 0."""
+    (experiments/symbiosis/backbone.py:58-68) without the padding multiply on the updates (padded rows are
+    don't-care), attention over the valid key prefix with padded query rows set to 0. The benchmark recipe has no
+    QK-norm; with ``query_norm.weight`` / ``key_norm.weight`` in ``w`` the query and key are normalised over the model
+    width as the reference layer does (backbone.py:33-36), with ``rope_base`` they are rotated (tokenformer/model.py:
+    153-154)."""
     h = rms_norm(x, w["attn_norm.weight"], eps)
     q, k, v = F.linear(h, w["qkv.weight"], w.get("qkv.bias")).chunk(3, dim=-1)
+    if "query_norm.weight" in w or rope_base is not None:
+        q, k = qk_norm_rope(q, k, w.get("query_norm.weight"), w.get("key_norm.weight"), num_heads=num_heads, eps=eps,
+                            rope_base=rope_base)
     a = scaled_dot_product_attention(q, k, v, num_heads=num_heads, key_lengths=key_lengths, zero_padded_queries=True)
     x = x + F.linear(a, w["out.weight"], w.get("out.bias"))
     h2 = rms_norm(x, w["ffn_norm.weight"], eps)
@@ -292,12 +299,12 @@ def block(x: torch.Tensor, key_lengths: torch.Tensor, w: dict[str, torch.Tensor]
 
 def backbone(emb: torch.Tensor, key_lengths: torch.Tensor, blocks: list[dict[str, torch.Tensor]],
              head_weight: torch.Tensor, head_bias: torch.Tensor | None, *, num_heads: int, eps: float = 1e-6,
-             return_hidden: bool = False):
+             return_hidden: bool = False, rope_base: float | None = None):
     """n pre-norm blocks (``_run_backbone``, experiments/symbiosis/model.py:283-292) + masked mean-pool
     (modeling/sequence.py:54-60) -> Linear(D, 1) -> sigmoid. Returns float32 probabilities [B]."""
     x = emb
     for w in blocks:
-        x = block(x, key_lengths, w, num_heads=num_heads, eps=eps)
+        x = block(x, key_lengths, w, num_heads=num_heads, eps=eps, rope_base=rope_base)
     padding = make_padding_mask(key_lengths.to(torch.int64), x.shape[1])
     pooled = masked_mean(x, padding)
     logits = F.linear(pooled, head_weight.reshape(1, -1), head_bias).squeeze(-1)

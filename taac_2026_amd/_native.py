@@ -22,7 +22,7 @@ TAAC_ERR_LAUNCH = -3
 TAAC_F32, TAAC_BF16, TAAC_F16 = 0, 1, 2
 EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _DTYPE_CODES = {torch.float32: TAAC_F32, torch.bfloat16: TAAC_BF16, torch.float16: TAAC_F16}
 
@@ -48,6 +48,8 @@ class BlockWeights(ctypes.Structure):
         ("up_bias", c_void_p),
         ("down_weight", c_void_p),
         ("down_bias", c_void_p),
+        ("query_norm_weight", c_void_p),
+        ("key_norm_weight", c_void_p),
     ]
 
 
@@ -63,6 +65,12 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "taac_flash_attn_fwd": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32]
+        + [ctypes.POINTER(c_int64)] * 4
+        + [c_int, c_int, c_int, c_void_p],
+    ),
+    "taac_flash_attn_scaled_fwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32]
         + [ctypes.POINTER(c_int64)] * 4
         + [c_int, c_int, c_int, c_void_p],
     ),
@@ -82,6 +90,12 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
          c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p],
     ),
     "taac_valid_rows": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p]),
+    "taac_norm_linear_qk_fwd": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32,
+         c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
+    "taac_row_rstd": (c_int, [c_void_p, c_int64, c_int32, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     "taac_qk_norm_rope_fwd": (
         c_int,
         [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p,
@@ -106,7 +120,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "taac_backbone_fwd": (
         c_int,
         [c_void_p, c_void_p, ctypes.POINTER(BlockWeights), c_int32, c_void_p, c_void_p, c_int32, c_int32, c_int32,
-         c_int32, c_int32, c_float, c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
+         c_int32, c_int32, c_float, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
     ),
 }
 

@@ -16,6 +16,7 @@ from taac_2026_amd.accelerators.linear import (
     linear,
     linear_fp8,
     norm_linear,
+    qkv_projection,
     quantize_fp8,
     swiglu_ffn,
     swiglu_linear,
@@ -51,6 +52,7 @@ __all__ = [
     "norm_linear",
     "plan_flash_attention_mask",
     "qk_norm_rope",
+    "qkv_projection",
     "quantize_fp8",
     "require_cuda_tensors",
     "require_same_device",

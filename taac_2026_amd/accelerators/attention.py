@@ -186,13 +186,17 @@ def hip_flash_attention_kernel(
     key_lengths: torch.Tensor | None,
     *,
     is_causal: bool = False,
-    zero_padded_queries: bool = False,
+    zero_padded_queries: bool | int = False,
+    q_row_scale: torch.Tensor | None = None,
+    k_row_scale: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """``(q, k, v: (B, H, T, d) bf16/fp16, key_lengths: int32[B]) -> (B, H, Tq, d)``.
 
     Same contract as a kernel handed to the reference's ``register_flash_attention_kernel``
-    (flash_attention.py:26,102-104, called at :351-352), extended by the two keyword flags. The output keeps
-    q's memory layout, so (B, T, H, d)-strided views stay copy-free in both directions.
+    (flash_attention.py:26,102-104, called at :351-352), extended by the keyword arguments. The output keeps
+    q's memory layout, so (B, T, H, d)-strided views stay copy-free in both directions. ``q_row_scale`` (B, Tq) /
+    ``k_row_scale`` (B, Tk): optional positive fp32 factors of the query / key rows, shared by the heads (a
+    normalisation statistic applied inside the kernel instead of in a pass of its own).
     """
     library = _native.load_library()
     require_cuda_tensors("hip flash_attention", q, k, v, key_lengths)
@@ -208,12 +212,19 @@ def hip_flash_attention_kernel(
         if key_lengths.dtype != torch.int32 or not key_lengths.is_contiguous():
             key_lengths = key_lengths.to(torch.int32).contiguous()
     batch, heads, query_len, head_dim = q.shape
-    status = library.taac_flash_attn_fwd(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), out.data_ptr(),
+    for scale, rows, label in ((q_row_scale, query_len, "q_row_scale"), (k_row_scale, k.shape[2], "k_row_scale")):
+        if scale is None:
+            continue
+        require_cuda_tensors("hip flash_attention", scale)
+        if scale.dtype != torch.float32 or scale.shape != (batch, rows) or not scale.is_contiguous():
+            raise ValueError(f"flash_attention {label} must be a contiguous float32 tensor of shape (batch, rows)")
+    status = library.taac_flash_attn_scaled_fwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), _native.ptr(q_row_scale),
+        _native.ptr(k_row_scale), out.data_ptr(),
         batch, heads, query_len, k.shape[2], head_dim,
         _native.Int64x4(*q.stride()), _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()),
         _native.Int64x4(*out.stride()),
-        int(bool(is_causal)), int(bool(zero_padded_queries)), _native.dtype_code(q.dtype),
+        int(bool(is_causal)), int(zero_padded_queries), _native.dtype_code(q.dtype),
         _native.current_stream(q.device),
     )
     _native.check(status, "flash_attention")
@@ -236,6 +247,8 @@ def flash_attention(
     threads: int = 128,
     key_lengths: torch.Tensor | None = None,
     zero_padded_queries: bool = False,
+    q_row_scale: torch.Tensor | None = None,
+    k_row_scale: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """``softmax(q k^T / sqrt(d) + mask) v`` for (B, H, T, d) tensors.
 
@@ -245,6 +258,8 @@ def flash_attention(
     (flash_attention.py:249-252, 300-309). ``block_m`` .. ``threads`` are TileLang launch hints, accepted and ignored.
     With ``zero_padded_queries`` the query rows at or beyond ``key_lengths[b]`` are returned as zeros; otherwise they
     attend to the valid keys like every other row (the behaviour of the reference's torch and TileLang paths).
+    ``q_row_scale`` / ``k_row_scale``: optional float32 (B, T) factors of the query / key rows, see
+    :func:`hip_flash_attention_kernel`.
     """
     del block_m, block_n, num_stages, threads
     q, k, v = _normalize_flash_attention_inputs(q, k, v)
@@ -261,7 +276,8 @@ def flash_attention(
         q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
     lengths = plan.key_lengths if (attn_mask is not None or key_lengths is not None) else None
     output = hip_flash_attention_kernel(
-        q, k, v, lengths, is_causal=plan.is_causal, zero_padded_queries=zero_padded_queries
+        q, k, v, lengths, is_causal=plan.is_causal, zero_padded_queries=zero_padded_queries,
+        q_row_scale=q_row_scale, k_row_scale=k_row_scale,
     )
     output = _apply_query_self_mask_fallback(output, v, plan.query_self_mask)
     return output if output.dtype == output_dtype else output.to(output_dtype)

@@ -334,6 +334,93 @@ def norm_linear(
     return out.reshape(*shape[:-1], out_features)
 
 
+def qkv_projection(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None = None,
+    *,
+    num_heads: int,
+    norm_weight: torch.Tensor | None = None,
+    eps: float = 1e-6,
+    query_weight: torch.Tensor | None = None,
+    key_weight: torch.Tensor | None = None,
+    qk_eps: float = 1e-6,
+    rope_base: float | None = None,
+    token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
+    out: torch.Tensor | None = None,
+    scales_out: torch.Tensor | None = None,
+) -> tuple[torch.Tensor, torch.Tensor | None, torch.Tensor | None]:
+    """The packed ``[q | k | v]`` projection of an attention layer with the query / key preparation of the reference's
+    layers folded into its epilogue: ``x (batch, tokens, d_model) -> (qkv (batch, tokens, 3 d_model), q_row_scale,
+    k_row_scale)``.
+
+    ``qkv = F.linear(rmsnorm(x, norm_weight, eps), weight, bias)``; its query and key columns are then multiplied by
+    ``query_weight`` / ``key_weight`` and, with ``rope_base``, rotated over the token positions. The remaining part of
+    ``RMSNorm(d_model)`` of the query and the key (experiments/symbiosis/backbone.py:33-36) is one positive factor per
+    token, ``rsqrt(mean(q^2) + qk_eps)``: it commutes with the weight and the rotation, is returned as
+    ``q_row_scale`` / ``k_row_scale`` (float32 (batch, tokens), None without norm weights) and is applied inside the
+    attention kernel (``hip_flash_attention_kernel(..., q_row_scale=, k_row_scale=)``), so the normalisation and the
+    rotary embedding (experiments/tokenformer/model.py:165-192) cost no pass over q and k. ``out`` (bf16, batch * tokens
+    rows of 3 d_model) and ``scales_out`` (float32 (2, batch, tokens)) let a caller reuse its buffers; with ``token_rows``
+    the rows outside the index are left as they are in them."""
+    name = "hip qkv_projection"
+    require_cuda_tensors(name, x, weight, bias, norm_weight, query_weight, key_weight)
+    require_inference(name, x, weight, bias, norm_weight, query_weight, key_weight)
+    _check_bf16(name, x, weight, bias, norm_weight, query_weight, key_weight)
+    if x.ndim != 3:
+        raise ValueError("qkv_projection expects x of shape (batch, tokens, d_model)")
+    batch, tokens, d_model = x.shape
+    rows, _ = _as_rows(x)
+    _check_weight(name, rows, weight, bias)
+    if weight.shape[0] != 3 * d_model:
+        raise ValueError("qkv_projection weight must have 3 * d_model rows")
+    if d_model % int(num_heads) != 0:
+        raise ValueError("d_model must be divisible by num_heads")
+    if (query_weight is None) != (key_weight is None):
+        raise ValueError("qkv_projection takes both norm weights or neither")
+    if query_weight is None and rope_base is None:
+        raise ValueError("qkv_projection needs norm weights, a rope_base, or both; use norm_linear otherwise")
+    if not (_fused_width(d_model) and d_model % 64 == 0):
+        raise RuntimeError("qkv_projection is built for d_model 128 / 256")
+    qk_weight = None
+    if query_weight is not None:
+        if query_weight.shape != (d_model,) or key_weight.shape != (d_model,):
+            raise ValueError("rms_norm weight must be 1D and match the normalized dimension")
+        qk_weight = torch.cat((query_weight.detach(), key_weight.detach())).contiguous()
+    table = None
+    if rope_base is not None:
+        from taac_2026_amd.accelerators.attention import rope_table
+
+        table = rope_table(tokens, d_model // int(num_heads), rope_base, x.dtype, x.device)
+    packed = _packed_cache.get((weight,), lambda: pack_linear_weight(weight))
+    index, count = _token_rows(name, token_rows, rows)
+    out = _output_rows(name, out, (rows.shape[0], 3 * d_model), index is not None, x)
+    sumsq = scales = None
+    if qk_weight is not None:
+        sumsq = torch.empty(2 * d_model // 64, rows.shape[0], dtype=torch.float32, device=x.device)
+        if scales_out is not None:
+            require_cuda_tensors(name, scales_out)
+            if scales_out.dtype != torch.float32 or scales_out.shape != (2, batch, tokens) or not scales_out.is_contiguous():
+                raise ValueError(f"{name}: scales_out must be a contiguous float32 tensor of shape (2, batch, tokens)")
+            scales = scales_out
+        else:
+            scales = (torch.ones if index is not None else torch.empty)(2, batch, tokens, dtype=torch.float32, device=x.device)
+    library = _native.load_library()
+    stream = _native.current_stream(x.device)
+    status = library.taac_norm_linear_qk_fwd(
+        rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), None, _native.ptr(bias), packed.data_ptr(),
+        out.data_ptr(), 3 * d_model, rows.shape[0], d_model, int(num_heads), tokens, _native.ptr(qk_weight),
+        _native.ptr(table), _native.ptr(sumsq), _native.ptr(index), _native.ptr(count), stream,
+    )
+    _native.check(status, "qkv_projection")
+    if scales is None:
+        return out.view(batch, tokens, 3 * d_model), None, None
+    status = library.taac_row_rstd(sumsq.data_ptr(), rows.shape[0], d_model, float(qk_eps), scales.data_ptr(),
+                                   _native.ptr(index), _native.ptr(count), stream)
+    _native.check(status, "row_rstd")
+    return out.view(batch, tokens, 3 * d_model), scales[0], scales[1]
+
+
 # ---- FP8 (OCP e4m3fn, per-tensor scale = amax / 448) ---------------------------------------------------------------
 
 
@@ -428,6 +515,7 @@ __all__ = [
     "pack_ffn_weights",
     "valid_rows",
     "pack_linear_weight",
+    "qkv_projection",
     "quantize_fp8",
     "swiglu_ffn",
     "swiglu_linear",

@@ -37,6 +37,8 @@ struct AttnParams {
   const void* v;
   void* o;
   const int32_t* key_lengths;
+  const float* q_row_scale;  // [B, Tq] / [B, Tk] factors of the query / key rows (shared by the heads), or null
+  const float* k_row_scale;
   int32_t B, H, Tq, Tk, d;
   int64_t qs[4], ks[4], vs[4], os[4];
   float scale_log2;  // log2(e) / sqrt(d)
@@ -82,7 +84,7 @@ __device__ __forceinline__ uint32_t pack2(T lo, T hi) {
 // hh = (k / 4) % 2 the keys {hh*4 .. hh*4+3} and {8 + hh*4 .. 8 + hh*4+3}; they become 8 consecutive elements.
 __device__ __forceinline__ int vt_pos16(int k) { return ((k >> 2) & 1) * 8 + (k >> 3) * 4 + (k & 3); }
 
-template <typename T, int DP, bool CAUSAL>
+template <typename T, int DP, bool CAUSAL, bool SCALED>
 __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnParams p) {
   typedef typename Vec8<T>::type vec_t;
   typedef typename Vec8<T>::half_type vec4_t;
@@ -159,7 +161,10 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
     for (int j = 0; j < 16; ++j) oacc[mb][j] = 0.f;
   float m_run = -INFINITY;
   float l_run = 0.f;
-  const float c = p.scale_log2;
+  // Row factors: the query's multiplies every score of its column, so it joins the softmax scale of the lane (it is
+  // positive, the running max keeps its meaning); the key's is applied to the key row on its way into LDS.
+  float c = p.scale_log2;
+  if (SCALED && p.q_row_scale != nullptr && qi < q_valid) c *= p.q_row_scale[static_cast<int64_t>(b) * p.Tq + qi];
 
   int wave_kv_end = kv_end;
   if (CAUSAL) {
@@ -175,15 +180,17 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   constexpr int KLD = (kKC * C8 + kThreads - 1) / kThreads;
   constexpr int VLD = ((kKC / 2) * C8 + kThreads - 1) / kThreads;
   vec_t kreg[KLD], vreg[VLD][2];
+  float kfac[SCALED ? KLD : 1];
+  const bool scale_keys = SCALED && p.k_row_scale != nullptr;
   auto fetch = [&](int kc0) {
 #pragma unroll
     for (int i = 0; i < KLD; ++i) {
       const int idx = tid + i * kThreads;
       const int kidx = kc0 + idx / C8;
       const int c8 = idx % C8;
-      kreg[i] = (idx < kKC * C8 && kidx < kv_end && c8 * 8 < p.d)
-                    ? *reinterpret_cast<const vec_t*>(kb + kidx * p.ks[2] + c8 * 8)
-                    : zero_vec;
+      const bool ok = idx < kKC * C8 && kidx < kv_end && c8 * 8 < p.d;
+      kreg[i] = ok ? *reinterpret_cast<const vec_t*>(kb + kidx * p.ks[2] + c8 * 8) : zero_vec;
+      if (SCALED) kfac[SCALED ? i : 0] = (ok && scale_keys) ? p.k_row_scale[static_cast<int64_t>(b) * p.Tk + kidx] : 1.0f;
     }
 #pragma unroll
     for (int i = 0; i < VLD; ++i) {
@@ -200,6 +207,10 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 #pragma unroll
     for (int i = 0; i < KLD; ++i) {
       const int idx = tid + i * kThreads;
+      if (SCALED) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) kreg[i][e] = static_cast<T>(static_cast<float>(kreg[i][e]) * kfac[SCALED ? i : 0]);
+      }
       if (idx < kKC * C8) *reinterpret_cast<vec_t*>(&sK[(idx / C8) * KSTR + (idx % C8) * 8]) = kreg[i];
     }
 #pragma unroll
@@ -335,10 +346,15 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 
 template <typename T, int DP>
 void launch(const AttnParams& p, bool causal, hipStream_t s) {
-  if (causal)
-    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  const bool scaled = p.q_row_scale != nullptr || p.k_row_scale != nullptr;
+  if (causal && scaled)
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  else if (causal)
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, true, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+  else if (scaled)
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
   else
-    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false, false>), dim3(p.total), dim3(kThreads), 0, s, p);
 }
 
 template <typename T>
@@ -358,16 +374,11 @@ bool strides_ok(const int64_t* st) {
   return true;
 }
 
-}  // namespace
-}  // namespace taac
-
-extern "C" int taac_flash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths, void* o,
-                                   int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
-                                   const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
-                                   const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype,
-                                   void* stream) {
-  using namespace taac;
-  const char* name = "taac_flash_attn_fwd";
+int attention_entry(const char* name, const void* q, const void* k, const void* v, const int32_t* key_lengths,
+                    const float* q_row_scale, const float* k_row_scale, void* o, int32_t B, int32_t H, int32_t Tq,
+                    int32_t Tk, int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
+                    const int64_t v_strides[4], const int64_t o_strides[4], int is_causal, int zero_padded_queries,
+                    int dtype, void* stream) {
   if (B < 0 || H < 0 || Tq < 0 || Tk < 0 || d <= 0)
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: negative dimension or non-positive head_dim", name);
   if (dtype != TAAC_BF16 && dtype != TAAC_F16)
@@ -392,6 +403,8 @@ extern "C" int taac_flash_attn_fwd(const void* q, const void* k, const void* v, 
   p.v = v;
   p.o = o;
   p.key_lengths = key_lengths;
+  p.q_row_scale = q_row_scale;
+  p.k_row_scale = k_row_scale;
   p.B = B;
   p.H = H;
   p.Tq = Tq;
@@ -416,4 +429,27 @@ extern "C" int taac_flash_attn_fwd(const void* q, const void* k, const void* v, 
   else
     launch_dp<f16_t>(p, is_causal != 0, s);
   return check_launch(name);
+}
+
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_flash_attn_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths, void* o,
+                                   int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                                   const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
+                                   const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype,
+                                   void* stream) {
+  return taac::attention_entry("taac_flash_attn_fwd", q, k, v, key_lengths, nullptr, nullptr, o, B, H, Tq, Tk, d,
+                               q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries, dtype, stream);
+}
+
+extern "C" int taac_flash_attn_scaled_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
+                                          const float* q_row_scale, const float* k_row_scale, void* o, int32_t B,
+                                          int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
+                                          const int64_t k_strides[4], const int64_t v_strides[4],
+                                          const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype,
+                                          void* stream) {
+  return taac::attention_entry("taac_flash_attn_scaled_fwd", q, k, v, key_lengths, q_row_scale, k_row_scale, o, B, H,
+                               Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries,
+                               dtype, stream);
 }

@@ -165,6 +165,11 @@ inline int64_t packed_block_bytes(int32_t D, int32_t F) {
   return align256(static_cast<int64_t>(3) * D * D * 2) + align256(static_cast<int64_t>(D) * D * 2) +
          align256(static_cast<int64_t>(3) * D * F * 2);
 }
+// Query / key norm scratch of the fused path: per-chunk sums of squares [2D / 64, M], factors [2, M], the
+// concatenated query | key norm weights [2D].
+inline int64_t qk_norm_bytes(int64_t M, int32_t D) {
+  return align256((2 * D / 64) * M * 4) + align256(2 * M * 4) + align256(static_cast<int64_t>(2) * D * 2);
+}
 }  // namespace
 }  // namespace taac
 
@@ -175,13 +180,14 @@ extern "C" int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D
   // x, h (shared with the attention output), qkv, then either the packed weights + the valid-row index (fused path)
   // or the gated hidden state
   const int64_t acts = align256(M * D * 2) * 2 + align256(M * 3 * D * 2);
-  return acts + (fused_shape(D, F) ? n_blocks * packed_block_bytes(D, F) + row_index_bytes(B, T) : align256(M * F * 2));
+  return acts + (fused_shape(D, F) ? n_blocks * packed_block_bytes(D, F) + row_index_bytes(B, T) + qk_norm_bytes(M, D)
+                                   : align256(M * F * 2));
 }
 
 extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, const taac_block_weights* blocks,
                                  int32_t n_blocks, const void* w_head, const void* b_head, int32_t B, int32_t T,
-                                 int32_t D, int32_t heads, int32_t F, float eps, void* workspace,
-                                 int64_t workspace_bytes, void* hidden_out, float* p, void* stream) {
+                                 int32_t D, int32_t heads, int32_t F, float eps, const void* rope_cos_sin,
+                                 void* workspace, int64_t workspace_bytes, void* hidden_out, float* p, void* stream) {
   using namespace taac;
   const char* name = "taac_backbone_fwd";
   if (B < 0 || T < 0 || D <= 0 || F <= 0 || heads <= 0 || n_blocks < 0)
@@ -213,8 +219,14 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
   // padded positions of the residual stream are never read or written. TAAC_DENSE_TOKENS switches this off.
   int32_t* rows = nullptr;
   int32_t* n_rows = nullptr;
+  char* after_packed = packed + static_cast<int64_t>(n_blocks) * packed_block_bytes(D, F);
+  float* qk_sumsq = reinterpret_cast<float*>(after_packed + row_index_bytes(B, T));
+  float* qk_rstd = reinterpret_cast<float*>(reinterpret_cast<char*>(qk_sumsq) + align256((2 * D / 64) * M * 4));
+  bf16_t* qk_weight = reinterpret_cast<bf16_t*>(reinterpret_cast<char*>(qk_rstd) + align256(2 * M * 4));
+  if (rope_cos_sin != nullptr && !aligned16(rope_cos_sin))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: the rotary table must be 16-byte aligned", name);
   if (fused && n_blocks > 0 && getenv("TAAC_DENSE_TOKENS") == nullptr) {
-    rows = reinterpret_cast<int32_t*>(packed + static_cast<int64_t>(n_blocks) * packed_block_bytes(D, F));
+    rows = reinterpret_cast<int32_t*>(after_packed);
     n_rows = rows + M + B + 1;
     const int rc_rows = taac_valid_rows(key_lengths, B, T, rows, n_rows, stream);
     if (rc_rows != TAAC_OK) return rc_rows;
@@ -253,7 +265,32 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
     char* pk_out = pk_qkv + align256(static_cast<int64_t>(3) * D * D * 2);
     char* pk_ffn = pk_out + align256(static_cast<int64_t>(D) * D * 2);
     // attention half
-    if (fused) {
+    if ((w.query_norm_weight == nullptr) != (w.key_norm_weight == nullptr))
+      return set_error(TAAC_ERR_INVALID_VALUE, "%s: block %d: query and key norm weights come together", name, i);
+    const bool qk_norm = w.query_norm_weight != nullptr;
+    const bool qk_prepare = qk_norm || rope_cos_sin != nullptr;
+    const float* q_scale = nullptr;
+    const float* k_scale = nullptr;
+    if (fused && qk_prepare) {
+      // Norm weight, rotation and the norm statistic in the projection's epilogue, the per-token factor of the norm in
+      // the attention kernel: no pass of its own over q and k.
+      if (qk_norm) {
+        if (hipMemcpyAsync(qk_weight, w.query_norm_weight, static_cast<size_t>(D) * 2, hipMemcpyDeviceToDevice,
+                           as_stream(stream)) != hipSuccess ||
+            hipMemcpyAsync(qk_weight + D, w.key_norm_weight, static_cast<size_t>(D) * 2, hipMemcpyDeviceToDevice,
+                           as_stream(stream)) != hipSuccess)
+          return set_error(TAAC_ERR_LAUNCH, "%s: copy of the query / key norm weights failed", name);
+      }
+      if ((rc = taac_norm_linear_qk_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, qkv, 3 * D, M, D,
+                                        heads, T, qk_norm ? qk_weight : nullptr, rope_cos_sin,
+                                        qk_norm ? qk_sumsq : nullptr, rows, n_rows, stream)) != TAAC_OK)
+        return rc;
+      if (qk_norm) {
+        if ((rc = taac_row_rstd(qk_sumsq, M, D, eps, qk_rstd, rows, n_rows, stream)) != TAAC_OK) return rc;
+        q_scale = qk_rstd;
+        k_scale = qk_rstd + M;
+      }
+    } else if (fused) {
       if ((rc = taac_norm_linear_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, nullptr, 0, qkv,
                                      3 * D, M, 3 * D, D, rows, n_rows, stream)) != TAAC_OK)
         return rc;
@@ -263,8 +300,15 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
                                  stream)) != TAAC_OK)
         return rc;
     }
-    if ((rc = taac_flash_attn_fwd(qkv, qkv + D, qkv + 2 * D, key_lengths, h, B, heads, T, T, dh, qkv_strides,
-                                  qkv_strides, qkv_strides, o_strides, 0, rows ? 2 : 1, TAAC_BF16, stream)) != TAAC_OK)
+    if (!fused && qk_prepare) {
+      if ((rc = taac_qk_norm_rope_fwd(qkv, qkv + D, 3 * D, qkv, qkv + D, 3 * D, M, T, D, heads, w.query_norm_weight,
+                                      w.key_norm_weight, eps, rope_cos_sin, nullptr, nullptr, TAAC_BF16, stream)) !=
+          TAAC_OK)
+        return rc;
+    }
+    if ((rc = taac_flash_attn_scaled_fwd(qkv, qkv + D, qkv + 2 * D, key_lengths, q_scale, k_scale, h, B, heads, T, T,
+                                         dh, qkv_strides, qkv_strides, qkv_strides, o_strides, 0, rows ? 2 : 1,
+                                         TAAC_BF16, stream)) != TAAC_OK)
       return rc;
     if (fused) {
       if ((rc = taac_norm_linear_fwd(h, D, nullptr, eps, nullptr, w.out_bias, pk_out, cur, D, x, D, M, D, D, rows,

@@ -55,6 +55,12 @@ struct TsParams {
   const int32_t* rows;      // optional row index: token i lives in row rows[i] of x / residual / out
   const int32_t* n_rows;    // with rows: device pointer to the number of tokens (at most M)
   int32_t units;            // FFN: compute units the last, partial round of workgroups is spread over
+  // Query / key mode of the linear kernel (the packed q | k | v projection of an attention layer):
+  const bf16_t* qk_w;       // [qk_chunks * 64] norm weights of the query and key features (q | k), or null (ones)
+  const bf16_t* cos_sin;    // rotary table [tokens_per_sample][head_dim] of (cos, sin) pairs, or null
+  float* qk_sumsq;          // [qk_chunks][M] sum of squares of a token's 64 features of one chunk
+  int32_t qk_chunks;        // leading 64-feature chunks that belong to the query and key projections
+  int32_t head_dim, tokens_per_sample;
 };
 
 __device__ __forceinline__ float silu_f(float v) {
@@ -238,6 +244,35 @@ __device__ __forceinline__ void tile_to_lds(uint8_t* tile, const f32x16& a0, con
       *reinterpret_cast<bf16x4*>(tile + l32 * kStageRow + col * 2) = ov;
     }
   }
+}
+
+// tile_to_lds that also returns the sum of squares of the lane's 32 rounded values (half of its token's 64 features).
+__device__ __forceinline__ float tile_to_lds_sumsq(uint8_t* tile, const f32x16& a0, const f32x16& a1,
+                                                   const bf16x4 (&bv)[8], int l32, int hh) {
+  float ss = 0.f;
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+    for (int jq = 0; jq < 4; ++jq) {
+      const int col = rb * 32 + jq * 8 + hh * 4;
+      bf16x4 ov;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        ov[e] = static_cast<bf16_t>((rb == 0 ? a0[jq * 4 + e] : a1[jq * 4 + e]) + static_cast<float>(bv[rb * 4 + jq][e]));
+        const float r = static_cast<float>(ov[e]);
+        ss = fmaf(r, r, ss);
+      }
+      *reinterpret_cast<bf16x4*>(tile + l32 * kStageRow + col * 2) = ov;
+    }
+  }
+  return ss;
+}
+
+// Sum of a value and the one held by lane ^ 32.
+__device__ __forceinline__ float half_wave_pair_sum(float v) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, static_cast<uint32_t>(r[0])) + __builtin_bit_cast(float, static_cast<uint32_t>(r[1]));
 }
 
 // Reads the epilogue tile back row-wise (lane -> token 8*i + lane/8, features 8*(lane%8) .. +7), adds the residual
@@ -565,8 +600,9 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 //   and the "memory" clobbers of the hand-written statements keep loads and stores on their side of them.
 // LDS: [3 weight buffers of 2*KS fragments][8 epilogue tiles][bias (N) | norm weight (D)]
 // ------------------------------------------------------------------------------------------------------------------
-template <int D, int TT, bool RES>
+template <int D, int TT, bool RES, bool QK>
 __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParams p) {
+  static_assert(!(QK && RES), "the query / key epilogue has no residual");
   constexpr int NWAVES = 8;
   constexpr int kTokPerWg = NWAVES * 32 * TT;  // TT token tiles of 32 per wavefront
   constexpr int KS = D / 16;
@@ -584,6 +620,9 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
   const int lane = tid % kWave;
   const int l32 = lane % 32;
   const int hh = lane / 32;
+  // QK: (memory row, position in the sample) of the wavefront's tokens, kept in LDS behind the bias and norm weights
+  // (written and read by the same wavefront only), instead of in registers.
+  int2* rowinfo = reinterpret_cast<int2*>(reinterpret_cast<uint8_t*>(bias_lds) + ((p.N + D) * 2 + 15) / 16 * 16) + wave * kWave;
   const int nchunks = p.N / kNC;
   const int64_t count = token_count(p);
   const int num_tiles = static_cast<int>((count + kTokPerWg - 1) / kTokPerWg);
@@ -652,12 +691,16 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     for (int t = 0; t < TT; ++t)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(xf[t][ks]));
+    if (QK) {  // lane <-> token `lane` of the wavefront's 32 * TT tokens
+      const int64_t r = token_row(p, count, tok_base + (lane < 32 * TT ? lane : 0));
+      rowinfo[lane] = make_int2(static_cast<int>(r), static_cast<int>(r % p.tokens_per_sample));
+    }
   };
 
   bf16x8 res_cur[NST], res_next[NST];
   int32_t prow[NST], prow_next[NST];  // rows of the current tile / of the tile the next step belongs to
   int64_t tok_wave = tokens_of_tile(tile_of(0));
-  rows_of_tile(tok_wave, prow);
+  if constexpr (!QK) rows_of_tile(tok_wave, prow);
   stage(chunk_of(0), 0);
   if (total > 1) stage(chunk_of(1), 1);
   if (RES) request_residual(prow, chunk_of(0), res_cur);
@@ -681,7 +724,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
       if (RES) {
 #pragma unroll
         for (int i = 0; i < NST; ++i) prow[i] = prow_next[i];
-      } else {
+      } else if constexpr (!QK) {
         rows_of_tile(tok_wave, prow);
       }
     }
@@ -747,8 +790,65 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     // ---- epilogue of this chunk: bias, rounding, transpose through LDS, residual, 4 stores ---------------------------
     bf16x4 bv[8];
     read_chunk_bias(bias_lds + chunk * kNC, hh, bv);
+    if constexpr (QK) {
+      // Query and key chunks: the sum of squares of the rounded projection goes to qk_sumsq (one value per token and
+      // chunk; the statistic of the norm over the model width is their sum), the features are multiplied by the norm
+      // weight and rotated. The per-token factor rsqrt(mean + eps) commutes with both and is applied by the attention
+      // kernel. Value chunks are stored as they are.
+      const bool qk_chunk = chunk < p.qk_chunks;  // wavefront-uniform
+      const int col8 = chunk * kNC + (lane % 8) * 8;
+      bf16x8 wn;
 #pragma unroll
-    for (int t = 0; t < TT; ++t) {
+      for (int e = 0; e < 8; ++e) wn[e] = static_cast<bf16_t>(1.0f);
+      if (qk_chunk && p.qk_w != nullptr) wn = *reinterpret_cast<const bf16x8*>(p.qk_w + col8);
+      const bool rotate = qk_chunk && p.cos_sin != nullptr;
+      const int d0 = rotate ? col8 % p.head_dim : 0;
+#pragma unroll
+      for (int t = 0; t < TT; ++t) {
+        if (qk_chunk) {
+          float ss = tile_to_lds_sumsq(tile_lds, acc0[t], acc1[t], bv, l32, hh);
+          ss = half_wave_pair_sum(ss);
+          const int row = rowinfo[t * 32 + l32].x;
+          if (hh == 0 && p.qk_sumsq != nullptr) p.qk_sumsq[static_cast<int64_t>(chunk) * p.M + row] = ss;
+        } else {
+          tile_to_lds(tile_lds, acc0[t], acc1[t], bv, l32, hh);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        int2 info[4];
+        bf16x8 cs[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          info[i] = rowinfo[t * 32 + i * 8 + lane / 8];
+          if (rotate)
+            cs[i] = *reinterpret_cast<const bf16x8*>(p.cos_sin + static_cast<int64_t>(info[i].y) * p.head_dim + d0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int row = i * 8 + lane / 8;
+          bf16x8 v = *reinterpret_cast<const bf16x8*>(tile_lds + row * kStageRow + (lane % 8) * 16);
+          if (qk_chunk) {
+            float f[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[e] = static_cast<float>(v[e]) * static_cast<float>(wn[e]);
+            if (rotate) {
+#pragma unroll
+              for (int e = 0; e < 8; e += 2) {
+                const float even = f[e], odd = f[e + 1];
+                const float cv = static_cast<float>(cs[i][e]), sv = static_cast<float>(cs[i][e + 1]);
+                f[e] = even * cv - odd * sv;
+                f[e + 1] = even * sv + odd * cv;
+              }
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = static_cast<bf16_t>(f[e]);
+          }
+          *reinterpret_cast<bf16x8*>(p.out + static_cast<int64_t>(info[i].x) * p.ldo + col8) = v;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < (QK ? 0 : TT); ++t) {
       tile_to_lds(tile_lds, acc0[t], acc1[t], bv, l32, hh);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
@@ -953,12 +1053,22 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
 #undef TAAC_FFN_LAUNCH
 }
 
-extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
-                                    const void* bias, const void* packed_weights, const void* residual, int64_t ldr,
-                                    void* out, int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows,
-                                    const int32_t* n_rows, void* stream) {
-  using namespace taac;
-  const char* name = "taac_norm_linear_fwd";
+namespace taac {
+namespace {
+
+// Query / key extras of the linear kernel; all null / zero for a plain layer.
+struct QkExtras {
+  const void* qk_weight = nullptr;
+  const void* cos_sin = nullptr;
+  float* qk_sumsq = nullptr;
+  int32_t qk_chunks = 0, head_dim = 0, tokens_per_sample = 0;
+  bool enabled = false;
+};
+
+int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
+                       const void* bias, const void* packed_weights, const void* residual, int64_t ldr, void* out,
+                       int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows, const int32_t* n_rows,
+                       const QkExtras& qk, void* stream) {
   if (M < 0 || N <= 0 || K <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, N and K > 0", name);
   if (K != 256 && K != 128)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: token-stationary kernel is built for K = 128 or 256 (got %d)", name, K);
@@ -971,10 +1081,13 @@ extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows and n_rows must be given together", name);
   if (M > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: at most 2^31 rows", name);
   if (!ptr_ok(x, 15) || !ptr_ok(w, 15) || !ptr_ok(out, 15) || !ptr_ok(residual, 15) || !ptr_ok(norm_weight, 15) ||
-      !ptr_ok(bias, 15) || !ptr_ok(packed_weights, 15))
+      !ptr_ok(bias, 15) || !ptr_ok(packed_weights, 15) || !ptr_ok(qk.qk_weight, 15) || !ptr_ok(qk.cos_sin, 15) ||
+      !ptr_ok(qk.qk_sumsq, 3))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
-  if (static_cast<size_t>(3 * 2 * (K / 16)) * kFrag + 8 * static_cast<size_t>(kStageWave) + static_cast<size_t>(N + K) * 2 >
-      kMaxLdsBytes)
+  const size_t rowinfo_bytes = qk.enabled ? 16 + 8 * static_cast<size_t>(kWave) * sizeof(int2) : 0;
+  const size_t lds_bytes = static_cast<size_t>(3 * 2 * (K / 16)) * kFrag + 8 * static_cast<size_t>(kStageWave) +
+                           static_cast<size_t>(N + K) * 2 + rowinfo_bytes;
+  if (lds_bytes > kMaxLdsBytes)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: N=%d does not fit the LDS (limit %d bytes)", name, N, kMaxLdsBytes);
   TsParams p{};
   p.x = static_cast<const bf16_t*>(x);
@@ -992,6 +1105,12 @@ extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm
   p.packed = packed_weights ? 1 : 0;
   p.rows = rows;
   p.n_rows = n_rows;
+  p.qk_w = static_cast<const bf16_t*>(qk.qk_weight);
+  p.cos_sin = static_cast<const bf16_t*>(qk.cos_sin);
+  p.qk_sumsq = qk.qk_sumsq;
+  p.qk_chunks = qk.qk_chunks;
+  p.head_dim = qk.head_dim;
+  p.tokens_per_sample = qk.tokens_per_sample;
   hipStream_t s = as_stream(stream);
   // Without a residual two token tiles per wavefront fit the register file: every weight fragment read from LDS then
   // feeds two MFMAs, which halves the LDS traffic that otherwise caps the kernel.
@@ -1007,21 +1126,91 @@ extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm
     const int limit = atoi(cap);
     if (limit > 0 && limit < grid) grid = limit;
   }
-  const size_t lds_bytes =
-      static_cast<size_t>(3 * 2 * (K / 16)) * kFrag + 8 * static_cast<size_t>(kStageWave) + static_cast<size_t>(N + K) * 2;
-#define TAAC_LIN_LAUNCH(KK, TT, RR)                                                                                  \
+#define TAAC_LIN_LAUNCH(KK, TT, RR, QQ)                                                                           \
   do {                                                                                                            \
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(norm_linear_kernel<KK, TT, RR>),                            \
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(norm_linear_kernel<KK, TT, RR, QQ>),                    \
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)) != hipSuccess) \
       return set_error(TAAC_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", name, lds_bytes);                  \
-    hipLaunchKernelGGL((norm_linear_kernel<KK, TT, RR>), dim3(grid), dim3(8 * kWave), lds_bytes, s, p);               \
+    hipLaunchKernelGGL((norm_linear_kernel<KK, TT, RR, QQ>), dim3(grid), dim3(8 * kWave), lds_bytes, s, p);       \
     return check_launch(name);                                                                                    \
   } while (0)
   if (K == 256) {
-    if (residual) TAAC_LIN_LAUNCH(256, 1, true);
-    TAAC_LIN_LAUNCH(256, 2, false);
+    if (qk.enabled) TAAC_LIN_LAUNCH(256, 2, false, true);
+    if (residual) TAAC_LIN_LAUNCH(256, 1, true, false);
+    TAAC_LIN_LAUNCH(256, 2, false, false);
   }
-  if (residual) TAAC_LIN_LAUNCH(128, 1, true);
-  TAAC_LIN_LAUNCH(128, 2, false);
+  if (qk.enabled) TAAC_LIN_LAUNCH(128, 2, false, true);
+  if (residual) TAAC_LIN_LAUNCH(128, 1, true, false);
+  TAAC_LIN_LAUNCH(128, 2, false, false);
 #undef TAAC_LIN_LAUNCH
+}
+
+// rstd[which][row] = rsqrt(sum over the `parts` chunks of the query (which = 0) / key (1) projection / d_model + eps).
+__global__ __launch_bounds__(256) void row_rstd_kernel(const float* __restrict__ sumsq, float* __restrict__ rstd,
+                                                       int64_t M, int parts, float inv_cols, float eps,
+                                                       const int32_t* __restrict__ rows,
+                                                       const int32_t* __restrict__ n_rows) {
+  const int64_t count = rows ? static_cast<int64_t>(*n_rows) : M;
+  const int64_t unit = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t slot = unit >> 1;
+  const int which = static_cast<int>(unit & 1);
+  if (slot >= count) return;
+  const int64_t row = rows ? static_cast<int64_t>(rows[slot]) : slot;
+  float ss = 0.f;
+  for (int c = 0; c < parts; ++c) ss += sumsq[(static_cast<int64_t>(which) * parts + c) * M + row];
+  rstd[which * M + row] = rsqrtf(ss * inv_cols + eps);
+}
+
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
+                                    const void* bias, const void* packed_weights, const void* residual, int64_t ldr,
+                                    void* out, int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows,
+                                    const int32_t* n_rows, void* stream) {
+  return taac::norm_linear_launch("taac_norm_linear_fwd", x, ldx, norm_weight, eps, w, bias, packed_weights, residual,
+                                  ldr, out, ldo, M, N, K, rows, n_rows, taac::QkExtras{}, stream);
+}
+
+extern "C" int taac_norm_linear_qk_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
+                                       const void* bias, const void* packed_weights, void* out, int64_t ldo, int64_t M,
+                                       int32_t d_model, int32_t num_heads, int32_t tokens_per_sample,
+                                       const void* qk_weight, const void* cos_sin, float* qk_sumsq,
+                                       const int32_t* rows, const int32_t* n_rows, void* stream) {
+  using namespace taac;
+  const char* name = "taac_norm_linear_qk_fwd";
+  if (d_model <= 0 || num_heads <= 0 || tokens_per_sample <= 0 || d_model % num_heads != 0)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: d_model, num_heads, tokens_per_sample > 0 and d_model divisible by num_heads", name);
+  if (d_model % kNC != 0) return set_error(TAAC_ERR_UNSUPPORTED, "%s: d_model must be a multiple of %d", name, kNC);
+  if (cos_sin && (d_model / num_heads) % 8 != 0)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: with a rotary table head_dim must be a multiple of 8", name);
+  if (!qk_sumsq && !qk_weight && !cos_sin)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: nothing to do for the query and key features", name);
+  QkExtras qk;
+  qk.enabled = true;
+  qk.qk_weight = qk_weight;
+  qk.cos_sin = cos_sin;
+  qk.qk_sumsq = qk_sumsq;
+  qk.qk_chunks = 2 * d_model / kNC;
+  qk.head_dim = d_model / num_heads;
+  qk.tokens_per_sample = tokens_per_sample;
+  return norm_linear_launch(name, x, ldx, norm_weight, eps, w, bias, packed_weights, nullptr, 0, out, ldo, M,
+                            3 * d_model, d_model, rows, n_rows, qk, stream);
+}
+
+extern "C" int taac_row_rstd(const float* qk_sumsq, int64_t M, int32_t d_model, float eps, float* rstd,
+                             const int32_t* rows, const int32_t* n_rows, void* stream) {
+  using namespace taac;
+  const char* name = "taac_row_rstd";
+  if (M < 0 || d_model <= 0 || d_model % kNC != 0)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: M >= 0 and d_model a positive multiple of %d required", name, kNC);
+  if (M == 0) return TAAC_OK;
+  if (!qk_sumsq || !rstd) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
+  if ((rows == nullptr) != (n_rows == nullptr))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows and n_rows must be given together", name);
+  if (M > 0x3fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: at most 2^30 rows", name);
+  const int64_t blocks = (2 * M + 255) / 256;
+  hipLaunchKernelGGL(row_rstd_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, as_stream(stream), qk_sumsq,
+                     rstd, M, d_model / kNC, 1.0f / static_cast<float>(d_model), eps, rows, n_rows);
+  return check_launch(name);
 }

@@ -18,8 +18,8 @@ import torch
 import torch.nn as nn
 
 from taac_2026_amd import _native
-from taac_2026_amd.accelerators.attention import qk_norm_rope
-from taac_2026_amd.accelerators.linear import norm_linear, swiglu_ffn
+from taac_2026_amd.accelerators.attention import qk_norm_rope, rope_table
+from taac_2026_amd.accelerators.linear import norm_linear, qkv_projection, swiglu_ffn
 from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference
 from taac_2026_amd.modeling.normalization import RMSNorm
 from taac_2026_amd.modeling.sequence import scaled_dot_product_attention
@@ -84,16 +84,24 @@ class UnifiedSelfAttention(nn.Module):
     ) -> torch.Tensor:
         output_dtype = tokens.dtype
         x = tokens if tokens.dtype == torch.bfloat16 else tokens.to(torch.bfloat16)
-        query, key, value = _dense(self.qkv, x).chunk(3, dim=-1)
-        if self.query_norm is not None or self.rope_base is not None:
-            # one pass over the q and k columns of the packed projection, in place
-            qk_norm_rope(
-                query, key,
-                None if self.query_norm is None else _bf16(self.query_norm.weight),
-                None if self.key_norm is None else _bf16(self.key_norm.weight),
-                num_heads=self.num_heads, eps=1e-6 if self.query_norm is None else self.query_norm.eps,
-                rope_base=self.rope_base, inplace=True,
+        prepare = self.query_norm is not None or self.rope_base is not None
+        query_weight = None if self.query_norm is None else _bf16(self.query_norm.weight)
+        key_weight = None if self.key_norm is None else _bf16(self.key_norm.weight)
+        qk_eps = 1e-6 if self.query_norm is None else self.query_norm.eps
+        q_row_scale = k_row_scale = None
+        if prepare and x.ndim == 3 and x.shape[-1] in (128, 256):
+            # weight, rotation and the norm statistic come out of the projection's epilogue; the per-token factor of
+            # the norm is applied inside the attention kernel: no pass over q and k at all
+            qkv, q_row_scale, k_row_scale = qkv_projection(
+                x, _bf16(self.qkv.weight), _bf16(self.qkv.bias), num_heads=self.num_heads, query_weight=query_weight,
+                key_weight=key_weight, qk_eps=qk_eps, rope_base=self.rope_base,
             )
+            query, key, value = qkv.chunk(3, dim=-1)
+        else:
+            query, key, value = _dense(self.qkv, x).chunk(3, dim=-1)
+            if prepare:  # one pass over the q and k columns of the packed projection, in place
+                qk_norm_rope(query, key, query_weight, key_weight, num_heads=self.num_heads, eps=qk_eps,
+                             rope_base=self.rope_base, inplace=True)
         attended = scaled_dot_product_attention(
             query,
             key,
@@ -104,6 +112,8 @@ class UnifiedSelfAttention(nn.Module):
             training=self.training,
             key_lengths=key_lengths,
             zero_padded_queries=zero_padded_queries,
+            q_row_scale=q_row_scale,
+            k_row_scale=k_row_scale,
         )
         out = _dense(self.out, attended, residual=_bf16(residual))
         return out if out.dtype == output_dtype else out.to(output_dtype)
@@ -150,10 +160,12 @@ class UnifiedInteractionBlock(nn.Module):
 class _PlainBlock(nn.Module):
     """Parameter container of one canonical block: RMSNorm -> MHA -> +res -> RMSNorm -> SwiGLU -> +res."""
 
-    def __init__(self, d_model: int, num_heads: int, d_ff: int) -> None:
+    def __init__(self, d_model: int, num_heads: int, d_ff: int, qk_norm: bool = False) -> None:
         super().__init__()
         self.attn_norm = RMSNorm(d_model)
         self.qkv = nn.Linear(d_model, 3 * d_model)
+        self.query_norm = RMSNorm(d_model) if qk_norm else None
+        self.key_norm = RMSNorm(d_model) if qk_norm else None
         self.out = nn.Linear(d_model, d_model)
         self.ffn_norm = RMSNorm(d_model)
         self.up = nn.Linear(d_model, 2 * d_ff)
@@ -167,14 +179,19 @@ class PCVRBackbone(nn.Module):
     Initialisation: Xavier-uniform weights, zero biases, unit norm weights.
     ``forward(emb[B, T, D] bf16, key_lengths[B] int32) -> p[B] float32``; ``return_hidden=True`` also returns the
     final hidden state (rows at or beyond ``key_lengths[b]`` are unspecified).
+    ``qk_norm=True`` adds the reference layer's ``RMSNorm(d_model)`` of the query and the key
+    (experiments/symbiosis/backbone.py:30-36), ``rope_base`` TokenFormer's rotary embedding of both over the token
+    positions (experiments/tokenformer/model.py:165-192); the benchmark recipe has neither.
     """
 
-    def __init__(self, d_model: int = 256, num_heads: int = 8, d_ff: int = 1024, n_blocks: int = 4, eps: float = 1e-6) -> None:
+    def __init__(self, d_model: int = 256, num_heads: int = 8, d_ff: int = 1024, n_blocks: int = 4, eps: float = 1e-6,
+                 *, qk_norm: bool = False, rope_base: float | None = None) -> None:
         super().__init__()
         if d_model % num_heads != 0:
             raise ValueError("d_model must be divisible by num_heads")
         self.d_model, self.num_heads, self.d_ff, self.eps = int(d_model), int(num_heads), int(d_ff), float(eps)
-        self.blocks = nn.ModuleList(_PlainBlock(d_model, num_heads, d_ff) for _ in range(n_blocks))
+        self.rope_base = None if rope_base is None else float(rope_base)
+        self.blocks = nn.ModuleList(_PlainBlock(d_model, num_heads, d_ff, qk_norm) for _ in range(n_blocks))
         self.head = nn.Linear(d_model, 1)
         self.reset_parameters()
         self._workspace: torch.Tensor | None = None
@@ -225,6 +242,12 @@ class PCVRBackbone(nn.Module):
             slot.ffn_norm_weight = dev(block.ffn_norm.weight)
             slot.up_weight, slot.up_bias = dev(block.up.weight), dev(block.up.bias)
             slot.down_weight, slot.down_bias = dev(block.down.weight), dev(block.down.bias)
+            if block.query_norm is not None:
+                slot.query_norm_weight = dev(block.query_norm.weight)
+                slot.key_norm_weight = dev(block.key_norm.weight)
+        table = None
+        if self.rope_base is not None:
+            table = rope_table(tokens, self.d_model // self.num_heads, self.rope_base, torch.bfloat16, emb.device)
 
         nbytes = library.taac_backbone_workspace_bytes(batch, tokens, self.d_model, self.d_ff, len(self.blocks))
         workspace = self._get_workspace(int(nbytes), emb.device)
@@ -233,7 +256,7 @@ class PCVRBackbone(nn.Module):
         status = library.taac_backbone_fwd(
             emb.data_ptr(), key_lengths.data_ptr(), packed, len(self.blocks), dev(self.head.weight.reshape(-1)),
             dev(self.head.bias), batch, tokens, self.d_model, self.num_heads, self.d_ff, ctypes.c_float(self.eps),
-            workspace.data_ptr(), workspace.numel(), _native.ptr(hidden), probabilities.data_ptr(),
+            _native.ptr(table), workspace.data_ptr(), workspace.numel(), _native.ptr(hidden), probabilities.data_ptr(),
             _native.current_stream(emb.device),
         )
         _native.check(status, "backbone_fwd")

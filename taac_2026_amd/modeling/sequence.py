@@ -80,8 +80,11 @@ def scaled_dot_product_attention(
     threads: int = 128,
     key_lengths: torch.Tensor | None = None,
     zero_padded_queries: bool = False,
+    q_row_scale: torch.Tensor | None = None,
+    k_row_scale: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """Multi-head attention over (B, T, D) projections; returns (B, Tq, D)."""
+    """Multi-head attention over (B, T, D) projections; returns (B, Tq, D). ``q_row_scale`` / ``k_row_scale``: optional
+    float32 (B, T) factors of the query / key rows applied inside the kernel."""
     batch, query_len, d_model = q.shape
     head_dim = d_model // num_heads
     q4 = q.view(batch, query_len, num_heads, head_dim).transpose(1, 2)
@@ -102,6 +105,8 @@ def scaled_dot_product_attention(
         threads=threads,
         key_lengths=key_lengths,
         zero_padded_queries=zero_padded_queries,
+        q_row_scale=q_row_scale,
+        k_row_scale=k_row_scale,
     )
     return output.transpose(1, 2).contiguous().view(batch, query_len, d_model)
 

@@ -71,9 +71,10 @@ def _xavier_uniform(out_features: int, in_features: int, g: torch.Generator) -> 
 
 def backbone_inputs(batch: int = 1024, n_feature_tokens: int = 32, n_sequence_tokens: int = 480, d_model: int = 256,
                     num_heads: int = 8, d_ff: int = 1024, n_blocks: int = 4, *, min_sequence_len: int = 32,
-                    seed: int = SEED) -> BackboneInputs:
+                    seed: int = SEED, qk_norm: bool = False) -> BackboneInputs:
     """Config 4: emb ~ N(0, 0.02) [B, 32 + 480, 256] bf16; sequence valid length ~ U{32..480}; Xavier-uniform
-    weights, zero biases, unit norm weights."""
+    weights, zero biases, unit norm weights. ``qk_norm`` adds the (unit) weights of the reference layer's query / key
+    RMSNorm, which the benchmark recipe leaves out."""
     g = _generator(seed)
     tokens = n_feature_tokens + n_sequence_tokens
     emb = (0.02 * torch.randn(batch, tokens, d_model, generator=g)).to(torch.bfloat16)
@@ -95,6 +96,10 @@ def backbone_inputs(batch: int = 1024, n_feature_tokens: int = 32, n_sequence_to
                 "down.bias": torch.zeros(d_model, dtype=torch.bfloat16),
             }
         )
+    if qk_norm:
+        for weights in blocks:
+            weights["query_norm.weight"] = torch.ones(d_model, dtype=torch.bfloat16)
+            weights["key_norm.weight"] = torch.ones(d_model, dtype=torch.bfloat16)
     head_weight = _xavier_uniform(1, d_model, g).to(torch.bfloat16)
     head_bias = torch.zeros(1, dtype=torch.bfloat16)
     return BackboneInputs(emb, key_lengths, blocks, head_weight, head_bias, num_heads, d_ff)

@@ -68,9 +68,9 @@ def test_host_side_argument_validation_without_gpu():
     assert library.taac_ffn_packed_bytes(256, 1024) == 3 * 256 * 1024 * 2 and library.taac_ffn_packed_bytes(96, 64) == -1
     assert library.taac_linear_packed_bytes(768, 256) == 768 * 256 * 2 and library.taac_linear_packed_bytes(72, 256) == -1
     weights = (_native.BlockWeights * 1)()
-    status = library.taac_backbone_fwd(fake, fake, weights, 1, fake, None, 2, 16, 32, 4, 64, 1e-6, fake, 16, None, fake, None)
+    status = library.taac_backbone_fwd(fake, fake, weights, 1, fake, None, 2, 16, 32, 4, 64, 1e-6, None, fake, 16, None, fake, None)
     assert status == _native.TAAC_ERR_INVALID_VALUE and b"workspace" in library.taac_last_error()
-    status = library.taac_backbone_fwd(fake, fake, weights, 1, fake, None, 2, 16, 32, 5, 64, 1e-6, fake, 1 << 20, None, fake, None)
+    status = library.taac_backbone_fwd(fake, fake, weights, 1, fake, None, 2, 16, 32, 5, 64, 1e-6, None, fake, 1 << 20, None, fake, None)
     assert status == _native.TAAC_ERR_UNSUPPORTED
 
 

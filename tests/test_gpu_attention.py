@@ -150,3 +150,38 @@ def test_errors(device):
     q7 = torch.randn(1, 1, 4, 12, dtype=torch.bfloat16, device=device)
     with pytest.raises(RuntimeError, match="head_dim"):
         flash_attention(q7, q7, q7)
+
+
+@pytest.mark.parametrize("dim,tokens,causal", [(32, 150, False), (64, 70, False), (128, 33, False), (32, 130, True)])
+def test_row_factors_of_queries_and_keys(device, dim, tokens, causal):
+    """One positive factor per query row and per key row (shared by the heads) applied inside the kernel equals attention
+    over the scaled tensors; factors at padded rows are never read (NaN there changes nothing); either may be absent."""
+    from taac_2026_amd.accelerators.attention import hip_flash_attention_kernel
+
+    batch, heads = 4, 3
+    q, k, v = _qkv(batch, heads, tokens, tokens, dim, torch.bfloat16, dim + tokens)
+    g = torch.Generator().manual_seed(9)
+    sq = 0.25 + 2.0 * torch.rand(batch, tokens, generator=g)
+    sk = 0.25 + 2.0 * torch.rand(batch, tokens, generator=g)
+    lengths = torch.tensor([tokens, 7, tokens // 2, 0], dtype=torch.int32)
+    expected = oracle.attention(q.float() * sq[:, None, :, None], k.float() * sk[:, None, :, None], v, lengths,
+                                is_causal=causal, zero_padded_queries=True)
+    valid = torch.arange(tokens)[None, :] < lengths[:, None]
+    sq_nan = torch.where(valid, sq, torch.full_like(sq, float("nan")))
+    sk_nan = torch.where(valid, sk, torch.full_like(sk, float("nan")))
+    with torch.no_grad():
+        args = (q.to(device), k.to(device), v.to(device), lengths.to(device))
+        got = hip_flash_attention_kernel(*args, is_causal=causal, zero_padded_queries=True,
+                                         q_row_scale=sq_nan.to(device), k_row_scale=sk_nan.to(device)).cpu()
+        only_q = hip_flash_attention_kernel(*args, is_causal=causal, zero_padded_queries=True,
+                                            q_row_scale=sq.to(device)).cpu()
+        only_k = hip_flash_attention_kernel(*args, is_causal=causal, zero_padded_queries=True,
+                                            k_row_scale=sk.to(device)).cpu()
+    assert torch.isfinite(got.float()).all()
+    torch.testing.assert_close(got.float(), expected.float(), **BF16_TOL)
+    expected_q = oracle.attention(q.float() * sq[:, None, :, None], k, v, lengths, is_causal=causal, zero_padded_queries=True)
+    expected_k = oracle.attention(q, k.float() * sk[:, None, :, None], v, lengths, is_causal=causal, zero_padded_queries=True)
+    torch.testing.assert_close(only_q.float(), expected_q.float(), **BF16_TOL)
+    torch.testing.assert_close(only_k.float(), expected_k.float(), **BF16_TOL)
+    with pytest.raises(ValueError, match="q_row_scale"):
+        hip_flash_attention_kernel(*args, q_row_scale=sq[:, :-1].contiguous().to(device))

@@ -14,9 +14,9 @@ from taac_2026_amd.api import PCVRBackbone, UnifiedInteractionBlock
 pytestmark = pytest.mark.gpu
 
 
-def _run(inputs, device, return_hidden=True):
+def _run(inputs, device, return_hidden=True, rope_base=None):
     model = PCVRBackbone(d_model=inputs.emb.shape[-1], num_heads=inputs.num_heads, d_ff=inputs.d_ff,
-                         n_blocks=len(inputs.blocks))
+                         n_blocks=len(inputs.blocks), qk_norm="query_norm.weight" in inputs.blocks[0], rope_base=rope_base)
     workloads.load_backbone_state(model, inputs)
     model = model.to(device=device, dtype=torch.bfloat16).eval()
     with torch.no_grad():
@@ -55,6 +55,47 @@ def test_backbone_matches_oracle(device, batch, n_feature, n_sequence):
     assert ours_err.max().item() <= max(3 * spacing, bf16_err.max().item()), (ours_err.max().item(), spacing)
     assert ours_err.mean().item() <= bf16_err.mean().item(), (ours_err.mean().item(), bf16_err.mean().item())
     assert torch.isfinite(hidden).all()
+
+
+@pytest.mark.parametrize("qk_norm,rope_base", [(True, None), (True, 10000.0), (False, 10000.0)])
+@pytest.mark.parametrize("d_model,heads,d_ff", [(256, 8, 512), (128, 4, 256), (64, 2, 96)])
+def test_backbone_with_normalised_and_rotated_queries_and_keys(device, monkeypatch, qk_norm, rope_base, d_model, heads, d_ff):
+    """The block as the reference's layers run it: RMSNorm(d_model) of the query and the key
+    (experiments/symbiosis/backbone.py:33-36) and TokenFormer's rotary embedding (experiments/tokenformer/model.py:
+    153-154). Widths 128 / 256 take the path without a pass over q and k (projection epilogue + attention row
+    factors), width 64 the in-place pass; with and without the valid-row index."""
+    inputs = workloads.backbone_inputs(batch=5, n_feature_tokens=8, n_sequence_tokens=120, d_model=d_model,
+                                       num_heads=heads, d_ff=d_ff, n_blocks=2, min_sequence_len=9, seed=11,
+                                       qk_norm=qk_norm)
+    g = torch.Generator().manual_seed(5)
+    for weights in inputs.blocks:
+        weights["qkv.bias"] = (0.05 * torch.randn(3 * d_model, generator=g)).to(torch.bfloat16)
+        if qk_norm:
+            weights["query_norm.weight"] = (1.0 + 0.1 * torch.randn(d_model, generator=g)).to(torch.bfloat16)
+            weights["key_norm.weight"] = (1.0 + 0.1 * torch.randn(d_model, generator=g)).to(torch.bfloat16)
+    expected_p, expected_h = oracle.backbone(inputs.emb, inputs.key_lengths, inputs.blocks, inputs.head_weight,
+                                             inputs.head_bias, num_heads=heads, return_hidden=True, rope_base=rope_base)
+    blocks32 = [{k: v.float() for k, v in w.items()} for w in inputs.blocks]
+    exact_p, exact_h = oracle.backbone(inputs.emb.float(), inputs.key_lengths, blocks32, inputs.head_weight.float(),
+                                       inputs.head_bias.float(), num_heads=heads, return_hidden=True, rope_base=rope_base)
+    valid = torch.arange(inputs.emb.shape[1])[None, :] < inputs.key_lengths[:, None]
+    results = [_run(inputs, device, rope_base=rope_base)]
+    monkeypatch.setenv("TAAC_DENSE_TOKENS", "1")
+    results.append(_run(inputs, device, rope_base=rope_base))
+    for p, hidden in results:
+        torch.testing.assert_close(p.cpu(), expected_p, rtol=0, atol=2e-2)
+        torch.testing.assert_close(p.cpu(), exact_p, rtol=0, atol=2e-2)
+        ours_err = (hidden.cpu().float()[valid] - exact_h[valid]).abs()
+        bf16_err = (expected_h.float()[valid] - exact_h[valid]).abs()
+        assert (ours_err > 2e-2 + 2e-2 * exact_h[valid].abs()).float().mean().item() <= 1e-3
+        assert ours_err.mean().item() <= 1.25 * bf16_err.mean().item() + 1e-4
+    if d_model != 64:
+        assert torch.equal(results[0][1][valid.to(device)], results[1][1][valid.to(device)])
+    # the preparation is not a no-op: the plain recipe gives measurably different hidden states
+    plain = [{k: v for k, v in w.items() if not k.startswith(("query_norm", "key_norm"))} for w in inputs.blocks]
+    _, plain_h = oracle.backbone(inputs.emb, inputs.key_lengths, plain, inputs.head_weight, inputs.head_bias,
+                                 num_heads=heads, return_hidden=True)
+    assert (plain_h.float()[valid] - expected_h.float()[valid]).abs().max().item() > 5e-2
 
 
 def test_backbone_skips_padded_positions(device, monkeypatch):

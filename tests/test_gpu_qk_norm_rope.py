@@ -150,3 +150,70 @@ def test_attention_layers_with_normalised_queries_and_keys(device, layer):
         with torch.no_grad():
             other = plain.to(device)(x.to(device), key_lengths=lengths.to(device), zero_padded_queries=True)
         assert (other.float() - got.float()).abs().max().item() > 5e-2
+
+
+@pytest.mark.parametrize("d_model,heads", [(256, 8), (128, 4)])
+@pytest.mark.parametrize("mode", ["norm", "rope", "norm+rope"])
+@pytest.mark.parametrize("workgroups", [None, 3])
+def test_qkv_projection_prepares_queries_and_keys_in_its_epilogue(device, monkeypatch, d_model, heads, mode, workgroups):
+    """The packed projection with the query / key preparation in its epilogue: q and k columns come out as
+    rotate(projection * weight), the value columns as the plain projection, and the returned per-token factors are
+    rsqrt(mean(projection^2) + eps); factor * columns equals the oracle's RMSNorm + rotary embedding. Run with one
+    tile per workgroup and with a capped grid (several tiles and the chunk-split last round per workgroup)."""
+    from taac_2026_amd.api import qkv_projection
+
+    if workgroups is not None:
+        monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+    batch, tokens = 5, 333
+    g = torch.Generator().manual_seed(d_model + len(mode))
+    x = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16)
+    nw = (1.0 + 0.1 * torch.randn(d_model, generator=g)).to(torch.bfloat16)
+    w = (torch.randn(3 * d_model, d_model, generator=g) * d_model ** -0.5).to(torch.bfloat16)
+    b = (0.1 * torch.randn(3 * d_model, generator=g)).to(torch.bfloat16)
+    wq = (1.0 + 0.1 * torch.randn(d_model, generator=g)).to(torch.bfloat16)
+    wk = (1.0 + 0.1 * torch.randn(d_model, generator=g)).to(torch.bfloat16)
+    weights = (wq, wk) if "norm" in mode else (None, None)
+    base = 10000.0 if "rope" in mode else None
+    projection = F.linear(oracle.rms_norm_fp32(x, nw).float(), w.float(), b.float()).to(torch.bfloat16)
+    q, k, v = projection.chunk(3, dim=-1)
+    expected_q, expected_k = oracle.qk_norm_rope(q, k, *weights, num_heads=heads, eps=1e-6, rope_base=base, fp32=True)
+    with torch.no_grad():
+        qkv, sq, sk = qkv_projection(x.to(device), w.to(device), b.to(device), num_heads=heads, norm_weight=nw.to(device),
+                                     query_weight=None if weights[0] is None else wq.to(device),
+                                     key_weight=None if weights[1] is None else wk.to(device), rope_base=base)
+    got_q, got_k, got_v = qkv.cpu().chunk(3, dim=-1)
+    torch.testing.assert_close(got_v.float(), v.float(), rtol=2e-2, atol=2e-2)
+    if "norm" in mode:
+        assert sq.shape == (batch, tokens) and sq.dtype == torch.float32
+        # the statistic is taken from the rounded projection the kernel itself produced
+        rstd = lambda t: torch.rsqrt(t.float().pow(2).mean(-1) + 1e-6)
+        torch.testing.assert_close(sq.cpu(), rstd(q), rtol=5e-3, atol=0)
+        torch.testing.assert_close(sk.cpu(), rstd(k), rtol=5e-3, atol=0)
+        got_q = got_q.float() * sq.cpu()[..., None]
+        got_k = got_k.float() * sk.cpu()[..., None]
+    else:
+        assert sq is None and sk is None
+    torch.testing.assert_close(got_q.float(), expected_q.float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(got_k.float(), expected_k.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_qkv_projection_skips_padded_rows(device):
+    from taac_2026_amd.api import qkv_projection
+
+    batch, tokens, d_model, heads = 4, 70, 256, 8
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16)
+    w = (torch.randn(3 * d_model, d_model, generator=g) * d_model ** -0.5).to(torch.bfloat16)
+    wq = (1.0 + 0.1 * torch.randn(d_model, generator=g)).to(torch.bfloat16)
+    lengths = torch.tensor([70, 3, 0, 41], dtype=torch.int32)
+    valid = torch.arange(tokens)[None, :] < lengths[:, None]
+    with torch.no_grad():
+        full, fq, fk = qkv_projection(x.to(device), w.to(device), None, num_heads=heads, query_weight=wq.to(device),
+                                      key_weight=wq.to(device), rope_base=500.0)
+        xn = torch.where(valid[..., None], x, torch.full_like(x, float("nan"))).to(device)
+        got, sq, sk = qkv_projection(xn, w.to(device), None, num_heads=heads, query_weight=wq.to(device),
+                                     key_weight=wq.to(device), rope_base=500.0,
+                                     token_rows=valid_rows(lengths.to(device), tokens))
+    mask = valid.to(device)
+    assert torch.equal(got[mask], full[mask]) and torch.equal(sq[mask], fq[mask]) and torch.equal(sk[mask], fk[mask])
+    assert torch.count_nonzero(got[~mask]) == 0 and torch.isfinite(sq).all() and torch.isfinite(sk).all()
