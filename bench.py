@@ -223,6 +223,69 @@ def _fp8_figures(inputs, device, iters: int) -> dict:
     return figures
 
 
+def _qk_variant_figures(device, batch: int, steps: int) -> dict:
+    """The same backbone with the attention layer as the reference's models run it: RMSNorm(d_model) of the query and
+    the key (Symbiosis) and additionally the rotary embedding (TokenFormer). Reported next to the headline recipe,
+    which has neither; each variant passes its own accuracy gate (2 samples against the CPU oracle) before it is timed.
+    Also the stand-alone one-pass query / key kernel at the step's shape, as an HBM-bound operator."""
+    from oracle import reference as oracle
+    from taac_2026_amd import workloads
+    from taac_2026_amd.api import PCVRBackbone, norm_linear, qk_norm_rope, qkv_projection, valid_rows
+
+    inputs = workloads.backbone_inputs(batch=batch, qk_norm=True)
+    B, T, D = inputs.emb.shape
+    H = inputs.num_heads
+    emb, lengths = inputs.emb.to(device), inputs.key_lengths.to(device)
+    pick = torch.tensor([0, B - 1])
+    out: dict[str, dict] = {}
+    for name, rope_base in (("qk_norm", None), ("qk_norm_rope", 10000.0)):
+        model = PCVRBackbone(d_model=D, num_heads=H, d_ff=inputs.d_ff, n_blocks=len(inputs.blocks), qk_norm=True,
+                             rope_base=rope_base)
+        workloads.load_backbone_state(model, inputs)
+        model = model.to(device=device, dtype=torch.bfloat16).eval()
+        with torch.no_grad():
+            p = model(emb, lengths).cpu()
+            expected = oracle.backbone(inputs.emb[pick], inputs.key_lengths[pick], inputs.blocks, inputs.head_weight,
+                                       inputs.head_bias, num_heads=H, rope_base=rope_base)
+            err = (p[pick] - expected).abs().max().item()
+            if not (torch.isfinite(p).all() and err <= 2e-2):
+                raise SystemExit(f"accuracy gate of the {name} variant failed: max |p - oracle| = {err}")
+            ms = _event_ms(lambda: model(emb, lengths), steps, 3)
+        out[name] = {"ms_per_step": ms, "samples_per_s": B / (ms * 1e-3), "max_abs_err": err}
+    w = {k: v.to(device) for k, v in inputs.blocks[0].items()}
+    with torch.no_grad():
+        index = valid_rows(lengths, T)
+        Mv = float(lengths.sum().item())
+        qkv = torch.zeros(B * T, 3 * D, dtype=torch.bfloat16, device=device)
+        scales = torch.ones(2, B, T, dtype=torch.float32, device=device)
+        plain = _event_ms(lambda: norm_linear(emb, w["qkv.weight"], w["qkv.bias"], norm_weight=w["attn_norm.weight"],
+                                              token_rows=index, out=qkv), 10, 3)
+        fused = _event_ms(lambda: qkv_projection(emb, w["qkv.weight"], w["qkv.bias"], num_heads=H,
+                                                 norm_weight=w["attn_norm.weight"], query_weight=w["query_norm.weight"],
+                                                 key_weight=w["key_norm.weight"], rope_base=10000.0, token_rows=index,
+                                                 out=qkv, scales_out=scales), 10, 3)
+        stats = _event_ms(lambda: qkv_projection(emb, w["qkv.weight"], w["qkv.bias"], num_heads=H,
+                                                 norm_weight=w["attn_norm.weight"], query_weight=w["query_norm.weight"],
+                                                 key_weight=w["key_norm.weight"], token_rows=index, out=qkv,
+                                                 scales_out=scales), 10, 3)
+        q, k, _ = qkv.view(B, T, 3 * D).chunk(3, dim=-1)
+        one_pass = _event_ms(lambda: qk_norm_rope(q, k, w["query_norm.weight"], w["key_norm.weight"], num_heads=H,
+                                                  rope_base=10000.0, token_rows=index, inplace=True), 10, 3)
+        nbytes = 2.0 * 2 * 2 * Mv * D  # q and k rows of the valid tokens, read and written, 2 bytes per element
+    out["kernels"] = {
+        "rmsnorm_qkv_plain_ms": plain,
+        "rmsnorm_qkv_with_norm_statistic_ms": stats,
+        "rmsnorm_qkv_with_weight_and_rotation_ms": fused,
+        "qk_norm_rope_one_pass": {"ms": one_pass, "algorithmic_bytes": nbytes, "gbs": nbytes / one_pass / 1e6,
+                                  "frac_hbm": nbytes / one_pass / 1e6 / HBM_PEAK_GBS},
+        "note": "the step uses the epilogue form (projection + row factors inside attention); the one-pass kernel is "
+                "the stand-alone operator for callers that hold q and k already; the two epilogue figures are whole "
+                "wrapper calls (projection kernel + factor kernel + small torch allocations), the kernel traces under "
+                "profiles/ hold the kernels alone",
+    }
+    return out
+
+
 def _cpu_baseline(inputs, budget_s: float = 20.0) -> dict:
     """The oracle's backbone forward (the reference's torch formulas) on the host cores, on a bounded sample."""
     from oracle import reference as oracle
@@ -268,6 +331,9 @@ def main() -> None:
     parser.add_argument("--skip-operators", action="store_true")
     parser.add_argument("--skip-all-positions", action="store_true",
                         help="do not time the comparison run over the padded positions (keeps kernel traces to one mode)")
+    parser.add_argument("--only-layer-variants", action="store_true",
+                        help="time only the backbone with the reference layers' query / key norm (and rotary embedding) "
+                             "and print those figures (for kernel traces of that mode)")
     args = parser.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU (the path has no cross-GPU stage); use --gpus 1")
@@ -278,6 +344,9 @@ def main() -> None:
     from taac_2026_amd.api import PCVRBackbone
 
     device = torch.device("cuda:0")
+    if args.only_layer_variants:
+        print(json.dumps({"reference_layer_variants": _qk_variant_figures(device, args.batch, args.steps)}))
+        return
     inputs = workloads.backbone_inputs(batch=args.batch)
     B, T, D = inputs.emb.shape
     model = PCVRBackbone(d_model=D, num_heads=inputs.num_heads, d_ff=inputs.d_ff, n_blocks=len(inputs.blocks))
@@ -361,6 +430,7 @@ def main() -> None:
     if not args.skip_operators:
         line["operators"] = _operator_figures(device, iters=20)
         line["fp8_dense_layers"] = _fp8_figures(inputs, device, iters=10)
+        line["reference_layer_variants"] = _qk_variant_figures(device, B, max(args.steps // 2, 1))
     if not args.skip_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(inputs)
         line["gpu_over_cpu"] = value / line["cpu_baseline"]["value"]

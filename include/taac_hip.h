@@ -89,19 +89,22 @@ int taac_flash_attn_fwd(const void* q, const void* k, const void* v, const int32
                         int is_causal, int zero_padded_queries, int dtype, void* stream);
 
 /*
- * taac_flash_attn_fwd with one positive factor per query row and per key row, shared by the heads:
- * scores = (q_row_scale[b, i] * q[b, h, i, :]) . (k_row_scale[b, j] * k[b, h, j, :]) / sqrt(d). q_row_scale: fp32
- * [B, Tq] contiguous or NULL (all ones); k_row_scale: fp32 [B, Tk] or NULL. The query factor joins the softmax scale
- * (no rounding); the key rows are multiplied in fp32 and rounded once to the storage dtype on their way to the MFMA.
- * Factors of rows in the padding are not read. Everything else as taac_flash_attn_fwd.
+ * taac_flash_attn_fwd with one positive factor per query row and per key row, shared by the heads, and one factor
+ * per query feature:
+ *   scores = (q_row_scale[b, i] * q[b, h, i, :] * q_col_scale[h, :]) . (k_row_scale[b, j] * k[b, h, j, :]) / sqrt(d).
+ * q_row_scale: fp32 [B, Tq] contiguous or NULL (all ones); k_row_scale: fp32 [B, Tk] or NULL; q_col_scale: fp32 [H, d]
+ * or NULL. The query row factor joins the softmax scale (no rounding); the query features and the key rows are
+ * multiplied in fp32 and rounded once to the storage dtype on their way to the MFMA. Factors of rows in the padding
+ * are not read. Everything else as taac_flash_attn_fwd. (The weights of a query norm and of a key norm act on a score
+ * only through their product, so q_col_scale = query weight * key weight applies both without touching the keys.)
  * Use: a per-token normalisation statistic that is only known after the projection that produced q and k has
  * finished (RMSNorm over the model width: the factor is rsqrt(mean(x^2) + eps), taac_norm_linear_qk_fwd +
  * taac_row_rstd), so that the normalisation costs no pass over q and k. Replaces, together with those, query_norm /
  * key_norm of UnifiedSelfAttention.forward (experiments/symbiosis/backbone.py:33-36).
  */
 int taac_flash_attn_scaled_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
-                               const float* q_row_scale, const float* k_row_scale, void* o, int32_t B, int32_t H,
-                               int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
+                               const float* q_row_scale, const float* k_row_scale, const float* q_col_scale, void* o,
+                               int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
                                const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4],
                                int is_causal, int zero_padded_queries, int dtype, void* stream);
 

@@ -70,7 +70,8 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "taac_flash_attn_scaled_fwd": (
         c_int,
-        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32]
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32,
+         c_int32]
         + [ctypes.POINTER(c_int64)] * 4
         + [c_int, c_int, c_int, c_void_p],
     ),

@@ -189,6 +189,7 @@ def hip_flash_attention_kernel(
     zero_padded_queries: bool | int = False,
     q_row_scale: torch.Tensor | None = None,
     k_row_scale: torch.Tensor | None = None,
+    q_col_scale: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """``(q, k, v: (B, H, T, d) bf16/fp16, key_lengths: int32[B]) -> (B, H, Tq, d)``.
 
@@ -196,7 +197,8 @@ def hip_flash_attention_kernel(
     (flash_attention.py:26,102-104, called at :351-352), extended by the keyword arguments. The output keeps
     q's memory layout, so (B, T, H, d)-strided views stay copy-free in both directions. ``q_row_scale`` (B, Tq) /
     ``k_row_scale`` (B, Tk): optional positive fp32 factors of the query / key rows, shared by the heads (a
-    normalisation statistic applied inside the kernel instead of in a pass of its own).
+    normalisation statistic applied inside the kernel instead of in a pass of its own); ``q_col_scale`` (H * d,):
+    optional fp32 factors of the query features (the product of a query and a key norm weight).
     """
     library = _native.load_library()
     require_cuda_tensors("hip flash_attention", q, k, v, key_lengths)
@@ -218,9 +220,13 @@ def hip_flash_attention_kernel(
         require_cuda_tensors("hip flash_attention", scale)
         if scale.dtype != torch.float32 or scale.shape != (batch, rows) or not scale.is_contiguous():
             raise ValueError(f"flash_attention {label} must be a contiguous float32 tensor of shape (batch, rows)")
+    if q_col_scale is not None:
+        require_cuda_tensors("hip flash_attention", q_col_scale)
+        if q_col_scale.dtype != torch.float32 or q_col_scale.numel() != heads * head_dim or not q_col_scale.is_contiguous():
+            raise ValueError("flash_attention q_col_scale must be a contiguous float32 tensor of heads * head_dim values")
     status = library.taac_flash_attn_scaled_fwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), _native.ptr(q_row_scale),
-        _native.ptr(k_row_scale), out.data_ptr(),
+        _native.ptr(k_row_scale), _native.ptr(q_col_scale), out.data_ptr(),
         batch, heads, query_len, k.shape[2], head_dim,
         _native.Int64x4(*q.stride()), _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()),
         _native.Int64x4(*out.stride()),
@@ -249,6 +255,7 @@ def flash_attention(
     zero_padded_queries: bool = False,
     q_row_scale: torch.Tensor | None = None,
     k_row_scale: torch.Tensor | None = None,
+    q_col_scale: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """``softmax(q k^T / sqrt(d) + mask) v`` for (B, H, T, d) tensors.
 
@@ -258,8 +265,8 @@ def flash_attention(
     (flash_attention.py:249-252, 300-309). ``block_m`` .. ``threads`` are TileLang launch hints, accepted and ignored.
     With ``zero_padded_queries`` the query rows at or beyond ``key_lengths[b]`` are returned as zeros; otherwise they
     attend to the valid keys like every other row (the behaviour of the reference's torch and TileLang paths).
-    ``q_row_scale`` / ``k_row_scale``: optional float32 (B, T) factors of the query / key rows, see
-    :func:`hip_flash_attention_kernel`.
+    ``q_row_scale`` / ``k_row_scale`` / ``q_col_scale``: optional float32 factors of the query / key rows and of the
+    query features, see :func:`hip_flash_attention_kernel`.
     """
     del block_m, block_n, num_stages, threads
     q, k, v = _normalize_flash_attention_inputs(q, k, v)
@@ -277,7 +284,7 @@ def flash_attention(
     lengths = plan.key_lengths if (attn_mask is not None or key_lengths is not None) else None
     output = hip_flash_attention_kernel(
         q, k, v, lengths, is_causal=plan.is_causal, zero_padded_queries=zero_padded_queries,
-        q_row_scale=q_row_scale, k_row_scale=k_row_scale,
+        q_row_scale=q_row_scale, k_row_scale=k_row_scale, q_col_scale=q_col_scale,
     )
     output = _apply_query_self_mask_fallback(output, v, plan.query_self_mask)
     return output if output.dtype == output_dtype else output.to(output_dtype)

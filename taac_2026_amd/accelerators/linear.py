@@ -349,18 +349,20 @@ def qkv_projection(
     token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
     out: torch.Tensor | None = None,
     scales_out: torch.Tensor | None = None,
-) -> tuple[torch.Tensor, torch.Tensor | None, torch.Tensor | None]:
+) -> tuple[torch.Tensor, torch.Tensor | None, torch.Tensor | None, torch.Tensor | None]:
     """The packed ``[q | k | v]`` projection of an attention layer with the query / key preparation of the reference's
     layers folded into its epilogue: ``x (batch, tokens, d_model) -> (qkv (batch, tokens, 3 d_model), q_row_scale,
-    k_row_scale)``.
+    k_row_scale, q_col_scale)``; hand the three factors to the attention call
+    (``scaled_dot_product_attention(..., q_row_scale=, k_row_scale=, q_col_scale=)``).
 
-    ``qkv = F.linear(rmsnorm(x, norm_weight, eps), weight, bias)``; its query and key columns are then multiplied by
-    ``query_weight`` / ``key_weight`` and, with ``rope_base``, rotated over the token positions. The remaining part of
-    ``RMSNorm(d_model)`` of the query and the key (experiments/symbiosis/backbone.py:33-36) is one positive factor per
-    token, ``rsqrt(mean(q^2) + qk_eps)``: it commutes with the weight and the rotation, is returned as
-    ``q_row_scale`` / ``k_row_scale`` (float32 (batch, tokens), None without norm weights) and is applied inside the
-    attention kernel (``hip_flash_attention_kernel(..., q_row_scale=, k_row_scale=)``), so the normalisation and the
-    rotary embedding (experiments/tokenformer/model.py:165-192) cost no pass over q and k. ``out`` (bf16, batch * tokens
+    ``qkv = F.linear(rmsnorm(x, norm_weight, eps), weight, bias)``. ``RMSNorm(d_model)`` of the query and of the key
+    (experiments/symbiosis/backbone.py:33-36) splits into one positive factor per token, ``rsqrt(mean(q^2) + qk_eps)``,
+    whose statistic the epilogue collects and which is returned as ``q_row_scale`` / ``k_row_scale`` (float32
+    (batch, tokens)), and the norm weights. Without a rotation the two weights act on a score only through their
+    product, returned as ``q_col_scale`` (float32 (d_model,)) and applied to the query inside the attention kernel: the
+    q and k columns of ``qkv`` are then the plain projection. With ``rope_base`` the epilogue multiplies the query and
+    key columns by their weights and rotates them over the token positions (experiments/tokenformer/model.py:165-192)
+    and ``q_col_scale`` is None. Either way the preparation costs no pass over q and k. ``out`` (bf16, batch * tokens
     rows of 3 d_model) and ``scales_out`` (float32 (2, batch, tokens)) let a caller reuse its buffers; with ``token_rows``
     the rows outside the index are left as they are in them."""
     name = "hip qkv_projection"
@@ -382,11 +384,14 @@ def qkv_projection(
         raise ValueError("qkv_projection needs norm weights, a rope_base, or both; use norm_linear otherwise")
     if not (_fused_width(d_model) and d_model % 64 == 0):
         raise RuntimeError("qkv_projection is built for d_model 128 / 256")
-    qk_weight = None
+    qk_weight = col_scale = None
     if query_weight is not None:
         if query_weight.shape != (d_model,) or key_weight.shape != (d_model,):
             raise ValueError("rms_norm weight must be 1D and match the normalized dimension")
-        qk_weight = torch.cat((query_weight.detach(), key_weight.detach())).contiguous()
+        if rope_base is None:
+            col_scale = (query_weight.detach().float() * key_weight.detach().float()).contiguous()
+        else:
+            qk_weight = torch.cat((query_weight.detach(), key_weight.detach())).contiguous()
     table = None
     if rope_base is not None:
         from taac_2026_amd.accelerators.attention import rope_table
@@ -396,7 +401,7 @@ def qkv_projection(
     index, count = _token_rows(name, token_rows, rows)
     out = _output_rows(name, out, (rows.shape[0], 3 * d_model), index is not None, x)
     sumsq = scales = None
-    if qk_weight is not None:
+    if query_weight is not None:
         sumsq = torch.empty(2 * d_model // 64, rows.shape[0], dtype=torch.float32, device=x.device)
         if scales_out is not None:
             require_cuda_tensors(name, scales_out)
@@ -414,11 +419,11 @@ def qkv_projection(
     )
     _native.check(status, "qkv_projection")
     if scales is None:
-        return out.view(batch, tokens, 3 * d_model), None, None
+        return out.view(batch, tokens, 3 * d_model), None, None, None
     status = library.taac_row_rstd(sumsq.data_ptr(), rows.shape[0], d_model, float(qk_eps), scales.data_ptr(),
                                    _native.ptr(index), _native.ptr(count), stream)
     _native.check(status, "row_rstd")
-    return out.view(batch, tokens, 3 * d_model), scales[0], scales[1]
+    return out.view(batch, tokens, 3 * d_model), scales[0], scales[1], col_scale
 
 
 # ---- FP8 (OCP e4m3fn, per-tensor scale = amax / 448) ---------------------------------------------------------------

@@ -39,6 +39,7 @@ struct AttnParams {
   const int32_t* key_lengths;
   const float* q_row_scale;  // [B, Tq] / [B, Tk] factors of the query / key rows (shared by the heads), or null
   const float* k_row_scale;
+  const float* q_col_scale;  // [H, d] factors of the query features, or null
   int32_t B, H, Tq, Tk, d;
   int64_t qs[4], ks[4], vs[4], os[4];
   float scale_log2;  // log2(e) / sqrt(d)
@@ -152,6 +153,11 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
     const int col = 16 * s + 8 * hh;
     // Query rows in the padding are not read (they may be uninitialised memory): a zero query keeps the arithmetic finite.
     qf[s] = (qi < q_valid && col < p.d) ? *reinterpret_cast<const vec_t*>(qb + qi * p.qs[2] + col) : zero_vec;
+    if (SCALED && p.q_col_scale != nullptr && col < p.d) {
+      const float* cf = p.q_col_scale + h * p.d + col;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<T>(static_cast<float>(qf[s][e]) * cf[e]);
+    }
   }
 
   f32x16 oacc[MB];
@@ -346,7 +352,7 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 
 template <typename T, int DP>
 void launch(const AttnParams& p, bool causal, hipStream_t s) {
-  const bool scaled = p.q_row_scale != nullptr || p.k_row_scale != nullptr;
+  const bool scaled = p.q_row_scale != nullptr || p.k_row_scale != nullptr || p.q_col_scale != nullptr;
   if (causal && scaled)
     hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
   else if (causal)
@@ -375,7 +381,8 @@ bool strides_ok(const int64_t* st) {
 }
 
 int attention_entry(const char* name, const void* q, const void* k, const void* v, const int32_t* key_lengths,
-                    const float* q_row_scale, const float* k_row_scale, void* o, int32_t B, int32_t H, int32_t Tq,
+                    const float* q_row_scale, const float* k_row_scale, const float* q_col_scale, void* o, int32_t B,
+                    int32_t H, int32_t Tq,
                     int32_t Tk, int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
                     const int64_t v_strides[4], const int64_t o_strides[4], int is_causal, int zero_padded_queries,
                     int dtype, void* stream) {
@@ -405,6 +412,7 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   p.key_lengths = key_lengths;
   p.q_row_scale = q_row_scale;
   p.k_row_scale = k_row_scale;
+  p.q_col_scale = q_col_scale;
   p.B = B;
   p.H = H;
   p.Tq = Tq;
@@ -439,17 +447,18 @@ extern "C" int taac_flash_attn_fwd(const void* q, const void* k, const void* v, 
                                    const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
                                    const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype,
                                    void* stream) {
-  return taac::attention_entry("taac_flash_attn_fwd", q, k, v, key_lengths, nullptr, nullptr, o, B, H, Tq, Tk, d,
+  return taac::attention_entry("taac_flash_attn_fwd", q, k, v, key_lengths, nullptr, nullptr, nullptr, o, B, H, Tq, Tk, d,
                                q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries, dtype, stream);
 }
 
 extern "C" int taac_flash_attn_scaled_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
-                                          const float* q_row_scale, const float* k_row_scale, void* o, int32_t B,
-                                          int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
+                                          const float* q_row_scale, const float* k_row_scale,
+                                          const float* q_col_scale, void* o, int32_t B, int32_t H, int32_t Tq,
+                                          int32_t Tk, int32_t d, const int64_t q_strides[4],
                                           const int64_t k_strides[4], const int64_t v_strides[4],
                                           const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype,
                                           void* stream) {
-  return taac::attention_entry("taac_flash_attn_scaled_fwd", q, k, v, key_lengths, q_row_scale, k_row_scale, o, B, H,
-                               Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries,
+  return taac::attention_entry("taac_flash_attn_scaled_fwd", q, k, v, key_lengths, q_row_scale, k_row_scale,
+                               q_col_scale, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries,
                                dtype, stream);
 }

@@ -100,6 +100,15 @@ __global__ __launch_bounds__(kBlock) void valid_rows_kernel(const int32_t* __res
   if (t < len) rows[offsets[b] + t] = b * T + t;
 }
 
+// prod[d] = wq[d] * wk[d] in fp32: the weights of a query and a key norm act on an attention score only through their
+// product, which the attention kernel applies to the query features.
+__global__ __launch_bounds__(kBlock) void weight_product_kernel(const bf16_t* __restrict__ wq,
+                                                                const bf16_t* __restrict__ wk,
+                                                                float* __restrict__ prod, int D) {
+  const int d = blockIdx.x * kBlock + threadIdx.x;
+  if (d < D) prod[d] = static_cast<float>(wq[d]) * static_cast<float>(wk[d]);
+}
+
 // Zero-fills the rows of the padded positions of x [B, T, D] (16 bytes per thread).
 __global__ __launch_bounds__(kBlock) void zero_padded_rows_kernel(bf16_t* __restrict__ x,
                                                                   const int32_t* __restrict__ lengths, int T, int D) {
@@ -168,7 +177,7 @@ inline int64_t packed_block_bytes(int32_t D, int32_t F) {
 // Query / key norm scratch of the fused path: per-chunk sums of squares [2D / 64, M], factors [2, M], the
 // concatenated query | key norm weights [2D].
 inline int64_t qk_norm_bytes(int64_t M, int32_t D) {
-  return align256((2 * D / 64) * M * 4) + align256(2 * M * 4) + align256(static_cast<int64_t>(2) * D * 2);
+  return align256((2 * D / 64) * M * 4) + align256(2 * M * 4) + align256(static_cast<int64_t>(D) * 4);
 }
 }  // namespace
 }  // namespace taac
@@ -271,10 +280,22 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
     const bool qk_prepare = qk_norm || rope_cos_sin != nullptr;
     const float* q_scale = nullptr;
     const float* k_scale = nullptr;
+    const float* q_col_scale = nullptr;
     if (fused && qk_prepare) {
-      // Norm weight, rotation and the norm statistic in the projection's epilogue, the per-token factor of the norm in
-      // the attention kernel: no pass of its own over q and k.
-      if (qk_norm) {
+      // The norm statistic comes out of the projection's epilogue and the per-token factor of the norm is applied by
+      // the attention kernel. Without a rotation the two norm weights go to the attention kernel as well, as their
+      // product on the query features; with one, the epilogue applies weight and rotation. Either way there is no
+      // pass of its own over q and k.
+      const bool weights_in_epilogue = qk_norm && rope_cos_sin != nullptr;
+      if (qk_norm && !weights_in_epilogue) {
+        float* prod = reinterpret_cast<float*>(qk_weight);
+        hipLaunchKernelGGL(weight_product_kernel, dim3((D + kBlock - 1) / kBlock), dim3(kBlock), 0, as_stream(stream),
+                           static_cast<const bf16_t*>(w.query_norm_weight),
+                           static_cast<const bf16_t*>(w.key_norm_weight), prod, D);
+        if ((rc = check_launch(name)) != TAAC_OK) return rc;
+        q_col_scale = prod;
+      }
+      if (weights_in_epilogue) {
         if (hipMemcpyAsync(qk_weight, w.query_norm_weight, static_cast<size_t>(D) * 2, hipMemcpyDeviceToDevice,
                            as_stream(stream)) != hipSuccess ||
             hipMemcpyAsync(qk_weight + D, w.key_norm_weight, static_cast<size_t>(D) * 2, hipMemcpyDeviceToDevice,
@@ -282,7 +303,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
           return set_error(TAAC_ERR_LAUNCH, "%s: copy of the query / key norm weights failed", name);
       }
       if ((rc = taac_norm_linear_qk_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, qkv, 3 * D, M, D,
-                                        heads, T, qk_norm ? qk_weight : nullptr, rope_cos_sin,
+                                        heads, T, weights_in_epilogue ? qk_weight : nullptr, rope_cos_sin,
                                         qk_norm ? qk_sumsq : nullptr, rows, n_rows, stream)) != TAAC_OK)
         return rc;
       if (qk_norm) {
@@ -306,8 +327,8 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
           TAAC_OK)
         return rc;
     }
-    if ((rc = taac_flash_attn_scaled_fwd(qkv, qkv + D, qkv + 2 * D, key_lengths, q_scale, k_scale, h, B, heads, T, T,
-                                         dh, qkv_strides, qkv_strides, qkv_strides, o_strides, 0, rows ? 2 : 1,
+    if ((rc = taac_flash_attn_scaled_fwd(qkv, qkv + D, qkv + 2 * D, key_lengths, q_scale, k_scale, q_col_scale, h, B,
+                                         heads, T, T, dh, qkv_strides, qkv_strides, qkv_strides, o_strides, 0, rows ? 2 : 1,
                                          TAAC_BF16, stream)) != TAAC_OK)
       return rc;
     if (fused) {

@@ -600,9 +600,9 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 //   and the "memory" clobbers of the hand-written statements keep loads and stores on their side of them.
 // LDS: [3 weight buffers of 2*KS fragments][8 epilogue tiles][bias (N) | norm weight (D)]
 // ------------------------------------------------------------------------------------------------------------------
-template <int D, int TT, bool RES, bool QK>
+template <int D, int TT, bool RES, int QK>
 __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParams p) {
-  static_assert(!(QK && RES), "the query / key epilogue has no residual");
+  static_assert(!(QK != 0 && RES), "the query / key epilogue has no residual");
   constexpr int NWAVES = 8;
   constexpr int kTokPerWg = NWAVES * 32 * TT;  // TT token tiles of 32 per wavefront
   constexpr int KS = D / 16;
@@ -691,7 +691,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     for (int t = 0; t < TT; ++t)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(xf[t][ks]));
-    if (QK) {  // lane <-> token `lane` of the wavefront's 32 * TT tokens
+    if (QK != 0) {  // lane <-> token `lane` of the wavefront's 32 * TT tokens
       const int64_t r = token_row(p, count, tok_base + (lane < 32 * TT ? lane : 0));
       rowinfo[lane] = make_int2(static_cast<int>(r), static_cast<int>(r % p.tokens_per_sample));
     }
@@ -700,7 +700,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
   bf16x8 res_cur[NST], res_next[NST];
   int32_t prow[NST], prow_next[NST];  // rows of the current tile / of the tile the next step belongs to
   int64_t tok_wave = tokens_of_tile(tile_of(0));
-  if constexpr (!QK) rows_of_tile(tok_wave, prow);
+  if constexpr (QK == 0) rows_of_tile(tok_wave, prow);
   stage(chunk_of(0), 0);
   if (total > 1) stage(chunk_of(1), 1);
   if (RES) request_residual(prow, chunk_of(0), res_cur);
@@ -724,7 +724,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
       if (RES) {
 #pragma unroll
         for (int i = 0; i < NST; ++i) prow[i] = prow_next[i];
-      } else if constexpr (!QK) {
+      } else if constexpr (QK == 0) {
         rows_of_tile(tok_wave, prow);
       }
     }
@@ -789,66 +789,75 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
 
     // ---- epilogue of this chunk: bias, rounding, transpose through LDS, residual, 4 stores ---------------------------
     bf16x4 bv[8];
-    read_chunk_bias(bias_lds + chunk * kNC, hh, bv);
-    if constexpr (QK) {
+    if constexpr (QK == 0) read_chunk_bias(bias_lds + chunk * kNC, hh, bv);
+    if constexpr (QK != 0) {
       // Query and key chunks: the sum of squares of the rounded projection goes to qk_sumsq (one value per token and
-      // chunk; the statistic of the norm over the model width is their sum), the features are multiplied by the norm
-      // weight and rotated. The per-token factor rsqrt(mean + eps) commutes with both and is applied by the attention
-      // kernel. Value chunks are stored as they are.
+      // chunk; the statistic of the norm over the model width is their sum). QK == 2 also multiplies the features by
+      // the norm weight and rotates them. The per-token factor rsqrt(mean + eps) commutes with both and is applied by
+      // the attention kernel. Value chunks are stored as they are.
+      constexpr bool XF = QK == 2;
       const bool qk_chunk = chunk < p.qk_chunks;  // wavefront-uniform
       const int col8 = chunk * kNC + (lane % 8) * 8;
+      const bool rotate = XF && qk_chunk && p.cos_sin != nullptr;
+      const bool transform = XF && qk_chunk;
       bf16x8 wn;
+      if (XF) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) wn[e] = static_cast<bf16_t>(1.0f);
-      if (qk_chunk && p.qk_w != nullptr) wn = *reinterpret_cast<const bf16x8*>(p.qk_w + col8);
-      const bool rotate = qk_chunk && p.cos_sin != nullptr;
+        for (int e = 0; e < 8; ++e) wn[e] = static_cast<bf16_t>(1.0f);
+        if (qk_chunk && p.qk_w != nullptr) wn = *reinterpret_cast<const bf16x8*>(p.qk_w + col8);
+      }
       const int d0 = rotate ? col8 % p.head_dim : 0;
 #pragma unroll
       for (int t = 0; t < TT; ++t) {
-        if (qk_chunk) {
+        read_chunk_bias(bias_lds + chunk * kNC, hh, bv);  // per tile: not held while the pieces are processed
+        if (qk_chunk && p.qk_sumsq != nullptr) {
           float ss = tile_to_lds_sumsq(tile_lds, acc0[t], acc1[t], bv, l32, hh);
           ss = half_wave_pair_sum(ss);
           const int row = rowinfo[t * 32 + l32].x;
-          if (hh == 0 && p.qk_sumsq != nullptr) p.qk_sumsq[static_cast<int64_t>(chunk) * p.M + row] = ss;
+          if (hh == 0) p.qk_sumsq[static_cast<int64_t>(chunk) * p.M + row] = ss;
         } else {
           tile_to_lds(tile_lds, acc0[t], acc1[t], bv, l32, hh);
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        int2 info[4];
-        bf16x8 cs[4];
+        // two pieces at a time: rows (and table pieces) first, then the arithmetic and the stores
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          info[i] = rowinfo[t * 32 + i * 8 + lane / 8];
-          if (rotate)
-            cs[i] = *reinterpret_cast<const bf16x8*>(p.cos_sin + static_cast<int64_t>(info[i].y) * p.head_dim + d0);
-        }
+        for (int i2 = 0; i2 < 4; i2 += 2) {
+          int2 info[2];
+          bf16x8 cs[2];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int row = i * 8 + lane / 8;
-          bf16x8 v = *reinterpret_cast<const bf16x8*>(tile_lds + row * kStageRow + (lane % 8) * 16);
-          if (qk_chunk) {
-            float f[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) f[e] = static_cast<float>(v[e]) * static_cast<float>(wn[e]);
-            if (rotate) {
-#pragma unroll
-              for (int e = 0; e < 8; e += 2) {
-                const float even = f[e], odd = f[e + 1];
-                const float cv = static_cast<float>(cs[i][e]), sv = static_cast<float>(cs[i][e + 1]);
-                f[e] = even * cv - odd * sv;
-                f[e + 1] = even * sv + odd * cv;
-              }
-            }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = static_cast<bf16_t>(f[e]);
+          for (int j = 0; j < 2; ++j) {
+            info[j] = rowinfo[t * 32 + (i2 + j) * 8 + lane / 8];
+            if (XF && rotate)
+              cs[j] = *reinterpret_cast<const bf16x8*>(p.cos_sin + static_cast<int64_t>(info[j].y) * p.head_dim + d0);
           }
-          *reinterpret_cast<bf16x8*>(p.out + static_cast<int64_t>(info[i].x) * p.ldo + col8) = v;
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const int row = (i2 + j) * 8 + lane / 8;
+            bf16x8 v = *reinterpret_cast<const bf16x8*>(tile_lds + row * kStageRow + (lane % 8) * 16);
+            if (XF && transform) {
+              float f[8];
+#pragma unroll
+              for (int e = 0; e < 8; ++e) f[e] = static_cast<float>(v[e]) * static_cast<float>(wn[e]);
+              if (rotate) {
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                  const float even = f[e], odd = f[e + 1];
+                  const float cv = static_cast<float>(cs[j][e]), sv = static_cast<float>(cs[j][e + 1]);
+                  f[e] = even * cv - odd * sv;
+                  f[e + 1] = even * sv + odd * cv;
+                }
+              }
+#pragma unroll
+              for (int e = 0; e < 8; ++e) v[e] = static_cast<bf16_t>(f[e]);
+            }
+            *reinterpret_cast<bf16x8*>(p.out + static_cast<int64_t>(info[j].x) * p.ldo + col8) = v;
+          }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       }
     }
 #pragma unroll
-    for (int t = 0; t < (QK ? 0 : TT); ++t) {
+    for (int t = 0; t < (QK != 0 ? 0 : TT); ++t) {
       tile_to_lds(tile_lds, acc0[t], acc1[t], bv, l32, hh);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
@@ -868,7 +877,11 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     // ---- close the step ------------------------------------------------------------------------------------------------
     if (has_next) {
       if (stage_ahead) {
-        vm_wait<FPW + NST>();
+        // The transfer that must have landed (step s + 1) was issued one step ago: behind it are the NST stores of step
+        // s - 1, the FPW transfers of step s + 2 and the NST stores of this step, whatever else was issued. The query /
+        // key epilogue issues more (statistic stores, table loads), so it uses the full count; the plain epilogue keeps
+        // the tighter one (it makes no difference there).
+        vm_wait<QK != 0 ? FPW + 2 * NST : FPW + NST>();
       } else {
         vm_wait<NST>();
       }
@@ -1134,14 +1147,17 @@ int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void*
     hipLaunchKernelGGL((norm_linear_kernel<KK, TT, RR, QQ>), dim3(grid), dim3(8 * kWave), lds_bytes, s, p);       \
     return check_launch(name);                                                                                    \
   } while (0)
+  const bool qk_transform = qk.enabled && (qk.qk_weight != nullptr || qk.cos_sin != nullptr);
   if (K == 256) {
-    if (qk.enabled) TAAC_LIN_LAUNCH(256, 2, false, true);
-    if (residual) TAAC_LIN_LAUNCH(256, 1, true, false);
-    TAAC_LIN_LAUNCH(256, 2, false, false);
+    if (qk_transform) TAAC_LIN_LAUNCH(256, 2, false, 2);
+    if (qk.enabled) TAAC_LIN_LAUNCH(256, 2, false, 1);
+    if (residual) TAAC_LIN_LAUNCH(256, 1, true, 0);
+    TAAC_LIN_LAUNCH(256, 2, false, 0);
   }
-  if (qk.enabled) TAAC_LIN_LAUNCH(128, 2, false, true);
-  if (residual) TAAC_LIN_LAUNCH(128, 1, true, false);
-  TAAC_LIN_LAUNCH(128, 2, false, false);
+  if (qk_transform) TAAC_LIN_LAUNCH(128, 2, false, 2);
+  if (qk.enabled) TAAC_LIN_LAUNCH(128, 2, false, 1);
+  if (residual) TAAC_LIN_LAUNCH(128, 1, true, 0);
+  TAAC_LIN_LAUNCH(128, 2, false, 0);
 #undef TAAC_LIN_LAUNCH
 }
 

@@ -88,11 +88,12 @@ class UnifiedSelfAttention(nn.Module):
         query_weight = None if self.query_norm is None else _bf16(self.query_norm.weight)
         key_weight = None if self.key_norm is None else _bf16(self.key_norm.weight)
         qk_eps = 1e-6 if self.query_norm is None else self.query_norm.eps
-        q_row_scale = k_row_scale = None
+        q_row_scale = k_row_scale = q_col_scale = None
         if prepare and x.ndim == 3 and x.shape[-1] in (128, 256):
-            # weight, rotation and the norm statistic come out of the projection's epilogue; the per-token factor of
-            # the norm is applied inside the attention kernel: no pass over q and k at all
-            qkv, q_row_scale, k_row_scale = qkv_projection(
+            # the norm statistic (and, with a rotation, weight and rotation) come out of the projection's epilogue; the
+            # per-token factor of the norm and the weights of the unrotated case are applied inside the attention
+            # kernel: no pass over q and k at all
+            qkv, q_row_scale, k_row_scale, q_col_scale = qkv_projection(
                 x, _bf16(self.qkv.weight), _bf16(self.qkv.bias), num_heads=self.num_heads, query_weight=query_weight,
                 key_weight=key_weight, qk_eps=qk_eps, rope_base=self.rope_base,
             )
@@ -114,6 +115,7 @@ class UnifiedSelfAttention(nn.Module):
             zero_padded_queries=zero_padded_queries,
             q_row_scale=q_row_scale,
             k_row_scale=k_row_scale,
+            q_col_scale=q_col_scale,
         )
         out = _dense(self.out, attended, residual=_bf16(residual))
         return out if out.dtype == output_dtype else out.to(output_dtype)

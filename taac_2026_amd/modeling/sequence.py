@@ -82,9 +82,11 @@ def scaled_dot_product_attention(
     zero_padded_queries: bool = False,
     q_row_scale: torch.Tensor | None = None,
     k_row_scale: torch.Tensor | None = None,
+    q_col_scale: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """Multi-head attention over (B, T, D) projections; returns (B, Tq, D). ``q_row_scale`` / ``k_row_scale``: optional
-    float32 (B, T) factors of the query / key rows applied inside the kernel."""
+    """Multi-head attention over (B, T, D) projections; returns (B, Tq, D). ``q_row_scale`` / ``k_row_scale``
+    (float32 (B, T)) and ``q_col_scale`` (float32 (D,)): optional factors of the query / key rows and of the query
+    features applied inside the kernel."""
     batch, query_len, d_model = q.shape
     head_dim = d_model // num_heads
     q4 = q.view(batch, query_len, num_heads, head_dim).transpose(1, 2)
@@ -107,6 +109,7 @@ def scaled_dot_product_attention(
         zero_padded_queries=zero_padded_queries,
         q_row_scale=q_row_scale,
         k_row_scale=k_row_scale,
+        q_col_scale=q_col_scale,
     )
     return output.transpose(1, 2).contiguous().view(batch, query_len, d_model)
 

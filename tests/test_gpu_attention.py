@@ -185,3 +185,18 @@ def test_row_factors_of_queries_and_keys(device, dim, tokens, causal):
     torch.testing.assert_close(only_k.float(), expected_k.float(), **BF16_TOL)
     with pytest.raises(ValueError, match="q_row_scale"):
         hip_flash_attention_kernel(*args, q_row_scale=sq[:, :-1].contiguous().to(device))
+    # one factor per query feature (the product of a query and a key norm weight)
+    col = 0.5 + torch.rand(heads * dim, generator=g)
+    expected_c = oracle.attention(q.float() * col.view(1, heads, 1, dim) * sq[:, None, :, None], k, v, lengths,
+                                  is_causal=causal, zero_padded_queries=True)
+    with torch.no_grad():
+        with_col = hip_flash_attention_kernel(*args, is_causal=causal, zero_padded_queries=True,
+                                              q_row_scale=sq.to(device), q_col_scale=col.to(device)).cpu()
+        only_col = hip_flash_attention_kernel(*args, is_causal=causal, zero_padded_queries=True,
+                                              q_col_scale=col.to(device)).cpu()
+    torch.testing.assert_close(with_col.float(), expected_c.float(), **BF16_TOL)
+    expected_oc = oracle.attention(q.float() * col.view(1, heads, 1, dim), k, v, lengths, is_causal=causal,
+                                   zero_padded_queries=True)
+    torch.testing.assert_close(only_col.float(), expected_oc.float(), **BF16_TOL)
+    with pytest.raises(ValueError, match="q_col_scale"):
+        hip_flash_attention_kernel(*args, q_col_scale=col[:-1].contiguous().to(device))

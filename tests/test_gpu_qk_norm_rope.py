@@ -178,9 +178,10 @@ def test_qkv_projection_prepares_queries_and_keys_in_its_epilogue(device, monkey
     q, k, v = projection.chunk(3, dim=-1)
     expected_q, expected_k = oracle.qk_norm_rope(q, k, *weights, num_heads=heads, eps=1e-6, rope_base=base, fp32=True)
     with torch.no_grad():
-        qkv, sq, sk = qkv_projection(x.to(device), w.to(device), b.to(device), num_heads=heads, norm_weight=nw.to(device),
-                                     query_weight=None if weights[0] is None else wq.to(device),
-                                     key_weight=None if weights[1] is None else wk.to(device), rope_base=base)
+        qkv, sq, sk, col = qkv_projection(x.to(device), w.to(device), b.to(device), num_heads=heads,
+                                          norm_weight=nw.to(device),
+                                          query_weight=None if weights[0] is None else wq.to(device),
+                                          key_weight=None if weights[1] is None else wk.to(device), rope_base=base)
     got_q, got_k, got_v = qkv.cpu().chunk(3, dim=-1)
     torch.testing.assert_close(got_v.float(), v.float(), rtol=2e-2, atol=2e-2)
     if "norm" in mode:
@@ -191,8 +192,18 @@ def test_qkv_projection_prepares_queries_and_keys_in_its_epilogue(device, monkey
         torch.testing.assert_close(sk.cpu(), rstd(k), rtol=5e-3, atol=0)
         got_q = got_q.float() * sq.cpu()[..., None]
         got_k = got_k.float() * sk.cpu()[..., None]
+        if base is None:
+            # without a rotation the columns are the plain projection and both weights ride on the query as their
+            # product: q * (wq * wk) and k give the same scores as (q * wq) and (k * wk)
+            torch.testing.assert_close(col.cpu(), wq.float() * wk.float(), rtol=0, atol=0)
+            torch.testing.assert_close(qkv.cpu()[..., :2 * d_model].float(), projection[..., :2 * d_model].float(),
+                                       rtol=2e-2, atol=2e-2)
+            got_q = got_q * col.cpu() / wk.float()
+            got_k = got_k * wk.float()
+        else:
+            assert col is None
     else:
-        assert sq is None and sk is None
+        assert sq is None and sk is None and col is None
     torch.testing.assert_close(got_q.float(), expected_q.float(), rtol=2e-2, atol=2e-2)
     torch.testing.assert_close(got_k.float(), expected_k.float(), rtol=2e-2, atol=2e-2)
 
@@ -208,10 +219,10 @@ def test_qkv_projection_skips_padded_rows(device):
     lengths = torch.tensor([70, 3, 0, 41], dtype=torch.int32)
     valid = torch.arange(tokens)[None, :] < lengths[:, None]
     with torch.no_grad():
-        full, fq, fk = qkv_projection(x.to(device), w.to(device), None, num_heads=heads, query_weight=wq.to(device),
+        full, fq, fk, _ = qkv_projection(x.to(device), w.to(device), None, num_heads=heads, query_weight=wq.to(device),
                                       key_weight=wq.to(device), rope_base=500.0)
         xn = torch.where(valid[..., None], x, torch.full_like(x, float("nan"))).to(device)
-        got, sq, sk = qkv_projection(xn, w.to(device), None, num_heads=heads, query_weight=wq.to(device),
+        got, sq, sk, _ = qkv_projection(xn, w.to(device), None, num_heads=heads, query_weight=wq.to(device),
                                      key_weight=wq.to(device), rope_base=500.0,
                                      token_rows=valid_rows(lengths.to(device), tokens))
     mask = valid.to(device)
