@@ -109,6 +109,38 @@ int taac_flash_attn_scaled_fwd(const void* q, const void* k, const void* v, cons
                                int is_causal, int zero_padded_queries, int dtype, void* stream);
 
 /*
+ * Attention under a structured mask: key j is visible to query i of sample b iff
+ *   structural[i, j] AND key_valid[b, j]      (AND j < key_lengths[b] when key_lengths is given),
+ * with structural shared by the batch and the heads. That is the form of the reference's model-level masks:
+ * TokenFormer's per-layer full / sliding-window mask with always-visible separator keys and an all-seeing target query
+ * (_bfts_attention_mask, experiments/tokenformer/model.py:474-503) and Symbiosis' role-metadata mask
+ * (MetadataAttentionMask.forward, experiments/symbiosis/attention.py:21-60), both ANDed with the key padding; the
+ * reference's accelerated attention path rejects them (flash_attention.py:183-209) and falls back to torch SDPA.
+ * struct_bits: uint32 [Tq, ceil(Tk / 32)], bit j % 32 of word j / 32 of row i = structural[i, j], bits beyond Tk zero
+ * (taac_mask_pack_bits); block_any: uint8 [ceil(Tq / 128), ceil(Tk / 64)] from taac_mask_block_any: 64-key chunks that
+ * no query of a 128-row block can see are neither loaded nor computed, 32-key tiles that no query of a wavefront sees
+ * are skipped, fully visible tiles skip the bit tests. valid_bits: uint32 [B, ceil(Tk / 32)] or NULL (all valid).
+ * self_bits: uint32 [B, ceil(Tq / 32)] or NULL; a flagged query row returns its own value row (the reference's
+ * fallback for padded queries, which attend to themselves only; requires Tq == Tk). Rows with no visible key give
+ * zeros. The row / feature factors are those of taac_flash_attn_scaled_fwd (NULL: none). Everything else as
+ * taac_flash_attn_fwd; no is_causal (put the triangle into structural).
+ */
+int taac_flash_attn_masked_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
+                               const uint32_t* struct_bits, const uint8_t* block_any, const uint32_t* valid_bits,
+                               const uint32_t* self_bits, const float* q_row_scale, const float* k_row_scale,
+                               const float* q_col_scale, void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk,
+                               int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
+                               const int64_t v_strides[4], const int64_t o_strides[4], int zero_padded_queries,
+                               int dtype, void* stream);
+
+/* Packs a row-major bool matrix (one byte per element, nonzero = true) [rows, cols] into bit rows
+ * [rows, ceil(cols / 32)]: the struct_bits / valid_bits / self_bits of taac_flash_attn_masked_fwd. */
+int taac_mask_pack_bits(const void* mask, int64_t rows, int32_t cols, uint32_t* bits, void* stream);
+
+/* block_any [ceil(Tq / 128), ceil(Tk / 64)] of struct_bits [Tq, ceil(Tk / 32)] for taac_flash_attn_masked_fwd. */
+int taac_mask_block_any(const uint32_t* struct_bits, int32_t Tq, int32_t Tk, uint8_t* block_any, void* stream);
+
+/*
  * Dense layer, bf16 storage / bf16 MFMA / fp32 accumulation: out = epilogue(a @ w^T + bias).
  * a: [M, K] with row stride lda (elements); w: [N, K] contiguous (torch nn.Linear layout, [out, in]);
  * bias: [N] bf16 or NULL; residual: [M, N_out] with row stride ldo or NULL; out: [M, N_out] with row stride ldo,

@@ -20,6 +20,11 @@ Puiching-Memory/TAAC_2026). How each function is pinned, independently of its ow
                       test_primitives.py:36-39, tests/contract/experiments/test_packages.py:597-617,
                       test_tilelang_ops.py:361-428), committed as tests/golden/mask_vectors.json.
   masked_mean         float64 brute force; all-padded rows give zeros (divisor clamp).
+  bfts_attention_mask / metadata_attention_mask
+                      the reference holds no known answer for them (its contract test checks the shape and that the
+                      readout rows see a key, tests/contract/experiments/test_packages.py:430-440); restated here as
+                      per-element rules, pinned by hand-derived small cases and invariants (every valid query sees
+                      itself, padded keys are never seen, target rows and separator columns are full, window counts).
   rotate_half_pairs / rope_tables / apply_rope / qk_norm_rope
                       the reference holds no numeric test for them; pinned by what a rotation fixes: multiplication of
                       even + i*odd by exp(i*angle) (numpy complex128), position 0 is the identity, pair norms are
@@ -179,6 +184,55 @@ def scaled_dot_product_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tens
     v4 = v.view(batch, v.shape[1], num_heads, head_dim).transpose(1, 2)
     out = attention(q4, k4, v4, key_lengths, zero_padded_queries=zero_padded_queries)
     return out.transpose(1, 2).contiguous().view(batch, query_len, d_model)
+
+
+# ---- model-level structured masks ------------------------------------------------------------------------------------
+
+
+def bfts_attention_mask(padding_mask: torch.Tensor, role_ids: torch.Tensor, layer_index: int, num_layers: int, *,
+                        seq_causal: bool, seq_keep_per_domain: int) -> torch.Tensor:
+    """``PCVRTokenFormer._bfts_attention_mask`` (experiments/tokenformer/model.py:474-503) restated element by element
+    (small inputs only): (B, 1, T, T) bool, True = attend. Roles: 3 = target, 4 = separator (model.py:32-37)."""
+    batch, tokens = padding_mask.shape
+    bottom = max(1, num_layers // 2)
+    window = None if layer_index < bottom else max(4, math.ceil(seq_keep_per_domain / (2 ** (layer_index - bottom))))
+    safe = safe_key_padding_mask(padding_mask)
+    mask = torch.zeros(batch, 1, tokens, tokens, dtype=torch.bool)
+    for b in range(batch):
+        for i in range(tokens):
+            if bool(padding_mask[b, i]):
+                mask[b, 0, i, i] = True  # a padded query attends to itself only
+                continue
+            for j in range(tokens):
+                if window is None:
+                    seen = j <= i if seq_causal else True
+                else:
+                    seen = 0 <= i - j <= window if seq_causal else abs(i - j) <= window
+                seen = seen or i == j or int(role_ids[i]) == 3 or int(role_ids[j]) == 4
+                mask[b, 0, i, j] = seen and not bool(safe[b, j])
+    return mask
+
+
+_METADATA_VISIBLE_KEY_ROLES = {
+    # query role -> key roles it may read (experiments/symbiosis/attention.py:29-58; roles: tokenization.py:22-30)
+    0: set(range(8)), 1: set(range(8)), 7: set(range(8)),
+    2: {0, 1, 2, 3, 4, 5, 7}, 3: {0, 1, 2, 3, 4, 5, 7}, 4: {0, 1, 2, 3, 4, 5, 7}, 5: {0, 1, 2, 3, 4, 5, 7},
+    6: {0, 1, 3, 6, 5, 7},
+}
+
+
+def metadata_attention_mask(padding_mask: torch.Tensor, role_ids: torch.Tensor, *, enabled: bool = True) -> torch.Tensor:
+    """``MetadataAttentionMask.forward`` (experiments/symbiosis/attention.py:22-60) restated element by element (small
+    inputs only): (B, 1, T, T) bool."""
+    batch, tokens = padding_mask.shape
+    safe = safe_key_padding_mask(padding_mask)
+    mask = torch.zeros(batch, 1, tokens, tokens, dtype=torch.bool)
+    for b in range(batch):
+        for i in range(tokens):
+            for j in range(tokens):
+                seen = True if not enabled else (i == j or int(role_ids[j]) in _METADATA_VISIBLE_KEY_ROLES[int(role_ids[i])])
+                mask[b, 0, i, j] = seen and not bool(safe[b, j])
+    return mask
 
 
 # ---- query / key normalisation and rotary embedding ------------------------------------------------------------------

@@ -75,6 +75,14 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         + [ctypes.POINTER(c_int64)] * 4
         + [c_int, c_int, c_int, c_void_p],
     ),
+    "taac_flash_attn_masked_fwd": (
+        c_int,
+        [c_void_p] * 12 + [c_int32, c_int32, c_int32, c_int32, c_int32]
+        + [ctypes.POINTER(c_int64)] * 4
+        + [c_int, c_int, c_void_p],
+    ),
+    "taac_mask_pack_bits": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p]),
+    "taac_mask_block_any": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
     "taac_linear_bf16": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_int, c_int,

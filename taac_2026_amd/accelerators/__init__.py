@@ -3,10 +3,13 @@
 
 from taac_2026_amd.accelerators.attention import (
     FlashAttentionMaskPlan,
+    StructuredAttentionMask,
     _plan_tilelang_flash_attention_mask,
+    build_structured_mask,
     flash_attention,
     hip_flash_attention_kernel,
     plan_flash_attention_mask,
+    plan_structured_attention_mask,
     qk_norm_rope,
     resolved_flash_attention_backend,
     rope_table,
@@ -39,8 +42,10 @@ from taac_2026_amd.accelerators.tensor_validation import (
 
 __all__ = [
     "FlashAttentionMaskPlan",
+    "StructuredAttentionMask",
     "_plan_tilelang_flash_attention_mask",
     "amax",
+    "build_structured_mask",
     "concrete_tensors",
     "flash_attention",
     "hip_flash_attention_kernel",
@@ -51,6 +56,7 @@ __all__ = [
     "linear_fp8",
     "norm_linear",
     "plan_flash_attention_mask",
+    "plan_structured_attention_mask",
     "qk_norm_rope",
     "qkv_projection",
     "quantize_fp8",

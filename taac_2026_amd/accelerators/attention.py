@@ -28,9 +28,109 @@ FLASH_ATTENTION_BACKENDS = ("hip", "torch", "tilelang")
 class FlashAttentionMaskPlan:
     """What the kernel needs to know about a mask (flash_attention.py:60-64)."""
 
-    key_lengths: torch.Tensor
+    key_lengths: torch.Tensor | None
     query_self_mask: torch.Tensor | None
     is_causal: bool
+
+
+@dataclass(frozen=True)
+class StructuredAttentionMask:
+    """Bit form of a mask ``visible[b, i, j] = structural[i, j] & key_valid[b, j]`` (shared by the heads), optionally with
+    query rows that attend to themselves only (``query_self``: their output is their value row). This is the shape of the
+    reference's model-level masks (experiments/tokenformer/model.py:474-503, experiments/symbiosis/attention.py:21-60).
+    Built by :func:`build_structured_mask`; ``dense()`` gives the (B, 1, Tq, Tk) bool mask the reference would pass."""
+
+    struct_bits: torch.Tensor          # int32 (Tq, ceil(Tk / 32))
+    block_any: torch.Tensor            # uint8 (ceil(Tq / 128), ceil(Tk / 64))
+    valid_bits: torch.Tensor | None    # int32 (B, ceil(Tk / 32))
+    self_bits: torch.Tensor | None     # int32 (B, ceil(Tq / 32))
+    structural: torch.Tensor           # bool (Tq, Tk)
+    key_valid: torch.Tensor | None     # bool (B, Tk)
+    query_self: torch.Tensor | None    # bool (B, Tq)
+
+    def dense(self) -> torch.Tensor:
+        query_len, kv_len = self.structural.shape
+        mask = self.structural[None]
+        if self.key_valid is not None:
+            mask = mask & self.key_valid[:, None, :]
+        if self.query_self is not None:
+            eye = torch.eye(query_len, kv_len, dtype=torch.bool, device=self.structural.device)
+            mask = torch.where(self.query_self[:, :, None], eye[None], mask)
+        return mask[:, None]
+
+
+def _pack_bits(mask: torch.Tensor) -> torch.Tensor:
+    rows, cols = mask.shape
+    bits = torch.empty(rows, (cols + 31) // 32, dtype=torch.int32, device=mask.device)
+    library = _native.load_library()
+    status = library.taac_mask_pack_bits(mask.data_ptr(), rows, cols, bits.data_ptr(), _native.current_stream(mask.device))
+    _native.check(status, "mask_pack_bits")
+    return bits
+
+
+def build_structured_mask(
+    structural: torch.Tensor, key_valid: torch.Tensor | None = None, query_self: torch.Tensor | None = None
+) -> StructuredAttentionMask:
+    """``structural`` (Tq, Tk) bool, True = attend; ``key_valid`` (B, Tk) bool or None; ``query_self`` (B, Tq) bool or
+    None (needs Tq == Tk). Everything stays on the device (no host synchronisation)."""
+    name = "hip build_structured_mask"
+    require_cuda_tensors(name, structural, key_valid, query_self)
+    for tensor, label in ((structural, "structural"), (key_valid, "key_valid"), (query_self, "query_self")):
+        if tensor is not None and (tensor.dtype is not torch.bool or tensor.ndim != 2):
+            raise ValueError(f"{name}: {label} must be a 2-D bool tensor")
+    query_len, kv_len = structural.shape
+    if key_valid is not None and key_valid.shape[1] != kv_len:
+        raise ValueError(f"{name}: key_valid must have shape (batch, kv_len)")
+    if query_self is not None and (query_len != kv_len or query_self.shape[1] != query_len):
+        raise ValueError(f"{name}: query_self must have shape (batch, query_len) and needs query_len == kv_len")
+    structural = structural.contiguous()
+    struct_bits = _pack_bits(structural)
+    block_any = torch.empty((query_len + 127) // 128, (kv_len + 63) // 64, dtype=torch.uint8, device=structural.device)
+    library = _native.load_library()
+    status = library.taac_mask_block_any(struct_bits.data_ptr(), query_len, kv_len, block_any.data_ptr(),
+                                         _native.current_stream(structural.device))
+    _native.check(status, "mask_block_any")
+    key_valid = None if key_valid is None else key_valid.contiguous()
+    query_self = None if query_self is None else query_self.contiguous()
+    return StructuredAttentionMask(
+        struct_bits, block_any, None if key_valid is None else _pack_bits(key_valid),
+        None if query_self is None else _pack_bits(query_self), structural, key_valid, query_self,
+    )
+
+
+def plan_structured_attention_mask(q: torch.Tensor, k: torch.Tensor, attn_mask: torch.Tensor) -> StructuredAttentionMask:
+    """Factor a (B, H | 1, Tq, Tk) bool mask into ``structural[i, j] & key_valid[b, j]`` with optional self-only query
+    rows, verifying the factorisation exactly; ``RuntimeError`` when the mask has no such form. This reads the full mask
+    several times and synchronises with the host (as the reference's planner does, flash_attention.py:149-198): callers
+    that know the factors pass ``structured_mask=build_structured_mask(...)`` instead."""
+    batch, heads, query_len, kv_len = q.shape[0], q.shape[1], q.shape[2], k.shape[2]
+    if attn_mask.dtype is not torch.bool:
+        raise RuntimeError("hip flash_attention only supports structured bool attention masks")
+    if attn_mask.ndim != 4 or attn_mask.shape[0] != batch or attn_mask.shape[1] not in (1, heads) or \
+            attn_mask.shape[2:] != (query_len, kv_len):
+        raise RuntimeError("hip flash_attention only supports 4D bool masks matching (batch, heads, query_len, kv_len)")
+    if attn_mask.shape[1] != 1 and not torch.equal(attn_mask, attn_mask[:, :1].expand_as(attn_mask)):
+        raise RuntimeError("hip flash_attention requires the bool attention mask to be shared across heads")
+    mask = attn_mask[:, 0]
+    query_self = None
+    live = mask
+    if query_len == kv_len:
+        eye = torch.eye(query_len, dtype=torch.bool, device=mask.device)
+        query_self = (mask == eye[None]).all(dim=-1)
+        live = mask & ~query_self[:, :, None]
+    key_valid = live.any(dim=1)
+    structural = live.any(dim=0)
+    expected = structural[None] & key_valid[:, None, :]
+    if query_self is not None:
+        expected = torch.where(query_self[:, :, None], eye[None], expected)
+    if not torch.equal(expected, mask):
+        raise RuntimeError(
+            "hip flash_attention only supports bool masks of the form structural[query, key] & key_valid[batch, key] "
+            "(shared by the heads), optionally with padded query rows that attend to themselves only"
+        )
+    if query_self is not None and not bool(query_self.any()):
+        query_self = None
+    return build_structured_mask(structural, key_valid, query_self)
 
 
 def _normalize_flash_attention_inputs(
@@ -190,6 +290,7 @@ def hip_flash_attention_kernel(
     q_row_scale: torch.Tensor | None = None,
     k_row_scale: torch.Tensor | None = None,
     q_col_scale: torch.Tensor | None = None,
+    structured_mask: StructuredAttentionMask | None = None,
 ) -> torch.Tensor:
     """``(q, k, v: (B, H, T, d) bf16/fp16, key_lengths: int32[B]) -> (B, H, Tq, d)``.
 
@@ -198,7 +299,8 @@ def hip_flash_attention_kernel(
     q's memory layout, so (B, T, H, d)-strided views stay copy-free in both directions. ``q_row_scale`` (B, Tq) /
     ``k_row_scale`` (B, Tk): optional positive fp32 factors of the query / key rows, shared by the heads (a
     normalisation statistic applied inside the kernel instead of in a pass of its own); ``q_col_scale`` (H * d,):
-    optional fp32 factors of the query features (the product of a query and a key norm weight).
+    optional fp32 factors of the query features (the product of a query and a key norm weight). ``structured_mask``:
+    a :class:`StructuredAttentionMask` (excludes ``is_causal``; combines with ``key_lengths``).
     """
     library = _native.load_library()
     require_cuda_tensors("hip flash_attention", q, k, v, key_lengths)
@@ -224,6 +326,25 @@ def hip_flash_attention_kernel(
         require_cuda_tensors("hip flash_attention", q_col_scale)
         if q_col_scale.dtype != torch.float32 or q_col_scale.numel() != heads * head_dim or not q_col_scale.is_contiguous():
             raise ValueError("flash_attention q_col_scale must be a contiguous float32 tensor of heads * head_dim values")
+    if structured_mask is not None:
+        if is_causal:
+            raise ValueError("flash_attention: a structured mask carries its own causal triangle (is_causal must be False)")
+        sm = structured_mask
+        if sm.structural.shape != (query_len, k.shape[2]) or (sm.key_valid is not None and sm.key_valid.shape[0] != batch) \
+                or (sm.query_self is not None and sm.query_self.shape[0] != batch):
+            raise ValueError("flash_attention: the structured mask does not match (batch, query_len, kv_len)")
+        require_cuda_tensors("hip flash_attention", sm.struct_bits)
+        status = library.taac_flash_attn_masked_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), sm.struct_bits.data_ptr(),
+            sm.block_any.data_ptr(), _native.ptr(sm.valid_bits), _native.ptr(sm.self_bits), _native.ptr(q_row_scale),
+            _native.ptr(k_row_scale), _native.ptr(q_col_scale), out.data_ptr(),
+            batch, heads, query_len, k.shape[2], head_dim,
+            _native.Int64x4(*q.stride()), _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()),
+            _native.Int64x4(*out.stride()), int(zero_padded_queries), _native.dtype_code(q.dtype),
+            _native.current_stream(q.device),
+        )
+        _native.check(status, "flash_attention")
+        return out
     status = library.taac_flash_attn_scaled_fwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), _native.ptr(q_row_scale),
         _native.ptr(k_row_scale), _native.ptr(q_col_scale), out.data_ptr(),
@@ -256,6 +377,7 @@ def flash_attention(
     q_row_scale: torch.Tensor | None = None,
     k_row_scale: torch.Tensor | None = None,
     q_col_scale: torch.Tensor | None = None,
+    structured_mask: StructuredAttentionMask | None = None,
 ) -> torch.Tensor:
     """``softmax(q k^T / sqrt(d) + mask) v`` for (B, H, T, d) tensors.
 
@@ -266,25 +388,37 @@ def flash_attention(
     With ``zero_padded_queries`` the query rows at or beyond ``key_lengths[b]`` are returned as zeros; otherwise they
     attend to the valid keys like every other row (the behaviour of the reference's torch and TileLang paths).
     ``q_row_scale`` / ``k_row_scale`` / ``q_col_scale``: optional float32 factors of the query / key rows and of the
-    query features, see :func:`hip_flash_attention_kernel`.
+    query features, see :func:`hip_flash_attention_kernel`. ``structured_mask``: a :class:`StructuredAttentionMask`
+    instead of ``attn_mask``; an ``attn_mask`` that is neither a key-prefix nor a causal-valid mask is factored into one
+    by :func:`plan_structured_attention_mask` (the reference's accelerated path rejects such masks).
     """
     del block_m, block_n, num_stages, threads
     q, k, v = _normalize_flash_attention_inputs(q, k, v)
     _resolve_flash_attention_backend(q, backend, dropout_p=dropout_p, training=training)
     require_inference("hip flash_attention", q, k, v)
+    if structured_mask is not None and attn_mask is not None:
+        raise ValueError("flash_attention takes either attn_mask or structured_mask, not both")
     if key_lengths is not None:
         if attn_mask is not None:
             raise ValueError("flash_attention takes either attn_mask or key_lengths, not both")
         plan = FlashAttentionMaskPlan(key_lengths, None, is_causal)
+    elif structured_mask is not None:
+        plan = FlashAttentionMaskPlan(None, None, is_causal)
     else:
-        plan = plan_flash_attention_mask(q, k, attn_mask, is_causal=is_causal)
+        try:
+            plan = plan_flash_attention_mask(q, k, attn_mask, is_causal=is_causal)
+        except RuntimeError:
+            if attn_mask is None or attn_mask.dtype is not torch.bool or attn_mask.ndim != 4 or is_causal:
+                raise
+            structured_mask = plan_structured_attention_mask(q, k, attn_mask)
+            plan = FlashAttentionMaskPlan(None, None, False)
     output_dtype = v.dtype
     if q.dtype == torch.float32:
         q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
-    lengths = plan.key_lengths if (attn_mask is not None or key_lengths is not None) else None
+    lengths = plan.key_lengths if (plan.key_lengths is not None and (attn_mask is not None or key_lengths is not None)) else None
     output = hip_flash_attention_kernel(
         q, k, v, lengths, is_causal=plan.is_causal, zero_padded_queries=zero_padded_queries,
-        q_row_scale=q_row_scale, k_row_scale=k_row_scale, q_col_scale=q_col_scale,
+        q_row_scale=q_row_scale, k_row_scale=k_row_scale, q_col_scale=q_col_scale, structured_mask=structured_mask,
     )
     output = _apply_query_self_mask_fallback(output, v, plan.query_self_mask)
     return output if output.dtype == output_dtype else output.to(output_dtype)
@@ -398,10 +532,13 @@ def qk_norm_rope(
 __all__ = [
     "FLASH_ATTENTION_BACKENDS",
     "FlashAttentionMaskPlan",
+    "StructuredAttentionMask",
     "_plan_tilelang_flash_attention_mask",
+    "build_structured_mask",
     "flash_attention",
     "hip_flash_attention_kernel",
     "plan_flash_attention_mask",
+    "plan_structured_attention_mask",
     "qk_norm_rope",
     "resolved_flash_attention_backend",
     "rope_table",

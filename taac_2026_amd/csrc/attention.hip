@@ -40,6 +40,13 @@ struct AttnParams {
   const float* q_row_scale;  // [B, Tq] / [B, Tk] factors of the query / key rows (shared by the heads), or null
   const float* k_row_scale;
   const float* q_col_scale;  // [H, d] factors of the query features, or null
+  // Structured mask: key j is visible to query i of sample b iff bit j of struct_bits[i] and of valid_bits[b] is set.
+  const uint32_t* struct_bits;  // [Tq][wpr] words, bit j % 32 of word j / 32; null: no structured mask
+  const uint32_t* valid_bits;   // [B][wpr] or null (every key valid)
+  const uint32_t* self_bits;    // [B][ceil(Tq / 32)] or null: flagged query rows return their own value row
+  const uint8_t* block_any;     // [nqc][nkc]: some query of the 128-row block sees some key of the 64-key chunk
+  int32_t wpr;                  // words per row of struct_bits / valid_bits = ceil(Tk / 32)
+  int32_t nkc;                  // key chunks = ceil(Tk / 64)
   int32_t B, H, Tq, Tk, d;
   int64_t qs[4], ks[4], vs[4], os[4];
   float scale_log2;  // log2(e) / sqrt(d)
@@ -85,8 +92,9 @@ __device__ __forceinline__ uint32_t pack2(T lo, T hi) {
 // hh = (k / 4) % 2 the keys {hh*4 .. hh*4+3} and {8 + hh*4 .. 8 + hh*4+3}; they become 8 consecutive elements.
 __device__ __forceinline__ int vt_pos16(int k) { return ((k >> 2) & 1) * 8 + (k >> 3) * 4 + (k & 3); }
 
-template <typename T, int DP, bool CAUSAL, bool SCALED>
+template <typename T, int DP, bool CAUSAL, bool SCALED, bool MASKED>
 __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnParams p) {
+  static_assert(!(MASKED && CAUSAL), "a structured mask carries its own causal triangle");
   typedef typename Vec8<T>::type vec_t;
   typedef typename Vec8<T>::half_type vec4_t;
   constexpr int KSTEPS = DP / 16;  // MFMA k-steps of the score product
@@ -188,7 +196,21 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   vec_t kreg[KLD], vreg[VLD][2];
   float kfac[SCALED ? KLD : 1];
   const bool scale_keys = SCALED && p.k_row_scale != nullptr;
+  // MASKED: the two 32-key words of the lane's query for the chunk being fetched / being consumed.
+  uint32_t mw_next[2] = {0u, 0u}, mw[2] = {0u, 0u};
   auto fetch = [&](int kc0) {
+    if (MASKED) {
+      const int w0 = kc0 / 32;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        uint32_t bits = 0u;
+        if (qi < p.Tq && w0 + kt < p.wpr) {
+          bits = p.struct_bits[static_cast<int64_t>(qi) * p.wpr + w0 + kt];
+          if (p.valid_bits != nullptr) bits &= p.valid_bits[static_cast<int64_t>(b) * p.wpr + w0 + kt];
+        }
+        mw_next[kt] = bits;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < KLD; ++i) {
       const int idx = tid + i * kThreads;
@@ -213,7 +235,7 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 #pragma unroll
     for (int i = 0; i < KLD; ++i) {
       const int idx = tid + i * kThreads;
-      if (SCALED) {
+      if (SCALED && scale_keys) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) kreg[i][e] = static_cast<T>(static_cast<float>(kreg[i][e]) * kfac[SCALED ? i : 0]);
       }
@@ -233,19 +255,37 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
     }
   };
 
-  if (kv_end > 0) fetch(0);
-  for (int kc0 = 0; kc0 < kv_end; kc0 += kKC) {
-    if (kc0 > 0) __syncthreads();  // every wavefront is done reading the previous chunk
+  // Chunks are walked in order; with a structured mask the chunks in which no query of this workgroup's block sees
+  // any key (block_any, shared by the batch) are skipped altogether: not staged, not synchronised on.
+  auto next_chunk = [&](int kc) -> int {
+    if (MASKED) {
+      while (kc * kKC < kv_end && p.block_any[qc * p.nkc + kc] == 0) ++kc;
+    }
+    return kc * kKC < kv_end ? kc : -1;
+  };
+  int kc = next_chunk(0);
+  if (kc >= 0) fetch(kc * kKC);
+  bool first_chunk = true;
+  while (kc >= 0) {
+    const int kc0 = kc * kKC;
+    if (!first_chunk) __syncthreads();  // every wavefront is done reading the previous chunk
+    first_chunk = false;
     commit();
+    if (MASKED) {
+      mw[0] = mw_next[0];
+      mw[1] = mw_next[1];
+    }
     __syncthreads();
-    if (kc0 + kKC < kv_end) fetch(kc0 + kKC);
+    kc = next_chunk(kc + 1);
+    if (kc >= 0) fetch(kc * kKC);
 
     // One softmax update per chunk: both 32-key tiles when the second one has a visible key for this wavefront
-    // (NT = 2), the first tile alone otherwise (NT = 1). Per update: scores S^T (NT tiles of 32 keys x 32 queries),
+    // (NT = 2), one tile alone otherwise (NT = 1, tile T0). Per update: scores S^T (NT tiles of 32 keys x 32 queries),
     // running max / sum of one query per lane pair, P rounded to the storage type, one rescale of O^T, O^T += V^T P^T.
     if (kc0 >= wave_kv_end) continue;  // wavefront-uniform: nothing visible in this chunk (padding / causal bound)
-    auto update = [&](auto nt_tag) {
+    auto update = [&](auto nt_tag, auto t0_tag) {
       constexpr int NT = decltype(nt_tag)::value;
+      constexpr int T0 = decltype(t0_tag)::value;  // first 32-key tile of the chunk taken by this update
       f32x16 sacc[NT];
 #pragma unroll
       for (int kt = 0; kt < NT; ++kt) {
@@ -253,21 +293,36 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
         for (int j = 0; j < 16; ++j) sacc[kt][j] = 0.f;
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
-          const vec_t a = *reinterpret_cast<const vec_t*>(&sK[(kt * 32 + l32) * KSTR + 16 * s + 8 * hh]);
+          const vec_t a = *reinterpret_cast<const vec_t*>(&sK[((T0 + kt) * 32 + l32) * KSTR + 16 * s + 8 * hh]);
           sacc[kt] = Mfma32<T>::run(a, qf[s], sacc[kt]);
         }
       }
-      const int k_last = kc0 + NT * 32;  // one past the last key of this update
+      const int k_last = kc0 + (T0 + NT) * 32;  // one past the last key of this update
       const bool tail = (k_last > kv_end) || (CAUSAL && (k_last - 1 > q_begin + wave * 32));
       if (tail) {
 #pragma unroll
         for (int kt = 0; kt < NT; ++kt)
 #pragma unroll
           for (int j = 0; j < 16; ++j) {
-            const int key = kc0 + kt * 32 + (j / 4) * 8 + hh * 4 + (j % 4);
+            const int key = kc0 + (T0 + kt) * 32 + (j / 4) * 8 + hh * 4 + (j % 4);
             const bool masked = key >= kv_end || (CAUSAL && key > qi);
             if (masked) sacc[kt][j] = -INFINITY;
           }
+      }
+      if (MASKED) {
+        // Accumulator register j of the lane is key (j / 4) * 8 + hh * 4 + j % 4 of the tile: bit of the lane's word.
+        bool all_visible = true;
+#pragma unroll
+        for (int kt = 0; kt < NT; ++kt) all_visible = all_visible && mw[T0 + kt] == 0xffffffffu;
+        if (__builtin_amdgcn_ballot_w64(!all_visible) != 0) {  // wavefront-uniform
+#pragma unroll
+          for (int kt = 0; kt < NT; ++kt) {
+            const uint32_t bits = mw[T0 + kt] >> (hh * 4);
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+              if (((bits >> ((j / 4) * 8 + (j % 4))) & 1u) == 0u) sacc[kt][j] = -INFINITY;
+          }
+        }
       }
       // ---- online softmax, one query per lane (pair of lanes l, l ^ 32) ------------------------------------
       float mx = sacc[0][0];
@@ -311,15 +366,29 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 #pragma unroll
           for (int s2 = 0; s2 < 2; ++s2) {
             const vec_t a =
-                *reinterpret_cast<const vec_t*>(&sVt[(mb * 32 + l32) * VSTR + kt * 32 + s2 * 16 + hh * 8]);
+                *reinterpret_cast<const vec_t*>(&sVt[(mb * 32 + l32) * VSTR + (T0 + kt) * 32 + s2 * 16 + hh * 8]);
             oacc[mb] = Mfma32<T>::run(a, pb[kt][s2], oacc[mb]);
           }
       }
     };
-    if (kc0 + 32 < wave_kv_end)
-      update(std::integral_constant<int, 2>{});
-    else
-      update(std::integral_constant<int, 1>{});
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 1> I1;
+    typedef std::integral_constant<int, 2> I2;
+    if (MASKED) {
+      // tiles in which no query of this wavefront sees a key are not computed
+      const bool any0 = __builtin_amdgcn_ballot_w64(mw[0] != 0u) != 0;
+      const bool any1 = __builtin_amdgcn_ballot_w64(mw[1] != 0u) != 0 && kc0 + 32 < wave_kv_end;
+      if (any0 && any1)
+        update(I2{}, I0{});
+      else if (any0)
+        update(I1{}, I0{});
+      else if (any1)
+        update(I1{}, I1{});
+    } else if (kc0 + 32 < wave_kv_end) {
+      update(I2{}, I0{});
+    } else {
+      update(I1{}, I0{});
+    }
   }
 
   // ---- finalise: O / l (0 for rows in the padding), transpose through a wavefront-private LDS tile, 16-byte stores --
@@ -344,7 +413,12 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   for (int pass = 0; pass < 32 / RPP; ++pass) {
     const int row = pass * RPP + lane / C8;
     const int q_row = q_begin + wave * 32 + row;
-    const vec_t v = *reinterpret_cast<const vec_t*>(tile + row * OROW + c8 * 16);
+    vec_t v = *reinterpret_cast<const vec_t*>(tile + row * OROW + c8 * 16);
+    if (MASKED && p.self_bits != nullptr && q_row < p.Tq && c8 * 8 < p.d) {
+      // a flagged query attends to itself only: its output is its own value row
+      const uint32_t word = p.self_bits[static_cast<int64_t>(b) * ((p.Tq + 31) / 32) + q_row / 32];
+      if ((word >> (q_row % 32)) & 1u) v = *reinterpret_cast<const vec_t*>(vb + q_row * p.vs[2] + c8 * 8);
+    }
     const int q_store_end = p.zero_pad == 2 ? q_valid : p.Tq;  // mode 2: rows in the padding are left untouched
     if (q_row < q_store_end && c8 * 8 < p.d) *reinterpret_cast<vec_t*>(ob + q_row * p.os[2] + c8 * 8) = v;
   }
@@ -353,14 +427,16 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 template <typename T, int DP>
 void launch(const AttnParams& p, bool causal, hipStream_t s) {
   const bool scaled = p.q_row_scale != nullptr || p.k_row_scale != nullptr || p.q_col_scale != nullptr;
-  if (causal && scaled)
-    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  if (p.struct_bits != nullptr)
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  else if (causal && scaled)
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, true, true, false>), dim3(p.total), dim3(kThreads), 0, s, p);
   else if (causal)
-    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, true, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, true, false, false>), dim3(p.total), dim3(kThreads), 0, s, p);
   else if (scaled)
-    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false, true, false>), dim3(p.total), dim3(kThreads), 0, s, p);
   else
-    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false, false, false>), dim3(p.total), dim3(kThreads), 0, s, p);
 }
 
 template <typename T>
@@ -380,12 +456,55 @@ bool strides_ok(const int64_t* st) {
   return true;
 }
 
+// One word per thread: bit c % 32 of word c / 32 of a row is set iff mask[row][c] != 0; bits beyond cols are zero.
+__global__ __launch_bounds__(256) void pack_bits_kernel(const uint8_t* __restrict__ mask, int64_t rows, int cols,
+                                                        int wpr, uint32_t* __restrict__ bits) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= rows * wpr) return;
+  const int64_t row = idx / wpr;
+  const int w = static_cast<int>(idx % wpr);
+  const uint8_t* src = mask + row * cols + w * 32;
+  const int n = cols - w * 32 < 32 ? cols - w * 32 : 32;
+  uint32_t word = 0u;
+  for (int c = 0; c < n; ++c) word |= (src[c] != 0 ? 1u : 0u) << c;
+  bits[idx] = word;
+}
+
+// block_any[qc][kc] = some query of rows [128 qc, 128 qc + 127] sees some key of [64 kc, 64 kc + 63].
+__global__ __launch_bounds__(256) void block_any_kernel(const uint32_t* __restrict__ bits, int Tq, int wpr, int nqc,
+                                                        int nkc, uint8_t* __restrict__ block_any) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= nqc * nkc) return;
+  const int qc = idx / nkc, kc = idx % nkc;
+  uint32_t acc = 0u;
+  for (int r = qc * kQB; r < (qc + 1) * kQB && r < Tq; ++r) {
+    acc |= bits[static_cast<int64_t>(r) * wpr + 2 * kc];
+    if (2 * kc + 1 < wpr) acc |= bits[static_cast<int64_t>(r) * wpr + 2 * kc + 1];
+  }
+  block_any[idx] = acc != 0u ? 1 : 0;
+}
+
+struct MaskArgs {
+  const uint32_t* struct_bits = nullptr;
+  const uint8_t* block_any = nullptr;
+  const uint32_t* valid_bits = nullptr;
+  const uint32_t* self_bits = nullptr;
+};
+
 int attention_entry(const char* name, const void* q, const void* k, const void* v, const int32_t* key_lengths,
-                    const float* q_row_scale, const float* k_row_scale, const float* q_col_scale, void* o, int32_t B,
-                    int32_t H, int32_t Tq,
-                    int32_t Tk, int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
-                    const int64_t v_strides[4], const int64_t o_strides[4], int is_causal, int zero_padded_queries,
-                    int dtype, void* stream) {
+                    const MaskArgs& mask, const float* q_row_scale, const float* k_row_scale, const float* q_col_scale,
+                    void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
+                    const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4], int is_causal,
+                    int zero_padded_queries, int dtype, void* stream) {
+  if (mask.struct_bits != nullptr) {
+    if (mask.block_any == nullptr) return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_bits needs block_any", name);
+    if (is_causal)
+      return set_error(TAAC_ERR_INVALID_VALUE, "%s: a structured mask carries its own causal triangle", name);
+    if (mask.self_bits != nullptr && Tq != Tk)
+      return set_error(TAAC_ERR_INVALID_VALUE, "%s: self rows require Tq == Tk", name);
+  } else if (mask.valid_bits != nullptr || mask.self_bits != nullptr || mask.block_any != nullptr) {
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: valid_bits / self_bits / block_any need struct_bits", name);
+  }
   if (B < 0 || H < 0 || Tq < 0 || Tk < 0 || d <= 0)
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: negative dimension or non-positive head_dim", name);
   if (dtype != TAAC_BF16 && dtype != TAAC_F16)
@@ -413,6 +532,12 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   p.q_row_scale = q_row_scale;
   p.k_row_scale = k_row_scale;
   p.q_col_scale = q_col_scale;
+  p.struct_bits = mask.struct_bits;
+  p.valid_bits = mask.valid_bits;
+  p.self_bits = mask.self_bits;
+  p.block_any = mask.block_any;
+  p.wpr = (Tk + 31) / 32;
+  p.nkc = (Tk + kKC - 1) / kKC;
   p.B = B;
   p.H = H;
   p.Tq = Tq;
@@ -447,7 +572,8 @@ extern "C" int taac_flash_attn_fwd(const void* q, const void* k, const void* v, 
                                    const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
                                    const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype,
                                    void* stream) {
-  return taac::attention_entry("taac_flash_attn_fwd", q, k, v, key_lengths, nullptr, nullptr, nullptr, o, B, H, Tq, Tk, d,
+  return taac::attention_entry("taac_flash_attn_fwd", q, k, v, key_lengths, taac::MaskArgs{}, nullptr, nullptr, nullptr, o,
+                               B, H, Tq, Tk, d,
                                q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries, dtype, stream);
 }
 
@@ -458,7 +584,53 @@ extern "C" int taac_flash_attn_scaled_fwd(const void* q, const void* k, const vo
                                           const int64_t k_strides[4], const int64_t v_strides[4],
                                           const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype,
                                           void* stream) {
-  return taac::attention_entry("taac_flash_attn_scaled_fwd", q, k, v, key_lengths, q_row_scale, k_row_scale,
-                               q_col_scale, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries,
+  return taac::attention_entry("taac_flash_attn_scaled_fwd", q, k, v, key_lengths, taac::MaskArgs{}, q_row_scale,
+                               k_row_scale, q_col_scale, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries,
                                dtype, stream);
+}
+
+extern "C" int taac_flash_attn_masked_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
+                                          const uint32_t* struct_bits, const uint8_t* block_any,
+                                          const uint32_t* valid_bits, const uint32_t* self_bits,
+                                          const float* q_row_scale, const float* k_row_scale, const float* q_col_scale,
+                                          void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                                          const int64_t q_strides[4], const int64_t k_strides[4],
+                                          const int64_t v_strides[4], const int64_t o_strides[4],
+                                          int zero_padded_queries, int dtype, void* stream) {
+  if (!struct_bits)
+    return taac::set_error(TAAC_ERR_INVALID_VALUE, "taac_flash_attn_masked_fwd: struct_bits must be given");
+  taac::MaskArgs mask;
+  mask.struct_bits = struct_bits;
+  mask.block_any = block_any;
+  mask.valid_bits = valid_bits;
+  mask.self_bits = self_bits;
+  return taac::attention_entry("taac_flash_attn_masked_fwd", q, k, v, key_lengths, mask, q_row_scale, k_row_scale,
+                               q_col_scale, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, 0,
+                               zero_padded_queries, dtype, stream);
+}
+
+extern "C" int taac_mask_pack_bits(const void* mask, int64_t rows, int32_t cols, uint32_t* bits, void* stream) {
+  using namespace taac;
+  const char* name = "taac_mask_pack_bits";
+  if (rows < 0 || cols <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows >= 0 and cols > 0 required", name);
+  if (rows == 0) return TAAC_OK;
+  if (!mask || !bits) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  const int wpr = (cols + 31) / 32;
+  const int64_t words = rows * wpr;
+  if (words > 0x7fffffffLL * 256) return set_error(TAAC_ERR_UNSUPPORTED, "%s: mask too large", name);
+  hipLaunchKernelGGL(pack_bits_kernel, dim3(static_cast<uint32_t>((words + 255) / 256)), dim3(256), 0, as_stream(stream),
+                     static_cast<const uint8_t*>(mask), rows, cols, wpr, bits);
+  return check_launch(name);
+}
+
+extern "C" int taac_mask_block_any(const uint32_t* struct_bits, int32_t Tq, int32_t Tk, uint8_t* block_any,
+                                   void* stream) {
+  using namespace taac;
+  const char* name = "taac_mask_block_any";
+  if (Tq <= 0 || Tk <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: Tq and Tk must be positive", name);
+  if (!struct_bits || !block_any) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  const int nqc = (Tq + kQB - 1) / kQB, nkc = (Tk + kKC - 1) / kKC;
+  hipLaunchKernelGGL(block_any_kernel, dim3((nqc * nkc + 255) / 256), dim3(256), 0, as_stream(stream), struct_bits, Tq,
+                     (Tk + 31) / 32, nqc, nkc, block_any);
+  return check_launch(name);
 }

@@ -7,6 +7,12 @@ from taac_2026_amd.modeling.backbone import (
     UnifiedInteractionBlock,
     UnifiedSelfAttention,
 )
+from taac_2026_amd.modeling.masks import (
+    MetadataAttentionMask,
+    bfts_attention_mask,
+    bfts_structural_mask,
+    metadata_structural_mask,
+)
 from taac_2026_amd.modeling.normalization import (
     LayerNorm,
     RMSNorm,
@@ -26,17 +32,21 @@ from taac_2026_amd.modeling.sequence import (
 __all__ = [
     "BFTSAttention",
     "LayerNorm",
+    "MetadataAttentionMask",
     "PCVRBackbone",
     "RMSNorm",
     "SwiGLUFeedForward",
     "UnifiedInteractionBlock",
     "UnifiedSelfAttention",
+    "bfts_attention_mask",
+    "bfts_structural_mask",
     "causal_valid_attention_mask",
     "configure_flash_attention_runtime",
     "configure_rms_norm_runtime",
     "flash_attention_runtime_state",
     "make_padding_mask",
     "masked_mean",
+    "metadata_structural_mask",
     "rms_norm_runtime_state",
     "safe_key_padding_mask",
     "scaled_dot_product_attention",

@@ -12,7 +12,7 @@ from contextvars import ContextVar
 
 import torch
 
-from taac_2026_amd.accelerators.attention import FLASH_ATTENTION_BACKENDS, flash_attention
+from taac_2026_amd.accelerators.attention import FLASH_ATTENTION_BACKENDS, StructuredAttentionMask, flash_attention
 
 _FLASH_ATTENTION_BACKEND: ContextVar[str] = ContextVar("taac_2026_amd_flash_attention_backend", default="hip")
 
@@ -83,10 +83,11 @@ def scaled_dot_product_attention(
     q_row_scale: torch.Tensor | None = None,
     k_row_scale: torch.Tensor | None = None,
     q_col_scale: torch.Tensor | None = None,
+    structured_mask: StructuredAttentionMask | None = None,
 ) -> torch.Tensor:
     """Multi-head attention over (B, T, D) projections; returns (B, Tq, D). ``q_row_scale`` / ``k_row_scale``
     (float32 (B, T)) and ``q_col_scale`` (float32 (D,)): optional factors of the query / key rows and of the query
-    features applied inside the kernel."""
+    features applied inside the kernel. ``structured_mask``: a :class:`StructuredAttentionMask` in place of ``attn_mask``."""
     batch, query_len, d_model = q.shape
     head_dim = d_model // num_heads
     q4 = q.view(batch, query_len, num_heads, head_dim).transpose(1, 2)
@@ -110,6 +111,7 @@ def scaled_dot_product_attention(
         q_row_scale=q_row_scale,
         k_row_scale=k_row_scale,
         q_col_scale=q_col_scale,
+        structured_mask=structured_mask,
     )
     return output.transpose(1, 2).contiguous().view(batch, query_len, d_model)
 

@@ -143,8 +143,16 @@ def test_errors(device):
     with pytest.raises(ValueError, match="matching head dimensions"):
         flash_attention(q.to(device), k.to(device), v[..., :4].to(device))
     bad = torch.tensor([[True, False, True, False, False]]).expand(2, 5)[:, None, None, :].expand(2, 3, 5, 5)
+    # the reference's planner refuses a key mask that is not a prefix (flash_attention.py:171-173), and so does its
+    # restatement here; flash_attention itself then serves the mask through the structured-mask kernel, as the
+    # reference serves it through its torch backend
+    from taac_2026_amd.accelerators.attention import plan_flash_attention_mask
+
     with pytest.raises(RuntimeError, match="prefix-valid"):
-        flash_attention(q.to(device), k.to(device), v.to(device), attn_mask=bad.to(device))
+        plan_flash_attention_mask(q.to(device), k.to(device), bad.to(device), is_causal=False)
+    got = flash_attention(q.to(device), k.to(device), v.to(device), attn_mask=bad.to(device)).cpu()
+    expected = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=bad)
+    torch.testing.assert_close(got.float(), expected, **BF16_TOL)
     with pytest.raises(RuntimeError, match="requires CUDA tensors"):
         flash_attention(q, k, v)
     q7 = torch.randn(1, 1, 4, 12, dtype=torch.bfloat16, device=device)

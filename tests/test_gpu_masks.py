@@ -1,0 +1,171 @@
+"""GPU parity: attention under structured masks (structural[query, key] & key_valid[batch, key], optional self-only query
+rows) through the C ABI, against the library SDPA with the dense bool mask and the oracle's per-element mask rules."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import reference as oracle
+from taac_2026_amd.api import (
+    MetadataAttentionMask,
+    bfts_attention_mask,
+    build_structured_mask,
+    flash_attention,
+    scaled_dot_product_attention,
+)
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = dict(rtol=2e-2, atol=2e-2)
+
+
+def _qkv(batch, heads, tokens, dim, seed):
+    g = torch.Generator().manual_seed(seed)
+    return tuple(torch.randn(batch, heads, tokens, dim, generator=g).to(torch.bfloat16) for _ in range(3))
+
+
+def _expected(q, k, v, dense):
+    """Library SDPA with the bool mask (the reference's torch backend, flash_attention.py:552-570); rows without any
+    visible key are defined as zeros, as the kernel and the reference's TileLang kernel define them."""
+    empty = ~dense.any(dim=-1, keepdim=True)
+    out = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=dense | empty)
+    return torch.where(empty.expand(-1, q.shape[1], -1, -1), torch.zeros_like(out), out)
+
+
+@pytest.mark.parametrize("tokens,dim", [(50, 32), (130, 64), (300, 32), (512, 32), (97, 128)])
+def test_random_structured_masks(device, tokens, dim):
+    batch, heads = 3, 2
+    q, k, v = _qkv(batch, heads, tokens, dim, tokens + dim)
+    g = torch.Generator().manual_seed(tokens)
+    structural = torch.rand(tokens, tokens, generator=g) < 0.4
+    structural[tokens // 3] = False                     # a query row that sees nothing: zeros
+    key_valid = torch.rand(batch, tokens, generator=g) < 0.7
+    key_valid[1] = True
+    query_self = torch.rand(batch, tokens, generator=g) < 0.1
+    with torch.no_grad():
+        plain = build_structured_mask(structural.to(device), key_valid.to(device))
+        with_self = build_structured_mask(structural.to(device), key_valid.to(device), query_self.to(device))
+        only_structural = build_structured_mask(structural.to(device))
+        args = (q.to(device), k.to(device), v.to(device))
+        got = flash_attention(*args, structured_mask=plain).cpu()
+        got_self = flash_attention(*args, structured_mask=with_self).cpu()
+        got_struct = flash_attention(*args, structured_mask=only_structural).cpu()
+    dense = (structural[None] & key_valid[:, None, :])[:, None]
+    assert torch.equal(plain.dense().cpu(), dense)
+    torch.testing.assert_close(got.float(), _expected(q, k, v, dense), **BF16_TOL)
+    assert got[:, :, tokens // 3].abs().max().item() == 0.0
+    torch.testing.assert_close(got_struct.float(), _expected(q, k, v, structural[None, None].expand(batch, 1, -1, -1)), **BF16_TOL)
+    # self-only rows return their value row bit for bit; the other rows are unchanged
+    flagged = query_self[:, None, :, None].expand_as(got_self)
+    assert torch.equal(got_self[flagged], v[flagged])
+    assert torch.equal(got_self[~flagged], got[~flagged])
+    assert torch.equal(with_self.dense().cpu(), torch.where(query_self[:, None, :, None], torch.eye(tokens, dtype=torch.bool)[None, None], dense))
+
+
+@pytest.mark.parametrize("seq_causal", [True, False])
+def test_tokenformer_layer_masks(device, seq_causal):
+    """Every layer's mask of a TokenFormer-like token layout (bottom layers full, upper layers sliding windows that shrink
+    by halves; separators seen by everyone, the target sees everyone, padded queries keep themselves): the factored mask
+    equals the oracle's per-element rule, and attention under it equals SDPA with the dense mask. At 512 tokens the
+    narrow windows leave most (query block, key chunk) pairs empty - those are skipped by the kernel."""
+    batch, heads, dim, layers = 3, 2, 32, 6
+    roles = torch.tensor([0] * 20 + [4] + [1] * 460 + [4] + [2] * 20 + [5] * 9 + [3])
+    tokens = roles.numel()
+    assert tokens == 512
+    g = torch.Generator().manual_seed(3)
+    padding = torch.zeros(batch, tokens, dtype=torch.bool)
+    padding[1, 200:481] = True
+    padding[2, 21 + 37:481] = True
+    padding[2, 5] = True
+    q, k, v = _qkv(batch, heads, tokens, dim, 5)
+    for layer in range(layers):
+        with torch.no_grad():
+            mask = bfts_attention_mask(padding.to(device), roles.to(device), layer, layers, seq_causal=seq_causal,
+                                       seq_keep_per_domain=64)
+            got = flash_attention(q.to(device), k.to(device), v.to(device), structured_mask=mask).cpu()
+        dense = mask.dense().cpu()
+        if layer in (0, 3, 5):  # the per-element oracle is slow: three layers cover full, first and narrowest window
+            assert torch.equal(dense[:1], oracle.bfts_attention_mask(padding[:1], roles, layer, layers, seq_causal=seq_causal,
+                                                                      seq_keep_per_domain=64))
+        torch.testing.assert_close(got.float(), _expected(q, k, v, dense), **BF16_TOL)
+        if layer == 5:  # window max(4, 64 / 4) = 16: far-away key chunks of the sequence span are empty for a query block
+            assert mask.block_any.cpu()[1].tolist().count(0) >= 2
+
+
+def test_symbiosis_metadata_mask(device):
+    batch, heads, dim = 4, 4, 64
+    roles = torch.tensor([0, 1] + [2] * 9 + [3] * 7 + [4] * 3 + [5] * 2 + [6] * 150 + [7] * 4)
+    tokens = roles.numel()
+    g = torch.Generator().manual_seed(1)
+    padding = torch.rand(batch, tokens, generator=g) < 0.3
+    padding[:, :2] = False
+    padding[3] = True                                           # an all-padded sample keeps key 0 (safe mask)
+    q, k, v = _qkv(batch, heads, tokens, dim, 2)
+    for enabled in (True, False):
+        module = MetadataAttentionMask(enabled=enabled)
+        with torch.no_grad():
+            mask = module(padding.to(device), roles.to(device))
+            got = flash_attention(q.to(device), k.to(device), v.to(device), structured_mask=mask).cpu()
+        dense = mask.dense().cpu()
+        assert torch.equal(dense[:2], oracle.metadata_attention_mask(padding[:2], roles, enabled=enabled))
+        assert dense[:, :, 0, :].any(dim=-1).all() and dense[:, :, 1, :].any(dim=-1).all()   # the reference's own check
+        torch.testing.assert_close(got.float(), _expected(q, k, v, dense), **BF16_TOL)
+
+
+def test_dense_bool_masks_are_factored(device):
+    """A (B, 1, T, T) or (B, H, T, T) bool mask that is neither a key prefix nor causal-valid is factored and verified by
+    the planner (the reference's accelerated path rejects it and runs torch SDPA); masks without the factored form are
+    refused with a RuntimeError."""
+    batch, heads, tokens, dim = 3, 2, 70, 32
+    roles = torch.tensor([0] * 5 + [4] + [1] * 50 + [4] + [2] * 12 + [3])
+    padding = torch.zeros(batch, tokens, dtype=torch.bool)
+    padding[1, 30:56] = True
+    q, k, v = _qkv(batch, heads, tokens, dim, 9)
+    dense = oracle.bfts_attention_mask(padding, roles, 2, 4, seq_causal=True, seq_keep_per_domain=8)
+    expected = _expected(q, k, v, dense)
+    with torch.no_grad():
+        args = (q.to(device), k.to(device), v.to(device))
+        got1 = flash_attention(*args, attn_mask=dense.to(device)).cpu()
+        got_h = flash_attention(*args, attn_mask=dense.expand(-1, heads, -1, -1).contiguous().to(device)).cpu()
+        torch.testing.assert_close(got1.float(), expected, **BF16_TOL)
+        assert torch.equal(got1, got_h)
+        # (B, T, D) front end used by the model packages
+        q3, k3, v3 = (t.transpose(1, 2).reshape(batch, tokens, heads * dim).to(device) for t in (q, k, v))
+        got3 = scaled_dot_product_attention(q3, k3, v3, num_heads=heads, attn_mask=dense.to(device), dropout_p=0.0,
+                                            training=False).cpu()
+        torch.testing.assert_close(got3.view(batch, tokens, heads, dim).transpose(1, 2).float(), expected, **BF16_TOL)
+        bad = dense.clone()
+        bad[0, 0, 10, 3] = ~bad[0, 0, 10, 3]        # differs between samples in a way no key_valid explains
+        bad[1, 0, 10, 3] = ~bad[0, 0, 10, 3]
+        with pytest.raises(RuntimeError, match="structural"):
+            flash_attention(*args, attn_mask=bad.to(device))
+        per_head = dense.expand(-1, heads, -1, -1).clone()
+        per_head[:, 1, 4, 2] = ~per_head[:, 1, 4, 2]
+        with pytest.raises(RuntimeError, match="shared across heads"):
+            flash_attention(*args, attn_mask=per_head.to(device))
+
+
+def test_structured_mask_with_key_lengths_and_row_factors(device):
+    from taac_2026_amd.accelerators.attention import hip_flash_attention_kernel
+
+    batch, heads, tokens, dim = 3, 2, 160, 32
+    q, k, v = _qkv(batch, heads, tokens, dim, 4)
+    g = torch.Generator().manual_seed(6)
+    structural = (torch.arange(tokens)[:, None] - torch.arange(tokens)[None, :]).abs() <= 20
+    lengths = torch.tensor([160, 33, 97], dtype=torch.int32)
+    sq = 0.5 + torch.rand(batch, tokens, generator=g)
+    sk = 0.5 + torch.rand(batch, tokens, generator=g)
+    key_valid = torch.arange(tokens)[None, :] < lengths[:, None]
+    dense = (structural[None] & key_valid[:, None, :])[:, None]
+    expected = _expected(q.float() * sq[:, None, :, None], k.float() * sk[:, None, :, None], v, dense)
+    expected = expected * key_valid[:, None, :, None]     # zero_padded_queries
+    with torch.no_grad():
+        mask = build_structured_mask(structural.to(device))
+        got = hip_flash_attention_kernel(q.to(device), k.to(device), v.to(device), lengths.to(device),
+                                         zero_padded_queries=True, q_row_scale=sq.to(device), k_row_scale=sk.to(device),
+                                         structured_mask=mask).cpu()
+        with pytest.raises(ValueError, match="causal"):
+            hip_flash_attention_kernel(q.to(device), k.to(device), v.to(device), None, is_causal=True, structured_mask=mask)
+    torch.testing.assert_close(got.float(), expected, **BF16_TOL)

@@ -184,3 +184,29 @@ def test_dense_layer_argument_errors():
         api.swiglu_linear(x, w)
     with pytest.raises(RuntimeError, match="requires CUDA tensors"):
         api.amax(x)
+
+
+def test_structural_masks_match_the_per_element_rules():
+    """The (T, T) structural parts of the two model-level masks (vectorised torch expressions) against the oracle's
+    per-element restatement, for every layer, both sequence modes and ragged padding."""
+    from oracle import reference as oracle
+    from taac_2026_amd.modeling.masks import bfts_structural_mask, metadata_structural_mask
+    from taac_2026_amd.modeling.sequence import safe_key_padding_mask
+
+    g = torch.Generator().manual_seed(0)
+    tokens, layers = 37, 5
+    roles = torch.tensor([0] * 3 + [4] + [1] * 24 + [4] + [2] * 4 + [5] * 3 + [3])
+    padding = torch.rand(3, tokens, generator=g) < 0.3
+    padding[2] = True
+    eye = torch.eye(tokens, dtype=torch.bool)
+    for layer in range(layers):
+        for causal in (True, False):
+            structural = bfts_structural_mask(roles, layer, layers, seq_causal=causal, seq_keep_per_domain=10)
+            dense = structural[None] & ~safe_key_padding_mask(padding)[:, None, :]
+            dense = torch.where(padding[:, :, None], eye[None], dense)
+            expected = oracle.bfts_attention_mask(padding, roles, layer, layers, seq_causal=causal, seq_keep_per_domain=10)
+            assert torch.equal(dense[:, None], expected), (layer, causal)
+    roles = torch.randint(0, 8, (29,), generator=g)
+    padding = torch.rand(2, 29, generator=g) < 0.25
+    dense = metadata_structural_mask(roles)[None] & ~safe_key_padding_mask(padding)[:, None, :]
+    assert torch.equal(dense[:, None], oracle.metadata_attention_mask(padding, roles))

@@ -367,3 +367,69 @@ def test_qk_norm_rope_normalises_over_the_model_width_then_rotates():
     b16q, _ = oracle.qk_norm_rope(qb, kb, wq, wk, num_heads=heads, rope_base=10000.0)
     assert f32q.dtype == torch.bfloat16
     torch.testing.assert_close(f32q.float(), b16q.float(), rtol=2e-2, atol=2e-2)
+
+
+# ---- model-level structured masks ------------------------------------------------------------------------------------
+
+
+def test_bfts_mask_hand_derived_case():
+    """Six tokens [user, sep, seq, seq, sep, target], last sequence token of sample 1 padded; 2 layers (one full, one
+    sliding with window max(4, ...) -> use a wider row to see the window: checked on a second, longer case)."""
+    roles = torch.tensor([0, 4, 1, 1, 4, 3])
+    padding = torch.tensor([[False] * 6, [False, False, False, True, False, False]])
+    full = oracle.bfts_attention_mask(padding, roles, 0, 2, seq_causal=True, seq_keep_per_domain=8)[:, 0]
+    # causal triangle + separator columns (1, 4) + the target row sees everything
+    expected0 = torch.tensor([
+        [1, 1, 0, 0, 1, 0],
+        [1, 1, 0, 0, 1, 0],
+        [1, 1, 1, 0, 1, 0],
+        [1, 1, 1, 1, 1, 0],
+        [1, 1, 1, 1, 1, 0],
+        [1, 1, 1, 1, 1, 1]], dtype=torch.bool)
+    assert torch.equal(full[0], expected0)
+    expected1 = expected0.clone()
+    expected1[:, 3] = False               # key 3 is padding in sample 1
+    expected1[3] = False
+    expected1[3, 3] = True                # the padded query keeps itself only
+    assert torch.equal(full[1], expected1)
+
+
+def test_bfts_mask_sliding_window_counts_and_invariants():
+    tokens, layers = 40, 6
+    roles = torch.tensor([0] * 4 + [4] + [1] * 28 + [4] + [2] * 5 + [3])
+    padding = torch.zeros(3, tokens, dtype=torch.bool)
+    padding[1, 20:33] = True
+    padding[2, 5:33] = True
+    for layer in range(layers):
+        for causal in (True, False):
+            m = oracle.bfts_attention_mask(padding, roles, layer, layers, seq_causal=causal, seq_keep_per_domain=16)[:, 0]
+            valid = ~padding
+            diag = torch.diagonal(m, dim1=1, dim2=2)
+            assert diag.all()                                         # every query sees itself
+            assert not (m & padding[:, None, :] & valid[:, :, None]).any()  # valid queries never see padded keys
+            assert (m[:, -1, :] == valid).all()                       # the target row sees every valid key
+            assert (m[0, :, 4]).all() and (m[0, :, 33]).all()          # separator columns are seen by everyone
+            if layer >= 3:
+                window = max(4, math.ceil(16 / 2 ** (layer - 3)))
+                row = 25  # an unpadded sequence query of sample 0, far from both ends of the sequence span
+                lo = max(0, row - window)
+                hi = row if causal else min(tokens - 1, row + window)
+                outside = sum(1 for sep in (4, 33) if not lo <= sep <= hi)  # separators are seen from anywhere
+                assert int(m[0, row].sum()) == (hi - lo + 1) + outside
+
+
+def test_metadata_mask_hand_derived_case_and_invariants():
+    # roles: cls, candidate, user, item, dense, missing, sequence, sequence, stats
+    roles = torch.tensor([0, 1, 2, 3, 4, 5, 6, 6, 7])
+    padding = torch.zeros(2, 9, dtype=torch.bool)
+    padding[1, 7] = True
+    m = oracle.metadata_attention_mask(padding, roles)[:, 0]
+    assert m[0, 0].all() and m[0, 1].all() and m[0, 8].all()            # readout and statistics queries read everything
+    assert m[0, 2].tolist() == [True, True, True, True, True, True, False, False, True]   # a field query skips sequence keys
+    assert m[0, 6].tolist() == [True, True, False, True, False, True, True, True, True]   # a sequence query skips user / dense
+    assert not m[1, :7, 7].any() and not m[1, 8, 7].any()                # the padded key is seen by no other query
+    off = oracle.metadata_attention_mask(padding, roles, enabled=False)[:, 0]
+    assert (off[1] == ~padding[1][None, :].expand(9, 9)).all()
+    # an all-padded sample keeps key 0 visible (safe_key_padding_mask) so that no softmax row is empty
+    allpad = oracle.metadata_attention_mask(torch.ones(1, 9, dtype=torch.bool), roles)[0, 0]
+    assert allpad[:, 0].all()
