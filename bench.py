@@ -286,6 +286,35 @@ def _qk_variant_figures(device, batch: int, steps: int) -> dict:
     return out
 
 
+def _structured_mask_figures(device, batch: int, iters: int) -> dict:
+    """Attention under the layer masks of a TokenFormer-like token layout (512 tokens: user fields, separator, a ragged
+    sequence span, separator, item fields, target) at the headline attention shape: the kernel skips key chunks and
+    tiles nobody sees. Useful FLOPs count visible (query, key) pairs only."""
+    from taac_2026_amd.api import bfts_attention_mask, flash_attention
+
+    g = torch.Generator().manual_seed(42)
+    T, D, H, layers = 512, 256, 8, 6
+    qkv = torch.randn(batch, T, 3 * D, generator=g).to(torch.bfloat16).to(device)
+    q, k, v = (t.view(batch, T, H, D // H).transpose(1, 2) for t in qkv.chunk(3, dim=-1))
+    roles = torch.tensor([0] * 20 + [4] + [1] * 460 + [4] + [2] * 20 + [5] * 9 + [3], device=device)
+    span = torch.randint(32, 461, (batch,), generator=g).to(device)
+    pos = torch.arange(T, device=device)
+    padding = (pos[None, :] >= 21 + span[:, None]) & (pos[None, :] < 481)
+    out: dict[str, dict] = {}
+    with torch.no_grad():
+        out["no_mask"] = {"ms": _event_ms(lambda: flash_attention(q, k, v), iters, 3)}
+        for name, layer in (("layer0_causal_full", 0), ("layer3_window_64", 3), ("layer5_window_16", 5)):
+            mask = bfts_attention_mask(padding, roles, layer, layers, seq_causal=True, seq_keep_per_domain=64)
+            visible = float((mask.structural[None] & mask.key_valid[:, None, :]).sum().item())
+            ms = _event_ms(lambda: flash_attention(q, k, v, structured_mask=mask), iters, 3)
+            out[name] = {"ms": ms, "visible_fraction": visible / (batch * T * T),
+                         "useful_tflops": 4.0 * D * visible / ms / 1e9,
+                         "skipped_key_chunks": int((mask.block_any == 0).sum().item()), "key_chunks": int(mask.block_any.numel())}
+        out["mask_build_ms"] = _event_ms(lambda: bfts_attention_mask(padding, roles, 5, layers, seq_causal=True,
+                                                                      seq_keep_per_domain=64), iters, 3)
+    return out
+
+
 def _cpu_baseline(inputs, budget_s: float = 20.0) -> dict:
     """The oracle's backbone forward (the reference's torch formulas) on the host cores, on a bounded sample."""
     from oracle import reference as oracle
@@ -431,6 +460,7 @@ def main() -> None:
         line["operators"] = _operator_figures(device, iters=20)
         line["fp8_dense_layers"] = _fp8_figures(inputs, device, iters=10)
         line["reference_layer_variants"] = _qk_variant_figures(device, B, max(args.steps // 2, 1))
+        line["structured_masks"] = _structured_mask_figures(device, B, iters=10)
     if not args.skip_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(inputs)
         line["gpu_over_cpu"] = value / line["cpu_baseline"]["value"]

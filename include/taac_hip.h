@@ -123,7 +123,7 @@ int taac_flash_attn_scaled_fwd(const void* q, const void* k, const void* v, cons
  * self_bits: uint32 [B, ceil(Tq / 32)] or NULL; a flagged query row returns its own value row (the reference's
  * fallback for padded queries, which attend to themselves only; requires Tq == Tk). Rows with no visible key give
  * zeros. The row / feature factors are those of taac_flash_attn_scaled_fwd (NULL: none). Everything else as
- * taac_flash_attn_fwd; no is_causal (put the triangle into structural).
+ * taac_flash_attn_fwd; no is_causal (put the triangle into structural); Tk <= 4096.
  */
 int taac_flash_attn_masked_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
                                const uint32_t* struct_bits, const uint8_t* block_any, const uint32_t* valid_bits,

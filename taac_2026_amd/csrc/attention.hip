@@ -257,9 +257,14 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 
   // Chunks are walked in order; with a structured mask the chunks in which no query of this workgroup's block sees
   // any key (block_any, shared by the batch) are skipped altogether: not staged, not synchronised on.
+  // The block's row of block_any is read once, as one bit per chunk (at most 64 chunks: Tk <= 4096 with a mask).
+  uint64_t chunk_bits = ~0ull;
+  if (MASKED) chunk_bits = __builtin_amdgcn_ballot_w64(lane < p.nkc && p.block_any[qc * p.nkc + (lane < p.nkc ? lane : 0)] != 0);
   auto next_chunk = [&](int kc) -> int {
     if (MASKED) {
-      while (kc * kKC < kv_end && p.block_any[qc * p.nkc + kc] == 0) ++kc;
+      const uint64_t rest = kc < 64 ? chunk_bits >> kc : 0ull;
+      if (rest == 0ull) return -1;
+      kc += __builtin_ctzll(rest);
     }
     return kc * kKC < kv_end ? kc : -1;
   };
@@ -498,6 +503,7 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
                     int zero_padded_queries, int dtype, void* stream) {
   if (mask.struct_bits != nullptr) {
     if (mask.block_any == nullptr) return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_bits needs block_any", name);
+    if (Tk > 64 * kKC) return set_error(TAAC_ERR_UNSUPPORTED, "%s: structured masks cover at most %d keys", name, 64 * kKC);
     if (is_causal)
       return set_error(TAAC_ERR_INVALID_VALUE, "%s: a structured mask carries its own causal triangle", name);
     if (mask.self_bits != nullptr && Tq != Tk)
