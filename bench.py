@@ -360,6 +360,11 @@ def main() -> None:
     parser.add_argument("--skip-operators", action="store_true")
     parser.add_argument("--skip-all-positions", action="store_true",
                         help="do not time the comparison run over the padded positions (keeps kernel traces to one mode)")
+    parser.add_argument("--skip-widened", action="store_true",
+                        help="leave out the reference-layer variants and the structured-mask figures (keeps kernel traces "
+                             "and counter runs of the headline recipe free of their dispatches)")
+    parser.add_argument("--only-structured-masks", action="store_true",
+                        help="time only attention under the TokenFormer layer masks and print those figures")
     parser.add_argument("--only-layer-variants", action="store_true",
                         help="time only the backbone with the reference layers' query / key norm (and rotary embedding) "
                              "and print those figures (for kernel traces of that mode)")
@@ -373,6 +378,9 @@ def main() -> None:
     from taac_2026_amd.api import PCVRBackbone
 
     device = torch.device("cuda:0")
+    if args.only_structured_masks:
+        print(json.dumps({"structured_masks": _structured_mask_figures(device, args.batch, iters=10)}))
+        return
     if args.only_layer_variants:
         print(json.dumps({"reference_layer_variants": _qk_variant_figures(device, args.batch, args.steps)}))
         return
@@ -459,8 +467,9 @@ def main() -> None:
     if not args.skip_operators:
         line["operators"] = _operator_figures(device, iters=20)
         line["fp8_dense_layers"] = _fp8_figures(inputs, device, iters=10)
-        line["reference_layer_variants"] = _qk_variant_figures(device, B, max(args.steps // 2, 1))
-        line["structured_masks"] = _structured_mask_figures(device, B, iters=10)
+        if not args.skip_widened:
+            line["reference_layer_variants"] = _qk_variant_figures(device, B, max(args.steps // 2, 1))
+            line["structured_masks"] = _structured_mask_figures(device, B, iters=10)
     if not args.skip_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(inputs)
         line["gpu_over_cpu"] = value / line["cpu_baseline"]["value"]

@@ -475,18 +475,18 @@ __global__ __launch_bounds__(256) void pack_bits_kernel(const uint8_t* __restric
   bits[idx] = word;
 }
 
-// block_any[qc][kc] = some query of rows [128 qc, 128 qc + 127] sees some key of [64 kc, 64 kc + 63].
-__global__ __launch_bounds__(256) void block_any_kernel(const uint32_t* __restrict__ bits, int Tq, int wpr, int nqc,
-                                                        int nkc, uint8_t* __restrict__ block_any) {
-  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= nqc * nkc) return;
-  const int qc = idx / nkc, kc = idx % nkc;
+// block_any[qc][kc] = some query of rows [128 qc, 128 qc + 127] sees some key of [64 kc, 64 kc + 63]. One wavefront
+// per (qc, kc): each lane ORs the two words of two rows.
+__global__ __launch_bounds__(kWave) void block_any_kernel(const uint32_t* __restrict__ bits, int Tq, int wpr, int nkc,
+                                                          uint8_t* __restrict__ block_any) {
+  const int qc = blockIdx.x / nkc, kc = blockIdx.x % nkc;
   uint32_t acc = 0u;
-  for (int r = qc * kQB; r < (qc + 1) * kQB && r < Tq; ++r) {
+  for (int r = qc * kQB + static_cast<int>(threadIdx.x); r < (qc + 1) * kQB && r < Tq; r += kWave) {
     acc |= bits[static_cast<int64_t>(r) * wpr + 2 * kc];
     if (2 * kc + 1 < wpr) acc |= bits[static_cast<int64_t>(r) * wpr + 2 * kc + 1];
   }
-  block_any[idx] = acc != 0u ? 1 : 0;
+  const bool any = __builtin_amdgcn_ballot_w64(acc != 0u) != 0;
+  if (threadIdx.x == 0) block_any[blockIdx.x] = any ? 1 : 0;
 }
 
 struct MaskArgs {
@@ -636,7 +636,7 @@ extern "C" int taac_mask_block_any(const uint32_t* struct_bits, int32_t Tq, int3
   if (Tq <= 0 || Tk <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: Tq and Tk must be positive", name);
   if (!struct_bits || !block_any) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
   const int nqc = (Tq + kQB - 1) / kQB, nkc = (Tk + kKC - 1) / kKC;
-  hipLaunchKernelGGL(block_any_kernel, dim3((nqc * nkc + 255) / 256), dim3(256), 0, as_stream(stream), struct_bits, Tq,
-                     (Tk + 31) / 32, nqc, nkc, block_any);
+  hipLaunchKernelGGL(block_any_kernel, dim3(nqc * nkc), dim3(kWave), 0, as_stream(stream), struct_bits, Tq,
+                     (Tk + 31) / 32, nkc, block_any);
   return check_launch(name);
 }
