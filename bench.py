@@ -170,6 +170,37 @@ def _operator_figures(device, iters: int) -> dict:
     return figures
 
 
+def _embedding_figures(device, iters: int) -> dict:
+    """Multi-hot embedding lookup with mean pooling, the step in front of the backbone: the reference operator
+    benchmark's table (1 000 000 x 64 fp16, bags of 4 ids, 25 % padding; pcvr_tilelang_ops_benchmark.py:59-62) at a batch
+    that fills the device, and a table that does not fit the last-level cache. Algorithmic bytes: the gathered rows, the
+    ids and the output."""
+    from oracle import reference as oracle
+    from taac_2026_amd.api import embedding_bag_mean
+
+    out = {}
+    g = torch.Generator().manual_seed(42)
+    for name, vocab, dim, bags, bag_size in (("vocab1M_dim64_bags1M_x4_fp16", 1_000_000, 64, 1 << 20, 4),
+                                             ("vocab4M_dim128_bags1M_x8_fp16", 4_000_000, 128, 1 << 20, 8)):
+        weight = torch.randn(vocab, dim, generator=g).to(torch.float16)
+        values = torch.randint(1, vocab, (bags, bag_size), generator=g)
+        values[torch.rand(bags, bag_size, generator=g) < 0.25] = 0
+        gathered = int((values != 0).sum().item())
+        dev_w, dev_v = weight.to(device), values.to(device)
+        with torch.no_grad():
+            got = embedding_bag_mean(dev_w, dev_v)
+            pick = torch.arange(0, bags, 4099)
+            err = (got[pick.to(device)].cpu().float() - oracle.embedding_bag_mean_closed_form(weight, values[pick])).abs().max().item()
+            if not err <= 1e-2:
+                raise SystemExit(f"accuracy gate of embedding_bag_mean failed: {err}")
+            ms = _event_ms(lambda: embedding_bag_mean(dev_w, dev_v), iters, 3)
+        nbytes = gathered * dim * 2 + bags * bag_size * 8 + bags * dim * 2
+        out[name] = {"ms": ms, "algorithmic_bytes": nbytes, "gbs": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS,
+                     "max_abs_err": err}
+        del dev_w, dev_v, weight, values
+    return out
+
+
 def _fp8_figures(inputs, device, iters: int) -> dict:
     """Configuration 5: the block's four dense layers with e4m3 operands (per-tensor scale amax / 448) over all
     M = B * T tokens, each checked on a slice of rows against the quantize -> matmul -> dequantize emulation."""
@@ -467,6 +498,7 @@ def main() -> None:
     if not args.skip_operators:
         line["operators"] = _operator_figures(device, iters=20)
         line["fp8_dense_layers"] = _fp8_figures(inputs, device, iters=10)
+        line["embedding_bag_mean"] = _embedding_figures(device, iters=20)
         if not args.skip_widened:
             line["reference_layer_variants"] = _qk_variant_figures(device, B, max(args.steps // 2, 1))
             line["structured_masks"] = _structured_mask_figures(device, B, iters=10)

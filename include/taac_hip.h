@@ -298,6 +298,22 @@ int taac_masked_mean_head(const void* x, const int32_t* lengths, const void* w_h
                           int32_t B, int32_t T, int32_t D, void* stream);
 
 /*
+ * Multi-hot embedding lookup with mean pooling: out[b, :] = mean of weight[id, :] over the ids of bag b that are not the
+ * padding id 0; a bag without any such id gives zeros. fp32 accumulation, one rounding to the table's dtype.
+ * weight: [num_embeddings, emb_dim] contiguous; values: [bags, bag_size] int32 (index_is_int64 == 0) or int64,
+ * contiguous; out: [bags, emb_dim] in weight's dtype. Ids outside [0, num_embeddings) are skipped like padding and, when
+ * invalid_count (one int32 on the device, zeroed by the caller) is given, counted there: the reference's torch backend
+ * raises an index error for them, a caller that wants that behaviour reads the counter.
+ * Replaces: embedding_bag_mean / _torch_embedding_bag_mean = F.embedding_bag(values, weight, mode="mean",
+ * padding_idx=0) (src/taac2026/infrastructure/accelerators/embedding/embedding_bag.py:82-83, 439-467), the step that
+ * feeds the token backbone (infrastructure/modeling/embeddings.py:65-71); same signature as a kernel registered
+ * through register_embedding_bag_mean_kernel (embedding_bag.py:39,77-79).
+ */
+int taac_embedding_bag_mean_fwd(const void* weight, int64_t num_embeddings, int32_t emb_dim, const void* values,
+                                int index_is_int64, int64_t bags, int32_t bag_size, void* out, int32_t* invalid_count,
+                                int dtype, void* stream);
+
+/*
  * Weights of one backbone block; every pointer is a device pointer to bf16 data in torch nn.Linear layout.
  * Field names follow the reference's parameter names (experiments/symbiosis/backbone.py:24-56).
  * Biases may be NULL (treated as zero). query_norm_weight / key_norm_weight are the attention layer's

@@ -20,6 +20,8 @@ Puiching-Memory/TAAC_2026). How each function is pinned, independently of its ow
                       test_primitives.py:36-39, tests/contract/experiments/test_packages.py:597-617,
                       test_tilelang_ops.py:361-428), committed as tests/golden/mask_vectors.json.
   masked_mean         float64 brute force; all-padded rows give zeros (divisor clamp).
+  embedding_bag_mean  the library routine F.embedding_bag and the closed form held by the reference's own test
+                      (test_tilelang_ops.py:123-140) on that test's literal id matrix; float64 loop brute force.
   bfts_attention_mask / metadata_attention_mask
                       the reference holds no known answer for them (its contract test checks the shape and that the
                       readout rows see a key, tests/contract/experiments/test_packages.py:430-440); restated here as
@@ -184,6 +186,23 @@ def scaled_dot_product_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tens
     v4 = v.view(batch, v.shape[1], num_heads, head_dim).transpose(1, 2)
     out = attention(q4, k4, v4, key_lengths, zero_padded_queries=zero_padded_queries)
     return out.transpose(1, 2).contiguous().view(batch, query_len, d_model)
+
+
+# ---- embedding bag -------------------------------------------------------------------------------------------------------
+
+
+def embedding_bag_mean(weight: torch.Tensor, values: torch.Tensor) -> torch.Tensor:
+    """``_torch_embedding_bag_mean`` (accelerators/embedding/embedding_bag.py:82-83): mean of the rows named by the
+    non-zero ids of each bag, zeros for a bag of padding only."""
+    return F.embedding_bag(values.long(), weight, mode="mean", padding_idx=0)
+
+
+def embedding_bag_mean_closed_form(weight: torch.Tensor, values: torch.Tensor) -> torch.Tensor:
+    """The expression the reference's own test and benchmark compare against (tests/unit/infrastructure/accelerators/
+    test_tilelang_ops.py:134-137, application/benchmarking/pcvr_tilelang_ops_benchmark.py:171-174), in float32."""
+    embedded = F.embedding(values.long(), weight.float(), padding_idx=0)
+    valid = values.ne(0).to(embedded.dtype).unsqueeze(-1)
+    return (embedded * valid).sum(dim=1) / valid.sum(dim=1).clamp_min(1.0)
 
 
 # ---- model-level structured masks ------------------------------------------------------------------------------------

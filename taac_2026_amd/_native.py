@@ -121,6 +121,10 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         [c_void_p, c_int, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
          c_int32, c_int32, c_int, c_int, c_void_p],
     ),
+    "taac_embedding_bag_mean_fwd": (
+        c_int,
+        [c_void_p, c_int64, c_int32, c_void_p, c_int, c_int64, c_int32, c_void_p, c_void_p, c_int, c_void_p],
+    ),
     "taac_masked_mean_head": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p],

@@ -14,6 +14,11 @@ from taac_2026_amd.accelerators.attention import (
     resolved_flash_attention_backend,
     rope_table,
 )
+from taac_2026_amd.accelerators.embedding import (
+    embedding_bag_mean,
+    hip_embedding_bag_mean_kernel,
+    resolved_embedding_bag_mean_backend,
+)
 from taac_2026_amd.accelerators.linear import (
     amax,
     linear,
@@ -47,7 +52,9 @@ __all__ = [
     "amax",
     "build_structured_mask",
     "concrete_tensors",
+    "embedding_bag_mean",
     "flash_attention",
+    "hip_embedding_bag_mean_kernel",
     "hip_flash_attention_kernel",
     "hip_layer_norm_kernel",
     "hip_rms_norm_kernel",
@@ -63,6 +70,7 @@ __all__ = [
     "require_cuda_tensors",
     "require_same_device",
     "require_same_dtype",
+    "resolved_embedding_bag_mean_backend",
     "resolved_flash_attention_backend",
     "resolved_layer_norm_backend",
     "resolved_rms_norm_backend",

@@ -7,6 +7,7 @@ from taac_2026_amd.modeling.backbone import (
     UnifiedInteractionBlock,
     UnifiedSelfAttention,
 )
+from taac_2026_amd.modeling.embeddings import hash_compress_ids, sparse_embedding_bag_mean
 from taac_2026_amd.modeling.masks import (
     MetadataAttentionMask,
     bfts_attention_mask,
@@ -44,10 +45,12 @@ __all__ = [
     "configure_flash_attention_runtime",
     "configure_rms_norm_runtime",
     "flash_attention_runtime_state",
+    "hash_compress_ids",
     "make_padding_mask",
     "masked_mean",
     "metadata_structural_mask",
     "rms_norm_runtime_state",
     "safe_key_padding_mask",
     "scaled_dot_product_attention",
+    "sparse_embedding_bag_mean",
 ]

@@ -1,0 +1,92 @@
+"""GPU parity: multi-hot embedding lookup with mean pooling (through the C ABI) against the CPU oracle."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from oracle import reference as oracle
+from taac_2026_amd.api import embedding_bag_mean
+
+pytestmark = pytest.mark.gpu
+
+# tolerances of the reference's operator benchmark (pcvr_tilelang_ops_benchmark.py:177-184)
+TOL = {torch.float32: 1e-5, torch.float16: 1e-2, torch.bfloat16: 2e-2}
+
+
+def test_reference_fixture(device):
+    """The id matrix of the reference's own test (tests/unit/infrastructure/accelerators/test_tilelang_ops.py:123-140)."""
+    weight = torch.randn(8, 5, generator=torch.Generator().manual_seed(0))
+    values = torch.tensor([[1, 2, 0, 4], [0, 0, 0, 0], [3, 3, 7, 0]], dtype=torch.long)
+    with torch.no_grad():
+        got = embedding_bag_mean(weight.to(device), values.to(device)).cpu()
+    torch.testing.assert_close(got, oracle.embedding_bag_mean(weight, values), rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(got, oracle.embedding_bag_mean_closed_form(weight, values), rtol=1e-6, atol=1e-6)
+    assert got[1].abs().max().item() == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("index_dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("vocab,dim,bags,bag_size", [(1000, 64, 257, 4), (50, 8, 33, 1), (4096, 128, 100, 7),
+                                                      (300, 100, 19, 5), (2000, 1024, 9, 3), (64, 4096, 3, 2), (77, 5, 40, 9)])
+def test_matches_oracle(device, dtype, index_dtype, vocab, dim, bags, bag_size):
+    g = torch.Generator().manual_seed(vocab + dim + bags)
+    weight = torch.randn(vocab, dim, generator=g).to(dtype)
+    values = torch.randint(0, vocab, (bags, bag_size), generator=g)
+    values[torch.rand(bags, bag_size, generator=g) < 0.25] = 0      # the reference benchmark's padding probability
+    values[0] = 0                                                    # a bag of padding only
+    expected = oracle.embedding_bag_mean_closed_form(weight, values)
+    with torch.no_grad():
+        got = embedding_bag_mean(weight.to(device), values.to(index_dtype).to(device))
+    assert got.shape == (bags, dim) and got.dtype == dtype
+    torch.testing.assert_close(got.cpu().float(), expected, rtol=TOL[dtype], atol=TOL[dtype])
+    assert got[0].abs().max().item() == 0.0
+    if dtype == torch.float32:
+        torch.testing.assert_close(got.cpu(), oracle.embedding_bag_mean(weight, values), rtol=1e-5, atol=1e-5)
+
+
+def test_benchmark_shape_and_properties(device):
+    """The reference benchmark's default shape (vocabulary 1 000 000 x 64, bags of 4, fp16) at a batch that fills the
+    device: a slice against the oracle, and two size-independent properties - a bag's mean does not depend on the
+    order of its ids, and a table of constant rows returns that constant for every non-empty bag."""
+    vocab, dim, bags, bag_size = 1_000_000, 64, 262_144, 4
+    g = torch.Generator().manual_seed(42)
+    weight = torch.randn(vocab, dim, generator=g).to(torch.float16)
+    values = torch.randint(1, vocab, (bags, bag_size), generator=g)
+    values[torch.rand(bags, bag_size, generator=g) < 0.25] = 0
+    with torch.no_grad():
+        dev_w, dev_v = weight.to(device), values.to(device)
+        got = embedding_bag_mean(dev_w, dev_v)
+        flipped = embedding_bag_mean(dev_w, dev_v.flip(1).contiguous())
+        ones = embedding_bag_mean(torch.full_like(dev_w, 0.5), dev_v)
+    pick = torch.arange(0, bags, 1021)
+    torch.testing.assert_close(got[pick.to(device)].cpu().float(), oracle.embedding_bag_mean_closed_form(weight, values[pick]),
+                               rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(got.float(), flipped.float(), rtol=0, atol=2e-3)
+    nonempty = (values != 0).any(dim=1).to(device)
+    assert (ones[nonempty] == 0.5).all() and (ones[~nonempty] == 0).all()
+
+
+def test_argument_errors_and_index_check(device):
+    weight = torch.randn(16, 8, device=device)
+    values = torch.tensor([[1, 2], [3, 0]], device=device)
+    with pytest.raises(ValueError, match="weight must be a 2D tensor"):
+        embedding_bag_mean(weight[0], values)
+    with pytest.raises(ValueError, match="values must be a 2D tensor"):
+        embedding_bag_mean(weight, values[0])
+    with pytest.raises(RuntimeError, match="int32 or int64"):
+        embedding_bag_mean(weight, values.float())
+    with pytest.raises(RuntimeError, match="does not support dtype"):
+        embedding_bag_mean(weight.double(), values)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        embedding_bag_mean(weight.cpu(), values.cpu())
+    with pytest.raises(ValueError, match="unsupported embedding_bag_mean backend"):
+        embedding_bag_mean(weight, values, backend="numpy")
+    bad = torch.tensor([[1, 99], [-3, 2]], device=device)
+    with torch.no_grad():
+        skipped = embedding_bag_mean(weight, bad)        # out-of-range ids are skipped like padding ...
+        torch.testing.assert_close(skipped[0], weight[1])
+        torch.testing.assert_close(skipped[1], weight[2])
+        with pytest.raises(IndexError, match="2 ids are outside"):   # ... or reported, at the price of a host sync
+            embedding_bag_mean(weight, bad, check_indices=True)
+        assert embedding_bag_mean(weight, values, check_indices=True).shape == (2, 8)

@@ -210,3 +210,15 @@ def test_structural_masks_match_the_per_element_rules():
     padding = torch.rand(2, 29, generator=g) < 0.25
     dense = metadata_structural_mask(roles)[None] & ~safe_key_padding_mask(padding)[:, None, :]
     assert torch.equal(dense[:, None], oracle.metadata_attention_mask(padding, roles))
+
+
+def test_hash_compress_ids_against_the_rule_stated_per_element():
+    from taac_2026_amd.api import hash_compress_ids
+
+    values = torch.tensor([[0, 1, 2, 7, 8, 9, -3, 15, 16, 17, 10**12]])
+    got = hash_compress_ids(values, 8)
+    expected = [[0 if v <= 0 else (v - 1) % 8 + 1 for v in values[0].tolist()]]
+    assert got.tolist() == expected and got.dtype == values.dtype
+    assert got.max().item() <= 8 and (got[values > 0] >= 1).all()
+    assert hash_compress_ids(values, 0).tolist() == [[0] * values.shape[1]]
+    assert hash_compress_ids(values.to(torch.int32)[:, :10], 3).dtype == torch.int32

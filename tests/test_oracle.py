@@ -433,3 +433,24 @@ def test_metadata_mask_hand_derived_case_and_invariants():
     # an all-padded sample keeps key 0 visible (safe_key_padding_mask) so that no softmax row is empty
     allpad = oracle.metadata_attention_mask(torch.ones(1, 9, dtype=torch.bool), roles)[0, 0]
     assert allpad[:, 0].all()
+
+
+# ---- embedding bag -----------------------------------------------------------------------------------------------------
+
+
+def test_embedding_bag_mean_reference_fixture_and_brute_force():
+    """The id matrix of the reference's own test (test_tilelang_ops.py:123-140): library routine, the test's closed
+    form and a float64 loop agree; the all-padding bag is zero, the repeated id counts twice."""
+    weight = torch.randn(8, 5, generator=torch.Generator().manual_seed(0))
+    values = torch.tensor([[1, 2, 0, 4], [0, 0, 0, 0], [3, 3, 7, 0]], dtype=torch.long)
+    got = oracle.embedding_bag_mean(weight, values)
+    torch.testing.assert_close(got, oracle.embedding_bag_mean_closed_form(weight, values))
+    expected = np.zeros((3, 5))
+    for b in range(3):
+        rows = [int(i) for i in values[b] if int(i) != 0]
+        for i in rows:
+            expected[b] += weight[i].double().numpy()
+        expected[b] /= max(1, len(rows))
+    np.testing.assert_allclose(got.double().numpy(), expected, rtol=1e-6, atol=1e-7)
+    assert got[1].abs().max().item() == 0.0
+    torch.testing.assert_close(got[2], (2 * weight[3] + weight[7]) / 3)
