@@ -34,17 +34,22 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 
 
 def _event_ms(fn, iters: int, warmup: int) -> float:
-    """Average duration of ``fn`` in ms, HIP events on the current stream (the stream the kernels are launched on)."""
+    """Duration of ``fn`` in ms per call, HIP events on the current stream (the stream the kernels are launched on):
+    the launches are timed in up to five groups and the median group is reported, so that a single stall on a shared
+    host (seen as one group several times slower than the others) does not end up in a kernel figure."""
     for _ in range(warmup):
         fn()
-    start = torch.cuda.Event(enable_timing=True)
-    stop = torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(iters):
-        fn()
-    stop.record()
-    stop.synchronize()
-    return start.elapsed_time(stop) / iters
+    groups = max(1, min(5, iters // 2))
+    per_group = max(1, iters // groups)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(groups + 1)]
+    marks[0].record()
+    for g in range(groups):
+        for _ in range(per_group):
+            fn()
+        marks[g + 1].record()
+    marks[-1].synchronize()
+    times = sorted(marks[g].elapsed_time(marks[g + 1]) / per_group for g in range(groups))
+    return times[len(times) // 2]
 
 
 def _measured_traffic(kernel_name: str) -> int | None:
@@ -146,7 +151,17 @@ def _operator_figures(device, iters: int) -> dict:
         ms = _event_ms(lambda: layer_norm(xd, gd, bd), iters, 5)
         figures["layernorm_bf16_1048576x256"] = {"ms": ms, "gbs": (nbytes + 512) / ms / 1e6,
                                                  "frac_hbm": (nbytes + 512) / ms / 1e6 / HBM_PEAK_GBS}
-        del xd
+        # backward of both norms at the same shape: x and dy read once, dx written once (dw / db are 512 bytes each)
+        from taac_2026_amd.accelerators.normalization import hip_layer_norm_backward_kernel, hip_rms_norm_backward_kernel
+
+        x2d = xd.view(-1, 256)
+        dy = torch.randn(x2d.shape, generator=torch.Generator().manual_seed(7)).to(torch.bfloat16).to(device)
+        bwd_bytes = 3.0 * x.numel() * 2
+        ms = _event_ms(lambda: hip_rms_norm_backward_kernel(x2d, gd, dy, 1e-6), iters, 5)
+        figures["rmsnorm_bwd_bf16_1048576x256"] = {"ms": ms, "gbs": bwd_bytes / ms / 1e6, "frac_hbm": bwd_bytes / ms / 1e6 / HBM_PEAK_GBS}
+        ms = _event_ms(lambda: hip_layer_norm_backward_kernel(x2d, gd, dy, 1e-5), iters, 5)
+        figures["layernorm_bwd_bf16_1048576x256"] = {"ms": ms, "gbs": bwd_bytes / ms / 1e6, "frac_hbm": bwd_bytes / ms / 1e6 / HBM_PEAK_GBS}
+        del xd, x2d, dy
 
         q, k, v, lengths = workloads.attention_inputs()
         qd, kd, vd, ld = q.to(device), k.to(device), v.to(device), lengths.to(device)

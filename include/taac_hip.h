@@ -69,6 +69,24 @@ int taac_layernorm_fwd(const void* x, const void* w, const void* b, void* y, int
                        int dtype, void* stream);
 
 /*
+ * Backward of taac_rmsnorm_fwd / taac_layernorm_fwd. With g = dy * w and x_hat the normalised row:
+ *   RMSNorm:   dx = rstd * (g - x_hat * mean(g * x_hat));            dw = sum over rows of dy * x_hat
+ *   LayerNorm: dx = rstd * (g - mean(g) - x_hat * mean(g * x_hat));  dw as above; db = sum over rows of dy
+ * The row statistics are recomputed from x (nothing is saved by the forward). x, dy, dx: [rows, cols] contiguous;
+ * w, dw, db: [cols]; all in `dtype`, fp32 arithmetic. dw / db may be NULL (not wanted). workspace: device memory for
+ * taac_norm_bwd_workspace_floats(rows, cols, layer_norm) floats (per-workgroup partial sums of dw / db, added in a
+ * fixed order: the result does not depend on scheduling). cols must be a multiple of the 16-byte vector (8 elements,
+ * 4 for fp32) and at most 256 vectors.
+ * Replaces: the Triton / TileLang backward kernels and their host-side partial sums
+ * (accelerators/normalization/kernels/triton.py:82-116, 276-320; rms_norm.py:294-340, layer_norm.py:170-258).
+ */
+int64_t taac_norm_bwd_workspace_floats(int64_t rows, int32_t cols, int layer_norm);
+int taac_rmsnorm_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw, float* workspace,
+                     int64_t workspace_floats, int64_t rows, int32_t cols, float eps, int dtype, void* stream);
+int taac_layernorm_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw, void* db, float* workspace,
+                       int64_t workspace_floats, int64_t rows, int32_t cols, float eps, int dtype, void* stream);
+
+/*
  * Key-padding-masked attention forward: o = softmax(q k^T / sqrt(d) + mask) v per (batch, head), softmax in
  * fp32, bf16/fp16 MFMA operands. Key j of batch b is visible iff j < key_lengths[b] (and j <= query index when
  * is_causal). key_lengths == NULL means every key is visible. Rows with no visible key produce zeros.

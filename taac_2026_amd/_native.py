@@ -62,6 +62,16 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_float, c_int, c_void_p],
     ),
+    "taac_norm_bwd_workspace_floats": (c_int64, [c_int64, c_int32, c_int]),
+    "taac_rmsnorm_bwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_float, c_int, c_void_p],
+    ),
+    "taac_layernorm_bwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_float, c_int,
+         c_void_p],
+    ),
     "taac_flash_attn_fwd": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32]

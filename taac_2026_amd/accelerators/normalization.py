@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from taac_2026_amd import _native
-from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference
+from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors
 
 RMS_NORM_BACKENDS = ("hip", "torch", "tilelang", "triton")
 LAYER_NORM_BACKENDS = ("hip", "torch", "triton")
@@ -104,6 +104,78 @@ def hip_layer_norm_kernel(x: torch.Tensor, weight: torch.Tensor, bias: torch.Ten
     return out
 
 
+def _backward_workspace(rows: torch.Tensor, layer_norm_parts: bool) -> torch.Tensor:
+    library = _native.load_library()
+    count = int(library.taac_norm_bwd_workspace_floats(rows.shape[0], rows.shape[1], int(layer_norm_parts)))
+    return torch.empty(count, dtype=torch.float32, device=rows.device)
+
+
+def hip_rms_norm_backward_kernel(x: torch.Tensor, weight: torch.Tensor, grad_out: torch.Tensor, eps: float
+                                 ) -> tuple[torch.Tensor, torch.Tensor]:
+    """``(rows [R, D], weight [D], grad_out [R, D], eps) -> (grad_rows [R, D], grad_weight [D])`` in x's dtype."""
+    library = _native.load_library()
+    require_cuda_tensors("hip rms_norm backward", x, weight, grad_out)
+    grad_x, grad_w = torch.empty_like(x), torch.empty_like(weight)
+    workspace = _backward_workspace(x, False)
+    status = library.taac_rmsnorm_bwd(
+        x.data_ptr(), weight.data_ptr(), grad_out.data_ptr(), grad_x.data_ptr(), grad_w.data_ptr(), workspace.data_ptr(),
+        workspace.numel(), x.shape[0], x.shape[1], float(eps), _native.dtype_code(x.dtype), _native.current_stream(x.device),
+    )
+    _native.check(status, "rms_norm backward")
+    return grad_x, grad_w
+
+
+def hip_layer_norm_backward_kernel(x: torch.Tensor, weight: torch.Tensor, grad_out: torch.Tensor, eps: float
+                                   ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``-> (grad_rows, grad_weight, grad_bias)`` in x's dtype."""
+    library = _native.load_library()
+    require_cuda_tensors("hip layer_norm backward", x, weight, grad_out)
+    grad_x, grad_w, grad_b = torch.empty_like(x), torch.empty_like(weight), torch.empty_like(weight)
+    workspace = _backward_workspace(x, True)
+    status = library.taac_layernorm_bwd(
+        x.data_ptr(), weight.data_ptr(), grad_out.data_ptr(), grad_x.data_ptr(), grad_w.data_ptr(), grad_b.data_ptr(),
+        workspace.data_ptr(), workspace.numel(), x.shape[0], x.shape[1], float(eps), _native.dtype_code(x.dtype),
+        _native.current_stream(x.device),
+    )
+    _native.check(status, "layer_norm backward")
+    return grad_x, grad_w, grad_b
+
+
+class _HipRMSNormFunction(torch.autograd.Function):
+    """Forward and backward on the HIP kernels (the role of _TritonRMSNormFunction, rms_norm.py:318-340); the backward
+    recomputes the row statistic from the saved input, so the forward is the inference kernel."""
+
+    @staticmethod
+    def forward(ctx, rows: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+        ctx.save_for_backward(rows, weight)
+        ctx.eps = float(eps)
+        return hip_rms_norm_kernel(rows, weight, eps)
+
+    @staticmethod
+    def backward(ctx, grad_out: torch.Tensor):
+        rows, weight = ctx.saved_tensors
+        grad_rows, grad_weight = hip_rms_norm_backward_kernel(rows, weight, grad_out.contiguous(), ctx.eps)
+        return grad_rows, grad_weight, None
+
+
+class _HipLayerNormFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, rows: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float) -> torch.Tensor:
+        ctx.save_for_backward(rows, weight)
+        ctx.eps = float(eps)
+        return hip_layer_norm_kernel(rows, weight, bias, eps)
+
+    @staticmethod
+    def backward(ctx, grad_out: torch.Tensor):
+        rows, weight = ctx.saved_tensors
+        grad_rows, grad_weight, grad_bias = hip_layer_norm_backward_kernel(rows, weight, grad_out.contiguous(), ctx.eps)
+        return grad_rows, grad_weight, grad_bias, None
+
+
+def _needs_grad(*tensors: torch.Tensor) -> bool:
+    return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+
+
 def rms_norm(
     x: torch.Tensor,
     weight: torch.Tensor,
@@ -112,11 +184,13 @@ def rms_norm(
     backend: str = "hip",
     block_rows: int | None = None,
 ) -> torch.Tensor:
-    """``x * rsqrt(mean(x^2, -1) + eps) * weight`` over the last dimension, fp32 accumulation."""
+    """``x * rsqrt(mean(x^2, -1) + eps) * weight`` over the last dimension, fp32 accumulation. Differentiable: with
+    autograd enabled and an input that requires grad, the backward runs on the HIP kernel too (rms_norm.py:345-360)."""
     del block_rows
     rows, normalized_weight, original_shape = _normalize_rms_norm_inputs(x, weight)
     _resolve_rms_norm_backend(rows, backend)
-    require_inference("hip rms_norm", x, weight)
+    if _needs_grad(x, weight):
+        return _HipRMSNormFunction.apply(rows, normalized_weight, eps).reshape(original_shape)
     return hip_rms_norm_kernel(rows, normalized_weight, eps).reshape(original_shape)
 
 
@@ -129,18 +203,22 @@ def layer_norm(
     backend: str = "hip",
     block_rows: int | None = None,
 ) -> torch.Tensor:
-    """``F.layer_norm(x, (D,), weight, bias, eps)`` over the last dimension, fp32 statistics."""
+    """``F.layer_norm(x, (D,), weight, bias, eps)`` over the last dimension, fp32 statistics. Differentiable like
+    :func:`rms_norm` (layer_norm.py:170-258)."""
     del block_rows
     rows, normalized_weight, normalized_bias, original_shape = _normalize_layer_norm_inputs(x, weight, bias)
     _resolve_layer_norm_backend(rows, backend)
-    require_inference("hip layer_norm", x, weight, bias)
+    if _needs_grad(x, weight, bias):
+        return _HipLayerNormFunction.apply(rows, normalized_weight, normalized_bias, eps).reshape(original_shape)
     return hip_layer_norm_kernel(rows, normalized_weight, normalized_bias, eps).reshape(original_shape)
 
 
 __all__ = [
     "LAYER_NORM_BACKENDS",
     "RMS_NORM_BACKENDS",
+    "hip_layer_norm_backward_kernel",
     "hip_layer_norm_kernel",
+    "hip_rms_norm_backward_kernel",
     "hip_rms_norm_kernel",
     "layer_norm",
     "resolved_layer_norm_backend",

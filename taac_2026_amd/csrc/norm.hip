@@ -266,6 +266,225 @@ int norm_entry(const char* name, const void* x, const void* w, const void* b, vo
 }
 
 
+// ---- backward ----------------------------------------------------------------------------------------------------------
+//
+// RMSNorm:   g = dy * w, x_hat = x * rstd:            dx = rstd * (g - x_hat * mean(g * x_hat)),           dw = sum_rows dy * x_hat
+// LayerNorm: g = dy * w, x_hat = (x - mean) * rstd:   dx = rstd * (g - mean(g) - x_hat * mean(g * x_hat)), dw as above,
+//                                                     db = sum_rows dy
+// (normalization/kernels/triton.py:82-116, 276-320). The row statistics are recomputed from x, which the kernel reads
+// anyway, so nothing has to be saved by the forward. One pass: x and dy read once, dx written once. A workgroup walks
+// several row tiles and keeps its share of dw / db in registers; per workgroup one partial row is written
+// (fixed order inside the workgroup, through LDS), and a second small kernel adds the partials in order: the result
+// does not depend on scheduling.
+template <typename T, int G, int NV, bool LN>
+__global__ __launch_bounds__(kBlock) void norm_bwd_rows_vec_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                    const T* __restrict__ dy, T* __restrict__ dx,
+                                                                    float* __restrict__ partial, int64_t rows, int cols,
+                                                                    int nvec, float eps) {
+  typedef Pack<T> P;
+  typedef typename P::vec vec_t;
+  constexpr int VEC = P::VEC;
+  constexpr int GPB = kBlock / G;
+  __shared__ float red[GPB][G * VEC];
+  const int lane = threadIdx.x % G;
+  const int gid = threadIdx.x / G;
+  const float inv_cols = 1.0f / static_cast<float>(cols);
+
+  float wf[NV][VEC];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = lane + i * G;
+    if (v < nvec) {
+      P::unpack(reinterpret_cast<const vec_t*>(w)[v], wf[i]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) wf[i][e] = 0.f;
+    }
+  }
+  float dwacc[NV][VEC], dbacc[LN ? NV : 1][VEC];
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      dwacc[i][e] = 0.f;
+      if (LN) dbacc[LN ? i : 0][e] = 0.f;
+    }
+
+  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * GPB; row0 < rows; row0 += static_cast<int64_t>(gridDim.x) * GPB) {
+    const int64_t row = row0 + gid;
+    const bool ok = row < rows;
+    vec_t xr[NV], gr[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = lane + i * G;
+      if (ok && v < nvec) {
+        xr[i] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(x + row * cols) + v);
+        gr[i] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(dy + row * cols) + v);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          xr[i][e] = 0;
+          gr[i][e] = 0;
+        }
+      }
+    }
+    float xf[NV][VEC], gf[NV][VEC];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      P::unpack(xr[i], xf[i]);
+      P::unpack(gr[i], gf[i]);
+    }
+    float mean = 0.f;
+    if (LN) {
+      float sum = 0.f;
+#pragma unroll
+      for (int i = 0; i < NV; ++i)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) sum += xf[i][e];
+      mean = group_sum<G>(sum) * inv_cols;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const bool live = (lane + i * G) < nvec;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        xf[i][e] = LN ? (live ? xf[i][e] - mean : 0.f) : xf[i][e];  // centred from here on
+        ss += xf[i][e] * xf[i][e];
+      }
+    }
+    const float rstd = rsqrtf(group_sum<G>(ss) * inv_cols + eps);
+    float sg = 0.f, sgx = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        xf[i][e] *= rstd;  // x_hat
+        const float g = gf[i][e] * wf[i][e];
+        sg += g;
+        sgx += g * xf[i][e];
+      }
+    const float mean_gx = group_sum<G>(sgx) * inv_cols;
+    const float mean_g = LN ? group_sum<G>(sg) * inv_cols : 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = lane + i * G;
+      float of[VEC];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        of[e] = rstd * (gf[i][e] * wf[i][e] - mean_g - xf[i][e] * mean_gx);
+        dwacc[i][e] += gf[i][e] * xf[i][e];  // rows beyond the end contribute zeros
+        if (LN) dbacc[LN ? i : 0][e] += gf[i][e];
+      }
+      if (ok && v < nvec) __builtin_nontemporal_store(P::pack(of), reinterpret_cast<vec_t*>(dx + row * cols) + v);
+    }
+  }
+
+  // Partial row of this workgroup: for every vector index the GPB lane groups meet in LDS and one thread per column adds
+  // them in group order.
+  float* out_w = partial + static_cast<int64_t>(blockIdx.x) * cols * (LN ? 2 : 1);
+#pragma unroll
+  for (int pass = 0; pass < (LN ? 2 : 1); ++pass) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      __syncthreads();
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) red[gid][lane * VEC + e] = pass == 0 ? dwacc[i][e] : dbacc[LN ? i : 0][e];
+      __syncthreads();
+      for (int t = threadIdx.x; t < G * VEC; t += kBlock) {
+        float sum = 0.f;
+#pragma unroll
+        for (int g = 0; g < GPB; ++g) sum += red[g][t];
+        // column of element e of vector lane + i * G is (lane + i * G) * VEC + e = i * G * VEC + t
+        const int col = i * G * VEC + t;
+        if (col < cols) out_w[pass * cols + col] = sum;
+      }
+    }
+  }
+}
+
+// dw[c] (and db[c]) = sum over the workgroups' partial rows, in workgroup order.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void norm_bwd_reduce_kernel(const float* __restrict__ partial, int nblocks, int cols,
+                                                                  int parts, T* __restrict__ dw, T* __restrict__ db) {
+  const int c = blockIdx.x * kBlock + threadIdx.x;
+  if (c >= cols) return;
+  for (int part = 0; part < parts; ++part) {
+    float sum = 0.f;
+    for (int b = 0; b < nblocks; ++b) sum += partial[(static_cast<int64_t>(b) * parts + part) * cols + c];
+    T* dst = part == 0 ? dw : db;
+    if (dst != nullptr) dst[c] = static_cast<T>(sum);
+  }
+}
+
+constexpr int kBwdMaxBlocks = 1024;
+
+template <typename T, bool LN>
+int dispatch_bwd(const void* xv, const void* wv, const void* dyv, void* dxv, void* dwv, void* dbv, float* workspace,
+                 int64_t workspace_floats, int64_t rows, int cols, float eps, hipStream_t s, const char* name) {
+  const T* x = static_cast<const T*>(xv);
+  const T* w = static_cast<const T*>(wv);
+  const T* dy = static_cast<const T*>(dyv);
+  T* dx = static_cast<T*>(dxv);
+  constexpr int VEC = Pack<T>::VEC;
+  if (cols % VEC != 0 || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(w) || cols / VEC > kWave * 4)
+    return set_error(TAAC_ERR_UNSUPPORTED,
+                     "%s: cols must be a multiple of %d and at most %d, tensors 16-byte aligned", name, VEC,
+                     kWave * 4 * VEC);
+  const int nvec = cols / VEC;
+  int G = 1;
+  while (G < nvec && G < kWave) G *= 2;
+  const int gpb = kBlock / G;
+  int64_t nblocks = (rows + gpb - 1) / gpb;
+  if (nblocks > kBwdMaxBlocks) nblocks = kBwdMaxBlocks;
+  const int parts = LN ? 2 : 1;
+  if (workspace == nullptr || workspace_floats < nblocks * parts * cols)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: workspace must hold %lld floats", name,
+                     (long long)(nblocks * parts * cols));
+#define TAAC_BWD_CASE(GG, NV)                                                                                           \
+  hipLaunchKernelGGL((norm_bwd_rows_vec_kernel<T, GG, NV, LN>), dim3(static_cast<uint32_t>(nblocks)), dim3(kBlock), 0, s, \
+                     x, w, dy, dx, workspace, rows, cols, nvec, eps);                                                    \
+  break;
+  if (rows > 0) switch (G) {
+    case 1: TAAC_BWD_CASE(1, 1)
+    case 2: TAAC_BWD_CASE(2, 1)
+    case 4: TAAC_BWD_CASE(4, 1)
+    case 8: TAAC_BWD_CASE(8, 1)
+    case 16: TAAC_BWD_CASE(16, 1)
+    case 32: TAAC_BWD_CASE(32, 1)
+    default:
+      if (nvec <= 64) {
+        TAAC_BWD_CASE(64, 1)
+      } else if (nvec <= 128) {
+        TAAC_BWD_CASE(64, 2)
+      } else {
+        TAAC_BWD_CASE(64, 4)
+      }
+  }
+#undef TAAC_BWD_CASE
+  hipLaunchKernelGGL((norm_bwd_reduce_kernel<T>), dim3((cols + kBlock - 1) / kBlock), dim3(kBlock), 0, s, workspace,
+                     static_cast<int>(nblocks), cols, parts, static_cast<T*>(dwv), static_cast<T*>(dbv));
+  return TAAC_OK;
+}
+
+template <bool LN>
+int norm_bwd_entry(const char* name, const void* x, const void* w, const void* dy, void* dx, void* dw, void* db,
+                   float* workspace, int64_t workspace_floats, int64_t rows, int32_t cols, float eps, int dtype,
+                   void* stream) {
+  if (rows < 0 || cols <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows must be >= 0 and cols > 0", name);
+  if (!x || !w || !dy || !dx) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
+  hipStream_t s = as_stream(stream);
+  int rc;
+  switch (dtype) {
+    case TAAC_F32: rc = dispatch_bwd<float, LN>(x, w, dy, dx, dw, db, workspace, workspace_floats, rows, cols, eps, s, name); break;
+    case TAAC_BF16: rc = dispatch_bwd<bf16_t, LN>(x, w, dy, dx, dw, db, workspace, workspace_floats, rows, cols, eps, s, name); break;
+    case TAAC_F16: rc = dispatch_bwd<f16_t, LN>(x, w, dy, dx, dw, db, workspace, workspace_floats, rows, cols, eps, s, name); break;
+    default: return set_error(TAAC_ERR_INVALID_VALUE, "%s: unknown dtype %d", name, dtype);
+  }
+  if (rc != TAAC_OK) return rc;
+  return check_launch(name);
+}
+
 // ---- query / key RMSNorm + rotary embedding ---------------------------------------------------------------------------
 //
 // Work unit u = (token slot u / 2, which = u % 2): the query (0) or key (1) row of one token; the two rows of a token
@@ -480,4 +699,23 @@ extern "C" int taac_qk_norm_rope_fwd(const void* q, const void* k, int64_t ld_in
   }
   if (rc != TAAC_OK) return rc;
   return check_launch(name);
+}
+
+extern "C" int64_t taac_norm_bwd_workspace_floats(int64_t rows, int32_t cols, int layer_norm) {
+  if (rows < 0 || cols <= 0) return -1;
+  return static_cast<int64_t>(taac::kBwdMaxBlocks) * cols * (layer_norm ? 2 : 1);
+}
+
+extern "C" int taac_rmsnorm_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw, float* workspace,
+                                int64_t workspace_floats, int64_t rows, int32_t cols, float eps, int dtype,
+                                void* stream) {
+  return taac::norm_bwd_entry<false>("taac_rmsnorm_bwd", x, w, dy, dx, dw, nullptr, workspace, workspace_floats, rows,
+                                     cols, eps, dtype, stream);
+}
+
+extern "C" int taac_layernorm_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw, void* db,
+                                  float* workspace, int64_t workspace_floats, int64_t rows, int32_t cols, float eps,
+                                  int dtype, void* stream) {
+  return taac::norm_bwd_entry<true>("taac_layernorm_bwd", x, w, dy, dx, dw, db, workspace, workspace_floats, rows, cols,
+                                    eps, dtype, stream);
 }

@@ -120,7 +120,83 @@ def test_modules_and_errors(device):
         torch.testing.assert_close(norm(x).cpu(), oracle.rms_norm(x.cpu(), torch.ones(64), 1e-6), rtol=1e-5, atol=1e-5)
         torch.testing.assert_close(ln(x).cpu(), oracle.layer_norm(x.cpu(), torch.ones(64), torch.zeros(64), 1e-5),
                                    rtol=1e-5, atol=1e-5)
-    with pytest.raises(RuntimeError, match="forward-only"):
-        norm(x)  # grad enabled and the weight requires grad
+    # with autograd on, the modules train: forward and backward both run on the HIP kernels
+    out = norm(x)
+    assert out.requires_grad
+    out.sum().backward()
+    assert norm.weight.grad is not None and norm.weight.grad.shape == (64,)
     with pytest.raises(ValueError, match="does not match weight size"):
         rms_norm(x, torch.ones(32, device=device))
+
+
+# ---- backward ----------------------------------------------------------------------------------------------------------
+
+# Gradient tolerances of the reference's GPU tests (tests/gpu/infrastructure/accelerators/test_tilelang_ops_cuda.py:
+# 98-141, 206-207): 1e-2 .. 3e-2 for 16-bit inputs; fp32 is held to 1e-4 here.
+GRAD_TOL = {torch.float32: 1e-4, torch.bfloat16: 3e-2, torch.float16: 1e-2}
+
+
+def _autograd_reference(fn, x, params, grad_out):
+    """Gradients of the oracle's closed form by torch autograd in float64 from the stored (rounded) inputs."""
+    xr = x.double().requires_grad_(True)
+    pr = [p.double().requires_grad_(True) for p in params]
+    fn(xr, *pr).backward(grad_out.double())
+    return [xr.grad] + [p.grad for p in pr]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows_shape,cols", [((37, 5), 64), ((3,), 8), ((1000,), 256), ((19, 3), 128), ((257,), 1024),
+                                             ((5, 7), 2048), ((4099,), 96)])
+def test_rmsnorm_backward_matches_autograd_of_the_oracle(device, dtype, rows_shape, cols):
+    if dtype == torch.float32 and cols > 1024:
+        pytest.skip("fp32 rows above 1024 columns are outside the backward kernel's envelope")
+    x, w, _ = _draw(rows_shape, cols, dtype, seed=cols + len(rows_shape))
+    grad_out = torch.randn(*rows_shape, cols, generator=torch.Generator().manual_seed(1)).to(dtype)
+    ref_dx, ref_dw = _autograd_reference(lambda a, b: oracle.rms_norm(a, b, 1e-6), x, [w], grad_out)
+    xd = x.to(device).requires_grad_(True)
+    wd = w.to(device).requires_grad_(True)
+    rms_norm(xd, wd, 1e-6).backward(grad_out.to(device))
+    tol = GRAD_TOL[dtype]
+    torch.testing.assert_close(xd.grad.cpu().double(), ref_dx, rtol=tol, atol=tol)
+    # dw sums rows * values of size ~1: the rounding of a 16-bit result scales with its magnitude
+    scale = max(1.0, ref_dw.abs().max().item())
+    torch.testing.assert_close(wd.grad.cpu().double(), ref_dw, rtol=tol, atol=tol * scale)
+    assert xd.grad.dtype == dtype and wd.grad.dtype == dtype
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows_shape,cols", [((37, 5), 64), ((3,), 8), ((1000,), 256), ((257,), 1024), ((4099,), 96)])
+def test_layernorm_backward_matches_autograd_of_the_oracle(device, dtype, rows_shape, cols):
+    x, w, b = _draw(rows_shape, cols, dtype, seed=7 + cols)
+    x = (x + 2.0).to(dtype)
+    grad_out = torch.randn(*rows_shape, cols, generator=torch.Generator().manual_seed(2)).to(dtype)
+    ref_dx, ref_dw, ref_db = _autograd_reference(lambda a, ww, bb: oracle.layer_norm(a, ww, bb, 1e-5), x, [w, b], grad_out)
+    xd, wd, bd = (t.to(device).requires_grad_(True) for t in (x, w, b))
+    layer_norm(xd, wd, bd, 1e-5).backward(grad_out.to(device))
+    tol = GRAD_TOL[dtype]
+    torch.testing.assert_close(xd.grad.cpu().double(), ref_dx, rtol=tol, atol=tol)
+    for got, ref in ((wd.grad, ref_dw), (bd.grad, ref_db)):
+        scale = max(1.0, ref.abs().max().item())
+        torch.testing.assert_close(got.cpu().double(), ref, rtol=tol, atol=tol * scale)
+
+
+def test_norm_backward_is_deterministic_and_modules_train(device):
+    x, w, b = _draw((5000,), 256, torch.bfloat16, seed=3)
+    grad_out = torch.randn(5000, 256, generator=torch.Generator().manual_seed(4)).to(torch.bfloat16).to(device)
+    grads = []
+    for _ in range(3):
+        xd, wd = x.to(device).requires_grad_(True), w.to(device).requires_grad_(True)
+        rms_norm(xd, wd, 1e-6).backward(grad_out)
+        grads.append((xd.grad.clone(), wd.grad.clone()))
+    assert all(torch.equal(g[0], grads[0][0]) and torch.equal(g[1], grads[0][1]) for g in grads[1:])
+    # fp32 master weights under a bf16 activation, as the reference's modules run under autocast: the gradient arrives
+    # in the parameter's dtype
+    norm = RMSNorm(256).to(device)
+    ln = LayerNorm(256).to(device)
+    h = x.to(device).requires_grad_(True)
+    (ln(norm(h)).float().pow(2).mean()).backward()
+    assert norm.weight.grad.dtype == torch.float32 and ln.bias.grad.dtype == torch.float32 and h.grad.dtype == torch.bfloat16
+    assert torch.isfinite(norm.weight.grad).all() and torch.isfinite(ln.weight.grad).all() and torch.isfinite(h.grad).all()
+    with pytest.raises(RuntimeError, match="multiple of"):
+        rms_norm(torch.randn(4, 100, device=device, dtype=torch.bfloat16).requires_grad_(True), torch.ones(100, device=device))\
+            .sum().backward()
