@@ -310,73 +310,84 @@ __global__ __launch_bounds__(kBlock) void norm_bwd_rows_vec_kernel(const T* __re
       if (LN) dbacc[LN ? i : 0][e] = 0.f;
     }
 
-  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * GPB; row0 < rows; row0 += static_cast<int64_t>(gridDim.x) * GPB) {
-    const int64_t row = row0 + gid;
-    const bool ok = row < rows;
-    vec_t xr[NV], gr[NV];
+  constexpr int R = NV == 1 ? 4 : (NV == 2 ? 2 : 1);  // rows in flight per lane group
+  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * (GPB * R); row0 < rows;
+       row0 += static_cast<int64_t>(gridDim.x) * (GPB * R)) {
+    // every load of the R rows is issued before any of them is used
+    vec_t xr[R][NV], gr[R][NV];
+    bool ok[R];
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const int v = lane + i * G;
-      if (ok && v < nvec) {
-        xr[i] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(x + row * cols) + v);
-        gr[i] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(dy + row * cols) + v);
-      } else {
+    for (int r = 0; r < R; ++r) {
+      const int64_t row = row0 + r * GPB + gid;
+      ok[r] = row < rows;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          xr[i][e] = 0;
-          gr[i][e] = 0;
+      for (int i = 0; i < NV; ++i) {
+        const int v = lane + i * G;
+        if (ok[r] && v < nvec) {
+          xr[r][i] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(x + row * cols) + v);
+          gr[r][i] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(dy + row * cols) + v);
+        } else {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            xr[r][i][e] = 0;
+            gr[r][i][e] = 0;
+          }
         }
       }
     }
-    float xf[NV][VEC], gf[NV][VEC];
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      P::unpack(xr[i], xf[i]);
-      P::unpack(gr[i], gf[i]);
-    }
-    float mean = 0.f;
-    if (LN) {
-      float sum = 0.f;
+    for (int r = 0; r < R; ++r) {
+      const int64_t row = row0 + r * GPB + gid;
+      float xf[NV][VEC], gf[NV][VEC];
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        P::unpack(xr[r][i], xf[i]);
+        P::unpack(gr[r][i], gf[i]);
+      }
+      float mean = 0.f;
+      if (LN) {
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) sum += xf[i][e];
+        mean = group_sum<G>(sum) * inv_cols;
+      }
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const bool live = (lane + i * G) < nvec;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          xf[i][e] = LN ? (live ? xf[i][e] - mean : 0.f) : xf[i][e];  // centred from here on
+          ss += xf[i][e] * xf[i][e];
+        }
+      }
+      const float rstd = rsqrtf(group_sum<G>(ss) * inv_cols + eps);
+      float sg = 0.f, sgx = 0.f;
 #pragma unroll
       for (int i = 0; i < NV; ++i)
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) sum += xf[i][e];
-      mean = group_sum<G>(sum) * inv_cols;
-    }
-    float ss = 0.f;
+        for (int e = 0; e < VEC; ++e) {
+          xf[i][e] *= rstd;  // x_hat
+          const float g = gf[i][e] * wf[i][e];
+          sg += g;
+          sgx += g * xf[i][e];
+        }
+      const float mean_gx = group_sum<G>(sgx) * inv_cols;
+      const float mean_g = LN ? group_sum<G>(sg) * inv_cols : 0.f;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const bool live = (lane + i * G) < nvec;
+      for (int i = 0; i < NV; ++i) {
+        const int v = lane + i * G;
+        float of[VEC];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        xf[i][e] = LN ? (live ? xf[i][e] - mean : 0.f) : xf[i][e];  // centred from here on
-        ss += xf[i][e] * xf[i][e];
+        for (int e = 0; e < VEC; ++e) {
+          of[e] = rstd * (gf[i][e] * wf[i][e] - mean_g - xf[i][e] * mean_gx);
+          dwacc[i][e] += gf[i][e] * xf[i][e];  // rows beyond the end contribute zeros
+          if (LN) dbacc[LN ? i : 0][e] += gf[i][e];
+        }
+        if (ok[r] && v < nvec) __builtin_nontemporal_store(P::pack(of), reinterpret_cast<vec_t*>(dx + row * cols) + v);
       }
-    }
-    const float rstd = rsqrtf(group_sum<G>(ss) * inv_cols + eps);
-    float sg = 0.f, sgx = 0.f;
-#pragma unroll
-    for (int i = 0; i < NV; ++i)
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        xf[i][e] *= rstd;  // x_hat
-        const float g = gf[i][e] * wf[i][e];
-        sg += g;
-        sgx += g * xf[i][e];
-      }
-    const float mean_gx = group_sum<G>(sgx) * inv_cols;
-    const float mean_g = LN ? group_sum<G>(sg) * inv_cols : 0.f;
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const int v = lane + i * G;
-      float of[VEC];
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        of[e] = rstd * (gf[i][e] * wf[i][e] - mean_g - xf[i][e] * mean_gx);
-        dwacc[i][e] += gf[i][e] * xf[i][e];  // rows beyond the end contribute zeros
-        if (LN) dbacc[LN ? i : 0][e] += gf[i][e];
-      }
-      if (ok && v < nvec) __builtin_nontemporal_store(P::pack(of), reinterpret_cast<vec_t*>(dx + row * cols) + v);
     }
   }
 
@@ -403,17 +414,31 @@ __global__ __launch_bounds__(kBlock) void norm_bwd_rows_vec_kernel(const T* __re
   }
 }
 
-// dw[c] (and db[c]) = sum over the workgroups' partial rows, in workgroup order.
+// dw[c] (and db[c]) = sum over the workgroups' partial rows in a fixed order: a workgroup owns 16 columns, thread
+// (column, slice) adds the partial rows slice, slice + 16, ... and the 16 slice sums of a column are added in slice order.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void norm_bwd_reduce_kernel(const float* __restrict__ partial, int nblocks, int cols,
                                                                   int parts, T* __restrict__ dw, T* __restrict__ db) {
-  const int c = blockIdx.x * kBlock + threadIdx.x;
-  if (c >= cols) return;
+  constexpr int CPB = 16, SLICES = kBlock / CPB;
+  __shared__ float red[SLICES][CPB];
+  const int cl = threadIdx.x % CPB, slice = threadIdx.x / CPB;
+  const int c = blockIdx.x * CPB + cl;
   for (int part = 0; part < parts; ++part) {
     float sum = 0.f;
-    for (int b = 0; b < nblocks; ++b) sum += partial[(static_cast<int64_t>(b) * parts + part) * cols + c];
-    T* dst = part == 0 ? dw : db;
-    if (dst != nullptr) dst[c] = static_cast<T>(sum);
+    if (c < cols) {
+#pragma unroll 4
+      for (int b = slice; b < nblocks; b += SLICES) sum += partial[(static_cast<int64_t>(b) * parts + part) * cols + c];
+    }
+    __syncthreads();
+    red[slice][cl] = sum;
+    __syncthreads();
+    if (slice == 0 && c < cols) {
+      float total = 0.f;
+#pragma unroll
+      for (int sl = 0; sl < SLICES; ++sl) total += red[sl][cl];
+      T* dst = part == 0 ? dw : db;
+      if (dst != nullptr) dst[c] = static_cast<T>(total);
+    }
   }
 }
 
@@ -434,7 +459,8 @@ int dispatch_bwd(const void* xv, const void* wv, const void* dyv, void* dxv, voi
   const int nvec = cols / VEC;
   int G = 1;
   while (G < nvec && G < kWave) G *= 2;
-  const int gpb = kBlock / G;
+  const int rows_in_flight = nvec <= kWave ? 4 : (nvec <= 2 * kWave ? 2 : 1);  // R of the kernel
+  const int gpb = (kBlock / G) * rows_in_flight;
   int64_t nblocks = (rows + gpb - 1) / gpb;
   if (nblocks > kBwdMaxBlocks) nblocks = kBwdMaxBlocks;
   const int parts = LN ? 2 : 1;
@@ -462,7 +488,7 @@ int dispatch_bwd(const void* xv, const void* wv, const void* dyv, void* dxv, voi
       }
   }
 #undef TAAC_BWD_CASE
-  hipLaunchKernelGGL((norm_bwd_reduce_kernel<T>), dim3((cols + kBlock - 1) / kBlock), dim3(kBlock), 0, s, workspace,
+  hipLaunchKernelGGL((norm_bwd_reduce_kernel<T>), dim3((cols + 15) / 16), dim3(kBlock), 0, s, workspace,
                      static_cast<int>(nblocks), cols, parts, static_cast<T*>(dwv), static_cast<T*>(dbv));
   return TAAC_OK;
 }
