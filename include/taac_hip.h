@@ -159,6 +159,32 @@ int taac_mask_pack_bits(const void* mask, int64_t rows, int32_t cols, uint32_t* 
 int taac_mask_block_any(const uint32_t* struct_bits, int32_t Tq, int32_t Tk, uint8_t* block_any, void* stream);
 
 /*
+ * Training pair of taac_flash_attn_fwd (key-length mask, optional causal triangle; head_dim <= 64 for the backward).
+ * taac_flash_attn_train_fwd additionally writes lse: fp32 [B, H, Tq] contiguous, the natural-log sum of exp of the
+ * scaled scores of every query row (-inf for rows without a visible key and for padded rows).
+ * taac_flash_attn_bwd: with P = exp(q k^T / sqrt(d) - lse) on the visible pairs and D_i = sum_d o[i, d] dout[i, d],
+ *   dv = P^T dout,  dS = P * (dout v^T - D) / sqrt(d),  dq = dS k,  dk = dS^T q
+ * for the same mask arguments as the forward. o is the forward's output, dout its gradient (logical (B, H, Tq, d) like
+ * q, own strides); dq / dk / dv have the logical shapes of q / k / v and their own element strides (same rules as the
+ * forward). delta: workspace, fp32 [B, H, Tq]. With zero_padded_queries the padded query rows carry no gradient (dq
+ * rows are zero); gradients of keys at or beyond key_lengths[b] are zero. Every output element has one writer and a
+ * fixed summation order (two kernels, each recomputing the scores), so results are reproducible run to run.
+ * Replaces: the TileLang training forward (accelerators/attention/kernels/tilelang.py:287-390) and backward
+ * preprocess + backward kernels (:405-435, 598-699), which accumulate dq with floating-point atomics.
+ */
+int taac_flash_attn_train_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths, void* o,
+                              float* lse, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                              const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
+                              const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype,
+                              void* stream);
+int taac_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,
+                        const int32_t* key_lengths, void* dq, void* dk, void* dv, float* delta, int32_t B, int32_t H,
+                        int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
+                        const int64_t v_strides[4], const int64_t o_strides[4], const int64_t do_strides[4],
+                        const int64_t dq_strides[4], const int64_t dk_strides[4], const int64_t dv_strides[4],
+                        int is_causal, int zero_padded_queries, int dtype, void* stream);
+
+/*
  * Dense layer, bf16 storage / bf16 MFMA / fp32 accumulation: out = epilogue(a @ w^T + bias).
  * a: [M, K] with row stride lda (elements); w: [N, K] contiguous (torch nn.Linear layout, [out, in]);
  * bias: [N] bf16 or NULL; residual: [M, N_out] with row stride ldo or NULL; out: [M, N_out] with row stride ldo,

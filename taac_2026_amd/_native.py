@@ -93,6 +93,18 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "taac_mask_pack_bits": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p]),
     "taac_mask_block_any": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
+    "taac_flash_attn_train_fwd": (
+        c_int,
+        [c_void_p] * 6 + [c_int32, c_int32, c_int32, c_int32, c_int32]
+        + [ctypes.POINTER(c_int64)] * 4
+        + [c_int, c_int, c_int, c_void_p],
+    ),
+    "taac_flash_attn_bwd": (
+        c_int,
+        [c_void_p] * 11 + [c_int32, c_int32, c_int32, c_int32, c_int32]
+        + [ctypes.POINTER(c_int64)] * 8
+        + [c_int, c_int, c_int, c_void_p],
+    ),
     "taac_linear_bf16": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_int, c_int,

@@ -358,6 +358,59 @@ def hip_flash_attention_kernel(
     return out
 
 
+def _dense_like(t: torch.Tensor) -> torch.Tensor:
+    out = torch.empty_like(t)
+    if out.stride(-1) != 1 or any(s % 8 for s in out.stride()[:-1]):
+        out = torch.empty(t.shape, dtype=t.dtype, device=t.device)
+    return out
+
+
+class _HipFlashAttentionFunction(torch.autograd.Function):
+    """Training path (key-length mask, optional causal triangle): the forward also saves the log-sum-exp of every query
+    row, the backward runs the two HIP backward kernels (the role of the reference's TileLang training functions,
+    flash_attention.py:397-525)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, key_lengths, is_causal: bool, zero_padded_queries: bool):
+        library = _native.load_library()
+        q, k, v = _kernel_view(q), _kernel_view(k), _kernel_view(v)
+        out = _dense_like(q)
+        batch, heads, query_len, head_dim = q.shape
+        lse = torch.empty(batch, heads, query_len, dtype=torch.float32, device=q.device)
+        status = library.taac_flash_attn_train_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), out.data_ptr(), lse.data_ptr(),
+            batch, heads, query_len, k.shape[2], head_dim,
+            _native.Int64x4(*q.stride()), _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()),
+            _native.Int64x4(*out.stride()), int(bool(is_causal)), int(bool(zero_padded_queries)),
+            _native.dtype_code(q.dtype), _native.current_stream(q.device),
+        )
+        _native.check(status, "flash_attention")
+        ctx.save_for_backward(q, k, v, out, lse, *(() if key_lengths is None else (key_lengths,)))
+        ctx.has_lengths = key_lengths is not None
+        ctx.flags = (bool(is_causal), bool(zero_padded_queries))
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        library = _native.load_library()
+        saved = ctx.saved_tensors
+        q, k, v, out, lse = saved[:5]
+        key_lengths = saved[5] if ctx.has_lengths else None
+        grad_out = _kernel_view(grad_out)
+        dq, dk, dv = _dense_like(q), _dense_like(k), _dense_like(v)
+        delta = torch.empty_like(lse)
+        batch, heads, query_len, head_dim = q.shape
+        strides = [_native.Int64x4(*t.stride()) for t in (q, k, v, out, grad_out, dq, dk, dv)]
+        status = library.taac_flash_attn_bwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), grad_out.data_ptr(), lse.data_ptr(),
+            _native.ptr(key_lengths), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(),
+            batch, heads, query_len, k.shape[2], head_dim, *strides, int(ctx.flags[0]), int(ctx.flags[1]),
+            _native.dtype_code(q.dtype), _native.current_stream(q.device),
+        )
+        _native.check(status, "flash_attention backward")
+        return dq, dk, dv, None, None, None
+
+
 def flash_attention(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -395,7 +448,11 @@ def flash_attention(
     del block_m, block_n, num_stages, threads
     q, k, v = _normalize_flash_attention_inputs(q, k, v)
     _resolve_flash_attention_backend(q, backend, dropout_p=dropout_p, training=training)
-    require_inference("hip flash_attention", q, k, v)
+    needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v))
+    if needs_grad and (structured_mask is not None or q_row_scale is not None or k_row_scale is not None
+                       or q_col_scale is not None or q.dtype == torch.float32):
+        raise RuntimeError("hip flash_attention backward covers bf16 / fp16 inputs under key-length and causal masks only; "
+                           "call it under torch.no_grad() for structured masks, row factors or fp32 inputs")
     if structured_mask is not None and attn_mask is not None:
         raise ValueError("flash_attention takes either attn_mask or structured_mask, not both")
     if key_lengths is not None:
@@ -416,6 +473,15 @@ def flash_attention(
     if q.dtype == torch.float32:
         q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
     lengths = plan.key_lengths if (plan.key_lengths is not None and (attn_mask is not None or key_lengths is not None)) else None
+    if needs_grad:
+        if structured_mask is not None:
+            raise RuntimeError("hip flash_attention backward does not cover structured masks")
+        if lengths is not None:
+            lengths = lengths.to(torch.int32).contiguous()
+        output = _HipFlashAttentionFunction.apply(q, k, v, lengths, plan.is_causal, zero_padded_queries)
+        if plan.query_self_mask is not None:
+            output = torch.where(plan.query_self_mask[:, None, :, None], v, output)
+        return output
     output = hip_flash_attention_kernel(
         q, k, v, lengths, is_causal=plan.is_causal, zero_padded_queries=zero_padded_queries,
         q_row_scale=q_row_scale, k_row_scale=k_row_scale, q_col_scale=q_col_scale, structured_mask=structured_mask,

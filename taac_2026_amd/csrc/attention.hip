@@ -45,6 +45,7 @@ struct AttnParams {
   const uint32_t* valid_bits;   // [B][wpr] or null (every key valid)
   const uint32_t* self_bits;    // [B][ceil(Tq / 32)] or null: flagged query rows return their own value row
   const uint8_t* block_any;     // [nqc][nkc]: some query of the 128-row block sees some key of the 64-key chunk
+  float* lse;                   // [B, H, Tq] log-sum-exp of the scaled scores (natural log) for the backward, or null
   int32_t wpr;                  // words per row of struct_bits / valid_bits = ceil(Tk / 32)
   int32_t nkc;                  // key chunks = ceil(Tk / 64)
   int32_t B, H, Tq, Tk, d;
@@ -140,6 +141,10 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 
   if (q_begin >= q_valid) {
     // Whole block lies in the padding: zero-fill its rows, or leave them alone.
+    if (p.lse != nullptr) {
+      for (int idx = tid; idx < kQB; idx += kThreads)
+        if (q_begin + idx < p.Tq) p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Tq + q_begin + idx] = -INFINITY;
+    }
     if (p.zero_pad == 2) return;
     const int c8n = p.d / 8;
     for (int idx = tid; idx < kQB * c8n; idx += kThreads) {
@@ -399,6 +404,9 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   // ---- finalise: O / l (0 for rows in the padding), transpose through a wavefront-private LDS tile, 16-byte stores --
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
   const float fin = (qi < q_valid) ? inv : 0.f;
+  if (p.lse != nullptr && hh == 0 && qi < p.Tq)
+    p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Tq + qi] =
+        (qi < q_valid && l_run > 0.f) ? (m_run * c + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f : -INFINITY;
   __syncthreads();  // every wavefront is done with sK / sVt: the buffer now holds the output tiles
   uint8_t* tile = smem + wave * (32 * OROW);
 #pragma unroll
@@ -498,7 +506,7 @@ struct MaskArgs {
 
 int attention_entry(const char* name, const void* q, const void* k, const void* v, const int32_t* key_lengths,
                     const MaskArgs& mask, const float* q_row_scale, const float* k_row_scale, const float* q_col_scale,
-                    void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
+                    float* lse, void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
                     const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4], int is_causal,
                     int zero_padded_queries, int dtype, void* stream) {
   if (mask.struct_bits != nullptr) {
@@ -538,6 +546,7 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   p.q_row_scale = q_row_scale;
   p.k_row_scale = k_row_scale;
   p.q_col_scale = q_col_scale;
+  p.lse = lse;
   p.struct_bits = mask.struct_bits;
   p.valid_bits = mask.valid_bits;
   p.self_bits = mask.self_bits;
@@ -578,8 +587,8 @@ extern "C" int taac_flash_attn_fwd(const void* q, const void* k, const void* v, 
                                    const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
                                    const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype,
                                    void* stream) {
-  return taac::attention_entry("taac_flash_attn_fwd", q, k, v, key_lengths, taac::MaskArgs{}, nullptr, nullptr, nullptr, o,
-                               B, H, Tq, Tk, d,
+  return taac::attention_entry("taac_flash_attn_fwd", q, k, v, key_lengths, taac::MaskArgs{}, nullptr, nullptr, nullptr,
+                               nullptr, o, B, H, Tq, Tk, d,
                                q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries, dtype, stream);
 }
 
@@ -591,7 +600,7 @@ extern "C" int taac_flash_attn_scaled_fwd(const void* q, const void* k, const vo
                                           const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype,
                                           void* stream) {
   return taac::attention_entry("taac_flash_attn_scaled_fwd", q, k, v, key_lengths, taac::MaskArgs{}, q_row_scale,
-                               k_row_scale, q_col_scale, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries,
+                               k_row_scale, q_col_scale, nullptr, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries,
                                dtype, stream);
 }
 
@@ -611,7 +620,7 @@ extern "C" int taac_flash_attn_masked_fwd(const void* q, const void* k, const vo
   mask.valid_bits = valid_bits;
   mask.self_bits = self_bits;
   return taac::attention_entry("taac_flash_attn_masked_fwd", q, k, v, key_lengths, mask, q_row_scale, k_row_scale,
-                               q_col_scale, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, 0,
+                               q_col_scale, nullptr, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, 0,
                                zero_padded_queries, dtype, stream);
 }
 
@@ -639,4 +648,15 @@ extern "C" int taac_mask_block_any(const uint32_t* struct_bits, int32_t Tq, int3
   hipLaunchKernelGGL(block_any_kernel, dim3(nqc * nkc), dim3(kWave), 0, as_stream(stream), struct_bits, Tq,
                      (Tk + 31) / 32, nkc, block_any);
   return check_launch(name);
+}
+
+extern "C" int taac_flash_attn_train_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
+                                         void* o, float* lse, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                                         const int64_t q_strides[4], const int64_t k_strides[4],
+                                         const int64_t v_strides[4], const int64_t o_strides[4], int is_causal,
+                                         int zero_padded_queries, int dtype, void* stream) {
+  if (!lse) return taac::set_error(TAAC_ERR_INVALID_VALUE, "taac_flash_attn_train_fwd: lse must be given");
+  return taac::attention_entry("taac_flash_attn_train_fwd", q, k, v, key_lengths, taac::MaskArgs{}, nullptr, nullptr,
+                               nullptr, lse, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, is_causal,
+                               zero_padded_queries, dtype, stream);
 }

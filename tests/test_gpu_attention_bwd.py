@@ -1,0 +1,82 @@
+"""GPU parity: attention training forward (log-sum-exp) and backward (through the C ABI) against torch autograd of the
+CPU oracle's closed form evaluated in float64."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from oracle import reference as oracle
+from taac_2026_amd.api import flash_attention, scaled_dot_product_attention
+
+pytestmark = pytest.mark.gpu
+
+# Gradient tolerance of the reference's GPU tests for 16-bit attention (tests/gpu/infrastructure/accelerators/
+# test_tilelang_ops_cuda.py:98-141): 3e-2.
+TOL = dict(rtol=3e-2, atol=3e-2)
+
+
+def _reference(q, k, v, lengths, grad_out, *, causal, zero_pad):
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    out = oracle.attention(qr, kr, vr, lengths, is_causal=causal, zero_padded_queries=zero_pad)
+    out.backward(grad_out.double())
+    return out.detach(), qr.grad, kr.grad, vr.grad
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tokens,dim", [(50, 32), (130, 64), (300, 32), (64, 16), (257, 64), (33, 8)])
+@pytest.mark.parametrize("causal,zero_pad", [(False, False), (False, True), (True, False)])
+def test_backward_matches_autograd_of_the_oracle(device, dtype, tokens, dim, causal, zero_pad):
+    batch, heads = 4, 2
+    g = torch.Generator().manual_seed(tokens * 7 + dim)
+    q, k, v = (torch.randn(batch, heads, tokens, dim, generator=g).to(dtype) for _ in range(3))
+    grad_out = torch.randn(batch, heads, tokens, dim, generator=g).to(dtype)
+    lengths = torch.tensor([tokens, 1, max(1, tokens // 2), max(1, tokens - 3)], dtype=torch.int32)
+    ref_out, ref_dq, ref_dk, ref_dv = _reference(q, k, v, lengths, grad_out, causal=causal, zero_pad=zero_pad)
+    qd, kd, vd = (t.to(device).requires_grad_(True) for t in (q, k, v))
+    out = flash_attention(qd, kd, vd, key_lengths=lengths.to(device), is_causal=causal, zero_padded_queries=zero_pad)
+    out.backward(grad_out.to(device))
+    torch.testing.assert_close(out.detach().cpu().double(), ref_out, rtol=2e-2, atol=2e-2)
+    for got, ref, name in ((qd.grad, ref_dq, "dq"), (kd.grad, ref_dk, "dk"), (vd.grad, ref_dv, "dv")):
+        assert got.dtype == dtype and got.shape == ref.shape
+        torch.testing.assert_close(got.cpu().double(), ref, msg=lambda m, n=name: f"{n}: {m}", **TOL)
+    # keys in the padding receive exactly zero gradient
+    for b in range(batch):
+        if lengths[b] < tokens:
+            assert kd.grad[b, :, int(lengths[b]):].abs().max().item() == 0.0
+            assert vd.grad[b, :, int(lengths[b]):].abs().max().item() == 0.0
+            if zero_pad:
+                assert qd.grad[b, :, int(lengths[b]):].abs().max().item() == 0.0
+
+
+def test_backward_is_reproducible_and_reads_the_projection_layout(device):
+    """(B, T, D) projections that are chunk views of one packed tensor, as the model packages produce them; two runs
+    give bit-identical gradients (one writer per element, fixed summation order)."""
+    batch, tokens, heads, dim = 3, 200, 4, 32
+    g = torch.Generator().manual_seed(0)
+    packed = torch.randn(batch, tokens, 3 * heads * dim, generator=g).to(torch.bfloat16)
+    lengths = torch.tensor([200, 77, 130], dtype=torch.int32)
+    grad_out = torch.randn(batch, tokens, heads * dim, generator=g).to(torch.bfloat16)
+    grads = []
+    for _ in range(2):
+        pd = packed.to(device).requires_grad_(True)
+        q, k, v = pd.chunk(3, dim=-1)
+        out = scaled_dot_product_attention(q, k, v, num_heads=heads, attn_mask=None, dropout_p=0.0, training=True,
+                                           key_lengths=lengths.to(device), zero_padded_queries=True)
+        out.backward(grad_out.to(device))
+        grads.append(pd.grad.clone())
+    assert torch.equal(grads[0], grads[1])
+    pr = packed.double().requires_grad_(True)
+    q, k, v = pr.chunk(3, dim=-1)
+    ref = oracle.scaled_dot_product_attention(q, k, v, num_heads=heads, key_lengths=lengths, zero_padded_queries=True)
+    ref.backward(grad_out.double())
+    torch.testing.assert_close(grads[0].cpu().double(), pr.grad, **TOL)
+
+
+def test_backward_envelope(device):
+    q = torch.randn(1, 1, 16, 128, device=device, dtype=torch.bfloat16, requires_grad=True)
+    with pytest.raises(RuntimeError, match="head_dim"):
+        flash_attention(q, q, q).sum().backward()
+    q32 = torch.randn(1, 1, 16, 32, device=device, requires_grad=True)
+    with pytest.raises(RuntimeError, match="backward covers"):
+        flash_attention(q32, q32, q32)
