@@ -182,6 +182,18 @@ def _operator_figures(device, iters: int) -> dict:
             "frac_mfma": useful / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS,
             "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS,
         }
+    # attention backward at the same shape (training forward + both backward kernels timed together, minus the training
+    # forward alone); algorithmic FLOPs: five products against the forward's two
+    qg, kg, vg = (t.clone().requires_grad_(True) for t in (qd, kd, vd))
+    go = torch.randn(q.shape, generator=torch.Generator().manual_seed(9)).to(torch.bfloat16).to(device)
+    fwd = lambda: flash_attention(qg, kg, vg, key_lengths=ld, zero_padded_queries=True)  # noqa: E731
+    ms_fwd = _event_ms(fwd, iters, 3)
+    ms_both = _event_ms(lambda: torch.autograd.grad(fwd(), (qg, kg, vg), go), iters, 3)
+    ms_bwd = ms_both - ms_fwd
+    figures["attention_bwd_bf16_B2048_H4_T256_d64"] = {
+        "training_fwd_ms": ms_fwd, "bwd_ms": ms_bwd, "useful_tflops": 2.5 * useful / ms_bwd / 1e9,
+        "frac_mfma": 2.5 * useful / ms_bwd / 1e9 / MFMA_BF16_PEAK_TFLOPS,
+    }
     return figures
 
 
