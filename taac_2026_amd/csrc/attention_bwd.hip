@@ -75,45 +75,78 @@ __device__ __forceinline__ uint32_t pack2(T lo, T hi) {
 // Position of row k (0..15 inside a 16-row group) in a transposed, permuted LDS row: accumulator order.
 __device__ __forceinline__ int vt_pos16(int k) { return ((k >> 2) & 1) * 8 + (k >> 3) * 4 + (k & 3); }
 
-// Stages rows [row0, row0 + kChunk) of a [rows, d] matrix (row stride `stride`) as dst[row][DP + 8]; rows at or beyond
-// row_end and features at or beyond d are zeros.
+// Staging of a chunk of streamed rows is split into a register fetch and an LDS commit, so that the global loads of
+// chunk c + 1 are in flight while chunk c is being consumed.
+//
+// RowStager: rows [row0, row0 + kChunk) of a [rows, d] matrix (row stride `stride`) -> dst[row][DP + 8]; rows at or
+// beyond row_end and features at or beyond d are zeros.
 template <typename T, int DP>
-__device__ __forceinline__ void stage_rows(const T* __restrict__ base, int64_t stride, int row0, int row_end, int d,
-                                           T* __restrict__ dst, int tid) {
+struct RowStager {
   typedef typename Vec8<T>::type vec_t;
-  constexpr int C8 = DP / 8, STR = DP + 8;
-  vec_t zero;
+  static constexpr int C8 = DP / 8, STR = DP + 8;
+  static constexpr int N = (kChunk * C8 + kThreads - 1) / kThreads;
+  vec_t reg[N];
+  __device__ __forceinline__ void fetch(const T* __restrict__ base, int64_t stride, int row0, int row_end, int d, int tid) {
 #pragma unroll
-  for (int e = 0; e < 8; ++e) zero[e] = static_cast<T>(0.f);
-  for (int idx = tid; idx < kChunk * C8; idx += kThreads) {
-    const int r = idx / C8, c8 = idx % C8;
-    const int row = row0 + r;
-    const vec_t val = (row < row_end && c8 * 8 < d) ? *reinterpret_cast<const vec_t*>(base + row * stride + c8 * 8) : zero;
-    *reinterpret_cast<vec_t*>(&dst[r * STR + c8 * 8]) = val;
+    for (int i = 0; i < N; ++i) {
+      const int idx = tid + i * kThreads;
+      const int row = row0 + idx / C8, c8 = idx % C8;
+      if (idx < kChunk * C8 && row < row_end && c8 * 8 < d) {
+        reg[i] = *reinterpret_cast<const vec_t*>(base + row * stride + c8 * 8);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) reg[i][e] = static_cast<T>(0.f);
+      }
+    }
   }
-}
+  __device__ __forceinline__ void commit(T* __restrict__ dst, int tid) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int idx = tid + i * kThreads;
+      if (idx < kChunk * C8) *reinterpret_cast<vec_t*>(&dst[(idx / C8) * STR + (idx % C8) * 8]) = reg[i];
+    }
+  }
+};
 
-// Stages the same rows transposed: dst[feature][pos(row)] with row stride kChunk + 8, the rows of every 16-row group in
-// accumulator order, two neighbouring rows per 32-bit store.
+// TransStager: the same rows transposed, dst[feature][pos(row)] with row stride kChunk + 8, the rows of every 16-row
+// group in accumulator order, two neighbouring rows per 32-bit store.
 template <typename T, int DP>
-__device__ __forceinline__ void stage_transposed(const T* __restrict__ base, int64_t stride, int row0, int row_end, int d,
-                                                 T* __restrict__ dst, int tid) {
+struct TransStager {
   typedef typename Vec8<T>::type vec_t;
-  constexpr int C8 = DP / 8, STR = kChunk + 8;
-  vec_t zero;
+  static constexpr int C8 = DP / 8, STR = kChunk + 8;
+  static constexpr int N = ((kChunk / 2) * C8 + kThreads - 1) / kThreads;
+  vec_t reg[N][2];
+  __device__ __forceinline__ void fetch(const T* __restrict__ base, int64_t stride, int row0, int row_end, int d, int tid) {
 #pragma unroll
-  for (int e = 0; e < 8; ++e) zero[e] = static_cast<T>(0.f);
-  for (int idx = tid; idx < (kChunk / 2) * C8; idx += kThreads) {
-    const int r0 = 2 * (idx / C8), c8 = idx % C8;
-    const int row = row0 + r0;
-    const bool col_ok = c8 * 8 < d;
-    const vec_t a = (col_ok && row < row_end) ? *reinterpret_cast<const vec_t*>(base + row * stride + c8 * 8) : zero;
-    const vec_t b = (col_ok && row + 1 < row_end) ? *reinterpret_cast<const vec_t*>(base + (row + 1) * stride + c8 * 8) : zero;
-    const int pos = (r0 & ~15) + vt_pos16(r0 & 15);  // even; row r0 + 1 lands at pos + 1
+    for (int i = 0; i < N; ++i) {
+      const int idx = tid + i * kThreads;
+      const int row = row0 + 2 * (idx / C8), c8 = idx % C8;
+      const bool ok = idx < (kChunk / 2) * C8 && c8 * 8 < d;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) *reinterpret_cast<uint32_t*>(&dst[(c8 * 8 + e) * STR + pos]) = pack2<T>(a[e], b[e]);
+      for (int r = 0; r < 2; ++r) {
+        if (ok && row + r < row_end) {
+          reg[i][r] = *reinterpret_cast<const vec_t*>(base + (row + r) * stride + c8 * 8);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) reg[i][r][e] = static_cast<T>(0.f);
+        }
+      }
+    }
   }
-}
+  __device__ __forceinline__ void commit(T* __restrict__ dst, int tid) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int idx = tid + i * kThreads;
+      if (idx < (kChunk / 2) * C8) {
+        const int r0 = 2 * (idx / C8), c8 = idx % C8;
+        const int pos = (r0 & ~15) + vt_pos16(r0 & 15);  // even; row r0 + 1 lands at pos + 1
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          *reinterpret_cast<uint32_t*>(&dst[(c8 * 8 + e) * STR + pos]) = pack2<T>(reg[i][0][e], reg[i][1][e]);
+      }
+    }
+  }
+};
 
 // Owned rows as B-operand fragments: lane (l32, hh) holds features 16 s + 8 hh .. + 7 of row `row` (zeros when !ok).
 template <typename T, int DP>
@@ -194,6 +227,9 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnBwdPara
   const bool q_ok = qi < q_valid;
   int kv_end = len;
   if (p.causal) kv_end = kv_end < q_begin + kOwn ? kv_end : q_begin + kOwn;
+  if (q_begin >= q_valid) kv_end = 0;  // a block of padded queries: zero gradient, no key is staged
+  // A wavefront whose 32 queries all lie in the padding only helps staging.
+  const bool wave_active = q_begin + wave * 32 < q_valid;
 
   vec_t qf[KSTEPS], dof[KSTEPS], of[KSTEPS];
   load_owned<T, DP>(qb, p.qs[2], qi, q_ok, p.d, hh, qf);
@@ -207,10 +243,11 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnBwdPara
   delta = pair_sum(delta);
   const int64_t stat = (static_cast<int64_t>(b) * p.H + h) * p.Tq + qi;
   if (hh == 0 && qi < p.Tq) p.delta[stat] = delta;
-  float lse = q_ok ? p.lse[stat] : -INFINITY;
-  const bool row_live = q_ok && lse > -INFINITY;
-  const float c = p.scale * 1.4426950408889634f;                // scores -> base-2 exponent
-  const float lse2 = row_live ? lse * 1.4426950408889634f : 0.f;
+  const float lse = q_ok ? p.lse[stat] : -INFINITY;
+  const float c = p.scale * 1.4426950408889634f;  // scores -> base-2 exponent
+  // a row without a visible key (or in the padding) gets +inf: exp2(x - inf) = 0 switches it off without a select
+  const float lse2 = lse > -INFINITY ? lse * 1.4426950408889634f : INFINITY;
+  const float delta_scaled = delta * p.scale;
 
   f32x16 dqacc[MB];
 #pragma unroll
@@ -218,15 +255,25 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnBwdPara
 #pragma unroll
     for (int j = 0; j < 16; ++j) dqacc[mb][j] = 0.f;
 
+  RowStager<T, DP> k_rows, v_rows;
+  TransStager<T, DP> k_cols;
+  auto fetch = [&](int kc0) {
+    k_rows.fetch(kb, p.ks[2], kc0, kv_end, p.d, tid);
+    v_rows.fetch(vb, p.vs[2], kc0, kv_end, p.d, tid);
+    k_cols.fetch(kb, p.ks[2], kc0, kv_end, p.d, tid);
+  };
+  if (kv_end > 0) fetch(0);
   for (int kc0 = 0; kc0 < kv_end; kc0 += kChunk) {
-    if (kc0 > 0) __syncthreads();
-    stage_rows<T, DP>(kb, p.ks[2], kc0, kv_end, p.d, sK, tid);
-    stage_rows<T, DP>(vb, p.vs[2], kc0, kv_end, p.d, sV, tid);
-    stage_transposed<T, DP>(kb, p.ks[2], kc0, kv_end, p.d, sKt, tid);
+    if (kc0 > 0) __syncthreads();  // every wavefront is done reading the previous chunk
+    k_rows.commit(sK, tid);
+    v_rows.commit(sV, tid);
+    k_cols.commit(sKt, tid);
     __syncthreads();
+    if (kc0 + kChunk < kv_end) fetch(kc0 + kChunk);
 #pragma unroll
     for (int kt = 0; kt < kChunk / 32; ++kt) {
-      if (kc0 + kt * 32 >= kv_end) continue;  // workgroup-uniform
+      if (kc0 + kt * 32 >= kv_end || !wave_active) continue;  // wavefront-uniform
+      if (p.causal && kc0 + kt * 32 > q_begin + wave * 32 + 31) continue;  // every key of the tile lies after the queries
       f32x16 sacc, dpacc;
 #pragma unroll
       for (int j = 0; j < 16; ++j) sacc[j] = dpacc[j] = 0.f;
@@ -237,13 +284,21 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnBwdPara
         sacc = Mfma32<T>::run(ka, qf[s], sacc);
         dpacc = Mfma32<T>::run(va, dof[s], dpacc);
       }
+      // only a tile that crosses the end of the keys or the causal diagonal needs per-element tests
+      const int k_tile = kc0 + kt * 32;
+      const bool tail = k_tile + 32 > kv_end || (p.causal && k_tile + 31 > q_begin + wave * 32);
+      if (tail) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const int key = k_tile + (j / 4) * 8 + hh * 4 + (j % 4);
+          if (key >= kv_end || (p.causal && key > qi)) sacc[j] = -INFINITY;
+        }
+      }
       vec_t dsb[2];
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
-        const int key = kc0 + kt * 32 + (j / 4) * 8 + hh * 4 + (j % 4);
-        const bool visible = row_live && key < kv_end && (!p.causal || key <= qi);
-        const float prob = visible ? __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -lse2)) : 0.f;
-        dsb[j / 8][j % 8] = static_cast<T>(prob * (dpacc[j] - delta) * p.scale);
+        const float prob = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -lse2));
+        dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -delta_scaled));
       }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
@@ -271,7 +326,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkv_kernel(const AttnBwdPar
   T* sQt = sDo + kChunk * RSTR;         // [DP][TSTR]
   T* sDot = sQt + DP * TSTR;            // [DP][TSTR]
   float* sLse = reinterpret_cast<float*>(sDot + DP * TSTR);  // [kChunk] base-2 log-sum-exp (+inf: row carries nothing)
-  float* sDelta = sLse + kChunk;                             // [kChunk]
+  float* sDelta = sLse + kChunk;                             // [kChunk] D_i / sqrt(d)
 
   const int blk = static_cast<int>(blockIdx.x % p.nblk);
   const int bh = static_cast<int>(blockIdx.x / p.nblk);
@@ -308,22 +363,37 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkv_kernel(const AttnBwdPar
   const int64_t stat0 = (static_cast<int64_t>(b) * p.H + h) * p.Tq;
 
   if (k_begin < len) {  // workgroup-uniform: a block of padding keys gets zero gradients without any work
-    for (int qc0 = q_start; qc0 < q_valid; qc0 += kChunk) {
-      if (qc0 > q_start) __syncthreads();
-      stage_rows<T, DP>(qb, p.qs[2], qc0, q_valid, p.d, sQ, tid);
-      stage_rows<T, DP>(dob, p.dos[2], qc0, q_valid, p.d, sDo, tid);
-      stage_transposed<T, DP>(qb, p.qs[2], qc0, q_valid, p.d, sQt, tid);
-      stage_transposed<T, DP>(dob, p.dos[2], qc0, q_valid, p.d, sDot, tid);
+    RowStager<T, DP> q_rows, do_rows;
+    TransStager<T, DP> q_cols, do_cols;
+    float lse_next = -INFINITY, delta_next = 0.f;
+    auto fetch = [&](int qc0) {
+      q_rows.fetch(qb, p.qs[2], qc0, q_valid, p.d, tid);
+      do_rows.fetch(dob, p.dos[2], qc0, q_valid, p.d, tid);
+      q_cols.fetch(qb, p.qs[2], qc0, q_valid, p.d, tid);
+      do_cols.fetch(dob, p.dos[2], qc0, q_valid, p.d, tid);
       if (tid < kChunk) {
         const int qi = qc0 + tid;
-        const float lse = qi < q_valid ? p.lse[stat0 + qi] : -INFINITY;
-        sLse[tid] = lse > -INFINITY ? lse * 1.4426950408889634f : INFINITY;  // exp2(x - inf) = 0
-        sDelta[tid] = qi < q_valid ? p.delta[stat0 + qi] : 0.f;
+        lse_next = qi < q_valid ? p.lse[stat0 + qi] : -INFINITY;
+        delta_next = qi < q_valid ? p.delta[stat0 + qi] : 0.f;
+      }
+    };
+    if (q_start < q_valid) fetch(q_start);
+    for (int qc0 = q_start; qc0 < q_valid; qc0 += kChunk) {
+      if (qc0 > q_start) __syncthreads();  // every wavefront is done reading the previous chunk
+      q_rows.commit(sQ, tid);
+      do_rows.commit(sDo, tid);
+      q_cols.commit(sQt, tid);
+      do_cols.commit(sDot, tid);
+      if (tid < kChunk) {
+        sLse[tid] = lse_next > -INFINITY ? lse_next * 1.4426950408889634f : INFINITY;  // exp2(x - inf) = 0
+        sDelta[tid] = delta_next * p.scale;
       }
       __syncthreads();
+      if (qc0 + kChunk < q_valid) fetch(qc0 + kChunk);
 #pragma unroll
       for (int qt = 0; qt < kChunk / 32; ++qt) {
-        if (qc0 + qt * 32 >= q_valid) continue;  // workgroup-uniform
+        if (qc0 + qt * 32 >= q_valid || k_begin + wave * 32 >= len) continue;  // wavefront-uniform
+        if (p.causal && qc0 + qt * 32 + 31 < k_begin + wave * 32) continue;     // every query of the tile lies before the keys
         f32x16 sacc, dpacc;
 #pragma unroll
         for (int j = 0; j < 16; ++j) sacc[j] = dpacc[j] = 0.f;
@@ -334,20 +404,23 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkv_kernel(const AttnBwdPar
           sacc = Mfma32<T>::run(qa, kf[s], sacc);
           dpacc = Mfma32<T>::run(da, vf[s], dpacc);
         }
+        // a padded key of the lane, or (causal) a query before the key: the score becomes -inf, the probability 0;
+        // only a tile that crosses the causal diagonal needs per-element tests
+        const bool diagonal = p.causal && qc0 + qt * 32 < k_begin + wave * 32 + 31;
         vec_t pb[2], dsb[2];
 #pragma unroll
         for (int jq = 0; jq < 4; ++jq) {
           const int r0 = qt * 32 + jq * 8 + hh * 4;  // four consecutive queries of the chunk
           const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sLse[r0]);
-          const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[r0]);
+          const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[r0]);  // already times 1 / sqrt(d)
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int j = jq * 4 + e;
-            const int qi = qc0 + r0 + e;
-            const bool visible = k_ok && (!p.causal || kj <= qi);
-            const float prob = visible ? __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -l4[e])) : 0.f;
+            float sc = k_ok ? sacc[j] : -INFINITY;
+            if (diagonal && kj > qc0 + r0 + e) sc = -INFINITY;
+            const float prob = __builtin_amdgcn_exp2f(fmaf(sc, c, -l4[e]));
             pb[j / 8][j % 8] = static_cast<T>(prob);
-            dsb[j / 8][j % 8] = static_cast<T>(prob * (dpacc[j] - d4[e]) * p.scale);
+            dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -d4[e]));
           }
         }
 #pragma unroll
