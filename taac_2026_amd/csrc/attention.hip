@@ -83,6 +83,28 @@ __device__ __forceinline__ float pair_sum(float v) {
   return __builtin_bit_cast(float, static_cast<uint32_t>(r[0])) + __builtin_bit_cast(float, static_cast<uint32_t>(r[1]));
 }
 
+// acc + the sum of the eight rounded values of a fragment: four two-element dot products with (1, 1).
+__device__ __forceinline__ float frag_sum(const bf16x8& v, float acc) {
+  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+  const bf16x2 ones = {static_cast<__bf16>(1.0f), static_cast<__bf16>(1.0f)};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const bf16x2 pair = {v[2 * i], v[2 * i + 1]};
+    acc = __builtin_amdgcn_fdot2_f32_bf16(pair, ones, acc, false);
+  }
+  return acc;
+}
+__device__ __forceinline__ float frag_sum(const f16x8& v, float acc) {
+  typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2;
+  const f16x2 ones = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const f16x2 pair = {v[2 * i], v[2 * i + 1]};
+    acc = __builtin_amdgcn_fdot2(pair, ones, acc, false);
+  }
+  return acc;
+}
+
 template <typename T>
 __device__ __forceinline__ uint32_t pack2(T lo, T hi) {
   return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, lo)) |
@@ -351,15 +373,15 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
       for (int kt = 0; kt < NT; ++kt) {
         float pr[16];
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          pr[j] = __builtin_amdgcn_exp2f(fmaf(sacc[kt][j], c, mc));
-          rs += pr[j];
-        }
+        for (int j = 0; j < 16; ++j) pr[j] = __builtin_amdgcn_exp2f(fmaf(sacc[kt][j], c, mc));
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           pb[kt][0][e] = static_cast<T>(pr[e]);
           pb[kt][1][e] = static_cast<T>(pr[8 + e]);
         }
+        // the normaliser sums the rounded probabilities, the values the second product uses: two per instruction
+        rs = frag_sum(pb[kt][0], rs);
+        rs = frag_sum(pb[kt][1], rs);
       }
       rs = pair_sum(rs);
       l_run = l_run * alpha + rs;
