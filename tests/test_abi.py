@@ -74,6 +74,85 @@ def test_host_side_argument_validation_without_gpu():
     assert status == _native.TAAC_ERR_UNSUPPORTED
 
 
+def test_host_side_validation_of_the_widened_entry_points_without_gpu():
+    library = _native.load_library()
+    fake = ctypes.c_void_p(256)
+    bf16, f32 = _native.TAAC_BF16, _native.TAAC_F32
+    invalid, unsupported, ok = _native.TAAC_ERR_INVALID_VALUE, _native.TAAC_ERR_UNSUPPORTED, _native.TAAC_OK
+
+    # query / key normalisation + rotation
+    def qk(**kw):
+        a = dict(q=fake, k=fake, ld_in=64, q_out=fake, k_out=fake, ld_out=64, rows=8, tps=4, d_model=64, heads=4,
+                 qw=fake, kw=fake, eps=1e-6, cos_sin=None, row_index=None, n_rows=None, dtype=bf16)
+        a.update(kw)
+        return library.taac_qk_norm_rope_fwd(a["q"], a["k"], a["ld_in"], a["q_out"], a["k_out"], a["ld_out"], a["rows"],
+                                             a["tps"], a["d_model"], a["heads"], a["qw"], a["kw"], a["eps"],
+                                             a["cos_sin"], a["row_index"], a["n_rows"], a["dtype"], None)
+
+    assert qk(heads=5) == invalid and b"divisible" in library.taac_last_error()
+    assert qk(kw=None) == invalid and b"come together" in library.taac_last_error()
+    assert qk(qw=None, kw=None) == invalid and b"neither" in library.taac_last_error()
+    assert qk(ld_in=32) == invalid and b"row stride" in library.taac_last_error()
+    assert qk(row_index=fake) == invalid
+    assert qk(rows=0) == ok
+    assert qk(dtype=9) == invalid
+
+    # embedding bag
+    def bag(**kw):
+        a = dict(weight=fake, n=16, e=8, values=fake, i64=0, bags=4, size=2, out=fake, count=None, dtype=f32)
+        a.update(kw)
+        return library.taac_embedding_bag_mean_fwd(a["weight"], a["n"], a["e"], a["values"], a["i64"], a["bags"],
+                                                   a["size"], a["out"], a["count"], a["dtype"], None)
+
+    assert bag(n=0) == invalid
+    assert bag(values=None) == invalid and b"null" in library.taac_last_error()
+    assert bag(bags=0) == ok
+    assert bag(dtype=9) == invalid
+
+    # normalisation backward: workspace size, too-small workspace, width outside the envelope
+    floats = library.taac_norm_bwd_workspace_floats(1000, 256, 0)
+    assert floats > 0 and library.taac_norm_bwd_workspace_floats(1000, 256, 1) == 2 * floats
+    assert library.taac_rmsnorm_bwd(fake, fake, fake, fake, fake, fake, 255, 1000, 256, 1e-6, bf16, None) == invalid
+    assert b"workspace" in library.taac_last_error()
+    assert library.taac_rmsnorm_bwd(fake, fake, fake, fake, fake, fake, 1 << 30, 8, 260, 1e-6, bf16, None) == unsupported
+    assert library.taac_layernorm_bwd(fake, fake, fake, None, fake, fake, fake, 1 << 30, 8, 256, 1e-5, bf16, None) == invalid
+
+    # attention with structured masks, the training forward and the backward
+    strides = _native.Int64x4(2048, 16, 128, 1)
+
+    def masked(**kw):
+        a = dict(lengths=None, struct=fake, any=fake, valid=None, self=None, tq=64, tk=64, d=16, zero=0, dtype=bf16)
+        a.update(kw)
+        return library.taac_flash_attn_masked_fwd(fake, fake, fake, a["lengths"], a["struct"], a["any"], a["valid"],
+                                                  a["self"], None, None, None, fake, 1, 8, a["tq"], a["tk"], a["d"],
+                                                  strides, strides, strides, strides, a["zero"], a["dtype"], None)
+
+    assert masked(struct=None) == invalid and b"struct_bits" in library.taac_last_error()
+    assert masked(any=None) == invalid and b"block_any" in library.taac_last_error()
+    assert masked(tk=4096 + 64) == unsupported and b"at most" in library.taac_last_error()
+    assert masked(self=fake, tk=128) == invalid and b"self rows" in library.taac_last_error()
+    assert masked(d=12) == unsupported
+    assert library.taac_mask_pack_bits(None, 4, 4, fake, None) == invalid
+    assert library.taac_mask_pack_bits(fake, 0, 4, fake, None) == ok
+    assert library.taac_mask_block_any(fake, 0, 4, fake, None) == invalid
+    status = library.taac_flash_attn_train_fwd(fake, fake, fake, None, fake, None, 1, 8, 64, 64, 16, strides, strides,
+                                               strides, strides, 0, 0, bf16, None)
+    assert status == invalid and b"lse" in library.taac_last_error()
+
+    def backward(**kw):
+        a = dict(lse=fake, delta=fake, tq=64, tk=64, d=16, zero=0, dtype=bf16)
+        a.update(kw)
+        return library.taac_flash_attn_bwd(fake, fake, fake, fake, fake, a["lse"], None, fake, fake, fake, a["delta"],
+                                           1, 8, a["tq"], a["tk"], a["d"], strides, strides, strides, strides, strides,
+                                           strides, strides, strides, 0, a["zero"], a["dtype"], None)
+
+    assert backward(d=72) == unsupported and b"head_dim" in library.taac_last_error()
+    assert backward(dtype=f32) == invalid
+    assert backward(lse=None) == invalid and b"null" in library.taac_last_error()
+    assert backward(tk=0) == unsupported
+    assert backward(tq=64, tk=128, zero=1) == invalid
+
+
 def test_status_mapping_to_python_exceptions():
     library = _native.load_library()
     fake = ctypes.c_void_p(256)
