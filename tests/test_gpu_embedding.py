@@ -25,6 +25,20 @@ def test_reference_fixture(device):
     assert got[1].abs().max().item() == 0.0
 
 
+def test_golden_vectors(device):
+    """The committed pure-Python float64 evaluations (tests/golden/qk_rope_embedding_small.json)."""
+    import json
+    from pathlib import Path
+
+    golden = json.loads((Path(__file__).resolve().parent / "golden" / "qk_rope_embedding_small.json").read_text())
+    for case in golden["bags"]:
+        weight, values = torch.tensor(case["weight"]), torch.tensor(case["values"])
+        for index_dtype in (torch.int32, torch.int64):
+            with torch.no_grad():
+                got = embedding_bag_mean(weight.to(device), values.to(index_dtype).to(device)).cpu()
+            torch.testing.assert_close(got.double(), torch.tensor(case["out"], dtype=torch.float64), rtol=1e-6, atol=1e-7)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("index_dtype", [torch.int32, torch.int64])
 @pytest.mark.parametrize("vocab,dim,bags,bag_size", [(1000, 64, 257, 4), (50, 8, 33, 1), (4096, 128, 100, 7),

@@ -228,3 +228,29 @@ def test_qkv_projection_skips_padded_rows(device):
     mask = valid.to(device)
     assert torch.equal(got[mask], full[mask]) and torch.equal(sq[mask], fq[mask]) and torch.equal(sk[mask], fk[mask])
     assert torch.count_nonzero(got[~mask]) == 0 and torch.isfinite(sq).all() and torch.isfinite(sk).all()
+
+
+def test_golden_vectors(device):
+    """The committed pure-Python float64 evaluations (tests/golden/qk_rope_embedding_small.json) against the float32
+    kernel; an odd head width (its last feature is not rotated) is reported by the host layer, not served."""
+    import json
+    from pathlib import Path
+
+    golden = json.loads((Path(__file__).resolve().parent / "golden" / "qk_rope_embedding_small.json").read_text())
+    served = 0
+    for case in golden["qk"]:
+        q, k = torch.tensor(case["query"]), torch.tensor(case["key"])
+        weights = [None if case[name] is None else torch.tensor(case[name]).to(device) for name in ("query_weight", "key_weight")]
+        head_dim = q.shape[-1] // case["num_heads"]
+        call = lambda: qk_norm_rope(q.to(device), k.to(device), *weights, num_heads=case["num_heads"], eps=case["eps"],
+                                    rope_base=case["rope_base"])
+        if case["rope_base"] is not None and head_dim % 4 != 0:
+            with pytest.raises((RuntimeError, ValueError), match="multiples of|must be even"):
+                call()
+            continue
+        with torch.no_grad():
+            got_q, got_k = call()
+        torch.testing.assert_close(got_q.cpu().double(), torch.tensor(case["query_out"], dtype=torch.float64), rtol=2e-5, atol=2e-6)
+        torch.testing.assert_close(got_k.cpu().double(), torch.tensor(case["key_out"], dtype=torch.float64), rtol=2e-5, atol=2e-6)
+        served += 1
+    assert served == 3

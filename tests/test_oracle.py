@@ -454,3 +454,25 @@ def test_embedding_bag_mean_reference_fixture_and_brute_force():
     np.testing.assert_allclose(got.double().numpy(), expected, rtol=1e-6, atol=1e-7)
     assert got[1].abs().max().item() == 0.0
     torch.testing.assert_close(got[2], (2 * weight[3] + weight[7]) / 3)
+
+
+# ---- pure-Python golden vectors of the widened operators ----------------------------------------------------------------
+
+
+def test_qk_norm_rope_and_embedding_bag_golden_vectors():
+    """tests/golden/qk_rope_embedding_small.json holds float64 pure-Python evaluations (make_widened_golden.py) of the
+    query / key normalisation + rotation and of the bag mean; the oracle's float32 routes reproduce them."""
+    golden = json.loads((GOLDEN / "qk_rope_embedding_small.json").read_text())
+    for case in golden["qk"]:
+        q, k = torch.tensor(case["query"]), torch.tensor(case["key"])
+        wq = None if case["query_weight"] is None else torch.tensor(case["query_weight"])
+        wk = None if case["key_weight"] is None else torch.tensor(case["key_weight"])
+        for fp32 in (False, True):
+            got_q, got_k = oracle.qk_norm_rope(q, k, wq, wk, num_heads=case["num_heads"], eps=case["eps"],
+                                               rope_base=case["rope_base"], fp32=fp32)
+            np.testing.assert_allclose(got_q.double().numpy(), np.array(case["query_out"]), rtol=2e-5, atol=2e-6)
+            np.testing.assert_allclose(got_k.double().numpy(), np.array(case["key_out"]), rtol=2e-5, atol=2e-6)
+    for case in golden["bags"]:
+        weight, values = torch.tensor(case["weight"]), torch.tensor(case["values"])
+        for route in (oracle.embedding_bag_mean, oracle.embedding_bag_mean_closed_form):
+            np.testing.assert_allclose(route(weight, values).double().numpy(), np.array(case["out"]), rtol=1e-6, atol=1e-7)
