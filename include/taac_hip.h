@@ -219,6 +219,25 @@ int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_weight, flo
                         int gate_first, const int32_t* rows, const int32_t* n_rows, void* stream);
 
 /*
+ * Attention output projection + residual and the feed-forward half of a block in one kernel:
+ *   x1  = residual + (attn @ w_out^T + out_bias)
+ *   out = x1 + down( silu(g) * u ) + b_down,   g, u = chunk2( up( norm_weight ? rmsnorm(x1, norm_weight, eps) : x1 ) )
+ * attn: [M, D] bf16 attention output (row stride ld_attn); residual: [M, D] block input (row stride ldr, required);
+ * out: [M, D] (row stride ldo), may alias residual, not attn. packed_out_weights: blob of taac_linear_pack_weights for
+ * the [D, D] projection; packed_ffn_weights: blob of taac_ffn_pack_weights with gate_first = 1 (both required);
+ * out_bias / b_up / b_down may be NULL. x1 is rounded to bf16 as the reference's residual stream is, but is never
+ * written to memory: it stays in the accumulators of the down projection, so the final sum x1 + down + b_down is
+ * rounded once (the two-kernel route rounds down + b_down first). D must be 128 or 256, F a multiple of 32.
+ * rows / n_rows: as in taac_swiglu_ffn_fwd.
+ * Replaces: attention.out + residual add and ffn_norm + SwiGLUFeedForward.forward + residual add of
+ * UnifiedInteractionBlock.forward (experiments/symbiosis/backbone.py:47, 64-67).
+ */
+int taac_attn_out_ffn_fwd(const void* attn, int64_t ld_attn, const void* out_bias, const void* packed_out_weights,
+                          const void* residual, int64_t ldr, const void* norm_weight, float eps, const void* b_up,
+                          const void* b_down, const void* packed_ffn_weights, void* out, int64_t ldo, int64_t M,
+                          int32_t D, int32_t F, const int32_t* rows, const int32_t* n_rows, void* stream);
+
+/*
  * Fused [RMSNorm ->] dense layer [-> + residual] with the token rows held in registers:
  *   out = (residual ? residual : 0) + (norm_weight ? rmsnorm(x, norm_weight, eps) : x) @ w^T + bias
  * x: [M, K] bf16; w: [N, K]; bias: [N] or NULL; residual / out: [M, N]; packed_weights: NULL or the blob written by

@@ -21,6 +21,7 @@ from taac_2026_amd.accelerators.embedding import (
 )
 from taac_2026_amd.accelerators.linear import (
     amax,
+    attention_out_ffn,
     linear,
     linear_fp8,
     norm_linear,
@@ -46,6 +47,7 @@ from taac_2026_amd.accelerators.tensor_validation import (
 )
 
 __all__ = [
+    "attention_out_ffn",
     "FlashAttentionMaskPlan",
     "StructuredAttentionMask",
     "_plan_tilelang_flash_attention_mask",

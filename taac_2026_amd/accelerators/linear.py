@@ -282,6 +282,59 @@ def swiglu_ffn(
     return out.reshape(shape)
 
 
+def attention_out_ffn(
+    attn: torch.Tensor,
+    out_weight: torch.Tensor,
+    out_bias: torch.Tensor | None,
+    residual: torch.Tensor,
+    up_weight: torch.Tensor,
+    up_bias: torch.Tensor | None,
+    down_weight: torch.Tensor,
+    down_bias: torch.Tensor | None,
+    *,
+    norm_weight: torch.Tensor | None = None,
+    eps: float = 1e-6,
+    token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Second half of a ``UnifiedInteractionBlock`` (experiments/symbiosis/backbone.py:47, 64-67) as ONE kernel:
+    ``x1 = residual + F.linear(attn, out_weight, out_bias)`` then ``x1 + down(silu(gate) * value)`` with
+    ``gate, value = up(rmsnorm(x1)).chunk(2, -1)``. ``x1`` never reaches memory. Model width 128 / 256 and a hidden
+    size that is a multiple of 32 only (``taac_attn_out_ffn_fwd``); ``token_rows`` / ``out`` as in :func:`swiglu_ffn`
+    (``out`` may be ``residual``)."""
+    name = "hip attention_out_ffn"
+    tensors = (attn, out_weight, out_bias, residual, up_weight, up_bias, down_weight, down_bias, norm_weight)
+    require_cuda_tensors(name, *tensors)
+    require_inference(name, *tensors)
+    _check_bf16(name, *tensors)
+    rows, shape = _as_rows(attn)
+    _check_weight(name, rows, out_weight, out_bias)
+    _check_weight(name, rows, up_weight, up_bias)
+    d_model, hidden = rows.shape[1], up_weight.shape[0] // 2
+    if out_weight.shape != (d_model, d_model) or up_weight.shape[0] % 2 != 0 or down_weight.shape != (d_model, hidden):
+        raise ValueError("attention_out_ffn expects out_weight [D, D], up_weight [2F, D] and down_weight [D, F]")
+    if residual.shape != shape:
+        raise ValueError("attention_out_ffn residual must have the shape of the attention output")
+    if not (_fused_width(d_model) and hidden % 32 == 0):
+        raise RuntimeError("attention_out_ffn: needs model width 128 / 256 and a hidden size that is a multiple of 32")
+    packed_out = _packed_cache.get((out_weight,), lambda: pack_linear_weight(out_weight))
+    packed_ffn = _packed_cache.get((up_weight, down_weight), lambda: pack_ffn_weights(up_weight, down_weight), variant=1)
+    res_rows = residual.reshape(-1, d_model)
+    if res_rows.stride(-1) != 1 or res_rows.stride(0) % 8 != 0:
+        res_rows = res_rows.contiguous()
+    index, count = _token_rows(name, token_rows, rows)
+    out = _output_rows(name, out, (rows.shape[0], d_model), index is not None, attn)
+    library = _native.load_library()
+    status = library.taac_attn_out_ffn_fwd(
+        rows.data_ptr(), rows.stride(0), _native.ptr(out_bias), packed_out.data_ptr(), res_rows.data_ptr(),
+        res_rows.stride(0), _native.ptr(norm_weight), float(eps), _native.ptr(up_bias), _native.ptr(down_bias),
+        packed_ffn.data_ptr(), out.data_ptr(), d_model, rows.shape[0], d_model, hidden, _native.ptr(index),
+        _native.ptr(count), _native.current_stream(attn.device),
+    )
+    _native.check(status, "attention_out_ffn")
+    return out.reshape(shape)
+
+
 def norm_linear(
     x: torch.Tensor,
     weight: torch.Tensor,

@@ -247,6 +247,8 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
 
   const bf16_t* cur = static_cast<const bf16_t*>(emb);
   int rc;
+  // TAAC_SPLIT_OUT_FFN: run the out projection and the feed-forward half as two kernels (tuning / comparison knob).
+  const bool split_out_ffn = getenv("TAAC_SPLIT_OUT_FFN") != nullptr;
   if (fused && n_blocks > 0) {
     // One launch re-lays the weights of all blocks into fragment order.
     std::vector<void*> pk(3 * static_cast<size_t>(n_blocks));
@@ -331,7 +333,12 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
                                          heads, T, T, dh, qkv_strides, qkv_strides, qkv_strides, o_strides, 0, rows ? 2 : 1,
                                          TAAC_BF16, stream)) != TAAC_OK)
       return rc;
-    if (fused) {
+    if (fused && !split_out_ffn) {
+      // out projection + residual and the whole feed-forward half in one kernel; the stream between them stays on chip
+      if ((rc = taac_attn_out_ffn_fwd(h, D, w.out_bias, pk_out, cur, D, w.ffn_norm_weight, eps, w.up_bias, w.down_bias,
+                                      pk_ffn, x_out, D, M, D, F, rows, n_rows, stream)) != TAAC_OK)
+        return rc;
+    } else if (fused) {
       if ((rc = taac_norm_linear_fwd(h, D, nullptr, eps, nullptr, w.out_bias, pk_out, cur, D, x, D, M, D, D, rows,
                                      n_rows, stream)) != TAAC_OK)
         return rc;

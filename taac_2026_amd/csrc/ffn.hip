@@ -61,6 +61,9 @@ struct TsParams {
   float* qk_sumsq;          // [qk_chunks][M] sum of squares of a token's 64 features of one chunk
   int32_t qk_chunks;        // leading 64-feature chunks that belong to the query and key projections
   int32_t head_dim, tokens_per_sample;
+  // Attention output projection in front of the FFN (x is then the attention output, residual the block input):
+  const bf16_t* w0;         // packed [D, D] projection (linear blob)
+  const bf16_t* b0;         // its bias [D] or null
 };
 
 __device__ __forceinline__ float silu_f(float v) {
@@ -308,9 +311,22 @@ __device__ __forceinline__ void load_residual(const bf16_t* residual, int64_t ld
 // rows, so ONE accumulator (16 registers per lane) holds g in registers 0..7 and u in registers 8..15 for the same
 // eight hidden units of the lane's token. silu(g) * u of those eight is exactly one B-operand fragment (k = 16) of
 // the down projection. Two chunks are staged and consumed per barrier.
-// LDS: [2 weight buffers][b_up (2F) | b_down (D) | norm weight (D)]; after the main loop the weight buffers hold the epilogue tiles.
+// LDS: [2 or 3 weight buffers][b_up (2F) | b_down (D) | norm weight (D) | OUTP: projection bias (D)]; after the main
+// loop the weight buffers hold the epilogue tiles.
+//
+// OUTP: the attention output projection and its residual run in front, in the same registers. p.x is then the
+// attention output A, p.residual the block input h, and the kernel evaluates
+//   x1 = bf16( bf16(A W0^T + b0) + h ),   out = bf16( x1 + down(silu(gate) * value) + b_down ),  gate, value = up(rmsnorm(x1))
+// The projection is formed transposed like the down projection, X1^T[feature, token] = W0 A^T, into the accumulators of
+// the final result; the packed W0 streams through weight buffers 1 and 2 one 64-feature chunk at a time. Bias and h
+// are added per chunk in accumulator order, the rounded x1 stays in the accumulators as the start value of the down
+// projection (so x1 never exists in memory and the final sum is rounded once), and its normalised copy is turned into
+// B-operand fragments with one half-wavefront exchange per register pair: the accumulator holds 4-feature runs of a
+// token per lane, a fragment needs 8-feature runs, and lanes l and l ^ 32 own the two halves of each run.
+// Replaces the out projection + residual and the feed-forward half of UnifiedInteractionBlock.forward
+// (experiments/symbiosis/backbone.py:60-67) in one pass over the tokens.
 // ------------------------------------------------------------------------------------------------------------------
-template <int D, int TT, int NWAVES, int CPB, bool DEFER>
+template <int D, int TT, int NWAVES, int CPB, bool DEFER, bool OUTP>
 __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_kernel(const TsParams p) {
   constexpr int kTokPerWg = NWAVES * 32 * TT;  // TT token tiles of 32 per wavefront
   constexpr int KS = D / 16;             // k-steps of the up projection = up fragments per chunk
@@ -391,10 +407,24 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
     }
   };
 
+  // OUTP: chunk c of the packed projection (2 * KS fragments) goes to weight buffer 1 + (c & 1).
+  [[maybe_unused]] auto stage_proj = [&](int c, int buf) {
+    constexpr int CF = 2 * KS, CFW = CF / NWAVES;
+    static_assert(CF % NWAVES == 0 && CF <= NFRAG, "a projection chunk is staged by all wavefronts into one buffer");
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    uint8_t* base = smem + buf * (NFRAG * kFrag) + wave * (CFW * kFrag);
+    const char* src = reinterpret_cast<const char*>(p.w0) + (static_cast<int64_t>(c) * CF + wave * CFW) * kFrag + ln * 16;
+#pragma unroll
+    for (int i = 0; i < CFW; ++i) lds_dma16(src + i * kFrag, base + i * kFrag);
+  };
+
   stage(0, 0);
+  if constexpr (OUTP) stage_proj(0, 1);
   stage_up_bias(p.b1, bias_lds, F, p.gate_first, tid, NWAVES * kWave);
   stage_bias(p.b2, bias_lds + 2 * F, D, tid, NWAVES * kWave);
   if (p.norm_w != nullptr) stage_bias(p.norm_w, bias_lds + 2 * F + D, D, tid, NWAVES * kWave);
+  if constexpr (OUTP) stage_bias(p.b0, bias_lds + 2 * F + 2 * D, D, tid, NWAVES * kWave);
 
   bf16x8 xf[TT][KS];
   if (active) load_token_rows<D, TT>(p, count, tok0, l32, hh, xf);
@@ -409,7 +439,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  if (active && p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + 2 * F + D, hh, xf);
+  if (!OUTP && active && p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + 2 * F + D, hh, xf);
 
   // One barrier step = CPB chunks = NFRAG fragments, consumed in their LDS order: per chunk KS up fragments, then MB
   // down fragments. Fragment reads run P fragments ahead of their MFMAs through a ring of P registers sets; the two
@@ -423,6 +453,105 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
   u32x4 ones_bits = {hh == 0 ? 0x3f80u : 0u, 0u, 0u, 0u};
   asm volatile("" : "+v"(ones_bits));
   const bf16x8 ones = __builtin_bit_cast(bf16x8, ones_bits);
+
+  if constexpr (OUTP) {
+    static_assert(DEFER, "the projection chunks use weight buffers 1 and 2");
+    constexpr int NCH = D / kNC;  // 64-feature chunks of the projection
+    constexpr int CF = 2 * KS;    // fragments of a chunk: (row block rb, k-step ks) at rb * KS + ks
+    const bf16_t* b0_lds = bias_lds + 2 * F + 2 * D;
+    float ss[TT];
+    const bf16_t* hrow[TT];
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+      ss[t] = 0.f;
+      hrow[t] = p.residual + token_row(p, count, tok0 + t * 32 + l32) * p.ldr + hh * 4;
+    }
+    static_for<NCH>([&](auto cc) {
+      constexpr int c = decltype(cc)::value;
+      // block input of this chunk's 64 features in accumulator order: piece rb*4 + jq = features rb*32 + jq*8 + hh*4 .. +3
+      bf16x4 hv[TT][8];
+      if (active) {
+#pragma unroll
+        for (int t = 0; t < TT; ++t)
+#pragma unroll
+          for (int q = 0; q < 8; ++q)
+            hv[t][q] = *reinterpret_cast<const bf16x4*>(hrow[t] + c * kNC + (q / 4) * 32 + (q % 4) * 8);
+      }
+      if constexpr (c + 1 < NCH) stage_proj(c + 1, 1 + ((c + 1) & 1));
+      if (active) {
+        const uint32_t wb0 = smem_off + (1 + (c & 1)) * (NFRAG * kFrag);
+        bf16x8 pring[P];
+        static_for<P>([&](auto ic) { lds_read_frag<decltype(ic)::value * kFrag>(pring[decltype(ic)::value], wb0); });
+        static_for<CF>([&](auto ic) {
+          constexpr int i = decltype(ic)::value;
+          constexpr int after = P - 1 < CF - 1 - i ? P - 1 : CF - 1 - i;
+          lds_wait_frag<after>(pring[i % P]);
+#pragma unroll
+          for (int t = 0; t < TT; ++t)
+            oacc[t][2 * c + i / KS] =
+                __builtin_amdgcn_mfma_f32_32x32x16_bf16(pring[i % P], xf[t][i % KS], oacc[t][2 * c + i / KS], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if constexpr (i + P < CF) lds_read_frag<(i + P) * kFrag>(pring[i % P], wb0);
+        });
+        // x1 = bf16( bf16(projection + b0) + h ), kept in the accumulators; sum of squares for the norm that follows
+        bf16x4 bv[8];
+        read_chunk_bias(b0_lds + c * kNC, hh, bv);
+#pragma unroll
+        for (int t = 0; t < TT; ++t)
+#pragma unroll
+          for (int q = 0; q < 8; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float a = oacc[t][2 * c + q / 4][(q % 4) * 4 + e];
+              const float lin = static_cast<float>(static_cast<bf16_t>(a + static_cast<float>(bv[q][e])));
+              const float x1 = static_cast<float>(static_cast<bf16_t>(lin + static_cast<float>(hv[t][q][e])));
+              oacc[t][2 * c + q / 4][(q % 4) * 4 + e] = x1;
+              ss[t] = fmaf(x1, x1, ss[t]);
+            }
+      }
+      // the next chunk has landed (and, with the first wait, the first step of the feed-forward weights)
+      vm_wait<0>();
+      __syncthreads();
+    });
+    if (active) {
+      // rmsnorm(x1) as B-operand fragments. k-step ks covers features 16*ks .. +15 = the 8-feature groups jq = 2*(ks%2)
+      // and jq + 1 of row block ks / 2; the lower half-wavefront needs all of the first group, the upper half all of
+      // the second, and each half holds 4 features of both.
+      const bf16_t* nw_lds = bias_lds + 2 * F + D;
+#pragma unroll
+      for (int t = 0; t < TT; ++t) {
+        const float scale = p.norm_w != nullptr ? rsqrtf(half_wave_pair_sum(ss[t]) * (1.0f / D) + p.eps) : 1.0f;
+        static_for<KS>([&](auto kc) {
+          constexpr int ks = decltype(kc)::value;
+          constexpr int mb = ks / 2, jq = 2 * (ks % 2);
+          bf16x4 lo, hi;
+          if (p.norm_w != nullptr) {
+            const bf16x4 wl = *reinterpret_cast<const bf16x4*>(nw_lds + mb * 32 + jq * 8 + hh * 4);
+            const bf16x4 wh = *reinterpret_cast<const bf16x4*>(nw_lds + mb * 32 + (jq + 1) * 8 + hh * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              lo[e] = static_cast<bf16_t>(oacc[t][mb][jq * 4 + e] * scale * static_cast<float>(wl[e]));
+              hi[e] = static_cast<bf16_t>(oacc[t][mb][(jq + 1) * 4 + e] * scale * static_cast<float>(wh[e]));
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              lo[e] = static_cast<bf16_t>(oacc[t][mb][jq * 4 + e]);
+              hi[e] = static_cast<bf16_t>(oacc[t][mb][(jq + 1) * 4 + e]);
+            }
+          }
+          const u32x2 ul = __builtin_bit_cast(u32x2, lo), uh = __builtin_bit_cast(u32x2, hi);
+          // swap: result 0 = (lower lanes of the first, lower lanes of the second), result 1 = the upper lanes
+          const auto r0 = __builtin_amdgcn_permlane32_swap(ul[0], uh[0], false, false);
+          const auto r1 = __builtin_amdgcn_permlane32_swap(ul[1], uh[1], false, false);
+          const u32x4 frag = {static_cast<uint32_t>(r0[0]), static_cast<uint32_t>(r1[0]), static_cast<uint32_t>(r0[1]),
+                              static_cast<uint32_t>(r1[1])};
+          xf[t][ks] = __builtin_bit_cast(bf16x8, frag);
+        });
+      }
+    }
+  }
+
   // DEFER: the down projection of a chunk is issued one chunk late, interleaved with the SiLU arithmetic of the next
   // chunk (MFMA j of the old chunk, then two gated values of the new one), so the matrix unit has work while the
   // wavefront evaluates the activation. hb is the gated hidden state whose down projection is pending; before the
@@ -564,12 +693,13 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 #pragma unroll
     for (int pr = 0; pr < MB / 2; ++pr) {  // 64 features at a time
       bf16x8 res[4];
-      if (p.residual != nullptr) load_residual(p.residual, p.ldr, prow, pr * 64, res, lane);
+      const bool add_residual = !OUTP && p.residual != nullptr;  // OUTP: the accumulators started from x1
+      if (add_residual) load_residual(p.residual, p.ldr, prow, pr * 64, res, lane);
       bf16x4 bv[8];
       read_chunk_bias(bdown_lds + pr * 64, hh, bv);
       tile_to_lds(tile, oacc[t][2 * pr], oacc[t][2 * pr + 1], bv, l32, hh);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      if (p.residual != nullptr)
+      if (add_residual)
         tile_to_global<true>(tile, p.out, p.ldo, prow, live, pr * 64, res, lane);
       else
         tile_to_global<false>(tile, p.out, p.ldo, prow, live, pr * 64, res, lane);
@@ -998,13 +1128,16 @@ extern "C" int taac_linear_pack_weights(const void* w, void* packed, int32_t N, 
   return check_launch(name);
 }
 
-extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w_up,
-                                   const void* b_up, const void* w_down, const void* b_down, const void* packed_weights,
-                                   const void* residual, int64_t ldr, void* out, int64_t ldo, int64_t M, int32_t D,
-                                   int32_t F, int gate_first, const int32_t* rows, const int32_t* n_rows,
-                                   void* stream) {
-  using namespace taac;
-  const char* name = "taac_swiglu_ffn_fwd";
+namespace taac {
+namespace {
+
+// Shared body of taac_swiglu_ffn_fwd and taac_attn_out_ffn_fwd (out_packed != null: the attention output projection
+// runs in front; x is then the attention output and residual the block input).
+int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias, const void* out_packed,
+              const void* norm_weight, float eps, const void* w_up, const void* b_up, const void* w_down,
+              const void* b_down, const void* packed_weights, const void* residual, int64_t ldr, void* out, int64_t ldo,
+              int64_t M, int32_t D, int32_t F, int gate_first, const int32_t* rows, const int32_t* n_rows, void* stream) {
+  const bool with_proj = out_packed != nullptr;
   if (M < 0 || D <= 0 || F <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, D and F > 0", name);
   if (D != 256 && D != 128)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: fused kernel is built for D = 128 or 256 (got %d)", name, D);
@@ -1015,13 +1148,19 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
   if (M == 0) return TAAC_OK;
   if (!x || !out || (!packed_weights && (!w_up || !w_down)))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
+  if (with_proj && (!residual || !packed_weights))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: the projection needs the block input and packed feed-forward weights", name);
   if ((rows == nullptr) != (n_rows == nullptr))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows and n_rows must be given together", name);
   if (rows && M > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: a row index covers at most 2^31 rows", name);
   if (!ptr_ok(x, 15) || !ptr_ok(w_up, 15) || !ptr_ok(w_down, 15) || !ptr_ok(out, 15) || !ptr_ok(residual, 15) ||
-      !ptr_ok(norm_weight, 15) || !ptr_ok(b_up, 15) || !ptr_ok(b_down, 15) || !ptr_ok(packed_weights, 15))
+      !ptr_ok(norm_weight, 15) || !ptr_ok(b_up, 15) || !ptr_ok(b_down, 15) || !ptr_ok(packed_weights, 15) ||
+      !ptr_ok(out_packed, 15) || !ptr_ok(out_bias, 15))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
-  if (static_cast<size_t>(2 * kCPB * (D / 16 + D / 32)) * kFrag + static_cast<size_t>(2 * F + 2 * D) * 2 > kMaxLdsBytes)
+  const int KS = D / 16, MB = D / 32;
+  const size_t bias_bytes = static_cast<size_t>(2 * F + (with_proj ? 3 : 2) * D) * 2;
+  const size_t buffer_bytes = static_cast<size_t>(kCPB * (KS + MB)) * kFrag;
+  if ((with_proj ? 3 : 2) * buffer_bytes + bias_bytes > kMaxLdsBytes)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: F=%d does not fit the LDS (limit %d bytes)", name, F, kMaxLdsBytes);
   TsParams p{};
   p.x = static_cast<const bf16_t*>(x);
@@ -1042,6 +1181,8 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
   p.packed = packed_weights ? 1 : 0;
   p.rows = rows;
   p.n_rows = n_rows;
+  p.w0 = static_cast<const bf16_t*>(out_packed);
+  p.b0 = static_cast<const bf16_t*>(out_bias);
   p.units = compute_units();
   if (p.units <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
   if (const char* cap = getenv("TAAC_TS_MAX_WORKGROUPS")) {  // test hook, as in the linear kernel
@@ -1049,21 +1190,47 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
     if (limit > 0 && limit < p.units) p.units = limit;
   }
   hipStream_t s = as_stream(stream);
-  const int KS = D / 16, MB = D / 32;
-  const size_t bias_bytes = static_cast<size_t>(2 * F + 2 * D) * 2;
-#define TAAC_FFN_LAUNCH(DD, TT, NW, CPB, DEFER)                                                               \
-  return launch_ts(swiglu_ffn_kernel<DD, TT, NW, CPB, DEFER>, p, NW * kWave, NW * 32 * TT,                   \
+#define TAAC_FFN_LAUNCH(DD, TT, NW, CPB, DEFER, OUTP)                                                        \
+  return launch_ts(swiglu_ffn_kernel<DD, TT, NW, CPB, DEFER, OUTP>, p, NW * kWave, NW * 32 * TT,             \
                    static_cast<size_t>((DEFER ? 3 : 2) * CPB * (KS + MB)) * kFrag + bias_bytes, s, name)
+  if (with_proj) {
+    if (D == 256) TAAC_FFN_LAUNCH(256, 1, 8, 2, true, true);
+    TAAC_FFN_LAUNCH(128, 1, 8, 2, true, true);
+  }
   int cfg = ts_config();
   // the deferred schedule needs a third weight buffer: fall back when a large F leaves no room for it next to the biases
-  if (cfg >= 1 && static_cast<size_t>(3 * kCPB * (KS + MB)) * kFrag + bias_bytes > kMaxLdsBytes) cfg = 0;
+  if (cfg >= 1 && 3 * buffer_bytes + bias_bytes > kMaxLdsBytes) cfg = 0;
   if (D == 256) {
-    if (cfg == 1) TAAC_FFN_LAUNCH(256, 1, 8, 2, true);
-    TAAC_FFN_LAUNCH(256, 1, 8, 2, false);
+    if (cfg == 1) TAAC_FFN_LAUNCH(256, 1, 8, 2, true, false);
+    TAAC_FFN_LAUNCH(256, 1, 8, 2, false, false);
   }
-  if (cfg == 1) TAAC_FFN_LAUNCH(128, 1, 8, 2, true);
-  TAAC_FFN_LAUNCH(128, 1, 8, 2, false);
+  if (cfg == 1) TAAC_FFN_LAUNCH(128, 1, 8, 2, true, false);
+  TAAC_FFN_LAUNCH(128, 1, 8, 2, false, false);
 #undef TAAC_FFN_LAUNCH
+}
+
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w_up,
+                                   const void* b_up, const void* w_down, const void* b_down, const void* packed_weights,
+                                   const void* residual, int64_t ldr, void* out, int64_t ldo, int64_t M, int32_t D,
+                                   int32_t F, int gate_first, const int32_t* rows, const int32_t* n_rows,
+                                   void* stream) {
+  return taac::ffn_entry("taac_swiglu_ffn_fwd", x, ldx, nullptr, nullptr, norm_weight, eps, w_up, b_up, w_down, b_down,
+                         packed_weights, residual, ldr, out, ldo, M, D, F, gate_first, rows, n_rows, stream);
+}
+
+extern "C" int taac_attn_out_ffn_fwd(const void* attn, int64_t ld_attn, const void* out_bias,
+                                     const void* packed_out_weights, const void* residual, int64_t ldr,
+                                     const void* norm_weight, float eps, const void* b_up, const void* b_down,
+                                     const void* packed_ffn_weights, void* out, int64_t ldo, int64_t M, int32_t D,
+                                     int32_t F, const int32_t* rows, const int32_t* n_rows, void* stream) {
+  const char* name = "taac_attn_out_ffn_fwd";
+  if (!packed_out_weights || !packed_ffn_weights)
+    return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: both weight sets must be packed", name);
+  return taac::ffn_entry(name, attn, ld_attn, out_bias, packed_out_weights, norm_weight, eps, nullptr, b_up, nullptr,
+                         b_down, packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, stream);
 }
 
 namespace taac {

@@ -117,6 +117,20 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
     assert library.taac_rmsnorm_bwd(fake, fake, fake, fake, fake, fake, 1 << 30, 8, 260, 1e-6, bf16, None) == unsupported
     assert library.taac_layernorm_bwd(fake, fake, fake, None, fake, fake, fake, 1 << 30, 8, 256, 1e-5, bf16, None) == invalid
 
+    # out projection + feed-forward half in one kernel: both weight sets packed, the block input required
+    def tail(**kw):
+        a = dict(packed_out=fake, residual=fake, packed_ffn=fake, d=256, f=64, m=8)
+        a.update(kw)
+        return library.taac_attn_out_ffn_fwd(fake, a["d"], None, a["packed_out"], a["residual"], a["d"], None, 1e-6, None,
+                                             None, a["packed_ffn"], fake, a["d"], a["m"], a["d"], a["f"], None, None, None)
+
+    assert tail(packed_out=None) == invalid and b"packed" in library.taac_last_error()
+    assert tail(packed_ffn=None) == invalid
+    assert tail(residual=None) == invalid and b"block input" in library.taac_last_error()
+    assert tail(d=192) == unsupported
+    assert tail(f=48) == unsupported
+    assert tail(m=0) == ok
+
     # attention with structured masks, the training forward and the backward
     strides = _native.Int64x4(2048, 16, 128, 1)
 

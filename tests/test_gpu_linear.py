@@ -230,6 +230,82 @@ def test_fused_swiglu_ffn(device, m, d, f, gate_first):
     torch.testing.assert_close(got.cpu().float(), ref_bf16.float(), rtol=4e-2, atol=4e-2)
 
 
+def _block_tail_inputs(m, d, f, seed):
+    g = torch.Generator().manual_seed(seed)
+    attn = torch.randn(m, d, generator=g).to(torch.bfloat16)
+    h = torch.randn(m, d, generator=g).to(torch.bfloat16)
+    nw = (1 + 0.1 * torch.randn(d, generator=g)).to(torch.bfloat16)
+    wo = (torch.randn(d, d, generator=g) * (1.0 / d) ** 0.5).to(torch.bfloat16)
+    bo = (0.1 * torch.randn(d, generator=g)).to(torch.bfloat16)
+    wu = (torch.randn(2 * f, d, generator=g) * (2.0 / (d + 2 * f)) ** 0.5).to(torch.bfloat16)
+    bu = (0.1 * torch.randn(2 * f, generator=g)).to(torch.bfloat16)
+    wd = (torch.randn(d, f, generator=g) * (2.0 / (d + f)) ** 0.5).to(torch.bfloat16)
+    bd = (0.1 * torch.randn(d, generator=g)).to(torch.bfloat16)
+    return attn, h, nw, wo, bo, wu, bu, wd, bd
+
+
+@pytest.mark.parametrize("m,d,f", [(1, 256, 32), (300, 256, 1024), (64, 128, 64), (1000, 256, 96), (257, 128, 256),
+                                   (2500, 256, 64)])
+@pytest.mark.parametrize("workgroups", [None, 3])
+def test_fused_attention_out_ffn(device, monkeypatch, m, d, f, workgroups):
+    """out projection + residual -> RMSNorm -> up -> SiLU-gate -> down -> + residual in one kernel, against the oracle's
+    pieces (dense layers evaluated in fp32 from the stored operands, the residual stream rounded to bf16 in between) and
+    against the two-kernel route of the same library."""
+    from taac_2026_amd.api import attention_out_ffn, norm_linear, swiglu_ffn
+
+    if workgroups is not None:
+        monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+    attn, h, nw, wo, bo, wu, bu, wd, bd = _block_tail_inputs(m, d, f, seed=m + d + f)
+    lin = F.linear(attn.float(), wo.float(), bo.float()).to(torch.bfloat16)
+    x1 = (lin.float() + h.float()).to(torch.bfloat16)
+    expected = x1.float() + oracle.swiglu_ffn(oracle.rms_norm_fp32(x1, nw).float(), wu.float(), bu.float(), wd.float(), bd.float())
+    to = lambda t: t.to(device)
+    with torch.no_grad():
+        got = attention_out_ffn(to(attn), to(wo), to(bo), to(h), to(wu), to(bu), to(wd), to(bd), norm_weight=to(nw))
+        mid = norm_linear(to(attn), to(wo), to(bo), residual=to(h))
+        two = swiglu_ffn(mid, to(wu), to(bu), to(wd), to(bd), residual=mid, norm_weight=to(nw))
+        bare = attention_out_ffn(to(attn), to(wo), None, to(h), to(wu), None, to(wd), None)
+    assert got.shape == attn.shape and got.dtype == torch.bfloat16
+    torch.testing.assert_close(got.cpu().float(), expected, **BF16_TOL)
+    # x1 is bit-identical on both routes; the one-kernel route rounds x1 + down + b_down once, the other twice
+    torch.testing.assert_close(got.cpu().float(), two.cpu().float(), rtol=2 ** -6, atol=2 ** -6)
+    x1_bare = (F.linear(attn.float(), wo.float()).to(torch.bfloat16).float() + h.float()).to(torch.bfloat16)
+    expected_bare = x1_bare.float() + oracle.swiglu_ffn(x1_bare.float(), wu.float(), None, wd.float(), None)
+    torch.testing.assert_close(bare.cpu().float(), expected_bare, **BF16_TOL)
+
+
+def test_fused_attention_out_ffn_in_place_on_valid_rows(device):
+    """With a row index and out = residual the kernel updates the residual stream in place: valid rows equal the dense
+    run bit for bit, padded rows (NaN in every operand here) are neither read nor written."""
+    from taac_2026_amd.api import attention_out_ffn, valid_rows
+
+    batch, tokens, d, f = 7, 150, 256, 64
+    lengths = torch.tensor([150, 0, 1, 77, 149, 33, 64], dtype=torch.int32)
+    valid = (torch.arange(tokens)[None, :] < lengths[:, None]).flatten()
+    attn, h, nw, wo, bo, wu, bu, wd, bd = _block_tail_inputs(batch * tokens, d, f, seed=5)
+    to = lambda t: t.to(device)
+    with torch.no_grad():
+        dense = attention_out_ffn(to(attn), to(wo), to(bo), to(h), to(wu), to(bu), to(wd), to(bd), norm_weight=to(nw))
+        attn_p, h_p = attn.clone(), h.clone()
+        attn_p[~valid] = float("nan")
+        h_p[~valid] = float("nan")
+        stream = to(h_p)
+        result = attention_out_ffn(to(attn_p), to(wo), to(bo), stream, to(wu), to(bu), to(wd), to(bd), norm_weight=to(nw),
+                                   token_rows=valid_rows(to(lengths), tokens), out=stream)
+    assert result.data_ptr() == stream.data_ptr()
+    assert torch.equal(result.cpu()[valid], dense.cpu()[valid])
+    assert torch.isnan(result.cpu()[~valid].float()).all()
+
+
+def test_fused_attention_out_ffn_rejects_other_shapes(device):
+    from taac_2026_amd.api import attention_out_ffn
+
+    attn, h, nw, wo, bo, wu, bu, wd, bd = _block_tail_inputs(8, 64, 32, seed=1)
+    to = lambda t: t.to(device)
+    with pytest.raises(RuntimeError, match="width 128 / 256"):
+        attention_out_ffn(to(attn), to(wo), to(bo), to(h), to(wu), to(bu), to(wd), to(bd))
+
+
 @pytest.mark.parametrize("m,k,n", [(1, 256, 64), (300, 256, 768), (64, 128, 256), (1000, 256, 256), (513, 128, 768)])
 def test_fused_norm_linear(device, m, k, n):
     from taac_2026_amd.api import norm_linear
