@@ -236,6 +236,40 @@ def _embedding_figures(device, iters: int) -> dict:
     return out
 
 
+def _readout_figures(inputs, device, iters: int) -> dict:
+    """The reference model's readout behind the backbone (final_norm -> cls | candidate | masked mean -> RMSNorm(3D) ->
+    Linear(3D, D) -> SiLU -> Linear(D, 1) -> sigmoid; experiments/symbiosis/model.py:215-222, pooling.py:16-32) as one
+    kernel at the headline batch. Algorithmic bytes: the valid token rows once plus the classifier weights."""
+    from oracle import reference as oracle
+    from taac_2026_amd.api import candidate_readout
+
+    B, T, D = inputs.emb.shape
+    g = torch.Generator().manual_seed(7)
+    bf = lambda t: t.to(torch.bfloat16)  # noqa: E731
+    x = bf(torch.randn(B, T, D, generator=g))
+    wt, wp = bf(1 + 0.1 * torch.randn(D, generator=g)), bf(1 + 0.1 * torch.randn(3 * D, generator=g))
+    w1, b1 = bf(torch.randn(D, 3 * D, generator=g) * (3 * D) ** -0.5), bf(0.1 * torch.randn(D, generator=g))
+    w2, b2 = bf(torch.randn(1, D, generator=g) * D ** -0.5), bf(torch.zeros(1))
+    lengths = inputs.key_lengths
+    to = lambda t: t.to(device)  # noqa: E731
+    kw = dict(cls_index=0, candidate_index=1, key_lengths=to(lengths), token_norm_weight=to(wt), pool_norm_weight=to(wp),
+              fc1_weight=to(w1), fc1_bias=to(b1), fc2_weight=to(w2), fc2_bias=to(b2), sigmoid=True)
+    dev_x = to(x)
+    with torch.no_grad():
+        got = candidate_readout(dev_x, **kw).cpu()
+        pick = slice(0, 32)
+        pad = torch.arange(T)[None, :] >= lengths[pick, None]
+        _, want = oracle.candidate_readout(x[pick], pad, cls_index=0, candidate_index=1, token_norm_weight=wt,
+                                           pool_norm_weight=wp, classifier=(w1, b1, w2, b2))
+        err = (got[pick] - torch.sigmoid(want)).abs().max().item()
+        if not err <= 2e-2:
+            raise SystemExit(f"accuracy gate of candidate_readout failed: {err}")
+        ms = _event_ms(lambda: candidate_readout(dev_x, **kw), iters, 3)
+    nbytes = float(lengths.clamp(0, T).sum().item()) * D * 2 + (3 * D * D + 5 * D) * 2
+    return {f"B{B}_T{T}_D{D}_hidden{D}": {"ms": ms, "algorithmic_bytes": nbytes, "gbs": nbytes / ms / 1e6,
+                                           "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS, "max_abs_err": err}}
+
+
 def _fp8_figures(inputs, device, iters: int) -> dict:
     """Configuration 5: the block's four dense layers with e4m3 operands (per-tensor scale amax / 448) over all
     M = B * T tokens, each checked on a slice of rows against the quantize -> matmul -> dequantize emulation."""
@@ -534,6 +568,7 @@ def main() -> None:
         line["operators"] = _operator_figures(device, iters=20)
         line["fp8_dense_layers"] = _fp8_figures(inputs, device, iters=10)
         line["embedding_bag_mean"] = _embedding_figures(device, iters=20)
+        line["candidate_readout"] = _readout_figures(inputs, device, iters=20)
         if not args.skip_widened:
             line["reference_layer_variants"] = _qk_variant_figures(device, B, max(args.steps // 2, 1))
             line["structured_masks"] = _structured_mask_figures(device, B, iters=10)

@@ -303,6 +303,29 @@ int taac_row_rstd(const float* qk_sumsq, int64_t M, int32_t d_model, float eps, 
                   const int32_t* n_rows, void* stream);
 
 /*
+ * Readout of the token backbone, one kernel:
+ *   n(t)  = token_norm_weight ? rmsnorm(tokens[b, t], token_norm_weight, eps) : tokens[b, t]
+ *   e[b]  = concat( n(cls_index), candidate_index >= 0 ? n(candidate_index) : 0, mean over the valid t of n(t) )
+ *   e[b]  = pool_norm_weight ? rmsnorm(e[b], pool_norm_weight, eps) : e[b]                       [3D]
+ *   z[b]  = fc2( silu( fc1(e[b]) ) ),  optionally sigmoid(z[b])                                  [actions]
+ * tokens: [B, T, D] bf16 contiguous. Valid tokens: t < key_lengths[b] (clamped to [0, T]) when key_lengths is given,
+ * bit t of valid_bits[b] (rows of ceil(T / 32) 32-bit words, as written by taac_mask_pack_bits from a [B, T] bool
+ * matrix, True = valid) when valid_bits is given, every token when both are NULL; the mean's divisor is clamped to
+ * >= 1 (modeling/sequence.py:54-60). The cls and candidate tokens are taken whether valid or not, as the reference
+ * does. fc1_weight: [hidden, 3D], fc2_weight: [actions, hidden] (torch nn.Linear layout), biases may be NULL;
+ * fc1_weight NULL skips the classifier. embedding_out: [B, 3D] bf16 or NULL; logits_out: [B, actions] fp32 (required
+ * with a classifier). D a multiple of 8, D and hidden at most 1024. Evaluated in fp32 from the stored operands.
+ * Replaces: final_norm + CandidateClsPooler.forward + classifier of PCVRSymbiosis (experiments/symbiosis/model.py:
+ * 215-222, 291, 309, 316-317; experiments/symbiosis/pooling.py:16-32).
+ */
+int taac_candidate_readout_fwd(const void* tokens, const int32_t* key_lengths, const uint32_t* valid_bits, int32_t B,
+                               int32_t T, int32_t D, int32_t cls_index, int32_t candidate_index,
+                               const void* token_norm_weight, const void* pool_norm_weight, float eps,
+                               const void* fc1_weight, const void* fc1_bias, int32_t hidden, const void* fc2_weight,
+                               const void* fc2_bias, int32_t actions, void* embedding_out, float* logits_out,
+                               int apply_sigmoid, void* stream);
+
+/*
  * Row index of the valid tokens of a padded batch: token t of sample b is valid iff t < key_lengths[b] (clamped to
  * [0, T]). Writes rows[i] = b * T + t for the valid tokens in increasing order, *n_rows = their number, and the
  * per-sample offsets (exclusive prefix sums of the lengths, B + 1 values, the last one equal to *n_rows) to

@@ -334,6 +334,34 @@ def qk_norm_rope(query: torch.Tensor, key: torch.Tensor, query_weight: torch.Ten
     return query.to(dtype), key.to(dtype)
 
 
+# ---- readout ---------------------------------------------------------------------------------------------------------------
+
+
+def candidate_readout(tokens: torch.Tensor, padding_mask: torch.Tensor | None, *, cls_index: int,
+                      candidate_index: int | None, token_norm_weight: torch.Tensor | None,
+                      pool_norm_weight: torch.Tensor | None, eps: float = 1e-6,
+                      classifier: tuple[torch.Tensor, torch.Tensor | None, torch.Tensor, torch.Tensor | None] | None = None,
+                      fp32: bool = True) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """``final_norm`` -> ``CandidateClsPooler.forward`` -> classifier of ``PCVRSymbiosis`` (experiments/symbiosis/
+    model.py:215-222, 291, 309, 316-317; experiments/symbiosis/pooling.py:24-32): the pieces are ``rms_norm``,
+    ``masked_mean`` and ``F.linear`` / ``F.silu`` above. ``fp32=True`` evaluates them in float32 from the stored operands
+    (the parity target of a fused kernel), ``fp32=False`` in the tensors' own dtype as the reference does.
+    Returns (pooled embedding (B, 3D), logits (B, actions) or None)."""
+    cast = (lambda t: None if t is None else t.float()) if fp32 else (lambda t: t)
+    x = cast(tokens)
+    if token_norm_weight is not None:
+        x = rms_norm(x, cast(token_norm_weight), eps)
+    cls_summary = x[:, cls_index, :]
+    candidate_summary = x[:, candidate_index, :] if candidate_index is not None else torch.zeros_like(cls_summary)
+    pooled = torch.cat([cls_summary, candidate_summary, masked_mean(x, padding_mask)], dim=-1)
+    if pool_norm_weight is not None:
+        pooled = rms_norm(pooled, cast(pool_norm_weight), eps)
+    if classifier is None:
+        return pooled, None
+    w1, b1, w2, b2 = (cast(t) for t in classifier)
+    return pooled, F.linear(F.silu(F.linear(pooled, w1, b1)), w2, b2)
+
+
 # ---- dense layers ----------------------------------------------------------------------------------------------------
 
 

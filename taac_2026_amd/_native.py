@@ -152,6 +152,11 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         c_int,
         [c_void_p, c_int64, c_int32, c_void_p, c_int, c_int64, c_int32, c_void_p, c_void_p, c_int, c_void_p],
     ),
+    "taac_candidate_readout_fwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_float,
+         c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_int, c_void_p],
+    ),
     "taac_masked_mean_head": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p],

@@ -31,6 +31,7 @@ from taac_2026_amd.accelerators.linear import (
     swiglu_linear,
     valid_rows,
 )
+from taac_2026_amd.accelerators.readout import candidate_readout
 from taac_2026_amd.accelerators.normalization import (
     hip_layer_norm_kernel,
     hip_rms_norm_kernel,
@@ -47,6 +48,7 @@ from taac_2026_amd.accelerators.tensor_validation import (
 )
 
 __all__ = [
+    "candidate_readout",
     "attention_out_ffn",
     "FlashAttentionMaskPlan",
     "StructuredAttentionMask",

@@ -20,6 +20,7 @@ from taac_2026_amd.modeling.normalization import (
     configure_rms_norm_runtime,
     rms_norm_runtime_state,
 )
+from taac_2026_amd.modeling.readout import CandidateClsPooler, CandidateReadoutHead
 from taac_2026_amd.modeling.sequence import (
     causal_valid_attention_mask,
     configure_flash_attention_runtime,
@@ -32,6 +33,8 @@ from taac_2026_amd.modeling.sequence import (
 
 __all__ = [
     "BFTSAttention",
+    "CandidateClsPooler",
+    "CandidateReadoutHead",
     "LayerNorm",
     "MetadataAttentionMask",
     "PCVRBackbone",

@@ -131,6 +131,24 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
     assert tail(f=48) == unsupported
     assert tail(m=0) == ok
 
+    # readout: indices inside the sequence, one kind of validity, a complete classifier, something to write
+    def readout(**kw):
+        a = dict(lengths=None, bits=None, t=16, d=64, cls=0, cand=3, fc1=fake, fc2=fake, hidden=32, actions=1, emb=None,
+                 logits=fake, b=2)
+        a.update(kw)
+        return library.taac_candidate_readout_fwd(fake, a["lengths"], a["bits"], a["b"], a["t"], a["d"], a["cls"], a["cand"],
+                                                  None, None, 1e-6, a["fc1"], None, a["hidden"], a["fc2"], None,
+                                                  a["actions"], a["emb"], a["logits"], 0, None)
+
+    assert readout(cls=16) == invalid and b"outside the sequence" in library.taac_last_error()
+    assert readout(cand=16) == invalid
+    assert readout(lengths=fake, bits=fake) == invalid and b"not both" in library.taac_last_error()
+    assert readout(d=12) == unsupported and readout(d=2048) == unsupported
+    assert readout(hidden=2048) == unsupported
+    assert readout(fc2=None) == invalid and readout(logits=None) == invalid
+    assert readout(fc1=None, emb=None) == invalid and b"nothing to compute" in library.taac_last_error()
+    assert readout(b=0) == ok
+
     # attention with structured masks, the training forward and the backward
     strides = _native.Int64x4(2048, 16, 128, 1)
 

@@ -476,3 +476,39 @@ def test_qk_norm_rope_and_embedding_bag_golden_vectors():
         weight, values = torch.tensor(case["weight"]), torch.tensor(case["values"])
         for route in (oracle.embedding_bag_mean, oracle.embedding_bag_mean_closed_form):
             np.testing.assert_allclose(route(weight, values).double().numpy(), np.array(case["out"]), rtol=1e-6, atol=1e-7)
+
+
+# ---- readout ---------------------------------------------------------------------------------------------------------------
+
+
+def test_candidate_readout_brute_force_and_special_cases():
+    """A float64 loop over a tiny case restates final_norm -> cls | candidate | masked mean -> RMSNorm(3D) ->
+    Linear -> SiLU -> Linear (experiments/symbiosis/pooling.py:24-32, model.py:217-222, 291); special cases: without
+    a candidate the middle third is zero, an all-padded sample's mean is zero, and without norms and classifier the
+    last third is the plain masked mean."""
+    g = torch.Generator().manual_seed(5)
+    batch, tokens, d, hidden, actions = 3, 6, 8, 5, 2
+    x = torch.randn(batch, tokens, d, generator=g)
+    pad = torch.tensor([[False, False, True, False, True, True], [True] * 6, [False] * 6])
+    wt, wp = 1 + 0.1 * torch.randn(d, generator=g), 1 + 0.1 * torch.randn(3 * d, generator=g)
+    w1, b1 = torch.randn(hidden, 3 * d, generator=g) / 4, torch.randn(hidden, generator=g) / 4
+    w2, b2 = torch.randn(actions, hidden, generator=g) / 2, torch.randn(actions, generator=g) / 4
+    emb, logits = oracle.candidate_readout(x, pad, cls_index=0, candidate_index=3, token_norm_weight=wt,
+                                           pool_norm_weight=wp, eps=1e-6, classifier=(w1, b1, w2, b2))
+    xn, eps = x.double().numpy(), 1e-6
+    for b in range(batch):
+        normed = np.stack([row / np.sqrt((row ** 2).mean() + eps) * wt.double().numpy() for row in xn[b]])
+        keep = [t for t in range(tokens) if not bool(pad[b, t])]
+        mean = sum(normed[t] for t in keep) / max(1, len(keep)) if keep else np.zeros(d)
+        pooled = np.concatenate([normed[0], normed[3], mean])
+        pooled = pooled / np.sqrt((pooled ** 2).mean() + eps) * wp.double().numpy()
+        np.testing.assert_allclose(emb[b].double().numpy(), pooled, rtol=1e-5, atol=1e-6)
+        z = w1.double().numpy() @ pooled + b1.double().numpy()
+        out = w2.double().numpy() @ (z / (1 + np.exp(-z))) + b2.double().numpy()
+        np.testing.assert_allclose(logits[b].double().numpy(), out, rtol=1e-5, atol=1e-6)
+    bare, none = oracle.candidate_readout(x, pad, cls_index=2, candidate_index=None, token_norm_weight=None,
+                                          pool_norm_weight=None)
+    assert none is None and bare[:, d:2 * d].abs().max().item() == 0.0
+    torch.testing.assert_close(bare[:, :d], x[:, 2])
+    torch.testing.assert_close(bare[:, 2 * d:], oracle.masked_mean(x, pad))
+    assert bare[1, 2 * d:].abs().max().item() == 0.0
