@@ -415,6 +415,43 @@ def _structured_mask_figures(device, batch: int, iters: int) -> dict:
     return out
 
 
+def _reference_block_figures(device, batch: int, iters: int) -> dict:
+    """One block as the reference model runs it (UnifiedInteractionBlock with query / key norms, experiments/symbiosis/
+    backbone.py:51-68): role-based attention mask, padding scattered inside the sequence part (not a prefix), updates
+    masked at padded rows. Timed: the fused route that leaves out the intermediate stream (3 heavy kernels + the row
+    index) and the route that returns it, plus a block checked against the oracle on a small slice."""
+    from oracle import reference as oracle
+    from taac_2026_amd.api import MetadataAttentionMask, UnifiedInteractionBlock
+
+    g = torch.Generator().manual_seed(42)
+    T, D, H = 512, 256, 8
+    block = UnifiedInteractionBlock(D, H, 4, 0.0).to(torch.bfloat16).eval()
+    x = (0.5 * torch.randn(batch, T, D, generator=g)).to(torch.bfloat16)
+    roles = torch.tensor([0] * 16 + [2] * 15 + [3] + [1] * 480)            # feature tokens, candidate, sequence tokens
+    keep_fraction = torch.rand(batch, 1, generator=g) * 0.9 + 0.1           # per sample, of the 480 sequence tokens
+    padding = torch.cat([torch.zeros(batch, 32, dtype=torch.bool), torch.rand(batch, 480, generator=g) > keep_fraction], dim=1)
+    small = slice(0, 4)
+    state = {k.replace("attention.", "").replace("ffn.", ""): v.detach().float() for k, v in block.state_dict().items()}
+    want, _ = oracle.interaction_block(x[small].float(), padding[small], oracle.metadata_attention_mask(padding[small], roles),
+                                       state, num_heads=H)
+    block = block.to(device)
+    dev_x, dev_pad = x.to(device), padding.to(device)
+    with torch.no_grad():
+        mask = MetadataAttentionMask(enabled=True)(dev_pad, roles.to(device))
+        got, _ = block(dev_x, dev_pad, mask, return_attention_tokens=False)
+        valid = ~padding[small]
+        err = (got[small].cpu().float()[valid] - want[valid]).abs().max().item()
+        if not err <= 5e-2:
+            raise SystemExit(f"accuracy gate of the reference block failed: {err}")
+        work = dev_x.clone()
+        fused = _event_ms(lambda: block(work, dev_pad, mask, return_attention_tokens=False, inplace=True), iters, 3)
+        both = _event_ms(lambda: block(dev_x, dev_pad, mask), iters, 3)
+    return {"valid_token_fraction": float((~padding).float().mean().item()), "one_kernel_tail_in_place_ms": fused,
+            "with_attention_tokens_ms": both, "max_abs_err_vs_oracle": err,
+            "note": "whole module calls: row index from the padding mask, projection + norm statistic, masked "
+                    "attention, out projection + feed-forward; the second figure also copies the stream twice"}
+
+
 def _cpu_baseline(inputs, budget_s: float = 20.0) -> dict:
     """The oracle's backbone forward (the reference's torch formulas) on the host cores, on a bounded sample."""
     from oracle import reference as oracle
@@ -468,6 +505,8 @@ def main() -> None:
     parser.add_argument("--only-layer-variants", action="store_true",
                         help="time only the backbone with the reference layers' query / key norm (and rotary embedding) "
                              "and print those figures (for kernel traces of that mode)")
+    parser.add_argument("--only-reference-block", action="store_true",
+                        help="time only the reference model's block (role mask, scattered padding) and print those figures")
     args = parser.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU (the path has no cross-GPU stage); use --gpus 1")
@@ -483,6 +522,9 @@ def main() -> None:
         return
     if args.only_layer_variants:
         print(json.dumps({"reference_layer_variants": _qk_variant_figures(device, args.batch, args.steps)}))
+        return
+    if args.only_reference_block:
+        print(json.dumps({"reference_block": _reference_block_figures(device, args.batch, 10)}))
         return
     inputs = workloads.backbone_inputs(batch=args.batch)
     B, T, D = inputs.emb.shape
@@ -571,6 +613,7 @@ def main() -> None:
         line["candidate_readout"] = _readout_figures(inputs, device, iters=20)
         if not args.skip_widened:
             line["reference_layer_variants"] = _qk_variant_figures(device, B, max(args.steps // 2, 1))
+            line["reference_block"] = _reference_block_figures(device, B, 10)
             line["structured_masks"] = _structured_mask_figures(device, B, iters=10)
     if not args.skip_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(inputs)

@@ -336,6 +336,15 @@ int taac_candidate_readout_fwd(const void* tokens, const int32_t* key_lengths, c
 int taac_valid_rows(const int32_t* key_lengths, int32_t B, int32_t T, int32_t* rows, int32_t* n_rows, void* stream);
 
 /*
+ * The same row index for padding that is not a prefix: token t of sample b is valid iff bit t of valid_bits[b] is set
+ * (rows of ceil(T / 32) 32-bit words, as written by taac_mask_pack_bits from a [B, T] bool matrix, True = valid).
+ * Output layout and sizes as in taac_valid_rows. This is what lets the dense layers honour the reference blocks'
+ * `update * ~padding_mask` (experiments/symbiosis/backbone.py:65, 67) by not touching the padded rows at all.
+ */
+int taac_valid_rows_from_bits(const uint32_t* valid_bits, int32_t B, int32_t T, int32_t* rows, int32_t* n_rows,
+                              void* stream);
+
+/*
  * Weight packing for the two fused kernels above: copies the weights into MFMA-fragment order (the order in which
  * the kernels stage them into LDS). Pack once per weight set; the blob has the size of the weights themselves.
  * The FFN blob depends on gate_first (which half of w_up is gated): taac_swiglu_ffn_fwd must be given the same value.

@@ -398,6 +398,28 @@ def block(x: torch.Tensor, key_lengths: torch.Tensor, w: dict[str, torch.Tensor]
     return x + swiglu_ffn(h2, w["up.weight"], w.get("up.bias"), w["down.weight"], w.get("down.bias"))
 
 
+def interaction_block(tokens: torch.Tensor, padding_mask: torch.Tensor, attention_mask: torch.Tensor | None,
+                      w: dict[str, torch.Tensor], *, num_heads: int, eps: float = 1e-6,
+                      rope_base: float | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """``UnifiedInteractionBlock.forward`` as written (experiments/symbiosis/backbone.py:58-68): both updates are
+    multiplied by ``~padding_mask``, so padded rows pass through unchanged; ``attention_mask`` is the bool
+    (B, 1 or H, T, T) mask the model's mask module built (True = attend) or None. Composed from the pinned pieces
+    above. Returns (output, attn_tokens)."""
+    batch, token_count, d_model = tokens.shape
+    keep = (~padding_mask).unsqueeze(-1).to(tokens.dtype)
+    h = rms_norm(tokens, w["attn_norm.weight"], eps)
+    q, k, v = F.linear(h, w["qkv.weight"], w.get("qkv.bias")).chunk(3, dim=-1)
+    if "query_norm.weight" in w or rope_base is not None:
+        q, k = qk_norm_rope(q, k, w.get("query_norm.weight"), w.get("key_norm.weight"), num_heads=num_heads, eps=eps,
+                            rope_base=rope_base)
+    heads = lambda t: t.view(batch, token_count, num_heads, d_model // num_heads).transpose(1, 2)  # noqa: E731
+    a = sdpa(heads(q), heads(k), heads(v), attn_mask=attention_mask).transpose(1, 2).reshape(batch, token_count, d_model)
+    attn_tokens = tokens + F.linear(a, w["out.weight"], w.get("out.bias")) * keep
+    h2 = rms_norm(attn_tokens, w["ffn_norm.weight"], eps)
+    output = attn_tokens + swiglu_ffn(h2, w["up.weight"], w.get("up.bias"), w["down.weight"], w.get("down.bias")) * keep
+    return output, attn_tokens
+
+
 def backbone(emb: torch.Tensor, key_lengths: torch.Tensor, blocks: list[dict[str, torch.Tensor]],
              head_weight: torch.Tensor, head_bias: torch.Tensor | None, *, num_heads: int, eps: float = 1e-6,
              return_hidden: bool = False, rope_base: float | None = None):

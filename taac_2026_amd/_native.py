@@ -126,6 +126,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
          c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p],
     ),
     "taac_valid_rows": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p]),
+    "taac_valid_rows_from_bits": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p]),
     "taac_norm_linear_qk_fwd": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32,

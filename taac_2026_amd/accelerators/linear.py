@@ -175,18 +175,36 @@ def pack_linear_weight(weight: torch.Tensor) -> torch.Tensor:
     return packed
 
 
-def valid_rows(key_lengths: torch.Tensor, tokens: int) -> tuple[torch.Tensor, torch.Tensor]:
-    """Row index of the valid tokens of a padded ``[B, tokens, ...]`` batch (token ``t`` of sample ``b`` is valid iff
-    ``t < key_lengths[b]``): ``(rows, n_rows)`` with ``rows[:n_rows] = b * tokens + t`` in increasing order, both int32
+def valid_rows(key_lengths: torch.Tensor | None, tokens: int, *,
+               padding_mask: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """Row index of the valid tokens of a padded ``[B, tokens, ...]`` batch: token ``t`` of sample ``b`` is valid iff
+    ``t < key_lengths[b]``, or - for padding that is not a prefix - iff ``not padding_mask[b, t]`` (bool ``[B, tokens]``,
+    True = padding). Returns ``(rows, n_rows)`` with ``rows[:n_rows] = b * tokens + t`` in increasing order, both int32
     on the device (no host synchronisation). ``rows[B * tokens : B * tokens + B + 1]`` holds the per-sample offsets.
-    Pass the pair as ``token_rows=`` to :func:`norm_linear` / :func:`swiglu_ffn` to skip the padded positions."""
+    Pass the pair as ``token_rows=`` to :func:`norm_linear` / :func:`swiglu_ffn` / :func:`attention_out_ffn` to skip the
+    padded positions."""
     name = "hip valid_rows"
-    require_cuda_tensors(name, key_lengths)
+    if (key_lengths is None) == (padding_mask is None):
+        raise ValueError(f"{name}: give key_lengths or padding_mask")
+    require_cuda_tensors(name, key_lengths, padding_mask)
+    library = _native.load_library()
+    if padding_mask is not None:
+        if padding_mask.dtype is not torch.bool or padding_mask.ndim != 2 or padding_mask.shape[1] != int(tokens):
+            raise ValueError(f"{name}: padding_mask must be a bool tensor of shape (batch, {int(tokens)})")
+        from taac_2026_amd.accelerators.attention import _pack_bits
+
+        batch = padding_mask.shape[0]
+        bits = _pack_bits((~padding_mask).contiguous())
+        rows = torch.empty(batch * int(tokens) + batch + 1, dtype=torch.int32, device=padding_mask.device)
+        count = torch.empty(1, dtype=torch.int32, device=padding_mask.device)
+        status = library.taac_valid_rows_from_bits(bits.data_ptr(), batch, int(tokens), rows.data_ptr(), count.data_ptr(),
+                                                   _native.current_stream(padding_mask.device))
+        _native.check(status, "valid_rows")
+        return rows, count
     lengths = key_lengths.to(torch.int32).contiguous()
     batch = lengths.numel()
     rows = torch.empty(batch * int(tokens) + batch + 1, dtype=torch.int32, device=lengths.device)
     count = torch.empty(1, dtype=torch.int32, device=lengths.device)
-    library = _native.load_library()
     status = library.taac_valid_rows(lengths.data_ptr(), batch, int(tokens), rows.data_ptr(), count.data_ptr(),
                                      _native.current_stream(lengths.device))
     _native.check(status, "valid_rows")

@@ -223,8 +223,32 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   vec_t kreg[KLD], vreg[VLD][2];
   float kfac[SCALED ? KLD : 1];
   const bool scale_keys = SCALED && p.k_row_scale != nullptr;
-  // MASKED: the two 32-key words of the lane's query for the chunk being fetched / being consumed.
+  // MASKED: the two 32-key words of the lane's query for the chunk being fetched / being consumed (structure only),
+  // and the sample's key-validity words of the same keys (all ones without valid_bits).
   uint32_t mw_next[2] = {0u, 0u}, mw[2] = {0u, 0u};
+  uint32_t vw_next[2] = {~0u, ~0u}, vw[2] = {~0u, ~0u};
+  // Key validity enters the scores through the matrix unit instead of per-element selects: one more k-step per tile
+  // whose key operand is -BIG at k = 0 for an invalid key (0 for a valid one) and whose query operand is the inverse of
+  // the query's row factor at k = 0 (1 without one), so that after the lane's scale the score of an invalid key is about
+  // -BIG * log2(e) / sqrt(d) (BIG = 2^30, 2^15 for fp16), whatever the factor, and its probability underflows to exactly 0, while valid keys get
+  // 0 added, exactly. Tiles whose structure is all ones then stay on the fast path however the padding is scattered.
+  // (A query with no valid key at all still ends at 0: the value rows of invalid keys are staged as zeros.)
+  vec_t qbias;
+  if (MASKED) {
+    const float factor = c / p.scale_log2;  // the query's row factor, 1 without one
+    const T inv = static_cast<T>(1.0f / factor);
+    u32x4 bits = {hh == 0 ? static_cast<uint32_t>(__builtin_bit_cast(uint16_t, inv)) : 0u, 0u, 0u, 0u};
+    qbias = __builtin_bit_cast(vec_t, bits);
+  }
+  constexpr uint32_t kNegBigBits = std::is_same<T, bf16_t>::value ? 0xCE80u : 0xF800u;  // -2^30 (bf16) / -32768 (fp16)
+  // MASKED with per-sample key validity: a key outside it reaches LDS as zeros whatever its rows hold - they may be
+  // uninitialised memory (a caller that skips the padded positions never writes them), and a masked probability of
+  // zero times a NaN would still poison the output. The rows are loaded like any other and cleared on their way into
+  // LDS (commit), against the chunk's two validity words, so that the loads do not wait for those words.
+  auto key_is_valid = [&](int key_in_chunk) -> bool {
+    if (!MASKED) return true;
+    return ((vw_next[key_in_chunk / 32] >> (key_in_chunk % 32)) & 1u) != 0u;
+  };
   auto fetch = [&](int kc0) {
     if (MASKED) {
       const int w0 = kc0 / 32;
@@ -233,9 +257,9 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
         uint32_t bits = 0u;
         if (qi < p.Tq && w0 + kt < p.wpr) {
           bits = p.struct_bits[static_cast<int64_t>(qi) * p.wpr + w0 + kt];
-          if (p.valid_bits != nullptr) bits &= p.valid_bits[static_cast<int64_t>(b) * p.wpr + w0 + kt];
         }
         mw_next[kt] = bits;
+        vw_next[kt] = (p.valid_bits != nullptr && w0 + kt < p.wpr) ? p.valid_bits[static_cast<int64_t>(b) * p.wpr + w0 + kt] : ~0u;
       }
     }
 #pragma unroll
@@ -266,7 +290,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 #pragma unroll
         for (int e = 0; e < 8; ++e) kreg[i][e] = static_cast<T>(static_cast<float>(kreg[i][e]) * kfac[SCALED ? i : 0]);
       }
-      if (idx < kKC * C8) *reinterpret_cast<vec_t*>(&sK[(idx / C8) * KSTR + (idx % C8) * 8]) = kreg[i];
+      if (idx < kKC * C8) *reinterpret_cast<vec_t*>(&sK[(idx / C8) * KSTR + (idx % C8) * 8]) =
+          key_is_valid(idx / C8) ? kreg[i] : zero_vec;
     }
 #pragma unroll
     for (int i = 0; i < VLD; ++i) {
@@ -275,9 +300,11 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
         const int key0 = 2 * (idx / C8);
         const int c8 = idx % C8;
         const int pos = (key0 & ~15) + vt_pos16(key0 & 15);  // even; key0 + 1 lands at pos + 1
+        const vec_t v0 = key_is_valid(key0) ? vreg[i][0] : zero_vec;
+        const vec_t v1 = key_is_valid(key0 + 1) ? vreg[i][1] : zero_vec;
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          *reinterpret_cast<uint32_t*>(&sVt[(c8 * 8 + e) * VSTR + pos]) = pack2<T>(vreg[i][0][e], vreg[i][1][e]);
+          *reinterpret_cast<uint32_t*>(&sVt[(c8 * 8 + e) * VSTR + pos]) = pack2<T>(v0[e], v1[e]);
       }
     }
   };
@@ -306,6 +333,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
     if (MASKED) {
       mw[0] = mw_next[0];
       mw[1] = mw_next[1];
+      vw[0] = vw_next[0];
+      vw[1] = vw_next[1];
     }
     __syncthreads();
     kc = next_chunk(kc + 1);
@@ -327,6 +356,14 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
         for (int s = 0; s < KSTEPS; ++s) {
           const vec_t a = *reinterpret_cast<const vec_t*>(&sK[((T0 + kt) * 32 + l32) * KSTR + 16 * s + 8 * hh]);
           sacc[kt] = Mfma32<T>::run(a, qf[s], sacc[kt]);
+        }
+        if (MASKED) {  // + (invalid key ? -BIG : 0) / (row factor of the query); the lane's key is key l32 of the tile
+          const uint32_t word = __builtin_amdgcn_readfirstlane(vw[T0 + kt]);  // the same for every lane: one sample
+          if (word != ~0u) {
+            const bool invalid = ((word >> l32) & 1u) == 0u;
+            const u32x4 kbits = {(hh == 0 && invalid) ? kNegBigBits : 0u, 0u, 0u, 0u};
+            sacc[kt] = Mfma32<T>::run(__builtin_bit_cast(vec_t, kbits), qbias, sacc[kt]);
+          }
         }
       }
       const int k_last = kc0 + (T0 + NT) * 32;  // one past the last key of this update
@@ -408,8 +445,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
     typedef std::integral_constant<int, 2> I2;
     if (MASKED) {
       // tiles in which no query of this wavefront sees a key are not computed
-      const bool any0 = __builtin_amdgcn_ballot_w64(mw[0] != 0u) != 0;
-      const bool any1 = __builtin_amdgcn_ballot_w64(mw[1] != 0u) != 0 && kc0 + 32 < wave_kv_end;
+      const bool any0 = __builtin_amdgcn_ballot_w64((mw[0] & vw[0]) != 0u) != 0;
+      const bool any1 = __builtin_amdgcn_ballot_w64((mw[1] & vw[1]) != 0u) != 0 && kc0 + 32 < wave_kv_end;
       if (any0 && any1)
         update(I2{}, I0{});
       else if (any0)

@@ -62,16 +62,34 @@ __global__ __launch_bounds__(kBlock) void masked_mean_head_kernel(const bf16_t* 
   }
 }
 
-// Exclusive prefix sums of the clamped lengths (one workgroup; B is walked in slabs of kBlock with a running carry).
-__global__ __launch_bounds__(kBlock) void length_offsets_kernel(const int32_t* __restrict__ lengths, int B, int T,
+// Number of valid tokens of sample b: its clamped length, or the set bits among the first T of its bit row.
+__device__ __forceinline__ int32_t valid_count(const int32_t* __restrict__ lengths, const uint32_t* __restrict__ bits,
+                                               int b, int T) {
+  if (lengths != nullptr) {
+    const int32_t len = lengths[b];
+    return len < 0 ? 0 : (len > T ? T : len);
+  }
+  const int wpr = (T + 31) / 32;
+  int32_t n = 0;
+  for (int w = 0; w < wpr; ++w) {
+    uint32_t word = bits[static_cast<int64_t>(b) * wpr + w];
+    if (w == wpr - 1 && T % 32 != 0) word &= (1u << (T % 32)) - 1u;
+    n += __popc(word);
+  }
+  return n;
+}
+
+// Exclusive prefix sums of the per-sample valid counts (one workgroup; B is walked in slabs of kBlock with a running
+// carry).
+__global__ __launch_bounds__(kBlock) void length_offsets_kernel(const int32_t* __restrict__ lengths,
+                                                                const uint32_t* __restrict__ bits, int B, int T,
                                                                 int32_t* __restrict__ offsets,
                                                                 int32_t* __restrict__ n_rows) {
   __shared__ int32_t s_scan[kBlock];
   int32_t carry = 0;
   for (int base = 0; base < B; base += kBlock) {
     const int b = base + threadIdx.x;
-    int32_t len = b < B ? lengths[b] : 0;
-    len = len < 0 ? 0 : (len > T ? T : len);
+    const int32_t len = b < B ? valid_count(lengths, bits, b, T) : 0;
     s_scan[threadIdx.x] = len;
     __syncthreads();
     for (int step = 1; step < kBlock; step <<= 1) {  // inclusive scan, Hillis-Steele
@@ -98,6 +116,22 @@ __global__ __launch_bounds__(kBlock) void valid_rows_kernel(const int32_t* __res
   len = len < 0 ? 0 : (len > T ? T : len);
   const int t = blockIdx.x * kBlock + threadIdx.x;
   if (t < len) rows[offsets[b] + t] = b * T + t;
+}
+
+// The same for a validity bit row per sample: token t goes to slot offsets[b] + (number of valid tokens before t).
+__global__ __launch_bounds__(kBlock) void valid_rows_bits_kernel(const uint32_t* __restrict__ bits,
+                                                                 const int32_t* __restrict__ offsets, int T,
+                                                                 int32_t* __restrict__ rows) {
+  const int b = blockIdx.y;
+  const int t = blockIdx.x * kBlock + threadIdx.x;
+  if (t >= T) return;
+  const int wpr = (T + 31) / 32;
+  const uint32_t* row = bits + static_cast<int64_t>(b) * wpr;
+  const uint32_t word = row[t / 32];
+  if (((word >> (t % 32)) & 1u) == 0u) return;
+  int32_t rank = __popc(word & ((1u << (t % 32)) - 1u));
+  for (int w = 0; w < t / 32; ++w) rank += __popc(row[w]);
+  rows[offsets[b] + rank] = b * T + t;
 }
 
 // prod[d] = wq[d] * wk[d] in fp32: the weights of a query and a key norm act on an attention score only through their
@@ -138,11 +172,29 @@ extern "C" int taac_valid_rows(const int32_t* key_lengths, int32_t B, int32_t T,
   if (!rows || !n_rows || (B > 0 && !key_lengths)) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
   if (B > 65535) return set_error(TAAC_ERR_UNSUPPORTED, "%s: at most 65535 samples", name);
   int32_t* offsets = rows + static_cast<int64_t>(B) * T;
-  hipLaunchKernelGGL(length_offsets_kernel, dim3(1), dim3(kBlock), 0, as_stream(stream), key_lengths, B, T, offsets,
-                     n_rows);
+  hipLaunchKernelGGL(length_offsets_kernel, dim3(1), dim3(kBlock), 0, as_stream(stream), key_lengths,
+                     static_cast<const uint32_t*>(nullptr), B, T, offsets, n_rows);
   if (B > 0 && T > 0)
     hipLaunchKernelGGL(valid_rows_kernel, dim3((T + kBlock - 1) / kBlock, B), dim3(kBlock), 0, as_stream(stream),
                        key_lengths, offsets, T, rows);
+  return check_launch(name);
+}
+
+extern "C" int taac_valid_rows_from_bits(const uint32_t* valid_bits, int32_t B, int32_t T, int32_t* rows,
+                                         int32_t* n_rows, void* stream) {
+  using namespace taac;
+  const char* name = "taac_valid_rows_from_bits";
+  if (B < 0 || T < 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: bad dimensions", name);
+  if (static_cast<int64_t>(B) * T > 0x7fffffffLL - B - 1)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: B * T must fit 32-bit row numbers", name);
+  if (!rows || !n_rows || (B > 0 && T > 0 && !valid_bits)) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  if (B > 65535) return set_error(TAAC_ERR_UNSUPPORTED, "%s: at most 65535 samples", name);
+  int32_t* offsets = rows + static_cast<int64_t>(B) * T;
+  hipLaunchKernelGGL(length_offsets_kernel, dim3(1), dim3(kBlock), 0, as_stream(stream),
+                     static_cast<const int32_t*>(nullptr), valid_bits, B, T, offsets, n_rows);
+  if (B > 0 && T > 0)
+    hipLaunchKernelGGL(valid_rows_bits_kernel, dim3((T + kBlock - 1) / kBlock, B), dim3(kBlock), 0, as_stream(stream),
+                       valid_bits, offsets, T, rows);
   return check_launch(name);
 }
 

@@ -18,8 +18,8 @@ import torch
 import torch.nn as nn
 
 from taac_2026_amd import _native
-from taac_2026_amd.accelerators.attention import qk_norm_rope, rope_table
-from taac_2026_amd.accelerators.linear import norm_linear, qkv_projection, swiglu_ffn
+from taac_2026_amd.accelerators.attention import StructuredAttentionMask, qk_norm_rope, rope_table
+from taac_2026_amd.accelerators.linear import attention_out_ffn, norm_linear, qkv_projection, swiglu_ffn, valid_rows
 from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference
 from taac_2026_amd.modeling.normalization import RMSNorm
 from taac_2026_amd.modeling.sequence import scaled_dot_product_attention
@@ -76,7 +76,7 @@ class UnifiedSelfAttention(nn.Module):
     def forward(
         self,
         tokens: torch.Tensor,
-        attention_mask: torch.Tensor | None = None,
+        attention_mask: torch.Tensor | StructuredAttentionMask | None = None,
         *,
         key_lengths: torch.Tensor | None = None,
         zero_padded_queries: bool = False,
@@ -103,12 +103,14 @@ class UnifiedSelfAttention(nn.Module):
             if prepare:  # one pass over the q and k columns of the packed projection, in place
                 qk_norm_rope(query, key, query_weight, key_weight, num_heads=self.num_heads, eps=qk_eps,
                              rope_base=self.rope_base, inplace=True)
+        structured = attention_mask if isinstance(attention_mask, StructuredAttentionMask) else None
         attended = scaled_dot_product_attention(
             query,
             key,
             value,
             num_heads=self.num_heads,
-            attn_mask=attention_mask,
+            attn_mask=None if structured is not None else attention_mask,
+            structured_mask=structured,
             dropout_p=self.dropout,
             training=self.training,
             key_lengths=key_lengths,
@@ -134,7 +136,16 @@ class BFTSAttention(UnifiedSelfAttention):
 
 
 class UnifiedInteractionBlock(nn.Module):
-    """Pre-RMSNorm self-attention and SwiGLU feed-forward with residuals masked at padded positions."""
+    """Pre-RMSNorm self-attention and SwiGLU feed-forward with residuals masked at padded positions
+    (experiments/symbiosis/backbone.py:51-68).
+
+    For bf16 GPU tokens of width 128 / 256 under ``torch.no_grad()`` the block runs on the fused kernels: the dense
+    layers walk the valid rows only (``update * ~padding_mask`` becomes "the padded rows are never touched": they keep
+    their input values, as ``x + 0`` does), ``attn_norm`` and the query / key norm statistic are part of the projection
+    kernel, and with ``return_attention_tokens=False`` the out projection, both residual adds, ``ffn_norm`` and the
+    feed-forward are one kernel. ``attention_mask`` may be a dense bool mask, a :class:`StructuredAttentionMask`
+    (what ``MetadataAttentionMask`` returns) or None; ``key_lengths`` states prefix padding without a mask.
+    ``inplace=True`` lets the fused route update ``tokens`` itself instead of a copy."""
 
     def __init__(self, d_model: int, num_heads: int, hidden_mult: int, dropout: float = 0.0, *, qk_norm: bool = True) -> None:
         super().__init__()
@@ -143,14 +154,68 @@ class UnifiedInteractionBlock(nn.Module):
         self.ffn_norm = RMSNorm(d_model)
         self.ffn = SwiGLUFeedForward(d_model, hidden_mult, dropout)
 
+    def _fused_route(self, tokens: torch.Tensor) -> bool:
+        if not (tokens.is_cuda and tokens.dtype == torch.bfloat16 and tokens.ndim == 3 and tokens.shape[-1] in (128, 256)):
+            return False
+        if self.ffn.down.weight.shape[1] % 32 != 0:
+            return False
+        if self.training and (self.attention.dropout > 0.0 or self.ffn.dropout.p > 0.0):
+            return False
+        return not (torch.is_grad_enabled() and (tokens.requires_grad or any(p.requires_grad for p in self.parameters())))
+
+    def _forward_fused(self, tokens, padding_mask, attention_mask, key_lengths, return_attention_tokens, inplace):
+        batch, token_count, d_model = tokens.shape
+        x = tokens.contiguous()
+        index = valid_rows(key_lengths, token_count) if key_lengths is not None else \
+            valid_rows(None, token_count, padding_mask=padding_mask)
+        attention = self.attention
+        qkv = torch.empty(batch * token_count, 3 * d_model, dtype=x.dtype, device=x.device)
+        q_row_scale = k_row_scale = q_col_scale = None
+        if attention.query_norm is not None or attention.rope_base is not None:
+            _, q_row_scale, k_row_scale, q_col_scale = qkv_projection(
+                x, _bf16(attention.qkv.weight), _bf16(attention.qkv.bias), num_heads=attention.num_heads,
+                norm_weight=_bf16(self.attn_norm.weight), eps=self.attn_norm.eps,
+                query_weight=None if attention.query_norm is None else _bf16(attention.query_norm.weight),
+                key_weight=None if attention.key_norm is None else _bf16(attention.key_norm.weight),
+                qk_eps=1e-6 if attention.query_norm is None else attention.query_norm.eps, rope_base=attention.rope_base,
+                token_rows=index, out=qkv)
+        else:
+            norm_linear(x, _bf16(attention.qkv.weight), _bf16(attention.qkv.bias), norm_weight=_bf16(self.attn_norm.weight),
+                        eps=self.attn_norm.eps, token_rows=index, out=qkv)
+        query, key, value = qkv.view(batch, token_count, 3 * d_model).chunk(3, dim=-1)
+        structured = attention_mask if isinstance(attention_mask, StructuredAttentionMask) else None
+        dense_mask = None if structured is not None else attention_mask
+        attended = scaled_dot_product_attention(
+            query, key, value, num_heads=attention.num_heads, attn_mask=dense_mask, structured_mask=structured,
+            dropout_p=0.0, training=False, key_lengths=key_lengths if attention_mask is None else None,
+            q_row_scale=q_row_scale, k_row_scale=k_row_scale, q_col_scale=q_col_scale)
+        ffn = self.ffn
+        dense = dict(norm_weight=_bf16(self.ffn_norm.weight), eps=self.ffn_norm.eps, token_rows=index)
+        if not return_attention_tokens and ffn.gate_first:
+            output = x if inplace else x.clone()
+            attention_out_ffn(attended, _bf16(attention.out.weight), _bf16(attention.out.bias), x, _bf16(ffn.up.weight),
+                              _bf16(ffn.up.bias), _bf16(ffn.down.weight), _bf16(ffn.down.bias), out=output, **dense)
+            return output, None
+        attn_tokens = x.clone()  # padded rows pass through
+        norm_linear(attended, _bf16(attention.out.weight), _bf16(attention.out.bias), residual=x, token_rows=index,
+                    out=attn_tokens)
+        output = attn_tokens.clone()
+        swiglu_ffn(attn_tokens, _bf16(ffn.up.weight), _bf16(ffn.up.bias), _bf16(ffn.down.weight), _bf16(ffn.down.bias),
+                   residual=attn_tokens, gate_first=ffn.gate_first, out=output, **dense)
+        return output, attn_tokens
+
     def forward(
         self,
         tokens: torch.Tensor,
         padding_mask: torch.Tensor,
-        attention_mask: torch.Tensor | None,
+        attention_mask: torch.Tensor | StructuredAttentionMask | None,
         *,
         key_lengths: torch.Tensor | None = None,
-    ) -> tuple[torch.Tensor, torch.Tensor]:
+        return_attention_tokens: bool = True,
+        inplace: bool = False,
+    ) -> tuple[torch.Tensor, torch.Tensor | None]:
+        if self._fused_route(tokens):
+            return self._forward_fused(tokens, padding_mask, attention_mask, key_lengths, return_attention_tokens, inplace)
         keep = (~padding_mask).unsqueeze(-1)
         attn_update = self.attention(self.attn_norm(tokens), attention_mask, key_lengths=key_lengths)
         attn_tokens = tokens + attn_update * keep.to(attn_update.dtype)

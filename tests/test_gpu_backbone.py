@@ -163,3 +163,92 @@ def test_interaction_block_module(device):
         got, got_attn = block(x.to(device), padding.to(device), mask.to(device))
     torch.testing.assert_close(got_attn.cpu().float(), attn_tokens.float(), rtol=2e-2, atol=2e-2)
     torch.testing.assert_close(got.cpu().float(), expected.float(), rtol=2e-2, atol=2e-2)
+
+
+def _symbiosis_block_case(d_model, heads, tokens, batch, seed):
+    from taac_2026_amd.api import MetadataAttentionMask
+
+    g = torch.Generator().manual_seed(seed)
+    block = UnifiedInteractionBlock(d_model, heads, 4, 0.0).to(torch.bfloat16).eval()
+    with torch.no_grad():
+        for name, parameter in block.named_parameters():
+            if name.endswith("norm.weight"):
+                parameter.add_((0.1 * torch.randn(parameter.shape, generator=g)).to(parameter.dtype))
+            elif name.endswith("bias"):
+                parameter.add_((0.05 * torch.randn(parameter.shape, generator=g)).to(parameter.dtype))
+    x = (0.5 * torch.randn(batch, tokens, d_model, generator=g)).to(torch.bfloat16)
+    padding = torch.rand(batch, tokens, generator=g) < 0.35   # padding anywhere, not a prefix
+    padding[0] = False
+    padding[1, 1:] = True                                      # a single valid token
+    padding[:, 0] = False                                      # every sample keeps its first token
+    roles = torch.randint(0, 8, (tokens,), generator=g)
+    state = {k.replace("attention.", "").replace("ffn.", ""): v.detach() for k, v in block.state_dict().items()}
+    return block, x, padding, roles, state, MetadataAttentionMask(enabled=True)
+
+
+@pytest.mark.parametrize("d_model,heads,tokens,batch", [(128, 4, 70, 5), (256, 8, 150, 4)])
+def test_interaction_block_fused_routes_under_role_masks_and_scattered_padding(device, d_model, heads, tokens, batch):
+    """The reference block as the model runs it: role-based attention mask, padding anywhere in the sequence, updates
+    masked at padded rows. Both fused routes against the oracle's statement of the block; padded rows pass through bit
+    for bit and are never read (NaN there changes nothing)."""
+    block, x, padding, roles, state, mask_module = _symbiosis_block_case(d_model, heads, tokens, batch, seed=d_model + tokens)
+    dense_mask = oracle.metadata_attention_mask(padding, roles)
+    want, want_attn = oracle.interaction_block(x.float(), padding, dense_mask, {k: v.float() for k, v in state.items()},
+                                               num_heads=heads)
+    valid = ~padding
+    block = block.to(device)
+    with torch.no_grad():
+        mask = mask_module(padding.to(device), roles.to(device))
+        two, two_attn = block(x.to(device), padding.to(device), mask)
+        one, none = block(x.to(device), padding.to(device), mask, return_attention_tokens=False)
+        from_dense, _ = block(x.to(device), padding.to(device), dense_mask.to(device))
+        poisoned = x.clone()
+        poisoned[padding] = float("nan")
+        stream = poisoned.to(device)
+        in_place, _ = block(stream, padding.to(device), mask, return_attention_tokens=False, inplace=True)
+    assert none is None and in_place.data_ptr() == stream.data_ptr()
+    torch.testing.assert_close(two_attn.cpu().float()[valid], want_attn[valid], rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(two.cpu().float()[valid], want[valid], rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(one.cpu().float()[valid], want[valid], rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(one.cpu().float(), two.cpu().float(), rtol=2 ** -6, atol=2 ** -6)
+    assert torch.equal(from_dense.cpu(), two.cpu())
+    for result in (two, one, two_attn):
+        assert torch.equal(result.cpu()[padding], x[padding])          # x + update * 0
+    assert torch.equal(in_place.cpu()[valid], one.cpu()[valid])
+    assert torch.isnan(in_place.cpu()[padding].float()).all()
+
+
+def test_interaction_block_routes_agree(device):
+    """fp32 tokens take the module-by-module route (norms, attention layer and feed-forward as separate calls with the
+    padding multiply in torch), bf16 tokens the fused one; both state the same block."""
+    block, x, padding, roles, _, mask_module = _symbiosis_block_case(128, 4, 48, 3, seed=9)
+    block = block.to(device)
+    with torch.no_grad():
+        mask = mask_module(padding.to(device), roles.to(device))
+        fused, fused_attn = block(x.to(device), padding.to(device), mask)
+        plain, plain_attn = block(x.to(device).float(), padding.to(device), mask)
+    valid = ~padding
+    torch.testing.assert_close(plain_attn.cpu()[valid], fused_attn.cpu().float()[valid], rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(plain.cpu()[valid], fused.cpu().float()[valid], rtol=2e-2, atol=2e-2)
+
+
+def test_valid_rows_from_a_padding_mask(device):
+    from taac_2026_amd.api import valid_rows
+
+    g = torch.Generator().manual_seed(2)
+    for batch, tokens in ((7, 100), (3, 32), (5, 513), (1, 1)):
+        padding = torch.rand(batch, tokens, generator=g) < 0.4
+        if batch > 1:
+            padding[1] = True
+        rows, count = valid_rows(None, tokens, padding_mask=padding.to(device))
+        expected = (~padding).flatten().nonzero().flatten()
+        assert int(count.item()) == expected.numel()
+        assert torch.equal(rows[:expected.numel()].cpu().long(), expected)
+        offsets = rows[batch * tokens:batch * tokens + batch + 1].cpu().long()
+        assert torch.equal(offsets, torch.cat([torch.zeros(1, dtype=torch.long), (~padding).sum(1).cumsum(0)]))
+    lengths = torch.tensor([5, 0, 9], dtype=torch.int32)
+    by_len = valid_rows(lengths.to(device), 9)
+    by_mask = valid_rows(None, 9, padding_mask=(torch.arange(9)[None, :] >= lengths[:, None]).to(device))
+    assert int(by_len[1].item()) == int(by_mask[1].item()) == 14 and torch.equal(by_len[0][:14], by_mask[0][:14])
+    with pytest.raises(ValueError, match="key_lengths or padding_mask"):
+        valid_rows(None, 9)
