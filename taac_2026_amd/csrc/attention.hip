@@ -19,10 +19,12 @@
 // online softmax with scale log2(e)/sqrt(d), key j visible iff j < key_lengths[b] (and j <= i when causal),
 // P rounded to the storage dtype before the second product, rows with an empty visible set produce 0.
 #include <math.h>
+#include <stdlib.h>
 
 #include <type_traits>
 
 #include "common.h"
+#include "ts_common.h"
 
 namespace taac {
 namespace {
@@ -496,9 +498,281 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   }
 }
 
+// ------------------------------------------------------------------------------------------------------------------
+// The plain case at head dim 32 (key-length / causal masking only, no row factors, no structured mask): K and V
+// chunks go from global memory straight into LDS (one 1 KB transfer per wavefront and operand, no staging registers,
+// no transposition arithmetic), into two buffers, so that chunk c + 1 is in flight while chunk c is consumed and one
+// barrier per chunk is enough.
+//   K: row-major [64 keys][32 features]; a transfer cannot pad rows, so the four 16-byte pieces of row r are stored
+//      at piece ^ ((r / 4) % 4): the 16 lanes that read the same piece of 16 consecutive rows hit 64 distinct banks.
+//   V: row-major as well. The A operand of O^T += V^T P^T needs, per lane, 8 keys of ONE feature: it is read with
+//      ds_read_b64_tr_b16, which hands element e of lane j of a 16-lane group element j % 4 of the 8-byte row supplied
+//      by lane 4 * e + j / 4 of that group. With lane 4 * e + q pointing at V[k0 + e][f0 + 4 * q ..] lane j receives
+//      V[k0 .. k0 + 3][f0 + j]: four keys of its feature; two such reads make a fragment, in the key order of P.
+// Rows at or beyond the valid length are never requested: the transfer repeats the last valid row (finite values; the
+// scores of those keys are masked), since uninitialised memory could hold NaNs that a zero probability would not cancel.
+// ------------------------------------------------------------------------------------------------------------------
+// lds_dma16 with the source given as a wavefront-uniform base (scalar registers) + a 32-bit per-lane byte offset.
+__device__ __forceinline__ void lds_dma16_offset(const void* base, uint32_t lane_offset, void* lds_wave_base) {
+  const uint32_t lds_base = __builtin_amdgcn_readfirstlane(lds_offset(lds_wave_base));
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %0, %1"
+      :
+      : "v"(lane_offset), "s"(base), "s"(lds_base)
+      : "memory", "m0");
+}
+
+__device__ __forceinline__ void lds_read_tr16(u32x2& dst, uint32_t addr) {
+  asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(dst) : "v"(addr) : "memory");
+}
+
+template <typename T, bool CAUSAL>
+__global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const AttnParams p) {
+  typedef typename Vec8<T>::type vec_t;
+  typedef typename Vec8<T>::half_type vec4_t;
+  constexpr int DP = 32;
+  constexpr int KSTEPS = DP / 16;
+  constexpr int C8 = DP / 8;
+  constexpr int ROWB = DP * 2;                      // bytes per staged row
+  constexpr int TILE_BYTES = kKC * ROWB;            // one operand of one chunk: 4 KB
+  constexpr int BUF_BYTES = 2 * TILE_BYTES;         // K then V
+  constexpr int OROW = DP * 2 + 16;
+  constexpr int OT_BYTES = (kThreads / kWave) * 32 * OROW;
+  static_assert(kKC * C8 == kThreads, "one 16-byte piece per lane and operand");
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * BUF_BYTES > OT_BYTES ? 2 * BUF_BYTES : OT_BYTES];
+
+  const uint32_t logical = xcd_remap(blockIdx.x, p.total);
+  const int qc = static_cast<int>(logical % p.nqc);
+  const int bh = static_cast<int>(logical / p.nqc);
+  const int h = bh % p.H;
+  const int b = bh / p.H;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int lane = tid % kWave;
+  const int l32 = lane % 32;
+  const int hh = lane / 32;
+
+  const T* qb = static_cast<const T*>(p.q) + b * p.qs[0] + h * p.qs[1];
+  const T* kb = static_cast<const T*>(p.k) + b * p.ks[0] + h * p.ks[1];
+  const T* vb = static_cast<const T*>(p.v) + b * p.vs[0] + h * p.vs[1];
+  T* ob = static_cast<T*>(p.o) + b * p.os[0] + h * p.os[1];
+
+  int len = p.Tk;
+  if (p.key_lengths != nullptr) {
+    len = p.key_lengths[b];
+    len = len < 0 ? 0 : (len > p.Tk ? p.Tk : len);
+  }
+  const int q_begin = qc * kQB;
+  const int q_valid = p.zero_pad ? (len < p.Tq ? len : p.Tq) : p.Tq;
+  vec_t zero_vec;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) zero_vec[e] = static_cast<T>(0.f);
+  if (q_begin >= q_valid) {  // whole block in the padding: zero-fill its rows, or leave them alone
+    if (p.lse != nullptr) {
+      for (int idx = tid; idx < kQB; idx += kThreads)
+        if (q_begin + idx < p.Tq) p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Tq + q_begin + idx] = -INFINITY;
+    }
+    if (p.zero_pad == 2) return;
+    for (int idx = tid; idx < kQB * C8; idx += kThreads) {
+      const int row = q_begin + idx / C8;
+      if (row < p.Tq) *reinterpret_cast<vec_t*>(ob + row * p.os[2] + (idx % C8) * 8) = zero_vec;
+    }
+    return;
+  }
+  int kv_end = len;
+  if (CAUSAL) kv_end = kv_end < q_begin + kQB ? kv_end : q_begin + kQB;
+
+  const int qi = q_begin + wave * 32 + l32;
+  vec_t qf[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s)
+    qf[s] = qi < q_valid ? *reinterpret_cast<const vec_t*>(qb + qi * p.qs[2] + 16 * s + 8 * hh) : zero_vec;
+
+  f32x16 oacc;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) oacc[j] = 0.f;
+  float m_run = -INFINITY;
+  float l_run = 0.f;
+  const float c = p.scale_log2;
+  int wave_kv_end = kv_end;
+  if (CAUSAL) {
+    const int wlim = q_begin + wave * 32 + 32;
+    wave_kv_end = wave_kv_end < wlim ? wave_kv_end : wlim;
+  }
+  if (q_begin + wave * 32 >= q_valid) wave_kv_end = 0;
+
+  // The lane's piece of a chunk: slot 64 * wave + lane = (row, stored piece); K's stored piece holds piece ^ swizzle.
+  // Sources are addressed as a wavefront-uniform base + a 32-bit per-lane byte offset (the host checks that the
+  // offsets fit): row * stride with a 24-bit multiply, plus the piece.
+  const int slot = wave * kWave + lane;
+  const int srow = slot / C8;
+  const uint32_t k_piece_off = static_cast<uint32_t>(((slot % C8) ^ ((srow / 4) % 4)) * 16);
+  const uint32_t v_piece_off = static_cast<uint32_t>((slot % C8) * 16);
+  const uint32_t k_row_bytes = static_cast<uint32_t>(p.ks[2]) * 2u, v_row_bytes = static_cast<uint32_t>(p.vs[2]) * 2u;
+  auto issue = [&](int chunk, int buffer) {
+    int row = chunk * kKC + srow;
+    row = row < kv_end ? row : kv_end - 1;  // kv_end >= 1 here
+    uint8_t* dst = smem + buffer * BUF_BYTES + wave * (kWave * 16);
+    lds_dma16_offset(kb, __umul24(static_cast<uint32_t>(row), k_row_bytes) + k_piece_off, dst);
+    lds_dma16_offset(vb, __umul24(static_cast<uint32_t>(row), v_row_bytes) + v_piece_off, dst + TILE_BYTES);
+  };
+  // Per-lane LDS offsets of the fragment reads (relative to the chunk buffer).
+  const uint32_t smem_off = lds_offset(smem);
+  //   K fragment (tile, k-step s): row tile * 32 + l32 (tile * 32 keeps (row / 4) % 4), piece (2 * s + hh) ^ ((row / 4) % 4):
+  //   the offset of k-step 1 is that of k-step 0 with bit 5 flipped
+  const uint32_t k_off0 = static_cast<uint32_t>(l32 * ROWB + ((hh ^ ((l32 / 4) % 4)) * 16));
+  //   V transposed read: group g = lane / 16 covers features 16 * (g % 2) .. + 15 and keys 4 * (g / 2) .. + 3 of a
+  //   16-key group; lane r = lane % 16 of the group points at key r / 4, features 4 * (r % 4) .. + 3
+  const uint32_t v_off = static_cast<uint32_t>(TILE_BYTES + (4 * (lane / 32) + (lane % 16) / 4) * ROWB +
+                                               (16 * ((lane / 16) % 2) + 4 * (lane % 4)) * 2);
+
+  const int nchunks = (kv_end + kKC - 1) / kKC;
+  if (nchunks > 0) issue(0, 0);
+  int buf = 0;
+  for (int chunk = 0; chunk < nchunks; ++chunk) {
+    vm_wait<0>();     // this wavefront's pieces of the chunk have landed ...
+    __syncthreads();  // ... everyone's have, and everyone is done reading the other buffer
+    if (chunk + 1 < nchunks) issue(chunk + 1, buf ^ 1);
+    const int kc0 = chunk * kKC;
+    const uint32_t base = smem_off + buf * BUF_BYTES;
+    buf ^= 1;
+    if (kc0 >= wave_kv_end) continue;  // wavefront-uniform: nothing visible in this chunk
+    auto update = [&](auto nt_tag) {
+      constexpr int NT = decltype(nt_tag)::value;
+      f32x16 sacc[NT];
+#pragma unroll
+      for (int kt = 0; kt < NT; ++kt) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) sacc[kt][j] = 0.f;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+          const vec_t a = *reinterpret_cast<const vec_t*>(smem + (base - smem_off) + kt * 32 * ROWB + (k_off0 ^ (s * 32)));
+          sacc[kt] = Mfma32<T>::run(a, qf[s], sacc[kt]);
+        }
+      }
+      const int k_last = kc0 + NT * 32;
+      const bool tail = (k_last > kv_end) || (CAUSAL && (k_last - 1 > q_begin + wave * 32));
+      if (tail) {
+#pragma unroll
+        for (int kt = 0; kt < NT; ++kt)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) {
+            const int key = kc0 + kt * 32 + (j / 4) * 8 + hh * 4 + (j % 4);
+            if (key >= kv_end || (CAUSAL && key > qi)) sacc[kt][j] = -INFINITY;
+          }
+      }
+      float mx = sacc[0][0];
+#pragma unroll
+      for (int kt = 0; kt < NT; ++kt)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) mx = fmaxf(mx, sacc[kt][j]);
+      mx = pair_max(mx);
+      const float m_new = fmaxf(m_run, mx);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
+      const float mc = -m_use * c;
+      float rs = 0.f;
+      vec_t pb[NT][2];
+#pragma unroll
+      for (int kt = 0; kt < NT; ++kt) {
+        float pr[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) pr[j] = __builtin_amdgcn_exp2f(fmaf(sacc[kt][j], c, mc));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          pb[kt][0][e] = static_cast<T>(pr[e]);
+          pb[kt][1][e] = static_cast<T>(pr[8 + e]);
+        }
+        rs = frag_sum(pb[kt][0], rs);
+        rs = frag_sum(pb[kt][1], rs);
+      }
+      // V fragments: requested once the scores are dead (registers), in flight during the bookkeeping below
+      u32x2 vt[NT][2][2];
+      const uint32_t v_addr = base + v_off;
+#pragma unroll
+      for (int kt = 0; kt < NT; ++kt)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          lds_read_tr16(vt[kt][s2][0], v_addr + (kt * 32 + s2 * 16) * ROWB);
+          lds_read_tr16(vt[kt][s2][1], v_addr + (kt * 32 + s2 * 16 + 8) * ROWB);
+        }
+      rs = pair_sum(rs);
+      l_run = l_run * alpha + rs;
+      m_run = m_new;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) oacc[j] *= alpha;  // unconditional, see the general kernel
+      // the transposed reads were issued by hand: wait for them by hand (everything of this wavefront's LDS queue);
+      // the fragments are tied to the wait so that their consumers cannot be scheduled above it
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vt[0][0][0]) : : "memory");
+#pragma unroll
+      for (int kt = 0; kt < NT; ++kt)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          asm volatile("" : "+v"(vt[kt][s2][0]));
+          asm volatile("" : "+v"(vt[kt][s2][1]));
+        }
+#pragma unroll
+      for (int kt = 0; kt < NT; ++kt)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const u32x4 bits = {vt[kt][s2][0][0], vt[kt][s2][0][1], vt[kt][s2][1][0], vt[kt][s2][1][1]};
+          oacc = Mfma32<T>::run(__builtin_bit_cast(vec_t, bits), pb[kt][s2], oacc);
+        }
+    };
+    if (kc0 + 32 < wave_kv_end)
+      update(std::integral_constant<int, 2>{});
+    else
+      update(std::integral_constant<int, 1>{});
+  }
+
+  const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+  const float fin = (qi < q_valid) ? inv : 0.f;
+  if (p.lse != nullptr && hh == 0 && qi < p.Tq)
+    p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Tq + qi] =
+        (qi < q_valid && l_run > 0.f) ? (m_run * c + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f : -INFINITY;
+  __syncthreads();  // every wavefront is done with the chunk buffers: they now hold the output tiles
+  uint8_t* tile = smem + wave * (32 * OROW);
+#pragma unroll
+  for (int jq = 0; jq < 4; ++jq) {
+    vec4_t ov;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ov[e] = static_cast<T>(oacc[jq * 4 + e] * fin);
+    *reinterpret_cast<vec4_t*>(tile + l32 * OROW + (jq * 8 + hh * 4) * 2) = ov;
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  constexpr int RPP = kWave / C8;
+  const int c8 = lane % C8;
+  const int q_store_end = p.zero_pad == 2 ? q_valid : p.Tq;
+#pragma unroll
+  for (int pass = 0; pass < 32 / RPP; ++pass) {
+    const int row = pass * RPP + lane / C8;
+    const int q_row = q_begin + wave * 32 + row;
+    const vec_t v = *reinterpret_cast<const vec_t*>(tile + row * OROW + c8 * 16);
+    if (q_row < q_store_end) *reinterpret_cast<vec_t*>(ob + q_row * p.os[2] + c8 * 8) = v;
+  }
+}
+
 template <typename T, int DP>
 void launch(const AttnParams& p, bool causal, hipStream_t s) {
   const bool scaled = p.q_row_scale != nullptr || p.k_row_scale != nullptr || p.q_col_scale != nullptr;
+  // TAAC_ATTN_STAGING=registers keeps the general kernel for the plain head-dim-32 case too (comparison knob).
+  static const bool dma_staging = [] {
+    const char* env = getenv("TAAC_ATTN_STAGING");
+    return !(env != nullptr && env[0] == 'r');
+  }();
+  // 32-bit source offsets with a 24-bit row multiply: row strides below 8 M elements, sequences below 2^31 bytes
+  const bool small_offsets = p.ks[2] < (1 << 22) && p.vs[2] < (1 << 22) && p.Tk < (1 << 22) &&
+                             static_cast<int64_t>(p.Tk) * p.ks[2] * 2 < (1ll << 31) &&
+                             static_cast<int64_t>(p.Tk) * p.vs[2] * 2 < (1ll << 31);
+  if (DP == 32 && p.d == 32 && !scaled && p.struct_bits == nullptr && dma_staging && small_offsets) {
+    if (causal)
+      hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+    else
+      hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+    return;
+  }
   if (p.struct_bits != nullptr)
     hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
   else if (causal && scaled)
