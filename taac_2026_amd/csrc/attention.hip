@@ -499,7 +499,7 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 }
 
 // ------------------------------------------------------------------------------------------------------------------
-// The plain case at head dim 32 (key-length / causal masking only, no row factors, no structured mask): K and V
+// The plain case at head dims 32 and 64 (key-length / causal masking only, no row factors, no structured mask): K and V
 // chunks go from global memory straight into LDS (one 1 KB transfer per wavefront and operand, no staging registers,
 // no transposition arithmetic), into two buffers, so that chunk c + 1 is in flight while chunk c is consumed and one
 // barrier per chunk is enough.
@@ -524,23 +524,26 @@ __device__ __forceinline__ void lds_dma16_offset(const void* base, uint32_t lane
       : "memory", "m0");
 }
 
+template <int OFFSET>
 __device__ __forceinline__ void lds_read_tr16(u32x2& dst, uint32_t addr) {
-  asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(dst) : "v"(addr) : "memory");
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFFSET) : "memory");
 }
 
-template <typename T, bool CAUSAL>
+template <typename T, int DP, bool CAUSAL>
 __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const AttnParams p) {
   typedef typename Vec8<T>::type vec_t;
   typedef typename Vec8<T>::half_type vec4_t;
-  constexpr int DP = 32;
+  static_assert(DP == 32 || DP == 64, "row swizzles are written for 64- and 128-byte rows");
   constexpr int KSTEPS = DP / 16;
+  constexpr int MB = DP / 32;
   constexpr int C8 = DP / 8;
   constexpr int ROWB = DP * 2;                      // bytes per staged row
-  constexpr int TILE_BYTES = kKC * ROWB;            // one operand of one chunk: 4 KB
+  constexpr int TILE_BYTES = kKC * ROWB;            // one operand of one chunk
   constexpr int BUF_BYTES = 2 * TILE_BYTES;         // K then V
+  constexpr int PPT = kKC * C8 / kThreads;          // 16-byte pieces per lane, operand and chunk
   constexpr int OROW = DP * 2 + 16;
   constexpr int OT_BYTES = (kThreads / kWave) * 32 * OROW;
-  static_assert(kKC * C8 == kThreads, "one 16-byte piece per lane and operand");
+  static_assert(kKC * C8 % kThreads == 0, "whole transfers per wavefront");
   __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * BUF_BYTES > OT_BYTES ? 2 * BUF_BYTES : OT_BYTES];
 
   const uint32_t logical = xcd_remap(blockIdx.x, p.total);
@@ -590,9 +593,11 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   for (int s = 0; s < KSTEPS; ++s)
     qf[s] = qi < q_valid ? *reinterpret_cast<const vec_t*>(qb + qi * p.qs[2] + 16 * s + 8 * hh) : zero_vec;
 
-  f32x16 oacc;
+  f32x16 oacc[MB];
 #pragma unroll
-  for (int j = 0; j < 16; ++j) oacc[j] = 0.f;
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) oacc[mb][j] = 0.f;
   float m_run = -INFINITY;
   float l_run = 0.f;
   const float c = p.scale_log2;
@@ -603,30 +608,42 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   }
   if (q_begin + wave * 32 >= q_valid) wave_kv_end = 0;
 
-  // The lane's piece of a chunk: slot 64 * wave + lane = (row, stored piece); K's stored piece holds piece ^ swizzle.
-  // Sources are addressed as a wavefront-uniform base + a 32-bit per-lane byte offset (the host checks that the
-  // offsets fit): row * stride with a 24-bit multiply, plus the piece.
+  // Row swizzles (a transfer cannot pad rows): the 16-byte piece `piece` of row r is stored at piece ^ swizzle(r).
+  //   K: (r / 4) % 4 for 64-byte rows, (r / 2) % 8 for 128-byte rows: the 16 lanes that read the same piece of 16
+  //      consecutive rows hit 64 distinct banks.
+  //   V: none for 64-byte rows; 4 * ((r / 2) % 2) for 128-byte rows, which keeps the four rows a 16-lane group of a
+  //      transposed read touches (and the neighbouring group's) on distinct banks.
+  auto k_swizzle = [](int r) -> int { return DP == 32 ? (r / 4) % 4 : (r / 2) % 8; };
+  auto v_swizzle = [](int r) -> int { return DP == 32 ? 0 : 4 * ((r / 2) % 2); };
+  // The lane's pieces of a chunk: slot i * 256 + 64 * wave + lane = (row, stored piece), i < PPT; rows of successive i
+  // are 256 / C8 apart, which leaves the swizzles unchanged. Sources are addressed as a wavefront-uniform base + a
+  // 32-bit per-lane byte offset (the host checks that the offsets fit): row * stride with a 24-bit multiply + the piece.
   const int slot = wave * kWave + lane;
   const int srow = slot / C8;
-  const uint32_t k_piece_off = static_cast<uint32_t>(((slot % C8) ^ ((srow / 4) % 4)) * 16);
-  const uint32_t v_piece_off = static_cast<uint32_t>((slot % C8) * 16);
+  const uint32_t k_piece_off = static_cast<uint32_t>(((slot % C8) ^ k_swizzle(srow)) * 16);
+  const uint32_t v_piece_off = static_cast<uint32_t>(((slot % C8) ^ v_swizzle(srow)) * 16);
   const uint32_t k_row_bytes = static_cast<uint32_t>(p.ks[2]) * 2u, v_row_bytes = static_cast<uint32_t>(p.vs[2]) * 2u;
   auto issue = [&](int chunk, int buffer) {
-    int row = chunk * kKC + srow;
-    row = row < kv_end ? row : kv_end - 1;  // kv_end >= 1 here
-    uint8_t* dst = smem + buffer * BUF_BYTES + wave * (kWave * 16);
-    lds_dma16_offset(kb, __umul24(static_cast<uint32_t>(row), k_row_bytes) + k_piece_off, dst);
-    lds_dma16_offset(vb, __umul24(static_cast<uint32_t>(row), v_row_bytes) + v_piece_off, dst + TILE_BYTES);
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+      int row = chunk * kKC + srow + i * (kThreads / C8);
+      row = row < kv_end ? row : kv_end - 1;  // kv_end >= 1 here
+      uint8_t* dst = smem + buffer * BUF_BYTES + i * (kThreads * 16) + wave * (kWave * 16);
+      lds_dma16_offset(kb, __umul24(static_cast<uint32_t>(row), k_row_bytes) + k_piece_off, dst);
+      lds_dma16_offset(vb, __umul24(static_cast<uint32_t>(row), v_row_bytes) + v_piece_off, dst + TILE_BYTES);
+    }
   };
   // Per-lane LDS offsets of the fragment reads (relative to the chunk buffer).
   const uint32_t smem_off = lds_offset(smem);
-  //   K fragment (tile, k-step s): row tile * 32 + l32 (tile * 32 keeps (row / 4) % 4), piece (2 * s + hh) ^ ((row / 4) % 4):
-  //   the offset of k-step 1 is that of k-step 0 with bit 5 flipped
-  const uint32_t k_off0 = static_cast<uint32_t>(l32 * ROWB + ((hh ^ ((l32 / 4) % 4)) * 16));
-  //   V transposed read: group g = lane / 16 covers features 16 * (g % 2) .. + 15 and keys 4 * (g / 2) .. + 3 of a
-  //   16-key group; lane r = lane % 16 of the group points at key r / 4, features 4 * (r % 4) .. + 3
-  const uint32_t v_off = static_cast<uint32_t>(TILE_BYTES + (4 * (lane / 32) + (lane % 16) / 4) * ROWB +
-                                               (16 * ((lane / 16) % 2) + 4 * (lane % 4)) * 2);
+  //   K fragment (tile, k-step s): row tile * 32 + l32 (tile * 32 leaves the swizzle alone), piece (2 * s + hh) ^ swizzle:
+  //   the offset of k-step s is that of k-step 0 with s * 32 XORed in
+  const uint32_t k_off0 = static_cast<uint32_t>(l32 * ROWB + ((hh ^ k_swizzle(l32)) * 16));
+  //   V transposed read: group g = lane / 16 covers features 16 * (g % 2) .. + 15 (of row block mb) and keys
+  //   4 * (g / 2) .. + 3 of a 16-key group; lane r = lane % 16 of the group points at key r / 4, features
+  //   4 * (r % 4) .. + 3 = half of piece 2 * (g % 2) + (r % 4) / 2 (+ 4 * mb: XORs 64 * mb into the address)
+  const int v_key = 4 * (lane / 32) + (lane % 16) / 4;
+  const uint32_t v_off = static_cast<uint32_t>(
+      TILE_BYTES + v_key * ROWB + ((2 * ((lane / 16) % 2) + (lane % 4) / 2) ^ v_swizzle(v_key)) * 16 + (lane % 2) * 8);
 
   const int nchunks = (kv_end + kKC - 1) / kKC;
   if (nchunks > 0) issue(0, 0);
@@ -688,38 +705,43 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
         rs = frag_sum(pb[kt][0], rs);
         rs = frag_sum(pb[kt][1], rs);
       }
-      // V fragments: requested once the scores are dead (registers), in flight during the bookkeeping below
-      u32x2 vt[NT][2][2];
+      // V fragments of one row block at a time: requested once the scores are dead (registers), in flight during the
+      // bookkeeping below
       const uint32_t v_addr = base + v_off;
-#pragma unroll
-      for (int kt = 0; kt < NT; ++kt)
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          lds_read_tr16(vt[kt][s2][0], v_addr + (kt * 32 + s2 * 16) * ROWB);
-          lds_read_tr16(vt[kt][s2][1], v_addr + (kt * 32 + s2 * 16 + 8) * ROWB);
-        }
-      rs = pair_sum(rs);
-      l_run = l_run * alpha + rs;
-      m_run = m_new;
-#pragma unroll
-      for (int j = 0; j < 16; ++j) oacc[j] *= alpha;  // unconditional, see the general kernel
-      // the transposed reads were issued by hand: wait for them by hand (everything of this wavefront's LDS queue);
-      // the fragments are tied to the wait so that their consumers cannot be scheduled above it
-      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vt[0][0][0]) : : "memory");
-#pragma unroll
-      for (int kt = 0; kt < NT; ++kt)
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          asm volatile("" : "+v"(vt[kt][s2][0]));
-          asm volatile("" : "+v"(vt[kt][s2][1]));
+      static_for<MB>([&](auto mc_tag) {
+        constexpr int mb = decltype(mc_tag)::value;
+        const uint32_t v_addr_mb = v_addr ^ (mb * 64);
+        u32x2 vt[NT][2][2];
+        static_for<NT * 2>([&](auto ic) {
+          constexpr int kt = decltype(ic)::value / 2, s2 = decltype(ic)::value % 2;
+          lds_read_tr16<(kt * 32 + s2 * 16) * ROWB>(vt[kt][s2][0], v_addr_mb);
+          lds_read_tr16<(kt * 32 + s2 * 16 + 8) * ROWB>(vt[kt][s2][1], v_addr_mb);
+        });
+        if (mb == 0) {
+          rs = pair_sum(rs);
+          l_run = l_run * alpha + rs;
+          m_run = m_new;
         }
 #pragma unroll
-      for (int kt = 0; kt < NT; ++kt)
+        for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;  // unconditional, see the general kernel
+        // the transposed reads were issued by hand: wait for them by hand (everything of this wavefront's LDS queue);
+        // the fragments are tied to the wait so that their consumers cannot be scheduled above it
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vt[0][0][0]) : : "memory");
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          const u32x4 bits = {vt[kt][s2][0][0], vt[kt][s2][0][1], vt[kt][s2][1][0], vt[kt][s2][1][1]};
-          oacc = Mfma32<T>::run(__builtin_bit_cast(vec_t, bits), pb[kt][s2], oacc);
-        }
+        for (int kt = 0; kt < NT; ++kt)
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            asm volatile("" : "+v"(vt[kt][s2][0]));
+            asm volatile("" : "+v"(vt[kt][s2][1]));
+          }
+#pragma unroll
+        for (int kt = 0; kt < NT; ++kt)
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            const u32x4 bits = {vt[kt][s2][0][0], vt[kt][s2][0][1], vt[kt][s2][1][0], vt[kt][s2][1][1]};
+            oacc[mb] = Mfma32<T>::run(__builtin_bit_cast(vec_t, bits), pb[kt][s2], oacc[mb]);
+          }
+      });
     };
     if (kc0 + 32 < wave_kv_end)
       update(std::integral_constant<int, 2>{});
@@ -735,11 +757,14 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   __syncthreads();  // every wavefront is done with the chunk buffers: they now hold the output tiles
   uint8_t* tile = smem + wave * (32 * OROW);
 #pragma unroll
-  for (int jq = 0; jq < 4; ++jq) {
-    vec4_t ov;
+  for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) ov[e] = static_cast<T>(oacc[jq * 4 + e] * fin);
-    *reinterpret_cast<vec4_t*>(tile + l32 * OROW + (jq * 8 + hh * 4) * 2) = ov;
+    for (int jq = 0; jq < 4; ++jq) {
+      vec4_t ov;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ov[e] = static_cast<T>(oacc[mb][jq * 4 + e] * fin);
+      *reinterpret_cast<vec4_t*>(tile + l32 * OROW + (mb * 32 + jq * 8 + hh * 4) * 2) = ov;
+    }
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   constexpr int RPP = kWave / C8;
@@ -766,12 +791,14 @@ void launch(const AttnParams& p, bool causal, hipStream_t s) {
   const bool small_offsets = p.ks[2] < (1 << 22) && p.vs[2] < (1 << 22) && p.Tk < (1 << 22) &&
                              static_cast<int64_t>(p.Tk) * p.ks[2] * 2 < (1ll << 31) &&
                              static_cast<int64_t>(p.Tk) * p.vs[2] * 2 < (1ll << 31);
-  if (DP == 32 && p.d == 32 && !scaled && p.struct_bits == nullptr && dma_staging && small_offsets) {
-    if (causal)
-      hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, true>), dim3(p.total), dim3(kThreads), 0, s, p);
-    else
-      hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, false>), dim3(p.total), dim3(kThreads), 0, s, p);
-    return;
+  if constexpr (DP == 32 || DP == 64) {
+    if (p.d == DP && !scaled && p.struct_bits == nullptr && dma_staging && small_offsets) {
+      if (causal)
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+      else
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+      return;
+    }
   }
   if (p.struct_bits != nullptr)
     hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
