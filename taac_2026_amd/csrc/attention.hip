@@ -529,7 +529,7 @@ __device__ __forceinline__ void lds_read_tr16(u32x2& dst, uint32_t addr) {
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFFSET) : "memory");
 }
 
-template <typename T, int DP, bool CAUSAL>
+template <typename T, int DP, bool CAUSAL, bool SCALED>
 __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const AttnParams p) {
   typedef typename Vec8<T>::type vec_t;
   typedef typename Vec8<T>::half_type vec4_t;
@@ -590,8 +590,14 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   const int qi = q_begin + wave * 32 + l32;
   vec_t qf[KSTEPS];
 #pragma unroll
-  for (int s = 0; s < KSTEPS; ++s)
+  for (int s = 0; s < KSTEPS; ++s) {
     qf[s] = qi < q_valid ? *reinterpret_cast<const vec_t*>(qb + qi * p.qs[2] + 16 * s + 8 * hh) : zero_vec;
+    if (SCALED && p.q_col_scale != nullptr) {
+      const float* cf = p.q_col_scale + h * p.d + 16 * s + 8 * hh;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<T>(static_cast<float>(qf[s][e]) * cf[e]);
+    }
+  }
 
   f32x16 oacc[MB];
 #pragma unroll
@@ -600,7 +606,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
     for (int j = 0; j < 16; ++j) oacc[mb][j] = 0.f;
   float m_run = -INFINITY;
   float l_run = 0.f;
-  const float c = p.scale_log2;
+  float c = p.scale_log2;  // SCALED: the query's row factor joins the lane's softmax scale
+  if (SCALED && p.q_row_scale != nullptr && qi < q_valid) c *= p.q_row_scale[static_cast<int64_t>(b) * p.Tq + qi];
   int wave_kv_end = kv_end;
   if (CAUSAL) {
     const int wlim = q_begin + wave * 32 + 32;
@@ -623,14 +630,36 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   const uint32_t k_piece_off = static_cast<uint32_t>(((slot % C8) ^ k_swizzle(srow)) * 16);
   const uint32_t v_piece_off = static_cast<uint32_t>(((slot % C8) ^ v_swizzle(srow)) * 16);
   const uint32_t k_row_bytes = static_cast<uint32_t>(p.ks[2]) * 2u, v_row_bytes = static_cast<uint32_t>(p.vs[2]) * 2u;
+  // SCALED with a key factor: the K rows are multiplied by it on their way into LDS, so they go through registers (into
+  // the same swizzled slots) while V still takes the direct route.
+  const bool scale_keys = SCALED && p.k_row_scale != nullptr;
+  vec_t kreg[SCALED ? PPT : 1];
+  float kfac[SCALED ? PPT : 1];
   auto issue = [&](int chunk, int buffer) {
 #pragma unroll
     for (int i = 0; i < PPT; ++i) {
       int row = chunk * kKC + srow + i * (kThreads / C8);
       row = row < kv_end ? row : kv_end - 1;  // kv_end >= 1 here
       uint8_t* dst = smem + buffer * BUF_BYTES + i * (kThreads * 16) + wave * (kWave * 16);
-      lds_dma16_offset(kb, __umul24(static_cast<uint32_t>(row), k_row_bytes) + k_piece_off, dst);
+      if (scale_keys) {
+        kreg[SCALED ? i : 0] = *reinterpret_cast<const vec_t*>(reinterpret_cast<const uint8_t*>(kb) +
+                                                              __umul24(static_cast<uint32_t>(row), k_row_bytes) + k_piece_off);
+        kfac[SCALED ? i : 0] = p.k_row_scale[static_cast<int64_t>(b) * p.Tk + row];
+      } else {
+        lds_dma16_offset(kb, __umul24(static_cast<uint32_t>(row), k_row_bytes) + k_piece_off, dst);
+      }
       lds_dma16_offset(vb, __umul24(static_cast<uint32_t>(row), v_row_bytes) + v_piece_off, dst + TILE_BYTES);
+    }
+  };
+  // The K pieces fetched by issue() for `buffer`, scaled and stored at this lane's slots.
+  auto commit_keys = [&](int buffer) {
+    if (!scale_keys) return;
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+      vec_t v = kreg[SCALED ? i : 0];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = static_cast<T>(static_cast<float>(v[e]) * kfac[SCALED ? i : 0]);
+      *reinterpret_cast<vec_t*>(smem + buffer * BUF_BYTES + i * (kThreads * 16) + wave * (kWave * 16) + lane * 16) = v;
     }
   };
   // Per-lane LDS offsets of the fragment reads (relative to the chunk buffer).
@@ -646,16 +675,23 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
       TILE_BYTES + v_key * ROWB + ((2 * ((lane / 16) % 2) + (lane % 4) / 2) ^ v_swizzle(v_key)) * 16 + (lane % 2) * 8);
 
   const int nchunks = (kv_end + kKC - 1) / kKC;
-  if (nchunks > 0) issue(0, 0);
+  if (nchunks > 0) {
+    issue(0, 0);
+    commit_keys(0);
+  }
   int buf = 0;
   for (int chunk = 0; chunk < nchunks; ++chunk) {
     vm_wait<0>();     // this wavefront's pieces of the chunk have landed ...
     __syncthreads();  // ... everyone's have, and everyone is done reading the other buffer
-    if (chunk + 1 < nchunks) issue(chunk + 1, buf ^ 1);
+    const bool more = chunk + 1 < nchunks;
+    if (more) issue(chunk + 1, buf ^ 1);
     const int kc0 = chunk * kKC;
     const uint32_t base = smem_off + buf * BUF_BYTES;
     buf ^= 1;
-    if (kc0 >= wave_kv_end) continue;  // wavefront-uniform: nothing visible in this chunk
+    if (kc0 >= wave_kv_end) {  // wavefront-uniform: nothing visible in this chunk
+      if (more) commit_keys(buf);
+      continue;
+    }
     auto update = [&](auto nt_tag) {
       constexpr int NT = decltype(nt_tag)::value;
       f32x16 sacc[NT];
@@ -747,6 +783,7 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
       update(std::integral_constant<int, 2>{});
     else
       update(std::integral_constant<int, 1>{});
+    if (more) commit_keys(buf);  // the next chunk's K, fetched before the update: the barrier above publishes it
   }
 
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
@@ -792,11 +829,15 @@ void launch(const AttnParams& p, bool causal, hipStream_t s) {
                              static_cast<int64_t>(p.Tk) * p.ks[2] * 2 < (1ll << 31) &&
                              static_cast<int64_t>(p.Tk) * p.vs[2] * 2 < (1ll << 31);
   if constexpr (DP == 32 || DP == 64) {
-    if (p.d == DP && !scaled && p.struct_bits == nullptr && dma_staging && small_offsets) {
-      if (causal)
-        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+    if (p.d == DP && p.struct_bits == nullptr && dma_staging && small_offsets) {
+      if (causal && scaled)
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+      else if (causal)
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, true, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+      else if (scaled)
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
       else
-        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, false>), dim3(p.total), dim3(kThreads), 0, s, p);
       return;
     }
   }
