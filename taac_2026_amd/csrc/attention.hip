@@ -820,10 +820,8 @@ template <typename T, int DP>
 void launch(const AttnParams& p, bool causal, hipStream_t s) {
   const bool scaled = p.q_row_scale != nullptr || p.k_row_scale != nullptr || p.q_col_scale != nullptr;
   // TAAC_ATTN_STAGING=registers keeps the general kernel for the plain head-dim-32 case too (comparison knob).
-  static const bool dma_staging = [] {
-    const char* env = getenv("TAAC_ATTN_STAGING");
-    return !(env != nullptr && env[0] == 'r');
-  }();
+  const char* staging_env = getenv("TAAC_ATTN_STAGING");  // read per call: tests compare the two kernels in one process
+  const bool dma_staging = !(staging_env != nullptr && staging_env[0] == 'r');
   // 32-bit source offsets with a 24-bit row multiply: row strides below 8 M elements, sequences below 2^31 bytes
   const bool small_offsets = p.ks[2] < (1 << 22) && p.vs[2] < (1 << 22) && p.Tk < (1 << 22) &&
                              static_cast<int64_t>(p.Tk) * p.ks[2] * 2 < (1ll << 31) &&

@@ -208,3 +208,38 @@ def test_row_factors_of_queries_and_keys(device, dim, tokens, causal):
     torch.testing.assert_close(only_col.float(), expected_oc.float(), **BF16_TOL)
     with pytest.raises(ValueError, match="q_col_scale"):
         hip_flash_attention_kernel(*args, q_col_scale=col[:-1].contiguous().to(device))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("head_dim", [32, 64])
+@pytest.mark.parametrize("causal", [False, True])
+def test_direct_transfer_kernel_equals_general_kernel_bit_for_bit(device, monkeypatch, dtype, head_dim, causal):
+    """Head dims 32 and 64 run a kernel that stages K and V by direct global->LDS transfers (swizzled rows, transposed
+    LDS reads); TAAC_ATTN_STAGING=registers selects the general kernel. Same arithmetic in the same order: identical
+    results, for ragged lengths (0, 1, not a multiple of the chunk), strided views of a packed projection, row factors
+    and the log-sum-exp output of the training forward."""
+    from taac_2026_amd.api import flash_attention
+    from taac_2026_amd.accelerators.attention import hip_flash_attention_kernel
+
+    g = torch.Generator().manual_seed(head_dim + int(causal))
+    batch, heads, tokens = 5, 3, 200
+    qkv = torch.randn(batch, tokens, 3 * heads * head_dim, generator=g).to(dtype).to(device)
+    q, k, v = (t.view(batch, tokens, heads, head_dim).transpose(1, 2) for t in qkv.chunk(3, dim=-1))
+    lengths = torch.tensor([200, 0, 1, 65, 130], dtype=torch.int32, device=device)
+    q_rows = (0.5 + torch.rand(batch, tokens, generator=g)).to(device)
+    k_rows = (0.5 + torch.rand(batch, tokens, generator=g)).to(device)
+    q_cols = (0.5 + torch.rand(heads * head_dim, generator=g)).to(device)
+
+    def run():
+        with torch.no_grad():
+            plain = flash_attention(q, k, v, key_lengths=lengths, is_causal=causal, zero_padded_queries=True)
+            full = flash_attention(q, k, v, is_causal=causal)
+            scaled = hip_flash_attention_kernel(q, k, v, lengths, is_causal=causal, zero_padded_queries=True,
+                                                q_row_scale=q_rows, k_row_scale=k_rows, q_col_scale=q_cols)
+        return plain, full, scaled
+
+    direct = run()
+    monkeypatch.setenv("TAAC_ATTN_STAGING", "registers")
+    general = run()
+    for a, b in zip(direct, general):
+        assert torch.equal(a, b)
