@@ -36,6 +36,12 @@ Puiching-Memory/TAAC_2026). How each function is pinned, independently of its ow
                       compositions of library routines F.linear, F.silu, the functions above; float64 loop brute
                       force on tiny shapes for swiglu_ffn; the reference holds no numeric test for these
                       (tests/contract/experiments/test_packages.py:170-192 checks shapes and finiteness only).
+  candidate_readout / interaction_block
+                      compositions of the functions above as the reference's modules write them (experiments/symbiosis/
+                      pooling.py:24-32, model.py:217-222, backbone.py:58-68); candidate_readout is pinned by a float64
+                      loop and special cases (no candidate -> zero third, all-padded sample -> zero mean, no norms ->
+                      picked rows and plain masked mean); qk_norm_rope and embedding_bag_mean additionally by the
+                      pure-Python float64 vectors of tests/golden/qk_rope_embedding_small.json.
   fp8 emulation       PARITY UNPINNED by the reference (it has no FP8 code). Defined by the configuration text:
                       s = amax/448, q = (t/s).to(float8_e4m3fn), y = (qa.float() @ qw.float().T) * s_a * s_w.
                       The e4m3 rounding itself is pinned against an exhaustive decode table of all 256 codes and
