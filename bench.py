@@ -529,6 +529,8 @@ def main() -> None:
     parser.add_argument("--only-layer-variants", action="store_true",
                         help="time only the backbone with the reference layers' query / key norm (and rotary embedding) "
                              "and print those figures (for kernel traces of that mode)")
+    parser.add_argument("--only-kernels", action="store_true",
+                        help="time only the stand-alone kernels of one block (short run for hardware-counter collection)")
     parser.add_argument("--only-reference-block", action="store_true",
                         help="time only the reference model's block (role mask, scattered padding) and print those figures")
     args = parser.parse_args()
@@ -546,6 +548,10 @@ def main() -> None:
         return
     if args.only_layer_variants:
         print(json.dumps({"reference_layer_variants": _qk_variant_figures(device, args.batch, args.steps)}))
+        return
+    if args.only_kernels:
+        inputs = workloads.backbone_inputs(batch=args.batch)
+        print(json.dumps({"kernels": _kernel_breakdown(inputs, device, iters=6)}))
         return
     if args.only_reference_block:
         print(json.dumps({"reference_block": _reference_block_figures(device, args.batch, 10)}))
