@@ -512,23 +512,6 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 // Rows at or beyond the valid length are never requested: the transfer repeats the last valid row (finite values; the
 // scores of those keys are masked), since uninitialised memory could hold NaNs that a zero probability would not cancel.
 // ------------------------------------------------------------------------------------------------------------------
-// lds_dma16 with the source given as a wavefront-uniform base (scalar registers) + a 32-bit per-lane byte offset.
-__device__ __forceinline__ void lds_dma16_offset(const void* base, uint32_t lane_offset, void* lds_wave_base) {
-  const uint32_t lds_base = __builtin_amdgcn_readfirstlane(lds_offset(lds_wave_base));
-  asm volatile(
-      "s_mov_b32 m0, %2\n\t"
-      "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %0, %1"
-      :
-      : "v"(lane_offset), "s"(base), "s"(lds_base)
-      : "memory", "m0");
-}
-
-template <int OFFSET>
-__device__ __forceinline__ void lds_read_tr16(u32x2& dst, uint32_t addr) {
-  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFFSET) : "memory");
-}
-
 template <typename T, int DP, bool CAUSAL, bool SCALED>
 __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const AttnParams p) {
   typedef typename Vec8<T>::type vec_t;

@@ -11,11 +11,12 @@
 // All products are formed transposed, as in the forward kernel: the streamed operand is the MFMA A operand (rows from
 // LDS), the lane-owned operand the B operand (registers), so the accumulator holds one owned column per lane and the
 // 16 registers run over the streamed rows (register r <-> row (r / 4) * 8 + hh * 4 + r % 4 of a 32-row tile). The
-// second product of each pair consumes those values as a B operand; the streamed A operand for it is staged
-// transposed with its 16-row groups permuted to that register order (vt_pos16).
+// second product of each pair consumes those values as a B operand; its streamed A operand is the same chunk read
+// column-wise with ds_read_b64_tr_b16, at row offsets that follow that register order, so every chunk is staged once,
+// row-major, and nothing is transposed on the way into LDS.
 #include <math.h>
 
-#include "common.h"
+#include "ts_common.h"
 
 namespace taac {
 namespace {
@@ -72,81 +73,94 @@ __device__ __forceinline__ uint32_t pack2(T lo, T hi) {
          (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, hi)) << 16);
 }
 
-// Position of row k (0..15 inside a 16-row group) in a transposed, permuted LDS row: accumulator order.
-__device__ __forceinline__ int vt_pos16(int k) { return ((k >> 2) & 1) * 8 + (k >> 3) * 4 + (k & 3); }
+// A streamed chunk (kChunk rows of DP features) lies row-major and unpadded in LDS, the 16-byte pieces of row r stored
+// at piece ^ row_swizzle(r), and serves two kinds of reads without bank conflicts:
+//   rows as MFMA A operands (lane l32 reads one piece of row l32: 16 consecutive rows of one piece cover all banks);
+//   columns as MFMA A operands through ds_read_b64_tr_b16: a 16-lane group reads 32 contiguous bytes of four
+//   consecutive rows and every lane receives four rows of one feature (see streamed_column_offset below).
+// +32 rows leave the swizzle unchanged, +16 rows too, +8 rows flip kSwizzleBit8 of it.
+template <int DP>
+__device__ __forceinline__ int row_swizzle(int r) {
+  static_assert(DP == 32 || DP == 64, "row swizzles are written for 64- and 128-byte rows");
+  return DP == 32 ? (r >> 2) & 3 : ((r >> 1) & 7) ^ (((r >> 1) & 1) << 2);
+}
+template <int DP>
+struct SwizzleStep {
+  static constexpr uint32_t kRows8 = (DP == 32 ? 2 : 4) * 16;  // address bits that +8 rows flip
+};
 
-// Staging of a chunk of streamed rows is split into a register fetch and an LDS commit, so that the global loads of
-// chunk c + 1 are in flight while chunk c is being consumed.
-//
-// RowStager: rows [row0, row0 + kChunk) of a [rows, d] matrix (row stride `stride`) -> dst[row][DP + 8]; rows at or
-// beyond row_end and features at or beyond d are zeros.
-template <typename T, int DP>
-struct RowStager {
+// Staging of one streamed operand. DMA: the chunk goes from global memory straight into LDS (one 1 KB transfer per
+// wavefront and piece slot, no staging registers); rows at or beyond row_end repeat the last valid row, whose products
+// the callers cancel (finite values times a zero probability); needs d == DP and 32-bit source offsets. Otherwise the
+// chunk travels through registers (fetch, then commit after the barrier), with zeros for rows at or beyond row_end and
+// features at or beyond d. The lane's slot i * 256 + tid is (row slot / C8, stored piece slot % C8).
+template <typename T, int DP, bool DMA>
+struct Streamed {
   typedef typename Vec8<T>::type vec_t;
-  static constexpr int C8 = DP / 8, STR = DP + 8;
-  static constexpr int N = (kChunk * C8 + kThreads - 1) / kThreads;
-  vec_t reg[N];
-  __device__ __forceinline__ void fetch(const T* __restrict__ base, int64_t stride, int row0, int row_end, int d, int tid) {
+  static constexpr int C8 = DP / 8, ROWB = DP * 2, TILE_BYTES = kChunk * ROWB;
+  static constexpr int PPT = kChunk * C8 / kThreads;
+  static_assert(kChunk * C8 % kThreads == 0, "whole transfers per wavefront");
+  const T* base;
+  int64_t stride;
+  int srow, piece;          // the lane's row inside a chunk (slot 0) and the logical piece stored at its slot
+  uint32_t row_bytes;
+  vec_t reg[DMA ? 1 : PPT];
+  __device__ __forceinline__ void init(const T* b, int64_t st, int tid) {
+    base = b;
+    stride = st;
+    srow = tid / C8;
+    piece = (tid % C8) ^ row_swizzle<DP>(srow);
+    row_bytes = static_cast<uint32_t>(st) * 2u;
+  }
+  __device__ __forceinline__ void fetch(int row0, int row_end, int d, uint8_t* tile, int tid) {
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-      const int idx = tid + i * kThreads;
-      const int row = row0 + idx / C8, c8 = idx % C8;
-      if (idx < kChunk * C8 && row < row_end && c8 * 8 < d) {
-        reg[i] = *reinterpret_cast<const vec_t*>(base + row * stride + c8 * 8);
+    for (int i = 0; i < PPT; ++i) {
+      int row = row0 + srow + i * (kThreads / C8);
+      if (DMA) {
+        row = row < row_end ? row : row_end - 1;  // row_end >= 1 here
+        lds_dma16_offset(base, __umul24(static_cast<uint32_t>(row), row_bytes) + static_cast<uint32_t>(piece * 16),
+                         tile + i * (kThreads * 16) + (tid / kWave) * (kWave * 16));
+      } else if (row < row_end && piece * 8 < d) {
+        reg[DMA ? 0 : i] = *reinterpret_cast<const vec_t*>(base + row * stride + piece * 8);
       } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) reg[i][e] = static_cast<T>(0.f);
+        for (int e = 0; e < 8; ++e) reg[DMA ? 0 : i][e] = static_cast<T>(0.f);
       }
     }
   }
-  __device__ __forceinline__ void commit(T* __restrict__ dst, int tid) const {
+  __device__ __forceinline__ void commit(uint8_t* tile, int tid) const {
+    if (DMA) return;
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-      const int idx = tid + i * kThreads;
-      if (idx < kChunk * C8) *reinterpret_cast<vec_t*>(&dst[(idx / C8) * STR + (idx % C8) * 8]) = reg[i];
-    }
+    for (int i = 0; i < PPT; ++i) *reinterpret_cast<vec_t*>(tile + i * (kThreads * 16) + tid * 16) = reg[DMA ? 0 : i];
   }
 };
 
-// TransStager: the same rows transposed, dst[feature][pos(row)] with row stride kChunk + 8, the rows of every 16-row
-// group in accumulator order, two neighbouring rows per 32-bit store.
-template <typename T, int DP>
-struct TransStager {
-  typedef typename Vec8<T>::type vec_t;
-  static constexpr int C8 = DP / 8, STR = kChunk + 8;
-  static constexpr int N = ((kChunk / 2) * C8 + kThreads - 1) / kThreads;
-  vec_t reg[N][2];
-  __device__ __forceinline__ void fetch(const T* __restrict__ base, int64_t stride, int row0, int row_end, int d, int tid) {
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-      const int idx = tid + i * kThreads;
-      const int row = row0 + 2 * (idx / C8), c8 = idx % C8;
-      const bool ok = idx < (kChunk / 2) * C8 && c8 * 8 < d;
-#pragma unroll
-      for (int r = 0; r < 2; ++r) {
-        if (ok && row + r < row_end) {
-          reg[i][r] = *reinterpret_cast<const vec_t*>(base + (row + r) * stride + c8 * 8);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) reg[i][r][e] = static_cast<T>(0.f);
-        }
-      }
-    }
-  }
-  __device__ __forceinline__ void commit(T* __restrict__ dst, int tid) const {
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-      const int idx = tid + i * kThreads;
-      if (idx < (kChunk / 2) * C8) {
-        const int r0 = 2 * (idx / C8), c8 = idx % C8;
-        const int pos = (r0 & ~15) + vt_pos16(r0 & 15);  // even; row r0 + 1 lands at pos + 1
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          *reinterpret_cast<uint32_t*>(&dst[(c8 * 8 + e) * STR + pos]) = pack2<T>(reg[i][0][e], reg[i][1][e]);
-      }
-    }
-  }
-};
+// Byte offset (inside a chunk tile) of the lane's row fragment of k-step 0 of a 32-row tile: row l32, piece hh; k-step s
+// is this offset with s * 32 XORed in, the next 32-row tile 32 * ROWB further.
+template <int DP>
+__device__ __forceinline__ uint32_t streamed_row_offset(int l32, int hh) {
+  return static_cast<uint32_t>(l32 * (DP * 2) + ((hh ^ row_swizzle<DP>(l32)) * 16));
+}
+
+// Byte offset of the lane's address for the transposed reads. Accumulator register j of a 32-row tile belongs to row
+// (j / 4) * 8 + hh * 4 + j % 4, so the B operand of the second product (registers 8 s2 .. 8 s2 + 7) runs over rows
+// 16 s2 + hh * 4 + 0..3 and 16 s2 + 8 + hh * 4 + 0..3. The matching A operand holds, for feature l32 (of row block mb),
+// those eight rows: two transposed reads, at row offsets 16 s2 and 16 s2 + 8, in each of which lane r of 16-lane group
+// g points at row hh * 4 + r / 4, features 16 (g % 2) + 4 (r % 4) .. + 3. Row block mb XORs 64 mb into the offset and
+// the read 8 rows further SwizzleStep<DP>::kRows8.
+template <int DP>
+__device__ __forceinline__ uint32_t streamed_column_offset(int lane) {
+  const int row = 4 * (lane / 32) + (lane % 16) / 4;
+  const int piece = 2 * ((lane / 16) % 2) + (lane % 4) / 2;
+  return static_cast<uint32_t>(row * (DP * 2) + ((piece ^ row_swizzle<DP>(row)) * 16) + (lane % 2) * 8);
+}
+
+// A operand of the second product for (32-row tile at byte offset tile_off, k-step s2) from a tile base address.
+template <typename T, int DP, int TILE_OFF>
+__device__ __forceinline__ void read_columns(u32x2 (&frag)[2], uint32_t addr) {
+  lds_read_tr16<TILE_OFF>(frag[0], addr);
+  lds_read_tr16<TILE_OFF + 8 * DP * 2>(frag[1], addr ^ SwizzleStep<DP>::kRows8);
+}
 
 // Owned rows as B-operand fragments: lane (l32, hh) holds features 16 s + 8 hh .. + 7 of row `row` (zeros when !ok).
 template <typename T, int DP>
@@ -193,20 +207,67 @@ __device__ __forceinline__ void store_owned(const f32x16 (&acc)[DP / 32], uint8_
   }
 }
 
-template <typename T, int DP>
-__global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnBwdParams p) {
+// The second product of a 32-row tile: acc[mb] += columns(tile)^T-fragments x b[s2], the column fragments read
+// transposed from the chunk tile at `addr` (tile base + streamed_column_offset), one row block at a time.
+template <typename T, int DP, int TILE_OFF>
+__device__ __forceinline__ void accumulate_columns(f32x16 (&acc)[DP / 32], const typename Vec8<T>::type (&b)[2], uint32_t addr) {
+  typedef typename Vec8<T>::type vec_t;
+  static_for<DP / 32>([&](auto mb_tag) {
+    constexpr int mb = decltype(mb_tag)::value;
+    u32x2 f[2][2];
+    read_columns<T, DP, TILE_OFF>(f[0], addr ^ (mb * 64));
+    read_columns<T, DP, TILE_OFF + 16 * DP * 2>(f[1], addr ^ (mb * 64));
+    // hand-issued reads are awaited by hand; the fragments are tied to the wait so that no consumer moves above it
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f[0][0]), "+v"(f[0][1]), "+v"(f[1][0]), "+v"(f[1][1]) : : "memory");
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      const u32x4 bits = {f[s2][0][0], f[s2][0][1], f[s2][1][0], f[s2][1][1]};
+      acc[mb] = Mfma32<T>::run(__builtin_bit_cast(vec_t, bits), b[s2], acc[mb]);
+    }
+  });
+}
+
+// Same for two accumulators that share the tile position (dV from dO and P, dK from Q and dS).
+template <typename T, int DP, int TILE_OFF>
+__device__ __forceinline__ void accumulate_columns2(f32x16 (&acc_a)[DP / 32], const typename Vec8<T>::type (&b_a)[2],
+                                                    uint32_t addr_a, f32x16 (&acc_b)[DP / 32],
+                                                    const typename Vec8<T>::type (&b_b)[2], uint32_t addr_b) {
+  typedef typename Vec8<T>::type vec_t;
+  static_for<DP / 32>([&](auto mb_tag) {
+    constexpr int mb = decltype(mb_tag)::value;
+    u32x2 fa[2][2], fb[2][2];
+    read_columns<T, DP, TILE_OFF>(fa[0], addr_a ^ (mb * 64));
+    read_columns<T, DP, TILE_OFF + 16 * DP * 2>(fa[1], addr_a ^ (mb * 64));
+    read_columns<T, DP, TILE_OFF>(fb[0], addr_b ^ (mb * 64));
+    read_columns<T, DP, TILE_OFF + 16 * DP * 2>(fb[1], addr_b ^ (mb * 64));
+    asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[1][0]), "+v"(fa[1][1]) : : "memory");
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      const u32x4 bits = {fa[s2][0][0], fa[s2][0][1], fa[s2][1][0], fa[s2][1][1]};
+      acc_a[mb] = Mfma32<T>::run(__builtin_bit_cast(vec_t, bits), b_a[s2], acc_a[mb]);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fb[0][0]), "+v"(fb[0][1]), "+v"(fb[1][0]), "+v"(fb[1][1]) : : "memory");
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      const u32x4 bits = {fb[s2][0][0], fb[s2][0][1], fb[s2][1][0], fb[s2][1][1]};
+      acc_b[mb] = Mfma32<T>::run(__builtin_bit_cast(vec_t, bits), b_b[s2], acc_b[mb]);
+    }
+  });
+}
+
+template <typename T, int DP, bool DMA>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 32 ? 4 : 3))) void attn_bwd_dq_kernel(const AttnBwdParams p) {
   typedef typename Vec8<T>::type vec_t;
   constexpr int KSTEPS = DP / 16, MB = DP / 32;
-  constexpr int RSTR = DP + 8, TSTR = kChunk + 8, OROW = DP * 2 + 16;
-  constexpr int STAGE_BYTES = (2 * kChunk * RSTR + DP * TSTR) * 2;
-  constexpr int TILE_BYTES = (kThreads / kWave) * 32 * OROW;
-  __shared__ __attribute__((aligned(16))) uint8_t smem[STAGE_BYTES > TILE_BYTES ? STAGE_BYTES : TILE_BYTES];
-  T* sK = reinterpret_cast<T*>(smem);   // [kChunk][RSTR]
-  T* sV = sK + kChunk * RSTR;           // [kChunk][RSTR]
-  T* sKt = sV + kChunk * RSTR;          // [DP][TSTR]
+  constexpr int ROWB = DP * 2, TILE_BYTES = kChunk * ROWB, BUF_BYTES = 2 * TILE_BYTES;  // a chunk of K, then of V
+  constexpr int NBUF = DMA ? 2 : 1;  // direct transfers land in the other buffer while this one is consumed
+  constexpr int OROW = DP * 2 + 16;
+  constexpr int OUT_BYTES = (kThreads / kWave) * 32 * OROW;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[NBUF * BUF_BYTES > OUT_BYTES ? NBUF * BUF_BYTES : OUT_BYTES];
 
-  const int blk = static_cast<int>(blockIdx.x % p.nblk);
-  const int bh = static_cast<int>(blockIdx.x / p.nblk);
+  const uint32_t logical = xcd_remap(blockIdx.x, p.total);
+  const int blk = static_cast<int>(logical % p.nblk);
+  const int bh = static_cast<int>(logical / p.nblk);
   const int h = bh % p.H, b = bh / p.H;
   const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave, l32 = lane % 32, hh = lane / 32;
   const T* qb = static_cast<const T*>(p.q) + b * p.qs[0] + h * p.qs[1];
@@ -255,32 +316,44 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnBwdPara
 #pragma unroll
     for (int j = 0; j < 16; ++j) dqacc[mb][j] = 0.f;
 
-  RowStager<T, DP> k_rows, v_rows;
-  TransStager<T, DP> k_cols;
-  auto fetch = [&](int kc0) {
-    k_rows.fetch(kb, p.ks[2], kc0, kv_end, p.d, tid);
-    v_rows.fetch(vb, p.vs[2], kc0, kv_end, p.d, tid);
-    k_cols.fetch(kb, p.ks[2], kc0, kv_end, p.d, tid);
+  Streamed<T, DP, DMA> k_rows, v_rows;
+  k_rows.init(kb, p.ks[2], tid);
+  v_rows.init(vb, p.vs[2], tid);
+  auto fetch = [&](int kc0, int buffer) {
+    k_rows.fetch(kc0, kv_end, p.d, smem + buffer * BUF_BYTES, tid);
+    v_rows.fetch(kc0, kv_end, p.d, smem + buffer * BUF_BYTES + TILE_BYTES, tid);
   };
-  if (kv_end > 0) fetch(0);
+  const uint32_t row_off = streamed_row_offset<DP>(l32, hh);
+  const uint32_t col_off = streamed_column_offset<DP>(lane);
+  if (kv_end > 0) fetch(0, 0);
+  int buf = 0;
   for (int kc0 = 0; kc0 < kv_end; kc0 += kChunk) {
-    if (kc0 > 0) __syncthreads();  // every wavefront is done reading the previous chunk
-    k_rows.commit(sK, tid);
-    v_rows.commit(sV, tid);
-    k_cols.commit(sKt, tid);
-    __syncthreads();
-    if (kc0 + kChunk < kv_end) fetch(kc0 + kChunk);
-#pragma unroll
-    for (int kt = 0; kt < kChunk / 32; ++kt) {
-      if (kc0 + kt * 32 >= kv_end || !wave_active) continue;  // wavefront-uniform
-      if (p.causal && kc0 + kt * 32 > q_begin + wave * 32 + 31) continue;  // every key of the tile lies after the queries
+    if (DMA) {
+      vm_wait<0>();     // this wavefront's pieces of the chunk have landed ...
+      __syncthreads();  // ... everyone's have, and everyone is done reading the other buffer
+      if (kc0 + kChunk < kv_end) fetch(kc0 + kChunk, buf ^ 1);
+    } else {
+      if (kc0 > 0) __syncthreads();  // every wavefront is done reading the previous chunk
+      k_rows.commit(smem, tid);
+      v_rows.commit(smem + TILE_BYTES, tid);
+      __syncthreads();
+      if (kc0 + kChunk < kv_end) fetch(kc0 + kChunk, 0);
+    }
+    const uint8_t* kt_rows = smem + buf * BUF_BYTES;
+    const uint32_t col_addr = lds_offset(kt_rows) + col_off;
+    if (DMA) buf ^= 1;
+    static_for<kChunk / 32>([&](auto kt_tag) {
+      constexpr int kt = decltype(kt_tag)::value;
+      if (kc0 + kt * 32 >= kv_end || !wave_active) return;  // wavefront-uniform
+      if (p.causal && kc0 + kt * 32 > q_begin + wave * 32 + 31) return;  // every key of the tile lies after the queries
       f32x16 sacc, dpacc;
 #pragma unroll
       for (int j = 0; j < 16; ++j) sacc[j] = dpacc[j] = 0.f;
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) {
-        const vec_t ka = *reinterpret_cast<const vec_t*>(&sK[(kt * 32 + l32) * RSTR + 16 * s + 8 * hh]);
-        const vec_t va = *reinterpret_cast<const vec_t*>(&sV[(kt * 32 + l32) * RSTR + 16 * s + 8 * hh]);
+        const uint32_t off = kt * 32 * ROWB + (row_off ^ (s * 32));
+        const vec_t ka = *reinterpret_cast<const vec_t*>(kt_rows + off);
+        const vec_t va = *reinterpret_cast<const vec_t*>(kt_rows + TILE_BYTES + off);
         sacc = Mfma32<T>::run(ka, qf[s], sacc);
         dpacc = Mfma32<T>::run(va, dof[s], dpacc);
       }
@@ -300,36 +373,27 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnBwdPara
         const float prob = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -lse2));
         dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -delta_scaled));
       }
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          const vec_t a = *reinterpret_cast<const vec_t*>(&sKt[(mb * 32 + l32) * TSTR + kt * 32 + s2 * 16 + hh * 8]);
-          dqacc[mb] = Mfma32<T>::run(a, dsb[s2], dqacc[mb]);
-        }
-    }
+      accumulate_columns<T, DP, kt * 32 * ROWB>(dqacc, dsb, col_addr);
+    });
   }
   __syncthreads();  // the staging buffers now hold the output tiles
   store_owned<T, DP>(dqacc, smem + wave * (32 * OROW), dqb, p.dqs[2], q_begin + wave * 32, p.Tq, p.d, lane);
 }
 
-template <typename T, int DP>
-__global__ __launch_bounds__(kThreads) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
+template <typename T, int DP, bool DMA>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP == 32 ? 4 : 3) - (DMA ? 0 : 1)))) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
   typedef typename Vec8<T>::type vec_t;
   constexpr int KSTEPS = DP / 16, MB = DP / 32;
-  constexpr int RSTR = DP + 8, TSTR = kChunk + 8, OROW = DP * 2 + 16;
-  constexpr int STAGE_BYTES = (2 * kChunk * RSTR + 2 * DP * TSTR) * 2 + 2 * kChunk * 4;
-  constexpr int TILE_BYTES = (kThreads / kWave) * 32 * OROW;
-  __shared__ __attribute__((aligned(16))) uint8_t smem[STAGE_BYTES > TILE_BYTES ? STAGE_BYTES : TILE_BYTES];
-  T* sQ = reinterpret_cast<T*>(smem);   // [kChunk][RSTR]
-  T* sDo = sQ + kChunk * RSTR;          // [kChunk][RSTR]
-  T* sQt = sDo + kChunk * RSTR;         // [DP][TSTR]
-  T* sDot = sQt + DP * TSTR;            // [DP][TSTR]
-  float* sLse = reinterpret_cast<float*>(sDot + DP * TSTR);  // [kChunk] base-2 log-sum-exp (+inf: row carries nothing)
-  float* sDelta = sLse + kChunk;                             // [kChunk] D_i / sqrt(d)
+  constexpr int ROWB = DP * 2, TILE_BYTES = kChunk * ROWB;
+  constexpr int BUF_BYTES = 2 * TILE_BYTES + 2 * kChunk * 4;  // a chunk of Q, of dO, then its row statistics
+  constexpr int NBUF = DMA ? 2 : 1;
+  constexpr int OROW = DP * 2 + 16;
+  constexpr int OUT_BYTES = (kThreads / kWave) * 32 * OROW;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[NBUF * BUF_BYTES > OUT_BYTES ? NBUF * BUF_BYTES : OUT_BYTES];
 
-  const int blk = static_cast<int>(blockIdx.x % p.nblk);
-  const int bh = static_cast<int>(blockIdx.x / p.nblk);
+  const uint32_t logical = xcd_remap(blockIdx.x, p.total);
+  const int blk = static_cast<int>(logical % p.nblk);
+  const int bh = static_cast<int>(logical / p.nblk);
   const int h = bh % p.H, b = bh / p.H;
   const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave, l32 = lane % 32, hh = lane / 32;
   const T* qb = static_cast<const T*>(p.q) + b * p.qs[0] + h * p.qs[1];
@@ -363,49 +427,72 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkv_kernel(const AttnBwdPar
   const int64_t stat0 = (static_cast<int64_t>(b) * p.H + h) * p.Tq;
 
   if (k_begin < len) {  // workgroup-uniform: a block of padding keys gets zero gradients without any work
-    RowStager<T, DP> q_rows, do_rows;
-    TransStager<T, DP> q_cols, do_cols;
+    Streamed<T, DP, DMA> q_rows, do_rows;
+    q_rows.init(qb, p.qs[2], tid);
+    do_rows.init(dob, p.dos[2], tid);
     float lse_next = -INFINITY, delta_next = 0.f;
-    auto fetch = [&](int qc0) {
-      q_rows.fetch(qb, p.qs[2], qc0, q_valid, p.d, tid);
-      do_rows.fetch(dob, p.dos[2], qc0, q_valid, p.d, tid);
-      q_cols.fetch(qb, p.qs[2], qc0, q_valid, p.d, tid);
-      do_cols.fetch(dob, p.dos[2], qc0, q_valid, p.d, tid);
+    auto fetch = [&](int qc0, int buffer) {
+      q_rows.fetch(qc0, q_valid, p.d, smem + buffer * BUF_BYTES, tid);
+      do_rows.fetch(qc0, q_valid, p.d, smem + buffer * BUF_BYTES + TILE_BYTES, tid);
       if (tid < kChunk) {
         const int qi = qc0 + tid;
         lse_next = qi < q_valid ? p.lse[stat0 + qi] : -INFINITY;
         delta_next = qi < q_valid ? p.delta[stat0 + qi] : 0.f;
       }
     };
-    if (q_start < q_valid) fetch(q_start);
-    for (int qc0 = q_start; qc0 < q_valid; qc0 += kChunk) {
-      if (qc0 > q_start) __syncthreads();  // every wavefront is done reading the previous chunk
-      q_rows.commit(sQ, tid);
-      do_rows.commit(sDo, tid);
-      q_cols.commit(sQt, tid);
-      do_cols.commit(sDot, tid);
+    // the row statistics travel through registers: base-2 log-sum-exp (+inf: the row carries nothing, exp2(x - inf) = 0)
+    // and D_i / sqrt(d)
+    auto commit_stats = [&](int buffer) {
       if (tid < kChunk) {
-        sLse[tid] = lse_next > -INFINITY ? lse_next * 1.4426950408889634f : INFINITY;  // exp2(x - inf) = 0
-        sDelta[tid] = delta_next * p.scale;
+        float* stats = reinterpret_cast<float*>(smem + buffer * BUF_BYTES + 2 * TILE_BYTES);
+        stats[tid] = lse_next > -INFINITY ? lse_next * 1.4426950408889634f : INFINITY;
+        stats[kChunk + tid] = delta_next * p.scale;
       }
-      __syncthreads();
-      if (qc0 + kChunk < q_valid) fetch(qc0 + kChunk);
-#pragma unroll
-      for (int qt = 0; qt < kChunk / 32; ++qt) {
-        if (qc0 + qt * 32 >= q_valid || k_begin + wave * 32 >= len) continue;  // wavefront-uniform
-        if (p.causal && qc0 + qt * 32 + 31 < k_begin + wave * 32) continue;     // every query of the tile lies before the keys
+    };
+    const uint32_t row_off = streamed_row_offset<DP>(l32, hh);
+    const uint32_t col_off = streamed_column_offset<DP>(lane);
+    if (q_start < q_valid) {
+      fetch(q_start, 0);
+      if (DMA) commit_stats(0);
+    }
+    int buf = 0;
+    for (int qc0 = q_start; qc0 < q_valid; qc0 += kChunk) {
+      const bool more = qc0 + kChunk < q_valid;
+      if (DMA) {
+        vm_wait<0>();     // this wavefront's pieces of the chunk have landed ...
+        __syncthreads();  // ... everyone's have (and the statistics), and everyone is done reading the other buffer
+        if (more) fetch(qc0 + kChunk, buf ^ 1);
+      } else {
+        if (qc0 > q_start) __syncthreads();  // every wavefront is done reading the previous chunk
+        q_rows.commit(smem, tid);
+        do_rows.commit(smem + TILE_BYTES, tid);
+        commit_stats(0);
+        __syncthreads();
+        if (more) fetch(qc0 + kChunk, 0);
+      }
+      const uint8_t* q_tile = smem + buf * BUF_BYTES;
+      const float* sLse = reinterpret_cast<const float*>(q_tile + 2 * TILE_BYTES);
+      const float* sDelta = sLse + kChunk;
+      const uint32_t q_col_addr = lds_offset(q_tile) + col_off;
+      if (DMA) buf ^= 1;
+      static_for<kChunk / 32>([&](auto qt_tag) {
+        constexpr int qt = decltype(qt_tag)::value;
+        if (qc0 + qt * 32 >= q_valid || k_begin + wave * 32 >= len) return;  // wavefront-uniform
+        if (p.causal && qc0 + qt * 32 + 31 < k_begin + wave * 32) return;     // every query of the tile lies before the keys
         f32x16 sacc, dpacc;
 #pragma unroll
         for (int j = 0; j < 16; ++j) sacc[j] = dpacc[j] = 0.f;
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
-          const vec_t qa = *reinterpret_cast<const vec_t*>(&sQ[(qt * 32 + l32) * RSTR + 16 * s + 8 * hh]);
-          const vec_t da = *reinterpret_cast<const vec_t*>(&sDo[(qt * 32 + l32) * RSTR + 16 * s + 8 * hh]);
+          const uint32_t off = qt * 32 * ROWB + (row_off ^ (s * 32));
+          const vec_t qa = *reinterpret_cast<const vec_t*>(q_tile + off);
+          const vec_t da = *reinterpret_cast<const vec_t*>(q_tile + TILE_BYTES + off);
           sacc = Mfma32<T>::run(qa, kf[s], sacc);
           dpacc = Mfma32<T>::run(da, vf[s], dpacc);
         }
-        // a padded key of the lane, or (causal) a query before the key: the score becomes -inf, the probability 0;
-        // only a tile that crosses the causal diagonal needs per-element tests
+        // (causal) a query before the key: the score becomes -inf, the probability 0; only a tile that crosses the
+        // causal diagonal needs per-element tests. A padded key of the lane (zeros in kf and vf) collects finite
+        // values in its own accumulator column only, which is cleared after the loop.
         const bool diagonal = p.causal && qc0 + qt * 32 < k_begin + wave * 32 + 31;
         vec_t pb[2], dsb[2];
 #pragma unroll
@@ -416,24 +503,23 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkv_kernel(const AttnBwdPar
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int j = jq * 4 + e;
-            float sc = k_ok ? sacc[j] : -INFINITY;
+            float sc = sacc[j];
             if (diagonal && kj > qc0 + r0 + e) sc = -INFINITY;
             const float prob = __builtin_amdgcn_exp2f(fmaf(sc, c, -l4[e]));
             pb[j / 8][j % 8] = static_cast<T>(prob);
             dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -d4[e]));
           }
         }
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2) {
-            const vec_t dot = *reinterpret_cast<const vec_t*>(&sDot[(mb * 32 + l32) * TSTR + qt * 32 + s2 * 16 + hh * 8]);
-            const vec_t qt_ = *reinterpret_cast<const vec_t*>(&sQt[(mb * 32 + l32) * TSTR + qt * 32 + s2 * 16 + hh * 8]);
-            dvacc[mb] = Mfma32<T>::run(dot, pb[s2], dvacc[mb]);
-            dkacc[mb] = Mfma32<T>::run(qt_, dsb[s2], dkacc[mb]);
-          }
-      }
+        accumulate_columns2<T, DP, qt * 32 * ROWB>(dvacc, pb, q_col_addr + TILE_BYTES, dkacc, dsb, q_col_addr);
+      });
+      if (DMA && more) commit_stats(buf);  // the next chunk's statistics: the barrier above publishes them
     }
+  }
+  if (!k_ok) {  // a key in the padding receives no gradient
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) dkacc[mb][j] = dvacc[mb][j] = 0.f;
   }
   __syncthreads();
   uint8_t* tile = smem + wave * (32 * OROW);
@@ -449,20 +535,36 @@ bool strides_ok(const int64_t* st) {
   return true;
 }
 
-template <typename T>
-void launch_bwd(AttnBwdParams p, hipStream_t s) {
+// 32-bit source offsets with a 24-bit row multiply: row strides below 4 M elements, sequences below 2^31 bytes.
+bool small_offsets(int64_t rows, int64_t stride) {
+  return stride < (1 << 22) && rows < (1 << 22) && rows * stride * 2 < (1ll << 31);
+}
+
+template <typename T, int DP>
+void launch_bwd_dp(AttnBwdParams p, hipStream_t s) {
+  // TAAC_ATTN_STAGING=registers keeps the register-staged kernels for full head dims too (comparison knob).
+  const char* staging_env = getenv("TAAC_ATTN_STAGING");  // read per call: tests compare the two routes in one process
+  const bool direct = p.d == DP && !(staging_env != nullptr && staging_env[0] == 'r');
   p.nblk = static_cast<uint32_t>((p.Tq + kOwn - 1) / kOwn);
   p.total = p.nblk * p.B * p.H;
-  if (p.d <= 32)
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, 32>), dim3(p.total), dim3(kThreads), 0, s, p);
+  if (direct && small_offsets(p.Tk, p.ks[2]) && small_offsets(p.Tk, p.vs[2]))
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, DP, true>), dim3(p.total), dim3(kThreads), 0, s, p);
   else
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, 64>), dim3(p.total), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, DP, false>), dim3(p.total), dim3(kThreads), 0, s, p);
   p.nblk = static_cast<uint32_t>((p.Tk + kOwn - 1) / kOwn);
   p.total = p.nblk * p.B * p.H;
-  if (p.d <= 32)
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, 32>), dim3(p.total), dim3(kThreads), 0, s, p);
+  if (direct && small_offsets(p.Tq, p.qs[2]) && small_offsets(p.Tq, p.dos[2]))
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, DP, true>), dim3(p.total), dim3(kThreads), 0, s, p);
   else
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, 64>), dim3(p.total), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, DP, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+}
+
+template <typename T>
+void launch_bwd(const AttnBwdParams& p, hipStream_t s) {
+  if (p.d <= 32)
+    launch_bwd_dp<T, 32>(p, s);
+  else
+    launch_bwd_dp<T, 64>(p, s);
 }
 
 }  // namespace

@@ -1,5 +1,5 @@
-// Pieces shared by the token-stationary kernels (ffn.hip, fp8_ts.hip): direct global->LDS staging and hand-issued,
-// hand-awaited LDS / global operations.
+// Pieces shared by the token-stationary kernels (ffn.hip, fp8_ts.hip) and the attention kernels: direct global->LDS
+// staging and hand-issued, hand-awaited LDS / global operations.
 #pragma once
 
 #include <type_traits>
@@ -32,6 +32,25 @@ __device__ __forceinline__ void lds_dma16(const void* gsrc, void* lds_wave_base)
       :
       : "v"(gsrc), "s"(base)
       : "memory", "m0");
+}
+
+// lds_dma16 with the source given as a wavefront-uniform base (scalar registers) + a 32-bit per-lane byte offset.
+__device__ __forceinline__ void lds_dma16_offset(const void* base, uint32_t lane_offset, void* lds_wave_base) {
+  const uint32_t lds_base = __builtin_amdgcn_readfirstlane(lds_offset(lds_wave_base));
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %0, %1"
+      :
+      : "v"(lane_offset), "s"(base), "s"(lds_base)
+      : "memory", "m0");
+}
+
+// Transposed 64-bit read: element e of lane j of a 16-lane group receives element j % 4 of the 8-byte row whose address
+// lane 4 * e + j / 4 of that group supplies.
+template <int OFFSET>
+__device__ __forceinline__ void lds_read_tr16(u32x2& dst, uint32_t addr) {
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFFSET) : "memory");
 }
 
 // Hand-issued LDS reads and hand-written waits: fragment reads run several MFMAs ahead of their use with exact

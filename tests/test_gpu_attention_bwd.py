@@ -24,7 +24,7 @@ def _reference(q, k, v, lengths, grad_out, *, causal, zero_pad):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("tokens,dim", [(50, 32), (130, 64), (300, 32), (64, 16), (257, 64), (33, 8)])
+@pytest.mark.parametrize("tokens,dim", [(50, 32), (130, 64), (300, 32), (64, 16), (257, 64), (33, 8), (150, 48)])
 @pytest.mark.parametrize("causal,zero_pad", [(False, False), (False, True), (True, False)])
 def test_backward_matches_autograd_of_the_oracle(device, dtype, tokens, dim, causal, zero_pad):
     batch, heads = 4, 2
@@ -71,6 +71,26 @@ def test_backward_is_reproducible_and_reads_the_projection_layout(device):
     ref = oracle.scaled_dot_product_attention(q, k, v, num_heads=heads, key_lengths=lengths, zero_padded_queries=True)
     ref.backward(grad_out.double())
     torch.testing.assert_close(grads[0].cpu().double(), pr.grad, **TOL)
+
+
+@pytest.mark.parametrize("dim,causal", [(32, False), (64, False), (64, True)])
+def test_direct_transfer_backward_equals_register_staged_backward(device, monkeypatch, dim, causal):
+    """Full head dims stream their chunks from global memory straight into LDS, where rows beyond the valid length repeat
+    the last valid row instead of zeros; their products are cancelled by zero probabilities, so both routes give the
+    same bits (the staging knob is read per call)."""
+    batch, heads, tokens = 5, 2, 333
+    g = torch.Generator().manual_seed(dim + causal)
+    q, k, v, grad_out = (torch.randn(batch, heads, tokens, dim, generator=g).to(torch.bfloat16).to(device) for _ in range(4))
+    lengths = torch.tensor([333, 1, 64, 65, 200], dtype=torch.int32, device=device)
+    grads = {}
+    for staging in ("direct", "registers"):
+        monkeypatch.setenv("TAAC_ATTN_STAGING", staging)
+        qd, kd, vd = (t.clone().requires_grad_(True) for t in (q, k, v))
+        flash_attention(qd, kd, vd, key_lengths=lengths, is_causal=causal, zero_padded_queries=not causal).backward(grad_out)
+        grads[staging] = (qd.grad, kd.grad, vd.grad)
+    for direct, staged in zip(grads["direct"], grads["registers"]):
+        assert torch.isfinite(direct.float()).all()
+        assert torch.equal(direct, staged)
 
 
 def test_backward_envelope(device):
