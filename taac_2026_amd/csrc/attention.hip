@@ -12,8 +12,9 @@
 //   Scores are computed transposed, S^T[key, query] = K Q^T, so that in the accumulator layout every lane owns ONE
 //   query column (lane % 32) and 16 of the tile's 32 keys: the softmax row reductions are in-register plus one
 //   exchange with lane ^ 32. The probabilities are then already in the B-operand layout of the second product
-//   O^T[d, query] = V^T P^T, so P never leaves registers. The accumulator's key order (4-key runs interleaved
-//   between the two lane halves) is matched by storing V^T in LDS with the same key permutation.
+//   O^T[d, query] = V^T P^T, so P never leaves registers. V stays row-major in LDS: its fragments (8 keys of one
+//   feature per lane) are read column-wise with ds_read_b64_tr_b16, at key offsets that follow the accumulator's key
+//   order (4-key runs interleaved between the two lane halves).
 //
 // Semantics follow the reference's inference kernel (accelerators/attention/kernels/tilelang.py:36-138): base-2
 // online softmax with scale log2(e)/sqrt(d), key j visible iff j < key_lengths[b] (and j <= i when causal),
@@ -107,16 +108,6 @@ __device__ __forceinline__ float frag_sum(const f16x8& v, float acc) {
   return acc;
 }
 
-template <typename T>
-__device__ __forceinline__ uint32_t pack2(T lo, T hi) {
-  return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, lo)) |
-         (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, hi)) << 16);
-}
-
-// Position of key k (0..15 inside a 16-key group) in the permuted V^T row: the accumulator layout gives lane half
-// hh = (k / 4) % 2 the keys {hh*4 .. hh*4+3} and {8 + hh*4 .. 8 + hh*4+3}; they become 8 consecutive elements.
-__device__ __forceinline__ int vt_pos16(int k) { return ((k >> 2) & 1) * 8 + (k >> 3) * 4 + (k & 3); }
-
 template <typename T, int DP, bool CAUSAL, bool SCALED, bool MASKED>
 __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnParams p) {
   static_assert(!(MASKED && CAUSAL), "a structured mask carries its own causal triangle");
@@ -125,14 +116,16 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   constexpr int KSTEPS = DP / 16;  // MFMA k-steps of the score product
   constexpr int MB = DP / 32;      // 32-row blocks of O^T
   constexpr int C8 = DP / 8;       // 128-bit column chunks per row
-  constexpr int KSTR = DP + 8;     // LDS row strides in elements (+16 bytes against bank conflicts)
-  constexpr int VSTR = kKC + 8;
+  constexpr int KSTR = DP + 8;     // K row stride in elements (+16 bytes: 16 lanes reading one piece of 16 rows hit all banks)
+  // V stays row-major as well; its fragments are read column-wise with ds_read_b64_tr_b16, where 32 lanes touch 64
+  // contiguous bytes of four consecutive rows: a row stride of 16 or 48 dwords (mod 64) spreads those over all banks.
+  constexpr int VSTR = DP == 32 ? DP : DP + 32;
   constexpr int OROW = DP * 2 + 16;                 // bytes per row of a wavefront's output tile
-  constexpr int KV_BYTES = (kKC * KSTR + DP * VSTR) * 2;
+  constexpr int KV_BYTES = (kKC * KSTR + kKC * VSTR) * 2;
   constexpr int OT_BYTES = (kThreads / kWave) * 32 * OROW;
   __shared__ __attribute__((aligned(16))) uint8_t smem[KV_BYTES > OT_BYTES ? KV_BYTES : OT_BYTES];
   T* sK = reinterpret_cast<T*>(smem);               // [kKC][KSTR]
-  T* sVt = sK + kKC * KSTR;                         // [DP][VSTR]
+  T* sV = sK + kKC * KSTR;                          // [kKC][VSTR]
 
   const uint32_t logical = xcd_remap(blockIdx.x, p.total);
   const int qc = static_cast<int>(logical % p.nqc);
@@ -218,11 +211,9 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   if (q_begin + wave * 32 >= q_valid) wave_kv_end = 0;
 
   // K / V staging is split into a register fetch and an LDS commit so that the global loads of chunk c + 1 are in
-  // flight while chunk c is being consumed. Piece idx of a chunk: K -> (key idx / C8, 8 features idx % C8);
-  // V -> (key pair idx / C8, 8 features idx % C8), written transposed and key-permuted as sVt[feature][pos(key)].
+  // flight while chunk c is being consumed. Piece idx of a chunk, of K and of V: (key idx / C8, 8 features idx % C8).
   constexpr int KLD = (kKC * C8 + kThreads - 1) / kThreads;
-  constexpr int VLD = ((kKC / 2) * C8 + kThreads - 1) / kThreads;
-  vec_t kreg[KLD], vreg[VLD][2];
+  vec_t kreg[KLD], vreg[KLD];
   float kfac[SCALED ? KLD : 1];
   const bool scale_keys = SCALED && p.k_row_scale != nullptr;
   // MASKED: the two 32-key words of the lane's query for the chunk being fetched / being consumed (structure only),
@@ -271,17 +262,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
       const int c8 = idx % C8;
       const bool ok = idx < kKC * C8 && kidx < kv_end && c8 * 8 < p.d;
       kreg[i] = ok ? *reinterpret_cast<const vec_t*>(kb + kidx * p.ks[2] + c8 * 8) : zero_vec;
+      vreg[i] = ok ? *reinterpret_cast<const vec_t*>(vb + kidx * p.vs[2] + c8 * 8) : zero_vec;
       if (SCALED) kfac[SCALED ? i : 0] = (ok && scale_keys) ? p.k_row_scale[static_cast<int64_t>(b) * p.Tk + kidx] : 1.0f;
-    }
-#pragma unroll
-    for (int i = 0; i < VLD; ++i) {
-      const int idx = tid + i * kThreads;
-      const int kidx = kc0 + 2 * (idx / C8);
-      const int c8 = idx % C8;
-      const bool ok = idx < (kKC / 2) * C8 && c8 * 8 < p.d;
-      vreg[i][0] = (ok && kidx < kv_end) ? *reinterpret_cast<const vec_t*>(vb + kidx * p.vs[2] + c8 * 8) : zero_vec;
-      vreg[i][1] =
-          (ok && kidx + 1 < kv_end) ? *reinterpret_cast<const vec_t*>(vb + (kidx + 1) * p.vs[2] + c8 * 8) : zero_vec;
     }
   };
   auto commit = [&]() {
@@ -292,24 +274,19 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 #pragma unroll
         for (int e = 0; e < 8; ++e) kreg[i][e] = static_cast<T>(static_cast<float>(kreg[i][e]) * kfac[SCALED ? i : 0]);
       }
-      if (idx < kKC * C8) *reinterpret_cast<vec_t*>(&sK[(idx / C8) * KSTR + (idx % C8) * 8]) =
-          key_is_valid(idx / C8) ? kreg[i] : zero_vec;
-    }
-#pragma unroll
-    for (int i = 0; i < VLD; ++i) {
-      const int idx = tid + i * kThreads;
-      if (idx < (kKC / 2) * C8) {
-        const int key0 = 2 * (idx / C8);
-        const int c8 = idx % C8;
-        const int pos = (key0 & ~15) + vt_pos16(key0 & 15);  // even; key0 + 1 lands at pos + 1
-        const vec_t v0 = key_is_valid(key0) ? vreg[i][0] : zero_vec;
-        const vec_t v1 = key_is_valid(key0 + 1) ? vreg[i][1] : zero_vec;
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          *reinterpret_cast<uint32_t*>(&sVt[(c8 * 8 + e) * VSTR + pos]) = pack2<T>(v0[e], v1[e]);
+      if (idx < kKC * C8) {
+        const bool valid = key_is_valid(idx / C8);
+        *reinterpret_cast<vec_t*>(&sK[(idx / C8) * KSTR + (idx % C8) * 8]) = valid ? kreg[i] : zero_vec;
+        *reinterpret_cast<vec_t*>(&sV[(idx / C8) * VSTR + (idx % C8) * 8]) = valid ? vreg[i] : zero_vec;
       }
     }
   };
+  // Address of the lane's transposed reads of V (see lds_read_tr16): lane r of 16-lane group g points at key
+  // 4 * hh + r / 4 of an 8-key group, features 16 (g % 2) + 4 (r % 4) .. + 3 of a 32-feature row block. With the read at
+  // key offset 16 s2 (+ 8) of a tile, lane (l32, hh) receives the keys 16 s2 (+ 8) + 4 hh + 0..3 of feature l32: the
+  // key order of the probabilities in its accumulator registers 8 s2 .. 8 s2 + 7.
+  const uint32_t v_addr = lds_offset(sV) + static_cast<uint32_t>((4 * hh + (lane % 16) / 4) * (VSTR * 2) +
+                                                                  (16 * ((lane / 16) % 2) + 4 * (lane % 4)) * 2);
 
   // Chunks are walked in order; with a structured mask the chunks in which no query of this workgroup's block sees
   // any key (block_any, shared by the batch) are skipped altogether: not staged, not synchronised on.
@@ -428,19 +405,28 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
       // ---- O^T += V^T P^T --------------------------------------------------------------------------------
       // The rescale is unconditional on purpose: a wavefront-uniform branch around it placed the accumulator read-back
       // of the preceding MFMA on a path without the required wait states (wrong values in the last accumulator register).
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
+      static_for<MB>([&](auto mb_tag) {
+        constexpr int mb = decltype(mb_tag)::value;
 #pragma unroll
         for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;
-#pragma unroll
-        for (int kt = 0; kt < NT; ++kt)
+        static_for<NT>([&](auto kt_tag) {
+          constexpr int kt = decltype(kt_tag)::value;
+          constexpr int key0 = (T0 + kt) * 32;
+          u32x2 vt[2][2];
+          lds_read_tr16<key0 * VSTR * 2 + mb * 64>(vt[0][0], v_addr);
+          lds_read_tr16<(key0 + 8) * VSTR * 2 + mb * 64>(vt[0][1], v_addr);
+          lds_read_tr16<(key0 + 16) * VSTR * 2 + mb * 64>(vt[1][0], v_addr);
+          lds_read_tr16<(key0 + 24) * VSTR * 2 + mb * 64>(vt[1][1], v_addr);
+          // the transposed reads were issued by hand: wait for them by hand (everything of this wavefront's LDS queue);
+          // the fragments are tied to the wait so that their consumers cannot be scheduled above it
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vt[0][0]), "+v"(vt[0][1]), "+v"(vt[1][0]), "+v"(vt[1][1]) : : "memory");
 #pragma unroll
           for (int s2 = 0; s2 < 2; ++s2) {
-            const vec_t a =
-                *reinterpret_cast<const vec_t*>(&sVt[(mb * 32 + l32) * VSTR + (T0 + kt) * 32 + s2 * 16 + hh * 8]);
-            oacc[mb] = Mfma32<T>::run(a, pb[kt][s2], oacc[mb]);
+            const u32x4 bits = {vt[s2][0][0], vt[s2][0][1], vt[s2][1][0], vt[s2][1][1]};
+            oacc[mb] = Mfma32<T>::run(__builtin_bit_cast(vec_t, bits), pb[kt][s2], oacc[mb]);
           }
-      }
+        });
+      });
     };
     typedef std::integral_constant<int, 0> I0;
     typedef std::integral_constant<int, 1> I1;
@@ -468,7 +454,7 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   if (p.lse != nullptr && hh == 0 && qi < p.Tq)
     p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Tq + qi] =
         (qi < q_valid && l_run > 0.f) ? (m_run * c + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f : -INFINITY;
-  __syncthreads();  // every wavefront is done with sK / sVt: the buffer now holds the output tiles
+  __syncthreads();  // every wavefront is done with sK / sV: the buffer now holds the output tiles
   uint8_t* tile = smem + wave * (32 * OROW);
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
