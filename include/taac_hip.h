@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define TAAC_ABI_VERSION 3
+#define TAAC_ABI_VERSION 4
 
 enum taac_status {
   TAAC_OK = 0,
@@ -142,9 +142,14 @@ int taac_flash_attn_scaled_fwd(const void* q, const void* k, const void* v, cons
  * fallback for padded queries, which attend to themselves only; requires Tq == Tk). Rows with no visible key give
  * zeros. The row / feature factors are those of taac_flash_attn_scaled_fwd (NULL: none). Everything else as
  * taac_flash_attn_fwd; no is_causal (put the triangle into structural); Tk <= 4096.
+ * struct_sample_stride: 0 for one structural matrix shared by the batch, else the number of 32-bit words between the
+ * matrices of consecutive samples (at least Tq * ceil(Tk / 32)): per-sample structure, as taac_mask_front_bits writes
+ * it for samples whose valid tokens were moved to the front; block_any may then be NULL (no chunk is skipped on
+ * structure).
  */
 int taac_flash_attn_masked_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
-                               const uint32_t* struct_bits, const uint8_t* block_any, const uint32_t* valid_bits,
+                               const uint32_t* struct_bits, int64_t struct_sample_stride, const uint8_t* block_any,
+                               const uint32_t* valid_bits,
                                const uint32_t* self_bits, const float* q_row_scale, const float* k_row_scale,
                                const float* q_col_scale, void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk,
                                int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
@@ -228,28 +233,31 @@ int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_weight, flo
  * out_bias / b_up / b_down may be NULL. x1 is rounded to bf16 as the reference's residual stream is, but is never
  * written to memory: it stays in the accumulators of the down projection, so the final sum x1 + down + b_down is
  * rounded once (the two-kernel route rounds down + b_down first). D must be 128 or 256, F a multiple of 32.
- * rows / n_rows: as in taac_swiglu_ffn_fwd.
+ * rows / n_rows: as in taac_swiglu_ffn_fwd (rows of residual and out). attn_rows: NULL, or (with rows) the row of attn
+ * that holds token i when attn is laid out differently (taac_front_rows).
  * Replaces: attention.out + residual add and ffn_norm + SwiGLUFeedForward.forward + residual add of
  * UnifiedInteractionBlock.forward (experiments/symbiosis/backbone.py:47, 64-67).
  */
 int taac_attn_out_ffn_fwd(const void* attn, int64_t ld_attn, const void* out_bias, const void* packed_out_weights,
                           const void* residual, int64_t ldr, const void* norm_weight, float eps, const void* b_up,
                           const void* b_down, const void* packed_ffn_weights, void* out, int64_t ldo, int64_t M,
-                          int32_t D, int32_t F, const int32_t* rows, const int32_t* n_rows, void* stream);
+                          int32_t D, int32_t F, const int32_t* rows, const int32_t* n_rows, const int32_t* attn_rows,
+                          void* stream);
 
 /*
  * Fused [RMSNorm ->] dense layer [-> + residual] with the token rows held in registers:
  *   out = (residual ? residual : 0) + (norm_weight ? rmsnorm(x, norm_weight, eps) : x) @ w^T + bias
  * x: [M, K] bf16; w: [N, K]; bias: [N] or NULL; residual / out: [M, N]; packed_weights: NULL or the blob written by
  * taac_linear_pack_weights for w. K must be 128 or 256, N a multiple of 64. out may alias residual, not x.
- * rows / n_rows: as in taac_swiglu_ffn_fwd.
+ * rows / n_rows: as in taac_swiglu_ffn_fwd (rows of residual and out). x_rows: NULL, or (with rows) the row of x that
+ * holds token i when x is laid out differently from residual / out (taac_front_rows).
  * Replaces: attn_norm + the qkv projection, and the out projection + residual add, of UnifiedInteractionBlock /
  * UnifiedSelfAttention (experiments/symbiosis/backbone.py:34-35, 47, 64-65).
  */
 int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
                          const void* bias, const void* packed_weights, const void* residual, int64_t ldr, void* out,
                          int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows, const int32_t* n_rows,
-                         void* stream);
+                         const int32_t* x_rows, void* stream);
 
 /*
  * Query / key preparation of the attention layers, one pass over q and k (each read once, written once; in place when
@@ -284,7 +292,8 @@ int taac_qk_norm_rope_fwd(const void* q, const void* k, int64_t ld_in, void* q_o
  *         the token at position r % tokens_per_sample.
  * The value features are stored unchanged. The per-token factor rsqrt(mean + eps) of the norm commutes with the weight
  * and the rotation and is left to the attention kernel (taac_flash_attn_scaled_fwd). d_model: 128 or 256; head_dim a
- * multiple of 8 with a table. Other arguments as taac_norm_linear_fwd.
+ * multiple of 8 with a table. Other arguments as taac_norm_linear_fwd; with x_rows the statistic is indexed by the row
+ * of out and the position is that of the row of x.
  * Replaces: qkv + query_norm + key_norm of UnifiedSelfAttention.forward (experiments/symbiosis/backbone.py:33-36)
  * and BFTSAttention._apply_rope (experiments/tokenformer/model.py:165-192) without a pass of their own over q and k.
  */
@@ -292,7 +301,7 @@ int taac_norm_linear_qk_fwd(const void* x, int64_t ldx, const void* norm_weight,
                             const void* bias, const void* packed_weights, void* out, int64_t ldo, int64_t M,
                             int32_t d_model, int32_t num_heads, int32_t tokens_per_sample, const void* qk_weight,
                             const void* cos_sin, float* qk_sumsq, const int32_t* rows, const int32_t* n_rows,
-                            void* stream);
+                            const int32_t* x_rows, void* stream);
 
 /*
  * rstd[0, r] = rsqrt(sum_c qk_sumsq[c, r] / d_model + eps) over the d_model / 64 chunks of the query projection,
@@ -343,6 +352,31 @@ int taac_valid_rows(const int32_t* key_lengths, int32_t B, int32_t T, int32_t* r
  */
 int taac_valid_rows_from_bits(const uint32_t* valid_bits, int32_t B, int32_t T, int32_t* rows, int32_t* n_rows,
                               void* stream);
+
+/*
+ * Second row index for a layout in which every sample's valid tokens sit at the front of its T rows, in their
+ * original order: front_rows[i] = b * T + (rank of token i among the valid tokens of its sample b), for the tokens of
+ * a row index written by taac_valid_rows / taac_valid_rows_from_bits (rows, with its offsets in rows[B * T ..]), and
+ * lengths[b] = number of valid tokens of sample b. A projection that reads x through rows and writes through
+ * front_rows (taac_norm_linear_fwd / taac_norm_linear_qk_fwd with rows = front_rows, x_rows = rows) turns scattered
+ * padding into prefix padding for the attention call (key_lengths = lengths, zero_padded_queries = 2), whose cost then
+ * follows the valid tokens instead of T; the out projection reads it back through attn_rows / x_rows = front_rows.
+ * front_rows holds B * T values, lengths B. No counterpart in the reference, whose attention visits every position.
+ */
+int taac_front_rows(const int32_t* rows, const int32_t* n_rows, int32_t B, int32_t T, int32_t* front_rows,
+                    int32_t* lengths, void* stream);
+
+/*
+ * A structural mask in that front layout: out_bits[b, r, :] (rows of ceil(T / 32) words, T rows per sample) holds, for
+ * the r-th valid token of sample b, bit j = struct_bits[position(b, r), position(b, j)] for j below the sample's
+ * number of valid tokens n_b and zeros up to the end of the 64-key group of key n_b - 1. Nothing else is written (rows
+ * at or beyond n_b, words beyond that group): the attention call below does not read it. struct_bits:
+ * [T, ceil(T / 32)] (taac_mask_pack_bits), rows: the index of taac_valid_rows_from_bits. Use with key_lengths =
+ * the lengths of taac_front_rows, zero_padded_queries = 1 or 2, struct_sample_stride = T * ceil(T / 32) and
+ * valid_bits = block_any = NULL in taac_flash_attn_masked_fwd. T <= 4096.
+ */
+int taac_mask_front_bits(const uint32_t* struct_bits, int32_t T, const int32_t* rows, int32_t B, uint32_t* out_bits,
+                         void* stream);
 
 /*
  * Weight packing for the two fused kernels above: copies the weights into MFMA-fragment order (the order in which

@@ -22,7 +22,7 @@ TAAC_ERR_LAUNCH = -3
 TAAC_F32, TAAC_BF16, TAAC_F16 = 0, 1, 2
 EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _DTYPE_CODES = {torch.float32: TAAC_F32, torch.bfloat16: TAAC_BF16, torch.float16: TAAC_F16}
 
@@ -87,7 +87,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "taac_flash_attn_masked_fwd": (
         c_int,
-        [c_void_p] * 12 + [c_int32, c_int32, c_int32, c_int32, c_int32]
+        [c_void_p] * 5 + [c_int64] + [c_void_p] * 7 + [c_int32, c_int32, c_int32, c_int32, c_int32]
         + [ctypes.POINTER(c_int64)] * 4
         + [c_int, c_int, c_void_p],
     ),
@@ -118,19 +118,21 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "taac_attn_out_ffn_fwd": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
-         c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p],
+         c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p],
     ),
     "taac_norm_linear_fwd": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
-         c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p],
+         c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p],
     ),
+    "taac_front_rows": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p]),
+    "taac_mask_front_bits": (c_int, [c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p]),
     "taac_valid_rows": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p]),
     "taac_valid_rows_from_bits": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p]),
     "taac_norm_linear_qk_fwd": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32,
-         c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+         c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     ),
     "taac_row_rstd": (c_int, [c_void_p, c_int64, c_int32, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     "taac_qk_norm_rope_fwd": (

@@ -10,7 +10,7 @@ pass ``key_lengths=`` and skip the planning (and its device-to-host synchronisat
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 
 import torch
 
@@ -40,15 +40,22 @@ class StructuredAttentionMask:
     reference's model-level masks (experiments/tokenformer/model.py:474-503, experiments/symbiosis/attention.py:21-60).
     Built by :func:`build_structured_mask`; ``dense()`` gives the (B, 1, Tq, Tk) bool mask the reference would pass."""
 
-    struct_bits: torch.Tensor          # int32 (Tq, ceil(Tk / 32))
-    block_any: torch.Tensor            # uint8 (ceil(Tq / 128), ceil(Tk / 64))
+    struct_bits: torch.Tensor          # int32 (Tq, ceil(Tk / 32)); front layout: (B * Tq, ceil(Tk / 32))
+    block_any: torch.Tensor | None     # uint8 (ceil(Tq / 128), ceil(Tk / 64)); front layout: None
     valid_bits: torch.Tensor | None    # int32 (B, ceil(Tk / 32))
     self_bits: torch.Tensor | None     # int32 (B, ceil(Tq / 32))
     structural: torch.Tensor           # bool (Tq, Tk)
     key_valid: torch.Tensor | None     # bool (B, Tk)
     query_self: torch.Tensor | None    # bool (B, Tq)
+    sample_stride: int = 0             # words between the bit matrices of consecutive samples (front layout), else 0
+    padding_source: torch.Tensor | None = None  # the (B, Tk) padding mask that key_valid is the complement of, if any
+    # what callers derive from this mask once per forward pass (row indices, its front-layout form): the blocks of a
+    # stack receive the same mask object and share it
+    cache: dict = field(default_factory=dict, compare=False, repr=False)
 
     def dense(self) -> torch.Tensor:
+        if self.sample_stride:
+            raise RuntimeError("a mask in the front layout has no dense form; use the mask it was made from")
         query_len, kv_len = self.structural.shape
         mask = self.structural[None]
         if self.key_valid is not None:
@@ -57,6 +64,29 @@ class StructuredAttentionMask:
             eye = torch.eye(query_len, kv_len, dtype=torch.bool, device=self.structural.device)
             mask = torch.where(self.query_self[:, :, None], eye[None], mask)
         return mask[:, None]
+
+
+def front_structured_mask(mask: StructuredAttentionMask, token_rows: tuple[torch.Tensor, torch.Tensor],
+                          batch: int) -> StructuredAttentionMask:
+    """``mask`` for samples whose valid tokens were moved to the front of their rows (``token_rows`` = the index of
+    ``valid_rows(..., padding_mask=)`` over the same validity as ``mask.key_valid``): one structural bit matrix per
+    sample, ``bits[b, r, j] = structural[position(b, r), position(b, j)]``, every listed key valid. Use it together
+    with ``key_lengths`` = the samples' numbers of valid tokens."""
+    name = "hip front_structured_mask"
+    query_len, kv_len = mask.structural.shape
+    if query_len != kv_len or mask.query_self is not None or mask.sample_stride:
+        raise ValueError(f"{name}: needs a square mask without self rows that is not in the front layout already")
+    rows, _ = token_rows
+    require_cuda_tensors(name, rows, mask.struct_bits)
+    words = (kv_len + 31) // 32
+    if rows.dtype != torch.int32 or rows.numel() < batch * query_len + batch + 1 or not rows.is_contiguous():
+        raise ValueError(f"{name}: token_rows must be the index returned by valid_rows for (batch, tokens)")
+    bits = torch.empty(batch * query_len, words, dtype=torch.int32, device=rows.device)
+    library = _native.load_library()
+    status = library.taac_mask_front_bits(mask.struct_bits.data_ptr(), query_len, rows.data_ptr(), int(batch),
+                                          bits.data_ptr(), _native.current_stream(rows.device))
+    _native.check(status, "mask_front_bits")
+    return StructuredAttentionMask(bits, None, None, None, mask.structural, None, None, query_len * words)
 
 
 def _pack_bits(mask: torch.Tensor) -> torch.Tensor:
@@ -69,10 +99,13 @@ def _pack_bits(mask: torch.Tensor) -> torch.Tensor:
 
 
 def build_structured_mask(
-    structural: torch.Tensor, key_valid: torch.Tensor | None = None, query_self: torch.Tensor | None = None
+    structural: torch.Tensor, key_valid: torch.Tensor | None = None, query_self: torch.Tensor | None = None,
+    *, padding_source: torch.Tensor | None = None,
 ) -> StructuredAttentionMask:
     """``structural`` (Tq, Tk) bool, True = attend; ``key_valid`` (B, Tk) bool or None; ``query_self`` (B, Tq) bool or
-    None (needs Tq == Tk). Everything stays on the device (no host synchronisation)."""
+    None (needs Tq == Tk). Everything stays on the device (no host synchronisation). ``padding_source``: the padding
+    mask whose non-padded positions are exactly the valid keys of every sample that has one (a caller that skips the
+    padded rows with the same mask can then run the attention over the valid tokens only)."""
     name = "hip build_structured_mask"
     require_cuda_tensors(name, structural, key_valid, query_self)
     for tensor, label in ((structural, "structural"), (key_valid, "key_valid"), (query_self, "query_self")):
@@ -94,7 +127,7 @@ def build_structured_mask(
     query_self = None if query_self is None else query_self.contiguous()
     return StructuredAttentionMask(
         struct_bits, block_any, None if key_valid is None else _pack_bits(key_valid),
-        None if query_self is None else _pack_bits(query_self), structural, key_valid, query_self,
+        None if query_self is None else _pack_bits(query_self), structural, key_valid, query_self, 0, padding_source,
     )
 
 
@@ -331,12 +364,14 @@ def hip_flash_attention_kernel(
             raise ValueError("flash_attention: a structured mask carries its own causal triangle (is_causal must be False)")
         sm = structured_mask
         if sm.structural.shape != (query_len, k.shape[2]) or (sm.key_valid is not None and sm.key_valid.shape[0] != batch) \
-                or (sm.query_self is not None and sm.query_self.shape[0] != batch):
+                or (sm.query_self is not None and sm.query_self.shape[0] != batch) \
+                or (sm.sample_stride and sm.struct_bits.shape[0] != batch * query_len):
             raise ValueError("flash_attention: the structured mask does not match (batch, query_len, kv_len)")
         require_cuda_tensors("hip flash_attention", sm.struct_bits)
         status = library.taac_flash_attn_masked_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), sm.struct_bits.data_ptr(),
-            sm.block_any.data_ptr(), _native.ptr(sm.valid_bits), _native.ptr(sm.self_bits), _native.ptr(q_row_scale),
+            int(sm.sample_stride), _native.ptr(sm.block_any), _native.ptr(sm.valid_bits), _native.ptr(sm.self_bits),
+            _native.ptr(q_row_scale),
             _native.ptr(k_row_scale), _native.ptr(q_col_scale), out.data_ptr(),
             batch, heads, query_len, k.shape[2], head_dim,
             _native.Int64x4(*q.stride()), _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()),

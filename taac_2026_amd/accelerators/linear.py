@@ -211,6 +211,38 @@ def valid_rows(key_lengths: torch.Tensor | None, tokens: int, *,
     return rows, count
 
 
+def front_rows(token_rows: tuple[torch.Tensor, torch.Tensor], batch: int, tokens: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Second index for the layout in which every sample's valid tokens sit at the front of its ``tokens`` rows, in
+    their original order: ``(front, lengths)`` with ``front[i] = b * tokens + rank`` for token ``i`` of
+    ``token_rows`` and ``lengths[b]`` = the sample's number of valid tokens (int32, on the device). A projection called
+    with ``token_rows=(front, count), input_rows=rows`` writes that layout, in which scattered padding has become
+    prefix padding (``key_lengths=lengths`` for the attention call); ``token_rows=(rows, count), input_rows=front``
+    reads it back."""
+    name = "hip front_rows"
+    rows, count = token_rows
+    require_cuda_tensors(name, rows, count)
+    if rows.dtype != torch.int32 or rows.numel() < batch * tokens + batch + 1 or not rows.is_contiguous():
+        raise ValueError(f"{name}: token_rows must be the index returned by valid_rows for (batch, tokens)")
+    front = torch.empty(max(1, batch * tokens), dtype=torch.int32, device=rows.device)
+    lengths = torch.empty(batch, dtype=torch.int32, device=rows.device)
+    library = _native.load_library()
+    status = library.taac_front_rows(rows.data_ptr(), count.data_ptr(), int(batch), int(tokens), front.data_ptr(),
+                                     lengths.data_ptr(), _native.current_stream(rows.device))
+    _native.check(status, "front_rows")
+    return front, lengths
+
+
+def _input_rows(name: str, input_rows: torch.Tensor | None, index: torch.Tensor | None, rows: torch.Tensor):
+    if input_rows is None:
+        return None
+    if index is None:
+        raise ValueError(f"{name}: input_rows needs token_rows")
+    require_cuda_tensors(name, input_rows)
+    if input_rows.dtype != torch.int32 or not input_rows.is_contiguous() or input_rows.numel() < rows.shape[0]:
+        raise ValueError(f"{name}: input_rows must be a contiguous int32 index that covers the {rows.shape[0]} rows of the input")
+    return input_rows
+
+
 def _output_rows(name: str, out: torch.Tensor | None, shape: tuple[int, int], sparse: bool, like: torch.Tensor):
     if out is None:
         return (torch.zeros if sparse else torch.empty)(shape, dtype=like.dtype, device=like.device)
@@ -313,13 +345,15 @@ def attention_out_ffn(
     norm_weight: torch.Tensor | None = None,
     eps: float = 1e-6,
     token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
+    input_rows: torch.Tensor | None = None,
     out: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Second half of a ``UnifiedInteractionBlock`` (experiments/symbiosis/backbone.py:47, 64-67) as ONE kernel:
     ``x1 = residual + F.linear(attn, out_weight, out_bias)`` then ``x1 + down(silu(gate) * value)`` with
     ``gate, value = up(rmsnorm(x1)).chunk(2, -1)``. ``x1`` never reaches memory. Model width 128 / 256 and a hidden
     size that is a multiple of 32 only (``taac_attn_out_ffn_fwd``); ``token_rows`` / ``out`` as in :func:`swiglu_ffn`
-    (``out`` may be ``residual``)."""
+    (``out`` may be ``residual``). ``input_rows`` (with ``token_rows``): the row of ``attn`` that holds each token when
+    ``attn`` is laid out differently from ``residual`` / ``out`` (:func:`front_rows`)."""
     name = "hip attention_out_ffn"
     tensors = (attn, out_weight, out_bias, residual, up_weight, up_bias, down_weight, down_bias, norm_weight)
     require_cuda_tensors(name, *tensors)
@@ -347,7 +381,7 @@ def attention_out_ffn(
         rows.data_ptr(), rows.stride(0), _native.ptr(out_bias), packed_out.data_ptr(), res_rows.data_ptr(),
         res_rows.stride(0), _native.ptr(norm_weight), float(eps), _native.ptr(up_bias), _native.ptr(down_bias),
         packed_ffn.data_ptr(), out.data_ptr(), d_model, rows.shape[0], d_model, hidden, _native.ptr(index),
-        _native.ptr(count), _native.current_stream(attn.device),
+        _native.ptr(count), _native.ptr(_input_rows(name, input_rows, index, rows)), _native.current_stream(attn.device),
     )
     _native.check(status, "attention_out_ffn")
     return out.reshape(shape)
@@ -362,11 +396,13 @@ def norm_linear(
     eps: float = 1e-6,
     residual: torch.Tensor | None = None,
     token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
+    input_rows: torch.Tensor | None = None,
     out: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """``residual + F.linear(rmsnorm(x, norm_weight, eps), weight, bias)`` (norm and residual optional) as one
     kernel when ``in_features`` is 128 / 256 and ``out_features`` a multiple of 64; otherwise composed from the
-    stand-alone kernels."""
+    stand-alone kernels. ``input_rows`` (with ``token_rows``, fused shapes): the row of ``x`` that holds each token when
+    ``x`` is laid out differently from ``residual`` / ``out`` (:func:`front_rows`)."""
     name = "hip norm_linear"
     require_cuda_tensors(name, x, weight, bias, residual, norm_weight)
     require_inference(name, x, weight, bias, residual, norm_weight)
@@ -375,7 +411,7 @@ def norm_linear(
     _check_weight(name, rows, weight, bias)
     in_features, out_features = weight.shape[1], weight.shape[0]
     if not (_fused_width(in_features) and out_features % 64 == 0):
-        if token_rows is not None or out is not None:
+        if token_rows is not None or out is not None or input_rows is not None:
             raise RuntimeError("norm_linear: token_rows / out need a fused shape (K 128 / 256, N a multiple of 64)")
         h = rows
         if norm_weight is not None:
@@ -399,7 +435,7 @@ def norm_linear(
         rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), None, _native.ptr(bias),
         packed.data_ptr(), _native.ptr(res_rows), res_rows.stride(0) if res_rows is not None else out_features, out.data_ptr(),
         out_features, rows.shape[0], out_features, in_features, _native.ptr(index), _native.ptr(count),
-        _native.current_stream(x.device),
+        _native.ptr(_input_rows(name, input_rows, index, rows)), _native.current_stream(x.device),
     )
     _native.check(status, "norm_linear")
     return out.reshape(*shape[:-1], out_features)
@@ -418,6 +454,7 @@ def qkv_projection(
     qk_eps: float = 1e-6,
     rope_base: float | None = None,
     token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
+    input_rows: torch.Tensor | None = None,
     out: torch.Tensor | None = None,
     scales_out: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor | None, torch.Tensor | None, torch.Tensor | None]:
@@ -435,7 +472,9 @@ def qkv_projection(
     key columns by their weights and rotates them over the token positions (experiments/tokenformer/model.py:165-192)
     and ``q_col_scale`` is None. Either way the preparation costs no pass over q and k. ``out`` (bf16, batch * tokens
     rows of 3 d_model) and ``scales_out`` (float32 (2, batch, tokens)) let a caller reuse its buffers; with ``token_rows``
-    the rows outside the index are left as they are in them."""
+    the rows outside the index are left as they are in them. ``input_rows`` (with ``token_rows``): the row of ``x`` that
+    holds each token when the projection is to be written in another layout (:func:`front_rows`); the factors follow the
+    rows of the output, the rotation the positions of the rows of ``x``."""
     name = "hip qkv_projection"
     require_cuda_tensors(name, x, weight, bias, norm_weight, query_weight, key_weight)
     require_inference(name, x, weight, bias, norm_weight, query_weight, key_weight)
@@ -486,7 +525,8 @@ def qkv_projection(
     status = library.taac_norm_linear_qk_fwd(
         rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), None, _native.ptr(bias), packed.data_ptr(),
         out.data_ptr(), 3 * d_model, rows.shape[0], d_model, int(num_heads), tokens, _native.ptr(qk_weight),
-        _native.ptr(table), _native.ptr(sumsq), _native.ptr(index), _native.ptr(count), stream,
+        _native.ptr(table), _native.ptr(sumsq), _native.ptr(index), _native.ptr(count),
+        _native.ptr(_input_rows(name, input_rows, index, rows)), stream,
     )
     _native.check(status, "qkv_projection")
     if scales is None:

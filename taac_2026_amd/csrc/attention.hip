@@ -45,9 +45,11 @@ struct AttnParams {
   const float* q_col_scale;  // [H, d] factors of the query features, or null
   // Structured mask: key j is visible to query i of sample b iff bit j of struct_bits[i] and of valid_bits[b] is set.
   const uint32_t* struct_bits;  // [Tq][wpr] words, bit j % 32 of word j / 32; null: no structured mask
+  int64_t struct_stride;        // words between the matrices of consecutive samples; 0: one matrix for the batch
   const uint32_t* valid_bits;   // [B][wpr] or null (every key valid)
   const uint32_t* self_bits;    // [B][ceil(Tq / 32)] or null: flagged query rows return their own value row
-  const uint8_t* block_any;     // [nqc][nkc]: some query of the 128-row block sees some key of the 64-key chunk
+  const uint8_t* block_any;     // [nqc][nkc]: some query of the 128-row block sees some key of the 64-key chunk;
+                                // null (per-sample structure only): every chunk is visited
   float* lse;                   // [B, H, Tq] log-sum-exp of the scaled scores (natural log) for the backward, or null
   int32_t wpr;                  // words per row of struct_bits / valid_bits = ceil(Tk / 32)
   int32_t nkc;                  // key chunks = ceil(Tk / 64)
@@ -248,8 +250,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt) {
         uint32_t bits = 0u;
-        if (qi < p.Tq && w0 + kt < p.wpr) {
-          bits = p.struct_bits[static_cast<int64_t>(qi) * p.wpr + w0 + kt];
+        if (qi < q_valid && w0 + kt < p.wpr) {  // a query row in the padding sees nothing (and has no row of bits)
+          bits = p.struct_bits[b * p.struct_stride + static_cast<int64_t>(qi) * p.wpr + w0 + kt];
         }
         mw_next[kt] = bits;
         vw_next[kt] = (p.valid_bits != nullptr && w0 + kt < p.wpr) ? p.valid_bits[static_cast<int64_t>(b) * p.wpr + w0 + kt] : ~0u;
@@ -292,7 +294,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   // any key (block_any, shared by the batch) are skipped altogether: not staged, not synchronised on.
   // The block's row of block_any is read once, as one bit per chunk (at most 64 chunks: Tk <= 4096 with a mask).
   uint64_t chunk_bits = ~0ull;
-  if (MASKED) chunk_bits = __builtin_amdgcn_ballot_w64(lane < p.nkc && p.block_any[qc * p.nkc + (lane < p.nkc ? lane : 0)] != 0);
+  if (MASKED && p.block_any != nullptr)
+    chunk_bits = __builtin_amdgcn_ballot_w64(lane < p.nkc && p.block_any[qc * p.nkc + (lane < p.nkc ? lane : 0)] != 0);
   auto next_chunk = [&](int kc) -> int {
     if (MASKED) {
       const uint64_t rest = kc < 64 ? chunk_bits >> kc : 0ull;
@@ -498,8 +501,12 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 // Rows at or beyond the valid length are never requested: the transfer repeats the last valid row (finite values; the
 // scores of those keys are masked), since uninitialised memory could hold NaNs that a zero probability would not cancel.
 // ------------------------------------------------------------------------------------------------------------------
-template <typename T, int DP, bool CAUSAL, bool SCALED>
+// MASKED: per-sample structure bits on top (struct_bits with a sample stride, every listed key valid, no chunk map): the
+// form in which samples with their valid tokens moved to the front arrive. The lane's two words of a chunk are fetched
+// with the chunk's transfers; tiles that are fully visible to the wavefront skip the bit tests.
+template <typename T, int DP, bool CAUSAL, bool SCALED, bool MASKED>
 __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const AttnParams p) {
+  static_assert(!(MASKED && CAUSAL), "a structured mask carries its own causal triangle");
   typedef typename Vec8<T>::type vec_t;
   typedef typename Vec8<T>::half_type vec4_t;
   static_assert(DP == 32 || DP == 64, "row swizzles are written for 64- and 128-byte rows");
@@ -604,7 +611,16 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   const bool scale_keys = SCALED && p.k_row_scale != nullptr;
   vec_t kreg[SCALED ? PPT : 1];
   float kfac[SCALED ? PPT : 1];
+  uint32_t mw_next[2] = {0u, 0u}, mw[2] = {0u, 0u};
   auto issue = [&](int chunk, int buffer) {
+    if (MASKED) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        const int w = chunk * 2 + kt;
+        mw_next[kt] = (qi < q_valid && w < p.wpr)
+                          ? p.struct_bits[b * p.struct_stride + static_cast<int64_t>(qi) * p.wpr + w] : 0u;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < PPT; ++i) {
       int row = chunk * kKC + srow + i * (kThreads / C8);
@@ -652,6 +668,10 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   for (int chunk = 0; chunk < nchunks; ++chunk) {
     vm_wait<0>();     // this wavefront's pieces of the chunk have landed ...
     __syncthreads();  // ... everyone's have, and everyone is done reading the other buffer
+    if (MASKED) {
+      mw[0] = mw_next[0];
+      mw[1] = mw_next[1];
+    }
     const bool more = chunk + 1 < nchunks;
     if (more) issue(chunk + 1, buf ^ 1);
     const int kc0 = chunk * kKC;
@@ -684,6 +704,21 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
             const int key = kc0 + kt * 32 + (j / 4) * 8 + hh * 4 + (j % 4);
             if (key >= kv_end || (CAUSAL && key > qi)) sacc[kt][j] = -INFINITY;
           }
+      }
+      if (MASKED) {
+        // Accumulator register j of the lane is key (j / 4) * 8 + hh * 4 + j % 4 of the tile: bit of the lane's word.
+        bool all_visible = true;
+#pragma unroll
+        for (int kt = 0; kt < NT; ++kt) all_visible = all_visible && mw[kt] == 0xffffffffu;
+        if (__builtin_amdgcn_ballot_w64(!all_visible) != 0) {  // wavefront-uniform
+#pragma unroll
+          for (int kt = 0; kt < NT; ++kt) {
+            const uint32_t bits = mw[kt] >> (hh * 4);
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+              if (((bits >> ((j / 4) * 8 + (j % 4))) & 1u) == 0u) sacc[kt][j] = -INFINITY;
+          }
+        }
       }
       float mx = sacc[0][0];
 #pragma unroll
@@ -796,15 +831,22 @@ void launch(const AttnParams& p, bool causal, hipStream_t s) {
                              static_cast<int64_t>(p.Tk) * p.ks[2] * 2 < (1ll << 31) &&
                              static_cast<int64_t>(p.Tk) * p.vs[2] * 2 < (1ll << 31);
   if constexpr (DP == 32 || DP == 64) {
-    if (p.d == DP && p.struct_bits == nullptr && dma_staging && small_offsets) {
-      if (causal && scaled)
-        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+    // structure bits ride along when they are all there is to the mask: per sample, no validity or self rows, no chunk map
+    const bool structure_only = p.struct_bits != nullptr && p.valid_bits == nullptr && p.self_bits == nullptr &&
+                                p.block_any == nullptr;
+    if (p.d == DP && (p.struct_bits == nullptr || structure_only) && dma_staging && small_offsets) {
+      if (structure_only && scaled)
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+      else if (structure_only)
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+      else if (causal && scaled)
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, true, true, false>), dim3(p.total), dim3(kThreads), 0, s, p);
       else if (causal)
-        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, true, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, true, false, false>), dim3(p.total), dim3(kThreads), 0, s, p);
       else if (scaled)
-        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, true, false>), dim3(p.total), dim3(kThreads), 0, s, p);
       else
-        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, false, false>), dim3(p.total), dim3(kThreads), 0, s, p);
       return;
     }
   }
@@ -867,6 +909,7 @@ __global__ __launch_bounds__(kWave) void block_any_kernel(const uint32_t* __rest
 
 struct MaskArgs {
   const uint32_t* struct_bits = nullptr;
+  int64_t struct_stride = 0;
   const uint8_t* block_any = nullptr;
   const uint32_t* valid_bits = nullptr;
   const uint32_t* self_bits = nullptr;
@@ -878,7 +921,10 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
                     const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4], int is_causal,
                     int zero_padded_queries, int dtype, void* stream) {
   if (mask.struct_bits != nullptr) {
-    if (mask.block_any == nullptr) return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_bits needs block_any", name);
+    if (mask.block_any == nullptr && mask.struct_stride == 0)
+      return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_bits shared by the batch needs block_any", name);
+    if (mask.struct_stride < 0 || (mask.struct_stride != 0 && mask.struct_stride < static_cast<int64_t>(Tq) * ((Tk + 31) / 32)))
+      return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_sample_stride must be 0 or cover a sample's matrix", name);
     if (Tk > 64 * kKC) return set_error(TAAC_ERR_UNSUPPORTED, "%s: structured masks cover at most %d keys", name, 64 * kKC);
     if (is_causal)
       return set_error(TAAC_ERR_INVALID_VALUE, "%s: a structured mask carries its own causal triangle", name);
@@ -916,6 +962,7 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   p.q_col_scale = q_col_scale;
   p.lse = lse;
   p.struct_bits = mask.struct_bits;
+  p.struct_stride = mask.struct_stride;
   p.valid_bits = mask.valid_bits;
   p.self_bits = mask.self_bits;
   p.block_any = mask.block_any;
@@ -973,7 +1020,8 @@ extern "C" int taac_flash_attn_scaled_fwd(const void* q, const void* k, const vo
 }
 
 extern "C" int taac_flash_attn_masked_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
-                                          const uint32_t* struct_bits, const uint8_t* block_any,
+                                          const uint32_t* struct_bits, int64_t struct_sample_stride,
+                                          const uint8_t* block_any,
                                           const uint32_t* valid_bits, const uint32_t* self_bits,
                                           const float* q_row_scale, const float* k_row_scale, const float* q_col_scale,
                                           void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
@@ -984,6 +1032,7 @@ extern "C" int taac_flash_attn_masked_fwd(const void* q, const void* k, const vo
     return taac::set_error(TAAC_ERR_INVALID_VALUE, "taac_flash_attn_masked_fwd: struct_bits must be given");
   taac::MaskArgs mask;
   mask.struct_bits = struct_bits;
+  mask.struct_stride = struct_sample_stride;
   mask.block_any = block_any;
   mask.valid_bits = valid_bits;
   mask.self_bits = self_bits;

@@ -134,6 +134,67 @@ __global__ __launch_bounds__(kBlock) void valid_rows_bits_kernel(const uint32_t*
   rows[offsets[b] + rank] = b * T + t;
 }
 
+// front_rows[i] = b * T + (i - offsets[b]) for token i of sample b = rows[i] / T; lengths[b] = offsets[b + 1] - offsets[b].
+__global__ __launch_bounds__(kBlock) void front_rows_kernel(const int32_t* __restrict__ rows,
+                                                            const int32_t* __restrict__ n_rows, int B, int T,
+                                                            int32_t* __restrict__ front_rows,
+                                                            int32_t* __restrict__ lengths) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  const int32_t* offsets = rows + static_cast<int64_t>(B) * T;
+  if (i < B) lengths[i] = offsets[i + 1] - offsets[i];
+  if (i >= *n_rows) return;
+  const int b = rows[i] / T;
+  front_rows[i] = b * T + static_cast<int32_t>(i - offsets[b]);
+}
+
+// One workgroup per (sample b, 32 front rows): the sample's key positions go to LDS once; a wavefront then takes 8
+// rows, holds a row's structure words across its lanes (lane l: words l and l + 64) and, 64 keys per step, lets lane j
+// pick the word of its key from them with a lane permute; a ballot gathers the bits. Only rows below the sample's
+// number of valid tokens n_b are written, and of those the words that hold a key below n_b (the attention kernel reads
+// nothing else), bits at or beyond n_b as zeros.
+constexpr int kFrontRowsPerBlock = 32;
+__global__ __launch_bounds__(kBlock) void mask_front_bits_kernel(const uint32_t* __restrict__ struct_bits, int T,
+                                                                 const int32_t* __restrict__ rows, int B,
+                                                                 uint32_t* __restrict__ out) {
+  __shared__ uint16_t kpos[4096];
+  const int wpr = (T + 31) / 32;
+  const int slabs = (T + kFrontRowsPerBlock - 1) / kFrontRowsPerBlock;
+  const int b = blockIdx.x / slabs, r0 = (blockIdx.x % slabs) * kFrontRowsPerBlock;
+  const int32_t* offsets = rows + static_cast<int64_t>(B) * T;
+  const int32_t off = offsets[b];
+  const int n = offsets[b + 1] - off;
+  if (r0 >= n) return;  // workgroup-uniform
+  for (int j = threadIdx.x; j < n; j += kBlock) kpos[j] = static_cast<uint16_t>(rows[off + j] - b * T);
+  __syncthreads();
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  constexpr int kRowsPerWave = kFrontRowsPerBlock / (kBlock / kWave);
+  // the structure words of the wavefront's rows first (independent loads), then the gathers
+  uint32_t w_lo[kRowsPerWave], w_hi[kRowsPerWave];
+#pragma unroll
+  for (int i = 0; i < kRowsPerWave; ++i) {
+    const int r = r0 + wave * kRowsPerWave + i;
+    const uint32_t* src = struct_bits + static_cast<int64_t>(kpos[r < n ? r : 0]) * wpr;
+    w_lo[i] = (r < n && lane < wpr) ? src[lane] : 0u;
+    w_hi[i] = (r < n && lane + kWave < wpr) ? src[lane + kWave] : 0u;
+  }
+  for (int j0 = 0; j0 < n; j0 += kWave) {
+    const int j = j0 + lane;
+    const int key = j < n ? kpos[j] : 0;
+    const int src_lane = (key >> 5) & (kWave - 1);
+    const bool upper = (key >> 5) >= kWave;
+#pragma unroll
+    for (int i = 0; i < kRowsPerWave; ++i) {
+      const int r = r0 + wave * kRowsPerWave + i;
+      if (r >= n) break;  // wavefront-uniform
+      const uint32_t lo = __shfl(w_lo[i], src_lane, kWave);
+      const uint32_t word = wpr > kWave ? (upper ? __shfl(w_hi[i], src_lane, kWave) : lo) : lo;
+      const uint64_t bits = __builtin_amdgcn_ballot_w64(j < n && ((word >> (key & 31)) & 1u) != 0u);
+      uint32_t* dst = out + (static_cast<int64_t>(b) * T + r) * wpr;
+      if (lane < 2 && j0 / 32 + lane < wpr) dst[j0 / 32 + lane] = static_cast<uint32_t>(bits >> (32 * lane));
+    }
+  }
+}
+
 // prod[d] = wq[d] * wk[d] in fp32: the weights of a query and a key norm act on an attention score only through their
 // product, which the attention kernel applies to the query features.
 __global__ __launch_bounds__(kBlock) void weight_product_kernel(const bf16_t* __restrict__ wq,
@@ -358,7 +419,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
       }
       if ((rc = taac_norm_linear_qk_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, qkv, 3 * D, M, D,
                                         heads, T, weights_in_epilogue ? qk_weight : nullptr, rope_cos_sin,
-                                        qk_norm ? qk_sumsq : nullptr, rows, n_rows, stream)) != TAAC_OK)
+                                        qk_norm ? qk_sumsq : nullptr, rows, n_rows, nullptr, stream)) != TAAC_OK)
         return rc;
       if (qk_norm) {
         if ((rc = taac_row_rstd(qk_sumsq, M, D, eps, qk_rstd, rows, n_rows, stream)) != TAAC_OK) return rc;
@@ -367,7 +428,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
       }
     } else if (fused) {
       if ((rc = taac_norm_linear_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, nullptr, 0, qkv,
-                                     3 * D, M, 3 * D, D, rows, n_rows, stream)) != TAAC_OK)
+                                     3 * D, M, 3 * D, D, rows, n_rows, nullptr, stream)) != TAAC_OK)
         return rc;
     } else {
       if ((rc = taac_rmsnorm_fwd(cur, w.attn_norm_weight, h, M, D, eps, TAAC_BF16, stream)) != TAAC_OK) return rc;
@@ -388,11 +449,11 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
     if (fused && !split_out_ffn) {
       // out projection + residual and the whole feed-forward half in one kernel; the stream between them stays on chip
       if ((rc = taac_attn_out_ffn_fwd(h, D, w.out_bias, pk_out, cur, D, w.ffn_norm_weight, eps, w.up_bias, w.down_bias,
-                                      pk_ffn, x_out, D, M, D, F, rows, n_rows, stream)) != TAAC_OK)
+                                      pk_ffn, x_out, D, M, D, F, rows, n_rows, nullptr, stream)) != TAAC_OK)
         return rc;
     } else if (fused) {
       if ((rc = taac_norm_linear_fwd(h, D, nullptr, eps, nullptr, w.out_bias, pk_out, cur, D, x, D, M, D, D, rows,
-                                     n_rows, stream)) != TAAC_OK)
+                                     n_rows, nullptr, stream)) != TAAC_OK)
         return rc;
       // feed-forward half: RMSNorm -> up -> SiLU-gate -> down -> + residual in one kernel
       if ((rc = taac_swiglu_ffn_fwd(x, D, w.ffn_norm_weight, eps, nullptr, w.up_bias, nullptr, w.down_bias, pk_ffn, x,
@@ -425,4 +486,36 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
       return set_error(TAAC_ERR_LAUNCH, "%s: copy of the embeddings failed", name);
   }
   return taac_masked_mean_head(cur, key_lengths, w_head, b_head, p, B, T, D, stream);
+}
+
+extern "C" int taac_front_rows(const int32_t* rows, const int32_t* n_rows, int32_t B, int32_t T, int32_t* front_rows,
+                               int32_t* lengths, void* stream) {
+  using namespace taac;
+  const char* name = "taac_front_rows";
+  if (B < 0 || T < 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: bad dimensions", name);
+  if (static_cast<int64_t>(B) * T > 0x7fffffffLL - B - 1)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: B * T must fit 32-bit row numbers", name);
+  if (B == 0) return TAAC_OK;
+  if (!rows || !n_rows || !lengths || (T > 0 && !front_rows)) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  const int64_t threads = static_cast<int64_t>(B) * T > B ? static_cast<int64_t>(B) * T : B;
+  hipLaunchKernelGGL(front_rows_kernel, dim3(static_cast<uint32_t>((threads + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                     as_stream(stream), rows, n_rows, B, T, front_rows, lengths);
+  return check_launch(name);
+}
+
+extern "C" int taac_mask_front_bits(const uint32_t* struct_bits, int32_t T, const int32_t* rows, int32_t B,
+                                    uint32_t* out_bits, void* stream) {
+  using namespace taac;
+  const char* name = "taac_mask_front_bits";
+  if (B < 0 || T < 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: bad dimensions", name);
+  if (T > 4096) return set_error(TAAC_ERR_UNSUPPORTED, "%s: at most 4096 tokens per sample", name);
+  if (static_cast<int64_t>(B) * T > 0x7fffffffLL - B - 1)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: B * T must fit 32-bit row numbers", name);
+  if (B == 0 || T == 0) return TAAC_OK;
+  if (!struct_bits || !rows || !out_bits) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  const int64_t blocks = static_cast<int64_t>(B) * ((T + kFrontRowsPerBlock - 1) / kFrontRowsPerBlock);
+  if (blocks > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many rows", name);
+  hipLaunchKernelGGL(mask_front_bits_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, as_stream(stream),
+                     struct_bits, T, rows, B, out_bits);
+  return check_launch(name);
 }

@@ -54,6 +54,8 @@ struct TsParams {
   int32_t packed;           // weights are in fragment order
   const int32_t* rows;      // optional row index: token i lives in row rows[i] of x / residual / out
   const int32_t* n_rows;    // with rows: device pointer to the number of tokens (at most M)
+  const int32_t* x_rows;    // optional, with rows: token i's row of x when it differs from rows[i] (x and residual / out
+                            // laid out differently: samples with their valid tokens moved to the front on one side)
   int32_t units;            // FFN: compute units the last, partial round of workgroups is spread over
   // Query / key mode of the linear kernel (the packed q | k | v projection of an attention layer):
   const bf16_t* qk_w;       // [qk_chunks * 64] norm weights of the query and key features (q | k), or null (ones)
@@ -162,6 +164,13 @@ __device__ __forceinline__ int64_t token_row(const TsParams& p, int64_t count, i
   return p.rows != nullptr ? static_cast<int64_t>(p.rows[tok]) : tok;
 }
 
+// Row of x that holds token `tok`: its own index when one is given, the common one otherwise.
+__device__ __forceinline__ int64_t input_row(const TsParams& p, int64_t count, int64_t tok) {
+  if (p.x_rows == nullptr) return token_row(p, count, tok);
+  tok = tok < count ? tok : count - 1;
+  return static_cast<int64_t>(p.x_rows[tok]);
+}
+
 // Loads the wavefront's token rows as B-operand fragments: lane (l32, hh) holds features 16*ks + 8*hh .. +7 of token
 // l32 of each 32-token tile.
 template <int D, int TT>
@@ -170,7 +179,7 @@ __device__ __forceinline__ void load_token_rows(const TsParams& p, int64_t count
   constexpr int KS = D / 16;
 #pragma unroll
   for (int t = 0; t < TT; ++t) {
-    const bf16_t* row = p.x + token_row(p, count, tok0 + t * 32 + l32) * p.ldx + hh * 8;
+    const bf16_t* row = p.x + input_row(p, count, tok0 + t * 32 + l32) * p.ldx + hh * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) xf[t][ks] = *reinterpret_cast<const bf16x8*>(row + ks * 16);
   }
@@ -822,8 +831,10 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(xf[t][ks]));
     if (QK != 0) {  // lane <-> token `lane` of the wavefront's 32 * TT tokens
-      const int64_t r = token_row(p, count, tok_base + (lane < 32 * TT ? lane : 0));
-      rowinfo[lane] = make_int2(static_cast<int>(r), static_cast<int>(r % p.tokens_per_sample));
+      // the token's position inside its sample is that of its row of x (the side that keeps the caller's layout)
+      const int64_t tok = tok_base + (lane < 32 * TT ? lane : 0);
+      rowinfo[lane] = make_int2(static_cast<int>(token_row(p, count, tok)),
+                                static_cast<int>(input_row(p, count, tok) % p.tokens_per_sample));
     }
   };
 
@@ -1136,7 +1147,8 @@ namespace {
 int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias, const void* out_packed,
               const void* norm_weight, float eps, const void* w_up, const void* b_up, const void* w_down,
               const void* b_down, const void* packed_weights, const void* residual, int64_t ldr, void* out, int64_t ldo,
-              int64_t M, int32_t D, int32_t F, int gate_first, const int32_t* rows, const int32_t* n_rows, void* stream) {
+              int64_t M, int32_t D, int32_t F, int gate_first, const int32_t* rows, const int32_t* n_rows,
+              const int32_t* x_rows, void* stream) {
   const bool with_proj = out_packed != nullptr;
   if (M < 0 || D <= 0 || F <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, D and F > 0", name);
   if (D != 256 && D != 128)
@@ -1152,6 +1164,7 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: the projection needs the block input and packed feed-forward weights", name);
   if ((rows == nullptr) != (n_rows == nullptr))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows and n_rows must be given together", name);
+  if (x_rows && !rows) return set_error(TAAC_ERR_INVALID_VALUE, "%s: x_rows needs rows and n_rows", name);
   if (rows && M > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: a row index covers at most 2^31 rows", name);
   if (!ptr_ok(x, 15) || !ptr_ok(w_up, 15) || !ptr_ok(w_down, 15) || !ptr_ok(out, 15) || !ptr_ok(residual, 15) ||
       !ptr_ok(norm_weight, 15) || !ptr_ok(b_up, 15) || !ptr_ok(b_down, 15) || !ptr_ok(packed_weights, 15) ||
@@ -1181,6 +1194,7 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
   p.packed = packed_weights ? 1 : 0;
   p.rows = rows;
   p.n_rows = n_rows;
+  p.x_rows = x_rows;
   p.w0 = static_cast<const bf16_t*>(out_packed);
   p.b0 = static_cast<const bf16_t*>(out_bias);
   p.units = compute_units();
@@ -1218,19 +1232,20 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
                                    int32_t F, int gate_first, const int32_t* rows, const int32_t* n_rows,
                                    void* stream) {
   return taac::ffn_entry("taac_swiglu_ffn_fwd", x, ldx, nullptr, nullptr, norm_weight, eps, w_up, b_up, w_down, b_down,
-                         packed_weights, residual, ldr, out, ldo, M, D, F, gate_first, rows, n_rows, stream);
+                         packed_weights, residual, ldr, out, ldo, M, D, F, gate_first, rows, n_rows, nullptr, stream);
 }
 
 extern "C" int taac_attn_out_ffn_fwd(const void* attn, int64_t ld_attn, const void* out_bias,
                                      const void* packed_out_weights, const void* residual, int64_t ldr,
                                      const void* norm_weight, float eps, const void* b_up, const void* b_down,
                                      const void* packed_ffn_weights, void* out, int64_t ldo, int64_t M, int32_t D,
-                                     int32_t F, const int32_t* rows, const int32_t* n_rows, void* stream) {
+                                     int32_t F, const int32_t* rows, const int32_t* n_rows,
+                                     const int32_t* attn_rows, void* stream) {
   const char* name = "taac_attn_out_ffn_fwd";
   if (!packed_out_weights || !packed_ffn_weights)
     return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: both weight sets must be packed", name);
   return taac::ffn_entry(name, attn, ld_attn, out_bias, packed_out_weights, norm_weight, eps, nullptr, b_up, nullptr,
-                         b_down, packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, stream);
+                         b_down, packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, attn_rows, stream);
 }
 
 namespace taac {
@@ -1248,7 +1263,7 @@ struct QkExtras {
 int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
                        const void* bias, const void* packed_weights, const void* residual, int64_t ldr, void* out,
                        int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows, const int32_t* n_rows,
-                       const QkExtras& qk, void* stream) {
+                       const int32_t* x_rows, const QkExtras& qk, void* stream) {
   if (M < 0 || N <= 0 || K <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, N and K > 0", name);
   if (K != 256 && K != 128)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: token-stationary kernel is built for K = 128 or 256 (got %d)", name, K);
@@ -1259,6 +1274,7 @@ int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void*
   if (!x || !out || (!packed_weights && !w)) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
   if ((rows == nullptr) != (n_rows == nullptr))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows and n_rows must be given together", name);
+  if (x_rows && !rows) return set_error(TAAC_ERR_INVALID_VALUE, "%s: x_rows needs rows and n_rows", name);
   if (M > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: at most 2^31 rows", name);
   if (!ptr_ok(x, 15) || !ptr_ok(w, 15) || !ptr_ok(out, 15) || !ptr_ok(residual, 15) || !ptr_ok(norm_weight, 15) ||
       !ptr_ok(bias, 15) || !ptr_ok(packed_weights, 15) || !ptr_ok(qk.qk_weight, 15) || !ptr_ok(qk.cos_sin, 15) ||
@@ -1285,6 +1301,7 @@ int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void*
   p.packed = packed_weights ? 1 : 0;
   p.rows = rows;
   p.n_rows = n_rows;
+  p.x_rows = x_rows;
   p.qk_w = static_cast<const bf16_t*>(qk.qk_weight);
   p.cos_sin = static_cast<const bf16_t*>(qk.cos_sin);
   p.qk_sumsq = qk.qk_sumsq;
@@ -1350,16 +1367,17 @@ __global__ __launch_bounds__(256) void row_rstd_kernel(const float* __restrict__
 extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
                                     const void* bias, const void* packed_weights, const void* residual, int64_t ldr,
                                     void* out, int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows,
-                                    const int32_t* n_rows, void* stream) {
+                                    const int32_t* n_rows, const int32_t* x_rows, void* stream) {
   return taac::norm_linear_launch("taac_norm_linear_fwd", x, ldx, norm_weight, eps, w, bias, packed_weights, residual,
-                                  ldr, out, ldo, M, N, K, rows, n_rows, taac::QkExtras{}, stream);
+                                  ldr, out, ldo, M, N, K, rows, n_rows, x_rows, taac::QkExtras{}, stream);
 }
 
 extern "C" int taac_norm_linear_qk_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
                                        const void* bias, const void* packed_weights, void* out, int64_t ldo, int64_t M,
                                        int32_t d_model, int32_t num_heads, int32_t tokens_per_sample,
                                        const void* qk_weight, const void* cos_sin, float* qk_sumsq,
-                                       const int32_t* rows, const int32_t* n_rows, void* stream) {
+                                       const int32_t* rows, const int32_t* n_rows, const int32_t* x_rows,
+                                       void* stream) {
   using namespace taac;
   const char* name = "taac_norm_linear_qk_fwd";
   if (d_model <= 0 || num_heads <= 0 || tokens_per_sample <= 0 || d_model % num_heads != 0)
@@ -1378,7 +1396,7 @@ extern "C" int taac_norm_linear_qk_fwd(const void* x, int64_t ldx, const void* n
   qk.head_dim = d_model / num_heads;
   qk.tokens_per_sample = tokens_per_sample;
   return norm_linear_launch(name, x, ldx, norm_weight, eps, w, bias, packed_weights, nullptr, 0, out, ldo, M,
-                            3 * d_model, d_model, rows, n_rows, qk, stream);
+                            3 * d_model, d_model, rows, n_rows, x_rows, qk, stream);
 }
 
 extern "C" int taac_row_rstd(const float* qk_sumsq, int64_t M, int32_t d_model, float eps, float* rstd,

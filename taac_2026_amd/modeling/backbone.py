@@ -13,13 +13,15 @@ sigmoid) executed by a single ``taac_backbone_fwd`` call.
 from __future__ import annotations
 
 import ctypes
+import os
 
 import torch
 import torch.nn as nn
 
 from taac_2026_amd import _native
-from taac_2026_amd.accelerators.attention import StructuredAttentionMask, qk_norm_rope, rope_table
-from taac_2026_amd.accelerators.linear import attention_out_ffn, norm_linear, qkv_projection, swiglu_ffn, valid_rows
+from taac_2026_amd.accelerators.attention import StructuredAttentionMask, front_structured_mask, qk_norm_rope, rope_table
+from taac_2026_amd.accelerators.linear import (attention_out_ffn, front_rows, norm_linear, qkv_projection, swiglu_ffn,
+                                               valid_rows)
 from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference
 from taac_2026_amd.modeling.normalization import RMSNorm
 from taac_2026_amd.modeling.sequence import scaled_dot_product_attention
@@ -166,9 +168,36 @@ class UnifiedInteractionBlock(nn.Module):
     def _forward_fused(self, tokens, padding_mask, attention_mask, key_lengths, return_attention_tokens, inplace):
         batch, token_count, d_model = tokens.shape
         x = tokens.contiguous()
-        index = valid_rows(key_lengths, token_count) if key_lengths is not None else \
-            valid_rows(None, token_count, padding_mask=padding_mask)
         attention = self.attention
+        structured = attention_mask if isinstance(attention_mask, StructuredAttentionMask) else None
+        dense_mask = None if structured is not None else attention_mask
+        # Padding scattered inside the samples, under a structured mask whose valid keys are exactly the non-padded
+        # positions: the projection writes every sample's valid tokens at the front of its rows, so that the attention
+        # call sees prefix padding (its cost follows the valid tokens, not the positions) with the mask's structure
+        # gathered per sample, and the out projection reads that layout back. TAAC_BLOCK_LAYOUT=positions keeps the
+        # tokens where they are (comparison knob).
+        # The indices and the gathered mask depend on the mask object only: the blocks of a stack, which all receive it,
+        # share them through its cache.
+        front = lengths = None
+        if (structured is not None and key_lengths is None and structured.padding_source is padding_mask
+                and structured.query_self is None and not structured.sample_stride
+                and structured.structural.shape == (token_count, token_count)
+                and os.environ.get("TAAC_BLOCK_LAYOUT", "front") != "positions"):
+            entry = structured.cache.get("front")
+            if entry is None:
+                index = valid_rows(None, token_count, padding_mask=padding_mask)
+                entry = (index, *front_rows(index, batch, token_count), front_structured_mask(structured, index, batch))
+                structured.cache["front"] = entry
+            index, front, lengths, structured = entry
+        elif key_lengths is not None:
+            index = valid_rows(key_lengths, token_count)
+        elif structured is not None and structured.padding_source is padding_mask:
+            index = structured.cache.get("rows")
+            if index is None:
+                index = structured.cache["rows"] = valid_rows(None, token_count, padding_mask=padding_mask)
+        else:
+            index = valid_rows(None, token_count, padding_mask=padding_mask)
+        qkv_rows = dict(token_rows=index) if front is None else dict(token_rows=(front, index[1]), input_rows=index[0])
         qkv = torch.empty(batch * token_count, 3 * d_model, dtype=x.dtype, device=x.device)
         q_row_scale = k_row_scale = q_col_scale = None
         if attention.query_norm is not None or attention.rope_base is not None:
@@ -178,19 +207,20 @@ class UnifiedInteractionBlock(nn.Module):
                 query_weight=None if attention.query_norm is None else _bf16(attention.query_norm.weight),
                 key_weight=None if attention.key_norm is None else _bf16(attention.key_norm.weight),
                 qk_eps=1e-6 if attention.query_norm is None else attention.query_norm.eps, rope_base=attention.rope_base,
-                token_rows=index, out=qkv)
+                out=qkv, **qkv_rows)
         else:
             norm_linear(x, _bf16(attention.qkv.weight), _bf16(attention.qkv.bias), norm_weight=_bf16(self.attn_norm.weight),
-                        eps=self.attn_norm.eps, token_rows=index, out=qkv)
+                        eps=self.attn_norm.eps, out=qkv, **qkv_rows)
         query, key, value = qkv.view(batch, token_count, 3 * d_model).chunk(3, dim=-1)
-        structured = attention_mask if isinstance(attention_mask, StructuredAttentionMask) else None
-        dense_mask = None if structured is not None else attention_mask
         attended = scaled_dot_product_attention(
             query, key, value, num_heads=attention.num_heads, attn_mask=dense_mask, structured_mask=structured,
-            dropout_p=0.0, training=False, key_lengths=key_lengths if attention_mask is None else None,
+            dropout_p=0.0, training=False, key_lengths=lengths if front is not None else (key_lengths if attention_mask is None else None),
+            zero_padded_queries=2 if front is not None else False,
             q_row_scale=q_row_scale, k_row_scale=k_row_scale, q_col_scale=q_col_scale)
         ffn = self.ffn
         dense = dict(norm_weight=_bf16(self.ffn_norm.weight), eps=self.ffn_norm.eps, token_rows=index)
+        if front is not None:
+            dense["input_rows"] = front
         if not return_attention_tokens and ffn.gate_first:
             output = x if inplace else x.clone()
             attention_out_ffn(attended, _bf16(attention.out.weight), _bf16(attention.out.bias), x, _bf16(ffn.up.weight),
@@ -198,8 +228,9 @@ class UnifiedInteractionBlock(nn.Module):
             return output, None
         attn_tokens = x.clone()  # padded rows pass through
         norm_linear(attended, _bf16(attention.out.weight), _bf16(attention.out.bias), residual=x, token_rows=index,
-                    out=attn_tokens)
+                    input_rows=front, out=attn_tokens)
         output = attn_tokens.clone()
+        dense.pop("input_rows", None)
         swiglu_ffn(attn_tokens, _bf16(ffn.up.weight), _bf16(ffn.up.bias), _bf16(ffn.down.weight), _bf16(ffn.down.bias),
                    residual=attn_tokens, gate_first=ffn.gate_first, out=output, **dense)
         return output, attn_tokens

@@ -97,7 +97,7 @@ class MetadataAttentionMask(nn.Module):
             structural = metadata_structural_mask(role_ids)
         else:
             structural = torch.ones(token_count, token_count, dtype=torch.bool, device=padding_mask.device)
-        return build_structured_mask(structural, ~safe_key_padding_mask(padding_mask), None)
+        return build_structured_mask(structural, ~safe_key_padding_mask(padding_mask), None, padding_source=padding_mask)
 
 
 __all__ = [

@@ -119,10 +119,11 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
 
     # out projection + feed-forward half in one kernel: both weight sets packed, the block input required
     def tail(**kw):
-        a = dict(packed_out=fake, residual=fake, packed_ffn=fake, d=256, f=64, m=8)
+        a = dict(packed_out=fake, residual=fake, packed_ffn=fake, d=256, f=64, m=8, rows=None, attn_rows=None)
         a.update(kw)
         return library.taac_attn_out_ffn_fwd(fake, a["d"], None, a["packed_out"], a["residual"], a["d"], None, 1e-6, None,
-                                             None, a["packed_ffn"], fake, a["d"], a["m"], a["d"], a["f"], None, None, None)
+                                             None, a["packed_ffn"], fake, a["d"], a["m"], a["d"], a["f"], a["rows"], a["rows"],
+                                             a["attn_rows"], None)
 
     assert tail(packed_out=None) == invalid and b"packed" in library.taac_last_error()
     assert tail(packed_ffn=None) == invalid
@@ -130,6 +131,10 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
     assert tail(d=192) == unsupported
     assert tail(f=48) == unsupported
     assert tail(m=0) == ok
+    assert tail(attn_rows=fake) == invalid and b"x_rows needs rows" in library.taac_last_error()
+    status = library.taac_norm_linear_fwd(fake, 256, None, 1e-6, fake, None, None, None, 0, fake, 64, 8, 64, 256, None, None,
+                                          fake, None)
+    assert status == invalid and b"x_rows needs rows" in library.taac_last_error()
 
     # readout: indices inside the sequence, one kind of validity, a complete classifier, something to write
     def readout(**kw):
@@ -153,14 +158,23 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
     strides = _native.Int64x4(2048, 16, 128, 1)
 
     def masked(**kw):
-        a = dict(lengths=None, struct=fake, any=fake, valid=None, self=None, tq=64, tk=64, d=16, zero=0, dtype=bf16)
+        a = dict(lengths=None, struct=fake, stride=0, any=fake, valid=None, self=None, tq=64, tk=64, d=16, zero=0, dtype=bf16)
         a.update(kw)
-        return library.taac_flash_attn_masked_fwd(fake, fake, fake, a["lengths"], a["struct"], a["any"], a["valid"],
+        return library.taac_flash_attn_masked_fwd(fake, fake, fake, a["lengths"], a["struct"], a["stride"], a["any"], a["valid"],
                                                   a["self"], None, None, None, fake, 1, 8, a["tq"], a["tk"], a["d"],
                                                   strides, strides, strides, strides, a["zero"], a["dtype"], None)
 
     assert masked(struct=None) == invalid and b"struct_bits" in library.taac_last_error()
     assert masked(any=None) == invalid and b"block_any" in library.taac_last_error()
+    assert masked(stride=64) == invalid and b"struct_sample_stride" in library.taac_last_error()
+    assert masked(stride=-1) == invalid
+    # the row index of the front layout and the mask gathered into it
+    assert library.taac_front_rows(None, fake, 2, 8, fake, fake, None) == invalid and b"null" in library.taac_last_error()
+    assert library.taac_front_rows(fake, fake, 0, 8, fake, fake, None) == ok
+    assert library.taac_front_rows(fake, fake, -1, 8, fake, fake, None) == invalid
+    assert library.taac_mask_front_bits(fake, 8192, fake, 2, fake, None) == unsupported
+    assert library.taac_mask_front_bits(None, 8, fake, 2, fake, None) == invalid
+    assert library.taac_mask_front_bits(fake, 8, fake, 0, fake, None) == ok
     assert masked(tk=4096 + 64) == unsupported and b"at most" in library.taac_last_error()
     assert masked(self=fake, tk=128) == invalid and b"self rows" in library.taac_last_error()
     assert masked(d=12) == unsupported

@@ -187,10 +187,12 @@ def _symbiosis_block_case(d_model, heads, tokens, batch, seed):
 
 
 @pytest.mark.parametrize("d_model,heads,tokens,batch", [(128, 4, 70, 5), (256, 8, 150, 4)])
-def test_interaction_block_fused_routes_under_role_masks_and_scattered_padding(device, d_model, heads, tokens, batch):
+def test_interaction_block_fused_routes_under_role_masks_and_scattered_padding(device, monkeypatch, d_model, heads, tokens,
+                                                                               batch):
     """The reference block as the model runs it: role-based attention mask, padding anywhere in the sequence, updates
     masked at padded rows. Both fused routes against the oracle's statement of the block; padded rows pass through bit
-    for bit and are never read (NaN there changes nothing)."""
+    for bit and are never read (NaN there changes nothing). With the model's own mask object the attention runs over
+    every sample's valid tokens moved to the front; a dense mask (or TAAC_BLOCK_LAYOUT=positions) keeps the positions."""
     block, x, padding, roles, state, mask_module = _symbiosis_block_case(d_model, heads, tokens, batch, seed=d_model + tokens)
     dense_mask = oracle.metadata_attention_mask(padding, roles)
     want, want_attn = oracle.interaction_block(x.float(), padding, dense_mask, {k: v.float() for k, v in state.items()},
@@ -202,6 +204,9 @@ def test_interaction_block_fused_routes_under_role_masks_and_scattered_padding(d
         two, two_attn = block(x.to(device), padding.to(device), mask)
         one, none = block(x.to(device), padding.to(device), mask, return_attention_tokens=False)
         from_dense, _ = block(x.to(device), padding.to(device), dense_mask.to(device))
+        monkeypatch.setenv("TAAC_BLOCK_LAYOUT", "positions")
+        by_position, by_position_attn = block(x.to(device), padding.to(device), mask)
+        monkeypatch.delenv("TAAC_BLOCK_LAYOUT")
         poisoned = x.clone()
         poisoned[padding] = float("nan")
         stream = poisoned.to(device)
@@ -211,7 +216,9 @@ def test_interaction_block_fused_routes_under_role_masks_and_scattered_padding(d
     torch.testing.assert_close(two.cpu().float()[valid], want[valid], rtol=2e-2, atol=2e-2)
     torch.testing.assert_close(one.cpu().float()[valid], want[valid], rtol=2e-2, atol=2e-2)
     torch.testing.assert_close(one.cpu().float(), two.cpu().float(), rtol=2 ** -6, atol=2 ** -6)
-    assert torch.equal(from_dense.cpu(), two.cpu())
+    assert torch.equal(from_dense.cpu(), by_position.cpu())
+    torch.testing.assert_close(by_position_attn.cpu().float()[valid], want_attn[valid], rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(by_position.cpu().float(), two.cpu().float(), rtol=2 ** -6, atol=2 ** -6)
     for result in (two, one, two_attn):
         assert torch.equal(result.cpu()[padding], x[padding])          # x + update * 0
     assert torch.equal(in_place.cpu()[valid], one.cpu()[valid])
