@@ -214,18 +214,36 @@ def _operator_figures(device, iters: int) -> dict:
             "frac_mfma": useful / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS,
             "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS,
         }
-    # attention backward at the same shape (training forward + both backward kernels timed together, minus the training
-    # forward alone); algorithmic FLOPs: five products against the forward's two
-    qg, kg, vg = (t.clone().requires_grad_(True) for t in (qd, kd, vd))
-    go = torch.randn(q.shape, generator=torch.Generator().manual_seed(9)).to(torch.bfloat16).to(device)
-    fwd = lambda: flash_attention(qg, kg, vg, key_lengths=ld, zero_padded_queries=True)  # noqa: E731
-    ms_fwd = _event_ms(fwd, iters, 3)
-    ms_both = _event_ms(lambda: torch.autograd.grad(fwd(), (qg, kg, vg), go), iters, 3)
-    ms_bwd = ms_both - ms_fwd
-    figures["attention_bwd_bf16_B2048_H4_T256_d64"] = {
-        "training_fwd_ms": ms_fwd, "bwd_ms": ms_bwd, "useful_tflops": 2.5 * useful / ms_bwd / 1e9,
-        "frac_mfma": 2.5 * useful / ms_bwd / 1e9 / MFMA_BF16_PEAK_TFLOPS,
-    }
+    del qd, kd, vd
+    figures.update(_attention_bwd_figures(device, iters))
+    return figures
+
+
+def _attention_bwd_figures(device, iters: int) -> dict:
+    """Attention backward at the configuration-3 shape and at the headline attention shape (training forward + both
+    backward kernels timed together, minus the training forward alone); algorithmic FLOPs: five products against the
+    forward's two."""
+    from taac_2026_amd import workloads
+    from taac_2026_amd.api import flash_attention
+
+    figures = {}
+    for label, kwargs in (("B2048_H4_T256_d64", {}),
+                          ("B1024_H8_T512_d32", dict(batch=1024, heads=8, tokens=512, head_dim=32, min_len=64))):
+        q, k, v, lengths = workloads.attention_inputs(**kwargs)
+        _, H, _, d = q.shape
+        useful = 4.0 * H * d * float((lengths.double() ** 2).sum().item())
+        ld = lengths.to(device)
+        qg, kg, vg = (t.to(device).requires_grad_(True) for t in (q, k, v))
+        go = torch.randn(q.shape, generator=torch.Generator().manual_seed(9)).to(torch.bfloat16).to(device)
+        fwd = lambda: flash_attention(qg, kg, vg, key_lengths=ld, zero_padded_queries=True)  # noqa: E731
+        ms_fwd = _event_ms(fwd, iters, 3)
+        ms_both = _event_ms(lambda: torch.autograd.grad(fwd(), (qg, kg, vg), go), iters, 3)
+        ms_bwd = ms_both - ms_fwd
+        figures[f"attention_bwd_bf16_{label}"] = {
+            "training_fwd_ms": ms_fwd, "bwd_ms": ms_bwd, "useful_tflops": 2.5 * useful / ms_bwd / 1e9,
+            "frac_mfma": 2.5 * useful / ms_bwd / 1e9 / MFMA_BF16_PEAK_TFLOPS,
+        }
+        del qg, kg, vg, go
     return figures
 
 
@@ -539,6 +557,8 @@ def main() -> None:
                              "and print those figures (for kernel traces of that mode)")
     parser.add_argument("--only-kernels", action="store_true",
                         help="time only the stand-alone kernels of one block (short run for hardware-counter collection)")
+    parser.add_argument("--only-attention-bwd", action="store_true",
+                        help="time only the attention backward at its two shapes (short run for traces and counters)")
     parser.add_argument("--only-reference-block", action="store_true",
                         help="time only the reference model's block (role mask, scattered padding) and print those figures")
     args = parser.parse_args()
@@ -560,6 +580,9 @@ def main() -> None:
     if args.only_kernels:
         inputs = workloads.backbone_inputs(batch=args.batch)
         print(json.dumps({"kernels": _kernel_breakdown(inputs, device, iters=6)}))
+        return
+    if args.only_attention_bwd:
+        print(json.dumps({"attention_bwd": _attention_bwd_figures(device, iters=6)}))
         return
     if args.only_reference_block:
         print(json.dumps({"reference_block": _reference_block_figures(device, args.batch, 10)}))
