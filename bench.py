@@ -463,7 +463,7 @@ def _reference_block_figures(device, batch: int, iters: int) -> dict:
     masked at padded rows. Timed: the fused route that leaves out the intermediate stream (3 heavy kernels + the row
     index) and the route that returns it, plus a block checked against the oracle on a small slice."""
     from oracle import reference as oracle
-    from taac_2026_amd.api import MetadataAttentionMask, UnifiedInteractionBlock
+    from taac_2026_amd.api import MetadataAttentionMask, UnifiedInteractionBlock, run_interaction_blocks
 
     g = torch.Generator().manual_seed(42)
     T, D, H = 512, 256, 8
@@ -479,7 +479,8 @@ def _reference_block_figures(device, batch: int, iters: int) -> dict:
     block = block.to(device)
     dev_x, dev_pad = x.to(device), padding.to(device)
     with torch.no_grad():
-        mask = MetadataAttentionMask(enabled=True)(dev_pad, roles.to(device))
+        mask_module, dev_roles = MetadataAttentionMask(enabled=True), roles.to(device)
+        mask = mask_module(dev_pad, dev_roles)
         got, _ = block(dev_x, dev_pad, mask, return_attention_tokens=False)
         valid = ~padding[small]
         err = (got[small].cpu().float()[valid] - want[valid]).abs().max().item()
@@ -494,8 +495,14 @@ def _reference_block_figures(device, batch: int, iters: int) -> dict:
 
         first = _event_ms(first_block, iters, 3)
         both = _event_ms(lambda: block(dev_x, dev_pad, mask), iters, 3)
+
+        def stack():  # the reference model's block loop, four blocks: one copy of the stream, a fresh mask per pass
+            return run_interaction_blocks([block] * 4, dev_x, dev_pad, mask_module(dev_pad, dev_roles))
+
+        stack_ms = _event_ms(stack, max(4, iters // 2), 2)
     return {"valid_token_fraction": float((~padding).float().mean().item()), "one_kernel_tail_in_place_ms": fused,
-            "first_block_of_a_stack_ms": first, "with_attention_tokens_ms": both, "max_abs_err_vs_oracle": err,
+            "first_block_of_a_stack_ms": first, "with_attention_tokens_ms": both,
+            "stack_of_4_blocks_with_mask_build_ms": stack_ms, "max_abs_err_vs_oracle": err,
             "note": "whole module calls: projection + norm statistic into the front layout, attention over the valid "
                     "tokens under the gathered mask, out projection + feed-forward; the row indices and the gathered "
                     "mask are shared by the blocks of a stack through the mask object (first_block_of_a_stack_ms "

@@ -5,6 +5,7 @@ from taac_2026_amd.modeling.backbone import (
     PCVRBackbone,
     SwiGLUFeedForward,
     UnifiedInteractionBlock,
+    run_interaction_blocks,
     UnifiedSelfAttention,
 )
 from taac_2026_amd.modeling.embeddings import hash_compress_ids, sparse_embedding_bag_mean
@@ -41,6 +42,7 @@ __all__ = [
     "RMSNorm",
     "SwiGLUFeedForward",
     "UnifiedInteractionBlock",
+    "run_interaction_blocks",
     "UnifiedSelfAttention",
     "bfts_attention_mask",
     "bfts_structural_mask",

@@ -184,17 +184,20 @@ class UnifiedInteractionBlock(nn.Module):
                 and structured.structural.shape == (token_count, token_count)
                 and os.environ.get("TAAC_BLOCK_LAYOUT", "front") != "positions"):
             entry = structured.cache.get("front")
-            if entry is None:
+            if entry is None or entry[0] != padding_mask._version:  # rebuilt when the padding mask was written to
                 index = valid_rows(None, token_count, padding_mask=padding_mask)
-                entry = (index, *front_rows(index, batch, token_count), front_structured_mask(structured, index, batch))
+                entry = (padding_mask._version, index, *front_rows(index, batch, token_count),
+                         front_structured_mask(structured, index, batch))
                 structured.cache["front"] = entry
-            index, front, lengths, structured = entry
+            _, index, front, lengths, structured = entry
         elif key_lengths is not None:
             index = valid_rows(key_lengths, token_count)
         elif structured is not None and structured.padding_source is padding_mask:
-            index = structured.cache.get("rows")
-            if index is None:
-                index = structured.cache["rows"] = valid_rows(None, token_count, padding_mask=padding_mask)
+            entry = structured.cache.get("rows")
+            if entry is None or entry[0] != padding_mask._version:
+                entry = structured.cache["rows"] = (padding_mask._version,
+                                                    valid_rows(None, token_count, padding_mask=padding_mask))
+            index = entry[1]
         else:
             index = valid_rows(None, token_count, padding_mask=padding_mask)
         qkv_rows = dict(token_rows=index) if front is None else dict(token_rows=(front, index[1]), input_rows=index[0])
@@ -253,6 +256,19 @@ class UnifiedInteractionBlock(nn.Module):
         ffn_update = self.ffn(self.ffn_norm(attn_tokens))
         output = attn_tokens + ffn_update * keep.to(ffn_update.dtype)
         return output, attn_tokens
+
+
+def run_interaction_blocks(blocks, tokens: torch.Tensor, padding_mask: torch.Tensor,
+                           attention_mask: torch.Tensor | StructuredAttentionMask | None) -> torch.Tensor:
+    """The block loop of the reference model's ``_run_backbone`` (experiments/symbiosis/model.py:283-292, without its
+    ``final_norm``, which the readout head applies): every block receives the same padding mask and attention mask and
+    only its output stream is kept. The stream is copied once and the blocks then update it in place; with a mask from
+    ``MetadataAttentionMask`` the row indices and the mask gathered per sample are built by the first block and shared
+    by the others. The padding mask must not be modified while the loop runs."""
+    stream = tokens
+    for position, block in enumerate(blocks):
+        stream, _ = block(stream, padding_mask, attention_mask, return_attention_tokens=False, inplace=position > 0)
+    return stream
 
 
 class _PlainBlock(nn.Module):

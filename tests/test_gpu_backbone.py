@@ -239,6 +239,31 @@ def test_interaction_block_routes_agree(device):
     torch.testing.assert_close(plain.cpu()[valid], fused.cpu().float()[valid], rtol=2e-2, atol=2e-2)
 
 
+def test_block_stack_shares_the_indices_of_its_mask(device):
+    """run_interaction_blocks = the blocks called one after the other on fresh tensors, bit for bit; the indices and the
+    gathered mask are built once (by the first block) and rebuilt when the padding mask is written to."""
+    from taac_2026_amd.api import run_interaction_blocks
+
+    block, x, padding, roles, _, mask_module = _symbiosis_block_case(128, 4, 70, 5, seed=21)
+    other, *_ = _symbiosis_block_case(128, 4, 70, 5, seed=22)
+    blocks = [block.to(device), other.to(device), block]
+    dev_x, dev_pad = x.to(device), padding.to(device)
+    with torch.no_grad():
+        mask = mask_module(dev_pad, roles.to(device))
+        expected = dev_x
+        for module in blocks:
+            expected, _ = module(expected, dev_pad, mask_module(dev_pad, roles.to(device)), return_attention_tokens=False)
+        before = dev_x.clone()
+        got = run_interaction_blocks(blocks, dev_x, dev_pad, mask)
+        assert torch.equal(dev_x, before) and got.data_ptr() != dev_x.data_ptr()
+        assert torch.equal(got, expected)
+        entry = mask.cache["front"]
+        assert run_interaction_blocks(blocks, dev_x, dev_pad, mask) is not None and mask.cache["front"] is entry
+        dev_pad[3, 5] = ~dev_pad[3, 5]     # an in-place write: the cached indices no longer describe the mask
+        run_interaction_blocks(blocks[:1], dev_x, dev_pad, mask)
+        assert mask.cache["front"] is not entry
+
+
 def test_valid_rows_from_a_padding_mask(device):
     from taac_2026_amd.api import valid_rows
 
