@@ -84,9 +84,11 @@ def test_direct_transfer_backward_equals_register_staged_backward(device, monkey
     lengths = torch.tensor([333, 1, 64, 65, 200], dtype=torch.int32, device=device)
     grads = {}
     for staging in ("direct", "registers"):
-        monkeypatch.setenv("TAAC_ATTN_STAGING", staging)
+        monkeypatch.setenv("TAAC_ATTN_STAGING", "direct")  # the same training forward (output, log-sum-exp) for both
         qd, kd, vd = (t.clone().requires_grad_(True) for t in (q, k, v))
-        flash_attention(qd, kd, vd, key_lengths=lengths, is_causal=causal, zero_padded_queries=not causal).backward(grad_out)
+        out = flash_attention(qd, kd, vd, key_lengths=lengths, is_causal=causal, zero_padded_queries=not causal)
+        monkeypatch.setenv("TAAC_ATTN_STAGING", staging)
+        out.backward(grad_out)
         grads[staging] = (qd.grad, kd.grad, vd.grad)
     for direct, staged in zip(grads["direct"], grads["registers"]):
         assert torch.isfinite(direct.float()).all()
