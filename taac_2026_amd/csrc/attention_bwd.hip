@@ -494,6 +494,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
         // causal diagonal needs per-element tests. A padded key of the lane (zeros in kf and vf) collects finite
         // values in its own accumulator column only, which is cleared after the loop.
         const bool diagonal = p.causal && qc0 + qt * 32 < k_begin + wave * 32 + 31;
+        if (diagonal) {  // wavefront-uniform: the other tiles pay nothing for the triangle
+#pragma unroll
+          for (int j = 0; j < 16; ++j)
+            if (kj > qc0 + qt * 32 + (j / 4) * 8 + hh * 4 + (j % 4)) sacc[j] = -INFINITY;
+        }
         vec_t pb[2], dsb[2];
 #pragma unroll
         for (int jq = 0; jq < 4; ++jq) {
@@ -503,9 +508,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int j = jq * 4 + e;
-            float sc = sacc[j];
-            if (diagonal && kj > qc0 + r0 + e) sc = -INFINITY;
-            const float prob = __builtin_amdgcn_exp2f(fmaf(sc, c, -l4[e]));
+            const float prob = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -l4[e]));
             pb[j / 8][j % 8] = static_cast<T>(prob);
             dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -d4[e]));
           }
