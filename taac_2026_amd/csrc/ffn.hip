@@ -394,9 +394,10 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
     asm volatile("" : "+v"(ln));
     uint8_t* base = smem + buf * (NFRAG * kFrag) + wave * (FPW * kFrag);
     if (p.packed) {
-      const char* src = w_up_bytes + (static_cast<int64_t>(step) * NFRAG + wave * FPW) * kFrag + ln * 16;
+      const char* src = w_up_bytes + (static_cast<int64_t>(step) * NFRAG + wave * FPW) * kFrag;  // scalar registers
+      const uint32_t lane_off = static_cast<uint32_t>(ln * 16);
 #pragma unroll
-      for (int i = 0; i < FPW; ++i) lds_dma16(src + i * kFrag, base + i * kFrag);
+      for (int i = 0; i < FPW; ++i) lds_dma16_offset(src + i * kFrag, lane_off, base + i * kFrag);
       return;
     }
     const int s32 = ln & 31, shh = ln >> 5;
@@ -423,9 +424,10 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
     int ln = lane;
     asm volatile("" : "+v"(ln));
     uint8_t* base = smem + buf * (NFRAG * kFrag) + wave * (CFW * kFrag);
-    const char* src = reinterpret_cast<const char*>(p.w0) + (static_cast<int64_t>(c) * CF + wave * CFW) * kFrag + ln * 16;
+    const char* src = reinterpret_cast<const char*>(p.w0) + (static_cast<int64_t>(c) * CF + wave * CFW) * kFrag;
+    const uint32_t lane_off = static_cast<uint32_t>(ln * 16);
 #pragma unroll
-    for (int i = 0; i < CFW; ++i) lds_dma16(src + i * kFrag, base + i * kFrag);
+    for (int i = 0; i < CFW; ++i) lds_dma16_offset(src + i * kFrag, lane_off, base + i * kFrag);
   };
 
   stage(0, 0);
@@ -794,9 +796,10 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     asm volatile("" : "+v"(ln));
     uint8_t* base = smem + buf * kBuf + wave * (FPW * kFrag);
     if (p.packed) {
-      const char* src = w_bytes + (static_cast<int64_t>(chunk) * NFRAG + wave * FPW) * kFrag + ln * 16;
+      const char* src = w_bytes + (static_cast<int64_t>(chunk) * NFRAG + wave * FPW) * kFrag;  // scalar registers
+      const uint32_t lane_off = static_cast<uint32_t>(ln * 16);
 #pragma unroll
-      for (int i = 0; i < FPW; ++i) lds_dma16(src + i * kFrag, base + i * kFrag);
+      for (int i = 0; i < FPW; ++i) lds_dma16_offset(src + i * kFrag, lane_off, base + i * kFrag);
       return;
     }
     const uint32_t lane_off = static_cast<uint32_t>(((ln & 31) * D + (ln >> 5) * 8) * 2);
