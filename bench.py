@@ -70,16 +70,49 @@ def _event_ms_after(prelude, fn, iters: int, warmup: int) -> float:
     return times[len(times) // 2]
 
 
-def _measured_traffic(kernel_name: str) -> int | None:
+TRAFFIC_SUMMARY = "profiles/pmc_traffic_backbone_c4.txt"
+
+
+def _measured_traffic(kernel_name: str) -> int:
     """HBM bytes per launch of ``kernel_name`` as measured with the FETCH_SIZE / WRITE_SIZE counters (scaled by a kernel
-    of known traffic); read from the committed counter summary, None if the kernel is not listed there."""
-    summary = REPO_ROOT / "profiles" / "pmc_traffic_backbone_c4.txt"
-    if not summary.exists():
-        return None
-    for line in summary.read_text().splitlines():
-        if line.startswith(kernel_name + ":") and "traffic_bytes=" in line:
-            return int(line.split("traffic_bytes=")[1].split()[0])
-    return None
+    of known traffic). The counters cannot be read from inside this process: the figure is taken from the committed
+    counter summary (the line says so) and the run fails when the kernel is not listed there, so that a renamed or new
+    dominant kernel cannot silently carry another kernel's traffic."""
+    summary = REPO_ROOT / TRAFFIC_SUMMARY
+    if summary.exists():
+        for line in summary.read_text().splitlines():
+            if line.startswith(kernel_name + ":") and "traffic_bytes=" in line:
+                return int(line.split("traffic_bytes=")[1].split()[0])
+    raise SystemExit(f"bench.py: no measured traffic for kernel '{kernel_name}' in {TRAFFIC_SUMMARY}; collect the "
+                     "FETCH_SIZE / WRITE_SIZE counters for it (commands in that file) before reporting a roofline")
+
+
+def _sustained(step, batch: int, *, heat_s: float = 2.0, repeats: int = 5, repeat_s: float = 0.4) -> dict:
+    """Back-to-back steps for ``heat_s`` seconds (the chip settles at its sustained clock after ~0.6 s of continuous
+    load), then ``repeats`` timed groups of ~``repeat_s`` seconds each, host clock around a device synchronisation:
+    median and 95th percentile of the per-step time over the groups."""
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    step()
+    torch.cuda.synchronize()
+    one = max(time.perf_counter() - t0, 1e-4)
+    heat_steps = max(10, int(heat_s / one))
+    per_group = max(10, int(repeat_s / one))
+    for _ in range(heat_steps):
+        step()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        for _ in range(per_group):
+            step()
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3 / per_group)
+    times.sort()
+    median = times[len(times) // 2]
+    p95 = times[min(len(times) - 1, int(round(0.95 * (len(times) - 1))))]
+    return {"ms_per_step_median": median, "ms_per_step_p95": p95, "samples_per_s": batch / (median * 1e-3),
+            "heat_steps": heat_steps, "repeats": repeats, "steps_per_repeat": per_group}
 
 
 def _accuracy_gate(model, inputs, device) -> dict:
@@ -134,7 +167,7 @@ def _kernel_breakdown(inputs, device, iters: int) -> dict:
                                           w["down.weight"], w["down.bias"], norm_weight=w["ffn_norm.weight"],
                                           token_rows=index, out=buf),
                 2.0 * Mv * (D * D + 3 * D * F), 2.0 * (3 * Mv * D + D * D + 3 * D * F)),
-            # the same two halves as kernels of their own (the route TAAC_SPLIT_OUT_FFN=1 takes; not part of the step)
+            # the same two halves as kernels of their own (the split_out_ffn=True route; not part of the step)
             "split:out_residual": (lambda: norm_linear(a, w["out.weight"], w["out.bias"], residual=x, token_rows=index, out=buf),
                                    2.0 * Mv * D * D, 2.0 * (3 * Mv * D + D * D)),
             "split:rmsnorm_swiglu_ffn_residual": (
@@ -209,7 +242,6 @@ def _operator_figures(device, iters: int) -> dict:
         figures["attention_bf16_B2048_H4_T256_d64"] = {
             "ms": ms,
             "useful_tflops": useful / ms / 1e9,
-            "dense_equivalent_tflops": 4.0 * B * H * T * T * d / ms / 1e9,
             "gbs": nbytes / ms / 1e6,
             "frac_mfma": useful / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS,
             "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS,
@@ -623,16 +655,22 @@ def main() -> None:
     ms_per_step = elapsed * 1e3 / args.steps
     value = B / (elapsed / args.steps)
 
+    # Sustained figure: the timed window above lies inside the first ~0.6 s of load, where the chip still runs at its
+    # boost clock; this one is taken after 2 s of back-to-back steps.
+    with torch.no_grad():
+        sustained = _sustained(lambda: model(emb, lengths), B)
+
     # The same step with the dense layers run over all B*T positions, padding included (what the reference's dense
     # [B, T, D] formulation does): reported next to the headline figure, never as the value.
-    dense_ms = None
+    dense = None
     if not args.skip_all_positions:
-        os.environ["TAAC_DENSE_TOKENS"] = "1"
-        try:
-            with torch.no_grad():
-                dense_ms = _event_ms(lambda: model(emb, lengths), max(args.steps // 2, 1), 2)
-        finally:
-            del os.environ["TAAC_DENSE_TOKENS"]
+        with torch.no_grad():
+            run_dense = lambda: model(emb, lengths, dense_tokens=True)  # noqa: E731
+            dense_ms = _event_ms(run_dense, max(args.steps // 2, 1), 2)
+            dense = {"ms_per_step": dense_ms, "samples_per_s": B / (dense_ms * 1e-3),
+                     "sustained": _sustained(run_dense, B),
+                     "note": "dense layers run over the padded positions too (dense_tokens=True): the figure "
+                             "comparable to a dense [B, T, D] formulation"}
     valid_fraction = float(inputs.key_lengths.clamp(0, T).sum().item()) / (B * T)
 
     kernels = _kernel_breakdown(inputs, device, iters=10)
@@ -652,11 +690,11 @@ def main() -> None:
         "unit": "TFLOP/s" if bound == "mfma" else "GB/s",
         "frac": tflops / MFMA_BF16_PEAK_TFLOPS if bound == "mfma" else gbs / HBM_PEAK_GBS,
         "traffic": _measured_traffic(dominant),
+        "traffic_source": f"{TRAFFIC_SUMMARY} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE; not measured in this run)",
         "launch_ms": launch_ms,
         "launch_ms_standalone": dom["ms"],
     }
 
-    dense_flops = len(inputs.blocks) * (2.0 * B * T * (3 * D * D + D * D + 3 * D * inputs.d_ff) + 4.0 * B * T * T * D)
     line = {
         "metric": "pCVR samples/s (4-block fwd, B=1024,T=512); attn TFLOP/s; norm HBM GB/s",
         "value": value,
@@ -678,11 +716,9 @@ def main() -> None:
             "batch": B,
             "tokens": T,
         },
-        "dense_equivalent_tflops": dense_flops / (elapsed / args.steps) / 1e12,
+        "sustained": sustained,
         "valid_token_fraction": valid_fraction,
-        "all_positions": None if dense_ms is None else {
-            "ms_per_step": dense_ms, "samples_per_s": B / (dense_ms * 1e-3),
-            "note": "dense layers run over the padded positions too (TAAC_DENSE_TOKENS=1)"},
+        "all_positions": dense,
         "roofline": roofline,
         "accuracy": accuracy,
         "kernels": kernels,

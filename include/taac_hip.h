@@ -10,8 +10,10 @@
  *     returns a human-readable message (thread-local storage, valid until the next call on that thread).
  *   - Arguments are validated on the host before any kernel is launched; a rejected call launches nothing.
  *   - `dtype` is a taac_dtype value.
- *   - No global mutable state besides the thread-local error string: calls from different host threads
- *     and on different streams are independent.
+ *   - No global mutable state besides the thread-local error string: calls from different host threads and on different streams are independent.
+ *     Behaviour is chosen by arguments only. Two environment variables exist as TEST HOOKS and change no result:
+ *     TAAC_TS_MAX_WORKGROUPS caps the grid of the persistent dense kernels (so that small test inputs walk several
+ *     tiles per workgroup), TAAC_FP8_TILED routes taac_linear_fp8 to its generic tiled kernel.
  *
  * Each declaration cites the reference interface it replaces (path:line under the reference tree,
  * Puiching-Memory/TAAC_2026). The reference has no C ABI on this path: its operators are Python
@@ -27,7 +29,7 @@
 extern "C" {
 #endif
 
-#define TAAC_ABI_VERSION 4
+#define TAAC_ABI_VERSION 5
 
 enum taac_status {
   TAAC_OK = 0,
@@ -44,6 +46,15 @@ enum taac_epilogue {
   TAAC_EPI_RESIDUAL = 1, /* out = residual + a @ w^T (+ bias); out may alias residual          */
   TAAC_EPI_SWIGLU = 2  /* w is [2F, K]; out[M, F] = silu(g) * u (gate_first) or g * silu(u)    */
 };
+
+/* Bits of the `is_causal` argument of the key-length attention entry points (forward, scaled, training pair). */
+#define TAAC_ATTN_CAUSAL 1           /* key j is visible to query i only if j <= i                                */
+#define TAAC_ATTN_REGISTER_STAGING 2 /* stage K / V chunks through registers instead of direct global -> LDS       */
+                                     /* transfers: same arithmetic and results, kept as a comparison route        */
+
+/* Bits of the `flags` argument of taac_backbone_fwd. */
+#define TAAC_BACKBONE_DENSE_TOKENS 1  /* run the dense layers over the padded positions too                        */
+#define TAAC_BACKBONE_SPLIT_OUT_FFN 2 /* out projection and feed-forward half as two kernels instead of one        */
 
 int taac_abi_version(void);
 const char* taac_last_error(void);
@@ -75,8 +86,9 @@ int taac_layernorm_fwd(const void* x, const void* w, const void* b, void* y, int
  * The row statistics are recomputed from x (nothing is saved by the forward). x, dy, dx: [rows, cols] contiguous;
  * w, dw, db: [cols]; all in `dtype`, fp32 arithmetic. dw / db may be NULL (not wanted). workspace: device memory for
  * taac_norm_bwd_workspace_floats(rows, cols, layer_norm) floats (per-workgroup partial sums of dw / db, added in a
- * fixed order: the result does not depend on scheduling). cols must be a multiple of the 16-byte vector (8 elements,
- * 4 for fp32) and at most 256 vectors.
+ * fixed order: the result does not depend on scheduling). Rows of whole 16-byte vectors (8 elements, 4 for fp32), at
+ * most 256 of them, with 16-byte aligned tensors take the one-pass vector kernel; every other shape takes a generic
+ * kernel (one workgroup per row at a time, the row swept four times).
  * Replaces: the Triton / TileLang backward kernels and their host-side partial sums
  * (accelerators/normalization/kernels/triton.py:82-116, 276-320; rms_norm.py:294-340, layer_norm.py:170-258).
  */
@@ -89,7 +101,8 @@ int taac_layernorm_bwd(const void* x, const void* w, const void* dy, void* dx, v
 /*
  * Key-padding-masked attention forward: o = softmax(q k^T / sqrt(d) + mask) v per (batch, head), softmax in
  * fp32, bf16/fp16 MFMA operands. Key j of batch b is visible iff j < key_lengths[b] (and j <= query index when
- * is_causal). key_lengths == NULL means every key is visible. Rows with no visible key produce zeros.
+ * is_causal has TAAC_ATTN_CAUSAL set; is_causal is a bit set, 0 / 1 keep their plain meaning).
+ * key_lengths == NULL means every key is visible. Rows with no visible key produce zeros.
  * q/o: logical shape (B, H, Tq, d); k/v: (B, H, Tk, d). *_strides are ELEMENT strides of the four logical
  * dimensions, so (B,H,T,d)-contiguous and (B,T,H,d)-contiguous tensors are both read in place; the last
  * stride must be 1, the others multiples of 8, and base pointers 16-byte aligned. d must be a multiple of 8, <= 128.
@@ -479,8 +492,9 @@ int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D, int32_t F
  * emb: [B, T, D] bf16 (not modified); key_lengths: int32 [B] valid-prefix lengths; hidden_out: [B, T, D] bf16
  * final hidden state or NULL; p: float [B]. heads divides D and D / heads is a multiple of 8.
  * rope_cos_sin: [T, D / heads / 2, 2] bf16 table of (cos, sin) as in taac_qk_norm_rope_fwd, or NULL (no rotation);
- * the same eps serves every norm. Rows at or beyond key_lengths[b] of hidden_out hold unspecified finite values (they
- * are never read by the readout).
+ * the same eps serves every norm. flags: TAAC_BACKBONE_* bits, 0 for the default route (the dense layers skip the
+ * padded positions; rows at or beyond key_lengths[b] of hidden_out are then zeros, with TAAC_BACKBONE_DENSE_TOKENS they
+ * hold the values the dense formulation computes there; the readout never reads them).
  * Replaces: the block loop _run_backbone (experiments/symbiosis/model.py:283-292) over UnifiedInteractionBlock
  * (experiments/symbiosis/backbone.py:50-68) in its canonical pre-norm form, plus masked_mean + Linear + sigmoid; with
  * the query / key norm weights UnifiedSelfAttention as the reference runs it (backbone.py:24-48), with the table
@@ -488,8 +502,8 @@ int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D, int32_t F
  */
 int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, const taac_block_weights* blocks, int32_t n_blocks,
                       const void* w_head, const void* b_head, int32_t B, int32_t T, int32_t D, int32_t heads, int32_t F,
-                      float eps, const void* rope_cos_sin, void* workspace, int64_t workspace_bytes, void* hidden_out,
-                      float* p, void* stream);
+                      float eps, const void* rope_cos_sin, int flags, void* workspace, int64_t workspace_bytes,
+                      void* hidden_out, float* p, void* stream);
 
 #ifdef __cplusplus
 }

@@ -21,8 +21,10 @@ TAAC_ERR_LAUNCH = -3
 
 TAAC_F32, TAAC_BF16, TAAC_F16 = 0, 1, 2
 EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
+ATTN_CAUSAL, ATTN_REGISTER_STAGING = 1, 2
+BACKBONE_DENSE_TOKENS, BACKBONE_SPLIT_OUT_FFN = 1, 2
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _DTYPE_CODES = {torch.float32: TAAC_F32, torch.bfloat16: TAAC_BF16, torch.float16: TAAC_F16}
 
@@ -168,7 +170,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "taac_backbone_fwd": (
         c_int,
         [c_void_p, c_void_p, ctypes.POINTER(BlockWeights), c_int32, c_void_p, c_void_p, c_int32, c_int32, c_int32,
-         c_int32, c_int32, c_float, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
+         c_int32, c_int32, c_float, c_void_p, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
     ),
 }
 

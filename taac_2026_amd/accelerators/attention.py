@@ -324,6 +324,7 @@ def hip_flash_attention_kernel(
     k_row_scale: torch.Tensor | None = None,
     q_col_scale: torch.Tensor | None = None,
     structured_mask: StructuredAttentionMask | None = None,
+    kv_staging: str = "direct",
 ) -> torch.Tensor:
     """``(q, k, v: (B, H, T, d) bf16/fp16, key_lengths: int32[B]) -> (B, H, Tq, d)``.
 
@@ -333,7 +334,9 @@ def hip_flash_attention_kernel(
     ``k_row_scale`` (B, Tk): optional positive fp32 factors of the query / key rows, shared by the heads (a
     normalisation statistic applied inside the kernel instead of in a pass of its own); ``q_col_scale`` (H * d,):
     optional fp32 factors of the query features (the product of a query and a key norm weight). ``structured_mask``:
-    a :class:`StructuredAttentionMask` (excludes ``is_causal``; combines with ``key_lengths``).
+    a :class:`StructuredAttentionMask` (excludes ``is_causal``; combines with ``key_lengths``). ``kv_staging``:
+    ``"direct"`` (K / V chunks go from global memory straight into LDS) or ``"registers"`` (the general kernel; same
+    results, kept as a comparison route).
     """
     library = _native.load_library()
     require_cuda_tensors("hip flash_attention", q, k, v, key_lengths)
@@ -386,11 +389,17 @@ def hip_flash_attention_kernel(
         batch, heads, query_len, k.shape[2], head_dim,
         _native.Int64x4(*q.stride()), _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()),
         _native.Int64x4(*out.stride()),
-        int(bool(is_causal)), int(zero_padded_queries), _native.dtype_code(q.dtype),
+        _mask_flags(is_causal, kv_staging), int(zero_padded_queries), _native.dtype_code(q.dtype),
         _native.current_stream(q.device),
     )
     _native.check(status, "flash_attention")
     return out
+
+
+def _mask_flags(is_causal: bool, kv_staging: str) -> int:
+    if kv_staging not in ("direct", "registers"):
+        raise ValueError(f"flash_attention kv_staging must be 'direct' or 'registers', got {kv_staging!r}")
+    return (_native.ATTN_CAUSAL if is_causal else 0) | (_native.ATTN_REGISTER_STAGING if kv_staging == "registers" else 0)
 
 
 def _dense_like(t: torch.Tensor) -> torch.Tensor:
@@ -406,7 +415,7 @@ class _HipFlashAttentionFunction(torch.autograd.Function):
     flash_attention.py:397-525)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, key_lengths, is_causal: bool, zero_padded_queries: bool):
+    def forward(ctx, q, k, v, key_lengths, is_causal: bool, zero_padded_queries: bool, kv_staging: str = "direct"):
         library = _native.load_library()
         q, k, v = _kernel_view(q), _kernel_view(k), _kernel_view(v)
         out = _dense_like(q)
@@ -416,13 +425,13 @@ class _HipFlashAttentionFunction(torch.autograd.Function):
             q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), out.data_ptr(), lse.data_ptr(),
             batch, heads, query_len, k.shape[2], head_dim,
             _native.Int64x4(*q.stride()), _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()),
-            _native.Int64x4(*out.stride()), int(bool(is_causal)), int(bool(zero_padded_queries)),
+            _native.Int64x4(*out.stride()), _mask_flags(is_causal, kv_staging), int(bool(zero_padded_queries)),
             _native.dtype_code(q.dtype), _native.current_stream(q.device),
         )
         _native.check(status, "flash_attention")
         ctx.save_for_backward(q, k, v, out, lse, *(() if key_lengths is None else (key_lengths,)))
         ctx.has_lengths = key_lengths is not None
-        ctx.flags = (bool(is_causal), bool(zero_padded_queries))
+        ctx.flags = (_mask_flags(is_causal, kv_staging), bool(zero_padded_queries))
         return out
 
     @staticmethod
@@ -443,7 +452,7 @@ class _HipFlashAttentionFunction(torch.autograd.Function):
             _native.dtype_code(q.dtype), _native.current_stream(q.device),
         )
         _native.check(status, "flash_attention backward")
-        return dq, dk, dv, None, None, None
+        return dq, dk, dv, None, None, None, None
 
 
 def flash_attention(
@@ -466,6 +475,7 @@ def flash_attention(
     k_row_scale: torch.Tensor | None = None,
     q_col_scale: torch.Tensor | None = None,
     structured_mask: StructuredAttentionMask | None = None,
+    kv_staging: str = "direct",
 ) -> torch.Tensor:
     """``softmax(q k^T / sqrt(d) + mask) v`` for (B, H, T, d) tensors.
 
@@ -478,7 +488,8 @@ def flash_attention(
     ``q_row_scale`` / ``k_row_scale`` / ``q_col_scale``: optional float32 factors of the query / key rows and of the
     query features, see :func:`hip_flash_attention_kernel`. ``structured_mask``: a :class:`StructuredAttentionMask`
     instead of ``attn_mask``; an ``attn_mask`` that is neither a key-prefix nor a causal-valid mask is factored into one
-    by :func:`plan_structured_attention_mask` (the reference's accelerated path rejects such masks).
+    by :func:`plan_structured_attention_mask` (the reference's accelerated path rejects such masks). ``kv_staging``:
+    see :func:`hip_flash_attention_kernel`.
     """
     del block_m, block_n, num_stages, threads
     q, k, v = _normalize_flash_attention_inputs(q, k, v)
@@ -513,13 +524,14 @@ def flash_attention(
             raise RuntimeError("hip flash_attention backward does not cover structured masks")
         if lengths is not None:
             lengths = lengths.to(torch.int32).contiguous()
-        output = _HipFlashAttentionFunction.apply(q, k, v, lengths, plan.is_causal, zero_padded_queries)
+        output = _HipFlashAttentionFunction.apply(q, k, v, lengths, plan.is_causal, zero_padded_queries, kv_staging)
         if plan.query_self_mask is not None:
             output = torch.where(plan.query_self_mask[:, None, :, None], v, output)
         return output
     output = hip_flash_attention_kernel(
         q, k, v, lengths, is_causal=plan.is_causal, zero_padded_queries=zero_padded_queries,
         q_row_scale=q_row_scale, k_row_scale=k_row_scale, q_col_scale=q_col_scale, structured_mask=structured_mask,
+        kv_staging=kv_staging,
     )
     output = _apply_query_self_mask_fallback(output, v, plan.query_self_mask)
     return output if output.dtype == output_dtype else output.to(output_dtype)

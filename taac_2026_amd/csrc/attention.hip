@@ -821,11 +821,10 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
 }
 
 template <typename T, int DP>
-void launch(const AttnParams& p, bool causal, hipStream_t s) {
+void launch(const AttnParams& p, bool causal, bool register_staging, hipStream_t s) {
   const bool scaled = p.q_row_scale != nullptr || p.k_row_scale != nullptr || p.q_col_scale != nullptr;
-  // TAAC_ATTN_STAGING=registers keeps the general kernel for the plain head-dim-32 case too (comparison knob).
-  const char* staging_env = getenv("TAAC_ATTN_STAGING");  // read per call: tests compare the two kernels in one process
-  const bool dma_staging = !(staging_env != nullptr && staging_env[0] == 'r');
+  // TAAC_ATTN_REGISTER_STAGING keeps the general kernel for full head dims too (comparison route of the caller).
+  const bool dma_staging = !register_staging;
   // 32-bit source offsets with a 24-bit row multiply: row strides below 8 M elements, sequences below 2^31 bytes
   const bool small_offsets = p.ks[2] < (1 << 22) && p.vs[2] < (1 << 22) && p.Tk < (1 << 22) &&
                              static_cast<int64_t>(p.Tk) * p.ks[2] * 2 < (1ll << 31) &&
@@ -863,13 +862,13 @@ void launch(const AttnParams& p, bool causal, hipStream_t s) {
 }
 
 template <typename T>
-void launch_dp(const AttnParams& p, bool causal, hipStream_t s) {
+void launch_dp(const AttnParams& p, bool causal, bool register_staging, hipStream_t s) {
   if (p.d <= 32)
-    launch<T, 32>(p, causal, s);
+    launch<T, 32>(p, causal, register_staging, s);
   else if (p.d <= 64)
-    launch<T, 64>(p, causal, s);
+    launch<T, 64>(p, causal, register_staging, s);
   else
-    launch<T, 128>(p, causal, s);
+    launch<T, 128>(p, causal, register_staging, s);
 }
 
 bool strides_ok(const int64_t* st) {
@@ -918,8 +917,12 @@ struct MaskArgs {
 int attention_entry(const char* name, const void* q, const void* k, const void* v, const int32_t* key_lengths,
                     const MaskArgs& mask, const float* q_row_scale, const float* k_row_scale, const float* q_col_scale,
                     float* lse, void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
-                    const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4], int is_causal,
+                    const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4], int mask_flags,
                     int zero_padded_queries, int dtype, void* stream) {
+  if (mask_flags & ~(TAAC_ATTN_CAUSAL | TAAC_ATTN_REGISTER_STAGING))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: unknown bits in is_causal (%d)", name, mask_flags);
+  const int is_causal = mask_flags & TAAC_ATTN_CAUSAL;
+  const bool register_staging = (mask_flags & TAAC_ATTN_REGISTER_STAGING) != 0;
   if (mask.struct_bits != nullptr) {
     if (mask.block_any == nullptr && mask.struct_stride == 0)
       return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_bits shared by the batch needs block_any", name);
@@ -988,9 +991,9 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
 
   hipStream_t s = as_stream(stream);
   if (dtype == TAAC_BF16)
-    launch_dp<bf16_t>(p, is_causal != 0, s);
+    launch_dp<bf16_t>(p, is_causal != 0, register_staging, s);
   else
-    launch_dp<f16_t>(p, is_causal != 0, s);
+    launch_dp<f16_t>(p, is_causal != 0, register_staging, s);
   return check_launch(name);
 }
 

@@ -544,10 +544,9 @@ bool small_offsets(int64_t rows, int64_t stride) {
 }
 
 template <typename T, int DP>
-void launch_bwd_dp(AttnBwdParams p, hipStream_t s) {
-  // TAAC_ATTN_STAGING=registers keeps the register-staged kernels for full head dims too (comparison knob).
-  const char* staging_env = getenv("TAAC_ATTN_STAGING");  // read per call: tests compare the two routes in one process
-  const bool direct = p.d == DP && !(staging_env != nullptr && staging_env[0] == 'r');
+void launch_bwd_dp(AttnBwdParams p, bool register_staging, hipStream_t s) {
+  // TAAC_ATTN_REGISTER_STAGING keeps the register-staged kernels for full head dims too (comparison route of the caller).
+  const bool direct = p.d == DP && !register_staging;
   p.nblk = static_cast<uint32_t>((p.Tq + kOwn - 1) / kOwn);
   p.total = p.nblk * p.B * p.H;
   if (direct && small_offsets(p.Tk, p.ks[2]) && small_offsets(p.Tk, p.vs[2]))
@@ -563,11 +562,11 @@ void launch_bwd_dp(AttnBwdParams p, hipStream_t s) {
 }
 
 template <typename T>
-void launch_bwd(const AttnBwdParams& p, hipStream_t s) {
+void launch_bwd(const AttnBwdParams& p, bool register_staging, hipStream_t s) {
   if (p.d <= 32)
-    launch_bwd_dp<T, 32>(p, s);
+    launch_bwd_dp<T, 32>(p, register_staging, s);
   else
-    launch_bwd_dp<T, 64>(p, s);
+    launch_bwd_dp<T, 64>(p, register_staging, s);
 }
 
 }  // namespace
@@ -584,6 +583,9 @@ extern "C" int taac_flash_attn_bwd(const void* q, const void* k, const void* v, 
   const char* name = "taac_flash_attn_bwd";
   if (B < 0 || H < 0 || Tq < 0 || Tk < 0 || d <= 0)
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: negative dimension or non-positive head_dim", name);
+  if (is_causal & ~(TAAC_ATTN_CAUSAL | TAAC_ATTN_REGISTER_STAGING))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: unknown bits in is_causal (%d)", name, is_causal);
+  const bool register_staging = (is_causal & TAAC_ATTN_REGISTER_STAGING) != 0;
   if (dtype != TAAC_BF16 && dtype != TAAC_F16)
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: dtype must be bf16 or fp16 (got %d)", name, dtype);
   if (d % 8 != 0 || d > 64)
@@ -634,11 +636,11 @@ extern "C" int taac_flash_attn_bwd(const void* q, const void* k, const void* v, 
   }
   p.scale = 1.0f / sqrtf(static_cast<float>(d));
   p.zero_pad = zero_padded_queries ? 1 : 0;
-  p.causal = is_causal ? 1 : 0;
+  p.causal = (is_causal & TAAC_ATTN_CAUSAL) ? 1 : 0;
   hipStream_t s = as_stream(stream);
   if (dtype == TAAC_BF16)
-    launch_bwd<bf16_t>(p, s);
+    launch_bwd<bf16_t>(p, register_staging, s);
   else
-    launch_bwd<f16_t>(p, s);
+    launch_bwd<f16_t>(p, register_staging, s);
   return check_launch(name);
 }

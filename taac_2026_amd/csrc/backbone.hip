@@ -309,9 +309,12 @@ extern "C" int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D
 extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, const taac_block_weights* blocks,
                                  int32_t n_blocks, const void* w_head, const void* b_head, int32_t B, int32_t T,
                                  int32_t D, int32_t heads, int32_t F, float eps, const void* rope_cos_sin,
-                                 void* workspace, int64_t workspace_bytes, void* hidden_out, float* p, void* stream) {
+                                 int flags, void* workspace, int64_t workspace_bytes, void* hidden_out, float* p,
+                                 void* stream) {
   using namespace taac;
   const char* name = "taac_backbone_fwd";
+  if (flags & ~(TAAC_BACKBONE_DENSE_TOKENS | TAAC_BACKBONE_SPLIT_OUT_FFN))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: unknown flag bits (%d)", name, flags);
   if (B < 0 || T < 0 || D <= 0 || F <= 0 || heads <= 0 || n_blocks < 0)
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: bad dimensions", name);
   if (D % heads != 0 || (D / heads) % 8 != 0 || D / heads > 128)
@@ -338,7 +341,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
   char* packed = ws;
   const bool fused = fused_shape(D, F);
   // Fused path: the dense layers walk the valid tokens only (row index built from key_lengths on the device); the
-  // padded positions of the residual stream are never read or written. TAAC_DENSE_TOKENS switches this off.
+  // padded positions of the residual stream are never read or written. TAAC_BACKBONE_DENSE_TOKENS switches this off.
   int32_t* rows = nullptr;
   int32_t* n_rows = nullptr;
   char* after_packed = packed + static_cast<int64_t>(n_blocks) * packed_block_bytes(D, F);
@@ -347,7 +350,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
   bf16_t* qk_weight = reinterpret_cast<bf16_t*>(reinterpret_cast<char*>(qk_rstd) + align256(2 * M * 4));
   if (rope_cos_sin != nullptr && !aligned16(rope_cos_sin))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: the rotary table must be 16-byte aligned", name);
-  if (fused && n_blocks > 0 && getenv("TAAC_DENSE_TOKENS") == nullptr) {
+  if (fused && n_blocks > 0 && !(flags & TAAC_BACKBONE_DENSE_TOKENS)) {
     rows = reinterpret_cast<int32_t*>(after_packed);
     n_rows = rows + M + B + 1;
     const int rc_rows = taac_valid_rows(key_lengths, B, T, rows, n_rows, stream);
@@ -360,8 +363,8 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
 
   const bf16_t* cur = static_cast<const bf16_t*>(emb);
   int rc;
-  // TAAC_SPLIT_OUT_FFN: run the out projection and the feed-forward half as two kernels (tuning / comparison knob).
-  const bool split_out_ffn = getenv("TAAC_SPLIT_OUT_FFN") != nullptr;
+  // TAAC_BACKBONE_SPLIT_OUT_FFN: the out projection and the feed-forward half as two kernels (comparison route).
+  const bool split_out_ffn = (flags & TAAC_BACKBONE_SPLIT_OUT_FFN) != 0;
   if (fused && n_blocks > 0) {
     // One launch re-lays the weights of all blocks into fragment order.
     std::vector<void*> pk(3 * static_cast<size_t>(n_blocks));

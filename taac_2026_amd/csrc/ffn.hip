@@ -1054,17 +1054,6 @@ int launch_ts(K kernel, const TsParams& p, int threads, int tokens_per_wg, size_
   return check_launch(name);
 }
 
-// Schedule of the fused FFN kernel (tuning knob, read once from TAAC_TS_CONFIG; default 1):
-//   0 = down projection of a chunk right after its activation, two weight buffers
-//   1 = down projection deferred by one chunk and interleaved with the next activation, three weight buffers
-int ts_config() {
-  static const int config = [] {
-    const char* env = getenv("TAAC_TS_CONFIG");
-    return (env != nullptr && env[0] >= '0' && env[0] <= '1') ? env[0] - '0' : 1;
-  }();
-  return config;
-}
-
 bool ptr_ok(const void* p, uintptr_t mask) { return (reinterpret_cast<uintptr_t>(p) & mask) == 0; }
 
 constexpr int kMaxLdsBytes = 160 * 1024;
@@ -1214,9 +1203,10 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
     if (D == 256) TAAC_FFN_LAUNCH(256, 1, 8, 2, true, true);
     TAAC_FFN_LAUNCH(128, 1, 8, 2, true, true);
   }
-  int cfg = ts_config();
-  // the deferred schedule needs a third weight buffer: fall back when a large F leaves no room for it next to the biases
-  if (cfg >= 1 && 3 * buffer_bytes + bias_bytes > kMaxLdsBytes) cfg = 0;
+  // Schedule: the down projection of a chunk is deferred by one chunk and interleaved with the next activation (three
+  // weight buffers); when a large F leaves no room for the third buffer next to the biases it follows its activation
+  // directly (two buffers).
+  const int cfg = 3 * buffer_bytes + bias_bytes > kMaxLdsBytes ? 0 : 1;
   if (D == 256) {
     if (cfg == 1) TAAC_FFN_LAUNCH(256, 1, 8, 2, true, false);
     TAAC_FFN_LAUNCH(256, 1, 8, 2, false, false);

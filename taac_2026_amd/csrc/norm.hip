@@ -442,6 +442,83 @@ __global__ __launch_bounds__(kBlock) void norm_bwd_reduce_kernel(const float* __
   }
 }
 
+// Sum over the workgroup of up to three values at once (wavefront shuffles, then one LDS round over the wavefronts);
+// every thread gets the totals. `red` is reused by consecutive calls: the leading barrier protects the previous round.
+template <int N>
+__device__ __forceinline__ void block_sum(float (&v)[N], float (*red)[kBlock / kWave]) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+#pragma unroll
+  for (int i = 0; i < N; ++i) v[i] = group_sum<kWave>(v[i]);
+  __syncthreads();
+  if (lane == 0) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) red[i][wave] = v[i];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < kBlock / kWave; ++w) total += red[i][w];
+    v[i] = total;
+  }
+}
+
+// Backward for shapes the vector kernel does not take (columns that are not whole 128-bit vectors, unaligned bases,
+// rows longer than its register budget): one workgroup per row at a time, thread t owns columns t, t + 256, ...; the
+// row is swept four times (mean, variance, the two projections, the result), sweeps after the first come from cache.
+// The workgroup's partial row of dw / db lives in the workspace and is updated in place by the thread that owns the
+// column, in row order, so the result is reproducible as in the vector kernel.
+template <typename T, bool LN>
+__global__ __launch_bounds__(kBlock) void norm_bwd_rows_generic_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                        const T* __restrict__ dy, T* __restrict__ dx,
+                                                                        float* __restrict__ partial, int64_t rows,
+                                                                        int cols, float eps) {
+  __shared__ float red[2][kBlock / kWave];
+  const int tid = threadIdx.x;
+  const float inv_cols = 1.0f / static_cast<float>(cols);
+  float* out_w = partial + static_cast<int64_t>(blockIdx.x) * cols * (LN ? 2 : 1);
+  for (int c = tid; c < cols; c += kBlock) {
+    out_w[c] = 0.f;
+    if (LN) out_w[cols + c] = 0.f;
+  }
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const T* xr = x + row * cols;
+    const T* gr = dy + row * cols;
+    T* dr = dx + row * cols;
+    float mean = 0.f;
+    if (LN) {
+      float s[1] = {0.f};
+      for (int c = tid; c < cols; c += kBlock) s[0] += static_cast<float>(xr[c]);
+      block_sum<1>(s, red);
+      mean = s[0] * inv_cols;
+    }
+    float ss[1] = {0.f};
+    for (int c = tid; c < cols; c += kBlock) {
+      const float d = static_cast<float>(xr[c]) - mean;
+      ss[0] += d * d;
+    }
+    block_sum<1>(ss, red);
+    const float rstd = rsqrtf(ss[0] * inv_cols + eps);
+    float proj[2] = {0.f, 0.f};  // sum of g, sum of g * x_hat
+    for (int c = tid; c < cols; c += kBlock) {
+      const float g = static_cast<float>(gr[c]) * static_cast<float>(w[c]);
+      proj[0] += g;
+      proj[1] += g * ((static_cast<float>(xr[c]) - mean) * rstd);
+    }
+    block_sum<2>(proj, red);
+    const float mean_g = LN ? proj[0] * inv_cols : 0.f;
+    const float mean_gx = proj[1] * inv_cols;
+    for (int c = tid; c < cols; c += kBlock) {
+      const float gy = static_cast<float>(gr[c]);
+      const float xh = (static_cast<float>(xr[c]) - mean) * rstd;
+      dr[c] = static_cast<T>(rstd * (gy * static_cast<float>(w[c]) - mean_g - xh * mean_gx));
+      out_w[c] += gy * xh;
+      if (LN) out_w[cols + c] += gy;
+    }
+  }
+}
+
 constexpr int kBwdMaxBlocks = 1024;
 
 template <typename T, bool LN>
@@ -452,10 +529,19 @@ int dispatch_bwd(const void* xv, const void* wv, const void* dyv, void* dxv, voi
   const T* dy = static_cast<const T*>(dyv);
   T* dx = static_cast<T*>(dxv);
   constexpr int VEC = Pack<T>::VEC;
-  if (cols % VEC != 0 || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(w) || cols / VEC > kWave * 4)
-    return set_error(TAAC_ERR_UNSUPPORTED,
-                     "%s: cols must be a multiple of %d and at most %d, tensors 16-byte aligned", name, VEC,
-                     kWave * 4 * VEC);
+  const int parts = LN ? 2 : 1;
+  if (cols % VEC != 0 || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(w) || cols / VEC > kWave * 4) {
+    // generic route: one workgroup per row at a time
+    const int64_t nb = rows < kBwdMaxBlocks ? rows : kBwdMaxBlocks;
+    if (workspace == nullptr || workspace_floats < nb * parts * cols)
+      return set_error(TAAC_ERR_INVALID_VALUE, "%s: workspace must hold %lld floats", name, (long long)(nb * parts * cols));
+    if (rows > 0)
+      hipLaunchKernelGGL((norm_bwd_rows_generic_kernel<T, LN>), dim3(static_cast<uint32_t>(nb)), dim3(kBlock), 0, s, x, w,
+                         dy, dx, workspace, rows, cols, eps);
+    hipLaunchKernelGGL((norm_bwd_reduce_kernel<T>), dim3((cols + 15) / 16), dim3(kBlock), 0, s, workspace,
+                       static_cast<int>(nb), cols, parts, static_cast<T*>(dwv), static_cast<T*>(dbv));
+    return TAAC_OK;
+  }
   const int nvec = cols / VEC;
   int G = 1;
   while (G < nvec && G < kWave) G *= 2;
@@ -463,7 +549,6 @@ int dispatch_bwd(const void* xv, const void* wv, const void* dyv, void* dxv, voi
   const int gpb = (kBlock / G) * rows_in_flight;
   int64_t nblocks = (rows + gpb - 1) / gpb;
   if (nblocks > kBwdMaxBlocks) nblocks = kBwdMaxBlocks;
-  const int parts = LN ? 2 : 1;
   if (workspace == nullptr || workspace_floats < nblocks * parts * cols)
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: workspace must hold %lld floats", name,
                      (long long)(nblocks * parts * cols));

@@ -13,7 +13,6 @@ sigmoid) executed by a single ``taac_backbone_fwd`` call.
 from __future__ import annotations
 
 import ctypes
-import os
 
 import torch
 import torch.nn as nn
@@ -147,10 +146,16 @@ class UnifiedInteractionBlock(nn.Module):
     kernel, and with ``return_attention_tokens=False`` the out projection, both residual adds, ``ffn_norm`` and the
     feed-forward are one kernel. ``attention_mask`` may be a dense bool mask, a :class:`StructuredAttentionMask`
     (what ``MetadataAttentionMask`` returns) or None; ``key_lengths`` states prefix padding without a mask.
-    ``inplace=True`` lets the fused route update ``tokens`` itself instead of a copy."""
+    ``inplace=True`` lets the fused route update ``tokens`` itself instead of a copy. ``token_layout``: ``"front"``
+    (default) lets the fused route move every sample's valid tokens to the front of its rows for the attention call
+    when the mask allows it, ``"positions"`` keeps them where they are (comparison route; same results)."""
 
-    def __init__(self, d_model: int, num_heads: int, hidden_mult: int, dropout: float = 0.0, *, qk_norm: bool = True) -> None:
+    def __init__(self, d_model: int, num_heads: int, hidden_mult: int, dropout: float = 0.0, *, qk_norm: bool = True,
+                 token_layout: str = "front") -> None:
         super().__init__()
+        if token_layout not in ("front", "positions"):
+            raise ValueError("token_layout must be 'front' or 'positions'")
+        self.token_layout = token_layout
         self.attn_norm = RMSNorm(d_model)
         self.attention = UnifiedSelfAttention(d_model, num_heads, dropout, qk_norm=qk_norm)
         self.ffn_norm = RMSNorm(d_model)
@@ -174,15 +179,15 @@ class UnifiedInteractionBlock(nn.Module):
         # Padding scattered inside the samples, under a structured mask whose valid keys are exactly the non-padded
         # positions: the projection writes every sample's valid tokens at the front of its rows, so that the attention
         # call sees prefix padding (its cost follows the valid tokens, not the positions) with the mask's structure
-        # gathered per sample, and the out projection reads that layout back. TAAC_BLOCK_LAYOUT=positions keeps the
-        # tokens where they are (comparison knob).
+        # gathered per sample, and the out projection reads that layout back. token_layout="positions" keeps the
+        # tokens where they are (comparison route).
         # The indices and the gathered mask depend on the mask object only: the blocks of a stack, which all receive it,
         # share them through its cache.
         front = lengths = None
         if (structured is not None and key_lengths is None and structured.padding_source is padding_mask
                 and structured.query_self is None and not structured.sample_stride
                 and structured.structural.shape == (token_count, token_count)
-                and os.environ.get("TAAC_BLOCK_LAYOUT", "front") != "positions"):
+                and self.token_layout != "positions"):
             entry = structured.cache.get("front")
             if entry is None or entry[0] != padding_mask._version:  # rebuilt when the padding mask was written to
                 index = valid_rows(None, token_count, padding_mask=padding_mask)
@@ -200,7 +205,17 @@ class UnifiedInteractionBlock(nn.Module):
             index = entry[1]
         else:
             index = valid_rows(None, token_count, padding_mask=padding_mask)
-        qkv_rows = dict(token_rows=index) if front is None else dict(token_rows=(front, index[1]), input_rows=index[0])
+        # The projection may skip the padded tokens only when the mask proves that no query can see a padded key: a key
+        # length handed to the attention call, or a structured mask whose key validity was derived from this padding
+        # mask. Otherwise (no mask, a dense mask, a structured mask of unknown origin) the padded tokens are projected
+        # like every other token, as the reference block does (experiments/symbiosis/backbone.py:58-63), and only the
+        # residual updates skip them.
+        padded_keys_hidden = (front is not None or (key_lengths is not None and attention_mask is None)
+                              or (structured is not None and structured.padding_source is padding_mask))
+        if front is not None:
+            qkv_rows = dict(token_rows=(front, index[1]), input_rows=index[0])
+        else:
+            qkv_rows = dict(token_rows=index) if padded_keys_hidden else {}
         qkv = torch.empty(batch * token_count, 3 * d_model, dtype=x.dtype, device=x.device)
         q_row_scale = k_row_scale = q_col_scale = None
         if attention.query_norm is not None or attention.rope_base is not None:
@@ -292,7 +307,9 @@ class PCVRBackbone(nn.Module):
 
     Initialisation: Xavier-uniform weights, zero biases, unit norm weights.
     ``forward(emb[B, T, D] bf16, key_lengths[B] int32) -> p[B] float32``; ``return_hidden=True`` also returns the
-    final hidden state (rows at or beyond ``key_lengths[b]`` are unspecified).
+    final hidden state (rows at or beyond ``key_lengths[b]`` are zeros). ``dense_tokens=True`` runs the dense layers over
+    the padded positions too (what the reference's dense ``[B, T, D]`` formulation does; same valid rows, bit for bit),
+    ``split_out_ffn=True`` runs the out projection and the feed-forward half as two kernels (comparison routes).
     ``qk_norm=True`` adds the reference layer's ``RMSNorm(d_model)`` of the query and the key
     (experiments/symbiosis/backbone.py:30-36), ``rope_base`` TokenFormer's rotary embedding of both over the token
     positions (experiments/tokenformer/model.py:165-192); the benchmark recipe has neither.
@@ -323,7 +340,8 @@ class PCVRBackbone(nn.Module):
             self._workspace = ws
         return ws
 
-    def forward(self, emb: torch.Tensor, key_lengths: torch.Tensor, *, return_hidden: bool = False):
+    def forward(self, emb: torch.Tensor, key_lengths: torch.Tensor, *, return_hidden: bool = False,
+                dense_tokens: bool = False, split_out_ffn: bool = False):
         name = "hip PCVRBackbone"
         require_cuda_tensors(name, emb, key_lengths)
         require_inference(name, emb)
@@ -366,11 +384,13 @@ class PCVRBackbone(nn.Module):
         nbytes = library.taac_backbone_workspace_bytes(batch, tokens, self.d_model, self.d_ff, len(self.blocks))
         workspace = self._get_workspace(int(nbytes), emb.device)
         hidden = torch.empty_like(emb) if return_hidden else None
+        flags = (_native.BACKBONE_DENSE_TOKENS if dense_tokens else 0) | (_native.BACKBONE_SPLIT_OUT_FFN if split_out_ffn else 0)
         probabilities = torch.empty(batch, dtype=torch.float32, device=emb.device)
         status = library.taac_backbone_fwd(
             emb.data_ptr(), key_lengths.data_ptr(), packed, len(self.blocks), dev(self.head.weight.reshape(-1)),
             dev(self.head.bias), batch, tokens, self.d_model, self.num_heads, self.d_ff, ctypes.c_float(self.eps),
-            _native.ptr(table), workspace.data_ptr(), workspace.numel(), _native.ptr(hidden), probabilities.data_ptr(),
+            _native.ptr(table), flags, workspace.data_ptr(), workspace.numel(), _native.ptr(hidden),
+            probabilities.data_ptr(),
             _native.current_stream(emb.device),
         )
         _native.check(status, "backbone_fwd")

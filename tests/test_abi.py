@@ -68,10 +68,16 @@ def test_host_side_argument_validation_without_gpu():
     assert library.taac_ffn_packed_bytes(256, 1024) == 3 * 256 * 1024 * 2 and library.taac_ffn_packed_bytes(96, 64) == -1
     assert library.taac_linear_packed_bytes(768, 256) == 768 * 256 * 2 and library.taac_linear_packed_bytes(72, 256) == -1
     weights = (_native.BlockWeights * 1)()
-    status = library.taac_backbone_fwd(fake, fake, weights, 1, fake, None, 2, 16, 32, 4, 64, 1e-6, None, fake, 16, None, fake, None)
+    status = library.taac_backbone_fwd(fake, fake, weights, 1, fake, None, 2, 16, 32, 4, 64, 1e-6, None, 0, fake, 16, None, fake, None)
     assert status == _native.TAAC_ERR_INVALID_VALUE and b"workspace" in library.taac_last_error()
-    status = library.taac_backbone_fwd(fake, fake, weights, 1, fake, None, 2, 16, 32, 5, 64, 1e-6, None, fake, 1 << 20, None, fake, None)
+    status = library.taac_backbone_fwd(fake, fake, weights, 1, fake, None, 2, 16, 32, 5, 64, 1e-6, None, 0, fake, 1 << 20, None, fake, None)
     assert status == _native.TAAC_ERR_UNSUPPORTED
+    # unknown flag bits of the backbone and of the attention mask argument are rejected, not ignored
+    status = library.taac_backbone_fwd(fake, fake, weights, 1, fake, None, 2, 16, 32, 4, 64, 1e-6, None, 64, fake, 1 << 20, None, fake, None)
+    assert status == _native.TAAC_ERR_INVALID_VALUE and b"flag" in library.taac_last_error()
+    status = library.taac_flash_attn_fwd(fake, fake, fake, None, fake, 1, 1, 4, 4, 16, strides, strides, strides, strides,
+                                         4, 0, _native.TAAC_BF16, None)
+    assert status == _native.TAAC_ERR_INVALID_VALUE and b"is_causal" in library.taac_last_error()
 
 
 def test_host_side_validation_of_the_widened_entry_points_without_gpu():
@@ -114,7 +120,9 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
     assert floats > 0 and library.taac_norm_bwd_workspace_floats(1000, 256, 1) == 2 * floats
     assert library.taac_rmsnorm_bwd(fake, fake, fake, fake, fake, fake, 255, 1000, 256, 1e-6, bf16, None) == invalid
     assert b"workspace" in library.taac_last_error()
-    assert library.taac_rmsnorm_bwd(fake, fake, fake, fake, fake, fake, 1 << 30, 8, 260, 1e-6, bf16, None) == unsupported
+    # a width that is not a whole number of 16-byte vectors takes the generic kernel, which needs its workspace too
+    assert library.taac_rmsnorm_bwd(fake, fake, fake, fake, fake, fake, 8 * 260 - 1, 8, 260, 1e-6, bf16, None) == invalid
+    assert b"workspace" in library.taac_last_error()
     assert library.taac_layernorm_bwd(fake, fake, fake, None, fake, fake, fake, 1 << 30, 8, 256, 1e-5, bf16, None) == invalid
 
     # out projection + feed-forward half in one kernel: both weight sets packed, the block input required

@@ -213,9 +213,9 @@ def test_row_factors_of_queries_and_keys(device, dim, tokens, causal):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("head_dim", [32, 64])
 @pytest.mark.parametrize("causal", [False, True])
-def test_direct_transfer_kernel_equals_general_kernel_bit_for_bit(device, monkeypatch, dtype, head_dim, causal):
+def test_direct_transfer_kernel_equals_general_kernel_bit_for_bit(device, dtype, head_dim, causal):
     """Head dims 32 and 64 run a kernel that stages K and V by direct global->LDS transfers (swizzled rows, transposed
-    LDS reads); TAAC_ATTN_STAGING=registers selects the general kernel. Same arithmetic in the same order: identical
+    LDS reads); kv_staging="registers" selects the general kernel. Same arithmetic in the same order: identical
     results, for ragged lengths (0, 1, not a multiple of the chunk), strided views of a packed projection, row factors
     and the log-sum-exp output of the training forward."""
     from taac_2026_amd.api import flash_attention
@@ -230,16 +230,17 @@ def test_direct_transfer_kernel_equals_general_kernel_bit_for_bit(device, monkey
     k_rows = (0.5 + torch.rand(batch, tokens, generator=g)).to(device)
     q_cols = (0.5 + torch.rand(heads * head_dim, generator=g)).to(device)
 
-    def run():
+    def run(staging):
         with torch.no_grad():
-            plain = flash_attention(q, k, v, key_lengths=lengths, is_causal=causal, zero_padded_queries=True)
-            full = flash_attention(q, k, v, is_causal=causal)
+            plain = flash_attention(q, k, v, key_lengths=lengths, is_causal=causal, zero_padded_queries=True,
+                                    kv_staging=staging)
+            full = flash_attention(q, k, v, is_causal=causal, kv_staging=staging)
             scaled = hip_flash_attention_kernel(q, k, v, lengths, is_causal=causal, zero_padded_queries=True,
-                                                q_row_scale=q_rows, k_row_scale=k_rows, q_col_scale=q_cols)
+                                                q_row_scale=q_rows, k_row_scale=k_rows, q_col_scale=q_cols,
+                                                kv_staging=staging)
         return plain, full, scaled
 
-    direct = run()
-    monkeypatch.setenv("TAAC_ATTN_STAGING", "registers")
-    general = run()
+    direct = run("direct")
+    general = run("registers")
     for a, b in zip(direct, general):
         assert torch.equal(a, b)

@@ -74,20 +74,20 @@ def test_backward_is_reproducible_and_reads_the_projection_layout(device):
 
 
 @pytest.mark.parametrize("dim,causal", [(32, False), (64, False), (64, True)])
-def test_direct_transfer_backward_equals_register_staged_backward(device, monkeypatch, dim, causal):
+def test_direct_transfer_backward_equals_register_staged_backward(device, dim, causal):
     """Full head dims stream their chunks from global memory straight into LDS, where rows beyond the valid length repeat
     the last valid row instead of zeros; their products are cancelled by zero probabilities, so both routes give the
-    same bits (the staging knob is read per call)."""
+    same bits (``kv_staging`` selects the route of the training forward and of its backward; the forwards are
+    bit-identical, see test_gpu_attention.py)."""
     batch, heads, tokens = 5, 2, 333
     g = torch.Generator().manual_seed(dim + causal)
     q, k, v, grad_out = (torch.randn(batch, heads, tokens, dim, generator=g).to(torch.bfloat16).to(device) for _ in range(4))
     lengths = torch.tensor([333, 1, 64, 65, 200], dtype=torch.int32, device=device)
     grads = {}
     for staging in ("direct", "registers"):
-        monkeypatch.setenv("TAAC_ATTN_STAGING", "direct")  # the same training forward (output, log-sum-exp) for both
         qd, kd, vd = (t.clone().requires_grad_(True) for t in (q, k, v))
-        out = flash_attention(qd, kd, vd, key_lengths=lengths, is_causal=causal, zero_padded_queries=not causal)
-        monkeypatch.setenv("TAAC_ATTN_STAGING", staging)
+        out = flash_attention(qd, kd, vd, key_lengths=lengths, is_causal=causal, zero_padded_queries=not causal,
+                              kv_staging=staging)
         out.backward(grad_out)
         grads[staging] = (qd.grad, kd.grad, vd.grad)
     for direct, staged in zip(grads["direct"], grads["registers"]):

@@ -14,13 +14,13 @@ from taac_2026_amd.api import PCVRBackbone, UnifiedInteractionBlock
 pytestmark = pytest.mark.gpu
 
 
-def _run(inputs, device, return_hidden=True, rope_base=None):
+def _run(inputs, device, return_hidden=True, rope_base=None, **routes):
     model = PCVRBackbone(d_model=inputs.emb.shape[-1], num_heads=inputs.num_heads, d_ff=inputs.d_ff,
                          n_blocks=len(inputs.blocks), qk_norm="query_norm.weight" in inputs.blocks[0], rope_base=rope_base)
     workloads.load_backbone_state(model, inputs)
     model = model.to(device=device, dtype=torch.bfloat16).eval()
     with torch.no_grad():
-        return model(inputs.emb.to(device), inputs.key_lengths.to(device), return_hidden=return_hidden)
+        return model(inputs.emb.to(device), inputs.key_lengths.to(device), return_hidden=return_hidden, **routes)
 
 
 @pytest.mark.parametrize("batch,n_feature,n_sequence", [(6, 32, 96), (3, 32, 480), (5, 8, 57)])
@@ -59,7 +59,7 @@ def test_backbone_matches_oracle(device, batch, n_feature, n_sequence):
 
 @pytest.mark.parametrize("qk_norm,rope_base", [(True, None), (True, 10000.0), (False, 10000.0)])
 @pytest.mark.parametrize("d_model,heads,d_ff", [(256, 8, 512), (128, 4, 256), (64, 2, 96)])
-def test_backbone_with_normalised_and_rotated_queries_and_keys(device, monkeypatch, qk_norm, rope_base, d_model, heads, d_ff):
+def test_backbone_with_normalised_and_rotated_queries_and_keys(device, qk_norm, rope_base, d_model, heads, d_ff):
     """The block as the reference's layers run it: RMSNorm(d_model) of the query and the key
     (experiments/symbiosis/backbone.py:33-36) and TokenFormer's rotary embedding (experiments/tokenformer/model.py:
     153-154). Widths 128 / 256 take the path without a pass over q and k (projection epilogue + attention row
@@ -79,9 +79,7 @@ def test_backbone_with_normalised_and_rotated_queries_and_keys(device, monkeypat
     exact_p, exact_h = oracle.backbone(inputs.emb.float(), inputs.key_lengths, blocks32, inputs.head_weight.float(),
                                        inputs.head_bias.float(), num_heads=heads, return_hidden=True, rope_base=rope_base)
     valid = torch.arange(inputs.emb.shape[1])[None, :] < inputs.key_lengths[:, None]
-    results = [_run(inputs, device, rope_base=rope_base)]
-    monkeypatch.setenv("TAAC_DENSE_TOKENS", "1")
-    results.append(_run(inputs, device, rope_base=rope_base))
+    results = [_run(inputs, device, rope_base=rope_base), _run(inputs, device, rope_base=rope_base, dense_tokens=True)]
     for p, hidden in results:
         torch.testing.assert_close(p.cpu(), expected_p, rtol=0, atol=2e-2)
         torch.testing.assert_close(p.cpu(), exact_p, rtol=0, atol=2e-2)
@@ -98,10 +96,11 @@ def test_backbone_with_normalised_and_rotated_queries_and_keys(device, monkeypat
     assert (plain_h.float()[valid] - expected_h.float()[valid]).abs().max().item() > 5e-2
 
 
-def test_backbone_skips_padded_positions(device, monkeypatch):
+def test_backbone_skips_padded_positions(device):
     """The fused forward walks the valid tokens only: garbage (NaN) at the padded positions of the embeddings changes
     nothing, the valid rows of the hidden state are bit-identical to the run over all B*T positions
-    (TAAC_DENSE_TOKENS), and the padded rows of the returned hidden state are zeros."""
+    (``dense_tokens=True``) and to the route with the out projection and the feed-forward half as two kernels, and the
+    padded rows of the returned hidden state are zeros."""
     inputs = workloads.backbone_inputs(batch=7, n_feature_tokens=32, n_sequence_tokens=224, min_sequence_len=16, seed=3)
     tokens = inputs.emb.shape[1]
     valid = torch.arange(tokens)[None, :] < inputs.key_lengths[:, None]
@@ -112,10 +111,14 @@ def test_backbone_skips_padded_positions(device, monkeypatch):
     p_poisoned, h_poisoned = _run(poisoned, device)
     assert torch.equal(p_poisoned, p_ref) and torch.equal(h_poisoned, h_ref)
     assert (h_ref.cpu()[~valid] == 0).all()
-    monkeypatch.setenv("TAAC_DENSE_TOKENS", "1")
-    p_dense, h_dense = _run(inputs, device)
+    p_dense, h_dense = _run(inputs, device, dense_tokens=True)
     assert torch.equal(p_dense, p_ref)
     assert torch.equal(h_dense.cpu()[valid], h_ref.cpu()[valid])
+    # two kernels round the feed-forward update before the residual add, one kernel rounds their sum once
+    p_split, h_split = _run(inputs, device, split_out_ffn=True)
+    torch.testing.assert_close(p_split, p_ref, rtol=0, atol=2e-3)
+    # (differences of one bf16 step per block, carried through four blocks)
+    torch.testing.assert_close(h_split.cpu().float()[valid], h_ref.cpu().float()[valid], rtol=2 ** -5, atol=2 ** -4)
 
 
 def test_backbone_config4_full_size(device):
@@ -187,12 +190,11 @@ def _symbiosis_block_case(d_model, heads, tokens, batch, seed):
 
 
 @pytest.mark.parametrize("d_model,heads,tokens,batch", [(128, 4, 70, 5), (256, 8, 150, 4)])
-def test_interaction_block_fused_routes_under_role_masks_and_scattered_padding(device, monkeypatch, d_model, heads, tokens,
-                                                                               batch):
+def test_interaction_block_fused_routes_under_role_masks_and_scattered_padding(device, d_model, heads, tokens, batch):
     """The reference block as the model runs it: role-based attention mask, padding anywhere in the sequence, updates
     masked at padded rows. Both fused routes against the oracle's statement of the block; padded rows pass through bit
     for bit and are never read (NaN there changes nothing). With the model's own mask object the attention runs over
-    every sample's valid tokens moved to the front; a dense mask (or TAAC_BLOCK_LAYOUT=positions) keeps the positions."""
+    every sample's valid tokens moved to the front; a dense mask (or token_layout="positions") keeps the positions."""
     block, x, padding, roles, state, mask_module = _symbiosis_block_case(d_model, heads, tokens, batch, seed=d_model + tokens)
     dense_mask = oracle.metadata_attention_mask(padding, roles)
     want, want_attn = oracle.interaction_block(x.float(), padding, dense_mask, {k: v.float() for k, v in state.items()},
@@ -204,9 +206,9 @@ def test_interaction_block_fused_routes_under_role_masks_and_scattered_padding(d
         two, two_attn = block(x.to(device), padding.to(device), mask)
         one, none = block(x.to(device), padding.to(device), mask, return_attention_tokens=False)
         from_dense, _ = block(x.to(device), padding.to(device), dense_mask.to(device))
-        monkeypatch.setenv("TAAC_BLOCK_LAYOUT", "positions")
+        block.token_layout = "positions"
         by_position, by_position_attn = block(x.to(device), padding.to(device), mask)
-        monkeypatch.delenv("TAAC_BLOCK_LAYOUT")
+        block.token_layout = "front"
         poisoned = x.clone()
         poisoned[padding] = float("nan")
         stream = poisoned.to(device)
@@ -223,6 +225,57 @@ def test_interaction_block_fused_routes_under_role_masks_and_scattered_padding(d
         assert torch.equal(result.cpu()[padding], x[padding])          # x + update * 0
     assert torch.equal(in_place.cpu()[valid], one.cpu()[valid])
     assert torch.isnan(in_place.cpu()[padding].float()).all()
+
+
+def test_interaction_block_projects_padded_tokens_when_the_mask_does_not_hide_them(device):
+    """Without a mask (or under a dense mask that does not exclude the padded keys) the reference block attends to the
+    projections of the padded tokens as well (experiments/symbiosis/backbone.py:58-63): the fused route must then
+    project every row instead of reading rows it never wrote. Checked against the oracle's statement of the block, with
+    the allocator's memory poisoned beforehand so that an unwritten row cannot pass by luck."""
+    block, x, padding, roles, state, _ = _symbiosis_block_case(128, 4, 70, 5, seed=33)
+    state32 = {k: v.float() for k, v in state.items()}
+    batch, tokens, _ = x.shape
+    structure = torch.rand(tokens, tokens, generator=torch.Generator().manual_seed(1)) < 0.6
+    structure |= torch.eye(tokens, dtype=torch.bool)           # every query sees itself: no empty rows
+    structure = structure[None, None].expand(batch, 1, tokens, tokens)   # shared by the batch, padded keys visible
+    valid = ~padding
+    block = block.to(device)
+    for mask in (None, structure):
+        want, want_attn = oracle.interaction_block(x.float(), padding, mask, state32, num_heads=4)
+        # fill the caching allocator's free blocks of the size the projection will ask for with NaN
+        poison = torch.full((batch * tokens, 3 * 128), float("nan"), dtype=torch.bfloat16, device=device)
+        del poison
+        with torch.no_grad():
+            got, got_attn = block(x.to(device), padding.to(device), None if mask is None else mask.to(device))
+            one, _ = block(x.to(device), padding.to(device), None if mask is None else mask.to(device),
+                           return_attention_tokens=False)
+        assert torch.isfinite(got.float()).all()
+        torch.testing.assert_close(got_attn.cpu().float()[valid], want_attn[valid], rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(got.cpu().float()[valid], want[valid], rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(one.cpu().float()[valid], want[valid], rtol=2e-2, atol=2e-2)
+        assert torch.equal(got.cpu()[padding], x[padding])
+    # the padded tokens matter in these cases: hiding them changes the result
+    hidden_keys, _ = oracle.interaction_block(x.float(), padding, valid[:, None, None, :].expand(batch, 1, tokens, tokens),
+                                              state32, num_heads=4)
+    no_mask, _ = oracle.interaction_block(x.float(), padding, None, state32, num_heads=4)
+    assert (hidden_keys[valid] - no_mask[valid]).abs().max().item() > 5e-2
+
+
+def test_one_block_at_the_headline_widths_holds_elementwise_tolerance(device):
+    """A single block at the headline widths (d_model 256, 8 heads, d_ff 1024, 512 tokens, key-length route through the
+    backbone entry point): every valid element of the hidden state within rtol = atol = 2e-2 of the fp32 evaluation of
+    the reference's formulas. (The looser statistical bound of the 4-block tests is accumulation over 28 rounding
+    points, not a property of a block.)"""
+    inputs = workloads.backbone_inputs(batch=6, n_blocks=1, seed=11)
+    assert inputs.emb.shape[1:] == (512, 256) and inputs.d_ff == 1024 and inputs.num_heads == 8
+    blocks32 = [{k: v.float() for k, v in w.items()} for w in inputs.blocks]
+    exact_p, exact_h = oracle.backbone(inputs.emb.float(), inputs.key_lengths, blocks32, inputs.head_weight.float(),
+                                       inputs.head_bias.float(), num_heads=inputs.num_heads, return_hidden=True)
+    valid = torch.arange(512)[None, :] < inputs.key_lengths[:, None]
+    for routes in ({}, {"dense_tokens": True}, {"split_out_ffn": True}):
+        p, hidden = _run(inputs, device, **routes)
+        torch.testing.assert_close(hidden.cpu().float()[valid], exact_h[valid], rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(p.cpu(), exact_p, rtol=0, atol=2e-2)
 
 
 def test_interaction_block_routes_agree(device):

@@ -239,6 +239,84 @@ def test_block_and_backbone_compose_the_pinned_pieces():
     torch.testing.assert_close(p0, p[:1])
 
 
+def test_interaction_block_float64_loop_with_scattered_padding_and_role_mask():
+    """``oracle.interaction_block`` (experiments/symbiosis/backbone.py:51-68) against a per-token float64 loop that
+    shares none of its code: query / key RMSNorm over the model width, per-head softmax over the keys the mask shows,
+    both residual updates multiplied by ``~padding`` (padding scattered inside the samples), under the role mask, under
+    no mask at all (padded keys are then visible to everyone) and without the query / key norm."""
+    g = torch.Generator().manual_seed(17)
+    batch, tokens, d, heads, f, eps = 2, 6, 8, 2, 12, 1e-6
+    dh = d // heads
+    x = torch.randn(batch, tokens, d, generator=g, dtype=torch.float64)
+    padding = torch.tensor([[False, True, False, False, True, False], [False, False, True, True, True, False]])
+    roles = torch.tensor([0, 1, 1, 2, 3, 3])
+    w = {"attn_norm.weight": 1 + 0.2 * torch.randn(d, generator=g, dtype=torch.float64),
+         "qkv.weight": torch.randn(3 * d, d, generator=g, dtype=torch.float64) * d ** -0.5,
+         "qkv.bias": 0.1 * torch.randn(3 * d, generator=g, dtype=torch.float64),
+         "query_norm.weight": 1 + 0.2 * torch.randn(d, generator=g, dtype=torch.float64),
+         "key_norm.weight": 1 + 0.2 * torch.randn(d, generator=g, dtype=torch.float64),
+         "out.weight": torch.randn(d, d, generator=g, dtype=torch.float64) * d ** -0.5,
+         "out.bias": 0.1 * torch.randn(d, generator=g, dtype=torch.float64),
+         "ffn_norm.weight": 1 + 0.2 * torch.randn(d, generator=g, dtype=torch.float64),
+         "up.weight": torch.randn(2 * f, d, generator=g, dtype=torch.float64) * d ** -0.5,
+         "up.bias": 0.1 * torch.randn(2 * f, generator=g, dtype=torch.float64),
+         "down.weight": torch.randn(d, f, generator=g, dtype=torch.float64) * f ** -0.5,
+         "down.bias": 0.1 * torch.randn(d, generator=g, dtype=torch.float64)}
+
+    def rms(row, weight):
+        scale = 1.0 / math.sqrt(sum(float(v) ** 2 for v in row) / len(row) + eps)
+        return [float(v) * scale * float(weight[i]) for i, v in enumerate(row)]
+
+    def dense(row, weight, bias):
+        return [sum(float(weight[o, c]) * row[c] for c in range(len(row))) + float(bias[o]) for o in range(weight.shape[0])]
+
+    def loop(mask, qk_norm):
+        out = torch.zeros_like(x)
+        mid = torch.zeros_like(x)
+        for b in range(batch):
+            q, k, v = [], [], []
+            for t in range(tokens):
+                proj = dense(rms(x[b, t].tolist(), w["attn_norm.weight"]), w["qkv.weight"], w["qkv.bias"])
+                qt, kt = proj[:d], proj[d:2 * d]
+                if qk_norm:
+                    qt, kt = rms(qt, w["query_norm.weight"]), rms(kt, w["key_norm.weight"])
+                q.append(qt), k.append(kt), v.append(proj[2 * d:])
+            for t in range(tokens):
+                attended = []
+                for h in range(heads):
+                    cols = range(h * dh, (h + 1) * dh)
+                    seen = [j for j in range(tokens) if mask is None or bool(mask[b, 0, t, j])]
+                    scores = [sum(q[t][c] * k[j][c] for c in cols) / math.sqrt(dh) for j in seen]
+                    top = max(scores)
+                    weights = [math.exp(sc - top) for sc in scores]
+                    total = sum(weights)
+                    attended += [sum(wt * v[j][c] for wt, j in zip(weights, seen)) / total for c in cols]
+                keep = 0.0 if bool(padding[b, t]) else 1.0
+                update = dense(attended, w["out.weight"], w["out.bias"])
+                x1 = [float(x[b, t, c]) + keep * update[c] for c in range(d)]
+                mid[b, t] = torch.tensor(x1, dtype=torch.float64)
+                up = dense(rms(x1, w["ffn_norm.weight"]), w["up.weight"], w["up.bias"])
+                hidden = [up[j] / (1.0 + math.exp(-up[j])) * up[f + j] for j in range(f)]
+                down = dense(hidden, w["down.weight"], w["down.bias"])
+                out[b, t] = torch.tensor([x1[c] + keep * down[c] for c in range(d)], dtype=torch.float64)
+        return out, mid
+
+    role_mask = oracle.metadata_attention_mask(padding, roles)
+    assert role_mask.shape[0] == batch and role_mask.shape[-2:] == (tokens, tokens)
+    assert role_mask.any(dim=-1).all()  # every query row sees a key, as the reference's contract test demands
+    plain = {k: v for k, v in w.items() if not k.startswith(("query_norm", "key_norm"))}
+    for mask, weights, qk_norm in ((role_mask, w, True), (None, w, True), (role_mask, plain, False)):
+        want, want_mid = loop(mask, qk_norm)
+        got, got_mid = oracle.interaction_block(x, padding, mask, weights, num_heads=heads, eps=eps)
+        torch.testing.assert_close(got_mid, want_mid, rtol=1e-9, atol=1e-9)
+        torch.testing.assert_close(got, want, rtol=1e-9, atol=1e-9)
+        assert torch.equal(got[padding], x[padding]) and torch.equal(got_mid[padding], x[padding])
+    # the mask matters: role mask and no mask give different streams
+    a, _ = oracle.interaction_block(x, padding, role_mask, w, num_heads=heads)
+    b, _ = oracle.interaction_block(x, padding, None, w, num_heads=heads)
+    assert (a - b).abs().max().item() > 1e-3
+
+
 # ---- FP8 (no reference counterpart; the rounding itself is pinned, the layer is defined by its formula) ----------------
 
 
