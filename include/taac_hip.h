@@ -10,7 +10,8 @@
  *     returns a human-readable message (thread-local storage, valid until the next call on that thread).
  *   - Arguments are validated on the host before any kernel is launched; a rejected call launches nothing.
  *   - `dtype` is a taac_dtype value.
- *   - No global mutable state besides the thread-local error string: calls from different host threads and on different streams are independent.
+ *   - No global mutable state besides the thread-local error string (and the scratch array of
+ *     taac_rmsnorm_bwd_static): calls from different host threads and on different streams are independent.
  *     Behaviour is chosen by arguments only. Two environment variables exist as TEST HOOKS and change no result:
  *     TAAC_TS_MAX_WORKGROUPS caps the grid of the persistent dense kernels (so that small test inputs walk several
  *     tiles per workgroup), TAAC_FP8_TILED routes taac_linear_fp8 to its generic tiled kernel.
@@ -97,6 +98,19 @@ int taac_rmsnorm_bwd(const void* x, const void* w, const void* dy, void* dx, voi
                      int64_t workspace_floats, int64_t rows, int32_t cols, float eps, int dtype, void* stream);
 int taac_layernorm_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw, void* db, float* workspace,
                        int64_t workspace_floats, int64_t rows, int32_t cols, float eps, int dtype, void* stream);
+
+/*
+ * taac_rmsnorm_bwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the per-workgroup partial sums of dw live in a device array that is part of the
+ * library image (TAAC_RMSNORM_BWD_STATIC_MAX_COLS * 1024 floats = 8 MiB per GPU, held until the process ends) instead
+ * of a caller workspace. No counterpart in the reference. Arguments and results as taac_rmsnorm_bwd (bit-identical);
+ * cols above TAAC_RMSNORM_BWD_STATIC_MAX_COLS are rejected with TAAC_ERR_UNSUPPORTED. The call allocates and frees
+ * nothing. All calls on one GPU share the array: calls that overlap on one GPU (different streams or host threads)
+ * race on it and must be serialised by the caller; calls on one stream are ordered and safe.
+ */
+#define TAAC_RMSNORM_BWD_STATIC_MAX_COLS 2048
+int taac_rmsnorm_bwd_static(const void* x, const void* w, const void* dy, void* dx, void* dw, int64_t rows,
+                            int32_t cols, float eps, int dtype, void* stream);
 
 /*
  * Key-padding-masked attention forward: o = softmax(q k^T / sqrt(d) + mask) v per (batch, head), softmax in

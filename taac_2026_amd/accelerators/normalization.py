@@ -125,6 +125,24 @@ def hip_rms_norm_backward_kernel(x: torch.Tensor, weight: torch.Tensor, grad_out
     return grad_x, grad_w
 
 
+def hip_rms_norm_backward_static_kernel(x: torch.Tensor, weight: torch.Tensor, grad_out: torch.Tensor, eps: float,
+                                        grad_x: torch.Tensor, grad_w: torch.Tensor) -> None:
+    """:func:`hip_rms_norm_backward_kernel` for callers that cannot allocate device memory (graph capture, serving loops):
+    writes into the given ``grad_x [R, D]`` / ``grad_w [D]`` and keeps the partial sums in the library's built-in device
+    array (``taac_rmsnorm_bwd_static``; at most 2048 columns; calls that overlap on one GPU must be serialised)."""
+    library = _native.load_library()
+    require_cuda_tensors("hip rms_norm backward", x, weight, grad_out, grad_x, grad_w)
+    if grad_x.shape != x.shape or grad_w.shape != weight.shape or grad_x.dtype != x.dtype or grad_w.dtype != x.dtype:
+        raise ValueError("rms_norm backward: grad_x / grad_w must have the shape and dtype of x / weight")
+    if not (x.is_contiguous() and grad_out.is_contiguous() and grad_x.is_contiguous() and grad_w.is_contiguous()):
+        raise ValueError("rms_norm backward: tensors must be contiguous")
+    status = library.taac_rmsnorm_bwd_static(
+        x.data_ptr(), weight.data_ptr(), grad_out.data_ptr(), grad_x.data_ptr(), grad_w.data_ptr(), x.shape[0], x.shape[1],
+        float(eps), _native.dtype_code(x.dtype), _native.current_stream(x.device),
+    )
+    _native.check(status, "rms_norm backward")
+
+
 def hip_layer_norm_backward_kernel(x: torch.Tensor, weight: torch.Tensor, grad_out: torch.Tensor, eps: float
                                    ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """``-> (grad_rows, grad_weight, grad_bias)`` in x's dtype."""
@@ -219,6 +237,7 @@ __all__ = [
     "hip_layer_norm_backward_kernel",
     "hip_layer_norm_kernel",
     "hip_rms_norm_backward_kernel",
+    "hip_rms_norm_backward_static_kernel",
     "hip_rms_norm_kernel",
     "layer_norm",
     "resolved_layer_norm_backend",

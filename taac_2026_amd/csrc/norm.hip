@@ -9,6 +9,8 @@
 //   RMSNorm:   y = x * rsqrt(mean(x^2) + eps) * w      (accelerators/normalization/rms_norm.py:71-73)
 //   LayerNorm: y = (x - mean) * rsqrt(var + eps) * w + b, var from centred values
 //                                                      (normalization/kernels/triton.py:224-247)
+#include <mutex>
+
 #include "common.h"
 
 namespace taac {
@@ -822,6 +824,55 @@ extern "C" int taac_rmsnorm_bwd(const void* x, const void* w, const void* dy, vo
                                 void* stream) {
   return taac::norm_bwd_entry<false>("taac_rmsnorm_bwd", x, w, dy, dx, dw, nullptr, workspace, workspace_floats, rows,
                                      cols, eps, dtype, stream);
+}
+
+// ---- taac_rmsnorm_bwd without a caller workspace -----------------------------------------------------------------------
+// The partial rows of dw live in a device array of the library image. In host code the array's name is only a handle:
+// its device address is looked up once per device (every GPU holds its own copy at its own address) and that pointer
+// is what the kernels receive, exactly as they receive the caller's workspace in taac_rmsnorm_bwd. Nothing has to be
+// cleared between calls: a launch writes every partial row it later reads.
+namespace taac {
+namespace {
+constexpr int64_t kStaticBwdFloats = static_cast<int64_t>(kBwdMaxBlocks) * TAAC_RMSNORM_BWD_STATIC_MAX_COLS;
+static __device__ __align__(256) float scratch[kStaticBwdFloats];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device; nullptr (with the error set) when it cannot be resolved.
+float* static_scratch(const char* name) {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+    set_error(TAAC_ERR_LAUNCH, "%s: cannot query the current device", name);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    float* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      set_error(TAAC_ERR_LAUNCH, "%s: cannot resolve the device scratch array: %s", name, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[device] = ptr;
+  }
+  return g_scratch_ptr[device];
+}
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_rmsnorm_bwd_static(const void* x, const void* w, const void* dy, void* dx, void* dw, int64_t rows,
+                                       int32_t cols, float eps, int dtype, void* stream) {
+  using namespace taac;
+  const char* name = "taac_rmsnorm_bwd_static";
+  if (cols > TAAC_RMSNORM_BWD_STATIC_MAX_COLS)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: cols=%d exceeds the %d columns the built-in scratch array covers", name,
+                     cols, TAAC_RMSNORM_BWD_STATIC_MAX_COLS);
+  if (rows < 0 || cols <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows must be >= 0 and cols > 0", name);
+  float* ptr = static_scratch(name);
+  if (ptr == nullptr) return TAAC_ERR_LAUNCH;
+  return norm_bwd_entry<false>(name, x, w, dy, dx, dw, nullptr, ptr, kStaticBwdFloats, rows, cols, eps, dtype, stream);
 }
 
 extern "C" int taac_layernorm_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw, void* db,

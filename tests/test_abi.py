@@ -123,6 +123,10 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
     # a width that is not a whole number of 16-byte vectors takes the generic kernel, which needs its workspace too
     assert library.taac_rmsnorm_bwd(fake, fake, fake, fake, fake, fake, 8 * 260 - 1, 8, 260, 1e-6, bf16, None) == invalid
     assert b"workspace" in library.taac_last_error()
+    # the variant with the built-in scratch array rejects widths beyond the array before it touches the device
+    assert library.taac_rmsnorm_bwd_static(fake, fake, fake, fake, fake, 8, 2056, 1e-6, bf16, None) == unsupported
+    assert b"2048" in library.taac_last_error()
+    assert library.taac_rmsnorm_bwd_static(fake, fake, fake, fake, fake, -1, 256, 1e-6, bf16, None) == invalid
     assert library.taac_layernorm_bwd(fake, fake, fake, None, fake, fake, fake, 1 << 30, 8, 256, 1e-5, bf16, None) == invalid
 
     # out projection + feed-forward half in one kernel: both weight sets packed, the block input required
