@@ -445,6 +445,34 @@ int taac_linear_fp8(const void* a, int a_is_fp8, int64_t lda, const void* w, con
                     int epilogue, int gate_first, void* stream);
 
 /*
+ * Fused feed-forward half with FP8 (e4m3fn) MFMA operands and per-tensor scales, the FP8 counterpart of
+ * taac_swiglu_ffn_fwd: the chain of two taac_linear_fp8 layers
+ *   h   = norm_weight ? bf16(rmsnorm(x, norm_weight, eps)) : x
+ *   hid = bf16( silu(g) * u ),  g, u = chunk2( (q(h) q(w_up)^T) (amax_x / 448)(amax_up / 448) + b_up )
+ *   out = bf16( (q(hid) q(w_down)^T) (amax_hidden / 448)(amax_down / 448) + b_down + residual )
+ * with q(t) = sat(t / (amax_t / 448)) in e4m3 and amax_hidden = max |hid| over all tokens, which the call computes
+ * itself: a first launch evaluates the up projection and the gate only to reduce max |hid| into *amax_hidden, a second
+ * launch evaluates the whole layer with that scale. The [M, F] hidden state is never written to memory.
+ * packed_weights: blob of taac_ffn_fp8_pack_weights (both weights quantised with their amax and laid out in fragment
+ * order; 3 * D * F bytes, taac_ffn_fp8_packed_bytes). amax_x: device float, max |h| over the tokens (of the normalised
+ * input when norm_weight is given: taac_amax of it, or the amax_next / amax_out of the producing call). amax_up /
+ * amax_down: the amax the weights were packed with. amax_hidden: device float, written. x, residual, out, rows / n_rows,
+ * gate_first: as in taac_swiglu_ffn_fwd (out may alias residual and x). D: 128 or 256, F a multiple of 64.
+ * amax_next (or NULL): receives max | bf16(rmsnorm(out, next_norm_weight, next_eps)) | over the tokens (max |out| when
+ * next_norm_weight is NULL): the amax_x of the layer that consumes out, so that no pass of its own is needed for it.
+ * No counterpart in the reference (it has no FP8 code); semantics follow the quantize -> matmul -> dequantize emulation.
+ */
+int64_t taac_ffn_fp8_packed_bytes(int32_t D, int32_t F);
+int taac_ffn_fp8_pack_weights(const void* w_up, const void* w_down, const float* amax_up, const float* amax_down,
+                              void* packed, int32_t D, int32_t F, int gate_first, void* stream);
+int taac_swiglu_ffn_fp8_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* packed_weights,
+                            const void* b_up, const void* b_down, const float* amax_x, const float* amax_up,
+                            const float* amax_down, float* amax_hidden, const void* residual, int64_t ldr, void* out,
+                            int64_t ldo, int64_t M, int32_t D, int32_t F, int gate_first, const int32_t* rows,
+                            const int32_t* n_rows, const void* next_norm_weight, float next_eps, float* amax_next,
+                            void* stream);
+
+/*
  * Readout of the backbone: p[b] = sigmoid( masked_mean(x[b, :L_b, :]) . w_head + b_head ), with
  * L_b = clamp(lengths[b], 0, T) and the mean's divisor clamped to >= 1.
  * x: [B, T, D] bf16 contiguous; lengths: int32 [B]; w_head: [D] bf16; b_head: [1] bf16 or NULL; p: float [B].

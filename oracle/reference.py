@@ -472,3 +472,17 @@ def linear_fp8(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None 
     if residual is not None:
         y = y + residual.float()
     return y.to(torch.bfloat16)
+
+
+def swiglu_ffn_fp8(x: torch.Tensor, norm_weight: torch.Tensor | None, up_weight: torch.Tensor, up_bias: torch.Tensor | None,
+                   down_weight: torch.Tensor, down_bias: torch.Tensor | None, *, residual: torch.Tensor | None = None,
+                   eps: float = 1e-6, gate_first: bool = True) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """The feed-forward half as a chain of two ``linear_fp8`` layers on bf16 tensors (FP8 configuration of the dense
+    layers; experiments/symbiosis/backbone.py:19-21, 66-67 for the recipe): ``h = rmsnorm(x)`` in fp32 statistics, one
+    rounding; ``hidden = linear_fp8(h, up, swiglu=True)``; ``out = linear_fp8(hidden, down, residual=residual)``, every
+    tensor quantised with its own ``amax / 448``. Returns (out, hidden, h). Parity unpinned by the reference like
+    ``linear_fp8`` itself; composed from it only."""
+    h = x if norm_weight is None else rms_norm_fp32(x, norm_weight, eps)
+    hidden = linear_fp8(h, up_weight, up_bias, swiglu=True, gate_first=gate_first)
+    out = linear_fp8(hidden, down_weight, down_bias, residual=residual)
+    return out, hidden, h

@@ -621,6 +621,92 @@ def linear_fp8(
     return out.reshape(*shape[:-1], out_features)
 
 
+def pack_ffn_weights_fp8(up_weight: torch.Tensor, down_weight: torch.Tensor, *, gate_first: bool = True
+                         ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Quantises ``(up_weight [2F, D], down_weight [D, F])`` to e4m3 with their per-tensor scales and lays them out in
+    the fragment order of :func:`swiglu_ffn_fp8`. Returns ``(blob uint8, amax_up, amax_down)``."""
+    name = "hip pack_ffn_weights_fp8"
+    require_cuda_tensors(name, up_weight, down_weight)
+    _check_bf16(name, up_weight, down_weight)
+    library = _native.load_library()
+    d_model, hidden = down_weight.shape
+    if up_weight.shape != (2 * hidden, d_model):
+        raise ValueError("pack_ffn_weights_fp8 expects up_weight [2F, D] and down_weight [D, F]")
+    nbytes = library.taac_ffn_fp8_packed_bytes(d_model, hidden)
+    if nbytes < 0:
+        raise RuntimeError(f"pack_ffn_weights_fp8: unsupported shape D={d_model}, F={hidden} (D 128 / 256, F a multiple of 64)")
+    up_weight, down_weight = up_weight.detach().contiguous(), down_weight.detach().contiguous()
+    amax_up, amax_down = amax(up_weight), amax(down_weight)
+    packed = torch.empty(nbytes, dtype=torch.uint8, device=up_weight.device)
+    status = library.taac_ffn_fp8_pack_weights(up_weight.data_ptr(), down_weight.data_ptr(), amax_up.data_ptr(),
+                                               amax_down.data_ptr(), packed.data_ptr(), d_model, hidden,
+                                               int(bool(gate_first)), _native.current_stream(up_weight.device))
+    _native.check(status, "pack_ffn_weights_fp8")
+    return packed, amax_up, amax_down
+
+
+def swiglu_ffn_fp8(
+    x: torch.Tensor,
+    packed_weights: tuple[torch.Tensor, torch.Tensor, torch.Tensor],
+    up_bias: torch.Tensor | None,
+    down_bias: torch.Tensor | None,
+    amax_x: torch.Tensor,
+    *,
+    hidden_size: int,
+    residual: torch.Tensor | None = None,
+    gate_first: bool = True,
+    norm_weight: torch.Tensor | None = None,
+    eps: float = 1e-6,
+    token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
+    out: torch.Tensor | None = None,
+    next_norm_weight: torch.Tensor | None = None,
+    next_eps: float = 1e-6,
+    want_amax_next: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
+    """The feed-forward half with e4m3 MFMA operands and per-tensor scales as ONE fused layer (two launches: the first
+    finds the scale of the gated hidden state, the second evaluates the layer; the hidden state never reaches memory):
+    ``residual + down_fp8(silu(gate) * value)``, ``gate, value = up_fp8(rmsnorm(x)).chunk(2, -1)``, each ``*_fp8`` the
+    quantize -> matmul -> dequantize layer of :func:`linear_fp8`. ``packed_weights`` is the triple returned by
+    :func:`pack_ffn_weights_fp8` (packed with the same ``gate_first``); ``amax_x`` the float32 scalar max of the tensor
+    the up projection quantises (``rmsnorm(x) * norm_weight`` rounded to bf16 when ``norm_weight`` is given). Returns
+    ``(out, amax_hidden, amax_next)``; ``amax_next`` (with ``want_amax_next``) is the max of
+    ``|rmsnorm(out, next_norm_weight)|`` (of ``|out|`` without a weight), i.e. the ``amax_x`` of the layer that consumes
+    ``out``. ``token_rows`` / ``out`` as in :func:`swiglu_ffn`."""
+    name = "hip swiglu_ffn_fp8"
+    blob, amax_up, amax_down = packed_weights
+    require_cuda_tensors(name, x, blob, amax_up, amax_down, up_bias, down_bias, amax_x, residual, norm_weight, next_norm_weight)
+    require_inference(name, x, up_bias, down_bias, residual, norm_weight)
+    _check_bf16(name, x, up_bias, down_bias, residual, norm_weight, next_norm_weight)
+    rows, shape = _as_rows(x)
+    d_model, hidden = rows.shape[1], int(hidden_size)
+    library = _native.load_library()
+    if library.taac_ffn_fp8_packed_bytes(d_model, hidden) != blob.numel():
+        raise ValueError(f"swiglu_ffn_fp8: the packed weights do not match D={d_model}, F={hidden}")
+    for scale in (amax_x, amax_up, amax_down):
+        if scale.dtype != torch.float32 or scale.numel() != 1:
+            raise ValueError("swiglu_ffn_fp8 scales must be float32 scalar tensors")
+    if residual is not None and residual.shape != shape:
+        raise ValueError("swiglu_ffn_fp8 residual must have the shape of the input")
+    res_rows = None
+    if residual is not None:
+        res_rows = residual.reshape(-1, d_model)
+        if res_rows.stride(-1) != 1 or res_rows.stride(0) % 8 != 0:
+            res_rows = res_rows.contiguous()
+    index, count = _token_rows(name, token_rows, rows)
+    out = _output_rows(name, out, (rows.shape[0], d_model), index is not None, x)
+    amax_hidden = torch.empty((), dtype=torch.float32, device=x.device)
+    amax_next = torch.empty((), dtype=torch.float32, device=x.device) if (want_amax_next or next_norm_weight is not None) else None
+    status = library.taac_swiglu_ffn_fp8_fwd(
+        rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), blob.data_ptr(), _native.ptr(up_bias),
+        _native.ptr(down_bias), amax_x.data_ptr(), amax_up.data_ptr(), amax_down.data_ptr(), amax_hidden.data_ptr(),
+        _native.ptr(res_rows), res_rows.stride(0) if res_rows is not None else d_model, out.data_ptr(), d_model,
+        rows.shape[0], d_model, hidden, int(bool(gate_first)), _native.ptr(index), _native.ptr(count),
+        _native.ptr(next_norm_weight), float(next_eps), _native.ptr(amax_next), _native.current_stream(x.device),
+    )
+    _native.check(status, "swiglu_ffn_fp8")
+    return out.reshape(shape), amax_hidden, amax_next
+
+
 __all__ = [
     "FP8_MAX",
     "amax",
@@ -629,6 +715,8 @@ __all__ = [
     "linear_fp8",
     "norm_linear",
     "pack_ffn_weights",
+    "pack_ffn_weights_fp8",
+    "swiglu_ffn_fp8",
     "valid_rows",
     "pack_linear_weight",
     "qkv_projection",
