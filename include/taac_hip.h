@@ -445,6 +445,26 @@ int taac_linear_fp8(const void* a, int a_is_fp8, int64_t lda, const void* w, con
                     int epilogue, int gate_first, void* stream);
 
 /*
+ * Fused [RMSNorm ->] FP8 dense layer [-> + residual], the FP8 counterpart of
+ * taac_norm_linear_fwd (K = 256, N a multiple of 64):
+ *   h   = norm_weight ? bf16(rmsnorm(x, norm_weight, eps)) : x                    quantised with scale amax_x / 448
+ *   out = bf16( (q(h) q(w)^T) (amax_x / 448)(amax_w / 448) + bias [+ residual] )  one rounding
+ * x: [M, K] bf16 (row stride ldx); w_fp8: [N, K] e4m3 bytes (taac_quantize_fp8 with amax_w); amax_x: max |h| over the
+ * tokens (device float; of the normalised rows when norm_weight is given). rows / n_rows: as in taac_swiglu_ffn_fwd
+ * (token i lives in row rows[i] of x / residual / out; other rows are neither read nor written).
+ * amax_out (or NULL): receives the per-tensor scale of the layer that consumes out, reduced in the epilogue (no pass of
+ * its own): max over the tokens of | bf16( rstd * max_f |out_f * out_norm_weight_f| ) | with rstd the RMSNorm statistic
+ * of the rounded output row (eps out_eps), or max |out| when out_norm_weight is NULL. The first form equals
+ * max | bf16(rmsnorm(out, out_norm_weight)) | up to the order of two fp32 multiplications.
+ * No counterpart in the reference (it has no FP8 code).
+ */
+int taac_norm_linear_fp8_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w_fp8,
+                             const void* bias, const float* amax_x, const float* amax_w, const void* residual, int64_t ldr,
+                             void* out, int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows,
+                             const int32_t* n_rows, const void* out_norm_weight, float out_eps, float* amax_out,
+                             void* stream);
+
+/*
  * Fused feed-forward half with FP8 (e4m3fn) MFMA operands and per-tensor scales, the FP8 counterpart of
  * taac_swiglu_ffn_fwd: the chain of two taac_linear_fp8 layers
  *   h   = norm_weight ? bf16(rmsnorm(x, norm_weight, eps)) : x

@@ -171,6 +171,11 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p],
     ),
     "taac_backbone_workspace_bytes": (c_int64, [c_int32, c_int32, c_int32, c_int32, c_int32]),
+    "taac_norm_linear_fp8_fwd": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
+         c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p],
+    ),
     "taac_ffn_fp8_packed_bytes": (c_int64, [c_int32, c_int32]),
     "taac_ffn_fp8_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int, c_void_p]),
     "taac_swiglu_ffn_fp8_fwd": (

@@ -621,6 +621,64 @@ def linear_fp8(
     return out.reshape(*shape[:-1], out_features)
 
 
+def norm_linear_fp8(
+    x: torch.Tensor,
+    weight_fp8: torch.Tensor,
+    amax_x: torch.Tensor,
+    amax_w: torch.Tensor,
+    bias: torch.Tensor | None = None,
+    *,
+    norm_weight: torch.Tensor | None = None,
+    eps: float = 1e-6,
+    residual: torch.Tensor | None = None,
+    token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
+    out: torch.Tensor | None = None,
+    out_norm_weight: torch.Tensor | None = None,
+    out_eps: float = 1e-6,
+    want_amax_out: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """``residual + linear_fp8(rmsnorm(x, norm_weight), weight_fp8)`` (norm and residual optional) as one kernel for
+    ``in_features == 256`` (``taac_norm_linear_fp8_fwd``): the rows are normalised, rounded to bf16 and quantised with
+    ``amax_x / 448`` on their way into registers. ``amax_x`` is the float32 scalar max of the tensor that is quantised
+    (of the normalised rows when ``norm_weight`` is given). ``token_rows`` / ``out`` as in :func:`norm_linear`.
+    Returns ``(out, amax_out)``; with ``want_amax_out`` (or an ``out_norm_weight``) the epilogue also reduces the scale
+    of the layer that consumes the output: the max of ``|rmsnorm(out, out_norm_weight)|`` (of ``|out|`` without a
+    weight), so that no pass of its own is needed for it."""
+    name = "hip norm_linear_fp8"
+    require_cuda_tensors(name, x, weight_fp8, amax_x, amax_w, bias, norm_weight, residual, out_norm_weight)
+    require_inference(name, x, bias, norm_weight, residual)
+    _check_bf16(name, x, bias, norm_weight, residual, out_norm_weight)
+    if weight_fp8.dtype != torch.float8_e4m3fn:
+        raise RuntimeError("norm_linear_fp8 weight must be float8_e4m3fn")
+    rows, shape = _as_rows(x)
+    _check_weight(name, rows, weight_fp8, bias)
+    out_features, in_features = weight_fp8.shape
+    if in_features != 256 or out_features % 64 != 0:
+        raise RuntimeError("norm_linear_fp8 is built for in_features = 256 and out_features a multiple of 64")
+    weight_fp8 = weight_fp8.contiguous()
+    res_rows = None
+    if residual is not None:
+        if residual.shape != (*shape[:-1], out_features):
+            raise ValueError("norm_linear_fp8 residual must have the shape of the output")
+        res_rows = residual.reshape(-1, out_features)
+        if res_rows.stride(-1) != 1 or res_rows.stride(0) % 8 != 0:
+            res_rows = res_rows.contiguous()
+    index, count = _token_rows(name, token_rows, rows)
+    out = _output_rows(name, out, (rows.shape[0], out_features), index is not None, x)
+    amax_out = None
+    if want_amax_out or out_norm_weight is not None:
+        amax_out = torch.empty((), dtype=torch.float32, device=x.device)
+    library = _native.load_library()
+    status = library.taac_norm_linear_fp8_fwd(
+        rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), weight_fp8.data_ptr(), _native.ptr(bias),
+        amax_x.data_ptr(), amax_w.data_ptr(), _native.ptr(res_rows), res_rows.stride(0) if res_rows is not None else out_features,
+        out.data_ptr(), out_features, rows.shape[0], out_features, in_features, _native.ptr(index), _native.ptr(count),
+        _native.ptr(out_norm_weight), float(out_eps), _native.ptr(amax_out), _native.current_stream(x.device),
+    )
+    _native.check(status, "norm_linear_fp8")
+    return out.reshape(*shape[:-1], out_features), amax_out
+
+
 def pack_ffn_weights_fp8(up_weight: torch.Tensor, down_weight: torch.Tensor, *, gate_first: bool = True
                          ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Quantises ``(up_weight [2F, D], down_weight [D, F])`` to e4m3 with their per-tensor scales and lays them out in
@@ -715,6 +773,7 @@ __all__ = [
     "linear_fp8",
     "norm_linear",
     "pack_ffn_weights",
+    "norm_linear_fp8",
     "pack_ffn_weights_fp8",
     "swiglu_ffn_fp8",
     "valid_rows",

@@ -49,9 +49,17 @@ struct Fp8TsParams {
   bf16_t* out;              // [M, N] (SwiGLU: [M, N / 2]) row stride ldo
   const float* amax_a;
   const float* amax_w;
-  int64_t M, lda, ldo;
+  int64_t M, lda, ldo, ldr;
   int32_t N;                // weight rows
   int32_t gate_first;
+  // taac_norm_linear_fp8_fwd only:
+  const bf16_t* norm_w;     // [K] RMSNorm weight applied to the rows before quantisation, or null
+  float eps;
+  const int32_t* rows;      // optional row index: token i lives in row rows[i] of a / residual / out
+  const int32_t* n_rows;    // with rows: device pointer to the number of tokens
+  float* amax_out;          // STATS: receives max |bf16(rmsnorm(out, out_norm_w))| (max |out| without a weight)
+  const bf16_t* out_norm_w; // [N] or null
+  float out_eps;
 };
 
 __device__ __forceinline__ float clamp448(float x) { return __builtin_fminf(__builtin_fmaxf(x, -448.f), 448.f); }
@@ -80,8 +88,13 @@ __device__ __forceinline__ void lds_wait_halves(u32x4& a, u32x4& b) {
   asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
 }
 
-template <int kK, int EPI, bool A_FP8>
-__global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const Fp8TsParams p, const int num_tiles) {
+// STATS (taac_norm_linear_fp8_fwd): the epilogue also reduces, per token, the sum of squares and max |out * weight| of
+// the rounded output over the steps of a tile, and from them the maximum over all tokens of |rmsnorm(out) * weight| - the
+// per-tensor scale of the layer that consumes the output - without a pass of its own over it.
+// NORM: the rows are RMS-normalised (weight p.norm_w) before they are quantised.
+template <int kK, int EPI, bool A_FP8, bool STATS, bool NORM = false>
+__global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const Fp8TsParams p, const int /*max_tiles*/) {
+  static_assert(!NORM || (kK == 256 && !A_FP8), "the normalisation is built for bf16 rows of 256 features");
   constexpr bool RES = EPI == TAAC_EPI_RESIDUAL;
   constexpr int kTT = tiles_per_wave(kK, EPI);
   constexpr int kTokPerWg = kWaves * 32 * kTT;
@@ -113,9 +126,25 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
   const int hh = lane / 32;
   const int F = p.N / 2;
   const int nsteps_tile = GLU ? F / 32 : p.N / kRows;
+  // tokens: M, or the device-side count of a row index
+  int64_t count = p.M;
+  if (p.rows != nullptr) {
+    const int64_t n = *p.n_rows;
+    count = n < p.M ? n : p.M;
+  }
+  const int num_tiles = static_cast<int>((count + kTokPerWg - 1) / kTokPerWg);
   const int my_tiles = (num_tiles - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) /
                        static_cast<int>(gridDim.x);
+  if (my_tiles <= 0) return;  // whole workgroup: no tile for it (fewer tokens than the grid was sized for)
   const int total = my_tiles * nsteps_tile;
+  // memory row of token `tok`; tokens at or beyond the count repeat the last one (same values, benign duplicate stores)
+  auto row_of = [&](int64_t tok) -> int64_t {
+    tok = tok < count ? tok : count - 1;
+    return p.rows != nullptr ? static_cast<int64_t>(p.rows[tok]) : tok;
+  };
+  bf16_t* normw_lds = bias_lds + p.N;           // [K] (taac_norm_linear_fp8_fwd)
+  bf16_t* outw_lds = normw_lds + kK;            // [N]
+  float* red = reinterpret_cast<float*>(outw_lds + p.N);
 
   const float amax_a = fmaxf(*p.amax_a, 1e-12f);
   const float amax_w = fmaxf(*p.amax_w, 1e-12f);
@@ -150,9 +179,8 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
   auto request_residual = [&](int64_t tok_base, int chunk, bf16x8 (&res)[NST]) {
 #pragma unroll
     for (int i = 0; i < NST; ++i) {
-      int64_t tok = tok_base + (i / NSTT) * 32 + (i % NSTT) * ROWS_PER_STORE + lane / PIECES;
-      tok = tok < p.M ? tok : p.M - 1;
-      res[i] = *reinterpret_cast<const bf16x8*>(p.residual + tok * p.ldo + chunk * OUTC + (lane % PIECES) * 8);
+      const int64_t row = row_of(tok_base + (i / NSTT) * 32 + (i % NSTT) * ROWS_PER_STORE + lane / PIECES);
+      res[i] = *reinterpret_cast<const bf16x8*>(p.residual + row * p.ldr + chunk * OUTC + (lane % PIECES) * 8);
     }
   };
   // Token rows -> e4m3 B-operand fragments.
@@ -160,8 +188,7 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
   auto load_tile = [&](int64_t tok_base) {
 #pragma unroll
     for (int t = 0; t < kTT; ++t) {
-      int64_t tok = tok_base + t * 32 + l32;
-      tok = tok < p.M ? tok : p.M - 1;
+      const int64_t tok = row_of(tok_base + t * 32 + l32);
       if (A_FP8) {
         const uint8_t* row = static_cast<const uint8_t*>(p.a) + tok * p.lda + hh * 32;
 #pragma unroll
@@ -180,6 +207,38 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
           for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
             for (int c = 0; c < 4; ++c) raw[ks][c] = *reinterpret_cast<const bf16x8*>(row + (k4 + ks) * 64 + c * 8);
+          if constexpr (NORM) {
+            // RMSNorm of the row (a lane and its partner lane ^ 32 hold its two halves), rounded to bf16 as the
+            // stand-alone norm rounds its output, then quantised
+            float ss = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+              for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                  const float v = static_cast<float>(raw[ks][c][e]);
+                  ss = fmaf(v, v, ss);
+                }
+            const uint32_t ssb = __builtin_bit_cast(uint32_t, ss);
+            const auto sw = __builtin_amdgcn_permlane32_swap(ssb, ssb, false, false);
+            ss = __builtin_bit_cast(float, static_cast<uint32_t>(sw[0])) + __builtin_bit_cast(float, static_cast<uint32_t>(sw[1]));
+            const float scale = rsqrtf(ss * (1.0f / kK) + p.eps);
+            // opaque here: otherwise the fp32 copies of the first sweep are kept alive for the second one
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+              for (int c = 0; c < 4; ++c) asm volatile("" : "+v"(raw[ks][c]));
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+              for (int c = 0; c < 4; ++c) {
+                const bf16x8 wv = *reinterpret_cast<const bf16x8*>(normw_lds + ks * 64 + hh * 32 + c * 8);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                  raw[ks][c][e] = static_cast<bf16_t>(static_cast<float>(raw[ks][c][e]) * scale * static_cast<float>(wv[e]));
+              }
+          }
 #pragma unroll
           for (int ks = 0; ks < 4; ++ks) {
             int q[8];
@@ -206,9 +265,19 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
   if (total > 1) stage(nsteps_tile > 1 ? 1 : 0, 1);
   if (RES) request_residual(tok_wave, 0, res_cur);
   stage_bias(p.bias, bias_lds, p.N, tid, kWaves * kWave);
+  if constexpr (NORM) {
+    stage_bias(p.norm_w, normw_lds, kK, tid, kWaves * kWave);
+    __syncthreads();  // the first tile is normalised before the common barrier below
+  }
+  if (STATS) stage_bias(p.out_norm_w, outw_lds, p.N, tid, kWaves * kWave);
   load_tile(tok_wave);
   vm_wait<0>();
   __syncthreads();
+  // STATS: per piece slot (token of the epilogue layout) the sum of squares and max |value * weight| over the tile's steps
+  [[maybe_unused]] float st_ss[NST], st_mw[NST];
+  [[maybe_unused]] float st_max = 0.f;
+#pragma unroll
+  for (int i = 0; i < NST; ++i) st_ss[i] = st_mw[i] = 0.f;
 
   uint8_t* tile_lds = tiles + wave * kTileWave;
   int chunk = 0;                    // step inside the tile
@@ -290,8 +359,7 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
 #pragma unroll
       for (int i = 0; i < NSTT; ++i) {
         const int row = i * ROWS_PER_STORE + lane / PIECES;
-        int64_t tok = tok_wave + t * 32 + row;
-        tok = tok < p.M ? tok : p.M - 1;
+        const int64_t tok = row_of(tok_wave + t * 32 + row);
         const f32x4 a0 = *reinterpret_cast<const f32x4*>(tile_lds + row * kTileRow + (lane % PIECES) * 32);
         const f32x4 a1 = *reinterpret_cast<const f32x4*>(tile_lds + row * kTileRow + (lane % PIECES) * 32 + 16);
         bf16x8 o;
@@ -306,8 +374,37 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
           o[4 + e] = static_cast<bf16_t>(x1);
         }
         *reinterpret_cast<bf16x8*>(p.out + tok * p.ldo + chunk * OUTC + (lane % PIECES) * 8) = o;
+        if constexpr (STATS) {
+          const bf16x8 wv = *reinterpret_cast<const bf16x8*>(outw_lds + chunk * OUTC + (lane % PIECES) * 8);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float r = static_cast<float>(o[e]);
+            st_ss[t * NSTT + i] = fmaf(r, r, st_ss[t * NSTT + i]);
+            const float rw = p.out_norm_w != nullptr ? r * static_cast<float>(wv[e]) : r;
+            st_mw[t * NSTT + i] = fmaxf(st_mw[t * NSTT + i], fabsf(rw));
+          }
+        }
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+    if constexpr (STATS) {
+      if (chunk == nsteps_tile - 1) {  // the tile is complete: a token's statistics are spread over PIECES lanes
+#pragma unroll
+        for (int i = 0; i < NST; ++i) {
+          float ss = st_ss[i], mw = st_mw[i];
+#pragma unroll
+          for (int off = 1; off < PIECES; off <<= 1) {
+            ss += __shfl_xor(ss, off, kWave);
+            mw = fmaxf(mw, __shfl_xor(mw, off, kWave));
+          }
+          const int64_t tok = tok_wave + (i / NSTT) * 32 + (i % NSTT) * ROWS_PER_STORE + lane / PIECES;
+          float v = mw;
+          if (p.out_norm_w != nullptr)
+            v = static_cast<float>(static_cast<bf16_t>(mw * rsqrtf(ss * (1.0f / static_cast<float>(p.N)) + p.out_eps)));
+          if (tok < count) st_max = fmaxf(st_max, v);
+          st_ss[i] = st_mw[i] = 0.f;
+        }
+      }
     }
     // ---- close the step ------------------------------------------------------------------------------------------------
     if (has_next) {
@@ -325,6 +422,17 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
     buf = buf == 2 ? 0 : buf + 1;
     if (++chunk == nsteps_tile) chunk = 0;
     if (++chunk2 == nsteps_tile) chunk2 = 0;
+  }
+  if constexpr (STATS) {
+    // maximum over the workgroup, one atomic on the float's bit pattern (non-negative floats order like their bits)
+    st_max = group_max<kWave>(st_max);
+    if (lane == 0) red[wave] = st_max;
+    __syncthreads();
+    if (tid == 0) {
+      for (int w = 1; w < kWaves; ++w) st_max = fmaxf(st_max, red[w]);
+      if (st_max > __builtin_nontemporal_load(p.amax_out))
+        atomicMax(reinterpret_cast<unsigned int*>(p.amax_out), __float_as_uint(st_max));
+    }
   }
 }
 
@@ -349,10 +457,10 @@ int launch_fp8_ts_for_k(const Fp8TsParams& p, int a_is_fp8, int epilogue, hipStr
   }
 #define TAAC_FP8_TS_LAUNCH(EPI, AF8)                                                                                \
   do {                                                                                                              \
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(linear_fp8_ts_kernel<K, EPI, AF8>),                       \
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(linear_fp8_ts_kernel<K, EPI, AF8, false>),                       \
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)) != hipSuccess) \
       return set_error(TAAC_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", name, lds_bytes);                    \
-    hipLaunchKernelGGL((linear_fp8_ts_kernel<K, EPI, AF8>), dim3(grid), dim3(kWaves * kWave), lds_bytes, s, p,      \
+    hipLaunchKernelGGL((linear_fp8_ts_kernel<K, EPI, AF8, false>), dim3(grid), dim3(kWaves * kWave), lds_bytes, s, p,      \
                        num_tiles);                                                                                  \
     return check_launch(name);                                                                                      \
   } while (0)
@@ -394,6 +502,7 @@ int launch_linear_fp8_ts(const void* a, int a_is_fp8, int64_t lda, const void* w
   p.M = M;
   p.lda = lda;
   p.ldo = ldo;
+  p.ldr = ldo;
   p.N = N;
   p.gate_first = gate_first ? 1 : 0;
   if (K == 256) return launch_fp8_ts_for_k<256>(p, a_is_fp8, epilogue, s, name);
@@ -401,3 +510,96 @@ int launch_linear_fp8_ts(const void* a, int a_is_fp8, int64_t lda, const void* w
 }
 
 }  // namespace taac
+
+namespace taac {
+namespace {
+__global__ void fp8_ts_clear_kernel(float* a) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) *a = 0.f;
+}
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_norm_linear_fp8_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w_fp8,
+                                        const void* bias, const float* amax_x, const float* amax_w, const void* residual,
+                                        int64_t ldr, void* out, int64_t ldo, int64_t M, int32_t N, int32_t K,
+                                        const int32_t* rows, const int32_t* n_rows, const void* out_norm_weight,
+                                        float out_eps, float* amax_out, void* stream) {
+  using namespace taac;
+  const char* name = "taac_norm_linear_fp8_fwd";
+  if (M < 0 || N <= 0 || K <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, N and K > 0", name);
+  if (K != 256) return set_error(TAAC_ERR_UNSUPPORTED, "%s: built for K = 256 (got %d)", name, K);
+  if (N % 64 != 0) return set_error(TAAC_ERR_UNSUPPORTED, "%s: N=%d must be a multiple of 64", name, N);
+  if (ldx < K || ldo < N || (residual && ldr < N) || ldx % 8 || ldo % 8 || (residual && ldr % 8))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: row strides must cover a row and be multiples of 8", name);
+  if (!amax_x || !amax_w) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null scale pointer", name);
+  if ((rows == nullptr) != (n_rows == nullptr))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows and n_rows must be given together", name);
+  if (out_norm_weight && !amax_out) return set_error(TAAC_ERR_INVALID_VALUE, "%s: out_norm_weight without amax_out", name);
+  hipStream_t s = as_stream(stream);
+  if (amax_out != nullptr) {
+    hipLaunchKernelGGL(fp8_ts_clear_kernel, dim3(1), dim3(kWave), 0, s, amax_out);
+    const int rc = check_launch(name);
+    if (rc != TAAC_OK) return rc;
+  }
+  if (M == 0) return TAAC_OK;
+  if (!x || !w_fp8 || !out) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
+  if (M > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: at most 2^31 rows", name);
+  const void* ptrs[7] = {x, w_fp8, out, residual, bias, norm_weight, out_norm_weight};
+  for (const void* ptr : ptrs)
+    if (reinterpret_cast<uintptr_t>(ptr) & 15u)
+      return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
+  Fp8TsParams p{};
+  p.a = x;
+  p.w = static_cast<const uint8_t*>(w_fp8);
+  p.bias = static_cast<const bf16_t*>(bias);
+  p.residual = static_cast<const bf16_t*>(residual);
+  p.out = static_cast<bf16_t*>(out);
+  p.amax_a = amax_x;
+  p.amax_w = amax_w;
+  p.M = M;
+  p.lda = ldx;
+  p.ldo = ldo;
+  p.ldr = ldr;
+  p.N = N;
+  p.norm_w = static_cast<const bf16_t*>(norm_weight);
+  p.eps = eps;
+  p.rows = rows;
+  p.n_rows = n_rows;
+  p.amax_out = amax_out;
+  p.out_norm_w = static_cast<const bf16_t*>(out_norm_weight);
+  p.out_eps = out_eps;
+  const int epilogue = residual ? TAAC_EPI_RESIDUAL : TAAC_EPI_NONE;
+  const size_t lds_bytes = static_cast<size_t>(3 * step_bytes(256)) + static_cast<size_t>(kWaves) * 32 * tile_row_bytes(256) +
+                           static_cast<size_t>(2 * N + 256) * 2 + 64;
+  if (lds_bytes > 160 * 1024) return set_error(TAAC_ERR_UNSUPPORTED, "%s: N=%d does not fit the LDS", name, N);
+  const int tok_per_wg = kWaves * 32 * tiles_per_wave(256, epilogue);
+  const int64_t tiles64 = (M + tok_per_wg - 1) / tok_per_wg;
+  const int num_tiles = static_cast<int>(tiles64);
+  const int cus = compute_units();
+  if (cus <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
+  int grid = num_tiles < cus ? num_tiles : cus;
+  if (const char* cap = getenv("TAAC_TS_MAX_WORKGROUPS")) {  // test hook, as in taac_linear_fp8
+    const int limit = atoi(cap);
+    if (limit > 0 && limit < grid) grid = limit;
+  }
+#define TAAC_NL_FP8(EPI, ST, NM)                                                                                          \
+  do {                                                                                                                    \
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(linear_fp8_ts_kernel<256, EPI, false, ST, NM>),                 \
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)) != hipSuccess)       \
+      return set_error(TAAC_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", name, lds_bytes);                          \
+    hipLaunchKernelGGL((linear_fp8_ts_kernel<256, EPI, false, ST, NM>), dim3(grid), dim3(kWaves * kWave), lds_bytes, s, p, \
+                       num_tiles);                                                                                        \
+    return check_launch(name);                                                                                            \
+  } while (0)
+#define TAAC_NL_FP8_EPI(EPI)                              \
+  do {                                                    \
+    if (amax_out && norm_weight) TAAC_NL_FP8(EPI, true, true);   \
+    if (amax_out) TAAC_NL_FP8(EPI, true, false);          \
+    if (norm_weight) TAAC_NL_FP8(EPI, false, true);       \
+    TAAC_NL_FP8(EPI, false, false);                       \
+  } while (0)
+  if (residual) TAAC_NL_FP8_EPI(TAAC_EPI_RESIDUAL);
+  TAAC_NL_FP8_EPI(TAAC_EPI_NONE);
+#undef TAAC_NL_FP8_EPI
+#undef TAAC_NL_FP8
+}

@@ -7,7 +7,8 @@ import pytest
 import torch
 
 from oracle import reference as oracle
-from taac_2026_amd.api import amax, pack_ffn_weights_fp8, rms_norm, swiglu_ffn_fp8, valid_rows
+from taac_2026_amd.api import (amax, linear_fp8, norm_linear_fp8, pack_ffn_weights_fp8, quantize_fp8, rms_norm,
+                               swiglu_ffn_fp8, valid_rows)
 
 pytestmark = pytest.mark.gpu
 
@@ -112,3 +113,49 @@ def test_fused_fp8_ffn_errors(device):
                              torch.zeros(256, 48, dtype=torch.bfloat16, device=device))
     with pytest.raises(RuntimeError, match="same device|CUDA"):
         swiglu_ffn_fp8(x, packed, None, None, amax(xd), hidden_size=64)
+
+
+@pytest.mark.parametrize("workgroups", [None, 2])
+@pytest.mark.parametrize("n,with_norm,with_residual", [(768, True, False), (256, False, True), (256, True, True), (64, False, False)])
+def test_norm_linear_fp8_fuses_norm_rows_and_the_next_scale(device, monkeypatch, n, with_norm, with_residual, workgroups):
+    """RMSNorm -> quantise -> e4m3 product -> (+ residual) in one kernel, over a row index, with the scale of the consuming
+    layer reduced in the epilogue; against the emulated layer on the normalised rows, and against the two-kernel route
+    (stand-alone norm, taac_linear_fp8), which computes the same thing."""
+    if workgroups is not None:
+        monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+    batch, tokens, k = 9, 150, 256
+    g = torch.Generator().manual_seed(n + with_norm)
+    bf = lambda t: t.to(torch.bfloat16)  # noqa: E731
+    x = bf(torch.randn(batch * tokens, k, generator=g) * (0.5 + torch.rand(batch * tokens, 1, generator=g)))
+    w = bf(torch.randn(n, k, generator=g) * k ** -0.5)
+    b = bf(0.1 * torch.randn(n, generator=g))
+    norm_w = bf(1 + 0.1 * torch.randn(k, generator=g))
+    next_w = bf(1 + 0.2 * torch.randn(n, generator=g))
+    res = bf(torch.randn(batch * tokens, n, generator=g)) if with_residual else None
+    lengths = torch.tensor([150, 0, 1, 77, 149, 150, 3, 64, 100], dtype=torch.int32)
+    valid = (torch.arange(tokens)[None, :] < lengths[:, None]).flatten()
+    h = oracle.rms_norm_fp32(x[valid], norm_w) if with_norm else x[valid]
+    want = oracle.linear_fp8(h, w, b, residual=None if res is None else res[valid])
+    poisoned = x.clone()
+    poisoned[~valid] = float("nan")
+    xd, wd, bd, nw, nxt = _to(device, poisoned, w, b, norm_w, next_w)
+    resd = None if res is None else res.to(device)
+    with torch.no_grad():
+        index = valid_rows(lengths.to(device), tokens)
+        wq, wa = quantize_fp8(wd)
+        h_dev = rms_norm(x[valid].to(device), nw) if with_norm else x[valid].to(device)
+        ax = amax(h_dev)
+        out = torch.full((batch * tokens, n), float("nan"), dtype=torch.bfloat16, device=device)
+        got, amax_out = norm_linear_fp8(xd, wq, ax, wa, bd, norm_weight=nw if with_norm else None, residual=resd,
+                                        token_rows=index, out=out, out_norm_weight=nxt)
+        plain, amax_plain = norm_linear_fp8(xd, wq, ax, wa, bd, norm_weight=nw if with_norm else None, residual=resd,
+                                            token_rows=index, out=out.clone(), want_amax_out=True)
+        two_kernels = linear_fp8(h_dev, wq, ax, wa, bd, residual=None if resd is None else resd[valid.to(device)])
+    got = got.cpu()
+    assert torch.isnan(got[~valid].float()).all()
+    assert _rel(got[valid], want) <= 5e-2
+    assert torch.equal(got[valid], two_kernels.cpu())
+    assert torch.equal(plain.cpu()[valid], got[valid])
+    assert amax_plain.item() == got[valid].float().abs().max().item()
+    expected_next = rms_norm(got[valid].to(device), nxt).float().abs().max().item()
+    assert abs(amax_out.item() - expected_next) <= 2 ** -7 * expected_next
