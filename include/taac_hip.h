@@ -56,6 +56,8 @@ enum taac_epilogue {
 /* Bits of the `flags` argument of taac_backbone_fwd. */
 #define TAAC_BACKBONE_DENSE_TOKENS 1  /* run the dense layers over the padded positions too                        */
 #define TAAC_BACKBONE_SPLIT_OUT_FFN 2 /* out projection and feed-forward half as two kernels instead of one        */
+#define TAAC_BACKBONE_FP8 4           /* the four dense layers of a block with e4m3 MFMA operands and per-tensor   */
+                                      /* scales (amax / 448); D = 256, F a multiple of 64, plain attention layer   */
 
 int taac_abi_version(void);
 const char* taac_last_error(void);
@@ -152,6 +154,18 @@ int taac_flash_attn_scaled_fwd(const void* q, const void* k, const void* v, cons
                                int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
                                const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4],
                                int is_causal, int zero_padded_queries, int dtype, void* stream);
+
+/*
+ * taac_flash_attn_scaled_fwd that also reduces max |o| over everything it writes into *amax_out (device float, cleared
+ * by the call): the per-tensor FP8 scale of the output projection that consumes o, taken in the kernel's epilogue
+ * instead of in a pass of its own. Padded query rows that are not written (zero_padded_queries = 2) do not count.
+ * No counterpart in the reference (it has no FP8 code).
+ */
+int taac_flash_attn_amax_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
+                             const float* q_row_scale, const float* k_row_scale, const float* q_col_scale, void* o,
+                             float* amax_out, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                             const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
+                             const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype, void* stream);
 
 /*
  * Attention under a structured mask: key j is visible to query i of sample b iff
@@ -468,13 +482,15 @@ int taac_norm_linear_fp8_fwd(const void* x, int64_t ldx, const void* norm_weight
  * Fused feed-forward half with FP8 (e4m3fn) MFMA operands and per-tensor scales, the FP8 counterpart of
  * taac_swiglu_ffn_fwd: the chain of two taac_linear_fp8 layers
  *   h   = norm_weight ? bf16(rmsnorm(x, norm_weight, eps)) : x
- *   hid = bf16( silu(g) * u ),  g, u = chunk2( (q(h) q(w_up)^T) (amax_x / 448)(amax_up / 448) + b_up )
+ *   hid = silu(g) * u,  g, u = chunk2( (q(h) q(w_up)^T) (amax_x / 448)(amax_up / 448) + b_up )      (kept in fp32)
  *   out = bf16( (q(hid) q(w_down)^T) (amax_hidden / 448)(amax_down / 448) + b_down + residual )
  * with q(t) = sat(t / (amax_t / 448)) in e4m3 and amax_hidden = max |hid| over all tokens, which the call computes
  * itself: a first launch evaluates the up projection and the gate only to reduce max |hid| into *amax_hidden, a second
- * launch evaluates the whole layer with that scale. The [M, F] hidden state is never written to memory.
+ * launch evaluates the whole layer with that scale. The [M, F] hidden state is never written to memory, so it is
+ * quantised from fp32 (the chain of two separate layers rounds it to bf16 in between: a difference of at most one bf16
+ * step before a quantisation to three mantissa bits).
  * packed_weights: blob of taac_ffn_fp8_pack_weights (both weights quantised with their amax and laid out in fragment
- * order; 3 * D * F bytes, taac_ffn_fp8_packed_bytes). amax_x: device float, max |h| over the tokens (of the normalised
+ * order; 3 * D * F + 64 * D bytes, taac_ffn_fp8_packed_bytes). amax_x: device float, max |h| over the tokens (of the normalised
  * input when norm_weight is given: taac_amax of it, or the amax_next / amax_out of the producing call). amax_up /
  * amax_down: the amax the weights were packed with. amax_hidden: device float, written. x, residual, out, rows / n_rows,
  * gate_first: as in taac_swiglu_ffn_fwd (out may alias residual and x). D: 128 or 256, F a multiple of 64.
@@ -542,6 +558,13 @@ typedef struct taac_block_weights {
  * plus, for the fused path, one fragment-ordered copy of every block's weights (repacked on each call). */
 int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D, int32_t F, int32_t n_blocks);
 
+/* Byte offset, inside the workspace of taac_backbone_fwd, of the per-tensor maxima a TAAC_BACKBONE_FP8 call leaves
+ * behind: float [n_blocks + 1][8] = per block {|w_qkv|, |w_out|, |w_up|, |w_down|, |rmsnorm(x)|, |attention|,
+ * |rmsnorm(x1)|, |silu(gate) * value|} (scale = maximum / 448); the last row holds nothing. -1 when the shape has no
+ * FP8 mode. No counterpart in the reference (its FP8 layers keep the scales inside the layer); for calibration and
+ * tests. */
+int64_t taac_backbone_fp8_scales_offset(int32_t B, int32_t T, int32_t D, int32_t F, int32_t n_blocks);
+
 /*
  * Forward of n_blocks pre-norm blocks plus the pCVR readout:
  *   for each block: h = rmsnorm(x); q,k,v = chunk3(h Wqkv^T + b);
@@ -556,7 +579,10 @@ int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D, int32_t F
  * rope_cos_sin: [T, D / heads / 2, 2] bf16 table of (cos, sin) as in taac_qk_norm_rope_fwd, or NULL (no rotation);
  * the same eps serves every norm. flags: TAAC_BACKBONE_* bits, 0 for the default route (the dense layers skip the
  * padded positions; rows at or beyond key_lengths[b] of hidden_out are then zeros, with TAAC_BACKBONE_DENSE_TOKENS they
- * hold the values the dense formulation computes there; the readout never reads them).
+ * hold the values the dense formulation computes there; the readout never reads them). With TAAC_BACKBONE_FP8 every
+ * dense layer is the quantize -> matmul -> dequantize layer of taac_linear_fp8 (weights quantised per call; every
+ * activation scale is the exact per-tensor maximum, reduced in the epilogue of the kernel that produces the tensor:
+ * taac_norm_linear_fp8_fwd, taac_flash_attn_amax_fwd, taac_swiglu_ffn_fp8_fwd).
  * Replaces: the block loop _run_backbone (experiments/symbiosis/model.py:283-292) over UnifiedInteractionBlock
  * (experiments/symbiosis/backbone.py:50-68) in its canonical pre-norm form, plus masked_mean + Linear + sigmoid; with
  * the query / key norm weights UnifiedSelfAttention as the reference runs it (backbone.py:24-48), with the table

@@ -486,3 +486,43 @@ def swiglu_ffn_fp8(x: torch.Tensor, norm_weight: torch.Tensor | None, up_weight:
     hidden = linear_fp8(h, up_weight, up_bias, swiglu=True, gate_first=gate_first)
     out = linear_fp8(hidden, down_weight, down_bias, residual=residual)
     return out, hidden, h
+
+
+def block_fp8(x: torch.Tensor, key_lengths: torch.Tensor, w: dict[str, torch.Tensor], *, num_heads: int, eps: float = 1e-6,
+              valid_only: bool = False, maxima: dict[str, torch.Tensor] | None = None) -> torch.Tensor:
+    """``block`` with its four dense layers replaced by ``linear_fp8`` (qkv, out, up, down; the recipe of
+    experiments/symbiosis/backbone.py:58-68, plain attention layer). ``valid_only=True`` takes every activation scale
+    over the rows before ``key_lengths`` only, which is what a route that never touches the padded positions computes;
+    the padded rows of the result are then don't-care. ``maxima`` fixes the per-tensor maxima of the four activations
+    (keys "attn_norm", "attention", "ffn_norm", "hidden") instead of taking them from ``x`` - for a slice of a batch
+    whose scales were taken over the whole batch. Parity unpinned like ``linear_fp8``; composed from it only."""
+    keep = ~make_padding_mask(key_lengths.to(torch.int64), x.shape[1])
+
+    def scale_of(name: str, t: torch.Tensor) -> torch.Tensor | None:
+        if maxima is not None:
+            return maxima[name].float().clamp_min(1e-12) / FP8_MAX
+        return fp8_scale(t[keep]) if valid_only else None
+
+    h = rms_norm_fp32(x, w["attn_norm.weight"], eps)
+    q, k, v = linear_fp8(h, w["qkv.weight"], w.get("qkv.bias"), x_scale=scale_of("attn_norm", h)).chunk(3, dim=-1)
+    a = scaled_dot_product_attention(q, k, v, num_heads=num_heads, key_lengths=key_lengths, zero_padded_queries=True)
+    x = linear_fp8(a, w["out.weight"], w.get("out.bias"), residual=x, x_scale=scale_of("attention", a))
+    h2 = rms_norm_fp32(x, w["ffn_norm.weight"], eps)
+    hidden = linear_fp8(h2, w["up.weight"], w.get("up.bias"), swiglu=True, x_scale=scale_of("ffn_norm", h2))
+    return linear_fp8(hidden, w["down.weight"], w.get("down.bias"), residual=x, x_scale=scale_of("hidden", hidden))
+
+
+def backbone_fp8(emb: torch.Tensor, key_lengths: torch.Tensor, blocks: list[dict[str, torch.Tensor]],
+                 head_weight: torch.Tensor, head_bias: torch.Tensor | None, *, num_heads: int, eps: float = 1e-6,
+                 return_hidden: bool = False, valid_only: bool = False,
+                 maxima: list[dict[str, torch.Tensor]] | None = None):
+    """``backbone`` over ``block_fp8``; the pooled readout stays in the activation dtype."""
+    x = emb
+    for index, w in enumerate(blocks):
+        x = block_fp8(x, key_lengths, w, num_heads=num_heads, eps=eps, valid_only=valid_only,
+                      maxima=None if maxima is None else maxima[index])
+    padding = make_padding_mask(key_lengths.to(torch.int64), x.shape[1])
+    pooled = masked_mean(x, padding)
+    logits = F.linear(pooled, head_weight.reshape(1, -1), head_bias).squeeze(-1)
+    probs = torch.sigmoid(logits.float())
+    return (probs, x) if return_hidden else probs

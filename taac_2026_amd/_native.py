@@ -22,7 +22,7 @@ TAAC_ERR_LAUNCH = -3
 TAAC_F32, TAAC_BF16, TAAC_F16 = 0, 1, 2
 EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
 ATTN_CAUSAL, ATTN_REGISTER_STAGING = 1, 2
-BACKBONE_DENSE_TOKENS, BACKBONE_SPLIT_OUT_FFN = 1, 2
+BACKBONE_DENSE_TOKENS, BACKBONE_SPLIT_OUT_FFN, BACKBONE_FP8 = 1, 2, 4
 
 ABI_VERSION = 5
 
@@ -88,6 +88,13 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32,
          c_int32]
+        + [ctypes.POINTER(c_int64)] * 4
+        + [c_int, c_int, c_int, c_void_p],
+    ),
+    "taac_flash_attn_amax_fwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32,
+         c_int32, c_int32]
         + [ctypes.POINTER(c_int64)] * 4
         + [c_int, c_int, c_int, c_void_p],
     ),
@@ -171,6 +178,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p],
     ),
     "taac_backbone_workspace_bytes": (c_int64, [c_int32, c_int32, c_int32, c_int32, c_int32]),
+    "taac_backbone_fp8_scales_offset": (c_int64, [c_int32, c_int32, c_int32, c_int32, c_int32]),
     "taac_norm_linear_fp8_fwd": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,

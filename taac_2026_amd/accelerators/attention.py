@@ -325,6 +325,7 @@ def hip_flash_attention_kernel(
     q_col_scale: torch.Tensor | None = None,
     structured_mask: StructuredAttentionMask | None = None,
     kv_staging: str = "direct",
+    amax_out: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """``(q, k, v: (B, H, T, d) bf16/fp16, key_lengths: int32[B]) -> (B, H, Tq, d)``.
 
@@ -336,7 +337,8 @@ def hip_flash_attention_kernel(
     optional fp32 factors of the query features (the product of a query and a key norm weight). ``structured_mask``:
     a :class:`StructuredAttentionMask` (excludes ``is_causal``; combines with ``key_lengths``). ``kv_staging``:
     ``"direct"`` (K / V chunks go from global memory straight into LDS) or ``"registers"`` (the general kernel; same
-    results, kept as a comparison route).
+    results, kept as a comparison route). ``amax_out``: a float32 scalar tensor that receives ``max |output|`` over the rows
+    the kernel writes (the FP8 scale of the layer that consumes the output; not with a structured mask).
     """
     library = _native.load_library()
     require_cuda_tensors("hip flash_attention", q, k, v, key_lengths)
@@ -363,6 +365,8 @@ def hip_flash_attention_kernel(
         if q_col_scale.dtype != torch.float32 or q_col_scale.numel() != heads * head_dim or not q_col_scale.is_contiguous():
             raise ValueError("flash_attention q_col_scale must be a contiguous float32 tensor of heads * head_dim values")
     if structured_mask is not None:
+        if amax_out is not None:
+            raise ValueError("flash_attention: amax_out is not available under a structured mask")
         if is_causal:
             raise ValueError("flash_attention: a structured mask carries its own causal triangle (is_causal must be False)")
         sm = structured_mask
@@ -379,6 +383,21 @@ def hip_flash_attention_kernel(
             batch, heads, query_len, k.shape[2], head_dim,
             _native.Int64x4(*q.stride()), _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()),
             _native.Int64x4(*out.stride()), int(zero_padded_queries), _native.dtype_code(q.dtype),
+            _native.current_stream(q.device),
+        )
+        _native.check(status, "flash_attention")
+        return out
+    if amax_out is not None:
+        require_cuda_tensors("hip flash_attention", amax_out)
+        if amax_out.dtype != torch.float32 or amax_out.numel() != 1:
+            raise ValueError("flash_attention amax_out must be a float32 scalar tensor")
+        status = library.taac_flash_attn_amax_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), _native.ptr(q_row_scale),
+            _native.ptr(k_row_scale), _native.ptr(q_col_scale), out.data_ptr(), amax_out.data_ptr(),
+            batch, heads, query_len, k.shape[2], head_dim,
+            _native.Int64x4(*q.stride()), _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()),
+            _native.Int64x4(*out.stride()),
+            _mask_flags(is_causal, kv_staging), int(zero_padded_queries), _native.dtype_code(q.dtype),
             _native.current_stream(q.device),
         )
         _native.check(status, "flash_attention")

@@ -43,6 +43,7 @@ struct AttnParams {
   const float* q_row_scale;  // [B, Tq] / [B, Tk] factors of the query / key rows (shared by the heads), or null
   const float* k_row_scale;
   const float* q_col_scale;  // [H, d] factors of the query features, or null
+  float* amax_out;           // receives max |o| over everything written (atomic max), or null
   // Structured mask: key j is visible to query i of sample b iff bit j of struct_bits[i] and of valid_bits[b] is set.
   const uint32_t* struct_bits;  // [Tq][wpr] words, bit j % 32 of word j / 32; null: no structured mask
   int64_t struct_stride;        // words between the matrices of consecutive samples; 0: one matrix for the batch
@@ -459,6 +460,7 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
         (qi < q_valid && l_run > 0.f) ? (m_run * c + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f : -INFINITY;
   __syncthreads();  // every wavefront is done with sK / sV: the buffer now holds the output tiles
   uint8_t* tile = smem + wave * (32 * OROW);
+  float omax = 0.f;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
@@ -467,7 +469,18 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
 #pragma unroll
       for (int e = 0; e < 4; ++e) ov[e] = static_cast<T>(oacc[mb][jq * 4 + e] * fin);
       *reinterpret_cast<vec4_t*>(tile + l32 * OROW + (mb * 32 + jq * 8 + hh * 4) * 2) = ov;
+      if (p.amax_out != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) omax = fmaxf(omax, fabsf(static_cast<float>(ov[e])));
+      }
     }
+  }
+  if (p.amax_out != nullptr) {
+    // per-tensor scale of the layer that consumes the output (FP8 dense layers): one atomic per wavefront on the float's
+    // bit pattern, skipped when the published value already covers it
+    omax = group_max<kWave>(omax);
+    if (lane == 0 && omax > __builtin_nontemporal_load(p.amax_out))
+      atomicMax(reinterpret_cast<unsigned int*>(p.amax_out), __float_as_uint(omax));
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   constexpr int RPP = kWave / C8;  // rows per pass: C8 lanes cover one row
@@ -797,6 +810,7 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
         (qi < q_valid && l_run > 0.f) ? (m_run * c + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f : -INFINITY;
   __syncthreads();  // every wavefront is done with the chunk buffers: they now hold the output tiles
   uint8_t* tile = smem + wave * (32 * OROW);
+  float omax = 0.f;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
@@ -805,7 +819,18 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
 #pragma unroll
       for (int e = 0; e < 4; ++e) ov[e] = static_cast<T>(oacc[mb][jq * 4 + e] * fin);
       *reinterpret_cast<vec4_t*>(tile + l32 * OROW + (mb * 32 + jq * 8 + hh * 4) * 2) = ov;
+      if (p.amax_out != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) omax = fmaxf(omax, fabsf(static_cast<float>(ov[e])));
+      }
     }
+  }
+  if (p.amax_out != nullptr) {
+    // per-tensor scale of the layer that consumes the output (FP8 dense layers): one atomic per wavefront on the float's
+    // bit pattern, skipped when the published value already covers it
+    omax = group_max<kWave>(omax);
+    if (lane == 0 && omax > __builtin_nontemporal_load(p.amax_out))
+      atomicMax(reinterpret_cast<unsigned int*>(p.amax_out), __float_as_uint(omax));
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   constexpr int RPP = kWave / C8;
@@ -916,7 +941,7 @@ struct MaskArgs {
 
 int attention_entry(const char* name, const void* q, const void* k, const void* v, const int32_t* key_lengths,
                     const MaskArgs& mask, const float* q_row_scale, const float* k_row_scale, const float* q_col_scale,
-                    float* lse, void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
+                    float* lse, float* amax_out, void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
                     const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4], int mask_flags,
                     int zero_padded_queries, int dtype, void* stream) {
   if (mask_flags & ~(TAAC_ATTN_CAUSAL | TAAC_ATTN_REGISTER_STAGING))
@@ -963,6 +988,7 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   p.q_row_scale = q_row_scale;
   p.k_row_scale = k_row_scale;
   p.q_col_scale = q_col_scale;
+  p.amax_out = amax_out;
   p.lse = lse;
   p.struct_bits = mask.struct_bits;
   p.struct_stride = mask.struct_stride;
@@ -1006,7 +1032,7 @@ extern "C" int taac_flash_attn_fwd(const void* q, const void* k, const void* v, 
                                    const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype,
                                    void* stream) {
   return taac::attention_entry("taac_flash_attn_fwd", q, k, v, key_lengths, taac::MaskArgs{}, nullptr, nullptr, nullptr,
-                               nullptr, o, B, H, Tq, Tk, d,
+                               nullptr, nullptr, o, B, H, Tq, Tk, d,
                                q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries, dtype, stream);
 }
 
@@ -1018,8 +1044,31 @@ extern "C" int taac_flash_attn_scaled_fwd(const void* q, const void* k, const vo
                                           const int64_t o_strides[4], int is_causal, int zero_padded_queries, int dtype,
                                           void* stream) {
   return taac::attention_entry("taac_flash_attn_scaled_fwd", q, k, v, key_lengths, taac::MaskArgs{}, q_row_scale,
-                               k_row_scale, q_col_scale, nullptr, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries,
-                               dtype, stream);
+                               k_row_scale, q_col_scale, nullptr, nullptr, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides,
+                               o_strides, is_causal, zero_padded_queries, dtype, stream);
+}
+
+namespace taac {
+namespace {
+__global__ void attn_clear_kernel(float* a) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) *a = 0.f;
+}
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_flash_attn_amax_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
+                                        const float* q_row_scale, const float* k_row_scale, const float* q_col_scale,
+                                        void* o, float* amax_out, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                                        const int64_t q_strides[4], const int64_t k_strides[4],
+                                        const int64_t v_strides[4], const int64_t o_strides[4], int is_causal,
+                                        int zero_padded_queries, int dtype, void* stream) {
+  if (!amax_out) return taac::set_error(TAAC_ERR_INVALID_VALUE, "taac_flash_attn_amax_fwd: amax_out must be given");
+  hipLaunchKernelGGL(taac::attn_clear_kernel, dim3(1), dim3(taac::kWave), 0, taac::as_stream(stream), amax_out);
+  const int rc = taac::check_launch("taac_flash_attn_amax_fwd");
+  if (rc != TAAC_OK) return rc;
+  return taac::attention_entry("taac_flash_attn_amax_fwd", q, k, v, key_lengths, taac::MaskArgs{}, q_row_scale,
+                               k_row_scale, q_col_scale, nullptr, amax_out, o, B, H, Tq, Tk, d, q_strides, k_strides,
+                               v_strides, o_strides, is_causal, zero_padded_queries, dtype, stream);
 }
 
 extern "C" int taac_flash_attn_masked_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
@@ -1040,8 +1089,8 @@ extern "C" int taac_flash_attn_masked_fwd(const void* q, const void* k, const vo
   mask.valid_bits = valid_bits;
   mask.self_bits = self_bits;
   return taac::attention_entry("taac_flash_attn_masked_fwd", q, k, v, key_lengths, mask, q_row_scale, k_row_scale,
-                               q_col_scale, nullptr, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, 0,
-                               zero_padded_queries, dtype, stream);
+                               q_col_scale, nullptr, nullptr, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides,
+                               0, zero_padded_queries, dtype, stream);
 }
 
 extern "C" int taac_mask_pack_bits(const void* mask, int64_t rows, int32_t cols, uint32_t* bits, void* stream) {
@@ -1077,6 +1126,6 @@ extern "C" int taac_flash_attn_train_fwd(const void* q, const void* k, const voi
                                          int zero_padded_queries, int dtype, void* stream) {
   if (!lse) return taac::set_error(TAAC_ERR_INVALID_VALUE, "taac_flash_attn_train_fwd: lse must be given");
   return taac::attention_entry("taac_flash_attn_train_fwd", q, k, v, key_lengths, taac::MaskArgs{}, nullptr, nullptr,
-                               nullptr, lse, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, is_causal,
-                               zero_padded_queries, dtype, stream);
+                               nullptr, lse, nullptr, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides,
+                               is_causal, zero_padded_queries, dtype, stream);
 }

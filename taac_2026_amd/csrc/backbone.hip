@@ -292,6 +292,17 @@ inline int64_t packed_block_bytes(int32_t D, int32_t F) {
 inline int64_t qk_norm_bytes(int64_t M, int32_t D) {
   return align256((2 * D / 64) * M * 4) + align256(2 * M * 4) + align256(static_cast<int64_t>(D) * 4);
 }
+// FP8 mode (TAAC_BACKBONE_FP8; D = 256, F a multiple of 64): per block the e4m3 qkv / out weights, the packed feed-forward
+// blob and 8 scales (weights: qkv, out, up, down; activations: block input, attention output, feed-forward input, gated
+// hidden state); one more set of scales behind the last block.
+inline bool fp8_shape(int32_t D, int32_t F) { return D == 256 && F % 64 == 0; }
+inline int64_t fp8_block_bytes(int32_t D, int32_t F) {
+  return align256(static_cast<int64_t>(3) * D * D) + align256(static_cast<int64_t>(D) * D) +
+         align256(taac_ffn_fp8_packed_bytes(D, F));
+}
+inline int64_t fp8_bytes(int32_t D, int32_t F, int32_t n_blocks) {
+  return fp8_shape(D, F) ? n_blocks * fp8_block_bytes(D, F) + align256((n_blocks + 1) * 8 * 4) : 0;
+}
 }  // namespace
 }  // namespace taac
 
@@ -302,8 +313,15 @@ extern "C" int64_t taac_backbone_workspace_bytes(int32_t B, int32_t T, int32_t D
   // x, h (shared with the attention output), qkv, then either the packed weights + the valid-row index (fused path)
   // or the gated hidden state
   const int64_t acts = align256(M * D * 2) * 2 + align256(M * 3 * D * 2);
-  return acts + (fused_shape(D, F) ? n_blocks * packed_block_bytes(D, F) + row_index_bytes(B, T) + qk_norm_bytes(M, D)
+  return acts + (fused_shape(D, F) ? n_blocks * packed_block_bytes(D, F) + row_index_bytes(B, T) + qk_norm_bytes(M, D) +
+                                         fp8_bytes(D, F, n_blocks)
                                    : align256(M * F * 2));
+}
+
+extern "C" int64_t taac_backbone_fp8_scales_offset(int32_t B, int32_t T, int32_t D, int32_t F, int32_t n_blocks) {
+  using namespace taac;
+  if (B < 0 || T < 0 || n_blocks < 0 || !fp8_shape(D, F)) return -1;
+  return taac_backbone_workspace_bytes(B, T, D, F, n_blocks) - align256((n_blocks + 1) * 8 * 4);
 }
 
 extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, const taac_block_weights* blocks,
@@ -313,8 +331,13 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
                                  void* stream) {
   using namespace taac;
   const char* name = "taac_backbone_fwd";
-  if (flags & ~(TAAC_BACKBONE_DENSE_TOKENS | TAAC_BACKBONE_SPLIT_OUT_FFN))
+  if (flags & ~(TAAC_BACKBONE_DENSE_TOKENS | TAAC_BACKBONE_SPLIT_OUT_FFN | TAAC_BACKBONE_FP8))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: unknown flag bits (%d)", name, flags);
+  const bool fp8 = (flags & TAAC_BACKBONE_FP8) != 0;
+  if (fp8 && !fp8_shape(D, F))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: the FP8 dense layers are built for D = 256 and F a multiple of 64", name);
+  if (fp8 && rope_cos_sin != nullptr)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: the FP8 mode covers the plain attention layer (no rotary embedding)", name);
   if (B < 0 || T < 0 || D <= 0 || F <= 0 || heads <= 0 || n_blocks < 0)
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: bad dimensions", name);
   if (D % heads != 0 || (D / heads) % 8 != 0 || D / heads > 128)
@@ -365,7 +388,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
   int rc;
   // TAAC_BACKBONE_SPLIT_OUT_FFN: the out projection and the feed-forward half as two kernels (comparison route).
   const bool split_out_ffn = (flags & TAAC_BACKBONE_SPLIT_OUT_FFN) != 0;
-  if (fused && n_blocks > 0) {
+  if (fused && !fp8 && n_blocks > 0) {
     // One launch re-lays the weights of all blocks into fragment order.
     std::vector<void*> pk(3 * static_cast<size_t>(n_blocks));
     for (int i = 0; i < n_blocks; ++i) {
@@ -381,12 +404,60 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
                                    as_stream(stream), name)) != TAAC_OK)
       return rc;
   }
+  // FP8 mode: scales and e4m3 weights of all blocks (three launches), then the scale of the first block's input
+  char* fp8_base = reinterpret_cast<char*>(qk_weight) + align256(static_cast<int64_t>(D) * 4);
+  float* fp8_scales = reinterpret_cast<float*>(fp8_base + static_cast<int64_t>(n_blocks) * (fp8 ? fp8_block_bytes(D, F) : 0));
+  auto fp8_qkv = [&](int i) { return fp8_base + static_cast<int64_t>(i) * fp8_block_bytes(D, F); };
+  auto fp8_out = [&](int i) { return fp8_qkv(i) + align256(static_cast<int64_t>(3) * D * D); };
+  auto fp8_ffn = [&](int i) { return fp8_out(i) + align256(static_cast<int64_t>(D) * D); };
+  if (fp8 && n_blocks > 0) {
+    std::vector<float*> sc(n_blocks);
+    std::vector<void*> wq(3 * static_cast<size_t>(n_blocks));
+    for (int i = 0; i < n_blocks; ++i) {
+      if (blocks[i].query_norm_weight || blocks[i].key_norm_weight)
+        return set_error(TAAC_ERR_UNSUPPORTED, "%s: the FP8 mode covers the plain attention layer (no query / key norm)", name);
+      if (!blocks[i].attn_norm_weight || !blocks[i].ffn_norm_weight)
+        return set_error(TAAC_ERR_INVALID_VALUE, "%s: block %d has a null weight", name, i);
+      sc[i] = fp8_scales + 8 * i;
+      wq[i] = fp8_qkv(i);
+      wq[n_blocks + i] = fp8_out(i);
+      wq[2 * n_blocks + i] = fp8_ffn(i);
+    }
+    if ((rc = prepare_backbone_fp8(blocks, n_blocks, D, F, sc.data(), wq.data(), wq.data() + n_blocks,
+                                   wq.data() + 2 * n_blocks, as_stream(stream), name)) != TAAC_OK)
+      return rc;
+    if ((rc = rmsnorm_amax_256(emb, D, blocks[0].attn_norm_weight, eps, M, rows, n_rows, fp8_scales + 4, as_stream(stream),
+                               name)) != TAAC_OK)
+      return rc;
+  }
   for (int i = 0; i < n_blocks; ++i) {
     const taac_block_weights& w = blocks[i];
     if (!w.attn_norm_weight || !w.qkv_weight || !w.out_weight || !w.ffn_norm_weight || !w.up_weight || !w.down_weight)
       return set_error(TAAC_ERR_INVALID_VALUE, "%s: block %d has a null weight", name, i);
     const bool last = (i == n_blocks - 1);
     bf16_t* x_out = (last && hidden_out != nullptr) ? static_cast<bf16_t*>(hidden_out) : x;
+    if (fp8) {
+      // Four dense layers with e4m3 operands and per-tensor scales; every activation scale comes out of the epilogue of the
+      // kernel that produces the tensor (scales[4..7] = block input, attention output, feed-forward input, hidden state).
+      float* sc = fp8_scales + 8 * i;
+      if ((rc = taac_norm_linear_fp8_fwd(cur, D, w.attn_norm_weight, eps, fp8_qkv(i), w.qkv_bias, sc + 4, sc + 0, nullptr, 0,
+                                         qkv, 3 * D, M, 3 * D, D, rows, n_rows, nullptr, 0.f, nullptr, stream)) != TAAC_OK)
+        return rc;
+      if ((rc = taac_flash_attn_amax_fwd(qkv, qkv + D, qkv + 2 * D, key_lengths, nullptr, nullptr, nullptr, h, sc + 5, B,
+                                         heads, T, T, D / heads, qkv_strides, qkv_strides, qkv_strides, o_strides, 0,
+                                         rows ? 2 : 1, TAAC_BF16, stream)) != TAAC_OK)
+        return rc;
+      if ((rc = taac_norm_linear_fp8_fwd(h, D, nullptr, eps, fp8_out(i), w.out_bias, sc + 5, sc + 1, cur, D, x, D, M, D, D,
+                                         rows, n_rows, w.ffn_norm_weight, eps, sc + 6, stream)) != TAAC_OK)
+        return rc;
+      if ((rc = taac_swiglu_ffn_fp8_fwd(x, D, w.ffn_norm_weight, eps, fp8_ffn(i), w.up_bias, w.down_bias, sc + 6, sc + 2,
+                                        sc + 3, sc + 7, x, D, x_out, D, M, D, F, 1, rows, n_rows,
+                                        last ? nullptr : blocks[i + 1].attn_norm_weight, eps, last ? nullptr : sc + 8 + 4,
+                                        stream)) != TAAC_OK)
+        return rc;
+      cur = x_out;
+      continue;
+    }
     // Fused path: token-stationary kernels with norms and residuals fused, weights repacked into fragment order.
     char* pk_qkv = packed + static_cast<int64_t>(i) * packed_block_bytes(D, F);
     char* pk_out = pk_qkv + align256(static_cast<int64_t>(3) * D * D * 2);

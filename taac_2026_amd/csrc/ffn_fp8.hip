@@ -119,14 +119,12 @@ __device__ __forceinline__ uint32_t f8_quant4(const bf16_t* v, float scale) {
   return static_cast<uint32_t>(w);
 }
 
-__global__ __launch_bounds__(256) void ffn_fp8_pack_kernel(const bf16_t* __restrict__ w_up, const bf16_t* __restrict__ w_down,
-                                                           const float* __restrict__ amax_up,
-                                                           const float* __restrict__ amax_down, u32x4* __restrict__ packed,
-                                                           int D, int F, int gate_first) {
+__device__ __forceinline__ void ffn_fp8_pack_piece(const bf16_t* __restrict__ w_up, const bf16_t* __restrict__ w_down,
+                                                   const float* __restrict__ amax_up, const float* __restrict__ amax_down,
+                                                   u32x4* __restrict__ packed, int D, int F, int gate_first, int64_t gid) {
   const int KS = D / 64, MB = D / 32, DPS = MB / 4, SUBF = KS + DPS, NC = F / kF8Chunk;
   const int64_t stream_frags = static_cast<int64_t>(NC) * 4 * SUBF;
   const int64_t total = (stream_frags + MB) * 128;  // 16-byte pieces
-  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (gid >= total) return;
   const int lane = static_cast<int>(gid % 64);
   const int half = static_cast<int>((gid / 64) % 2);
@@ -167,6 +165,14 @@ __global__ __launch_bounds__(256) void ffn_fp8_pack_kernel(const bf16_t* __restr
   }
   const u32x4 q = {f8_quant4(v, scale), f8_quant4(v + 4, scale), f8_quant4(v + 8, scale), f8_quant4(v + 12, scale)};
   packed[gid] = q;
+}
+
+__global__ __launch_bounds__(256) void ffn_fp8_pack_kernel(const bf16_t* __restrict__ w_up, const bf16_t* __restrict__ w_down,
+                                                           const float* __restrict__ amax_up,
+                                                           const float* __restrict__ amax_down, u32x4* __restrict__ packed,
+                                                           int D, int F, int gate_first) {
+  ffn_fp8_pack_piece(w_up, w_down, amax_up, amax_down, packed, D, F, gate_first,
+                     static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x);
 }
 
 // ---- shared pieces ----------------------------------------------------------------------------------------------------
@@ -656,6 +662,157 @@ int f8_launch(K kernel, const FfnFp8Params& p, int waves, int tokens_per_wg, siz
 }
 
 }  // namespace
+}  // namespace taac
+
+namespace taac {
+namespace {
+
+// ---- FP8 preparation of a whole backbone: scales and quantised / packed weights of all blocks in three launches -------
+constexpr int kPrepBatch = 16;
+struct PrepBatch {
+  const bf16_t* w[kPrepBatch][4];   // qkv, out, up, down
+  uint8_t* qkv_q[kPrepBatch];
+  uint8_t* out_q[kPrepBatch];
+  u32x4* ffn_blob[kPrepBatch];
+  float* scales[kPrepBatch];        // 4 floats: amax of qkv, out, up, down
+};
+
+__global__ __launch_bounds__(256) void f8_fill_zero_kernel(float* a, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) a[i] = 0.f;
+}
+
+// blockIdx.y = block * 4 + tensor; grid-stride absolute maximum, one atomic per workgroup.
+__global__ __launch_bounds__(256) void f8_weights_amax_kernel(const PrepBatch batch, int D, int F) {
+  __shared__ float part[4];
+  const int blk = blockIdx.y / 4, which = blockIdx.y % 4;
+  const int64_t n = which == 0 ? static_cast<int64_t>(3) * D * D : (which == 1 ? static_cast<int64_t>(D) * D
+                                                                                : (which == 2 ? static_cast<int64_t>(2) * F * D
+                                                                                              : static_cast<int64_t>(D) * F));
+  const bf16x8* w = reinterpret_cast<const bf16x8*>(batch.w[blk][which]);
+  float m = 0.f;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n / 8;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const bf16x8 v = w[i];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) m = fmaxf(m, fabsf(static_cast<float>(v[e])));
+  }
+  m = group_max<kWave>(m);
+  if (threadIdx.x % kWave == 0) part[threadIdx.x / kWave] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    m = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+    atomicMax(reinterpret_cast<unsigned int*>(batch.scales[blk] + which), __float_as_uint(m));
+  }
+}
+
+// blockIdx.y = block; blockIdx.x walks 16-byte output pieces: the row-major e4m3 copies of qkv and out, then the FFN blob.
+__global__ __launch_bounds__(256) void f8_weights_quant_kernel(const PrepBatch batch, int D, int F) {
+  const int blk = blockIdx.y;
+  const int64_t n_qkv = static_cast<int64_t>(3) * D * D / 16, n_out = static_cast<int64_t>(D) * D / 16;
+  int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const float* scales = batch.scales[blk];
+  if (gid < n_qkv + n_out) {
+    const bool is_out = gid >= n_qkv;
+    const int64_t piece = is_out ? gid - n_qkv : gid;
+    const bf16_t* src = batch.w[blk][is_out ? 1 : 0] + piece * 16;
+    const float scale = fmaxf(scales[is_out ? 1 : 0], 1e-12f) / 448.0f;
+    bf16_t v[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) v[e] = src[e];
+    const u32x4 q = {f8_quant4(v, scale), f8_quant4(v + 4, scale), f8_quant4(v + 8, scale), f8_quant4(v + 12, scale)};
+    reinterpret_cast<u32x4*>(is_out ? batch.out_q[blk] : batch.qkv_q[blk])[piece] = q;
+    return;
+  }
+  gid -= n_qkv + n_out;
+  ffn_fp8_pack_piece(batch.w[blk][2], batch.w[blk][3], scales + 2, scales + 3, batch.ffn_blob[blk], D, F, 1, gid);
+}
+
+// max over the listed rows of | bf16(rmsnorm(x, w)) |: 32 lanes per row of 256 features (the scale of a block's first
+// dense layer when no producing kernel could deliver it: the embeddings come from outside).
+__global__ __launch_bounds__(256) void f8_norm_amax_kernel(const bf16_t* __restrict__ x, int64_t ldx,
+                                                           const bf16_t* __restrict__ w, float eps, int64_t M,
+                                                           const int32_t* __restrict__ rows,
+                                                           const int32_t* __restrict__ n_rows, float* __restrict__ out) {
+  __shared__ float part[4];
+  const int64_t count = rows != nullptr ? (static_cast<int64_t>(*n_rows) < M ? static_cast<int64_t>(*n_rows) : M) : M;
+  const int lane = threadIdx.x % 32;
+  float wf[8];
+  {
+    const bf16x8 wv = *reinterpret_cast<const bf16x8*>(w + lane * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) wf[e] = static_cast<float>(wv[e]);
+  }
+  float m = 0.f;
+  for (int64_t tok = static_cast<int64_t>(blockIdx.x) * 8 + threadIdx.x / 32; tok < count;
+       tok += static_cast<int64_t>(gridDim.x) * 8) {
+    const int64_t row = rows != nullptr ? static_cast<int64_t>(rows[tok]) : tok;
+    const bf16x8 v = *reinterpret_cast<const bf16x8*>(x + row * ldx + lane * 8);
+    float f[8], ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      f[e] = static_cast<float>(v[e]);
+      ss = fmaf(f[e], f[e], ss);
+    }
+    const float scale = rsqrtf(group_sum<32>(ss) * (1.0f / 256.0f) + eps);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) m = fmaxf(m, fabsf(static_cast<float>(static_cast<bf16_t>(f[e] * scale * wf[e]))));
+  }
+  m = group_max<kWave>(m);
+  if (threadIdx.x % kWave == 0) part[threadIdx.x / kWave] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    m = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+    if (m > __builtin_nontemporal_load(out)) atomicMax(reinterpret_cast<unsigned int*>(out), __float_as_uint(m));
+  }
+}
+
+}  // namespace
+
+// Scales (4 floats per block: qkv, out, up, down) and the e4m3 weights of n backbone blocks: row-major qkv / out copies and
+// the feed-forward blob (gate first). D = 256, F a multiple of 64.
+int prepare_backbone_fp8(const taac_block_weights* blocks, int n, int32_t D, int32_t F, float* const* scales,
+                         void* const* qkv_q, void* const* out_q, void* const* ffn_blob, hipStream_t s, const char* name) {
+  for (int base = 0; base < n; base += kPrepBatch) {
+    PrepBatch batch{};
+    const int m = n - base < kPrepBatch ? n - base : kPrepBatch;
+    for (int i = 0; i < m; ++i) {
+      const taac_block_weights& w = blocks[base + i];
+      const void* ptrs[4] = {w.qkv_weight, w.out_weight, w.up_weight, w.down_weight};
+      for (int t = 0; t < 4; ++t) {
+        if (!ptrs[t] || (reinterpret_cast<uintptr_t>(ptrs[t]) & 15u))
+          return set_error(TAAC_ERR_UNSUPPORTED, "%s: weights must be given and 16-byte aligned", name);
+        batch.w[i][t] = static_cast<const bf16_t*>(ptrs[t]);
+      }
+      batch.qkv_q[i] = static_cast<uint8_t*>(qkv_q[base + i]);
+      batch.out_q[i] = static_cast<uint8_t*>(out_q[base + i]);
+      batch.ffn_blob[i] = static_cast<u32x4*>(ffn_blob[base + i]);
+      batch.scales[i] = scales[base + i];
+      hipLaunchKernelGGL(f8_fill_zero_kernel, dim3(1), dim3(256), 0, s, scales[base + i], 4);
+    }
+    hipLaunchKernelGGL(f8_weights_amax_kernel, dim3(16, 4 * m), dim3(256), 0, s, batch, D, F);
+    const int64_t pieces = (static_cast<int64_t>(4) * D * D + taac_ffn_fp8_packed_bytes(D, F)) / 16;
+    hipLaunchKernelGGL(f8_weights_quant_kernel, dim3(static_cast<uint32_t>((pieces + 255) / 256), m), dim3(256), 0, s, batch,
+                       D, F);
+    const int rc = check_launch(name);
+    if (rc != TAAC_OK) return rc;
+  }
+  return TAAC_OK;
+}
+
+// *out = max over the (listed) rows of | bf16(rmsnorm(x, w, eps)) |, rows of 256 bf16 features.
+int rmsnorm_amax_256(const void* x, int64_t ldx, const void* w, float eps, int64_t M, const int32_t* rows,
+                     const int32_t* n_rows, float* out, hipStream_t s, const char* name) {
+  hipLaunchKernelGGL(f8_fill_zero_kernel, dim3(1), dim3(256), 0, s, out, 1);
+  if (M > 0) {
+    int64_t grid = (M + 7) / 8;
+    if (grid > 4096) grid = 4096;
+    hipLaunchKernelGGL(f8_norm_amax_kernel, dim3(static_cast<uint32_t>(grid)), dim3(256), 0, s, static_cast<const bf16_t*>(x),
+                       ldx, static_cast<const bf16_t*>(w), eps, M, rows, n_rows, out);
+  }
+  return check_launch(name);
+}
+
 }  // namespace taac
 
 extern "C" int64_t taac_ffn_fp8_packed_bytes(int32_t D, int32_t F) {

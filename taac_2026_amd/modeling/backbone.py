@@ -310,6 +310,8 @@ class PCVRBackbone(nn.Module):
     final hidden state (rows at or beyond ``key_lengths[b]`` are zeros). ``dense_tokens=True`` runs the dense layers over
     the padded positions too (what the reference's dense ``[B, T, D]`` formulation does; same valid rows, bit for bit),
     ``split_out_ffn=True`` runs the out projection and the feed-forward half as two kernels (comparison routes).
+    ``fp8=True`` runs the four dense layers of every block with e4m3 operands and per-tensor scales (d_model 256, plain
+    attention layer).
     ``qk_norm=True`` adds the reference layer's ``RMSNorm(d_model)`` of the query and the key
     (experiments/symbiosis/backbone.py:30-36), ``rope_base`` TokenFormer's rotary embedding of both over the token
     positions (experiments/tokenformer/model.py:165-192); the benchmark recipe has neither.
@@ -341,7 +343,7 @@ class PCVRBackbone(nn.Module):
         return ws
 
     def forward(self, emb: torch.Tensor, key_lengths: torch.Tensor, *, return_hidden: bool = False,
-                dense_tokens: bool = False, split_out_ffn: bool = False):
+                dense_tokens: bool = False, split_out_ffn: bool = False, fp8: bool = False):
         name = "hip PCVRBackbone"
         require_cuda_tensors(name, emb, key_lengths)
         require_inference(name, emb)
@@ -384,7 +386,8 @@ class PCVRBackbone(nn.Module):
         nbytes = library.taac_backbone_workspace_bytes(batch, tokens, self.d_model, self.d_ff, len(self.blocks))
         workspace = self._get_workspace(int(nbytes), emb.device)
         hidden = torch.empty_like(emb) if return_hidden else None
-        flags = (_native.BACKBONE_DENSE_TOKENS if dense_tokens else 0) | (_native.BACKBONE_SPLIT_OUT_FFN if split_out_ffn else 0)
+        flags = ((_native.BACKBONE_DENSE_TOKENS if dense_tokens else 0) | (_native.BACKBONE_SPLIT_OUT_FFN if split_out_ffn else 0)
+                 | (_native.BACKBONE_FP8 if fp8 else 0))
         probabilities = torch.empty(batch, dtype=torch.float32, device=emb.device)
         status = library.taac_backbone_fwd(
             emb.data_ptr(), key_lengths.data_ptr(), packed, len(self.blocks), dev(self.head.weight.reshape(-1)),
@@ -394,9 +397,25 @@ class PCVRBackbone(nn.Module):
             _native.current_stream(emb.device),
         )
         _native.check(status, "backbone_fwd")
+        self._fp8_maxima = None
+        if fp8:
+            offset = library.taac_backbone_fp8_scales_offset(batch, tokens, self.d_model, self.d_ff, len(self.blocks))
+            count = (len(self.blocks) + 1) * 8
+            self._fp8_maxima = workspace[offset:offset + 4 * count].view(torch.float32).view(-1, 8)
         if return_hidden:
             return probabilities, hidden
         return probabilities
+
+    FP8_MAXIMA = ("qkv.weight", "out.weight", "up.weight", "down.weight", "attn_norm", "attention", "ffn_norm", "hidden")
+
+    def fp8_maxima(self) -> list[dict[str, torch.Tensor]]:
+        """Per block, the per-tensor maxima (scale = maximum / 448) the last ``fp8=True`` forward quantised with: the four
+        weights, the two normalised streams, the attention output and the gated hidden state (host tensors; waits for
+        the forward)."""
+        if getattr(self, "_fp8_maxima", None) is None:
+            raise RuntimeError("hip PCVRBackbone: no fp8 forward has run on this module")
+        table = self._fp8_maxima[:len(self.blocks)].cpu()
+        return [dict(zip(self.FP8_MAXIMA, row)) for row in table]
 
 
 __all__ = [

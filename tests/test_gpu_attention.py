@@ -244,3 +244,24 @@ def test_direct_transfer_kernel_equals_general_kernel_bit_for_bit(device, dtype,
     general = run("registers")
     for a, b in zip(direct, general):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("head_dim,zero_pad", [(32, 2), (64, 1), (16, 0)])
+def test_attention_reduces_the_scale_of_its_output(device, head_dim, zero_pad):
+    """``amax_out`` receives max |o| over the rows the kernel writes (the FP8 scale of the layer behind it), from both
+    kernels (direct-transfer and general), with the output itself unchanged."""
+    from taac_2026_amd.accelerators.attention import hip_flash_attention_kernel
+
+    g = torch.Generator().manual_seed(head_dim)
+    batch, heads, tokens = 6, 3, 190
+    q, k, v = (torch.randn(batch, heads, tokens, head_dim, generator=g).to(torch.bfloat16).to(device) for _ in range(3))
+    lengths = torch.tensor([190, 1, 64, 65, 130, 17], dtype=torch.int32, device=device)
+    for staging in ("direct", "registers"):
+        amax = torch.full((), -1.0, dtype=torch.float32, device=device)
+        with torch.no_grad():
+            plain = hip_flash_attention_kernel(q, k, v, lengths, zero_padded_queries=zero_pad, kv_staging=staging)
+            got = hip_flash_attention_kernel(q, k, v, lengths, zero_padded_queries=zero_pad, kv_staging=staging, amax_out=amax)
+        valid = torch.arange(tokens, device=device)[None, :] < lengths[:, None]
+        rows = valid[:, None, :, None].expand_as(got) if zero_pad else torch.ones_like(got, dtype=torch.bool)
+        assert torch.equal(got[rows], plain[rows])
+        assert amax.item() == got[rows].float().abs().max().item()

@@ -1,0 +1,226 @@
+"""GPU parity: the backbone forward with e4m3 dense layers (TAAC_BACKBONE_FP8) against the CPU oracle's chain of quantize ->
+matmul -> dequantize layers. Tolerance of the FP8 configuration: probabilities 2e-2 absolute; hidden state 5e-2 relative to
+the largest expected value, and an error against the float32 evaluation no larger than the emulation's own."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from oracle import reference as oracle
+from taac_2026_amd import workloads
+from taac_2026_amd.accelerators.attention import hip_flash_attention_kernel
+from taac_2026_amd.api import (PCVRBackbone, amax, norm_linear_fp8, pack_ffn_weights_fp8, quantize_fp8, rms_norm,
+                               swiglu_ffn_fp8, valid_rows)
+
+pytestmark = pytest.mark.gpu
+
+
+def _model(inputs, device):
+    model = PCVRBackbone(d_model=inputs.emb.shape[-1], num_heads=inputs.num_heads, d_ff=inputs.d_ff,
+                         n_blocks=len(inputs.blocks))
+    workloads.load_backbone_state(model, inputs)
+    return model.to(device=device, dtype=torch.bfloat16).eval()
+
+
+def _run(inputs, device, **routes):
+    model = _model(inputs, device)
+    with torch.no_grad():
+        p, hidden = model(inputs.emb.to(device), inputs.key_lengths.to(device), return_hidden=True, **routes)
+    return p.cpu(), hidden.cpu(), model
+
+
+def _with_biases(inputs, seed):
+    g = torch.Generator().manual_seed(seed)
+    for w in inputs.blocks:
+        for name in ("qkv", "out", "up", "down"):
+            w[f"{name}.bias"] = (0.05 * torch.randn(w[f"{name}.weight"].shape[0], generator=g)).to(torch.bfloat16)
+    return inputs
+
+
+def _exact(inputs):
+    blocks32 = [{k: v.float() for k, v in w.items()} for w in inputs.blocks]
+    return oracle.backbone(inputs.emb.float(), inputs.key_lengths, blocks32, inputs.head_weight.float(),
+                           inputs.head_bias.float(), num_heads=inputs.num_heads, return_hidden=True)
+
+
+@pytest.mark.parametrize("batch,n_feature,n_sequence,n_blocks,d_ff", [(6, 32, 96, 4, 512), (3, 32, 480, 2, 1024),
+                                                                      (5, 8, 57, 1, 64)])
+def test_fp8_backbone_matches_the_emulated_chain(device, batch, n_feature, n_sequence, n_blocks, d_ff):
+    inputs = _with_biases(workloads.backbone_inputs(batch=batch, n_feature_tokens=n_feature, n_sequence_tokens=n_sequence,
+                                                    min_sequence_len=min(32, n_sequence), n_blocks=n_blocks, d_ff=d_ff,
+                                                    seed=batch), seed=batch)
+    tokens = inputs.emb.shape[1]
+    valid = torch.arange(tokens)[None, :] < inputs.key_lengths[:, None]
+    exact_p, exact_h = _exact(inputs)
+    # valid_only: the scales of the route over the valid-row index; dense: the scales over all B*T positions
+    for routes, valid_only in (({}, True), ({"dense_tokens": True}, False)):
+        want_p, want_h = oracle.backbone_fp8(inputs.emb, inputs.key_lengths, inputs.blocks, inputs.head_weight,
+                                             inputs.head_bias, num_heads=inputs.num_heads, return_hidden=True,
+                                             valid_only=valid_only)
+        p, hidden, model = _run(inputs, device, fp8=True, **routes)
+        assert torch.isfinite(p).all() and torch.isfinite(hidden).all()
+        torch.testing.assert_close(p, want_p, rtol=0, atol=2e-2)
+        # against float32 the kernels stray no further than the emulation itself does (what e4m3 operands cost)
+        assert (p - exact_p).abs().max().item() <= (want_p - exact_p).abs().max().item() + 2e-2
+        scale = want_h.float()[valid].abs().max().item()
+        assert (hidden.float()[valid] - want_h.float()[valid]).abs().max().item() <= 5e-2 * scale
+        ours = (hidden.float()[valid] - exact_h[valid]).abs().mean().item()
+        emulated = (want_h.float()[valid] - exact_h[valid]).abs().mean().item()
+        assert ours <= 1.1 * emulated + 1e-4, (ours, emulated)
+        # the maxima the kernels reduced are those of the emulated tensors of the first block
+        first = model.fp8_maxima()[0]
+        keep = valid if valid_only else torch.ones_like(valid)
+        h = oracle.rms_norm_fp32(inputs.emb, inputs.blocks[0]["attn_norm.weight"])
+        assert first["attn_norm"].item() == h[keep].float().abs().max().item()
+        for name in ("qkv", "out", "up", "down"):
+            assert first[f"{name}.weight"].item() == inputs.blocks[0][f"{name}.weight"].float().abs().max().item()
+    # FP8 is not the bf16 route under another name
+    _, bf16_h, _ = _run(inputs, device)
+    assert not torch.equal(bf16_h[valid], hidden[valid])
+
+
+def test_every_kernel_of_the_fp8_block_is_tight_against_its_emulated_layer(device):
+    """The four kernels of one FP8 block, each against the emulated layer on the tensor the previous kernel wrote and with
+    the maximum that kernel reduced, so that no quantisation bucket flipped upstream is carried along: what is left is
+    accumulation order and rounding points, 1e-2 of the largest value at most and 1e-3 on average (the chain of four
+    kernels on its own input stays inside the 5e-2 of the configuration, test above)."""
+    inputs = _with_biases(workloads.backbone_inputs(batch=4, n_feature_tokens=16, n_sequence_tokens=112, n_blocks=1, seed=2),
+                          seed=4)
+    w = inputs.blocks[0]
+    batch, tokens, width = inputs.emb.shape
+    heads = inputs.num_heads
+    valid = torch.arange(tokens)[None, :] < inputs.key_lengths[:, None]
+    flat = valid.flatten()
+    d = {k: v.to(device) for k, v in w.items()}
+    x = inputs.emb.reshape(-1, width).to(device)
+    lengths = inputs.key_lengths.to(device)
+
+    def tight(got, want, mask):
+        diff = (got.float().cpu()[mask] - want.float()[mask]).abs()
+        top = want.float()[mask].abs().max().item()
+        assert diff.max().item() <= 1e-2 * top and diff.mean().item() <= 1e-3 * top, (diff.max().item(), diff.mean().item(), top)
+
+    with torch.no_grad():
+        rows = valid_rows(lengths, tokens)
+        h = rms_norm(x, d["attn_norm.weight"])
+        amax_h = amax(h[flat.to(device)])
+        w_qkv, amax_w = quantize_fp8(d["qkv.weight"])
+        qkv, _ = norm_linear_fp8(x, w_qkv, amax_h, amax_w, d["qkv.bias"], norm_weight=d["attn_norm.weight"], token_rows=rows,
+                                 out=torch.zeros(batch * tokens, 3 * width, dtype=torch.bfloat16, device=device))
+        tight(qkv, oracle.linear_fp8(h.cpu(), w["qkv.weight"], w["qkv.bias"], x_scale=amax_h.cpu() / 448), flat)
+
+        q, k, v = qkv.view(batch, tokens, 3 * width).chunk(3, dim=-1)
+        split = lambda t: t.reshape(batch, tokens, heads, width // heads).transpose(1, 2)  # noqa: E731
+        amax_a = torch.zeros((), dtype=torch.float32, device=device)
+        a = hip_flash_attention_kernel(split(q), split(k), split(v), lengths, zero_padded_queries=2, amax_out=amax_a)
+        a = a.transpose(1, 2).reshape(batch * tokens, width).contiguous()
+        want_a = oracle.scaled_dot_product_attention(q.cpu(), k.cpu(), v.cpu(), num_heads=heads, key_lengths=inputs.key_lengths,
+                                                     zero_padded_queries=True).reshape(-1, width)
+        tight(a, want_a, flat)
+        assert amax_a.item() == a[flat.to(device)].float().abs().max().item()
+
+        w_out, amax_wo = quantize_fp8(d["out.weight"])
+        x1, amax_h2 = norm_linear_fp8(a, w_out, amax_a, amax_wo, d["out.bias"], residual=x, token_rows=rows,
+                                      out=torch.zeros_like(x), out_norm_weight=d["ffn_norm.weight"])
+        tight(x1, oracle.linear_fp8(a.cpu(), w["out.weight"], w["out.bias"], residual=x.cpu(), x_scale=amax_a.cpu() / 448), flat)
+        h2 = rms_norm(x1, d["ffn_norm.weight"])
+        assert amax_h2.item() == h2[flat.to(device)].float().abs().max().item()
+
+        packed = pack_ffn_weights_fp8(d["up.weight"], d["down.weight"])
+        y, amax_hidden, _ = swiglu_ffn_fp8(x1, packed, d["up.bias"], d["down.bias"], amax_h2, hidden_size=inputs.d_ff,
+                                           residual=x1, norm_weight=d["ffn_norm.weight"], token_rows=rows,
+                                           out=torch.zeros_like(x))
+    # the fused layer quantises the float32 hidden state (the emulated chain rounds it to bf16 in between)
+    qh2, s_h2 = oracle.fp8_quantize(h2.cpu(), amax_h2.cpu() / 448)
+    q_up, s_up = oracle.fp8_quantize(w["up.weight"])
+    gate, value = (torch.matmul(qh2.float(), q_up.float().t()) * (s_h2 * s_up) + w["up.bias"].float()).chunk(2, dim=-1)
+    hidden = torch.nn.functional.silu(gate) * value
+    assert abs(amax_hidden.item() - hidden[flat].abs().max().item()) <= 1e-5 * amax_hidden.item()
+    q_hidden, s_hidden = oracle.fp8_quantize(hidden, amax_hidden.cpu() / 448)
+    q_down, s_down = oracle.fp8_quantize(w["down.weight"])
+    want = torch.matmul(q_hidden.float(), q_down.float().t()) * (s_hidden * s_down) + w["down.bias"].float() + x1.cpu().float()
+    tight(y, want.to(torch.bfloat16), flat)
+    # and the backbone call runs exactly these kernels
+    _, hidden_state, _ = _run(inputs, device, fp8=True)
+    assert torch.equal(hidden_state.reshape(-1, width)[flat], y.cpu()[flat])
+
+
+def test_fp8_backbone_skips_padded_positions_and_repeats_bit_for_bit(device):
+    inputs = workloads.backbone_inputs(batch=7, n_feature_tokens=32, n_sequence_tokens=224, min_sequence_len=16, seed=3)
+    valid = torch.arange(inputs.emb.shape[1])[None, :] < inputs.key_lengths[:, None]
+    p_ref, h_ref, _ = _run(inputs, device, fp8=True)
+    poisoned = workloads.BackboneInputs(inputs.emb.clone(), inputs.key_lengths, inputs.blocks, inputs.head_weight,
+                                        inputs.head_bias, inputs.num_heads, inputs.d_ff)
+    poisoned.emb[~valid] = float("nan")
+    p, hidden, _ = _run(poisoned, device, fp8=True)
+    assert torch.equal(p, p_ref) and torch.equal(hidden, h_ref)
+    assert (h_ref[~valid] == 0).all()
+
+
+def test_fp8_backbone_rejects_what_it_does_not_cover(device):
+    inputs = workloads.backbone_inputs(batch=2, n_feature_tokens=8, n_sequence_tokens=24, d_model=128, num_heads=4, d_ff=256, min_sequence_len=4,
+                                       n_blocks=1, seed=1)
+    with pytest.raises(RuntimeError, match="D = 256"):
+        _run(inputs, device, fp8=True)
+    inputs = workloads.backbone_inputs(batch=2, n_feature_tokens=8, n_sequence_tokens=24, n_blocks=1, seed=1, qk_norm=True,
+                                       min_sequence_len=4)
+    model = PCVRBackbone(d_model=256, num_heads=inputs.num_heads, d_ff=inputs.d_ff, n_blocks=1, qk_norm=True)
+    workloads.load_backbone_state(model, inputs)
+    model = model.to(device=device, dtype=torch.bfloat16).eval()
+    with pytest.raises(RuntimeError, match="query / key norm"):
+        model(inputs.emb.to(device), inputs.key_lengths.to(device), fp8=True)
+    with pytest.raises(RuntimeError, match="no fp8 forward"):
+        model.fp8_maxima()
+
+
+def test_fp8_backbone_full_size_slice_against_the_emulation(device):
+    """Config 4 at full size (B=1024, T=512, 285k valid tokens) with e4m3 dense layers: all outputs finite, and a slice of
+    samples against the oracle quantising with the whole batch's maxima (which the slice alone does not determine)."""
+    inputs = workloads.backbone_inputs()
+    p, hidden, model = _run(inputs, device, fp8=True)
+    assert torch.isfinite(p).all() and torch.isfinite(hidden).all()
+    assert ((p > 0) & (p < 1)).all()
+    maxima = model.fp8_maxima()
+    assert all(torch.isfinite(v) and v > 0 for row in maxima for v in row.values())
+    pick = torch.tensor([0, 257, 511, 1023])
+    want_p, want_h = oracle.backbone_fp8(inputs.emb[pick], inputs.key_lengths[pick], inputs.blocks, inputs.head_weight,
+                                         inputs.head_bias, num_heads=inputs.num_heads, return_hidden=True, maxima=maxima)
+    torch.testing.assert_close(p[pick], want_p, rtol=0, atol=2e-2)
+    valid = torch.arange(inputs.emb.shape[1])[None, :] < inputs.key_lengths[pick][:, None]
+    got, want = hidden[pick].float()[valid], want_h.float()[valid]
+    assert (got - want).abs().max().item() <= 5e-2 * want.abs().max().item()
+    bf16_p = oracle.backbone(inputs.emb[pick], inputs.key_lengths[pick], inputs.blocks, inputs.head_weight, inputs.head_bias,
+                             num_heads=inputs.num_heads)
+    # e4m3 operands move these probabilities by up to ~0.06 against the bf16 recipe; the kernels add nothing to that
+    assert (p[pick] - bf16_p).abs().max().item() <= (want_p - bf16_p).abs().max().item() + 2e-2
+
+
+def test_fp8_dense_layers_at_full_size_on_backbone_activations(device):
+    """The two fused FP8 layers at M = 524288 rows, on the residual stream the bf16 backbone produces for config 4 (not on
+    Gaussian noise): RMSNorm + QKV projection and the whole feed-forward half against the emulated layers, every element
+    inside 5e-2 of the largest expected value."""
+    inputs = workloads.backbone_inputs()
+    model = _model(inputs, device)
+    with torch.no_grad():
+        _, hidden = model(inputs.emb.to(device), inputs.key_lengths.to(device), return_hidden=True, dense_tokens=True)
+    w = inputs.blocks[-1]
+    x = hidden.reshape(-1, hidden.shape[-1])
+    assert x.shape[0] == 524288
+    dev = {k: v.to(device) for k, v in w.items()}
+    with torch.no_grad():
+        wq, amax_w = quantize_fp8(dev["qkv.weight"])
+        h = rms_norm(x, dev["attn_norm.weight"])
+        qkv, _ = norm_linear_fp8(x, wq, amax(h), amax_w, norm_weight=dev["attn_norm.weight"])
+        packed = pack_ffn_weights_fp8(dev["up.weight"], dev["down.weight"])
+        h2 = rms_norm(x, dev["ffn_norm.weight"])
+        out, amax_hidden, _ = swiglu_ffn_fp8(x, packed, None, None, amax(h2), hidden_size=inputs.d_ff, residual=x,
+                                             norm_weight=dev["ffn_norm.weight"])
+    xc = x.cpu()
+    want_qkv = oracle.linear_fp8(oracle.rms_norm_fp32(xc, w["attn_norm.weight"]), w["qkv.weight"])
+    assert (qkv.cpu().float() - want_qkv.float()).abs().max().item() <= 5e-2 * want_qkv.float().abs().max().item()
+    want, want_hidden, _ = oracle.swiglu_ffn_fp8(xc, w["ffn_norm.weight"], w["up.weight"], None, w["down.weight"], None,
+                                                 residual=xc)
+    assert (out.cpu().float() - want.float()).abs().max().item() <= 5e-2 * want.float().abs().max().item()
+    top = want_hidden.float().abs().max().item()
+    assert abs(amax_hidden.item() - top) <= 2e-2 * top
