@@ -345,56 +345,109 @@ def _readout_figures(inputs, device, iters: int) -> dict:
                                            "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS, "max_abs_err": err}}
 
 
-def _fp8_figures(inputs, device, iters: int) -> dict:
-    """Configuration 5: the block's four dense layers with e4m3 operands (per-tensor scale amax / 448) over all
-    M = B * T tokens, each checked on a slice of rows against the quantize -> matmul -> dequantize emulation."""
+def _fp8_figures(inputs, device, iters: int, all_positions: bool = True) -> dict:
+    """Configuration 5: the block's four dense layers with e4m3 operands (per-tensor scale = maximum / 448, every
+    activation maximum reduced in the epilogue of the kernel that produces the tensor). Reports the three fused kernels of
+    one block over the valid tokens and over all M = B * T positions, each checked on a slice of rows against the
+    quantize -> matmul -> dequantize emulation run with the maxima the kernels found, and the whole backbone step with
+    ``fp8=True`` next to the bf16 step, timed in alternation."""
     from oracle import reference as oracle
-    from taac_2026_amd.api import (amax, flash_attention, linear_fp8, norm_linear, quantize_fp8, rms_norm,
-                                   scaled_dot_product_attention, swiglu_linear)
+    from taac_2026_amd.accelerators.attention import hip_flash_attention_kernel
+    from taac_2026_amd.api import (PCVRBackbone, amax, norm_linear_fp8, pack_ffn_weights_fp8, quantize_fp8, rms_norm,
+                                   swiglu_ffn_fp8, valid_rows)
+    from taac_2026_amd import workloads
 
-    del flash_attention
     B, T, D = inputs.emb.shape
     M, F, H = B * T, inputs.d_ff, inputs.num_heads
-    w = {k: v.to(device) for k, v in inputs.blocks[0].items()}
-    x = inputs.emb.to(device)
+    cpu_w = inputs.blocks[0]
+    w = {k: v.to(device) for k, v in cpu_w.items()}
+    x = inputs.emb.to(device).view(M, D)
     lengths = inputs.key_lengths.to(device)
+    n_valid = int(inputs.key_lengths.clamp(0, T).sum().item())
     figures: dict[str, dict] = {}
+    split = lambda t: t.reshape(B, T, H, D // H).transpose(1, 2)  # noqa: E731
     with torch.no_grad():
-        h = rms_norm(x, w["attn_norm.weight"])
-        q, k, v = norm_linear(h, w["qkv.weight"], w["qkv.bias"]).chunk(3, dim=-1)
-        a = scaled_dot_product_attention(q, k, v, num_heads=H, attn_mask=None, dropout_p=0.0, training=False,
-                                         key_lengths=lengths, zero_padded_queries=True)
-        x1 = norm_linear(a, w["out.weight"], w["out.bias"], residual=x)
-        h2 = rms_norm(x1, w["ffn_norm.weight"])
-        g = swiglu_linear(h2, w["up.weight"], w["up.bias"])
-        layers = {
-            "qkv": (h.view(M, D), "qkv", False, None),
-            "out": (a.view(M, D), "out", False, x.view(M, D)),
-            "up_swiglu": (h2.view(M, D), "up", True, None),
-            "down": (g.view(M, F), "down", False, x1.view(M, D)),
-        }
-        total_flops, total_ms = 0.0, 0.0
-        for name, (act, key, swiglu, residual) in layers.items():
-            weight, bias = w[f"{key}.weight"], w[f"{key}.bias"]
-            wq, wa = quantize_fp8(weight)
-            xa = amax(act)
-            run = lambda act=act, wq=wq, xa=xa, wa=wa, bias=bias, residual=residual, swiglu=swiglu: linear_fp8(  # noqa: E731
-                act, wq, xa, wa, bias, residual=residual, swiglu=swiglu)
-            got = run()[:512].cpu().float()
-            expected = oracle.linear_fp8(act[:512].cpu(), weight.cpu(), bias.cpu(),
-                                         residual=None if residual is None else residual[:512].cpu(), swiglu=swiglu,
-                                         x_scale=(xa.cpu() / 448.0), w_scale=(wa.cpu() / 448.0)).float()
-            rel = ((got - expected).abs().max() / expected.abs().max()).item()
-            if rel > 5e-2:
-                raise SystemExit(f"fp8 accuracy gate failed for {name}: relative error {rel}")
-            flops = 2.0 * M * weight.shape[0] * weight.shape[1]
-            ms = _event_ms(run, iters, 3)
-            ms_amax = _event_ms(lambda act=act: amax(act), iters, 3)
-            figures[name] = {"ms": ms, "amax_ms": ms_amax, "tflops": flops / ms / 1e9,
-                             "frac_mfma_fp8": flops / ms / 1e9 / 5000.0, "rel_err": rel}
-            total_flops += flops
-            total_ms += ms + ms_amax
-        figures["block_set"] = {"ms_including_amax": total_ms, "tflops": total_flops / total_ms / 1e9}
+        index = valid_rows(lengths, T)
+        flat_valid = (torch.arange(T, device=device)[None, :] < lengths[:, None]).flatten()
+        w_qkv, amax_wqkv = quantize_fp8(w["qkv.weight"])
+        w_out, amax_wout = quantize_fp8(w["out.weight"])
+        packed = pack_ffn_weights_fp8(w["up.weight"], w["down.weight"])
+        for label, rows, tokens in (("valid_tokens", index, n_valid), ("all_positions", None, M))[:2 if all_positions else 1]:
+            h = rms_norm(x, w["attn_norm.weight"])
+            amax_h = amax(h[flat_valid] if rows is not None else h)
+            qkv = torch.zeros(M, 3 * D, dtype=torch.bfloat16, device=device)
+            x1 = torch.zeros(M, D, dtype=torch.bfloat16, device=device)
+            y = torch.zeros(M, D, dtype=torch.bfloat16, device=device)
+            amax_a = torch.zeros((), dtype=torch.float32, device=device)
+            run_qkv = lambda: norm_linear_fp8(x, w_qkv, amax_h, amax_wqkv, w["qkv.bias"],  # noqa: E731
+                                              norm_weight=w["attn_norm.weight"], token_rows=rows, out=qkv)
+            run_qkv()
+            q, k, v = qkv.view(B, T, 3 * D).chunk(3, dim=-1)
+            run_attn = lambda: hip_flash_attention_kernel(split(q), split(k), split(v), lengths,  # noqa: E731
+                                                          zero_padded_queries=2 if rows is not None else 1, amax_out=amax_a)
+            a = run_attn().transpose(1, 2).reshape(M, D)
+            run_out = lambda: norm_linear_fp8(a, w_out, amax_a, amax_wout, w["out.bias"], residual=x, token_rows=rows,  # noqa: E731
+                                              out=x1, out_norm_weight=w["ffn_norm.weight"])
+            _, amax_h2 = run_out()
+            run_ffn = lambda: swiglu_ffn_fp8(x1, packed, w["up.bias"], w["down.bias"], amax_h2, hidden_size=F,  # noqa: E731
+                                             residual=x1, norm_weight=w["ffn_norm.weight"], token_rows=rows, out=y,
+                                             next_norm_weight=w["attn_norm.weight"])
+            _, amax_hidden, _ = run_ffn()
+            # accuracy gates on the first 512 valid rows, the emulation quantising with the kernels' maxima
+            pick = (index[0][:512].long() if rows is not None else torch.arange(512, device=device))
+            scale = lambda t: t.cpu() / 448.0  # noqa: E731
+            cases = {
+                "norm_qkv": (qkv, oracle.linear_fp8(h[pick].cpu(), cpu_w["qkv.weight"], cpu_w["qkv.bias"], x_scale=scale(amax_h))),
+                "out_residual": (x1, oracle.linear_fp8(a[pick].cpu(), cpu_w["out.weight"], cpu_w["out.bias"],
+                                                       residual=x[pick].cpu(), x_scale=scale(amax_a))),
+            }
+            h2 = oracle.rms_norm_fp32(x1[pick].cpu(), cpu_w["ffn_norm.weight"])
+            hidden = oracle.linear_fp8(h2, cpu_w["up.weight"], cpu_w["up.bias"], swiglu=True, x_scale=scale(amax_h2))
+            cases["feed_forward"] = (y, oracle.linear_fp8(hidden, cpu_w["down.weight"], cpu_w["down.bias"],
+                                                          residual=x1[pick].cpu(), x_scale=scale(amax_hidden)))
+            errors = {}
+            for name, (got, expected) in cases.items():
+                rel = ((got[pick].cpu().float() - expected.float()).abs().max() / expected.float().abs().max()).item()
+                if not rel <= 5e-2:
+                    raise SystemExit(f"fp8 accuracy gate failed for {name} ({label}): relative error {rel}")
+                errors[name] = rel
+            flops = {"norm_qkv": 2.0 * tokens * 3 * D * D, "out_residual": 2.0 * tokens * D * D,
+                     "feed_forward": 2.0 * tokens * 3 * D * F}
+            runs = {"norm_qkv": run_qkv, "out_residual": run_out, "feed_forward": run_ffn}
+            entry: dict[str, dict | float] = {}
+            for _ in range(30):                       # clocks and caches settle before any kernel is timed
+                run_ffn()
+            total_ms, total_flops = 0.0, 0.0
+            for name, run in runs.items():
+                ms = _event_ms(run, iters, 5)
+                entry[name] = {"ms": ms, "tflops": flops[name] / ms / 1e9, "frac_mfma_fp8": flops[name] / ms / 1e9 / 5000.0,
+                               "rel_err": errors[name]}
+                total_ms += ms
+                total_flops += flops[name]
+            entry["attention_with_maximum"] = {"ms": _event_ms(run_attn, iters, 5)}
+            entry["block_set"] = {"ms": total_ms, "tflops": total_flops / total_ms / 1e9,
+                                  "frac_mfma_fp8": total_flops / total_ms / 1e9 / 5000.0,
+                                  "note": "three launches sequences (qkv; out; feed-forward = two passes), every scale "
+                                          "included: no stand-alone maximum pass is left"}
+            figures[label] = entry
+
+        model = PCVRBackbone(d_model=D, num_heads=H, d_ff=F, n_blocks=len(inputs.blocks))
+        workloads.load_backbone_state(model, inputs)
+        model = model.to(device=device, dtype=torch.bfloat16).eval()
+        emb = inputs.emb.to(device)
+        p_fp8 = model(emb, lengths, fp8=True)
+        p_bf16 = model(emb, lengths)
+        step: dict[str, float] = {"max_abs_diff_of_probabilities_to_bf16": (p_fp8 - p_bf16).abs().max().item()}
+        for _ in range(10):
+            model(emb, lengths, fp8=True)
+        fp8_ms, bf16_ms = [], []
+        for _ in range(3):                            # alternate, so that neither is the one measured on a cold chip
+            fp8_ms.append(_event_ms(lambda: model(emb, lengths, fp8=True), iters, 3))
+            bf16_ms.append(_event_ms(lambda: model(emb, lengths), iters, 3))
+        step["fp8_ms_per_step"] = sorted(fp8_ms)[1]
+        step["bf16_ms_per_step"] = sorted(bf16_ms)[1]
+        step["fp8_samples_per_s"] = B / (step["fp8_ms_per_step"] * 1e-3)
+        figures["backbone_step"] = step
     return figures
 
 
@@ -599,6 +652,8 @@ def main() -> None:
                         help="time only the stand-alone kernels of one block (short run for hardware-counter collection)")
     parser.add_argument("--only-attention-bwd", action="store_true",
                         help="time only the attention backward at its two shapes (short run for traces and counters)")
+    parser.add_argument("--only-fp8", action="store_true",
+                        help="time only the FP8 dense layers and the FP8 backbone step (short run for traces and counters)")
     parser.add_argument("--only-reference-block", action="store_true",
                         help="time only the reference model's block (role mask, scattered padding) and print those figures")
     args = parser.parse_args()
@@ -623,6 +678,11 @@ def main() -> None:
         return
     if args.only_attention_bwd:
         print(json.dumps({"attention_bwd": _attention_bwd_figures(device, iters=6)}))
+        return
+    if args.only_fp8:
+        inputs = workloads.backbone_inputs(batch=args.batch)
+        print(json.dumps({"fp8_dense_layers": _fp8_figures(inputs, device, iters=6,
+                                                           all_positions=not args.skip_all_positions)}))
         return
     if args.only_reference_block:
         print(json.dumps({"reference_block": _reference_block_figures(device, args.batch, 10)}))

@@ -1063,9 +1063,11 @@ extern "C" int taac_flash_attn_amax_fwd(const void* q, const void* k, const void
                                         const int64_t v_strides[4], const int64_t o_strides[4], int is_causal,
                                         int zero_padded_queries, int dtype, void* stream) {
   if (!amax_out) return taac::set_error(TAAC_ERR_INVALID_VALUE, "taac_flash_attn_amax_fwd: amax_out must be given");
-  hipLaunchKernelGGL(taac::attn_clear_kernel, dim3(1), dim3(taac::kWave), 0, taac::as_stream(stream), amax_out);
-  const int rc = taac::check_launch("taac_flash_attn_amax_fwd");
-  if (rc != TAAC_OK) return rc;
+  if (!taac::maxima_precleared) {
+    hipLaunchKernelGGL(taac::attn_clear_kernel, dim3(1), dim3(taac::kWave), 0, taac::as_stream(stream), amax_out);
+    const int rc = taac::check_launch("taac_flash_attn_amax_fwd");
+    if (rc != TAAC_OK) return rc;
+  }
   return taac::attention_entry("taac_flash_attn_amax_fwd", q, k, v, key_lengths, taac::MaskArgs{}, q_row_scale,
                                k_row_scale, q_col_scale, nullptr, amax_out, o, B, H, Tq, Tk, d, q_strides, k_strides,
                                v_strides, o_strides, is_causal, zero_padded_queries, dtype, stream);

@@ -423,6 +423,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
       wq[n_blocks + i] = fp8_out(i);
       wq[2 * n_blocks + i] = fp8_ffn(i);
     }
+    if ((rc = fill_zero(fp8_scales, (n_blocks + 1) * 8, as_stream(stream), name)) != TAAC_OK) return rc;
     if ((rc = prepare_backbone_fp8(blocks, n_blocks, D, F, sc.data(), wq.data(), wq.data() + n_blocks,
                                    wq.data() + 2 * n_blocks, as_stream(stream), name)) != TAAC_OK)
       return rc;
@@ -440,6 +441,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
       // Four dense layers with e4m3 operands and per-tensor scales; every activation scale comes out of the epilogue of the
       // kernel that produces the tensor (scales[4..7] = block input, attention output, feed-forward input, hidden state).
       float* sc = fp8_scales + 8 * i;
+      PreclearedMaxima precleared;
       if ((rc = taac_norm_linear_fp8_fwd(cur, D, w.attn_norm_weight, eps, fp8_qkv(i), w.qkv_bias, sc + 4, sc + 0, nullptr, 0,
                                          qkv, 3 * D, M, 3 * D, D, rows, n_rows, nullptr, 0.f, nullptr, stream)) != TAAC_OK)
         return rc;

@@ -39,13 +39,24 @@ int launch_linear_fp8_ts(const void* a, int a_is_fp8, int64_t lda, const void* w
                          int64_t M, int32_t N, int32_t K, int epilogue, int gate_first, hipStream_t s,
                          const char* name);
 
-// FP8 preparation of a backbone (ffn_fp8.hip): per block four weight scales (qkv, out, up, down), the row-major e4m3
+// FP8 preparation of a backbone (ffn_fp8.hip): per block four weight scales (qkv, out, up, down; zeroed by the caller), the row-major e4m3
 // copies of the qkv / out weights and the packed feed-forward blob.
 int prepare_backbone_fp8(const taac_block_weights* blocks, int n, int32_t D, int32_t F, float* const* scales,
                          void* const* qkv_q, void* const* out_q, void* const* ffn_blob, hipStream_t s, const char* name);
-// *out = max over the (listed) rows of | bf16(rmsnorm(x, w, eps)) | for rows of 256 bf16 features (ffn_fp8.hip).
+// p[0..n) = 0 with a kernel (ffn_fp8.hip).
+int fill_zero(float* p, int n, hipStream_t s, const char* name);
+// *out (zeroed by the caller) = max over the (listed) rows of | bf16(rmsnorm(x, w, eps)) |, rows of 256 bf16 features
+// (ffn_fp8.hip).
 int rmsnorm_amax_256(const void* x, int64_t ldx, const void* w, float eps, int64_t M, const int32_t* rows,
                      const int32_t* n_rows, float* out, hipStream_t s, const char* name);
+
+// Set (per host thread) while taac_backbone_fwd drives the FP8 entry points: it has zeroed every maximum of the forward in
+// one launch, so the entry points skip the clearing launch each of them issues for its own outputs.
+inline thread_local bool maxima_precleared = false;
+struct PreclearedMaxima {
+  PreclearedMaxima() { maxima_precleared = true; }
+  ~PreclearedMaxima() { maxima_precleared = false; }
+};
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 __host__ __device__ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

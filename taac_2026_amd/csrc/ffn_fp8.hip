@@ -769,7 +769,7 @@ __global__ __launch_bounds__(256) void f8_norm_amax_kernel(const bf16_t* __restr
 
 }  // namespace
 
-// Scales (4 floats per block: qkv, out, up, down) and the e4m3 weights of n backbone blocks: row-major qkv / out copies and
+// Scales (4 floats per block: qkv, out, up, down; zeroed by the caller) and the e4m3 weights of n backbone blocks: row-major qkv / out copies and
 // the feed-forward blob (gate first). D = 256, F a multiple of 64.
 int prepare_backbone_fp8(const taac_block_weights* blocks, int n, int32_t D, int32_t F, float* const* scales,
                          void* const* qkv_q, void* const* out_q, void* const* ffn_blob, hipStream_t s, const char* name) {
@@ -788,7 +788,6 @@ int prepare_backbone_fp8(const taac_block_weights* blocks, int n, int32_t D, int
       batch.out_q[i] = static_cast<uint8_t*>(out_q[base + i]);
       batch.ffn_blob[i] = static_cast<u32x4*>(ffn_blob[base + i]);
       batch.scales[i] = scales[base + i];
-      hipLaunchKernelGGL(f8_fill_zero_kernel, dim3(1), dim3(256), 0, s, scales[base + i], 4);
     }
     hipLaunchKernelGGL(f8_weights_amax_kernel, dim3(16, 4 * m), dim3(256), 0, s, batch, D, F);
     const int64_t pieces = (static_cast<int64_t>(4) * D * D + taac_ffn_fp8_packed_bytes(D, F)) / 16;
@@ -800,10 +799,14 @@ int prepare_backbone_fp8(const taac_block_weights* blocks, int n, int32_t D, int
   return TAAC_OK;
 }
 
-// *out = max over the (listed) rows of | bf16(rmsnorm(x, w, eps)) |, rows of 256 bf16 features.
+// *out (zeroed by the caller) = max over the (listed) rows of | bf16(rmsnorm(x, w, eps)) |, rows of 256 bf16 features.
+int fill_zero(float* p, int n, hipStream_t s, const char* name) {
+  hipLaunchKernelGGL(f8_fill_zero_kernel, dim3((n + 255) / 256), dim3(256), 0, s, p, n);
+  return check_launch(name);
+}
+
 int rmsnorm_amax_256(const void* x, int64_t ldx, const void* w, float eps, int64_t M, const int32_t* rows,
                      const int32_t* n_rows, float* out, hipStream_t s, const char* name) {
-  hipLaunchKernelGGL(f8_fill_zero_kernel, dim3(1), dim3(256), 0, s, out, 1);
   if (M > 0) {
     int64_t grid = (M + 7) / 8;
     if (grid > 4096) grid = 4096;
@@ -896,9 +899,11 @@ extern "C" int taac_swiglu_ffn_fp8_fwd(const void* x, int64_t ldx, const void* n
   p.next_eps = next_eps;
   p.rows = rows;
   p.n_rows = n_rows;
-  hipLaunchKernelGGL(f8_clear_kernel, dim3(1), dim3(kWave), 0, s, amax_hidden, amax_next);
-  int rc = check_launch(name);
-  if (rc != TAAC_OK) return rc;
+  int rc = TAAC_OK;
+  if (!maxima_precleared) {
+    hipLaunchKernelGGL(f8_clear_kernel, dim3(1), dim3(kWave), 0, s, amax_hidden, amax_next);
+    if ((rc = check_launch(name)) != TAAC_OK) return rc;
+  }
 // pass 1: 4 wavefronts x 2 tiles; pass 2: 4 wavefronts x 1 tile; two workgroups per compute unit
 #define TAAC_F8_FFN(DD, BB)                                                                                             \
   do {                                                                                                                  \

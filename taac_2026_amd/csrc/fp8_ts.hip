@@ -536,7 +536,7 @@ extern "C" int taac_norm_linear_fp8_fwd(const void* x, int64_t ldx, const void* 
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows and n_rows must be given together", name);
   if (out_norm_weight && !amax_out) return set_error(TAAC_ERR_INVALID_VALUE, "%s: out_norm_weight without amax_out", name);
   hipStream_t s = as_stream(stream);
-  if (amax_out != nullptr) {
+  if (amax_out != nullptr && !maxima_precleared) {
     hipLaunchKernelGGL(fp8_ts_clear_kernel, dim3(1), dim3(kWave), 0, s, amax_out);
     const int rc = check_launch(name);
     if (rc != TAAC_OK) return rc;
