@@ -533,7 +533,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   constexpr int OROW = DP * 2 + 16;
   constexpr int OT_BYTES = (kThreads / kWave) * 32 * OROW;
   static_assert(kKC * C8 % kThreads == 0, "whole transfers per wavefront");
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * BUF_BYTES > OT_BYTES ? 2 * BUF_BYTES : OT_BYTES];
+  constexpr int NBUF = 3;                           // chunk c is consumed while c + 1 and c + 2 are in flight
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[NBUF * BUF_BYTES > OT_BYTES ? NBUF * BUF_BYTES : OT_BYTES];
 
   const uint32_t logical = xcd_remap(blockIdx.x, p.total);
   const int qc = static_cast<int>(logical % p.nqc);
@@ -577,15 +578,18 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   if (CAUSAL) kv_end = kv_end < q_begin + kQB ? kv_end : q_begin + kQB;
 
   const int qi = q_begin + wave * 32 + l32;
+  float c = p.scale_log2;  // SCALED: the query's row factor joins the lane's softmax scale
+  if (SCALED && p.q_row_scale != nullptr && qi < q_valid) c *= p.q_row_scale[static_cast<int64_t>(b) * p.Tq + qi];
+  // The query enters the products already multiplied by the softmax scale (and log2 e), rounded once more to the storage
+  // type: the score tiles then come out of the matrix unit in the exponent's units.
   vec_t qf[KSTEPS];
 #pragma unroll
   for (int s = 0; s < KSTEPS; ++s) {
     qf[s] = qi < q_valid ? *reinterpret_cast<const vec_t*>(qb + qi * p.qs[2] + 16 * s + 8 * hh) : zero_vec;
-    if (SCALED && p.q_col_scale != nullptr) {
-      const float* cf = p.q_col_scale + h * p.d + 16 * s + 8 * hh;
+    const float* cf = (SCALED && p.q_col_scale != nullptr) ? p.q_col_scale + h * p.d + 16 * s + 8 * hh : nullptr;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<T>(static_cast<float>(qf[s][e]) * cf[e]);
-    }
+    for (int e = 0; e < 8; ++e)
+      qf[s][e] = static_cast<T>(static_cast<float>(qf[s][e]) * (cf != nullptr ? cf[e] * c : c));
   }
 
   f32x16 oacc[MB];
@@ -593,10 +597,23 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
     for (int j = 0; j < 16; ++j) oacc[mb][j] = 0.f;
-  float m_run = -INFINITY;
-  float l_run = 0.f;
-  float c = p.scale_log2;  // SCALED: the query's row factor joins the lane's softmax scale
-  if (SCALED && p.q_row_scale != nullptr && qi < q_valid) c *= p.q_row_scale[static_cast<int64_t>(b) * p.Tq + qi];
+  // Softmax with a lazily moved reference: the exponent's offset -m is the C operand of the first score product (sixteen
+  // equal registers), so a tile arrives as s - m and goes straight into exp2; m is moved (and the accumulators rescaled)
+  // only when a score exceeds it by more than kLazyBits, which keeps every probability below 2^kLazyBits - exact in the
+  // float32 accumulators and neutral for the relative rounding of the 16-bit probabilities. The row sums are a product
+  // with a fragment of ones (all sixteen registers of lacc hold the sum over the keys of both lanes of the query).
+  constexpr float kLazyBits = 8.f;
+  f32x16 negm, lacc;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    negm[j] = 0.f;
+    lacc[j] = 0.f;
+  }
+  bool m_set = false;                 // the query has seen a visible key (its reference is meaningful)
+  float thr = -3.0e38f;               // the lane's tile maximum above this moves the reference: any finite score at first
+  vec_t ones_frag;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ones_frag[e] = static_cast<T>(1.0f);
   int wave_kv_end = kv_end;
   if (CAUSAL) {
     const int wlim = q_begin + wave * 32 + 32;
@@ -624,14 +641,19 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   const bool scale_keys = SCALED && p.k_row_scale != nullptr;
   vec_t kreg[SCALED ? PPT : 1];
   float kfac[SCALED ? PPT : 1];
-  uint32_t mw_next[2] = {0u, 0u}, mw[2] = {0u, 0u};
+  // mask words of the two chunks in flight (even / odd chunk) and of the chunk being consumed
+  uint32_t mw_even[2] = {0u, 0u}, mw_odd[2] = {0u, 0u}, mw[2] = {0u, 0u};
   auto issue = [&](int chunk, int buffer) {
     if (MASKED) {
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt) {
         const int w = chunk * 2 + kt;
-        mw_next[kt] = (qi < q_valid && w < p.wpr)
-                          ? p.struct_bits[b * p.struct_stride + static_cast<int64_t>(qi) * p.wpr + w] : 0u;
+        const uint32_t word = (qi < q_valid && w < p.wpr)
+                                  ? p.struct_bits[b * p.struct_stride + static_cast<int64_t>(qi) * p.wpr + w] : 0u;
+        if (chunk & 1)
+          mw_odd[kt] = word;
+        else
+          mw_even[kt] = word;
       }
     }
 #pragma unroll
@@ -677,34 +699,44 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
     issue(0, 0);
     commit_keys(0);
   }
+  if (nchunks > 1) {
+    issue(1, 1);
+    commit_keys(1);
+  }
   int buf = 0;
-  for (int chunk = 0; chunk < nchunks; ++chunk) {
-    vm_wait<0>();     // this wavefront's pieces of the chunk have landed ...
-    __syncthreads();  // ... everyone's have, and everyone is done reading the other buffer
+  // transfers (and mask words) of one chunk per wavefront: what may stay in flight while the chunk before it is awaited.
+  // With key factors the keys pass through registers and are waited for when they are committed: wait for everything.
+  constexpr int kInFlight = 2 * PPT + (MASKED ? 2 : 0);
+  // One chunk: wait for its transfers, publish them, start the next chunk's, then (NT > 0) take the chunk's first NT key
+  // tiles into the running softmax. NT is a compile-time property of the call site: a wavefront sees whole chunks first,
+  // then at most one chunk of which only the first tile holds visible keys, then chunks that only the other wavefronts of
+  // the workgroup still need - three straight-line loops instead of one loop whose paths merge the accumulators.
+  auto step = [&](int chunk, auto nt_tag) {
+    constexpr int NT = decltype(nt_tag)::value;
+    // this wavefront's pieces of the chunk have landed (the next chunk's, issued after them, may still be in flight) ...
+    if (chunk + 1 < nchunks && !scale_keys)
+      vm_wait<kInFlight>();
+    else
+      vm_wait<0>();
+    __syncthreads();  // ... everyone's have, and everyone is done reading the buffer of the chunk before
     if (MASKED) {
-      mw[0] = mw_next[0];
-      mw[1] = mw_next[1];
+      mw[0] = (chunk & 1) ? mw_odd[0] : mw_even[0];
+      mw[1] = (chunk & 1) ? mw_odd[1] : mw_even[1];
     }
-    const bool more = chunk + 1 < nchunks;
-    if (more) issue(chunk + 1, buf ^ 1);
+    const bool more = chunk + 2 < nchunks;
+    const int ahead = buf == 0 ? 2 : buf - 1;  // (buf + 2) % 3
+    if (more) issue(chunk + 2, ahead);
     const int kc0 = chunk * kKC;
     const uint32_t base = smem_off + buf * BUF_BYTES;
-    buf ^= 1;
-    if (kc0 >= wave_kv_end) {  // wavefront-uniform: nothing visible in this chunk
-      if (more) commit_keys(buf);
-      continue;
-    }
-    auto update = [&](auto nt_tag) {
-      constexpr int NT = decltype(nt_tag)::value;
+    buf = buf == 2 ? 0 : buf + 1;
+    if constexpr (NT > 0) {
       f32x16 sacc[NT];
 #pragma unroll
       for (int kt = 0; kt < NT; ++kt) {
 #pragma unroll
-        for (int j = 0; j < 16; ++j) sacc[kt][j] = 0.f;
-#pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
           const vec_t a = *reinterpret_cast<const vec_t*>(smem + (base - smem_off) + kt * 32 * ROWB + (k_off0 ^ (s * 32)));
-          sacc[kt] = Mfma32<T>::run(a, qf[s], sacc[kt]);
+          sacc[kt] = Mfma32<T>::run(a, qf[s], s == 0 ? negm : sacc[kt]);
         }
       }
       const int k_last = kc0 + NT * 32;
@@ -738,25 +770,43 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
       for (int kt = 0; kt < NT; ++kt)
 #pragma unroll
         for (int j = 0; j < 16; ++j) mx = fmaxf(mx, sacc[kt][j]);
-      mx = pair_max(mx);
-      const float m_new = fmaxf(m_run, mx);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
-      const float mc = -m_use * c;
-      float rs = 0.f;
+      if (__builtin_amdgcn_ballot_w64(mx > thr) != 0) {  // wavefront-uniform, rare after a query's first tile
+        // Both lanes of a query decide on the pair's maximum, so they keep one reference between them.
+        const float mxp = pair_max(mx);
+        const bool move = mxp > thr;
+        const float shift = move ? mxp : 0.f;
+        const float alpha = (move && m_set) ? __builtin_amdgcn_exp2f(-mxp) : 1.f;
+#pragma unroll
+        for (int kt = 0; kt < NT; ++kt)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) sacc[kt][j] -= shift;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          negm[j] -= shift;
+          lacc[j] *= alpha;
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;
+        if (move) {
+          m_set = true;
+          thr = kLazyBits;
+        }
+      }
       vec_t pb[NT][2];
 #pragma unroll
       for (int kt = 0; kt < NT; ++kt) {
         float pr[16];
 #pragma unroll
-        for (int j = 0; j < 16; ++j) pr[j] = __builtin_amdgcn_exp2f(fmaf(sacc[kt][j], c, mc));
+        for (int j = 0; j < 16; ++j) pr[j] = __builtin_amdgcn_exp2f(sacc[kt][j]);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           pb[kt][0][e] = static_cast<T>(pr[e]);
           pb[kt][1][e] = static_cast<T>(pr[8 + e]);
         }
-        rs = frag_sum(pb[kt][0], rs);
-        rs = frag_sum(pb[kt][1], rs);
+        lacc = Mfma32<T>::run(ones_frag, pb[kt][0], lacc);
+        lacc = Mfma32<T>::run(ones_frag, pb[kt][1], lacc);
       }
       // V fragments of one row block at a time: requested once the scores are dead (registers), in flight during the
       // bookkeeping below
@@ -770,13 +820,6 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
           lds_read_tr16<(kt * 32 + s2 * 16) * ROWB>(vt[kt][s2][0], v_addr_mb);
           lds_read_tr16<(kt * 32 + s2 * 16 + 8) * ROWB>(vt[kt][s2][1], v_addr_mb);
         });
-        if (mb == 0) {
-          rs = pair_sum(rs);
-          l_run = l_run * alpha + rs;
-          m_run = m_new;
-        }
-#pragma unroll
-        for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;  // unconditional, see the general kernel
         // the transposed reads were issued by hand: wait for them by hand (everything of this wavefront's LDS queue);
         // the fragments are tied to the wait so that their consumers cannot be scheduled above it
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vt[0][0][0]) : : "memory");
@@ -795,19 +838,25 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
             oacc[mb] = Mfma32<T>::run(__builtin_bit_cast(vec_t, bits), pb[kt][s2], oacc[mb]);
           }
       });
-    };
-    if (kc0 + 32 < wave_kv_end)
-      update(std::integral_constant<int, 2>{});
-    else
-      update(std::integral_constant<int, 1>{});
-    if (more) commit_keys(buf);  // the next chunk's K, fetched before the update: the barrier above publishes it
+    }
+    if (more) commit_keys(ahead);  // that chunk's K, fetched before the update: the next barrier publishes it
+  };
+  // chunks of which both tiles hold keys visible to this wavefront: 64 * chunk + 32 < wave_kv_end
+  const int whole = wave_kv_end >= 33 ? (wave_kv_end - 33) / kKC + 1 : 0;
+  int chunk = 0;
+  for (; chunk < whole; ++chunk) step(chunk, std::integral_constant<int, 2>{});
+  if (chunk < nchunks && chunk * kKC < wave_kv_end) {
+    step(chunk, std::integral_constant<int, 1>{});
+    ++chunk;
   }
+  for (; chunk < nchunks; ++chunk) step(chunk, std::integral_constant<int, 0>{});
 
+  const float l_run = lacc[0];
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
   const float fin = (qi < q_valid) ? inv : 0.f;
   if (p.lse != nullptr && hh == 0 && qi < p.Tq)
     p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Tq + qi] =
-        (qi < q_valid && l_run > 0.f) ? (m_run * c + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f : -INFINITY;
+        (qi < q_valid && l_run > 0.f) ? (__builtin_amdgcn_logf(l_run) - negm[0]) * 0.6931471805599453f : -INFINITY;
   __syncthreads();  // every wavefront is done with the chunk buffers: they now hold the output tiles
   uint8_t* tile = smem + wave * (32 * OROW);
   float omax = 0.f;

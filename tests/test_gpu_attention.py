@@ -213,11 +213,13 @@ def test_row_factors_of_queries_and_keys(device, dim, tokens, causal):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("head_dim", [32, 64])
 @pytest.mark.parametrize("causal", [False, True])
-def test_direct_transfer_kernel_equals_general_kernel_bit_for_bit(device, dtype, head_dim, causal):
+def test_direct_transfer_kernel_agrees_with_general_kernel(device, dtype, head_dim, causal):
     """Head dims 32 and 64 run a kernel that stages K and V by direct global->LDS transfers (swizzled rows, transposed
-    LDS reads); kv_staging="registers" selects the general kernel. Same arithmetic in the same order: identical
-    results, for ragged lengths (0, 1, not a multiple of the chunk), strided views of a packed projection, row factors
-    and the log-sum-exp output of the training forward."""
+    LDS reads) and a softmax whose reference moves lazily (query pre-multiplied by the softmax scale, row sums through the
+    matrix unit); kv_staging="registers" selects the general kernel with the textbook running maximum. The two differ by
+    one more rounding of the scaled query and by the order of the sums: a few steps of the storage type, for ragged
+    lengths (0, 1, not a multiple of the chunk), strided views of a packed projection and row factors. Rows a kernel must
+    not touch or must zero are identical."""
     from taac_2026_amd.api import flash_attention
     from taac_2026_amd.accelerators.attention import hip_flash_attention_kernel
 
@@ -242,8 +244,12 @@ def test_direct_transfer_kernel_equals_general_kernel_bit_for_bit(device, dtype,
 
     direct = run("direct")
     general = run("registers")
+    step = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
     for a, b in zip(direct, general):
-        assert torch.equal(a, b)
+        torch.testing.assert_close(a.float(), b.float(), rtol=4 * step, atol=4 * step)
+        assert torch.equal(a == 0, b == 0) or (a.float() - b.float()).abs().max().item() <= 4 * step
+    padded = torch.arange(tokens, device=device)[None, :] >= lengths[:, None]
+    assert (direct[0].transpose(1, 2)[padded] == 0).all() and (direct[2].transpose(1, 2)[padded] == 0).all()
 
 
 @pytest.mark.parametrize("head_dim,zero_pad", [(32, 2), (64, 1), (16, 0)])
