@@ -60,7 +60,21 @@ struct AttnParams {
   int32_t zero_pad;
   uint32_t nqc;    // query chunks per (batch, head)
   uint32_t total;  // workgroups
+  uint32_t nqc_magic, h_magic;  // floor(2^32 / nqc), floor(2^32 / H) (0 for a divisor of 1): divisions without a divide
 };
+
+// x / d and x % d for a divisor known to the host: q = mulhi(x, floor(2^32 / d)) is at most two short of the quotient.
+__device__ __forceinline__ void magic_divmod(uint32_t x, uint32_t d, uint32_t magic, uint32_t& q, uint32_t& r) {
+  q = magic == 0u ? x : __umulhi(x, magic);
+  r = x - q * d;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    if (r >= d) {
+      ++q;
+      r -= d;
+    }
+}
+inline uint32_t magic_of(uint32_t d) { return d <= 1u ? 0u : static_cast<uint32_t>((1ull << 32) / d); }
 
 template <typename T>
 struct Mfma32;
@@ -537,10 +551,10 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   __shared__ __attribute__((aligned(1024))) uint8_t smem[NBUF * BUF_BYTES > OT_BYTES ? NBUF * BUF_BYTES : OT_BYTES];
 
   const uint32_t logical = xcd_remap(blockIdx.x, p.total);
-  const int qc = static_cast<int>(logical % p.nqc);
-  const int bh = static_cast<int>(logical / p.nqc);
-  const int h = bh % p.H;
-  const int b = bh / p.H;
+  uint32_t bh_u, qc_u, b_u, h_u;
+  magic_divmod(logical, p.nqc, p.nqc_magic, bh_u, qc_u);
+  magic_divmod(bh_u, static_cast<uint32_t>(p.H), p.h_magic, b_u, h_u);
+  const int qc = static_cast<int>(qc_u), h = static_cast<int>(h_u), b = static_cast<int>(b_u);
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int lane = tid % kWave;
@@ -600,20 +614,15 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   // Softmax with a lazily moved reference: the exponent's offset -m is the C operand of the first score product (sixteen
   // equal registers), so a tile arrives as s - m and goes straight into exp2; m is moved (and the accumulators rescaled)
   // only when a score exceeds it by more than kLazyBits, which keeps every probability below 2^kLazyBits - exact in the
-  // float32 accumulators and neutral for the relative rounding of the 16-bit probabilities. The row sums are a product
-  // with a fragment of ones (all sixteen registers of lacc hold the sum over the keys of both lanes of the query).
+  // float32 accumulators and neutral for the relative rounding of the 16-bit probabilities. Each lane sums the rounded
+  // probabilities of its own keys; the two lanes of a query are added once, at the end.
   constexpr float kLazyBits = 8.f;
-  f32x16 negm, lacc;
+  f32x16 negm;
 #pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    negm[j] = 0.f;
-    lacc[j] = 0.f;
-  }
+  for (int j = 0; j < 16; ++j) negm[j] = 0.f;
+  float l_lane = 0.f;
   bool m_set = false;                 // the query has seen a visible key (its reference is meaningful)
   float thr = -3.0e38f;               // the lane's tile maximum above this moves the reference: any finite score at first
-  vec_t ones_frag;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) ones_frag[e] = static_cast<T>(1.0f);
   int wave_kv_end = kv_end;
   if (CAUSAL) {
     const int wlim = q_begin + wave * 32 + 32;
@@ -742,13 +751,15 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
       const int k_last = kc0 + NT * 32;
       const bool tail = (k_last > kv_end) || (CAUSAL && (k_last - 1 > q_begin + wave * 32));
       if (tail) {
+        // register j of tile kt is key kc0 + hh * 4 + (kt * 32 + (j / 4) * 8 + j % 4): one lane-dependent limit, then a
+        // compare against a constant per register
+        int lim = kv_end - kc0 - hh * 4;
+        if (CAUSAL) lim = min(lim, qi + 1 - kc0 - hh * 4);
 #pragma unroll
         for (int kt = 0; kt < NT; ++kt)
 #pragma unroll
-          for (int j = 0; j < 16; ++j) {
-            const int key = kc0 + kt * 32 + (j / 4) * 8 + hh * 4 + (j % 4);
-            if (key >= kv_end || (CAUSAL && key > qi)) sacc[kt][j] = -INFINITY;
-          }
+          for (int j = 0; j < 16; ++j)
+            sacc[kt][j] = (kt * 32 + (j / 4) * 8 + (j % 4)) < lim ? sacc[kt][j] : -INFINITY;
       }
       if (MASKED) {
         // Accumulator register j of the lane is key (j / 4) * 8 + hh * 4 + j % 4 of the tile: bit of the lane's word.
@@ -781,10 +792,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
 #pragma unroll
           for (int j = 0; j < 16; ++j) sacc[kt][j] -= shift;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          negm[j] -= shift;
-          lacc[j] *= alpha;
-        }
+        for (int j = 0; j < 16; ++j) negm[j] -= shift;
+        l_lane *= alpha;
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -805,8 +814,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
           pb[kt][0][e] = static_cast<T>(pr[e]);
           pb[kt][1][e] = static_cast<T>(pr[8 + e]);
         }
-        lacc = Mfma32<T>::run(ones_frag, pb[kt][0], lacc);
-        lacc = Mfma32<T>::run(ones_frag, pb[kt][1], lacc);
+        l_lane = frag_sum(pb[kt][0], l_lane);
+        l_lane = frag_sum(pb[kt][1], l_lane);
       }
       // V fragments of one row block at a time: requested once the scores are dead (registers), in flight during the
       // bookkeeping below
@@ -851,7 +860,7 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   }
   for (; chunk < nchunks; ++chunk) step(chunk, std::integral_constant<int, 0>{});
 
-  const float l_run = lacc[0];
+  const float l_run = pair_sum(l_lane);
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
   const float fin = (qi < q_valid) ? inv : 0.f;
   if (p.lse != nullptr && hh == 0 && qi < p.Tq)
@@ -1063,6 +1072,8 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   const int64_t total = static_cast<int64_t>(p.nqc) * B * H;
   if (total > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many workgroups (%lld)", name, (long long)total);
   p.total = static_cast<uint32_t>(total);
+  p.nqc_magic = magic_of(p.nqc);
+  p.h_magic = magic_of(static_cast<uint32_t>(H));
 
   hipStream_t s = as_stream(stream);
   if (dtype == TAAC_BF16)
