@@ -76,23 +76,47 @@ def test_backward_is_reproducible_and_reads_the_projection_layout(device):
 @pytest.mark.parametrize("dim,causal", [(32, False), (64, False), (64, True)])
 def test_direct_transfer_backward_equals_register_staged_backward(device, dim, causal):
     """Full head dims stream their chunks from global memory straight into LDS, where rows beyond the valid length repeat
-    the last valid row instead of zeros; their products are cancelled by zero probabilities, so both routes give the
-    same bits (``kv_staging`` selects the route of the training forward and of its backward; the forwards are
-    bit-identical, see test_gpu_attention.py)."""
+    the last valid row instead of zeros; their products are cancelled by zero probabilities, so both backward routes give
+    the same bits from the same saved forward (taac_flash_attn_bwd through the C ABI with and without
+    TAAC_ATTN_REGISTER_STAGING; the two forwards differ by roundings, see test_gpu_attention.py, so one forward feeds
+    both)."""
+    from taac_2026_amd import _native
+
     batch, heads, tokens = 5, 2, 333
     g = torch.Generator().manual_seed(dim + causal)
     q, k, v, grad_out = (torch.randn(batch, heads, tokens, dim, generator=g).to(torch.bfloat16).to(device) for _ in range(4))
     lengths = torch.tensor([333, 1, 64, 65, 200], dtype=torch.int32, device=device)
+    library = _native.load_library()
+    stream = _native.current_stream(q.device)
+    out = torch.empty_like(q)
+    lse = torch.empty(batch, heads, tokens, dtype=torch.float32, device=device)
+    strides = lambda *ts: [_native.Int64x4(*t.stride()) for t in ts]  # noqa: E731
+    flags = _native.ATTN_CAUSAL if causal else 0
+    zero_pad = int(not causal)
+    _native.check(library.taac_flash_attn_train_fwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), lengths.data_ptr(), out.data_ptr(), lse.data_ptr(), batch, heads, tokens,
+        tokens, dim, *strides(q, k, v, out), flags, zero_pad, _native.dtype_code(q.dtype), stream), "train_fwd")
     grads = {}
-    for staging in ("direct", "registers"):
-        qd, kd, vd = (t.clone().requires_grad_(True) for t in (q, k, v))
-        out = flash_attention(qd, kd, vd, key_lengths=lengths, is_causal=causal, zero_padded_queries=not causal,
-                              kv_staging=staging)
-        out.backward(grad_out)
-        grads[staging] = (qd.grad, kd.grad, vd.grad)
+    for name, route in (("direct", 0), ("registers", _native.ATTN_REGISTER_STAGING)):
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        delta = torch.empty_like(lse)
+        _native.check(library.taac_flash_attn_bwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), grad_out.data_ptr(), lse.data_ptr(),
+            lengths.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(), batch, heads, tokens, tokens,
+            dim, *strides(q, k, v, out, grad_out, dq, dk, dv), flags | route, zero_pad, _native.dtype_code(q.dtype), stream),
+            "bwd")
+        grads[name] = (dq, dk, dv)
     for direct, staged in zip(grads["direct"], grads["registers"]):
         assert torch.isfinite(direct.float()).all()
         assert torch.equal(direct, staged)
+    # and the module-level route switch reaches both kernels: gradients of the two routes agree to rounding
+    for staging in ("direct", "registers"):
+        qd, kd, vd = (t.clone().requires_grad_(True) for t in (q, k, v))
+        flash_attention(qd, kd, vd, key_lengths=lengths, is_causal=causal, zero_padded_queries=not causal,
+                        kv_staging=staging).backward(grad_out)
+        for got, want in zip((qd.grad, kd.grad, vd.grad), grads["direct"]):
+            # (a step or two of bf16 at the largest gradients: the two forwards round differently)
+            torch.testing.assert_close(got.float(), want.float(), rtol=2 ** -5, atol=2 ** -6 * want.float().abs().max().item())
 
 
 def test_backward_envelope(device):
