@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define TAAC_ABI_VERSION 5
+#define TAAC_ABI_VERSION 6
 
 enum taac_status {
   TAAC_OK = 0,
@@ -229,6 +229,30 @@ int taac_flash_attn_bwd(const void* q, const void* k, const void* v, const void*
                         const int64_t v_strides[4], const int64_t o_strides[4], const int64_t do_strides[4],
                         const int64_t dq_strides[4], const int64_t dk_strides[4], const int64_t dv_strides[4],
                         int is_causal, int zero_padded_queries, int dtype, void* stream);
+
+/*
+ * Training forward and backward with dropout on the attention probabilities, the mask supplied by the caller:
+ * dropout_mask is uint8 [B, H, Tq, Tk] contiguous (non-zero = keep), dropout_scale = 1 / (1 - p) >= 1. The softmax
+ * normaliser and lse are those of the undropped probabilities; out = ((keep ? P * dropout_scale : 0) V); the backward
+ * forms dV from the dropped probabilities and dS = P * ((keep ? dP * dropout_scale : 0) - D) / sqrt(d) with
+ * D = rowsum(dO * out). Every other argument as in taac_flash_attn_train_fwd / taac_flash_attn_bwd (key-length and
+ * causal masks; the backward for head dims up to 64).
+ * Replaces: flash_attention_training_forward_kernel / flash_attention_backward_kernel with use_dropout
+ * (infrastructure/accelerators/attention/kernels/tilelang.py:165-283, 463-597); the mask is the one
+ * _build_tilelang_dropout_mask draws (attention/flash_attention.py:316-325).
+ */
+int taac_flash_attn_train_dropout_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
+                                      const uint8_t* dropout_mask, float dropout_scale, void* o, float* lse, int32_t B,
+                                      int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
+                                      const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4],
+                                      int is_causal, int zero_padded_queries, int dtype, void* stream);
+int taac_flash_attn_dropout_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout,
+                                const float* lse, const int32_t* key_lengths, const uint8_t* dropout_mask,
+                                float dropout_scale, void* dq, void* dk, void* dv, float* delta, int32_t B, int32_t H,
+                                int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
+                                const int64_t v_strides[4], const int64_t o_strides[4], const int64_t do_strides[4],
+                                const int64_t dq_strides[4], const int64_t dk_strides[4], const int64_t dv_strides[4],
+                                int is_causal, int zero_padded_queries, int dtype, void* stream);
 
 /*
  * Dense layer, bf16 storage / bf16 MFMA / fp32 accumulation: out = epilogue(a @ w^T + bias).

@@ -182,6 +182,34 @@ def attention(
     return out.to(v.dtype)
 
 
+def attention_dropout(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, key_lengths: torch.Tensor | None,
+                      dropout_mask: torch.Tensor, dropout_p: float, *, is_causal: bool = False,
+                      zero_padded_queries: bool = False) -> torch.Tensor:
+    """Training attention with dropout on the probabilities under a fixed keep mask, (B, H, T, d) tensors:
+    ``softmax(scores)`` over the visible keys, then ``P * keep / (1 - p)``, then ``@ v`` - the semantics of the
+    reference's training kernel (attention/kernels/tilelang.py:224-247: the normaliser sums the undropped probabilities)
+    and of the manual reference its own test compares with
+    (tests/gpu/infrastructure/accelerators/test_tilelang_ops_cuda.py:103-141). Differentiable; evaluate in float64 for
+    gradient targets. Rows without a visible key give 0."""
+    batch, heads, query_len, dim = q.shape
+    kv_len = k.shape[2]
+    scores = torch.matmul(q, k.transpose(-1, -2)) * (dim ** -0.5)
+    visible = torch.ones(batch, 1, query_len, kv_len, dtype=torch.bool)
+    if key_lengths is not None:
+        visible = visible & (torch.arange(kv_len)[None, None, None, :] < key_lengths.to(torch.int64)[:, None, None, None])
+    if is_causal:
+        visible = visible & (torch.arange(kv_len)[None, None, None, :] <= torch.arange(query_len)[None, None, :, None])
+    scores = scores.masked_fill(~visible, float("-inf"))
+    probs = torch.softmax(scores, dim=-1)
+    probs = torch.where(visible.any(dim=-1, keepdim=True), probs, torch.zeros_like(probs))
+    probs = probs * dropout_mask.to(probs.dtype) / (1.0 - dropout_p)
+    out = torch.matmul(probs, v)
+    if zero_padded_queries and key_lengths is not None:
+        keep_rows = torch.arange(query_len)[None, :] < key_lengths.to(torch.int64)[:, None]
+        out = out * keep_rows[:, None, :, None].to(out.dtype)
+    return out
+
+
 def scaled_dot_product_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, num_heads: int,
                                  key_lengths: torch.Tensor | None = None, zero_padded_queries: bool = False) -> torch.Tensor:
     """modeling/sequence.py:81-116 on (B, T, D) projections, with the key-length mask."""

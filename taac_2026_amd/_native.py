@@ -24,7 +24,7 @@ EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
 ATTN_CAUSAL, ATTN_REGISTER_STAGING = 1, 2
 BACKBONE_DENSE_TOKENS, BACKBONE_SPLIT_OUT_FFN, BACKBONE_FP8 = 1, 2, 4
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _DTYPE_CODES = {torch.float32: TAAC_F32, torch.bfloat16: TAAC_BF16, torch.float16: TAAC_F16}
 
@@ -115,6 +115,18 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "taac_flash_attn_bwd": (
         c_int,
         [c_void_p] * 11 + [c_int32, c_int32, c_int32, c_int32, c_int32]
+        + [ctypes.POINTER(c_int64)] * 8
+        + [c_int, c_int, c_int, c_void_p],
+    ),
+    "taac_flash_attn_train_dropout_fwd": (
+        c_int,
+        [c_void_p] * 5 + [c_float] + [c_void_p] * 2 + [c_int32, c_int32, c_int32, c_int32, c_int32]
+        + [ctypes.POINTER(c_int64)] * 4
+        + [c_int, c_int, c_int, c_void_p],
+    ),
+    "taac_flash_attn_dropout_bwd": (
+        c_int,
+        [c_void_p] * 8 + [c_float] + [c_void_p] * 4 + [c_int32, c_int32, c_int32, c_int32, c_int32]
         + [ctypes.POINTER(c_int64)] * 8
         + [c_int, c_int, c_int, c_void_p],
     ),

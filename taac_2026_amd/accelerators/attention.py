@@ -12,6 +12,8 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
+import ctypes
+
 import torch
 
 from taac_2026_amd import _native
@@ -281,8 +283,8 @@ def _resolve_flash_attention_backend(q: torch.Tensor, backend: str, *, dropout_p
         raise ValueError(f"unsupported flash attention backend: {backend}")
     if dropout_p < 0.0 or dropout_p >= 1.0:
         raise RuntimeError("hip flash_attention requires dropout_p to be in [0, 1)")
-    if training and dropout_p != 0.0:
-        raise RuntimeError("hip flash_attention is forward-only inference and does not apply dropout")
+    if dropout_p != 0.0 and not training:
+        raise RuntimeError("hip flash_attention only supports dropout during training")
     require_cuda_tensors("hip flash_attention", q)
     return "hip"
 
@@ -428,50 +430,84 @@ def _dense_like(t: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def build_dropout_mask(q: torch.Tensor, k: torch.Tensor, dropout_p: float) -> torch.Tensor:
+    """uint8 keep mask (B, H, Tq, Tk) drawn as the reference's ``_build_tilelang_dropout_mask`` does
+    (attention/flash_attention.py:316-325): ``rand >= p``."""
+    if not 0.0 < dropout_p < 1.0:
+        raise RuntimeError("hip flash_attention requires dropout_p to be in [0, 1)")
+    return (torch.rand((q.shape[0], q.shape[1], q.shape[2], k.shape[2]), device=q.device) >= dropout_p).to(torch.uint8).contiguous()
+
+
 class _HipFlashAttentionFunction(torch.autograd.Function):
-    """Training path (key-length mask, optional causal triangle): the forward also saves the log-sum-exp of every query
-    row, the backward runs the two HIP backward kernels (the role of the reference's TileLang training functions,
-    flash_attention.py:397-525)."""
+    """Training path (key-length mask, optional causal triangle, optional dropout with a caller-supplied keep mask): the
+    forward also saves the log-sum-exp of every query row, the backward runs the two HIP backward kernels (the role of
+    the reference's TileLang training functions, flash_attention.py:397-525, 575-650)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, key_lengths, is_causal: bool, zero_padded_queries: bool, kv_staging: str = "direct"):
+    def forward(ctx, q, k, v, key_lengths, is_causal: bool, zero_padded_queries: bool, kv_staging: str = "direct",
+                dropout_mask: torch.Tensor | None = None, dropout_p: float = 0.0):
         library = _native.load_library()
         q, k, v = _kernel_view(q), _kernel_view(k), _kernel_view(v)
         out = _dense_like(q)
         batch, heads, query_len, head_dim = q.shape
         lse = torch.empty(batch, heads, query_len, dtype=torch.float32, device=q.device)
-        status = library.taac_flash_attn_train_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), out.data_ptr(), lse.data_ptr(),
-            batch, heads, query_len, k.shape[2], head_dim,
-            _native.Int64x4(*q.stride()), _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()),
-            _native.Int64x4(*out.stride()), _mask_flags(is_causal, kv_staging), int(bool(zero_padded_queries)),
-            _native.dtype_code(q.dtype), _native.current_stream(q.device),
-        )
+        shape = (batch, heads, query_len, k.shape[2], head_dim)
+        strides = (_native.Int64x4(*q.stride()), _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()),
+                   _native.Int64x4(*out.stride()))
+        tail = (_mask_flags(is_causal, kv_staging), int(bool(zero_padded_queries)), _native.dtype_code(q.dtype),
+                _native.current_stream(q.device))
+        scale = 1.0
+        if dropout_mask is not None:
+            if dropout_mask.dtype != torch.uint8 or tuple(dropout_mask.shape) != (batch, heads, query_len, k.shape[2]):
+                raise ValueError("flash_attention dropout_mask must be uint8 of shape (B, H, Tq, Tk)")
+            require_cuda_tensors("hip flash_attention", dropout_mask)
+            dropout_mask = dropout_mask.contiguous()
+            scale = 1.0 / (1.0 - dropout_p)
+            status = library.taac_flash_attn_train_dropout_fwd(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), dropout_mask.data_ptr(),
+                ctypes.c_float(scale), out.data_ptr(), lse.data_ptr(), *shape, *strides, *tail)
+        else:
+            status = library.taac_flash_attn_train_fwd(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), out.data_ptr(), lse.data_ptr(),
+                *shape, *strides, *tail)
         _native.check(status, "flash_attention")
-        ctx.save_for_backward(q, k, v, out, lse, *(() if key_lengths is None else (key_lengths,)))
+        saved = [q, k, v, out, lse]
         ctx.has_lengths = key_lengths is not None
+        ctx.has_dropout = dropout_mask is not None
+        if ctx.has_lengths:
+            saved.append(key_lengths)
+        if ctx.has_dropout:
+            saved.append(dropout_mask)
+        ctx.save_for_backward(*saved)
+        ctx.dropout_scale = scale
         ctx.flags = (_mask_flags(is_causal, kv_staging), bool(zero_padded_queries))
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
         library = _native.load_library()
-        saved = ctx.saved_tensors
+        saved = list(ctx.saved_tensors)
         q, k, v, out, lse = saved[:5]
-        key_lengths = saved[5] if ctx.has_lengths else None
+        rest = saved[5:]
+        key_lengths = rest.pop(0) if ctx.has_lengths else None
+        dropout_mask = rest.pop(0) if ctx.has_dropout else None
         grad_out = _kernel_view(grad_out)
         dq, dk, dv = _dense_like(q), _dense_like(k), _dense_like(v)
         delta = torch.empty_like(lse)
         batch, heads, query_len, head_dim = q.shape
         strides = [_native.Int64x4(*t.stride()) for t in (q, k, v, out, grad_out, dq, dk, dv)]
-        status = library.taac_flash_attn_bwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), grad_out.data_ptr(), lse.data_ptr(),
-            _native.ptr(key_lengths), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(),
-            batch, heads, query_len, k.shape[2], head_dim, *strides, int(ctx.flags[0]), int(ctx.flags[1]),
-            _native.dtype_code(q.dtype), _native.current_stream(q.device),
-        )
+        head = (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), grad_out.data_ptr(), lse.data_ptr(),
+                _native.ptr(key_lengths))
+        tail = (dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(), batch, heads, query_len, k.shape[2],
+                head_dim, *strides, int(ctx.flags[0]), int(ctx.flags[1]), _native.dtype_code(q.dtype),
+                _native.current_stream(q.device))
+        if dropout_mask is not None:
+            status = library.taac_flash_attn_dropout_bwd(*head, dropout_mask.data_ptr(), ctypes.c_float(ctx.dropout_scale),
+                                                         *tail)
+        else:
+            status = library.taac_flash_attn_bwd(*head, *tail)
         _native.check(status, "flash_attention backward")
-        return dq, dk, dv, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None, None
 
 
 def flash_attention(
@@ -495,8 +531,13 @@ def flash_attention(
     q_col_scale: torch.Tensor | None = None,
     structured_mask: StructuredAttentionMask | None = None,
     kv_staging: str = "direct",
+    dropout_mask: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """``softmax(q k^T / sqrt(d) + mask) v`` for (B, H, T, d) tensors.
+
+    ``dropout_p`` with ``training=True`` drops attention probabilities as the reference's training kernels do: a uint8
+    keep mask (B, H, Tq, Tk) - ``dropout_mask`` if given, else drawn by :func:`build_dropout_mask` - multiplies the
+    probabilities by ``keep / (1 - p)`` behind the softmax normaliser (flash_attention.py:316-325, 575-650).
 
     ``attn_mask`` is a bool mask with True = attend (structured as described in :func:`plan_flash_attention_mask`);
     ``key_lengths`` (int32 [B]) states the valid key prefix directly and excludes ``attn_mask``.
@@ -514,6 +555,10 @@ def flash_attention(
     q, k, v = _normalize_flash_attention_inputs(q, k, v)
     _resolve_flash_attention_backend(q, backend, dropout_p=dropout_p, training=training)
     needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v))
+    use_dropout = training and dropout_p > 0.0
+    if use_dropout and (structured_mask is not None or q_row_scale is not None or k_row_scale is not None
+                        or q_col_scale is not None):
+        raise RuntimeError("hip flash_attention dropout covers key-length and causal masks only")
     if needs_grad and (structured_mask is not None or q_row_scale is not None or k_row_scale is not None
                        or q_col_scale is not None or q.dtype == torch.float32):
         raise RuntimeError("hip flash_attention backward covers bf16 / fp16 inputs under key-length and causal masks only; "
@@ -538,15 +583,19 @@ def flash_attention(
     if q.dtype == torch.float32:
         q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
     lengths = plan.key_lengths if (plan.key_lengths is not None and (attn_mask is not None or key_lengths is not None)) else None
-    if needs_grad:
+    if needs_grad or use_dropout:
         if structured_mask is not None:
-            raise RuntimeError("hip flash_attention backward does not cover structured masks")
+            raise RuntimeError("hip flash_attention backward and dropout do not cover structured masks")
         if lengths is not None:
             lengths = lengths.to(torch.int32).contiguous()
-        output = _HipFlashAttentionFunction.apply(q, k, v, lengths, plan.is_causal, zero_padded_queries, kv_staging)
+        mask = None
+        if use_dropout:
+            mask = dropout_mask if dropout_mask is not None else build_dropout_mask(q, k, dropout_p)
+        output = _HipFlashAttentionFunction.apply(q, k, v, lengths, plan.is_causal, zero_padded_queries, kv_staging, mask,
+                                                  float(dropout_p) if use_dropout else 0.0)
         if plan.query_self_mask is not None:
             output = torch.where(plan.query_self_mask[:, None, :, None], v, output)
-        return output
+        return output if output.dtype == output_dtype else output.to(output_dtype)
     output = hip_flash_attention_kernel(
         q, k, v, lengths, is_causal=plan.is_causal, zero_padded_queries=zero_padded_queries,
         q_row_scale=q_row_scale, k_row_scale=k_row_scale, q_col_scale=q_col_scale, structured_mask=structured_mask,

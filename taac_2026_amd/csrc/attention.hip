@@ -44,6 +44,8 @@ struct AttnParams {
   const float* k_row_scale;
   const float* q_col_scale;  // [H, d] factors of the query features, or null
   float* amax_out;           // receives max |o| over everything written (atomic max), or null
+  const uint8_t* drop_mask;  // training dropout: [B, H, Tq, Tk] keep mask (non-zero = keep), or null
+  float drop_scale;          // 1 / (1 - p)
   // Structured mask: key j is visible to query i of sample b iff bit j of struct_bits[i] and of valid_bits[b] is set.
   const uint32_t* struct_bits;  // [Tq][wpr] words, bit j % 32 of word j / 32; null: no structured mask
   int64_t struct_stride;        // words between the matrices of consecutive samples; 0: one matrix for the batch
@@ -125,8 +127,20 @@ __device__ __forceinline__ float frag_sum(const f16x8& v, float acc) {
   return acc;
 }
 
-template <typename T, int DP, bool CAUSAL, bool SCALED, bool MASKED>
+// Keep bytes of four consecutive keys of one mask row as one word (byte e = key key0 + e); keys at or beyond Tk read as 0.
+// `aligned`: Tk is a multiple of 4 and the mask is 4-byte aligned, so a word never straddles rows.
+__device__ __forceinline__ uint32_t keep_bytes4(const uint8_t* row, int key0, int Tk, bool aligned) {
+  if (aligned && key0 + 3 < Tk) return *reinterpret_cast<const uint32_t*>(row + key0);
+  uint32_t w = 0u;
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    if (key0 + e < Tk) w |= static_cast<uint32_t>(row[key0 + e]) << (8 * e);
+  return w;
+}
+
+template <typename T, int DP, bool CAUSAL, bool SCALED, bool MASKED, bool DROPOUT = false>
 __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnParams p) {
+  static_assert(!(DROPOUT && (SCALED || MASKED)), "dropout comes with the key-length / causal masks of the training path");
   static_assert(!(MASKED && CAUSAL), "a structured mask carries its own causal triangle");
   typedef typename Vec8<T>::type vec_t;
   typedef typename Vec8<T>::half_type vec4_t;
@@ -413,9 +427,30 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
           pb[kt][0][e] = static_cast<T>(pr[e]);
           pb[kt][1][e] = static_cast<T>(pr[8 + e]);
         }
-        // the normaliser sums the rounded probabilities, the values the second product uses: two per instruction
-        rs = frag_sum(pb[kt][0], rs);
-        rs = frag_sum(pb[kt][1], rs);
+        if (DROPOUT) {
+          // Training dropout with the caller's keep mask (tilelang.py:224-247 of the reference kernel): the normaliser
+          // sums the probabilities before the mask, the second product takes keep ? P / (1 - p) : 0.
+          const bool aligned = (p.Tk % 4 == 0) && (reinterpret_cast<uintptr_t>(p.drop_mask) % 4 == 0);
+          const uint8_t* row = p.drop_mask + ((static_cast<int64_t>(b) * p.H + h) * p.Tq + (qi < p.Tq ? qi : 0)) * p.Tk;
+#pragma unroll
+          for (int jq = 0; jq < 4; ++jq) {
+            const uint32_t keep = qi < p.Tq ? keep_bytes4(row, kc0 + (T0 + kt) * 32 + jq * 8 + hh * 4, p.Tk, aligned) : 0u;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              rs += pr[jq * 4 + e];
+              pr[jq * 4 + e] = ((keep >> (8 * e)) & 0xffu) != 0u ? pr[jq * 4 + e] * p.drop_scale : 0.f;
+            }
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            pb[kt][0][e] = static_cast<T>(pr[e]);
+            pb[kt][1][e] = static_cast<T>(pr[8 + e]);
+          }
+        } else {
+          // the normaliser sums the rounded probabilities, the values the second product uses: two per instruction
+          rs = frag_sum(pb[kt][0], rs);
+          rs = frag_sum(pb[kt][1], rs);
+        }
       }
       rs = pair_sum(rs);
       l_run = l_run * alpha + rs;
@@ -916,7 +951,7 @@ void launch(const AttnParams& p, bool causal, bool register_staging, hipStream_t
     // structure bits ride along when they are all there is to the mask: per sample, no validity or self rows, no chunk map
     const bool structure_only = p.struct_bits != nullptr && p.valid_bits == nullptr && p.self_bits == nullptr &&
                                 p.block_any == nullptr;
-    if (p.d == DP && (p.struct_bits == nullptr || structure_only) && dma_staging && small_offsets) {
+    if (p.d == DP && (p.struct_bits == nullptr || structure_only) && dma_staging && small_offsets && p.drop_mask == nullptr) {
       if (structure_only && scaled)
         hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
       else if (structure_only)
@@ -932,7 +967,11 @@ void launch(const AttnParams& p, bool causal, bool register_staging, hipStream_t
       return;
     }
   }
-  if (p.struct_bits != nullptr)
+  if (p.drop_mask != nullptr && causal)
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, true, false, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  else if (p.drop_mask != nullptr)
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false, false, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  else if (p.struct_bits != nullptr)
     hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
   else if (causal && scaled)
     hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, true, true, false>), dim3(p.total), dim3(kThreads), 0, s, p);
@@ -1001,7 +1040,13 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
                     const MaskArgs& mask, const float* q_row_scale, const float* k_row_scale, const float* q_col_scale,
                     float* lse, float* amax_out, void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
                     const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4], int mask_flags,
-                    int zero_padded_queries, int dtype, void* stream) {
+                    int zero_padded_queries, int dtype, void* stream, const uint8_t* drop_mask = nullptr,
+                    float drop_scale = 1.f) {
+  if (drop_mask != nullptr && (mask.struct_bits != nullptr || q_row_scale != nullptr || k_row_scale != nullptr ||
+                               q_col_scale != nullptr))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: dropout comes with key-length and causal masks only", name);
+  if (drop_mask != nullptr && !(drop_scale >= 1.f))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: dropout_scale = 1 / (1 - p) must be >= 1", name);
   if (mask_flags & ~(TAAC_ATTN_CAUSAL | TAAC_ATTN_REGISTER_STAGING))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: unknown bits in is_causal (%d)", name, mask_flags);
   const int is_causal = mask_flags & TAAC_ATTN_CAUSAL;
@@ -1047,6 +1092,8 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   p.k_row_scale = k_row_scale;
   p.q_col_scale = q_col_scale;
   p.amax_out = amax_out;
+  p.drop_mask = drop_mask;
+  p.drop_scale = drop_scale;
   p.lse = lse;
   p.struct_bits = mask.struct_bits;
   p.struct_stride = mask.struct_stride;
@@ -1179,6 +1226,20 @@ extern "C" int taac_mask_block_any(const uint32_t* struct_bits, int32_t Tq, int3
   hipLaunchKernelGGL(block_any_kernel, dim3(nqc * nkc), dim3(kWave), 0, as_stream(stream), struct_bits, Tq,
                      (Tk + 31) / 32, nkc, block_any);
   return check_launch(name);
+}
+
+extern "C" int taac_flash_attn_train_dropout_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
+                                                 const uint8_t* dropout_mask, float dropout_scale, void* o, float* lse,
+                                                 int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                                                 const int64_t q_strides[4], const int64_t k_strides[4],
+                                                 const int64_t v_strides[4], const int64_t o_strides[4], int is_causal,
+                                                 int zero_padded_queries, int dtype, void* stream) {
+  const char* name = "taac_flash_attn_train_dropout_fwd";
+  if (!lse) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: lse must be given", name);
+  if (!dropout_mask) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: dropout_mask must be given", name);
+  return taac::attention_entry(name, q, k, v, key_lengths, taac::MaskArgs{}, nullptr, nullptr, nullptr, lse, nullptr, o, B,
+                               H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, is_causal, zero_padded_queries,
+                               dtype, stream, dropout_mask, dropout_scale);
 }
 
 extern "C" int taac_flash_attn_train_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,

@@ -37,6 +37,8 @@ struct AttnBwdParams {
   void* dk;
   void* dv;
   const int32_t* key_lengths;
+  const uint8_t* drop_mask;  // training dropout: [B, H, Tq, Tk] keep mask (non-zero = keep), or null
+  float drop_scale;          // 1 / (1 - p)
   int32_t B, H, Tq, Tk, d;
   int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4];
   float scale;            // 1 / sqrt(d)
@@ -255,7 +257,19 @@ __device__ __forceinline__ void accumulate_columns2(f32x16 (&acc_a)[DP / 32], co
   });
 }
 
-template <typename T, int DP, bool DMA>
+// Keep bytes of four consecutive keys of one mask row as one word (byte e = key key0 + e); keys at or beyond Tk read as 0.
+__device__ __forceinline__ uint32_t keep_bytes4(const uint8_t* row, int key0, int Tk, bool aligned) {
+  if (aligned && key0 + 3 < Tk) return *reinterpret_cast<const uint32_t*>(row + key0);
+  uint32_t w = 0u;
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    if (key0 + e < Tk) w |= static_cast<uint32_t>(row[key0 + e]) << (8 * e);
+  return w;
+}
+
+// DROPOUT (both kernels): the caller's keep mask of the training forward; dV takes keep ? P / (1 - p) : 0 and the score
+// gradient P * ((keep ? dP / (1 - p) : 0) - D) / sqrt(d), as the reference's backward kernel does (tilelang.py:535-570).
+template <typename T, int DP, bool DMA, bool DROPOUT = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 32 ? 4 : 3))) void attn_bwd_dq_kernel(const AttnBwdParams p) {
   typedef typename Vec8<T>::type vec_t;
   constexpr int KSTEPS = DP / 16, MB = DP / 32;
@@ -368,10 +382,26 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 
         }
       }
       vec_t dsb[2];
+      if (DROPOUT) {
+        const bool aligned = (p.Tk % 4 == 0) && (reinterpret_cast<uintptr_t>(p.drop_mask) % 4 == 0);
+        const uint8_t* row = p.drop_mask + ((static_cast<int64_t>(b) * p.H + h) * p.Tq + (qi < p.Tq ? qi : 0)) * p.Tk;
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const float prob = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -lse2));
-        dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -delta_scaled));
+        for (int jq = 0; jq < 4; ++jq) {
+          const uint32_t keep = qi < p.Tq ? keep_bytes4(row, k_tile + jq * 8 + hh * 4, p.Tk, aligned) : 0u;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int j = jq * 4 + e;
+            const float prob = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -lse2));
+            const float dp = ((keep >> (8 * e)) & 0xffu) != 0u ? dpacc[j] * p.drop_scale : 0.f;
+            dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dp, p.scale, -delta_scaled));
+          }
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const float prob = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -lse2));
+          dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -delta_scaled));
+        }
       }
       accumulate_columns<T, DP, kt * 32 * ROWB>(dqacc, dsb, col_addr);
     });
@@ -380,7 +410,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 
   store_owned<T, DP>(dqacc, smem + wave * (32 * OROW), dqb, p.dqs[2], q_begin + wave * 32, p.Tq, p.d, lane);
 }
 
-template <typename T, int DP, bool DMA>
+template <typename T, int DP, bool DMA, bool DROPOUT = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP == 32 ? 4 : 3) - (DMA ? 0 : 1)))) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
   typedef typename Vec8<T>::type vec_t;
   constexpr int KSTEPS = DP / 16, MB = DP / 32;
@@ -509,8 +539,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
           for (int e = 0; e < 4; ++e) {
             const int j = jq * 4 + e;
             const float prob = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -l4[e]));
-            pb[j / 8][j % 8] = static_cast<T>(prob);
-            dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -d4[e]));
+            if (DROPOUT) {
+              // the lane owns key kj; register j is query qc0 + r0 + e: one keep byte per register
+              const int qrow = qc0 + r0 + e;
+              const bool keep = qrow < p.Tq && kj < p.Tk &&
+                                p.drop_mask[((static_cast<int64_t>(b) * p.H + h) * p.Tq + qrow) * p.Tk + kj] != 0;
+              pb[j / 8][j % 8] = static_cast<T>(keep ? prob * p.drop_scale : 0.f);
+              dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(keep ? dpacc[j] * p.drop_scale : 0.f, p.scale, -d4[e]));
+            } else {
+              pb[j / 8][j % 8] = static_cast<T>(prob);
+              dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -d4[e]));
+            }
           }
         }
         accumulate_columns2<T, DP, qt * 32 * ROWB>(dvacc, pb, q_col_addr + TILE_BYTES, dkacc, dsb, q_col_addr);
@@ -547,16 +586,27 @@ template <typename T, int DP>
 void launch_bwd_dp(AttnBwdParams p, bool register_staging, hipStream_t s) {
   // TAAC_ATTN_REGISTER_STAGING keeps the register-staged kernels for full head dims too (comparison route of the caller).
   const bool direct = p.d == DP && !register_staging;
+  const bool dropout = p.drop_mask != nullptr;
   p.nblk = static_cast<uint32_t>((p.Tq + kOwn - 1) / kOwn);
   p.total = p.nblk * p.B * p.H;
-  if (direct && small_offsets(p.Tk, p.ks[2]) && small_offsets(p.Tk, p.vs[2]))
+  const bool dq_direct = direct && small_offsets(p.Tk, p.ks[2]) && small_offsets(p.Tk, p.vs[2]);
+  if (dq_direct && dropout)
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, DP, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  else if (dq_direct)
     hipLaunchKernelGGL((attn_bwd_dq_kernel<T, DP, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  else if (dropout)
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, DP, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
   else
     hipLaunchKernelGGL((attn_bwd_dq_kernel<T, DP, false>), dim3(p.total), dim3(kThreads), 0, s, p);
   p.nblk = static_cast<uint32_t>((p.Tk + kOwn - 1) / kOwn);
   p.total = p.nblk * p.B * p.H;
-  if (direct && small_offsets(p.Tq, p.qs[2]) && small_offsets(p.Tq, p.dos[2]))
+  const bool dkv_direct = direct && small_offsets(p.Tq, p.qs[2]) && small_offsets(p.Tq, p.dos[2]);
+  if (dkv_direct && dropout)
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, DP, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  else if (dkv_direct)
     hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, DP, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  else if (dropout)
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, DP, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
   else
     hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, DP, false>), dim3(p.total), dim3(kThreads), 0, s, p);
 }
@@ -572,15 +622,17 @@ void launch_bwd(const AttnBwdParams& p, bool register_staging, hipStream_t s) {
 }  // namespace
 }  // namespace taac
 
-extern "C" int taac_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout,
-                                   const float* lse, const int32_t* key_lengths, void* dq, void* dk, void* dv,
-                                   float* delta, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
-                                   const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
-                                   const int64_t o_strides[4], const int64_t do_strides[4], const int64_t dq_strides[4],
-                                   const int64_t dk_strides[4], const int64_t dv_strides[4], int is_causal,
-                                   int zero_padded_queries, int dtype, void* stream) {
-  using namespace taac;
-  const char* name = "taac_flash_attn_bwd";
+namespace taac {
+namespace {
+int attention_bwd_entry(const char* name, const void* q, const void* k, const void* v, const void* o, const void* dout,
+                        const float* lse, const int32_t* key_lengths, const uint8_t* drop_mask, float drop_scale, void* dq,
+                        void* dk, void* dv, float* delta, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                        const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
+                        const int64_t o_strides[4], const int64_t do_strides[4], const int64_t dq_strides[4],
+                        const int64_t dk_strides[4], const int64_t dv_strides[4], int is_causal, int zero_padded_queries,
+                        int dtype, void* stream) {
+  if (drop_mask != nullptr && !(drop_scale >= 1.f))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: dropout_scale = 1 / (1 - p) must be >= 1", name);
   if (B < 0 || H < 0 || Tq < 0 || Tk < 0 || d <= 0)
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: negative dimension or non-positive head_dim", name);
   if (is_causal & ~(TAAC_ATTN_CAUSAL | TAAC_ATTN_REGISTER_STAGING))
@@ -619,6 +671,8 @@ extern "C" int taac_flash_attn_bwd(const void* q, const void* k, const void* v, 
   p.dk = dk;
   p.dv = dv;
   p.key_lengths = key_lengths;
+  p.drop_mask = drop_mask;
+  p.drop_scale = drop_scale;
   p.B = B;
   p.H = H;
   p.Tq = Tq;
@@ -643,4 +697,34 @@ extern "C" int taac_flash_attn_bwd(const void* q, const void* k, const void* v, 
   else
     launch_bwd<f16_t>(p, register_staging, s);
   return check_launch(name);
+}
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout,
+                                   const float* lse, const int32_t* key_lengths, void* dq, void* dk, void* dv,
+                                   float* delta, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                                   const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
+                                   const int64_t o_strides[4], const int64_t do_strides[4], const int64_t dq_strides[4],
+                                   const int64_t dk_strides[4], const int64_t dv_strides[4], int is_causal,
+                                   int zero_padded_queries, int dtype, void* stream) {
+  return taac::attention_bwd_entry("taac_flash_attn_bwd", q, k, v, o, dout, lse, key_lengths, nullptr, 1.f, dq, dk, dv, delta,
+                                   B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, do_strides, dq_strides,
+                                   dk_strides, dv_strides, is_causal, zero_padded_queries, dtype, stream);
+}
+
+extern "C" int taac_flash_attn_dropout_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout,
+                                           const float* lse, const int32_t* key_lengths, const uint8_t* dropout_mask,
+                                           float dropout_scale, void* dq, void* dk, void* dv, float* delta, int32_t B,
+                                           int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
+                                           const int64_t k_strides[4], const int64_t v_strides[4],
+                                           const int64_t o_strides[4], const int64_t do_strides[4],
+                                           const int64_t dq_strides[4], const int64_t dk_strides[4],
+                                           const int64_t dv_strides[4], int is_causal, int zero_padded_queries, int dtype,
+                                           void* stream) {
+  const char* name = "taac_flash_attn_dropout_bwd";
+  if (!dropout_mask) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: dropout_mask must be given", name);
+  return taac::attention_bwd_entry(name, q, k, v, o, dout, lse, key_lengths, dropout_mask, dropout_scale, dq, dk, dv, delta,
+                                   B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, do_strides, dq_strides,
+                                   dk_strides, dv_strides, is_causal, zero_padded_queries, dtype, stream);
 }

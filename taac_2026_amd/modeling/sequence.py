@@ -84,8 +84,10 @@ def scaled_dot_product_attention(
     k_row_scale: torch.Tensor | None = None,
     q_col_scale: torch.Tensor | None = None,
     structured_mask: StructuredAttentionMask | None = None,
+    dropout_mask: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """Multi-head attention over (B, T, D) projections; returns (B, Tq, D). ``q_row_scale`` / ``k_row_scale``
+    """Multi-head attention over (B, T, D) projections; returns (B, Tq, D). ``dropout_mask``: the uint8 keep mask
+    (B, H, Tq, Tk) of a training forward with ``dropout_p > 0`` (drawn when not given). ``q_row_scale`` / ``k_row_scale``
     (float32 (B, T)) and ``q_col_scale`` (float32 (D,)): optional factors of the query / key rows and of the query
     features applied inside the kernel. ``structured_mask``: a :class:`StructuredAttentionMask` in place of ``attn_mask``."""
     batch, query_len, d_model = q.shape
@@ -112,6 +114,7 @@ def scaled_dot_product_attention(
         k_row_scale=k_row_scale,
         q_col_scale=q_col_scale,
         structured_mask=structured_mask,
+        dropout_mask=dropout_mask,
     )
     return output.transpose(1, 2).contiguous().view(batch, query_len, d_model)
 

@@ -126,3 +126,51 @@ def test_backward_envelope(device):
     q32 = torch.randn(1, 1, 16, 32, device=device, requires_grad=True)
     with pytest.raises(RuntimeError, match="backward covers"):
         flash_attention(q32, q32, q32)
+
+
+@pytest.mark.parametrize("dtype,dim,causal,tokens", [(torch.float16, 16, False, 32), (torch.bfloat16, 32, False, 150),
+                                                     (torch.bfloat16, 64, True, 200), (torch.float16, 64, False, 77)])
+def test_training_dropout_with_a_fixed_keep_mask(device, dtype, dim, causal, tokens):
+    """Dropout on the attention probabilities with the caller's uint8 keep mask, forward and backward, against float64
+    autograd of the oracle under the same mask - the check the reference runs on its TileLang kernels
+    (tests/gpu/infrastructure/accelerators/test_tilelang_ops_cuda.py:103-141: output 2e-2, gradients 3e-2), here also with
+    ragged key lengths, a causal triangle and a key count that is no multiple of four (unaligned mask rows)."""
+    batch, heads, dropout_p = 3, 4, 0.125
+    g = torch.Generator().manual_seed(tokens + dim)
+    q, k, v, grad_out = (torch.randn(batch, heads, tokens, dim, generator=g).to(dtype) for _ in range(4))
+    lengths = torch.tensor([tokens, max(1, tokens // 3), tokens - 5], dtype=torch.int32)
+    mask = (torch.rand(batch, heads, tokens, tokens, generator=g) >= dropout_p).to(torch.uint8)
+    qd, kd, vd = (t.to(device).requires_grad_(True) for t in (q, k, v))
+    out = flash_attention(qd, kd, vd, key_lengths=lengths.to(device), is_causal=causal, zero_padded_queries=not causal,
+                          dropout_p=dropout_p, training=True, dropout_mask=mask.to(device))
+    out.backward(grad_out.to(device))
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    want = oracle.attention_dropout(qr, kr, vr, lengths, mask, dropout_p, is_causal=causal, zero_padded_queries=not causal)
+    want.backward(grad_out.double())
+    torch.testing.assert_close(out.detach().cpu().double(), want.detach(), rtol=2e-2, atol=2e-2)
+    for got, ref in ((qd.grad, qr.grad), (kd.grad, kr.grad), (vd.grad, vr.grad)):
+        torch.testing.assert_close(got.cpu().double(), ref, rtol=3e-2, atol=3e-2)
+    # the mask matters (a run without it differs) and an all-ones mask at p -> 0 is the plain training path
+    plain = flash_attention(qd.detach(), kd.detach(), vd.detach(), key_lengths=lengths.to(device), is_causal=causal,
+                            zero_padded_queries=not causal)
+    assert (plain.float() - out.detach().float()).abs().max().item() > 5e-2
+    ones = torch.ones_like(mask).to(device)
+    q1 = qd.detach().clone().requires_grad_(True)
+    same = flash_attention(q1, kd.detach(), vd.detach(), key_lengths=lengths.to(device), is_causal=causal,
+                           zero_padded_queries=not causal, dropout_p=1e-9, training=True, dropout_mask=ones)
+    torch.testing.assert_close(same.detach().float(), plain.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_dropout_draws_its_own_mask_and_rejects_what_it_does_not_cover(device):
+    g = torch.Generator().manual_seed(3)
+    q, k, v = (torch.randn(2, 2, 64, 32, generator=g).to(torch.bfloat16).to(device) for _ in range(3))
+    torch.manual_seed(0)
+    a = flash_attention(q, k, v, dropout_p=0.5, training=True)
+    torch.manual_seed(0)
+    b = flash_attention(q, k, v, dropout_p=0.5, training=True)
+    c = flash_attention(q, k, v, dropout_p=0.5, training=True)
+    assert torch.equal(a, b) and not torch.equal(a, c)
+    with pytest.raises(RuntimeError, match="only supports dropout during training"):
+        flash_attention(q, k, v, dropout_p=0.5, training=False)
+    with pytest.raises(ValueError, match="dropout_mask must be uint8"):
+        flash_attention(q, k, v, dropout_p=0.5, training=True, dropout_mask=torch.ones(2, 2, 64, 63, dtype=torch.uint8, device=device))

@@ -71,8 +71,8 @@ def test_flash_attention_argument_errors():
         api.flash_attention(q, q, q, backend="triton")
     with pytest.raises(RuntimeError, match=r"dropout_p to be in \[0, 1\)"):
         api.flash_attention(q, q, q, dropout_p=1.0, training=True)
-    with pytest.raises(RuntimeError, match="does not apply dropout"):
-        api.flash_attention(q, q, q, dropout_p=0.1, training=True)
+    with pytest.raises(RuntimeError, match="only supports dropout during training"):
+        api.flash_attention(q, q, q, dropout_p=0.1, training=False)
     with pytest.raises(RuntimeError, match="requires CUDA tensors"):
         api.flash_attention(q, q, q)
 

@@ -590,3 +590,29 @@ def test_candidate_readout_brute_force_and_special_cases():
     torch.testing.assert_close(bare[:, :d], x[:, 2])
     torch.testing.assert_close(bare[:, 2 * d:], oracle.masked_mean(x, pad))
     assert bare[1, 2 * d:].abs().max().item() == 0.0
+
+
+def test_attention_dropout_reduces_to_attention_and_matches_a_loop():
+    """``attention_dropout``: with an all-ones mask and p = 0 it is ``attention``; on a tiny case it equals a per-element
+    loop (softmax over the visible keys, then keep / (1 - p), then the value sum); dropping a key changes only that key's
+    contribution (the normaliser is that of the undropped probabilities)."""
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(2, 2, 5, 4, generator=g, dtype=torch.float64) for _ in range(3))
+    lengths = torch.tensor([5, 3], dtype=torch.int32)
+    ones = torch.ones(2, 2, 5, 5, dtype=torch.uint8)
+    torch.testing.assert_close(oracle.attention_dropout(q, k, v, lengths, ones, 0.0, zero_padded_queries=True),
+                               oracle.attention(q, k, v, lengths, zero_padded_queries=True), rtol=1e-5, atol=1e-6)      # (that one works in float32)
+    p = 0.25
+    mask = (torch.rand(2, 2, 5, 5, generator=g) >= p).to(torch.uint8)
+    for causal in (False, True):
+        got = oracle.attention_dropout(q, k, v, lengths, mask, p, is_causal=causal)
+        for b in range(2):
+            for h in range(2):
+                for i in range(5):
+                    keys = [j for j in range(int(lengths[b])) if not causal or j <= i]
+                    scores = [float(q[b, h, i] @ k[b, h, j]) / 2.0 for j in keys]
+                    top = max(scores)
+                    weights = [math.exp(s - top) for s in scores]
+                    total = sum(weights)
+                    want = sum(w / total * float(mask[b, h, i, j]) / (1 - p) * v[b, h, j] for w, j in zip(weights, keys))
+                    torch.testing.assert_close(got[b, h, i], want, rtol=1e-10, atol=1e-12)
