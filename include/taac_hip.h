@@ -269,6 +269,25 @@ int taac_linear_bf16(const void* a, int64_t lda, const void* w, const void* bias
                      int64_t ldo, int64_t M, int32_t N, int32_t K, int epilogue, int gate_first, void* stream);
 
 /*
+ * Backward pieces of a dense layer y = a w^T + b that are not themselves a forward-shaped product (the input gradient
+ * dy w is one: taac_linear_bf16 with the transposed weight):
+ *   taac_linear_wgrad: dw[n, k] = sum_m dy[m, n] * a[m, k] and (db != NULL) db[n] = sum_m dy[m, n].
+ *     dy: [M, N] bf16 (row stride ldy), a: [M, K] bf16 (row stride lda), dw: [N, K], db: [N], both of out_dtype
+ *     (TAAC_BF16 or TAAC_F32), contiguous. fp32 accumulation; the token range is split over workgroups and the splits
+ *     are added in a fixed order (bit-reproducible). workspace: taac_linear_wgrad_workspace_floats(M, N, K) floats.
+ *   taac_swiglu_bwd: gu: [M, 2F] pre-activations (g | u); hidden (or NULL) = silu(g) * u (gate_first) or g * silu(u);
+ *     with dhidden [M, F]: dgu (or NULL) = (dg | du), dg = dhidden * u * silu'(g), du = dhidden * silu(g) (roles swapped
+ *     without gate_first). bf16, fp32 arithmetic, one rounding per output.
+ * Replaces: what torch autograd derives for nn.Linear and F.silu(gate) * value in the reference's training runs
+ * (experiments/symbiosis/backbone.py:11-21, 24-48).
+ */
+int64_t taac_linear_wgrad_workspace_floats(int64_t M, int32_t N, int32_t K);
+int taac_linear_wgrad(const void* dy, int64_t ldy, const void* a, int64_t lda, void* dw, void* db, float* workspace,
+                      int64_t workspace_floats, int64_t M, int32_t N, int32_t K, int out_dtype, void* stream);
+int taac_swiglu_bwd(const void* gu, int64_t ldgu, const void* dhidden, int64_t lddh, void* dgu, int64_t lddgu, void* hidden,
+                    int64_t ldh, int64_t M, int32_t F, int gate_first, void* stream);
+
+/*
  * Fused feed-forward half of a block, one kernel:
  *   out = residual + down( silu(g) * u ),   g, u = chunk2( up( norm_weight ? rmsnorm(x, norm_weight, eps) : x ) )
  * x: [M, D] bf16 (row stride ldx); w_up: [2F, D]; b_up: [2F] or NULL; w_down: [D, F]; b_down: [D] or NULL;

@@ -118,6 +118,15 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         + [ctypes.POINTER(c_int64)] * 8
         + [c_int, c_int, c_int, c_void_p],
     ),
+    "taac_linear_wgrad_workspace_floats": (c_int64, [c_int64, c_int32, c_int32]),
+    "taac_linear_wgrad": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_int, c_void_p],
+    ),
+    "taac_swiglu_bwd": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int32, c_int, c_void_p],
+    ),
     "taac_flash_attn_train_dropout_fwd": (
         c_int,
         [c_void_p] * 5 + [c_float] + [c_void_p] * 2 + [c_int32, c_int32, c_int32, c_int32, c_int32]

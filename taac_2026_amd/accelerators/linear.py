@@ -43,6 +43,150 @@ def _check_weight(operator_name: str, rows: torch.Tensor, weight: torch.Tensor, 
         raise ValueError(f"{operator_name} bias must have shape ({weight.shape[0]},)")
 
 
+def _needs_grad(*tensors: torch.Tensor | None) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+def linear_wgrad(grad_out: torch.Tensor, inputs: torch.Tensor, *, with_bias: bool = True,
+                 dtype: torch.dtype = torch.bfloat16) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """Weight and bias gradient of ``y = inputs @ w.T + b``: ``(grad_out.T @ inputs, grad_out.sum(0))`` over the flattened
+    rows, fp32 accumulation with a fixed summation order (``taac_linear_wgrad``). Returns tensors of ``dtype``."""
+    name = "hip linear_wgrad"
+    require_cuda_tensors(name, grad_out, inputs)
+    _check_bf16(name, grad_out, inputs)
+    dy, _ = _as_rows(grad_out)
+    a, _ = _as_rows(inputs)
+    if dy.shape[0] != a.shape[0]:
+        raise ValueError("linear_wgrad: grad_out and inputs must have the same number of rows")
+    if dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("linear_wgrad returns bfloat16 or float32 gradients")
+    rows, out_features, in_features = dy.shape[0], dy.shape[1], a.shape[1]
+    grad_w = torch.empty(out_features, in_features, dtype=dtype, device=dy.device)
+    grad_b = torch.empty(out_features, dtype=dtype, device=dy.device) if with_bias else None
+    library = _native.load_library()
+    count = int(library.taac_linear_wgrad_workspace_floats(rows, out_features, in_features))
+    workspace = torch.empty(max(count, 1), dtype=torch.float32, device=dy.device)
+    status = library.taac_linear_wgrad(
+        dy.data_ptr(), dy.stride(0), a.data_ptr(), a.stride(0), grad_w.data_ptr(), _native.ptr(grad_b), workspace.data_ptr(),
+        workspace.numel(), rows, out_features, in_features, _native.dtype_code(dtype), _native.current_stream(dy.device),
+    )
+    _native.check(status, "linear_wgrad")
+    return grad_w, grad_b
+
+
+def swiglu_backward(pre_activation: torch.Tensor, grad_hidden: torch.Tensor | None, *, gate_first: bool = True,
+                    want_hidden: bool = True) -> tuple[torch.Tensor | None, torch.Tensor | None]:
+    """From the up projection ``[.., 2F]`` (gate | value): the gated hidden state ``silu(gate) * value`` and, with
+    ``grad_hidden``, the gradient of the up projection ``[.., 2F]`` (``taac_swiglu_bwd``). Returns (hidden, grad)."""
+    name = "hip swiglu_backward"
+    require_cuda_tensors(name, pre_activation, grad_hidden)
+    _check_bf16(name, pre_activation, grad_hidden)
+    gu, shape = _as_rows(pre_activation)
+    hidden_size = gu.shape[1] // 2
+    dh = None
+    if grad_hidden is not None:
+        dh, _ = _as_rows(grad_hidden)
+    hidden = torch.empty(gu.shape[0], hidden_size, dtype=gu.dtype, device=gu.device) if want_hidden else None
+    grad = torch.empty_like(gu, memory_format=torch.contiguous_format) if dh is not None else None
+    library = _native.load_library()
+    status = library.taac_swiglu_bwd(
+        gu.data_ptr(), gu.stride(0), _native.ptr(dh), dh.stride(0) if dh is not None else hidden_size, _native.ptr(grad),
+        2 * hidden_size, _native.ptr(hidden), hidden_size, gu.shape[0], hidden_size, int(bool(gate_first)),
+        _native.current_stream(gu.device),
+    )
+    _native.check(status, "swiglu_backward")
+    return (None if hidden is None else hidden.reshape(*shape[:-1], hidden_size),
+            None if grad is None else grad.reshape(*shape[:-1], 2 * hidden_size))
+
+
+def _input_grad(grad_rows: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``grad_rows @ weight``: a forward-shaped product with the transposed weight."""
+    with torch.no_grad():
+        return linear(grad_rows, weight.detach().t().contiguous())
+
+
+class _NormLinearFunction(torch.autograd.Function):
+    """``residual + linear(rmsnorm(x))`` (norm and residual optional) for training: the forward is the inference kernel and
+    saves only its inputs; the backward recomputes the normalised rows and runs the input-gradient product, the weight
+    gradient and the norm backward as HIP kernels (what torch autograd derives for the reference's nn.Linear layers,
+    experiments/symbiosis/backbone.py:24-48)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, norm_weight, residual, eps):
+        with torch.no_grad():
+            out = norm_linear(x, weight, bias, norm_weight=norm_weight, eps=eps, residual=residual)
+        ctx.save_for_backward(x, weight, *(() if norm_weight is None else (norm_weight,)))
+        ctx.has_norm, ctx.has_bias, ctx.has_residual, ctx.eps = norm_weight is not None, bias is not None, residual is not None, eps
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        from taac_2026_amd.accelerators.normalization import hip_rms_norm_backward_kernel, hip_rms_norm_kernel
+
+        x, weight = ctx.saved_tensors[:2]
+        norm_weight = ctx.saved_tensors[2] if ctx.has_norm else None
+        rows, shape = _as_rows(x)
+        rows = rows.contiguous()
+        dy, _ = _as_rows(grad_out if grad_out.dtype == torch.bfloat16 else grad_out.to(torch.bfloat16))
+        dy = dy.contiguous()
+        with torch.no_grad():
+            h = hip_rms_norm_kernel(rows, norm_weight, ctx.eps) if ctx.has_norm else rows
+            grad_w, grad_b = linear_wgrad(dy, h, with_bias=ctx.has_bias)
+            grad_h = _input_grad(dy, weight)
+            grad_norm = None
+            if ctx.has_norm:
+                grad_rows, grad_norm = hip_rms_norm_backward_kernel(rows, norm_weight, grad_h.contiguous(), ctx.eps)
+            else:
+                grad_rows = grad_h
+        return (grad_rows.reshape(shape), grad_w, grad_b, grad_norm, grad_out if ctx.has_residual else None, None)
+
+
+class _SwigluFfnFunction(torch.autograd.Function):
+    """``residual + down(silu(gate) * value)``, ``gate, value = up(rmsnorm(x))``, for training: the forward is the fused
+    inference kernel and saves only its inputs; the backward recomputes the up projection and the hidden state
+    (experiments/symbiosis/backbone.py:11-21)."""
+
+    @staticmethod
+    def forward(ctx, x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight, gate_first, eps):
+        with torch.no_grad():
+            out = swiglu_ffn(x, up_weight, up_bias, down_weight, down_bias, residual=residual, gate_first=gate_first,
+                             norm_weight=norm_weight, eps=eps)
+        ctx.save_for_backward(x, up_weight, down_weight, *(t for t in (up_bias, norm_weight) if t is not None))
+        ctx.flags = (up_bias is not None, down_bias is not None, residual is not None, norm_weight is not None,
+                     bool(gate_first), eps)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        from taac_2026_amd.accelerators.normalization import hip_rms_norm_backward_kernel, hip_rms_norm_kernel
+
+        has_up_bias, has_down_bias, has_residual, has_norm, gate_first, eps = ctx.flags
+        saved = list(ctx.saved_tensors)
+        x, up_weight, down_weight = saved[:3]
+        rest = saved[3:]
+        up_bias = rest.pop(0) if has_up_bias else None
+        norm_weight = rest.pop(0) if has_norm else None
+        rows, shape = _as_rows(x)
+        rows = rows.contiguous()
+        dy, _ = _as_rows(grad_out if grad_out.dtype == torch.bfloat16 else grad_out.to(torch.bfloat16))
+        dy = dy.contiguous()
+        with torch.no_grad():
+            h = hip_rms_norm_kernel(rows, norm_weight, eps) if has_norm else rows
+            pre = linear(h, up_weight.detach(), None if up_bias is None else up_bias.detach())   # [M, 2F]
+            grad_hidden = _input_grad(dy, down_weight)                                           # [M, F]
+            hidden, grad_pre = swiglu_backward(pre, grad_hidden, gate_first=gate_first)
+            grad_down_w, grad_down_b = linear_wgrad(dy, hidden, with_bias=has_down_bias)
+            grad_up_w, grad_up_b = linear_wgrad(grad_pre, h, with_bias=has_up_bias)
+            grad_h = _input_grad(grad_pre, up_weight)
+            grad_norm = None
+            if has_norm:
+                grad_rows, grad_norm = hip_rms_norm_backward_kernel(rows, norm_weight, grad_h.contiguous(), eps)
+            else:
+                grad_rows = grad_h
+        return (grad_rows.reshape(shape), grad_up_w, grad_up_b, grad_down_w, grad_down_b,
+                grad_out if has_residual else None, grad_norm, None, None)
+
+
 def linear(
     x: torch.Tensor,
     weight: torch.Tensor,
@@ -53,7 +197,8 @@ def linear(
     """``F.linear(x, weight, bias)`` (+ ``residual``) in bf16 with fp32 accumulation."""
     name = "hip linear"
     require_cuda_tensors(name, x, weight, bias, residual)
-    require_inference(name, x, weight, bias, residual)
+    if _needs_grad(x, weight, bias, residual):
+        return _NormLinearFunction.apply(x, weight, bias, None, residual, 1e-6)
     _check_bf16(name, x, weight, bias, residual)
     rows, shape = _as_rows(x)
     _check_weight(name, rows, weight, bias)
@@ -291,7 +436,12 @@ def swiglu_ffn(
     """
     name = "hip swiglu_ffn"
     require_cuda_tensors(name, x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight)
-    require_inference(name, x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight)
+    if _needs_grad(x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight):
+        if token_rows is not None or out is not None:
+            raise RuntimeError("hip swiglu_ffn: token_rows / out belong to the inference route; call it under "
+                               "torch.no_grad() or pass dense tensors when a gradient is needed")
+        return _SwigluFfnFunction.apply(x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight,
+                                        bool(gate_first), float(eps))
     _check_bf16(name, x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight)
     rows, shape = _as_rows(x)
     _check_weight(name, rows, up_weight, up_bias)
@@ -405,7 +555,11 @@ def norm_linear(
     ``x`` is laid out differently from ``residual`` / ``out`` (:func:`front_rows`)."""
     name = "hip norm_linear"
     require_cuda_tensors(name, x, weight, bias, residual, norm_weight)
-    require_inference(name, x, weight, bias, residual, norm_weight)
+    if _needs_grad(x, weight, bias, residual, norm_weight):
+        if token_rows is not None or input_rows is not None or out is not None:
+            raise RuntimeError("hip norm_linear: token_rows / input_rows / out belong to the inference route; "
+                               "call it under torch.no_grad() or pass dense tensors when a gradient is needed")
+        return _NormLinearFunction.apply(x, weight, bias, norm_weight, residual, float(eps))
     _check_bf16(name, x, weight, bias, residual, norm_weight)
     rows, shape = _as_rows(x)
     _check_weight(name, rows, weight, bias)
@@ -771,6 +925,8 @@ __all__ = [
     "clear_packed_weight_cache",
     "linear",
     "linear_fp8",
+    "linear_wgrad",
+    "swiglu_backward",
     "norm_linear",
     "pack_ffn_weights",
     "norm_linear_fp8",

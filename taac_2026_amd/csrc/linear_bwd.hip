@@ -1,0 +1,266 @@
+// Backward pieces of the dense layers (gfx950): the weight gradient of a linear layer as a product over the tokens, the
+// column sums for the bias gradient, and the elementwise backward of the SiLU gate.
+//
+//   taac_linear_wgrad : dW[n, k] = sum_m dy[m, n] * a[m, k],  db[n] = sum_m dy[m, n]
+//   taac_swiglu_bwd   : hidden = silu(g) * u,  dg = dhidden * u * silu'(g),  du = dhidden * silu(g)
+//
+// The reference trains its dense layers through torch autograd of nn.Linear / F.silu (experiments/symbiosis/backbone.py:
+// 11-21, 24-48); these are the two products of that backward that are not themselves a forward-shaped linear layer (the
+// input gradient dy W is one, with the transposed weight).
+//
+// Weight gradient: both operands are [tokens, features] row-major, and the MFMA needs, per lane, eight consecutive tokens
+// of one feature from each - a transposed read. A workgroup stages 32 tokens of a 128-feature slab of dy and of a into LDS
+// row-major (rows padded to 288 bytes: the four rows and four 8-byte pieces a 16-lane group touches fall on distinct
+// banks) and reads both fragments with ds_read_b64_tr_b16. The token range is split over workgroups; every split writes its
+// fp32 partial tile, and a second kernel adds the splits in a fixed order, so the gradient is bit-reproducible.
+
+#include <hip/hip_runtime.h>
+#include <math.h>
+
+#include "common.h"
+#include "ts_common.h"
+
+namespace taac {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kTile = 128;      // features of dy / of a per workgroup tile
+constexpr int kChunk = 32;      // tokens per staged chunk
+constexpr int kRowBytes = kTile * 2 + 32;  // padded LDS row
+constexpr int kMaxSplits = 256;
+
+// Stage rows [m0, m0 + 32) x columns [c0, c0 + 128) of src (bf16, row stride ld) into dst; out-of-range pieces are zeros.
+__device__ __forceinline__ void stage_chunk(const bf16_t* __restrict__ src, int64_t ld, int64_t m0, int64_t m_end, int c0,
+                                            int cols, uint8_t* dst, int tid) {
+#pragma unroll
+  for (int i = 0; i < kChunk * (kTile / 8) / kThreads; ++i) {
+    const int idx = tid + i * kThreads;
+    const int row = idx / (kTile / 8), piece = idx % (kTile / 8);
+    const int64_t m = m0 + row;
+    const int c = c0 + piece * 8;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (m < m_end && c < cols) v = *reinterpret_cast<const u32x4*>(src + m * ld + c);
+    *reinterpret_cast<u32x4*>(dst + row * kRowBytes + piece * 16) = v;
+  }
+}
+
+// grid = (tiles of N x tiles of K, splits). partial: [splits][N][K] fp32.
+__global__ __launch_bounds__(kThreads) void wgrad_partial_kernel(const bf16_t* __restrict__ dy, int64_t ldy,
+                                                                 const bf16_t* __restrict__ a, int64_t lda,
+                                                                 float* __restrict__ partial, int64_t M, int N, int K,
+                                                                 int64_t rows_per_split) {
+  __shared__ __attribute__((aligned(16))) uint8_t smem[2 * kChunk * kRowBytes];
+  uint8_t* sA = smem;                       // dy slab
+  uint8_t* sB = smem + kChunk * kRowBytes;  // activation slab
+  const int tiles_k = (K + kTile - 1) / kTile;
+  const int n0 = (blockIdx.x / tiles_k) * kTile, k0 = (blockIdx.x % tiles_k) * kTile;
+  const int64_t m_begin = static_cast<int64_t>(blockIdx.y) * rows_per_split;
+  const int64_t m_end = m_begin + rows_per_split < M ? m_begin + rows_per_split : M;
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  const int wn = wave / 2, wk = wave % 2;  // the wavefront's 64 x 64 block of the tile
+  // transposed read: lane r of a 16-lane group g points at token t0 + r / 4, features f0 + 4 * (r % 4) .. + 3 and receives
+  // tokens t0 .. t0 + 3 of feature f0 + r; group g covers features 16 * (g % 2) .. + 15 and the token half g / 2
+  const int g = lane / 16, r = lane % 16;
+  const uint32_t lane_off = static_cast<uint32_t>((8 * (g / 2) + r / 4) * kRowBytes + (16 * (g % 2) + 4 * (r % 4)) * 2);
+  const uint32_t a_addr = lds_offset(sA) + lane_off + wn * 64 * 2;
+  const uint32_t b_addr = lds_offset(sB) + lane_off + wk * 64 * 2;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  for (int64_t m0 = m_begin; m0 < m_end; m0 += kChunk) {
+    __syncthreads();  // everyone is done reading the previous chunk
+    stage_chunk(dy, ldy, m0, m_end, n0, N, sA, tid);
+    stage_chunk(a, lda, m0, m_end, k0, K, sB, tid);
+    __syncthreads();
+    static_for<kChunk / 16>([&](auto ks_tag) {
+      constexpr int ks = decltype(ks_tag)::value;
+      u32x2 fa[2][2], fb[2][2];
+      static_for<2>([&](auto t_tag) {
+        constexpr int t = decltype(t_tag)::value;
+        lds_read_tr16<(ks * 16) * kRowBytes + t * 64>(fa[t][0], a_addr);
+        lds_read_tr16<(ks * 16 + 4) * kRowBytes + t * 64>(fa[t][1], a_addr);
+        lds_read_tr16<(ks * 16) * kRowBytes + t * 64>(fb[t][0], b_addr);
+        lds_read_tr16<(ks * 16 + 4) * kRowBytes + t * 64>(fb[t][1], b_addr);
+      });
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[1][0]), "+v"(fa[1][1]) : : "memory");
+      asm volatile("" : "+v"(fb[0][0]), "+v"(fb[0][1]), "+v"(fb[1][0]), "+v"(fb[1][1]));
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const u32x4 abits = {fa[i][0][0], fa[i][0][1], fa[i][1][0], fa[i][1][1]};
+          const u32x4 bbits = {fb[j][0][0], fb[j][0][1], fb[j][1][0], fb[j][1][1]};
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, abits),
+                                                              __builtin_bit_cast(bf16x8, bbits), acc[i][j], 0, 0, 0);
+        }
+    });
+  }
+  // accumulator register e of a lane: row (e / 4) * 8 + (lane / 32) * 4 + e % 4 of the 32 x 32 tile, column lane % 32
+  float* out = partial + static_cast<int64_t>(blockIdx.y) * N * K;
+  const int l32 = lane % 32, hh = lane / 32;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = k0 + wk * 64 + j * 32 + l32;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = n0 + wn * 64 + i * 32 + (e / 4) * 8 + hh * 4 + (e % 4);
+        if (row < N && col < K) out[static_cast<int64_t>(row) * K + col] = acc[i][j][e];
+      }
+    }
+}
+
+// out[i] = sum over the splits of partial[s][i], in split order; one rounding to the output type.
+template <typename TOut>
+__global__ __launch_bounds__(kThreads) void reduce_splits_kernel(const float* __restrict__ partial, TOut* __restrict__ out,
+                                                                 int64_t n, int splits) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i >= n) return;
+  float s = 0.f;
+  for (int k = 0; k < splits; ++k) s += partial[static_cast<int64_t>(k) * n + i];
+  out[i] = static_cast<TOut>(s);
+}
+
+// partial[split][c] = sum over the split's rows of dy[m][c]; a thread owns eight columns.
+__global__ __launch_bounds__(kThreads) void colsum_partial_kernel(const bf16_t* __restrict__ dy, int64_t ldy,
+                                                                  float* __restrict__ partial, int64_t M, int N,
+                                                                  int64_t rows_per_split) {
+  const int64_t m_begin = static_cast<int64_t>(blockIdx.y) * rows_per_split;
+  const int64_t m_end = m_begin + rows_per_split < M ? m_begin + rows_per_split : M;
+  const int c = (blockIdx.x * kThreads + threadIdx.x) * 8;
+  if (c >= N) return;
+  float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int64_t m = m_begin; m < m_end; ++m) {
+    const bf16x8 v = *reinterpret_cast<const bf16x8*>(dy + m * ldy + c);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s[e] += static_cast<float>(v[e]);
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) partial[static_cast<int64_t>(blockIdx.y) * N + c + e] = s[e];
+}
+
+int splits_for(int64_t M) {
+  int64_t s = (M + 2047) / 2048;
+  if (s < 1) s = 1;
+  if (s > kMaxSplits) s = kMaxSplits;
+  return static_cast<int>(s);
+}
+
+// gu: [M, 2F] pre-activations (first half g, second half u); dh: [M, F]. gate_first: hidden = silu(g) * u, else g * silu(u).
+__global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const bf16_t* __restrict__ gu, int64_t ldgu,
+                                                              const bf16_t* __restrict__ dh, int64_t lddh,
+                                                              bf16_t* __restrict__ dgu, int64_t lddgu,
+                                                              bf16_t* __restrict__ hidden, int64_t ldh, int64_t M, int F,
+                                                              int gate_first) {
+  const int pieces = F / 8;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (idx >= M * pieces) return;
+  const int64_t m = idx / pieces;
+  const int c = static_cast<int>(idx % pieces) * 8;
+  const bf16x8 gv = *reinterpret_cast<const bf16x8*>(gu + m * ldgu + c);
+  const bf16x8 uv = *reinterpret_cast<const bf16x8*>(gu + m * ldgu + F + c);
+  bf16x8 dv;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) dv[e] = static_cast<bf16_t>(0.f);
+  if (dh != nullptr) dv = *reinterpret_cast<const bf16x8*>(dh + m * lddh + c);
+  bf16x8 dg, du, hv;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    // act: the operand that goes through SiLU; lin: the one that multiplies it
+    const float act = static_cast<float>(gate_first ? gv[e] : uv[e]);
+    const float lin = static_cast<float>(gate_first ? uv[e] : gv[e]);
+    const float d = static_cast<float>(dv[e]);
+    const float sig = 1.f / (1.f + __expf(-act));
+    const float silu = act * sig;
+    const float dact = d * lin * (sig * (1.f + act * (1.f - sig)));
+    const float dlin = d * silu;
+    hv[e] = static_cast<bf16_t>(silu * lin);
+    dg[e] = static_cast<bf16_t>(gate_first ? dact : dlin);
+    du[e] = static_cast<bf16_t>(gate_first ? dlin : dact);
+  }
+  if (dgu != nullptr) {
+    *reinterpret_cast<bf16x8*>(dgu + m * lddgu + c) = dg;
+    *reinterpret_cast<bf16x8*>(dgu + m * lddgu + F + c) = du;
+  }
+  if (hidden != nullptr) *reinterpret_cast<bf16x8*>(hidden + m * ldh + c) = hv;
+}
+
+}  // namespace
+}  // namespace taac
+
+extern "C" int64_t taac_linear_wgrad_workspace_floats(int64_t M, int32_t N, int32_t K) {
+  if (M < 0 || N <= 0 || K <= 0) return -1;
+  return static_cast<int64_t>(taac::splits_for(M)) * N * (static_cast<int64_t>(K) + 1);
+}
+
+extern "C" int taac_linear_wgrad(const void* dy, int64_t ldy, const void* a, int64_t lda, void* dw, void* db,
+                                 float* workspace, int64_t workspace_floats, int64_t M, int32_t N, int32_t K, int out_dtype,
+                                 void* stream) {
+  using namespace taac;
+  const char* name = "taac_linear_wgrad";
+  if (M < 0 || N <= 0 || K <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, N and K > 0", name);
+  if (N % 8 != 0 || K % 8 != 0 || ldy % 8 != 0 || lda % 8 != 0 || ldy < N || lda < K)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: N, K and the row strides must be multiples of 8 and cover a row", name);
+  if (out_dtype != TAAC_BF16 && out_dtype != TAAC_F32)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: out_dtype must be bf16 or fp32 (got %d)", name, out_dtype);
+  if (!dw || (M > 0 && (!dy || !a))) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
+  if (!aligned16(dy) || !aligned16(a)) return set_error(TAAC_ERR_UNSUPPORTED, "%s: dy and a must be 16-byte aligned", name);
+  const int64_t need = taac_linear_wgrad_workspace_floats(M, N, K);
+  if (!workspace || workspace_floats < need)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: workspace must hold %lld floats", name, (long long)need);
+  hipStream_t s = as_stream(stream);
+  const int splits = splits_for(M);
+  const int64_t rows_per_split = ((M + splits - 1) / splits + kChunk - 1) / kChunk * kChunk;
+  const int64_t nk = static_cast<int64_t>(N) * K;
+  float* part_w = workspace;
+  float* part_b = workspace + static_cast<int64_t>(splits) * nk;
+  const int tiles = ((N + kTile - 1) / kTile) * ((K + kTile - 1) / kTile);
+  hipLaunchKernelGGL(wgrad_partial_kernel, dim3(tiles, splits), dim3(kThreads), 0, s, static_cast<const bf16_t*>(dy), ldy,
+                     static_cast<const bf16_t*>(a), lda, part_w, M, N, K, rows_per_split);
+  const uint32_t blocks = static_cast<uint32_t>((nk + kThreads - 1) / kThreads);
+  if (out_dtype == TAAC_BF16)
+    hipLaunchKernelGGL(reduce_splits_kernel<bf16_t>, dim3(blocks), dim3(kThreads), 0, s, part_w, static_cast<bf16_t*>(dw), nk,
+                       splits);
+  else
+    hipLaunchKernelGGL(reduce_splits_kernel<float>, dim3(blocks), dim3(kThreads), 0, s, part_w, static_cast<float*>(dw), nk,
+                       splits);
+  if (db != nullptr) {
+    hipLaunchKernelGGL(colsum_partial_kernel, dim3((N / 8 + kThreads - 1) / kThreads, splits), dim3(kThreads), 0, s,
+                       static_cast<const bf16_t*>(dy), ldy, part_b, M, N, rows_per_split);
+    const uint32_t bblocks = static_cast<uint32_t>((N + kThreads - 1) / kThreads);
+    if (out_dtype == TAAC_BF16)
+      hipLaunchKernelGGL(reduce_splits_kernel<bf16_t>, dim3(bblocks), dim3(kThreads), 0, s, part_b, static_cast<bf16_t*>(db),
+                         static_cast<int64_t>(N), splits);
+    else
+      hipLaunchKernelGGL(reduce_splits_kernel<float>, dim3(bblocks), dim3(kThreads), 0, s, part_b, static_cast<float*>(db),
+                         static_cast<int64_t>(N), splits);
+  }
+  return check_launch(name);
+}
+
+extern "C" int taac_swiglu_bwd(const void* gu, int64_t ldgu, const void* dhidden, int64_t lddh, void* dgu, int64_t lddgu,
+                               void* hidden, int64_t ldh, int64_t M, int32_t F, int gate_first, void* stream) {
+  using namespace taac;
+  const char* name = "taac_swiglu_bwd";
+  if (M < 0 || F <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0 and F > 0", name);
+  if (F % 8 != 0 || ldgu % 8 != 0 || ldgu < 2 * F || (dhidden && (lddh % 8 != 0 || lddh < F)) ||
+      (dgu && (lddgu % 8 != 0 || lddgu < 2 * F)) || (hidden && (ldh % 8 != 0 || ldh < F)))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: F and the row strides must be multiples of 8 and cover a row", name);
+  if (M == 0) return TAAC_OK;
+  if (!gu || (!dgu && !hidden)) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null tensor pointer", name);
+  if (dgu && !dhidden) return set_error(TAAC_ERR_INVALID_VALUE, "%s: dgu needs dhidden", name);
+  if (!aligned16(gu) || !aligned16(dhidden) || !aligned16(dgu) || !aligned16(hidden))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
+  const int64_t work = M * (F / 8);
+  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(static_cast<uint32_t>((work + kThreads - 1) / kThreads)), dim3(kThreads), 0,
+                     as_stream(stream), static_cast<const bf16_t*>(gu), ldgu, static_cast<const bf16_t*>(dhidden), lddh,
+                     static_cast<bf16_t*>(dgu), lddgu, static_cast<bf16_t*>(hidden), ldh, M, F, gate_first ? 1 : 0);
+  return check_launch(name);
+}

@@ -1,0 +1,191 @@
+"""GPU parity: backward of the dense layers (weight gradient, SiLU-gate backward, and the autograd routes of norm_linear /
+swiglu_ffn / the interaction block) against torch autograd of the CPU oracle's formulas evaluated in float64. Tolerance:
+the reference's gradient tolerance for its 16-bit GPU kernels (tests/gpu/infrastructure/accelerators/
+test_tilelang_ops_cuda.py:98-141), 3e-2, relative to the largest expected value of each gradient."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import reference as oracle
+from taac_2026_amd.api import (UnifiedInteractionBlock, linear, linear_wgrad, norm_linear, swiglu_backward, swiglu_ffn)
+
+pytestmark = pytest.mark.gpu
+
+
+def _close(got: torch.Tensor, want: torch.Tensor, tol: float = 3e-2) -> None:
+    want = want.double()
+    scale = want.abs().max().item()
+    assert (got.detach().cpu().double() - want).abs().max().item() <= tol * max(scale, 1e-6), (
+        (got.detach().cpu().double() - want).abs().max().item(), scale)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 8, 8), (33, 64, 256), (1000, 768, 256), (5000, 256, 1024), (4099, 2048, 256),
+                                   (777, 72, 40)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_weight_gradient_is_the_product_over_the_tokens(device, m, n, k, dtype):
+    g = torch.Generator().manual_seed(m + n)
+    dy = torch.randn(m, n, generator=g).to(torch.bfloat16)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    grad_w, grad_b = linear_wgrad(dy.to(device), a.to(device), dtype=dtype)
+    assert grad_w.dtype == dtype and grad_w.shape == (n, k) and grad_b.shape == (n,)
+    _close(grad_w, dy.double().t() @ a.double(), 1e-2)
+    _close(grad_b, dy.double().sum(0), 1e-2)
+    again_w, again_b = linear_wgrad(dy.to(device), a.to(device), dtype=dtype)
+    assert torch.equal(again_w, grad_w) and torch.equal(again_b, grad_b)      # fixed summation order
+    without, none = linear_wgrad(dy.to(device), a.to(device), with_bias=False, dtype=dtype)
+    assert none is None and torch.equal(without, grad_w)
+
+
+def test_weight_gradient_of_strided_rows_and_errors(device):
+    g = torch.Generator().manual_seed(2)
+    packed = torch.randn(300, 3 * 64, generator=g).to(torch.bfloat16).to(device)
+    a = torch.randn(300, 128, generator=g).to(torch.bfloat16).to(device)
+    dy = packed[:, 64:128]                                                   # a column slice: row stride 192
+    grad_w, _ = linear_wgrad(dy, a, dtype=torch.float32)
+    _close(grad_w, dy.cpu().double().t() @ a.cpu().double(), 1e-2)
+    with pytest.raises(ValueError, match="same number of rows"):
+        linear_wgrad(dy[:10], a)
+    with pytest.raises(RuntimeError, match="multiples of 8"):
+        linear_wgrad(torch.zeros(4, 12, dtype=torch.bfloat16, device=device), torch.zeros(4, 16, dtype=torch.bfloat16, device=device))
+
+
+@pytest.mark.parametrize("gate_first", [True, False])
+def test_silu_gate_backward(device, gate_first):
+    g = torch.Generator().manual_seed(int(gate_first))
+    pre = (2 * torch.randn(257, 2 * 96, generator=g)).to(torch.bfloat16)
+    grad_hidden = torch.randn(257, 96, generator=g).to(torch.bfloat16)
+    hidden, grad_pre = swiglu_backward(pre.to(device), grad_hidden.to(device), gate_first=gate_first)
+    ref = pre.double().requires_grad_(True)
+    gate, value = ref.chunk(2, dim=-1)
+    want = F.silu(gate) * value if gate_first else gate * F.silu(value)
+    want.backward(grad_hidden.double())
+    _close(hidden, want.detach(), 1e-2)
+    _close(grad_pre, ref.grad, 1e-2)
+    only_hidden, none = swiglu_backward(pre.to(device), None, gate_first=gate_first)
+    assert none is None and torch.equal(only_hidden, hidden)
+
+
+def _dense_case(m, d, n, seed):
+    g = torch.Generator().manual_seed(seed)
+    bf = lambda t: t.to(torch.bfloat16)  # noqa: E731
+    x = bf(torch.randn(m, d, generator=g))
+    w = bf(torch.randn(n, d, generator=g) * d ** -0.5)
+    b = bf(0.1 * torch.randn(n, generator=g))
+    nw = bf(1 + 0.1 * torch.randn(d, generator=g))
+    res = bf(torch.randn(m, n, generator=g))
+    dy = bf(torch.randn(m, n, generator=g))
+    return x, w, b, nw, res, dy
+
+
+@pytest.mark.parametrize("m,d,n", [(300, 256, 768), (129, 128, 128), (50, 64, 96)])
+@pytest.mark.parametrize("with_norm,with_residual", [(True, False), (False, True), (True, True)])
+def test_norm_linear_takes_a_gradient(device, m, d, n, with_norm, with_residual):
+    """RMSNorm -> linear -> + residual, fused widths (128 / 256) and the composed route (64): every gradient against float64
+    autograd of the oracle's formulas."""
+    x, w, b, nw, res, dy = _dense_case(m, d, n, seed=m + n)
+    dev = [t.to(device).requires_grad_(True) for t in (x, w, b, nw, res)]
+    out = norm_linear(dev[0], dev[1], dev[2], norm_weight=dev[3] if with_norm else None,
+                      residual=dev[4] if with_residual else None)
+    out.backward(dy.to(device))
+    ref = [t.double().requires_grad_(True) for t in (x, w, b, nw, res)]
+    h = oracle.rms_norm(ref[0], ref[3]) if with_norm else ref[0]
+    want = F.linear(h, ref[1], ref[2]) + (ref[4] if with_residual else 0)
+    want.backward(dy.double())
+    _close(out, want.detach(), 2e-2)
+    for index, (got, expected) in enumerate(zip(dev, ref)):
+        if (index == 3 and not with_norm) or (index == 4 and not with_residual):
+            assert got.grad is None
+        else:
+            _close(got.grad, expected.grad)
+
+
+def test_linear_takes_a_gradient_and_the_forward_is_the_inference_kernel(device):
+    x, w, b, _, _, dy = _dense_case(200, 256, 512, seed=9)
+    xd, wd, bd = (t.to(device).requires_grad_(True) for t in (x, w, b))
+    out = linear(xd.view(4, 50, 256), wd, bd)
+    with torch.no_grad():
+        assert torch.equal(out.detach(), linear(xd.view(4, 50, 256), wd, bd))
+    out.backward(dy.to(device).view(4, 50, 512))
+    _close(wd.grad, dy.double().t() @ x.double())
+    _close(xd.grad, dy.double() @ w.double())
+    _close(bd.grad, dy.double().sum(0))
+    with pytest.raises(RuntimeError, match="inference route"):
+        norm_linear(xd, wd, bd, out=torch.empty(200, 512, dtype=torch.bfloat16, device=device))
+
+
+@pytest.mark.parametrize("m,d,f,gate_first,with_norm", [(300, 256, 512, True, True), (100, 128, 96, False, True),
+                                                          (64, 64, 80, True, False), (513, 256, 1024, True, True)])
+def test_swiglu_ffn_takes_a_gradient(device, m, d, f, gate_first, with_norm):
+    g = torch.Generator().manual_seed(m + f)
+    bf = lambda t: t.to(torch.bfloat16)  # noqa: E731
+    x = bf(torch.randn(m, d, generator=g))
+    nw = bf(1 + 0.1 * torch.randn(d, generator=g))
+    up_w, up_b = bf(torch.randn(2 * f, d, generator=g) * d ** -0.5), bf(0.1 * torch.randn(2 * f, generator=g))
+    down_w, down_b = bf(torch.randn(d, f, generator=g) * f ** -0.5), bf(0.1 * torch.randn(d, generator=g))
+    dy = bf(torch.randn(m, d, generator=g))
+    tensors = (x, nw, up_w, up_b, down_w, down_b)
+    dev = [t.to(device).requires_grad_(True) for t in tensors]
+    out = swiglu_ffn(dev[0], dev[2], dev[3], dev[4], dev[5], residual=dev[0], gate_first=gate_first,
+                     norm_weight=dev[1] if with_norm else None)
+    out.backward(dy.to(device))
+    ref = [t.double().requires_grad_(True) for t in tensors]
+    h = oracle.rms_norm(ref[0], ref[1]) if with_norm else ref[0]
+    want = ref[0] + oracle.swiglu_ffn(h, ref[2], ref[3], ref[4], ref[5], gate_first=gate_first)
+    want.backward(dy.double())
+    _close(out, want.detach(), 2e-2)
+    for index, (got, expected) in enumerate(zip(dev, ref)):
+        if index == 1 and not with_norm:
+            assert got.grad is None
+        else:
+            _close(got.grad, expected.grad)
+
+
+def test_interaction_block_takes_a_gradient_end_to_end(device):
+    """``UnifiedInteractionBlock`` in training mode (plain attention layer, key-length mask): output and the gradient of
+    the input and of every parameter against float64 autograd of ``oracle.interaction_block``
+    (experiments/symbiosis/backbone.py:58-68)."""
+    batch, tokens, d_model, heads, mult = 3, 48, 128, 4, 2
+    g = torch.Generator().manual_seed(1)
+    block = UnifiedInteractionBlock(d_model, heads, mult, qk_norm=False)
+    with torch.no_grad():
+        for parameter in block.parameters():
+            if parameter.ndim == 1:
+                parameter.copy_((1.0 if parameter.shape[0] == d_model and parameter.mean() > 0.5 else 0.0)
+                                + 0.1 * torch.randn(parameter.shape, generator=g))
+            else:
+                parameter.copy_(torch.randn(parameter.shape, generator=g) * parameter.shape[1] ** -0.5)
+    block = block.to(torch.bfloat16)
+    weights = {
+        "attn_norm.weight": block.attn_norm.weight, "qkv.weight": block.attention.qkv.weight,
+        "qkv.bias": block.attention.qkv.bias, "out.weight": block.attention.out.weight, "out.bias": block.attention.out.bias,
+        "ffn_norm.weight": block.ffn_norm.weight, "up.weight": block.ffn.up.weight, "up.bias": block.ffn.up.bias,
+        "down.weight": block.ffn.down.weight, "down.bias": block.ffn.down.bias,
+    }
+    reference = {name: value.detach().double().requires_grad_(True) for name, value in weights.items()}
+    x = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16)
+    lengths = torch.tensor([48, 17, 33], dtype=torch.int32)
+    padding = torch.arange(tokens)[None, :] >= lengths[:, None]
+    grad_out = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16)
+
+    block = block.to(device).train()
+    xd = x.to(device).requires_grad_(True)
+    out, _ = block(xd, padding.to(device), None, key_lengths=lengths.to(device))
+    out.backward(grad_out.to(device))
+
+    xr = x.double().requires_grad_(True)
+    mask = (~padding)[:, None, None, :].expand(batch, 1, tokens, tokens)
+    want, _ = oracle.interaction_block(xr, padding, mask, reference, num_heads=heads)
+    want.backward(grad_out.double())
+    _close(out, want.detach(), 2e-2)
+    _close(xd.grad, xr.grad)
+    named = dict(block.named_parameters())
+    lookup = {"attn_norm.weight": "attn_norm.weight", "qkv.weight": "attention.qkv.weight", "qkv.bias": "attention.qkv.bias",
+              "out.weight": "attention.out.weight", "out.bias": "attention.out.bias", "ffn_norm.weight": "ffn_norm.weight",
+              "up.weight": "ffn.up.weight", "up.bias": "ffn.up.bias", "down.weight": "ffn.down.weight",
+              "down.bias": "ffn.down.bias"}
+    for name, parameter_name in lookup.items():
+        assert named[parameter_name].grad is not None, parameter_name
+        _close(named[parameter_name].grad, reference[name].grad)
