@@ -197,7 +197,8 @@ def _kernel_breakdown(inputs, device, iters: int) -> dict:
 
 
 def _operator_figures(device, iters: int) -> dict:
-    """Stand-alone operators at configurations 2 and 3: norm HBM GB/s and masked-attention TFLOP/s."""
+    """Stand-alone operators at configurations 2 and 3: norm HBM GB/s and masked-attention TFLOP/s. Each figure: 20 warm-up
+    launches, then 5 groups of ``iters`` launches between HIP events, the median group."""
     from oracle import reference as oracle
     from taac_2026_amd import workloads
     from taac_2026_amd.api import flash_attention, layer_norm, rms_norm
@@ -211,9 +212,9 @@ def _operator_figures(device, iters: int) -> dict:
         got = layer_norm(xd[:16], gd, bd).cpu().float()
         torch.testing.assert_close(got, oracle.layer_norm_fp32(x[:16], gamma, beta).float(), rtol=2e-2, atol=2e-2)
         nbytes = 2.0 * x.numel() * 2 + 2 * 256
-        ms = _event_ms(lambda: rms_norm(xd, gd), iters, 5)
+        ms = _event_ms(lambda: rms_norm(xd, gd), 5 * iters, 20)
         figures["rmsnorm_bf16_1048576x256"] = {"ms": ms, "gbs": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS}
-        ms = _event_ms(lambda: layer_norm(xd, gd, bd), iters, 5)
+        ms = _event_ms(lambda: layer_norm(xd, gd, bd), 5 * iters, 20)
         figures["layernorm_bf16_1048576x256"] = {"ms": ms, "gbs": (nbytes + 512) / ms / 1e6,
                                                  "frac_hbm": (nbytes + 512) / ms / 1e6 / HBM_PEAK_GBS}
         # backward of both norms at the same shape: x and dy read once, dx written once (dw / db are 512 bytes each)
@@ -222,9 +223,9 @@ def _operator_figures(device, iters: int) -> dict:
         x2d = xd.view(-1, 256)
         dy = torch.randn(x2d.shape, generator=torch.Generator().manual_seed(7)).to(torch.bfloat16).to(device)
         bwd_bytes = 3.0 * x.numel() * 2
-        ms = _event_ms(lambda: hip_rms_norm_backward_kernel(x2d, gd, dy, 1e-6), iters, 5)
+        ms = _event_ms(lambda: hip_rms_norm_backward_kernel(x2d, gd, dy, 1e-6), 5 * iters, 20)
         figures["rmsnorm_bwd_bf16_1048576x256"] = {"ms": ms, "gbs": bwd_bytes / ms / 1e6, "frac_hbm": bwd_bytes / ms / 1e6 / HBM_PEAK_GBS}
-        ms = _event_ms(lambda: hip_layer_norm_backward_kernel(x2d, gd, dy, 1e-5), iters, 5)
+        ms = _event_ms(lambda: hip_layer_norm_backward_kernel(x2d, gd, dy, 1e-5), 5 * iters, 20)
         figures["layernorm_bwd_bf16_1048576x256"] = {"ms": ms, "gbs": bwd_bytes / ms / 1e6, "frac_hbm": bwd_bytes / ms / 1e6 / HBM_PEAK_GBS}
         del xd, x2d, dy
 
@@ -238,7 +239,7 @@ def _operator_figures(device, iters: int) -> dict:
         sum_sq = float((lengths.double() ** 2).sum().item())
         useful = 4.0 * H * d * sum_sq
         nbytes = 3.0 * H * d * 2 * float(lengths.sum().item()) + B * H * T * d * 2
-        ms = _event_ms(lambda: flash_attention(qd, kd, vd, key_lengths=ld, zero_padded_queries=True), iters, 5)
+        ms = _event_ms(lambda: flash_attention(qd, kd, vd, key_lengths=ld, zero_padded_queries=True), 5 * iters, 20)
         figures["attention_bf16_B2048_H4_T256_d64"] = {
             "ms": ms,
             "useful_tflops": useful / ms / 1e9,
