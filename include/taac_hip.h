@@ -577,6 +577,23 @@ int taac_embedding_bag_mean_fwd(const void* weight, int64_t num_embeddings, int3
                                 int dtype, void* stream);
 
 /*
+ * Gradient of the table under taac_embedding_bag_mean_fwd: grad_weight[id, :] = sum over the bags b and their slots j
+ * with values[b, j] == id of grad_out[b, :] / max(count_b, 1), count_b = the number of ids of bag b that are neither the
+ * padding id 0 nor outside [0, num_embeddings); rows no bag names are zero. The whole [num_embeddings, emb_dim] gradient
+ * is written (it is cleared here, not by the caller). Sums are formed in fp32 by float add-to-memory, so a row named
+ * by several bags adds in an order that may differ from launch to launch (last-bit differences, as with the
+ * reference's atomic adds); a 16-bit table needs workspace = num_embeddings * emb_dim floats (16-byte aligned) for
+ * those sums and is rounded once at the end, an fp32 table is accumulated in place (workspace may be NULL).
+ * values: [bags, bag_size] int32 / int64 contiguous; grad_out: [bags, emb_dim] contiguous in the table's dtype;
+ * grad_weight: [num_embeddings, emb_dim] in the table's dtype.
+ * Replaces: the embedding-bag mean backward kernels (src/taac2026/infrastructure/accelerators/embedding/kernels/
+ * triton.py:91-150, tilelang.py:95-140) called from the autograd functions' backward (embedding_bag.py:345-353).
+ */
+int taac_embedding_bag_mean_bwd(const void* values, int index_is_int64, int64_t bags, int32_t bag_size,
+                                const void* grad_out, void* grad_weight, int64_t num_embeddings, int32_t emb_dim,
+                                void* workspace, int dtype, void* stream);
+
+/*
  * Weights of one backbone block; every pointer is a device pointer to bf16 data in torch nn.Linear layout.
  * Field names follow the reference's parameter names (experiments/symbiosis/backbone.py:24-56).
  * Biases may be NULL (treated as zero). query_norm_weight / key_norm_weight are the attention layer's

@@ -189,6 +189,10 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         c_int,
         [c_void_p, c_int64, c_int32, c_void_p, c_int, c_int64, c_int32, c_void_p, c_void_p, c_int, c_void_p],
     ),
+    "taac_embedding_bag_mean_bwd": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int32, c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_int, c_void_p],
+    ),
     "taac_candidate_readout_fwd": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_float,

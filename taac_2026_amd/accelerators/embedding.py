@@ -9,7 +9,7 @@ from __future__ import annotations
 import torch
 
 from taac_2026_amd import _native
-from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference, require_same_device
+from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_same_device
 
 EMBEDDING_BAG_MEAN_BACKENDS = ("hip", "torch", "tilelang", "triton", "cuembed")
 
@@ -65,6 +65,46 @@ def hip_embedding_bag_mean_kernel(embedding_weight: torch.Tensor, values: torch.
     return out
 
 
+def hip_embedding_bag_mean_backward_kernel(values: torch.Tensor, grad_out: torch.Tensor, num_embeddings: int) -> torch.Tensor:
+    """``(values (B, L), grad_out (B, E)) -> grad_weight (N, E)`` in grad_out's dtype: the backward kernels of the
+    reference (embedding/kernels/triton.py:91-150, tilelang.py:95-140). fp32 sums; a 16-bit gradient is rounded once."""
+    library = _native.load_library()
+    require_cuda_tensors("hip embedding_bag_mean backward", values, grad_out)
+    grad_out = grad_out.contiguous()
+    emb_dim = grad_out.shape[1]
+    grad_weight = torch.empty(num_embeddings, emb_dim, dtype=grad_out.dtype, device=grad_out.device)
+    workspace = None
+    if grad_out.dtype != torch.float32:
+        workspace = torch.empty(num_embeddings, emb_dim, dtype=torch.float32, device=grad_out.device)
+    status = library.taac_embedding_bag_mean_bwd(
+        values.data_ptr(), int(values.dtype == torch.int64), values.shape[0], values.shape[1], grad_out.data_ptr(),
+        grad_weight.data_ptr(), num_embeddings, emb_dim, _native.ptr(workspace), _native.dtype_code(grad_out.dtype),
+        _native.current_stream(grad_out.device),
+    )
+    _native.check(status, "embedding_bag_mean backward")
+    return grad_weight
+
+
+class _HipEmbeddingBagMeanFunction(torch.autograd.Function):
+    """embedding_bag.py:327-353: the ids are saved, the table's gradient comes from the backward kernel."""
+
+    @staticmethod
+    def forward(ctx, embedding_weight: torch.Tensor, values: torch.Tensor, check_indices: bool) -> torch.Tensor:
+        out = hip_embedding_bag_mean_kernel(embedding_weight, values, check_indices=check_indices)
+        ctx.save_for_backward(values)
+        ctx.num_embeddings = embedding_weight.shape[0]
+        ctx.weight_dtype = embedding_weight.dtype
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out: torch.Tensor):
+        if not ctx.needs_input_grad[0]:
+            return None, None, None
+        (values,) = ctx.saved_tensors
+        grad_weight = hip_embedding_bag_mean_backward_kernel(values, grad_out.to(ctx.weight_dtype), ctx.num_embeddings)
+        return grad_weight, None, None
+
+
 def embedding_bag_mean(embedding_weight: torch.Tensor, values: torch.Tensor, *, backend: str = "hip",
                        block_rows: int | None = None, block_cols: int | None = None,
                        check_indices: bool = False) -> torch.Tensor:
@@ -73,13 +113,15 @@ def embedding_bag_mean(embedding_weight: torch.Tensor, values: torch.Tensor, *, 
     del block_rows, block_cols
     weight, ids, _ = _normalize_embedding_bag_mean_inputs(embedding_weight, values)
     _resolve_embedding_bag_mean_backend(weight, ids, backend)
-    require_inference("hip embedding_bag_mean", weight)
+    if torch.is_grad_enabled() and weight.requires_grad:
+        return _HipEmbeddingBagMeanFunction.apply(weight, ids, check_indices)
     return hip_embedding_bag_mean_kernel(weight, ids, check_indices=check_indices)
 
 
 __all__ = [
     "EMBEDDING_BAG_MEAN_BACKENDS",
     "embedding_bag_mean",
+    "hip_embedding_bag_mean_backward_kernel",
     "hip_embedding_bag_mean_kernel",
     "resolved_embedding_bag_mean_backend",
 ]

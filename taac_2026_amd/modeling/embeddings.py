@@ -1,7 +1,8 @@
 """Embedding primitives in front of the token backbone (src/taac2026/infrastructure/modeling/embeddings.py:65-80).
 
-``sparse_embedding_bag_mean`` is the forward of the reference helper of the same name: the reference wraps it in an
-autograd function only to build a sparse weight gradient for training, which this forward-only build does not have.
+``sparse_embedding_bag_mean`` follows the reference helper of the same name in the forward. The reference wraps it in an
+autograd function that hands the optimiser an uncoalesced sparse COO gradient (embeddings.py:17-63); here a table that
+requires a gradient takes the dense gradient of the accelerator's autograd route (the embedding-bag backward kernel).
 ``hash_compress_ids`` is the small integer helper that folds raw ids into a table's bucket range before the lookup.
 """
 
@@ -13,7 +14,7 @@ from taac_2026_amd.accelerators.embedding import embedding_bag_mean
 
 
 def sparse_embedding_bag_mean(weight: torch.Tensor, values: torch.Tensor) -> torch.Tensor:
-    """Mean of ``weight`` rows over each bag's non-zero ids (embeddings.py:65-71, forward only)."""
+    """Mean of ``weight`` rows over each bag's non-zero ids (embeddings.py:65-71)."""
     return embedding_bag_mean(weight, values)
 
 

@@ -115,6 +115,17 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
     assert bag(bags=0) == ok
     assert bag(dtype=9) == invalid
 
+    def bag_bwd(**kw):
+        a = dict(values=fake, i64=0, bags=4, size=2, grad_out=fake, grad_weight=fake, n=16, e=8, workspace=None, dtype=f32)
+        a.update(kw)
+        return library.taac_embedding_bag_mean_bwd(a["values"], a["i64"], a["bags"], a["size"], a["grad_out"],
+                                                   a["grad_weight"], a["n"], a["e"], a["workspace"], a["dtype"], None)
+
+    assert bag_bwd(e=0) == invalid
+    assert bag_bwd(grad_weight=None) == invalid and b"null" in library.taac_last_error()
+    assert bag_bwd(dtype=bf16) == invalid and b"workspace" in library.taac_last_error()
+    assert bag_bwd(dtype=9) == invalid
+
     # normalisation backward: workspace size, too-small workspace, width outside the envelope
     floats = library.taac_norm_bwd_workspace_floats(1000, 256, 0)
     assert floats > 0 and library.taac_norm_bwd_workspace_floats(1000, 256, 1) == 2 * floats
