@@ -51,6 +51,9 @@ class StructuredAttentionMask:
     query_self: torch.Tensor | None    # bool (B, Tq)
     sample_stride: int = 0             # words between the bit matrices of consecutive samples (front layout), else 0
     padding_source: torch.Tensor | None = None  # the (B, Tk) padding mask that key_valid is the complement of, if any
+    # few visible 32 x 32 tiles per query tile (sliding windows, a few global rows / columns): the kernel that gives every
+    # 32-query tile its own wavefront and visits only that tile's visible key tiles pays; dense masks keep the chunked one
+    sparse: bool = False
     # what callers derive from this mask once per forward pass (row indices, its front-layout form): the blocks of a
     # stack receive the same mask object and share it
     cache: dict = field(default_factory=dict, compare=False, repr=False)
@@ -102,12 +105,14 @@ def _pack_bits(mask: torch.Tensor) -> torch.Tensor:
 
 def build_structured_mask(
     structural: torch.Tensor, key_valid: torch.Tensor | None = None, query_self: torch.Tensor | None = None,
-    *, padding_source: torch.Tensor | None = None,
+    *, padding_source: torch.Tensor | None = None, sparse: bool = False,
 ) -> StructuredAttentionMask:
     """``structural`` (Tq, Tk) bool, True = attend; ``key_valid`` (B, Tk) bool or None; ``query_self`` (B, Tq) bool or
     None (needs Tq == Tk). Everything stays on the device (no host synchronisation). ``padding_source``: the padding
     mask whose non-padded positions are exactly the valid keys of every sample that has one (a caller that skips the
-    padded rows with the same mask can then run the attention over the valid tokens only)."""
+    padded rows with the same mask can then run the attention over the valid tokens only). ``sparse``: the caller knows
+    that a query tile sees few key tiles (a sliding window plus a few global rows and columns) and prefers the kernel
+    built for that; the result does not depend on it."""
     name = "hip build_structured_mask"
     require_cuda_tensors(name, structural, key_valid, query_self)
     for tensor, label in ((structural, "structural"), (key_valid, "key_valid"), (query_self, "query_self")):
@@ -130,6 +135,7 @@ def build_structured_mask(
     return StructuredAttentionMask(
         struct_bits, block_any, None if key_valid is None else _pack_bits(key_valid),
         None if query_self is None else _pack_bits(query_self), structural, key_valid, query_self, 0, padding_source,
+        sparse=bool(sparse),
     )
 
 
@@ -165,7 +171,34 @@ def plan_structured_attention_mask(q: torch.Tensor, k: torch.Tensor, attn_mask: 
         )
     if query_self is not None and not bool(query_self.any()):
         query_self = None
-    return build_structured_mask(structural, key_valid, query_self)
+    return build_structured_mask(structural, key_valid, query_self, sparse=_few_visible_tiles(structural))
+
+
+def _few_visible_tiles(structural: torch.Tensor) -> bool:
+    """True when at most a third of the 32 x 32 tiles of the (Tq, Tk) structure hold a visible pair (one host sync)."""
+    query_len, kv_len = structural.shape
+    if kv_len > 2048:
+        return False
+    padded = torch.zeros((query_len + 31) // 32 * 32, (kv_len + 31) // 32 * 32, dtype=torch.bool, device=structural.device)
+    padded[:query_len, :kv_len] = structural
+    tiles = padded.view(padded.shape[0] // 32, 32, padded.shape[1] // 32, 32).any(dim=3).any(dim=1)
+    return bool(tiles.float().mean().item() <= 1.0 / 3.0)
+
+
+def _tile_words(mask: StructuredAttentionMask, batch: int) -> torch.Tensor:
+    """The mask's structure ORed over the 32 query rows of each tile (made once per mask object)."""
+    words = mask.cache.get("tile_words")
+    if words is None:
+        query_len, kv_len = mask.structural.shape
+        samples = batch if mask.sample_stride else 1
+        words = torch.empty(samples, (query_len + 31) // 32, (kv_len + 31) // 32, dtype=torch.int32,
+                            device=mask.struct_bits.device)
+        library = _native.load_library()
+        status = library.taac_mask_tile_words(mask.struct_bits.data_ptr(), samples, query_len, kv_len, int(mask.sample_stride),
+                                              words.data_ptr(), _native.current_stream(words.device))
+        _native.check(status, "mask_tile_words")
+        mask.cache["tile_words"] = words
+    return words
 
 
 def _normalize_flash_attention_inputs(
@@ -377,9 +410,12 @@ def hip_flash_attention_kernel(
                 or (sm.sample_stride and sm.struct_bits.shape[0] != batch * query_len):
             raise ValueError("flash_attention: the structured mask does not match (batch, query_len, kv_len)")
         require_cuda_tensors("hip flash_attention", sm.struct_bits)
-        status = library.taac_flash_attn_masked_fwd(
+        per_tile = sm.sparse and head_dim in (32, 64) and k.shape[2] <= 2048 and k.stride(2) < (1 << 20) and v.stride(2) < (1 << 20)
+        entry = library.taac_flash_attn_sparse_fwd if per_tile else library.taac_flash_attn_masked_fwd
+        status = entry(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), sm.struct_bits.data_ptr(),
-            int(sm.sample_stride), _native.ptr(sm.block_any), _native.ptr(sm.valid_bits), _native.ptr(sm.self_bits),
+            int(sm.sample_stride), _tile_words(sm, batch).data_ptr() if per_tile else _native.ptr(sm.block_any),
+            _native.ptr(sm.valid_bits), _native.ptr(sm.self_bits),
             _native.ptr(q_row_scale),
             _native.ptr(k_row_scale), _native.ptr(q_col_scale), out.data_ptr(),
             batch, heads, query_len, k.shape[2], head_dim,

@@ -53,6 +53,7 @@ struct AttnParams {
   const uint32_t* self_bits;    // [B][ceil(Tq / 32)] or null: flagged query rows return their own value row
   const uint8_t* block_any;     // [nqc][nkc]: some query of the 128-row block sees some key of the 64-key chunk;
                                 // null (per-sample structure only): every chunk is visited
+  const uint32_t* tile_words;   // per-tile kernel: [samples][ceil(Tq / 32)][wpr], struct_bits ORed over a tile's 32 rows
   float* lse;                   // [B, H, Tq] log-sum-exp of the scaled scores (natural log) for the backward, or null
   int32_t wpr;                  // words per row of struct_bits / valid_bits = ceil(Tk / 32)
   int32_t nkc;                  // key chunks = ceil(Tk / 64)
@@ -938,6 +939,262 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------------------------
+// Structured masks whose visible part is a small fraction of the score matrix (sliding windows plus a few always-visible
+// columns and rows): one wavefront per 32-query tile, on its own - no workgroup, no barrier, no shared chunk list.
+//   * The lane's row of structure bits (ANDed with the sample's key validity and the valid length) is read once, 16
+//     words at a time; a ballot per word gives the 32-key tiles in which some query of the wavefront sees some key, and
+//     only those tiles are visited. Query rows in the padding and self-only rows contribute nothing to that set.
+//   * K fragments (the A operand of S^T = K Q^T: key l32, 8 features) come straight from global memory - a tile's rows
+//     are read completely by the 64 lanes - and the V tile's pieces are requested one tile ahead of their use. V passes
+//     through a wavefront-private LDS tile (row-major, rows of 128 bytes swizzled like the chunked kernel's) and is read
+//     column-wise with transposed LDS reads. Rows of invalid keys may be uninitialised memory: their scores are replaced
+//     by selects, their V rows stored as zeros.
+// Same arithmetic per tile as the general kernel taken one tile at a time.
+// ------------------------------------------------------------------------------------------------------------------
+template <typename T, int DP, bool SCALED>
+__global__ __launch_bounds__(kWave) void flash_attn_fwd_sparse_kernel(const AttnParams p) {
+  typedef typename Vec8<T>::type vec_t;
+  typedef typename Vec8<T>::half_type vec4_t;
+  static_assert(DP == 32 || DP == 64, "row swizzles are written for 64- and 128-byte rows");
+  constexpr int KSTEPS = DP / 16;
+  constexpr int MB = DP / 32;
+  constexpr int C8 = DP / 8;
+  constexpr int ROWB = DP * 2;
+  constexpr int VT_BYTES = 32 * ROWB;       // the V tile
+  constexpr int PPT = 32 * C8 / kWave;      // 16-byte pieces per lane and tile
+  constexpr int OROW = DP * 2 + 16;
+  constexpr int OT_BYTES = 32 * OROW;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[VT_BYTES > OT_BYTES ? VT_BYTES : OT_BYTES];
+
+  const uint32_t nqt = static_cast<uint32_t>((p.Tq + 31) / 32);
+  const uint32_t logical = xcd_remap(blockIdx.x, gridDim.x);
+  const int qt = static_cast<int>(logical % nqt);
+  const int bh = static_cast<int>(logical / nqt);
+  const int h = bh % p.H;
+  const int b = bh / p.H;
+  const int lane = threadIdx.x;
+  const int l32 = lane % 32;
+  const int hh = lane / 32;
+
+  const T* qb = static_cast<const T*>(p.q) + b * p.qs[0] + h * p.qs[1];
+  const T* kb = static_cast<const T*>(p.k) + b * p.ks[0] + h * p.ks[1];
+  const T* vb = static_cast<const T*>(p.v) + b * p.vs[0] + h * p.vs[1];
+  T* ob = static_cast<T*>(p.o) + b * p.os[0] + h * p.os[1];
+
+  int len = p.Tk;
+  if (p.key_lengths != nullptr) {
+    len = p.key_lengths[b];
+    len = len < 0 ? 0 : (len > p.Tk ? p.Tk : len);
+  }
+  const int q_begin = qt * 32;
+  const int q_valid = p.zero_pad ? (len < p.Tq ? len : p.Tq) : p.Tq;
+  vec_t zero_vec;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) zero_vec[e] = static_cast<T>(0.f);
+  const int c8 = lane % C8;
+  constexpr int RPP = kWave / C8;
+  if (q_begin >= q_valid) {  // whole tile in the padding: zero-fill its rows, or leave them alone
+    if (p.zero_pad == 2) return;
+#pragma unroll
+    for (int pass = 0; pass < 32 / RPP; ++pass) {
+      const int row = q_begin + pass * RPP + lane / C8;
+      if (row < p.Tq) *reinterpret_cast<vec_t*>(ob + row * p.os[2] + c8 * 8) = zero_vec;
+    }
+    return;
+  }
+
+  const int qi = q_begin + l32;
+  // self-only rows return their value row (epilogue) and take no part in the products
+  uint32_t self_word = 0u;
+  if (p.self_bits != nullptr) self_word = p.self_bits[static_cast<int64_t>(b) * ((p.Tq + 31) / 32) + qt];
+  const bool row_active = qi < q_valid && ((self_word >> l32) & 1u) == 0u;
+  const uint32_t* bits_row = p.struct_bits + b * p.struct_stride + static_cast<int64_t>(qi < p.Tq ? qi : 0) * p.wpr;
+  // Lane w holds word w of the sample's key validity, cut at the valid length (at most 64 words: Tk <= 2048), and word w
+  // of the structure bits ORed over the tile's 32 query rows: one ballot then names the key tiles to visit.
+  uint32_t valid_lane = 0u, tile_lane = 0u;
+  if (lane < p.wpr) {
+    valid_lane = p.valid_bits != nullptr ? p.valid_bits[static_cast<int64_t>(b) * p.wpr + lane] : ~0u;
+    tile_lane = p.tile_words[(p.struct_stride != 0 ? static_cast<int64_t>(b) * nqt * p.wpr : 0) + static_cast<int64_t>(qt) * p.wpr + lane];
+  }
+  {
+    const int rest = len - lane * 32;
+    if (rest < 32) valid_lane &= rest <= 0 ? 0u : ((1u << rest) - 1u);
+  }
+  auto valid_word = [&](int w) -> uint32_t { return __builtin_amdgcn_readlane(valid_lane, w); };
+
+  float c = p.scale_log2;
+  if (SCALED && p.q_row_scale != nullptr && qi < q_valid) c *= p.q_row_scale[static_cast<int64_t>(b) * p.Tq + qi];
+  vec_t qf[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    qf[s] = qi < q_valid ? *reinterpret_cast<const vec_t*>(qb + qi * p.qs[2] + 16 * s + 8 * hh) : zero_vec;
+    if (SCALED && p.q_col_scale != nullptr) {
+      const float* cf = p.q_col_scale + h * p.d + 16 * s + 8 * hh;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<T>(static_cast<float>(qf[s][e]) * cf[e]);
+    }
+  }
+  // ---- the tiles this wavefront visits: bit kt of `tiles` (none when every row is in the padding or self-only) -------
+  uint64_t tiles = __builtin_amdgcn_ballot_w64((tile_lane & valid_lane) != 0u);
+  if (__builtin_amdgcn_ballot_w64(row_active) == 0ull) tiles = 0ull;
+
+  f32x16 oacc[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) oacc[mb][j] = 0.f;
+  float m_run = -INFINITY;
+  float l_run = 0.f;
+
+  auto v_swizzle = [](int r) -> int { return DP == 32 ? 0 : 4 * ((r / 2) % 2); };
+  const uint32_t k_row_bytes = static_cast<uint32_t>(p.ks[2]) * 2u, v_row_bytes = static_cast<uint32_t>(p.vs[2]) * 2u;
+  const bool scale_keys = SCALED && p.k_row_scale != nullptr;
+  // Operands of a tile: the lane's pieces of the V tile (piece i * 64 + lane = row / C8, 16 bytes / C8), its K fragments,
+  // its word of the mask and its key's factor. Two sets: a tile is consumed while the one after it is in flight.
+  struct TileOperands {
+    vec_t v[PPT], kf[KSTEPS];
+    uint32_t word;
+    float kfac;
+  };
+  auto issue = [&](int kt, TileOperands& t) {
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+      const int slot = i * kWave + lane;
+      int row = kt * 32 + slot / C8;
+      row = row < p.Tk ? row : p.Tk - 1;
+      t.v[i] = *reinterpret_cast<const vec_t*>(reinterpret_cast<const uint8_t*>(vb) +
+                                               __umul24(static_cast<uint32_t>(row), v_row_bytes) + (slot % C8) * 16);
+    }
+    int krow = kt * 32 + l32;
+    krow = krow < p.Tk ? krow : p.Tk - 1;
+    const uint8_t* ksrc = reinterpret_cast<const uint8_t*>(kb) + __umul24(static_cast<uint32_t>(krow), k_row_bytes) + hh * 16;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) t.kf[s] = *reinterpret_cast<const vec_t*>(ksrc + s * 32);
+    t.word = row_active ? bits_row[kt] : 0u;
+    t.kfac = 1.f;
+    if (SCALED && scale_keys) t.kfac = p.k_row_scale[static_cast<int64_t>(b) * p.Tk + krow];
+  };
+
+  const uint32_t smem_off = lds_offset(smem);
+  const int v_key = 4 * (lane / 32) + (lane % 16) / 4;
+  const uint32_t v_addr = smem_off + static_cast<uint32_t>(
+      v_key * ROWB + ((2 * ((lane / 16) % 2) + (lane % 4) / 2) ^ v_swizzle(v_key)) * 16 + (lane % 2) * 8);
+
+  auto consume = [&](int kt, TileOperands& t) {
+    const uint32_t vword = valid_word(kt);
+    const uint32_t word = t.word & vword;
+    // The V tile goes into the wavefront's LDS tile (the transposed reads of the tile before it have been waited for);
+    // rows of invalid keys are stored as zeros.
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+      const int slot = i * kWave + lane;
+      const int r = slot / C8;
+      const bool ok = ((vword >> r) & 1u) != 0u;
+      *reinterpret_cast<vec_t*>(smem + r * ROWB + ((slot % C8) ^ v_swizzle(r)) * 16) = ok ? t.v[i] : zero_vec;
+    }
+    if (SCALED && scale_keys) {
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t.kf[s][e] = static_cast<T>(static_cast<float>(t.kf[s][e]) * t.kfac);
+    }
+    f32x16 sacc;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) sacc[j] = 0.f;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) sacc = Mfma32<T>::run(t.kf[s], qf[s], sacc);
+    if (__builtin_amdgcn_ballot_w64(word != 0xffffffffu) != 0ull) {  // wavefront-uniform
+      const uint32_t bits = word >> (hh * 4);
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        if (((bits >> ((j / 4) * 8 + (j % 4))) & 1u) == 0u) sacc[j] = -INFINITY;
+    }
+    float mx = sacc[0];
+#pragma unroll
+    for (int j = 1; j < 16; ++j) mx = fmaxf(mx, sacc[j]);
+    mx = pair_max(mx);
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
+    const float mc = -m_use * c;
+    float pr[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) pr[j] = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, mc));
+    vec_t pb[2];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      pb[0][e] = static_cast<T>(pr[e]);
+      pb[1][e] = static_cast<T>(pr[8 + e]);
+    }
+    float rs = frag_sum(pb[0], 0.f);
+    rs = frag_sum(pb[1], rs);
+    rs = pair_sum(rs);
+    l_run = l_run * alpha + rs;
+    m_run = m_new;
+    static_for<MB>([&](auto mb_tag) {
+      constexpr int mb = decltype(mb_tag)::value;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;
+      const uint32_t v_addr_mb = v_addr ^ (mb * 64);
+      u32x2 vt[2][2];
+      lds_read_tr16<0>(vt[0][0], v_addr_mb);
+      lds_read_tr16<8 * ROWB>(vt[0][1], v_addr_mb);
+      lds_read_tr16<16 * ROWB>(vt[1][0], v_addr_mb);
+      lds_read_tr16<24 * ROWB>(vt[1][1], v_addr_mb);
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vt[0][0]), "+v"(vt[0][1]), "+v"(vt[1][0]), "+v"(vt[1][1]) : : "memory");
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const u32x4 bits = {vt[s2][0][0], vt[s2][0][1], vt[s2][1][0], vt[s2][1][1]};
+        oacc[mb] = Mfma32<T>::run(__builtin_bit_cast(vec_t, bits), pb[s2], oacc[mb]);
+      }
+    });
+  };
+
+  auto pop_tile = [&]() -> int {
+    if (tiles == 0ull) return -1;
+    const int kt = __builtin_ctzll(tiles);
+    tiles &= tiles - 1ull;
+    return kt;
+  };
+  TileOperands next;
+  int kt = pop_tile();
+  if (kt >= 0) issue(kt, next);
+  while (kt >= 0) {
+    TileOperands cur = next;
+    const int kt_next = pop_tile();
+    if (kt_next >= 0) issue(kt_next, next);
+    consume(kt, cur);
+    kt = kt_next;
+  }
+
+  // ---- finalise: O / l, transpose through the wavefront's LDS tile, self rows, 16-byte stores -------------------------
+  const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+  const float fin = (qi < q_valid) ? inv : 0.f;
+  uint8_t* tile = smem;
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+    for (int jq = 0; jq < 4; ++jq) {
+      vec4_t ov;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ov[e] = static_cast<T>(oacc[mb][jq * 4 + e] * fin);
+      *reinterpret_cast<vec4_t*>(tile + l32 * OROW + (mb * 32 + jq * 8 + hh * 4) * 2) = ov;
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  const int q_store_end = p.zero_pad == 2 ? q_valid : p.Tq;
+#pragma unroll
+  for (int pass = 0; pass < 32 / RPP; ++pass) {
+    const int row = pass * RPP + lane / C8;
+    const int q_row = q_begin + row;
+    vec_t v = *reinterpret_cast<const vec_t*>(tile + row * OROW + c8 * 16);
+    if (((self_word >> row) & 1u) != 0u && q_row < p.Tq) v = *reinterpret_cast<const vec_t*>(vb + q_row * p.vs[2] + c8 * 8);
+    if (q_row < q_store_end) *reinterpret_cast<vec_t*>(ob + q_row * p.os[2] + c8 * 8) = v;
+  }
+}
+
 template <typename T, int DP>
 void launch(const AttnParams& p, bool causal, bool register_staging, hipStream_t s) {
   const bool scaled = p.q_row_scale != nullptr || p.k_row_scale != nullptr || p.q_col_scale != nullptr;
@@ -948,6 +1205,14 @@ void launch(const AttnParams& p, bool causal, bool register_staging, hipStream_t
                              static_cast<int64_t>(p.Tk) * p.ks[2] * 2 < (1ll << 31) &&
                              static_cast<int64_t>(p.Tk) * p.vs[2] * 2 < (1ll << 31);
   if constexpr (DP == 32 || DP == 64) {
+    if (p.tile_words != nullptr) {  // the entry point has checked the shape
+      const int64_t waves = static_cast<int64_t>((p.Tq + 31) / 32) * p.B * p.H;
+      if (scaled)
+        hipLaunchKernelGGL((flash_attn_fwd_sparse_kernel<T, DP, true>), dim3(static_cast<uint32_t>(waves)), dim3(kWave), 0, s, p);
+      else
+        hipLaunchKernelGGL((flash_attn_fwd_sparse_kernel<T, DP, false>), dim3(static_cast<uint32_t>(waves)), dim3(kWave), 0, s, p);
+      return;
+    }
     // structure bits ride along when they are all there is to the mask: per sample, no validity or self rows, no chunk map
     const bool structure_only = p.struct_bits != nullptr && p.valid_bits == nullptr && p.self_bits == nullptr &&
                                 p.block_any == nullptr;
@@ -1034,6 +1299,7 @@ struct MaskArgs {
   const uint8_t* block_any = nullptr;
   const uint32_t* valid_bits = nullptr;
   const uint32_t* self_bits = nullptr;
+  const uint32_t* tile_words = nullptr;  // given: the one-wavefront-per-query-tile kernel
 };
 
 int attention_entry(const char* name, const void* q, const void* k, const void* v, const int32_t* key_lengths,
@@ -1052,7 +1318,7 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   const int is_causal = mask_flags & TAAC_ATTN_CAUSAL;
   const bool register_staging = (mask_flags & TAAC_ATTN_REGISTER_STAGING) != 0;
   if (mask.struct_bits != nullptr) {
-    if (mask.block_any == nullptr && mask.struct_stride == 0)
+    if (mask.block_any == nullptr && mask.struct_stride == 0 && mask.tile_words == nullptr)
       return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_bits shared by the batch needs block_any", name);
     if (mask.struct_stride < 0 || (mask.struct_stride != 0 && mask.struct_stride < static_cast<int64_t>(Tq) * ((Tk + 31) / 32)))
       return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_sample_stride must be 0 or cover a sample's matrix", name);
@@ -1100,6 +1366,7 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   p.valid_bits = mask.valid_bits;
   p.self_bits = mask.self_bits;
   p.block_any = mask.block_any;
+  p.tile_words = mask.tile_words;
   p.wpr = (Tk + 31) / 32;
   p.nkc = (Tk + kKC - 1) / kKC;
   p.B = B;
@@ -1200,6 +1467,70 @@ extern "C" int taac_flash_attn_masked_fwd(const void* q, const void* k, const vo
   return taac::attention_entry("taac_flash_attn_masked_fwd", q, k, v, key_lengths, mask, q_row_scale, k_row_scale,
                                q_col_scale, nullptr, nullptr, o, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides,
                                0, zero_padded_queries, dtype, stream);
+}
+
+extern "C" int taac_flash_attn_sparse_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
+                                          const uint32_t* struct_bits, int64_t struct_sample_stride,
+                                          const uint32_t* tile_words, const uint32_t* valid_bits,
+                                          const uint32_t* self_bits, const float* q_row_scale, const float* k_row_scale,
+                                          const float* q_col_scale, void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk,
+                                          int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
+                                          const int64_t v_strides[4], const int64_t o_strides[4],
+                                          int zero_padded_queries, int dtype, void* stream) {
+  using namespace taac;
+  const char* name = "taac_flash_attn_sparse_fwd";
+  if (!struct_bits || !tile_words) return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_bits and tile_words must be given", name);
+  if (d != 32 && d != 64) return set_error(TAAC_ERR_UNSUPPORTED, "%s: head_dim must be 32 or 64 (got %d)", name, d);
+  if (Tk < 1 || Tk > 2048) return set_error(TAAC_ERR_UNSUPPORTED, "%s: 1 <= Tk <= 2048 required (got %d)", name, Tk);
+  if (!k_strides || !v_strides) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null stride array", name);
+  if (k_strides[2] >= (1 << 22) || v_strides[2] >= (1 << 22) || static_cast<int64_t>(Tk) * k_strides[2] * 2 >= (1ll << 31) ||
+      static_cast<int64_t>(Tk) * v_strides[2] * 2 >= (1ll << 31))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: key / value row strides must fit 32-bit byte offsets", name);
+  if (static_cast<int64_t>((Tq + 31) / 32) * B * H > 0x7fffffffLL)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many query tiles", name);
+  MaskArgs mask;
+  mask.struct_bits = struct_bits;
+  mask.struct_stride = struct_sample_stride;
+  mask.valid_bits = valid_bits;
+  mask.self_bits = self_bits;
+  mask.tile_words = tile_words;
+  return attention_entry(name, q, k, v, key_lengths, mask, q_row_scale, k_row_scale, q_col_scale, nullptr, nullptr, o, B, H,
+                         Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, 0, zero_padded_queries, dtype, stream);
+}
+
+namespace taac {
+namespace {
+// tile_words[s][t][w] = OR over the rows 32 t .. 32 t + 31 (below Tq) of sample s of struct_bits[row][w]; one lane per word.
+__global__ __launch_bounds__(256) void tile_words_kernel(const uint32_t* __restrict__ bits, int samples, int Tq, int wpr,
+                                                         int64_t stride, uint32_t* __restrict__ tile_words) {
+  const int nqt = (Tq + 31) / 32;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= static_cast<int64_t>(samples) * nqt * wpr) return;
+  const int w = static_cast<int>(idx % wpr);
+  const int t = static_cast<int>((idx / wpr) % nqt);
+  const int64_t smp = idx / wpr / nqt;
+  const uint32_t* src = bits + smp * stride;
+  uint32_t acc = 0u;
+  for (int r = t * 32; r < t * 32 + 32 && r < Tq; ++r) acc |= src[static_cast<int64_t>(r) * wpr + w];
+  tile_words[idx] = acc;
+}
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_mask_tile_words(const uint32_t* struct_bits, int32_t samples, int32_t Tq, int32_t Tk,
+                                    int64_t struct_sample_stride, uint32_t* tile_words, void* stream) {
+  using namespace taac;
+  const char* name = "taac_mask_tile_words";
+  if (samples <= 0 || Tq <= 0 || Tk <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: samples, Tq and Tk must be positive", name);
+  if (!struct_bits || !tile_words) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  const int wpr = (Tk + 31) / 32;
+  if (samples > 1 && struct_sample_stride < static_cast<int64_t>(Tq) * wpr)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_sample_stride must cover a sample's matrix", name);
+  const int64_t words = static_cast<int64_t>(samples) * ((Tq + 31) / 32) * wpr;
+  if (words > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: mask too large", name);
+  hipLaunchKernelGGL(tile_words_kernel, dim3(static_cast<uint32_t>((words + 255) / 256)), dim3(256), 0, as_stream(stream),
+                     struct_bits, samples, Tq, wpr, struct_sample_stride, tile_words);
+  return check_launch(name);
 }
 
 extern "C" int taac_mask_pack_bits(const void* mask, int64_t rows, int32_t cols, uint32_t* bits, void* stream) {

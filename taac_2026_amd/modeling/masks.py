@@ -52,7 +52,12 @@ def bfts_attention_mask(padding_mask: torch.Tensor, role_ids: torch.Tensor, laye
     """``structural & key_valid`` with padded query rows attending to themselves only (model.py:499-503)."""
     structural = bfts_structural_mask(role_ids, layer_index, num_layers, seq_causal=seq_causal,
                                       seq_keep_per_domain=seq_keep_per_domain)
-    return build_structured_mask(structural, ~safe_key_padding_mask(padding_mask), padding_mask)
+    # window layers: a 32-query tile sees its band (two or three key tiles) and the separator columns
+    bottom_full_layers = max(1, int(num_layers) // 2)
+    window = None if layer_index < bottom_full_layers else max(
+        4, math.ceil(int(seq_keep_per_domain) / (2 ** (layer_index - bottom_full_layers))))
+    sparse = window is not None and role_ids.shape[0] <= 2048 and 4 * (window + 64) <= role_ids.shape[0]
+    return build_structured_mask(structural, ~safe_key_padding_mask(padding_mask), padding_mask, sparse=sparse)
 
 
 def metadata_structural_mask(role_ids: torch.Tensor) -> torch.Tensor:

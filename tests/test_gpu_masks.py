@@ -3,6 +3,8 @@ rows) through the C ABI, against the library SDPA with the dense bool mask and t
 
 from __future__ import annotations
 
+from dataclasses import replace
+
 import pytest
 import torch
 import torch.nn.functional as F
@@ -34,8 +36,11 @@ def _expected(q, k, v, dense):
     return torch.where(empty.expand(-1, q.shape[1], -1, -1), torch.zeros_like(out), out)
 
 
+@pytest.mark.parametrize("sparse", [False, True])
 @pytest.mark.parametrize("tokens,dim", [(50, 32), (130, 64), (300, 32), (512, 32), (97, 128)])
-def test_random_structured_masks(device, tokens, dim):
+def test_random_structured_masks(device, tokens, dim, sparse):
+    """``sparse``: the kernel that gives every 32-query tile its own wavefront (head dims 32 and 64; 128 runs the chunked
+    kernel either way)."""
     batch, heads = 3, 2
     q, k, v = _qkv(batch, heads, tokens, dim, tokens + dim)
     g = torch.Generator().manual_seed(tokens)
@@ -45,9 +50,9 @@ def test_random_structured_masks(device, tokens, dim):
     key_valid[1] = True
     query_self = torch.rand(batch, tokens, generator=g) < 0.1
     with torch.no_grad():
-        plain = build_structured_mask(structural.to(device), key_valid.to(device))
-        with_self = build_structured_mask(structural.to(device), key_valid.to(device), query_self.to(device))
-        only_structural = build_structured_mask(structural.to(device))
+        plain = build_structured_mask(structural.to(device), key_valid.to(device), sparse=sparse)
+        with_self = build_structured_mask(structural.to(device), key_valid.to(device), query_self.to(device), sparse=sparse)
+        only_structural = build_structured_mask(structural.to(device), sparse=sparse)
         args = (q.to(device), k.to(device), v.to(device))
         got = flash_attention(*args, structured_mask=plain).cpu()
         got_self = flash_attention(*args, structured_mask=with_self).cpu()
@@ -85,7 +90,11 @@ def test_tokenformer_layer_masks(device, seq_causal):
             mask = bfts_attention_mask(padding.to(device), roles.to(device), layer, layers, seq_causal=seq_causal,
                                        seq_keep_per_domain=64)
             got = flash_attention(q.to(device), k.to(device), v.to(device), structured_mask=mask).cpu()
+            other = flash_attention(q.to(device), k.to(device), v.to(device),
+                                    structured_mask=replace(mask, sparse=not mask.sparse)).cpu()
+        assert mask.sparse == (layer >= 3)               # the window layers prefer the per-tile kernel
         dense = mask.dense().cpu()
+        torch.testing.assert_close(other.float(), got.float(), rtol=2 ** -6, atol=2 ** -6)   # same result from either kernel
         if layer in (0, 3, 5):  # the per-element oracle is slow: three layers cover full, first and narrowest window
             assert torch.equal(dense[:1], oracle.bfts_attention_mask(padding[:1], roles, layer, layers, seq_causal=seq_causal,
                                                                       seq_keep_per_domain=64))
@@ -108,7 +117,9 @@ def test_symbiosis_metadata_mask(device):
         with torch.no_grad():
             mask = module(padding.to(device), roles.to(device))
             got = flash_attention(q.to(device), k.to(device), v.to(device), structured_mask=mask).cpu()
+            per_tile = flash_attention(q.to(device), k.to(device), v.to(device), structured_mask=replace(mask, sparse=True)).cpu()
         dense = mask.dense().cpu()
+        torch.testing.assert_close(per_tile.float(), _expected(q, k, v, dense), **BF16_TOL)
         assert torch.equal(dense[:2], oracle.metadata_attention_mask(padding[:2], roles, enabled=enabled))
         assert dense[:, :, 0, :].any(dim=-1).all() and dense[:, :, 1, :].any(dim=-1).all()   # the reference's own check
         torch.testing.assert_close(got.float(), _expected(q, k, v, dense), **BF16_TOL)
@@ -147,10 +158,12 @@ def test_dense_bool_masks_are_factored(device):
             flash_attention(*args, attn_mask=per_head.to(device))
 
 
-def test_structured_mask_with_key_lengths_and_row_factors(device):
+@pytest.mark.parametrize("sparse", [False, True])
+@pytest.mark.parametrize("dim", [32, 64])
+def test_structured_mask_with_key_lengths_and_row_factors(device, sparse, dim):
     from taac_2026_amd.accelerators.attention import hip_flash_attention_kernel
 
-    batch, heads, tokens, dim = 3, 2, 160, 32
+    batch, heads, tokens = 3, 2, 160
     q, k, v = _qkv(batch, heads, tokens, dim, 4)
     g = torch.Generator().manual_seed(6)
     structural = (torch.arange(tokens)[:, None] - torch.arange(tokens)[None, :]).abs() <= 20
@@ -162,10 +175,39 @@ def test_structured_mask_with_key_lengths_and_row_factors(device):
     expected = _expected(q.float() * sq[:, None, :, None], k.float() * sk[:, None, :, None], v, dense)
     expected = expected * key_valid[:, None, :, None]     # zero_padded_queries
     with torch.no_grad():
-        mask = build_structured_mask(structural.to(device))
+        mask = build_structured_mask(structural.to(device), sparse=sparse)
         got = hip_flash_attention_kernel(q.to(device), k.to(device), v.to(device), lengths.to(device),
                                          zero_padded_queries=True, q_row_scale=sq.to(device), k_row_scale=sk.to(device),
                                          structured_mask=mask).cpu()
         with pytest.raises(ValueError, match="causal"):
             hip_flash_attention_kernel(q.to(device), k.to(device), v.to(device), None, is_causal=True, structured_mask=mask)
     torch.testing.assert_close(got.float(), expected, **BF16_TOL)
+
+
+@pytest.mark.parametrize("dim", [32, 64])
+def test_per_tile_kernel_ignores_the_rows_of_invalid_keys_and_padded_queries(device, dim):
+    """Scattered padding, NaN in the q / k / v rows of padded positions (a caller that skips them never writes them): the
+    valid rows are unchanged, padded query rows return their value row (self-only), tiles nobody sees cost nothing."""
+    batch, heads, tokens = 4, 2, 200
+    q, k, v = _qkv(batch, heads, tokens, dim, 11)
+    g = torch.Generator().manual_seed(12)
+    padding = torch.rand(batch, tokens, generator=g) < 0.4
+    padding[0] = False
+    padding[3, 40:] = True
+    positions = torch.arange(tokens)
+    distance = positions[:, None] - positions[None, :]
+    structural = ((distance >= 0) & (distance <= 9)) | (positions[None, :] == 7) | (positions[:, None] == tokens - 1)
+    poisoned = [t.clone() for t in (q, k, v)]
+    for t in poisoned[:2]:
+        t[padding[:, None, :, None].expand_as(t)] = float("nan")
+    with torch.no_grad():
+        mask = build_structured_mask(structural.to(device), (~padding).to(device), padding.to(device), sparse=True)
+        clean = flash_attention(q.to(device), k.to(device), v.to(device), structured_mask=mask).cpu()
+        got = flash_attention(*(t.to(device) for t in poisoned), structured_mask=mask).cpu()
+        chunked = flash_attention(q.to(device), k.to(device), v.to(device), structured_mask=replace(mask, sparse=False)).cpu()
+    dense = (structural[None] & ~padding[:, None, :])[:, None]
+    valid = (~padding)[:, None, :, None].expand_as(got)
+    assert torch.equal(got[valid], clean[valid]) and torch.isfinite(got[valid]).all()
+    torch.testing.assert_close(clean.float()[valid], _expected(q, k, v, dense)[valid], **BF16_TOL)
+    assert torch.equal(clean[~valid], v[~valid])                 # self-only rows: the value row, bit for bit
+    torch.testing.assert_close(clean.float(), chunked.float(), rtol=2 ** -6, atol=2 ** -6)
