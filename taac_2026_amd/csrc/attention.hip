@@ -64,6 +64,7 @@ struct AttnParams {
   uint32_t nqc;    // query chunks per (batch, head)
   uint32_t total;  // workgroups
   uint32_t nqc_magic, h_magic;  // floor(2^32 / nqc), floor(2^32 / H) (0 for a divisor of 1): divisions without a divide
+  uint32_t nqt_magic;           // the same for the number of 32-query tiles
 };
 
 // x / d and x % d for a divisor known to the host: q = mulhi(x, floor(2^32 / d)) is at most two short of the quotient.
@@ -953,8 +954,10 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
 //     by selects, their V rows stored as zeros.
 // Same arithmetic per tile as the general kernel taken one tile at a time.
 // ------------------------------------------------------------------------------------------------------------------
+constexpr int kSparseWaves = 4;  // independent wavefronts per workgroup: the same query tile of consecutive (batch, head)s
+
 template <typename T, int DP, bool SCALED>
-__global__ __launch_bounds__(kWave) void flash_attn_fwd_sparse_kernel(const AttnParams p) {
+__global__ __launch_bounds__(kSparseWaves * kWave) void flash_attn_fwd_sparse_kernel(const AttnParams p) {
   typedef typename Vec8<T>::type vec_t;
   typedef typename Vec8<T>::half_type vec4_t;
   static_assert(DP == 32 || DP == 64, "row swizzles are written for 64- and 128-byte rows");
@@ -966,15 +969,22 @@ __global__ __launch_bounds__(kWave) void flash_attn_fwd_sparse_kernel(const Attn
   constexpr int PPT = 32 * C8 / kWave;      // 16-byte pieces per lane and tile
   constexpr int OROW = DP * 2 + 16;
   constexpr int OT_BYTES = 32 * OROW;
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[VT_BYTES > OT_BYTES ? VT_BYTES : OT_BYTES];
+  constexpr int WAVE_LDS = ((VT_BYTES > OT_BYTES ? VT_BYTES : OT_BYTES) + 1023) / 1024 * 1024;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem_all[kSparseWaves * WAVE_LDS];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  uint8_t* smem = smem_all + wave * WAVE_LDS;
 
+  // Workgroup g takes query tile g % nqt of the (batch, head)s 4 (g / nqt) .. + 3, one per wavefront: wavefronts of a
+  // workgroup have like amounts of work, the tiles of one (batch, head) sit in neighbouring workgroups (one die's L2).
   const uint32_t nqt = static_cast<uint32_t>((p.Tq + 31) / 32);
   const uint32_t logical = xcd_remap(blockIdx.x, gridDim.x);
-  const int qt = static_cast<int>(logical % nqt);
-  const int bh = static_cast<int>(logical / nqt);
-  const int h = bh % p.H;
-  const int b = bh / p.H;
-  const int lane = threadIdx.x;
+  uint32_t group_u, qt_u, b_u, h_u;
+  magic_divmod(logical, nqt, p.nqt_magic, group_u, qt_u);
+  const uint32_t bh_u = group_u * kSparseWaves + static_cast<uint32_t>(wave);
+  if (bh_u >= static_cast<uint32_t>(p.B) * static_cast<uint32_t>(p.H)) return;
+  magic_divmod(bh_u, static_cast<uint32_t>(p.H), p.h_magic, b_u, h_u);
+  const int qt = static_cast<int>(qt_u), h = static_cast<int>(h_u), b = static_cast<int>(b_u);
+  const int lane = threadIdx.x % kWave;
   const int l32 = lane % 32;
   const int hh = lane / 32;
 
@@ -1024,17 +1034,17 @@ __global__ __launch_bounds__(kWave) void flash_attn_fwd_sparse_kernel(const Attn
   }
   auto valid_word = [&](int w) -> uint32_t { return __builtin_amdgcn_readlane(valid_lane, w); };
 
+  // The query enters the products already multiplied by the softmax scale, log2 e and its row / feature factors, rounded
+  // once more to the storage type: the score tiles come out of the matrix unit in the exponent's units.
   float c = p.scale_log2;
   if (SCALED && p.q_row_scale != nullptr && qi < q_valid) c *= p.q_row_scale[static_cast<int64_t>(b) * p.Tq + qi];
   vec_t qf[KSTEPS];
 #pragma unroll
   for (int s = 0; s < KSTEPS; ++s) {
     qf[s] = qi < q_valid ? *reinterpret_cast<const vec_t*>(qb + qi * p.qs[2] + 16 * s + 8 * hh) : zero_vec;
-    if (SCALED && p.q_col_scale != nullptr) {
-      const float* cf = p.q_col_scale + h * p.d + 16 * s + 8 * hh;
+    const float* cf = (SCALED && p.q_col_scale != nullptr) ? p.q_col_scale + h * p.d + 16 * s + 8 * hh : nullptr;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<T>(static_cast<float>(qf[s][e]) * cf[e]);
-    }
+    for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<T>(static_cast<float>(qf[s][e]) * (cf != nullptr ? cf[e] * c : c));
   }
   // ---- the tiles this wavefront visits: bit kt of `tiles` (none when every row is in the padding or self-only) -------
   uint64_t tiles = __builtin_amdgcn_ballot_w64((tile_lane & valid_lane) != 0u);
@@ -1045,8 +1055,15 @@ __global__ __launch_bounds__(kWave) void flash_attn_fwd_sparse_kernel(const Attn
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
     for (int j = 0; j < 16; ++j) oacc[mb][j] = 0.f;
-  float m_run = -INFINITY;
-  float l_run = 0.f;
+  // Softmax with a lazily moved reference, as in the chunked direct-transfer kernel: -m is the C operand of the first
+  // score product, m moves (and the accumulators are rescaled) only when a score exceeds it by more than kLazyBits.
+  constexpr float kLazyBits = 8.f;
+  f32x16 negm;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) negm[j] = 0.f;
+  float l_lane = 0.f;
+  bool m_set = false;
+  float thr = -3.0e38f;
 
   auto v_swizzle = [](int r) -> int { return DP == 32 ? 0 : 4 * ((r / 2) % 2); };
   const uint32_t k_row_bytes = static_cast<uint32_t>(p.ks[2]) * 2u, v_row_bytes = static_cast<uint32_t>(p.vs[2]) * 2u;
@@ -1102,9 +1119,7 @@ __global__ __launch_bounds__(kWave) void flash_attn_fwd_sparse_kernel(const Attn
     }
     f32x16 sacc;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) sacc[j] = 0.f;
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) sacc = Mfma32<T>::run(t.kf[s], qf[s], sacc);
+    for (int s = 0; s < KSTEPS; ++s) sacc = Mfma32<T>::run(t.kf[s], qf[s], s == 0 ? negm : sacc);
     if (__builtin_amdgcn_ballot_w64(word != 0xffffffffu) != 0ull) {  // wavefront-uniform
       const uint32_t bits = word >> (hh * 4);
 #pragma unroll
@@ -1114,29 +1129,38 @@ __global__ __launch_bounds__(kWave) void flash_attn_fwd_sparse_kernel(const Attn
     float mx = sacc[0];
 #pragma unroll
     for (int j = 1; j < 16; ++j) mx = fmaxf(mx, sacc[j]);
-    mx = pair_max(mx);
-    const float m_new = fmaxf(m_run, mx);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
-    const float mc = -m_use * c;
+    if (__builtin_amdgcn_ballot_w64(mx > thr) != 0ull) {  // wavefront-uniform, rare after a query's first visible tile
+      const float mxp = pair_max(mx);  // both lanes of a query keep one reference between them
+      const bool move = mxp > thr;
+      const float shift = move ? mxp : 0.f;
+      const float alpha = (move && m_set) ? __builtin_amdgcn_exp2f(-mxp) : 1.f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) sacc[j] -= shift;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) negm[j] -= shift;
+      l_lane *= alpha;
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;
+      if (move) {
+        m_set = true;
+        thr = kLazyBits;
+      }
+    }
     float pr[16];
 #pragma unroll
-    for (int j = 0; j < 16; ++j) pr[j] = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, mc));
+    for (int j = 0; j < 16; ++j) pr[j] = __builtin_amdgcn_exp2f(sacc[j]);
     vec_t pb[2];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       pb[0][e] = static_cast<T>(pr[e]);
       pb[1][e] = static_cast<T>(pr[8 + e]);
     }
-    float rs = frag_sum(pb[0], 0.f);
-    rs = frag_sum(pb[1], rs);
-    rs = pair_sum(rs);
-    l_run = l_run * alpha + rs;
-    m_run = m_new;
+    l_lane = frag_sum(pb[0], l_lane);
+    l_lane = frag_sum(pb[1], l_lane);
     static_for<MB>([&](auto mb_tag) {
       constexpr int mb = decltype(mb_tag)::value;
-#pragma unroll
-      for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;
       const uint32_t v_addr_mb = v_addr ^ (mb * 64);
       u32x2 vt[2][2];
       lds_read_tr16<0>(vt[0][0], v_addr_mb);
@@ -1170,6 +1194,7 @@ __global__ __launch_bounds__(kWave) void flash_attn_fwd_sparse_kernel(const Attn
   }
 
   // ---- finalise: O / l, transpose through the wavefront's LDS tile, self rows, 16-byte stores -------------------------
+  const float l_run = pair_sum(l_lane);
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
   const float fin = (qi < q_valid) ? inv : 0.f;
   uint8_t* tile = smem;
@@ -1206,11 +1231,13 @@ void launch(const AttnParams& p, bool causal, bool register_staging, hipStream_t
                              static_cast<int64_t>(p.Tk) * p.vs[2] * 2 < (1ll << 31);
   if constexpr (DP == 32 || DP == 64) {
     if (p.tile_words != nullptr) {  // the entry point has checked the shape
-      const int64_t waves = static_cast<int64_t>((p.Tq + 31) / 32) * p.B * p.H;
+      const int64_t groups = static_cast<int64_t>((p.Tq + 31) / 32) * ((static_cast<int64_t>(p.B) * p.H + kSparseWaves - 1) / kSparseWaves);
       if (scaled)
-        hipLaunchKernelGGL((flash_attn_fwd_sparse_kernel<T, DP, true>), dim3(static_cast<uint32_t>(waves)), dim3(kWave), 0, s, p);
+        hipLaunchKernelGGL((flash_attn_fwd_sparse_kernel<T, DP, true>), dim3(static_cast<uint32_t>(groups)),
+                           dim3(kSparseWaves * kWave), 0, s, p);
       else
-        hipLaunchKernelGGL((flash_attn_fwd_sparse_kernel<T, DP, false>), dim3(static_cast<uint32_t>(waves)), dim3(kWave), 0, s, p);
+        hipLaunchKernelGGL((flash_attn_fwd_sparse_kernel<T, DP, false>), dim3(static_cast<uint32_t>(groups)),
+                           dim3(kSparseWaves * kWave), 0, s, p);
       return;
     }
     // structure bits ride along when they are all there is to the mask: per sample, no validity or self rows, no chunk map
@@ -1388,6 +1415,7 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   p.total = static_cast<uint32_t>(total);
   p.nqc_magic = magic_of(p.nqc);
   p.h_magic = magic_of(static_cast<uint32_t>(H));
+  p.nqt_magic = magic_of(static_cast<uint32_t>((Tq + 31) / 32));
 
   hipStream_t s = as_stream(stream);
   if (dtype == TAAC_BF16)
