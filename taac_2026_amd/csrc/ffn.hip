@@ -432,13 +432,19 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 
   stage(0, 0);
   if constexpr (OUTP) stage_proj(0, 1);
+  // The token rows (a row-index load, then the rows) are requested before the bias vectors are staged, so that the two
+  // chains of memory latencies run side by side; OUTP: so is the row number of the block input read by the projection.
+  bf16x8 xf[TT][KS];
+  if (active) load_token_rows<D, TT>(p, count, tok0, l32, hh, xf);
+  [[maybe_unused]] int64_t hrow_index[TT];
+  if constexpr (OUTP) {
+#pragma unroll
+    for (int t = 0; t < TT; ++t) hrow_index[t] = token_row(p, count, tok0 + t * 32 + l32);
+  }
   stage_up_bias(p.b1, bias_lds, F, p.gate_first, tid, NWAVES * kWave);
   stage_bias(p.b2, bias_lds + 2 * F, D, tid, NWAVES * kWave);
   if (p.norm_w != nullptr) stage_bias(p.norm_w, bias_lds + 2 * F + D, D, tid, NWAVES * kWave);
   if constexpr (OUTP) stage_bias(p.b0, bias_lds + 2 * F + 2 * D, D, tid, NWAVES * kWave);
-
-  bf16x8 xf[TT][KS];
-  if (active) load_token_rows<D, TT>(p, count, tok0, l32, hh, xf);
 
   f32x16 oacc[TT][MB];
 #pragma unroll
@@ -475,7 +481,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
       ss[t] = 0.f;
-      hrow[t] = p.residual + token_row(p, count, tok0 + t * 32 + l32) * p.ldr + hh * 4;
+      hrow[t] = p.residual + hrow_index[t] * p.ldr + hh * 4;
     }
     static_for<NCH>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
