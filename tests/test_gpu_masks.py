@@ -211,3 +211,28 @@ def test_per_tile_kernel_ignores_the_rows_of_invalid_keys_and_padded_queries(dev
     torch.testing.assert_close(clean.float()[valid], _expected(q, k, v, dense)[valid], **BF16_TOL)
     assert torch.equal(clean[~valid], v[~valid])                 # self-only rows: the value row, bit for bit
     torch.testing.assert_close(clean.float(), chunked.float(), rtol=2 ** -6, atol=2 ** -6)
+
+
+def test_per_tile_kernel_at_the_headline_attention_shape(device):
+    """B=1024, H=8, T=512, head dim 32 under TokenFormer's narrowest window layer (2.3 % of the pairs visible): the
+    per-tile kernel against the chunked kernel on every sample, and a slice of samples against SDPA with the dense mask."""
+    batch, heads, tokens, dim, layers = 1024, 8, 512, 32, 6
+    g = torch.Generator().manual_seed(42)
+    qkv = torch.randn(batch, tokens, 3 * heads * dim, generator=g).to(torch.bfloat16).to(device)
+    q, k, v = (t.view(batch, tokens, heads, dim).transpose(1, 2) for t in qkv.chunk(3, dim=-1))
+    roles = torch.tensor([0] * 20 + [4] + [1] * 460 + [4] + [2] * 20 + [5] * 9 + [3], device=device)
+    span = torch.randint(32, 461, (batch,), generator=g).to(device)
+    positions = torch.arange(tokens, device=device)
+    padding = (positions[None, :] >= 21 + span[:, None]) & (positions[None, :] < 481)
+    with torch.no_grad():
+        mask = bfts_attention_mask(padding, roles, 5, layers, seq_causal=True, seq_keep_per_domain=64)
+        assert mask.sparse
+        got = flash_attention(q, k, v, structured_mask=mask)
+        chunked = flash_attention(q, k, v, structured_mask=replace(mask, sparse=False))
+    torch.testing.assert_close(got.float(), chunked.float(), rtol=2 ** -6, atol=2 ** -6)
+    pick = torch.tensor([0, 333, 1023])
+    dense = mask.dense()[pick.to(device)].cpu()
+    want = _expected(q[pick.to(device)].cpu(), k[pick.to(device)].cpu(), v[pick.to(device)].cpu(), dense)
+    self_rows = padding[pick.to(device)].cpu()[:, None, :, None].expand_as(want)
+    torch.testing.assert_close(got[pick.to(device)].cpu().float()[~self_rows], want[~self_rows], **BF16_TOL)
+    assert torch.equal(got[pick.to(device)].cpu()[self_rows], v[pick.to(device)].cpu()[self_rows])
