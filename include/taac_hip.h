@@ -199,33 +199,40 @@ int taac_flash_attn_masked_fwd(const void* q, const void* k, const void* v, cons
 
 /*
  * taac_flash_attn_masked_fwd (same mask, same result up to the summation order of the softmax) for masks in which a
- * 32-query tile sees only a few 32-key tiles: sliding windows with a few always-visible key columns and query rows, the
- * upper layers of TokenFormer's mask (experiments/tokenformer/model.py:474-503). One wavefront per 32-query tile works
- * on its own: tile_words (taac_mask_tile_words: the tile's rows of struct_bits ORed together) ANDed with valid_bits and
- * key_lengths names the key tiles in which one of its queries can see a key, and exactly those are visited - K fragments
- * straight from global memory, V through a wavefront-private LDS tile. A tile whose query rows are all self-only or in
- * the padding visits nothing. The time follows the number of visible tiles instead of the number of key chunks a
- * 128-query block touches; for dense masks the chunked kernel is faster, so the caller chooses.
- * tile_words: uint32 [samples, ceil(Tq / 32), ceil(Tk / 32)], samples = 1 (struct_sample_stride = 0) or B.
+ * 32-query tile sees only a few key columns: sliding windows with a few always-visible key columns and query rows, the
+ * upper layers of TokenFormer's mask (experiments/tokenformer/model.py:474-503). The structure arrives in compact form
+ * (taac_mask_compact): per 32-query tile the ascending list of key columns some query of the tile can see, cut into
+ * compact tiles of 32 keys, and per query row one word per compact tile. One wavefront per 32-query tile works on its
+ * own: it visits the compact tiles that can hold a valid key of the sample (valid_bits, key_lengths), gathers their K
+ * rows straight from global memory into MFMA fragments and their V rows through a wavefront-private LDS tile, and
+ * applies the row's word. A tile whose query rows are all self-only or in the padding visits nothing. The time follows
+ * the number of visible key columns per query tile (in units of 32) instead of the number of 64-key chunks a 128-query
+ * block touches; for dense masks the chunked kernel is faster, so the caller chooses.
+ * compact_bits: uint32 [samples, Tq, ceil(Tk / 32)]; compact_keys: int32 [samples, ceil(Tq / 32), 32 ceil(Tk / 32)];
+ * compact_tiles: uint64 [samples, ceil(Tq / 32), 64]; samples = 1 (compact_sample_stride = 0) for a structure shared by
+ * the batch, else B with compact_sample_stride = Tq * ceil(Tk / 32).
  * Head dims 32 and 64, Tk <= 2048, key / value row strides that fit 32-bit byte offsets; anything else is
  * TAAC_ERR_UNSUPPORTED (use taac_flash_attn_masked_fwd). Other arguments as taac_flash_attn_masked_fwd.
  */
 int taac_flash_attn_sparse_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
-                               const uint32_t* struct_bits, int64_t struct_sample_stride, const uint32_t* tile_words,
-                               const uint32_t* valid_bits,
-                               const uint32_t* self_bits, const float* q_row_scale, const float* k_row_scale,
-                               const float* q_col_scale, void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk,
-                               int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
-                               const int64_t v_strides[4], const int64_t o_strides[4], int zero_padded_queries,
-                               int dtype, void* stream);
+                               const uint32_t* compact_bits, int64_t compact_sample_stride, const int32_t* compact_keys,
+                               const uint64_t* compact_tiles, const uint32_t* valid_bits, const uint32_t* self_bits,
+                               const float* q_row_scale, const float* k_row_scale, const float* q_col_scale, void* o,
+                               int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
+                               const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4],
+                               int zero_padded_queries, int dtype, void* stream);
 
 /*
- * tile_words[s, t, w] = OR over the query rows 32 t .. 32 t + 31 (below Tq) of sample s of struct_bits[row, w]: which keys
- * some query of the tile can see. samples = 1 for a structure shared by the batch, else B with struct_sample_stride words
- * between the samples' matrices. No counterpart in the reference (its fallback passes a dense bool mask to torch SDPA).
+ * Compact form of a structure matrix for taac_flash_attn_sparse_fwd. For sample s and query tile t (rows 32 t .. 32 t + 31
+ * below Tq): compact_keys[s, t, :] = the key columns j with struct_bits[row, j] set for some row of the tile, ascending,
+ * then -1; compact_tiles[s, t, c] = bit w set iff compact tile c (keys 32 c .. 32 c + 31 of that list) holds a key of
+ * word w (keys 32 w .. 32 w + 31 of Tk), 0 for tiles beyond the list; compact_bits[s, row, c] = bit j set iff the row
+ * sees key compact_keys[s, row / 32, 32 c + j]. samples = 1 for a structure shared by the batch, else B with
+ * struct_sample_stride words between the samples' matrices. Tk <= 2048.
+ * No counterpart in the reference (its fallback passes a dense bool mask to torch SDPA).
  */
-int taac_mask_tile_words(const uint32_t* struct_bits, int32_t samples, int32_t Tq, int32_t Tk,
-                         int64_t struct_sample_stride, uint32_t* tile_words, void* stream);
+int taac_mask_compact(const uint32_t* struct_bits, int32_t samples, int32_t Tq, int32_t Tk, int64_t struct_sample_stride,
+                      uint32_t* compact_bits, int32_t* compact_keys, uint64_t* compact_tiles, void* stream);
 
 /* Packs a row-major bool matrix (one byte per element, nonzero = true) [rows, cols] into bit rows
  * [rows, ceil(cols / 32)]: the struct_bits / valid_bits / self_bits of taac_flash_attn_masked_fwd. */

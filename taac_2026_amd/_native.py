@@ -106,11 +106,11 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "taac_flash_attn_sparse_fwd": (
         c_int,
-        [c_void_p] * 5 + [c_int64] + [c_void_p] * 7 + [c_int32, c_int32, c_int32, c_int32, c_int32]
+        [c_void_p] * 5 + [c_int64] + [c_void_p] * 8 + [c_int32, c_int32, c_int32, c_int32, c_int32]
         + [ctypes.POINTER(c_int64)] * 4
         + [c_int, c_int, c_void_p],
     ),
-    "taac_mask_tile_words": (c_int, [c_void_p, c_int32, c_int32, c_int32, c_int64, c_void_p, c_void_p]),
+    "taac_mask_compact": (c_int, [c_void_p, c_int32, c_int32, c_int32, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "taac_mask_pack_bits": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p]),
     "taac_mask_block_any": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
     "taac_flash_attn_train_fwd": (

@@ -185,20 +185,27 @@ def _few_visible_tiles(structural: torch.Tensor) -> bool:
     return bool(tiles.float().mean().item() <= 1.0 / 3.0)
 
 
-def _tile_words(mask: StructuredAttentionMask, batch: int) -> torch.Tensor:
-    """The mask's structure ORed over the 32 query rows of each tile (made once per mask object)."""
-    words = mask.cache.get("tile_words")
-    if words is None:
+def _compact_tables(mask: StructuredAttentionMask, batch: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """The mask's structure in the per-tile kernel's compact form (made once per mask object): per 32-query tile the
+    visible key columns, per compact tile of 32 such keys the key words it draws from, per query row its words."""
+    tables = mask.cache.get("compact_tables")
+    if tables is None:
         query_len, kv_len = mask.structural.shape
         samples = batch if mask.sample_stride else 1
-        words = torch.empty(samples, (query_len + 31) // 32, (kv_len + 31) // 32, dtype=torch.int32,
-                            device=mask.struct_bits.device)
+        words = (kv_len + 31) // 32
+        tiles = (query_len + 31) // 32
+        device = mask.struct_bits.device
+        bits = torch.empty(samples, query_len, words, dtype=torch.int32, device=device)
+        keys = torch.empty(samples, tiles, 32 * words, dtype=torch.int32, device=device)
+        tile_words = torch.empty(samples, tiles, 64, dtype=torch.int64, device=device)
         library = _native.load_library()
-        status = library.taac_mask_tile_words(mask.struct_bits.data_ptr(), samples, query_len, kv_len, int(mask.sample_stride),
-                                              words.data_ptr(), _native.current_stream(words.device))
-        _native.check(status, "mask_tile_words")
-        mask.cache["tile_words"] = words
-    return words
+        status = library.taac_mask_compact(mask.struct_bits.data_ptr(), samples, query_len, kv_len, int(mask.sample_stride),
+                                           bits.data_ptr(), keys.data_ptr(), tile_words.data_ptr(),
+                                           _native.current_stream(device))
+        _native.check(status, "mask_compact")
+        tables = (bits, keys, tile_words)
+        mask.cache["compact_tables"] = tables
+    return tables
 
 
 def _normalize_flash_attention_inputs(
@@ -411,18 +418,23 @@ def hip_flash_attention_kernel(
             raise ValueError("flash_attention: the structured mask does not match (batch, query_len, kv_len)")
         require_cuda_tensors("hip flash_attention", sm.struct_bits)
         per_tile = sm.sparse and head_dim in (32, 64) and k.shape[2] <= 2048 and k.stride(2) < (1 << 20) and v.stride(2) < (1 << 20)
-        entry = library.taac_flash_attn_sparse_fwd if per_tile else library.taac_flash_attn_masked_fwd
-        status = entry(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), sm.struct_bits.data_ptr(),
-            int(sm.sample_stride), _tile_words(sm, batch).data_ptr() if per_tile else _native.ptr(sm.block_any),
-            _native.ptr(sm.valid_bits), _native.ptr(sm.self_bits),
-            _native.ptr(q_row_scale),
+        tail = (
+            _native.ptr(sm.valid_bits), _native.ptr(sm.self_bits), _native.ptr(q_row_scale),
             _native.ptr(k_row_scale), _native.ptr(q_col_scale), out.data_ptr(),
             batch, heads, query_len, k.shape[2], head_dim,
             _native.Int64x4(*q.stride()), _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()),
             _native.Int64x4(*out.stride()), int(zero_padded_queries), _native.dtype_code(q.dtype),
             _native.current_stream(q.device),
         )
+        if per_tile:
+            bits, keys, tile_words = _compact_tables(sm, batch)
+            status = library.taac_flash_attn_sparse_fwd(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), bits.data_ptr(),
+                query_len * bits.shape[2] if sm.sample_stride else 0, keys.data_ptr(), tile_words.data_ptr(), *tail)
+        else:
+            status = library.taac_flash_attn_masked_fwd(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), sm.struct_bits.data_ptr(),
+                int(sm.sample_stride), _native.ptr(sm.block_any), *tail)
         _native.check(status, "flash_attention")
         return out
     if amax_out is not None:

@@ -53,7 +53,11 @@ struct AttnParams {
   const uint32_t* self_bits;    // [B][ceil(Tq / 32)] or null: flagged query rows return their own value row
   const uint8_t* block_any;     // [nqc][nkc]: some query of the 128-row block sees some key of the 64-key chunk;
                                 // null (per-sample structure only): every chunk is visited
-  const uint32_t* tile_words;   // per-tile kernel: [samples][ceil(Tq / 32)][wpr], struct_bits ORed over a tile's 32 rows
+  // Per-tile kernel (compact form of the structure, taac_mask_compact): for every 32-query tile the key columns some
+  // query of the tile can see, in ascending order, cut into compact tiles of 32; struct_bits then holds, per query row,
+  // one word per compact tile (bit j = the row sees key compact_keys[32 c + j]).
+  const int32_t* compact_keys;   // [samples][nqt][32 wpr], -1 beyond the tile's keys
+  const uint64_t* compact_tiles; // [samples][nqt][64]: the 32-key words of Tk that hold keys of compact tile c (0: no such tile)
   float* lse;                   // [B, H, Tq] log-sum-exp of the scaled scores (natural log) for the backward, or null
   int32_t wpr;                  // words per row of struct_bits / valid_bits = ceil(Tk / 32)
   int32_t nkc;                  // key chunks = ceil(Tk / 64)
@@ -1021,18 +1025,27 @@ __global__ __launch_bounds__(kSparseWaves * kWave) void flash_attn_fwd_sparse_ke
   if (p.self_bits != nullptr) self_word = p.self_bits[static_cast<int64_t>(b) * ((p.Tq + 31) / 32) + qt];
   const bool row_active = qi < q_valid && ((self_word >> l32) & 1u) == 0u;
   const uint32_t* bits_row = p.struct_bits + b * p.struct_stride + static_cast<int64_t>(qi < p.Tq ? qi : 0) * p.wpr;
-  // Lane w holds word w of the sample's key validity, cut at the valid length (at most 64 words: Tk <= 2048), and word w
-  // of the structure bits ORed over the tile's 32 query rows: one ballot then names the key tiles to visit.
-  uint32_t valid_lane = 0u, tile_lane = 0u;
-  if (lane < p.wpr) {
-    valid_lane = p.valid_bits != nullptr ? p.valid_bits[static_cast<int64_t>(b) * p.wpr + lane] : ~0u;
-    tile_lane = p.tile_words[(p.struct_stride != 0 ? static_cast<int64_t>(b) * nqt * p.wpr : 0) + static_cast<int64_t>(qt) * p.wpr + lane];
-  }
+  // Lane w holds word w of the sample's key validity, cut at the valid length (at most 64 words: Tk <= 2048); lane c the
+  // set of key words that compact tile c of this query tile draws its keys from: one ballot names the compact tiles
+  // that can hold a valid key (a tile none of whose words has a valid key is never visited).
+  const int64_t compact_base = (p.struct_stride != 0 ? static_cast<int64_t>(b) * nqt : 0) + qt;
+  const int32_t* keys_tile = p.compact_keys + compact_base * (32 * p.wpr);
+  uint32_t valid_lane = 0u;
+  if (lane < p.wpr) valid_lane = p.valid_bits != nullptr ? p.valid_bits[static_cast<int64_t>(b) * p.wpr + lane] : ~0u;
+  const uint64_t words_of_tile = p.compact_tiles[compact_base * 64 + lane];
+  // The keys of the first two compact tiles are requested now, with everything else the prologue loads: they are
+  // almost always the first tiles visited, and their K / V rows can then be requested as soon as the tile set is known.
+  const int key_first = keys_tile[l32];
+  const int key_second = p.wpr > 1 ? keys_tile[32 + l32] : -1;
   {
     const int rest = len - lane * 32;
     if (rest < 32) valid_lane &= rest <= 0 ? 0u : ((1u << rest) - 1u);
   }
-  auto valid_word = [&](int w) -> uint32_t { return __builtin_amdgcn_readlane(valid_lane, w); };
+  // validity of key `key` (per lane): the bit of the word held by lane key / 32
+  auto key_is_valid = [&](int key) -> bool {
+    const uint32_t word = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute((key >> 5) << 2, static_cast<int>(valid_lane)));
+    return key >= 0 && ((word >> (key & 31)) & 1u) != 0u;
+  };
 
   // The query enters the products already multiplied by the softmax scale, log2 e and its row / feature factors, rounded
   // once more to the storage type: the score tiles come out of the matrix unit in the exponent's units.
@@ -1047,7 +1060,8 @@ __global__ __launch_bounds__(kSparseWaves * kWave) void flash_attn_fwd_sparse_ke
     for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<T>(static_cast<float>(qf[s][e]) * (cf != nullptr ? cf[e] * c : c));
   }
   // ---- the tiles this wavefront visits: bit kt of `tiles` (none when every row is in the padding or self-only) -------
-  uint64_t tiles = __builtin_amdgcn_ballot_w64((tile_lane & valid_lane) != 0u);
+  const uint64_t words_with_valid_keys = __builtin_amdgcn_ballot_w64(valid_lane != 0u);
+  uint64_t tiles = __builtin_amdgcn_ballot_w64((words_of_tile & words_with_valid_keys) != 0ull);
   if (__builtin_amdgcn_ballot_w64(row_active) == 0ull) tiles = 0ull;
 
   f32x16 oacc[MB];
@@ -1073,23 +1087,24 @@ __global__ __launch_bounds__(kSparseWaves * kWave) void flash_attn_fwd_sparse_ke
   struct TileOperands {
     vec_t v[PPT], kf[KSTEPS];
     uint32_t word;
+    uint32_t valid;  // the lane's key (key l32 of the compact tile) is valid
     float kfac;
   };
-  auto issue = [&](int kt, TileOperands& t) {
+  // `key` = the lane's key of compact tile kt (compact_keys[32 kt + l32], fetched a tile earlier still), -1: none.
+  auto issue = [&](int kt, int key, TileOperands& t) {
+    const int krow = key < 0 ? 0 : key;
 #pragma unroll
     for (int i = 0; i < PPT; ++i) {
       const int slot = i * kWave + lane;
-      int row = kt * 32 + slot / C8;
-      row = row < p.Tk ? row : p.Tk - 1;
+      const int row = __builtin_amdgcn_ds_bpermute((slot / C8) << 2, krow);  // the key of row slot / C8 of the tile
       t.v[i] = *reinterpret_cast<const vec_t*>(reinterpret_cast<const uint8_t*>(vb) +
                                                __umul24(static_cast<uint32_t>(row), v_row_bytes) + (slot % C8) * 16);
     }
-    int krow = kt * 32 + l32;
-    krow = krow < p.Tk ? krow : p.Tk - 1;
     const uint8_t* ksrc = reinterpret_cast<const uint8_t*>(kb) + __umul24(static_cast<uint32_t>(krow), k_row_bytes) + hh * 16;
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) t.kf[s] = *reinterpret_cast<const vec_t*>(ksrc + s * 32);
     t.word = row_active ? bits_row[kt] : 0u;
+    t.valid = key_is_valid(key) ? 1u : 0u;
     t.kfac = 1.f;
     if (SCALED && scale_keys) t.kfac = p.k_row_scale[static_cast<int64_t>(b) * p.Tk + krow];
   };
@@ -1100,7 +1115,7 @@ __global__ __launch_bounds__(kSparseWaves * kWave) void flash_attn_fwd_sparse_ke
       v_key * ROWB + ((2 * ((lane / 16) % 2) + (lane % 4) / 2) ^ v_swizzle(v_key)) * 16 + (lane % 2) * 8);
 
   auto consume = [&](int kt, TileOperands& t) {
-    const uint32_t vword = valid_word(kt);
+    const uint32_t vword = static_cast<uint32_t>(__builtin_amdgcn_ballot_w64(t.valid != 0u));  // lanes 0 .. 31: key l32
     const uint32_t word = t.word & vword;
     // The V tile goes into the wavefront's LDS tile (the transposed reads of the tile before it have been waited for);
     // rows of invalid keys are stored as zeros.
@@ -1182,15 +1197,27 @@ __global__ __launch_bounds__(kSparseWaves * kWave) void flash_attn_fwd_sparse_ke
     tiles &= tiles - 1ull;
     return kt;
   };
+  // Pipeline: the keys of a compact tile are fetched two tiles ahead, its K / V rows and mask word one tile ahead.
+  auto load_key = [&](int kt) -> int {
+    if (kt < 0) return -1;
+    if (kt == 0) return key_first;
+    if (kt == 1) return key_second;
+    return keys_tile[kt * 32 + l32];
+  };
   TileOperands next;
   int kt = pop_tile();
-  if (kt >= 0) issue(kt, next);
+  int kt_next = pop_tile();
+  int key_next = load_key(kt_next);
+  if (kt >= 0) issue(kt, load_key(kt), next);
   while (kt >= 0) {
     TileOperands cur = next;
-    const int kt_next = pop_tile();
-    if (kt_next >= 0) issue(kt_next, next);
+    const int kt_after = pop_tile();
+    const int key_after = load_key(kt_after);
+    if (kt_next >= 0) issue(kt_next, key_next, next);
     consume(kt, cur);
     kt = kt_next;
+    kt_next = kt_after;
+    key_next = key_after;
   }
 
   // ---- finalise: O / l, transpose through the wavefront's LDS tile, self rows, 16-byte stores -------------------------
@@ -1230,7 +1257,7 @@ void launch(const AttnParams& p, bool causal, bool register_staging, hipStream_t
                              static_cast<int64_t>(p.Tk) * p.ks[2] * 2 < (1ll << 31) &&
                              static_cast<int64_t>(p.Tk) * p.vs[2] * 2 < (1ll << 31);
   if constexpr (DP == 32 || DP == 64) {
-    if (p.tile_words != nullptr) {  // the entry point has checked the shape
+    if (p.compact_keys != nullptr) {  // the entry point has checked the shape
       const int64_t groups = static_cast<int64_t>((p.Tq + 31) / 32) * ((static_cast<int64_t>(p.B) * p.H + kSparseWaves - 1) / kSparseWaves);
       if (scaled)
         hipLaunchKernelGGL((flash_attn_fwd_sparse_kernel<T, DP, true>), dim3(static_cast<uint32_t>(groups)),
@@ -1326,7 +1353,8 @@ struct MaskArgs {
   const uint8_t* block_any = nullptr;
   const uint32_t* valid_bits = nullptr;
   const uint32_t* self_bits = nullptr;
-  const uint32_t* tile_words = nullptr;  // given: the one-wavefront-per-query-tile kernel
+  const int32_t* compact_keys = nullptr;    // given (with compact_tiles): the one-wavefront-per-query-tile kernel
+  const uint64_t* compact_tiles = nullptr;
 };
 
 int attention_entry(const char* name, const void* q, const void* k, const void* v, const int32_t* key_lengths,
@@ -1345,7 +1373,7 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   const int is_causal = mask_flags & TAAC_ATTN_CAUSAL;
   const bool register_staging = (mask_flags & TAAC_ATTN_REGISTER_STAGING) != 0;
   if (mask.struct_bits != nullptr) {
-    if (mask.block_any == nullptr && mask.struct_stride == 0 && mask.tile_words == nullptr)
+    if (mask.block_any == nullptr && mask.struct_stride == 0 && mask.compact_keys == nullptr)
       return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_bits shared by the batch needs block_any", name);
     if (mask.struct_stride < 0 || (mask.struct_stride != 0 && mask.struct_stride < static_cast<int64_t>(Tq) * ((Tk + 31) / 32)))
       return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_sample_stride must be 0 or cover a sample's matrix", name);
@@ -1393,7 +1421,8 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   p.valid_bits = mask.valid_bits;
   p.self_bits = mask.self_bits;
   p.block_any = mask.block_any;
-  p.tile_words = mask.tile_words;
+  p.compact_keys = mask.compact_keys;
+  p.compact_tiles = mask.compact_tiles;
   p.wpr = (Tk + 31) / 32;
   p.nkc = (Tk + kKC - 1) / kKC;
   p.B = B;
@@ -1498,16 +1527,18 @@ extern "C" int taac_flash_attn_masked_fwd(const void* q, const void* k, const vo
 }
 
 extern "C" int taac_flash_attn_sparse_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
-                                          const uint32_t* struct_bits, int64_t struct_sample_stride,
-                                          const uint32_t* tile_words, const uint32_t* valid_bits,
-                                          const uint32_t* self_bits, const float* q_row_scale, const float* k_row_scale,
-                                          const float* q_col_scale, void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk,
-                                          int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
+                                          const uint32_t* compact_bits, int64_t compact_sample_stride,
+                                          const int32_t* compact_keys, const uint64_t* compact_tiles,
+                                          const uint32_t* valid_bits, const uint32_t* self_bits,
+                                          const float* q_row_scale, const float* k_row_scale, const float* q_col_scale,
+                                          void* o, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                                          const int64_t q_strides[4], const int64_t k_strides[4],
                                           const int64_t v_strides[4], const int64_t o_strides[4],
                                           int zero_padded_queries, int dtype, void* stream) {
   using namespace taac;
   const char* name = "taac_flash_attn_sparse_fwd";
-  if (!struct_bits || !tile_words) return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_bits and tile_words must be given", name);
+  if (!compact_bits || !compact_keys || !compact_tiles)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: compact_bits, compact_keys and compact_tiles must be given", name);
   if (d != 32 && d != 64) return set_error(TAAC_ERR_UNSUPPORTED, "%s: head_dim must be 32 or 64 (got %d)", name, d);
   if (Tk < 1 || Tk > 2048) return set_error(TAAC_ERR_UNSUPPORTED, "%s: 1 <= Tk <= 2048 required (got %d)", name, Tk);
   if (!k_strides || !v_strides) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null stride array", name);
@@ -1517,47 +1548,98 @@ extern "C" int taac_flash_attn_sparse_fwd(const void* q, const void* k, const vo
   if (static_cast<int64_t>((Tq + 31) / 32) * B * H > 0x7fffffffLL)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many query tiles", name);
   MaskArgs mask;
-  mask.struct_bits = struct_bits;
-  mask.struct_stride = struct_sample_stride;
+  mask.struct_bits = compact_bits;
+  mask.struct_stride = compact_sample_stride;
   mask.valid_bits = valid_bits;
   mask.self_bits = self_bits;
-  mask.tile_words = tile_words;
+  mask.compact_keys = compact_keys;
+  mask.compact_tiles = compact_tiles;
   return attention_entry(name, q, k, v, key_lengths, mask, q_row_scale, k_row_scale, q_col_scale, nullptr, nullptr, o, B, H,
                          Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, 0, zero_padded_queries, dtype, stream);
 }
 
 namespace taac {
 namespace {
-// tile_words[s][t][w] = OR over the rows 32 t .. 32 t + 31 (below Tq) of sample s of struct_bits[row][w]; one lane per word.
-__global__ __launch_bounds__(256) void tile_words_kernel(const uint32_t* __restrict__ bits, int samples, int Tq, int wpr,
-                                                         int64_t stride, uint32_t* __restrict__ tile_words) {
+// One wavefront per (sample, 32-query tile): the key columns some row of the tile can see, in ascending order
+// (compact_keys, -1 behind them), per compact tile of 32 such keys the set of 32-key words of Tk it draws from
+// (compact_tiles), and per query row one word per compact tile (compact_bits: bit j = the row sees key 32 c + j of the list).
+__global__ __launch_bounds__(kWave) void mask_compact_kernel(const uint32_t* __restrict__ bits, int Tq, int wpr, int64_t stride,
+                                                            uint32_t* __restrict__ compact_bits,
+                                                            int32_t* __restrict__ compact_keys,
+                                                            uint64_t* __restrict__ compact_tiles) {
+  __shared__ int32_t keys[2048];
   const int nqt = (Tq + 31) / 32;
-  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (idx >= static_cast<int64_t>(samples) * nqt * wpr) return;
-  const int w = static_cast<int>(idx % wpr);
-  const int t = static_cast<int>((idx / wpr) % nqt);
-  const int64_t smp = idx / wpr / nqt;
+  const int t = blockIdx.x % nqt;
+  const int64_t smp = blockIdx.x / nqt;
+  const int lane = threadIdx.x;
   const uint32_t* src = bits + smp * stride;
-  uint32_t acc = 0u;
-  for (int r = t * 32; r < t * 32 + 32 && r < Tq; ++r) acc |= src[static_cast<int64_t>(r) * wpr + w];
-  tile_words[idx] = acc;
+  // union of the tile's rows, word `lane`
+  uint32_t seen = 0u;
+  if (lane < wpr)
+    for (int r = t * 32; r < t * 32 + 32 && r < Tq; ++r) seen |= src[static_cast<int64_t>(r) * wpr + lane];
+  // exclusive prefix sum of the words' population counts over the lanes
+  const int count = __builtin_popcount(seen);
+  int before = count;
+#pragma unroll
+  for (int d = 1; d < kWave; d *= 2) {
+    const int up = __shfl_up(before, d, kWave);
+    if (lane >= d) before += up;
+  }
+  const int total = __shfl(before, kWave - 1, kWave);
+  before -= count;
+  for (int j = lane; j < 32 * wpr; j += kWave) keys[j] = -1;
+  __syncthreads();
+  uint32_t rest = seen;
+  for (int i = 0; rest != 0u; ++i) {
+    const int bit = __builtin_ctz(rest);
+    rest &= rest - 1u;
+    keys[before + i] = lane * 32 + bit;
+  }
+  __syncthreads();
+  const int ntiles = (total + 31) / 32;
+  int32_t* keys_out = compact_keys + (smp * nqt + t) * (32 * static_cast<int64_t>(wpr));
+  for (int j = lane; j < 32 * wpr; j += kWave) keys_out[j] = keys[j];
+  uint64_t words = 0ull;
+  if (lane < ntiles)
+    for (int j = 0; j < 32; ++j) {
+      const int key = keys[lane * 32 + j];
+      if (key >= 0) words |= 1ull << (key >> 5);
+    }
+  compact_tiles[(smp * nqt + t) * 64 + lane] = words;
+  // two rows per pass: lanes 0 .. 31 the even row of the pair, lanes 32 .. 63 the odd one
+  for (int r2 = 0; r2 < 32; r2 += 2) {
+    const int row = t * 32 + r2 + lane / 32;
+    for (int c = 0; c < wpr; ++c) {
+      bool bit = false;
+      if (row < Tq && c < ntiles) {
+        const int key = keys[c * 32 + lane % 32];
+        bit = key >= 0 && ((src[static_cast<int64_t>(row) * wpr + (key >> 5)] >> (key & 31)) & 1u) != 0u;
+      }
+      const uint64_t both = __builtin_amdgcn_ballot_w64(bit);
+      if (row < Tq && lane % 32 == 0)
+        compact_bits[(smp * Tq + row) * static_cast<int64_t>(wpr) + c] = static_cast<uint32_t>(lane == 0 ? both : both >> 32);
+    }
+  }
 }
 }  // namespace
 }  // namespace taac
 
-extern "C" int taac_mask_tile_words(const uint32_t* struct_bits, int32_t samples, int32_t Tq, int32_t Tk,
-                                    int64_t struct_sample_stride, uint32_t* tile_words, void* stream) {
+extern "C" int taac_mask_compact(const uint32_t* struct_bits, int32_t samples, int32_t Tq, int32_t Tk,
+                                 int64_t struct_sample_stride, uint32_t* compact_bits, int32_t* compact_keys,
+                                 uint64_t* compact_tiles, void* stream) {
   using namespace taac;
-  const char* name = "taac_mask_tile_words";
+  const char* name = "taac_mask_compact";
   if (samples <= 0 || Tq <= 0 || Tk <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: samples, Tq and Tk must be positive", name);
-  if (!struct_bits || !tile_words) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  if (Tk > 2048) return set_error(TAAC_ERR_UNSUPPORTED, "%s: Tk <= 2048 required (got %d)", name, Tk);
+  if (!struct_bits || !compact_bits || !compact_keys || !compact_tiles)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
   const int wpr = (Tk + 31) / 32;
   if (samples > 1 && struct_sample_stride < static_cast<int64_t>(Tq) * wpr)
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_sample_stride must cover a sample's matrix", name);
-  const int64_t words = static_cast<int64_t>(samples) * ((Tq + 31) / 32) * wpr;
-  if (words > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: mask too large", name);
-  hipLaunchKernelGGL(tile_words_kernel, dim3(static_cast<uint32_t>((words + 255) / 256)), dim3(256), 0, as_stream(stream),
-                     struct_bits, samples, Tq, wpr, struct_sample_stride, tile_words);
+  const int64_t groups = static_cast<int64_t>(samples) * ((Tq + 31) / 32);
+  if (groups > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: mask too large", name);
+  hipLaunchKernelGGL(mask_compact_kernel, dim3(static_cast<uint32_t>(groups)), dim3(kWave), 0, as_stream(stream), struct_bits,
+                     Tq, wpr, struct_sample_stride, compact_bits, compact_keys, compact_tiles);
   return check_launch(name);
 }
 

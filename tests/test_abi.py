@@ -206,19 +206,21 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
     assert library.taac_mask_block_any(fake, 0, 4, fake, None) == invalid
 
     def per_tile(**kw):
-        a = dict(struct=fake, tiles=fake, tq=64, tk=64, d=32, strides=strides)
+        a = dict(bits=fake, keys=fake, tiles=fake, tq=64, tk=64, d=32, strides=strides)
         a.update(kw)
-        return library.taac_flash_attn_sparse_fwd(fake, fake, fake, None, a["struct"], 0, a["tiles"], None, None, None, None,
-                                                  None, fake, 1, 8, a["tq"], a["tk"], a["d"], strides, a["strides"],
+        return library.taac_flash_attn_sparse_fwd(fake, fake, fake, None, a["bits"], 0, a["keys"], a["tiles"], None, None, None,
+                                                  None, None, fake, 1, 8, a["tq"], a["tk"], a["d"], strides, a["strides"],
                                                   a["strides"], strides, 0, bf16, None)
 
-    assert per_tile(tiles=None) == invalid and b"tile_words" in library.taac_last_error()
+    assert per_tile(keys=None) == invalid and b"compact_keys" in library.taac_last_error()
+    assert per_tile(tiles=None) == invalid and per_tile(bits=None) == invalid
     assert per_tile(d=128) == unsupported and b"head_dim" in library.taac_last_error()
     assert per_tile(tk=4096) == unsupported and b"2048" in library.taac_last_error()
     assert per_tile(strides=_native.Int64x4(1 << 40, 1 << 30, 1 << 23, 1)) == unsupported and b"32-bit" in library.taac_last_error()
-    assert library.taac_mask_tile_words(fake, 1, 0, 64, 0, fake, None) == invalid
-    assert library.taac_mask_tile_words(None, 1, 64, 64, 0, fake, None) == invalid
-    assert library.taac_mask_tile_words(fake, 2, 64, 64, 16, fake, None) == invalid and b"stride" in library.taac_last_error()
+    assert library.taac_mask_compact(fake, 1, 0, 64, 0, fake, fake, fake, None) == invalid
+    assert library.taac_mask_compact(None, 1, 64, 64, 0, fake, fake, fake, None) == invalid
+    assert library.taac_mask_compact(fake, 1, 64, 4096, 0, fake, fake, fake, None) == unsupported
+    assert library.taac_mask_compact(fake, 2, 64, 64, 16, fake, fake, fake, None) == invalid and b"stride" in library.taac_last_error()
     status = library.taac_flash_attn_train_fwd(fake, fake, fake, None, fake, None, 1, 8, 64, 64, 16, strides, strides,
                                                strides, strides, 0, 0, bf16, None)
     assert status == invalid and b"lse" in library.taac_last_error()
