@@ -236,3 +236,33 @@ def test_per_tile_kernel_at_the_headline_attention_shape(device):
     self_rows = padding[pick.to(device)].cpu()[:, None, :, None].expand_as(want)
     torch.testing.assert_close(got[pick.to(device)].cpu().float()[~self_rows], want[~self_rows], **BF16_TOL)
     assert torch.equal(got[pick.to(device)].cpu()[self_rows], v[pick.to(device)].cpu()[self_rows])
+
+
+def test_compact_tables_follow_their_definition(device):
+    """``taac_mask_compact``: per 32-query tile the ascending list of visible key columns, per compact tile of 32 such keys
+    the key words it draws from, per query row one word per compact tile - against loops over a random structure."""
+    from taac_2026_amd.accelerators.attention import _compact_tables
+
+    tokens_q, tokens_k = 70, 200
+    g = torch.Generator().manual_seed(5)
+    structural = torch.rand(tokens_q, tokens_k, generator=g) < 0.08
+    structural[40:] &= torch.arange(tokens_k)[None, :] < 90            # a tile with few columns
+    mask = build_structured_mask(structural.to(device), sparse=True)
+    bits, keys, tile_words = (t.cpu() for t in _compact_tables(mask, 1))
+    words = (tokens_k + 31) // 32
+    assert bits.shape == (1, tokens_q, words) and keys.shape == (1, 3, 32 * words) and tile_words.shape == (1, 3, 64)
+    for tile in range(3):
+        rows = structural[tile * 32:(tile + 1) * 32]
+        columns = rows.any(dim=0).nonzero().flatten().tolist()
+        assert keys[0, tile, :len(columns)].tolist() == columns and (keys[0, tile, len(columns):] == -1).all()
+        for c in range(64):
+            chunk = columns[c * 32:(c + 1) * 32]
+            expected = 0
+            for key in chunk:
+                expected |= 1 << (key // 32)
+            assert int(tile_words[0, tile, c]) == expected
+        for r in range(rows.shape[0]):
+            for c in range(words):
+                chunk = columns[c * 32:(c + 1) * 32]
+                expected = sum(1 << j for j, key in enumerate(chunk) if bool(rows[r, key]))
+                assert int(bits[0, tile * 32 + r, c]) & 0xffffffff == expected
