@@ -325,6 +325,23 @@ int taac_swiglu_bwd(const void* gu, int64_t ldgu, const void* dhidden, int64_t l
                     int64_t ldh, int64_t M, int32_t F, int gate_first, void* stream);
 
 /*
+ * The activation part of the feed-forward backward in one kernel (model width D = 128 / 256, F a multiple of 32):
+ *   pre = bf16(h w_up^T + b_up), dhidden = bf16(dy w_down)   -- recomputed in registers, never written --
+ *   hidden [M, F] = act(pre), grad_pre [M, 2F] = d act / d pre * dhidden      (formulas of taac_swiglu_bwd)
+ * h: [M, D] input of the up projection (the normalised rows), dy: [M, D] gradient of the feed-forward output; both bf16.
+ * packed: the blob written by taac_swiglu_ffn_bwd_pack_weights for (w_up [2F, D], w_down [D, F]),
+ * taac_swiglu_ffn_bwd_packed_bytes(D, F) bytes (-1: shape not covered). b_up: [2F] or NULL.
+ * The outputs are the operands of the two weight gradients (taac_linear_wgrad) and of the input gradient
+ * grad_pre w_up. Replaces: the up projection, dy w_down and the activation backward that torch autograd runs as
+ * separate kernels for SwiGLUFeedForward (experiments/symbiosis/backbone.py:11-21).
+ */
+int64_t taac_swiglu_ffn_bwd_packed_bytes(int32_t D, int32_t F);
+int taac_swiglu_ffn_bwd_pack_weights(const void* w_up, const void* w_down, void* packed, int32_t D, int32_t F, void* stream);
+int taac_swiglu_ffn_bwd_hidden(const void* h, int64_t ldh, const void* dy, int64_t lddy, const void* packed,
+                               const void* b_up, void* hidden, int64_t ldhid, void* grad_pre, int64_t ldgp, int64_t M,
+                               int32_t D, int32_t F, int gate_first, void* stream);
+
+/*
  * Fused feed-forward half of a block, one kernel:
  *   out = residual + down( silu(g) * u ),   g, u = chunk2( up( norm_weight ? rmsnorm(x, norm_weight, eps) : x ) )
  * x: [M, D] bf16 (row stride ldx); w_up: [2F, D]; b_up: [2F] or NULL; w_down: [D, F]; b_down: [D] or NULL;

@@ -134,6 +134,13 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         c_int,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int32, c_int, c_void_p],
     ),
+    "taac_swiglu_ffn_bwd_packed_bytes": (c_int64, [c_int32, c_int32]),
+    "taac_swiglu_ffn_bwd_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
+    "taac_swiglu_ffn_bwd_hidden": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int32,
+         c_int32, c_int, c_void_p],
+    ),
     "taac_flash_attn_train_dropout_fwd": (
         c_int,
         [c_void_p] * 5 + [c_float] + [c_void_p] * 2 + [c_int32, c_int32, c_int32, c_int32, c_int32]

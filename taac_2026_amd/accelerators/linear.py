@@ -99,10 +99,57 @@ def swiglu_backward(pre_activation: torch.Tensor, grad_hidden: torch.Tensor | No
             None if grad is None else grad.reshape(*shape[:-1], 2 * hidden_size))
 
 
+def swiglu_ffn_backward_hidden(h: torch.Tensor, grad_out: torch.Tensor, up_weight: torch.Tensor,
+                               up_bias: torch.Tensor | None, down_weight: torch.Tensor, *,
+                               gate_first: bool = True) -> tuple[torch.Tensor, torch.Tensor] | None:
+    """The activation part of the feed-forward backward as one kernel (``taac_swiglu_ffn_bwd_hidden``): from the input
+    ``h [.., D]`` of the up projection and the gradient ``grad_out [.., D]`` of the feed-forward output, the hidden state
+    ``[.., F]`` and the gradient ``[.., 2F]`` of the up projection; the up projection itself and ``grad_out @ down_weight``
+    stay in registers. Returns ``None`` for shapes the kernel is not built for (width 128 / 256, F a multiple of 32)."""
+    name = "hip swiglu_ffn_backward_hidden"
+    require_cuda_tensors(name, h, grad_out, up_weight, up_bias, down_weight)
+    _check_bf16(name, h, grad_out, up_weight, up_bias, down_weight)
+    rows, shape = _as_rows(h)
+    dy, _ = _as_rows(grad_out)
+    d_model, hidden_size = down_weight.shape
+    if rows.shape != dy.shape or rows.shape[1] != d_model or up_weight.shape != (2 * hidden_size, d_model):
+        raise ValueError(f"{name}: expected h and grad_out [.., D], up_weight [2F, D], down_weight [D, F]")
+    library = _native.load_library()
+    nbytes = int(library.taac_swiglu_ffn_bwd_packed_bytes(d_model, hidden_size))
+    if nbytes < 0:
+        return None
+
+    def pack() -> torch.Tensor:
+        blob = torch.empty(nbytes, dtype=torch.uint8, device=rows.device)
+        status = library.taac_swiglu_ffn_bwd_pack_weights(
+            up_weight.detach().contiguous().data_ptr(), down_weight.detach().contiguous().data_ptr(), blob.data_ptr(),
+            d_model, hidden_size, _native.current_stream(rows.device))
+        _native.check(status, "swiglu_ffn_backward_hidden (pack)")
+        return blob
+
+    packed = _packed_cache.get((up_weight, down_weight), pack, variant=2)
+    hidden = torch.empty(rows.shape[0], hidden_size, dtype=rows.dtype, device=rows.device)
+    grad_pre = torch.empty(rows.shape[0], 2 * hidden_size, dtype=rows.dtype, device=rows.device)
+    status = library.taac_swiglu_ffn_bwd_hidden(
+        rows.data_ptr(), rows.stride(0), dy.data_ptr(), dy.stride(0), packed.data_ptr(), _native.ptr(up_bias),
+        hidden.data_ptr(), hidden_size, grad_pre.data_ptr(), 2 * hidden_size, rows.shape[0], d_model, hidden_size,
+        int(bool(gate_first)), _native.current_stream(rows.device))
+    _native.check(status, "swiglu_ffn_backward_hidden")
+    return hidden.reshape(*shape[:-1], hidden_size), grad_pre.reshape(*shape[:-1], 2 * hidden_size)
+
+
+def _plain_product(rows: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """``F.linear(rows, weight, bias)`` without autograd, by the token-stationary kernel where its shapes allow
+    (:func:`norm_linear` without a norm), else by the tiled one."""
+    with torch.no_grad():
+        if _fused_width(weight.shape[1]) and weight.shape[0] % 64 == 0:
+            return norm_linear(rows, weight, bias)
+        return linear(rows, weight, bias)
+
+
 def _input_grad(grad_rows: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``grad_rows @ weight``: a forward-shaped product with the transposed weight."""
-    with torch.no_grad():
-        return linear(grad_rows, weight.detach().t().contiguous())
+    return _plain_product(grad_rows, weight.detach().t().contiguous())
 
 
 class _NormLinearFunction(torch.autograd.Function):
@@ -172,9 +219,13 @@ class _SwigluFfnFunction(torch.autograd.Function):
         dy = dy.contiguous()
         with torch.no_grad():
             h = hip_rms_norm_kernel(rows, norm_weight, eps) if has_norm else rows
-            pre = linear(h, up_weight.detach(), None if up_bias is None else up_bias.detach())   # [M, 2F]
-            grad_hidden = _input_grad(dy, down_weight)                                           # [M, F]
-            hidden, grad_pre = swiglu_backward(pre, grad_hidden, gate_first=gate_first)
+            fused = swiglu_ffn_backward_hidden(h, dy, up_weight, up_bias, down_weight, gate_first=gate_first)
+            if fused is not None:
+                hidden, grad_pre = fused
+            else:
+                pre = _plain_product(h, up_weight.detach(), None if up_bias is None else up_bias.detach())   # [M, 2F]
+                grad_hidden = _input_grad(dy, down_weight)                                           # [M, F]
+                hidden, grad_pre = swiglu_backward(pre, grad_hidden, gate_first=gate_first)
             grad_down_w, grad_down_b = linear_wgrad(dy, hidden, with_bias=has_down_bias)
             grad_up_w, grad_up_b = linear_wgrad(grad_pre, h, with_bias=has_up_bias)
             grad_h = _input_grad(grad_pre, up_weight)
@@ -926,6 +977,7 @@ __all__ = [
     "linear",
     "linear_fp8",
     "linear_wgrad",
+    "swiglu_ffn_backward_hidden",
     "swiglu_backward",
     "norm_linear",
     "pack_ffn_weights",

@@ -19,7 +19,7 @@ CSRC_DIR = PACKAGE_DIR / "csrc"
 BUILD_DIR = PACKAGE_DIR / "csrc" / "build"
 LIBRARY_PATH = PACKAGE_DIR / "libtaac_hip.so"
 
-SOURCES = ("runtime.hip", "norm.hip", "attention.hip", "linear.hip", "ffn.hip", "fp8.hip", "fp8_ts.hip", "ffn_fp8.hip", "backbone.hip", "embedding.hip", "attention_bwd.hip", "readout.hip", "linear_bwd.hip")
+SOURCES = ("runtime.hip", "norm.hip", "attention.hip", "linear.hip", "ffn.hip", "fp8.hip", "fp8_ts.hip", "ffn_fp8.hip", "backbone.hip", "embedding.hip", "attention_bwd.hip", "readout.hip", "linear_bwd.hip", "ffn_bwd.hip")
 
 # -packed-fp32-ops: keep the compiler from forming packed-fp32 VALU instructions from scalar float code.
 HIPCC_FLAGS = (

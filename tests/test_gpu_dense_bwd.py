@@ -10,7 +10,8 @@ import torch
 import torch.nn.functional as F
 
 from oracle import reference as oracle
-from taac_2026_amd.api import (UnifiedInteractionBlock, linear, linear_wgrad, norm_linear, swiglu_backward, swiglu_ffn)
+from taac_2026_amd.api import (UnifiedInteractionBlock, linear, linear_wgrad, norm_linear, swiglu_backward, swiglu_ffn,
+                               swiglu_ffn_backward_hidden)
 
 pytestmark = pytest.mark.gpu
 
@@ -66,6 +67,47 @@ def test_silu_gate_backward(device, gate_first):
     _close(grad_pre, ref.grad, 1e-2)
     only_hidden, none = swiglu_backward(pre.to(device), None, gate_first=gate_first)
     assert none is None and torch.equal(only_hidden, hidden)
+
+
+@pytest.mark.parametrize("m,d,f,gate_first,with_bias", [(1, 128, 32, True, True), (255, 256, 96, False, True),
+                                                          (257, 256, 1024, True, True), (1000, 128, 2048, True, False),
+                                                          (4096, 256, 512, False, False)])
+def test_feed_forward_backward_hidden_kernel(device, m, d, f, gate_first, with_bias):
+    """The one-kernel activation backward (up projection and ``dy @ w_down`` recomputed in registers) against float64
+    autograd of the same expression, and against the three-kernel route it replaces (equal up to the roundings of
+    bfloat16: that route rounds the same intermediate values)."""
+    g = torch.Generator().manual_seed(m + f)
+    bf = lambda t: t.to(torch.bfloat16)  # noqa: E731
+    h = bf(torch.randn(m, d, generator=g))
+    dy = bf(torch.randn(m, d, generator=g))
+    up_w = bf(torch.randn(2 * f, d, generator=g) * d ** -0.5)
+    up_b = bf(0.5 * torch.randn(2 * f, generator=g)) if with_bias else None
+    down_w = bf(torch.randn(d, f, generator=g) * f ** -0.5)
+    on = lambda t: None if t is None else t.to(device)  # noqa: E731
+    hidden, grad_pre = swiglu_ffn_backward_hidden(on(h), on(dy), on(up_w), on(up_b), on(down_w), gate_first=gate_first)
+    assert hidden.shape == (m, f) and grad_pre.shape == (m, 2 * f)
+    pre = (F.linear(h.double(), up_w.double(), None if up_b is None else up_b.double())).requires_grad_(True)
+    gate, value = pre.chunk(2, dim=-1)
+    want = F.silu(gate) * value if gate_first else gate * F.silu(value)
+    want.backward(dy.double() @ down_w.double())
+    _close(hidden, want.detach(), 1e-2)
+    _close(grad_pre, pre.grad, 1.5e-2)
+    with torch.no_grad():
+        pre_rows = linear(on(h), on(up_w), on(up_b))
+        grad_hidden = linear(on(dy), on(down_w).t().contiguous())
+    hidden_steps, grad_steps = swiglu_backward(pre_rows, grad_hidden, gate_first=gate_first)
+    _close(hidden, hidden_steps.cpu(), 1e-2)
+    _close(grad_pre, grad_steps.cpu(), 1e-2)
+
+
+def test_feed_forward_backward_hidden_kernel_shapes(device):
+    z = lambda *shape: torch.zeros(*shape, dtype=torch.bfloat16, device=device)  # noqa: E731
+    assert swiglu_ffn_backward_hidden(z(4, 64), z(4, 64), z(2 * 32, 64), None, z(64, 32)) is None     # width 64: not built
+    assert swiglu_ffn_backward_hidden(z(4, 256), z(4, 256), z(2 * 40, 256), None, z(256, 40)) is None  # F not a multiple of 32
+    with pytest.raises(ValueError, match="expected h and grad_out"):
+        swiglu_ffn_backward_hidden(z(4, 256), z(5, 256), z(64, 256), None, z(256, 32))
+    hidden, grad_pre = swiglu_ffn_backward_hidden(z(0, 256), z(0, 256), z(64, 256), None, z(256, 32))
+    assert hidden.shape == (0, 32) and grad_pre.shape == (0, 64)
 
 
 def _dense_case(m, d, n, seed):
