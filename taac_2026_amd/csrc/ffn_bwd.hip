@@ -15,8 +15,10 @@
 // blocks - rows 32 s.. of the first half of W_up, of its second half, and of W_down^T - multiply h, h and dy into three
 // 32 x 32 accumulators in which a lane holds, for ITS token, the same 16 hidden units of all three, so the activation
 // backward is lane-local arithmetic. The weights come as a blob in fragment order (taac_swiglu_ffn_bwd_pack_weights)
-// and stream L2 -> LDS by direct transfers through two buffers, one step ahead; results leave through a
-// wavefront-private LDS tile as 16-byte stores that cover 64-byte runs of a row.
+// and stream L2 -> LDS by direct transfers through a ring of four 24 KB buffers, three sub-steps ahead (a sub-step is
+// eight k-steps of the three blocks: half a step at D = 256, a whole one at D = 128; with two whole-step buffers, one
+// step ahead, the wait for the weights was exposed in every step: 1.54 ms against the time below at 524 288 tokens);
+// results leave through a wavefront-private LDS tile as 16-byte stores that cover 64-byte runs of a row.
 #include "ts_common.h"
 
 namespace taac {
@@ -26,6 +28,8 @@ constexpr int kFrag = 1024;                     // bytes of one 32 x 16 bf16 MFM
 constexpr int kWaves = 8;
 constexpr int kTokPerWg = kWaves * 32;
 constexpr int kUnits = 32;                      // hidden units per step
+constexpr int kSubK = 8;                        // k-steps (of 16 features) per sub-step
+constexpr int kRing = 4;                        // weight buffers
 constexpr int kTileRow = 3 * kUnits * 2 + 16;   // epilogue tile row: hidden | grad first half | grad second half | pad
 constexpr int kTileWave = 32 * kTileRow;
 
@@ -40,19 +44,20 @@ struct FfnBwdParams {
   int32_t F;
 };
 
-// Blob: step s (32 hidden units) holds fragments (block b, k-step ks) at index b * KS + ks; block 0 = rows 32 s .. of
-// the first half of w_up, block 1 = the same rows of its second half, block 2 = columns 32 s .. of w_down (rows of its
-// transpose). Lane (l32, hh) of a fragment holds k = 16 ks + 8 hh .. + 7 of row l32.
+// Blob: step s (32 hidden units), sub-step u (k-steps 8 u .. 8 u + 7) holds fragments (block b, k-step 8 u + j) at index
+// b * 8 + j; block 0 = rows 32 s .. of the first half of w_up, block 1 = the same rows of its second half, block 2 =
+// columns 32 s .. of w_down (rows of its transpose). Lane (l32, hh) of a fragment holds k = 16 ks + 8 hh .. + 7 of row l32.
 __global__ void ffn_bwd_pack_kernel(const bf16_t* __restrict__ w_up, const bf16_t* __restrict__ w_down,
                                     bf16x8* __restrict__ packed, int D, int F) {
   const int64_t total = static_cast<int64_t>(3) * D * F / 8;
   const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (gid >= total) return;
-  const int KS = D / 16, NFRAG = 3 * KS;
+  const int NSUB = D / 16 / kSubK, NFRAG = 3 * kSubK;
   const int lane = static_cast<int>(gid % 64);
   const int f = static_cast<int>((gid / 64) % NFRAG);
-  const int64_t step = gid / 64 / NFRAG;
-  const int b = f / KS, ks = f % KS;
+  const int64_t sub = gid / 64 / NFRAG;  // step * NSUB + u
+  const int64_t step = sub / NSUB;
+  const int b = f / kSubK, ks = static_cast<int>(sub % NSUB) * kSubK + f % kSubK;
   const int l32 = lane % 32, hh = lane / 32;
   const int64_t unit = step * kUnits + l32;
   const int k0 = ks * 16 + hh * 8;
@@ -76,14 +81,15 @@ __device__ __forceinline__ float round_bf16(float v) { return static_cast<float>
 template <int D, bool GATE_FIRST>
 __global__ __launch_bounds__(kWaves * kWave, 2) void swiglu_ffn_bwd_hidden_kernel(const FfnBwdParams p) {
   constexpr int KS = D / 16;
-  constexpr int NFRAG = 3 * KS;
-  constexpr int FPW = NFRAG / kWaves;   // transfers per wavefront and step
+  constexpr int NSUB = KS / kSubK;      // sub-steps per step
+  constexpr int NFRAG = 3 * kSubK;      // fragments per sub-step
+  constexpr int FPW = NFRAG / kWaves;   // transfers per wavefront and sub-step
   constexpr int kBuf = NFRAG * kFrag;
   constexpr int PRE = 3;                // fragment triples in flight
   constexpr int NST = 6;                // output stores per wavefront and step
-  static_assert(NFRAG % kWaves == 0, "every wavefront stages the same number of fragments");
+  static_assert(KS % kSubK == 0 && NFRAG % kWaves == 0, "every wavefront stages the same number of fragments");
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  uint8_t* tiles = smem + 2 * kBuf;
+  uint8_t* tiles = smem + kRing * kBuf;
   bf16_t* bias_lds = reinterpret_cast<bf16_t*>(tiles + kWaves * kTileWave);
 
   const int tid = threadIdx.x;
@@ -92,23 +98,26 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void swiglu_ffn_bwd_hidden_kerne
   const int l32 = lane % 32;
   const int hh = lane / 32;
   const int nsteps = p.F / kUnits;
+  const int nsub = nsteps * NSUB;
   const int64_t tok0 = static_cast<int64_t>(blockIdx.x) * kTokPerWg + wave * 32;
   // Tokens at or beyond M are mapped to the last token: they compute the same values, so the duplicate stores are
   // benign and every wavefront issues the same number of memory operations (the hand-counted waits rely on that).
   auto row_of = [&](int64_t tok) -> int64_t { return tok < p.M ? tok : p.M - 1; };
 
   const char* w_bytes = reinterpret_cast<const char*>(p.packed);
-  auto stage = [&](int step, int buf) {
+  auto stage = [&](int q) {  // sub-step q -> ring slot q % kRing
     int ln = lane;
     asm volatile("" : "+v"(ln));
-    uint8_t* base = smem + buf * kBuf + wave * (FPW * kFrag);
-    const char* src = w_bytes + (static_cast<int64_t>(step) * NFRAG + wave * FPW) * kFrag;  // scalar registers
+    uint8_t* base = smem + (q % kRing) * kBuf + wave * (FPW * kFrag);
+    const char* src = w_bytes + (static_cast<int64_t>(q) * NFRAG + wave * FPW) * kFrag;  // scalar registers
     const uint32_t lane_off = static_cast<uint32_t>(ln * 16);
 #pragma unroll
     for (int i = 0; i < FPW; ++i) lds_dma16_offset(src + i * kFrag, lane_off, base + i * kFrag);
   };
 
-  stage(0, 0);
+#pragma unroll
+  for (int q = 0; q < kRing - 1; ++q)
+    if (q < nsub) stage(q);
   stage_bias(p.b_up, bias_lds, 2 * p.F, tid, kWaves * kWave);
   bf16x8 hf[KS], df[KS];
   {
@@ -132,89 +141,98 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void swiglu_ffn_bwd_hidden_kerne
 
   uint8_t* tile = tiles + wave * kTileWave;
   for (int s = 0; s < nsteps; ++s) {
-    const bool has_next = s + 1 < nsteps;
-    if (has_next) stage(s + 1, (s + 1) & 1);  // that buffer was last read in step s - 1, which every wavefront has left
-
-    const uint32_t wb = lds_offset(smem) + (s & 1) * kBuf + lane * 16;
     f32x16 acc_a, acc_b, acc_d;
 #pragma unroll
     for (int j = 0; j < 16; ++j) acc_a[j] = acc_b[j] = acc_d[j] = 0.f;
-    bf16x8 fa[PRE], fb[PRE], fd[PRE];
-    static_for<PRE>([&](auto k) {
-      constexpr int K_ = decltype(k)::value;
-      lds_read_frag<K_ * kFrag>(fa[K_], wb);
-      lds_read_frag<(KS + K_) * kFrag>(fb[K_], wb);
-      lds_read_frag<(2 * KS + K_) * kFrag>(fd[K_], wb);
-    });
-    static_for<KS>([&](auto k) {
-      constexpr int K_ = decltype(k)::value;
-      constexpr int R = K_ % PRE;
-      // reads issued behind triple K_: the triples up to min(K_ + PRE - 1, KS - 1)
-      constexpr int newest = K_ + PRE - 1 < KS - 1 ? K_ + PRE - 1 : KS - 1;
-      lds_wait_triple<3 * (newest - K_)>(fa[R], fb[R], fd[R]);
-      acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[R], hf[K_], acc_a, 0, 0, 0);
-      acc_b = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[R], hf[K_], acc_b, 0, 0, 0);
-      acc_d = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fd[R], df[K_], acc_d, 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      if constexpr (K_ + PRE < KS) {
-        lds_read_frag<(K_ + PRE) * kFrag>(fa[R], wb);
-        lds_read_frag<(KS + K_ + PRE) * kFrag>(fb[R], wb);
-        lds_read_frag<(2 * KS + K_ + PRE) * kFrag>(fd[R], wb);
+    static_for<NSUB>([&](auto u) {
+      constexpr int U = decltype(u)::value;
+      const int q = s * NSUB + U;
+      // slot (q + 3) % 4 was last read in sub-step q - 1, which every wavefront has left
+      if (q + kRing - 1 < nsub) stage(q + kRing - 1);
+      const uint32_t wb = lds_offset(smem) + (q % kRing) * kBuf + lane * 16;
+      bf16x8 fa[PRE], fb[PRE], fd[PRE];
+      static_for<PRE>([&](auto k) {
+        constexpr int K_ = decltype(k)::value;
+        lds_read_frag<K_ * kFrag>(fa[K_], wb);
+        lds_read_frag<(kSubK + K_) * kFrag>(fb[K_], wb);
+        lds_read_frag<(2 * kSubK + K_) * kFrag>(fd[K_], wb);
+      });
+      static_for<kSubK>([&](auto k) {
+        constexpr int K_ = decltype(k)::value;
+        constexpr int R = K_ % PRE;
+        // reads issued behind triple K_: the triples up to min(K_ + PRE - 1, kSubK - 1)
+        constexpr int newest = K_ + PRE - 1 < kSubK - 1 ? K_ + PRE - 1 : kSubK - 1;
+        lds_wait_triple<3 * (newest - K_)>(fa[R], fb[R], fd[R]);
+        acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[R], hf[U * kSubK + K_], acc_a, 0, 0, 0);
+        acc_b = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[R], hf[U * kSubK + K_], acc_b, 0, 0, 0);
+        acc_d = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fd[R], df[U * kSubK + K_], acc_d, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (K_ + PRE < kSubK) {
+          lds_read_frag<(K_ + PRE) * kFrag>(fa[R], wb);
+          lds_read_frag<(kSubK + K_ + PRE) * kFrag>(fb[R], wb);
+          lds_read_frag<(2 * kSubK + K_ + PRE) * kFrag>(fd[R], wb);
+        }
+      });
+      if constexpr (U == NSUB - 1) {
+        // ---- activation backward in accumulator order: register jq * 4 + e of lane (l32, hh) is hidden unit
+        //      32 s + jq * 8 + hh * 4 + e of token l32 ----------------------------------------------------------------------
+        const bf16_t* bias = bias_lds + s * kUnits + hh * 4;
+#pragma unroll
+        for (int jq = 0; jq < 4; ++jq) {
+          const bf16x4 ba = *reinterpret_cast<const bf16x4*>(bias + jq * 8);
+          const bf16x4 bb = *reinterpret_cast<const bf16x4*>(bias + p.F + jq * 8);
+          bf16x4 hv, ga, gb;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float a = round_bf16(acc_a[jq * 4 + e] + static_cast<float>(ba[e]));
+            const float b = round_bf16(acc_b[jq * 4 + e] + static_cast<float>(bb[e]));
+            const float d = round_bf16(acc_d[jq * 4 + e]);
+            const float act = GATE_FIRST ? a : b;  // the operand that goes through SiLU
+            const float lin = GATE_FIRST ? b : a;  // the one that multiplies it
+            const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * act));
+            const float silu = act * sig;
+            const float dact = d * lin * (sig * (1.f + act * (1.f - sig)));
+            const float dlin = d * silu;
+            hv[e] = static_cast<bf16_t>(silu * lin);
+            ga[e] = static_cast<bf16_t>(GATE_FIRST ? dact : dlin);
+            gb[e] = static_cast<bf16_t>(GATE_FIRST ? dlin : dact);
+          }
+          uint8_t* dst = tile + l32 * kTileRow + (jq * 8 + hh * 4) * 2;
+          *reinterpret_cast<bf16x4*>(dst) = hv;
+          *reinterpret_cast<bf16x4*>(dst + kUnits * 2) = ga;
+          *reinterpret_cast<bf16x4*>(dst + 2 * kUnits * 2) = gb;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        // ---- row-wise out of the tile: lane -> token 16 * i + lane / 4, 16-byte piece lane % 4 of each 64-byte run --------
+        const int unit0 = s * kUnits + (lane % 4) * 8;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const uint8_t* src = tile + (i * 16 + lane / 4) * kTileRow + (lane % 4) * 16;
+          const bf16x8 hv = *reinterpret_cast<const bf16x8*>(src);
+          const bf16x8 ga = *reinterpret_cast<const bf16x8*>(src + kUnits * 2);
+          const bf16x8 gb = *reinterpret_cast<const bf16x8*>(src + 2 * kUnits * 2);
+          *reinterpret_cast<bf16x8*>(p.hidden + prow[i] * p.ldhid + unit0) = hv;
+          *reinterpret_cast<bf16x8*>(p.grad_pre + prow[i] * p.ldgp + unit0) = ga;
+          *reinterpret_cast<bf16x8*>(p.grad_pre + prow[i] * p.ldgp + p.F + unit0) = gb;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      }
+      if (q + 1 < nsub) {
+        // The transfers of sub-step q + 1 were issued at the start of sub-step q - 2 (or in front of the loop, where
+        // everything was awaited). Behind them this wavefront has issued at least: the transfers of q + 2 and q + 3 (where
+        // those exist) and the stores of the epilogues in sub-steps q - 1 and q (one of the two at D = 256, both at D = 128).
+        constexpr int kStores = NST * (NSUB == 1 ? 2 : 1);
+        if (q + 3 < nsub) vm_wait<kStores + 2 * FPW>();
+        else if (q + 2 < nsub) vm_wait<kStores + FPW>();
+        else vm_wait<kStores>();
+        __syncthreads();
       }
     });
-
-    // ---- activation backward in accumulator order: register jq * 4 + e of lane (l32, hh) is hidden unit
-    //      32 s + jq * 8 + hh * 4 + e of token l32 ----------------------------------------------------------------------
-    const bf16_t* bias = bias_lds + s * kUnits + hh * 4;
-#pragma unroll
-    for (int jq = 0; jq < 4; ++jq) {
-      const bf16x4 ba = *reinterpret_cast<const bf16x4*>(bias + jq * 8);
-      const bf16x4 bb = *reinterpret_cast<const bf16x4*>(bias + p.F + jq * 8);
-      bf16x4 hv, ga, gb;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float a = round_bf16(acc_a[jq * 4 + e] + static_cast<float>(ba[e]));
-        const float b = round_bf16(acc_b[jq * 4 + e] + static_cast<float>(bb[e]));
-        const float d = round_bf16(acc_d[jq * 4 + e]);
-        const float act = GATE_FIRST ? a : b;  // the operand that goes through SiLU
-        const float lin = GATE_FIRST ? b : a;  // the one that multiplies it
-        const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * act));
-        const float silu = act * sig;
-        const float dact = d * lin * (sig * (1.f + act * (1.f - sig)));
-        const float dlin = d * silu;
-        hv[e] = static_cast<bf16_t>(silu * lin);
-        ga[e] = static_cast<bf16_t>(GATE_FIRST ? dact : dlin);
-        gb[e] = static_cast<bf16_t>(GATE_FIRST ? dlin : dact);
-      }
-      uint8_t* dst = tile + l32 * kTileRow + (jq * 8 + hh * 4) * 2;
-      *reinterpret_cast<bf16x4*>(dst) = hv;
-      *reinterpret_cast<bf16x4*>(dst + kUnits * 2) = ga;
-      *reinterpret_cast<bf16x4*>(dst + 2 * kUnits * 2) = gb;
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    // ---- row-wise out of the tile: lane -> token 16 * i + lane / 4, 16-byte piece lane % 4 of each 64-byte run --------
-    const int unit0 = s * kUnits + (lane % 4) * 8;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const uint8_t* src = tile + (i * 16 + lane / 4) * kTileRow + (lane % 4) * 16;
-      const bf16x8 hv = *reinterpret_cast<const bf16x8*>(src);
-      const bf16x8 ga = *reinterpret_cast<const bf16x8*>(src + kUnits * 2);
-      const bf16x8 gb = *reinterpret_cast<const bf16x8*>(src + 2 * kUnits * 2);
-      *reinterpret_cast<bf16x8*>(p.hidden + prow[i] * p.ldhid + unit0) = hv;
-      *reinterpret_cast<bf16x8*>(p.grad_pre + prow[i] * p.ldgp + unit0) = ga;
-      *reinterpret_cast<bf16x8*>(p.grad_pre + prow[i] * p.ldgp + p.F + unit0) = gb;
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if (has_next) {
-      // behind the transfers of step s + 1 this wavefront has issued the NST stores of this step: they may stay in flight
-      vm_wait<NST>();
-      __syncthreads();
-    }
   }
 }
 
 size_t bwd_lds_bytes(int32_t D, int32_t F) {
-  return static_cast<size_t>(2) * 3 * (D / 16) * kFrag + kWaves * kTileWave + static_cast<size_t>(2) * F * 2;
+  return static_cast<size_t>(kRing) * 3 * kSubK * kFrag + kWaves * kTileWave + static_cast<size_t>(2) * F * 2;
 }
 
 bool bwd_shape_ok(int32_t D, int32_t F) {

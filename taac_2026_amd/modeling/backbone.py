@@ -22,6 +22,7 @@ from taac_2026_amd.accelerators.attention import StructuredAttentionMask, front_
 from taac_2026_amd.accelerators.linear import (attention_out_ffn, front_rows, norm_linear, qkv_projection, swiglu_ffn,
                                                valid_rows)
 from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference
+from taac_2026_amd.modeling.block_training import run_training_block, training_route_applies
 from taac_2026_amd.modeling.normalization import RMSNorm
 from taac_2026_amd.modeling.sequence import scaled_dot_product_attention
 
@@ -265,6 +266,11 @@ class UnifiedInteractionBlock(nn.Module):
     ) -> tuple[torch.Tensor, torch.Tensor | None]:
         if self._fused_route(tokens):
             return self._forward_fused(tokens, padding_mask, attention_mask, key_lengths, return_attention_tokens, inplace)
+        if torch.is_grad_enabled() and training_route_applies(self, tokens, attention_mask, key_lengths):
+            # prefix padding, plain attention layer, no dropout: the whole block as one autograd function over the valid rows
+            result = run_training_block(self, tokens, key_lengths, return_attention_tokens)
+            if result is not None:
+                return result
         keep = (~padding_mask).unsqueeze(-1)
         attn_update = self.attention(self.attn_norm(tokens), attention_mask, key_lengths=key_lengths)
         attn_tokens = tokens + attn_update * keep.to(attn_update.dtype)

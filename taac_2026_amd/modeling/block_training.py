@@ -1,0 +1,225 @@
+"""Training route of ``UnifiedInteractionBlock`` (experiments/symbiosis/backbone.py:51-68) under prefix padding: one
+autograd function for the whole block whose forward and backward run over the VALID tokens only.
+
+The reference multiplies both residual updates by ``~padding_mask``, so a padded position passes its input through and
+contributes nothing to any weight gradient. The function therefore gathers the valid rows of the token stream once
+into a compact ``[valid, D]`` tensor and runs every dense layer, norm and weight gradient on compact tensors; only the
+attention kernels see the padded ``[B, T, .]`` layout, which the projections on either side of them write and read
+through the row index of :func:`valid_rows` (no copy). At the benchmark's lengths (54 % of the positions valid) the dense
+forward and backward kernels do 54 % of the work of the layer-by-layer route, the packed q | k | v gradient is written
+in place (no concatenation) and the mask multiplications and residual adds of autograd disappear.
+
+The number of valid rows sizes the compact tensors, so it is read back from the device once per ``key_lengths`` tensor
+(one host synchronisation, shared by the blocks of a stack).
+"""
+
+from __future__ import annotations
+
+import importlib
+import weakref
+
+import torch
+
+from taac_2026_amd import _native
+
+# the package re-exports a function of the same name, which shadows the module as an attribute
+_linear = importlib.import_module("taac_2026_amd.accelerators.linear")
+from taac_2026_amd.accelerators.normalization import hip_rms_norm_backward_kernel, hip_rms_norm_kernel
+
+
+class _RowIndex:
+    """Valid-row index of the last ``key_lengths`` tensor seen: ``rows`` (int32, :func:`valid_rows`), ``count`` (device
+    scalar), ``valid`` (the same number on the host), ``gather`` (int64 ``rows[:valid]`` for torch's index kernels) and
+    ``identity`` (int32 ``0..valid-1``: the row numbers of a compact tensor)."""
+
+    _last: tuple | None = None
+
+    @classmethod
+    def get(cls, key_lengths: torch.Tensor, tokens: int):
+        stamp = cls._last
+        if stamp is not None:
+            ref, version, pointer, width, entry = stamp
+            if ref() is key_lengths and version == key_lengths._version and pointer == key_lengths.data_ptr() and width == tokens:
+                return entry
+        rows, count = _linear.valid_rows(key_lengths, tokens)
+        valid = int(count.item())
+        gather = rows[:valid].to(torch.int64)
+        identity = torch.arange(max(valid, 1), dtype=torch.int32, device=rows.device)
+        entry = (rows, count, valid, gather, identity)
+        cls._last = (weakref.ref(key_lengths), key_lengths._version, key_lengths.data_ptr(), tokens, entry)
+        return entry
+
+
+def _indexed_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor, *, tokens: int,
+                    out_rows: torch.Tensor, count: torch.Tensor, x_rows: torch.Tensor, norm_weight: torch.Tensor | None = None,
+                    eps: float = 1e-6, residual: torch.Tensor | None = None, cache_weight: bool = True) -> None:
+    """``out[out_rows[i]] = residual[out_rows[i]] + linear(rmsnorm(x[x_rows[i]]))`` for ``i < tokens``
+    (``taac_norm_linear_fwd`` with both of its row indices): the projection that crosses between the compact and the padded
+    layout."""
+    out_features, in_features = weight.shape
+    pack = lambda: _linear.pack_linear_weight(weight)  # noqa: E731
+    packed = _linear._packed_cache.get((weight,), pack) if cache_weight else pack()
+    library = _native.load_library()
+    status = library.taac_norm_linear_fwd(
+        x.data_ptr(), x.stride(0), _native.ptr(norm_weight), float(eps), None, _native.ptr(bias), packed.data_ptr(),
+        _native.ptr(residual), residual.stride(0) if residual is not None else out_features, out.data_ptr(), out.stride(0),
+        tokens, out_features, in_features, out_rows.data_ptr(), count.data_ptr(), x_rows.data_ptr(),
+        _native.current_stream(x.device))
+    _native.check(status, "interaction block (training): projection")
+
+
+def _attention_strides(width: int, heads: int, row_stride: int, tokens: int):
+    """Element strides of a logical (B, H, T, d) view of ``[B * T, row_stride]`` rows whose heads lie side by side."""
+    return _native.Int64x4(tokens * row_stride, width // heads, row_stride, 1)
+
+
+class InteractionBlockFunction(torch.autograd.Function):
+    """``UnifiedInteractionBlock.forward`` without query / key norm, dropout or an attention mask other than the key
+    lengths. Inputs: tokens ``[B, T, D]`` bf16, ``key_lengths`` int32 ``[B]``, then the block's parameters. Returns
+    ``(output, attn_tokens)`` like the module (``attn_tokens`` is None unless asked for)."""
+
+    @staticmethod
+    def forward(ctx, tokens, key_lengths, want_attn_tokens, num_heads, attn_eps, ffn_eps, gate_first, attn_norm_w, w_qkv,
+                b_qkv, w_out, b_out, ffn_norm_w, w_up, b_up, w_down, b_down):
+        batch, token_count, width = tokens.shape
+        total = batch * token_count
+        rows, count, valid, gather, identity = _RowIndex.get(key_lengths, token_count)
+        flat = tokens.detach().reshape(total, width)
+        if not flat.is_contiguous():
+            flat = flat.contiguous()
+        library = _native.load_library()
+        stream = _native.current_stream(tokens.device)
+        xc = flat.index_select(0, gather)                                               # [valid, D]
+        qkv = torch.empty(total, 3 * width, dtype=flat.dtype, device=flat.device)      # padded layout; padded rows unused
+        _indexed_linear(xc, w_qkv, b_qkv, qkv, tokens=valid, out_rows=rows, count=count, x_rows=identity,
+                        norm_weight=attn_norm_w, eps=attn_eps)
+        attended = torch.zeros(total, width, dtype=flat.dtype, device=flat.device)
+        lse = torch.empty(batch, num_heads, token_count, dtype=torch.float32, device=flat.device)
+        qkv_strides = _attention_strides(width, num_heads, 3 * width, token_count)
+        out_strides = _attention_strides(width, num_heads, width, token_count)
+        element = qkv.element_size()
+        status = library.taac_flash_attn_train_fwd(
+            qkv.data_ptr(), qkv.data_ptr() + width * element, qkv.data_ptr() + 2 * width * element, key_lengths.data_ptr(),
+            attended.data_ptr(), lse.data_ptr(), batch, num_heads, token_count, token_count, width // num_heads,
+            qkv_strides, qkv_strides, qkv_strides, out_strides, 0, 1, _native.dtype_code(flat.dtype), stream)
+        _native.check(status, "interaction block (training): attention")
+        x1c = torch.empty(valid, width, dtype=flat.dtype, device=flat.device)
+        _indexed_linear(attended, w_out, b_out, x1c, tokens=valid, out_rows=identity, count=count, x_rows=rows, residual=xc)
+        yc = _linear.swiglu_ffn(x1c, w_up, b_up, w_down, b_down, residual=x1c, gate_first=gate_first,
+                                norm_weight=ffn_norm_w, eps=ffn_eps)
+        output = flat.clone()
+        output.index_copy_(0, gather, yc)
+        attn_tokens = None
+        if want_attn_tokens:
+            attn_tokens = flat.clone()
+            attn_tokens.index_copy_(0, gather, x1c)
+            attn_tokens = attn_tokens.view(batch, token_count, width)
+        ctx.save_for_backward(xc, qkv, attended, lse, x1c, key_lengths, attn_norm_w, w_qkv, w_out, ffn_norm_w, w_up, w_down,
+                              *(t for t in (b_up,) if t is not None))
+        ctx.index = (rows, count, valid, gather, identity)
+        ctx.config = (batch, token_count, width, int(num_heads), float(attn_eps), float(ffn_eps), bool(gate_first),
+                      b_qkv is not None, b_out is not None, b_up is not None, b_down is not None)
+        ctx.set_materialize_grads(False)
+        return output.view(batch, token_count, width), attn_tokens
+
+    @staticmethod
+    def backward(ctx, grad_output, grad_attn_tokens):
+        (xc, qkv, attended, lse, x1c, key_lengths, attn_norm_w, w_qkv, w_out, ffn_norm_w, w_up, w_down, *rest) = ctx.saved_tensors
+        (batch, token_count, width, num_heads, attn_eps, ffn_eps, gate_first, has_b_qkv, has_b_out, has_b_up,
+         has_b_down) = ctx.config
+        b_up = rest[0] if has_b_up else None
+        rows, count, valid, gather, identity = ctx.index
+        total = batch * token_count
+        dtype, device = xc.dtype, xc.device
+
+        def flat_grad(g):
+            g = g.reshape(total, width)
+            return g if g.dtype == dtype and g.is_contiguous() else g.to(dtype).contiguous()
+
+        grad_tokens = None
+        grad_x1c = None
+        if grad_attn_tokens is not None:       # the caller used attn_tokens: identity on padded rows, x1 on valid ones
+            g_attn = flat_grad(grad_attn_tokens)
+            grad_tokens = g_attn.clone()
+            grad_x1c = g_attn.index_select(0, gather)
+        weight_grads = dict.fromkeys(("up", "b_up", "down", "b_down", "ffn_norm"))
+        if grad_output is not None:
+            g_out = flat_grad(grad_output)
+            grad_tokens = g_out.clone() if grad_tokens is None else grad_tokens.add_(g_out)
+            gc = g_out.index_select(0, gather)                                           # [valid, D]
+            # ---- feed-forward half ---------------------------------------------------------------------------------------
+            h2 = hip_rms_norm_kernel(x1c, ffn_norm_w, ffn_eps)
+            hidden, grad_pre = _linear.swiglu_ffn_backward_hidden(h2, gc, w_up, b_up, w_down, gate_first=gate_first)
+            weight_grads["down"], weight_grads["b_down"] = _linear.linear_wgrad(gc, hidden, with_bias=has_b_down)
+            weight_grads["up"], weight_grads["b_up"] = _linear.linear_wgrad(grad_pre, h2, with_bias=has_b_up)
+            grad_h2 = _linear._input_grad(grad_pre, w_up)
+            del hidden, grad_pre
+            grad_x1_norm, weight_grads["ffn_norm"] = hip_rms_norm_backward_kernel(x1c, ffn_norm_w, grad_h2, ffn_eps)
+            grad_x1c = gc.add_(grad_x1_norm) if grad_x1c is None else grad_x1c.add_(gc).add_(grad_x1_norm)
+        if grad_x1c is None:
+            return (None,) * 17
+        # ---- out projection: weight gradient on compact rows, input gradient written into the padded layout ------------
+        attended_c = attended.index_select(0, gather)
+        grad_w_out, grad_b_out = _linear.linear_wgrad(grad_x1c, attended_c, with_bias=has_b_out)
+        del attended_c
+        grad_attended = torch.zeros(total, width, dtype=dtype, device=device)
+        _indexed_linear(grad_x1c, w_out.t().contiguous(), None, grad_attended, tokens=valid, out_rows=rows, count=count,
+                        x_rows=identity, cache_weight=False)
+        # ---- attention: the gradient of the packed q | k | v projection in place ---------------------------------------------
+        grad_qkv = torch.empty(total, 3 * width, dtype=dtype, device=device)
+        delta = torch.empty_like(lse)
+        library = _native.load_library()
+        qkv_strides = _attention_strides(width, num_heads, 3 * width, token_count)
+        out_strides = _attention_strides(width, num_heads, width, token_count)
+        element = qkv.element_size()
+        q_ptr, g_ptr = qkv.data_ptr(), grad_qkv.data_ptr()
+        status = library.taac_flash_attn_bwd(
+            q_ptr, q_ptr + width * element, q_ptr + 2 * width * element, attended.data_ptr(), grad_attended.data_ptr(),
+            lse.data_ptr(), key_lengths.data_ptr(), g_ptr, g_ptr + width * element, g_ptr + 2 * width * element,
+            delta.data_ptr(), batch, num_heads, token_count, token_count, width // num_heads, qkv_strides, qkv_strides,
+            qkv_strides, out_strides, out_strides, qkv_strides, qkv_strides, qkv_strides, 0, 1, _native.dtype_code(dtype),
+            _native.current_stream(device))
+        _native.check(status, "interaction block (training): attention backward")
+        grad_qkv_c = grad_qkv.index_select(0, gather)                                    # [valid, 3D]
+        del grad_qkv, grad_attended
+        # ---- q | k | v projection and its norm ------------------------------------------------------------------------------
+        h1 = hip_rms_norm_kernel(xc, attn_norm_w, attn_eps)
+        grad_w_qkv, grad_b_qkv = _linear.linear_wgrad(grad_qkv_c, h1, with_bias=has_b_qkv)
+        grad_h1 = _linear._input_grad(grad_qkv_c, w_qkv)
+        grad_xc_norm, grad_attn_norm = hip_rms_norm_backward_kernel(xc, attn_norm_w, grad_h1, attn_eps)
+        grad_xc = grad_x1c.add_(grad_xc_norm)
+        grad_tokens.index_copy_(0, gather, grad_xc)
+        return (grad_tokens.view(batch, token_count, width), None, None, None, None, None, None, grad_attn_norm, grad_w_qkv,
+                grad_b_qkv, grad_w_out, grad_b_out, weight_grads["ffn_norm"], weight_grads["up"], weight_grads["b_up"],
+                weight_grads["down"], weight_grads["b_down"])
+
+
+def training_route_applies(block, tokens: torch.Tensor, attention_mask, key_lengths) -> bool:
+    """Whether :class:`InteractionBlockFunction` covers this call of ``block`` (a ``UnifiedInteractionBlock``)."""
+    if attention_mask is not None or key_lengths is None:
+        return False
+    if not (tokens.is_cuda and tokens.dtype == torch.bfloat16 and tokens.ndim == 3 and tokens.shape[-1] in (128, 256)):
+        return False
+    attention, ffn = block.attention, block.ffn
+    width = tokens.shape[-1]
+    head_dim = width // attention.num_heads
+    if attention.query_norm is not None or attention.rope_base is not None or head_dim not in (32, 64) or width % attention.num_heads:
+        return False
+    if ffn.down.weight.shape[1] % 32 != 0:
+        return False
+    if block.training and (attention.dropout > 0.0 or ffn.dropout.p > 0.0):
+        return False
+    if key_lengths.dtype != torch.int32 or not key_lengths.is_cuda or not key_lengths.is_contiguous():
+        return False
+    return all(p.dtype == torch.bfloat16 and p.is_cuda for p in block.parameters())
+
+
+def run_training_block(block, tokens: torch.Tensor, key_lengths: torch.Tensor, return_attention_tokens: bool):
+    """The block through :class:`InteractionBlockFunction`; None when no token is valid (nothing to compact)."""
+    if _RowIndex.get(key_lengths, tokens.shape[1])[2] == 0:
+        return None
+    attention, ffn = block.attention, block.ffn
+    return InteractionBlockFunction.apply(
+        tokens, key_lengths, bool(return_attention_tokens), attention.num_heads, block.attn_norm.eps, block.ffn_norm.eps,
+        ffn.gate_first, block.attn_norm.weight, attention.qkv.weight, attention.qkv.bias, attention.out.weight,
+        attention.out.bias, block.ffn_norm.weight, ffn.up.weight, ffn.up.bias, ffn.down.weight, ffn.down.bias)

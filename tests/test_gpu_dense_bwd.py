@@ -231,3 +231,52 @@ def test_interaction_block_takes_a_gradient_end_to_end(device):
     for name, parameter_name in lookup.items():
         assert named[parameter_name].grad is not None, parameter_name
         _close(named[parameter_name].grad, reference[name].grad)
+
+
+@pytest.mark.parametrize("d_model,heads,mult,use_attn_tokens", [(256, 8, 4, False), (256, 4, 2, True), (128, 4, 2, True)])
+def test_block_training_route_over_the_valid_rows_equals_the_layer_by_layer_route(device, monkeypatch, d_model, heads, mult,
+                                                                                 use_attn_tokens):
+    """The one-function training route (valid rows compacted, gradients of the packed projection written in place)
+    against the layer-by-layer autograd route of the same module: outputs, input gradient and every parameter gradient,
+    with a sample of length zero, a full one, and a loss that also uses the block's second output."""
+    import taac_2026_amd.modeling.backbone as backbone_module
+
+    batch, tokens = 6, 96
+    g = torch.Generator().manual_seed(d_model + heads)
+    block = UnifiedInteractionBlock(d_model, heads, mult, qk_norm=False)
+    with torch.no_grad():
+        for parameter in block.parameters():
+            if parameter.ndim == 1:
+                parameter.copy_((1.0 if parameter.shape[0] == d_model and parameter.mean() > 0.5 else 0.0)
+                                + 0.1 * torch.randn(parameter.shape, generator=g))
+            else:
+                parameter.copy_(torch.randn(parameter.shape, generator=g) * parameter.shape[1] ** -0.5)
+    block = block.to(torch.bfloat16).to(device).train()
+    x = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16).to(device)
+    lengths = torch.tensor([96, 0, 33, 1, 64, 17], dtype=torch.int32, device=device)
+    padding = torch.arange(tokens, device=device)[None, :] >= lengths[:, None]
+    grad_out = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16).to(device)
+    grad_attn = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16).to(device)
+
+    def run(compact: bool):
+        if not compact:
+            monkeypatch.setattr(backbone_module, "training_route_applies", lambda *a, **k: False)
+        xd = x.clone().requires_grad_(True)
+        block.zero_grad(set_to_none=True)
+        out, attn_tokens = block(xd, padding, None, key_lengths=lengths)
+        loss_grads = [grad_out] + ([grad_attn] if use_attn_tokens else [])
+        torch.autograd.backward([out] + ([attn_tokens] if use_attn_tokens else []), loss_grads)
+        monkeypatch.undo()
+        return out.detach(), attn_tokens.detach(), xd.grad, {n: p.grad.clone() for n, p in block.named_parameters()}
+
+    out_c, attn_c, gx_c, grads_c = run(True)
+    out_s, attn_s, gx_s, grads_s = run(False)
+    _close(out_c, out_s.cpu(), 1e-2)
+    _close(attn_c, attn_s.cpu(), 1e-2)
+    valid = ~padding.cpu()
+    assert torch.equal(out_c.cpu()[~valid], x.cpu()[~valid]) and torch.equal(attn_c.cpu()[~valid], x.cpu()[~valid])
+    _close(gx_c, gx_s.cpu(), 2e-2)
+    expected_padded = (grad_out + grad_attn if use_attn_tokens else grad_out).cpu()
+    assert torch.equal(gx_c.cpu()[~valid], expected_padded[~valid])             # padded positions: identity
+    for name in grads_s:
+        _close(grads_c[name], grads_s[name].cpu(), 2e-2)
