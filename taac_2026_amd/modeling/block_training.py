@@ -28,34 +28,43 @@ from taac_2026_amd.accelerators.normalization import hip_rms_norm_backward_kerne
 
 
 class _RowIndex:
-    """Valid-row index of the last ``key_lengths`` tensor seen: ``rows`` (int32, :func:`valid_rows`), ``count`` (device
-    scalar), ``valid`` (the same number on the host), ``gather`` (int64 ``rows[:valid]`` for torch's index kernels) and
-    ``identity`` (int32 ``0..valid-1``: the row numbers of a compact tensor)."""
+    """Valid-row index of a ``key_lengths`` tensor: ``rows`` (int32, :func:`valid_rows`) and ``count`` (device scalar) at
+    once; ``compact()`` adds what the backward needs and what costs the host synchronisation: ``valid`` (the count on the
+    host), ``gather`` (int64 ``rows[:valid]`` for torch's index kernels) and ``identity`` (int32 ``0..valid-1``: the row
+    numbers of a compact tensor). The index of the last tensor seen is kept, so the blocks of a stack share it."""
 
     _last: tuple | None = None
 
+    def __init__(self, key_lengths: torch.Tensor, tokens: int) -> None:
+        self.rows, self.count = _linear.valid_rows(key_lengths, tokens)
+        self.valid: int | None = None
+        self.gather = self.identity = None
+
+    def compact(self) -> "_RowIndex":
+        if self.valid is None:
+            self.valid = int(self.count.item())
+            self.gather = self.rows[: self.valid].to(torch.int64)
+            self.identity = torch.arange(max(self.valid, 1), dtype=torch.int32, device=self.rows.device)
+        return self
+
     @classmethod
-    def get(cls, key_lengths: torch.Tensor, tokens: int):
+    def get(cls, key_lengths: torch.Tensor, tokens: int) -> "_RowIndex":
         stamp = cls._last
         if stamp is not None:
             ref, version, pointer, width, entry = stamp
             if ref() is key_lengths and version == key_lengths._version and pointer == key_lengths.data_ptr() and width == tokens:
                 return entry
-        rows, count = _linear.valid_rows(key_lengths, tokens)
-        valid = int(count.item())
-        gather = rows[:valid].to(torch.int64)
-        identity = torch.arange(max(valid, 1), dtype=torch.int32, device=rows.device)
-        entry = (rows, count, valid, gather, identity)
+        entry = cls(key_lengths, tokens)
         cls._last = (weakref.ref(key_lengths), key_lengths._version, key_lengths.data_ptr(), tokens, entry)
         return entry
 
 
 def _indexed_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor, *, tokens: int,
-                    out_rows: torch.Tensor, count: torch.Tensor, x_rows: torch.Tensor, norm_weight: torch.Tensor | None = None,
+                    out_rows: torch.Tensor, count: torch.Tensor, x_rows: torch.Tensor | None, norm_weight: torch.Tensor | None = None,
                     eps: float = 1e-6, residual: torch.Tensor | None = None, cache_weight: bool = True) -> None:
-    """``out[out_rows[i]] = residual[out_rows[i]] + linear(rmsnorm(x[x_rows[i]]))`` for ``i < tokens``
-    (``taac_norm_linear_fwd`` with both of its row indices): the projection that crosses between the compact and the padded
-    layout."""
+    """``out[out_rows[i]] = residual[out_rows[i]] + linear(rmsnorm(x[x_rows[i]]))`` for ``i < min(tokens, count)``
+    (``taac_norm_linear_fwd`` with its row indices; ``x_rows`` None: the rows of ``x`` are ``out_rows`` too): a projection
+    over the valid rows of the padded layout, or one that crosses between the compact and the padded layout."""
     out_features, in_features = weight.shape
     pack = lambda: _linear.pack_linear_weight(weight)  # noqa: E731
     packed = _linear._packed_cache.get((weight,), pack) if cache_weight else pack()
@@ -63,7 +72,7 @@ def _indexed_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | 
     status = library.taac_norm_linear_fwd(
         x.data_ptr(), x.stride(0), _native.ptr(norm_weight), float(eps), None, _native.ptr(bias), packed.data_ptr(),
         _native.ptr(residual), residual.stride(0) if residual is not None else out_features, out.data_ptr(), out.stride(0),
-        tokens, out_features, in_features, out_rows.data_ptr(), count.data_ptr(), x_rows.data_ptr(),
+        tokens, out_features, in_features, out_rows.data_ptr(), count.data_ptr(), _native.ptr(x_rows),
         _native.current_stream(x.device))
     _native.check(status, "interaction block (training): projection")
 
@@ -83,17 +92,17 @@ class InteractionBlockFunction(torch.autograd.Function):
                 b_qkv, w_out, b_out, ffn_norm_w, w_up, b_up, w_down, b_down):
         batch, token_count, width = tokens.shape
         total = batch * token_count
-        rows, count, valid, gather, identity = _RowIndex.get(key_lengths, token_count)
+        index = _RowIndex.get(key_lengths, token_count)
+        rows, count = index.rows, index.count
         flat = tokens.detach().reshape(total, width)
         if not flat.is_contiguous():
             flat = flat.contiguous()
         library = _native.load_library()
-        stream = _native.current_stream(tokens.device)
-        xc = flat.index_select(0, gather)                                               # [valid, D]
-        qkv = torch.empty(total, 3 * width, dtype=flat.dtype, device=flat.device)      # padded layout; padded rows unused
-        _indexed_linear(xc, w_qkv, b_qkv, qkv, tokens=valid, out_rows=rows, count=count, x_rows=identity,
+        # q | k | v of the valid rows, in the padded layout (the attention kernel never reads a padded key or query row)
+        qkv = torch.empty(total, 3 * width, dtype=flat.dtype, device=flat.device)
+        _indexed_linear(flat, w_qkv, b_qkv, qkv, tokens=total, out_rows=rows, count=count, x_rows=None,
                         norm_weight=attn_norm_w, eps=attn_eps)
-        attended = torch.zeros(total, width, dtype=flat.dtype, device=flat.device)
+        attended = torch.empty(total, width, dtype=flat.dtype, device=flat.device)
         lse = torch.empty(batch, num_heads, token_count, dtype=torch.float32, device=flat.device)
         qkv_strides = _attention_strides(width, num_heads, 3 * width, token_count)
         out_strides = _attention_strides(width, num_heads, width, token_count)
@@ -101,36 +110,56 @@ class InteractionBlockFunction(torch.autograd.Function):
         status = library.taac_flash_attn_train_fwd(
             qkv.data_ptr(), qkv.data_ptr() + width * element, qkv.data_ptr() + 2 * width * element, key_lengths.data_ptr(),
             attended.data_ptr(), lse.data_ptr(), batch, num_heads, token_count, token_count, width // num_heads,
-            qkv_strides, qkv_strides, qkv_strides, out_strides, 0, 1, _native.dtype_code(flat.dtype), stream)
+            qkv_strides, qkv_strides, qkv_strides, out_strides, 0, 1, _native.dtype_code(flat.dtype),
+            _native.current_stream(tokens.device))
         _native.check(status, "interaction block (training): attention")
-        x1c = torch.empty(valid, width, dtype=flat.dtype, device=flat.device)
-        _indexed_linear(attended, w_out, b_out, x1c, tokens=valid, out_rows=identity, count=count, x_rows=rows, residual=xc)
-        yc = _linear.swiglu_ffn(x1c, w_up, b_up, w_down, b_down, residual=x1c, gate_first=gate_first,
-                                norm_weight=ffn_norm_w, eps=ffn_eps)
-        output = flat.clone()
-        output.index_copy_(0, gather, yc)
+        # Second half on the valid rows of copies of the stream (padded rows pass through): one kernel when the caller
+        # does not want the tokens between the halves, two otherwise.
         attn_tokens = None
-        if want_attn_tokens:
+        if want_attn_tokens or not gate_first:
             attn_tokens = flat.clone()
-            attn_tokens.index_copy_(0, gather, x1c)
-            attn_tokens = attn_tokens.view(batch, token_count, width)
-        ctx.save_for_backward(xc, qkv, attended, lse, x1c, key_lengths, attn_norm_w, w_qkv, w_out, ffn_norm_w, w_up, w_down,
-                              *(t for t in (b_up,) if t is not None))
-        ctx.index = (rows, count, valid, gather, identity)
+            _indexed_linear(attended, w_out, b_out, attn_tokens, tokens=total, out_rows=rows, count=count, x_rows=None,
+                            residual=flat)
+            output = attn_tokens.clone()
+            _linear.swiglu_ffn(attn_tokens, w_up, b_up, w_down, b_down, residual=attn_tokens, gate_first=gate_first,
+                               norm_weight=ffn_norm_w, eps=ffn_eps, token_rows=(rows, count), out=output)
+        else:
+            output = flat.clone()
+            _linear.attention_out_ffn(attended, w_out, b_out, flat, w_up, b_up, w_down, b_down, norm_weight=ffn_norm_w,
+                                      eps=ffn_eps, token_rows=(rows, count), out=output)
+        ctx.save_for_backward(flat, qkv, attended, lse, key_lengths, attn_norm_w, w_qkv, w_out, ffn_norm_w, w_up, w_down,
+                              *(t for t in (b_out, b_up, attn_tokens) if t is not None))
+        ctx.index = index
         ctx.config = (batch, token_count, width, int(num_heads), float(attn_eps), float(ffn_eps), bool(gate_first),
-                      b_qkv is not None, b_out is not None, b_up is not None, b_down is not None)
+                      b_qkv is not None, b_out is not None, b_up is not None, b_down is not None, attn_tokens is not None)
         ctx.set_materialize_grads(False)
+        if attn_tokens is not None:
+            attn_tokens = attn_tokens.view(batch, token_count, width) if want_attn_tokens else None
         return output.view(batch, token_count, width), attn_tokens
 
     @staticmethod
     def backward(ctx, grad_output, grad_attn_tokens):
-        (xc, qkv, attended, lse, x1c, key_lengths, attn_norm_w, w_qkv, w_out, ffn_norm_w, w_up, w_down, *rest) = ctx.saved_tensors
-        (batch, token_count, width, num_heads, attn_eps, ffn_eps, gate_first, has_b_qkv, has_b_out, has_b_up,
-         has_b_down) = ctx.config
-        b_up = rest[0] if has_b_up else None
-        rows, count, valid, gather, identity = ctx.index
+        (flat, qkv, attended, lse, key_lengths, attn_norm_w, w_qkv, w_out, ffn_norm_w, w_up, w_down, *rest) = ctx.saved_tensors
+        (batch, token_count, width, num_heads, attn_eps, ffn_eps, gate_first, has_b_qkv, has_b_out, has_b_up, has_b_down,
+         has_attn_tokens) = ctx.config
+        rest = list(rest)
+        b_out = rest.pop(0) if has_b_out else None
+        b_up = rest.pop(0) if has_b_up else None
+        index = ctx.index.compact()
+        rows, count, valid, gather, identity = index.rows, index.count, index.valid, index.gather, index.identity
         total = batch * token_count
-        dtype, device = xc.dtype, xc.device
+        dtype, device = flat.dtype, flat.device
+        if valid == 0:                              # no valid token: the block is the identity
+            grads = [g for g in (grad_output, grad_attn_tokens) if g is not None]
+            return (sum(grads[1:], grads[0]) if grads else None,) + (None,) * 16
+        # the compact rows of the stream and of the tokens between the halves (gathered, or recomputed from the attention
+        # output when the forward ran the one-kernel second half)
+        xc = flat.index_select(0, gather)
+        if has_attn_tokens:
+            x1c = rest.pop(0).index_select(0, gather)
+        else:
+            x1c = torch.empty(valid, width, dtype=dtype, device=device)
+            _indexed_linear(attended, w_out, b_out, x1c, tokens=valid, out_rows=identity, count=count, x_rows=rows, residual=xc)
 
         def flat_grad(g):
             g = g.reshape(total, width)
@@ -215,9 +244,7 @@ def training_route_applies(block, tokens: torch.Tensor, attention_mask, key_leng
 
 
 def run_training_block(block, tokens: torch.Tensor, key_lengths: torch.Tensor, return_attention_tokens: bool):
-    """The block through :class:`InteractionBlockFunction`; None when no token is valid (nothing to compact)."""
-    if _RowIndex.get(key_lengths, tokens.shape[1])[2] == 0:
-        return None
+    """The block through :class:`InteractionBlockFunction`."""
     attention, ffn = block.attention, block.ffn
     return InteractionBlockFunction.apply(
         tokens, key_lengths, bool(return_attention_tokens), attention.num_heads, block.attn_norm.eps, block.ffn_norm.eps,
