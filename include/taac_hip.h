@@ -326,7 +326,7 @@ int taac_swiglu_bwd(const void* gu, int64_t ldgu, const void* dhidden, int64_t l
 
 /*
  * The activation part of the feed-forward backward in one kernel (model width D = 128 / 256, F a multiple of 32):
- *   pre = bf16(h w_up^T + b_up), dhidden = bf16(dy w_down)   -- recomputed in registers, never written --
+ *   pre = h w_up^T + b_up, dhidden = dy w_down               -- recomputed in fp32 registers, never written --
  *   hidden [M, F] = act(pre), grad_pre [M, 2F] = d act / d pre * dhidden      (formulas of taac_swiglu_bwd)
  * h: [M, D] input of the up projection (the normalised rows), dy: [M, D] gradient of the feed-forward output; both bf16.
  * packed: the blob written by taac_swiglu_ffn_bwd_pack_weights for (w_up [2F, D], w_down [D, F]),

@@ -75,7 +75,8 @@ def test_silu_gate_backward(device, gate_first):
 def test_feed_forward_backward_hidden_kernel(device, m, d, f, gate_first, with_bias):
     """The one-kernel activation backward (up projection and ``dy @ w_down`` recomputed in registers) against float64
     autograd of the same expression, and against the three-kernel route it replaces (equal up to the roundings of
-    bfloat16: that route rounds the same intermediate values)."""
+    bfloat16: that route rounds the up projection and ``dy @ w_down`` to bfloat16 on the way, the kernel keeps them in
+    float32)."""
     g = torch.Generator().manual_seed(m + f)
     bf = lambda t: t.to(torch.bfloat16)  # noqa: E731
     h = bf(torch.randn(m, d, generator=g))
