@@ -249,6 +249,7 @@ def _operator_figures(device, iters: int) -> dict:
         }
     del qd, kd, vd
     figures.update(_attention_bwd_figures(device, iters))
+    figures.update(_training_block_figures(device))
     return figures
 
 
@@ -279,6 +280,40 @@ def _attention_bwd_figures(device, iters: int) -> dict:
         }
         del qg, kg, vg, go
     return figures
+
+
+def _training_block_figures(device) -> dict:
+    """One training step (forward + backward, every parameter and the input taking a gradient) of a
+    ``UnifiedInteractionBlock`` at the headline shape: the one-function route over the valid rows, and the layer-by-layer
+    autograd route of the same module over all positions for comparison."""
+    import taac_2026_amd.modeling.backbone as backbone_module
+    from taac_2026_amd import workloads
+    from taac_2026_amd.api import UnifiedInteractionBlock
+
+    inputs = workloads.backbone_inputs(batch=1024)
+    batch, tokens, width = inputs.emb.shape
+    torch.manual_seed(0)
+    block = UnifiedInteractionBlock(width, inputs.num_heads, 4, qk_norm=False).to(torch.bfloat16).to(device).train()
+    x = inputs.emb.to(device).requires_grad_(True)
+    lengths = inputs.key_lengths.to(device)
+    padding = torch.arange(tokens, device=device)[None, :] >= lengths[:, None]
+    grad = torch.randn(batch, tokens, width, device=device).to(torch.bfloat16)
+
+    def step():
+        out, _ = block(x, padding, None, key_lengths=lengths, return_attention_tokens=False)
+        out.backward(grad)
+        block.zero_grad(set_to_none=True)
+        x.grad = None
+
+    figures = {"valid_rows_ms": _event_ms(step, 5, 3)}
+    applies = backbone_module.training_route_applies
+    backbone_module.training_route_applies = lambda *a, **k: False
+    try:
+        figures["layer_by_layer_ms"] = _event_ms(step, 3, 2)
+    finally:
+        backbone_module.training_route_applies = applies
+    figures["valid_token_fraction"] = float(lengths.sum().item()) / (batch * tokens)
+    return {"interaction_block_training_step_B1024_T512": figures}
 
 
 def _embedding_figures(device, iters: int) -> dict:

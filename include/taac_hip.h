@@ -483,6 +483,17 @@ int taac_candidate_readout_fwd(const void* tokens, const int32_t* key_lengths, c
 int taac_valid_rows(const int32_t* key_lengths, int32_t B, int32_t T, int32_t* rows, int32_t* n_rows, void* stream);
 
 /*
+ * Merge of a padded and a compact layout (bf16 rows of W elements, W a multiple of 8): row (b, t) of out [B * T, W] is
+ * compact_a[offsets[b] + t] (+ compact_b of the same row when compact_b is not NULL; fp32 add, one rounding) for
+ * t < key_lengths[b], and the row of `padded` otherwise. offsets: the per-sample offsets taac_valid_rows writes behind
+ * its row index (rows + B * T). out may be `padded`.
+ * Replaces: the scatter of a valid-row gradient (or output) into the padded token stream that
+ * `update * ~padding_mask` + residual adds amount to in UnifiedInteractionBlock (experiments/symbiosis/backbone.py:58-68).
+ */
+int taac_rows_merge(const void* padded, const void* compact_a, const void* compact_b, const int32_t* key_lengths,
+                    const int32_t* offsets, void* out, int32_t B, int32_t T, int32_t W, void* stream);
+
+/*
  * The same row index for padding that is not a prefix: token t of sample b is valid iff bit t of valid_bits[b] is set
  * (rows of ceil(T / 32) 32-bit words, as written by taac_mask_pack_bits from a [B, T] bool matrix, True = valid).
  * Output layout and sizes as in taac_valid_rows. This is what lets the dense layers honour the reference blocks'

@@ -223,6 +223,59 @@ __global__ __launch_bounds__(kBlock) void zero_padded_rows_kernel(bf16_t* __rest
 }  // namespace
 }  // namespace taac
 
+namespace taac {
+namespace {
+// One 16-byte piece per thread: row (b, t) of out is a[offsets[b] + t] (+ b2 of the same row) when t < lengths[b], else
+// the row of `padded`.
+__global__ __launch_bounds__(kBlock) void rows_merge_kernel(const bf16x8* __restrict__ padded, const bf16x8* __restrict__ a,
+                                                            const bf16x8* __restrict__ b2,
+                                                            const int32_t* __restrict__ lengths,
+                                                            const int32_t* __restrict__ offsets, bf16x8* __restrict__ out,
+                                                            int64_t pieces_total, int T, int pieces) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= pieces_total) return;
+  const int64_t row = idx / pieces;
+  const int c = static_cast<int>(idx % pieces);
+  const int b = static_cast<int>(row / T), t = static_cast<int>(row % T);
+  int32_t len = lengths[b];
+  len = len < 0 ? 0 : (len > T ? T : len);
+  bf16x8 v;
+  if (t < len) {
+    const int64_t src = (static_cast<int64_t>(offsets[b]) + t) * pieces + c;
+    v = a[src];
+    if (b2 != nullptr) {
+      const bf16x8 w = b2[src];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = static_cast<bf16_t>(static_cast<float>(v[e]) + static_cast<float>(w[e]));
+    }
+  } else {
+    v = padded[idx];
+  }
+  out[idx] = v;
+}
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_rows_merge(const void* padded, const void* compact_a, const void* compact_b, const int32_t* key_lengths,
+                               const int32_t* offsets, void* out, int32_t B, int32_t T, int32_t W, void* stream) {
+  using namespace taac;
+  const char* name = "taac_rows_merge";
+  if (B < 0 || T < 0 || W <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: bad dimensions", name);
+  if (W % 8 != 0) return set_error(TAAC_ERR_UNSUPPORTED, "%s: W=%d must be a multiple of 8", name, W);
+  if (B == 0 || T == 0) return TAAC_OK;
+  if (!padded || !compact_a || !key_lengths || !offsets || !out) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  if (!aligned16(padded) || !aligned16(compact_a) || !aligned16(compact_b) || !aligned16(out))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
+  const int64_t pieces_total = static_cast<int64_t>(B) * T * (W / 8);
+  const int64_t blocks = (pieces_total + kBlock - 1) / kBlock;
+  if (blocks > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many workgroups", name);
+  hipLaunchKernelGGL(rows_merge_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, as_stream(stream),
+                     static_cast<const bf16x8*>(padded), static_cast<const bf16x8*>(compact_a),
+                     static_cast<const bf16x8*>(compact_b), key_lengths, offsets, static_cast<bf16x8*>(out), pieces_total, T,
+                     W / 8);
+  return check_launch(name);
+}
+
 extern "C" int taac_valid_rows(const int32_t* key_lengths, int32_t B, int32_t T, int32_t* rows, int32_t* n_rows,
                                void* stream) {
   using namespace taac;

@@ -165,16 +165,16 @@ class InteractionBlockFunction(torch.autograd.Function):
             g = g.reshape(total, width)
             return g if g.dtype == dtype and g.is_contiguous() else g.to(dtype).contiguous()
 
-        grad_tokens = None
+        # gradient arriving at the padded rows (they pass through the block) and, gathered, at the valid ones
+        grad_padded = None
         grad_x1c = None
         if grad_attn_tokens is not None:       # the caller used attn_tokens: identity on padded rows, x1 on valid ones
-            g_attn = flat_grad(grad_attn_tokens)
-            grad_tokens = g_attn.clone()
-            grad_x1c = g_attn.index_select(0, gather)
+            grad_padded = flat_grad(grad_attn_tokens)
+            grad_x1c = grad_padded.index_select(0, gather)
         weight_grads = dict.fromkeys(("up", "b_up", "down", "b_down", "ffn_norm"))
         if grad_output is not None:
             g_out = flat_grad(grad_output)
-            grad_tokens = g_out.clone() if grad_tokens is None else grad_tokens.add_(g_out)
+            grad_padded = g_out if grad_padded is None else grad_padded + g_out
             gc = g_out.index_select(0, gather)                                           # [valid, D]
             # ---- feed-forward half ---------------------------------------------------------------------------------------
             h2 = hip_rms_norm_kernel(x1c, ffn_norm_w, ffn_eps)
@@ -216,8 +216,12 @@ class InteractionBlockFunction(torch.autograd.Function):
         grad_w_qkv, grad_b_qkv = _linear.linear_wgrad(grad_qkv_c, h1, with_bias=has_b_qkv)
         grad_h1 = _linear._input_grad(grad_qkv_c, w_qkv)
         grad_xc_norm, grad_attn_norm = hip_rms_norm_backward_kernel(xc, attn_norm_w, grad_h1, attn_eps)
-        grad_xc = grad_x1c.add_(grad_xc_norm)
-        grad_tokens.index_copy_(0, gather, grad_xc)
+        # valid rows: the gradient of the tokens between the halves + that of the norm's input; padded rows: what arrived
+        grad_tokens = torch.empty(total, width, dtype=dtype, device=device)
+        status = library.taac_rows_merge(grad_padded.data_ptr(), grad_x1c.data_ptr(), grad_xc_norm.data_ptr(),
+                                         key_lengths.data_ptr(), rows.data_ptr() + 4 * total, grad_tokens.data_ptr(), batch,
+                                         token_count, width, _native.current_stream(device))
+        _native.check(status, "interaction block (training): gradient merge")
         return (grad_tokens.view(batch, token_count, width), None, None, None, None, None, None, grad_attn_norm, grad_w_qkv,
                 grad_b_qkv, grad_w_out, grad_b_out, weight_grads["ffn_norm"], weight_grads["up"], weight_grads["b_up"],
                 weight_grads["down"], weight_grads["b_down"])
