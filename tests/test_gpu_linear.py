@@ -46,6 +46,23 @@ def test_linear_matches_oracle(device, m, n, k, use_bias):
     torch.testing.assert_close(got.cpu().float(), F.linear(x, w, bias).float(), **BF16_TOL)
 
 
+@pytest.mark.parametrize("m,n,k", [(1024, 256, 512), (1500, 256, 2048), (1025, 136, 520), (4096, 192, 768)])
+@pytest.mark.parametrize("epilogue", ["none", "bias", "residual"])
+def test_linear_long_contraction_into_a_narrow_output(device, m, n, k, epilogue):
+    """Shapes served by the 256-token x all-features kernel (128 < N <= 256, K >= 512, M >= 1024): ragged token, feature
+    and contraction tails, bias and residual epilogues."""
+    x, w, b = _draw(m, n, k, seed=m + n + k)
+    res = torch.randn(m, n, generator=torch.Generator().manual_seed(k)).to(torch.bfloat16)
+    bias = None if epilogue == "none" else b
+    expected = F.linear(x.float(), w.float(), None if bias is None else bias.float())
+    if epilogue == "residual":
+        expected = expected + res.float()
+    with torch.no_grad():
+        got = linear(x.to(device), w.to(device), None if bias is None else bias.to(device),
+                     residual=res.to(device) if epilogue == "residual" else None)
+    torch.testing.assert_close(got.cpu().float(), expected, **BF16_TOL)
+
+
 def test_linear_residual_and_batch_dims(device):
     x, w, b = _draw(6 * 50, 256, 256, seed=4)
     x3 = x.view(6, 50, 256)
