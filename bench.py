@@ -282,7 +282,7 @@ def _attention_bwd_figures(device, iters: int) -> dict:
     return figures
 
 
-def _training_block_figures(device) -> dict:
+def _training_block_figures(device, with_comparison: bool = True) -> dict:
     """One training step (forward + backward, every parameter and the input taking a gradient) of a
     ``UnifiedInteractionBlock`` at the headline shape: the one-function route over the valid rows, and the layer-by-layer
     autograd route of the same module over all positions for comparison."""
@@ -306,12 +306,13 @@ def _training_block_figures(device) -> dict:
         x.grad = None
 
     figures = {"valid_rows_ms": _event_ms(step, 5, 3)}
-    applies = backbone_module.training_route_applies
-    backbone_module.training_route_applies = lambda *a, **k: False
-    try:
-        figures["layer_by_layer_ms"] = _event_ms(step, 3, 2)
-    finally:
-        backbone_module.training_route_applies = applies
+    if with_comparison:
+        applies = backbone_module.training_route_applies
+        backbone_module.training_route_applies = lambda *a, **k: False
+        try:
+            figures["layer_by_layer_ms"] = _event_ms(step, 3, 2)
+        finally:
+            backbone_module.training_route_applies = applies
     figures["valid_token_fraction"] = float(lengths.sum().item()) / (batch * tokens)
     return {"interaction_block_training_step_B1024_T512": figures}
 
@@ -688,6 +689,9 @@ def main() -> None:
                         help="time only the stand-alone kernels of one block (short run for hardware-counter collection)")
     parser.add_argument("--only-attention-bwd", action="store_true",
                         help="time only the attention backward at its two shapes (short run for traces and counters)")
+    parser.add_argument("--only-training-block", action="store_true",
+                        help="time only one training step of the interaction block, valid-row route and layer-by-layer route "
+                             "(short run for traces)")
     parser.add_argument("--only-fp8", action="store_true",
                         help="time only the FP8 dense layers and the FP8 backbone step (short run for traces and counters)")
     parser.add_argument("--only-reference-block", action="store_true",
@@ -714,6 +718,9 @@ def main() -> None:
         return
     if args.only_attention_bwd:
         print(json.dumps({"attention_bwd": _attention_bwd_figures(device, iters=6)}))
+        return
+    if args.only_training_block:
+        print(json.dumps({"training_block": _training_block_figures(device, with_comparison=False)}))
         return
     if args.only_fp8:
         inputs = workloads.backbone_inputs(batch=args.batch)

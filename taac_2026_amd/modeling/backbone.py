@@ -3,8 +3,10 @@
 ``SwiGLUFeedForward`` / ``UnifiedSelfAttention`` / ``BFTSAttention`` / ``UnifiedInteractionBlock`` keep the constructor signatures,
 parameter names (``up``, ``down``, ``qkv``, ``out``, ``attn_norm`` ...) and forward semantics of
 experiments/symbiosis/backbone.py:11-68 (TokenFormer's feed-forward, experiments/tokenformer/model.py:118-128, is the
-same module), with every dense layer, norm and attention call routed to libtaac_hip.so. They are inference modules:
-dropout probabilities are stored but only the eval-mode behaviour (identity) exists.
+same module), with every dense layer, norm and attention call routed to libtaac_hip.so. Dropout probabilities are stored
+but only the eval-mode behaviour (identity) exists for the feed-forward dropout; tensors that require grad take the
+autograd routes of the operators, and ``UnifiedInteractionBlock`` under prefix padding the one-function training route of
+``block_training``.
 
 ``PCVRBackbone`` is the canonical pre-norm stack + pCVR readout (mean-pool over valid tokens -> Linear(D, 1) ->
 sigmoid) executed by a single ``taac_backbone_fwd`` call.
