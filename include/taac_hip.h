@@ -483,6 +483,13 @@ int taac_candidate_readout_fwd(const void* tokens, const int32_t* key_lengths, c
 int taac_valid_rows(const int32_t* key_lengths, int32_t B, int32_t T, int32_t* rows, int32_t* n_rows, void* stream);
 
 /*
+ * dst[i, 0..W) = src[rows[i], 0..W) for i < n: rows of 16-bit elements (W a multiple of 8; src row stride ld_src elements,
+ * dst contiguous). With the index of taac_valid_rows and n = the number of valid rows it compacts the valid tokens of a
+ * padded [B * T, W] tensor. No counterpart in the reference (torch.index_select in its place).
+ */
+int taac_rows_gather(const void* src, int64_t ld_src, const int32_t* rows, int64_t n, void* dst, int32_t W, void* stream);
+
+/*
  * Merge of a padded and a compact layout (bf16 rows of W elements, W a multiple of 8): row (b, t) of out [B * T, W] is
  * compact_a[offsets[b] + t] (+ compact_b of the same row when compact_b is not NULL; fp32 add, one rounding) for
  * t < key_lengths[b], and the row of `padded` otherwise. offsets: the per-sample offsets taac_valid_rows writes behind

@@ -253,8 +253,37 @@ __global__ __launch_bounds__(kBlock) void rows_merge_kernel(const bf16x8* __rest
   }
   out[idx] = v;
 }
+
+// dst[i] = src[rows[i]] for i < n: one 16-byte piece per thread.
+__global__ __launch_bounds__(kBlock) void rows_gather_kernel(const bf16x8* __restrict__ src, int64_t src_pieces,
+                                                             const int32_t* __restrict__ rows, bf16x8* __restrict__ dst,
+                                                             int64_t pieces_total, int pieces) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= pieces_total) return;
+  const int64_t i = idx / pieces;
+  const int c = static_cast<int>(idx % pieces);
+  dst[idx] = __builtin_nontemporal_load(src + static_cast<int64_t>(rows[i]) * src_pieces + c);
+}
 }  // namespace
 }  // namespace taac
+
+extern "C" int taac_rows_gather(const void* src, int64_t ld_src, const int32_t* rows, int64_t n, void* dst, int32_t W,
+                                void* stream) {
+  using namespace taac;
+  const char* name = "taac_rows_gather";
+  if (n < 0 || W <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: bad dimensions", name);
+  if (W % 8 != 0 || ld_src % 8 != 0 || ld_src < W)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: W and the source row stride must be multiples of 8 and cover a row", name);
+  if (n == 0) return TAAC_OK;
+  if (!src || !rows || !dst) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  if (!aligned16(src) || !aligned16(dst)) return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
+  const int64_t pieces_total = n * (W / 8);
+  const int64_t blocks = (pieces_total + kBlock - 1) / kBlock;
+  if (blocks > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many workgroups", name);
+  hipLaunchKernelGGL(rows_gather_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, as_stream(stream),
+                     static_cast<const bf16x8*>(src), ld_src / 8, rows, static_cast<bf16x8*>(dst), pieces_total, W / 8);
+  return check_launch(name);
+}
 
 extern "C" int taac_rows_merge(const void* padded, const void* compact_a, const void* compact_b, const int32_t* key_lengths,
                                const int32_t* offsets, void* out, int32_t B, int32_t T, int32_t W, void* stream) {

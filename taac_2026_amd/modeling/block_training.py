@@ -30,20 +30,19 @@ from taac_2026_amd.accelerators.normalization import hip_rms_norm_backward_kerne
 class _RowIndex:
     """Valid-row index of a ``key_lengths`` tensor: ``rows`` (int32, :func:`valid_rows`) and ``count`` (device scalar) at
     once; ``compact()`` adds what the backward needs and what costs the host synchronisation: ``valid`` (the count on the
-    host), ``gather`` (int64 ``rows[:valid]`` for torch's index kernels) and ``identity`` (int32 ``0..valid-1``: the row
-    numbers of a compact tensor). The index of the last tensor seen is kept, so the blocks of a stack share it."""
+    host) and ``identity`` (int32 ``0..valid-1``: the row numbers of a compact tensor). The index of the last tensor seen
+    is kept, so the blocks of a stack share it."""
 
     _last: tuple | None = None
 
     def __init__(self, key_lengths: torch.Tensor, tokens: int) -> None:
         self.rows, self.count = _linear.valid_rows(key_lengths, tokens)
         self.valid: int | None = None
-        self.gather = self.identity = None
+        self.identity = None
 
     def compact(self) -> "_RowIndex":
         if self.valid is None:
             self.valid = int(self.count.item())
-            self.gather = self.rows[: self.valid].to(torch.int64)
             self.identity = torch.arange(max(self.valid, 1), dtype=torch.int32, device=self.rows.device)
         return self
 
@@ -75,6 +74,15 @@ def _indexed_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | 
         tokens, out_features, in_features, out_rows.data_ptr(), count.data_ptr(), _native.ptr(x_rows),
         _native.current_stream(x.device))
     _native.check(status, "interaction block (training): projection")
+
+
+def _gather_rows(src: torch.Tensor, index: "_RowIndex") -> torch.Tensor:
+    """The valid rows of a padded ``[B * T, W]`` tensor as a compact ``[valid, W]`` one (``taac_rows_gather``)."""
+    out = torch.empty(index.valid, src.shape[1], dtype=src.dtype, device=src.device)
+    status = _native.load_library().taac_rows_gather(src.data_ptr(), src.stride(0), index.rows.data_ptr(), index.valid,
+                                                     out.data_ptr(), src.shape[1], _native.current_stream(src.device))
+    _native.check(status, "interaction block (training): gather")
+    return out
 
 
 def _attention_strides(width: int, heads: int, row_stride: int, tokens: int):
@@ -146,7 +154,7 @@ class InteractionBlockFunction(torch.autograd.Function):
         b_out = rest.pop(0) if has_b_out else None
         b_up = rest.pop(0) if has_b_up else None
         index = ctx.index.compact()
-        rows, count, valid, gather, identity = index.rows, index.count, index.valid, index.gather, index.identity
+        rows, count, valid, identity = index.rows, index.count, index.valid, index.identity
         total = batch * token_count
         dtype, device = flat.dtype, flat.device
         if valid == 0:                              # no valid token: the block is the identity
@@ -154,9 +162,9 @@ class InteractionBlockFunction(torch.autograd.Function):
             return (sum(grads[1:], grads[0]) if grads else None,) + (None,) * 16
         # the compact rows of the stream and of the tokens between the halves (gathered, or recomputed from the attention
         # output when the forward ran the one-kernel second half)
-        xc = flat.index_select(0, gather)
+        xc = _gather_rows(flat, index)
         if has_attn_tokens:
-            x1c = rest.pop(0).index_select(0, gather)
+            x1c = _gather_rows(rest.pop(0), index)
         else:
             x1c = torch.empty(valid, width, dtype=dtype, device=device)
             _indexed_linear(attended, w_out, b_out, x1c, tokens=valid, out_rows=identity, count=count, x_rows=rows, residual=xc)
@@ -170,12 +178,12 @@ class InteractionBlockFunction(torch.autograd.Function):
         grad_x1c = None
         if grad_attn_tokens is not None:       # the caller used attn_tokens: identity on padded rows, x1 on valid ones
             grad_padded = flat_grad(grad_attn_tokens)
-            grad_x1c = grad_padded.index_select(0, gather)
+            grad_x1c = _gather_rows(grad_padded, index)
         weight_grads = dict.fromkeys(("up", "b_up", "down", "b_down", "ffn_norm"))
         if grad_output is not None:
             g_out = flat_grad(grad_output)
             grad_padded = g_out if grad_padded is None else grad_padded + g_out
-            gc = g_out.index_select(0, gather)                                           # [valid, D]
+            gc = _gather_rows(g_out, index)                                           # [valid, D]
             # ---- feed-forward half ---------------------------------------------------------------------------------------
             h2 = hip_rms_norm_kernel(x1c, ffn_norm_w, ffn_eps)
             hidden, grad_pre = _linear.swiglu_ffn_backward_hidden(h2, gc, w_up, b_up, w_down, gate_first=gate_first)
@@ -188,7 +196,7 @@ class InteractionBlockFunction(torch.autograd.Function):
         if grad_x1c is None:
             return (None,) * 17
         # ---- out projection: weight gradient on compact rows, input gradient written into the padded layout ------------
-        attended_c = attended.index_select(0, gather)
+        attended_c = _gather_rows(attended, index)
         grad_w_out, grad_b_out = _linear.linear_wgrad(grad_x1c, attended_c, with_bias=has_b_out)
         del attended_c
         grad_attended = torch.zeros(total, width, dtype=dtype, device=device)
@@ -209,7 +217,7 @@ class InteractionBlockFunction(torch.autograd.Function):
             qkv_strides, out_strides, out_strides, qkv_strides, qkv_strides, qkv_strides, 0, 1, _native.dtype_code(dtype),
             _native.current_stream(device))
         _native.check(status, "interaction block (training): attention backward")
-        grad_qkv_c = grad_qkv.index_select(0, gather)                                    # [valid, 3D]
+        grad_qkv_c = _gather_rows(grad_qkv, index)                                    # [valid, 3D]
         del grad_qkv, grad_attended
         # ---- q | k | v projection and its norm ------------------------------------------------------------------------------
         h1 = hip_rms_norm_kernel(xc, attn_norm_w, attn_eps)

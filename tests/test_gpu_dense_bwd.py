@@ -281,3 +281,39 @@ def test_block_training_route_over_the_valid_rows_equals_the_layer_by_layer_rout
     assert torch.equal(gx_c.cpu()[~valid], expected_padded[~valid])             # padded positions: identity
     for name in grads_s:
         _close(grads_c[name], grads_s[name].cpu(), 2e-2)
+
+
+def test_rows_gather_and_merge_through_the_c_abi(device):
+    """``taac_rows_gather`` compacts the valid rows of a padded tensor (also out of a column slice), ``taac_rows_merge``
+    puts compact rows (one part, or the rounded sum of two) back between the pass-through rows: bit-exact against
+    indexing, with an empty and a full sample."""
+    from taac_2026_amd import _native
+    from taac_2026_amd.api import valid_rows
+
+    library = _native.load_library()
+    batch, tokens, width = 5, 40, 72
+    g = torch.Generator().manual_seed(3)
+    lengths = torch.tensor([40, 0, 7, 1, 23], dtype=torch.int32, device=device)
+    padded = torch.randn(batch * tokens, 2 * width, generator=g).to(torch.bfloat16).to(device)
+    rows, count = valid_rows(lengths, tokens)
+    valid = int(count.item())
+    index = rows[:valid].long()
+    stream = _native.current_stream(padded.device)
+    source = padded[:, width:]                                                  # row stride 2 * width
+    compact = torch.empty(valid, width, dtype=torch.bfloat16, device=device)
+    _native.check(library.taac_rows_gather(source.data_ptr(), source.stride(0), rows.data_ptr(), valid, compact.data_ptr(),
+                                           width, stream), "gather")
+    assert torch.equal(compact, source[index])
+    a = torch.randn(valid, width, generator=g).to(torch.bfloat16).to(device)
+    b = torch.randn(valid, width, generator=g).to(torch.bfloat16).to(device)
+    base = padded[:, :width].contiguous()
+    for second in (None, b):
+        out = torch.empty_like(base)
+        _native.check(library.taac_rows_merge(base.data_ptr(), a.data_ptr(), _native.ptr(second), lengths.data_ptr(),
+                                              rows.data_ptr() + 4 * batch * tokens, out.data_ptr(), batch, tokens, width,
+                                              stream), "merge")
+        expected = base.clone()
+        expected[index] = a if second is None else (a.float() + b.float()).to(torch.bfloat16)
+        assert torch.equal(out, expected)
+    assert library.taac_rows_gather(source.data_ptr(), source.stride(0), rows.data_ptr(), valid, compact.data_ptr(), 12,
+                                    stream) == _native.TAAC_ERR_UNSUPPORTED
