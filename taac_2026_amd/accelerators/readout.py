@@ -10,7 +10,41 @@ from __future__ import annotations
 import torch
 
 from taac_2026_amd import _native
-from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference
+from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors
+
+
+def _candidate_readout_training(tokens, cls_index, candidate_index, key_lengths, padding_mask, token_norm_weight,
+                                pool_norm_weight, eps, classifier, sigmoid, return_embedding):
+    """The readout for tensors that take a gradient: the same expression from differentiable pieces - the HIP RMSNorm
+    (forward and backward kernels) over the tokens and over the pooled vector, torch for the masked mean and for the
+    classifier's two small products (``CandidateClsPooler.forward``, experiments/symbiosis/pooling.py:24-32, and the
+    classifier of experiments/symbiosis/model.py:215-222, as the reference evaluates them under autograd)."""
+    from taac_2026_amd.accelerators.normalization import rms_norm
+
+    batch, token_count, _ = tokens.shape
+    x = tokens if token_norm_weight is None else rms_norm(tokens, token_norm_weight, eps)
+    if padding_mask is not None:
+        keep = ~padding_mask
+    elif key_lengths is not None:
+        keep = torch.arange(token_count, device=tokens.device)[None, :] < key_lengths[:, None]
+    else:
+        keep = torch.ones(batch, token_count, dtype=torch.bool, device=tokens.device)
+    weights = keep.to(torch.float32)
+    counts = weights.sum(dim=1, keepdim=True).clamp_min(1.0)
+    mean = torch.einsum("btd,bt->bd", x.float(), weights / counts).to(x.dtype)      # masked mean, fp32 accumulation
+    cls_summary = x[:, cls_index, :]
+    candidate_summary = x[:, candidate_index, :] if candidate_index is not None else torch.zeros_like(cls_summary)
+    pooled = torch.cat([cls_summary, candidate_summary, mean], dim=-1)
+    if pool_norm_weight is not None:
+        pooled = rms_norm(pooled, pool_norm_weight, eps)
+    if classifier is None:
+        return pooled
+    fc1_weight, fc1_bias, fc2_weight, fc2_bias = classifier
+    hidden = torch.nn.functional.silu(torch.nn.functional.linear(pooled, fc1_weight, fc1_bias))
+    logits = torch.nn.functional.linear(hidden, fc2_weight, fc2_bias).float()
+    if sigmoid:
+        logits = torch.sigmoid(logits)
+    return (logits, pooled) if return_embedding else logits
 
 
 def candidate_readout(
@@ -36,12 +70,12 @@ def candidate_readout(
     ``token_norm_weight`` fuses the per-token RMSNorm in front (``final_norm``), ``pool_norm_weight`` the pooler's
     ``RMSNorm(3D)``. Without ``fc1_weight`` only the embedding is computed. Returns the logits (probabilities with
     ``sigmoid=True``), the embedding, or ``(logits, embedding)`` with ``return_embedding=True``, like
-    ``PCVRSymbiosis.forward`` / ``predict``.
+    ``PCVRSymbiosis.forward`` / ``predict``. Tensors that require a gradient take a differentiable route (the HIP norm
+    kernels with their backward, torch for the mean and the classifier) instead of the one-kernel inference route.
     """
     name = "hip candidate_readout"
     weights = (token_norm_weight, pool_norm_weight, fc1_weight, fc1_bias, fc2_weight, fc2_bias)
     require_cuda_tensors(name, tokens, key_lengths, padding_mask, *weights)
-    require_inference(name, tokens, *weights)
     if tokens.ndim != 3:
         raise ValueError(f"{name} expects tokens of shape (batch, tokens, d_model)")
     for t in (tokens, *weights):
@@ -73,6 +107,13 @@ def candidate_readout(
     lengths = None if key_lengths is None else key_lengths.to(torch.int32).contiguous()
     if lengths is not None and lengths.shape != (batch,):
         raise ValueError(f"{name}: key_lengths must have shape ({batch},)")
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (tokens, *weights)):
+        if padding_mask is not None and (padding_mask.dtype is not torch.bool or padding_mask.shape != (batch, token_count)):
+            raise ValueError(f"{name}: padding_mask must be a bool tensor of shape ({batch}, {token_count})")
+        return _candidate_readout_training(
+            tokens, int(cls_index), None if candidate_index is None else int(candidate_index), lengths, padding_mask,
+            token_norm_weight, pool_norm_weight, float(eps),
+            (fc1_weight, fc1_bias, fc2_weight, fc2_bias) if classifier else None, bool(sigmoid), bool(return_embedding))
     valid_bits = None
     if padding_mask is not None:
         if padding_mask.dtype is not torch.bool or padding_mask.shape != (batch, token_count):

@@ -118,6 +118,42 @@ def test_modules_mirror_the_reference_readout(device):
     torch.testing.assert_close(cpu(pooler_only).float(), want_plain, **TOL)
 
 
+@pytest.mark.parametrize("candidate,use_lengths", [(True, False), (False, True)])
+def test_readout_takes_a_gradient(device, candidate, use_lengths):
+    """Under autograd the readout runs its differentiable route: outputs equal to the one-kernel route, gradients of the
+    tokens and of every weight against float64 autograd of the oracle's expression."""
+    batch, tokens, d, hidden, actions = 6, 50, 256, 128, 2
+    x, wt, wp, w1, b1, w2, b2, pad = _draw(batch, tokens, d, hidden, actions, seed=77)
+    lengths = torch.tensor([50, 0, 13, 1, 30, 44], dtype=torch.int32)
+    if use_lengths:
+        pad = torch.arange(tokens)[None, :] >= lengths[:, None]
+    cls_index, cand_index = 2, (tokens - 1 if candidate else None)
+    dev = [t.to(device).requires_grad_(True) for t in (x, wt, wp, w1, b1, w2, b2)]
+    where = dict(key_lengths=lengths.to(device)) if use_lengths else dict(padding_mask=pad.to(device))
+    logits, emb = candidate_readout(dev[0], cls_index=cls_index, candidate_index=cand_index, token_norm_weight=dev[1],
+                                    pool_norm_weight=dev[2], fc1_weight=dev[3], fc1_bias=dev[4], fc2_weight=dev[5],
+                                    fc2_bias=dev[6], return_embedding=True, **where)
+    g = torch.Generator().manual_seed(5)
+    grad_logits, grad_emb = torch.randn(batch, actions, generator=g), torch.randn(batch, 3 * d, generator=g).to(torch.bfloat16)
+    torch.autograd.backward([logits, emb], [grad_logits.to(device), grad_emb.to(device)])
+    ref = [t.double().requires_grad_(True) for t in (x, wt, wp, w1, b1, w2, b2)]
+    want_emb, want_logits = oracle.candidate_readout(ref[0], pad, cls_index=cls_index, candidate_index=cand_index,
+                                                     token_norm_weight=ref[1], pool_norm_weight=ref[2], eps=1e-6,
+                                                     classifier=tuple(ref[3:]), fp32=False)
+    torch.autograd.backward([want_logits, want_emb], [grad_logits.double(), grad_emb.double()])
+    with torch.no_grad():
+        fused_logits, fused_emb = candidate_readout(
+            dev[0].detach(), cls_index=cls_index, candidate_index=cand_index, token_norm_weight=dev[1].detach(),
+            pool_norm_weight=dev[2].detach(), fc1_weight=dev[3].detach(), fc1_bias=dev[4].detach(),
+            fc2_weight=dev[5].detach(), fc2_bias=dev[6].detach(), return_embedding=True, **where)
+    torch.testing.assert_close(emb.detach().float(), fused_emb.float(), **TOL)
+    torch.testing.assert_close(logits.detach(), fused_logits, rtol=4e-2, atol=4e-2)
+    for got, expected in zip(dev, ref):
+        scale = expected.grad.abs().max().item()
+        error = (got.grad.detach().cpu().double() - expected.grad).abs().max().item()
+        assert error <= 3e-2 * max(scale, 1e-6), (error, scale)
+
+
 def test_errors(device):
     x = torch.randn(2, 8, 64).to(torch.bfloat16).to(device)
     with pytest.raises(ValueError, match="outside the sequence"):
