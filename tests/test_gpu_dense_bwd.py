@@ -317,3 +317,63 @@ def test_rows_gather_and_merge_through_the_c_abi(device):
         assert torch.equal(out, expected)
     assert library.taac_rows_gather(source.data_ptr(), source.stride(0), rows.data_ptr(), valid, compact.data_ptr(), 12,
                                     stream) == _native.TAAC_ERR_UNSUPPORTED
+
+
+def test_two_blocks_and_the_readout_train_end_to_end(device):
+    """A stack of two blocks (shared key lengths: one row index, one host synchronisation) and the readout head under a
+    binary cross-entropy loss: the loss and the gradient of the input and of every parameter against float64 autograd of
+    the oracle's blocks and readout."""
+    from types import SimpleNamespace
+
+    from taac_2026_amd.api import CandidateReadoutHead
+
+    batch, tokens, d_model, heads, mult = 4, 40, 128, 4, 2
+    g = torch.Generator().manual_seed(11)
+    modules = torch.nn.ModuleList([UnifiedInteractionBlock(d_model, heads, mult, qk_norm=False) for _ in range(2)]
+                                  + [CandidateReadoutHead(d_model, 1)])
+    with torch.no_grad():
+        for parameter in modules.parameters():
+            if parameter.ndim == 1:
+                parameter.copy_((1.0 if parameter.mean() > 0.5 else 0.0) + 0.1 * torch.randn(parameter.shape, generator=g))
+            else:
+                parameter.copy_(torch.randn(parameter.shape, generator=g) * parameter.shape[1] ** -0.5)
+    modules = modules.to(torch.bfloat16)
+    reference = {name: value.detach().double().requires_grad_(True) for name, value in modules.named_parameters()}
+    x = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16)
+    lengths = torch.tensor([40, 9, 1, 25], dtype=torch.int32)
+    padding = torch.arange(tokens)[None, :] >= lengths[:, None]
+    labels = torch.tensor([[1.0], [0.0], [1.0], [0.0]])
+    meta = SimpleNamespace(cls_index=0, candidate_index=3, padding_mask=None)
+
+    modules = modules.to(device).train()
+    xd = x.to(device).requires_grad_(True)
+    stream, lengths_d, padding_d = xd, lengths.to(device), padding.to(device)
+    for block in modules[:2]:
+        stream, _ = block(stream, padding_d, None, key_lengths=lengths_d, return_attention_tokens=False)
+    meta.padding_mask = padding_d
+    logits = modules[2](stream, meta)
+    loss = F.binary_cross_entropy_with_logits(logits, labels.to(device))
+    loss.backward()
+
+    xr = x.double().requires_grad_(True)
+    mask = (~padding)[:, None, None, :].expand(batch, 1, tokens, tokens)
+    stream_r = xr
+    names = {"attn_norm.weight": "attn_norm.weight", "qkv.weight": "attention.qkv.weight", "qkv.bias": "attention.qkv.bias",
+             "out.weight": "attention.out.weight", "out.bias": "attention.out.bias", "ffn_norm.weight": "ffn_norm.weight",
+             "up.weight": "ffn.up.weight", "up.bias": "ffn.up.bias", "down.weight": "ffn.down.weight",
+             "down.bias": "ffn.down.bias"}
+    for index in range(2):
+        weights = {short: reference[f"{index}.{full}"] for short, full in names.items()}
+        stream_r, _ = oracle.interaction_block(stream_r, padding, mask, weights, num_heads=heads)
+    _, logits_r = oracle.candidate_readout(
+        stream_r, padding, cls_index=0, candidate_index=3, token_norm_weight=reference["2.final_norm.weight"],
+        pool_norm_weight=reference["2.pooler.norm.weight"], eps=1e-6,
+        classifier=(reference["2.classifier.0.weight"], reference["2.classifier.0.bias"], reference["2.classifier.3.weight"],
+                    reference["2.classifier.3.bias"]), fp32=False)
+    loss_r = F.binary_cross_entropy_with_logits(logits_r, labels.double())
+    loss_r.backward()
+    assert abs(loss.item() - loss_r.item()) <= 2e-2
+    _close(xd.grad, xr.grad, 5e-2)
+    for name, parameter in modules.named_parameters():
+        assert parameter.grad is not None, name
+        _close(parameter.grad, reference[name].grad, 5e-2)
