@@ -17,7 +17,7 @@
 // [F+n0, F+n0+64); each wavefront holds gate and value of the same (token, feature) in the same lane and
 // register index, so silu(g) * u is formed in registers and the [M, 2F] projection is never written.
 // Follows SwiGLUFeedForward.forward (experiments/symbiosis/backbone.py:19-21): gate, value = up(x).chunk(2, -1).
-#include "common.h"
+#include "ts_common.h"
 
 namespace taac {
 namespace {
@@ -227,73 +227,74 @@ __global__ __launch_bounds__(kThreads) void linear_bf16_kernel(const LinearParam
 }
 
 // ------------------------------------------------------------------------------------------------------------------
-// bf16 operands, narrow outputs from a long contraction (128 < N <= 256, large K): the input-gradient products of the
-// backward (dy w with K = 2F or 3D, N = D). One workgroup owns 256 tokens x ALL output features, so the activations are
-// read from memory exactly once (the 128 x 128 kernel reads them once per feature tile, and with two tiles per token
-// block it was 0.80 ms against 0.56 ms for the library at M = 524 288, K = 2048). Eight wavefronts, 4 token groups of 64
-// x 2 feature halves of 128: 4 weight fragments and 2 token fragments from LDS feed 8 MFMAs. K is walked in slabs of 64
-// through two padded LDS buffers, the next slab travelling through registers while the current one is consumed: one
-// barrier per slab.
+// bf16 operands, narrow outputs from a long contraction (128 < N <= 256, K a multiple of 32): the input-gradient
+// products of the backward (dy w with K = 2F or 3D, N = D). One workgroup owns 256 tokens x ALL output features, so the
+// activations are read from memory exactly once (the 128 x 128 kernel reads them once per feature tile: 0.80 ms against
+// 0.57 ms for the library at M = 524 288, K = 2048). Eight wavefronts, 4 token groups of 64 x 2 feature halves of 128:
+// per k-step 4 weight fragments and 2 token fragments from LDS feed 8 MFMAs. K is walked in slabs of 32: the slab of
+// both operands goes from global memory straight into LDS (16 rows x 64 bytes per transfer instruction, 4 instructions
+// per wavefront and slab) into a ring of four 32 KB stages, three slabs ahead (a first version staged 64-wide slabs
+// through registers, one slab ahead: the same 0.73 ms, so it is not the latency of the loads that bounds the kernel at
+// 3.3-3.5 TB/s; half of the wavefronts' time is spent waiting for the transfers). A transfer cannot pad rows, so the four 16-byte pieces of a row are XOR-swizzled
+// by (row / 4) % 4: the 16 lanes of a fragment read hit 16 distinct bank groups. Rows beyond M (or N) repeat the last
+// row; their results are not stored.
 // ------------------------------------------------------------------------------------------------------------------
 constexpr int kWideThreads = 512;
 constexpr int kWideTile = 256;
-constexpr int kWideSlab = 64;
-constexpr int kWideStride = kWideSlab + 8;  // LDS row stride in elements (+16 bytes)
-constexpr int kWideOperand = kWideTile * kWideStride;
-constexpr size_t kWideLdsBytes = static_cast<size_t>(2) * 2 * kWideOperand * sizeof(bf16_t);
+constexpr int kWideSlab = 32;
+constexpr int kWideRing = 4;
+constexpr int kWideOperandBytes = kWideTile * kWideSlab * 2;   // 16 KB
+constexpr int kWideStageBytes = 2 * kWideOperandBytes;         // tokens | weights
+constexpr size_t kWideLdsBytes = static_cast<size_t>(kWideRing) * kWideStageBytes;
 
 template <int EPI>
 __global__ __launch_bounds__(kWideThreads, 2) void linear_bf16_wide_kernel(const LinearParams p) {
-  constexpr int CH = kWideSlab / 8;                        // 16-byte pieces per tile row
-  constexpr int LD = kWideTile * CH / kWideThreads;        // pieces per thread and operand (4)
-  extern __shared__ __attribute__((aligned(16))) uint8_t wide_smem[];
-  bf16_t* lds = reinterpret_cast<bf16_t*>(wide_smem);      // [buffer][operand: tokens, weights][row][kWideStride]
+  extern __shared__ __attribute__((aligned(1024))) uint8_t wide_smem[];
 
   const int64_t m0 = static_cast<int64_t>(blockIdx.x) * kWideTile;
   const int tid = threadIdx.x;
-  const int wave = tid / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int lane = tid % kWave;
   const int l32 = lane % 32;
   const int hh = lane / 32;
   const int wt = wave % 4;  // token group of 64
   const int wn = wave / 4;  // feature half of 128
+  const int nslabs = p.K / kWideSlab;
 
-  const bf16_t* A = static_cast<const bf16_t*>(p.a);
-  const bf16_t* W = static_cast<const bf16_t*>(p.w);
-  bf16x8 zero_vec;
+  // Transfers of this wavefront: instructions j = 2 * wave, 2 * wave + 1 of both operands; lane -> row 16 j + lane / 4,
+  // LDS piece lane % 4, which holds global piece (lane % 4) ^ (row / 4) % 4 of the slab.
+  const bf16_t* a_src[2];
+  const bf16_t* w_src[2];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) zero_vec[e] = static_cast<bf16_t>(0.f);
-
-  // staging slots: piece c = tid + 512 * i -> tile row c / CH, 8-element column c % CH
-  const bf16_t* a_src[LD];
-  const bf16_t* w_src[LD];
-  int lds_off[LD];
-  const int col_off = (tid % CH) * 8;
-#pragma unroll
-  for (int i = 0; i < LD; ++i) {
-    const int r = (tid + kWideThreads * i) / CH;
-    lds_off[i] = r * kWideStride + col_off;
-    a_src[i] = (m0 + r < p.M) ? A + (m0 + r) * p.lda + col_off : nullptr;
-    w_src[i] = (r < p.N) ? W + static_cast<int64_t>(r) * p.K + col_off : nullptr;
+  for (int i = 0; i < 2; ++i) {
+    const int row = 16 * (2 * wave + i) + lane / 4;
+    const int piece = (lane % 4) ^ ((row >> 2) & 3);
+    const int64_t arow = m0 + row < p.M ? m0 + row : p.M - 1;
+    const int wrow = row < p.N ? row : p.N - 1;
+    a_src[i] = static_cast<const bf16_t*>(p.a) + arow * p.lda + piece * 8;
+    w_src[i] = static_cast<const bf16_t*>(p.w) + static_cast<int64_t>(wrow) * p.K + piece * 8;
   }
-  bf16x8 ra[LD], rw[LD];
-  auto fetch = [&](int k0) {
-    const bool kin = k0 + col_off < p.K;
+  // Every workgroup starts its walk over K at a different slab (the sum is the same; its order differs per workgroup,
+  // not per run): with all workgroups on the same columns of a matrix whose row pitch is a power of two their requests
+  // crowded the same memory channels (0.73 -> 0.69 ms at K = 2048).
+  const int rot = static_cast<int>((blockIdx.x * 5u) % static_cast<uint32_t>(nslabs));
+  auto stage = [&](int slab) {
+    uint8_t* base = wide_smem + (slab % kWideRing) * kWideStageBytes + (2 * wave) * 1024;
+    const int turned = slab + rot;
+    const int k0 = (turned >= nslabs ? turned - nslabs : turned) * kWideSlab;
 #pragma unroll
-    for (int i = 0; i < LD; ++i) {
-      ra[i] = (a_src[i] != nullptr && kin) ? *reinterpret_cast<const bf16x8*>(a_src[i] + k0) : zero_vec;
-      rw[i] = (w_src[i] != nullptr && kin) ? *reinterpret_cast<const bf16x8*>(w_src[i] + k0) : zero_vec;
+    for (int i = 0; i < 2; ++i) {
+      lds_dma16(a_src[i] + k0, base + i * 1024);
+      lds_dma16(w_src[i] + k0, base + kWideOperandBytes + i * 1024);
     }
   };
-  auto commit = [&](int buf) {
-    bf16_t* sa = lds + buf * 2 * kWideOperand;
-    bf16_t* sw = sa + kWideOperand;
+  // Fragment reads: lane (l32, hh) takes piece 2 ks + hh of its row, stored at piece ^ (l32 / 4) % 4.
+  const int swz = (l32 >> 2) & 3;
+  int piece_off[2];
 #pragma unroll
-    for (int i = 0; i < LD; ++i) {
-      *reinterpret_cast<bf16x8*>(&sa[lds_off[i]]) = ra[i];
-      *reinterpret_cast<bf16x8*>(&sw[lds_off[i]]) = rw[i];
-    }
-  };
+  for (int ks = 0; ks < 2; ++ks) piece_off[ks] = ((2 * ks + hh) ^ swz) * 16;
+  const int a_row_off = (wt * 64 + l32) * (kWideSlab * 2);
+  const int w_row_off = kWideOperandBytes + (wn * 128 + l32) * (kWideSlab * 2);
 
   f32x16 acc[4][2];
 #pragma unroll
@@ -303,33 +304,40 @@ __global__ __launch_bounds__(kWideThreads, 2) void linear_bf16_wide_kernel(const
 #pragma unroll
       for (int j = 0; j < 16; ++j) acc[ni][mi][j] = 0.f;
 
-  fetch(0);
-  commit(0);
+#pragma unroll
+  for (int q = 0; q < kWideRing - 1; ++q)
+    if (q < nslabs) stage(q);
+  // slab 0 has landed when at most the transfers of slabs 1 and 2 are outstanding
+  if (nslabs > 2) vm_wait<8>();
+  else if (nslabs > 1) vm_wait<4>();
+  else vm_wait<0>();
   __syncthreads();
-  int buf = 0;
-  for (int k0 = 0; k0 < p.K; k0 += kWideSlab) {
-    const bool has_next = k0 + kWideSlab < p.K;
-    if (has_next) fetch(k0 + kWideSlab);
-    const bf16_t* sa = lds + buf * 2 * kWideOperand;
-    const bf16_t* sw = sa + kWideOperand;
+  for (int s = 0; s < nslabs; ++s) {
+    // slot (s + 3) % 4 was last read in slab s - 1, which every wavefront has left
+    if (s + kWideRing - 1 < nslabs) stage(s + kWideRing - 1);
+    const uint8_t* st = wide_smem + (s % kWideRing) * kWideStageBytes;
 #pragma unroll
     for (int ks = 0; ks < kWideSlab / 16; ++ks) {
       bf16x8 wf[4], af[2];
 #pragma unroll
       for (int mi = 0; mi < 2; ++mi)
-        af[mi] = *reinterpret_cast<const bf16x8*>(&sa[(wt * 64 + mi * 32 + l32) * kWideStride + ks * 16 + hh * 8]);
+        af[mi] = *reinterpret_cast<const bf16x8*>(st + a_row_off + mi * 32 * (kWideSlab * 2) + piece_off[ks]);
 #pragma unroll
       for (int ni = 0; ni < 4; ++ni)
-        wf[ni] = *reinterpret_cast<const bf16x8*>(&sw[(wn * 128 + ni * 32 + l32) * kWideStride + ks * 16 + hh * 8]);
+        wf[ni] = *reinterpret_cast<const bf16x8*>(st + w_row_off + ni * 32 * (kWideSlab * 2) + piece_off[ks]);
 #pragma unroll
       for (int ni = 0; ni < 4; ++ni)
 #pragma unroll
         for (int mi = 0; mi < 2; ++mi)
           acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ni], af[mi], acc[ni][mi], 0, 0, 0);
     }
-    if (has_next) commit(buf ^ 1);  // that buffer was last read in the previous slab, which every wavefront has left
-    __syncthreads();
-    buf ^= 1;
+    if (s + 1 < nslabs) {
+      // the transfers of slab s + 1 were issued three slabs ago; behind them are those of slabs s + 2 and s + 3
+      if (s + 3 < nslabs) vm_wait<8>();
+      else if (s + 2 < nslabs) vm_wait<4>();
+      else vm_wait<0>();
+      __syncthreads();
+    }
   }
 
   // acc[ni][mi][jq * 4 + e]: feature wn * 128 + ni * 32 + jq * 8 + hh * 4 + e of token wt * 64 + mi * 32 + l32
@@ -583,7 +591,7 @@ extern "C" int taac_linear_bf16(const void* a, int64_t lda, const void* w, const
   rc = fill_params(name, p, M, N, epilogue);
   if (rc != TAAC_OK) return rc;
   hipStream_t s = as_stream(stream);
-  if (epilogue != TAAC_EPI_SWIGLU && N > 128 && N <= kWideTile && K >= 512 && M >= 1024) {
+  if (epilogue != TAAC_EPI_SWIGLU && N > 128 && N <= kWideTile && K >= 512 && K % kWideSlab == 0 && M >= 1024) {
     // long contraction into a narrow output: one workgroup per 256 tokens with all output features
     const int64_t blocks = (M + kWideTile - 1) / kWideTile;
     if (blocks > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many workgroups", name);
