@@ -54,19 +54,28 @@ def _event_ms(fn, iters: int, warmup: int) -> float:
 
 def _event_ms_after(prelude, fn, iters: int, warmup: int) -> float:
     """Duration of ``fn`` in ms per call when every call follows ``prelude`` on the same stream, as it does inside the
-    step (its inputs were just written by the kernel before it): one pair of HIP events around each ``fn`` launch, the
-    median over the launches. The events bracket ``fn`` alone; ``prelude`` runs outside them."""
+    step (its inputs were just written by the kernel before it). HIP events on the launch stream around runs of
+    back-to-back launches: the time of ``n x [prelude, fn]`` minus the time of ``n x [prelude]``, per call, median over
+    interleaved groups. (A pair of events around every single ``fn`` launch also counts the gap between the event and the
+    kernel on either side, which read 5 - 7 % above the kernel trace's duration of the same launches.)"""
     for _ in range(warmup):
         prelude()
         fn()
-    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
-    for start, stop in pairs:
-        prelude()
+    groups = max(1, min(5, iters // 2))
+    per_group = max(2, iters // groups)
+
+    def run(with_fn: bool) -> float:
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
-        fn()
+        for _ in range(per_group):
+            prelude()
+            if with_fn:
+                fn()
         stop.record()
-    pairs[-1][1].synchronize()
-    times = sorted(start.elapsed_time(stop) for start, stop in pairs)
+        stop.synchronize()
+        return start.elapsed_time(stop) / per_group
+
+    times = sorted(run(True) - run(False) for _ in range(groups))
     return times[len(times) // 2]
 
 
@@ -192,7 +201,7 @@ def _kernel_breakdown(inputs, device, iters: int) -> dict:
                 "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS,
             }
             if name in in_sequence:
-                out[name]["ms_in_sequence"] = _event_ms_after(in_sequence[name], fn, iters, 2)
+                out[name]["ms_in_sequence"] = _event_ms_after(in_sequence[name], fn, 4 * iters, 2)
     return out
 
 
