@@ -52,12 +52,13 @@ def _event_ms(fn, iters: int, warmup: int) -> float:
     return times[len(times) // 2]
 
 
-def _event_ms_after(prelude, fn, iters: int, warmup: int) -> float:
+def _event_ms_after(prelude, fn, iters: int, warmup: int, reset=None) -> float:
     """Duration of ``fn`` in ms per call when every call follows ``prelude`` on the same stream, as it does inside the
     step (its inputs were just written by the kernel before it). HIP events on the launch stream around runs of
     back-to-back launches: the time of ``n x [prelude, fn]`` minus the time of ``n x [prelude]``, per call, median over
     interleaved groups. (A pair of events around every single ``fn`` launch also counts the gap between the event and the
-    kernel on either side, which read 5 - 7 % above the kernel trace's duration of the same launches.)"""
+    kernel on either side, which read 5 - 7 % above the kernel trace's duration of the same launches.) ``reset`` runs
+    in front of every run, outside the events (for an ``fn`` that updates its input in place)."""
     for _ in range(warmup):
         prelude()
         fn()
@@ -66,6 +67,8 @@ def _event_ms_after(prelude, fn, iters: int, warmup: int) -> float:
 
     def run(with_fn: bool) -> float:
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        if reset is not None:
+            reset()
         start.record()
         for _ in range(per_group):
             prelude()
@@ -187,7 +190,13 @@ def _kernel_breakdown(inputs, device, iters: int) -> dict:
         # Inside the step every kernel reads what the kernel before it just wrote. The block's last kernel is timed that
         # way too (attention launched in front of every timed launch, outside the events): "ms" is the stand-alone figure
         # on inputs that are cold in the caches, "ms_in_sequence" the one that matches the kernel trace of the step.
-        in_sequence = {"out_residual_rmsnorm_swiglu_ffn_residual": attn}
+        # The step's launch also updates the residual stream in place (out = the block input), which the timed launch
+        # here does on a working copy that is restored in front of every run of eight launches.
+        x_work = x.clone()
+        in_place = lambda: attention_out_ffn(a, w["out.weight"], w["out.bias"], x_work, w["up.weight"], w["up.bias"],  # noqa: E731
+                                             w["down.weight"], w["down.bias"], norm_weight=w["ffn_norm.weight"],
+                                             token_rows=index, out=x_work)
+        in_sequence = {"out_residual_rmsnorm_swiglu_ffn_residual": (attn, in_place, lambda: x_work.copy_(x))}
         for name, (fn, flops, nbytes) in cases.items():
             ms = _event_ms(fn, iters, 3)
             out[name] = {
@@ -201,7 +210,8 @@ def _kernel_breakdown(inputs, device, iters: int) -> dict:
                 "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS,
             }
             if name in in_sequence:
-                out[name]["ms_in_sequence"] = _event_ms_after(in_sequence[name], fn, 4 * iters, 2)
+                prelude, step_fn, restore = in_sequence[name]
+                out[name]["ms_in_sequence"] = _event_ms_after(prelude, step_fn, 4 * iters, 2, reset=restore)
     return out
 
 
