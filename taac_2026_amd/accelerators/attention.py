@@ -658,20 +658,23 @@ def flash_attention(
 _ROPE_TABLES: dict[tuple, torch.Tensor] = {}
 
 
-def rope_table(token_count: int, head_dim: int, rope_base: float, dtype: torch.dtype, device: torch.device) -> torch.Tensor:
+def rope_table(token_count: int, head_dim: int, rope_base: float, dtype: torch.dtype, device: torch.device, *,
+               inverse: bool = False) -> torch.Tensor:
     """``[tokens, head_dim / 2, 2]`` table of (cos, sin) of ``position * rope_base ** (-2i / head_dim)``, computed in
     float32 and rounded to the activation dtype as ``BFTSAttention._apply_rope`` does
-    (experiments/tokenformer/model.py:174-179); cached per shape, base, dtype and device."""
+    (experiments/tokenformer/model.py:174-179); cached per shape, base, dtype and device. ``inverse``: (cos, -sin), the
+    rotation by the opposite angles - the transpose of the rotation, which is what its backward applies."""
     if head_dim % 2 != 0:
         raise ValueError("hip qk_norm_rope rotates whole heads: head_dim must be even")
-    key = (int(token_count), int(head_dim), float(rope_base), dtype, str(device))
+    key = (int(token_count), int(head_dim), float(rope_base), dtype, str(device), bool(inverse))
     table = _ROPE_TABLES.get(key)
     if table is None:
         positions = torch.arange(token_count, dtype=torch.float32)
         frequencies = torch.arange(0, head_dim, 2, dtype=torch.float32)
         inv_freq = torch.pow(torch.tensor(float(rope_base)), -frequencies / max(1, head_dim))
         angles = positions[:, None] * inv_freq[None, :]
-        table = torch.stack((angles.cos().to(dtype), angles.sin().to(dtype)), dim=-1).contiguous().to(device)
+        sin = angles.sin().to(dtype)
+        table = torch.stack((angles.cos().to(dtype), -sin if inverse else sin), dim=-1).contiguous().to(device)
         _ROPE_TABLES[key] = table
     return table
 
@@ -697,19 +700,25 @@ def qk_norm_rope(
     rope_base: float | None = None,
     token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
     inplace: bool = False,
+    inverse_rotation: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """What the reference's attention layers do to the query and key projections before attention, in one pass:
     ``RMSNorm(d_model)`` of each (experiments/symbiosis/backbone.py:33-36) and, with ``rope_base``, the rotary embedding
     over the token positions (experiments/tokenformer/model.py:165-192). ``query`` / ``key``: (batch, tokens, d_model),
     possibly the ``chunk(3, -1)`` views of a packed projection (rows are read with their stride). ``inplace`` writes the
     result over the inputs. ``token_rows`` (:func:`valid_rows`) restricts the pass to the valid tokens; the other rows
-    of the result are then zero (new tensors) or untouched (in place)."""
+    of the result are then zero (new tensors) or untouched (in place). Tensors that require a gradient take the
+    differentiable route :func:`qk_norm_rope_autograd`. ``inverse_rotation`` rotates by the opposite angles."""
     name = "hip qk_norm_rope"
     if query.ndim != 3 or key.shape != query.shape:
         raise ValueError("qk_norm_rope expects query and key of the same shape (batch, tokens, d_model)")
     require_same_dtype("qk_norm_rope", query, key)
     require_cuda_tensors(name, query, key)
-    require_inference(name, query, key)
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (query, key, query_weight, key_weight)):
+        if token_rows is not None or inplace or inverse_rotation:
+            raise RuntimeError(f"{name}: token_rows / inplace belong to the inference route; call it under "
+                               "torch.no_grad() or pass plain tensors when a gradient is needed")
+        return qk_norm_rope_autograd(query, key, query_weight, key_weight, num_heads=num_heads, eps=eps, rope_base=rope_base)
     batch, tokens, d_model = query.shape
     if d_model % int(num_heads) != 0:
         raise ValueError("d_model must be divisible by num_heads")
@@ -728,7 +737,7 @@ def qk_norm_rope(
         weights.append(weight.detach().to(dtype=query.dtype).contiguous())
     table = None
     if rope_base is not None:
-        table = rope_table(tokens, d_model // int(num_heads), rope_base, query.dtype, query.device)
+        table = rope_table(tokens, d_model // int(num_heads), rope_base, query.dtype, query.device, inverse=inverse_rotation)
     strides = (_row_stride(name, query), _row_stride(name, key))
     if strides[0] is None or strides[0] != strides[1]:
         if inplace:
@@ -758,6 +767,44 @@ def qk_norm_rope(
     return query_out, key_out
 
 
+class _RotaryFunction(torch.autograd.Function):
+    """The rotary embedding of query and key as one pass of the preparation kernel; the backward is the same pass with
+    the opposite angles (a rotation's transpose), applied to the incoming gradients."""
+
+    @staticmethod
+    def forward(ctx, query, key, num_heads: int, rope_base: float):
+        ctx.config = (int(num_heads), float(rope_base))
+        with torch.no_grad():
+            return qk_norm_rope(query.detach(), key.detach(), None, None, num_heads=num_heads, rope_base=rope_base)
+
+    @staticmethod
+    def backward(ctx, grad_query, grad_key):
+        num_heads, rope_base = ctx.config
+        with torch.no_grad():
+            grad_query, grad_key = qk_norm_rope(grad_query.contiguous(), grad_key.contiguous(), None, None, num_heads=num_heads,
+                                                rope_base=rope_base, inverse_rotation=True)
+        return grad_query, grad_key, None, None
+
+
+def qk_norm_rope_autograd(query: torch.Tensor, key: torch.Tensor, query_weight: torch.Tensor | None,
+                          key_weight: torch.Tensor | None, *, num_heads: int, eps: float = 1e-6,
+                          rope_base: float | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """:func:`qk_norm_rope` for tensors that take a gradient, as two differentiable steps the way the reference's layers
+    run them (experiments/symbiosis/backbone.py:33-36, experiments/tokenformer/model.py:149-154): ``RMSNorm(d_model)`` of
+    the query and of the key through the norm kernels and their backward, then the rotation (its backward is the
+    rotation by the opposite angles)."""
+    from taac_2026_amd.accelerators.normalization import rms_norm
+
+    if (query_weight is None) != (key_weight is None):
+        raise ValueError("qk_norm_rope takes both norm weights or neither")
+    if query_weight is not None:
+        query = rms_norm(query.contiguous(), query_weight, eps)
+        key = rms_norm(key.contiguous(), key_weight, eps)
+    if rope_base is not None:
+        query, key = _RotaryFunction.apply(query, key, int(num_heads), float(rope_base))
+    return query, key
+
+
 __all__ = [
     "FLASH_ATTENTION_BACKENDS",
     "FlashAttentionMaskPlan",
@@ -769,6 +816,7 @@ __all__ = [
     "plan_flash_attention_mask",
     "plan_structured_attention_mask",
     "qk_norm_rope",
+    "qk_norm_rope_autograd",
     "resolved_flash_attention_backend",
     "rope_table",
 ]

@@ -93,7 +93,13 @@ class UnifiedSelfAttention(nn.Module):
         key_weight = None if self.key_norm is None else _bf16(self.key_norm.weight)
         qk_eps = 1e-6 if self.query_norm is None else self.query_norm.eps
         q_row_scale = k_row_scale = q_col_scale = None
-        if prepare and x.ndim == 3 and x.shape[-1] in (128, 256):
+        needs_grad = torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))
+        if prepare and needs_grad:
+            # training: projection, query / key norm and rotation as differentiable steps
+            query, key, value = _dense(self.qkv, x).chunk(3, dim=-1)
+            query, key = qk_norm_rope(query, key, query_weight, key_weight, num_heads=self.num_heads, eps=qk_eps,
+                                      rope_base=self.rope_base)
+        elif prepare and x.ndim == 3 and x.shape[-1] in (128, 256):
             # the norm statistic (and, with a rotation, weight and rotation) come out of the projection's epilogue; the
             # per-token factor of the norm and the weights of the unrotated case are applied inside the attention
             # kernel: no pass over q and k at all

@@ -186,13 +186,14 @@ def test_swiglu_ffn_takes_a_gradient(device, m, d, f, gate_first, with_norm):
             _close(got.grad, expected.grad)
 
 
-def test_interaction_block_takes_a_gradient_end_to_end(device):
-    """``UnifiedInteractionBlock`` in training mode (plain attention layer, key-length mask): output and the gradient of
-    the input and of every parameter against float64 autograd of ``oracle.interaction_block``
-    (experiments/symbiosis/backbone.py:58-68)."""
+@pytest.mark.parametrize("qk_norm", [False, True])
+def test_interaction_block_takes_a_gradient_end_to_end(device, qk_norm):
+    """``UnifiedInteractionBlock`` in training mode (plain attention layer or the reference's default with query / key
+    norms, key-length mask): output and the gradient of the input and of every parameter against float64 autograd of
+    ``oracle.interaction_block`` (experiments/symbiosis/backbone.py:58-68)."""
     batch, tokens, d_model, heads, mult = 3, 48, 128, 4, 2
     g = torch.Generator().manual_seed(1)
-    block = UnifiedInteractionBlock(d_model, heads, mult, qk_norm=False)
+    block = UnifiedInteractionBlock(d_model, heads, mult, qk_norm=qk_norm)
     with torch.no_grad():
         for parameter in block.parameters():
             if parameter.ndim == 1:
@@ -207,6 +208,9 @@ def test_interaction_block_takes_a_gradient_end_to_end(device):
         "ffn_norm.weight": block.ffn_norm.weight, "up.weight": block.ffn.up.weight, "up.bias": block.ffn.up.bias,
         "down.weight": block.ffn.down.weight, "down.bias": block.ffn.down.bias,
     }
+    if qk_norm:
+        weights["query_norm.weight"] = block.attention.query_norm.weight
+        weights["key_norm.weight"] = block.attention.key_norm.weight
     reference = {name: value.detach().double().requires_grad_(True) for name, value in weights.items()}
     x = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16)
     lengths = torch.tensor([48, 17, 33], dtype=torch.int32)
@@ -229,6 +233,8 @@ def test_interaction_block_takes_a_gradient_end_to_end(device):
               "out.weight": "attention.out.weight", "out.bias": "attention.out.bias", "ffn_norm.weight": "ffn_norm.weight",
               "up.weight": "ffn.up.weight", "up.bias": "ffn.up.bias", "down.weight": "ffn.down.weight",
               "down.bias": "ffn.down.bias"}
+    if qk_norm:
+        lookup.update({"query_norm.weight": "attention.query_norm.weight", "key_norm.weight": "attention.key_norm.weight"})
     for name, parameter_name in lookup.items():
         assert named[parameter_name].grad is not None, parameter_name
         _close(named[parameter_name].grad, reference[name].grad)

@@ -254,3 +254,39 @@ def test_golden_vectors(device):
         torch.testing.assert_close(got_k.cpu().double(), torch.tensor(case["key_out"], dtype=torch.float64), rtol=2e-5, atol=2e-6)
         served += 1
     assert served == 3
+
+
+@pytest.mark.parametrize("mode", ["norm", "rope", "norm_rope"])
+def test_qk_norm_rope_takes_a_gradient(device, mode):
+    """Under autograd the preparation runs as differentiable steps (norm kernels with their backward, the rotation with
+    the opposite angles as its backward): outputs equal to the one-pass route, gradients of query, key and the norm
+    weights against float64 autograd of the oracle's expression at the reference's gradient tolerance."""
+    batch, tokens, d_model, heads = 3, 50, 128, 4
+    g = torch.Generator().manual_seed(21)
+    q = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16)
+    k = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16)
+    wq = (1 + 0.1 * torch.randn(d_model, generator=g)).to(torch.bfloat16)
+    wk = (1 + 0.1 * torch.randn(d_model, generator=g)).to(torch.bfloat16)
+    gq = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16)
+    gk = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16)
+    with_norm, rope_base = mode != "rope", (None if mode == "norm" else 10000.0)
+    dev = [t.to(device).requires_grad_(True) for t in (q, k, wq, wk)]
+    out_q, out_k = qk_norm_rope(dev[0], dev[1], dev[2] if with_norm else None, dev[3] if with_norm else None,
+                                num_heads=heads, rope_base=rope_base)
+    torch.autograd.backward([out_q, out_k], [gq.to(device), gk.to(device)])
+    with torch.no_grad():
+        one_q, one_k = qk_norm_rope(dev[0].detach(), dev[1].detach(), dev[2].detach() if with_norm else None,
+                                    dev[3].detach() if with_norm else None, num_heads=heads, rope_base=rope_base)
+    torch.testing.assert_close(out_q.detach().float(), one_q.float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(out_k.detach().float(), one_k.float(), rtol=2e-2, atol=2e-2)
+    ref = [t.double().requires_grad_(True) for t in (q, k, wq, wk)]
+    want_q, want_k = oracle.qk_norm_rope(ref[0], ref[1], ref[2] if with_norm else None, ref[3] if with_norm else None,
+                                         num_heads=heads, rope_base=rope_base)
+    torch.autograd.backward([want_q, want_k], [gq.double(), gk.double()])
+    for index, (got, expected) in enumerate(zip(dev, ref)):
+        if index >= 2 and not with_norm:
+            assert got.grad is None
+            continue
+        scale = expected.grad.abs().max().item()
+        error = (got.grad.cpu().double() - expected.grad).abs().max().item()
+        assert error <= 3e-2 * scale, (index, error, scale)
