@@ -311,28 +311,32 @@ def _training_block_figures(device, with_comparison: bool = True) -> dict:
 
     inputs = workloads.backbone_inputs(batch=1024)
     batch, tokens, width = inputs.emb.shape
-    torch.manual_seed(0)
-    block = UnifiedInteractionBlock(width, inputs.num_heads, 4, qk_norm=False).to(torch.bfloat16).to(device).train()
-    x = inputs.emb.to(device).requires_grad_(True)
     lengths = inputs.key_lengths.to(device)
     padding = torch.arange(tokens, device=device)[None, :] >= lengths[:, None]
     grad = torch.randn(batch, tokens, width, device=device).to(torch.bfloat16)
+    figures = {"valid_token_fraction": float(lengths.sum().item()) / (batch * tokens)}
+    # the benchmark recipe's plain attention layer, and the reference block's default with query / key norms
+    for label, qk_norm in (("plain_attention_layer", False), ("query_key_norm", True)):
+        torch.manual_seed(0)
+        block = UnifiedInteractionBlock(width, inputs.num_heads, 4, qk_norm=qk_norm).to(torch.bfloat16).to(device).train()
+        x = inputs.emb.to(device).requires_grad_(True)
 
-    def step():
-        out, _ = block(x, padding, None, key_lengths=lengths, return_attention_tokens=False)
-        out.backward(grad)
-        block.zero_grad(set_to_none=True)
-        x.grad = None
+        def step():
+            out, _ = block(x, padding, None, key_lengths=lengths, return_attention_tokens=False)
+            out.backward(grad)
+            block.zero_grad(set_to_none=True)
+            x.grad = None
 
-    figures = {"valid_rows_ms": _event_ms(step, 5, 3)}
-    if with_comparison:
-        applies = backbone_module.training_route_applies
-        backbone_module.training_route_applies = lambda *a, **k: False
-        try:
-            figures["layer_by_layer_ms"] = _event_ms(step, 3, 2)
-        finally:
-            backbone_module.training_route_applies = applies
-    figures["valid_token_fraction"] = float(lengths.sum().item()) / (batch * tokens)
+        entry = {"valid_rows_ms": _event_ms(step, 5, 3)}
+        if with_comparison:
+            applies = backbone_module.training_route_applies
+            backbone_module.training_route_applies = lambda *a, **k: False
+            try:
+                entry["layer_by_layer_ms"] = _event_ms(step, 3, 2)
+            finally:
+                backbone_module.training_route_applies = applies
+        figures[label] = entry
+        del block, x
     return {"interaction_block_training_step_B1024_T512": figures}
 
 

@@ -91,13 +91,13 @@ def _attention_strides(width: int, heads: int, row_stride: int, tokens: int):
 
 
 class InteractionBlockFunction(torch.autograd.Function):
-    """``UnifiedInteractionBlock.forward`` without query / key norm, dropout or an attention mask other than the key
-    lengths. Inputs: tokens ``[B, T, D]`` bf16, ``key_lengths`` int32 ``[B]``, then the block's parameters. Returns
+    """``UnifiedInteractionBlock.forward`` (with or without the query / key norms) without rotary embedding, dropout or an
+    attention mask other than the key lengths. Inputs: tokens ``[B, T, D]`` bf16, ``key_lengths`` int32 ``[B]``, then the block's parameters. Returns
     ``(output, attn_tokens)`` like the module (``attn_tokens`` is None unless asked for)."""
 
     @staticmethod
-    def forward(ctx, tokens, key_lengths, want_attn_tokens, num_heads, attn_eps, ffn_eps, gate_first, attn_norm_w, w_qkv,
-                b_qkv, w_out, b_out, ffn_norm_w, w_up, b_up, w_down, b_down):
+    def forward(ctx, tokens, key_lengths, want_attn_tokens, num_heads, attn_eps, ffn_eps, gate_first, qk_eps, attn_norm_w,
+                w_qkv, b_qkv, w_out, b_out, ffn_norm_w, w_up, b_up, w_down, b_down, query_norm_w, key_norm_w):
         batch, token_count, width = tokens.shape
         total = batch * token_count
         index = _RowIndex.get(key_lengths, token_count)
@@ -110,11 +110,20 @@ class InteractionBlockFunction(torch.autograd.Function):
         qkv = torch.empty(total, 3 * width, dtype=flat.dtype, device=flat.device)
         _indexed_linear(flat, w_qkv, b_qkv, qkv, tokens=total, out_rows=rows, count=count, x_rows=None,
                         norm_weight=attn_norm_w, eps=attn_eps)
+        element = qkv.element_size()
+        if query_norm_w is not None:
+            # RMSNorm(d_model) of the query and of the key, in place on the valid rows of the packed projection; the
+            # backward recomputes the projection for the norms' own backward
+            status = library.taac_qk_norm_rope_fwd(
+                qkv.data_ptr(), qkv.data_ptr() + width * element, 3 * width, qkv.data_ptr(), qkv.data_ptr() + width * element,
+                3 * width, total, token_count, width, int(num_heads), query_norm_w.data_ptr(), key_norm_w.data_ptr(),
+                float(qk_eps), None, rows.data_ptr(), count.data_ptr(), _native.dtype_code(flat.dtype),
+                _native.current_stream(tokens.device))
+            _native.check(status, "interaction block (training): query / key norm")
         attended = torch.empty(total, width, dtype=flat.dtype, device=flat.device)
         lse = torch.empty(batch, num_heads, token_count, dtype=torch.float32, device=flat.device)
         qkv_strides = _attention_strides(width, num_heads, 3 * width, token_count)
         out_strides = _attention_strides(width, num_heads, width, token_count)
-        element = qkv.element_size()
         status = library.taac_flash_attn_train_fwd(
             qkv.data_ptr(), qkv.data_ptr() + width * element, qkv.data_ptr() + 2 * width * element, key_lengths.data_ptr(),
             attended.data_ptr(), lse.data_ptr(), batch, num_heads, token_count, token_count, width // num_heads,
@@ -136,10 +145,12 @@ class InteractionBlockFunction(torch.autograd.Function):
             _linear.attention_out_ffn(attended, w_out, b_out, flat, w_up, b_up, w_down, b_down, norm_weight=ffn_norm_w,
                                       eps=ffn_eps, token_rows=(rows, count), out=output)
         ctx.save_for_backward(flat, qkv, attended, lse, key_lengths, attn_norm_w, w_qkv, w_out, ffn_norm_w, w_up, w_down,
-                              *(t for t in (b_out, b_up, attn_tokens) if t is not None))
+                              *(t for t in (b_out, b_up, attn_tokens, b_qkv if query_norm_w is not None else None,
+                                            query_norm_w, key_norm_w) if t is not None))
         ctx.index = index
         ctx.config = (batch, token_count, width, int(num_heads), float(attn_eps), float(ffn_eps), bool(gate_first),
-                      b_qkv is not None, b_out is not None, b_up is not None, b_down is not None, attn_tokens is not None)
+                      b_qkv is not None, b_out is not None, b_up is not None, b_down is not None, attn_tokens is not None,
+                      query_norm_w is not None, float(qk_eps))
         ctx.set_materialize_grads(False)
         if attn_tokens is not None:
             attn_tokens = attn_tokens.view(batch, token_count, width) if want_attn_tokens else None
@@ -149,22 +160,25 @@ class InteractionBlockFunction(torch.autograd.Function):
     def backward(ctx, grad_output, grad_attn_tokens):
         (flat, qkv, attended, lse, key_lengths, attn_norm_w, w_qkv, w_out, ffn_norm_w, w_up, w_down, *rest) = ctx.saved_tensors
         (batch, token_count, width, num_heads, attn_eps, ffn_eps, gate_first, has_b_qkv, has_b_out, has_b_up, has_b_down,
-         has_attn_tokens) = ctx.config
+         has_attn_tokens, has_qk_norm, qk_eps) = ctx.config
         rest = list(rest)
         b_out = rest.pop(0) if has_b_out else None
         b_up = rest.pop(0) if has_b_up else None
+        attn_tokens_saved = rest.pop(0) if has_attn_tokens else None
+        b_qkv = rest.pop(0) if (has_qk_norm and has_b_qkv) else None
+        query_norm_w, key_norm_w = (rest.pop(0), rest.pop(0)) if has_qk_norm else (None, None)
         index = ctx.index.compact()
         rows, count, valid, identity = index.rows, index.count, index.valid, index.identity
         total = batch * token_count
         dtype, device = flat.dtype, flat.device
         if valid == 0:                              # no valid token: the block is the identity
             grads = [g for g in (grad_output, grad_attn_tokens) if g is not None]
-            return (sum(grads[1:], grads[0]) if grads else None,) + (None,) * 16
+            return (sum(grads[1:], grads[0]) if grads else None,) + (None,) * 19
         # the compact rows of the stream and of the tokens between the halves (gathered, or recomputed from the attention
         # output when the forward ran the one-kernel second half)
         xc = _gather_rows(flat, index)
         if has_attn_tokens:
-            x1c = _gather_rows(rest.pop(0), index)
+            x1c = _gather_rows(attn_tokens_saved, index)
         else:
             x1c = torch.empty(valid, width, dtype=dtype, device=device)
             _indexed_linear(attended, w_out, b_out, x1c, tokens=valid, out_rows=identity, count=count, x_rows=rows, residual=xc)
@@ -194,7 +208,7 @@ class InteractionBlockFunction(torch.autograd.Function):
             grad_x1_norm, weight_grads["ffn_norm"] = hip_rms_norm_backward_kernel(x1c, ffn_norm_w, grad_h2, ffn_eps)
             grad_x1c = gc.add_(grad_x1_norm) if grad_x1c is None else grad_x1c.add_(gc).add_(grad_x1_norm)
         if grad_x1c is None:
-            return (None,) * 17
+            return (None,) * 20
         # ---- out projection: weight gradient on compact rows, input gradient written into the padded layout ------------
         attended_c = _gather_rows(attended, index)
         grad_w_out, grad_b_out = _linear.linear_wgrad(grad_x1c, attended_c, with_bias=has_b_out)
@@ -219,6 +233,23 @@ class InteractionBlockFunction(torch.autograd.Function):
         _native.check(status, "interaction block (training): attention backward")
         grad_qkv_c = _gather_rows(grad_qkv, index)                                    # [valid, 3D]
         del grad_qkv, grad_attended
+        grad_query_norm = grad_key_norm = None
+        if has_qk_norm:
+            # the attention backward produced the gradients of the NORMALISED query and key: the projection's q | k columns
+            # are recomputed on the compact rows and each norm's backward runs on contiguous copies of its columns
+            qk_pre = torch.empty(valid, 2 * width, dtype=dtype, device=device)
+            _indexed_linear(xc, w_qkv[: 2 * width], None if b_qkv is None else b_qkv[: 2 * width], qk_pre, tokens=valid,
+                            out_rows=identity, count=count, x_rows=None, norm_weight=attn_norm_w, eps=attn_eps,
+                            cache_weight=False)
+            norm_grads = []
+            for part, norm_w in enumerate((query_norm_w, key_norm_w)):
+                columns = slice(part * width, (part + 1) * width)
+                grad_part, grad_w = hip_rms_norm_backward_kernel(qk_pre[:, columns].contiguous(), norm_w,
+                                                                 grad_qkv_c[:, columns].contiguous(), qk_eps)
+                grad_qkv_c[:, columns].copy_(grad_part)
+                norm_grads.append(grad_w)
+            grad_query_norm, grad_key_norm = norm_grads
+            del qk_pre
         # ---- q | k | v projection and its norm ------------------------------------------------------------------------------
         h1 = hip_rms_norm_kernel(xc, attn_norm_w, attn_eps)
         grad_w_qkv, grad_b_qkv = _linear.linear_wgrad(grad_qkv_c, h1, with_bias=has_b_qkv)
@@ -230,9 +261,9 @@ class InteractionBlockFunction(torch.autograd.Function):
                                          key_lengths.data_ptr(), rows.data_ptr() + 4 * total, grad_tokens.data_ptr(), batch,
                                          token_count, width, _native.current_stream(device))
         _native.check(status, "interaction block (training): gradient merge")
-        return (grad_tokens.view(batch, token_count, width), None, None, None, None, None, None, grad_attn_norm, grad_w_qkv,
-                grad_b_qkv, grad_w_out, grad_b_out, weight_grads["ffn_norm"], weight_grads["up"], weight_grads["b_up"],
-                weight_grads["down"], weight_grads["b_down"])
+        return (grad_tokens.view(batch, token_count, width), None, None, None, None, None, None, None, grad_attn_norm,
+                grad_w_qkv, grad_b_qkv, grad_w_out, grad_b_out, weight_grads["ffn_norm"], weight_grads["up"],
+                weight_grads["b_up"], weight_grads["down"], weight_grads["b_down"], grad_query_norm, grad_key_norm)
 
 
 def training_route_applies(block, tokens: torch.Tensor, attention_mask, key_lengths) -> bool:
@@ -244,7 +275,9 @@ def training_route_applies(block, tokens: torch.Tensor, attention_mask, key_leng
     attention, ffn = block.attention, block.ffn
     width = tokens.shape[-1]
     head_dim = width // attention.num_heads
-    if attention.query_norm is not None or attention.rope_base is not None or head_dim not in (32, 64) or width % attention.num_heads:
+    if attention.rope_base is not None or head_dim not in (32, 64) or width % attention.num_heads:
+        return False
+    if (attention.query_norm is None) != (attention.key_norm is None):
         return False
     if ffn.down.weight.shape[1] % 32 != 0:
         return False
@@ -258,7 +291,10 @@ def training_route_applies(block, tokens: torch.Tensor, attention_mask, key_leng
 def run_training_block(block, tokens: torch.Tensor, key_lengths: torch.Tensor, return_attention_tokens: bool):
     """The block through :class:`InteractionBlockFunction`."""
     attention, ffn = block.attention, block.ffn
+    qk_norm = attention.query_norm is not None
     return InteractionBlockFunction.apply(
         tokens, key_lengths, bool(return_attention_tokens), attention.num_heads, block.attn_norm.eps, block.ffn_norm.eps,
-        ffn.gate_first, block.attn_norm.weight, attention.qkv.weight, attention.qkv.bias, attention.out.weight,
-        attention.out.bias, block.ffn_norm.weight, ffn.up.weight, ffn.up.bias, ffn.down.weight, ffn.down.bias)
+        ffn.gate_first, attention.query_norm.eps if qk_norm else 1e-6, block.attn_norm.weight, attention.qkv.weight,
+        attention.qkv.bias, attention.out.weight, attention.out.bias, block.ffn_norm.weight, ffn.up.weight, ffn.up.bias,
+        ffn.down.weight, ffn.down.bias, attention.query_norm.weight if qk_norm else None,
+        attention.key_norm.weight if qk_norm else None)

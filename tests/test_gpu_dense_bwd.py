@@ -240,9 +240,11 @@ def test_interaction_block_takes_a_gradient_end_to_end(device, qk_norm):
         _close(named[parameter_name].grad, reference[name].grad)
 
 
-@pytest.mark.parametrize("d_model,heads,mult,use_attn_tokens", [(256, 8, 4, False), (256, 4, 2, True), (128, 4, 2, True)])
+@pytest.mark.parametrize("d_model,heads,mult,use_attn_tokens,qk_norm", [(256, 8, 4, False, False), (256, 4, 2, True, False),
+                                                                        (128, 4, 2, True, False), (256, 8, 4, False, True),
+                                                                        (128, 2, 2, True, True)])
 def test_block_training_route_over_the_valid_rows_equals_the_layer_by_layer_route(device, monkeypatch, d_model, heads, mult,
-                                                                                 use_attn_tokens):
+                                                                                 use_attn_tokens, qk_norm):
     """The one-function training route (valid rows compacted, gradients of the packed projection written in place)
     against the layer-by-layer autograd route of the same module: outputs, input gradient and every parameter gradient,
     with a sample of length zero, a full one, and a loss that also uses the block's second output."""
@@ -250,7 +252,7 @@ def test_block_training_route_over_the_valid_rows_equals_the_layer_by_layer_rout
 
     batch, tokens = 6, 96
     g = torch.Generator().manual_seed(d_model + heads)
-    block = UnifiedInteractionBlock(d_model, heads, mult, qk_norm=False)
+    block = UnifiedInteractionBlock(d_model, heads, mult, qk_norm=qk_norm)
     with torch.no_grad():
         for parameter in block.parameters():
             if parameter.ndim == 1:
