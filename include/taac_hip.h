@@ -268,6 +268,34 @@ int taac_flash_attn_bwd(const void* q, const void* k, const void* v, const void*
                         int is_causal, int zero_padded_queries, int dtype, void* stream);
 
 /*
+ * Training pair for attention under a mask that is not a key prefix or a causal triangle.
+ * taac_flash_attn_masked_train_fwd: taac_flash_attn_masked_fwd (structured mask, no row / feature factors) that also
+ * writes lse as taac_flash_attn_train_fwd does (-inf for rows without a visible key; the value written for a flagged
+ * self row is not used by the backward).
+ * taac_flash_attn_mask_bwd: taac_flash_attn_bwd with the visible pairs given as bytes: visible[b * visible_batch_stride +
+ * h * visible_head_stride + i * Tk + j] != 0 iff key j is visible to query i (strides in elements, 0 = shared by the
+ * batch / the heads; AND j < key_lengths[b] when key_lengths is given). An invisible pair has probability 0 in dV and dS.
+ * Any bool mask the forward applied can be written out this way; rows of flagged self queries are written as all
+ * invisible, and the caller adds dout of those rows to dv (o = v there).
+ * Replaces: what torch autograd derives for F.scaled_dot_product_attention under the bool masks of the reference's models
+ * (experiments/symbiosis/attention.py:21-60, experiments/tokenformer/model.py:474-503, flash_attention.py:183-209), which
+ * its accelerated path rejects.
+ */
+int taac_flash_attn_masked_train_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
+                                     const uint32_t* struct_bits, int64_t struct_sample_stride, const uint8_t* block_any,
+                                     const uint32_t* valid_bits, const uint32_t* self_bits, void* o, float* lse, int32_t B,
+                                     int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
+                                     const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4],
+                                     int zero_padded_queries, int dtype, void* stream);
+int taac_flash_attn_mask_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,
+                             const int32_t* key_lengths, const uint8_t* visible, int64_t visible_batch_stride,
+                             int64_t visible_head_stride, void* dq, void* dk, void* dv, float* delta, int32_t B, int32_t H,
+                             int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
+                             const int64_t v_strides[4], const int64_t o_strides[4], const int64_t do_strides[4],
+                             const int64_t dq_strides[4], const int64_t dk_strides[4], const int64_t dv_strides[4],
+                             int zero_padded_queries, int dtype, void* stream);
+
+/*
  * Training forward and backward with dropout on the attention probabilities, the mask supplied by the caller:
  * dropout_mask is uint8 [B, H, Tq, Tk] contiguous (non-zero = keep), dropout_scale = 1 / (1 - p) >= 1. The softmax
  * normaliser and lse are those of the undropped probabilities; out = ((keep ? P * dropout_scale : 0) V); the backward

@@ -558,6 +558,74 @@ class _HipFlashAttentionFunction(torch.autograd.Function):
         return dq, dk, dv, None, None, None, None, None, None
 
 
+def _visible_pairs(mask: StructuredAttentionMask, batch: int) -> tuple[torch.Tensor, int]:
+    """The pairs a structured mask lets through, written out as bytes for the backward kernels: ``(visible, batch
+    stride)`` with ``visible`` uint8 ``[Tq, Tk]`` (stride 0: no key validity, shared by the batch) or ``[B, Tq, Tk]``;
+    rows of self-only queries are all zero (their gradient is added outside the kernels). Cached on the mask."""
+    entry = mask.cache.get("visible_pairs")
+    if entry is None:
+        visible = mask.structural
+        if mask.key_valid is not None:
+            visible = visible[None, :, :] & mask.key_valid[:, None, :]
+        if mask.query_self is not None:
+            if visible.ndim == 2:
+                visible = visible[None, :, :].expand(batch, -1, -1)
+            visible = visible & ~mask.query_self[:, :, None]
+        visible = visible.to(torch.uint8).contiguous()
+        entry = mask.cache["visible_pairs"] = (visible, 0 if visible.ndim == 2 else visible.shape[1] * visible.shape[2])
+    return entry
+
+
+class _HipMaskedAttentionFunction(torch.autograd.Function):
+    """Training path under a :class:`StructuredAttentionMask`: the structured forward kernel also saves the log-sum-exp;
+    the backward kernels take the visible pairs as bytes. What torch autograd derives for SDPA under the reference models'
+    bool masks, which the reference's accelerated path rejects (flash_attention.py:183-209)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, key_lengths, mask: StructuredAttentionMask, zero_padded_queries: bool):
+        library = _native.load_library()
+        q, k, v = _kernel_view(q), _kernel_view(k), _kernel_view(v)
+        out = _dense_like(q)
+        batch, heads, query_len, head_dim = q.shape
+        if mask.sample_stride or mask.structural.shape != (query_len, k.shape[2]) \
+                or (mask.key_valid is not None and mask.key_valid.shape[0] != batch) \
+                or (mask.query_self is not None and mask.query_self.shape[0] != batch):
+            raise ValueError("flash_attention: the structured mask does not match (batch, query_len, kv_len)")
+        require_cuda_tensors("hip flash_attention", q, k, v, mask.struct_bits)
+        lse = torch.empty(batch, heads, query_len, dtype=torch.float32, device=q.device)
+        status = library.taac_flash_attn_masked_train_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), mask.struct_bits.data_ptr(), 0,
+            _native.ptr(mask.block_any), _native.ptr(mask.valid_bits), _native.ptr(mask.self_bits), out.data_ptr(),
+            lse.data_ptr(), batch, heads, query_len, k.shape[2], head_dim, _native.Int64x4(*q.stride()),
+            _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()), _native.Int64x4(*out.stride()),
+            int(bool(zero_padded_queries)), _native.dtype_code(q.dtype), _native.current_stream(q.device))
+        _native.check(status, "flash_attention")
+        ctx.save_for_backward(q, k, v, out, lse, *(() if key_lengths is None else (key_lengths,)))
+        ctx.mask, ctx.has_lengths, ctx.zero_padded_queries = mask, key_lengths is not None, bool(zero_padded_queries)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        library = _native.load_library()
+        q, k, v, out, lse, *rest = ctx.saved_tensors
+        key_lengths = rest[0] if ctx.has_lengths else None
+        batch, heads, query_len, head_dim = q.shape
+        visible, batch_stride = _visible_pairs(ctx.mask, batch)
+        grad_out = _kernel_view(grad_out)
+        dq, dk, dv = _dense_like(q), _dense_like(k), _dense_like(v)
+        delta = torch.empty_like(lse)
+        strides = [_native.Int64x4(*t.stride()) for t in (q, k, v, out, grad_out, dq, dk, dv)]
+        status = library.taac_flash_attn_mask_bwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), grad_out.data_ptr(), lse.data_ptr(),
+            _native.ptr(key_lengths), visible.data_ptr(), batch_stride, 0, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+            delta.data_ptr(), batch, heads, query_len, k.shape[2], head_dim, *strides, int(ctx.zero_padded_queries),
+            _native.dtype_code(q.dtype), _native.current_stream(q.device))
+        _native.check(status, "flash_attention backward")
+        if ctx.mask.query_self is not None:  # a self-only query returned its own value row
+            dv = dv + grad_out * ctx.mask.query_self[:, None, :, None].to(grad_out.dtype)
+        return dq, dk, dv, None, None, None
+
+
 def flash_attention(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -607,10 +675,10 @@ def flash_attention(
     if use_dropout and (structured_mask is not None or q_row_scale is not None or k_row_scale is not None
                         or q_col_scale is not None):
         raise RuntimeError("hip flash_attention dropout covers key-length and causal masks only")
-    if needs_grad and (structured_mask is not None or q_row_scale is not None or k_row_scale is not None
-                       or q_col_scale is not None or q.dtype == torch.float32):
-        raise RuntimeError("hip flash_attention backward covers bf16 / fp16 inputs under key-length and causal masks only; "
-                           "call it under torch.no_grad() for structured masks, row factors or fp32 inputs")
+    if needs_grad and (q_row_scale is not None or k_row_scale is not None or q_col_scale is not None
+                       or q.dtype == torch.float32 or (structured_mask is not None and structured_mask.sample_stride)):
+        raise RuntimeError("hip flash_attention backward covers bf16 / fp16 inputs without row factors; call it under "
+                           "torch.no_grad() for row factors, fp32 inputs or per-sample mask structure")
     if structured_mask is not None and attn_mask is not None:
         raise ValueError("flash_attention takes either attn_mask or structured_mask, not both")
     if key_lengths is not None:
@@ -632,10 +700,11 @@ def flash_attention(
         q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
     lengths = plan.key_lengths if (plan.key_lengths is not None and (attn_mask is not None or key_lengths is not None)) else None
     if needs_grad or use_dropout:
-        if structured_mask is not None:
-            raise RuntimeError("hip flash_attention backward and dropout do not cover structured masks")
         if lengths is not None:
             lengths = lengths.to(torch.int32).contiguous()
+        if structured_mask is not None:
+            output = _HipMaskedAttentionFunction.apply(q, k, v, lengths, structured_mask, zero_padded_queries)
+            return output if output.dtype == output_dtype else output.to(output_dtype)
         mask = None
         if use_dropout:
             mask = dropout_mask if dropout_mask is not None else build_dropout_mask(q, k, dropout_p)

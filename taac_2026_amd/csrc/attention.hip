@@ -1526,6 +1526,27 @@ extern "C" int taac_flash_attn_masked_fwd(const void* q, const void* k, const vo
                                0, zero_padded_queries, dtype, stream);
 }
 
+extern "C" int taac_flash_attn_masked_train_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
+                                                const uint32_t* struct_bits, int64_t struct_sample_stride,
+                                                const uint8_t* block_any, const uint32_t* valid_bits,
+                                                const uint32_t* self_bits, void* o, float* lse, int32_t B, int32_t H,
+                                                int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
+                                                const int64_t k_strides[4], const int64_t v_strides[4],
+                                                const int64_t o_strides[4], int zero_padded_queries, int dtype,
+                                                void* stream) {
+  const char* name = "taac_flash_attn_masked_train_fwd";
+  if (!struct_bits) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_bits must be given", name);
+  if (!lse && B > 0 && H > 0 && Tq > 0) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: lse must be given", name);
+  taac::MaskArgs mask;
+  mask.struct_bits = struct_bits;
+  mask.struct_stride = struct_sample_stride;
+  mask.block_any = block_any;
+  mask.valid_bits = valid_bits;
+  mask.self_bits = self_bits;
+  return taac::attention_entry(name, q, k, v, key_lengths, mask, nullptr, nullptr, nullptr, lse, nullptr, o, B, H, Tq, Tk, d,
+                               q_strides, k_strides, v_strides, o_strides, 0, zero_padded_queries, dtype, stream);
+}
+
 extern "C" int taac_flash_attn_sparse_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
                                           const uint32_t* compact_bits, int64_t compact_sample_stride,
                                           const int32_t* compact_keys, const uint64_t* compact_tiles,

@@ -37,7 +37,9 @@ struct AttnBwdParams {
   void* dk;
   void* dv;
   const int32_t* key_lengths;
-  const uint8_t* drop_mask;  // training dropout: [B, H, Tq, Tk] keep mask (non-zero = keep), or null
+  const uint8_t* drop_mask;  // byte mask with rows [Tq][Tk] at batch / head strides mask_bs / mask_hs, or null:
+                             // training dropout (keep mask, non-zero = keep) or pair visibility (non-zero = visible)
+  int64_t mask_bs, mask_hs;  // elements between the mask matrices of consecutive samples / heads (0: shared)
   float drop_scale;          // 1 / (1 - p)
   int32_t B, H, Tq, Tk, d;
   int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4];
@@ -267,10 +269,15 @@ __device__ __forceinline__ uint32_t keep_bytes4(const uint8_t* row, int key0, in
   return w;
 }
 
-// DROPOUT (both kernels): the caller's keep mask of the training forward; dV takes keep ? P / (1 - p) : 0 and the score
-// gradient P * ((keep ? dP / (1 - p) : 0) - D) / sqrt(d), as the reference's backward kernel does (tilelang.py:535-570).
-template <typename T, int DP, bool DMA, bool DROPOUT = false>
+// MODE (both kernels) says what the byte mask is. kMaskDropout: the caller's keep mask of the training forward; dV takes
+// keep ? P / (1 - p) : 0 and the score gradient P * ((keep ? dP / (1 - p) : 0) - D) / sqrt(d), as the reference's backward
+// kernel does (tilelang.py:535-570). kMaskVisible: the pairs the forward's mask let through (any bool mask, e.g. a
+// structured one written out); an invisible pair has probability 0 - the log-sum-exp was taken over the visible ones.
+constexpr int kMaskNone = 0, kMaskDropout = 1, kMaskVisible = 2;
+
+template <typename T, int DP, bool DMA, int MODE = kMaskNone>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 32 ? 4 : 3))) void attn_bwd_dq_kernel(const AttnBwdParams p) {
+  constexpr bool DROPOUT = MODE == kMaskDropout;
   typedef typename Vec8<T>::type vec_t;
   constexpr int KSTEPS = DP / 16, MB = DP / 32;
   constexpr int ROWB = DP * 2, TILE_BYTES = kChunk * ROWB, BUF_BYTES = 2 * TILE_BYTES;  // a chunk of K, then of V
@@ -382,18 +389,25 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 
         }
       }
       vec_t dsb[2];
-      if (DROPOUT) {
-        const bool aligned = (p.Tk % 4 == 0) && (reinterpret_cast<uintptr_t>(p.drop_mask) % 4 == 0);
-        const uint8_t* row = p.drop_mask + ((static_cast<int64_t>(b) * p.H + h) * p.Tq + (qi < p.Tq ? qi : 0)) * p.Tk;
+      if (MODE != kMaskNone) {
+        const bool aligned = (p.Tk % 4 == 0) && (reinterpret_cast<uintptr_t>(p.drop_mask) % 4 == 0) &&
+                             p.mask_bs % 4 == 0 && p.mask_hs % 4 == 0;
+        const uint8_t* row = p.drop_mask + b * p.mask_bs + h * p.mask_hs + static_cast<int64_t>(qi < p.Tq ? qi : 0) * p.Tk;
 #pragma unroll
         for (int jq = 0; jq < 4; ++jq) {
           const uint32_t keep = qi < p.Tq ? keep_bytes4(row, k_tile + jq * 8 + hh * 4, p.Tk, aligned) : 0u;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int j = jq * 4 + e;
-            const float prob = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -lse2));
-            const float dp = ((keep >> (8 * e)) & 0xffu) != 0u ? dpacc[j] * p.drop_scale : 0.f;
-            dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dp, p.scale, -delta_scaled));
+            const bool on = ((keep >> (8 * e)) & 0xffu) != 0u;
+            float prob = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -lse2));
+            if (DROPOUT) {
+              const float dp = on ? dpacc[j] * p.drop_scale : 0.f;
+              dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dp, p.scale, -delta_scaled));
+            } else {
+              prob = on ? prob : 0.f;
+              dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -delta_scaled));
+            }
           }
         }
       } else {
@@ -410,8 +424,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 
   store_owned<T, DP>(dqacc, smem + wave * (32 * OROW), dqb, p.dqs[2], q_begin + wave * 32, p.Tq, p.d, lane);
 }
 
-template <typename T, int DP, bool DMA, bool DROPOUT = false>
+template <typename T, int DP, bool DMA, int MODE = kMaskNone>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP == 32 ? 4 : 3) - (DMA ? 0 : 1)))) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
+  constexpr bool DROPOUT = MODE == kMaskDropout;
   typedef typename Vec8<T>::type vec_t;
   constexpr int KSTEPS = DP / 16, MB = DP / 32;
   constexpr int ROWB = DP * 2, TILE_BYTES = kChunk * ROWB;
@@ -538,14 +553,20 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int j = jq * 4 + e;
-            const float prob = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -l4[e]));
-            if (DROPOUT) {
-              // the lane owns key kj; register j is query qc0 + r0 + e: one keep byte per register
+            float prob = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -l4[e]));
+            if (MODE != kMaskNone) {
+              // the lane owns key kj; register j is query qc0 + r0 + e: one mask byte per register
               const int qrow = qc0 + r0 + e;
               const bool keep = qrow < p.Tq && kj < p.Tk &&
-                                p.drop_mask[((static_cast<int64_t>(b) * p.H + h) * p.Tq + qrow) * p.Tk + kj] != 0;
-              pb[j / 8][j % 8] = static_cast<T>(keep ? prob * p.drop_scale : 0.f);
-              dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(keep ? dpacc[j] * p.drop_scale : 0.f, p.scale, -d4[e]));
+                                p.drop_mask[b * p.mask_bs + h * p.mask_hs + static_cast<int64_t>(qrow) * p.Tk + kj] != 0;
+              if (DROPOUT) {
+                pb[j / 8][j % 8] = static_cast<T>(keep ? prob * p.drop_scale : 0.f);
+                dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(keep ? dpacc[j] * p.drop_scale : 0.f, p.scale, -d4[e]));
+              } else {
+                prob = keep ? prob : 0.f;
+                pb[j / 8][j % 8] = static_cast<T>(prob);
+                dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -d4[e]));
+              }
             } else {
               pb[j / 8][j % 8] = static_cast<T>(prob);
               dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -d4[e]));
@@ -582,41 +603,40 @@ bool small_offsets(int64_t rows, int64_t stride) {
   return stride < (1 << 22) && rows < (1 << 22) && rows * stride * 2 < (1ll << 31);
 }
 
-template <typename T, int DP>
-void launch_bwd_dp(AttnBwdParams p, bool register_staging, hipStream_t s) {
+template <typename T, int DP, int MODE>
+void launch_bwd_mode(AttnBwdParams p, bool register_staging, hipStream_t s) {
   // TAAC_ATTN_REGISTER_STAGING keeps the register-staged kernels for full head dims too (comparison route of the caller).
   const bool direct = p.d == DP && !register_staging;
-  const bool dropout = p.drop_mask != nullptr;
   p.nblk = static_cast<uint32_t>((p.Tq + kOwn - 1) / kOwn);
   p.total = p.nblk * p.B * p.H;
-  const bool dq_direct = direct && small_offsets(p.Tk, p.ks[2]) && small_offsets(p.Tk, p.vs[2]);
-  if (dq_direct && dropout)
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, DP, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
-  else if (dq_direct)
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, DP, true>), dim3(p.total), dim3(kThreads), 0, s, p);
-  else if (dropout)
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, DP, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  if (direct && small_offsets(p.Tk, p.ks[2]) && small_offsets(p.Tk, p.vs[2]))
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, DP, true, MODE>), dim3(p.total), dim3(kThreads), 0, s, p);
   else
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, DP, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, DP, false, MODE>), dim3(p.total), dim3(kThreads), 0, s, p);
   p.nblk = static_cast<uint32_t>((p.Tk + kOwn - 1) / kOwn);
   p.total = p.nblk * p.B * p.H;
-  const bool dkv_direct = direct && small_offsets(p.Tq, p.qs[2]) && small_offsets(p.Tq, p.dos[2]);
-  if (dkv_direct && dropout)
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, DP, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
-  else if (dkv_direct)
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, DP, true>), dim3(p.total), dim3(kThreads), 0, s, p);
-  else if (dropout)
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, DP, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  if (direct && small_offsets(p.Tq, p.qs[2]) && small_offsets(p.Tq, p.dos[2]))
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, DP, true, MODE>), dim3(p.total), dim3(kThreads), 0, s, p);
   else
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, DP, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, DP, false, MODE>), dim3(p.total), dim3(kThreads), 0, s, p);
+}
+
+template <typename T, int DP>
+void launch_bwd_dp(const AttnBwdParams& p, int mode, bool register_staging, hipStream_t s) {
+  if (mode == kMaskDropout)
+    launch_bwd_mode<T, DP, kMaskDropout>(p, register_staging, s);
+  else if (mode == kMaskVisible)
+    launch_bwd_mode<T, DP, kMaskVisible>(p, register_staging, s);
+  else
+    launch_bwd_mode<T, DP, kMaskNone>(p, register_staging, s);
 }
 
 template <typename T>
-void launch_bwd(const AttnBwdParams& p, bool register_staging, hipStream_t s) {
+void launch_bwd(const AttnBwdParams& p, int mode, bool register_staging, hipStream_t s) {
   if (p.d <= 32)
-    launch_bwd_dp<T, 32>(p, register_staging, s);
+    launch_bwd_dp<T, 32>(p, mode, register_staging, s);
   else
-    launch_bwd_dp<T, 64>(p, register_staging, s);
+    launch_bwd_dp<T, 64>(p, mode, register_staging, s);
 }
 
 }  // namespace
@@ -630,7 +650,14 @@ int attention_bwd_entry(const char* name, const void* q, const void* k, const vo
                         const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
                         const int64_t o_strides[4], const int64_t do_strides[4], const int64_t dq_strides[4],
                         const int64_t dk_strides[4], const int64_t dv_strides[4], int is_causal, int zero_padded_queries,
-                        int dtype, void* stream) {
+                        int dtype, void* stream, int mask_mode = -1, int64_t mask_bs = 0, int64_t mask_hs = 0) {
+  // mask_mode -1: dropout when a mask is given (its matrices follow the (B, H) order), nothing otherwise
+  if (mask_mode < 0) {
+    mask_mode = drop_mask != nullptr ? kMaskDropout : kMaskNone;
+    mask_hs = static_cast<int64_t>(Tq) * Tk;
+    mask_bs = mask_hs * H;
+  }
+  if (mask_bs < 0 || mask_hs < 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: negative mask stride", name);
   if (drop_mask != nullptr && !(drop_scale >= 1.f))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: dropout_scale = 1 / (1 - p) must be >= 1", name);
   if (B < 0 || H < 0 || Tq < 0 || Tk < 0 || d <= 0)
@@ -672,6 +699,8 @@ int attention_bwd_entry(const char* name, const void* q, const void* k, const vo
   p.dv = dv;
   p.key_lengths = key_lengths;
   p.drop_mask = drop_mask;
+  p.mask_bs = mask_bs;
+  p.mask_hs = mask_hs;
   p.drop_scale = drop_scale;
   p.B = B;
   p.H = H;
@@ -693,9 +722,9 @@ int attention_bwd_entry(const char* name, const void* q, const void* k, const vo
   p.causal = (is_causal & TAAC_ATTN_CAUSAL) ? 1 : 0;
   hipStream_t s = as_stream(stream);
   if (dtype == TAAC_BF16)
-    launch_bwd<bf16_t>(p, register_staging, s);
+    launch_bwd<bf16_t>(p, mask_mode, register_staging, s);
   else
-    launch_bwd<f16_t>(p, register_staging, s);
+    launch_bwd<f16_t>(p, mask_mode, register_staging, s);
   return check_launch(name);
 }
 }  // namespace
@@ -727,4 +756,20 @@ extern "C" int taac_flash_attn_dropout_bwd(const void* q, const void* k, const v
   return taac::attention_bwd_entry(name, q, k, v, o, dout, lse, key_lengths, dropout_mask, dropout_scale, dq, dk, dv, delta,
                                    B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides, do_strides, dq_strides,
                                    dk_strides, dv_strides, is_causal, zero_padded_queries, dtype, stream);
+}
+
+extern "C" int taac_flash_attn_mask_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout,
+                                        const float* lse, const int32_t* key_lengths, const uint8_t* visible,
+                                        int64_t visible_batch_stride, int64_t visible_head_stride, void* dq, void* dk,
+                                        void* dv, float* delta, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                                        const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
+                                        const int64_t o_strides[4], const int64_t do_strides[4],
+                                        const int64_t dq_strides[4], const int64_t dk_strides[4],
+                                        const int64_t dv_strides[4], int zero_padded_queries, int dtype, void* stream) {
+  const char* name = "taac_flash_attn_mask_bwd";
+  if (!visible) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: the visibility mask must be given", name);
+  return taac::attention_bwd_entry(name, q, k, v, o, dout, lse, key_lengths, visible, 1.f, dq, dk, dv, delta, B, H, Tq, Tk, d,
+                                   q_strides, k_strides, v_strides, o_strides, do_strides, dq_strides, dk_strides,
+                                   dv_strides, 0, zero_padded_queries, dtype, stream, taac::kMaskVisible,
+                                   visible_batch_stride, visible_head_stride);
 }

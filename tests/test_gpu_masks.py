@@ -266,3 +266,141 @@ def test_compact_tables_follow_their_definition(device):
                 chunk = columns[c * 32:(c + 1) * 32]
                 expected = sum(1 << j for j, key in enumerate(chunk) if bool(rows[r, key]))
                 assert int(bits[0, tile * 32 + r, c]) & 0xffffffff == expected
+
+
+# ---- training under structured masks ---------------------------------------------------------------------------------
+
+# Gradient tolerance of the reference's GPU tests for 16-bit attention (tests/gpu/infrastructure/accelerators/
+# test_tilelang_ops_cuda.py:98-141): 3e-2.
+GRAD_TOL = dict(rtol=3e-2, atol=3e-2)
+
+
+def _autograd_expected(q, k, v, dense, grad_out):
+    """float64 autograd of the oracle's SDPA under the dense bool mask (what the reference's models train with,
+    flash_attention.py:552-570); rows without a visible key are zeros and pass no gradient."""
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    empty = ~dense.any(dim=-1, keepdim=True)
+    out = oracle.sdpa(qr, kr, vr, dense | empty)
+    out = torch.where(empty.expand(-1, q.shape[1], -1, -1), torch.zeros_like(out), out)
+    out.backward(grad_out.double())
+    return out.detach(), qr.grad, kr.grad, vr.grad
+
+
+def _check_training(device, q, k, v, mask, grad_out, key_lengths=None, dense=None):
+    dense = mask.dense().cpu() if dense is None else dense
+    want_out, *want_grads = _autograd_expected(q, k, v, dense, grad_out)
+    qd, kd, vd = (t.to(device).requires_grad_(True) for t in (q, k, v))
+    out = flash_attention(qd, kd, vd, structured_mask=mask, key_lengths=key_lengths)
+    with torch.no_grad():
+        serving = flash_attention(qd, kd, vd, structured_mask=mask, key_lengths=key_lengths)
+    if mask.sparse:                                    # serving prefers the per-tile kernel there; training runs the chunked one
+        torch.testing.assert_close(out.detach().float(), serving.float(), rtol=2 ** -6, atol=2 ** -6)
+    else:                                              # the training forward is the serving kernel plus the log-sum-exp
+        assert torch.equal(out.detach(), serving)
+    out.backward(grad_out.to(device))
+    torch.testing.assert_close(out.detach().cpu().double(), want_out, **BF16_TOL)
+    for got, want, name in zip((qd.grad, kd.grad, vd.grad), want_grads, ("dq", "dk", "dv")):
+        assert got.dtype == q.dtype and got.shape == want.shape
+        torch.testing.assert_close(got.cpu().double(), want, msg=lambda m, n=name: f"{n}: {m}", **GRAD_TOL)
+    return qd.grad.cpu(), kd.grad.cpu(), vd.grad.cpu()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tokens,dim", [(50, 32), (130, 64), (300, 32), (257, 16), (96, 48)])
+def test_structured_masks_take_a_gradient(device, dtype, tokens, dim):
+    """Random structure, invalid keys, self-only queries and a query that sees nothing: the gradients equal float64
+    autograd under the dense mask; invisible keys and the empty query row receive exactly zero."""
+    batch, heads = 3, 2
+    g = torch.Generator().manual_seed(tokens * 3 + dim)
+    q, k, v, grad_out = (torch.randn(batch, heads, tokens, dim, generator=g).to(dtype) for _ in range(4))
+    structural = torch.rand(tokens, tokens, generator=g) < 0.4
+    structural[tokens // 3] = False
+    key_valid = torch.rand(batch, tokens, generator=g) < 0.7
+    key_valid[1] = True
+    query_self = torch.rand(batch, tokens, generator=g) < 0.1
+    query_self[:, tokens // 3] = False
+    for mask in (build_structured_mask(structural.to(device), key_valid.to(device), query_self.to(device)),
+                 build_structured_mask(structural.to(device), key_valid.to(device)),
+                 build_structured_mask(structural.to(device))):
+        dq, dk, dv = _check_training(device, q, k, v, mask, grad_out)
+        assert dq[:, :, tokens // 3].abs().max().item() == 0.0
+        if mask.key_valid is not None and mask.query_self is None:
+            dead = ~key_valid[:, None, :, None].expand_as(dk)
+            assert dk[dead].abs().max().item() == 0.0 and dv[dead].abs().max().item() == 0.0
+        if mask.query_self is not None:                # a self-only query passes its gradient to its own value row only
+            flagged = query_self[:, None, :, None].expand_as(dq)
+            assert dq[flagged].abs().max().item() == 0.0
+
+
+def test_model_masks_take_a_gradient(device):
+    """The masks the reference's models build: TokenFormer layers (full, first and narrowest window, padded queries keep
+    themselves - experiments/tokenformer/model.py:474-503) and the Symbiosis role mask
+    (experiments/symbiosis/attention.py:21-60)."""
+    batch, heads, dim, layers = 3, 2, 32, 6
+    roles = torch.tensor([0] * 20 + [4] + [1] * 460 + [4] + [2] * 20 + [5] * 9 + [3])
+    tokens = roles.numel()
+    padding = torch.zeros(batch, tokens, dtype=torch.bool)
+    padding[1, 200:481] = True
+    padding[2, 21 + 37:481] = True
+    padding[2, 5] = True
+    g = torch.Generator().manual_seed(11)
+    q, k, v, grad_out = (torch.randn(batch, heads, tokens, dim, generator=g).to(torch.bfloat16) for _ in range(4))
+    for layer in (0, 3, 5):
+        mask = bfts_attention_mask(padding.to(device), roles.to(device), layer, layers, seq_causal=True, seq_keep_per_domain=64)
+        _check_training(device, q, k, v, mask, grad_out)
+    roles = torch.tensor([0, 1] + [2] * 9 + [3] * 7 + [4] * 3 + [5] * 2 + [6] * 150 + [7] * 4)
+    tokens = roles.numel()
+    padding = torch.rand(4, tokens, generator=g) < 0.3
+    padding[:, :2] = False
+    padding[3] = True
+    q, k, v, grad_out = (torch.randn(4, 4, tokens, 64, generator=g).to(torch.bfloat16) for _ in range(4))
+    mask = MetadataAttentionMask(enabled=True)(padding.to(device), roles.to(device))
+    _check_training(device, q, k, v, mask, grad_out)
+
+
+def test_structured_mask_gradient_with_key_lengths(device):
+    """``key_lengths`` on top of the structure (keys beyond the prefix invisible, padded query rows zero)."""
+    batch, heads, tokens, dim = 3, 2, 200, 32
+    g = torch.Generator().manual_seed(4)
+    q, k, v, grad_out = (torch.randn(batch, heads, tokens, dim, generator=g).to(torch.bfloat16) for _ in range(4))
+    structural = torch.tril(torch.ones(tokens, tokens, dtype=torch.bool)) & (torch.rand(tokens, tokens, generator=g) < 0.8)
+    structural |= torch.eye(tokens, dtype=torch.bool)
+    lengths = torch.tensor([200, 33, 129], dtype=torch.int32)
+    inside = torch.arange(tokens)[None, :] < lengths[:, None]
+    dense = (structural[None] & inside[:, None, :])[:, None]
+    mask = build_structured_mask(structural.to(device))
+    _check_training(device, q, k, v, mask, grad_out, key_lengths=lengths.to(device), dense=dense)
+
+
+@pytest.mark.parametrize("per_head,per_sample", [(True, True), (False, True), (True, False), (False, False)])
+def test_mask_bwd_abi_reads_any_bool_mask(device, per_head, per_sample):
+    """``taac_flash_attn_mask_bwd`` alone: a random mask per sample and / or head (strides 0 = shared), the log-sum-exp
+    and the output taken from the float64 reference."""
+    from taac_2026_amd import _native
+
+    batch, heads, tokens, dim = 2, 3, 150, 64
+    g = torch.Generator().manual_seed(int(per_head) * 2 + int(per_sample))
+    q, k, v, grad_out = (torch.randn(batch, heads, tokens, dim, generator=g).to(torch.bfloat16) for _ in range(4))
+    visible = torch.rand(batch if per_sample else 1, heads if per_head else 1, tokens, tokens, generator=g) < 0.5
+    visible[..., 0] = True                              # every query sees a key
+    dense = visible.expand(batch, heads, -1, -1)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    scores = (qr @ kr.transpose(-1, -2)) / dim ** 0.5
+    scores = scores.masked_fill(~dense, float("-inf"))
+    lse = torch.logsumexp(scores, dim=-1)
+    out = torch.softmax(scores, dim=-1) @ vr
+    out.backward(grad_out.double())
+    dev = [t.to(device) for t in (q, k, v, out.detach().to(torch.bfloat16), grad_out)]
+    lse_d = lse.detach().float().to(device)
+    vis_d = visible.to(torch.uint8).contiguous().to(device)
+    grads = [torch.empty_like(dev[0]) for _ in range(3)]
+    delta = torch.empty_like(lse_d)
+    strides = [_native.Int64x4(*t.stride()) for t in (*dev, *grads)]
+    status = _native.load_library().taac_flash_attn_mask_bwd(
+        *(t.data_ptr() for t in dev), lse_d.data_ptr(), None, vis_d.data_ptr(),
+        heads * tokens * tokens if per_sample and per_head else (tokens * tokens if per_sample else 0),
+        tokens * tokens if per_head else 0, *(t.data_ptr() for t in grads), delta.data_ptr(), batch, heads, tokens,
+        tokens, dim, *strides, 0, _native.dtype_code(torch.bfloat16), _native.current_stream(dev[0].device))
+    _native.check(status, "taac_flash_attn_mask_bwd")
+    for got, want, name in zip(grads, (qr.grad, kr.grad, vr.grad), ("dq", "dk", "dv")):
+        torch.testing.assert_close(got.cpu().double(), want, msg=lambda m, n=name: f"{n}: {m}", **GRAD_TOL)
