@@ -337,6 +337,35 @@ def _training_block_figures(device, with_comparison: bool = True) -> dict:
                 backbone_module.training_route_applies = applies
         figures[label] = entry
         del block, x
+    # the reference block as its model trains it: query / key norms, the role mask, padding scattered inside the sequence
+    # part (the workload of the reference_block figures)
+    from taac_2026_amd.api import MetadataAttentionMask
+
+    g = torch.Generator().manual_seed(42)
+    roles = torch.tensor([0] * 16 + [2] * 15 + [3] + [1] * (tokens - 32), device=device)
+    keep_fraction = torch.rand(batch, 1, generator=g) * 0.9 + 0.1
+    scattered = torch.cat([torch.zeros(batch, 32, dtype=torch.bool),
+                           torch.rand(batch, tokens - 32, generator=g) > keep_fraction], dim=1).to(device)
+    mask = MetadataAttentionMask(enabled=True)(scattered, roles)
+    torch.manual_seed(0)
+    block = UnifiedInteractionBlock(width, inputs.num_heads, 4, qk_norm=True).to(torch.bfloat16).to(device).train()
+    x = inputs.emb.to(device).requires_grad_(True)
+
+    def masked_step():
+        out, _ = block(x, scattered, mask, return_attention_tokens=False)
+        out.backward(grad)
+        block.zero_grad(set_to_none=True)
+        x.grad = None
+
+    entry = {"valid_token_fraction": 1.0 - float(scattered.float().mean().item()), "valid_rows_ms": _event_ms(masked_step, 5, 3)}
+    if with_comparison:
+        applies = backbone_module.training_route_applies
+        backbone_module.training_route_applies = lambda *a, **k: False
+        try:
+            entry["layer_by_layer_ms"] = _event_ms(masked_step, 3, 2)
+        finally:
+            backbone_module.training_route_applies = applies
+    figures["query_key_norm_role_mask_scattered_padding"] = entry
     return {"interaction_block_training_step_B1024_T512": figures}
 
 

@@ -274,7 +274,10 @@ int taac_flash_attn_bwd(const void* q, const void* k, const void* v, const void*
  * self row is not used by the backward).
  * taac_flash_attn_mask_bwd: taac_flash_attn_bwd with the visible pairs given as bytes: visible[b * visible_batch_stride +
  * h * visible_head_stride + i * Tk + j] != 0 iff key j is visible to query i (strides in elements, 0 = shared by the
- * batch / the heads; AND j < key_lengths[b] when key_lengths is given). An invisible pair has probability 0 in dV and dS.
+ * batch / the heads; AND j < key_lengths[b] when key_lengths is given; AND key_valid[b * Tk + j] != 0 when key_valid is
+ * given - the factored form structure[i, j] & key_valid[b, j] then needs one shared matrix and B * Tk bytes instead of B
+ * matrices). An invisible pair has probability 0 in dV and dS. A query row whose lse is +inf contributes nothing and
+ * receives a zero gradient (how a caller takes rows out: the self-only rows of a structured mask).
  * Any bool mask the forward applied can be written out this way; rows of flagged self queries are written as all
  * invisible, and the caller adds dout of those rows to dv (o = v there).
  * Replaces: what torch autograd derives for F.scaled_dot_product_attention under the bool masks of the reference's models
@@ -289,7 +292,8 @@ int taac_flash_attn_masked_train_fwd(const void* q, const void* k, const void* v
                                      int zero_padded_queries, int dtype, void* stream);
 int taac_flash_attn_mask_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,
                              const int32_t* key_lengths, const uint8_t* visible, int64_t visible_batch_stride,
-                             int64_t visible_head_stride, void* dq, void* dk, void* dv, float* delta, int32_t B, int32_t H,
+                             int64_t visible_head_stride, const uint8_t* key_valid, void* dq, void* dk, void* dv,
+                             float* delta, int32_t B, int32_t H,
                              int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
                              const int64_t v_strides[4], const int64_t o_strides[4], const int64_t do_strides[4],
                              const int64_t dq_strides[4], const int64_t dk_strides[4], const int64_t dv_strides[4],
@@ -527,6 +531,33 @@ int taac_rows_gather(const void* src, int64_t ld_src, const int32_t* rows, int64
  */
 int taac_rows_merge(const void* padded, const void* compact_a, const void* compact_b, const int32_t* key_lengths,
                     const int32_t* offsets, void* out, int32_t B, int32_t T, int32_t W, void* stream);
+
+/*
+ * taac_flash_attn_mask_bwd with the mask in the bit form of taac_flash_attn_masked_train_fwd: struct_bits rows of
+ * ceil(Tk / 32) words per query (struct_sample_stride words between the matrices of consecutive samples, 0 = one matrix
+ * for the batch), valid_bits [B, ceil(Tk / 32)] or NULL; pair (i, j) of sample b is visible iff both bits are set (and
+ * j < key_lengths[b] when key_lengths is given). One word per 32-key tile where the byte form reads 32 bytes. With the
+ * samples' valid tokens at the front of their rows (taac_front_rows, taac_mask_front_bits) and key_lengths = their
+ * numbers, the cost follows the valid tokens as in taac_flash_attn_bwd.
+ * Replaces: as taac_flash_attn_mask_bwd.
+ */
+int taac_flash_attn_bits_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,
+                             const int32_t* key_lengths, const uint32_t* struct_bits, int64_t struct_sample_stride,
+                             const uint32_t* valid_bits, void* dq, void* dk, void* dv, float* delta, int32_t B, int32_t H,
+                             int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
+                             const int64_t v_strides[4], const int64_t o_strides[4], const int64_t do_strides[4],
+                             const int64_t dq_strides[4], const int64_t dk_strides[4], const int64_t dv_strides[4],
+                             int zero_padded_queries, int dtype, void* stream);
+
+/*
+ * taac_rows_merge for padding that is not a prefix: token t of sample b is valid iff bit t of valid_bits[b] is set (rows
+ * of ceil(T / 32) words, as for taac_valid_rows_from_bits, whose per-sample offsets are `offsets`); its compact row is
+ * offsets[b] + the number of valid tokens of the sample in front of it.
+ * Replaces: the same `update * ~padding_mask` + residual arithmetic under the scattered padding of the reference's
+ * token layout (experiments/symbiosis/backbone.py:58-68, experiments/symbiosis/attention.py:21-60).
+ */
+int taac_rows_merge_bits(const void* padded, const void* compact_a, const void* compact_b, const uint32_t* valid_bits,
+                         const int32_t* offsets, void* out, int32_t B, int32_t T, int32_t W, void* stream);
 
 /*
  * The same row index for padding that is not a prefix: token t of sample b is valid iff bit t of valid_bits[b] is set

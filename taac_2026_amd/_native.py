@@ -136,6 +136,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "taac_rows_gather": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int32, c_void_p]),
     "taac_rows_merge": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p]),
+    "taac_rows_merge_bits": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p]),
     "taac_swiglu_ffn_bwd_packed_bytes": (c_int64, [c_int32, c_int32]),
     "taac_swiglu_ffn_bwd_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
     "taac_swiglu_ffn_bwd_hidden": (
@@ -149,8 +150,12 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "taac_flash_attn_mask_bwd": (
         c_int,
-        [c_void_p] * 8 + [c_int64, c_int64] + [c_void_p] * 4 + [c_int32] * 5 + [ctypes.POINTER(c_int64)] * 8
+        [c_void_p] * 8 + [c_int64, c_int64] + [c_void_p] * 5 + [c_int32] * 5 + [ctypes.POINTER(c_int64)] * 8
         + [c_int, c_int, c_void_p],
+    ),
+    "taac_flash_attn_bits_bwd": (
+        c_int,
+        [c_void_p] * 8 + [c_int64] + [c_void_p] * 5 + [c_int32] * 5 + [ctypes.POINTER(c_int64)] * 8 + [c_int, c_int, c_void_p],
     ),
     "taac_flash_attn_train_dropout_fwd": (
         c_int,

@@ -558,22 +558,26 @@ class _HipFlashAttentionFunction(torch.autograd.Function):
         return dq, dk, dv, None, None, None, None, None, None
 
 
-def _visible_pairs(mask: StructuredAttentionMask, batch: int) -> tuple[torch.Tensor, int]:
-    """The pairs a structured mask lets through, written out as bytes for the backward kernels: ``(visible, batch
-    stride)`` with ``visible`` uint8 ``[Tq, Tk]`` (stride 0: no key validity, shared by the batch) or ``[B, Tq, Tk]``;
-    rows of self-only queries are all zero (their gradient is added outside the kernels). Cached on the mask."""
-    entry = mask.cache.get("visible_pairs")
-    if entry is None:
-        visible = mask.structural
-        if mask.key_valid is not None:
-            visible = visible[None, :, :] & mask.key_valid[:, None, :]
-        if mask.query_self is not None:
-            if visible.ndim == 2:
-                visible = visible[None, :, :].expand(batch, -1, -1)
-            visible = visible & ~mask.query_self[:, :, None]
-        visible = visible.to(torch.uint8).contiguous()
-        entry = mask.cache["visible_pairs"] = (visible, 0 if visible.ndim == 2 else visible.shape[1] * visible.shape[2])
-    return entry
+def masked_attention_backward(q, k, v, out, grad_out, lse, key_lengths, mask: StructuredAttentionMask, dq, dk, dv, *,
+                              zero_padded_queries: bool = False) -> None:
+    """``taac_flash_attn_bits_bwd`` for (B, H, T, d) views under a structured mask (either layout: one structure for the
+    batch, or one per sample with the valid tokens in front), writing into ``dq`` / ``dk`` / ``dv`` (any element strides
+    with a unit last one). A self-only query returned its own value row: its row is taken out of the kernels
+    (log-sum-exp +inf: zero probabilities) and ``grad_out`` of that row is added to ``dv``."""
+    library = _native.load_library()
+    batch, heads, query_len, head_dim = q.shape
+    if mask.query_self is not None:
+        lse = torch.where(mask.query_self[:, None, :], torch.full_like(lse, float("inf")), lse)
+    delta = torch.empty_like(lse)
+    strides = [_native.Int64x4(*t.stride()) for t in (q, k, v, out, grad_out, dq, dk, dv)]
+    status = library.taac_flash_attn_bits_bwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), grad_out.data_ptr(), lse.data_ptr(),
+        _native.ptr(key_lengths), mask.struct_bits.data_ptr(), int(mask.sample_stride), _native.ptr(mask.valid_bits),
+        dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(), batch, heads, query_len, k.shape[2], head_dim,
+        *strides, int(bool(zero_padded_queries)), _native.dtype_code(q.dtype), _native.current_stream(q.device))
+    _native.check(status, "flash_attention backward")
+    if mask.query_self is not None:
+        dv.add_(grad_out * mask.query_self[:, None, :, None].to(grad_out.dtype))
 
 
 class _HipMaskedAttentionFunction(torch.autograd.Function):
@@ -587,15 +591,17 @@ class _HipMaskedAttentionFunction(torch.autograd.Function):
         q, k, v = _kernel_view(q), _kernel_view(k), _kernel_view(v)
         out = _dense_like(q)
         batch, heads, query_len, head_dim = q.shape
-        if mask.sample_stride or mask.structural.shape != (query_len, k.shape[2]) \
+        if mask.structural.shape != (query_len, k.shape[2]) \
                 or (mask.key_valid is not None and mask.key_valid.shape[0] != batch) \
-                or (mask.query_self is not None and mask.query_self.shape[0] != batch):
+                or (mask.query_self is not None and mask.query_self.shape[0] != batch) \
+                or (mask.sample_stride and mask.struct_bits.shape[0] != batch * query_len):
             raise ValueError("flash_attention: the structured mask does not match (batch, query_len, kv_len)")
         require_cuda_tensors("hip flash_attention", q, k, v, mask.struct_bits)
         lse = torch.empty(batch, heads, query_len, dtype=torch.float32, device=q.device)
         status = library.taac_flash_attn_masked_train_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), mask.struct_bits.data_ptr(), 0,
-            _native.ptr(mask.block_any), _native.ptr(mask.valid_bits), _native.ptr(mask.self_bits), out.data_ptr(),
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), mask.struct_bits.data_ptr(),
+            int(mask.sample_stride), _native.ptr(mask.block_any), _native.ptr(mask.valid_bits), _native.ptr(mask.self_bits),
+            out.data_ptr(),
             lse.data_ptr(), batch, heads, query_len, k.shape[2], head_dim, _native.Int64x4(*q.stride()),
             _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()), _native.Int64x4(*out.stride()),
             int(bool(zero_padded_queries)), _native.dtype_code(q.dtype), _native.current_stream(q.device))
@@ -606,23 +612,12 @@ class _HipMaskedAttentionFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_out):
-        library = _native.load_library()
         q, k, v, out, lse, *rest = ctx.saved_tensors
         key_lengths = rest[0] if ctx.has_lengths else None
-        batch, heads, query_len, head_dim = q.shape
-        visible, batch_stride = _visible_pairs(ctx.mask, batch)
         grad_out = _kernel_view(grad_out)
         dq, dk, dv = _dense_like(q), _dense_like(k), _dense_like(v)
-        delta = torch.empty_like(lse)
-        strides = [_native.Int64x4(*t.stride()) for t in (q, k, v, out, grad_out, dq, dk, dv)]
-        status = library.taac_flash_attn_mask_bwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), grad_out.data_ptr(), lse.data_ptr(),
-            _native.ptr(key_lengths), visible.data_ptr(), batch_stride, 0, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-            delta.data_ptr(), batch, heads, query_len, k.shape[2], head_dim, *strides, int(ctx.zero_padded_queries),
-            _native.dtype_code(q.dtype), _native.current_stream(q.device))
-        _native.check(status, "flash_attention backward")
-        if ctx.mask.query_self is not None:  # a self-only query returned its own value row
-            dv = dv + grad_out * ctx.mask.query_self[:, None, :, None].to(grad_out.dtype)
+        masked_attention_backward(q, k, v, out, grad_out, lse, key_lengths, ctx.mask, dq, dk, dv,
+                                  zero_padded_queries=ctx.zero_padded_queries)
         return dq, dk, dv, None, None, None
 
 
@@ -676,9 +671,9 @@ def flash_attention(
                         or q_col_scale is not None):
         raise RuntimeError("hip flash_attention dropout covers key-length and causal masks only")
     if needs_grad and (q_row_scale is not None or k_row_scale is not None or q_col_scale is not None
-                       or q.dtype == torch.float32 or (structured_mask is not None and structured_mask.sample_stride)):
+                       or q.dtype == torch.float32):
         raise RuntimeError("hip flash_attention backward covers bf16 / fp16 inputs without row factors; call it under "
-                           "torch.no_grad() for row factors, fp32 inputs or per-sample mask structure")
+                           "torch.no_grad() for row factors or fp32 inputs")
     if structured_mask is not None and attn_mask is not None:
         raise ValueError("flash_attention takes either attn_mask or structured_mask, not both")
     if key_lengths is not None:

@@ -40,6 +40,7 @@ struct AttnBwdParams {
   const uint8_t* drop_mask;  // byte mask with rows [Tq][Tk] at batch / head strides mask_bs / mask_hs, or null:
                              // training dropout (keep mask, non-zero = keep) or pair visibility (non-zero = visible)
   int64_t mask_bs, mask_hs;  // elements between the mask matrices of consecutive samples / heads (0: shared)
+  const uint8_t* key_valid;  // visibility mode: [B, Tk] bytes, non-zero = the key can be seen at all; or null
   float drop_scale;          // 1 / (1 - p)
   int32_t B, H, Tq, Tk, d;
   int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4];
@@ -273,7 +274,10 @@ __device__ __forceinline__ uint32_t keep_bytes4(const uint8_t* row, int key0, in
 // keep ? P / (1 - p) : 0 and the score gradient P * ((keep ? dP / (1 - p) : 0) - D) / sqrt(d), as the reference's backward
 // kernel does (tilelang.py:535-570). kMaskVisible: the pairs the forward's mask let through (any bool mask, e.g. a
 // structured one written out); an invisible pair has probability 0 - the log-sum-exp was taken over the visible ones.
-constexpr int kMaskNone = 0, kMaskDropout = 1, kMaskVisible = 2;
+// kMaskBits: the same as bits, in the layout of the structured forward: drop_mask holds 32-bit words, row i of a sample's
+// matrix at word (b * mask_bs + i * wpr), wpr = ceil(Tk / 32), bit j % 32 of word j / 32 = pair (i, j); key_valid holds
+// [B, wpr] words. One word per 32-key tile instead of 32 bytes.
+constexpr int kMaskNone = 0, kMaskDropout = 1, kMaskVisible = 2, kMaskBits = 3;
 
 template <typename T, int DP, bool DMA, int MODE = kMaskNone>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 32 ? 4 : 3))) void attn_bwd_dq_kernel(const AttnBwdParams p) {
@@ -346,9 +350,25 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 
   };
   const uint32_t row_off = streamed_row_offset<DP>(l32, hh);
   const uint32_t col_off = streamed_column_offset<DP>(lane);
+  // bit mode: the lane's query row of the mask, two words (64 keys) per chunk, requested one chunk ahead of their use
+  [[maybe_unused]] uint32_t chunk_words[kChunk / 32] = {}, next_words[kChunk / 32] = {};
+  auto fetch_words = [&](int kc0, uint32_t (&dst)[kChunk / 32]) {
+    const int wpr = (p.Tk + 31) / 32;
+    const uint32_t* row = reinterpret_cast<const uint32_t*>(p.drop_mask) + b * p.mask_bs + static_cast<int64_t>(qi < p.Tq ? qi : 0) * wpr;
+    const uint32_t* valid = p.key_valid != nullptr ? reinterpret_cast<const uint32_t*>(p.key_valid) + static_cast<int64_t>(b) * wpr : nullptr;
+#pragma unroll
+    for (int t = 0; t < kChunk / 32; ++t) {
+      const int w = kc0 / 32 + t;
+      const bool inside = qi < p.Tq && w < wpr;  // a tile at or beyond Tk has no word
+      dst[t] = inside ? row[w] : 0u;
+      if (inside && valid != nullptr) dst[t] &= valid[w];
+    }
+  };
+  if (MODE == kMaskBits && kv_end > 0) fetch_words(0, chunk_words);
   if (kv_end > 0) fetch(0, 0);
   int buf = 0;
   for (int kc0 = 0; kc0 < kv_end; kc0 += kChunk) {
+    if (MODE == kMaskBits && kc0 + kChunk < kv_end) fetch_words(kc0 + kChunk, next_words);
     if (DMA) {
       vm_wait<0>();     // this wavefront's pieces of the chunk have landed ...
       __syncthreads();  // ... everyone's have, and everyone is done reading the other buffer
@@ -389,17 +409,29 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 
         }
       }
       vec_t dsb[2];
-      if (MODE != kMaskNone) {
+      if (MODE == kMaskBits) {
+        const uint32_t word = chunk_words[kt];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const bool on = ((word >> ((j / 4) * 8 + hh * 4 + (j % 4))) & 1u) != 0u;
+          const float prob = on ? __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -lse2)) : 0.f;
+          dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -delta_scaled));
+        }
+      } else if (MODE != kMaskNone) {
         const bool aligned = (p.Tk % 4 == 0) && (reinterpret_cast<uintptr_t>(p.drop_mask) % 4 == 0) &&
                              p.mask_bs % 4 == 0 && p.mask_hs % 4 == 0;
         const uint8_t* row = p.drop_mask + b * p.mask_bs + h * p.mask_hs + static_cast<int64_t>(qi < p.Tq ? qi : 0) * p.Tk;
+        const bool with_valid = MODE == kMaskVisible && p.key_valid != nullptr;  // uniform
+        const uint8_t* valid_row = with_valid ? p.key_valid + static_cast<int64_t>(b) * p.Tk : nullptr;
+        const bool valid_aligned = with_valid && (p.Tk % 4 == 0) && (reinterpret_cast<uintptr_t>(p.key_valid) % 4 == 0);
 #pragma unroll
         for (int jq = 0; jq < 4; ++jq) {
           const uint32_t keep = qi < p.Tq ? keep_bytes4(row, k_tile + jq * 8 + hh * 4, p.Tk, aligned) : 0u;
+          const uint32_t kval = with_valid ? keep_bytes4(valid_row, k_tile + jq * 8 + hh * 4, p.Tk, valid_aligned) : ~0u;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int j = jq * 4 + e;
-            const bool on = ((keep >> (8 * e)) & 0xffu) != 0u;
+            const bool on = ((keep >> (8 * e)) & 0xffu) != 0u && ((kval >> (8 * e)) & 0xffu) != 0u;
             float prob = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -lse2));
             if (DROPOUT) {
               const float dp = on ? dpacc[j] * p.drop_scale : 0.f;
@@ -419,6 +451,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 
       }
       accumulate_columns<T, DP, kt * 32 * ROWB>(dqacc, dsb, col_addr);
     });
+    if (MODE == kMaskBits) {
+#pragma unroll
+      for (int t = 0; t < kChunk / 32; ++t) chunk_words[t] = next_words[t];
+    }
   }
   __syncthreads();  // the staging buffers now hold the output tiles
   store_owned<T, DP>(dqacc, smem + wave * (32 * OROW), dqb, p.dqs[2], q_begin + wave * 32, p.Tq, p.d, lane);
@@ -430,7 +466,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
   typedef typename Vec8<T>::type vec_t;
   constexpr int KSTEPS = DP / 16, MB = DP / 32;
   constexpr int ROWB = DP * 2, TILE_BYTES = kChunk * ROWB;
-  constexpr int BUF_BYTES = 2 * TILE_BYTES + 2 * kChunk * 4;  // a chunk of Q, of dO, then its row statistics
+  // a chunk of Q, of dO, then its row statistics; bit mode: then the mask words of the chunk's rows for the 32 keys of
+  // each wavefront, [wavefront][row]
+  constexpr int kWaves = kThreads / kWave;
+  static_assert(kThreads == kWaves * kChunk, "one mask word per thread and chunk");
+  constexpr int BUF_BYTES = 2 * TILE_BYTES + 2 * kChunk * 4 + (MODE == kMaskBits ? kWaves * kChunk * 4 : 0);
   constexpr int NBUF = DMA ? 2 : 1;
   constexpr int OROW = DP * 2 + 16;
   constexpr int OUT_BYTES = (kThreads / kWave) * 32 * OROW;
@@ -456,6 +496,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
   const int q_valid = p.zero_pad ? (len < p.Tq ? len : p.Tq) : p.Tq;
   const int k_begin = blk * kOwn;
   const int kj = k_begin + wave * 32 + l32;
+  // visibility mode: whether the lane's key can be seen at all (its own byte of the key validity, if one was given)
+  // bit mode: column (kj / 32) of the sample's word matrix; (k_begin + wave * 32) is a multiple of 32, so the wavefront's
+  // keys share the word and key kj is bit l32
+  [[maybe_unused]] const int bit_wpr = (p.Tk + 31) / 32;
+  [[maybe_unused]] bool key_seen = kj < p.Tk;
+  if (MODE == kMaskVisible && key_seen && p.key_valid != nullptr) key_seen = p.key_valid[static_cast<int64_t>(b) * p.Tk + kj] != 0;
+  if (MODE == kMaskBits && key_seen && p.key_valid != nullptr)
+    key_seen = ((reinterpret_cast<const uint32_t*>(p.key_valid)[static_cast<int64_t>(b) * ((p.Tk + 31) / 32) + kj / 32] >> (kj % 32)) & 1u) != 0u;
   const bool k_ok = kj < len;
   // queries that can see a key of this block: all valid ones, or (causal) those at or after the block's first key
   const int q_start = p.causal ? (k_begin / kChunk) * kChunk : 0;
@@ -476,6 +524,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
     q_rows.init(qb, p.qs[2], tid);
     do_rows.init(dob, p.dos[2], tid);
     float lse_next = -INFINITY, delta_next = 0.f;
+    [[maybe_unused]] uint32_t word_next = 0u;
     auto fetch = [&](int qc0, int buffer) {
       q_rows.fetch(qc0, q_valid, p.d, smem + buffer * BUF_BYTES, tid);
       do_rows.fetch(qc0, q_valid, p.d, smem + buffer * BUF_BYTES + TILE_BYTES, tid);
@@ -483,6 +532,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
         const int qi = qc0 + tid;
         lse_next = qi < q_valid ? p.lse[stat0 + qi] : -INFINITY;
         delta_next = qi < q_valid ? p.delta[stat0 + qi] : 0.f;
+      }
+      if (MODE == kMaskBits) {  // thread (w, r): the word of query row qc0 + r that covers the keys of wavefront w
+        const int qi = qc0 + tid % kChunk, key0 = k_begin + (tid / kChunk) * 32;
+        word_next = (qi < q_valid && key0 < p.Tk)
+                        ? reinterpret_cast<const uint32_t*>(p.drop_mask)[b * p.mask_bs + static_cast<int64_t>(qi) * bit_wpr + key0 / 32]
+                        : 0u;
       }
     };
     // the row statistics travel through registers: base-2 log-sum-exp (+inf: the row carries nothing, exp2(x - inf) = 0)
@@ -493,6 +548,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
         stats[tid] = lse_next > -INFINITY ? lse_next * 1.4426950408889634f : INFINITY;
         stats[kChunk + tid] = delta_next * p.scale;
       }
+      if (MODE == kMaskBits)
+        reinterpret_cast<uint32_t*>(smem + buffer * BUF_BYTES + 2 * TILE_BYTES + 2 * kChunk * 4)[tid] = word_next;
     };
     const uint32_t row_off = streamed_row_offset<DP>(l32, hh);
     const uint32_t col_off = streamed_column_offset<DP>(lane);
@@ -518,6 +575,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
       const uint8_t* q_tile = smem + buf * BUF_BYTES;
       const float* sLse = reinterpret_cast<const float*>(q_tile + 2 * TILE_BYTES);
       const float* sDelta = sLse + kChunk;
+      [[maybe_unused]] const uint32_t* sWords = reinterpret_cast<const uint32_t*>(sDelta + kChunk) + wave * kChunk;
       const uint32_t q_col_addr = lds_offset(q_tile) + col_off;
       if (DMA) buf ^= 1;
       static_for<kChunk / 32>([&](auto qt_tag) {
@@ -550,14 +608,21 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
           const int r0 = qt * 32 + jq * 8 + hh * 4;  // four consecutive queries of the chunk
           const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sLse[r0]);
           const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[r0]);  // already times 1 / sqrt(d)
+          [[maybe_unused]] u32x4 w4 = {0u, 0u, 0u, 0u};
+          if (MODE == kMaskBits) w4 = *reinterpret_cast<const u32x4*>(&sWords[r0]);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int j = jq * 4 + e;
             float prob = __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -l4[e]));
-            if (MODE != kMaskNone) {
+            if (MODE == kMaskBits) {
+              // the lane owns key kj; register j is query qc0 + r0 + e: bit l32 of that row's word for the wavefront's keys
+              prob = (key_seen && ((w4[e] >> l32) & 1u) != 0u) ? prob : 0.f;
+              pb[j / 8][j % 8] = static_cast<T>(prob);
+              dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -d4[e]));
+            } else if (MODE != kMaskNone) {
               // the lane owns key kj; register j is query qc0 + r0 + e: one mask byte per register
               const int qrow = qc0 + r0 + e;
-              const bool keep = qrow < p.Tq && kj < p.Tk &&
+              const bool keep = qrow < p.Tq && key_seen &&
                                 p.drop_mask[b * p.mask_bs + h * p.mask_hs + static_cast<int64_t>(qrow) * p.Tk + kj] != 0;
               if (DROPOUT) {
                 pb[j / 8][j % 8] = static_cast<T>(keep ? prob * p.drop_scale : 0.f);
@@ -627,6 +692,8 @@ void launch_bwd_dp(const AttnBwdParams& p, int mode, bool register_staging, hipS
     launch_bwd_mode<T, DP, kMaskDropout>(p, register_staging, s);
   else if (mode == kMaskVisible)
     launch_bwd_mode<T, DP, kMaskVisible>(p, register_staging, s);
+  else if (mode == kMaskBits)
+    launch_bwd_mode<T, DP, kMaskBits>(p, register_staging, s);
   else
     launch_bwd_mode<T, DP, kMaskNone>(p, register_staging, s);
 }
@@ -650,7 +717,8 @@ int attention_bwd_entry(const char* name, const void* q, const void* k, const vo
                         const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
                         const int64_t o_strides[4], const int64_t do_strides[4], const int64_t dq_strides[4],
                         const int64_t dk_strides[4], const int64_t dv_strides[4], int is_causal, int zero_padded_queries,
-                        int dtype, void* stream, int mask_mode = -1, int64_t mask_bs = 0, int64_t mask_hs = 0) {
+                        int dtype, void* stream, int mask_mode = -1, int64_t mask_bs = 0, int64_t mask_hs = 0,
+                        const uint8_t* key_valid = nullptr) {
   // mask_mode -1: dropout when a mask is given (its matrices follow the (B, H) order), nothing otherwise
   if (mask_mode < 0) {
     mask_mode = drop_mask != nullptr ? kMaskDropout : kMaskNone;
@@ -701,6 +769,7 @@ int attention_bwd_entry(const char* name, const void* q, const void* k, const vo
   p.drop_mask = drop_mask;
   p.mask_bs = mask_bs;
   p.mask_hs = mask_hs;
+  p.key_valid = key_valid;
   p.drop_scale = drop_scale;
   p.B = B;
   p.H = H;
@@ -760,7 +829,8 @@ extern "C" int taac_flash_attn_dropout_bwd(const void* q, const void* k, const v
 
 extern "C" int taac_flash_attn_mask_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout,
                                         const float* lse, const int32_t* key_lengths, const uint8_t* visible,
-                                        int64_t visible_batch_stride, int64_t visible_head_stride, void* dq, void* dk,
+                                        int64_t visible_batch_stride, int64_t visible_head_stride,
+                                        const uint8_t* key_valid, void* dq, void* dk,
                                         void* dv, float* delta, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
                                         const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
                                         const int64_t o_strides[4], const int64_t do_strides[4],
@@ -771,5 +841,23 @@ extern "C" int taac_flash_attn_mask_bwd(const void* q, const void* k, const void
   return taac::attention_bwd_entry(name, q, k, v, o, dout, lse, key_lengths, visible, 1.f, dq, dk, dv, delta, B, H, Tq, Tk, d,
                                    q_strides, k_strides, v_strides, o_strides, do_strides, dq_strides, dk_strides,
                                    dv_strides, 0, zero_padded_queries, dtype, stream, taac::kMaskVisible,
-                                   visible_batch_stride, visible_head_stride);
+                                   visible_batch_stride, visible_head_stride, key_valid);
+}
+
+extern "C" int taac_flash_attn_bits_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout,
+                                        const float* lse, const int32_t* key_lengths, const uint32_t* struct_bits,
+                                        int64_t struct_sample_stride, const uint32_t* valid_bits, void* dq, void* dk,
+                                        void* dv, float* delta, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                                        const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
+                                        const int64_t o_strides[4], const int64_t do_strides[4],
+                                        const int64_t dq_strides[4], const int64_t dk_strides[4],
+                                        const int64_t dv_strides[4], int zero_padded_queries, int dtype, void* stream) {
+  const char* name = "taac_flash_attn_bits_bwd";
+  if (!struct_bits) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_bits must be given", name);
+  if (struct_sample_stride < 0) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: negative sample stride", name);
+  return taac::attention_bwd_entry(name, q, k, v, o, dout, lse, key_lengths, reinterpret_cast<const uint8_t*>(struct_bits),
+                                   1.f, dq, dk, dv, delta, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides,
+                                   do_strides, dq_strides, dk_strides, dv_strides, 0, zero_padded_queries, dtype, stream,
+                                   taac::kMaskBits, struct_sample_stride, 0,
+                                   reinterpret_cast<const uint8_t*>(valid_bits));
 }

@@ -254,6 +254,37 @@ __global__ __launch_bounds__(kBlock) void rows_merge_kernel(const bf16x8* __rest
   out[idx] = v;
 }
 
+// The same merge for padding that is not a prefix: (b, t) is valid iff bit t of valid_bits[b] is set, and its compact row
+// is offsets[b] + the number of valid tokens of the sample in front of it.
+__global__ __launch_bounds__(kBlock) void rows_merge_bits_kernel(const bf16x8* __restrict__ padded,
+                                                                 const bf16x8* __restrict__ a, const bf16x8* __restrict__ b2,
+                                                                 const uint32_t* __restrict__ valid_bits,
+                                                                 const int32_t* __restrict__ offsets, bf16x8* __restrict__ out,
+                                                                 int64_t pieces_total, int T, int pieces) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= pieces_total) return;
+  const int64_t row = idx / pieces;
+  const int c = static_cast<int>(idx % pieces);
+  const int b = static_cast<int>(row / T), t = static_cast<int>(row % T);
+  const uint32_t* bits = valid_bits + static_cast<int64_t>(b) * ((T + 31) / 32);
+  const uint32_t word = bits[t / 32];
+  bf16x8 v;
+  if ((word >> (t % 32)) & 1u) {
+    int rank = __popc(word & ((1u << (t % 32)) - 1u));
+    for (int w = 0; w < t / 32; ++w) rank += __popc(bits[w]);
+    const int64_t src = (static_cast<int64_t>(offsets[b]) + rank) * pieces + c;
+    v = a[src];
+    if (b2 != nullptr) {
+      const bf16x8 w2 = b2[src];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = static_cast<bf16_t>(static_cast<float>(v[e]) + static_cast<float>(w2[e]));
+    }
+  } else {
+    v = padded[idx];
+  }
+  out[idx] = v;
+}
+
 // dst[i] = src[rows[i]] for i < n: one 16-byte piece per thread.
 __global__ __launch_bounds__(kBlock) void rows_gather_kernel(const bf16x8* __restrict__ src, int64_t src_pieces,
                                                              const int32_t* __restrict__ rows, bf16x8* __restrict__ dst,
@@ -301,6 +332,27 @@ extern "C" int taac_rows_merge(const void* padded, const void* compact_a, const 
   hipLaunchKernelGGL(rows_merge_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, as_stream(stream),
                      static_cast<const bf16x8*>(padded), static_cast<const bf16x8*>(compact_a),
                      static_cast<const bf16x8*>(compact_b), key_lengths, offsets, static_cast<bf16x8*>(out), pieces_total, T,
+                     W / 8);
+  return check_launch(name);
+}
+
+extern "C" int taac_rows_merge_bits(const void* padded, const void* compact_a, const void* compact_b,
+                                    const uint32_t* valid_bits, const int32_t* offsets, void* out, int32_t B, int32_t T,
+                                    int32_t W, void* stream) {
+  using namespace taac;
+  const char* name = "taac_rows_merge_bits";
+  if (B < 0 || T < 0 || W <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: bad dimensions", name);
+  if (W % 8 != 0) return set_error(TAAC_ERR_UNSUPPORTED, "%s: W=%d must be a multiple of 8", name, W);
+  if (B == 0 || T == 0) return TAAC_OK;
+  if (!padded || !compact_a || !valid_bits || !offsets || !out) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  if (!aligned16(padded) || !aligned16(compact_a) || !aligned16(compact_b) || !aligned16(out))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
+  const int64_t pieces_total = static_cast<int64_t>(B) * T * (W / 8);
+  const int64_t blocks = (pieces_total + kBlock - 1) / kBlock;
+  if (blocks > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many workgroups", name);
+  hipLaunchKernelGGL(rows_merge_bits_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, as_stream(stream),
+                     static_cast<const bf16x8*>(padded), static_cast<const bf16x8*>(compact_a),
+                     static_cast<const bf16x8*>(compact_b), valid_bits, offsets, static_cast<bf16x8*>(out), pieces_total, T,
                      W / 8);
   return check_launch(name);
 }

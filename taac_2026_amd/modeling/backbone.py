@@ -274,9 +274,12 @@ class UnifiedInteractionBlock(nn.Module):
     ) -> tuple[torch.Tensor, torch.Tensor | None]:
         if self._fused_route(tokens):
             return self._forward_fused(tokens, padding_mask, attention_mask, key_lengths, return_attention_tokens, inplace)
-        if torch.is_grad_enabled() and training_route_applies(self, tokens, attention_mask, key_lengths):
-            # prefix padding, plain attention layer, no dropout: the whole block as one autograd function over the valid rows
-            result = run_training_block(self, tokens, key_lengths, return_attention_tokens)
+        if torch.is_grad_enabled() and training_route_applies(self, tokens, attention_mask, key_lengths, padding_mask):
+            # key lengths or a structured mask built from the padding mask, no rotary embedding, no dropout: the whole block
+            # as one autograd function over the valid rows
+            structured = attention_mask if isinstance(attention_mask, StructuredAttentionMask) else None
+            result = run_training_block(self, tokens, key_lengths, return_attention_tokens, structured,
+                                        padding_mask if structured is not None else None)
             if result is not None:
                 return result
         keep = (~padding_mask).unsqueeze(-1)

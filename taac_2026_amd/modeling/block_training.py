@@ -1,5 +1,7 @@
-"""Training route of ``UnifiedInteractionBlock`` (experiments/symbiosis/backbone.py:51-68) under prefix padding: one
-autograd function for the whole block whose forward and backward run over the VALID tokens only.
+"""Training route of ``UnifiedInteractionBlock`` (experiments/symbiosis/backbone.py:51-68) under prefix padding (key
+lengths) or under a structured mask built from the padding mask (scattered padding, e.g. the role mask of
+experiments/symbiosis/attention.py:21-60): one autograd function for the whole block whose forward and backward run over
+the VALID tokens only.
 
 The reference multiplies both residual updates by ``~padding_mask``, so a padded position passes its input through and
 contributes nothing to any weight gradient. The function therefore gathers the valid rows of the token stream once
@@ -10,7 +12,7 @@ forward and backward kernels do 54 % of the work of the layer-by-layer route, th
 in place (no concatenation) and the mask multiplications and residual adds of autograd disappear.
 
 The number of valid rows sizes the compact tensors, so it is read back from the device once per ``key_lengths`` tensor
-(one host synchronisation, shared by the blocks of a stack).
+or mask object (one host synchronisation, shared by the blocks of a stack).
 """
 
 from __future__ import annotations
@@ -47,6 +49,31 @@ class _RowIndex:
         return self
 
     @classmethod
+    def for_mask(cls, mask, padding_mask: torch.Tensor, tokens: int) -> "_RowIndex":
+        """Index of the positions ``~padding_mask`` (any pattern), kept on the mask object the blocks of a stack share;
+        ``bits``: the same validity as packed words, for ``taac_rows_merge_bits``."""
+        entry = mask.cache.get("training_rows")
+        if entry is None or entry[0] != padding_mask._version:
+            from taac_2026_amd.accelerators.attention import _pack_bits
+
+            from taac_2026_amd.accelerators.attention import front_structured_mask
+
+            index = cls.__new__(cls)
+            index.rows, index.count = _linear.valid_rows(None, tokens, padding_mask=padding_mask)
+            index.bits = _pack_bits((~padding_mask).contiguous())
+            index.valid = None
+            index.identity = None
+            # Without self-only queries the attention side runs in the layout that has every sample's valid tokens at the
+            # front of its rows (prefix padding: its cost follows the valid tokens), under the structure gathered per sample.
+            index.front = index.lengths = index.front_mask = None
+            if mask.query_self is None:
+                batch = padding_mask.shape[0]
+                index.front, index.lengths = _linear.front_rows((index.rows, index.count), batch, tokens)
+                index.front_mask = front_structured_mask(mask, (index.rows, index.count), batch)
+            entry = mask.cache["training_rows"] = (padding_mask._version, index)
+        return entry[1]
+
+    @classmethod
     def get(cls, key_lengths: torch.Tensor, tokens: int) -> "_RowIndex":
         stamp = cls._last
         if stamp is not None:
@@ -76,10 +103,12 @@ def _indexed_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | 
     _native.check(status, "interaction block (training): projection")
 
 
-def _gather_rows(src: torch.Tensor, index: "_RowIndex") -> torch.Tensor:
-    """The valid rows of a padded ``[B * T, W]`` tensor as a compact ``[valid, W]`` one (``taac_rows_gather``)."""
+def _gather_rows(src: torch.Tensor, index: "_RowIndex", rows: torch.Tensor | None = None) -> torch.Tensor:
+    """The valid rows of a padded ``[B * T, W]`` tensor as a compact ``[valid, W]`` one (``taac_rows_gather``); ``rows``:
+    where the valid tokens lie when that is not their position (the front layout of the attention side)."""
     out = torch.empty(index.valid, src.shape[1], dtype=src.dtype, device=src.device)
-    status = _native.load_library().taac_rows_gather(src.data_ptr(), src.stride(0), index.rows.data_ptr(), index.valid,
+    rows = index.rows if rows is None else rows
+    status = _native.load_library().taac_rows_gather(src.data_ptr(), src.stride(0), rows.data_ptr(), index.valid,
                                                      out.data_ptr(), src.shape[1], _native.current_stream(src.device))
     _native.check(status, "interaction block (training): gather")
     return out
@@ -91,25 +120,37 @@ def _attention_strides(width: int, heads: int, row_stride: int, tokens: int):
 
 
 class InteractionBlockFunction(torch.autograd.Function):
-    """``UnifiedInteractionBlock.forward`` (with or without the query / key norms) without rotary embedding, dropout or an
-    attention mask other than the key lengths. Inputs: tokens ``[B, T, D]`` bf16, ``key_lengths`` int32 ``[B]``, then the block's parameters. Returns
-    ``(output, attn_tokens)`` like the module (``attn_tokens`` is None unless asked for)."""
+    """``UnifiedInteractionBlock.forward`` (with or without the query / key norms) without rotary embedding or dropout,
+    under key lengths (``mask`` None) or under a structured mask whose key validity comes from ``padding_mask`` (``key_lengths``
+    None). Inputs: tokens ``[B, T, D]`` bf16, ``key_lengths`` int32 ``[B]`` or None, the mask and its padding mask or None,
+    then the block's parameters. Returns ``(output, attn_tokens)`` like the module (``attn_tokens`` is None unless asked for)."""
 
     @staticmethod
-    def forward(ctx, tokens, key_lengths, want_attn_tokens, num_heads, attn_eps, ffn_eps, gate_first, qk_eps, attn_norm_w,
-                w_qkv, b_qkv, w_out, b_out, ffn_norm_w, w_up, b_up, w_down, b_down, query_norm_w, key_norm_w):
+    def forward(ctx, tokens, key_lengths, mask, padding_mask, want_attn_tokens, num_heads, attn_eps, ffn_eps, gate_first,
+                qk_eps, attn_norm_w, w_qkv, b_qkv, w_out, b_out, ffn_norm_w, w_up, b_up, w_down, b_down, query_norm_w,
+                key_norm_w):
         batch, token_count, width = tokens.shape
         total = batch * token_count
-        index = _RowIndex.get(key_lengths, token_count)
+        index = _RowIndex.get(key_lengths, token_count) if mask is None else _RowIndex.for_mask(mask, padding_mask, token_count)
         rows, count = index.rows, index.count
         flat = tokens.detach().reshape(total, width)
         if not flat.is_contiguous():
             flat = flat.contiguous()
         library = _native.load_library()
-        # q | k | v of the valid rows, in the padded layout (the attention kernel never reads a padded key or query row)
-        qkv = torch.empty(total, 3 * width, dtype=flat.dtype, device=flat.device)
-        _indexed_linear(flat, w_qkv, b_qkv, qkv, tokens=total, out_rows=rows, count=count, x_rows=None,
-                        norm_weight=attn_norm_w, eps=attn_eps)
+        # q | k | v of the valid rows, in the padded layout. Under key lengths the attention kernels never read a padded
+        # key or query row; under a mask they do (an invisible pair is a zero factor, not a skipped one), so the padded
+        # rows hold zeros there.
+        # Layout of the attention side: the positions (key lengths, or a mask with self-only queries), or the samples'
+        # valid tokens in front (any other mask), where the mask's structure is the one gathered per sample and the
+        # samples' numbers of valid tokens are the key lengths.
+        front = getattr(index, "front", None) if mask is not None else None
+        arows = rows if front is None else front
+        if front is not None:
+            mask, key_lengths = index.front_mask, index.lengths
+        in_positions = mask is not None and front is None
+        qkv = (torch.zeros if in_positions else torch.empty)(total, 3 * width, dtype=flat.dtype, device=flat.device)
+        _indexed_linear(flat, w_qkv, b_qkv, qkv, tokens=total, out_rows=arows, count=count,
+                        x_rows=None if front is None else rows, norm_weight=attn_norm_w, eps=attn_eps)
         element = qkv.element_size()
         if query_norm_w is not None:
             # RMSNorm(d_model) of the query and of the key, in place on the valid rows of the packed projection; the
@@ -117,25 +158,33 @@ class InteractionBlockFunction(torch.autograd.Function):
             status = library.taac_qk_norm_rope_fwd(
                 qkv.data_ptr(), qkv.data_ptr() + width * element, 3 * width, qkv.data_ptr(), qkv.data_ptr() + width * element,
                 3 * width, total, token_count, width, int(num_heads), query_norm_w.data_ptr(), key_norm_w.data_ptr(),
-                float(qk_eps), None, rows.data_ptr(), count.data_ptr(), _native.dtype_code(flat.dtype),
+                float(qk_eps), None, arows.data_ptr(), count.data_ptr(), _native.dtype_code(flat.dtype),
                 _native.current_stream(tokens.device))
             _native.check(status, "interaction block (training): query / key norm")
         attended = torch.empty(total, width, dtype=flat.dtype, device=flat.device)
         lse = torch.empty(batch, num_heads, token_count, dtype=torch.float32, device=flat.device)
         qkv_strides = _attention_strides(width, num_heads, 3 * width, token_count)
         out_strides = _attention_strides(width, num_heads, width, token_count)
-        status = library.taac_flash_attn_train_fwd(
-            qkv.data_ptr(), qkv.data_ptr() + width * element, qkv.data_ptr() + 2 * width * element, key_lengths.data_ptr(),
-            attended.data_ptr(), lse.data_ptr(), batch, num_heads, token_count, token_count, width // num_heads,
-            qkv_strides, qkv_strides, qkv_strides, out_strides, 0, 1, _native.dtype_code(flat.dtype),
-            _native.current_stream(tokens.device))
+        if mask is None:
+            status = library.taac_flash_attn_train_fwd(
+                qkv.data_ptr(), qkv.data_ptr() + width * element, qkv.data_ptr() + 2 * width * element, key_lengths.data_ptr(),
+                attended.data_ptr(), lse.data_ptr(), batch, num_heads, token_count, token_count, width // num_heads,
+                qkv_strides, qkv_strides, qkv_strides, out_strides, 0, 1, _native.dtype_code(flat.dtype),
+                _native.current_stream(tokens.device))
+        else:
+            status = library.taac_flash_attn_masked_train_fwd(
+                qkv.data_ptr(), qkv.data_ptr() + width * element, qkv.data_ptr() + 2 * width * element,
+                _native.ptr(key_lengths), mask.struct_bits.data_ptr(), int(mask.sample_stride), _native.ptr(mask.block_any),
+                _native.ptr(mask.valid_bits), _native.ptr(mask.self_bits), attended.data_ptr(), lse.data_ptr(), batch,
+                num_heads, token_count, token_count, width // num_heads, qkv_strides, qkv_strides, qkv_strides, out_strides,
+                0 if front is None else 1, _native.dtype_code(flat.dtype), _native.current_stream(tokens.device))
         _native.check(status, "interaction block (training): attention")
         # Second half on the valid rows of copies of the stream (padded rows pass through): one kernel when the caller
         # does not want the tokens between the halves, two otherwise.
         attn_tokens = None
         if want_attn_tokens or not gate_first:
             attn_tokens = flat.clone()
-            _indexed_linear(attended, w_out, b_out, attn_tokens, tokens=total, out_rows=rows, count=count, x_rows=None,
+            _indexed_linear(attended, w_out, b_out, attn_tokens, tokens=total, out_rows=rows, count=count, x_rows=front,
                             residual=flat)
             output = attn_tokens.clone()
             _linear.swiglu_ffn(attn_tokens, w_up, b_up, w_down, b_down, residual=attn_tokens, gate_first=gate_first,
@@ -143,8 +192,11 @@ class InteractionBlockFunction(torch.autograd.Function):
         else:
             output = flat.clone()
             _linear.attention_out_ffn(attended, w_out, b_out, flat, w_up, b_up, w_down, b_down, norm_weight=ffn_norm_w,
-                                      eps=ffn_eps, token_rows=(rows, count), out=output)
-        ctx.save_for_backward(flat, qkv, attended, lse, key_lengths, attn_norm_w, w_qkv, w_out, ffn_norm_w, w_up, w_down,
+                                      eps=ffn_eps, token_rows=(rows, count), input_rows=front, out=output)
+        ctx.mask, ctx.front = mask, front
+        ctx.save_for_backward(flat, qkv, attended, lse, key_lengths if key_lengths is not None else lse, attn_norm_w, w_qkv,
+                              w_out,
+                              ffn_norm_w, w_up, w_down,
                               *(t for t in (b_out, b_up, attn_tokens, b_qkv if query_norm_w is not None else None,
                                             query_norm_w, key_norm_w) if t is not None))
         ctx.index = index
@@ -169,11 +221,13 @@ class InteractionBlockFunction(torch.autograd.Function):
         query_norm_w, key_norm_w = (rest.pop(0), rest.pop(0)) if has_qk_norm else (None, None)
         index = ctx.index.compact()
         rows, count, valid, identity = index.rows, index.count, index.valid, index.identity
+        mask, front = ctx.mask, ctx.front
+        arows = rows if front is None else front       # where the attention side keeps the valid tokens
         total = batch * token_count
         dtype, device = flat.dtype, flat.device
         if valid == 0:                              # no valid token: the block is the identity
             grads = [g for g in (grad_output, grad_attn_tokens) if g is not None]
-            return (sum(grads[1:], grads[0]) if grads else None,) + (None,) * 19
+            return (sum(grads[1:], grads[0]) if grads else None,) + (None,) * 21
         # the compact rows of the stream and of the tokens between the halves (gathered, or recomputed from the attention
         # output when the forward ran the one-kernel second half)
         xc = _gather_rows(flat, index)
@@ -181,7 +235,7 @@ class InteractionBlockFunction(torch.autograd.Function):
             x1c = _gather_rows(attn_tokens_saved, index)
         else:
             x1c = torch.empty(valid, width, dtype=dtype, device=device)
-            _indexed_linear(attended, w_out, b_out, x1c, tokens=valid, out_rows=identity, count=count, x_rows=rows, residual=xc)
+            _indexed_linear(attended, w_out, b_out, x1c, tokens=valid, out_rows=identity, count=count, x_rows=arows, residual=xc)
 
         def flat_grad(g):
             g = g.reshape(total, width)
@@ -208,13 +262,13 @@ class InteractionBlockFunction(torch.autograd.Function):
             grad_x1_norm, weight_grads["ffn_norm"] = hip_rms_norm_backward_kernel(x1c, ffn_norm_w, grad_h2, ffn_eps)
             grad_x1c = gc.add_(grad_x1_norm) if grad_x1c is None else grad_x1c.add_(gc).add_(grad_x1_norm)
         if grad_x1c is None:
-            return (None,) * 20
+            return (None,) * 22
         # ---- out projection: weight gradient on compact rows, input gradient written into the padded layout ------------
-        attended_c = _gather_rows(attended, index)
+        attended_c = _gather_rows(attended, index, arows)
         grad_w_out, grad_b_out = _linear.linear_wgrad(grad_x1c, attended_c, with_bias=has_b_out)
         del attended_c
         grad_attended = torch.zeros(total, width, dtype=dtype, device=device)
-        _indexed_linear(grad_x1c, w_out.t().contiguous(), None, grad_attended, tokens=valid, out_rows=rows, count=count,
+        _indexed_linear(grad_x1c, w_out.t().contiguous(), None, grad_attended, tokens=valid, out_rows=arows, count=count,
                         x_rows=identity, cache_weight=False)
         # ---- attention: the gradient of the packed q | k | v projection in place ---------------------------------------------
         grad_qkv = torch.empty(total, 3 * width, dtype=dtype, device=device)
@@ -224,14 +278,27 @@ class InteractionBlockFunction(torch.autograd.Function):
         out_strides = _attention_strides(width, num_heads, width, token_count)
         element = qkv.element_size()
         q_ptr, g_ptr = qkv.data_ptr(), grad_qkv.data_ptr()
-        status = library.taac_flash_attn_bwd(
-            q_ptr, q_ptr + width * element, q_ptr + 2 * width * element, attended.data_ptr(), grad_attended.data_ptr(),
-            lse.data_ptr(), key_lengths.data_ptr(), g_ptr, g_ptr + width * element, g_ptr + 2 * width * element,
-            delta.data_ptr(), batch, num_heads, token_count, token_count, width // num_heads, qkv_strides, qkv_strides,
-            qkv_strides, out_strides, out_strides, qkv_strides, qkv_strides, qkv_strides, 0, 1, _native.dtype_code(dtype),
-            _native.current_stream(device))
-        _native.check(status, "interaction block (training): attention backward")
-        grad_qkv_c = _gather_rows(grad_qkv, index)                                    # [valid, 3D]
+        if mask is None:
+            status = library.taac_flash_attn_bwd(
+                q_ptr, q_ptr + width * element, q_ptr + 2 * width * element, attended.data_ptr(), grad_attended.data_ptr(),
+                lse.data_ptr(), key_lengths.data_ptr(), g_ptr, g_ptr + width * element, g_ptr + 2 * width * element,
+                delta.data_ptr(), batch, num_heads, token_count, token_count, width // num_heads, qkv_strides, qkv_strides,
+                qkv_strides, out_strides, out_strides, qkv_strides, qkv_strides, qkv_strides, 0, 1, _native.dtype_code(dtype),
+                _native.current_stream(device))
+            _native.check(status, "interaction block (training): attention backward")
+        else:
+            from taac_2026_amd.accelerators.attention import masked_attention_backward
+
+            head_dim = width // num_heads
+            heads_of = lambda t, parts: t.view(batch, token_count, parts, num_heads, head_dim).permute(2, 0, 3, 1, 4)  # noqa: E731
+            q4, k4, v4 = heads_of(qkv, 3)
+            dq4, dk4, dv4 = heads_of(grad_qkv, 3)
+            (o4,), (do4,) = heads_of(attended, 1), heads_of(grad_attended, 1)
+            # positions: the padded rows of q | k | v are zeros and receive finite values that nobody reads; front layout:
+            # the rows beyond a sample's number of valid tokens are never touched
+            masked_attention_backward(q4, k4, v4, o4, do4, lse, None if front is None else key_lengths, mask, dq4, dk4, dv4,
+                                      zero_padded_queries=front is not None)
+        grad_qkv_c = _gather_rows(grad_qkv, index, arows)                             # [valid, 3D]
         del grad_qkv, grad_attended
         grad_query_norm = grad_key_norm = None
         if has_qk_norm:
@@ -257,18 +324,38 @@ class InteractionBlockFunction(torch.autograd.Function):
         grad_xc_norm, grad_attn_norm = hip_rms_norm_backward_kernel(xc, attn_norm_w, grad_h1, attn_eps)
         # valid rows: the gradient of the tokens between the halves + that of the norm's input; padded rows: what arrived
         grad_tokens = torch.empty(total, width, dtype=dtype, device=device)
-        status = library.taac_rows_merge(grad_padded.data_ptr(), grad_x1c.data_ptr(), grad_xc_norm.data_ptr(),
-                                         key_lengths.data_ptr(), rows.data_ptr() + 4 * total, grad_tokens.data_ptr(), batch,
-                                         token_count, width, _native.current_stream(device))
+        if not hasattr(index, "bits"):
+            status = library.taac_rows_merge(grad_padded.data_ptr(), grad_x1c.data_ptr(), grad_xc_norm.data_ptr(),
+                                             key_lengths.data_ptr(), rows.data_ptr() + 4 * total, grad_tokens.data_ptr(),
+                                             batch, token_count, width, _native.current_stream(device))
+        else:
+            status = library.taac_rows_merge_bits(grad_padded.data_ptr(), grad_x1c.data_ptr(), grad_xc_norm.data_ptr(),
+                                                  ctx.index.bits.data_ptr(), rows.data_ptr() + 4 * total,
+                                                  grad_tokens.data_ptr(), batch, token_count, width,
+                                                  _native.current_stream(device))
         _native.check(status, "interaction block (training): gradient merge")
-        return (grad_tokens.view(batch, token_count, width), None, None, None, None, None, None, None, grad_attn_norm,
+        return (grad_tokens.view(batch, token_count, width), None, None, None, None, None, None, None, None, None,
+                grad_attn_norm,
                 grad_w_qkv, grad_b_qkv, grad_w_out, grad_b_out, weight_grads["ffn_norm"], weight_grads["up"],
                 weight_grads["b_up"], weight_grads["down"], weight_grads["b_down"], grad_query_norm, grad_key_norm)
 
 
-def training_route_applies(block, tokens: torch.Tensor, attention_mask, key_lengths) -> bool:
-    """Whether :class:`InteractionBlockFunction` covers this call of ``block`` (a ``UnifiedInteractionBlock``)."""
-    if attention_mask is not None or key_lengths is None:
+def training_route_applies(block, tokens: torch.Tensor, attention_mask, key_lengths, padding_mask=None) -> bool:
+    """Whether :class:`InteractionBlockFunction` covers this call of ``block`` (a ``UnifiedInteractionBlock``): key lengths
+    and no mask, or a structured mask (same for every sample apart from key validity) that was built from
+    ``padding_mask``, so that no query can see a padded key."""
+    from taac_2026_amd.accelerators.attention import StructuredAttentionMask
+
+    if isinstance(attention_mask, StructuredAttentionMask):
+        if key_lengths is not None or padding_mask is None or attention_mask.padding_source is not padding_mask:
+            return False
+        if attention_mask.sample_stride or attention_mask.key_valid is None or tokens.ndim != 3:
+            return False
+        if attention_mask.structural.shape != (tokens.shape[1], tokens.shape[1]):
+            return False
+        if padding_mask.dtype is not torch.bool or not padding_mask.is_cuda or padding_mask.shape != tokens.shape[:2]:
+            return False
+    elif attention_mask is not None or key_lengths is None:
         return False
     if not (tokens.is_cuda and tokens.dtype == torch.bfloat16 and tokens.ndim == 3 and tokens.shape[-1] in (128, 256)):
         return False
@@ -283,17 +370,19 @@ def training_route_applies(block, tokens: torch.Tensor, attention_mask, key_leng
         return False
     if block.training and (attention.dropout > 0.0 or ffn.dropout.p > 0.0):
         return False
-    if key_lengths.dtype != torch.int32 or not key_lengths.is_cuda or not key_lengths.is_contiguous():
+    if key_lengths is not None and (key_lengths.dtype != torch.int32 or not key_lengths.is_cuda
+                                    or not key_lengths.is_contiguous()):
         return False
     return all(p.dtype == torch.bfloat16 and p.is_cuda for p in block.parameters())
 
 
-def run_training_block(block, tokens: torch.Tensor, key_lengths: torch.Tensor, return_attention_tokens: bool):
+def run_training_block(block, tokens: torch.Tensor, key_lengths: torch.Tensor | None, return_attention_tokens: bool,
+                       mask=None, padding_mask: torch.Tensor | None = None):
     """The block through :class:`InteractionBlockFunction`."""
     attention, ffn = block.attention, block.ffn
     qk_norm = attention.query_norm is not None
     return InteractionBlockFunction.apply(
-        tokens, key_lengths, bool(return_attention_tokens), attention.num_heads, block.attn_norm.eps, block.ffn_norm.eps,
+        tokens, key_lengths, mask, padding_mask, bool(return_attention_tokens), attention.num_heads, block.attn_norm.eps, block.ffn_norm.eps,
         ffn.gate_first, attention.query_norm.eps if qk_norm else 1e-6, block.attn_norm.weight, attention.qkv.weight,
         attention.qkv.bias, attention.out.weight, attention.out.bias, block.ffn_norm.weight, ffn.up.weight, ffn.up.bias,
         ffn.down.weight, ffn.down.bias, attention.query_norm.weight if qk_norm else None,

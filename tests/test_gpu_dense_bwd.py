@@ -435,3 +435,71 @@ def test_block_trains_under_the_role_mask(device, qk_norm):
     for name, parameter in block.named_parameters():
         assert parameter.grad is not None, name
         _close(parameter.grad, reference[name].grad, 5e-2)
+
+
+@pytest.mark.parametrize("model_mask", ["role", "window"])
+def test_block_training_route_under_a_structured_mask_equals_the_layer_by_layer_route(device, monkeypatch, model_mask):
+    """Scattered padding and a structured mask built from it (the Symbiosis role mask; a TokenFormer window layer whose
+    padded queries keep themselves): the one-function route over the valid rows against the layer-by-layer autograd
+    route of the same module - outputs, input gradient, every parameter gradient; padded positions pass through bit
+    for bit, an all-padded sample included."""
+    import taac_2026_amd.modeling.backbone as backbone_module
+    from taac_2026_amd.api import MetadataAttentionMask, bfts_attention_mask, build_structured_mask
+
+    batch, d_model, heads, mult = 4, 256, 8, 2
+    if model_mask == "role":
+        roles = torch.tensor([0, 1] + [2] * 9 + [3] * 7 + [4] * 3 + [5] * 2 + [6] * 100 + [7] * 5)
+    else:
+        roles = torch.tensor([0] * 10 + [4] + [1] * 90 + [4] + [2] * 10 + [5] * 7 + [3])
+    tokens = roles.numel()
+    g = torch.Generator().manual_seed(5)
+    block = UnifiedInteractionBlock(d_model, heads, mult, qk_norm=True)
+    with torch.no_grad():
+        for parameter in block.parameters():
+            if parameter.ndim == 1:
+                parameter.copy_((1.0 if parameter.mean() > 0.5 else 0.0) + 0.1 * torch.randn(parameter.shape, generator=g))
+            else:
+                parameter.copy_(torch.randn(parameter.shape, generator=g) * parameter.shape[1] ** -0.5)
+    block = block.to(torch.bfloat16).to(device).train()
+    x = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16).to(device)
+    padding = torch.rand(batch, tokens, generator=g) < 0.35
+    padding[:, :2] = False
+    padding[:, -1] = False
+    padding[2] = True                                          # an all-padded sample
+    padding = padding.to(device)
+    if model_mask == "role":
+        mask = MetadataAttentionMask(enabled=True)(padding, roles.to(device))
+    else:
+        layer = bfts_attention_mask(padding, roles.to(device), 4, 6, seq_causal=True, seq_keep_per_domain=32)
+        # the layer's structure over exactly the non-padded keys, padded queries keeping themselves, stated as built from
+        # this padding mask (which is what lets a block skip the padded rows)
+        mask = build_structured_mask(layer.structural, ~padding, padding, padding_source=padding)
+    assert mask.padding_source is padding
+    grad_out = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16).to(device)
+    grad_attn = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16).to(device)
+    taken = []
+    real = backbone_module.run_training_block
+
+    def run(compact: bool):
+        if compact:
+            monkeypatch.setattr(backbone_module, "run_training_block", lambda *a, **k: (taken.append(1), real(*a, **k))[1])
+        else:
+            monkeypatch.setattr(backbone_module, "training_route_applies", lambda *a, **k: False)
+        xd = x.clone().requires_grad_(True)
+        block.zero_grad(set_to_none=True)
+        out, attn_tokens = block(xd, padding, mask)
+        torch.autograd.backward([out, attn_tokens], [grad_out, grad_attn])
+        monkeypatch.undo()
+        return out.detach(), attn_tokens.detach(), xd.grad, {n: p.grad.clone() for n, p in block.named_parameters()}
+
+    out_c, attn_c, gx_c, grads_c = run(True)
+    assert taken == [1]                                        # the call took the one-function route
+    out_s, attn_s, gx_s, grads_s = run(False)
+    _close(out_c, out_s.cpu(), 1e-2)
+    _close(attn_c, attn_s.cpu(), 1e-2)
+    pad = padding.cpu()
+    assert torch.equal(out_c.cpu()[pad], x.cpu()[pad]) and torch.equal(attn_c.cpu()[pad], x.cpu()[pad])
+    assert torch.equal(gx_c.cpu()[pad], (grad_out + grad_attn).cpu()[pad])
+    _close(gx_c, gx_s.cpu(), 3e-2)
+    for name in grads_s:
+        _close(grads_c[name], grads_s[name].cpu(), 3e-2)

@@ -151,3 +151,41 @@ def test_attention_over_the_front_layout_matches_the_masked_attention_over_posit
     got = got_front.transpose(1, 2).reshape(batch * tokens, heads, dim).cpu().float()[front_cpu]
     expected = want.transpose(1, 2).reshape(batch * tokens, heads, dim)[rows]
     torch.testing.assert_close(got, expected, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("tokens,dim", [(150, 32), (96, 64)])
+def test_attention_over_the_front_layout_takes_a_gradient(device, tokens, dim):
+    """The same comparison for the backward: gradients of attention over the front layout (structure bits per sample,
+    key lengths = the samples' numbers of valid tokens, rows beyond them never read: they hold NaN here) against
+    float64 autograd under the dense mask over the positions."""
+    batch, heads = 5, 2
+    g = torch.Generator().manual_seed(tokens + dim + 1)
+    padding = _padding(batch, tokens, seed=tokens)
+    padding[1, 0] = False
+    structural = (torch.rand(tokens, tokens, generator=g) < 0.5) | torch.eye(tokens, dtype=torch.bool)
+    q, k, v, grad_out = (torch.randn(batch, heads, tokens, dim, generator=g).to(torch.bfloat16) for _ in range(4))
+    dense = structural[None, None] & (~padding)[:, None, None, :]
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    keep = (~padding)[:, None, :, None].double()           # padded query rows carry no loss
+    (oracle.sdpa(qr, kr, vr, dense) * keep).backward(grad_out.double())
+    mask = build_structured_mask(structural.to(device), (~padding).to(device))
+    index = valid_rows(None, tokens, padding_mask=padding.to(device))
+    front, lengths = front_rows(index, batch, tokens)
+    front_mask = front_structured_mask(mask, index, batch)
+    count = int(index[1].item())
+    rows, front_cpu = index[0][:count].long().cpu(), front[:count].long().cpu()
+
+    def moved(t, fill):
+        flat = t.transpose(1, 2).reshape(batch * tokens, heads, dim)
+        out = torch.full_like(flat, fill)
+        out[front_cpu] = flat[rows]
+        return out.view(batch, tokens, heads, dim).transpose(1, 2).to(device)
+
+    qd, kd, vd = (moved(t, float("nan")).requires_grad_(True) for t in (q, k, v))
+    out = flash_attention(qd, kd, vd, key_lengths=lengths, structured_mask=front_mask, zero_padded_queries=True)
+    out.backward(moved(grad_out, float("nan")))
+    for got, want, name in zip((qd.grad, kd.grad, vd.grad), (qr.grad, kr.grad, vr.grad), ("dq", "dk", "dv")):
+        got = got.transpose(1, 2).reshape(batch * tokens, heads, dim).cpu().double()[front_cpu]
+        want = want.transpose(1, 2).reshape(batch * tokens, heads, dim)[rows]
+        assert torch.isfinite(got).all(), name
+        torch.testing.assert_close(got, want, rtol=3e-2, atol=3e-2, msg=lambda m, n=name: f"{n}: {m}")

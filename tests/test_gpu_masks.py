@@ -372,10 +372,11 @@ def test_structured_mask_gradient_with_key_lengths(device):
     _check_training(device, q, k, v, mask, grad_out, key_lengths=lengths.to(device), dense=dense)
 
 
-@pytest.mark.parametrize("per_head,per_sample", [(True, True), (False, True), (True, False), (False, False)])
-def test_mask_bwd_abi_reads_any_bool_mask(device, per_head, per_sample):
-    """``taac_flash_attn_mask_bwd`` alone: a random mask per sample and / or head (strides 0 = shared), the log-sum-exp
-    and the output taken from the float64 reference."""
+@pytest.mark.parametrize("per_head,per_sample,with_valid", [(True, True, False), (False, True, False), (True, False, False),
+                                                          (False, False, False), (False, False, True), (True, False, True)])
+def test_mask_bwd_abi_reads_any_bool_mask(device, per_head, per_sample, with_valid):
+    """``taac_flash_attn_mask_bwd`` alone: a random mask per sample and / or head (strides 0 = shared), optionally times a
+    key validity per sample, the log-sum-exp and the output taken from the float64 reference."""
     from taac_2026_amd import _native
 
     batch, heads, tokens, dim = 2, 3, 150, 64
@@ -384,6 +385,11 @@ def test_mask_bwd_abi_reads_any_bool_mask(device, per_head, per_sample):
     visible = torch.rand(batch if per_sample else 1, heads if per_head else 1, tokens, tokens, generator=g) < 0.5
     visible[..., 0] = True                              # every query sees a key
     dense = visible.expand(batch, heads, -1, -1)
+    key_valid = None
+    if with_valid:
+        key_valid = torch.rand(batch, tokens, generator=g) < 0.7
+        key_valid[:, 0] = True
+        dense = dense & key_valid[:, None, None, :]
     qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
     scores = (qr @ kr.transpose(-1, -2)) / dim ** 0.5
     scores = scores.masked_fill(~dense, float("-inf"))
@@ -393,13 +399,15 @@ def test_mask_bwd_abi_reads_any_bool_mask(device, per_head, per_sample):
     dev = [t.to(device) for t in (q, k, v, out.detach().to(torch.bfloat16), grad_out)]
     lse_d = lse.detach().float().to(device)
     vis_d = visible.to(torch.uint8).contiguous().to(device)
+    valid_d = None if key_valid is None else key_valid.to(torch.uint8).contiguous().to(device)
     grads = [torch.empty_like(dev[0]) for _ in range(3)]
     delta = torch.empty_like(lse_d)
     strides = [_native.Int64x4(*t.stride()) for t in (*dev, *grads)]
     status = _native.load_library().taac_flash_attn_mask_bwd(
         *(t.data_ptr() for t in dev), lse_d.data_ptr(), None, vis_d.data_ptr(),
         heads * tokens * tokens if per_sample and per_head else (tokens * tokens if per_sample else 0),
-        tokens * tokens if per_head else 0, *(t.data_ptr() for t in grads), delta.data_ptr(), batch, heads, tokens,
+        tokens * tokens if per_head else 0, None if key_valid is None else valid_d.data_ptr(),
+        *(t.data_ptr() for t in grads), delta.data_ptr(), batch, heads, tokens,
         tokens, dim, *strides, 0, _native.dtype_code(torch.bfloat16), _native.current_stream(dev[0].device))
     _native.check(status, "taac_flash_attn_mask_bwd")
     for got, want, name in zip(grads, (qr.grad, kr.grad, vr.grad), ("dq", "dk", "dv")):
