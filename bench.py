@@ -366,6 +366,24 @@ def _training_block_figures(device, with_comparison: bool = True) -> dict:
         finally:
             backbone_module.training_route_applies = applies
     figures["query_key_norm_role_mask_scattered_padding"] = entry
+    del block, x, mask
+    # the whole benchmark network (4 blocks + masked mean -> Linear -> sigmoid) under autograd: forward, loss, backward
+    from taac_2026_amd.api import PCVRBackbone
+
+    model = PCVRBackbone(d_model=width, num_heads=inputs.num_heads, d_ff=inputs.d_ff, n_blocks=len(inputs.blocks))
+    workloads.load_backbone_state(model, inputs)
+    model = model.to(device=device, dtype=torch.bfloat16).train()
+    emb = inputs.emb.to(device).requires_grad_(True)
+    labels = (torch.arange(batch, device=device) % 2).float()
+
+    def model_step():
+        loss = torch.nn.functional.binary_cross_entropy(model(emb, lengths), labels)
+        loss.backward()
+        model.zero_grad(set_to_none=True)
+        emb.grad = None
+
+    ms = _event_ms(model_step, 5, 3)
+    figures["backbone_4_blocks_forward_loss_backward"] = {"ms_per_step": ms, "samples_per_s": batch / (ms * 1e-3)}
     return {"interaction_block_training_step_B1024_T512": figures}
 
 

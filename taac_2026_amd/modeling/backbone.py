@@ -363,7 +363,11 @@ class PCVRBackbone(nn.Module):
                 dense_tokens: bool = False, split_out_ffn: bool = False, fp8: bool = False):
         name = "hip PCVRBackbone"
         require_cuda_tensors(name, emb, key_lengths)
-        require_inference(name, emb)
+        if torch.is_grad_enabled() and (emb.requires_grad or any(p.requires_grad for p in self.parameters())):
+            if dense_tokens or split_out_ffn or fp8:
+                raise RuntimeError(f"{name}: dense_tokens, split_out_ffn and fp8 are inference routes: call them under "
+                                   "torch.no_grad()")
+            return self._forward_training(emb, key_lengths, return_hidden)
         if emb.ndim != 3 or emb.shape[-1] != self.d_model:
             raise ValueError(f"PCVRBackbone expects embeddings of shape (batch, tokens, {self.d_model})")
         if emb.dtype != torch.bfloat16:
@@ -421,6 +425,42 @@ class PCVRBackbone(nn.Module):
             self._fp8_maxima = workspace[offset:offset + 4 * count].view(torch.float32).view(-1, 8)
         if return_hidden:
             return probabilities, hidden
+        return probabilities
+
+    def _forward_training(self, emb: torch.Tensor, key_lengths: torch.Tensor, return_hidden: bool):
+        """The same network under autograd: every block as one function over the valid rows
+        (:class:`InteractionBlockFunction`), then the masked mean over the valid tokens, the head and the sigmoid as
+        differentiable tensor operations (``masked_mean``, modeling/sequence.py:54-60). One host synchronisation per
+        ``key_lengths`` tensor (the number of valid rows sizes the backward's tensors)."""
+        from taac_2026_amd.modeling.block_training import InteractionBlockFunction
+
+        name = "hip PCVRBackbone"
+        if emb.ndim != 3 or emb.shape[-1] != self.d_model or emb.dtype != torch.bfloat16:
+            raise ValueError(f"{name} expects bfloat16 embeddings of shape (batch, tokens, {self.d_model})")
+        if key_lengths.shape != (emb.shape[0],):
+            raise ValueError("key_lengths must have shape (batch,)")
+        head_dim = self.d_model // self.num_heads
+        if self.rope_base is not None or self.d_model not in (128, 256) or head_dim not in (32, 64) or self.d_ff % 32 != 0 \
+                or any(p.dtype != torch.bfloat16 for p in self.parameters()):
+            raise RuntimeError(f"{name}: the training route covers bf16 parameters, d_model 128 / 256, head dims 32 / 64, "
+                               "d_ff a multiple of 32 and no rotary embedding")
+        if key_lengths.dtype != torch.int32 or not key_lengths.is_contiguous():
+            key_lengths = key_lengths.to(torch.int32).contiguous()
+        stream = emb
+        for block in self.blocks:
+            qk = block.query_norm is not None
+            stream, _ = InteractionBlockFunction.apply(
+                stream, key_lengths, None, None, False, self.num_heads, self.eps, self.eps, True, self.eps, block.attn_norm.weight,
+                block.qkv.weight, block.qkv.bias, block.out.weight, block.out.bias, block.ffn_norm.weight, block.up.weight,
+                block.up.bias, block.down.weight, block.down.bias, block.query_norm.weight if qk else None,
+                block.key_norm.weight if qk else None)
+        tokens = emb.shape[1]
+        valid = (torch.arange(tokens, device=emb.device)[None, :] < key_lengths[:, None]).to(stream.dtype).unsqueeze(-1)
+        pooled = (stream * valid).sum(dim=1) / valid.sum(dim=1).clamp_min(1.0)
+        logits = torch.nn.functional.linear(pooled, self.head.weight, self.head.bias).squeeze(-1)
+        probabilities = torch.sigmoid(logits.float())
+        if return_hidden:
+            return probabilities, stream * valid      # rows at or beyond key_lengths[b] are zeros, as in the forward-only route
         return probabilities
 
     FP8_MAXIMA = ("qkv.weight", "out.weight", "up.weight", "down.weight", "attn_norm", "attention", "ffn_norm", "hidden")

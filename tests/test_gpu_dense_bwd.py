@@ -503,3 +503,47 @@ def test_block_training_route_under_a_structured_mask_equals_the_layer_by_layer_
     _close(gx_c, gx_s.cpu(), 3e-2)
     for name in grads_s:
         _close(grads_c[name], grads_s[name].cpu(), 3e-2)
+
+
+@pytest.mark.parametrize("qk_norm", [False, True])
+def test_backbone_module_trains(device, qk_norm):
+    """``PCVRBackbone`` under autograd (blocks through the one-function route, masked mean + head as tensor operations):
+    probabilities, and the gradient of a binary cross-entropy loss with respect to the embeddings and every parameter,
+    against float64 autograd of the oracle's backbone; under ``torch.no_grad()`` the same module runs the one-call
+    forward and returns the same probabilities."""
+    from taac_2026_amd.api import PCVRBackbone
+
+    batch, tokens, d_model, heads, d_ff = 4, 40, 128, 4, 256
+    g = torch.Generator().manual_seed(31)
+    model = PCVRBackbone(d_model=d_model, num_heads=heads, d_ff=d_ff, n_blocks=2, qk_norm=qk_norm)
+    with torch.no_grad():
+        for parameter in model.parameters():
+            if parameter.ndim == 1:
+                parameter.copy_((1.0 if parameter.mean() > 0.5 else 0.0) + 0.1 * torch.randn(parameter.shape, generator=g))
+            else:
+                parameter.copy_(torch.randn(parameter.shape, generator=g) * parameter.shape[1] ** -0.5)
+    model = model.to(torch.bfloat16)
+    reference = {name: value.detach().double().requires_grad_(True) for name, value in model.named_parameters()}
+    emb = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16)
+    lengths = torch.tensor([40, 9, 1, 25], dtype=torch.int32)
+    labels = torch.tensor([1.0, 0.0, 1.0, 0.0])
+
+    model = model.to(device).train()
+    emb_d = emb.to(device).requires_grad_(True)
+    p = model(emb_d, lengths.to(device))
+    assert p.dtype == torch.float32 and p.shape == (batch,)
+    F.binary_cross_entropy(p, labels.to(device)).backward()
+    with torch.no_grad():
+        served = model(emb.to(device), lengths.to(device))
+    torch.testing.assert_close(p.detach(), served, rtol=0, atol=1e-2)
+
+    emb_r = emb.double().requires_grad_(True)
+    blocks = [{name.split(".", 2)[2]: value for name, value in reference.items() if name.startswith(f"blocks.{i}.")}
+              for i in range(2)]
+    want = oracle.backbone(emb_r, lengths, blocks, reference["head.weight"], reference["head.bias"], num_heads=heads)
+    F.binary_cross_entropy(want.double(), labels.double()).backward()
+    torch.testing.assert_close(p.detach().cpu().double(), want.detach().double(), rtol=0, atol=2e-2)
+    _close(emb_d.grad, emb_r.grad, 5e-2)
+    for name, parameter in model.named_parameters():
+        assert parameter.grad is not None, name
+        _close(parameter.grad, reference[name].grad, 5e-2)
