@@ -172,7 +172,9 @@ def test_fp8_backbone_rejects_what_it_does_not_cover(device):
     model = PCVRBackbone(d_model=256, num_heads=inputs.num_heads, d_ff=inputs.d_ff, n_blocks=1, qk_norm=True)
     workloads.load_backbone_state(model, inputs)
     model = model.to(device=device, dtype=torch.bfloat16).eval()
-    with pytest.raises(RuntimeError, match="query / key norm"):
+    with pytest.raises(RuntimeError, match="query / key norm"), torch.no_grad():
+        model(inputs.emb.to(device), inputs.key_lengths.to(device), fp8=True)
+    with pytest.raises(RuntimeError, match="inference routes"):      # parameters that take a gradient, autograd on
         model(inputs.emb.to(device), inputs.key_lengths.to(device), fp8=True)
     with pytest.raises(RuntimeError, match="no fp8 forward"):
         model.fp8_maxima()
