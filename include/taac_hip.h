@@ -271,7 +271,8 @@ int taac_flash_attn_bwd(const void* q, const void* k, const void* v, const void*
  * Training pair for attention under a mask that is not a key prefix or a causal triangle.
  * taac_flash_attn_masked_train_fwd: taac_flash_attn_masked_fwd (structured mask, no row / feature factors) that also
  * writes lse as taac_flash_attn_train_fwd does (-inf for rows without a visible key; the value written for a flagged
- * self row is not used by the backward).
+ * self row is not used by the backward). dropout_mask (NULL: none): the keep mask [B, H, Tq, Tk] and scale 1 / (1 - p) of
+ * taac_flash_attn_train_dropout_fwd, applied behind the normaliser over the visible keys; not with self_bits.
  * taac_flash_attn_mask_bwd: taac_flash_attn_bwd with the visible pairs given as bytes: visible[b * visible_batch_stride +
  * h * visible_head_stride + i * Tk + j] != 0 iff key j is visible to query i (strides in elements, 0 = shared by the
  * batch / the heads; AND j < key_lengths[b] when key_lengths is given; AND key_valid[b * Tk + j] != 0 when key_valid is
@@ -286,7 +287,8 @@ int taac_flash_attn_bwd(const void* q, const void* k, const void* v, const void*
  */
 int taac_flash_attn_masked_train_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
                                      const uint32_t* struct_bits, int64_t struct_sample_stride, const uint8_t* block_any,
-                                     const uint32_t* valid_bits, const uint32_t* self_bits, void* o, float* lse, int32_t B,
+                                     const uint32_t* valid_bits, const uint32_t* self_bits, const uint8_t* dropout_mask,
+                                     float dropout_scale, void* o, float* lse, int32_t B,
                                      int32_t H, int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
                                      const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4],
                                      int zero_padded_queries, int dtype, void* stream);
@@ -538,12 +540,15 @@ int taac_rows_merge(const void* padded, const void* compact_a, const void* compa
  * for the batch), valid_bits [B, ceil(Tk / 32)] or NULL; pair (i, j) of sample b is visible iff both bits are set (and
  * j < key_lengths[b] when key_lengths is given). One word per 32-key tile where the byte form reads 32 bytes. With the
  * samples' valid tokens at the front of their rows (taac_front_rows, taac_mask_front_bits) and key_lengths = their
- * numbers, the cost follows the valid tokens as in taac_flash_attn_bwd.
- * Replaces: as taac_flash_attn_mask_bwd.
+ * numbers, the cost follows the valid tokens as in taac_flash_attn_bwd. dropout_mask (NULL: none): the keep mask and
+ * scale of the forward, as in taac_flash_attn_dropout_bwd.
+ * Replaces: as taac_flash_attn_mask_bwd; with dropout, what the reference's models train with by default
+ * (experiments/symbiosis/__init__.py:87).
  */
 int taac_flash_attn_bits_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,
                              const int32_t* key_lengths, const uint32_t* struct_bits, int64_t struct_sample_stride,
-                             const uint32_t* valid_bits, void* dq, void* dk, void* dv, float* delta, int32_t B, int32_t H,
+                             const uint32_t* valid_bits, const uint8_t* dropout_mask, float dropout_scale, void* dq,
+                             void* dk, void* dv, float* delta, int32_t B, int32_t H,
                              int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4], const int64_t k_strides[4],
                              const int64_t v_strides[4], const int64_t o_strides[4], const int64_t do_strides[4],
                              const int64_t dq_strides[4], const int64_t dk_strides[4], const int64_t dv_strides[4],

@@ -184,13 +184,14 @@ def attention(
 
 def attention_dropout(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, key_lengths: torch.Tensor | None,
                       dropout_mask: torch.Tensor, dropout_p: float, *, is_causal: bool = False,
-                      zero_padded_queries: bool = False) -> torch.Tensor:
+                      zero_padded_queries: bool = False, attn_mask: torch.Tensor | None = None) -> torch.Tensor:
     """Training attention with dropout on the probabilities under a fixed keep mask, (B, H, T, d) tensors:
     ``softmax(scores)`` over the visible keys, then ``P * keep / (1 - p)``, then ``@ v`` - the semantics of the
     reference's training kernel (attention/kernels/tilelang.py:224-247: the normaliser sums the undropped probabilities)
     and of the manual reference its own test compares with
     (tests/gpu/infrastructure/accelerators/test_tilelang_ops_cuda.py:103-141). Differentiable; evaluate in float64 for
-    gradient targets. Rows without a visible key give 0."""
+    gradient targets. Rows without a visible key give 0. ``attn_mask``: a bool mask of the models on top (what
+    ``F.scaled_dot_product_attention(attn_mask=, dropout_p=)`` computes for them, with the keep mask fixed)."""
     batch, heads, query_len, dim = q.shape
     kv_len = k.shape[2]
     scores = torch.matmul(q, k.transpose(-1, -2)) * (dim ** -0.5)
@@ -199,6 +200,8 @@ def attention_dropout(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, key_len
         visible = visible & (torch.arange(kv_len)[None, None, None, :] < key_lengths.to(torch.int64)[:, None, None, None])
     if is_causal:
         visible = visible & (torch.arange(kv_len)[None, None, None, :] <= torch.arange(query_len)[None, None, :, None])
+    if attn_mask is not None:  # a bool mask (B, 1 or H, Tq, Tk), True = attend, as the models build them
+        visible = visible & attn_mask
     scores = scores.masked_fill(~visible, float("-inf"))
     probs = torch.softmax(scores, dim=-1)
     probs = torch.where(visible.any(dim=-1, keepdim=True), probs, torch.zeros_like(probs))

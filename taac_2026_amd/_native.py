@@ -146,7 +146,8 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "taac_flash_attn_masked_train_fwd": (
         c_int,
-        [c_void_p] * 5 + [c_int64] + [c_void_p] * 5 + [c_int32] * 5 + [ctypes.POINTER(c_int64)] * 4 + [c_int, c_int, c_void_p],
+        [c_void_p] * 5 + [c_int64] + [c_void_p] * 4 + [c_float] + [c_void_p] * 2 + [c_int32] * 5
+        + [ctypes.POINTER(c_int64)] * 4 + [c_int, c_int, c_void_p],
     ),
     "taac_flash_attn_mask_bwd": (
         c_int,
@@ -155,7 +156,8 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "taac_flash_attn_bits_bwd": (
         c_int,
-        [c_void_p] * 8 + [c_int64] + [c_void_p] * 5 + [c_int32] * 5 + [ctypes.POINTER(c_int64)] * 8 + [c_int, c_int, c_void_p],
+        [c_void_p] * 8 + [c_int64] + [c_void_p] * 2 + [c_float] + [c_void_p] * 4 + [c_int32] * 5
+        + [ctypes.POINTER(c_int64)] * 8 + [c_int, c_int, c_void_p],
     ),
     "taac_flash_attn_train_dropout_fwd": (
         c_int,

@@ -559,7 +559,8 @@ class _HipFlashAttentionFunction(torch.autograd.Function):
 
 
 def masked_attention_backward(q, k, v, out, grad_out, lse, key_lengths, mask: StructuredAttentionMask, dq, dk, dv, *,
-                              zero_padded_queries: bool = False) -> None:
+                              zero_padded_queries: bool = False, dropout_mask: torch.Tensor | None = None,
+                              dropout_scale: float = 1.0) -> None:
     """``taac_flash_attn_bits_bwd`` for (B, H, T, d) views under a structured mask (either layout: one structure for the
     batch, or one per sample with the valid tokens in front), writing into ``dq`` / ``dk`` / ``dv`` (any element strides
     with a unit last one). A self-only query returned its own value row: its row is taken out of the kernels
@@ -573,7 +574,8 @@ def masked_attention_backward(q, k, v, out, grad_out, lse, key_lengths, mask: St
     status = library.taac_flash_attn_bits_bwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), grad_out.data_ptr(), lse.data_ptr(),
         _native.ptr(key_lengths), mask.struct_bits.data_ptr(), int(mask.sample_stride), _native.ptr(mask.valid_bits),
-        dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(), batch, heads, query_len, k.shape[2], head_dim,
+        _native.ptr(dropout_mask), ctypes.c_float(dropout_scale), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+        delta.data_ptr(), batch, heads, query_len, k.shape[2], head_dim,
         *strides, int(bool(zero_padded_queries)), _native.dtype_code(q.dtype), _native.current_stream(q.device))
     _native.check(status, "flash_attention backward")
     if mask.query_self is not None:
@@ -586,7 +588,8 @@ class _HipMaskedAttentionFunction(torch.autograd.Function):
     bool masks, which the reference's accelerated path rejects (flash_attention.py:183-209)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, key_lengths, mask: StructuredAttentionMask, zero_padded_queries: bool):
+    def forward(ctx, q, k, v, key_lengths, mask: StructuredAttentionMask, zero_padded_queries: bool,
+                dropout_mask: torch.Tensor | None = None, dropout_p: float = 0.0):
         library = _native.load_library()
         q, k, v = _kernel_view(q), _kernel_view(k), _kernel_view(v)
         out = _dense_like(q)
@@ -597,17 +600,27 @@ class _HipMaskedAttentionFunction(torch.autograd.Function):
                 or (mask.sample_stride and mask.struct_bits.shape[0] != batch * query_len):
             raise ValueError("flash_attention: the structured mask does not match (batch, query_len, kv_len)")
         require_cuda_tensors("hip flash_attention", q, k, v, mask.struct_bits)
+        scale = 1.0
+        if dropout_mask is not None:
+            if mask.query_self is not None:
+                raise RuntimeError("hip flash_attention: dropout does not come with self-only query rows")
+            if dropout_mask.dtype != torch.uint8 or tuple(dropout_mask.shape) != (batch, heads, query_len, k.shape[2]):
+                raise ValueError("flash_attention dropout_mask must be uint8 of shape (B, H, Tq, Tk)")
+            require_cuda_tensors("hip flash_attention", dropout_mask)
+            dropout_mask = dropout_mask.contiguous()
+            scale = 1.0 / (1.0 - dropout_p)
         lse = torch.empty(batch, heads, query_len, dtype=torch.float32, device=q.device)
         status = library.taac_flash_attn_masked_train_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), mask.struct_bits.data_ptr(),
             int(mask.sample_stride), _native.ptr(mask.block_any), _native.ptr(mask.valid_bits), _native.ptr(mask.self_bits),
-            out.data_ptr(),
+            _native.ptr(dropout_mask), ctypes.c_float(scale), out.data_ptr(),
             lse.data_ptr(), batch, heads, query_len, k.shape[2], head_dim, _native.Int64x4(*q.stride()),
             _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()), _native.Int64x4(*out.stride()),
             int(bool(zero_padded_queries)), _native.dtype_code(q.dtype), _native.current_stream(q.device))
         _native.check(status, "flash_attention")
         ctx.save_for_backward(q, k, v, out, lse, *(() if key_lengths is None else (key_lengths,)))
         ctx.mask, ctx.has_lengths, ctx.zero_padded_queries = mask, key_lengths is not None, bool(zero_padded_queries)
+        ctx.dropout_mask, ctx.dropout_scale = dropout_mask, scale
         return out
 
     @staticmethod
@@ -617,8 +630,9 @@ class _HipMaskedAttentionFunction(torch.autograd.Function):
         grad_out = _kernel_view(grad_out)
         dq, dk, dv = _dense_like(q), _dense_like(k), _dense_like(v)
         masked_attention_backward(q, k, v, out, grad_out, lse, key_lengths, ctx.mask, dq, dk, dv,
-                                  zero_padded_queries=ctx.zero_padded_queries)
-        return dq, dk, dv, None, None, None
+                                  zero_padded_queries=ctx.zero_padded_queries, dropout_mask=ctx.dropout_mask,
+                                  dropout_scale=ctx.dropout_scale)
+        return dq, dk, dv, None, None, None, None, None
 
 
 def flash_attention(
@@ -667,9 +681,8 @@ def flash_attention(
     _resolve_flash_attention_backend(q, backend, dropout_p=dropout_p, training=training)
     needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v))
     use_dropout = training and dropout_p > 0.0
-    if use_dropout and (structured_mask is not None or q_row_scale is not None or k_row_scale is not None
-                        or q_col_scale is not None):
-        raise RuntimeError("hip flash_attention dropout covers key-length and causal masks only")
+    if use_dropout and (q_row_scale is not None or k_row_scale is not None or q_col_scale is not None):
+        raise RuntimeError("hip flash_attention dropout does not come with row factors")
     if needs_grad and (q_row_scale is not None or k_row_scale is not None or q_col_scale is not None
                        or q.dtype == torch.float32):
         raise RuntimeError("hip flash_attention backward covers bf16 / fp16 inputs without row factors; call it under "
@@ -697,12 +710,13 @@ def flash_attention(
     if needs_grad or use_dropout:
         if lengths is not None:
             lengths = lengths.to(torch.int32).contiguous()
-        if structured_mask is not None:
-            output = _HipMaskedAttentionFunction.apply(q, k, v, lengths, structured_mask, zero_padded_queries)
-            return output if output.dtype == output_dtype else output.to(output_dtype)
         mask = None
         if use_dropout:
             mask = dropout_mask if dropout_mask is not None else build_dropout_mask(q, k, dropout_p)
+        if structured_mask is not None:
+            output = _HipMaskedAttentionFunction.apply(q, k, v, lengths, structured_mask, zero_padded_queries, mask,
+                                                       float(dropout_p) if use_dropout else 0.0)
+            return output if output.dtype == output_dtype else output.to(output_dtype)
         output = _HipFlashAttentionFunction.apply(q, k, v, lengths, plan.is_causal, zero_padded_queries, kv_staging, mask,
                                                   float(dropout_p) if use_dropout else 0.0)
         if plan.query_self_mask is not None:

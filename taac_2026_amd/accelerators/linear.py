@@ -238,6 +238,67 @@ class _SwigluFfnFunction(torch.autograd.Function):
                 grad_out if has_residual else None, grad_norm, None, None)
 
 
+class _SwigluDropoutFfnFunction(torch.autograd.Function):
+    """``residual + down(keep / (1 - p) * silu(gate) * value)``, ``gate, value = up(x)``: the feed-forward of the reference's
+    blocks in training mode (``down(dropout(silu(gate) * value))``, experiments/symbiosis/backbone.py:11-21) under a keep
+    mask ``[.., F]`` of the hidden state drawn by the caller. The hidden state reaches memory here (the mask applies to
+    it): up projection with the activation in its epilogue, the mask as an element-wise product, down projection; the
+    backward recomputes the up projection and runs the activation backward, both weight gradients and both input
+    gradients as HIP kernels."""
+
+    @staticmethod
+    def forward(ctx, x, up_weight, up_bias, down_weight, down_bias, residual, keep, scale, gate_first):
+        with torch.no_grad():
+            hidden = swiglu_linear(x, up_weight, up_bias, gate_first=gate_first)
+            dropped = hidden * keep.to(hidden.dtype) * scale
+            out = _plain_product(dropped, down_weight, down_bias)
+            if residual is not None:
+                out = out + residual
+        ctx.save_for_backward(x, up_weight, down_weight, dropped, keep, *(() if up_bias is None else (up_bias,)))
+        ctx.flags = (up_bias is not None, down_bias is not None, residual is not None, bool(gate_first), float(scale))
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        has_up_bias, has_down_bias, has_residual, gate_first, scale = ctx.flags
+        x, up_weight, down_weight, dropped, keep, *rest = ctx.saved_tensors
+        up_bias = rest[0] if has_up_bias else None
+        rows, shape = _as_rows(x)
+        rows = rows.contiguous()
+        dy, _ = _as_rows(grad_out if grad_out.dtype == torch.bfloat16 else grad_out.to(torch.bfloat16))
+        dy = dy.contiguous()
+        with torch.no_grad():
+            dropped_rows, _ = _as_rows(dropped)
+            grad_down_w, grad_down_b = linear_wgrad(dy, dropped_rows.contiguous(), with_bias=has_down_bias)
+            grad_hidden = _input_grad(dy, down_weight) * (_as_rows(keep)[0].to(dy.dtype) * scale)
+            pre = _plain_product(rows, up_weight.detach(), None if up_bias is None else up_bias.detach())
+            _, grad_pre = swiglu_backward(pre, grad_hidden.contiguous(), gate_first=gate_first, want_hidden=False)
+            grad_up_w, grad_up_b = linear_wgrad(grad_pre, rows, with_bias=has_up_bias)
+            grad_rows = _input_grad(grad_pre, up_weight)
+        return (grad_rows.reshape(shape), grad_up_w, grad_up_b, grad_down_w, grad_down_b,
+                grad_out if has_residual else None, None, None, None)
+
+
+def swiglu_ffn_dropout(x: torch.Tensor, up_weight: torch.Tensor, up_bias: torch.Tensor | None, down_weight: torch.Tensor,
+                       down_bias: torch.Tensor | None, *, dropout_p: float, residual: torch.Tensor | None = None,
+                       gate_first: bool = True, keep_mask: torch.Tensor | None = None) -> torch.Tensor:
+    """The reference's feed-forward in training mode: ``residual + down(dropout(silu(gate) * value))``. ``keep_mask``
+    (bool or uint8 ``[.., F]``, non-zero = keep) fixes the dropped units; without it one is drawn from torch's generator
+    (``rand >= p``). Differentiable; bf16 tensors."""
+    name = "hip swiglu_ffn_dropout"
+    require_cuda_tensors(name, x, up_weight, up_bias, down_weight, down_bias, residual, keep_mask)
+    _check_bf16(name, x, up_weight, up_bias, down_weight, down_bias, residual)
+    if not 0.0 <= dropout_p < 1.0:
+        raise ValueError(f"{name}: dropout_p must be in [0, 1)")
+    hidden_shape = (*x.shape[:-1], down_weight.shape[1])
+    if keep_mask is None:
+        keep_mask = torch.rand(hidden_shape, device=x.device) >= dropout_p
+    elif tuple(keep_mask.shape) != hidden_shape:
+        raise ValueError(f"{name}: keep_mask must have shape {hidden_shape}")
+    return _SwigluDropoutFfnFunction.apply(x, up_weight, up_bias, down_weight, down_bias, residual, keep_mask,
+                                           1.0 / (1.0 - dropout_p), bool(gate_first))
+
+
 def linear(
     x: torch.Tensor,
     weight: torch.Tensor,
@@ -978,6 +1039,7 @@ __all__ = [
     "linear_fp8",
     "linear_wgrad",
     "swiglu_ffn_backward_hidden",
+    "swiglu_ffn_dropout",
     "swiglu_backward",
     "norm_linear",
     "pack_ffn_weights",

@@ -146,7 +146,7 @@ __device__ __forceinline__ uint32_t keep_bytes4(const uint8_t* row, int key0, in
 
 template <typename T, int DP, bool CAUSAL, bool SCALED, bool MASKED, bool DROPOUT = false>
 __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnParams p) {
-  static_assert(!(DROPOUT && (SCALED || MASKED)), "dropout comes with the key-length / causal masks of the training path");
+  static_assert(!(DROPOUT && SCALED && !MASKED), "dropout comes with the masks of the training path, not with row factors");
   static_assert(!(MASKED && CAUSAL), "a structured mask carries its own causal triangle");
   typedef typename Vec8<T>::type vec_t;
   typedef typename Vec8<T>::half_type vec4_t;
@@ -1286,7 +1286,9 @@ void launch(const AttnParams& p, bool causal, bool register_staging, hipStream_t
       return;
     }
   }
-  if (p.drop_mask != nullptr && causal)
+  if (p.drop_mask != nullptr && p.struct_bits != nullptr)
+    hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false, true, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+  else if (p.drop_mask != nullptr && causal)
     hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, true, false, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
   else if (p.drop_mask != nullptr)
     hipLaunchKernelGGL((flash_attn_fwd_kernel<T, DP, false, false, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
@@ -1363,9 +1365,9 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
                     const int64_t k_strides[4], const int64_t v_strides[4], const int64_t o_strides[4], int mask_flags,
                     int zero_padded_queries, int dtype, void* stream, const uint8_t* drop_mask = nullptr,
                     float drop_scale = 1.f) {
-  if (drop_mask != nullptr && (mask.struct_bits != nullptr || q_row_scale != nullptr || k_row_scale != nullptr ||
-                               q_col_scale != nullptr))
-    return set_error(TAAC_ERR_UNSUPPORTED, "%s: dropout comes with key-length and causal masks only", name);
+  if (drop_mask != nullptr && (mask.self_bits != nullptr || mask.compact_keys != nullptr || q_row_scale != nullptr ||
+                               k_row_scale != nullptr || q_col_scale != nullptr))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: dropout does not come with self-only query rows or row factors", name);
   if (drop_mask != nullptr && !(drop_scale >= 1.f))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: dropout_scale = 1 / (1 - p) must be >= 1", name);
   if (mask_flags & ~(TAAC_ATTN_CAUSAL | TAAC_ATTN_REGISTER_STAGING))
@@ -1529,7 +1531,8 @@ extern "C" int taac_flash_attn_masked_fwd(const void* q, const void* k, const vo
 extern "C" int taac_flash_attn_masked_train_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,
                                                 const uint32_t* struct_bits, int64_t struct_sample_stride,
                                                 const uint8_t* block_any, const uint32_t* valid_bits,
-                                                const uint32_t* self_bits, void* o, float* lse, int32_t B, int32_t H,
+                                                const uint32_t* self_bits, const uint8_t* dropout_mask,
+                                                float dropout_scale, void* o, float* lse, int32_t B, int32_t H,
                                                 int32_t Tq, int32_t Tk, int32_t d, const int64_t q_strides[4],
                                                 const int64_t k_strides[4], const int64_t v_strides[4],
                                                 const int64_t o_strides[4], int zero_padded_queries, int dtype,
@@ -1544,7 +1547,8 @@ extern "C" int taac_flash_attn_masked_train_fwd(const void* q, const void* k, co
   mask.valid_bits = valid_bits;
   mask.self_bits = self_bits;
   return taac::attention_entry(name, q, k, v, key_lengths, mask, nullptr, nullptr, nullptr, lse, nullptr, o, B, H, Tq, Tk, d,
-                               q_strides, k_strides, v_strides, o_strides, 0, zero_padded_queries, dtype, stream);
+                               q_strides, k_strides, v_strides, o_strides, 0, zero_padded_queries, dtype, stream,
+                               dropout_mask, dropout_mask != nullptr ? dropout_scale : 1.f);
 }
 
 extern "C" int taac_flash_attn_sparse_fwd(const void* q, const void* k, const void* v, const int32_t* key_lengths,

@@ -41,6 +41,9 @@ struct AttnBwdParams {
                              // training dropout (keep mask, non-zero = keep) or pair visibility (non-zero = visible)
   int64_t mask_bs, mask_hs;  // elements between the mask matrices of consecutive samples / heads (0: shared)
   const uint8_t* key_valid;  // visibility mode: [B, Tk] bytes, non-zero = the key can be seen at all; or null
+                             // (bit modes: [B, ceil(Tk / 32)] words)
+  const uint32_t* bit_words; // bit modes: rows of ceil(Tk / 32) words per query, bits_bs words between the samples' matrices
+  int64_t bits_bs;
   float drop_scale;          // 1 / (1 - p)
   int32_t B, H, Tq, Tk, d;
   int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4];
@@ -277,11 +280,13 @@ __device__ __forceinline__ uint32_t keep_bytes4(const uint8_t* row, int key0, in
 // kMaskBits: the same as bits, in the layout of the structured forward: drop_mask holds 32-bit words, row i of a sample's
 // matrix at word (b * mask_bs + i * wpr), wpr = ceil(Tk / 32), bit j % 32 of word j / 32 = pair (i, j); key_valid holds
 // [B, wpr] words. One word per 32-key tile instead of 32 bytes.
-constexpr int kMaskNone = 0, kMaskDropout = 1, kMaskVisible = 2, kMaskBits = 3;
+// kMaskBitsDropout: the bit form for the pairs AND the byte keep mask of dropout (both pointers).
+constexpr int kMaskNone = 0, kMaskDropout = 1, kMaskVisible = 2, kMaskBits = 3, kMaskBitsDropout = 4;
 
 template <typename T, int DP, bool DMA, int MODE = kMaskNone>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 32 ? 4 : 3))) void attn_bwd_dq_kernel(const AttnBwdParams p) {
-  constexpr bool DROPOUT = MODE == kMaskDropout;
+  constexpr bool DROPOUT = MODE == kMaskDropout || MODE == kMaskBitsDropout;
+  constexpr bool BITS = MODE == kMaskBits || MODE == kMaskBitsDropout;
   typedef typename Vec8<T>::type vec_t;
   constexpr int KSTEPS = DP / 16, MB = DP / 32;
   constexpr int ROWB = DP * 2, TILE_BYTES = kChunk * ROWB, BUF_BYTES = 2 * TILE_BYTES;  // a chunk of K, then of V
@@ -354,7 +359,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 
   [[maybe_unused]] uint32_t chunk_words[kChunk / 32] = {}, next_words[kChunk / 32] = {};
   auto fetch_words = [&](int kc0, uint32_t (&dst)[kChunk / 32]) {
     const int wpr = (p.Tk + 31) / 32;
-    const uint32_t* row = reinterpret_cast<const uint32_t*>(p.drop_mask) + b * p.mask_bs + static_cast<int64_t>(qi < p.Tq ? qi : 0) * wpr;
+    const uint32_t* row = p.bit_words + b * p.bits_bs + static_cast<int64_t>(qi < p.Tq ? qi : 0) * wpr;
     const uint32_t* valid = p.key_valid != nullptr ? reinterpret_cast<const uint32_t*>(p.key_valid) + static_cast<int64_t>(b) * wpr : nullptr;
 #pragma unroll
     for (int t = 0; t < kChunk / 32; ++t) {
@@ -364,11 +369,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 
       if (inside && valid != nullptr) dst[t] &= valid[w];
     }
   };
-  if (MODE == kMaskBits && kv_end > 0) fetch_words(0, chunk_words);
+  if (BITS && kv_end > 0) fetch_words(0, chunk_words);
   if (kv_end > 0) fetch(0, 0);
   int buf = 0;
   for (int kc0 = 0; kc0 < kv_end; kc0 += kChunk) {
-    if (MODE == kMaskBits && kc0 + kChunk < kv_end) fetch_words(kc0 + kChunk, next_words);
+    if (BITS && kc0 + kChunk < kv_end) fetch_words(kc0 + kChunk, next_words);
     if (DMA) {
       vm_wait<0>();     // this wavefront's pieces of the chunk have landed ...
       __syncthreads();  // ... everyone's have, and everyone is done reading the other buffer
@@ -417,6 +422,23 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 
           const float prob = on ? __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -lse2)) : 0.f;
           dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -delta_scaled));
         }
+      } else if (MODE == kMaskBitsDropout) {
+        const uint32_t word = chunk_words[kt];
+        const bool aligned = (p.Tk % 4 == 0) && (reinterpret_cast<uintptr_t>(p.drop_mask) % 4 == 0) &&
+                             p.mask_bs % 4 == 0 && p.mask_hs % 4 == 0;
+        const uint8_t* row = p.drop_mask + b * p.mask_bs + h * p.mask_hs + static_cast<int64_t>(qi < p.Tq ? qi : 0) * p.Tk;
+#pragma unroll
+        for (int jq = 0; jq < 4; ++jq) {
+          const uint32_t keep = qi < p.Tq ? keep_bytes4(row, k_tile + jq * 8 + hh * 4, p.Tk, aligned) : 0u;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int j = jq * 4 + e;
+            const bool visible = ((word >> (jq * 8 + hh * 4 + e)) & 1u) != 0u;
+            const float prob = visible ? __builtin_amdgcn_exp2f(fmaf(sacc[j], c, -lse2)) : 0.f;
+            const float dp = ((keep >> (8 * e)) & 0xffu) != 0u ? dpacc[j] * p.drop_scale : 0.f;
+            dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dp, p.scale, -delta_scaled));
+          }
+        }
       } else if (MODE != kMaskNone) {
         const bool aligned = (p.Tk % 4 == 0) && (reinterpret_cast<uintptr_t>(p.drop_mask) % 4 == 0) &&
                              p.mask_bs % 4 == 0 && p.mask_hs % 4 == 0;
@@ -451,7 +473,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 
       }
       accumulate_columns<T, DP, kt * 32 * ROWB>(dqacc, dsb, col_addr);
     });
-    if (MODE == kMaskBits) {
+    if (BITS) {
 #pragma unroll
       for (int t = 0; t < kChunk / 32; ++t) chunk_words[t] = next_words[t];
     }
@@ -462,7 +484,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DP == 
 
 template <typename T, int DP, bool DMA, int MODE = kMaskNone>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP == 32 ? 4 : 3) - (DMA ? 0 : 1)))) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
-  constexpr bool DROPOUT = MODE == kMaskDropout;
+  constexpr bool DROPOUT = MODE == kMaskDropout || MODE == kMaskBitsDropout;
+  constexpr bool BITS = MODE == kMaskBits || MODE == kMaskBitsDropout;
   typedef typename Vec8<T>::type vec_t;
   constexpr int KSTEPS = DP / 16, MB = DP / 32;
   constexpr int ROWB = DP * 2, TILE_BYTES = kChunk * ROWB;
@@ -470,7 +493,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
   // each wavefront, [wavefront][row]
   constexpr int kWaves = kThreads / kWave;
   static_assert(kThreads == kWaves * kChunk, "one mask word per thread and chunk");
-  constexpr int BUF_BYTES = 2 * TILE_BYTES + 2 * kChunk * 4 + (MODE == kMaskBits ? kWaves * kChunk * 4 : 0);
+  constexpr int BUF_BYTES = 2 * TILE_BYTES + 2 * kChunk * 4 + (BITS ? kWaves * kChunk * 4 : 0);
   constexpr int NBUF = DMA ? 2 : 1;
   constexpr int OROW = DP * 2 + 16;
   constexpr int OUT_BYTES = (kThreads / kWave) * 32 * OROW;
@@ -502,7 +525,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
   [[maybe_unused]] const int bit_wpr = (p.Tk + 31) / 32;
   [[maybe_unused]] bool key_seen = kj < p.Tk;
   if (MODE == kMaskVisible && key_seen && p.key_valid != nullptr) key_seen = p.key_valid[static_cast<int64_t>(b) * p.Tk + kj] != 0;
-  if (MODE == kMaskBits && key_seen && p.key_valid != nullptr)
+  if (BITS && key_seen && p.key_valid != nullptr)
     key_seen = ((reinterpret_cast<const uint32_t*>(p.key_valid)[static_cast<int64_t>(b) * ((p.Tk + 31) / 32) + kj / 32] >> (kj % 32)) & 1u) != 0u;
   const bool k_ok = kj < len;
   // queries that can see a key of this block: all valid ones, or (causal) those at or after the block's first key
@@ -533,11 +556,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
         lse_next = qi < q_valid ? p.lse[stat0 + qi] : -INFINITY;
         delta_next = qi < q_valid ? p.delta[stat0 + qi] : 0.f;
       }
-      if (MODE == kMaskBits) {  // thread (w, r): the word of query row qc0 + r that covers the keys of wavefront w
+      if (BITS) {  // thread (w, r): the word of query row qc0 + r that covers the keys of wavefront w
         const int qi = qc0 + tid % kChunk, key0 = k_begin + (tid / kChunk) * 32;
-        word_next = (qi < q_valid && key0 < p.Tk)
-                        ? reinterpret_cast<const uint32_t*>(p.drop_mask)[b * p.mask_bs + static_cast<int64_t>(qi) * bit_wpr + key0 / 32]
-                        : 0u;
+        word_next = (qi < q_valid && key0 < p.Tk) ? p.bit_words[b * p.bits_bs + static_cast<int64_t>(qi) * bit_wpr + key0 / 32] : 0u;
       }
     };
     // the row statistics travel through registers: base-2 log-sum-exp (+inf: the row carries nothing, exp2(x - inf) = 0)
@@ -548,7 +569,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
         stats[tid] = lse_next > -INFINITY ? lse_next * 1.4426950408889634f : INFINITY;
         stats[kChunk + tid] = delta_next * p.scale;
       }
-      if (MODE == kMaskBits)
+      if (BITS)
         reinterpret_cast<uint32_t*>(smem + buffer * BUF_BYTES + 2 * TILE_BYTES + 2 * kChunk * 4)[tid] = word_next;
     };
     const uint32_t row_off = streamed_row_offset<DP>(l32, hh);
@@ -609,7 +630,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
           const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sLse[r0]);
           const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[r0]);  // already times 1 / sqrt(d)
           [[maybe_unused]] u32x4 w4 = {0u, 0u, 0u, 0u};
-          if (MODE == kMaskBits) w4 = *reinterpret_cast<const u32x4*>(&sWords[r0]);
+          if (BITS) w4 = *reinterpret_cast<const u32x4*>(&sWords[r0]);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int j = jq * 4 + e;
@@ -619,6 +640,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((DP ==
               prob = (key_seen && ((w4[e] >> l32) & 1u) != 0u) ? prob : 0.f;
               pb[j / 8][j % 8] = static_cast<T>(prob);
               dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(dpacc[j], p.scale, -d4[e]));
+            } else if (MODE == kMaskBitsDropout) {
+              const int qrow = qc0 + r0 + e;
+              prob = (key_seen && ((w4[e] >> l32) & 1u) != 0u) ? prob : 0.f;
+              const bool keep = qrow < p.Tq && kj < p.Tk &&
+                                p.drop_mask[b * p.mask_bs + h * p.mask_hs + static_cast<int64_t>(qrow) * p.Tk + kj] != 0;
+              pb[j / 8][j % 8] = static_cast<T>(keep ? prob * p.drop_scale : 0.f);
+              dsb[j / 8][j % 8] = static_cast<T>(prob * fmaf(keep ? dpacc[j] * p.drop_scale : 0.f, p.scale, -d4[e]));
             } else if (MODE != kMaskNone) {
               // the lane owns key kj; register j is query qc0 + r0 + e: one mask byte per register
               const int qrow = qc0 + r0 + e;
@@ -694,6 +722,8 @@ void launch_bwd_dp(const AttnBwdParams& p, int mode, bool register_staging, hipS
     launch_bwd_mode<T, DP, kMaskVisible>(p, register_staging, s);
   else if (mode == kMaskBits)
     launch_bwd_mode<T, DP, kMaskBits>(p, register_staging, s);
+  else if (mode == kMaskBitsDropout)
+    launch_bwd_mode<T, DP, kMaskBitsDropout>(p, register_staging, s);
   else
     launch_bwd_mode<T, DP, kMaskNone>(p, register_staging, s);
 }
@@ -718,10 +748,10 @@ int attention_bwd_entry(const char* name, const void* q, const void* k, const vo
                         const int64_t o_strides[4], const int64_t do_strides[4], const int64_t dq_strides[4],
                         const int64_t dk_strides[4], const int64_t dv_strides[4], int is_causal, int zero_padded_queries,
                         int dtype, void* stream, int mask_mode = -1, int64_t mask_bs = 0, int64_t mask_hs = 0,
-                        const uint8_t* key_valid = nullptr) {
+                        const uint8_t* key_valid = nullptr, const uint32_t* bit_words = nullptr, int64_t bits_bs = 0) {
   // mask_mode -1: dropout when a mask is given (its matrices follow the (B, H) order), nothing otherwise
-  if (mask_mode < 0) {
-    mask_mode = drop_mask != nullptr ? kMaskDropout : kMaskNone;
+  if (mask_mode < 0 || mask_mode == kMaskBitsDropout) {
+    if (mask_mode < 0) mask_mode = drop_mask != nullptr ? kMaskDropout : kMaskNone;
     mask_hs = static_cast<int64_t>(Tq) * Tk;
     mask_bs = mask_hs * H;
   }
@@ -770,6 +800,8 @@ int attention_bwd_entry(const char* name, const void* q, const void* k, const vo
   p.mask_bs = mask_bs;
   p.mask_hs = mask_hs;
   p.key_valid = key_valid;
+  p.bit_words = bit_words;
+  p.bits_bs = bits_bs;
   p.drop_scale = drop_scale;
   p.B = B;
   p.H = H;
@@ -846,8 +878,9 @@ extern "C" int taac_flash_attn_mask_bwd(const void* q, const void* k, const void
 
 extern "C" int taac_flash_attn_bits_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout,
                                         const float* lse, const int32_t* key_lengths, const uint32_t* struct_bits,
-                                        int64_t struct_sample_stride, const uint32_t* valid_bits, void* dq, void* dk,
-                                        void* dv, float* delta, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
+                                        int64_t struct_sample_stride, const uint32_t* valid_bits,
+                                        const uint8_t* dropout_mask, float dropout_scale, void* dq, void* dk, void* dv,
+                                        float* delta, int32_t B, int32_t H, int32_t Tq, int32_t Tk, int32_t d,
                                         const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
                                         const int64_t o_strides[4], const int64_t do_strides[4],
                                         const int64_t dq_strides[4], const int64_t dk_strides[4],
@@ -855,9 +888,10 @@ extern "C" int taac_flash_attn_bits_bwd(const void* q, const void* k, const void
   const char* name = "taac_flash_attn_bits_bwd";
   if (!struct_bits) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: struct_bits must be given", name);
   if (struct_sample_stride < 0) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: negative sample stride", name);
-  return taac::attention_bwd_entry(name, q, k, v, o, dout, lse, key_lengths, reinterpret_cast<const uint8_t*>(struct_bits),
-                                   1.f, dq, dk, dv, delta, B, H, Tq, Tk, d, q_strides, k_strides, v_strides, o_strides,
-                                   do_strides, dq_strides, dk_strides, dv_strides, 0, zero_padded_queries, dtype, stream,
-                                   taac::kMaskBits, struct_sample_stride, 0,
-                                   reinterpret_cast<const uint8_t*>(valid_bits));
+  return taac::attention_bwd_entry(name, q, k, v, o, dout, lse, key_lengths, dropout_mask,
+                                   dropout_mask != nullptr ? dropout_scale : 1.f, dq, dk, dv, delta, B, H, Tq, Tk, d,
+                                   q_strides, k_strides, v_strides, o_strides, do_strides, dq_strides, dk_strides,
+                                   dv_strides, 0, zero_padded_queries, dtype, stream,
+                                   dropout_mask != nullptr ? taac::kMaskBitsDropout : taac::kMaskBits, 0, 0,
+                                   reinterpret_cast<const uint8_t*>(valid_bits), struct_bits, struct_sample_stride);
 }

@@ -22,7 +22,7 @@ import torch.nn as nn
 from taac_2026_amd import _native
 from taac_2026_amd.accelerators.attention import StructuredAttentionMask, front_structured_mask, qk_norm_rope, rope_table
 from taac_2026_amd.accelerators.linear import (attention_out_ffn, front_rows, norm_linear, qkv_projection, swiglu_ffn,
-                                               valid_rows)
+                                               swiglu_ffn_dropout, valid_rows)
 from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference
 from taac_2026_amd.modeling.block_training import run_training_block, training_route_applies
 from taac_2026_amd.modeling.normalization import RMSNorm
@@ -52,10 +52,14 @@ class SwiGLUFeedForward(nn.Module):
         self.gate_first = bool(gate_first)
 
     def forward(self, tokens: torch.Tensor, *, residual: torch.Tensor | None = None) -> torch.Tensor:
-        if self.training and self.dropout.p > 0.0:
-            raise RuntimeError("hip SwiGLUFeedForward is forward-only inference and does not apply dropout")
         output_dtype = tokens.dtype
         x = tokens if tokens.dtype == torch.bfloat16 else tokens.to(torch.bfloat16)
+        if self.training and self.dropout.p > 0.0:
+            # dropout of the hidden state (experiments/symbiosis/backbone.py:19-21): the hidden state reaches memory
+            out = swiglu_ffn_dropout(x, _bf16(self.up.weight), _bf16(self.up.bias), _bf16(self.down.weight),
+                                     _bf16(self.down.bias), dropout_p=self.dropout.p, residual=_bf16(residual),
+                                     gate_first=self.gate_first)
+            return out if out.dtype == output_dtype else out.to(output_dtype)
         out = swiglu_ffn(x, _bf16(self.up.weight), _bf16(self.up.bias), _bf16(self.down.weight), _bf16(self.down.bias),
                          residual=_bf16(residual), gate_first=self.gate_first)
         return out if out.dtype == output_dtype else out.to(output_dtype)

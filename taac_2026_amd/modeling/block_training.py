@@ -17,6 +17,7 @@ or mask object (one host synchronisation, shared by the blocks of a stack).
 
 from __future__ import annotations
 
+import ctypes
 import importlib
 import weakref
 
@@ -175,7 +176,8 @@ class InteractionBlockFunction(torch.autograd.Function):
             status = library.taac_flash_attn_masked_train_fwd(
                 qkv.data_ptr(), qkv.data_ptr() + width * element, qkv.data_ptr() + 2 * width * element,
                 _native.ptr(key_lengths), mask.struct_bits.data_ptr(), int(mask.sample_stride), _native.ptr(mask.block_any),
-                _native.ptr(mask.valid_bits), _native.ptr(mask.self_bits), attended.data_ptr(), lse.data_ptr(), batch,
+                _native.ptr(mask.valid_bits), _native.ptr(mask.self_bits), None, ctypes.c_float(1.0), attended.data_ptr(),
+                lse.data_ptr(), batch,
                 num_heads, token_count, token_count, width // num_heads, qkv_strides, qkv_strides, qkv_strides, out_strides,
                 0 if front is None else 1, _native.dtype_code(flat.dtype), _native.current_stream(tokens.device))
         _native.check(status, "interaction block (training): attention")

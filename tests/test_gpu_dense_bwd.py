@@ -547,3 +547,38 @@ def test_backbone_module_trains(device, qk_norm):
     for name, parameter in model.named_parameters():
         assert parameter.grad is not None, name
         _close(parameter.grad, reference[name].grad, 5e-2)
+
+
+@pytest.mark.parametrize("gate_first", [True, False])
+def test_feed_forward_with_dropout_of_the_hidden_state(device, gate_first):
+    """``down(dropout(silu(gate) * value))`` (experiments/symbiosis/backbone.py:19-21) under a fixed keep mask: output and
+    every gradient against float64 autograd of the same formula; without a mask one is drawn from torch's generator."""
+    from taac_2026_amd.api import swiglu_ffn_dropout
+
+    rows, d_model, hidden, p = 300, 128, 256, 0.25
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(rows, d_model, generator=g).to(torch.bfloat16)
+    w_up = (torch.randn(2 * hidden, d_model, generator=g) * d_model ** -0.5).to(torch.bfloat16)
+    b_up = (0.1 * torch.randn(2 * hidden, generator=g)).to(torch.bfloat16)
+    w_down = (torch.randn(d_model, hidden, generator=g) * hidden ** -0.5).to(torch.bfloat16)
+    b_down = (0.1 * torch.randn(d_model, generator=g)).to(torch.bfloat16)
+    keep = torch.rand(rows, hidden, generator=g) >= p
+    grad_out = torch.randn(rows, d_model, generator=g).to(torch.bfloat16)
+    ref = [t.double().requires_grad_(True) for t in (x, w_up, b_up, w_down, b_down)]
+    first, second = F.linear(ref[0], ref[1], ref[2]).chunk(2, dim=-1)
+    hidden_r = (F.silu(first) * second) if gate_first else (first * F.silu(second))
+    want = ref[0] + F.linear(hidden_r * keep.double() / (1.0 - p), ref[3], ref[4])
+    want.backward(grad_out.double())
+    dev = [t.to(device).requires_grad_(True) for t in (x, w_up, b_up, w_down, b_down)]
+    out = swiglu_ffn_dropout(dev[0], dev[1], dev[2], dev[3], dev[4], dropout_p=p, residual=dev[0], gate_first=gate_first,
+                             keep_mask=keep.to(device))
+    out.backward(grad_out.to(device))
+    _close(out, want.detach(), 2e-2)
+    for got, expected in zip(dev, ref):
+        _close(got.grad, expected.grad, 3e-2)
+    torch.manual_seed(3)
+    a = swiglu_ffn_dropout(dev[0].detach(), dev[1], dev[2], dev[3], dev[4], dropout_p=p)
+    torch.manual_seed(3)
+    b = swiglu_ffn_dropout(dev[0].detach(), dev[1], dev[2], dev[3], dev[4], dropout_p=p)
+    c = swiglu_ffn_dropout(dev[0].detach(), dev[1], dev[2], dev[3], dev[4], dropout_p=p)
+    assert torch.equal(a, b) and not torch.equal(a, c)

@@ -412,3 +412,74 @@ def test_mask_bwd_abi_reads_any_bool_mask(device, per_head, per_sample, with_val
     _native.check(status, "taac_flash_attn_mask_bwd")
     for got, want, name in zip(grads, (qr.grad, kr.grad, vr.grad), ("dq", "dk", "dv")):
         torch.testing.assert_close(got.cpu().double(), want, msg=lambda m, n=name: f"{n}: {m}", **GRAD_TOL)
+
+
+@pytest.mark.parametrize("tokens,dim,with_lengths", [(130, 32, False), (200, 64, True), (96, 16, False)])
+def test_structured_mask_with_dropout_takes_a_gradient(device, tokens, dim, with_lengths):
+    """Dropout on the probabilities under a structured mask with a fixed keep mask - what the reference's models train
+    with by default (``F.scaled_dot_product_attention(attn_mask=, dropout_p=)``, experiments/symbiosis/__init__.py:87):
+    output and gradients against float64 autograd of the oracle's closed form (normaliser over the visible keys, then
+    keep / (1 - p))."""
+    batch, heads, dropout_p = 3, 2, 0.125
+    g = torch.Generator().manual_seed(tokens + dim)
+    q, k, v, grad_out = (torch.randn(batch, heads, tokens, dim, generator=g).to(torch.bfloat16) for _ in range(4))
+    structural = (torch.rand(tokens, tokens, generator=g) < 0.5) | torch.eye(tokens, dtype=torch.bool)
+    structural[tokens // 2] = False                     # a query that sees nothing
+    key_valid = torch.rand(batch, tokens, generator=g) < 0.7
+    key_valid[1] = True
+    keep = (torch.rand(batch, heads, tokens, tokens, generator=g) >= dropout_p).to(torch.uint8)
+    lengths = torch.tensor([tokens, tokens // 3, tokens - 5], dtype=torch.int32) if with_lengths else None
+    dense = (structural[None] & key_valid[:, None, :])[:, None]
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    want = oracle.attention_dropout(qr, kr, vr, lengths, keep, dropout_p, attn_mask=dense)
+    want.backward(grad_out.double())
+    mask = build_structured_mask(structural.to(device), key_valid.to(device))
+    qd, kd, vd = (t.to(device).requires_grad_(True) for t in (q, k, v))
+    out = flash_attention(qd, kd, vd, structured_mask=mask, key_lengths=None if lengths is None else lengths.to(device),
+                          dropout_p=dropout_p, training=True, dropout_mask=keep.to(device))
+    out.backward(grad_out.to(device))
+    torch.testing.assert_close(out.detach().cpu().double(), want.detach(), **BF16_TOL)
+    assert out[:, :, tokens // 2].abs().max().item() == 0.0
+    for got, ref, name in zip((qd.grad, kd.grad, vd.grad), (qr.grad, kr.grad, vr.grad), ("dq", "dk", "dv")):
+        torch.testing.assert_close(got.cpu().double(), ref, msg=lambda m, n=name: f"{n}: {m}", **GRAD_TOL)
+    # a keep mask of ones at a vanishing rate is the plain masked attention
+    ones = torch.ones_like(keep).to(device)
+    same = flash_attention(qd.detach(), kd.detach(), vd.detach(), structured_mask=mask,
+                           key_lengths=None if lengths is None else lengths.to(device), dropout_p=1e-9, training=True,
+                           dropout_mask=ones)
+    plain = flash_attention(qd.detach(), kd.detach(), vd.detach(), structured_mask=mask,
+                            key_lengths=None if lengths is None else lengths.to(device))
+    torch.testing.assert_close(same.float(), plain.float(), rtol=2 ** -6, atol=2 ** -6)
+    with pytest.raises(RuntimeError, match="self-only"):
+        flash_attention(qd, kd, vd, structured_mask=build_structured_mask(structural.to(device), key_valid.to(device),
+                                                                          key_valid.to(device)),
+                        dropout_p=dropout_p, training=True, dropout_mask=keep.to(device))
+
+
+def test_reference_block_trains_with_its_default_dropout(device):
+    """``UnifiedInteractionBlock`` in training mode with dropout (the reference's default hyperparameters) under the role
+    mask: the layer-by-layer route runs on the HIP attention with a drawn keep mask; same seed, same result; every
+    parameter receives a finite gradient."""
+    from taac_2026_amd.api import UnifiedInteractionBlock
+
+    batch, d_model, heads = 3, 128, 4
+    roles = torch.tensor([0, 1] + [2] * 5 + [3] * 4 + [4] * 3 + [5] * 2 + [6] * 40 + [7] * 4)
+    tokens = roles.numel()
+    g = torch.Generator().manual_seed(2)
+    block = UnifiedInteractionBlock(d_model, heads, 2, 0.04).to(torch.bfloat16).to(device).train()
+    x = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16).to(device)
+    padding = (torch.rand(batch, tokens, generator=g) < 0.3).to(device)
+    padding[:, :2] = False
+    mask = MetadataAttentionMask(enabled=True)(padding, roles.to(device))
+    results = []
+    for _ in range(2):
+        torch.manual_seed(7)
+        block.zero_grad(set_to_none=True)
+        xd = x.clone().requires_grad_(True)
+        out, _ = block(xd, padding, mask)
+        out.float().square().mean().backward()
+        results.append((out.detach().clone(), xd.grad.clone()))
+        for name, parameter in block.named_parameters():
+            assert parameter.grad is not None and torch.isfinite(parameter.grad).all(), name
+    assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
+    assert torch.isfinite(results[0][0]).all() and torch.isfinite(results[0][1]).all()
