@@ -560,7 +560,7 @@ class _HipFlashAttentionFunction(torch.autograd.Function):
 
 def masked_attention_backward(q, k, v, out, grad_out, lse, key_lengths, mask: StructuredAttentionMask, dq, dk, dv, *,
                               zero_padded_queries: bool = False, dropout_mask: torch.Tensor | None = None,
-                              dropout_scale: float = 1.0) -> None:
+                              dropout_scale: float = 1.0, self_factor: torch.Tensor | None = None) -> None:
     """``taac_flash_attn_bits_bwd`` for (B, H, T, d) views under a structured mask (either layout: one structure for the
     batch, or one per sample with the valid tokens in front), writing into ``dq`` / ``dk`` / ``dv`` (any element strides
     with a unit last one). A self-only query returned its own value row: its row is taken out of the kernels
@@ -578,8 +578,9 @@ def masked_attention_backward(q, k, v, out, grad_out, lse, key_lengths, mask: St
         delta.data_ptr(), batch, heads, query_len, k.shape[2], head_dim,
         *strides, int(bool(zero_padded_queries)), _native.dtype_code(q.dtype), _native.current_stream(q.device))
     _native.check(status, "flash_attention backward")
-    if mask.query_self is not None:
-        dv.add_(grad_out * mask.query_self[:, None, :, None].to(grad_out.dtype))
+    if mask.query_self is not None:  # ``self_factor`` (B, H, T): keep / (1 - p) of the row's own key under dropout
+        factor = mask.query_self[:, None, :, None].to(grad_out.dtype) if self_factor is None else self_factor[..., None]
+        dv.add_(grad_out * factor)
 
 
 class _HipMaskedAttentionFunction(torch.autograd.Function):
@@ -601,26 +602,34 @@ class _HipMaskedAttentionFunction(torch.autograd.Function):
             raise ValueError("flash_attention: the structured mask does not match (batch, query_len, kv_len)")
         require_cuda_tensors("hip flash_attention", q, k, v, mask.struct_bits)
         scale = 1.0
+        self_bits, self_factor = mask.self_bits, None
         if dropout_mask is not None:
-            if mask.query_self is not None:
-                raise RuntimeError("hip flash_attention: dropout does not come with self-only query rows")
             if dropout_mask.dtype != torch.uint8 or tuple(dropout_mask.shape) != (batch, heads, query_len, k.shape[2]):
                 raise ValueError("flash_attention dropout_mask must be uint8 of shape (B, H, Tq, Tk)")
             require_cuda_tensors("hip flash_attention", dropout_mask)
             dropout_mask = dropout_mask.contiguous()
             scale = 1.0 / (1.0 - dropout_p)
+            if mask.query_self is not None:
+                # A self-only query has probability 1 on its own key, which dropout keeps or drops like any other: its
+                # output is keep[i, i] / (1 - p) * v[i]. The kernels run without the self rows (whatever they compute
+                # for them is replaced here, and the backward takes the rows out through their log-sum-exp).
+                self_bits = None
+                diagonal = torch.diagonal(dropout_mask, dim1=-2, dim2=-1).to(v.dtype) * scale        # (B, H, T)
+                self_factor = diagonal * mask.query_self[:, None, :].to(v.dtype)
         lse = torch.empty(batch, heads, query_len, dtype=torch.float32, device=q.device)
         status = library.taac_flash_attn_masked_train_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), _native.ptr(key_lengths), mask.struct_bits.data_ptr(),
-            int(mask.sample_stride), _native.ptr(mask.block_any), _native.ptr(mask.valid_bits), _native.ptr(mask.self_bits),
+            int(mask.sample_stride), _native.ptr(mask.block_any), _native.ptr(mask.valid_bits), _native.ptr(self_bits),
             _native.ptr(dropout_mask), ctypes.c_float(scale), out.data_ptr(),
             lse.data_ptr(), batch, heads, query_len, k.shape[2], head_dim, _native.Int64x4(*q.stride()),
             _native.Int64x4(*k.stride()), _native.Int64x4(*v.stride()), _native.Int64x4(*out.stride()),
             int(bool(zero_padded_queries)), _native.dtype_code(q.dtype), _native.current_stream(q.device))
         _native.check(status, "flash_attention")
+        if self_factor is not None:
+            out = torch.where(mask.query_self[:, None, :, None], v * self_factor[..., None], out)
         ctx.save_for_backward(q, k, v, out, lse, *(() if key_lengths is None else (key_lengths,)))
         ctx.mask, ctx.has_lengths, ctx.zero_padded_queries = mask, key_lengths is not None, bool(zero_padded_queries)
-        ctx.dropout_mask, ctx.dropout_scale = dropout_mask, scale
+        ctx.dropout_mask, ctx.dropout_scale, ctx.self_factor = dropout_mask, scale, self_factor
         return out
 
     @staticmethod
@@ -631,7 +640,7 @@ class _HipMaskedAttentionFunction(torch.autograd.Function):
         dq, dk, dv = _dense_like(q), _dense_like(k), _dense_like(v)
         masked_attention_backward(q, k, v, out, grad_out, lse, key_lengths, ctx.mask, dq, dk, dv,
                                   zero_padded_queries=ctx.zero_padded_queries, dropout_mask=ctx.dropout_mask,
-                                  dropout_scale=ctx.dropout_scale)
+                                  dropout_scale=ctx.dropout_scale, self_factor=ctx.self_factor)
         return dq, dk, dv, None, None, None, None, None
 
 

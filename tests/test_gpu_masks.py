@@ -450,10 +450,22 @@ def test_structured_mask_with_dropout_takes_a_gradient(device, tokens, dim, with
     plain = flash_attention(qd.detach(), kd.detach(), vd.detach(), structured_mask=mask,
                             key_lengths=None if lengths is None else lengths.to(device))
     torch.testing.assert_close(same.float(), plain.float(), rtol=2 ** -6, atol=2 ** -6)
-    with pytest.raises(RuntimeError, match="self-only"):
-        flash_attention(qd, kd, vd, structured_mask=build_structured_mask(structural.to(device), key_valid.to(device),
-                                                                          key_valid.to(device)),
-                        dropout_p=dropout_p, training=True, dropout_mask=keep.to(device))
+    # self-only queries: probability 1 on their own key, kept or dropped like any other
+    if lengths is None:
+        query_self = torch.rand(batch, tokens, generator=g) < 0.2
+        eye = torch.eye(tokens, dtype=torch.bool)
+        dense_self = torch.where(query_self[:, None, :, None], eye[None, None], dense)
+        qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+        want = oracle.attention_dropout(qr, kr, vr, None, keep, dropout_p, attn_mask=dense_self)
+        want.backward(grad_out.double())
+        with_self = build_structured_mask(structural.to(device), key_valid.to(device), query_self.to(device))
+        qd, kd, vd = (t.to(device).requires_grad_(True) for t in (q, k, v))
+        out = flash_attention(qd, kd, vd, structured_mask=with_self, dropout_p=dropout_p, training=True,
+                              dropout_mask=keep.to(device))
+        out.backward(grad_out.to(device))
+        torch.testing.assert_close(out.detach().cpu().double(), want.detach(), **BF16_TOL)
+        for got, ref, name in zip((qd.grad, kd.grad, vd.grad), (qr.grad, kr.grad, vr.grad), ("dq", "dk", "dv")):
+            torch.testing.assert_close(got.cpu().double(), ref, msg=lambda m, n=name: f"{n} (self rows): {m}", **GRAD_TOL)
 
 
 def test_reference_block_trains_with_its_default_dropout(device):
