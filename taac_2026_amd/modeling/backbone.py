@@ -445,23 +445,24 @@ class PCVRBackbone(nn.Module):
             raise ValueError("key_lengths must have shape (batch,)")
         head_dim = self.d_model // self.num_heads
         if self.rope_base is not None or self.d_model not in (128, 256) or head_dim not in (32, 64) or self.d_ff % 32 != 0 \
-                or any(p.dtype != torch.bfloat16 for p in self.parameters()):
-            raise RuntimeError(f"{name}: the training route covers bf16 parameters, d_model 128 / 256, head dims 32 / 64, "
-                               "d_ff a multiple of 32 and no rotary embedding")
+                or any(p.dtype not in (torch.bfloat16, torch.float32) for p in self.parameters()):
+            raise RuntimeError(f"{name}: the training route covers bf16 (or float32 master) parameters, d_model 128 / 256, "
+                               "head dims 32 / 64, d_ff a multiple of 32 and no rotary embedding")
         if key_lengths.dtype != torch.int32 or not key_lengths.is_contiguous():
             key_lengths = key_lengths.to(torch.int32).contiguous()
         stream = emb
         for block in self.blocks:
             qk = block.query_norm is not None
             stream, _ = InteractionBlockFunction.apply(
-                stream, key_lengths, None, None, False, self.num_heads, self.eps, self.eps, True, self.eps, block.attn_norm.weight,
-                block.qkv.weight, block.qkv.bias, block.out.weight, block.out.bias, block.ffn_norm.weight, block.up.weight,
-                block.up.bias, block.down.weight, block.down.bias, block.query_norm.weight if qk else None,
-                block.key_norm.weight if qk else None)
+                stream, key_lengths, None, None, False, self.num_heads, self.eps, self.eps, True, self.eps,
+                _bf16(block.attn_norm.weight), _bf16(block.qkv.weight), _bf16(block.qkv.bias), _bf16(block.out.weight),
+                _bf16(block.out.bias), _bf16(block.ffn_norm.weight), _bf16(block.up.weight), _bf16(block.up.bias),
+                _bf16(block.down.weight), _bf16(block.down.bias), _bf16(block.query_norm.weight) if qk else None,
+                _bf16(block.key_norm.weight) if qk else None)
         tokens = emb.shape[1]
         valid = (torch.arange(tokens, device=emb.device)[None, :] < key_lengths[:, None]).to(stream.dtype).unsqueeze(-1)
         pooled = (stream * valid).sum(dim=1) / valid.sum(dim=1).clamp_min(1.0)
-        logits = torch.nn.functional.linear(pooled, self.head.weight, self.head.bias).squeeze(-1)
+        logits = torch.nn.functional.linear(pooled, _bf16(self.head.weight), _bf16(self.head.bias)).squeeze(-1)
         probabilities = torch.sigmoid(logits.float())
         if return_hidden:
             return probabilities, stream * valid      # rows at or beyond key_lengths[b] are zeros, as in the forward-only route

@@ -375,7 +375,9 @@ def training_route_applies(block, tokens: torch.Tensor, attention_mask, key_leng
     if key_lengths is not None and (key_lengths.dtype != torch.int32 or not key_lengths.is_cuda
                                     or not key_lengths.is_contiguous()):
         return False
-    return all(p.dtype == torch.bfloat16 and p.is_cuda for p in block.parameters())
+    # float32 parameters (master weights of mixed-precision training) are cast to bf16 on the way in, as every route of the
+    # module does; autograd carries the gradient back through the cast
+    return all(p.dtype in (torch.bfloat16, torch.float32) and p.is_cuda for p in block.parameters())
 
 
 def run_training_block(block, tokens: torch.Tensor, key_lengths: torch.Tensor | None, return_attention_tokens: bool,
@@ -383,9 +385,13 @@ def run_training_block(block, tokens: torch.Tensor, key_lengths: torch.Tensor | 
     """The block through :class:`InteractionBlockFunction`."""
     attention, ffn = block.attention, block.ffn
     qk_norm = attention.query_norm is not None
+
+    def bf16(parameter):
+        return parameter if parameter is None or parameter.dtype == torch.bfloat16 else parameter.to(torch.bfloat16)
+
     return InteractionBlockFunction.apply(
-        tokens, key_lengths, mask, padding_mask, bool(return_attention_tokens), attention.num_heads, block.attn_norm.eps, block.ffn_norm.eps,
-        ffn.gate_first, attention.query_norm.eps if qk_norm else 1e-6, block.attn_norm.weight, attention.qkv.weight,
-        attention.qkv.bias, attention.out.weight, attention.out.bias, block.ffn_norm.weight, ffn.up.weight, ffn.up.bias,
-        ffn.down.weight, ffn.down.bias, attention.query_norm.weight if qk_norm else None,
-        attention.key_norm.weight if qk_norm else None)
+        tokens, key_lengths, mask, padding_mask, bool(return_attention_tokens), attention.num_heads, block.attn_norm.eps,
+        block.ffn_norm.eps, ffn.gate_first, attention.query_norm.eps if qk_norm else 1e-6, bf16(block.attn_norm.weight),
+        bf16(attention.qkv.weight), bf16(attention.qkv.bias), bf16(attention.out.weight), bf16(attention.out.bias),
+        bf16(block.ffn_norm.weight), bf16(ffn.up.weight), bf16(ffn.up.bias), bf16(ffn.down.weight), bf16(ffn.down.bias),
+        bf16(attention.query_norm.weight) if qk_norm else None, bf16(attention.key_norm.weight) if qk_norm else None)

@@ -582,3 +582,40 @@ def test_feed_forward_with_dropout_of_the_hidden_state(device, gate_first):
     b = swiglu_ffn_dropout(dev[0].detach(), dev[1], dev[2], dev[3], dev[4], dropout_p=p)
     c = swiglu_ffn_dropout(dev[0].detach(), dev[1], dev[2], dev[3], dev[4], dropout_p=p)
     assert torch.equal(a, b) and not torch.equal(a, c)
+
+
+def test_block_training_route_takes_float32_master_parameters(device, monkeypatch):
+    """Mixed-precision training keeps float32 parameters: the one-function route casts them to bf16 on the way in and the
+    gradients arrive in float32, equal to those of the layer-by-layer route of the same module."""
+    import taac_2026_amd.modeling.backbone as backbone_module
+
+    batch, tokens, d_model, heads = 3, 64, 128, 4
+    g = torch.Generator().manual_seed(13)
+    block = UnifiedInteractionBlock(d_model, heads, 2, qk_norm=True).to(device).train()      # float32 parameters
+    x = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16).to(device)
+    lengths = torch.tensor([64, 20, 1], dtype=torch.int32, device=device)
+    padding = torch.arange(tokens, device=device)[None, :] >= lengths[:, None]
+    grad_out = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16).to(device)
+    taken = []
+    real = backbone_module.run_training_block
+
+    def run(compact: bool):
+        if compact:
+            monkeypatch.setattr(backbone_module, "run_training_block", lambda *a, **k: (taken.append(1), real(*a, **k))[1])
+        else:
+            monkeypatch.setattr(backbone_module, "training_route_applies", lambda *a, **k: False)
+        xd = x.clone().requires_grad_(True)
+        block.zero_grad(set_to_none=True)
+        out, _ = block(xd, padding, None, key_lengths=lengths, return_attention_tokens=False)
+        out.backward(grad_out)
+        monkeypatch.undo()
+        return out.detach(), xd.grad, {n: p.grad.clone() for n, p in block.named_parameters()}
+
+    out_c, gx_c, grads_c = run(True)
+    assert taken == [1]
+    out_s, gx_s, grads_s = run(False)
+    _close(out_c, out_s.cpu(), 1e-2)
+    _close(gx_c, gx_s.cpu(), 3e-2)
+    for name, grad in grads_c.items():
+        assert grad.dtype == torch.float32, name
+        _close(grad, grads_s[name].cpu(), 3e-2)
