@@ -584,9 +584,10 @@ def masked_attention_backward(q, k, v, out, grad_out, lse, key_lengths, mask: St
 
 
 class _HipMaskedAttentionFunction(torch.autograd.Function):
-    """Training path under a :class:`StructuredAttentionMask`: the structured forward kernel also saves the log-sum-exp;
-    the backward kernels take the visible pairs as bytes. What torch autograd derives for SDPA under the reference models'
-    bool masks, which the reference's accelerated path rejects (flash_attention.py:183-209)."""
+    """Training path under a :class:`StructuredAttentionMask` (either layout), optionally with dropout under a keep mask:
+    the structured forward kernel also saves the log-sum-exp; the backward kernels read the mask in the same bit form.
+    What torch autograd derives for SDPA under the reference models' bool masks, which the reference's accelerated path
+    rejects (flash_attention.py:183-209)."""
 
     @staticmethod
     def forward(ctx, q, k, v, key_lengths, mask: StructuredAttentionMask, zero_padded_queries: bool,
