@@ -301,6 +301,38 @@ def _attention_bwd_figures(device, iters: int) -> dict:
     return figures
 
 
+def _compare_training_routes(backbone_module, block, x, grad, step, forward) -> dict:
+    """The layer-by-layer autograd route of the same module at the same (full) size: its time, and the largest difference
+    of the two routes' gradients (input and every parameter) relative to the largest gradient value - the run stops when
+    they disagree by more than the 16-bit gradient tolerance of the reference's GPU tests (3e-2,
+    tests/gpu/infrastructure/accelerators/test_tilelang_ops_cuda.py:98-141)."""
+    def gradients():
+        block.zero_grad(set_to_none=True)
+        x.grad = None
+        forward().backward(grad)
+        out = {"input": x.grad.float().clone()}
+        out.update({name: p.grad.float().clone() for name, p in block.named_parameters()})
+        block.zero_grad(set_to_none=True)
+        x.grad = None
+        return out
+
+    compact = gradients()
+    applies = backbone_module.training_route_applies
+    backbone_module.training_route_applies = lambda *a, **k: False
+    try:
+        layered = gradients()
+        ms = _event_ms(step, 3, 2)
+    finally:
+        backbone_module.training_route_applies = applies
+    worst = 0.0
+    for name, reference in layered.items():
+        scale = max(reference.abs().max().item(), 1e-12)
+        worst = max(worst, (compact[name] - reference).abs().max().item() / scale)
+    if not worst <= 3e-2:
+        raise SystemExit(f"accuracy gate of the block's training routes failed: gradients differ by {worst} of their range")
+    return {"layer_by_layer_ms": ms, "max_gradient_difference_between_routes": worst}
+
+
 def _training_block_figures(device, with_comparison: bool = True) -> dict:
     """One training step (forward + backward, every parameter and the input taking a gradient) of a
     ``UnifiedInteractionBlock`` at the headline shape: the one-function route over the valid rows, and the layer-by-layer
@@ -329,12 +361,8 @@ def _training_block_figures(device, with_comparison: bool = True) -> dict:
 
         entry = {"valid_rows_ms": _event_ms(step, 5, 3)}
         if with_comparison:
-            applies = backbone_module.training_route_applies
-            backbone_module.training_route_applies = lambda *a, **k: False
-            try:
-                entry["layer_by_layer_ms"] = _event_ms(step, 3, 2)
-            finally:
-                backbone_module.training_route_applies = applies
+            entry.update(_compare_training_routes(backbone_module, block, x, grad, step,
+                                                  lambda: block(x, padding, None, key_lengths=lengths, return_attention_tokens=False)[0]))
         figures[label] = entry
         del block, x
     # the reference block as its model trains it: query / key norms, the role mask, padding scattered inside the sequence
@@ -359,12 +387,8 @@ def _training_block_figures(device, with_comparison: bool = True) -> dict:
 
     entry = {"valid_token_fraction": 1.0 - float(scattered.float().mean().item()), "valid_rows_ms": _event_ms(masked_step, 5, 3)}
     if with_comparison:
-        applies = backbone_module.training_route_applies
-        backbone_module.training_route_applies = lambda *a, **k: False
-        try:
-            entry["layer_by_layer_ms"] = _event_ms(masked_step, 3, 2)
-        finally:
-            backbone_module.training_route_applies = applies
+        entry.update(_compare_training_routes(backbone_module, block, x, grad, masked_step,
+                                              lambda: block(x, scattered, mask, return_attention_tokens=False)[0]))
     figures["query_key_norm_role_mask_scattered_padding"] = entry
     del block, x, mask
     # the whole benchmark network (4 blocks + masked mean -> Linear -> sigmoid) under autograd: forward, loss, backward
