@@ -138,16 +138,16 @@ class InteractionBlockFunction(torch.autograd.Function):
         if not flat.is_contiguous():
             flat = flat.contiguous()
         library = _native.load_library()
-        # q | k | v of the valid rows, in the padded layout. Under key lengths the attention kernels never read a padded
-        # key or query row; under a mask they do (an invisible pair is a zero factor, not a skipped one), so the padded
-        # rows hold zeros there.
-        # Layout of the attention side: the positions (key lengths, or a mask with self-only queries), or the samples'
-        # valid tokens in front (any other mask), where the mask's structure is the one gathered per sample and the
-        # samples' numbers of valid tokens are the key lengths.
+        # Layout of the attention side (q | k | v, the attention output and their gradients): the positions (key lengths,
+        # or a mask with self-only queries), or the samples' valid tokens in front (any other mask), where the mask's
+        # structure is the one gathered per sample and the samples' numbers of valid tokens are the key lengths.
         front = getattr(index, "front", None) if mask is not None else None
         arows = rows if front is None else front
         if front is not None:
             mask, key_lengths = index.front_mask, index.lengths
+        # q | k | v of the valid rows. Under key lengths the attention kernels never read a row beyond a sample's length;
+        # under a mask over the positions they do (an invisible pair is a zero factor, not a skipped one), so the padded
+        # rows hold zeros there.
         in_positions = mask is not None and front is None
         qkv = (torch.zeros if in_positions else torch.empty)(total, 3 * width, dtype=flat.dtype, device=flat.device)
         _indexed_linear(flat, w_qkv, b_qkv, qkv, tokens=total, out_rows=arows, count=count,
@@ -177,9 +177,9 @@ class InteractionBlockFunction(torch.autograd.Function):
                 qkv.data_ptr(), qkv.data_ptr() + width * element, qkv.data_ptr() + 2 * width * element,
                 _native.ptr(key_lengths), mask.struct_bits.data_ptr(), int(mask.sample_stride), _native.ptr(mask.block_any),
                 _native.ptr(mask.valid_bits), _native.ptr(mask.self_bits), None, ctypes.c_float(1.0), attended.data_ptr(),
-                lse.data_ptr(), batch,
-                num_heads, token_count, token_count, width // num_heads, qkv_strides, qkv_strides, qkv_strides, out_strides,
-                0 if front is None else 1, _native.dtype_code(flat.dtype), _native.current_stream(tokens.device))
+                lse.data_ptr(), batch, num_heads, token_count, token_count, width // num_heads, qkv_strides, qkv_strides,
+                qkv_strides, out_strides, 0 if front is None else 1, _native.dtype_code(flat.dtype),
+                _native.current_stream(tokens.device))
         _native.check(status, "interaction block (training): attention")
         # Second half on the valid rows of copies of the stream (padded rows pass through): one kernel when the caller
         # does not want the tokens between the halves, two otherwise.
@@ -196,9 +196,9 @@ class InteractionBlockFunction(torch.autograd.Function):
             _linear.attention_out_ffn(attended, w_out, b_out, flat, w_up, b_up, w_down, b_down, norm_weight=ffn_norm_w,
                                       eps=ffn_eps, token_rows=(rows, count), input_rows=front, out=output)
         ctx.mask, ctx.front = mask, front
+        # (a mask over the positions has no key lengths: the slot keeps a tensor it never reads)
         ctx.save_for_backward(flat, qkv, attended, lse, key_lengths if key_lengths is not None else lse, attn_norm_w, w_qkv,
-                              w_out,
-                              ffn_norm_w, w_up, w_down,
+                              w_out, ffn_norm_w, w_up, w_down,
                               *(t for t in (b_out, b_up, attn_tokens, b_qkv if query_norm_w is not None else None,
                                             query_norm_w, key_norm_w) if t is not None))
         ctx.index = index
