@@ -557,12 +557,14 @@ int taac_flash_attn_bits_bwd(const void* q, const void* k, const void* v, const 
 /*
  * taac_rows_merge for padding that is not a prefix: token t of sample b is valid iff bit t of valid_bits[b] is set (rows
  * of ceil(T / 32) words, as for taac_valid_rows_from_bits, whose per-sample offsets are `offsets`); its compact row is
- * offsets[b] + the number of valid tokens of the sample in front of it.
+ * offsets[b] + the number of valid tokens of the sample in front of it. word_prefix (NULL: the kernel counts): int32
+ * [B, ceil(T / 32)], the number of valid tokens of the sample in the words before each word.
  * Replaces: the same `update * ~padding_mask` + residual arithmetic under the scattered padding of the reference's
  * token layout (experiments/symbiosis/backbone.py:58-68, experiments/symbiosis/attention.py:21-60).
  */
 int taac_rows_merge_bits(const void* padded, const void* compact_a, const void* compact_b, const uint32_t* valid_bits,
-                         const int32_t* offsets, void* out, int32_t B, int32_t T, int32_t W, void* stream);
+                         const int32_t* word_prefix, const int32_t* offsets, void* out, int32_t B, int32_t T, int32_t W,
+                         void* stream);
 
 /*
  * The same row index for padding that is not a prefix: token t of sample b is valid iff bit t of valid_bits[b] is set

@@ -136,7 +136,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "taac_rows_gather": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int32, c_void_p]),
     "taac_rows_merge": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p]),
-    "taac_rows_merge_bits": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p]),
+    "taac_rows_merge_bits": (c_int, [c_void_p] * 7 + [c_int32, c_int32, c_int32, c_void_p]),
     "taac_swiglu_ffn_bwd_packed_bytes": (c_int64, [c_int32, c_int32]),
     "taac_swiglu_ffn_bwd_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
     "taac_swiglu_ffn_bwd_hidden": (

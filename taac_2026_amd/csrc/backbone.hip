@@ -255,10 +255,12 @@ __global__ __launch_bounds__(kBlock) void rows_merge_kernel(const bf16x8* __rest
 }
 
 // The same merge for padding that is not a prefix: (b, t) is valid iff bit t of valid_bits[b] is set, and its compact row
-// is offsets[b] + the number of valid tokens of the sample in front of it.
+// is offsets[b] + the number of valid tokens of the sample in front of it (word_prefix[b][w], if given, = the number of
+// valid tokens in the words before word w, which saves the walk over those words).
 __global__ __launch_bounds__(kBlock) void rows_merge_bits_kernel(const bf16x8* __restrict__ padded,
                                                                  const bf16x8* __restrict__ a, const bf16x8* __restrict__ b2,
                                                                  const uint32_t* __restrict__ valid_bits,
+                                                                 const int32_t* __restrict__ word_prefix,
                                                                  const int32_t* __restrict__ offsets, bf16x8* __restrict__ out,
                                                                  int64_t pieces_total, int T, int pieces) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
@@ -271,7 +273,11 @@ __global__ __launch_bounds__(kBlock) void rows_merge_bits_kernel(const bf16x8* _
   bf16x8 v;
   if ((word >> (t % 32)) & 1u) {
     int rank = __popc(word & ((1u << (t % 32)) - 1u));
-    for (int w = 0; w < t / 32; ++w) rank += __popc(bits[w]);
+    if (word_prefix != nullptr) {
+      rank += word_prefix[static_cast<int64_t>(b) * ((T + 31) / 32) + t / 32];
+    } else {
+      for (int w = 0; w < t / 32; ++w) rank += __popc(bits[w]);
+    }
     const int64_t src = (static_cast<int64_t>(offsets[b]) + rank) * pieces + c;
     v = a[src];
     if (b2 != nullptr) {
@@ -337,8 +343,8 @@ extern "C" int taac_rows_merge(const void* padded, const void* compact_a, const 
 }
 
 extern "C" int taac_rows_merge_bits(const void* padded, const void* compact_a, const void* compact_b,
-                                    const uint32_t* valid_bits, const int32_t* offsets, void* out, int32_t B, int32_t T,
-                                    int32_t W, void* stream) {
+                                    const uint32_t* valid_bits, const int32_t* word_prefix, const int32_t* offsets,
+                                    void* out, int32_t B, int32_t T, int32_t W, void* stream) {
   using namespace taac;
   const char* name = "taac_rows_merge_bits";
   if (B < 0 || T < 0 || W <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: bad dimensions", name);
@@ -352,8 +358,8 @@ extern "C" int taac_rows_merge_bits(const void* padded, const void* compact_a, c
   if (blocks > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many workgroups", name);
   hipLaunchKernelGGL(rows_merge_bits_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, as_stream(stream),
                      static_cast<const bf16x8*>(padded), static_cast<const bf16x8*>(compact_a),
-                     static_cast<const bf16x8*>(compact_b), valid_bits, offsets, static_cast<bf16x8*>(out), pieces_total, T,
-                     W / 8);
+                     static_cast<const bf16x8*>(compact_b), valid_bits, word_prefix, offsets, static_cast<bf16x8*>(out),
+                     pieces_total, T, W / 8);
   return check_launch(name);
 }
 

@@ -62,6 +62,10 @@ class _RowIndex:
             index = cls.__new__(cls)
             index.rows, index.count = _linear.valid_rows(None, tokens, padding_mask=padding_mask)
             index.bits = _pack_bits((~padding_mask).contiguous())
+            # valid tokens in the 32-token words before each word: the rank of a position without a walk over the words
+            words = index.bits.shape[1]
+            per_word = torch.nn.functional.pad(~padding_mask, (0, words * 32 - tokens)).view(-1, words, 32).sum(-1)
+            index.word_prefix = (per_word.cumsum(1) - per_word).to(torch.int32).contiguous()
             index.valid = None
             index.identity = None
             # Without self-only queries the attention side runs in the layout that has every sample's valid tokens at the
@@ -332,7 +336,8 @@ class InteractionBlockFunction(torch.autograd.Function):
                                              batch, token_count, width, _native.current_stream(device))
         else:
             status = library.taac_rows_merge_bits(grad_padded.data_ptr(), grad_x1c.data_ptr(), grad_xc_norm.data_ptr(),
-                                                  ctx.index.bits.data_ptr(), rows.data_ptr() + 4 * total,
+                                                  ctx.index.bits.data_ptr(), ctx.index.word_prefix.data_ptr(),
+                                                  rows.data_ptr() + 4 * total,
                                                   grad_tokens.data_ptr(), batch, token_count, width,
                                                   _native.current_stream(device))
         _native.check(status, "interaction block (training): gradient merge")

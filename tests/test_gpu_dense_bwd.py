@@ -325,6 +325,32 @@ def test_rows_gather_and_merge_through_the_c_abi(device):
         assert torch.equal(out, expected)
     assert library.taac_rows_gather(source.data_ptr(), source.stride(0), rows.data_ptr(), valid, compact.data_ptr(), 12,
                                     stream) == _native.TAAC_ERR_UNSUPPORTED
+    # padding that is not a prefix: validity bits, with and without the table of valid tokens in front of each word
+    from taac_2026_amd.accelerators.attention import _pack_bits
+
+    padding = torch.rand(batch, tokens, generator=g) < 0.4
+    padding[1] = True
+    padding[0] = False
+    padding = padding.to(device)
+    rows, count = valid_rows(None, tokens, padding_mask=padding)
+    valid = int(count.item())
+    index = rows[:valid].long()
+    assert torch.equal(index, (~padding).flatten().nonzero().flatten())
+    bits = _pack_bits((~padding).contiguous())
+    words = bits.shape[1]
+    per_word = torch.nn.functional.pad(~padding, (0, words * 32 - tokens)).view(batch, words, 32).sum(-1)
+    prefix = (per_word.cumsum(1) - per_word).to(torch.int32).contiguous()
+    a = torch.randn(valid, width, generator=g).to(torch.bfloat16).to(device)
+    b = torch.randn(valid, width, generator=g).to(torch.bfloat16).to(device)
+    for second in (None, b):
+        for table in (None, prefix):
+            out = torch.empty_like(base)
+            _native.check(library.taac_rows_merge_bits(base.data_ptr(), a.data_ptr(), _native.ptr(second), bits.data_ptr(),
+                                                       _native.ptr(table), rows.data_ptr() + 4 * batch * tokens,
+                                                       out.data_ptr(), batch, tokens, width, stream), "merge_bits")
+            expected = base.clone()
+            expected[index] = a if second is None else (a.float() + b.float()).to(torch.bfloat16)
+            assert torch.equal(out, expected)
 
 
 def test_two_blocks_and_the_readout_train_end_to_end(device):
