@@ -238,6 +238,46 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
     assert backward(tk=0) == unsupported
     assert backward(tq=64, tk=128, zero=1) == invalid
 
+    # training under structured masks: the structured forward with the log-sum-exp, the bit-form and byte-form backward
+    def masked_train(**kw):
+        a = dict(bits=fake, stride=0, block_any=fake, self=None, keep=None, scale=1.0, lse=fake, tq=64, tk=64)
+        a.update(kw)
+        return library.taac_flash_attn_masked_train_fwd(fake, fake, fake, None, a["bits"], a["stride"], a["block_any"], None,
+                                                        a["self"], a["keep"], a["scale"], fake, a["lse"], 1, 8, a["tq"],
+                                                        a["tk"], 16, strides, strides, strides, strides, 0, bf16, None)
+
+    assert masked_train(bits=None) == invalid and b"struct_bits" in library.taac_last_error()
+    assert masked_train(lse=None) == invalid and b"lse" in library.taac_last_error()
+    assert masked_train(block_any=None) == invalid and b"block_any" in library.taac_last_error()
+    assert masked_train(keep=fake, scale=0.5) == invalid and b"dropout_scale" in library.taac_last_error()
+    assert masked_train(keep=fake, scale=1.25, self=fake) == unsupported and b"self-only" in library.taac_last_error()
+
+    def bits_backward(**kw):
+        a = dict(bits=fake, stride=0, keep=None, scale=1.0, d=16, lse=fake)
+        a.update(kw)
+        return library.taac_flash_attn_bits_bwd(fake, fake, fake, fake, fake, a["lse"], None, a["bits"], a["stride"], None,
+                                                a["keep"], a["scale"], fake, fake, fake, fake, 1, 8, 64, 64, a["d"], strides,
+                                                strides, strides, strides, strides, strides, strides, strides, 0, bf16, None)
+
+    assert bits_backward(bits=None) == invalid and b"struct_bits" in library.taac_last_error()
+    assert bits_backward(stride=-4) == invalid and b"stride" in library.taac_last_error()
+    assert bits_backward(d=72) == unsupported and b"head_dim" in library.taac_last_error()
+    assert bits_backward(keep=fake, scale=0.5) == invalid and b"dropout_scale" in library.taac_last_error()
+    assert bits_backward(lse=None) == invalid
+    status = library.taac_flash_attn_mask_bwd(fake, fake, fake, fake, fake, fake, None, None, 0, 0, None, fake, fake, fake, fake,
+                                              1, 8, 64, 64, 16, strides, strides, strides, strides, strides, strides, strides,
+                                              strides, 0, bf16, None)
+    assert status == invalid and b"visibility" in library.taac_last_error()
+    status = library.taac_flash_attn_mask_bwd(fake, fake, fake, fake, fake, fake, None, fake, -1, 0, None, fake, fake, fake, fake,
+                                              1, 8, 64, 64, 16, strides, strides, strides, strides, strides, strides, strides,
+                                              strides, 0, bf16, None)
+    assert status == invalid and b"stride" in library.taac_last_error()
+    # the gradient merge for scattered padding
+    assert library.taac_rows_merge_bits(fake, fake, None, fake, None, fake, fake, 2, 8, 12, None) == unsupported
+    assert library.taac_rows_merge_bits(fake, fake, None, None, None, fake, fake, 2, 8, 16, None) == invalid
+    assert library.taac_rows_merge_bits(fake, fake, None, fake, None, fake, fake, 0, 8, 16, None) == ok
+    assert library.taac_rows_merge_bits(fake, fake, None, fake, None, fake, fake, -1, 8, 16, None) == invalid
+
 
 def test_status_mapping_to_python_exceptions():
     library = _native.load_library()
