@@ -306,7 +306,7 @@ def _check_training(device, q, k, v, mask, grad_out, key_lengths=None, dense=Non
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("tokens,dim", [(50, 32), (130, 64), (300, 32), (257, 16), (96, 48)])
+@pytest.mark.parametrize("tokens,dim", [(50, 32), (130, 64), (300, 32), (257, 16), (96, 48), (1100, 32)])
 def test_structured_masks_take_a_gradient(device, dtype, tokens, dim):
     """Random structure, invalid keys, self-only queries and a query that sees nothing: the gradients equal float64
     autograd under the dense mask; invisible keys and the empty query row receive exactly zero."""
