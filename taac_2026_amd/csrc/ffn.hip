@@ -1000,7 +1000,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
 #pragma unroll
               for (int e = 0; e < 8; ++e) v[e] = static_cast<bf16_t>(f[e]);
             }
-            *reinterpret_cast<bf16x8*>(p.out + static_cast<int64_t>(info[j].x) * p.ldo + col8) = v;
+            __builtin_nontemporal_store(v, reinterpret_cast<bf16x8*>(p.out + static_cast<int64_t>(info[j].x) * p.ldo + col8));
           }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
