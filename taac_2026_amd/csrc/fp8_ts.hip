@@ -373,7 +373,7 @@ __global__ __launch_bounds__(kWaves * kWave, 2) void linear_fp8_ts_kernel(const 
           o[e] = static_cast<bf16_t>(x0);
           o[4 + e] = static_cast<bf16_t>(x1);
         }
-        *reinterpret_cast<bf16x8*>(p.out + tok * p.ldo + chunk * OUTC + (lane % PIECES) * 8) = o;
+        __builtin_nontemporal_store(o, reinterpret_cast<bf16x8*>(p.out + tok * p.ldo + chunk * OUTC + (lane % PIECES) * 8));
         if constexpr (STATS) {
           const bf16x8 wv = *reinterpret_cast<const bf16x8*>(outw_lds + chunk * OUTC + (lane % PIECES) * 8);
 #pragma unroll
