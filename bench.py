@@ -52,49 +52,72 @@ def _event_ms(fn, iters: int, warmup: int) -> float:
     return times[len(times) // 2]
 
 
-def _event_ms_after(prelude, fn, iters: int, warmup: int, reset=None) -> float:
-    """Duration of ``fn`` in ms per call when every call follows ``prelude`` on the same stream, as it does inside the
-    step (its inputs were just written by the kernel before it). HIP events on the launch stream around runs of
-    back-to-back launches: the time of ``n x [prelude, fn]`` minus the time of ``n x [prelude]``, per call, median over
-    interleaved groups. (A pair of events around every single ``fn`` launch also counts the gap between the event and the
-    kernel on either side, which read 5 - 7 % above the kernel trace's duration of the same launches.) ``reset`` runs
-    in front of every run, outside the events (for an ``fn`` that updates its input in place)."""
-    for _ in range(warmup):
-        prelude()
-        fn()
-    groups = max(1, min(5, iters // 2))
-    per_group = max(2, iters // groups)
+class _CallRecorder:
+    """Stands in for the loaded library while one operator call runs and notes every compute entry point it calls with
+    the exact ctypes arguments (device pointers, sizes, stream)."""
 
-    def run(with_fn: bool) -> float:
-        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        if reset is not None:
-            reset()
-        start.record()
-        for _ in range(per_group):
-            prelude()
-            if with_fn:
-                fn()
-        stop.record()
-        stop.synchronize()
-        return start.elapsed_time(stop) / per_group
+    def __init__(self, library):
+        self._library = library
+        self.calls: list[tuple[object, tuple]] = []
 
-    times = sorted(run(True) - run(False) for _ in range(groups))
-    return times[len(times) // 2]
+    def __getattr__(self, name):
+        function = getattr(self._library, name)
+        if not name.startswith("taac_") or name in ("taac_last_error", "taac_abi_version") or name.endswith("_bytes"):
+            return function
+
+        def recorded(*args):
+            self.calls.append((function, args))
+            return function(*args)
+
+        return recorded
+
+
+def _native_replay(fn):
+    """Runs ``fn`` (a call of one of the package's operators) once and returns a callable that repeats exactly the
+    C-ABI calls it made, with the same arguments, and nothing else. The Python operator wrappers validate, reshape and
+    allocate for 0.1 - 0.3 ms per call, which is as long as the kernels they launch: timed through them the GPU waits
+    for the host and the events measure the host. The replay costs a few microseconds per launch, so back-to-back
+    launches keep the GPU busy and the event time per launch is the kernel's duration, as a kernel trace shows it. The
+    tensors the recorded pointers refer to are kept alive by the returned callable (``fn``'s result) and by the caller
+    (its inputs and ``out=`` buffers)."""
+    from taac_2026_amd import _native
+
+    library = _native.load_library()
+    recorder = _CallRecorder(library)
+    _native._library = recorder
+    try:
+        result = fn()
+    finally:
+        _native._library = library
+    calls = recorder.calls
+    if not calls:
+        raise SystemExit("bench.py: the operator made no library call to replay")
+
+    def replay(_keep=result):
+        for function, args in calls:
+            if function(*args) != 0:
+                raise SystemExit("bench.py: a replayed library call failed: " + library.taac_last_error().decode())
+
+    return replay
 
 
 TRAFFIC_SUMMARY = "profiles/pmc_traffic_backbone_c4.txt"
 
 
-def _measured_traffic(kernel_name: str) -> int:
+def _measured_traffic(kernel_name: str) -> tuple[int, str]:
     """HBM bytes per launch of ``kernel_name`` as measured with the FETCH_SIZE / WRITE_SIZE counters (scaled by a kernel
-    of known traffic). The counters cannot be read from inside this process: the figure is taken from the committed
-    counter summary (the line says so) and the run fails when the kernel is not listed there, so that a renamed or new
-    dominant kernel cannot silently carry another kernel's traffic."""
+    of known traffic), and the provenance line of that measurement (the commit of the kernel sources the counters were
+    collected on, so that a figure taken before a kernel changed is visible as such). The counters cannot be read from
+    inside this process: the figure is taken from the committed counter summary (the line says so) and the run fails
+    when the kernel is not listed there, so that a renamed or new dominant kernel cannot silently carry another
+    kernel's traffic."""
     summary = REPO_ROOT / TRAFFIC_SUMMARY
     if summary.exists():
-        for line in summary.read_text().splitlines():
+        lines = summary.read_text().splitlines()
+        collected = next((line[2:].strip() for line in lines if line.startswith("# collected on")), "collected on: not recorded")
+        for line in lines:
             if line.startswith(kernel_name + ":") and "traffic_bytes=" in line:
-                return int(line.split("traffic_bytes=")[1].split()[0])
+                return int(line.split("traffic_bytes=")[1].split()[0]), collected
     raise SystemExit(f"bench.py: no measured traffic for kernel '{kernel_name}' in {TRAFFIC_SUMMARY}; collect the "
                      "FETCH_SIZE / WRITE_SIZE counters for it (commands in that file) before reporting a roofline")
 
@@ -128,10 +151,12 @@ def _sustained(step, batch: int, *, heat_s: float = 2.0, repeats: int = 5, repea
 
 
 def _accuracy_gate(model, inputs, device) -> dict:
-    """Probabilities of a slice of the batch against the CPU oracle (2e-2 absolute)."""
+    """Probabilities of 64 samples spread over the batch against the CPU oracle (2e-2 absolute; about a second of host
+    time), and every probability of the batch finite."""
     from oracle import reference as oracle
 
-    pick = torch.tensor([0, 341, 682, 1023]) % inputs.emb.shape[0]
+    batch = inputs.emb.shape[0]
+    pick = torch.unique(torch.linspace(0, batch - 1, 64).round().long())
     with torch.no_grad():
         p = model(inputs.emb.to(device), inputs.key_lengths.to(device)).cpu()
     expected = oracle.backbone(inputs.emb[pick], inputs.key_lengths[pick], inputs.blocks, inputs.head_weight,
@@ -143,8 +168,9 @@ def _accuracy_gate(model, inputs, device) -> dict:
 
 
 def _kernel_breakdown(inputs, device, iters: int) -> dict:
-    """Stand-alone timing of each kernel of one block at the step's shapes (HIP events on the launch stream). The dense
-    layers walk the valid tokens only, as they do inside the step; their algorithmic work counts those tokens."""
+    """Stand-alone timing of each kernel of one block at the step's shapes (HIP events on the launch stream around
+    back-to-back replays of the library calls). The dense layers walk the valid tokens only, as they do inside the step;
+    their algorithmic work counts those tokens."""
     from taac_2026_amd.api import attention_out_ffn, norm_linear, scaled_dot_product_attention, swiglu_ffn, valid_rows
 
     B, T, D = inputs.emb.shape
@@ -187,20 +213,49 @@ def _kernel_breakdown(inputs, device, iters: int) -> dict:
                                    norm_weight=w["ffn_norm.weight"], token_rows=index, out=buf),
                 2.0 * Mv * 3 * D * F, 2.0 * (2 * Mv * D + 3 * D * F)),
         }
-        # Inside the step every kernel reads what the kernel before it just wrote. The block's last kernel is timed that
-        # way too (attention launched in front of every timed launch, outside the events): "ms" is the stand-alone figure
-        # on inputs that are cold in the caches, "ms_in_sequence" the one that matches the kernel trace of the step.
-        # The step's launch also updates the residual stream in place (out = the block input), which the timed launch
-        # here does on a working copy that is restored in front of every run of eight launches.
+        # Inside the step every kernel reads what the kernel before it just wrote and the block's last kernel updates the
+        # residual stream in place. "ms" of the three kernels of the step is measured that way, as the kernel trace of the
+        # step shows them: the block's three launches [RMSNorm+QKV on the stream, attention, out-projection+FFN in place on
+        # the stream] are replayed back to back between HIP events, once complete and once without the kernel in question
+        # (its outputs of the run before are still in place), and the difference per block is that kernel's time. The
+        # stream is a working copy that is restored in front of every run of eight blocks. "ms_standalone" is the same
+        # launch repeated on its own (inputs cold in the caches, no neighbours).
         x_work = x.clone()
-        in_place = lambda: attention_out_ffn(a, w["out.weight"], w["out.bias"], x_work, w["up.weight"], w["up.bias"],  # noqa: E731
-                                             w["down.weight"], w["down.bias"], norm_weight=w["ffn_norm.weight"],
-                                             token_rows=index, out=x_work)
-        in_sequence = {"out_residual_rmsnorm_swiglu_ffn_residual": (attn, in_place, lambda: x_work.copy_(x))}
+        sequence = {
+            "rmsnorm_qkv": _native_replay(lambda: norm_linear(x_work, w["qkv.weight"], w["qkv.bias"],
+                                                              norm_weight=w["attn_norm.weight"], token_rows=index, out=qkv)),
+            "attention": _native_replay(attn),
+            "out_residual_rmsnorm_swiglu_ffn_residual": _native_replay(
+                lambda: attention_out_ffn(a, w["out.weight"], w["out.bias"], x_work, w["up.weight"], w["up.bias"],
+                                          w["down.weight"], w["down.bias"], norm_weight=w["ffn_norm.weight"],
+                                          token_rows=index, out=x_work)),
+        }
+
+        def run_blocks(skip: str | None, blocks: int = 8) -> float:
+            x_work.copy_(x)
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(blocks):
+                for kernel_name, launch in sequence.items():
+                    if kernel_name != skip:
+                        launch()
+            stop.record()
+            stop.synchronize()
+            return start.elapsed_time(stop) / blocks
+
+        for _ in range(3):
+            run_blocks(None)
+        in_sequence = {}
+        for name in sequence:
+            diffs = sorted(run_blocks(None) - run_blocks(name) for _ in range(max(5, iters)))
+            in_sequence[name] = diffs[len(diffs) // 2]
         for name, (fn, flops, nbytes) in cases.items():
-            ms = _event_ms(fn, iters, 3)
+            standalone = _event_ms(sequence["attention"] if fn is attn else _native_replay(fn), 5 * iters, 5)
+            ms = in_sequence.get(name, standalone)
             out[name] = {
                 "ms": ms,
+                "ms_standalone": standalone,
+                "timed": "in the block's launch sequence" if name in in_sequence else "stand-alone",
                 "tokens": int(Mv) if name != "attention" else int(M),
                 "algorithmic_flops": flops,
                 "algorithmic_bytes": nbytes,
@@ -209,21 +264,72 @@ def _kernel_breakdown(inputs, device, iters: int) -> dict:
                 "frac_mfma": flops / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS,
                 "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS,
             }
-            if name in in_sequence:
-                prelude, step_fn, restore = in_sequence[name]
-                out[name]["ms_in_sequence"] = _event_ms_after(prelude, step_fn, 4 * iters, 2, reset=restore)
+        out["block_launch_sequence_ms"] = {"ms": sorted(run_blocks(None) for _ in range(5))[2],
+                                           "note": "the three launches of one block, replayed back to back"}
     return out
 
 
-def _operator_figures(device, iters: int) -> dict:
-    """Stand-alone operators at configurations 2 and 3: norm HBM GB/s and masked-attention TFLOP/s. Each figure: 20 warm-up
-    launches, then 5 groups of ``iters`` launches between HIP events, the median group."""
+def _host_cores() -> int:
+    """Host threads for the CPU baselines: the machine's cores, capped by OMP_NUM_THREADS when the environment sets it
+    (a box that shares its host between several GPUs exports its share there)."""
+    cores = os.cpu_count() or 1
+    try:
+        cores = min(cores, max(1, int(os.environ["OMP_NUM_THREADS"])))
+    except (KeyError, ValueError):
+        pass
+    return cores
+
+
+def _cpu_ms(fn, *, warmup: int = 3, iters: int = 10, budget_s: float = 8.0) -> tuple[float, int]:
+    """Mean host time of ``fn`` in ms: ``warmup`` untimed calls, then up to ``iters`` timed ones (the protocol of the
+    reference's operator benchmark, pcvr_tilelang_ops_benchmark.py:217-250), cut short once ``budget_s`` seconds of timed
+    calls have passed. Returns (ms per call, timed calls)."""
+    for _ in range(warmup):
+        fn()
+    done, t0 = 0, time.perf_counter()
+    while done < iters:
+        fn()
+        done += 1
+        if time.perf_counter() - t0 > budget_s:
+            break
+    return (time.perf_counter() - t0) * 1e3 / done, done
+
+
+def _operator_figures(device, iters: int, cpu_baselines: bool = True) -> dict:
+    """Stand-alone operators at configurations 1, 2 and 3: norm HBM GB/s and masked-attention TFLOP/s. Each GPU figure: 20
+    warm-up launches, then 5 groups of ``iters`` launches between HIP events, the median group, on replays of the
+    operators' library calls. Beside each, the reference's torch formulas (the oracle) on the host cores at the same
+    shape, 3 warm-up and up to 10 timed calls (configuration 3 on the first 256 samples, scaled to the batch; flagged)."""
     from oracle import reference as oracle
     from taac_2026_amd import workloads
     from taac_2026_amd.api import flash_attention, layer_norm, rms_norm
 
     figures: dict[str, dict] = {}
+    cores = _host_cores()
+    if cpu_baselines:
+        torch.set_num_threads(cores)
+
+    def cpu_entry(fn, scale: float = 1.0, note: str | None = None) -> dict:
+        ms, calls = _cpu_ms(fn)
+        entry = {"ms": ms * scale, "cores": cores, "timed_calls": calls, "kind": "port"}
+        if note:
+            entry["note"] = note
+        return entry
+
     with torch.no_grad():
+        # configuration 1: fp32, 65 536 rows x 128 (64 MiB in all: a launch-bound correctness case, reported for completeness)
+        x1, w1, eps1 = workloads.rmsnorm_fp32_inputs()
+        x1d, w1d = x1.to(device), w1.to(device)
+        got = rms_norm(x1d, w1d, eps1).cpu()
+        torch.testing.assert_close(got, oracle.rms_norm(x1, w1, eps1), rtol=1e-5, atol=1e-5)
+        nbytes1 = 2.0 * x1.numel() * 4 + 4 * 128
+        ms = _event_ms(_native_replay(lambda: rms_norm(x1d, w1d, eps1)), 5 * iters, 20)
+        figures["rmsnorm_fp32_65536x128"] = {"ms": ms, "gbs": nbytes1 / ms / 1e6, "frac_hbm": nbytes1 / ms / 1e6 / HBM_PEAK_GBS,
+                                             "algorithmic_bytes": nbytes1, "atol": 1e-5}
+        if cpu_baselines:
+            figures["rmsnorm_fp32_65536x128"]["cpu_baseline"] = cpu_entry(lambda: oracle.rms_norm(x1, w1, eps1))
+        del x1d
+
         x, gamma, beta = workloads.norm_bf16_inputs()
         xd, gd, bd = x.to(device), gamma.to(device), beta.to(device)
         got = rms_norm(xd[:16], gd).cpu().float()
@@ -231,11 +337,14 @@ def _operator_figures(device, iters: int) -> dict:
         got = layer_norm(xd[:16], gd, bd).cpu().float()
         torch.testing.assert_close(got, oracle.layer_norm_fp32(x[:16], gamma, beta).float(), rtol=2e-2, atol=2e-2)
         nbytes = 2.0 * x.numel() * 2 + 2 * 256
-        ms = _event_ms(lambda: rms_norm(xd, gd), 5 * iters, 20)
+        ms = _event_ms(_native_replay(lambda: rms_norm(xd, gd)), 5 * iters, 20)
         figures["rmsnorm_bf16_1048576x256"] = {"ms": ms, "gbs": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS}
-        ms = _event_ms(lambda: layer_norm(xd, gd, bd), 5 * iters, 20)
+        ms = _event_ms(_native_replay(lambda: layer_norm(xd, gd, bd)), 5 * iters, 20)
         figures["layernorm_bf16_1048576x256"] = {"ms": ms, "gbs": (nbytes + 512) / ms / 1e6,
                                                  "frac_hbm": (nbytes + 512) / ms / 1e6 / HBM_PEAK_GBS}
+        if cpu_baselines:
+            figures["rmsnorm_bf16_1048576x256"]["cpu_baseline"] = cpu_entry(lambda: oracle.rms_norm(x, gamma))
+            figures["layernorm_bf16_1048576x256"]["cpu_baseline"] = cpu_entry(lambda: oracle.layer_norm(x, gamma, beta, 1e-5))
         # backward of both norms at the same shape: x and dy read once, dx written once (dw / db are 512 bytes each)
         from taac_2026_amd.accelerators.normalization import hip_layer_norm_backward_kernel, hip_rms_norm_backward_kernel
 
@@ -258,7 +367,7 @@ def _operator_figures(device, iters: int) -> dict:
         sum_sq = float((lengths.double() ** 2).sum().item())
         useful = 4.0 * H * d * sum_sq
         nbytes = 3.0 * H * d * 2 * float(lengths.sum().item()) + B * H * T * d * 2
-        ms = _event_ms(lambda: flash_attention(qd, kd, vd, key_lengths=ld, zero_padded_queries=True), 5 * iters, 20)
+        ms = _event_ms(_native_replay(lambda: flash_attention(qd, kd, vd, key_lengths=ld, zero_padded_queries=True)), 5 * iters, 20)
         figures["attention_bf16_B2048_H4_T256_d64"] = {
             "ms": ms,
             "useful_tflops": useful / ms / 1e9,
@@ -266,6 +375,11 @@ def _operator_figures(device, iters: int) -> dict:
             "frac_mfma": useful / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS,
             "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS,
         }
+        if cpu_baselines:
+            part = 256
+            figures["attention_bf16_B2048_H4_T256_d64"]["cpu_baseline"] = cpu_entry(
+                lambda: oracle.attention(q[:part], k[:part], v[:part], lengths[:part], zero_padded_queries=True),
+                scale=B / part, note=f"timed on the first {part} of {B} samples and scaled to the batch")
     del qd, kd, vd
     figures.update(_attention_bwd_figures(device, iters))
     figures.update(_training_block_figures(device))
@@ -730,7 +844,7 @@ def _cpu_baseline(inputs, budget_s: float = 20.0) -> dict:
     """The oracle's backbone forward (the reference's torch formulas) on the host cores, on a bounded sample."""
     from oracle import reference as oracle
 
-    cores = os.cpu_count() or 1
+    cores = _host_cores()
     torch.set_num_threads(cores)
     results = {}
     for label, cast in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
@@ -871,14 +985,16 @@ def main() -> None:
     valid_fraction = float(inputs.key_lengths.clamp(0, T).sum().item()) / (B * T)
 
     kernels = _kernel_breakdown(inputs, device, iters=10)
-    dominant = max((name for name in kernels if not name.startswith("split:")), key=lambda name: kernels[name]["ms"])
+    dominant = max((name for name in kernels if not name.startswith("split:") and "tflops" in kernels[name]),
+                   key=lambda name: kernels[name]["ms"])
     dom = kernels[dominant]
-    # Roofline position from the launch duration in sequence (behind the kernel that precedes it in the step), which is
-    # what the kernel trace of the step shows; the stand-alone duration on cache-cold inputs is reported next to it.
-    launch_ms = dom.get("ms_in_sequence", dom["ms"])
+    # Roofline position from the launch duration inside the block's launch sequence, which is what the kernel trace of the
+    # step shows; the stand-alone duration on cache-cold inputs is reported next to it.
+    launch_ms = dom["ms"]
     tflops = dom["algorithmic_flops"] / launch_ms / 1e9
     gbs = dom["algorithmic_bytes"] / launch_ms / 1e6
     bound = "mfma" if tflops / MFMA_BF16_PEAK_TFLOPS >= gbs / HBM_PEAK_GBS else "hbm"
+    traffic_bytes, traffic_origin = _measured_traffic(dominant)
     roofline = {
         "kernel": dominant,
         "bound": bound,
@@ -886,10 +1002,11 @@ def main() -> None:
         "peak": MFMA_BF16_PEAK_TFLOPS if bound == "mfma" else HBM_PEAK_GBS,
         "unit": "TFLOP/s" if bound == "mfma" else "GB/s",
         "frac": tflops / MFMA_BF16_PEAK_TFLOPS if bound == "mfma" else gbs / HBM_PEAK_GBS,
-        "traffic": _measured_traffic(dominant),
-        "traffic_source": f"{TRAFFIC_SUMMARY} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE; not measured in this run)",
+        "traffic": traffic_bytes,
+        "traffic_source": f"{TRAFFIC_SUMMARY} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE; not measured in this run; "
+                          f"{traffic_origin})",
         "launch_ms": launch_ms,
-        "launch_ms_standalone": dom["ms"],
+        "launch_ms_standalone": dom["ms_standalone"],
     }
 
     line = {
@@ -921,7 +1038,7 @@ def main() -> None:
         "kernels": kernels,
     }
     if not args.skip_operators:
-        line["operators"] = _operator_figures(device, iters=20)
+        line["operators"] = _operator_figures(device, iters=20, cpu_baselines=not args.skip_cpu_baseline)
         line["fp8_dense_layers"] = _fp8_figures(inputs, device, iters=10)
         line["embedding_bag_mean"] = _embedding_figures(device, iters=20)
         line["candidate_readout"] = _readout_figures(inputs, device, iters=20)

@@ -12,9 +12,8 @@
  *   - `dtype` is a taac_dtype value.
  *   - No global mutable state besides the thread-local error string (and the scratch array of
  *     taac_rmsnorm_bwd_static): calls from different host threads and on different streams are independent.
- *     Behaviour is chosen by arguments only. Two environment variables exist as TEST HOOKS and change no result:
- *     TAAC_TS_MAX_WORKGROUPS caps the grid of the persistent dense kernels (so that small test inputs walk several
- *     tiles per workgroup), TAAC_FP8_TILED routes taac_linear_fp8 to its generic tiled kernel.
+ *     Behaviour is chosen by arguments only; no environment variable is read. taac_test_hooks (last declaration) sets
+ *     two process-wide test switches that change no result.
  *
  * Each declaration cites the reference interface it replaces (path:line under the reference tree,
  * Puiching-Memory/TAAC_2026). The reference has no C ABI on this path: its operators are Python
@@ -30,7 +29,7 @@
 extern "C" {
 #endif
 
-#define TAAC_ABI_VERSION 6
+#define TAAC_ABI_VERSION 7
 
 enum taac_status {
   TAAC_OK = 0,
@@ -61,6 +60,13 @@ enum taac_epilogue {
 
 int taac_abi_version(void);
 const char* taac_last_error(void);
+
+/* TEST-ONLY, not part of the drop-in surface (no counterpart in the reference): process-wide switches for the test
+ * suite that change scheduling and never a result. max_workgroups > 0 caps the grid of the persistent dense kernels
+ * (taac_norm_linear*_fwd, taac_linear_fp8, taac_norm_linear_fp8_fwd) and the number of units the fused feed-forward
+ * kernels spread their last round over, so that small test inputs walk several token tiles per workgroup; 0 removes
+ * the cap. fp8_tiled != 0 routes taac_linear_fp8 to its generic tiled kernel for every shape. Both start at 0. */
+void taac_test_hooks(int32_t max_workgroups, int32_t fp8_tiled);
 
 /*
  * RMSNorm forward: y[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * w, fp32 accumulation, one rounding

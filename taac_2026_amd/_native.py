@@ -24,7 +24,7 @@ EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
 ATTN_CAUSAL, ATTN_REGISTER_STAGING = 1, 2
 BACKBONE_DENSE_TOKENS, BACKBONE_SPLIT_OUT_FFN, BACKBONE_FP8 = 1, 2, 4
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _DTYPE_CODES = {torch.float32: TAAC_F32, torch.bfloat16: TAAC_BF16, torch.float16: TAAC_F16}
 
@@ -59,6 +59,7 @@ class BlockWeights(ctypes.Structure):
 SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "taac_abi_version": (c_int, []),
     "taac_last_error": (ctypes.c_char_p, []),
+    "taac_test_hooks": (None, [c_int32, c_int32]),
     "taac_rmsnorm_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_float, c_int, c_void_p]),
     "taac_layernorm_fwd": (
         c_int,

@@ -29,6 +29,10 @@ int set_error(int code, const char* fmt, ...);
 int check_launch(const char* what);
 // Compute units of the current device, cached per device; -1 when the query fails.
 int compute_units();
+// Values set through taac_test_hooks: a cap on the grid of the persistent kernels (0: none) and whether taac_linear_fp8
+// is routed to its tiled kernel.
+int test_max_workgroups();
+bool test_fp8_tiled();
 // Packs the qkv / out / feed-forward weights (gate first) of n backbone blocks into fragment order (ffn.hip).
 int pack_backbone_blocks(const taac_block_weights* blocks, int n, int32_t D, int32_t F, void* const* packed_qkv,
                          void* const* packed_out, void* const* packed_ffn, hipStream_t s, const char* name);

@@ -22,8 +22,6 @@
 // bf16, transposed through a wavefront-private LDS tile and written as 16-byte pieces, eight lanes per 128-byte row
 // segment; the residual is read the same way and added after the rounding of the layer output, which is the order
 // of roundings of the reference's bf16 evaluation (linear output rounded, then the residual add rounded).
-#include <cstdlib>
-
 #include "common.h"
 #include "ts_common.h"
 
@@ -1200,10 +1198,7 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
   p.b0 = static_cast<const bf16_t*>(out_bias);
   p.units = compute_units();
   if (p.units <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
-  if (const char* cap = getenv("TAAC_TS_MAX_WORKGROUPS")) {  // test hook, as in the linear kernel
-    const int limit = atoi(cap);
-    if (limit > 0 && limit < p.units) p.units = limit;
-  }
+  if (const int limit = test_max_workgroups(); limit > 0 && limit < p.units) p.units = limit;  // taac_test_hooks
   hipStream_t s = as_stream(stream);
 #define TAAC_FFN_LAUNCH(DD, TT, NW, CPB, DEFER, OUTP)                                                        \
   return launch_ts(swiglu_ffn_kernel<DD, TT, NW, CPB, DEFER, OUTP>, p, NW * kWave, NW * 32 * TT,             \
@@ -1320,11 +1315,8 @@ int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void*
   const int cus = compute_units();
   if (cus <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
   int grid = num_tiles < cus ? num_tiles : cus;
-  // Test hook: cap the number of persistent workgroups so that small inputs exercise the multi-tile path.
-  if (const char* cap = getenv("TAAC_TS_MAX_WORKGROUPS")) {
-    const int limit = atoi(cap);
-    if (limit > 0 && limit < grid) grid = limit;
-  }
+  // taac_test_hooks: cap the number of persistent workgroups so that small inputs exercise the multi-tile path.
+  if (const int limit = test_max_workgroups(); limit > 0 && limit < grid) grid = limit;
 #define TAAC_LIN_LAUNCH(KK, TT, RR, QQ)                                                                           \
   do {                                                                                                            \
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(norm_linear_kernel<KK, TT, RR, QQ>),                    \

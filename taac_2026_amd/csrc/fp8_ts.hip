@@ -451,10 +451,7 @@ int launch_fp8_ts_for_k(const Fp8TsParams& p, int a_is_fp8, int epilogue, hipStr
   const int cus = compute_units();
   if (cus <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
   int grid = num_tiles < cus ? num_tiles : cus;
-  if (const char* cap = getenv("TAAC_TS_MAX_WORKGROUPS")) {  // test hook, as in the bf16 kernel
-    const int limit = atoi(cap);
-    if (limit > 0 && limit < grid) grid = limit;
-  }
+  if (const int limit = test_max_workgroups(); limit > 0 && limit < grid) grid = limit;  // taac_test_hooks
 #define TAAC_FP8_TS_LAUNCH(EPI, AF8)                                                                                \
   do {                                                                                                              \
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(linear_fp8_ts_kernel<K, EPI, AF8, false>),                       \
@@ -490,7 +487,7 @@ int launch_linear_fp8_ts(const void* a, int a_is_fp8, int64_t lda, const void* w
   if (N % (row_blocks(K) * 32) != 0) return 1;
   if (K == 1024 && epilogue == TAAC_EPI_SWIGLU) return 1;
   if (lda % (a_is_fp8 ? 16 : 8) != 0 || ldo % 8 != 0 || (reinterpret_cast<uintptr_t>(bias) & 15u)) return 1;
-  if (getenv("TAAC_FP8_TILED") != nullptr) return 1;  // tuning / test hook: force the tiled kernel
+  if (test_fp8_tiled()) return 1;  // taac_test_hooks: force the tiled kernel
   Fp8TsParams p{};
   p.a = a;
   p.w = static_cast<const uint8_t*>(w);
@@ -578,10 +575,7 @@ extern "C" int taac_norm_linear_fp8_fwd(const void* x, int64_t ldx, const void* 
   const int cus = compute_units();
   if (cus <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
   int grid = num_tiles < cus ? num_tiles : cus;
-  if (const char* cap = getenv("TAAC_TS_MAX_WORKGROUPS")) {  // test hook, as in taac_linear_fp8
-    const int limit = atoi(cap);
-    if (limit > 0 && limit < grid) grid = limit;
-  }
+  if (const int limit = test_max_workgroups(); limit > 0 && limit < grid) grid = limit;  // taac_test_hooks
 #define TAAC_NL_FP8(EPI, ST, NM)                                                                                          \
   do {                                                                                                                    \
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(linear_fp8_ts_kernel<256, EPI, false, ST, NM>),                 \

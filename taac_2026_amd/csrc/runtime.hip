@@ -1,4 +1,5 @@
 // Error reporting and ABI version of libtaac_hip.so.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 
@@ -34,7 +35,18 @@ int compute_units() {
   return count;
 }
 
+// Test hooks (taac_test_hooks): process-wide, changed by tests only.
+static std::atomic<int> g_max_workgroups{0};
+static std::atomic<int> g_fp8_tiled{0};
+int test_max_workgroups() { return g_max_workgroups.load(std::memory_order_relaxed); }
+bool test_fp8_tiled() { return g_fp8_tiled.load(std::memory_order_relaxed) != 0; }
+
 }  // namespace taac
+
+extern "C" void taac_test_hooks(int32_t max_workgroups, int32_t fp8_tiled) {
+  taac::g_max_workgroups.store(max_workgroups > 0 ? max_workgroups : 0, std::memory_order_relaxed);
+  taac::g_fp8_tiled.store(fp8_tiled != 0 ? 1 : 0, std::memory_order_relaxed);
+}
 
 extern "C" int taac_abi_version(void) { return TAAC_ABI_VERSION; }
 extern "C" const char* taac_last_error(void) { return taac::g_last_error; }

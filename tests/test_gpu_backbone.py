@@ -122,13 +122,13 @@ def test_backbone_skips_padded_positions(device):
 
 
 def test_backbone_config4_full_size(device):
-    """Config 4 at full size (B=1024, T=512): a slice of samples against the oracle; all outputs finite; batch rows
-    independent (a sample gives the same probability alone and inside the batch)."""
+    """Config 4 at full size (B=1024, T=512): 64 samples spread over the batch against the oracle; all outputs finite;
+    batch rows independent (a sample gives the same probability alone and inside the batch)."""
     inputs = workloads.backbone_inputs()
     p, hidden = _run(inputs, device)
     assert torch.isfinite(p).all() and torch.isfinite(hidden).all()
     assert ((p > 0) & (p < 1)).all()
-    pick = torch.tensor([0, 257, 511, 1023])
+    pick = torch.unique(torch.linspace(0, 1023, 64).round().long())
     sub = workloads.BackboneInputs(inputs.emb[pick], inputs.key_lengths[pick], inputs.blocks, inputs.head_weight,
                                    inputs.head_bias, inputs.num_heads, inputs.d_ff)
     expected = oracle.backbone(sub.emb, sub.key_lengths, sub.blocks, sub.head_weight, sub.head_bias,

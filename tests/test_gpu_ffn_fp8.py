@@ -117,12 +117,12 @@ def test_fused_fp8_ffn_errors(device):
 
 @pytest.mark.parametrize("workgroups", [None, 2])
 @pytest.mark.parametrize("n,with_norm,with_residual", [(768, True, False), (256, False, True), (256, True, True), (64, False, False)])
-def test_norm_linear_fp8_fuses_norm_rows_and_the_next_scale(device, monkeypatch, n, with_norm, with_residual, workgroups):
+def test_norm_linear_fp8_fuses_norm_rows_and_the_next_scale(device, test_hooks, n, with_norm, with_residual, workgroups):
     """RMSNorm -> quantise -> e4m3 product -> (+ residual) in one kernel, over a row index, with the scale of the consuming
     layer reduced in the epilogue; against the emulated layer on the normalised rows, and against the two-kernel route
     (stand-alone norm, taac_linear_fp8), which computes the same thing."""
     if workgroups is not None:
-        monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+        test_hooks(max_workgroups=workgroups)
     batch, tokens, k = 9, 150, 256
     g = torch.Generator().manual_seed(n + with_norm)
     bf = lambda t: t.to(torch.bfloat16)  # noqa: E731

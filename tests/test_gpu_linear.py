@@ -159,12 +159,12 @@ def test_linear_fp8_epilogues(device):
 
 @pytest.mark.parametrize("workgroups", [None, 1, 2])
 @pytest.mark.parametrize("epilogue", ["none", "residual", "swiglu", "swiglu_value_first"])
-def test_linear_fp8_token_stationary_path(device, monkeypatch, epilogue, workgroups):
+def test_linear_fp8_token_stationary_path(device, test_hooks, epilogue, workgroups):
     """K = 256 layers run on the token-stationary e4m3 kernel: every epilogue, bf16 and pre-quantised activations,
     ragged M, one and several token tiles per workgroup; and the tiled kernel (forced) gives the same numbers up to the
     rounding of the output."""
     if workgroups is not None:
-        monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+        test_hooks(max_workgroups=workgroups)
     m, k = 1333, 256
     swiglu = epilogue.startswith("swiglu")
     gate_first = epilogue != "swiglu_value_first"
@@ -180,7 +180,7 @@ def test_linear_fp8_token_stationary_path(device, monkeypatch, epilogue, workgro
         xq, _ = quantize_fp8(x.to(device), xa)
         got_q = linear_fp8(xq, wq, xa, wa, b.to(device), **kwargs)
         no_bias = linear_fp8(x.to(device), wq, xa, wa, None, **kwargs)
-        monkeypatch.setenv("TAAC_FP8_TILED", "1")
+        test_hooks(fp8_tiled=True)
         tiled = linear_fp8(x.to(device), wq, xa, wa, b.to(device), **kwargs)
         tiled_no_bias = linear_fp8(x.to(device), wq, xa, wa, None, **kwargs)
     assert got.shape == expected.shape
@@ -193,11 +193,11 @@ def test_linear_fp8_token_stationary_path(device, monkeypatch, epilogue, workgro
 
 @pytest.mark.parametrize("epilogue", ["none", "residual"])
 @pytest.mark.parametrize("workgroups", [None, 2])
-def test_linear_fp8_token_stationary_long_reduction(device, monkeypatch, epilogue, workgroups):
+def test_linear_fp8_token_stationary_long_reduction(device, test_hooks, epilogue, workgroups):
     """K = 1024 (the FFN down projection) on the token-stationary e4m3 kernel: one 32-row weight block per step, ragged
     M, several token tiles per workgroup, bf16 and pre-quantised activations, against the oracle and the tiled kernel."""
     if workgroups is not None:
-        monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+        test_hooks(max_workgroups=workgroups)
     m, n, k = 1111, 96, 1024
     x, w, b = _draw(m, n, k, seed=17 + (workgroups or 0))
     res = torch.randn(m, n, generator=torch.Generator().manual_seed(6)).to(torch.bfloat16) if epilogue == "residual" else None
@@ -209,7 +209,7 @@ def test_linear_fp8_token_stationary_long_reduction(device, monkeypatch, epilogu
         got = linear_fp8(x.to(device), wq, xa, wa, b.to(device), **kwargs)
         xq, _ = quantize_fp8(x.to(device), xa)
         got_q = linear_fp8(xq, wq, xa, wa, b.to(device), **kwargs)
-        monkeypatch.setenv("TAAC_FP8_TILED", "1")
+        test_hooks(fp8_tiled=True)
         tiled = linear_fp8(x.to(device), wq, xa, wa, b.to(device), **kwargs)
     assert _rel_err(got.cpu(), expected) <= 5e-2
     assert _rel_err(got_q.cpu(), expected) <= 5e-2
@@ -264,14 +264,14 @@ def _block_tail_inputs(m, d, f, seed):
 @pytest.mark.parametrize("m,d,f", [(1, 256, 32), (300, 256, 1024), (64, 128, 64), (1000, 256, 96), (257, 128, 256),
                                    (2500, 256, 64)])
 @pytest.mark.parametrize("workgroups", [None, 3])
-def test_fused_attention_out_ffn(device, monkeypatch, m, d, f, workgroups):
+def test_fused_attention_out_ffn(device, test_hooks, m, d, f, workgroups):
     """out projection + residual -> RMSNorm -> up -> SiLU-gate -> down -> + residual in one kernel, against the oracle's
     pieces (dense layers evaluated in fp32 from the stored operands, the residual stream rounded to bf16 in between) and
     against the two-kernel route of the same library."""
     from taac_2026_amd.api import attention_out_ffn, norm_linear, swiglu_ffn
 
     if workgroups is not None:
-        monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+        test_hooks(max_workgroups=workgroups)
     attn, h, nw, wo, bo, wu, bu, wd, bd = _block_tail_inputs(m, d, f, seed=m + d + f)
     lin = F.linear(attn.float(), wo.float(), bo.float()).to(torch.bfloat16)
     x1 = (lin.float() + h.float()).to(torch.bfloat16)
@@ -341,13 +341,13 @@ def test_fused_norm_linear(device, m, k, n):
 
 @pytest.mark.parametrize("workgroups", [1, 2, 3])
 @pytest.mark.parametrize("m,k,n", [(3000, 256, 768), (2049, 128, 256), (1500, 256, 64)])
-def test_fused_norm_linear_walks_several_token_tiles(device, monkeypatch, workgroups, m, k, n):
+def test_fused_norm_linear_walks_several_token_tiles(device, test_hooks, workgroups, m, k, n):
     """The linear kernel is persistent: with few workgroups each one walks several token tiles (what happens at full
     size on 256 compute units), including the out-of-phase tile changes of its two wavefront groups and the residual
     pieces requested one step ahead across a tile boundary."""
     from taac_2026_amd.api import norm_linear
 
-    monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+    test_hooks(max_workgroups=workgroups)
     x, w, b = _draw(m, n, k, seed=m + n + workgroups)
     g = torch.Generator().manual_seed(11)
     nw = (1 + 0.1 * torch.randn(k, generator=g)).to(torch.bfloat16)
@@ -383,13 +383,13 @@ def test_valid_rows_index(device):
 
 
 @pytest.mark.parametrize("workgroups", [None, 2])
-def test_fused_layers_skip_padded_rows(device, monkeypatch, workgroups):
+def test_fused_layers_skip_padded_rows(device, test_hooks, workgroups):
     """With a row index the fused layers process exactly the valid rows of a padded batch: those rows are bit-identical
     to the dense run, all other rows are neither read (they hold NaN here) nor written."""
     from taac_2026_amd.api import norm_linear, swiglu_ffn, valid_rows
 
     if workgroups is not None:
-        monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+        test_hooks(max_workgroups=workgroups)
     g = torch.Generator().manual_seed(21)
     batch, tokens, d, f = 9, 200, 256, 96
     lengths = torch.tensor([200, 1, 0, 77, 128, 199, 33, 64, 160], dtype=torch.int32)

@@ -105,11 +105,34 @@ def test_norm_full_size_properties(device):
         # scale equivariance: rms_norm(4x) == rms_norm(x) up to eps (an exact power of two: at most one bf16 step)
         y4 = rms_norm(x * 4.0, w, 1e-6)
         torch.testing.assert_close(y4.float(), y.float(), rtol=2e-2, atol=2e-2)
-        # a random sample of rows agrees with the oracle
+        # a random sample of rows agrees with the oracle, for both norms
         idx = torch.randint(0, 4096 * 256, (2048,), generator=torch.Generator().manual_seed(3))
         rows = x.view(-1, 256)[idx.to(device)].cpu()
         torch.testing.assert_close(y.view(-1, 256)[idx.to(device)].cpu().float(),
                                    oracle.rms_norm_fp32(rows, w.cpu(), 1e-6).float(), rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(z.view(-1, 256)[idx.to(device)].cpu().float(),
+                                   oracle.layer_norm_fp32(rows, w.cpu(), b.cpu(), 1e-5).float(), rtol=2e-2, atol=2e-2)
+
+
+def test_norm_config2_full_size_sampled_rows(device):
+    """Config 2 as the workload draws it (1 048 576 x 256 bf16, 1 % of the rows scaled x50, gamma ~ N(1, 0.1),
+    beta ~ N(0, 0.02)) at full size: 4 096 rows spread over the tensor, the outlier rows among them, against the oracle
+    for RMSNorm and LayerNorm."""
+    x, gamma, beta = workloads.norm_bf16_inputs()
+    rows = x.view(-1, 256)
+    xd, gd, bd = x.to(device), gamma.to(device), beta.to(device)
+    with torch.no_grad():
+        y = rms_norm(xd, gd, 1e-6).view(-1, 256)
+        z = layer_norm(xd, gd, bd, 1e-5).view(-1, 256)
+    assert torch.isfinite(y).all() and torch.isfinite(z).all()
+    outliers = torch.nonzero(rows.float().abs().amax(dim=-1) > 25.0).flatten()[:1024]
+    assert outliers.numel() > 0
+    idx = torch.cat([torch.randint(0, rows.shape[0], (3072,), generator=torch.Generator().manual_seed(5)), outliers])
+    sample = rows[idx]
+    torch.testing.assert_close(y[idx.to(device)].cpu().float(), oracle.rms_norm_fp32(sample, gamma, 1e-6).float(),
+                               rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(z[idx.to(device)].cpu().float(), oracle.layer_norm_fp32(sample, gamma, beta, 1e-5).float(),
+                               rtol=2e-2, atol=2e-2)
 
 
 def test_modules_and_errors(device):

@@ -155,7 +155,7 @@ def test_attention_layers_with_normalised_queries_and_keys(device, layer):
 @pytest.mark.parametrize("d_model,heads", [(256, 8), (128, 4)])
 @pytest.mark.parametrize("mode", ["norm", "rope", "norm+rope"])
 @pytest.mark.parametrize("workgroups", [None, 3])
-def test_qkv_projection_prepares_queries_and_keys_in_its_epilogue(device, monkeypatch, d_model, heads, mode, workgroups):
+def test_qkv_projection_prepares_queries_and_keys_in_its_epilogue(device, test_hooks, d_model, heads, mode, workgroups):
     """The packed projection with the query / key preparation in its epilogue: q and k columns come out as
     rotate(projection * weight), the value columns as the plain projection, and the returned per-token factors are
     rsqrt(mean(projection^2) + eps); factor * columns equals the oracle's RMSNorm + rotary embedding. Run with one
@@ -163,7 +163,7 @@ def test_qkv_projection_prepares_queries_and_keys_in_its_epilogue(device, monkey
     from taac_2026_amd.api import qkv_projection
 
     if workgroups is not None:
-        monkeypatch.setenv("TAAC_TS_MAX_WORKGROUPS", str(workgroups))
+        test_hooks(max_workgroups=workgroups)
     batch, tokens = 5, 333
     g = torch.Generator().manual_seed(d_model + len(mode))
     x = torch.randn(batch, tokens, d_model, generator=g).to(torch.bfloat16)
