@@ -817,10 +817,21 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
   // First token of this wavefront in token tile `tile`.
   auto tokens_of_tile = [&](int tile) -> int64_t { return static_cast<int64_t>(tile) * kTokPerWg + wave * (32 * TT); };
   // Memory rows of a tile in the layout of the epilogue stores: piece i = token (i / 4) * 32 + 8 * (i % 4) + lane / 8.
+  // Without a residual the row numbers are only needed for the stores, so the lane's store offset is kept instead, in
+  // units of 16 bytes (row * ldo / 8 + lane % 8; the host checks that it fits 32 bits): a store then needs one
+  // multiply-add for its address instead of a 64-bit row * stride product per piece and step.
+  const uint32_t ld16 = static_cast<uint32_t>(p.ldo >> 3);
   auto rows_of_tile = [&](int64_t tok_base, int32_t (&prow)[NST]) {
 #pragma unroll
-    for (int i = 0; i < NST; ++i)
-      prow[i] = static_cast<int32_t>(token_row(p, count, tok_base + (i / 4) * 32 + (i % 4) * 8 + lane / 8));
+    for (int i = 0; i < NST; ++i) {
+      const int32_t row = static_cast<int32_t>(token_row(p, count, tok_base + (i / 4) * 32 + (i % 4) * 8 + lane / 8));
+      prow[i] = RES ? row : static_cast<int32_t>(static_cast<uint32_t>(row) * ld16 + static_cast<uint32_t>(lane % 8));
+    }
+  };
+  // Address of the lane's 16-byte piece of output chunk `chunk` for piece slot value v (a row with RES, an offset without).
+  auto out_piece = [&](int32_t v, int chunk) -> bf16x8* {
+    const uint32_t off16 = RES ? static_cast<uint32_t>(v) * ld16 + static_cast<uint32_t>(lane % 8) : static_cast<uint32_t>(v);
+    return reinterpret_cast<bf16x8*>(reinterpret_cast<char*>(p.out) + chunk * (kNC * 2) + (static_cast<uint64_t>(off16) << 4));
   };
   auto request_residual = [&](const int32_t (&prow)[NST], int chunk, bf16x8 (&res)[NST]) {
 #pragma unroll
@@ -829,6 +840,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
                                                 (lane % 8) * 8);
   };
   bf16x8 xf[TT][KS];
+  int32_t prow[NST], prow_next[NST];  // piece slots (see rows_of_tile) of the current tile / of the tile the next step belongs to
   auto load_tile = [&](int64_t tok_base) {
     load_token_rows<D, TT>(p, count, tok_base, l32, hh, xf);
     // Consume the rows right here: otherwise the compiler's wait for them lands in front of the first MFMA of EVERY
@@ -837,6 +849,13 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     for (int t = 0; t < TT; ++t)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(xf[t][ks]));
+    if constexpr (QK == 0 && !RES) {
+      // the same for the store offsets (their row numbers were loaded just before the rows): otherwise the compiler
+      // waits for them in front of the first store of every step, with a count that also covers the weight transfers
+      // and the stores that are meant to stay in flight
+#pragma unroll
+      for (int i = 0; i < NST; ++i) asm volatile("" : "+v"(prow[i]));
+    }
     if (QK != 0) {  // lane <-> token `lane` of the wavefront's 32 * TT tokens
       // the token's position inside its sample is that of its row of x (the side that keeps the caller's layout)
       const int64_t tok = tok_base + (lane < 32 * TT ? lane : 0);
@@ -846,7 +865,6 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
   };
 
   bf16x8 res_cur[NST], res_next[NST];
-  int32_t prow[NST], prow_next[NST];  // rows of the current tile / of the tile the next step belongs to
   int64_t tok_wave = tokens_of_tile(tile_of(0));
   if constexpr (QK == 0) rows_of_tile(tok_wave, prow);
   stage(chunk_of(0), 0);
@@ -1020,8 +1038,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
         // non-temporal: the 64 KB a workgroup stores per step are not read again by this kernel; as ordinary stores they
         // wait for the cache lines they displace (stand-alone 0.166 against 0.176 ms for q | k | v, 0.093 against 0.112 ms
         // for the out projection; inside the step the kernel behind reads the rows from memory either way)
-        __builtin_nontemporal_store(v, reinterpret_cast<bf16x8*>(p.out + static_cast<int64_t>(prow[t * 4 + i]) * p.ldo +
-                                                                 chunk * kNC + (lane % 8) * 8));
+        __builtin_nontemporal_store(v, out_piece(prow[t * 4 + i], chunk));
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
@@ -1273,6 +1290,8 @@ int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void*
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: rows and n_rows must be given together", name);
   if (x_rows && !rows) return set_error(TAAC_ERR_INVALID_VALUE, "%s: x_rows needs rows and n_rows", name);
   if (M > 0x7fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: at most 2^31 rows", name);
+  if (M * (ldo / 8) + 8 > 0xffffffffLL)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: the output spans more than 2^32 16-byte pieces", name);
   if (!ptr_ok(x, 15) || !ptr_ok(w, 15) || !ptr_ok(out, 15) || !ptr_ok(residual, 15) || !ptr_ok(norm_weight, 15) ||
       !ptr_ok(bias, 15) || !ptr_ok(packed_weights, 15) || !ptr_ok(qk.qk_weight, 15) || !ptr_ok(qk.cos_sin, 15) ||
       !ptr_ok(qk.qk_sumsq, 3))
