@@ -423,6 +423,24 @@ int taac_attn_out_ffn_fwd(const void* attn, int64_t ld_attn, const void* out_bia
                           void* stream);
 
 /*
+ * taac_attn_out_ffn_fwd with a sigmoid gate on the projected update (TokenFormer's NLIR gate):
+ *   x1  = residual + sigmoid(update_gate) * (attn @ w_out^T + out_bias)
+ *   out = x1 + down( silu(g) * u ) + b_down,   g, u = chunk2( up( norm_weight ? rmsnorm(x1, norm_weight, eps) : x1 ) )
+ * update_gate: [M, D] bf16 (row stride ld_gate, rows laid out like residual / out), the gate layer's output BEFORE the
+ * sigmoid: nlir_gate(attn_norm(tokens)), e.g. from taac_norm_linear_fwd on the block input. Roundings follow the
+ * reference's 16-bit evaluation: the projection, the sigmoid, their product and the sum with the residual are each
+ * rounded to bf16. Everything else as in taac_attn_out_ffn_fwd.
+ * Replaces: nlir_gate's sigmoid, the gated residual update and ffn_norm + SwiGLUFeedForward.forward + residual add of
+ * TokenFormerBlock.forward (experiments/tokenformer/model.py:209-214); the `* valid` factors of that forward are the
+ * row index (padded rows are never touched).
+ */
+int taac_attn_out_gate_ffn_fwd(const void* attn, int64_t ld_attn, const void* out_bias, const void* packed_out_weights,
+                               const void* update_gate, int64_t ld_gate, const void* residual, int64_t ldr,
+                               const void* norm_weight, float eps, const void* b_up, const void* b_down,
+                               const void* packed_ffn_weights, void* out, int64_t ldo, int64_t M, int32_t D, int32_t F,
+                               const int32_t* rows, const int32_t* n_rows, const int32_t* attn_rows, void* stream);
+
+/*
  * Fused [RMSNorm ->] dense layer [-> + residual] with the token rows held in registers:
  *   out = (residual ? residual : 0) + (norm_weight ? rmsnorm(x, norm_weight, eps) : x) @ w^T + bias
  * x: [M, K] bf16; w: [N, K]; bias: [N] or NULL; residual / out: [M, N]; packed_weights: NULL or the blob written by

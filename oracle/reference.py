@@ -42,6 +42,13 @@ Puiching-Memory/TAAC_2026). How each function is pinned, independently of its ow
                       loop and special cases (no candidate -> zero third, all-padded sample -> zero mean, no norms ->
                       picked rows and plain masked mean); qk_norm_rope and embedding_bag_mean additionally by the
                       pure-Python float64 vectors of tests/golden/qk_rope_embedding_small.json.
+  tokenformer_block / silu_mlp / mixed_feed_forward
+                      the reference holds no numeric test for them (shape / finiteness contract tests only); compositions
+                      of the functions above as the modules write them (experiments/tokenformer/model.py:203-215,
+                      experiments/onetrans/model.py:33-44, 80-94), pinned by float64 per-element loops on tiny shapes
+                      (gate = 1 / (1 + exp(-z)) applied to the update before the residual add; padded rows pass
+                      through; a zero gate layer halves the update), the gated block reducing to interaction_block's
+                      arithmetic when the gate is forced to one, and token replacement checked slot by slot.
   fp8 emulation       PARITY UNPINNED by the reference (it has no FP8 code). Defined by the configuration text:
                       s = amax/448, q = (t/s).to(float8_e4m3fn), y = (qa.float() @ qw.float().T) * s_a * s_w.
                       The e4m3 rounding itself is pinned against an exhaustive decode table of all 256 codes and
@@ -455,6 +462,51 @@ def interaction_block(tokens: torch.Tensor, padding_mask: torch.Tensor, attentio
     h2 = rms_norm(attn_tokens, w["ffn_norm.weight"], eps)
     output = attn_tokens + swiglu_ffn(h2, w["up.weight"], w.get("up.bias"), w["down.weight"], w.get("down.bias")) * keep
     return output, attn_tokens
+
+
+def tokenformer_block(tokens: torch.Tensor, padding_mask: torch.Tensor, attention_mask: torch.Tensor | None,
+                      w: dict[str, torch.Tensor], *, num_heads: int, eps: float = 1e-6,
+                      rope_base: float | None = None) -> torch.Tensor:
+    """``TokenFormerBlock.forward`` as written (experiments/tokenformer/model.py:203-215): the attention layer
+    (``BFTSAttention.forward``, :150-163: packed projection, RMSNorm(d_model) of query and key, optional rotary
+    embedding, attention, out projection) reads ``attn_norm(tokens)``; its update is multiplied by
+    ``sigmoid(nlir_gate(attn_norm(tokens)))`` and by ``~padding_mask`` before it joins the stream; the SwiGLU feed-forward
+    update is multiplied by ``~padding_mask`` as well. ``w`` holds the block's parameters under the names of
+    :func:`interaction_block` plus ``nlir_gate.weight`` / ``nlir_gate.bias``."""
+    batch, token_count, d_model = tokens.shape
+    keep = (~padding_mask).unsqueeze(-1).to(tokens.dtype)
+    h = rms_norm(tokens, w["attn_norm.weight"], eps)
+    q, k, v = F.linear(h, w["qkv.weight"], w.get("qkv.bias")).chunk(3, dim=-1)
+    q, k = qk_norm_rope(q, k, w.get("query_norm.weight"), w.get("key_norm.weight"), num_heads=num_heads, eps=eps,
+                        rope_base=rope_base)
+    heads = lambda t: t.view(batch, token_count, num_heads, d_model // num_heads).transpose(1, 2)  # noqa: E731
+    a = sdpa(heads(q), heads(k), heads(v), attn_mask=attention_mask).transpose(1, 2).reshape(batch, token_count, d_model)
+    attention_update = F.linear(a, w["out.weight"], w.get("out.bias"))
+    nlir_update = torch.sigmoid(F.linear(h, w["nlir_gate.weight"], w.get("nlir_gate.bias"))) * attention_update
+    tokens = tokens + nlir_update * keep
+    h2 = rms_norm(tokens, w["ffn_norm.weight"], eps)
+    return tokens + swiglu_ffn(h2, w["up.weight"], w.get("up.bias"), w["down.weight"], w.get("down.bias")) * keep
+
+
+def silu_mlp(x: torch.Tensor, fc1_weight: torch.Tensor, fc1_bias: torch.Tensor | None, fc2_weight: torch.Tensor,
+             fc2_bias: torch.Tensor | None) -> torch.Tensor:
+    """OneTrans' ``FeedForward.forward`` in eval mode (experiments/onetrans/model.py:33-44):
+    ``Linear(d_model, d_model * hidden_mult) -> SiLU -> Dropout -> Linear(d_model * hidden_mult, d_model)``."""
+    return F.linear(F.silu(F.linear(x, fc1_weight, fc1_bias)), fc2_weight, fc2_bias)
+
+
+def mixed_feed_forward(tokens: torch.Tensor, seq_token_count: int, shared: tuple, ns_specific: list[tuple]) -> torch.Tensor:
+    """OneTrans' ``MixedFeedForward.forward`` (experiments/onetrans/model.py:87-94): the shared feed-forward over every
+    token, then the token at position ``seq_token_count + i`` is replaced by the output of the i-th token-specific
+    feed-forward on that token (positions beyond the sequence are skipped). ``shared`` and every entry of
+    ``ns_specific`` are ``(fc1_weight, fc1_bias, fc2_weight, fc2_bias)``."""
+    output = silu_mlp(tokens, *shared).clone()
+    for ns_index, weights in enumerate(ns_specific):
+        position = seq_token_count + ns_index
+        if position >= tokens.shape[1]:
+            continue
+        output[:, position, :] = silu_mlp(tokens[:, position, :], *weights)
+    return output
 
 
 def backbone(emb: torch.Tensor, key_lengths: torch.Tensor, blocks: list[dict[str, torch.Tensor]],

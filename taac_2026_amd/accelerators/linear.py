@@ -609,15 +609,20 @@ def attention_out_ffn(
     token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
     input_rows: torch.Tensor | None = None,
     out: torch.Tensor | None = None,
+    update_gate: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Second half of a ``UnifiedInteractionBlock`` (experiments/symbiosis/backbone.py:47, 64-67) as ONE kernel:
     ``x1 = residual + F.linear(attn, out_weight, out_bias)`` then ``x1 + down(silu(gate) * value)`` with
     ``gate, value = up(rmsnorm(x1)).chunk(2, -1)``. ``x1`` never reaches memory. Model width 128 / 256 and a hidden
     size that is a multiple of 32 only (``taac_attn_out_ffn_fwd``); ``token_rows`` / ``out`` as in :func:`swiglu_ffn`
     (``out`` may be ``residual``). ``input_rows`` (with ``token_rows``): the row of ``attn`` that holds each token when
-    ``attn`` is laid out differently from ``residual`` / ``out`` (:func:`front_rows`)."""
+    ``attn`` is laid out differently from ``residual`` / ``out`` (:func:`front_rows`).
+
+    ``update_gate`` (shape of ``residual``): the second half of a ``TokenFormerBlock`` (experiments/tokenformer/
+    model.py:209-214) instead - ``x1 = residual + sigmoid(update_gate) * F.linear(attn, out_weight, out_bias)``, with
+    ``update_gate`` the output of the block's ``nlir_gate`` layer before the sigmoid (``taac_attn_out_gate_ffn_fwd``)."""
     name = "hip attention_out_ffn"
-    tensors = (attn, out_weight, out_bias, residual, up_weight, up_bias, down_weight, down_bias, norm_weight)
+    tensors = (attn, out_weight, out_bias, residual, up_weight, up_bias, down_weight, down_bias, norm_weight, update_gate)
     require_cuda_tensors(name, *tensors)
     require_inference(name, *tensors)
     _check_bf16(name, *tensors)
@@ -639,6 +644,21 @@ def attention_out_ffn(
     index, count = _token_rows(name, token_rows, rows)
     out = _output_rows(name, out, (rows.shape[0], d_model), index is not None, attn)
     library = _native.load_library()
+    if update_gate is not None:
+        if update_gate.shape != shape:
+            raise ValueError("attention_out_ffn update_gate must have the shape of the attention output")
+        gate_rows = update_gate.reshape(-1, d_model)
+        if gate_rows.stride(-1) != 1 or gate_rows.stride(0) % 8 != 0:
+            gate_rows = gate_rows.contiguous()
+        status = library.taac_attn_out_gate_ffn_fwd(
+            rows.data_ptr(), rows.stride(0), _native.ptr(out_bias), packed_out.data_ptr(), gate_rows.data_ptr(),
+            gate_rows.stride(0), res_rows.data_ptr(), res_rows.stride(0), _native.ptr(norm_weight), float(eps),
+            _native.ptr(up_bias), _native.ptr(down_bias), packed_ffn.data_ptr(), out.data_ptr(), d_model, rows.shape[0],
+            d_model, hidden, _native.ptr(index), _native.ptr(count),
+            _native.ptr(_input_rows(name, input_rows, index, rows)), _native.current_stream(attn.device),
+        )
+        _native.check(status, "attention_out_ffn")
+        return out.reshape(shape)
     status = library.taac_attn_out_ffn_fwd(
         rows.data_ptr(), rows.stride(0), _native.ptr(out_bias), packed_out.data_ptr(), res_rows.data_ptr(),
         res_rows.stride(0), _native.ptr(norm_weight), float(eps), _native.ptr(up_bias), _native.ptr(down_bias),

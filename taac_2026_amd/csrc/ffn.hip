@@ -64,6 +64,8 @@ struct TsParams {
   // Attention output projection in front of the FFN (x is then the attention output, residual the block input):
   const bf16_t* w0;         // packed [D, D] projection (linear blob)
   const bf16_t* b0;         // its bias [D] or null
+  const bf16_t* gate;       // GATE: [M, D] pre-activation of the update's gate (rows like residual), row stride ldg
+  int64_t ldg;
 };
 
 __device__ __forceinline__ float silu_f(float v) {
@@ -332,9 +334,17 @@ __device__ __forceinline__ void load_residual(const bf16_t* residual, int64_t ld
 // token per lane, a fragment needs 8-feature runs, and lanes l and l ^ 32 own the two halves of each run.
 // Replaces the out projection + residual and the feed-forward half of UnifiedInteractionBlock.forward
 // (experiments/symbiosis/backbone.py:60-67) in one pass over the tokens.
+//
+// GATE (with OUTP): the projected update is multiplied by a sigmoid gate before it joins the residual stream,
+//   x1 = bf16( h + bf16( bf16(sigmoid(g)) * bf16(A W0^T + b0) ) ),
+// g = p.gate, the gate layer's output in 16 bits (TokenFormerBlock.forward, experiments/tokenformer/model.py:209-214:
+// the gate layer reads the normalised block input, which only the projection kernel in front of attention holds, so
+// it arrives as a tensor). Its pieces of a chunk are requested behind the chunk's MFMAs, into the registers the weight
+// fragments have left, so the variant takes no registers of its own.
 // ------------------------------------------------------------------------------------------------------------------
-template <int D, int TT, int NWAVES, int CPB, bool DEFER, bool OUTP>
+template <int D, int TT, int NWAVES, int CPB, bool DEFER, bool OUTP, bool GATE = false>
 __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_kernel(const TsParams p) {
+  static_assert(!GATE || OUTP, "the gate belongs to the projection in front");
   constexpr int kTokPerWg = NWAVES * 32 * TT;  // TT token tiles of 32 per wavefront
   constexpr int KS = D / 16;             // k-steps of the up projection = up fragments per chunk
   constexpr int MB = D / 32;             // 32-feature row blocks of the down projection = down fragments per chunk
@@ -476,10 +486,12 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
     const bf16_t* b0_lds = bias_lds + 2 * F + 2 * D;
     float ss[TT];
     const bf16_t* hrow[TT];
+    [[maybe_unused]] const bf16_t* grow[TT];
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
       ss[t] = 0.f;
       hrow[t] = p.residual + hrow_index[t] * p.ldr + hh * 4;
+      if constexpr (GATE) grow[t] = p.gate + hrow_index[t] * p.ldg + hh * 4;
     }
     static_for<NCH>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
@@ -511,6 +523,14 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
         // x1 = bf16( bf16(projection + b0) + h ), kept in the accumulators; sum of squares for the norm that follows
         bf16x4 bv[8];
         read_chunk_bias(b0_lds + c * kNC, hh, bv);
+        [[maybe_unused]] bf16x4 gv[TT][8];
+        if constexpr (GATE) {
+#pragma unroll
+          for (int t = 0; t < TT; ++t)
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+              gv[t][q] = *reinterpret_cast<const bf16x4*>(grow[t] + c * kNC + (q / 4) * 32 + (q % 4) * 8);
+        }
 #pragma unroll
         for (int t = 0; t < TT; ++t)
 #pragma unroll
@@ -518,7 +538,12 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const float a = oacc[t][2 * c + q / 4][(q % 4) * 4 + e];
-              const float lin = static_cast<float>(static_cast<bf16_t>(a + static_cast<float>(bv[q][e])));
+              float lin = static_cast<float>(static_cast<bf16_t>(a + static_cast<float>(bv[q][e])));
+              if constexpr (GATE) {
+                const float g = static_cast<float>(gv[t][q][e]);
+                const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
+                lin = static_cast<float>(static_cast<bf16_t>(static_cast<float>(static_cast<bf16_t>(sg)) * lin));
+              }
               const float x1 = static_cast<float>(static_cast<bf16_t>(lin + static_cast<float>(hv[t][q][e])));
               oacc[t][2 * c + q / 4][(q % 4) * 4 + e] = x1;
               ss[t] = fmaf(x1, x1, ss[t]);
@@ -1164,8 +1189,12 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
               const void* norm_weight, float eps, const void* w_up, const void* b_up, const void* w_down,
               const void* b_down, const void* packed_weights, const void* residual, int64_t ldr, void* out, int64_t ldo,
               int64_t M, int32_t D, int32_t F, int gate_first, const int32_t* rows, const int32_t* n_rows,
-              const int32_t* x_rows, void* stream) {
+              const int32_t* x_rows, void* stream, const void* update_gate = nullptr, int64_t ldg = 0) {
   const bool with_proj = out_packed != nullptr;
+  if (update_gate && !with_proj)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: an update gate needs the projection in front", name);
+  if (update_gate && (ldg < D || ldg % 8 || !ptr_ok(update_gate, 15)))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: the gate's row stride must cover a row and be a multiple of 8, its base 16-byte aligned", name);
   if (M < 0 || D <= 0 || F <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, D and F > 0", name);
   if (D != 256 && D != 128)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: fused kernel is built for D = 128 or 256 (got %d)", name, D);
@@ -1213,13 +1242,19 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
   p.x_rows = x_rows;
   p.w0 = static_cast<const bf16_t*>(out_packed);
   p.b0 = static_cast<const bf16_t*>(out_bias);
+  p.gate = static_cast<const bf16_t*>(update_gate);
+  p.ldg = ldg;
   p.units = compute_units();
   if (p.units <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
   if (const int limit = test_max_workgroups(); limit > 0 && limit < p.units) p.units = limit;  // taac_test_hooks
   hipStream_t s = as_stream(stream);
-#define TAAC_FFN_LAUNCH(DD, TT, NW, CPB, DEFER, OUTP)                                                        \
-  return launch_ts(swiglu_ffn_kernel<DD, TT, NW, CPB, DEFER, OUTP>, p, NW * kWave, NW * 32 * TT,             \
+#define TAAC_FFN_LAUNCH(DD, TT, NW, CPB, DEFER, ...)                                                         \
+  return launch_ts(swiglu_ffn_kernel<DD, TT, NW, CPB, DEFER, __VA_ARGS__>, p, NW * kWave, NW * 32 * TT,      \
                    static_cast<size_t>((DEFER ? 3 : 2) * CPB * (KS + MB)) * kFrag + bias_bytes, s, name)
+  if (with_proj && update_gate) {
+    if (D == 256) TAAC_FFN_LAUNCH(256, 1, 8, 2, true, true, true);
+    TAAC_FFN_LAUNCH(128, 1, 8, 2, true, true, true);
+  }
   if (with_proj) {
     if (D == 256) TAAC_FFN_LAUNCH(256, 1, 8, 2, true, true);
     TAAC_FFN_LAUNCH(128, 1, 8, 2, true, true);
@@ -1260,6 +1295,22 @@ extern "C" int taac_attn_out_ffn_fwd(const void* attn, int64_t ld_attn, const vo
     return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: both weight sets must be packed", name);
   return taac::ffn_entry(name, attn, ld_attn, out_bias, packed_out_weights, norm_weight, eps, nullptr, b_up, nullptr,
                          b_down, packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, attn_rows, stream);
+}
+
+extern "C" int taac_attn_out_gate_ffn_fwd(const void* attn, int64_t ld_attn, const void* out_bias,
+                                          const void* packed_out_weights, const void* update_gate, int64_t ld_gate,
+                                          const void* residual, int64_t ldr, const void* norm_weight, float eps,
+                                          const void* b_up, const void* b_down, const void* packed_ffn_weights,
+                                          void* out, int64_t ldo, int64_t M, int32_t D, int32_t F,
+                                          const int32_t* rows, const int32_t* n_rows, const int32_t* attn_rows,
+                                          void* stream) {
+  const char* name = "taac_attn_out_gate_ffn_fwd";
+  if (!packed_out_weights || !packed_ffn_weights)
+    return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: both weight sets must be packed", name);
+  if (!update_gate) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: null gate pointer", name);
+  return taac::ffn_entry(name, attn, ld_attn, out_bias, packed_out_weights, norm_weight, eps, nullptr, b_up, nullptr,
+                         b_down, packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, attn_rows, stream,
+                         update_gate, ld_gate);
 }
 
 namespace taac {

@@ -4,6 +4,7 @@ from taac_2026_amd.modeling.backbone import (
     BFTSAttention,
     PCVRBackbone,
     SwiGLUFeedForward,
+    TokenFormerBlock,
     UnifiedInteractionBlock,
     run_interaction_blocks,
     UnifiedSelfAttention,
@@ -41,6 +42,7 @@ __all__ = [
     "PCVRBackbone",
     "RMSNorm",
     "SwiGLUFeedForward",
+    "TokenFormerBlock",
     "UnifiedInteractionBlock",
     "run_interaction_blocks",
     "UnifiedSelfAttention",

@@ -252,6 +252,18 @@ class UnifiedInteractionBlock(nn.Module):
         dense = dict(norm_weight=_bf16(self.ffn_norm.weight), eps=self.ffn_norm.eps, token_rows=index)
         if front is not None:
             dense["input_rows"] = front
+        gate_layer = getattr(self, "nlir_gate", None)
+        if gate_layer is not None:
+            # the gate layer reads the normalised block input, like the projection in front of attention; its output (before
+            # the sigmoid) is written at the valid rows and consumed by the kernel that applies the update
+            gate = torch.empty(batch * token_count, d_model, dtype=x.dtype, device=x.device)
+            norm_linear(x, _bf16(gate_layer.weight), _bf16(gate_layer.bias), norm_weight=_bf16(self.attn_norm.weight),
+                        eps=self.attn_norm.eps, token_rows=index, out=gate)
+            output = x if inplace else x.clone()
+            attention_out_ffn(attended, _bf16(attention.out.weight), _bf16(attention.out.bias), x, _bf16(ffn.up.weight),
+                              _bf16(ffn.up.bias), _bf16(ffn.down.weight), _bf16(ffn.down.bias), out=output,
+                              update_gate=gate.view(batch, token_count, d_model), **dense)
+            return output, None
         if not return_attention_tokens and ffn.gate_first:
             output = x if inplace else x.clone()
             attention_out_ffn(attended, _bf16(attention.out.weight), _bf16(attention.out.bias), x, _bf16(ffn.up.weight),
@@ -292,6 +304,37 @@ class UnifiedInteractionBlock(nn.Module):
         ffn_update = self.ffn(self.ffn_norm(attn_tokens))
         output = attn_tokens + ffn_update * keep.to(ffn_update.dtype)
         return output, attn_tokens
+
+
+class TokenFormerBlock(UnifiedInteractionBlock):
+    """TokenFormer's block (experiments/tokenformer/model.py:195-215): the interaction block with ``BFTSAttention`` as its
+    attention layer and the NLIR gate on the attention update,
+    ``tokens + sigmoid(nlir_gate(attn_norm(tokens))) * attention(attn_norm(tokens)) * valid``, followed by the same
+    feed-forward half. Same constructor signature, parameter names and ``forward(tokens, padding_mask, attention_mask)``
+    -> tokens. For bf16 GPU tokens of width 128 / 256 under ``torch.no_grad()`` the block runs on the fused kernels: the
+    gate layer's output comes from the projection kernel over the valid rows, and its sigmoid, the gated update, both
+    residual adds, ``ffn_norm`` and the feed-forward are one kernel (``taac_attn_out_gate_ffn_fwd``); padded rows are
+    never touched. Other inputs (and tensors that take a gradient) run layer by layer."""
+
+    def __init__(self, d_model: int, num_heads: int, hidden_mult: int, dropout: float = 0.0, *, use_rope: bool,
+                 rope_base: float, token_layout: str = "front") -> None:
+        super().__init__(d_model, num_heads, hidden_mult, dropout, qk_norm=True, token_layout=token_layout)
+        self.attention = BFTSAttention(d_model, num_heads, dropout, use_rope=use_rope, rope_base=rope_base)
+        self.nlir_gate = nn.Linear(d_model, d_model)
+
+    def forward(self, tokens: torch.Tensor, padding_mask: torch.Tensor,
+                attention_mask: torch.Tensor | StructuredAttentionMask | None, *, key_lengths: torch.Tensor | None = None,
+                inplace: bool = False) -> torch.Tensor:
+        if self._fused_route(tokens) and self.ffn.gate_first:
+            return self._forward_fused(tokens, padding_mask, attention_mask, key_lengths, False, inplace)[0]
+        keep = (~padding_mask).unsqueeze(-1)
+        attention_input = self.attn_norm(tokens)
+        attention_update = self.attention(attention_input, attention_mask, key_lengths=key_lengths)
+        gate_input = attention_input if attention_input.dtype == torch.bfloat16 else attention_input.to(torch.bfloat16)
+        gate = torch.sigmoid(_dense(self.nlir_gate, gate_input)).to(attention_update.dtype)
+        tokens = tokens + gate * attention_update * keep.to(attention_update.dtype)
+        ffn_update = self.ffn(self.ffn_norm(tokens))
+        return tokens + ffn_update * keep.to(ffn_update.dtype)
 
 
 def run_interaction_blocks(blocks, tokens: torch.Tensor, padding_mask: torch.Tensor,

@@ -317,6 +317,104 @@ def test_interaction_block_float64_loop_with_scattered_padding_and_role_mask():
     assert (a - b).abs().max().item() > 1e-3
 
 
+def test_tokenformer_block_float64_loop_with_gate_and_padding():
+    """``oracle.tokenformer_block`` (experiments/tokenformer/model.py:203-215) against a per-token float64 loop that
+    shares none of its code: query / key RMSNorm over the model width, softmax over the keys the mask shows, the update
+    multiplied by ``sigmoid(nlir_gate(attn_norm(x)))`` and by ``~padding``, then the gated-linear feed-forward. Special
+    cases: a zero gate layer halves the attention update exactly; padded rows pass through."""
+    g = torch.Generator().manual_seed(23)
+    batch, tokens, d, heads, f, eps = 2, 5, 8, 2, 12, 1e-6
+    dh = d // heads
+    x = torch.randn(batch, tokens, d, generator=g, dtype=torch.float64)
+    padding = torch.tensor([[False, False, True, False, True], [False, True, False, False, False]])
+    mask = (torch.rand(batch, 1, tokens, tokens, generator=g) > 0.3) | torch.eye(tokens, dtype=torch.bool)
+    mask = mask & ~padding[:, None, None, :] | torch.eye(tokens, dtype=torch.bool)
+    rnd = lambda *shape, scale=1.0: scale * torch.randn(*shape, generator=g, dtype=torch.float64)  # noqa: E731
+    w = {"attn_norm.weight": 1 + rnd(d, scale=0.2), "qkv.weight": rnd(3 * d, d, scale=d ** -0.5), "qkv.bias": rnd(3 * d, scale=0.1),
+         "query_norm.weight": 1 + rnd(d, scale=0.2), "key_norm.weight": 1 + rnd(d, scale=0.2),
+         "out.weight": rnd(d, d, scale=d ** -0.5), "out.bias": rnd(d, scale=0.1),
+         "nlir_gate.weight": rnd(d, d, scale=d ** -0.5), "nlir_gate.bias": rnd(d, scale=0.3),
+         "ffn_norm.weight": 1 + rnd(d, scale=0.2), "up.weight": rnd(2 * f, d, scale=d ** -0.5), "up.bias": rnd(2 * f, scale=0.1),
+         "down.weight": rnd(d, f, scale=f ** -0.5), "down.bias": rnd(d, scale=0.1)}
+
+    def rms(row, weight):
+        scale = 1.0 / math.sqrt(sum(float(v) ** 2 for v in row) / len(row) + eps)
+        return [float(v) * scale * float(weight[i]) for i, v in enumerate(row)]
+
+    def dense(row, weight, bias):
+        return [sum(float(weight[o, c]) * row[c] for c in range(len(row))) + float(bias[o]) for o in range(weight.shape[0])]
+
+    def loop(weights):
+        out = torch.zeros_like(x)
+        for b in range(batch):
+            h = [rms(x[b, t].tolist(), weights["attn_norm.weight"]) for t in range(tokens)]
+            proj = [dense(h[t], weights["qkv.weight"], weights["qkv.bias"]) for t in range(tokens)]
+            q = [rms(p[:d], weights["query_norm.weight"]) for p in proj]
+            k = [rms(p[d:2 * d], weights["key_norm.weight"]) for p in proj]
+            v = [p[2 * d:] for p in proj]
+            for t in range(tokens):
+                attended = []
+                for hd in range(heads):
+                    cols = range(hd * dh, (hd + 1) * dh)
+                    seen = [j for j in range(tokens) if bool(mask[b, 0, t, j])]
+                    scores = [sum(q[t][c] * k[j][c] for c in cols) / math.sqrt(dh) for j in seen]
+                    top = max(scores)
+                    weights_ = [math.exp(sc - top) for sc in scores]
+                    total = sum(weights_)
+                    attended += [sum(wt * v[j][c] for wt, j in zip(weights_, seen)) / total for c in cols]
+                keep = 0.0 if bool(padding[b, t]) else 1.0
+                update = dense(attended, weights["out.weight"], weights["out.bias"])
+                z = dense(h[t], weights["nlir_gate.weight"], weights["nlir_gate.bias"])
+                x1 = [float(x[b, t, c]) + keep * update[c] / (1.0 + math.exp(-z[c])) for c in range(d)]
+                up = dense(rms(x1, weights["ffn_norm.weight"]), weights["up.weight"], weights["up.bias"])
+                hidden = [up[j] / (1.0 + math.exp(-up[j])) * up[f + j] for j in range(f)]
+                down = dense(hidden, weights["down.weight"], weights["down.bias"])
+                out[b, t] = torch.tensor([x1[c] + keep * down[c] for c in range(d)], dtype=torch.float64)
+        return out
+
+    got = oracle.tokenformer_block(x, padding, mask, w, num_heads=heads, eps=eps)
+    torch.testing.assert_close(got, loop(w), rtol=1e-9, atol=1e-9)
+    assert torch.equal(got[padding], x[padding])
+    # a zero gate layer: sigmoid(0) = 1/2 scales the attention update, i.e. the block with the out projection halved
+    zero_gate = dict(w, **{"nlir_gate.weight": torch.zeros(d, d, dtype=torch.float64), "nlir_gate.bias": torch.zeros(d, dtype=torch.float64)})
+    halved = {k: v for k, v in w.items() if not k.startswith("nlir_gate")}
+    halved["out.weight"], halved["out.bias"] = 0.5 * w["out.weight"], 0.5 * w["out.bias"]
+    want, _ = oracle.interaction_block(x, padding, mask, halved, num_heads=heads, eps=eps)
+    torch.testing.assert_close(oracle.tokenformer_block(x, padding, mask, zero_gate, num_heads=heads, eps=eps), want,
+                               rtol=1e-12, atol=1e-12)
+    # the gate matters
+    assert (got - oracle.tokenformer_block(x, padding, mask, zero_gate, num_heads=heads, eps=eps)).abs().max().item() > 1e-3
+
+
+def test_silu_mlp_and_mixed_feed_forward_float64_loops():
+    """OneTrans' feed-forward (experiments/onetrans/model.py:33-44) and its mixed form (:80-94) against per-element loops:
+    Linear -> x / (1 + exp(-x)) -> Linear; the token at ``seq_token_count + i`` goes through the i-th token-specific
+    feed-forward instead of the shared one, positions beyond the sequence are skipped."""
+    g = torch.Generator().manual_seed(29)
+    d, f, batch, tokens = 4, 6, 2, 5
+    rnd = lambda *shape: torch.randn(*shape, generator=g, dtype=torch.float64)  # noqa: E731
+    make = lambda: (rnd(f, d), rnd(f), rnd(d, f), rnd(d))  # noqa: E731
+    shared, specific = make(), [make(), make(), make()]
+    x = rnd(batch, tokens, d)
+
+    def mlp(row, weights):
+        w1, b1, w2, b2 = weights
+        hidden = [sum(float(w1[j, c]) * row[c] for c in range(d)) + float(b1[j]) for j in range(f)]
+        hidden = [v / (1.0 + math.exp(-v)) for v in hidden]
+        return [sum(float(w2[o, j]) * hidden[j] for j in range(f)) + float(b2[o]) for o in range(d)]
+
+    want = torch.tensor([[mlp(x[b, t].tolist(), shared) for t in range(tokens)] for b in range(batch)], dtype=torch.float64)
+    torch.testing.assert_close(oracle.silu_mlp(x, *shared), want, rtol=1e-12, atol=1e-12)
+    seq_token_count = 3  # positions 3, 4 are token-specific; the third specific layer falls beyond the sequence
+    mixed = want.clone()
+    for i in range(2):
+        for b in range(batch):
+            mixed[b, seq_token_count + i] = torch.tensor(mlp(x[b, seq_token_count + i].tolist(), specific[i]), dtype=torch.float64)
+    got = oracle.mixed_feed_forward(x, seq_token_count, shared, specific)
+    torch.testing.assert_close(got, mixed, rtol=1e-12, atol=1e-12)
+    assert torch.equal(got[:, :seq_token_count], oracle.silu_mlp(x, *shared)[:, :seq_token_count])
+
+
 # ---- FP8 (no reference counterpart; the rounding itself is pinned, the layer is defined by its formula) ----------------
 
 
