@@ -402,6 +402,21 @@ int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_weight, flo
                         int gate_first, const int32_t* rows, const int32_t* n_rows, void* stream);
 
 /*
+ * Plain SiLU feed-forward (OneTrans' FeedForward), one kernel with the hidden state in registers:
+ *   out = residual + fc2( silu( fc1( norm_weight ? rmsnorm(x, norm_weight, eps) : x ) ) )
+ * fc1: [F, D] with bias b1 [F] or NULL, fc2: [D, F] with bias b2 [D] or NULL, both handed over as the blob written by
+ * taac_silu_mlp_pack_weights (taac_silu_mlp_packed_bytes bytes; -1: unsupported shape). x, residual (or NULL), out,
+ * row strides, rows / n_rows as in taac_swiglu_ffn_fwd. D must be 128 or 256, F a multiple of 32.
+ * Replaces: FeedForward.forward in eval mode (experiments/onetrans/model.py:33-44: Linear -> SiLU -> Dropout ->
+ * Linear), with the ffn_norm and the residual add of OneTransBlock.forward (:107) when they are passed.
+ */
+int64_t taac_silu_mlp_packed_bytes(int32_t D, int32_t F);
+int taac_silu_mlp_pack_weights(const void* w1, const void* w2, void* packed, int32_t D, int32_t F, void* stream);
+int taac_silu_mlp_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* b1, const void* b2,
+                      const void* packed_weights, const void* residual, int64_t ldr, void* out, int64_t ldo, int64_t M,
+                      int32_t D, int32_t F, const int32_t* rows, const int32_t* n_rows, void* stream);
+
+/*
  * Attention output projection + residual and the feed-forward half of a block in one kernel:
  *   x1  = residual + (attn @ w_out^T + out_bias)
  *   out = x1 + down( silu(g) * u ) + b_down,   g, u = chunk2( up( norm_weight ? rmsnorm(x1, norm_weight, eps) : x1 ) )

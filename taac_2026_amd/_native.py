@@ -187,6 +187,13 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
          c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p],
     ),
+    "taac_silu_mlp_packed_bytes": (c_int64, [c_int32, c_int32]),
+    "taac_silu_mlp_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
+    "taac_silu_mlp_fwd": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
+         c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p],
+    ),
     "taac_attn_out_gate_ffn_fwd": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_float, c_void_p,

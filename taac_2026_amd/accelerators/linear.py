@@ -594,6 +594,78 @@ def swiglu_ffn(
     return out.reshape(shape)
 
 
+def pack_mlp_weights(fc1_weight: torch.Tensor, fc2_weight: torch.Tensor) -> torch.Tensor:
+    """Fragment-ordered blob of ``(fc1_weight [F, D], fc2_weight [D, F])`` for :func:`silu_mlp` (uint8 tensor)."""
+    library = _native.load_library()
+    d_model, hidden = fc2_weight.shape
+    nbytes = library.taac_silu_mlp_packed_bytes(d_model, hidden)
+    if nbytes < 0:
+        raise RuntimeError(f"pack_mlp_weights: unsupported shape D={d_model}, F={hidden}")
+    fc1_weight, fc2_weight = fc1_weight.contiguous(), fc2_weight.contiguous()
+    packed = torch.empty(nbytes, dtype=torch.uint8, device=fc1_weight.device)
+    status = library.taac_silu_mlp_pack_weights(fc1_weight.data_ptr(), fc2_weight.data_ptr(), packed.data_ptr(), d_model,
+                                                hidden, _native.current_stream(fc1_weight.device))
+    _native.check(status, "pack_mlp_weights")
+    return packed
+
+
+def silu_mlp(
+    x: torch.Tensor,
+    fc1_weight: torch.Tensor,
+    fc1_bias: torch.Tensor | None,
+    fc2_weight: torch.Tensor,
+    fc2_bias: torch.Tensor | None,
+    *,
+    residual: torch.Tensor | None = None,
+    norm_weight: torch.Tensor | None = None,
+    eps: float = 1e-6,
+    token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """``residual + fc2(silu(fc1(rmsnorm(x))))`` (norm and residual optional): OneTrans' feed-forward
+    (experiments/onetrans/model.py:33-44) in eval mode. For model widths 128 / 256 with a hidden size that is a multiple
+    of 32, under ``torch.no_grad()``, the whole expression is ONE kernel (``taac_silu_mlp_fwd``: the hidden state stays in
+    registers); other shapes, and tensors that take a gradient, run the two dense layers as kernels of their own with
+    the activation between them. ``token_rows`` / ``out`` (fused route only) as in :func:`swiglu_ffn`."""
+    name = "hip silu_mlp"
+    tensors = (x, fc1_weight, fc1_bias, fc2_weight, fc2_bias, residual, norm_weight)
+    require_cuda_tensors(name, *tensors)
+    hidden, d_model = fc1_weight.shape
+    if fc2_weight.shape != (d_model, hidden) or x.shape[-1] != d_model:
+        raise ValueError("silu_mlp expects fc1_weight [F, D], fc2_weight [D, F] and input rows of D features")
+    if residual is not None and residual.shape != x.shape:
+        raise ValueError("silu_mlp residual must have the shape of the input")
+    needs_grad = _needs_grad(*tensors)
+    if needs_grad or not (_fused_width(d_model) and hidden % 32 == 0):
+        if token_rows is not None or out is not None:
+            raise RuntimeError("silu_mlp: token_rows / out belong to the fused inference route (width 128 / 256, hidden "
+                               "size a multiple of 32, no gradient)")
+        h = x
+        if norm_weight is not None:
+            from taac_2026_amd.accelerators.normalization import rms_norm
+
+            h = rms_norm(x, norm_weight, eps)
+        return linear(torch.nn.functional.silu(linear(h, fc1_weight, fc1_bias)), fc2_weight, fc2_bias, residual=residual)
+    _check_bf16(name, *tensors)
+    rows, shape = _as_rows(x)
+    packed = _packed_cache.get((fc1_weight, fc2_weight), lambda: pack_mlp_weights(fc1_weight, fc2_weight), variant=2)
+    res_rows = None
+    if residual is not None:
+        res_rows = residual.reshape(-1, d_model)
+        if res_rows.stride(-1) != 1 or res_rows.stride(0) % 8 != 0:
+            res_rows = res_rows.contiguous()
+    index, count = _token_rows(name, token_rows, rows)
+    out = _output_rows(name, out, (rows.shape[0], d_model), index is not None, x)
+    library = _native.load_library()
+    status = library.taac_silu_mlp_fwd(
+        rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), _native.ptr(fc1_bias), _native.ptr(fc2_bias),
+        packed.data_ptr(), _native.ptr(res_rows), res_rows.stride(0) if res_rows is not None else d_model, out.data_ptr(),
+        d_model, rows.shape[0], d_model, hidden, _native.ptr(index), _native.ptr(count), _native.current_stream(x.device),
+    )
+    _native.check(status, "silu_mlp")
+    return out.reshape(shape)
+
+
 def attention_out_ffn(
     attn: torch.Tensor,
     out_weight: torch.Tensor,
@@ -1063,6 +1135,8 @@ __all__ = [
     "swiglu_backward",
     "norm_linear",
     "pack_ffn_weights",
+    "pack_mlp_weights",
+    "silu_mlp",
     "norm_linear_fp8",
     "pack_ffn_weights_fp8",
     "swiglu_ffn_fp8",

@@ -105,6 +105,27 @@ __global__ void ffn_pack_kernel(const bf16_t* __restrict__ w_up, const bf16_t* _
   if (gid < total) ffn_pack_piece(w_up, w_down, packed, D, F, gate_first, gid);
 }
 
+// Plain SiLU MLP blob (fc1 [F, D], fc2 [D, F]): chunk c (32 hidden units) holds KS fc1 fragments (k-step r; row slots
+// 0..15 the chunk's first 16 units, 16..31 its second 16, each in the slot order of up_unit_of_slot) and then 2 * MB fc2
+// fragments (k-step (r - KS) / MB of the chunk, row block (r - KS) % MB).
+__global__ void mlp_pack_kernel(const bf16_t* __restrict__ w1, const bf16_t* __restrict__ w2, bf16x8* __restrict__ packed,
+                                int D, int F) {
+  const int64_t total = static_cast<int64_t>(2) * D * F / 8;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (gid >= total) return;
+  const int KS = D / 16, MB = D / 32, CFRAG = KS + 2 * MB;
+  const int lane = static_cast<int>(gid % 64);
+  const int r = static_cast<int>((gid / 64) % CFRAG);
+  const int64_t unit0 = gid / 64 / CFRAG * 32;
+  const int l32 = lane % 32, hh = lane / 32;
+  const bf16_t* src;
+  if (r < KS)
+    src = w1 + (unit0 + 16 * (l32 / 16) + up_unit_of_slot(l32 & 15)) * D + r * 16 + hh * 8;
+  else
+    src = w2 + static_cast<int64_t>(((r - KS) % MB) * 32 + l32) * F + unit0 + ((r - KS) / MB) * 16 + hh * 8;
+  packed[gid] = *reinterpret_cast<const bf16x8*>(src);
+}
+
 // Linear blob: chunk c (64 output features) holds fragments (row block rb, k-step ks) at index rb * KS + ks.
 __device__ __forceinline__ void linear_pack_piece(const bf16_t* __restrict__ w, bf16x8* __restrict__ packed, int K,
                                                   int64_t gid) {
@@ -233,6 +254,13 @@ __device__ __forceinline__ void stage_up_bias(const bf16_t* b_up, bf16_t* dst, i
     dst[i] = b_up != nullptr ? b_up[src] : static_cast<bf16_t>(0.f);
   }
 }
+// The same for the plain MLP: a chunk's fragment has 32 hidden units, slots 0..15 the first 16, slots 16..31 the others.
+__device__ __forceinline__ void stage_mlp_bias(const bf16_t* b1, bf16_t* dst, int F, int tid, int nthreads) {
+  for (int i = tid; i < F; i += nthreads) {
+    const int m = i % 32;
+    dst[i] = b1 != nullptr ? b1[(i / 32) * 32 + 16 * (m / 16) + up_unit_of_slot(m % 16)] : static_cast<bf16_t>(0.f);
+  }
+}
 
 // Bias values of a 64-feature chunk in accumulator order: piece rb*4 + jq holds features rb*32 + jq*8 + hh*4 .. +3.
 __device__ __forceinline__ void read_chunk_bias(const bf16_t* bias_lds, int hh, bf16x4 (&bv)[8]) {
@@ -342,13 +370,17 @@ __device__ __forceinline__ void load_residual(const bf16_t* residual, int64_t ld
 // it arrives as a tensor). Its pieces of a chunk are requested behind the chunk's MFMAs, into the registers the weight
 // fragments have left, so the variant takes no registers of its own.
 // ------------------------------------------------------------------------------------------------------------------
-template <int D, int TT, int NWAVES, int CPB, bool DEFER, bool OUTP, bool GATE = false>
+template <int D, int TT, int NWAVES, int CPB, bool DEFER, bool OUTP, bool GATE = false, bool GLU = true>
 __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_kernel(const TsParams p) {
   static_assert(!GATE || OUTP, "the gate belongs to the projection in front");
   constexpr int kTokPerWg = NWAVES * 32 * TT;  // TT token tiles of 32 per wavefront
   constexpr int KS = D / 16;             // k-steps of the up projection = up fragments per chunk
-  constexpr int MB = D / 32;             // 32-feature row blocks of the down projection = down fragments per chunk
-  constexpr int CFRAG = KS + MB;         // fragments per chunk
+  constexpr int MB = D / 32;             // 32-feature row blocks of the down projection
+  // GLU: a chunk is 16 hidden units (16 gated rows + 16 partner rows) and one k-step of the down projection. Plain MLP
+  // (!GLU: down(silu(up(x)))): all 32 rows of a chunk's fragment are hidden units, whose activations fill two k-steps.
+  constexpr int DK = GLU ? 1 : 2;        // k-steps of the down projection per chunk
+  constexpr int NDOWN = DK * MB;         // down fragments per chunk
+  constexpr int CFRAG = KS + NDOWN;      // fragments per chunk
   constexpr int NFRAG = CPB * CFRAG;     // fragments per barrier step
   constexpr int FPW = NFRAG / NWAVES;    // fragments staged per wavefront
   static_assert(NFRAG % NWAVES == 0, "fragments must divide over the wavefronts");
@@ -387,7 +419,8 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
   const bool active = wave * (32 * TT) < wg_ntok;
   const int64_t tok0 = wg_tok0 + wave * (32 * TT);
   const int F = p.F;
-  const int nsteps = F / (kHU * CPB);
+  const int UPB = GLU ? 2 * F : F;  // entries of the staged first-layer bias
+  const int nsteps = F / (kHU * DK * CPB);
 
   // Source address of a staged fragment = wavefront-uniform base (scalar registers) + a 32-bit per-lane byte offset.
   //   packed:   blob + (step * NFRAG + f) KB + 16 * lane
@@ -408,6 +441,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
       for (int i = 0; i < FPW; ++i) lds_dma16_offset(src + i * kFrag, lane_off, base + i * kFrag);
       return;
     }
+    if constexpr (!GLU) return;  // the plain MLP takes packed weights only (checked on the host)
     const int s32 = ln & 31, shh = ln >> 5;
     const uint32_t up_lane_off =
         static_cast<uint32_t>(((((s32 < 16) == (p.gate_first != 0) ? 0 : F) + up_unit_of_slot(s32 & 15)) * D + shh * 8) * 2);
@@ -449,10 +483,13 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 #pragma unroll
     for (int t = 0; t < TT; ++t) hrow_index[t] = token_row(p, count, tok0 + t * 32 + l32);
   }
-  stage_up_bias(p.b1, bias_lds, F, p.gate_first, tid, NWAVES * kWave);
-  stage_bias(p.b2, bias_lds + 2 * F, D, tid, NWAVES * kWave);
-  if (p.norm_w != nullptr) stage_bias(p.norm_w, bias_lds + 2 * F + D, D, tid, NWAVES * kWave);
-  if constexpr (OUTP) stage_bias(p.b0, bias_lds + 2 * F + 2 * D, D, tid, NWAVES * kWave);
+  if constexpr (GLU)
+    stage_up_bias(p.b1, bias_lds, F, p.gate_first, tid, NWAVES * kWave);
+  else
+    stage_mlp_bias(p.b1, bias_lds, F, tid, NWAVES * kWave);
+  stage_bias(p.b2, bias_lds + UPB, D, tid, NWAVES * kWave);
+  if (p.norm_w != nullptr) stage_bias(p.norm_w, bias_lds + UPB + D, D, tid, NWAVES * kWave);
+  if constexpr (OUTP) stage_bias(p.b0, bias_lds + UPB + 2 * D, D, tid, NWAVES * kWave);
 
   f32x16 oacc[TT][MB];
 #pragma unroll
@@ -464,7 +501,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  if (!OUTP && active && p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + 2 * F + D, hh, xf);
+  if (!OUTP && active && p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + UPB + D, hh, xf);
 
   // One barrier step = CPB chunks = NFRAG fragments, consumed in their LDS order: per chunk KS up fragments, then MB
   // down fragments. Fragment reads run P fragments ahead of their MFMAs through a ring of P registers sets; the two
@@ -483,7 +520,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
     static_assert(DEFER, "the projection chunks use weight buffers 1 and 2");
     constexpr int NCH = D / kNC;  // 64-feature chunks of the projection
     constexpr int CF = 2 * KS;    // fragments of a chunk: (row block rb, k-step ks) at rb * KS + ks
-    const bf16_t* b0_lds = bias_lds + 2 * F + 2 * D;
+    const bf16_t* b0_lds = bias_lds + UPB + 2 * D;
     float ss[TT];
     const bf16_t* hrow[TT];
     [[maybe_unused]] const bf16_t* grow[TT];
@@ -557,7 +594,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
       // rmsnorm(x1) as B-operand fragments. k-step ks covers features 16*ks .. +15 = the 8-feature groups jq = 2*(ks%2)
       // and jq + 1 of row block ks / 2; the lower half-wavefront needs all of the first group, the upper half all of
       // the second, and each half holds 4 features of both.
-      const bf16_t* nw_lds = bias_lds + 2 * F + D;
+      const bf16_t* nw_lds = bias_lds + UPB + D;
 #pragma unroll
       for (int t = 0; t < TT; ++t) {
         const float scale = p.norm_w != nullptr ? rsqrtf(half_wave_pair_sum(ss[t]) * (1.0f / D) + p.eps) : 1.0f;
@@ -596,11 +633,17 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
   // chunk (MFMA j of the old chunk, then two gated values of the new one), so the matrix unit has work while the
   // wavefront evaluates the activation. hb is the gated hidden state whose down projection is pending; before the
   // first chunk it is zero and the (finite) fragments it is multiplied with do not matter.
-  bf16x8 hb[TT];
+  bf16x8 hb[TT][DK];
 #pragma unroll
   for (int t = 0; t < TT; ++t)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) hb[t][e] = static_cast<bf16_t>(0.f);
+    for (int k = 0; k < DK; ++k)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) hb[t][k][e] = static_cast<bf16_t>(0.f);
+  // Activation of accumulator register e of a chunk (e < 8 * DK): the B-operand element it becomes.
+  auto activate = [](const f32x16& gu, int e) -> bf16_t {
+    return static_cast<bf16_t>(GLU ? silu_f(gu[e]) * gu[8 + e] : silu_f(gu[e]));
+  };
   int buf = 0;
   uint32_t wb_prev = smem_off;
   for (int step = 0; step < nsteps; ++step) {
@@ -613,7 +656,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
     bf16x8 ring[P];
     uint32_t brow[CPB];  // bias of this lane's fragment row, one per chunk, zero-extended bf16
     f32x16 gu[TT];
-    bf16x8 hb_new[TT];
+    bf16x8 hb_new[TT][DK];
     // Fragment i of the step's stream: chunk q = i / CFRAG; r < KS is up fragment r of chunk q, r >= KS is down
     // fragment r - KS of chunk q (of the chunk before q with DEFER, which for q = 0 lives in the previous buffer).
     auto read_stream = [&](auto ic, bf16x8& dst) {
@@ -657,9 +700,10 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
         }
       } else {
         // ---- down projection: O^T[feature, token] += W_down[feature, chunk] H^T --------------------------------------
+        constexpr int jd = r - KS;  // k-step jd / MB of the chunk, row block jd % MB
 #pragma unroll
         for (int t = 0; t < TT; ++t)
-          oacc[t][r - KS] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % P], hb[t], oacc[t][r - KS], 0, 0, 0);
+          oacc[t][jd % MB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % P], hb[t][jd / MB], oacc[t][jd % MB], 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (i + P < NFRAG) {
@@ -671,21 +715,22 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 #pragma unroll
         for (int t = 0; t < TT; ++t)
 #pragma unroll
-          for (int e = 0; e < 8; ++e) hb[t][e] = static_cast<bf16_t>(silu_f(gu[t][e]) * gu[t][8 + e]);
+          for (int e = 0; e < 8 * DK; ++e) hb[t][e / 8][e % 8] = activate(gu[t], e);
         __builtin_amdgcn_sched_barrier(0);
       }
       if constexpr (DEFER && r >= KS) {
-        constexpr int j = r - KS;  // down MFMA just issued; the 4 pairs of gated values are spread over the MB MFMAs
+        constexpr int j = r - KS;  // down MFMA just issued; the 4 * DK pairs of activations are spread over the NDOWN MFMAs
 #pragma unroll
         for (int t = 0; t < TT; ++t)
 #pragma unroll
-          for (int g = (j * 4) / MB; g < ((j + 1) * 4) / MB; ++g)
+          for (int g = (j * 4 * DK) / NDOWN; g < ((j + 1) * 4 * DK) / NDOWN; ++g)
 #pragma unroll
-            for (int e = 2 * g; e < 2 * g + 2; ++e)
-              hb_new[t][e] = static_cast<bf16_t>(silu_f(gu[t][e]) * gu[t][8 + e]);
+            for (int e = 2 * g; e < 2 * g + 2; ++e) hb_new[t][e / 8][e % 8] = activate(gu[t], e);
         if constexpr (r == CFRAG - 1) {
 #pragma unroll
-          for (int t = 0; t < TT; ++t) hb[t] = hb_new[t];
+          for (int t = 0; t < TT; ++t)
+#pragma unroll
+            for (int k = 0; k < DK; ++k) hb[t][k] = hb_new[t][k];
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -700,17 +745,17 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
   if constexpr (DEFER) {
     // The down projection of the last chunk is still pending; its fragments are in the last step's buffer.
     if (active) {
-    bf16x8 tail[MB];
-    static_for<MB>([&](auto ic) {
+    bf16x8 tail[NDOWN];
+    static_for<NDOWN>([&](auto ic) {
       constexpr int j = decltype(ic)::value;
       lds_read_frag<((CPB - 1) * CFRAG + KS + j) * kFrag>(tail[j], wb_prev);
     });
-    static_for<MB>([&](auto ic) {
+    static_for<NDOWN>([&](auto ic) {
       constexpr int j = decltype(ic)::value;
-      lds_wait_frag<MB - 1 - j>(tail[j]);
+      lds_wait_frag<NDOWN - 1 - j>(tail[j]);
 #pragma unroll
       for (int t = 0; t < TT; ++t)
-        oacc[t][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tail[j], hb[t], oacc[t][j], 0, 0, 0);
+        oacc[t][j % MB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tail[j], hb[t][j / MB], oacc[t][j % MB], 0, 0, 0);
     });
     }
     __syncthreads();  // the epilogue tiles below overwrite the weight buffers
@@ -719,7 +764,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
   // ---- epilogue: + b_down, round, transpose through the wavefront's LDS tile, + residual, coalesced bf16 stores ----
   if (!active) return;  // no barrier below
   uint8_t* tile = smem + wave * kStageWave;  // the weight buffers are free after the last barrier
-  const bf16_t* bdown_lds = bias_lds + 2 * F;
+  const bf16_t* bdown_lds = bias_lds + UPB;
 #pragma unroll
   for (int t = 0; t < TT; ++t) {
     const int64_t tok_base = tok0 + t * 32;
@@ -1189,8 +1234,11 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
               const void* norm_weight, float eps, const void* w_up, const void* b_up, const void* w_down,
               const void* b_down, const void* packed_weights, const void* residual, int64_t ldr, void* out, int64_t ldo,
               int64_t M, int32_t D, int32_t F, int gate_first, const int32_t* rows, const int32_t* n_rows,
-              const int32_t* x_rows, void* stream, const void* update_gate = nullptr, int64_t ldg = 0) {
+              const int32_t* x_rows, void* stream, const void* update_gate = nullptr, int64_t ldg = 0,
+              bool glu = true) {
   const bool with_proj = out_packed != nullptr;
+  if (!glu && (with_proj || !packed_weights))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: the plain MLP takes packed weights and no projection in front", name);
   if (update_gate && !with_proj)
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: an update gate needs the projection in front", name);
   if (update_gate && (ldg < D || ldg % 8 || !ptr_ok(update_gate, 15)))
@@ -1216,9 +1264,9 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
       !ptr_ok(out_packed, 15) || !ptr_ok(out_bias, 15))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
   const int KS = D / 16, MB = D / 32;
-  const size_t bias_bytes = static_cast<size_t>(2 * F + (with_proj ? 3 : 2) * D) * 2;
-  const size_t buffer_bytes = static_cast<size_t>(kCPB * (KS + MB)) * kFrag;
-  if ((with_proj ? 3 : 2) * buffer_bytes + bias_bytes > kMaxLdsBytes)
+  const size_t bias_bytes = static_cast<size_t>((glu ? 2 : 1) * F + (with_proj ? 3 : 2) * D) * 2;
+  const size_t buffer_bytes = glu ? static_cast<size_t>(kCPB * (KS + MB)) * kFrag : static_cast<size_t>(KS + 2 * MB) * kFrag;
+  if ((with_proj || !glu ? 3 : 2) * buffer_bytes + bias_bytes > kMaxLdsBytes)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: F=%d does not fit the LDS (limit %d bytes)", name, F, kMaxLdsBytes);
   TsParams p{};
   p.x = static_cast<const bf16_t*>(x);
@@ -1251,6 +1299,14 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
 #define TAAC_FFN_LAUNCH(DD, TT, NW, CPB, DEFER, ...)                                                         \
   return launch_ts(swiglu_ffn_kernel<DD, TT, NW, CPB, DEFER, __VA_ARGS__>, p, NW * kWave, NW * 32 * TT,      \
                    static_cast<size_t>((DEFER ? 3 : 2) * CPB * (KS + MB)) * kFrag + bias_bytes, s, name)
+  if (!glu) {  // one 32-unit chunk per barrier step, deferred down projection: three buffers of KS + 2 * MB fragments
+#define TAAC_MLP_LAUNCH(DD)                                                                              \
+  return launch_ts(swiglu_ffn_kernel<DD, 1, 8, 1, true, false, false, false>, p, 8 * kWave, 8 * 32,      \
+                   3 * buffer_bytes + bias_bytes, s, name)
+    if (D == 256) TAAC_MLP_LAUNCH(256);
+    TAAC_MLP_LAUNCH(128);
+#undef TAAC_MLP_LAUNCH
+  }
   if (with_proj && update_gate) {
     if (D == 256) TAAC_FFN_LAUNCH(256, 1, 8, 2, true, true, true);
     TAAC_FFN_LAUNCH(128, 1, 8, 2, true, true, true);
@@ -1295,6 +1351,36 @@ extern "C" int taac_attn_out_ffn_fwd(const void* attn, int64_t ld_attn, const vo
     return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: both weight sets must be packed", name);
   return taac::ffn_entry(name, attn, ld_attn, out_bias, packed_out_weights, norm_weight, eps, nullptr, b_up, nullptr,
                          b_down, packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, attn_rows, stream);
+}
+
+extern "C" int64_t taac_silu_mlp_packed_bytes(int32_t D, int32_t F) {
+  if ((D != 128 && D != 256) || F <= 0 || F % 32 != 0) return -1;
+  return static_cast<int64_t>(2) * D * F * 2;
+}
+
+extern "C" int taac_silu_mlp_pack_weights(const void* w1, const void* w2, void* packed, int32_t D, int32_t F,
+                                          void* stream) {
+  using namespace taac;
+  const char* name = "taac_silu_mlp_pack_weights";
+  if (taac_silu_mlp_packed_bytes(D, F) < 0)
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: D must be 128 or 256 and F a positive multiple of 32", name);
+  if (!w1 || !w2 || !packed) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
+  if (!ptr_ok(w1, 15) || !ptr_ok(w2, 15) || !ptr_ok(packed, 15))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: pointers must be 16-byte aligned", name);
+  const int64_t pieces = static_cast<int64_t>(2) * D * F / 8;
+  hipLaunchKernelGGL(mlp_pack_kernel, dim3(static_cast<uint32_t>((pieces + 255) / 256)), dim3(256), 0, as_stream(stream),
+                     static_cast<const bf16_t*>(w1), static_cast<const bf16_t*>(w2), static_cast<bf16x8*>(packed), D, F);
+  return check_launch(name);
+}
+
+extern "C" int taac_silu_mlp_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* b1,
+                                 const void* b2, const void* packed_weights, const void* residual, int64_t ldr, void* out,
+                                 int64_t ldo, int64_t M, int32_t D, int32_t F, const int32_t* rows, const int32_t* n_rows,
+                                 void* stream) {
+  const char* name = "taac_silu_mlp_fwd";
+  if (!packed_weights) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: the weights must be packed", name);
+  return taac::ffn_entry(name, x, ldx, nullptr, nullptr, norm_weight, eps, nullptr, b1, nullptr, b2, packed_weights,
+                         residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, nullptr, stream, nullptr, 0, false);
 }
 
 extern "C" int taac_attn_out_gate_ffn_fwd(const void* attn, int64_t ld_attn, const void* out_bias,

@@ -2,6 +2,8 @@
 
 from taac_2026_amd.modeling.backbone import (
     BFTSAttention,
+    FeedForward,
+    MixedFeedForward,
     PCVRBackbone,
     SwiGLUFeedForward,
     TokenFormerBlock,
@@ -35,6 +37,8 @@ from taac_2026_amd.modeling.sequence import (
 
 __all__ = [
     "BFTSAttention",
+    "FeedForward",
+    "MixedFeedForward",
     "CandidateClsPooler",
     "CandidateReadoutHead",
     "LayerNorm",

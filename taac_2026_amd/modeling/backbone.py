@@ -21,8 +21,8 @@ import torch.nn as nn
 
 from taac_2026_amd import _native
 from taac_2026_amd.accelerators.attention import StructuredAttentionMask, front_structured_mask, qk_norm_rope, rope_table
-from taac_2026_amd.accelerators.linear import (attention_out_ffn, front_rows, norm_linear, qkv_projection, swiglu_ffn,
-                                               swiglu_ffn_dropout, valid_rows)
+from taac_2026_amd.accelerators.linear import (attention_out_ffn, front_rows, norm_linear, qkv_projection, silu_mlp,
+                                               swiglu_ffn, swiglu_ffn_dropout, valid_rows)
 from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference
 from taac_2026_amd.modeling.block_training import run_training_block, training_route_applies
 from taac_2026_amd.modeling.normalization import RMSNorm
@@ -63,6 +63,73 @@ class SwiGLUFeedForward(nn.Module):
         out = swiglu_ffn(x, _bf16(self.up.weight), _bf16(self.up.bias), _bf16(self.down.weight), _bf16(self.down.bias),
                          residual=_bf16(residual), gate_first=self.gate_first)
         return out if out.dtype == output_dtype else out.to(output_dtype)
+
+
+class FeedForward(nn.Module):
+    """OneTrans' feed-forward (experiments/onetrans/model.py:33-44): ``net = Sequential(Linear(d_model, d_model *
+    hidden_mult), SiLU, Dropout, Linear(d_model * hidden_mult, d_model))``, same constructor and parameter names
+    (``net.0``, ``net.3``). Under ``torch.no_grad()`` bf16 tokens of width 128 / 256 run as one kernel with the hidden
+    state in registers; ``norm_weight`` / ``residual`` additionally fuse the RMSNorm in front and the residual add
+    behind (``tokens + ffn(ffn_norm(tokens))`` of ``OneTransBlock.forward``, :107). Training-mode dropout of the hidden
+    state runs the two layers as kernels of their own with torch's dropout between them."""
+
+    def __init__(self, d_model: int, hidden_mult: int, dropout: float = 0.0) -> None:
+        super().__init__()
+        self.net = nn.Sequential(
+            nn.Linear(d_model, d_model * hidden_mult),
+            nn.SiLU(),
+            nn.Dropout(dropout),
+            nn.Linear(d_model * hidden_mult, d_model),
+        )
+
+    def forward(self, x: torch.Tensor, *, residual: torch.Tensor | None = None, norm_weight: torch.Tensor | None = None,
+                eps: float = 1e-6) -> torch.Tensor:
+        output_dtype = x.dtype
+        tokens = x if x.dtype == torch.bfloat16 else x.to(torch.bfloat16)
+        fc1, fc2 = self.net[0], self.net[3]
+        if self.training and self.net[2].p > 0.0:
+            from taac_2026_amd.accelerators.linear import linear
+            from taac_2026_amd.accelerators.normalization import rms_norm
+
+            h = tokens if norm_weight is None else rms_norm(tokens, _bf16(norm_weight), eps)
+            hidden = self.net[2](torch.nn.functional.silu(linear(h, _bf16(fc1.weight), _bf16(fc1.bias))))
+            out = linear(hidden, _bf16(fc2.weight), _bf16(fc2.bias), residual=_bf16(residual))
+        else:
+            out = silu_mlp(tokens, _bf16(fc1.weight), _bf16(fc1.bias), _bf16(fc2.weight), _bf16(fc2.bias),
+                           residual=_bf16(residual), norm_weight=_bf16(norm_weight), eps=eps)
+        return out if out.dtype == output_dtype else out.to(output_dtype)
+
+
+class MixedFeedForward(nn.Module):
+    """OneTrans' mixed feed-forward (experiments/onetrans/model.py:80-94): a shared ``FeedForward`` over every token, and
+    for the i-th non-sequence token (position ``seq_token_count + i``) a feed-forward of its own whose output replaces
+    the shared one. The token-specific layers read their token as a strided ``[B, D]`` view of the stream."""
+
+    def __init__(self, d_model: int, hidden_mult: int, num_ns_tokens: int, dropout: float = 0.0) -> None:
+        super().__init__()
+        self.shared = FeedForward(d_model, hidden_mult, dropout)
+        self.ns_specific = nn.ModuleList(FeedForward(d_model, hidden_mult, dropout) for _ in range(num_ns_tokens))
+
+    def forward(self, tokens: torch.Tensor, seq_token_count: int) -> torch.Tensor:
+        output = self.shared(tokens)
+        if not output.requires_grad:
+            for ns_index, ffn in enumerate(self.ns_specific):
+                position = seq_token_count + ns_index
+                if position >= tokens.shape[1]:
+                    continue
+                output[:, position, :] = ffn(tokens[:, position, :])
+            return output
+        pieces = []  # under autograd: no in-place writes into a tensor the graph holds
+        for ns_index, ffn in enumerate(self.ns_specific):
+            position = seq_token_count + ns_index
+            if position < tokens.shape[1]:
+                pieces.append((position, ffn(tokens[:, position, :])))
+        if not pieces:
+            return output
+        replaced = output.clone()
+        for position, value in pieces:
+            replaced[:, position, :] = value
+        return replaced
 
 
 class UnifiedSelfAttention(nn.Module):
