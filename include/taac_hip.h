@@ -346,6 +346,15 @@ int taac_linear_bf16(const void* a, int64_t lda, const void* w, const void* bias
                      int64_t ldo, int64_t M, int32_t N, int32_t K, int epilogue, int gate_first, void* stream);
 
 /*
+ * taac_linear_bf16 with float16 operands, bias, residual and output (fp32 accumulation, v_mfma_f32_32x32x16_f16): the
+ * dense layers of a model that runs in float16, the 16-bit type of the reference's GPU tests
+ * (tests/gpu/infrastructure/accelerators/test_tilelang_ops_cuda.py:61-73). Same arguments, epilogues and alignment rules.
+ * Replaces: nn.Linear / F.linear on float16 tensors (experiments/symbiosis/backbone.py:14-21, 29, 32).
+ */
+int taac_linear_f16(const void* a, int64_t lda, const void* w, const void* bias, const void* residual, void* out,
+                    int64_t ldo, int64_t M, int32_t N, int32_t K, int epilogue, int gate_first, void* stream);
+
+/*
  * Backward pieces of a dense layer y = a w^T + b that are not themselves a forward-shaped product (the input gradient
  * dy w is one: taac_linear_bf16 with the transposed weight):
  *   taac_linear_wgrad: dw[n, k] = sum_m dy[m, n] * a[m, k] and (db != NULL) db[n] = sum_m dy[m, n].

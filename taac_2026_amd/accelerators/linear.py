@@ -28,6 +28,24 @@ def _as_rows(x: torch.Tensor) -> tuple[torch.Tensor, torch.Size]:
     return rows, x.shape
 
 
+def _check_16(operator_name: str, *tensors: torch.Tensor | None) -> torch.dtype:
+    """All tensors bfloat16, or all float16 (the tiled dense kernel exists for both): returns the common dtype."""
+    dtypes = {t.dtype for t in tensors if t is not None}
+    if len(dtypes) != 1 or not dtypes <= {torch.bfloat16, torch.float16}:
+        raise RuntimeError(f"{operator_name} expects tensors of one 16-bit dtype (bfloat16 or float16), got {sorted(map(str, dtypes))}")
+    return next(iter(dtypes))
+
+
+def _is_f16(*tensors: torch.Tensor | None) -> bool:
+    return any(t is not None and t.dtype == torch.float16 for t in tensors)
+
+
+def _f16_inference_only(operator_name: str, *tensors: torch.Tensor | None) -> None:
+    if _needs_grad(*tensors):
+        raise RuntimeError(f"{operator_name}: the float16 dense layers are forward-only; train in bfloat16 or call "
+                           "them under torch.no_grad()")
+
+
 def _check_bf16(operator_name: str, *tensors: torch.Tensor | None) -> None:
     for t in tensors:
         if t is not None and t.dtype != torch.bfloat16:
@@ -306,12 +324,15 @@ def linear(
     *,
     residual: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """``F.linear(x, weight, bias)`` (+ ``residual``) in bf16 with fp32 accumulation."""
+    """``F.linear(x, weight, bias)`` (+ ``residual``) on bfloat16 or float16 tensors with fp32 accumulation (float16:
+    forward only)."""
     name = "hip linear"
     require_cuda_tensors(name, x, weight, bias, residual)
-    if _needs_grad(x, weight, bias, residual):
+    if _is_f16(x, weight, bias, residual):
+        _f16_inference_only(name, x, weight, bias, residual)
+    elif _needs_grad(x, weight, bias, residual):
         return _NormLinearFunction.apply(x, weight, bias, None, residual, 1e-6)
-    _check_bf16(name, x, weight, bias, residual)
+    dtype = _check_16(name, x, weight, bias, residual)
     rows, shape = _as_rows(x)
     _check_weight(name, rows, weight, bias)
     weight = weight.contiguous()
@@ -323,7 +344,8 @@ def linear(
             raise ValueError("linear residual must have the shape of the output")
         res_rows = residual.reshape(-1, out_features).contiguous()
     library = _native.load_library()
-    status = library.taac_linear_bf16(
+    entry = library.taac_linear_f16 if dtype == torch.float16 else library.taac_linear_bf16
+    status = entry(
         rows.data_ptr(), rows.stride(0), weight.data_ptr(), _native.ptr(bias), _native.ptr(res_rows), out.data_ptr(),
         out_features, rows.shape[0], out_features, weight.shape[1],
         _native.EPI_RESIDUAL if res_rows is not None else _native.EPI_NONE, 1, _native.current_stream(x.device),
@@ -343,7 +365,7 @@ def swiglu_linear(
     name = "hip swiglu_linear"
     require_cuda_tensors(name, x, weight, bias)
     require_inference(name, x, weight, bias)
-    _check_bf16(name, x, weight, bias)
+    dtype = _check_16(name, x, weight, bias)
     rows, shape = _as_rows(x)
     _check_weight(name, rows, weight, bias)
     if weight.shape[0] % 2 != 0:
@@ -352,7 +374,8 @@ def swiglu_linear(
     hidden = weight.shape[0] // 2
     out = torch.empty((rows.shape[0], hidden), dtype=x.dtype, device=x.device)
     library = _native.load_library()
-    status = library.taac_linear_bf16(
+    entry = library.taac_linear_f16 if dtype == torch.float16 else library.taac_linear_bf16
+    status = entry(
         rows.data_ptr(), rows.stride(0), weight.data_ptr(), _native.ptr(bias), None, out.data_ptr(), hidden,
         rows.shape[0], weight.shape[0], weight.shape[1], _native.EPI_SWIGLU, int(bool(gate_first)),
         _native.current_stream(x.device),
@@ -548,13 +571,15 @@ def swiglu_ffn(
     """
     name = "hip swiglu_ffn"
     require_cuda_tensors(name, x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight)
-    if _needs_grad(x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight):
+    if _is_f16(x, up_weight, down_weight):
+        _f16_inference_only(name, x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight)
+    elif _needs_grad(x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight):
         if token_rows is not None or out is not None:
             raise RuntimeError("hip swiglu_ffn: token_rows / out belong to the inference route; call it under "
                                "torch.no_grad() or pass dense tensors when a gradient is needed")
         return _SwigluFfnFunction.apply(x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight,
                                         bool(gate_first), float(eps))
-    _check_bf16(name, x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight)
+    half = _check_16(name, x, up_weight, up_bias, down_weight, down_bias, residual, norm_weight) == torch.float16
     rows, shape = _as_rows(x)
     _check_weight(name, rows, up_weight, up_bias)
     d_model, hidden = rows.shape[1], up_weight.shape[0] // 2
@@ -562,7 +587,7 @@ def swiglu_ffn(
         raise ValueError("swiglu_ffn expects up_weight [2F, D] and down_weight [D, F]")
     if residual is not None and residual.shape != shape:
         raise ValueError("swiglu_ffn residual must have the shape of the input")
-    if not (_fused_width(d_model) and hidden % 32 == 0):
+    if half or not (_fused_width(d_model) and hidden % 32 == 0):  # float16: the tiled kernels, layer by layer
         if token_rows is not None or out is not None:
             raise RuntimeError("swiglu_ffn: token_rows / out need a fused shape (width 128 / 256, hidden size a multiple of 32)")
         h = rows
@@ -636,7 +661,7 @@ def silu_mlp(
     if residual is not None and residual.shape != x.shape:
         raise ValueError("silu_mlp residual must have the shape of the input")
     needs_grad = _needs_grad(*tensors)
-    if needs_grad or not (_fused_width(d_model) and hidden % 32 == 0):
+    if needs_grad or _is_f16(x, fc1_weight) or not (_fused_width(d_model) and hidden % 32 == 0):
         if token_rows is not None or out is not None:
             raise RuntimeError("silu_mlp: token_rows / out belong to the fused inference route (width 128 / 256, hidden "
                                "size a multiple of 32, no gradient)")
@@ -759,16 +784,18 @@ def norm_linear(
     ``x`` is laid out differently from ``residual`` / ``out`` (:func:`front_rows`)."""
     name = "hip norm_linear"
     require_cuda_tensors(name, x, weight, bias, residual, norm_weight)
-    if _needs_grad(x, weight, bias, residual, norm_weight):
+    if _is_f16(x, weight):
+        _f16_inference_only(name, x, weight, bias, residual, norm_weight)
+    elif _needs_grad(x, weight, bias, residual, norm_weight):
         if token_rows is not None or input_rows is not None or out is not None:
             raise RuntimeError("hip norm_linear: token_rows / input_rows / out belong to the inference route; "
                                "call it under torch.no_grad() or pass dense tensors when a gradient is needed")
         return _NormLinearFunction.apply(x, weight, bias, norm_weight, residual, float(eps))
-    _check_bf16(name, x, weight, bias, residual, norm_weight)
+    half = _check_16(name, x, weight, bias, residual, norm_weight) == torch.float16
     rows, shape = _as_rows(x)
     _check_weight(name, rows, weight, bias)
     in_features, out_features = weight.shape[1], weight.shape[0]
-    if not (_fused_width(in_features) and out_features % 64 == 0):
+    if half or not (_fused_width(in_features) and out_features % 64 == 0):  # float16: the tiled kernel
         if token_rows is not None or out is not None or input_rows is not None:
             raise RuntimeError("norm_linear: token_rows / out need a fused shape (K 128 / 256, N a multiple of 64)")
         h = rows

@@ -29,9 +29,9 @@ constexpr int kBN = 128;  // weight rows per workgroup
 struct LinearParams {
   const void* a;
   const void* w;
-  const bf16_t* bias;
-  const bf16_t* residual;
-  bf16_t* out;
+  const void* bias;      // 16-bit elements of the kernel's output type
+  const void* residual;
+  void* out;
   const float* amax_a;  // fp8 only
   const float* amax_w;  // fp8 only
   int64_t lda, ldo, M;
@@ -48,15 +48,17 @@ __device__ __forceinline__ float silu_f(float x) {
 
 // Accumulator -> bf16 output for one wavefront. acc[ni][mi][j]: feature sub-tile ni, token sub-tile mi,
 // j -> feature (j/4)*8 + hh*4 + j%4 inside the 32-feature sub-tile, token l32 inside the 32-token sub-tile.
-template <int EPI>
+template <int EPI, typename T = bf16_t>
 __device__ __forceinline__ void store_tile(const LinearParams& p, f32x16 (&acc)[2][2], float dq, int64_t m0, int n0,
                                            int wt, int wn, int l32, int hh) {
+  typedef typename Vec8<T>::half_type vec4_t;
 #pragma unroll
   for (int mi = 0; mi < 2; ++mi) {
     const int64_t row = m0 + wt * 64 + mi * 32 + l32;
     if (row >= p.M) continue;
-    bf16_t* orow = p.out + row * p.ldo;
-    const bf16_t* rrow = (EPI == TAAC_EPI_RESIDUAL) ? p.residual + row * p.ldo : nullptr;
+    T* orow = reinterpret_cast<T*>(p.out) + row * p.ldo;
+    const T* rrow = (EPI == TAAC_EPI_RESIDUAL) ? reinterpret_cast<const T*>(p.residual) + row * p.ldo : nullptr;
+    const T* bias = reinterpret_cast<const T*>(p.bias);
     if (EPI == TAAC_EPI_SWIGLU) {
 #pragma unroll
       for (int jq = 0; jq < 4; ++jq) {
@@ -69,19 +71,19 @@ __device__ __forceinline__ void store_tile(const LinearParams& p, f32x16 (&acc)[
           u[e] = acc[1][mi][jq * 4 + e] * dq;
         }
         if (p.bias != nullptr) {
-          const bf16x4 bg = *reinterpret_cast<const bf16x4*>(p.bias + col);
-          const bf16x4 bu = *reinterpret_cast<const bf16x4*>(p.bias + p.F + col);
+          const vec4_t bg = *reinterpret_cast<const vec4_t*>(bias + col);
+          const vec4_t bu = *reinterpret_cast<const vec4_t*>(bias + p.F + col);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             g[e] += static_cast<float>(bg[e]);
             u[e] += static_cast<float>(bu[e]);
           }
         }
-        bf16x4 ov;
+        vec4_t ov;
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          ov[e] = static_cast<bf16_t>(p.gate_first ? silu_f(g[e]) * u[e] : g[e] * silu_f(u[e]));
-        *reinterpret_cast<bf16x4*>(orow + col) = ov;
+          ov[e] = static_cast<T>(p.gate_first ? silu_f(g[e]) * u[e] : g[e] * silu_f(u[e]));
+        *reinterpret_cast<vec4_t*>(orow + col) = ov;
       }
     } else {
 #pragma unroll
@@ -94,19 +96,19 @@ __device__ __forceinline__ void store_tile(const LinearParams& p, f32x16 (&acc)[
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = acc[ni][mi][jq * 4 + e] * dq;
           if (p.bias != nullptr) {
-            const bf16x4 bv = *reinterpret_cast<const bf16x4*>(p.bias + col);
+            const vec4_t bv = *reinterpret_cast<const vec4_t*>(bias + col);
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] += static_cast<float>(bv[e]);
           }
           if (EPI == TAAC_EPI_RESIDUAL) {
-            const bf16x4 rv = *reinterpret_cast<const bf16x4*>(rrow + col);
+            const vec4_t rv = *reinterpret_cast<const vec4_t*>(rrow + col);
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] += static_cast<float>(rv[e]);
           }
-          bf16x4 ov;
+          vec4_t ov;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) ov[e] = static_cast<bf16_t>(v[e]);
-          *reinterpret_cast<bf16x4*>(orow + col) = ov;
+          for (int e = 0; e < 4; ++e) ov[e] = static_cast<T>(v[e]);
+          *reinterpret_cast<vec4_t*>(orow + col) = ov;
         }
       }
     }
@@ -128,7 +130,24 @@ __device__ __forceinline__ bool weight_row_ok(const LinearParams& p, int n0, int
 // ------------------------------------------------------------------------------------------------------------------
 // bf16 operands
 // ------------------------------------------------------------------------------------------------------------------
-template <int EPI>
+template <typename T>
+struct Mfma16;
+template <>
+struct Mfma16<bf16_t> {
+  static __device__ __forceinline__ f32x16 run(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma16<f16_t> {  // the staged 16-byte pieces are opaque: reinterpret them as eight halves
+  static __device__ __forceinline__ f32x16 run(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+
+// T: the 16-bit element type of operands, bias, residual and output (bf16_t or f16_t); the staging below moves opaque
+// 16-byte pieces, only the MFMA and the epilogue depend on it.
+template <int EPI, typename T = bf16_t>
 __global__ __launch_bounds__(kThreads) void linear_bf16_kernel(const LinearParams p) {
   constexpr int BK = 64;
   constexpr int STR = BK + 8;          // LDS row stride in elements (+16 bytes)
@@ -220,10 +239,10 @@ __global__ __launch_bounds__(kThreads) void linear_bf16_kernel(const LinearParam
       for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
         for (int mi = 0; mi < 2; ++mi)
-          acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ni], af[mi], acc[ni][mi], 0, 0, 0);
+          acc[ni][mi] = Mfma16<T>::run(wf[ni], af[mi], acc[ni][mi]);
     }
   }
-  store_tile<EPI>(p, acc, 1.0f, m0, n0, wt, wn, l32, hh);
+  store_tile<EPI, T>(p, acc, 1.0f, m0, n0, wt, wn, l32, hh);
 }
 
 // ------------------------------------------------------------------------------------------------------------------
@@ -345,8 +364,8 @@ __global__ __launch_bounds__(kWideThreads, 2) void linear_bf16_wide_kernel(const
   for (int mi = 0; mi < 2; ++mi) {
     const int64_t row = m0 + wt * 64 + mi * 32 + l32;
     if (row >= p.M) continue;
-    bf16_t* orow = p.out + row * p.ldo;
-    const bf16_t* rrow = (EPI == TAAC_EPI_RESIDUAL) ? p.residual + row * p.ldo : nullptr;
+    bf16_t* orow = static_cast<bf16_t*>(p.out) + row * p.ldo;
+    const bf16_t* rrow = (EPI == TAAC_EPI_RESIDUAL) ? static_cast<const bf16_t*>(p.residual) + row * p.ldo : nullptr;
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni) {
 #pragma unroll
@@ -357,7 +376,7 @@ __global__ __launch_bounds__(kWideThreads, 2) void linear_bf16_wide_kernel(const
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = acc[ni][mi][jq * 4 + e];
         if (p.bias != nullptr) {
-          const bf16x4 bv = *reinterpret_cast<const bf16x4*>(p.bias + col);
+          const bf16x4 bv = *reinterpret_cast<const bf16x4*>(static_cast<const bf16_t*>(p.bias) + col);
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] += static_cast<float>(bv[e]);
         }
@@ -579,9 +598,9 @@ extern "C" int taac_linear_bf16(const void* a, int64_t lda, const void* w, const
   LinearParams p{};
   p.a = a;
   p.w = w;
-  p.bias = static_cast<const bf16_t*>(bias);
-  p.residual = static_cast<const bf16_t*>(residual);
-  p.out = static_cast<bf16_t*>(out);
+  p.bias = bias;
+  p.residual = residual;
+  p.out = out;
   p.lda = lda;
   p.ldo = ldo;
   p.M = M;
@@ -621,6 +640,44 @@ extern "C" int taac_linear_bf16(const void* a, int64_t lda, const void* w, const
   return check_launch(name);
 }
 
+extern "C" int taac_linear_f16(const void* a, int64_t lda, const void* w, const void* bias, const void* residual,
+                               void* out, int64_t ldo, int64_t M, int32_t N, int32_t K, int epilogue, int gate_first,
+                               void* stream) {
+  using namespace taac;
+  const char* name = "taac_linear_f16";
+  int rc = validate_common(name, a, w, out, residual, lda, ldo, M, N, K, epilogue, 8);
+  if (rc != TAAC_OK || M == 0) return rc;
+  if (bias && (reinterpret_cast<uintptr_t>(bias) & 7u))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: bias must be 8-byte aligned", name);
+  LinearParams p{};
+  p.a = a;
+  p.w = w;
+  p.bias = bias;
+  p.residual = residual;
+  p.out = out;
+  p.lda = lda;
+  p.ldo = ldo;
+  p.M = M;
+  p.N = N;
+  p.K = K;
+  p.gate_first = gate_first ? 1 : 0;
+  rc = fill_params(name, p, M, N, epilogue);
+  if (rc != TAAC_OK) return rc;
+  hipStream_t s = as_stream(stream);
+  switch (epilogue) {
+    case TAAC_EPI_NONE:
+      hipLaunchKernelGGL((linear_bf16_kernel<TAAC_EPI_NONE, f16_t>), dim3(p.total), dim3(kThreads), 0, s, p);
+      break;
+    case TAAC_EPI_RESIDUAL:
+      hipLaunchKernelGGL((linear_bf16_kernel<TAAC_EPI_RESIDUAL, f16_t>), dim3(p.total), dim3(kThreads), 0, s, p);
+      break;
+    default:
+      hipLaunchKernelGGL((linear_bf16_kernel<TAAC_EPI_SWIGLU, f16_t>), dim3(p.total), dim3(kThreads), 0, s, p);
+      break;
+  }
+  return check_launch(name);
+}
+
 extern "C" int taac_linear_fp8(const void* a, int a_is_fp8, int64_t lda, const void* w, const float* amax_a,
                                const float* amax_w, const void* bias, const void* residual, void* out, int64_t ldo,
                                int64_t M, int32_t N, int32_t K, int epilogue, int gate_first, void* stream) {
@@ -636,9 +693,9 @@ extern "C" int taac_linear_fp8(const void* a, int a_is_fp8, int64_t lda, const v
   LinearParams p{};
   p.a = a;
   p.w = w;
-  p.bias = static_cast<const bf16_t*>(bias);
-  p.residual = static_cast<const bf16_t*>(residual);
-  p.out = static_cast<bf16_t*>(out);
+  p.bias = bias;
+  p.residual = residual;
+  p.out = out;
   p.amax_a = amax_a;
   p.amax_w = amax_w;
   p.lda = lda;

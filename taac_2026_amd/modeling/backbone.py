@@ -35,8 +35,20 @@ def _bf16(parameter: torch.Tensor | None) -> torch.Tensor | None:
     return parameter if parameter.dtype == torch.bfloat16 else parameter.to(torch.bfloat16)
 
 
+def _compute_dtype(tokens: torch.Tensor) -> torch.dtype:
+    """The 16-bit type a layer computes in: float16 tokens stay float16 (tiled kernels, forward only), everything else
+    runs in bfloat16."""
+    return torch.float16 if tokens.dtype == torch.float16 else torch.bfloat16
+
+
+def _as(parameter: torch.Tensor | None, dtype: torch.dtype) -> torch.Tensor | None:
+    if parameter is None:
+        return None
+    return parameter if parameter.dtype == dtype else parameter.to(dtype)
+
+
 def _dense(layer: nn.Linear, x: torch.Tensor, *, residual: torch.Tensor | None = None) -> torch.Tensor:
-    return norm_linear(x, _bf16(layer.weight), _bf16(layer.bias), residual=residual)
+    return norm_linear(x, _as(layer.weight, x.dtype), _as(layer.bias, x.dtype), residual=residual)
 
 
 class SwiGLUFeedForward(nn.Module):
@@ -53,15 +65,16 @@ class SwiGLUFeedForward(nn.Module):
 
     def forward(self, tokens: torch.Tensor, *, residual: torch.Tensor | None = None) -> torch.Tensor:
         output_dtype = tokens.dtype
-        x = tokens if tokens.dtype == torch.bfloat16 else tokens.to(torch.bfloat16)
+        dtype = _compute_dtype(tokens)
+        x = _as(tokens, dtype)
         if self.training and self.dropout.p > 0.0:
             # dropout of the hidden state (experiments/symbiosis/backbone.py:19-21): the hidden state reaches memory
-            out = swiglu_ffn_dropout(x, _bf16(self.up.weight), _bf16(self.up.bias), _bf16(self.down.weight),
-                                     _bf16(self.down.bias), dropout_p=self.dropout.p, residual=_bf16(residual),
+            out = swiglu_ffn_dropout(x, _as(self.up.weight, dtype), _as(self.up.bias, dtype), _as(self.down.weight, dtype),
+                                     _as(self.down.bias, dtype), dropout_p=self.dropout.p, residual=_as(residual, dtype),
                                      gate_first=self.gate_first)
             return out if out.dtype == output_dtype else out.to(output_dtype)
-        out = swiglu_ffn(x, _bf16(self.up.weight), _bf16(self.up.bias), _bf16(self.down.weight), _bf16(self.down.bias),
-                         residual=_bf16(residual), gate_first=self.gate_first)
+        out = swiglu_ffn(x, _as(self.up.weight, dtype), _as(self.up.bias, dtype), _as(self.down.weight, dtype),
+                         _as(self.down.bias, dtype), residual=_as(residual, dtype), gate_first=self.gate_first)
         return out if out.dtype == output_dtype else out.to(output_dtype)
 
 
@@ -85,18 +98,19 @@ class FeedForward(nn.Module):
     def forward(self, x: torch.Tensor, *, residual: torch.Tensor | None = None, norm_weight: torch.Tensor | None = None,
                 eps: float = 1e-6) -> torch.Tensor:
         output_dtype = x.dtype
-        tokens = x if x.dtype == torch.bfloat16 else x.to(torch.bfloat16)
+        dtype = _compute_dtype(x)
+        tokens = _as(x, dtype)
         fc1, fc2 = self.net[0], self.net[3]
         if self.training and self.net[2].p > 0.0:
             from taac_2026_amd.accelerators.linear import linear
             from taac_2026_amd.accelerators.normalization import rms_norm
 
-            h = tokens if norm_weight is None else rms_norm(tokens, _bf16(norm_weight), eps)
-            hidden = self.net[2](torch.nn.functional.silu(linear(h, _bf16(fc1.weight), _bf16(fc1.bias))))
-            out = linear(hidden, _bf16(fc2.weight), _bf16(fc2.bias), residual=_bf16(residual))
+            h = tokens if norm_weight is None else rms_norm(tokens, _as(norm_weight, dtype), eps)
+            hidden = self.net[2](torch.nn.functional.silu(linear(h, _as(fc1.weight, dtype), _as(fc1.bias, dtype))))
+            out = linear(hidden, _as(fc2.weight, dtype), _as(fc2.bias, dtype), residual=_as(residual, dtype))
         else:
-            out = silu_mlp(tokens, _bf16(fc1.weight), _bf16(fc1.bias), _bf16(fc2.weight), _bf16(fc2.bias),
-                           residual=_bf16(residual), norm_weight=_bf16(norm_weight), eps=eps)
+            out = silu_mlp(tokens, _as(fc1.weight, dtype), _as(fc1.bias, dtype), _as(fc2.weight, dtype), _as(fc2.bias, dtype),
+                           residual=_as(residual, dtype), norm_weight=_as(norm_weight, dtype), eps=eps)
         return out if out.dtype == output_dtype else out.to(output_dtype)
 
 
@@ -158,10 +172,11 @@ class UnifiedSelfAttention(nn.Module):
         residual: torch.Tensor | None = None,
     ) -> torch.Tensor:
         output_dtype = tokens.dtype
-        x = tokens if tokens.dtype == torch.bfloat16 else tokens.to(torch.bfloat16)
+        dtype = _compute_dtype(tokens)
+        x = _as(tokens, dtype)
         prepare = self.query_norm is not None or self.rope_base is not None
-        query_weight = None if self.query_norm is None else _bf16(self.query_norm.weight)
-        key_weight = None if self.key_norm is None else _bf16(self.key_norm.weight)
+        query_weight = None if self.query_norm is None else _as(self.query_norm.weight, dtype)
+        key_weight = None if self.key_norm is None else _as(self.key_norm.weight, dtype)
         qk_eps = 1e-6 if self.query_norm is None else self.query_norm.eps
         q_row_scale = k_row_scale = q_col_scale = None
         needs_grad = torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))
@@ -170,7 +185,7 @@ class UnifiedSelfAttention(nn.Module):
             query, key, value = _dense(self.qkv, x).chunk(3, dim=-1)
             query, key = qk_norm_rope(query, key, query_weight, key_weight, num_heads=self.num_heads, eps=qk_eps,
                                       rope_base=self.rope_base)
-        elif prepare and x.ndim == 3 and x.shape[-1] in (128, 256):
+        elif prepare and dtype == torch.bfloat16 and x.ndim == 3 and x.shape[-1] in (128, 256):
             # the norm statistic (and, with a rotation, weight and rotation) come out of the projection's epilogue; the
             # per-token factor of the norm and the weights of the unrotated case are applied inside the attention
             # kernel: no pass over q and k at all
@@ -200,7 +215,7 @@ class UnifiedSelfAttention(nn.Module):
             k_row_scale=k_row_scale,
             q_col_scale=q_col_scale,
         )
-        out = _dense(self.out, attended, residual=_bf16(residual))
+        out = _dense(self.out, attended, residual=_as(residual, dtype))
         return out if out.dtype == output_dtype else out.to(output_dtype)
 
 
