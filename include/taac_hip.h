@@ -471,13 +471,19 @@ int taac_attn_out_gate_ffn_fwd(const void* attn, int64_t ld_attn, const void* ou
  * taac_linear_pack_weights for w. K must be 128 or 256, N a multiple of 64. out may alias residual, not x.
  * rows / n_rows: as in taac_swiglu_ffn_fwd (rows of residual and out). x_rows: NULL, or (with rows) the row of x that
  * holds token i when x is laid out differently from residual / out (taac_front_rows).
+ * norm_folded != 0 (needs norm_weight and packed_weights): packed_weights is the blob of taac_linear_pack_weights_norm
+ * for (w, norm_weight), i.e. the norm's weight is already part of the layer. The kernel then leaves the rows as they
+ * are and multiplies its fp32 accumulators by the token's rsqrt(mean(x^2) + eps) before bias and rounding
+ * (linear(x * r * g) = r * linear_g(x)): the normalised rows are never formed, which saves about five vector
+ * instructions per input element; the result differs from the unfolded form by roundings only (g is rounded into the
+ * weights instead of into the rows; exactly equal for g = 1).
  * Replaces: attn_norm + the qkv projection, and the out projection + residual add, of UnifiedInteractionBlock /
  * UnifiedSelfAttention (experiments/symbiosis/backbone.py:34-35, 47, 64-65).
  */
 int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
                          const void* bias, const void* packed_weights, const void* residual, int64_t ldr, void* out,
                          int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows, const int32_t* n_rows,
-                         const int32_t* x_rows, void* stream);
+                         const int32_t* x_rows, int norm_folded, void* stream);
 
 /*
  * Query / key preparation of the attention layers, one pass over q and k (each read once, written once; in place when
@@ -512,7 +518,7 @@ int taac_qk_norm_rope_fwd(const void* q, const void* k, int64_t ld_in, void* q_o
  *         the token at position r % tokens_per_sample.
  * The value features are stored unchanged. The per-token factor rsqrt(mean + eps) of the norm commutes with the weight
  * and the rotation and is left to the attention kernel (taac_flash_attn_scaled_fwd). d_model: 128 or 256; head_dim a
- * multiple of 8 with a table. Other arguments as taac_norm_linear_fwd; with x_rows the statistic is indexed by the row
+ * multiple of 8 with a table. Other arguments (norm_folded included) as taac_norm_linear_fwd; with x_rows the statistic is indexed by the row
  * of out and the position is that of the row of x.
  * Replaces: qkv + query_norm + key_norm of UnifiedSelfAttention.forward (experiments/symbiosis/backbone.py:33-36)
  * and BFTSAttention._apply_rope (experiments/tokenformer/model.py:165-192) without a pass of their own over q and k.
@@ -521,7 +527,7 @@ int taac_norm_linear_qk_fwd(const void* x, int64_t ldx, const void* norm_weight,
                             const void* bias, const void* packed_weights, void* out, int64_t ldo, int64_t M,
                             int32_t d_model, int32_t num_heads, int32_t tokens_per_sample, const void* qk_weight,
                             const void* cos_sin, float* qk_sumsq, const int32_t* rows, const int32_t* n_rows,
-                            const int32_t* x_rows, void* stream);
+                            const int32_t* x_rows, int norm_folded, void* stream);
 
 /*
  * rstd[0, r] = rsqrt(sum_c qk_sumsq[c, r] / d_model + eps) over the d_model / 64 chunks of the query projection,
@@ -660,6 +666,9 @@ int taac_ffn_pack_weights(const void* w_up, const void* w_down, void* packed, in
                           void* stream);
 int64_t taac_linear_packed_bytes(int32_t N, int32_t K);
 int taac_linear_pack_weights(const void* w, void* packed, int32_t N, int32_t K, void* stream);
+/* The same blob with the weight of an RMSNorm in front of the layer folded in (packed[n, k] = bf16(w[n, k] *
+ * norm_weight[k])), for taac_norm_linear_fwd / taac_norm_linear_qk_fwd with norm_folded = 1. */
+int taac_linear_pack_weights_norm(const void* w, const void* norm_weight, void* packed, int32_t N, int32_t K, void* stream);
 
 /*
  * Per-tensor absolute maximum, for the FP8 scale (scale = amax / 448). Writes max(|x|) over n elements to

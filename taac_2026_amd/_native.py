@@ -207,7 +207,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "taac_norm_linear_fwd": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
-         c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p],
+         c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     ),
     "taac_front_rows": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p]),
     "taac_mask_front_bits": (c_int, [c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p]),
@@ -216,7 +216,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "taac_norm_linear_qk_fwd": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32,
-         c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+         c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     ),
     "taac_row_rstd": (c_int, [c_void_p, c_int64, c_int32, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     "taac_qk_norm_rope_fwd": (
@@ -228,6 +228,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "taac_ffn_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int, c_void_p]),
     "taac_linear_packed_bytes": (c_int64, [c_int32, c_int32]),
     "taac_linear_pack_weights": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
+    "taac_linear_pack_weights_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
     "taac_amax": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p]),
     "taac_quantize_fp8": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p]),
     "taac_linear_fp8": (

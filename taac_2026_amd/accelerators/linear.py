@@ -440,8 +440,10 @@ def pack_ffn_weights(up_weight: torch.Tensor, down_weight: torch.Tensor, *, gate
     return packed
 
 
-def pack_linear_weight(weight: torch.Tensor) -> torch.Tensor:
-    """Fragment-ordered blob of ``weight [N, K]`` for ``norm_linear`` (uint8 tensor)."""
+def pack_linear_weight(weight: torch.Tensor, norm_weight: torch.Tensor | None = None) -> torch.Tensor:
+    """Fragment-ordered blob of ``weight [N, K]`` for ``norm_linear`` (uint8 tensor). ``norm_weight`` ``[K]``: the weight
+    of the RMSNorm in front of the layer, folded into the blob (``taac_linear_pack_weights_norm``); the kernel is then
+    called with ``norm_folded = 1`` and applies only the norm's per-token factor, to its accumulators."""
     library = _native.load_library()
     out_features, in_features = weight.shape
     nbytes = library.taac_linear_packed_bytes(out_features, in_features)
@@ -449,10 +451,24 @@ def pack_linear_weight(weight: torch.Tensor) -> torch.Tensor:
         raise RuntimeError(f"pack_linear_weight: unsupported shape N={out_features}, K={in_features}")
     weight = weight.contiguous()
     packed = torch.empty(nbytes, dtype=torch.uint8, device=weight.device)
-    status = library.taac_linear_pack_weights(weight.data_ptr(), packed.data_ptr(), out_features, in_features,
-                                              _native.current_stream(weight.device))
+    if norm_weight is not None:
+        if norm_weight.shape != (in_features,):
+            raise ValueError("rms_norm weight must be 1D and match the normalized dimension")
+        status = library.taac_linear_pack_weights_norm(weight.data_ptr(), norm_weight.contiguous().data_ptr(),
+                                                       packed.data_ptr(), out_features, in_features,
+                                                       _native.current_stream(weight.device))
+    else:
+        status = library.taac_linear_pack_weights(weight.data_ptr(), packed.data_ptr(), out_features, in_features,
+                                                  _native.current_stream(weight.device))
     _native.check(status, "pack_linear_weight")
     return packed
+
+
+def _packed_linear(weight: torch.Tensor, norm_weight: torch.Tensor | None) -> torch.Tensor:
+    """Cached blob of a layer, with the weight of the norm in front of it folded in when there is one."""
+    if norm_weight is None:
+        return _packed_cache.get((weight,), lambda: pack_linear_weight(weight))
+    return _packed_cache.get((weight, norm_weight), lambda: pack_linear_weight(weight, norm_weight), variant=3)
 
 
 def valid_rows(key_lengths: torch.Tensor | None, tokens: int, *,
@@ -805,7 +821,7 @@ def norm_linear(
             h = rms_norm(rows, norm_weight, eps)
         res = residual.reshape(-1, out_features) if residual is not None else None
         return linear(h, weight, bias, residual=res).reshape(*shape[:-1], out_features)
-    packed = _packed_cache.get((weight,), lambda: pack_linear_weight(weight))
+    packed = _packed_linear(weight, norm_weight)
     res_rows = None
     if residual is not None:
         if residual.shape != (*shape[:-1], out_features):
@@ -820,7 +836,8 @@ def norm_linear(
         rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), None, _native.ptr(bias),
         packed.data_ptr(), _native.ptr(res_rows), res_rows.stride(0) if res_rows is not None else out_features, out.data_ptr(),
         out_features, rows.shape[0], out_features, in_features, _native.ptr(index), _native.ptr(count),
-        _native.ptr(_input_rows(name, input_rows, index, rows)), _native.current_stream(x.device),
+        _native.ptr(_input_rows(name, input_rows, index, rows)), int(norm_weight is not None),
+        _native.current_stream(x.device),
     )
     _native.check(status, "norm_linear")
     return out.reshape(*shape[:-1], out_features)
@@ -892,7 +909,7 @@ def qkv_projection(
         from taac_2026_amd.accelerators.attention import rope_table
 
         table = rope_table(tokens, d_model // int(num_heads), rope_base, x.dtype, x.device)
-    packed = _packed_cache.get((weight,), lambda: pack_linear_weight(weight))
+    packed = _packed_linear(weight, norm_weight)
     index, count = _token_rows(name, token_rows, rows)
     out = _output_rows(name, out, (rows.shape[0], 3 * d_model), index is not None, x)
     sumsq = scales = None
@@ -911,7 +928,7 @@ def qkv_projection(
         rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), None, _native.ptr(bias), packed.data_ptr(),
         out.data_ptr(), 3 * d_model, rows.shape[0], d_model, int(num_heads), tokens, _native.ptr(qk_weight),
         _native.ptr(table), _native.ptr(sumsq), _native.ptr(index), _native.ptr(count),
-        _native.ptr(_input_rows(name, input_rows, index, rows)), stream,
+        _native.ptr(_input_rows(name, input_rows, index, rows)), int(norm_weight is not None), stream,
     )
     _native.check(status, "qkv_projection")
     if scales is None:

@@ -635,7 +635,8 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
       }
       if ((rc = taac_norm_linear_qk_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, qkv, 3 * D, M, D,
                                         heads, T, weights_in_epilogue ? qk_weight : nullptr, rope_cos_sin,
-                                        qk_norm ? qk_sumsq : nullptr, rows, n_rows, nullptr, stream)) != TAAC_OK)
+                                        qk_norm ? qk_sumsq : nullptr, rows, n_rows, nullptr,
+                                        w.attn_norm_weight != nullptr, stream)) != TAAC_OK)
         return rc;
       if (qk_norm) {
         if ((rc = taac_row_rstd(qk_sumsq, M, D, eps, qk_rstd, rows, n_rows, stream)) != TAAC_OK) return rc;
@@ -644,7 +645,8 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
       }
     } else if (fused) {
       if ((rc = taac_norm_linear_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, nullptr, 0, qkv,
-                                     3 * D, M, 3 * D, D, rows, n_rows, nullptr, stream)) != TAAC_OK)
+                                     3 * D, M, 3 * D, D, rows, n_rows, nullptr, w.attn_norm_weight != nullptr,
+                                     stream)) != TAAC_OK)
         return rc;
     } else {
       if ((rc = taac_rmsnorm_fwd(cur, w.attn_norm_weight, h, M, D, eps, TAAC_BF16, stream)) != TAAC_OK) return rc;
@@ -669,7 +671,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
         return rc;
     } else if (fused) {
       if ((rc = taac_norm_linear_fwd(h, D, nullptr, eps, nullptr, w.out_bias, pk_out, cur, D, x, D, M, D, D, rows,
-                                     n_rows, nullptr, stream)) != TAAC_OK)
+                                     n_rows, nullptr, 0, stream)) != TAAC_OK)
         return rc;
       // feed-forward half: RMSNorm -> up -> SiLU-gate -> down -> + residual in one kernel
       if ((rc = taac_swiglu_ffn_fwd(x, D, w.ffn_norm_weight, eps, nullptr, w.up_bias, nullptr, w.down_bias, pk_ffn, x,

@@ -64,6 +64,9 @@ struct TsParams {
   // Attention output projection in front of the FFN (x is then the attention output, residual the block input):
   const bf16_t* w0;         // packed [D, D] projection (linear blob)
   const bf16_t* b0;         // its bias [D] or null
+  int32_t norm_folded;      // linear kernel: norm_w is already part of the packed weights (taac_linear_pack_weights_norm):
+                            // the rows enter the products as they are and only the factor rsqrt(mean + eps) is applied, to the
+                            // accumulators
   const bf16_t* gate;       // GATE: [M, D] pre-activation of the update's gate (rows like residual), row stride ldg
   int64_t ldg;
 };
@@ -127,21 +130,31 @@ __global__ void mlp_pack_kernel(const bf16_t* __restrict__ w1, const bf16_t* __r
 }
 
 // Linear blob: chunk c (64 output features) holds fragments (row block rb, k-step ks) at index rb * KS + ks.
+// col_scale (optional, [K]): every weight is multiplied by the factor of its input feature and rounded once - the weight
+// of an RMSNorm in front of the layer, folded into the layer (linear(x * r * g) = r * linear_g(x) with linear_g's weights
+// w[n, k] * g[k]; the kernel then applies the per-token factor r to its accumulators).
 __device__ __forceinline__ void linear_pack_piece(const bf16_t* __restrict__ w, bf16x8* __restrict__ packed, int K,
-                                                  int64_t gid) {
+                                                  int64_t gid, const bf16_t* __restrict__ col_scale = nullptr) {
   const int KS = K / 16, NFRAG = 2 * KS;
   const int lane = static_cast<int>(gid % 64);
   const int f = static_cast<int>((gid / 64) % NFRAG);
   const int64_t chunk = gid / 64 / NFRAG;
   const int l32 = lane % 32, hh = lane / 32;
-  const bf16_t* src = w + (chunk * kNC + (f / KS) * 32 + l32) * K + (f % KS) * 16 + hh * 8;
-  packed[gid] = *reinterpret_cast<const bf16x8*>(src);
+  const int col = (f % KS) * 16 + hh * 8;
+  bf16x8 v = *reinterpret_cast<const bf16x8*>(w + (chunk * kNC + (f / KS) * 32 + l32) * K + col);
+  if (col_scale != nullptr) {
+    const bf16x8 g = *reinterpret_cast<const bf16x8*>(col_scale + col);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = static_cast<bf16_t>(static_cast<float>(v[e]) * static_cast<float>(g[e]));
+  }
+  packed[gid] = v;
 }
 
-__global__ void linear_pack_kernel(const bf16_t* __restrict__ w, bf16x8* __restrict__ packed, int N, int K) {
+__global__ void linear_pack_kernel(const bf16_t* __restrict__ w, bf16x8* __restrict__ packed, int N, int K,
+                                   const bf16_t* __restrict__ col_scale) {
   const int64_t total = static_cast<int64_t>(N) * K / 8;
   const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (gid < total) linear_pack_piece(w, packed, K, gid);
+  if (gid < total) linear_pack_piece(w, packed, K, gid, col_scale);
 }
 
 // All weights of up to kPackBatch backbone blocks in one launch: blockIdx.y = block, blockIdx.x walks the 16-byte
@@ -149,6 +162,7 @@ __global__ void linear_pack_kernel(const bf16_t* __restrict__ w, bf16x8* __restr
 constexpr int kPackBatch = 16;
 struct PackBatch {
   const bf16_t* qkv[kPackBatch];
+  const bf16_t* qkv_norm[kPackBatch];  // weight of the RMSNorm in front of the projection (folded into its blob), or null
   const bf16_t* out[kPackBatch];
   const bf16_t* up[kPackBatch];
   const bf16_t* down[kPackBatch];
@@ -161,7 +175,7 @@ __global__ void pack_blocks_kernel(const PackBatch batch, int D, int F) {
   const int64_t n_qkv = static_cast<int64_t>(3) * D * D / 8, n_out = static_cast<int64_t>(D) * D / 8;
   const int64_t n_ffn = static_cast<int64_t>(3) * D * F / 8;
   int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (gid < n_qkv) return linear_pack_piece(batch.qkv[blk], batch.packed_qkv[blk], D, gid);
+  if (gid < n_qkv) return linear_pack_piece(batch.qkv[blk], batch.packed_qkv[blk], D, gid, batch.qkv_norm[blk]);
   gid -= n_qkv;
   if (gid < n_out) return linear_pack_piece(batch.out[blk], batch.packed_out[blk], D, gid);
   gid -= n_out;
@@ -243,6 +257,27 @@ __device__ __forceinline__ void normalize_tokens(float eps, const bf16_t* norm_w
   }
 }
 
+// rsqrt(mean(x^2) + eps) of the loaded rows, per lane for its token of each tile; the rows themselves stay as they are
+// (the norm's weight is part of the packed layer, the factor goes to the accumulators). The squares are summed two
+// elements per instruction (v_dot2_f32_bf16).
+template <int D, int TT>
+__device__ __forceinline__ void token_rstd(float eps, const bf16x8 (&xf)[TT][D / 16], float (&rstd)[TT]) {
+  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+#pragma unroll
+  for (int t = 0; t < TT; ++t) {
+    float ss = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks)
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        const bf16x2 pair = {xf[t][ks][e], xf[t][ks][e + 1]};
+        ss = __builtin_amdgcn_fdot2_f32_bf16(pair, pair, ss, false);
+      }
+    ss += __shfl_xor(ss, 32, kWave);
+    rstd[t] = rsqrtf(ss * (1.0f / D) + eps);
+  }
+}
+
 // Up-projection bias in fragment row order: entry chunk * 32 + m belongs to row slot m of the chunk's up fragment
 // (slots 0..15 the gated half, 16..31 the other half), so lane l32 of a wavefront finds the bias of its fragment row at
 // chunk * 32 + l32. Zeros when there is no bias.
@@ -271,7 +306,7 @@ __device__ __forceinline__ void read_chunk_bias(const bf16_t* bias_lds, int hh, 
 // Writes two 32-feature accumulator blocks (64 features) of one 32-token tile into the wavefront's epilogue tile,
 // adding the bias and rounding to bf16. Accumulator register jq*4 + e of lane (l32, hh) is feature jq*8 + hh*4 + e.
 __device__ __forceinline__ void tile_to_lds(uint8_t* tile, const f32x16& a0, const f32x16& a1, const bf16x4 (&bv)[8],
-                                            int l32, int hh) {
+                                            int l32, int hh, float scale = 1.0f) {
 #pragma unroll
   for (int rb = 0; rb < 2; ++rb) {
 #pragma unroll
@@ -280,7 +315,7 @@ __device__ __forceinline__ void tile_to_lds(uint8_t* tile, const f32x16& a0, con
       bf16x4 ov;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        ov[e] = static_cast<bf16_t>((rb == 0 ? a0[jq * 4 + e] : a1[jq * 4 + e]) + static_cast<float>(bv[rb * 4 + jq][e]));
+        ov[e] = static_cast<bf16_t>(fmaf(rb == 0 ? a0[jq * 4 + e] : a1[jq * 4 + e], scale, static_cast<float>(bv[rb * 4 + jq][e])));
       *reinterpret_cast<bf16x4*>(tile + l32 * kStageRow + col * 2) = ov;
     }
   }
@@ -288,7 +323,7 @@ __device__ __forceinline__ void tile_to_lds(uint8_t* tile, const f32x16& a0, con
 
 // tile_to_lds that also returns the sum of squares of the lane's 32 rounded values (half of its token's 64 features).
 __device__ __forceinline__ float tile_to_lds_sumsq(uint8_t* tile, const f32x16& a0, const f32x16& a1,
-                                                   const bf16x4 (&bv)[8], int l32, int hh) {
+                                                   const bf16x4 (&bv)[8], int l32, int hh, float scale = 1.0f) {
   float ss = 0.f;
 #pragma unroll
   for (int rb = 0; rb < 2; ++rb) {
@@ -298,7 +333,7 @@ __device__ __forceinline__ float tile_to_lds_sumsq(uint8_t* tile, const f32x16& 
       bf16x4 ov;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        ov[e] = static_cast<bf16_t>((rb == 0 ? a0[jq * 4 + e] : a1[jq * 4 + e]) + static_cast<float>(bv[rb * 4 + jq][e]));
+        ov[e] = static_cast<bf16_t>(fmaf(rb == 0 ? a0[jq * 4 + e] : a1[jq * 4 + e], scale, static_cast<float>(bv[rb * 4 + jq][e])));
         const float r = static_cast<float>(ov[e]);
         ss = fmaf(r, r, ss);
       }
@@ -945,7 +980,19 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
   load_tile(tok_wave);
   vm_wait<0>();
   __syncthreads();
-  if (p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + p.N, hh, xf);
+  // The norm in front of the layer: either its weight is part of the packed layer and only the per-token factor is formed
+  // here (it multiplies the accumulators in the epilogue), or the rows are normalised in place.
+  float rstd[TT];
+#pragma unroll
+  for (int t = 0; t < TT; ++t) rstd[t] = 1.0f;
+  auto apply_norm = [&]() {
+    if (p.norm_w == nullptr) return;
+    if (p.norm_folded)
+      token_rstd<D, TT>(p.eps, xf, rstd);
+    else
+      normalize_tokens<D, TT>(p.eps, bias_lds + p.N, hh, xf);
+  };
+  apply_norm();
 
   uint8_t* tile_lds = tiles + wave * kStageWave;
   int buf = 0;                                        // ring slot of step s
@@ -977,7 +1024,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
       // The rows are requested after the weights and residual pieces of the later steps, so that those are not held
       // back by the wait for the rows.
       load_tile(tok_wave);
-      if (p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + p.N, hh, xf);
+      apply_norm();
     }
 
     // ---- the products of this chunk ------------------------------------------------------------------------------------
@@ -1047,12 +1094,12 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
       for (int t = 0; t < TT; ++t) {
         read_chunk_bias(bias_lds + chunk * kNC, hh, bv);  // per tile: not held while the pieces are processed
         if (qk_chunk && p.qk_sumsq != nullptr) {
-          float ss = tile_to_lds_sumsq(tile_lds, acc0[t], acc1[t], bv, l32, hh);
+          float ss = tile_to_lds_sumsq(tile_lds, acc0[t], acc1[t], bv, l32, hh, rstd[t]);
           ss = half_wave_pair_sum(ss);
           const int row = rowinfo[t * 32 + l32].x;
           if (hh == 0) p.qk_sumsq[static_cast<int64_t>(chunk) * p.M + row] = ss;
         } else {
-          tile_to_lds(tile_lds, acc0[t], acc1[t], bv, l32, hh);
+          tile_to_lds(tile_lds, acc0[t], acc1[t], bv, l32, hh, rstd[t]);
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         // two pieces at a time: rows (and table pieces) first, then the arithmetic and the stores
@@ -1094,7 +1141,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     }
 #pragma unroll
     for (int t = 0; t < (QK != 0 ? 0 : TT); ++t) {
-      tile_to_lds(tile_lds, acc0[t], acc1[t], bv, l32, hh);
+      tile_to_lds(tile_lds, acc0[t], acc1[t], bv, l32, hh, rstd[t]);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -1165,9 +1212,10 @@ int pack_backbone_blocks(const taac_block_weights* blocks, int n, int32_t D, int
     for (int i = 0; i < m; ++i) {
       const taac_block_weights& w = blocks[base + i];
       if (!ptr_ok(w.qkv_weight, 15) || !ptr_ok(w.out_weight, 15) || !ptr_ok(w.up_weight, 15) ||
-          !ptr_ok(w.down_weight, 15))
+          !ptr_ok(w.down_weight, 15) || !ptr_ok(w.attn_norm_weight, 15))
         return set_error(TAAC_ERR_UNSUPPORTED, "%s: weights must be 16-byte aligned", name);
       batch.qkv[i] = static_cast<const bf16_t*>(w.qkv_weight);
+      batch.qkv_norm[i] = static_cast<const bf16_t*>(w.attn_norm_weight);
       batch.out[i] = static_cast<const bf16_t*>(w.out_weight);
       batch.up[i] = static_cast<const bf16_t*>(w.up_weight);
       batch.down[i] = static_cast<const bf16_t*>(w.down_weight);
@@ -1211,18 +1259,32 @@ extern "C" int64_t taac_linear_packed_bytes(int32_t N, int32_t K) {
   return static_cast<int64_t>(N) * K * 2;
 }
 
-extern "C" int taac_linear_pack_weights(const void* w, void* packed, int32_t N, int32_t K, void* stream) {
-  using namespace taac;
-  const char* name = "taac_linear_pack_weights";
+namespace taac {
+namespace {
+int linear_pack(const char* name, const void* w, const void* norm_weight, void* packed, int32_t N, int32_t K, void* stream) {
   if (taac_linear_packed_bytes(N, K) < 0)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: K must be 128 or 256 and N a positive multiple of 64", name);
   if (!w || !packed) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
-  if (!ptr_ok(w, 15) || !ptr_ok(packed, 15))
+  if (!ptr_ok(w, 15) || !ptr_ok(packed, 15) || !ptr_ok(norm_weight, 15))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: pointers must be 16-byte aligned", name);
   const int64_t pieces = static_cast<int64_t>(N) * K / 8;
   hipLaunchKernelGGL(linear_pack_kernel, dim3(static_cast<uint32_t>((pieces + 255) / 256)), dim3(256), 0,
-                     as_stream(stream), static_cast<const bf16_t*>(w), static_cast<bf16x8*>(packed), N, K);
+                     as_stream(stream), static_cast<const bf16_t*>(w), static_cast<bf16x8*>(packed), N, K,
+                     static_cast<const bf16_t*>(norm_weight));
   return check_launch(name);
+}
+}  // namespace
+}  // namespace taac
+
+extern "C" int taac_linear_pack_weights(const void* w, void* packed, int32_t N, int32_t K, void* stream) {
+  return taac::linear_pack("taac_linear_pack_weights", w, nullptr, packed, N, K, stream);
+}
+
+extern "C" int taac_linear_pack_weights_norm(const void* w, const void* norm_weight, void* packed, int32_t N, int32_t K,
+                                             void* stream) {
+  const char* name = "taac_linear_pack_weights_norm";
+  if (!norm_weight) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: null norm weight", name);
+  return taac::linear_pack(name, w, norm_weight, packed, N, K, stream);
 }
 
 namespace taac {
@@ -1414,7 +1476,9 @@ struct QkExtras {
 int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
                        const void* bias, const void* packed_weights, const void* residual, int64_t ldr, void* out,
                        int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows, const int32_t* n_rows,
-                       const int32_t* x_rows, const QkExtras& qk, void* stream) {
+                       const int32_t* x_rows, const QkExtras& qk, int norm_folded, void* stream) {
+  if (norm_folded && (!norm_weight || !packed_weights))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: norm_folded needs the norm weight and the packed weights it was folded into", name);
   if (M < 0 || N <= 0 || K <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, N and K > 0", name);
   if (K != 256 && K != 128)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: token-stationary kernel is built for K = 128 or 256 (got %d)", name, K);
@@ -1452,6 +1516,7 @@ int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void*
   p.N = N;
   p.eps = eps;
   p.packed = packed_weights ? 1 : 0;
+  p.norm_folded = norm_folded ? 1 : 0;
   p.rows = rows;
   p.n_rows = n_rows;
   p.x_rows = x_rows;
@@ -1517,9 +1582,9 @@ __global__ __launch_bounds__(256) void row_rstd_kernel(const float* __restrict__
 extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
                                     const void* bias, const void* packed_weights, const void* residual, int64_t ldr,
                                     void* out, int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows,
-                                    const int32_t* n_rows, const int32_t* x_rows, void* stream) {
+                                    const int32_t* n_rows, const int32_t* x_rows, int norm_folded, void* stream) {
   return taac::norm_linear_launch("taac_norm_linear_fwd", x, ldx, norm_weight, eps, w, bias, packed_weights, residual,
-                                  ldr, out, ldo, M, N, K, rows, n_rows, x_rows, taac::QkExtras{}, stream);
+                                  ldr, out, ldo, M, N, K, rows, n_rows, x_rows, taac::QkExtras{}, norm_folded, stream);
 }
 
 extern "C" int taac_norm_linear_qk_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
@@ -1527,7 +1592,7 @@ extern "C" int taac_norm_linear_qk_fwd(const void* x, int64_t ldx, const void* n
                                        int32_t d_model, int32_t num_heads, int32_t tokens_per_sample,
                                        const void* qk_weight, const void* cos_sin, float* qk_sumsq,
                                        const int32_t* rows, const int32_t* n_rows, const int32_t* x_rows,
-                                       void* stream) {
+                                       int norm_folded, void* stream) {
   using namespace taac;
   const char* name = "taac_norm_linear_qk_fwd";
   if (d_model <= 0 || num_heads <= 0 || tokens_per_sample <= 0 || d_model % num_heads != 0)
@@ -1546,7 +1611,7 @@ extern "C" int taac_norm_linear_qk_fwd(const void* x, int64_t ldx, const void* n
   qk.head_dim = d_model / num_heads;
   qk.tokens_per_sample = tokens_per_sample;
   return norm_linear_launch(name, x, ldx, norm_weight, eps, w, bias, packed_weights, nullptr, 0, out, ldo, M,
-                            3 * d_model, d_model, rows, n_rows, x_rows, qk, stream);
+                            3 * d_model, d_model, rows, n_rows, x_rows, qk, norm_folded, stream);
 }
 
 extern "C" int taac_row_rstd(const float* qk_sumsq, int64_t M, int32_t d_model, float eps, float* rstd,

@@ -97,14 +97,13 @@ def _indexed_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | 
     (``taac_norm_linear_fwd`` with its row indices; ``x_rows`` None: the rows of ``x`` are ``out_rows`` too): a projection
     over the valid rows of the padded layout, or one that crosses between the compact and the padded layout."""
     out_features, in_features = weight.shape
-    pack = lambda: _linear.pack_linear_weight(weight)  # noqa: E731
-    packed = _linear._packed_cache.get((weight,), pack) if cache_weight else pack()
+    packed = _linear._packed_linear(weight, norm_weight) if cache_weight else _linear.pack_linear_weight(weight, norm_weight)
     library = _native.load_library()
     status = library.taac_norm_linear_fwd(
         x.data_ptr(), x.stride(0), _native.ptr(norm_weight), float(eps), None, _native.ptr(bias), packed.data_ptr(),
         _native.ptr(residual), residual.stride(0) if residual is not None else out_features, out.data_ptr(), out.stride(0),
         tokens, out_features, in_features, out_rows.data_ptr(), count.data_ptr(), _native.ptr(x_rows),
-        _native.current_stream(x.device))
+        int(norm_weight is not None), _native.current_stream(x.device))
     _native.check(status, "interaction block (training): projection")
 
 

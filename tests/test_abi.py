@@ -156,8 +156,11 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
     assert tail(m=0) == ok
     assert tail(attn_rows=fake) == invalid and b"x_rows needs rows" in library.taac_last_error()
     status = library.taac_norm_linear_fwd(fake, 256, None, 1e-6, fake, None, None, None, 0, fake, 64, 8, 64, 256, None, None,
-                                          fake, None)
+                                          fake, 0, None)
     assert status == invalid and b"x_rows needs rows" in library.taac_last_error()
+    status = library.taac_norm_linear_fwd(fake, 256, fake, 1e-6, fake, None, None, None, 0, fake, 64, 8, 64, 256, None, None,
+                                          None, 1, None)
+    assert status == invalid and b"norm_folded needs" in library.taac_last_error()
 
     # readout: indices inside the sequence, one kind of validity, a complete classifier, something to write
     def readout(**kw):
