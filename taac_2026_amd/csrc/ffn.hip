@@ -562,19 +562,53 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
       ss[t] = 0.f;
-      hrow[t] = p.residual + hrow_index[t] * p.ldr + hh * 4;
+      // GATE: block input in accumulator order (4-feature runs); otherwise as B-operand fragments (8-feature runs)
+      hrow[t] = p.residual + hrow_index[t] * p.ldr + (GATE ? hh * 4 : hh * 8);
       if constexpr (GATE) grow[t] = p.gate + hrow_index[t] * p.ldg + hh * 4;
+    }
+    // Without a gate the bias and the block input join the projection inside the matrix unit: per 32-feature row block
+    // one more product multiplies a bias fragment with the ones fragment of the feed-forward's bias trick, and - after
+    // the rounding of the layer output - two more multiply an identity fragment (row l32 of the block = k index l32 of a
+    // 32-feature slice) with the block input held as B-operand fragments, which adds h exactly in fp32. The roundings stay
+    // those of the 16-bit evaluation layer by layer, x1 = bf16(bf16(A W0^T + b0) + h); what is left for the vector unit
+    // per element is the two roundings with their widening back to fp32 and half a dot-product instruction for the
+    // norm's sum of squares (3.5 instead of 8 instructions per element).
+    [[maybe_unused]] bf16x8 ident[2];
+    if constexpr (!GATE) {
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int e0 = l32 - 16 * k - 8 * hh;  // element of this lane's eight k slots that is the row's own feature
+        u32x4 bits = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          bits[d] = (e0 >> 1) == d && e0 >= 0 && e0 < 8 ? ((e0 & 1) ? 0x3f800000u : 0x00003f80u) : 0u;
+        ident[k] = __builtin_bit_cast(bf16x8, bits);
+      }
     }
     static_for<NCH>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
-      // block input of this chunk's 64 features in accumulator order: piece rb*4 + jq = features rb*32 + jq*8 + hh*4 .. +3
-      bf16x4 hv[TT][8];
+      // GATE: block input of this chunk's 64 features in accumulator order: piece rb*4 + jq = features rb*32 + jq*8 + hh*4 .. +3
+      [[maybe_unused]] bf16x4 hv[TT][GATE ? 8 : 1];
+      // !GATE: the same 64 features as four B-operand fragments (k-steps 4c .. 4c+3 of the model width)
+      [[maybe_unused]] bf16x8 hf[TT][GATE ? 1 : 4];
+      [[maybe_unused]] uint32_t b0row[2] = {0u, 0u};  // !GATE: bias of this lane's feature row of the chunk's two row blocks
       if (active) {
 #pragma unroll
-        for (int t = 0; t < TT; ++t)
+        for (int t = 0; t < TT; ++t) {
+          if constexpr (GATE) {
 #pragma unroll
-          for (int q = 0; q < 8; ++q)
-            hv[t][q] = *reinterpret_cast<const bf16x4*>(hrow[t] + c * kNC + (q / 4) * 32 + (q % 4) * 8);
+            for (int q = 0; q < 8; ++q)
+              hv[t][q] = *reinterpret_cast<const bf16x4*>(hrow[t] + c * kNC + (q / 4) * 32 + (q % 4) * 8);
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) hf[t][j] = *reinterpret_cast<const bf16x8*>(hrow[t] + c * kNC + j * 16);
+          }
+        }
+        if constexpr (!GATE) {
+#pragma unroll
+          for (int rb = 0; rb < 2; ++rb)
+            b0row[rb] = static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(b0_lds)[c * kNC + rb * 32 + l32]);
+        }
       }
       if constexpr (c + 1 < NCH) stage_proj(c + 1, 1 + ((c + 1) & 1));
       if (active) {
@@ -592,34 +626,60 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
           __builtin_amdgcn_sched_barrier(0);
           if constexpr (i + P < CF) lds_read_frag<(i + P) * kFrag>(pring[i % P], wb0);
         });
-        // x1 = bf16( bf16(projection + b0) + h ), kept in the accumulators; sum of squares for the norm that follows
-        bf16x4 bv[8];
-        read_chunk_bias(b0_lds + c * kNC, hh, bv);
-        [[maybe_unused]] bf16x4 gv[TT][8];
         if constexpr (GATE) {
+          // x1 = bf16( bf16(sigmoid(g)) * bf16(projection + b0) + h ), kept in the accumulators; sum of squares for the
+          // norm that follows
+          bf16x4 bv[8];
+          read_chunk_bias(b0_lds + c * kNC, hh, bv);
+          bf16x4 gv[TT][8];
 #pragma unroll
           for (int t = 0; t < TT; ++t)
 #pragma unroll
             for (int q = 0; q < 8; ++q)
               gv[t][q] = *reinterpret_cast<const bf16x4*>(grow[t] + c * kNC + (q / 4) * 32 + (q % 4) * 8);
-        }
 #pragma unroll
-        for (int t = 0; t < TT; ++t)
+          for (int t = 0; t < TT; ++t)
 #pragma unroll
-          for (int q = 0; q < 8; ++q)
+            for (int q = 0; q < 8; ++q)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const float a = oacc[t][2 * c + q / 4][(q % 4) * 4 + e];
-              float lin = static_cast<float>(static_cast<bf16_t>(a + static_cast<float>(bv[q][e])));
-              if constexpr (GATE) {
+              for (int e = 0; e < 4; ++e) {
+                const float a = oacc[t][2 * c + q / 4][(q % 4) * 4 + e];
+                float lin = static_cast<float>(static_cast<bf16_t>(a + static_cast<float>(bv[q][e])));
                 const float g = static_cast<float>(gv[t][q][e]);
                 const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
                 lin = static_cast<float>(static_cast<bf16_t>(static_cast<float>(static_cast<bf16_t>(sg)) * lin));
+                const float x1 = static_cast<float>(static_cast<bf16_t>(lin + static_cast<float>(hv[t][q][e])));
+                oacc[t][2 * c + q / 4][(q % 4) * 4 + e] = x1;
+                ss[t] = fmaf(x1, x1, ss[t]);
               }
-              const float x1 = static_cast<float>(static_cast<bf16_t>(lin + static_cast<float>(hv[t][q][e])));
-              oacc[t][2 * c + q / 4][(q % 4) * 4 + e] = x1;
-              ss[t] = fmaf(x1, x1, ss[t]);
+        } else {
+          // + b0 through the matrix unit, lin = bf16(accumulator); + h through the matrix unit (exact in fp32),
+          // x1 = bf16(accumulator), kept in the accumulators as fp32
+          typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+#pragma unroll
+          for (int t = 0; t < TT; ++t)
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb) {
+              f32x16& acc = oacc[t][2 * c + rb];
+              const u32x4 bias_bits = {b0row[rb], 0u, 0u, 0u};
+              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, bias_bits), ones, acc, 0, 0, 0);
+#pragma unroll
+              for (int j = 0; j < 16; j += 2) {
+                const bf16x2 pair = {static_cast<bf16_t>(acc[j]), static_cast<bf16_t>(acc[j + 1])};
+                acc[j] = static_cast<float>(pair[0]);
+                acc[j + 1] = static_cast<float>(pair[1]);
+              }
+              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ident[0], hf[t][2 * rb], acc, 0, 0, 0);
+              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ident[1], hf[t][2 * rb + 1], acc, 0, 0, 0);
+#pragma unroll
+              for (int j = 0; j < 16; j += 2) {
+                const bf16x2 pair = {static_cast<bf16_t>(acc[j]), static_cast<bf16_t>(acc[j + 1])};
+                acc[j] = static_cast<float>(pair[0]);
+                acc[j + 1] = static_cast<float>(pair[1]);
+                ss[t] = __builtin_amdgcn_fdot2_f32_bf16(pair, pair, ss[t], false);
+              }
             }
+        }
       }
       // the next chunk has landed (and, with the first wait, the first step of the feed-forward weights)
       vm_wait<0>();
