@@ -402,13 +402,15 @@ int taac_swiglu_ffn_bwd_hidden(const void* h, int64_t ldh, const void* dy, int64
  * rows / n_rows: both NULL (every row 0..M-1 is a token), or a row index as written by taac_valid_rows: the tokens are
  * rows[0 .. *n_rows) of x / residual / out (*n_rows <= M, read on the device), all other rows are neither read nor
  * written - this is how the layers skip the padded positions of a padded [B, T, D] batch.
+ * norm_folded != 0 (needs norm_weight and packed_weights): the blob is that of taac_ffn_pack_weights_norm, i.e. the norm's
+ * weight is already part of the up projection, and the kernel multiplies the rows by rsqrt(mean(x^2) + eps) only.
  * Replaces: ffn_norm + SwiGLUFeedForward.forward + residual add of UnifiedInteractionBlock.forward
  * (experiments/symbiosis/backbone.py:19-21, 66-67).
  */
 int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w_up,
                         const void* b_up, const void* w_down, const void* b_down, const void* packed_weights,
                         const void* residual, int64_t ldr, void* out, int64_t ldo, int64_t M, int32_t D, int32_t F,
-                        int gate_first, const int32_t* rows, const int32_t* n_rows, void* stream);
+                        int gate_first, const int32_t* rows, const int32_t* n_rows, int norm_folded, void* stream);
 
 /*
  * Plain SiLU feed-forward (OneTrans' FeedForward), one kernel with the hidden state in registers:
@@ -435,8 +437,8 @@ int taac_silu_mlp_fwd(const void* x, int64_t ldx, const void* norm_weight, float
  * out_bias / b_up / b_down may be NULL. x1 is rounded to bf16 as the reference's residual stream is, but is never
  * written to memory: it stays in the accumulators of the down projection, so the final sum x1 + down + b_down is
  * rounded once (the two-kernel route rounds down + b_down first). D must be 128 or 256, F a multiple of 32.
- * rows / n_rows: as in taac_swiglu_ffn_fwd (rows of residual and out). attn_rows: NULL, or (with rows) the row of attn
- * that holds token i when attn is laid out differently (taac_front_rows).
+ * rows / n_rows, norm_folded: as in taac_swiglu_ffn_fwd (rows of residual and out). attn_rows: NULL, or (with rows) the
+ * row of attn that holds token i when attn is laid out differently (taac_front_rows).
  * Replaces: attention.out + residual add and ffn_norm + SwiGLUFeedForward.forward + residual add of
  * UnifiedInteractionBlock.forward (experiments/symbiosis/backbone.py:47, 64-67).
  */
@@ -444,7 +446,7 @@ int taac_attn_out_ffn_fwd(const void* attn, int64_t ld_attn, const void* out_bia
                           const void* residual, int64_t ldr, const void* norm_weight, float eps, const void* b_up,
                           const void* b_down, const void* packed_ffn_weights, void* out, int64_t ldo, int64_t M,
                           int32_t D, int32_t F, const int32_t* rows, const int32_t* n_rows, const int32_t* attn_rows,
-                          void* stream);
+                          int norm_folded, void* stream);
 
 /*
  * taac_attn_out_ffn_fwd with a sigmoid gate on the projected update (TokenFormer's NLIR gate):
@@ -462,7 +464,8 @@ int taac_attn_out_gate_ffn_fwd(const void* attn, int64_t ld_attn, const void* ou
                                const void* update_gate, int64_t ld_gate, const void* residual, int64_t ldr,
                                const void* norm_weight, float eps, const void* b_up, const void* b_down,
                                const void* packed_ffn_weights, void* out, int64_t ldo, int64_t M, int32_t D, int32_t F,
-                               const int32_t* rows, const int32_t* n_rows, const int32_t* attn_rows, void* stream);
+                               const int32_t* rows, const int32_t* n_rows, const int32_t* attn_rows,
+                               int norm_folded, void* stream);
 
 /*
  * Fused [RMSNorm ->] dense layer [-> + residual] with the token rows held in registers:
@@ -664,6 +667,10 @@ int taac_mask_front_bits(const uint32_t* struct_bits, int32_t T, const int32_t* 
 int64_t taac_ffn_packed_bytes(int32_t D, int32_t F);
 int taac_ffn_pack_weights(const void* w_up, const void* w_down, void* packed, int32_t D, int32_t F, int gate_first,
                           void* stream);
+/* The same blob with the weight of the RMSNorm in front of the up projection folded into its fragments
+ * (w_up[n, k] * norm_weight[k], rounded once), for the feed-forward entry points with norm_folded = 1. */
+int taac_ffn_pack_weights_norm(const void* w_up, const void* w_down, const void* norm_weight, void* packed, int32_t D,
+                               int32_t F, int gate_first, void* stream);
 int64_t taac_linear_packed_bytes(int32_t N, int32_t K);
 int taac_linear_pack_weights(const void* w, void* packed, int32_t N, int32_t K, void* stream);
 /* The same blob with the weight of an RMSNorm in front of the layer folded in (packed[n, k] = bf16(w[n, k] *

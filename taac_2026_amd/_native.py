@@ -185,12 +185,12 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "taac_swiglu_ffn_fwd": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
-         c_void_p, c_int64, c_int64, c_int32, c_int32, c_int, c_void_p, c_void_p, c_void_p],
+         c_void_p, c_int64, c_int64, c_int32, c_int32, c_int, c_void_p, c_void_p, c_int, c_void_p],
     ),
     "taac_attn_out_ffn_fwd": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
-         c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p],
+         c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     ),
     "taac_silu_mlp_packed_bytes": (c_int64, [c_int32, c_int32]),
     "taac_silu_mlp_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
@@ -202,7 +202,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "taac_attn_out_gate_ffn_fwd": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_float, c_void_p,
-         c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p],
+         c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     ),
     "taac_norm_linear_fwd": (
         c_int,
@@ -226,6 +226,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "taac_ffn_packed_bytes": (c_int64, [c_int32, c_int32]),
     "taac_ffn_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int, c_void_p]),
+    "taac_ffn_pack_weights_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int, c_void_p]),
     "taac_linear_packed_bytes": (c_int64, [c_int32, c_int32]),
     "taac_linear_pack_weights": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
     "taac_linear_pack_weights_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),

@@ -421,11 +421,13 @@ def clear_packed_weight_cache() -> None:
     _packed_cache.clear()
 
 
-def pack_ffn_weights(up_weight: torch.Tensor, down_weight: torch.Tensor, *, gate_first: bool = True) -> torch.Tensor:
+def pack_ffn_weights(up_weight: torch.Tensor, down_weight: torch.Tensor, *, gate_first: bool = True,
+                     norm_weight: torch.Tensor | None = None) -> torch.Tensor:
     """Fragment-ordered blob of ``(up_weight [2F, D], down_weight [D, F])`` for ``swiglu_ffn`` (uint8 tensor).
 
     The blob depends on ``gate_first`` (which half of ``up_weight`` goes through SiLU): pass the same value to
-    ``swiglu_ffn``."""
+    ``swiglu_ffn``. ``norm_weight`` ``[D]``: the weight of the RMSNorm in front of the up projection, folded into the
+    blob (``taac_ffn_pack_weights_norm``; the kernels are then called with ``norm_folded = 1``)."""
     library = _native.load_library()
     d_model, hidden = down_weight.shape
     nbytes = library.taac_ffn_packed_bytes(d_model, hidden)
@@ -433,11 +435,29 @@ def pack_ffn_weights(up_weight: torch.Tensor, down_weight: torch.Tensor, *, gate
         raise RuntimeError(f"pack_ffn_weights: unsupported shape D={d_model}, F={hidden}")
     up_weight, down_weight = up_weight.contiguous(), down_weight.contiguous()
     packed = torch.empty(nbytes, dtype=torch.uint8, device=up_weight.device)
-    status = library.taac_ffn_pack_weights(up_weight.data_ptr(), down_weight.data_ptr(), packed.data_ptr(), d_model,
-                                           hidden, int(bool(gate_first)),
-                                           _native.current_stream(up_weight.device))
+    if norm_weight is not None:
+        if norm_weight.shape != (d_model,):
+            raise ValueError("rms_norm weight must be 1D and match the normalized dimension")
+        status = library.taac_ffn_pack_weights_norm(up_weight.data_ptr(), down_weight.data_ptr(),
+                                                    norm_weight.contiguous().data_ptr(), packed.data_ptr(), d_model, hidden,
+                                                    int(bool(gate_first)), _native.current_stream(up_weight.device))
+    else:
+        status = library.taac_ffn_pack_weights(up_weight.data_ptr(), down_weight.data_ptr(), packed.data_ptr(), d_model,
+                                               hidden, int(bool(gate_first)),
+                                               _native.current_stream(up_weight.device))
     _native.check(status, "pack_ffn_weights")
     return packed
+
+
+def _packed_ffn(up_weight: torch.Tensor, down_weight: torch.Tensor, gate_first: bool, norm_weight: torch.Tensor | None):
+    """Cached feed-forward blob, with the weight of the norm in front of it folded in when there is one."""
+    if norm_weight is None:
+        return _packed_cache.get((up_weight, down_weight),
+                                 lambda: pack_ffn_weights(up_weight, down_weight, gate_first=gate_first),
+                                 variant=int(bool(gate_first)))
+    return _packed_cache.get((up_weight, down_weight, norm_weight),
+                             lambda: pack_ffn_weights(up_weight, down_weight, gate_first=gate_first, norm_weight=norm_weight),
+                             variant=4 + int(bool(gate_first)))
 
 
 def pack_linear_weight(weight: torch.Tensor, norm_weight: torch.Tensor | None = None) -> torch.Tensor:
@@ -614,9 +634,7 @@ def swiglu_ffn(
         gated = swiglu_linear(h, up_weight, up_bias, gate_first=gate_first)
         res_rows = residual.reshape(-1, d_model) if residual is not None else None
         return linear(gated, down_weight, down_bias, residual=res_rows).reshape(shape)
-    packed = _packed_cache.get((up_weight, down_weight),
-                               lambda: pack_ffn_weights(up_weight, down_weight, gate_first=gate_first),
-                               variant=int(bool(gate_first)))
+    packed = _packed_ffn(up_weight, down_weight, gate_first, norm_weight)
     res_rows = None
     if residual is not None:
         res_rows = residual.reshape(-1, d_model)
@@ -629,7 +647,8 @@ def swiglu_ffn(
         rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), None,
         _native.ptr(up_bias), None, _native.ptr(down_bias), packed.data_ptr(), _native.ptr(res_rows),
         res_rows.stride(0) if res_rows is not None else d_model, out.data_ptr(), d_model, rows.shape[0], d_model,
-        hidden, int(bool(gate_first)), _native.ptr(index), _native.ptr(count), _native.current_stream(x.device),
+        hidden, int(bool(gate_first)), _native.ptr(index), _native.ptr(count), int(norm_weight is not None),
+        _native.current_stream(x.device),
     )
     _native.check(status, "swiglu_ffn")
     return out.reshape(shape)
@@ -750,7 +769,7 @@ def attention_out_ffn(
     if not (_fused_width(d_model) and hidden % 32 == 0):
         raise RuntimeError("attention_out_ffn: needs model width 128 / 256 and a hidden size that is a multiple of 32")
     packed_out = _packed_cache.get((out_weight,), lambda: pack_linear_weight(out_weight))
-    packed_ffn = _packed_cache.get((up_weight, down_weight), lambda: pack_ffn_weights(up_weight, down_weight), variant=1)
+    packed_ffn = _packed_ffn(up_weight, down_weight, True, norm_weight)
     res_rows = residual.reshape(-1, d_model)
     if res_rows.stride(-1) != 1 or res_rows.stride(0) % 8 != 0:
         res_rows = res_rows.contiguous()
@@ -768,7 +787,8 @@ def attention_out_ffn(
             gate_rows.stride(0), res_rows.data_ptr(), res_rows.stride(0), _native.ptr(norm_weight), float(eps),
             _native.ptr(up_bias), _native.ptr(down_bias), packed_ffn.data_ptr(), out.data_ptr(), d_model, rows.shape[0],
             d_model, hidden, _native.ptr(index), _native.ptr(count),
-            _native.ptr(_input_rows(name, input_rows, index, rows)), _native.current_stream(attn.device),
+            _native.ptr(_input_rows(name, input_rows, index, rows)), int(norm_weight is not None),
+            _native.current_stream(attn.device),
         )
         _native.check(status, "attention_out_ffn")
         return out.reshape(shape)
@@ -776,7 +796,8 @@ def attention_out_ffn(
         rows.data_ptr(), rows.stride(0), _native.ptr(out_bias), packed_out.data_ptr(), res_rows.data_ptr(),
         res_rows.stride(0), _native.ptr(norm_weight), float(eps), _native.ptr(up_bias), _native.ptr(down_bias),
         packed_ffn.data_ptr(), out.data_ptr(), d_model, rows.shape[0], d_model, hidden, _native.ptr(index),
-        _native.ptr(count), _native.ptr(_input_rows(name, input_rows, index, rows)), _native.current_stream(attn.device),
+        _native.ptr(count), _native.ptr(_input_rows(name, input_rows, index, rows)), int(norm_weight is not None),
+        _native.current_stream(attn.device),
     )
     _native.check(status, "attention_out_ffn")
     return out.reshape(shape)

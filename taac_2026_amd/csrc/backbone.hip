@@ -667,7 +667,8 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
     if (fused && !split_out_ffn) {
       // out projection + residual and the whole feed-forward half in one kernel; the stream between them stays on chip
       if ((rc = taac_attn_out_ffn_fwd(h, D, w.out_bias, pk_out, cur, D, w.ffn_norm_weight, eps, w.up_bias, w.down_bias,
-                                      pk_ffn, x_out, D, M, D, F, rows, n_rows, nullptr, stream)) != TAAC_OK)
+                                      pk_ffn, x_out, D, M, D, F, rows, n_rows, nullptr, w.ffn_norm_weight != nullptr,
+                                      stream)) != TAAC_OK)
         return rc;
     } else if (fused) {
       if ((rc = taac_norm_linear_fwd(h, D, nullptr, eps, nullptr, w.out_bias, pk_out, cur, D, x, D, M, D, D, rows,
@@ -675,7 +676,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
         return rc;
       // feed-forward half: RMSNorm -> up -> SiLU-gate -> down -> + residual in one kernel
       if ((rc = taac_swiglu_ffn_fwd(x, D, w.ffn_norm_weight, eps, nullptr, w.up_bias, nullptr, w.down_bias, pk_ffn, x,
-                                    D, x_out, D, M, D, F, 1, rows, n_rows, stream)) != TAAC_OK)
+                                    D, x_out, D, M, D, F, 1, rows, n_rows, w.ffn_norm_weight != nullptr, stream)) != TAAC_OK)
         return rc;
     } else {
       if ((rc = taac_linear_bf16(h, D, w.out_weight, w.out_bias, cur, x, D, M, D, D, TAAC_EPI_RESIDUAL, 1, stream)) !=

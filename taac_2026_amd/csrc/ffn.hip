@@ -84,8 +84,11 @@ __host__ __device__ __forceinline__ int up_unit_of_slot(int m16) {
 // ---- fragment-order packing ------------------------------------------------------------------------------------------
 // FFN blob: step s (32 hidden units) holds, for chunk q = 0, 1: KS up fragments (k-step r) then MB down fragments
 // (row block r - KS); exactly the image one barrier step needs in LDS. A fragment is 64 lanes x 16 bytes.
+// col_scale (optional, [D]): weight of the RMSNorm in front of the up projection, folded into its fragments (see
+// linear_pack_piece).
 __device__ __forceinline__ void ffn_pack_piece(const bf16_t* __restrict__ w_up, const bf16_t* __restrict__ w_down,
-                                               bf16x8* __restrict__ packed, int D, int F, int gate_first, int64_t gid) {
+                                               bf16x8* __restrict__ packed, int D, int F, int gate_first, int64_t gid,
+                                               const bf16_t* __restrict__ col_scale = nullptr) {
   const int KS = D / 16, MB = D / 32, CFRAG = KS + MB, NFRAG = kCPB * CFRAG;
   const int lane = static_cast<int>(gid % 64);
   const int f = static_cast<int>((gid / 64) % NFRAG);
@@ -98,14 +101,21 @@ __device__ __forceinline__ void ffn_pack_piece(const bf16_t* __restrict__ w_up, 
     src = w_up + (((l32 < 16) == (gate_first != 0) ? 0 : F) + unit0 + up_unit_of_slot(l32 & 15)) * D + r * 16 + hh * 8;
   else
     src = w_down + static_cast<int64_t>((r - KS) * 32 + l32) * F + unit0 + hh * 8;
-  packed[gid] = *reinterpret_cast<const bf16x8*>(src);
+  bf16x8 v = *reinterpret_cast<const bf16x8*>(src);
+  if (col_scale != nullptr && r < KS) {
+    const bf16x8 g = *reinterpret_cast<const bf16x8*>(col_scale + r * 16 + hh * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = static_cast<bf16_t>(static_cast<float>(v[e]) * static_cast<float>(g[e]));
+  }
+  packed[gid] = v;
 }
 
 __global__ void ffn_pack_kernel(const bf16_t* __restrict__ w_up, const bf16_t* __restrict__ w_down,
-                                bf16x8* __restrict__ packed, int D, int F, int gate_first) {
+                                bf16x8* __restrict__ packed, int D, int F, int gate_first,
+                                const bf16_t* __restrict__ col_scale) {
   const int64_t total = static_cast<int64_t>(3) * D * F / 8;
   const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (gid < total) ffn_pack_piece(w_up, w_down, packed, D, F, gate_first, gid);
+  if (gid < total) ffn_pack_piece(w_up, w_down, packed, D, F, gate_first, gid, col_scale);
 }
 
 // Plain SiLU MLP blob (fc1 [F, D], fc2 [D, F]): chunk c (32 hidden units) holds KS fc1 fragments (k-step r; row slots
@@ -165,6 +175,7 @@ struct PackBatch {
   const bf16_t* qkv_norm[kPackBatch];  // weight of the RMSNorm in front of the projection (folded into its blob), or null
   const bf16_t* out[kPackBatch];
   const bf16_t* up[kPackBatch];
+  const bf16_t* ffn_norm[kPackBatch];  // weight of the RMSNorm in front of the up projection (folded into its blob), or null
   const bf16_t* down[kPackBatch];
   bf16x8* packed_qkv[kPackBatch];
   bf16x8* packed_out[kPackBatch];
@@ -179,7 +190,7 @@ __global__ void pack_blocks_kernel(const PackBatch batch, int D, int F) {
   gid -= n_qkv;
   if (gid < n_out) return linear_pack_piece(batch.out[blk], batch.packed_out[blk], D, gid);
   gid -= n_out;
-  if (gid < n_ffn) ffn_pack_piece(batch.up[blk], batch.down[blk], batch.packed_ffn[blk], D, F, 1, gid);
+  if (gid < n_ffn) ffn_pack_piece(batch.up[blk], batch.down[blk], batch.packed_ffn[blk], D, F, 1, gid, batch.ffn_norm[blk]);
 }
 
 // ---- shared pieces ---------------------------------------------------------------------------------------------------
@@ -221,8 +232,10 @@ __device__ __forceinline__ void load_token_rows(const TsParams& p, int64_t count
 }
 
 // RMS-normalises the loaded rows in place: y = bf16( x * rsqrt(mean(x^2) + eps) * w ), w read from its LDS copy.
+// folded: the norm's weight is part of the layer that consumes the rows; only the per-token factor is applied.
 template <int D, int TT>
-__device__ __forceinline__ void normalize_tokens(float eps, const bf16_t* norm_w_lds, int hh, bf16x8 (&xf)[TT][D / 16]) {
+__device__ __forceinline__ void normalize_tokens(float eps, const bf16_t* norm_w_lds, int hh, bf16x8 (&xf)[TT][D / 16],
+                                                 bool folded = false) {
   constexpr int KS = D / 16;
   float scale[TT];
 #pragma unroll
@@ -244,6 +257,17 @@ __device__ __forceinline__ void normalize_tokens(float eps, const bf16_t* norm_w
   for (int t = 0; t < TT; ++t)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(xf[t][ks]));
+  if (folded) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int t = 0; t < TT; ++t) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xf[t][ks][e] = static_cast<bf16_t>(static_cast<float>(xf[t][ks][e]) * scale[t]);
+        asm volatile("" : "+v"(xf[t][ks]));
+      }
+    return;
+  }
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     const bf16x8 wv = *reinterpret_cast<const bf16x8*>(norm_w_lds + ks * 16 + hh * 8);
@@ -536,7 +560,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  if (!OUTP && active && p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + UPB + D, hh, xf);
+  if (!OUTP && active && p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + UPB + D, hh, xf, p.norm_folded != 0);
 
   // One barrier step = CPB chunks = NFRAG fragments, consumed in their LDS order: per chunk KS up fragments, then MB
   // down fragments. Fragment reads run P fragments ahead of their MFMAs through a ring of P registers sets; the two
@@ -697,7 +721,13 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
           constexpr int ks = decltype(kc)::value;
           constexpr int mb = ks / 2, jq = 2 * (ks % 2);
           bf16x4 lo, hi;
-          if (p.norm_w != nullptr) {
+          if (p.norm_w != nullptr && p.norm_folded) {  // the norm's weight is part of the packed up projection
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              lo[e] = static_cast<bf16_t>(oacc[t][mb][jq * 4 + e] * scale);
+              hi[e] = static_cast<bf16_t>(oacc[t][mb][(jq + 1) * 4 + e] * scale);
+            }
+          } else if (p.norm_w != nullptr) {
             const bf16x4 wl = *reinterpret_cast<const bf16x4*>(nw_lds + mb * 32 + jq * 8 + hh * 4);
             const bf16x4 wh = *reinterpret_cast<const bf16x4*>(nw_lds + mb * 32 + (jq + 1) * 8 + hh * 4);
 #pragma unroll
@@ -1272,12 +1302,13 @@ int pack_backbone_blocks(const taac_block_weights* blocks, int n, int32_t D, int
     for (int i = 0; i < m; ++i) {
       const taac_block_weights& w = blocks[base + i];
       if (!ptr_ok(w.qkv_weight, 15) || !ptr_ok(w.out_weight, 15) || !ptr_ok(w.up_weight, 15) ||
-          !ptr_ok(w.down_weight, 15) || !ptr_ok(w.attn_norm_weight, 15))
+          !ptr_ok(w.down_weight, 15) || !ptr_ok(w.attn_norm_weight, 15) || !ptr_ok(w.ffn_norm_weight, 15))
         return set_error(TAAC_ERR_UNSUPPORTED, "%s: weights must be 16-byte aligned", name);
       batch.qkv[i] = static_cast<const bf16_t*>(w.qkv_weight);
       batch.qkv_norm[i] = static_cast<const bf16_t*>(w.attn_norm_weight);
       batch.out[i] = static_cast<const bf16_t*>(w.out_weight);
       batch.up[i] = static_cast<const bf16_t*>(w.up_weight);
+      batch.ffn_norm[i] = static_cast<const bf16_t*>(w.ffn_norm_weight);
       batch.down[i] = static_cast<const bf16_t*>(w.down_weight);
       batch.packed_qkv[i] = static_cast<bf16x8*>(packed_qkv[base + i]);
       batch.packed_out[i] = static_cast<bf16x8*>(packed_out[base + i]);
@@ -1298,21 +1329,43 @@ extern "C" int64_t taac_ffn_packed_bytes(int32_t D, int32_t F) {
   return static_cast<int64_t>(3) * D * F * 2;
 }
 
+namespace taac {
+namespace {
+int ffn_pack(const char* name, const void* w_up, const void* w_down, const void* norm_weight, void* packed, int32_t D,
+             int32_t F, int gate_first, void* stream);
+}
+}  // namespace taac
+
 extern "C" int taac_ffn_pack_weights(const void* w_up, const void* w_down, void* packed, int32_t D, int32_t F,
                                      int gate_first, void* stream) {
-  using namespace taac;
-  const char* name = "taac_ffn_pack_weights";
+  return taac::ffn_pack("taac_ffn_pack_weights", w_up, w_down, nullptr, packed, D, F, gate_first, stream);
+}
+
+extern "C" int taac_ffn_pack_weights_norm(const void* w_up, const void* w_down, const void* norm_weight, void* packed,
+                                          int32_t D, int32_t F, int gate_first, void* stream) {
+  const char* name = "taac_ffn_pack_weights_norm";
+  if (!norm_weight) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: null norm weight", name);
+  return taac::ffn_pack(name, w_up, w_down, norm_weight, packed, D, F, gate_first, stream);
+}
+
+namespace taac {
+namespace {
+int ffn_pack(const char* name, const void* w_up, const void* w_down, const void* norm_weight, void* packed, int32_t D,
+             int32_t F, int gate_first, void* stream) {
   if (taac_ffn_packed_bytes(D, F) < 0)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: D must be 128 or 256 and F a positive multiple of 32", name);
   if (!w_up || !w_down || !packed) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
-  if (!ptr_ok(w_up, 15) || !ptr_ok(w_down, 15) || !ptr_ok(packed, 15))
+  if (!ptr_ok(w_up, 15) || !ptr_ok(w_down, 15) || !ptr_ok(packed, 15) || !ptr_ok(norm_weight, 15))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: pointers must be 16-byte aligned", name);
   const int64_t pieces = static_cast<int64_t>(3) * D * F / 8;
   hipLaunchKernelGGL(ffn_pack_kernel, dim3(static_cast<uint32_t>((pieces + 255) / 256)), dim3(256), 0,
                      as_stream(stream), static_cast<const bf16_t*>(w_up), static_cast<const bf16_t*>(w_down),
-                     static_cast<bf16x8*>(packed), D, F, gate_first ? 1 : 0);
+                     static_cast<bf16x8*>(packed), D, F, gate_first ? 1 : 0, static_cast<const bf16_t*>(norm_weight));
   return check_launch(name);
 }
+}  // namespace
+}  // namespace taac
+
 
 extern "C" int64_t taac_linear_packed_bytes(int32_t N, int32_t K) {
   if ((K != 128 && K != 256) || N <= 0 || N % taac::kNC != 0) return -1;
@@ -1356,9 +1409,11 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
               const void* norm_weight, float eps, const void* w_up, const void* b_up, const void* w_down,
               const void* b_down, const void* packed_weights, const void* residual, int64_t ldr, void* out, int64_t ldo,
               int64_t M, int32_t D, int32_t F, int gate_first, const int32_t* rows, const int32_t* n_rows,
-              const int32_t* x_rows, void* stream, const void* update_gate = nullptr, int64_t ldg = 0,
+              const int32_t* x_rows, int norm_folded, void* stream, const void* update_gate = nullptr, int64_t ldg = 0,
               bool glu = true) {
   const bool with_proj = out_packed != nullptr;
+  if (norm_folded && (!norm_weight || !packed_weights))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: norm_folded needs the norm weight and the packed weights it was folded into", name);
   if (!glu && (with_proj || !packed_weights))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: the plain MLP takes packed weights and no projection in front", name);
   if (update_gate && !with_proj)
@@ -1414,6 +1469,7 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
   p.b0 = static_cast<const bf16_t*>(out_bias);
   p.gate = static_cast<const bf16_t*>(update_gate);
   p.ldg = ldg;
+  p.norm_folded = norm_folded ? 1 : 0;
   p.units = compute_units();
   if (p.units <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
   if (const int limit = test_max_workgroups(); limit > 0 && limit < p.units) p.units = limit;  // taac_test_hooks
@@ -1457,9 +1513,10 @@ extern "C" int taac_swiglu_ffn_fwd(const void* x, int64_t ldx, const void* norm_
                                    const void* b_up, const void* w_down, const void* b_down, const void* packed_weights,
                                    const void* residual, int64_t ldr, void* out, int64_t ldo, int64_t M, int32_t D,
                                    int32_t F, int gate_first, const int32_t* rows, const int32_t* n_rows,
-                                   void* stream) {
+                                   int norm_folded, void* stream) {
   return taac::ffn_entry("taac_swiglu_ffn_fwd", x, ldx, nullptr, nullptr, norm_weight, eps, w_up, b_up, w_down, b_down,
-                         packed_weights, residual, ldr, out, ldo, M, D, F, gate_first, rows, n_rows, nullptr, stream);
+                         packed_weights, residual, ldr, out, ldo, M, D, F, gate_first, rows, n_rows, nullptr, norm_folded,
+                         stream);
 }
 
 extern "C" int taac_attn_out_ffn_fwd(const void* attn, int64_t ld_attn, const void* out_bias,
@@ -1467,12 +1524,13 @@ extern "C" int taac_attn_out_ffn_fwd(const void* attn, int64_t ld_attn, const vo
                                      const void* norm_weight, float eps, const void* b_up, const void* b_down,
                                      const void* packed_ffn_weights, void* out, int64_t ldo, int64_t M, int32_t D,
                                      int32_t F, const int32_t* rows, const int32_t* n_rows,
-                                     const int32_t* attn_rows, void* stream) {
+                                     const int32_t* attn_rows, int norm_folded, void* stream) {
   const char* name = "taac_attn_out_ffn_fwd";
   if (!packed_out_weights || !packed_ffn_weights)
     return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: both weight sets must be packed", name);
   return taac::ffn_entry(name, attn, ld_attn, out_bias, packed_out_weights, norm_weight, eps, nullptr, b_up, nullptr,
-                         b_down, packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, attn_rows, stream);
+                         b_down, packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, attn_rows,
+                         norm_folded, stream);
 }
 
 extern "C" int64_t taac_silu_mlp_packed_bytes(int32_t D, int32_t F) {
@@ -1502,7 +1560,7 @@ extern "C" int taac_silu_mlp_fwd(const void* x, int64_t ldx, const void* norm_we
   const char* name = "taac_silu_mlp_fwd";
   if (!packed_weights) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: the weights must be packed", name);
   return taac::ffn_entry(name, x, ldx, nullptr, nullptr, norm_weight, eps, nullptr, b1, nullptr, b2, packed_weights,
-                         residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, nullptr, stream, nullptr, 0, false);
+                         residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, nullptr, 0, stream, nullptr, 0, false);
 }
 
 extern "C" int taac_attn_out_gate_ffn_fwd(const void* attn, int64_t ld_attn, const void* out_bias,
@@ -1511,14 +1569,14 @@ extern "C" int taac_attn_out_gate_ffn_fwd(const void* attn, int64_t ld_attn, con
                                           const void* b_up, const void* b_down, const void* packed_ffn_weights,
                                           void* out, int64_t ldo, int64_t M, int32_t D, int32_t F,
                                           const int32_t* rows, const int32_t* n_rows, const int32_t* attn_rows,
-                                          void* stream) {
+                                          int norm_folded, void* stream) {
   const char* name = "taac_attn_out_gate_ffn_fwd";
   if (!packed_out_weights || !packed_ffn_weights)
     return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: both weight sets must be packed", name);
   if (!update_gate) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: null gate pointer", name);
   return taac::ffn_entry(name, attn, ld_attn, out_bias, packed_out_weights, norm_weight, eps, nullptr, b_up, nullptr,
-                         b_down, packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, attn_rows, stream,
-                         update_gate, ld_gate);
+                         b_down, packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, attn_rows,
+                         norm_folded, stream, update_gate, ld_gate);
 }
 
 namespace taac {

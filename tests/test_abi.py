@@ -146,8 +146,9 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
         a.update(kw)
         return library.taac_attn_out_ffn_fwd(fake, a["d"], None, a["packed_out"], a["residual"], a["d"], None, 1e-6, None,
                                              None, a["packed_ffn"], fake, a["d"], a["m"], a["d"], a["f"], a["rows"], a["rows"],
-                                             a["attn_rows"], None)
+                                             a["attn_rows"], a.get("folded", 0), None)
 
+    assert tail(folded=1) == invalid and b"norm_folded needs" in library.taac_last_error()
     assert tail(packed_out=None) == invalid and b"packed" in library.taac_last_error()
     assert tail(packed_ffn=None) == invalid
     assert tail(residual=None) == invalid and b"block input" in library.taac_last_error()
