@@ -115,6 +115,9 @@ int taac_layernorm_bwd(const void* x, const void* w, const void* dy, void* dx, v
  * cols above TAAC_RMSNORM_BWD_STATIC_MAX_COLS are rejected with TAAC_ERR_UNSUPPORTED. The call allocates and frees
  * nothing. All calls on one GPU share the array: calls that overlap on one GPU (different streams or host threads)
  * race on it and must be serialised by the caller; calls on one stream are ordered and safe.
+ * The array's device address is looked up (hipGetSymbolAddress) by the first call on each GPU: make one ordinary call
+ * per GPU (rows = 0 is enough) before the first call under stream capture, so that the lookup, which may load the code
+ * object, does not happen inside a capture.
  */
 #define TAAC_RMSNORM_BWD_STATIC_MAX_COLS 2048
 int taac_rmsnorm_bwd_static(const void* x, const void* w, const void* dy, void* dx, void* dw, int64_t rows,

@@ -628,20 +628,24 @@ class _HipMaskedAttentionFunction(torch.autograd.Function):
         _native.check(status, "flash_attention")
         if self_factor is not None:
             out = torch.where(mask.query_self[:, None, :, None], v * self_factor[..., None], out)
-        ctx.save_for_backward(q, k, v, out, lse, *(() if key_lengths is None else (key_lengths,)))
-        ctx.mask, ctx.has_lengths, ctx.zero_padded_queries = mask, key_lengths is not None, bool(zero_padded_queries)
-        ctx.dropout_mask, ctx.dropout_scale, ctx.self_factor = dropout_mask, scale, self_factor
+        # optional tensors travel through save_for_backward as well (in-place version checks, saved-tensor hooks, and the
+        # (B, H, Tq, Tk) keep mask is released with the graph); `present` records which of them follow the fixed five
+        optional = (key_lengths, dropout_mask, self_factor)
+        ctx.save_for_backward(q, k, v, out, lse, *(t for t in optional if t is not None))
+        ctx.present = tuple(t is not None for t in optional)
+        ctx.mask, ctx.zero_padded_queries, ctx.dropout_scale = mask, bool(zero_padded_queries), scale
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
         q, k, v, out, lse, *rest = ctx.saved_tensors
-        key_lengths = rest[0] if ctx.has_lengths else None
+        rest = iter(rest)
+        key_lengths, dropout_mask, self_factor = (next(rest) if here else None for here in ctx.present)
         grad_out = _kernel_view(grad_out)
         dq, dk, dv = _dense_like(q), _dense_like(k), _dense_like(v)
         masked_attention_backward(q, k, v, out, grad_out, lse, key_lengths, ctx.mask, dq, dk, dv,
-                                  zero_padded_queries=ctx.zero_padded_queries, dropout_mask=ctx.dropout_mask,
-                                  dropout_scale=ctx.dropout_scale, self_factor=ctx.self_factor)
+                                  zero_padded_queries=ctx.zero_padded_queries, dropout_mask=dropout_mask,
+                                  dropout_scale=ctx.dropout_scale, self_factor=self_factor)
         return dq, dk, dv, None, None, None, None, None
 
 
@@ -861,17 +865,25 @@ class _RotaryFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, query, key, num_heads: int, rope_base: float):
-        ctx.config = (int(num_heads), float(rope_base))
+        ctx.config = (int(num_heads), float(rope_base), query.shape, key.shape, query.dtype, query.device)
         with torch.no_grad():
             return qk_norm_rope(query.detach(), key.detach(), None, None, num_heads=num_heads, rope_base=rope_base)
 
     @staticmethod
     def backward(ctx, grad_query, grad_key):
-        num_heads, rope_base = ctx.config
+        num_heads, rope_base, query_shape, key_shape, dtype, device = ctx.config
+        if grad_query is None and grad_key is None:
+            return None, None, None, None
+        # only one of the two outputs fed the loss: the pass rotates both, so the other one's gradient enters as zeros
+        has_query, has_key = grad_query is not None, grad_key is not None
+        if not has_query:
+            grad_query = torch.zeros(query_shape, dtype=dtype, device=device)
+        if not has_key:
+            grad_key = torch.zeros(key_shape, dtype=dtype, device=device)
         with torch.no_grad():
             grad_query, grad_key = qk_norm_rope(grad_query.contiguous(), grad_key.contiguous(), None, None, num_heads=num_heads,
                                                 rope_base=rope_base, inverse_rotation=True)
-        return grad_query, grad_key, None, None
+        return (grad_query if has_query else None), (grad_key if has_key else None), None, None
 
 
 def qk_norm_rope_autograd(query: torch.Tensor, key: torch.Tensor, query_weight: torch.Tensor | None,

@@ -117,6 +117,11 @@ def swiglu_backward(pre_activation: torch.Tensor, grad_hidden: torch.Tensor | No
             None if grad is None else grad.reshape(*shape[:-1], 2 * hidden_size))
 
 
+def swiglu_ffn_backward_supported(d_model: int, hidden_size: int) -> bool:
+    """Whether ``swiglu_ffn_backward_hidden`` covers these widths (its weight steps must fit the LDS, which bounds F)."""
+    return int(_native.load_library().taac_swiglu_ffn_bwd_packed_bytes(int(d_model), int(hidden_size))) >= 0
+
+
 def swiglu_ffn_backward_hidden(h: torch.Tensor, grad_out: torch.Tensor, up_weight: torch.Tensor,
                                up_bias: torch.Tensor | None, down_weight: torch.Tensor, *,
                                gate_first: bool = True) -> tuple[torch.Tensor, torch.Tensor] | None:

@@ -22,7 +22,7 @@ import torch.nn as nn
 from taac_2026_amd import _native
 from taac_2026_amd.accelerators.attention import StructuredAttentionMask, front_structured_mask, qk_norm_rope, rope_table
 from taac_2026_amd.accelerators.linear import (attention_out_ffn, front_rows, norm_linear, qkv_projection, silu_mlp,
-                                               swiglu_ffn, swiglu_ffn_dropout, valid_rows)
+                                               swiglu_ffn, swiglu_ffn_backward_supported, swiglu_ffn_dropout, valid_rows)
 from taac_2026_amd.accelerators.tensor_validation import require_cuda_tensors, require_inference
 from taac_2026_amd.modeling.block_training import run_training_block, training_route_applies
 from taac_2026_amd.modeling.normalization import RMSNorm
@@ -185,10 +185,12 @@ class UnifiedSelfAttention(nn.Module):
             query, key, value = _dense(self.qkv, x).chunk(3, dim=-1)
             query, key = qk_norm_rope(query, key, query_weight, key_weight, num_heads=self.num_heads, eps=qk_eps,
                                       rope_base=self.rope_base)
-        elif prepare and dtype == torch.bfloat16 and x.ndim == 3 and x.shape[-1] in (128, 256):
+        elif (prepare and dtype == torch.bfloat16 and x.ndim == 3 and x.shape[-1] in (128, 256)
+              and not (self.training and self.dropout > 0.0)):
             # the norm statistic (and, with a rotation, weight and rotation) come out of the projection's epilogue; the
             # per-token factor of the norm and the weights of the unrotated case are applied inside the attention
-            # kernel: no pass over q and k at all
+            # kernel: no pass over q and k at all (the attention call with dropout takes no row factors: a train-mode
+            # block with dropout goes through the explicit pass below, also when nothing requires a gradient)
             qkv, q_row_scale, k_row_scale, q_col_scale = qkv_projection(
                 x, _bf16(self.qkv.weight), _bf16(self.qkv.bias), num_heads=self.num_heads, query_weight=query_weight,
                 key_weight=key_weight, qk_eps=qk_eps, rope_base=self.rope_base,
@@ -231,6 +233,19 @@ class BFTSAttention(UnifiedSelfAttention):
         self.rope_base = float(rope_base) if use_rope else None
 
 
+# Debugging aid: verify on every block call that padding_mask is the prefix mask of key_lengths (see the block's docstring).
+CHECK_PADDING_CONTRACT = False
+
+
+def check_padding_contract(padding_mask: torch.Tensor, key_lengths: torch.Tensor) -> None:
+    """Raise ValueError unless ``padding_mask[b, t] == (t >= key_lengths[b])`` everywhere (synchronises the device)."""
+    positions = torch.arange(padding_mask.shape[1], device=padding_mask.device)
+    expected = positions[None, :] >= key_lengths.to(padding_mask.device)[:, None]
+    if padding_mask.shape != expected.shape or not bool((padding_mask.bool() == expected).all()):
+        raise ValueError("padding_mask is not the prefix mask of key_lengths: the routes that walk the valid rows of "
+                         "key_lengths and the layer-by-layer route would disagree")
+
+
 class UnifiedInteractionBlock(nn.Module):
     """Pre-RMSNorm self-attention and SwiGLU feed-forward with residuals masked at padded positions
     (experiments/symbiosis/backbone.py:51-68).
@@ -241,6 +256,11 @@ class UnifiedInteractionBlock(nn.Module):
     kernel, and with ``return_attention_tokens=False`` the out projection, both residual adds, ``ffn_norm`` and the
     feed-forward are one kernel. ``attention_mask`` may be a dense bool mask, a :class:`StructuredAttentionMask`
     (what ``MetadataAttentionMask`` returns) or None; ``key_lengths`` states prefix padding without a mask.
+    Contract of ``key_lengths``: when it is given, ``padding_mask`` must be exactly its prefix mask
+    (``padding_mask[b, t] == (t >= key_lengths[b])``) - the fused route and the training route take the valid rows from
+    ``key_lengths`` alone and never read ``padding_mask``, while the layer-by-layer route multiplies the updates by
+    ``~padding_mask``. ``taac_2026_amd.modeling.backbone.CHECK_PADDING_CONTRACT = True`` makes ``forward`` verify this
+    (one device synchronisation per call: a debugging aid, off by default) and raise ``ValueError`` on a mismatch.
     ``inplace=True`` lets the fused route update ``tokens`` itself instead of a copy. ``token_layout``: ``"front"``
     (default) lets the fused route move every sample's valid tokens to the front of its rows for the attention call
     when the mask allows it, ``"positions"`` keeps them where they are (comparison route; same results)."""
@@ -370,6 +390,8 @@ class UnifiedInteractionBlock(nn.Module):
         return_attention_tokens: bool = True,
         inplace: bool = False,
     ) -> tuple[torch.Tensor, torch.Tensor | None]:
+        if CHECK_PADDING_CONTRACT and key_lengths is not None:
+            check_padding_contract(padding_mask, key_lengths)
         if self._fused_route(tokens):
             return self._forward_fused(tokens, padding_mask, attention_mask, key_lengths, return_attention_tokens, inplace)
         if torch.is_grad_enabled() and training_route_applies(self, tokens, attention_mask, key_lengths, padding_mask):
@@ -407,6 +429,8 @@ class TokenFormerBlock(UnifiedInteractionBlock):
     def forward(self, tokens: torch.Tensor, padding_mask: torch.Tensor,
                 attention_mask: torch.Tensor | StructuredAttentionMask | None, *, key_lengths: torch.Tensor | None = None,
                 inplace: bool = False) -> torch.Tensor:
+        if CHECK_PADDING_CONTRACT and key_lengths is not None:
+            check_padding_contract(padding_mask, key_lengths)
         if self._fused_route(tokens) and self.ffn.gate_first:
             return self._forward_fused(tokens, padding_mask, attention_mask, key_lengths, False, inplace)[0]
         keep = (~padding_mask).unsqueeze(-1)
@@ -570,9 +594,11 @@ class PCVRBackbone(nn.Module):
             raise ValueError("key_lengths must have shape (batch,)")
         head_dim = self.d_model // self.num_heads
         if self.rope_base is not None or self.d_model not in (128, 256) or head_dim not in (32, 64) or self.d_ff % 32 != 0 \
-                or any(p.dtype not in (torch.bfloat16, torch.float32) for p in self.parameters()):
+                or any(p.dtype not in (torch.bfloat16, torch.float32) for p in self.parameters()) \
+                or not swiglu_ffn_backward_supported(self.d_model, self.d_ff):
             raise RuntimeError(f"{name}: the training route covers bf16 (or float32 master) parameters, d_model 128 / 256, "
-                               "head dims 32 / 64, d_ff a multiple of 32 and no rotary embedding")
+                               "head dims 32 / 64, d_ff a multiple of 32 within the backward kernel's bound "
+                               "(taac_swiglu_ffn_bwd_packed_bytes) and no rotary embedding")
         if key_lengths.dtype != torch.int32 or not key_lengths.is_contiguous():
             key_lengths = key_lengths.to(torch.int32).contiguous()
         stream = emb

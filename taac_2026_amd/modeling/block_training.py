@@ -372,8 +372,8 @@ def training_route_applies(block, tokens: torch.Tensor, attention_mask, key_leng
         return False
     if (attention.query_norm is None) != (attention.key_norm is None):
         return False
-    if ffn.down.weight.shape[1] % 32 != 0:
-        return False
+    if ffn.down.weight.shape[1] % 32 != 0 or not _linear.swiglu_ffn_backward_supported(width, ffn.down.weight.shape[1]):
+        return False  # (the forward kernels take any such F; the backward's hidden-state kernel bounds it)
     if block.training and (attention.dropout > 0.0 or ffn.dropout.p > 0.0):
         return False
     if key_lengths is not None and (key_lengths.dtype != torch.int32 or not key_lengths.is_cuda

@@ -11,11 +11,22 @@ from taac_2026_amd import _native
 pytestmark = pytest.mark.gpu
 
 
-def _call_pair(device, rows, cols, dtype, seed):
+def _unaligned(t: torch.Tensor, device) -> torch.Tensor:
+    """A contiguous device copy of ``t`` whose base address is one element past a 16-byte boundary."""
+    flat = torch.empty(t.numel() + 1, dtype=t.dtype, device=device)
+    view = flat[1:].view(t.shape)
+    view.copy_(t)
+    assert view.data_ptr() % 16 != 0
+    return view
+
+
+def _call_pair(device, rows, cols, dtype, seed, *, unaligned=False, check_oracle=False):
     g = torch.Generator().manual_seed(seed)
-    x = torch.randn(rows, cols, generator=g).to(dtype).to(device)
-    w = (1 + 0.1 * torch.randn(cols, generator=g)).to(dtype).to(device)
-    dy = torch.randn(rows, cols, generator=g).to(dtype).to(device)
+    place = (lambda t: _unaligned(t, device)) if unaligned else (lambda t: t.to(device))
+    x_cpu = torch.randn(rows, cols, generator=g).to(dtype)
+    w_cpu = (1 + 0.1 * torch.randn(cols, generator=g)).to(dtype)
+    dy_cpu = torch.randn(rows, cols, generator=g).to(dtype)
+    x, w, dy = place(x_cpu), place(w_cpu), place(dy_cpu)
     library = _native.load_library()
     stream = _native.current_stream(device)
     code = _native.dtype_code(dtype)
@@ -31,6 +42,14 @@ def _call_pair(device, rows, cols, dtype, seed):
     assert torch.equal(dx, dx_ref), (rows, cols, dtype)
     assert torch.equal(dw, dw_ref), (rows, cols, dtype)
     assert torch.isfinite(dw.float()).all()
+    if check_oracle:  # float64 autograd of the oracle's closed form from the stored (rounded) inputs
+        import oracle.reference as oracle
+
+        xr, wr = x_cpu.double().requires_grad_(True), w_cpu.double().requires_grad_(True)
+        oracle.rms_norm(xr, wr, 1e-6).backward(dy_cpu.double())
+        tol = 3e-2 if dtype == torch.bfloat16 else 1e-4
+        torch.testing.assert_close(dx.cpu().double(), xr.grad, rtol=tol, atol=tol)
+        torch.testing.assert_close(dw.cpu().double(), wr.grad, rtol=tol, atol=tol * max(1.0, wr.grad.abs().max().item()))
 
 
 def test_static_scratch_variant_matches_the_workspace_variant(device):
@@ -41,6 +60,9 @@ def test_static_scratch_variant_matches_the_workspace_variant(device):
     # a width that takes the generic kernel, fp32, then a wide fp32 row
     _call_pair(device, 300, 100, torch.float32, seed=3)
     _call_pair(device, 64, 2048, torch.float32, seed=4)
+    # the generic kernel with 16-bit rows of an odd width at base addresses off the 16-byte grid, against the oracle too
+    _call_pair(device, 1201, 101, torch.bfloat16, seed=5, unaligned=True, check_oracle=True)
+    _call_pair(device, 97, 7, torch.bfloat16, seed=6, unaligned=True, check_oracle=True)
 
 
 def test_static_scratch_variant_rejects_widths_beyond_the_array(device):
