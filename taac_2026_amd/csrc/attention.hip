@@ -69,6 +69,9 @@ struct AttnParams {
   uint32_t total;  // workgroups
   uint32_t nqc_magic, h_magic;  // floor(2^32 / nqc), floor(2^32 / H) (0 for a divisor of 1): divisions without a divide
   uint32_t nqt_magic;           // the same for the number of 32-query tiles
+  // direct-transfer kernel: whether a workgroup takes a pair of query blocks, workgroups per (batch, head), their grid
+  int32_t pair_blocks;
+  uint32_t nqg, nqg_magic, total_g;
 };
 
 // x / d and x % d for a divisor known to the host: q = mulhi(x, floor(2^32 / d)) is at most two short of the quotient.
@@ -591,16 +594,17 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   constexpr int NBUF = 3;                           // chunk c is consumed while c + 1 and c + 2 are in flight
   __shared__ __attribute__((aligned(1024))) uint8_t smem[NBUF * BUF_BYTES > OT_BYTES ? NBUF * BUF_BYTES : OT_BYTES];
 
-  const uint32_t logical = xcd_remap(blockIdx.x, p.total);
-  uint32_t bh_u, qc_u, b_u, h_u;
-  magic_divmod(logical, p.nqc, p.nqc_magic, bh_u, qc_u);
+  // A workgroup takes two query blocks of one (sample, head), g and nqc - 1 - g (one, for the middle block of an odd
+  // count): under key lengths the first is the one more likely to hold valid queries, so few workgroups find nothing to
+  // do (a workgroup that only learns from the sample's length that it is idle has held its registers and LDS for two
+  // memory latencies), and under a causal mask the pair's work is the same for every g.
+  const uint32_t logical = xcd_remap(blockIdx.x, p.total_g);
+  uint32_t bh_u, qg_u, b_u, h_u;
+  magic_divmod(logical, p.nqg, p.nqg_magic, bh_u, qg_u);
   magic_divmod(bh_u, static_cast<uint32_t>(p.H), p.h_magic, b_u, h_u);
-  const int qc = static_cast<int>(qc_u), h = static_cast<int>(h_u), b = static_cast<int>(b_u);
-  const int tid = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int lane = tid % kWave;
-  const int l32 = lane % 32;
-  const int hh = lane / 32;
+  const int h = static_cast<int>(h_u), b = static_cast<int>(b_u);
+  const int qc_a = static_cast<int>(qg_u);
+  const int qc_b = p.pair_blocks ? static_cast<int>(p.nqc) - 1 - qc_a : qc_a;
 
   const T* qb = static_cast<const T*>(p.q) + b * p.qs[0] + h * p.qs[1];
   const T* kb = static_cast<const T*>(p.k) + b * p.ks[0] + h * p.ks[1];
@@ -612,8 +616,20 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
     len = p.key_lengths[b];
     len = len < 0 ? 0 : (len > p.Tk ? p.Tk : len);
   }
-  const int q_begin = qc * kQB;
   const int q_valid = p.zero_pad ? (len < p.Tq ? len : p.Tq) : p.Tq;
+  // One query block. The body is instantiated once per block of the pair (no loop around it: a loop's preheader
+  // collects constants and lane offsets in registers for the whole kernel), and everything a block derives from the lane
+  // index is derived from an opaque copy of it, so that the second instance shares no vector register with the first
+  // (the kernel lives on its 96 registers: five wavefronts per SIMD).
+  auto block = [&](const int qc, auto second_tag) __attribute__((always_inline)) {
+  uint32_t opaque_tid = threadIdx.x;
+  if constexpr (decltype(second_tag)::value) asm volatile("" : "+v"(opaque_tid));
+  const int tid = static_cast<int>(opaque_tid & (kThreads - 1));
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int lane = tid % kWave;
+  const int l32 = lane % 32;
+  const int hh = lane / 32;
+  const int q_begin = qc * kQB;
   vec_t zero_vec;
 #pragma unroll
   for (int e = 0; e < 8; ++e) zero_vec[e] = static_cast<T>(0.f);
@@ -622,7 +638,7 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
       for (int idx = tid; idx < kQB; idx += kThreads)
         if (q_begin + idx < p.Tq) p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Tq + q_begin + idx] = -INFINITY;
     }
-    if (p.zero_pad == 2) return;
+    if (p.zero_pad == 2) return;  // the blocks behind this one lie in the padding as well
     for (int idx = tid; idx < kQB * C8; idx += kThreads) {
       const int row = q_begin + idx / C8;
       if (row < p.Tq) *reinterpret_cast<vec_t*>(ob + row * p.os[2] + (idx % C8) * 8) = zero_vec;
@@ -800,16 +816,19 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
         // the same slots of every query - so the masked scores leave the matrix unit at about -2^33 (16-bit floats: -2^18)
         // and their probabilities are exact zeros. Two vector instructions per tile instead of two per score register.
         // (the operands are formed here, from the thread index, so that nothing of them is live across the chunk loop)
-        uint32_t t = threadIdx.x;
+        // (the two constants sit in scalar registers: as vector-register literals they would be hoisted out of the loop)
+        uint32_t t = static_cast<uint32_t>(tid);
         asm volatile("" : "+v"(t));
+        uint32_t masked_pair = kMaskedKeyPair, one_pair = kOnePair;
+        asm volatile("" : "+s"(masked_pair), "+s"(one_pair));
         const bool lower = (t & 32u) == 0u;
-        const uint32_t one = lower ? kOnePair : 0u;
+        const uint32_t one = lower ? one_pair : 0u;
         const u32x4 b_bits = {one, one, one, one};
         const int key0 = kc0 + static_cast<int>(t & 31u);
 #pragma unroll
         for (int kt = 0; kt < NT; ++kt) {
           if (kc0 + kt * 32 + 32 > kv_end) {  // wavefront-uniform
-            const uint32_t bits = (lower && key0 + kt * 32 >= kv_end) ? kMaskedKeyPair : 0u;
+            const uint32_t bits = (lower && key0 + kt * 32 >= kv_end) ? masked_pair : 0u;
             const u32x4 a_bits = {bits, bits, bits, bits};
             sacc[kt] = Mfma32<T>::run(__builtin_bit_cast(vec_t, a_bits), __builtin_bit_cast(vec_t, b_bits), sacc[kt]);
           }
@@ -966,6 +985,12 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
     const int q_row = q_begin + wave * 32 + row;
     const vec_t v = *reinterpret_cast<const vec_t*>(tile + row * OROW + c8 * 16);
     if (q_row < q_store_end) *reinterpret_cast<vec_t*>(ob + q_row * p.os[2] + c8 * 8) = v;
+  }
+  };
+  block(qc_a, std::false_type{});
+  if (qc_b != qc_a) {
+    __syncthreads();  // the second block's first chunks land in the buffers the output tiles were read from
+    block(qc_b, std::true_type{});
   }
 }
 
@@ -1297,17 +1322,17 @@ void launch(const AttnParams& p, bool causal, bool register_staging, hipStream_t
                                 p.block_any == nullptr;
     if (p.d == DP && (p.struct_bits == nullptr || structure_only) && dma_staging && small_offsets && p.drop_mask == nullptr) {
       if (structure_only && scaled)
-        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, true, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, true, true>), dim3(p.total_g), dim3(kThreads), 0, s, p);
       else if (structure_only)
-        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, false, true>), dim3(p.total), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, false, true>), dim3(p.total_g), dim3(kThreads), 0, s, p);
       else if (causal && scaled)
-        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, true, true, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, true, true, false>), dim3(p.total_g), dim3(kThreads), 0, s, p);
       else if (causal)
-        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, true, false, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, true, false, false>), dim3(p.total_g), dim3(kThreads), 0, s, p);
       else if (scaled)
-        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, true, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, true, false>), dim3(p.total_g), dim3(kThreads), 0, s, p);
       else
-        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, false, false>), dim3(p.total), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((flash_attn_fwd_dma_kernel<T, DP, false, false, false>), dim3(p.total_g), dim3(kThreads), 0, s, p);
       return;
     }
   }
@@ -1472,6 +1497,12 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   p.nqc_magic = magic_of(p.nqc);
   p.h_magic = magic_of(static_cast<uint32_t>(H));
   p.nqt_magic = magic_of(static_cast<uint32_t>((Tq + 31) / 32));
+  // Pairs of query blocks per workgroup where blocks differ in work or may be empty (key lengths, a causal triangle);
+  // with neither, every block is the same and single blocks fill the last round of the launch better.
+  p.pair_blocks = (p.nqc > 1 && (key_lengths != nullptr || is_causal != 0)) ? 1 : 0;
+  p.nqg = p.pair_blocks ? (p.nqc + 1) / 2 : p.nqc;
+  p.nqg_magic = magic_of(p.nqg);
+  p.total_g = p.nqg * static_cast<uint32_t>(B) * static_cast<uint32_t>(H);
 
   hipStream_t s = as_stream(stream);
   if (dtype == TAAC_BF16)

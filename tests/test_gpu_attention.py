@@ -53,6 +53,32 @@ def test_key_lengths_bf16(device, dim, tokens):
         assert got_zero[b, :, int(lengths[b]):].abs().max().item() == 0.0 if lengths[b] < tokens else True
 
 
+@pytest.mark.parametrize("dim", [32, 64])
+@pytest.mark.parametrize("tokens", [129, 300, 512, 640])
+def test_workgroups_that_take_two_query_blocks(device, dim, tokens):
+    """Under key lengths (or a causal triangle) a workgroup of the direct-transfer kernel takes query blocks g and
+    nqc - 1 - g: 2, 3, 4 and 5 blocks of 128 queries here (odd counts leave the middle block alone), with samples whose
+    second block is full, partly valid, empty, and whose first block is empty too."""
+    batch, heads = 6, 2
+    q, k, v = _qkv(batch, heads, tokens, tokens, dim, torch.bfloat16, 7 * tokens + dim)
+    lengths = torch.tensor([tokens, 0, 1, 128, min(tokens, 200), tokens - 1], dtype=torch.int32)
+    for zero_pad in (False, True):
+        expected = oracle.attention(q, k, v, lengths, zero_padded_queries=zero_pad)
+        got = _run(q, k, v, device, key_lengths=lengths.to(device), zero_padded_queries=zero_pad)
+        torch.testing.assert_close(got.float(), expected.float(), **BF16_TOL)
+    # rows left alone (the backbone's mode): the valid rows as above
+    got = _run(q, k, v, device, key_lengths=lengths.to(device), zero_padded_queries=2)
+    expected = oracle.attention(q, k, v, lengths, zero_padded_queries=True)
+    for b in range(batch):
+        n = int(lengths[b])
+        torch.testing.assert_close(got[b, :, :n].float(), expected[b, :, :n].float(), **BF16_TOL)
+    # the causal triangle pairs blocks as well (no key lengths: every sample full)
+    causal = torch.ones(tokens, tokens, dtype=torch.bool).tril()
+    want = oracle.sdpa(q.float(), k.float(), v.float(), attn_mask=causal[None, None])
+    got = _run(q, k, v, device, is_causal=True)
+    torch.testing.assert_close(got.float(), want, **BF16_TOL)
+
+
 def test_cross_attention_lengths_differ(device):
     q, k, v = _qkv(2, 3, 5, 7, 8, torch.bfloat16, 11)
     got = _run(q, k, v, device)
