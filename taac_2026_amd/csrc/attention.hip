@@ -591,7 +591,10 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   constexpr int OROW = DP * 2 + 16;
   constexpr int OT_BYTES = (kThreads / kWave) * 32 * OROW;
   static_assert(kKC * C8 % kThreads == 0, "whole transfers per wavefront");
-  constexpr int NBUF = 3;                           // chunk c is consumed while c + 1 and c + 2 are in flight
+  // Head dim 32: three chunk buffers, chunk c is consumed while c + 1 and c + 2 are in flight. Head dim 64: two (a chunk is
+  // 16 KB: with three a compute unit holds three workgroups, with two it holds as many as the registers allow), chunk c + 1
+  // is requested once every wavefront has left chunk c - 1.
+  constexpr int NBUF = DP == 64 ? 2 : 3;
   __shared__ __attribute__((aligned(1024))) uint8_t smem[NBUF * BUF_BYTES > OT_BYTES ? NBUF * BUF_BYTES : OT_BYTES];
 
   // A workgroup takes two query blocks of one (sample, head), g and nqc - 1 - g (one, for the middle block of an odd
@@ -784,7 +787,8 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   auto step = [&](int chunk, auto nt_tag) {
     constexpr int NT = decltype(nt_tag)::value;
     // this wavefront's pieces of the chunk have landed (the next chunk's, issued after them, may still be in flight) ...
-    if (chunk + 1 < nchunks && !scale_keys)
+    // (two buffers: only chunk 1, requested with chunk 0 in front of the loop, can be in flight behind the awaited one)
+    if (chunk + 1 < nchunks && !scale_keys && (NBUF == 3 || chunk == 0))
       vm_wait<kInFlight>();
     else
       vm_wait<0>();
@@ -793,12 +797,13 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
       mw[0] = (chunk & 1) ? mw_odd[0] : mw_even[0];
       mw[1] = (chunk & 1) ? mw_odd[1] : mw_even[1];
     }
-    const bool more = chunk + 2 < nchunks;
-    const int ahead = buf == 0 ? 2 : buf - 1;  // (buf + 2) % 3
-    if (more) issue(chunk + 2, ahead);
+    // the chunk requested now: two ahead into the buffer (buf + 2) % 3, or the next one into the buffer left last
+    const bool more = NBUF == 3 ? chunk + 2 < nchunks : (chunk >= 1 && chunk + 1 < nchunks);
+    const int ahead = NBUF == 3 ? (buf == 0 ? 2 : buf - 1) : 1 - buf;
+    if (more) issue(NBUF == 3 ? chunk + 2 : chunk + 1, ahead);
     const int kc0 = chunk * kKC;
     const uint32_t base = smem_off + buf * BUF_BYTES;
-    buf = buf == 2 ? 0 : buf + 1;
+    buf = buf == NBUF - 1 ? 0 : buf + 1;
     if constexpr (NT > 0) {
       f32x16 sacc[NT];
 #pragma unroll
