@@ -93,11 +93,12 @@ def _native_replay(fn):
     if not calls:
         raise SystemExit("bench.py: the operator made no library call to replay")
 
-    def replay(_keep=result):
+    def replay():
         for function, args in calls:
             if function(*args) != 0:
                 raise SystemExit("bench.py: a replayed library call failed: " + library.taac_last_error().decode())
 
+    replay.result = result  # what fn returned: kept alive with the callable, and the buffer the replays write
     return replay
 
 
@@ -171,42 +172,50 @@ def _kernel_breakdown(inputs, device, iters: int) -> dict:
     """Stand-alone timing of each kernel of one block at the step's shapes (HIP events on the launch stream around
     back-to-back replays of the library calls). The dense layers walk the valid tokens only, as they do inside the step;
     their algorithmic work counts those tokens."""
-    from taac_2026_amd.api import attention_out_ffn, norm_linear, scaled_dot_product_attention, swiglu_ffn, valid_rows
+    from taac_2026_amd.accelerators.attention import hip_flash_attention_kernel
+    from taac_2026_amd.api import attention_out_ffn_heads, norm_linear, norm_linear_heads, swiglu_ffn, valid_rows
 
     B, T, D = inputs.emb.shape
     M, F, H = B * T, inputs.d_ff, inputs.num_heads
+    dh = D // H
     w = {k: v.to(device) for k, v in inputs.blocks[0].items()}
     x = inputs.emb.to(device)
     lengths = inputs.key_lengths.to(device)
     out: dict[str, dict] = {}
     with torch.no_grad():
         index = valid_rows(lengths, T)
-        qkv = norm_linear(x, w["qkv.weight"], w["qkv.bias"], norm_weight=w["attn_norm.weight"], token_rows=index)
+        # q | k | v and the attention output as the step keeps them: one plane [M, dh] per head
+        qkv = norm_linear_heads(x, w["qkv.weight"], w["qkv.bias"], head_dim=dh, norm_weight=w["attn_norm.weight"],
+                                token_rows=index)
+        q, k, v = (qkv.view(3, H, B, T, dh)[i].transpose(0, 1) for i in range(3))
         buf = torch.zeros_like(x)  # output buffer of the [M, D] layers (rows outside the index are never touched)
-        q, k, v = qkv.chunk(3, dim=-1)
-        attn = lambda: scaled_dot_product_attention(q, k, v, num_heads=H, attn_mask=None, dropout_p=0.0,  # noqa: E731
-                                                    training=False, key_lengths=lengths, zero_padded_queries=True)
-        a = attn()
+        # rows of padded queries are skipped, as in the step (the block's last kernel never reads them)
+        attn = _native_replay(lambda: hip_flash_attention_kernel(q, k, v, lengths, zero_padded_queries=2))
+        a = attn.result.transpose(0, 1)               # [H, B, T, dh], contiguous: the output keeps q's layout
+        if not a.is_contiguous():
+            raise SystemExit("bench.py: the attention output did not keep the plane layout")
+        a = a.reshape(H, M, dh)
+        a_rows = a.permute(1, 0, 2).reshape(B, T, D)  # row-major copy for the split route's out projection
         valid_tokens = float(lengths.sum().item())
         Mv = valid_tokens
         sum_sq = float((lengths.double() ** 2).sum().item())
-        dh = D // H
         # (callable, algorithmic flops, algorithmic HBM bytes) per launch; bf16 = 2 bytes per element
         cases = {
-            "rmsnorm_qkv": (lambda: norm_linear(x, w["qkv.weight"], w["qkv.bias"], norm_weight=w["attn_norm.weight"],
-                                                token_rows=index, out=qkv),
+            "rmsnorm_qkv": (lambda: norm_linear_heads(x, w["qkv.weight"], w["qkv.bias"], head_dim=dh,
+                                                      norm_weight=w["attn_norm.weight"], token_rows=index, out=qkv),
                             2.0 * Mv * 3 * D * D, 2.0 * (Mv * D + 3 * D * D + Mv * 3 * D)),
-            # useful work only: visible (query, key) pairs; Q/K/V valid rows read, O written in full
-            "attention": (attn, 4.0 * H * dh * sum_sq, 2.0 * (3 * D * valid_tokens + M * D)),
+            # useful work only: visible (query, key) pairs; Q / K / V valid rows read, O valid rows written
+            "attention": (attn, 4.0 * H * dh * sum_sq, 2.0 * 4 * D * valid_tokens),
             # out projection + residual and the feed-forward half, one kernel: reads the attention output and the block
             # input, writes the block output; the residual stream between the two halves stays on chip
             "out_residual_rmsnorm_swiglu_ffn_residual": (
-                lambda: attention_out_ffn(a, w["out.weight"], w["out.bias"], x, w["up.weight"], w["up.bias"],
-                                          w["down.weight"], w["down.bias"], norm_weight=w["ffn_norm.weight"],
-                                          token_rows=index, out=buf),
+                lambda: attention_out_ffn_heads(a, w["out.weight"], w["out.bias"], x, w["up.weight"], w["up.bias"],
+                                                w["down.weight"], w["down.bias"], norm_weight=w["ffn_norm.weight"],
+                                                token_rows=index, out=buf),
                 2.0 * Mv * (D * D + 3 * D * F), 2.0 * (3 * Mv * D + D * D + 3 * D * F)),
-            # the same two halves as kernels of their own (the split_out_ffn=True route; not part of the step)
-            "split:out_residual": (lambda: norm_linear(a, w["out.weight"], w["out.bias"], residual=x, token_rows=index, out=buf),
+            # the same two halves as kernels of their own (the split_out_ffn=True route, row-major; not part of the step)
+            "split:out_residual": (lambda: norm_linear(a_rows, w["out.weight"], w["out.bias"], residual=x, token_rows=index,
+                                                       out=buf),
                                    2.0 * Mv * D * D, 2.0 * (3 * Mv * D + D * D)),
             "split:rmsnorm_swiglu_ffn_residual": (
                 lambda: swiglu_ffn(x, w["up.weight"], w["up.bias"], w["down.weight"], w["down.bias"], residual=x,
@@ -222,13 +231,14 @@ def _kernel_breakdown(inputs, device, iters: int) -> dict:
         # launch repeated on its own (inputs cold in the caches, no neighbours).
         x_work = x.clone()
         sequence = {
-            "rmsnorm_qkv": _native_replay(lambda: norm_linear(x_work, w["qkv.weight"], w["qkv.bias"],
-                                                              norm_weight=w["attn_norm.weight"], token_rows=index, out=qkv)),
-            "attention": _native_replay(attn),
+            "rmsnorm_qkv": _native_replay(lambda: norm_linear_heads(x_work, w["qkv.weight"], w["qkv.bias"], head_dim=dh,
+                                                                    norm_weight=w["attn_norm.weight"], token_rows=index,
+                                                                    out=qkv)),
+            "attention": attn,
             "out_residual_rmsnorm_swiglu_ffn_residual": _native_replay(
-                lambda: attention_out_ffn(a, w["out.weight"], w["out.bias"], x_work, w["up.weight"], w["up.bias"],
-                                          w["down.weight"], w["down.bias"], norm_weight=w["ffn_norm.weight"],
-                                          token_rows=index, out=x_work)),
+                lambda: attention_out_ffn_heads(a, w["out.weight"], w["out.bias"], x_work, w["up.weight"], w["up.bias"],
+                                                w["down.weight"], w["down.bias"], norm_weight=w["ffn_norm.weight"],
+                                                token_rows=index, out=x_work)),
         }
 
         def run_blocks(skip: str | None, blocks: int = 8) -> float:
@@ -250,7 +260,7 @@ def _kernel_breakdown(inputs, device, iters: int) -> dict:
             diffs = sorted(run_blocks(None) - run_blocks(name) for _ in range(max(5, iters)))
             in_sequence[name] = diffs[len(diffs) // 2]
         for name, (fn, flops, nbytes) in cases.items():
-            standalone = _event_ms(sequence["attention"] if fn is attn else _native_replay(fn), 5 * iters, 5)
+            standalone = _event_ms(fn if fn is attn else _native_replay(fn), 5 * iters, 5)
             ms = in_sequence.get(name, standalone)
             out[name] = {
                 "ms": ms,

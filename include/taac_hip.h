@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define TAAC_ABI_VERSION 7
+#define TAAC_ABI_VERSION 8
 
 enum taac_status {
   TAAC_OK = 0,
@@ -57,6 +57,8 @@ enum taac_epilogue {
 #define TAAC_BACKBONE_SPLIT_OUT_FFN 2 /* out projection and feed-forward half as two kernels instead of one        */
 #define TAAC_BACKBONE_FP8 4           /* the four dense layers of a block with e4m3 MFMA operands and per-tensor   */
                                       /* scales (amax / 448); D = 256, F a multiple of 64, plain attention layer   */
+#define TAAC_BACKBONE_ROW_MAJOR_QKV 8 /* keep q | k | v and the attention output of the workspace as [M, 3D] / [M, D] */
+                                      /* rows instead of per-head planes (comparison route; same results)          */
 
 int taac_abi_version(void);
 const char* taac_last_error(void);
@@ -450,6 +452,31 @@ int taac_attn_out_ffn_fwd(const void* attn, int64_t ld_attn, const void* out_bia
                           const void* b_down, const void* packed_ffn_weights, void* out, int64_t ldo, int64_t M,
                           int32_t D, int32_t F, const int32_t* rows, const int32_t* n_rows, const int32_t* attn_rows,
                           int norm_folded, void* stream);
+
+/*
+ * The packed q | k | v projection and the block's second half on PER-HEAD PLANES: between the projection, the attention
+ * kernel and the out projection a tensor [M, N] may be kept as a stack of N / head_dim planes [M, head_dim] - element
+ * (row, col) at ((col / head_dim) * M + row) * head_dim + col % head_dim - so that the rows of one head are contiguous
+ * (64 or 128 bytes apart instead of pieces of a 3 * D row): the attention kernel, which takes any strides, then runs 8 %
+ * faster at the headline shape, and the dense kernels address the planes at no cost. head_dim = 32 or 64.
+ *   taac_norm_linear_heads_fwd: taac_norm_linear_fwd for packed weights without residual whose output is such a stack
+ *     (N / head_dim planes; q = planes 0 .. H-1, k = H .. 2H-1, v = 2H .. 3H-1 of a packed projection: pass them to
+ *     taac_flash_attn_fwd as base pointers H * M * head_dim elements apart with strides {T * head_dim, M * head_dim,
+ *     head_dim, 1}, and let it write its output with the same strides).
+ *   taac_attn_out_ffn_heads_fwd: taac_attn_out_ffn_fwd whose attention output `attn` is such a stack of D / head_dim
+ *     planes (rows indexed like residual / out: no attn_rows).
+ * Results are bit-identical to the row-major entry points. taac_backbone_fwd keeps its q | k | v and attention-output
+ * workspace this way for plain attention layers. Replaces: as taac_norm_linear_fwd / taac_attn_out_ffn_fwd; the layout
+ * takes the place of the reference's q / k / v transposes to (B, H, T, d) (modeling/sequence.py:100-116).
+ */
+int taac_norm_linear_heads_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* bias,
+                               const void* packed_weights, void* out, int32_t head_dim, int64_t M, int32_t N, int32_t K,
+                               const int32_t* rows, const int32_t* n_rows, int norm_folded, void* stream);
+int taac_attn_out_ffn_heads_fwd(const void* attn, int32_t head_dim, const void* out_bias, const void* packed_out_weights,
+                                const void* residual, int64_t ldr, const void* norm_weight, float eps, const void* b_up,
+                                const void* b_down, const void* packed_ffn_weights, void* out, int64_t ldo, int64_t M,
+                                int32_t D, int32_t F, const int32_t* rows, const int32_t* n_rows, int norm_folded,
+                                void* stream);
 
 /*
  * taac_attn_out_ffn_fwd with a sigmoid gate on the projected update (TokenFormer's NLIR gate):

@@ -22,9 +22,9 @@ TAAC_ERR_LAUNCH = -3
 TAAC_F32, TAAC_BF16, TAAC_F16 = 0, 1, 2
 EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
 ATTN_CAUSAL, ATTN_REGISTER_STAGING = 1, 2
-BACKBONE_DENSE_TOKENS, BACKBONE_SPLIT_OUT_FFN, BACKBONE_FP8 = 1, 2, 4
+BACKBONE_DENSE_TOKENS, BACKBONE_SPLIT_OUT_FFN, BACKBONE_FP8, BACKBONE_ROW_MAJOR_QKV = 1, 2, 4, 8
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _DTYPE_CODES = {torch.float32: TAAC_F32, torch.bfloat16: TAAC_BF16, torch.float16: TAAC_F16}
 
@@ -191,6 +191,16 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         c_int,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
          c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
+    ),
+    "taac_norm_linear_heads_fwd": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p,
+         c_void_p, c_int, c_void_p],
+    ),
+    "taac_attn_out_ffn_heads_fwd": (
+        c_int,
+        [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
+         c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_int, c_void_p],
     ),
     "taac_silu_mlp_packed_bytes": (c_int64, [c_int32, c_int32]),
     "taac_silu_mlp_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),

@@ -869,6 +869,98 @@ def norm_linear(
     return out.reshape(*shape[:-1], out_features)
 
 
+def norm_linear_heads(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None = None,
+    *,
+    head_dim: int,
+    norm_weight: torch.Tensor | None = None,
+    eps: float = 1e-6,
+    token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """:func:`norm_linear` (model width 128 / 256, no residual) writing its output as a stack of per-head planes
+    ``[out_features / head_dim, rows, head_dim]`` instead of rows ``[rows, out_features]`` (``taac_norm_linear_heads_fwd``;
+    ``head_dim`` 32 or 64): plane ``p`` holds columns ``p * head_dim ..`` of every row, so the rows of one head are
+    contiguous. For a packed q | k | v projection ``planes.view(3, H, B, T, head_dim)[i].transpose(0, 1)`` is q / k / v as
+    a ``(B, H, T, head_dim)`` view for :func:`flash_attention`, whose output keeps that layout and is what
+    :func:`attention_out_ffn_heads` reads. Same values as :func:`norm_linear`, bit for bit."""
+    name = "hip norm_linear_heads"
+    require_cuda_tensors(name, x, weight, bias, norm_weight)
+    require_inference(name, x, weight, bias, norm_weight)
+    _check_bf16(name, x, weight, bias, norm_weight)
+    rows, _ = _as_rows(x)
+    _check_weight(name, rows, weight, bias)
+    out_features, in_features = weight.shape
+    if not _fused_width(in_features) or out_features % 64 != 0 or head_dim not in (32, 64):
+        raise RuntimeError(f"{name}: needs in_features 128 / 256, out_features a multiple of 64 and head_dim 32 or 64")
+    packed = _packed_linear(weight, norm_weight)
+    index, count = _token_rows(name, token_rows, rows)
+    shape = (out_features // head_dim, rows.shape[0], head_dim)
+    if out is None:
+        out = (torch.zeros if index is not None else torch.empty)(shape, dtype=x.dtype, device=x.device)
+    elif out.dtype != x.dtype or out.numel() != out_features * rows.shape[0] or not out.is_contiguous():
+        raise ValueError(f"{name}: out must be a contiguous {x.dtype} tensor of {out_features * rows.shape[0]} elements")
+    library = _native.load_library()
+    status = library.taac_norm_linear_heads_fwd(
+        rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), _native.ptr(bias), packed.data_ptr(),
+        out.data_ptr(), int(head_dim), rows.shape[0], out_features, in_features, _native.ptr(index), _native.ptr(count),
+        int(norm_weight is not None), _native.current_stream(x.device))
+    _native.check(status, "norm_linear_heads")
+    return out.view(shape)
+
+
+def attention_out_ffn_heads(
+    attn: torch.Tensor,
+    out_weight: torch.Tensor,
+    out_bias: torch.Tensor | None,
+    residual: torch.Tensor,
+    up_weight: torch.Tensor,
+    up_bias: torch.Tensor | None,
+    down_weight: torch.Tensor,
+    down_bias: torch.Tensor | None,
+    *,
+    norm_weight: torch.Tensor | None = None,
+    eps: float = 1e-6,
+    token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """:func:`attention_out_ffn` whose attention output is a contiguous stack of per-head planes ``[H, rows, head_dim]``
+    (``taac_attn_out_ffn_heads_fwd``; the layout :func:`flash_attention` leaves behind for queries taken from
+    :func:`norm_linear_heads`). ``residual`` / ``out`` are ``[.., D]`` rows as usual. Same values, bit for bit."""
+    name = "hip attention_out_ffn_heads"
+    tensors = (attn, out_weight, out_bias, residual, up_weight, up_bias, down_weight, down_bias, norm_weight)
+    require_cuda_tensors(name, *tensors)
+    require_inference(name, *tensors)
+    _check_bf16(name, *tensors)
+    if attn.ndim != 3 or not attn.is_contiguous() or attn.shape[2] not in (32, 64):
+        raise ValueError(f"{name}: attn must be a contiguous [H, rows, head_dim] stack with head_dim 32 or 64")
+    heads, row_count, head_dim = attn.shape
+    d_model, hidden = heads * head_dim, up_weight.shape[0] // 2
+    res_rows, shape = _as_rows(residual)
+    if res_rows.shape != (row_count, d_model):
+        raise ValueError(f"{name}: residual must hold {row_count} rows of {d_model}")
+    if out_weight.shape != (d_model, d_model) or up_weight.shape != (2 * hidden, d_model) or down_weight.shape != (d_model, hidden):
+        raise ValueError(f"{name} expects out_weight [D, D], up_weight [2F, D] and down_weight [D, F]")
+    if not (_fused_width(d_model) and hidden % 32 == 0):
+        raise RuntimeError(f"{name}: needs model width 128 / 256 and a hidden size that is a multiple of 32")
+    packed_out = _packed_cache.get((out_weight,), lambda: pack_linear_weight(out_weight))
+    packed_ffn = _packed_ffn(up_weight, down_weight, True, norm_weight)
+    if res_rows.stride(-1) != 1 or res_rows.stride(0) % 8 != 0:
+        res_rows = res_rows.contiguous()
+    index, count = _token_rows(name, token_rows, res_rows)
+    out = _output_rows(name, out, (row_count, d_model), index is not None, residual)
+    library = _native.load_library()
+    status = library.taac_attn_out_ffn_heads_fwd(
+        attn.data_ptr(), int(head_dim), _native.ptr(out_bias), packed_out.data_ptr(), res_rows.data_ptr(), res_rows.stride(0),
+        _native.ptr(norm_weight), float(eps), _native.ptr(up_bias), _native.ptr(down_bias), packed_ffn.data_ptr(),
+        out.data_ptr(), d_model, row_count, d_model, hidden, _native.ptr(index), _native.ptr(count),
+        int(norm_weight is not None), _native.current_stream(attn.device))
+    _native.check(status, "attention_out_ffn_heads")
+    return out.reshape(shape)
+
+
 def qkv_projection(
     x: torch.Tensor,
     weight: torch.Tensor,

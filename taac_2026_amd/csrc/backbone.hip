@@ -471,7 +471,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
                                  void* stream) {
   using namespace taac;
   const char* name = "taac_backbone_fwd";
-  if (flags & ~(TAAC_BACKBONE_DENSE_TOKENS | TAAC_BACKBONE_SPLIT_OUT_FFN | TAAC_BACKBONE_FP8))
+  if (flags & ~(TAAC_BACKBONE_DENSE_TOKENS | TAAC_BACKBONE_SPLIT_OUT_FFN | TAAC_BACKBONE_FP8 | TAAC_BACKBONE_ROW_MAJOR_QKV))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: unknown flag bits (%d)", name, flags);
   const bool fp8 = (flags & TAAC_BACKBONE_FP8) != 0;
   if (fp8 && !fp8_shape(D, F))
@@ -571,6 +571,16 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
                                name)) != TAAC_OK)
       return rc;
   }
+  // Plain attention layers (no query / key norm, no rotary embedding) with heads of 32 or 64 features keep q | k | v and
+  // the attention output as stacks of per-head planes [3 * heads][M][dh] / [heads][M][dh] instead of [M][3 * D] / [M][D]
+  // rows: a head's rows are then contiguous for the attention kernel (64-byte pieces of 1 536-byte rows otherwise), and the
+  // dense kernels on either side address the planes directly. TAAC_BACKBONE_ROW_MAJOR_QKV keeps the rows (same results).
+  bool planes = fused && !fp8 && !split_out_ffn && rope_cos_sin == nullptr && (dh == 32 || dh == 64) &&
+                !(flags & TAAC_BACKBONE_ROW_MAJOR_QKV);
+  for (int i = 0; i < n_blocks && planes; ++i)
+    planes = blocks[i].query_norm_weight == nullptr && blocks[i].key_norm_weight == nullptr;
+  const int64_t plane_elems = M * dh;
+  const int64_t plane_strides[4] = {static_cast<int64_t>(T) * dh, plane_elems, dh, 1};
   for (int i = 0; i < n_blocks; ++i) {
     const taac_block_weights& w = blocks[i];
     if (!w.attn_norm_weight || !w.qkv_weight || !w.out_weight || !w.ffn_norm_weight || !w.up_weight || !w.down_weight)
@@ -643,6 +653,10 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
         q_scale = qk_rstd;
         k_scale = qk_rstd + M;
       }
+    } else if (planes) {
+      if ((rc = taac_norm_linear_heads_fwd(cur, D, w.attn_norm_weight, eps, w.qkv_bias, pk_qkv, qkv, dh, M, 3 * D, D, rows,
+                                           n_rows, w.attn_norm_weight != nullptr, stream)) != TAAC_OK)
+        return rc;
     } else if (fused) {
       if ((rc = taac_norm_linear_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, nullptr, 0, qkv,
                                      3 * D, M, 3 * D, D, rows, n_rows, nullptr, w.attn_norm_weight != nullptr,
@@ -659,6 +673,18 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
                                       w.key_norm_weight, eps, rope_cos_sin, nullptr, nullptr, TAAC_BF16, stream)) !=
           TAAC_OK)
         return rc;
+    }
+    if (planes) {
+      if ((rc = taac_flash_attn_scaled_fwd(qkv, qkv + heads * plane_elems, qkv + 2 * heads * plane_elems, key_lengths,
+                                           nullptr, nullptr, nullptr, h, B, heads, T, T, dh, plane_strides, plane_strides,
+                                           plane_strides, plane_strides, 0, rows ? 2 : 1, TAAC_BF16, stream)) != TAAC_OK)
+        return rc;
+      if ((rc = taac_attn_out_ffn_heads_fwd(h, dh, w.out_bias, pk_out, cur, D, w.ffn_norm_weight, eps, w.up_bias,
+                                            w.down_bias, pk_ffn, x_out, D, M, D, F, rows, n_rows,
+                                            w.ffn_norm_weight != nullptr, stream)) != TAAC_OK)
+        return rc;
+      cur = x_out;
+      continue;
     }
     if ((rc = taac_flash_attn_scaled_fwd(qkv, qkv + D, qkv + 2 * D, key_lengths, q_scale, k_scale, q_col_scale, h, B,
                                          heads, T, T, dh, qkv_strides, qkv_strides, qkv_strides, o_strides, 0, rows ? 2 : 1,

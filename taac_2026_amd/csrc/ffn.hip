@@ -69,6 +69,11 @@ struct TsParams {
                             // accumulators
   const bf16_t* gate;       // GATE: [M, D] pre-activation of the update's gate (rows like residual), row stride ldg
   int64_t ldg;
+  // Feature planes (the backbone's private q | k | v and attention-output buffers): with a shift s > 0 the tensor is a
+  // stack of planes of 2^s features, [cols / 2^s][M][2^s] - element (row, col) at ((col >> s) * M + row) * 2^s + col % 2^s -
+  // instead of [M][cols] rows; a head's rows are then contiguous for the attention kernel.
+  int32_t x_plane_shift;    // layout of x (0: rows of ldx elements)
+  int32_t out_plane_shift;  // layout of out (linear kernel without residual or query / key epilogue; 0: rows of ldo elements)
 };
 
 __device__ __forceinline__ float silu_f(float v) {
@@ -225,7 +230,17 @@ __device__ __forceinline__ void load_token_rows(const TsParams& p, int64_t count
   constexpr int KS = D / 16;
 #pragma unroll
   for (int t = 0; t < TT; ++t) {
-    const bf16_t* row = p.x + input_row(p, count, tok0 + t * 32 + l32) * p.ldx + hh * 8;
+    const int64_t r = input_row(p, count, tok0 + t * 32 + l32);
+    if (p.x_plane_shift > 0) {  // feature planes: k-step ks lies in plane (16 * ks) >> shift
+      const int sh = p.x_plane_shift;
+      const bf16_t* row = p.x + (r << sh) + hh * 8;
+      const int64_t plane_elems = p.M << sh;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        xf[t][ks] = *reinterpret_cast<const bf16x8*>(row + ((ks * 16) >> sh) * plane_elems + ((ks * 16) & ((1 << sh) - 1)));
+      continue;
+    }
+    const bf16_t* row = p.x + r * p.ldx + hh * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) xf[t][ks] = *reinterpret_cast<const bf16x8*>(row + ks * 16);
   }
@@ -1020,13 +1035,24 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
 #pragma unroll
     for (int i = 0; i < NST; ++i) {
       const int32_t row = static_cast<int32_t>(token_row(p, count, tok_base + (i / 4) * 32 + (i % 4) * 8 + lane / 8));
+      if (!RES && p.out_plane_shift > 0) {
+        // feature planes: the lane's piece j = lane % 8 of a 64-feature chunk lies in plane (8 * j) >> shift of the chunk's
+        // planes, at 16-byte piece j % (plane width / 8) of the row
+        const int psh = p.out_plane_shift - 3;  // log2 of the 16-byte pieces per plane row
+        const uint32_t j = static_cast<uint32_t>(lane % 8);
+        prow[i] = static_cast<int32_t>((((j >> psh) * static_cast<uint32_t>(p.M) + static_cast<uint32_t>(row)) << psh) +
+                                       (j & ((1u << psh) - 1u)));
+        continue;
+      }
       prow[i] = RES ? row : static_cast<int32_t>(static_cast<uint32_t>(row) * ld16 + static_cast<uint32_t>(lane % 8));
     }
   };
+  // bytes between the 64-feature chunks of the output: 128 in a row, 64 features of M rows in the plane layout
+  const int64_t chunk_bytes = (!RES && p.out_plane_shift > 0) ? static_cast<int64_t>(kNC) * 2 * p.M : kNC * 2;
   // Address of the lane's 16-byte piece of output chunk `chunk` for piece slot value v (a row with RES, an offset without).
   auto out_piece = [&](int32_t v, int chunk) -> bf16x8* {
     const uint32_t off16 = RES ? static_cast<uint32_t>(v) * ld16 + static_cast<uint32_t>(lane % 8) : static_cast<uint32_t>(v);
-    return reinterpret_cast<bf16x8*>(reinterpret_cast<char*>(p.out) + chunk * (kNC * 2) + (static_cast<uint64_t>(off16) << 4));
+    return reinterpret_cast<bf16x8*>(reinterpret_cast<char*>(p.out) + chunk * chunk_bytes + (static_cast<uint64_t>(off16) << 4));
   };
   auto request_residual = [&](const int32_t (&prow)[NST], int chunk, bf16x8 (&res)[NST]) {
 #pragma unroll
@@ -1410,8 +1436,10 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
               const void* b_down, const void* packed_weights, const void* residual, int64_t ldr, void* out, int64_t ldo,
               int64_t M, int32_t D, int32_t F, int gate_first, const int32_t* rows, const int32_t* n_rows,
               const int32_t* x_rows, int norm_folded, void* stream, const void* update_gate = nullptr, int64_t ldg = 0,
-              bool glu = true) {
+              bool glu = true, int x_plane = 0) {
   const bool with_proj = out_packed != nullptr;
+  if (x_plane != 0 && ((x_plane != 32 && x_plane != 64) || D % x_plane != 0))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: input planes are 32 or 64 features wide", name);
   if (norm_folded && (!norm_weight || !packed_weights))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: norm_folded needs the norm weight and the packed weights it was folded into", name);
   if (!glu && (with_proj || !packed_weights))
@@ -1470,6 +1498,7 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
   p.gate = static_cast<const bf16_t*>(update_gate);
   p.ldg = ldg;
   p.norm_folded = norm_folded ? 1 : 0;
+  p.x_plane_shift = x_plane == 32 ? 5 : (x_plane == 64 ? 6 : 0);
   p.units = compute_units();
   if (p.units <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
   if (const int limit = test_max_workgroups(); limit > 0 && limit < p.units) p.units = limit;  // taac_test_hooks
@@ -1594,7 +1623,9 @@ struct QkExtras {
 int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
                        const void* bias, const void* packed_weights, const void* residual, int64_t ldr, void* out,
                        int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows, const int32_t* n_rows,
-                       const int32_t* x_rows, const QkExtras& qk, int norm_folded, void* stream) {
+                       const int32_t* x_rows, const QkExtras& qk, int norm_folded, void* stream, int out_plane = 0) {
+  if (out_plane != 0 && (residual || qk.enabled || (out_plane != 32 && out_plane != 64) || static_cast<int64_t>(8) * M + 8 > 0xffffffffLL))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: output planes are 32 or 64 features wide, without residual or query / key epilogue", name);
   if (norm_folded && (!norm_weight || !packed_weights))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: norm_folded needs the norm weight and the packed weights it was folded into", name);
   if (M < 0 || N <= 0 || K <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, N and K > 0", name);
@@ -1638,6 +1669,7 @@ int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void*
   p.rows = rows;
   p.n_rows = n_rows;
   p.x_rows = x_rows;
+  p.out_plane_shift = out_plane == 32 ? 5 : (out_plane == 64 ? 6 : 0);
   p.qk_w = static_cast<const bf16_t*>(qk.qk_weight);
   p.cos_sin = static_cast<const bf16_t*>(qk.cos_sin);
   p.qk_sumsq = qk.qk_sumsq;
@@ -1696,6 +1728,34 @@ __global__ __launch_bounds__(256) void row_rstd_kernel(const float* __restrict__
 
 }  // namespace
 }  // namespace taac
+
+extern "C" int taac_norm_linear_heads_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* bias,
+                                          const void* packed_weights, void* out, int32_t head_dim, int64_t M, int32_t N,
+                                          int32_t K, const int32_t* rows, const int32_t* n_rows, int norm_folded,
+                                          void* stream) {
+  const char* name = "taac_norm_linear_heads_fwd";
+  if (!packed_weights) return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: the weights must be packed", name);
+  if (head_dim != 32 && head_dim != 64)
+    return taac::set_error(TAAC_ERR_UNSUPPORTED, "%s: head_dim must be 32 or 64 (got %d)", name, head_dim);
+  return taac::norm_linear_launch(name, x, ldx, norm_weight, eps, nullptr, bias, packed_weights, nullptr, 0, out, N, M, N,
+                                  K, rows, n_rows, nullptr, taac::QkExtras{}, norm_folded, stream, head_dim);
+}
+
+extern "C" int taac_attn_out_ffn_heads_fwd(const void* attn, int32_t head_dim, const void* out_bias,
+                                           const void* packed_out_weights, const void* residual, int64_t ldr,
+                                           const void* norm_weight, float eps, const void* b_up, const void* b_down,
+                                           const void* packed_ffn_weights, void* out, int64_t ldo, int64_t M, int32_t D,
+                                           int32_t F, const int32_t* rows, const int32_t* n_rows, int norm_folded,
+                                           void* stream) {
+  const char* name = "taac_attn_out_ffn_heads_fwd";
+  if (!packed_out_weights || !packed_ffn_weights)
+    return taac::set_error(TAAC_ERR_INVALID_VALUE, "%s: both weight sets must be packed", name);
+  if (head_dim != 32 && head_dim != 64)
+    return taac::set_error(TAAC_ERR_UNSUPPORTED, "%s: head_dim must be 32 or 64 (got %d)", name, head_dim);
+  return taac::ffn_entry(name, attn, D, out_bias, packed_out_weights, norm_weight, eps, nullptr, b_up, nullptr, b_down,
+                         packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, nullptr, norm_folded,
+                         stream, nullptr, 0, true, head_dim);
+}
 
 extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
                                     const void* bias, const void* packed_weights, const void* residual, int64_t ldr,

@@ -479,7 +479,9 @@ class PCVRBackbone(nn.Module):
     ``forward(emb[B, T, D] bf16, key_lengths[B] int32) -> p[B] float32``; ``return_hidden=True`` also returns the
     final hidden state (rows at or beyond ``key_lengths[b]`` are zeros). ``dense_tokens=True`` runs the dense layers over
     the padded positions too (what the reference's dense ``[B, T, D]`` formulation does; same valid rows, bit for bit),
-    ``split_out_ffn=True`` runs the out projection and the feed-forward half as two kernels (comparison routes).
+    ``split_out_ffn=True`` runs the out projection and the feed-forward half as two kernels, ``row_major_qkv=True`` keeps
+    q | k | v and the attention output of the workspace as rows instead of per-head planes (comparison routes;
+    ``row_major_qkv`` gives bit-identical results).
     ``fp8=True`` runs the four dense layers of every block with e4m3 operands and per-tensor scales (d_model 256, plain
     attention layer).
     ``qk_norm=True`` adds the reference layer's ``RMSNorm(d_model)`` of the query and the key
@@ -513,13 +515,13 @@ class PCVRBackbone(nn.Module):
         return ws
 
     def forward(self, emb: torch.Tensor, key_lengths: torch.Tensor, *, return_hidden: bool = False,
-                dense_tokens: bool = False, split_out_ffn: bool = False, fp8: bool = False):
+                dense_tokens: bool = False, split_out_ffn: bool = False, fp8: bool = False, row_major_qkv: bool = False):
         name = "hip PCVRBackbone"
         require_cuda_tensors(name, emb, key_lengths)
         if torch.is_grad_enabled() and (emb.requires_grad or any(p.requires_grad for p in self.parameters())):
-            if dense_tokens or split_out_ffn or fp8:
-                raise RuntimeError(f"{name}: dense_tokens, split_out_ffn and fp8 are inference routes: call them under "
-                                   "torch.no_grad()")
+            if dense_tokens or split_out_ffn or fp8 or row_major_qkv:
+                raise RuntimeError(f"{name}: dense_tokens, split_out_ffn, fp8 and row_major_qkv are inference routes: call "
+                                   "them under torch.no_grad()")
             return self._forward_training(emb, key_lengths, return_hidden)
         if emb.ndim != 3 or emb.shape[-1] != self.d_model:
             raise ValueError(f"PCVRBackbone expects embeddings of shape (batch, tokens, {self.d_model})")
@@ -561,7 +563,7 @@ class PCVRBackbone(nn.Module):
         workspace = self._get_workspace(int(nbytes), emb.device)
         hidden = torch.empty_like(emb) if return_hidden else None
         flags = ((_native.BACKBONE_DENSE_TOKENS if dense_tokens else 0) | (_native.BACKBONE_SPLIT_OUT_FFN if split_out_ffn else 0)
-                 | (_native.BACKBONE_FP8 if fp8 else 0))
+                 | (_native.BACKBONE_FP8 if fp8 else 0) | (_native.BACKBONE_ROW_MAJOR_QKV if row_major_qkv else 0))
         probabilities = torch.empty(batch, dtype=torch.float32, device=emb.device)
         status = library.taac_backbone_fwd(
             emb.data_ptr(), key_lengths.data_ptr(), packed, len(self.blocks), dev(self.head.weight.reshape(-1)),
