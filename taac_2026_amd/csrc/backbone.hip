@@ -62,6 +62,27 @@ __global__ __launch_bounds__(kBlock) void masked_mean_head_kernel(const bf16_t* 
   }
 }
 
+// The same readout from per-token dot products with the head weight (left behind by the last block's kernel): one
+// wavefront per sample adds the dots of its valid prefix in a fixed order, mean, bias, sigmoid.
+__global__ __launch_bounds__(kBlock) void token_dots_head_kernel(const float* __restrict__ dots,
+                                                                 const int32_t* __restrict__ lengths,
+                                                                 const bf16_t* __restrict__ b_head, float* __restrict__ p,
+                                                                 int B, int T) {
+  const int b = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  if (b >= B) return;
+  int len = lengths[b];
+  len = len < 0 ? 0 : (len > T ? T : len);
+  const float* row = dots + static_cast<int64_t>(b) * T;
+  float s = 0.f;
+  for (int t = lane; t < len; t += kWave) s += row[t];
+  s = group_sum<kWave>(s);
+  if (lane == 0) {
+    const float z = (b_head != nullptr ? static_cast<float>(b_head[0]) : 0.f) + s / static_cast<float>(len < 1 ? 1 : len);
+    p[b] = 1.0f / (1.0f + expf(-z));
+  }
+}
+
 // Number of valid tokens of sample b: its clamped length, or the set bits among the first T of its bit row.
 __device__ __forceinline__ int32_t valid_count(const int32_t* __restrict__ lengths, const uint32_t* __restrict__ bits,
                                                int b, int T) {
@@ -581,11 +602,18 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
     planes = blocks[i].query_norm_weight == nullptr && blocks[i].key_norm_weight == nullptr;
   const int64_t plane_elems = M * dh;
   const int64_t plane_strides[4] = {static_cast<int64_t>(T) * dh, plane_elems, dh, 1};
+  // The last block's kernel (out projection + feed-forward in one) also leaves every token's dot product with the head
+  // weight behind, in the q | k | v buffer that is free by then: the readout adds M floats instead of reading the final
+  // hidden state again.
+  float* token_dots = reinterpret_cast<float*>(qkv);
+  const bool head_rides = aligned16(w_head);
+  bool dots_ready = false;
   for (int i = 0; i < n_blocks; ++i) {
     const taac_block_weights& w = blocks[i];
     if (!w.attn_norm_weight || !w.qkv_weight || !w.out_weight || !w.ffn_norm_weight || !w.up_weight || !w.down_weight)
       return set_error(TAAC_ERR_INVALID_VALUE, "%s: block %d has a null weight", name, i);
     const bool last = (i == n_blocks - 1);
+    const bool ride = last && head_rides;
     bf16_t* x_out = (last && hidden_out != nullptr) ? static_cast<bf16_t*>(hidden_out) : x;
     if (fp8) {
       // Four dense layers with e4m3 operands and per-tensor scales; every activation scale comes out of the epilogue of the
@@ -679,10 +707,11 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
                                            nullptr, nullptr, nullptr, h, B, heads, T, T, dh, plane_strides, plane_strides,
                                            plane_strides, plane_strides, 0, rows ? 2 : 1, TAAC_BF16, stream)) != TAAC_OK)
         return rc;
-      if ((rc = taac_attn_out_ffn_heads_fwd(h, dh, w.out_bias, pk_out, cur, D, w.ffn_norm_weight, eps, w.up_bias,
-                                            w.down_bias, pk_ffn, x_out, D, M, D, F, rows, n_rows,
-                                            w.ffn_norm_weight != nullptr, stream)) != TAAC_OK)
+      if ((rc = attn_out_ffn_readout(h, D, dh, w.out_bias, pk_out, cur, D, w.ffn_norm_weight, eps, w.up_bias, w.down_bias,
+                                     pk_ffn, x_out, D, M, D, F, rows, n_rows, w.ffn_norm_weight != nullptr,
+                                     ride ? w_head : nullptr, ride ? token_dots : nullptr, stream)) != TAAC_OK)
         return rc;
+      dots_ready = ride;
       cur = x_out;
       continue;
     }
@@ -692,10 +721,11 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
       return rc;
     if (fused && !split_out_ffn) {
       // out projection + residual and the whole feed-forward half in one kernel; the stream between them stays on chip
-      if ((rc = taac_attn_out_ffn_fwd(h, D, w.out_bias, pk_out, cur, D, w.ffn_norm_weight, eps, w.up_bias, w.down_bias,
-                                      pk_ffn, x_out, D, M, D, F, rows, n_rows, nullptr, w.ffn_norm_weight != nullptr,
-                                      stream)) != TAAC_OK)
+      if ((rc = attn_out_ffn_readout(h, D, 0, w.out_bias, pk_out, cur, D, w.ffn_norm_weight, eps, w.up_bias, w.down_bias,
+                                     pk_ffn, x_out, D, M, D, F, rows, n_rows, w.ffn_norm_weight != nullptr,
+                                     ride ? w_head : nullptr, ride ? token_dots : nullptr, stream)) != TAAC_OK)
         return rc;
+      dots_ready = ride;
     } else if (fused) {
       if ((rc = taac_norm_linear_fwd(h, D, nullptr, eps, nullptr, w.out_bias, pk_out, cur, D, x, D, M, D, D, rows,
                                      n_rows, nullptr, 0, stream)) != TAAC_OK)
@@ -729,6 +759,12 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
     if (hipMemcpyAsync(hidden_out, emb, static_cast<size_t>(M) * D * 2, hipMemcpyDeviceToDevice, as_stream(stream)) !=
         hipSuccess)
       return set_error(TAAC_ERR_LAUNCH, "%s: copy of the embeddings failed", name);
+  }
+  if (dots_ready) {  // the last block's kernel left every token's dot product with the head weight behind
+    const int per = kBlock / kWave;
+    hipLaunchKernelGGL(token_dots_head_kernel, dim3((B + per - 1) / per), dim3(kBlock), 0, as_stream(stream), token_dots,
+                       key_lengths, static_cast<const bf16_t*>(b_head), p, B, T);
+    return check_launch(name);
   }
   return taac_masked_mean_head(cur, key_lengths, w_head, b_head, p, B, T, D, stream);
 }

@@ -36,6 +36,13 @@ bool test_fp8_tiled();
 // Packs the qkv / out / feed-forward weights (gate first) of n backbone blocks into fragment order (ffn.hip).
 int pack_backbone_blocks(const taac_block_weights* blocks, int n, int32_t D, int32_t F, void* const* packed_qkv,
                          void* const* packed_out, void* const* packed_ffn, hipStream_t s, const char* name);
+// Out projection + feed-forward half of a block (ffn.hip; attn_plane: 0 = rows of ld_attn elements, 32 / 64 = per-head
+// planes) that also writes the dot product of every stored output row with head_w to token_dots[row].
+int attn_out_ffn_readout(const void* attn, int64_t ld_attn, int attn_plane, const void* out_bias,
+                         const void* packed_out_weights, const void* residual, int64_t ldr, const void* norm_weight,
+                         float eps, const void* b_up, const void* b_down, const void* packed_ffn_weights, void* out,
+                         int64_t ldo, int64_t M, int32_t D, int32_t F, const int32_t* rows, const int32_t* n_rows,
+                         int norm_folded, const void* head_w, float* token_dots, void* stream);
 // Token-stationary e4m3 dense layer (fp8_ts.hip): TAAC_OK after a launch, a negative status on an error, 1 when the shape
 // is not covered and the caller must use the tiled kernel.
 int launch_linear_fp8_ts(const void* a, int a_is_fp8, int64_t lda, const void* w, const float* amax_a,

@@ -74,6 +74,10 @@ struct TsParams {
   // instead of [M][cols] rows; a head's rows are then contiguous for the attention kernel.
   int32_t x_plane_shift;    // layout of x (0: rows of ldx elements)
   int32_t out_plane_shift;  // layout of out (linear kernel without residual or query / key epilogue; 0: rows of ldo elements)
+  // Readout riding on the feed-forward epilogue: token_dots[row] = sum over the features of out[row] * head_w (fp32, from
+  // the rounded output), so that a mean-pooling linear head behind the layer need not read the rows again.
+  const bf16_t* head_w;     // [D] or null
+  float* token_dots;        // [M] (rows like out), written for the tokens the kernel stores
 };
 
 __device__ __forceinline__ float silu_f(float v) {
@@ -392,9 +396,13 @@ __device__ __forceinline__ float half_wave_pair_sum(float v) {
 // Reads the epilogue tile back row-wise (lane -> token 8*i + lane/8, features 8*(lane%8) .. +7), adds the residual
 // pieces loaded earlier and stores 16 bytes per lane: every 128-byte row segment is written by 8 consecutive lanes.
 // prow[i] is the memory row of token 8*i + lane/8 of the tile, live[i] whether that token exists.
+// head_w (optional): the lane's share of the dot product of each stored row with head_w is added to hdot[i].
 template <bool RES>
 __device__ __forceinline__ void tile_to_global(const uint8_t* tile, bf16_t* out, int64_t ldo, const int64_t (&prow)[4],
-                                               const bool (&live)[4], int col0, const bf16x8 (&res)[4], int lane) {
+                                               const bool (&live)[4], int col0, const bf16x8 (&res)[4], int lane,
+                                               const bf16_t* head_w, float (&hdot)[4]) {
+  bf16x8 hw;
+  if (head_w != nullptr) hw = *reinterpret_cast<const bf16x8*>(head_w + col0 + (lane % 8) * 8);
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int row = i * 8 + lane / 8;
@@ -405,6 +413,10 @@ __device__ __forceinline__ void tile_to_global(const uint8_t* tile, bf16_t* out,
         v[e] = static_cast<bf16_t>(static_cast<float>(v[e]) + static_cast<float>(res[i][e]));
     }
     if (live[i]) *reinterpret_cast<bf16x8*>(out + prow[i] * ldo + col0 + (lane % 8) * 8) = v;
+    if (head_w != nullptr) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) hdot[i] = fmaf(static_cast<float>(v[e]), static_cast<float>(hw[e]), hdot[i]);
+    }
   }
 }
 
@@ -915,6 +927,7 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
       prow[i] = token_row(p, count, tok_base + i * 8 + lane / 8);
       live[i] = tok_base + i * 8 + lane / 8 < wg_tok0 + wg_ntok;
     }
+    float hdot[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int pr = 0; pr < MB / 2; ++pr) {  // 64 features at a time
       bf16x8 res[4];
@@ -925,11 +938,22 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
       tile_to_lds(tile, oacc[t][2 * pr], oacc[t][2 * pr + 1], bv, l32, hh);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       if (add_residual)
-        tile_to_global<true>(tile, p.out, p.ldo, prow, live, pr * 64, res, lane);
+        tile_to_global<true>(tile, p.out, p.ldo, prow, live, pr * 64, res, lane, p.head_w, hdot);
       else
-        tile_to_global<false>(tile, p.out, p.ldo, prow, live, pr * 64, res, lane);
+        tile_to_global<false>(tile, p.out, p.ldo, prow, live, pr * 64, res, lane, p.head_w, hdot);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if (p.head_w != nullptr) {
+      // the eight lanes of a row hold its eight 8-feature shares: add them in a fixed order, lane % 8 == 0 stores
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float d = hdot[i];
+        d += __shfl_xor(d, 1);
+        d += __shfl_xor(d, 2);
+        d += __shfl_xor(d, 4);
+        if (lane % 8 == 0 && live[i]) p.token_dots[prow[i]] = d;
+      }
     }
   }
 }
@@ -1436,8 +1460,10 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
               const void* b_down, const void* packed_weights, const void* residual, int64_t ldr, void* out, int64_t ldo,
               int64_t M, int32_t D, int32_t F, int gate_first, const int32_t* rows, const int32_t* n_rows,
               const int32_t* x_rows, int norm_folded, void* stream, const void* update_gate = nullptr, int64_t ldg = 0,
-              bool glu = true, int x_plane = 0) {
+              bool glu = true, int x_plane = 0, const void* head_w = nullptr, float* token_dots = nullptr) {
   const bool with_proj = out_packed != nullptr;
+  if ((head_w == nullptr) != (token_dots == nullptr) || !ptr_ok(head_w, 15))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: the readout needs a 16-byte aligned head weight and a buffer of token dots", name);
   if (x_plane != 0 && ((x_plane != 32 && x_plane != 64) || D % x_plane != 0))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: input planes are 32 or 64 features wide", name);
   if (norm_folded && (!norm_weight || !packed_weights))
@@ -1499,6 +1525,8 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
   p.ldg = ldg;
   p.norm_folded = norm_folded ? 1 : 0;
   p.x_plane_shift = x_plane == 32 ? 5 : (x_plane == 64 ? 6 : 0);
+  p.head_w = static_cast<const bf16_t*>(head_w);
+  p.token_dots = token_dots;
   p.units = compute_units();
   if (p.units <= 0) return set_error(TAAC_ERR_LAUNCH, "%s: cannot query the device", name);
   if (const int limit = test_max_workgroups(); limit > 0 && limit < p.units) p.units = limit;  // taac_test_hooks
@@ -1756,6 +1784,20 @@ extern "C" int taac_attn_out_ffn_heads_fwd(const void* attn, int32_t head_dim, c
                          packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, nullptr, norm_folded,
                          stream, nullptr, 0, true, head_dim);
 }
+
+namespace taac {
+// taac_attn_out_ffn_fwd (attn_plane = 0) / taac_attn_out_ffn_heads_fwd (attn_plane = head_dim) that also leaves, for every
+// token it stores, the dot product of the output row with head_w in token_dots[row] (see TsParams::head_w).
+int attn_out_ffn_readout(const void* attn, int64_t ld_attn, int attn_plane, const void* out_bias,
+                         const void* packed_out_weights, const void* residual, int64_t ldr, const void* norm_weight,
+                         float eps, const void* b_up, const void* b_down, const void* packed_ffn_weights, void* out,
+                         int64_t ldo, int64_t M, int32_t D, int32_t F, const int32_t* rows, const int32_t* n_rows,
+                         int norm_folded, const void* head_w, float* token_dots, void* stream) {
+  return ffn_entry("taac_backbone_fwd", attn, ld_attn, out_bias, packed_out_weights, norm_weight, eps, nullptr, b_up, nullptr,
+                   b_down, packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, nullptr, norm_folded,
+                   stream, nullptr, 0, true, attn_plane, head_w, token_dots);
+}
+}  // namespace taac
 
 extern "C" int taac_norm_linear_fwd(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* w,
                                     const void* bias, const void* packed_weights, const void* residual, int64_t ldr,

@@ -137,3 +137,41 @@ def test_backbone_plane_route_equals_its_row_major_route(device, d_model, heads,
     assert torch.equal(hidden[valid], hidden_rows[valid])
     if not dense_tokens:
         assert torch.equal(hidden, hidden_rows)
+
+
+@pytest.mark.parametrize("d_model,heads,d_ff", [(256, 8, 1024), (128, 2, 256)])
+@pytest.mark.parametrize("dense_tokens", [False, True])
+def test_readout_riding_on_the_last_block_equals_the_readout_kernel(device, d_model, heads, d_ff, dense_tokens):
+    """The last block's kernel leaves every token's dot product with the head weight behind and the readout adds those;
+    the stand-alone readout kernel (``taac_masked_mean_head``: mean of the rows, then the dot product) on the returned
+    hidden state gives the same probabilities up to fp32 summation order. Lengths 0 and T included."""
+    from taac_2026_amd import _native
+
+    inputs = workloads.backbone_inputs(batch=9, n_feature_tokens=8, n_sequence_tokens=192, d_model=d_model,
+                                       num_heads=heads, d_ff=d_ff, n_blocks=2, min_sequence_len=1, seed=77)
+    inputs.key_lengths[0] = 0
+    inputs.key_lengths[1] = inputs.emb.shape[1]
+    g = torch.Generator().manual_seed(4)
+    inputs.head_weight.copy_((0.5 * torch.randn(inputs.head_weight.shape, generator=g)).to(torch.bfloat16))
+    inputs.head_bias.fill_(0.25)
+    model = PCVRBackbone(d_model=d_model, num_heads=heads, d_ff=d_ff, n_blocks=2)
+    workloads.load_backbone_state(model, inputs)
+    model = model.to(device=device, dtype=torch.bfloat16).eval()
+    emb, lengths = inputs.emb.to(device), inputs.key_lengths.to(device)
+    with torch.no_grad():
+        p, hidden = model(emb, lengths, return_hidden=True, dense_tokens=dense_tokens)
+        p_only = model(emb, lengths, dense_tokens=dense_tokens)
+    assert torch.equal(p, p_only)
+    batch, tokens, _ = emb.shape
+    library = _native.load_library()
+    expected = torch.empty(batch, dtype=torch.float32, device=device)
+    w_head = inputs.head_weight.to(device).reshape(-1).contiguous()
+    b_head = inputs.head_bias.to(device).reshape(-1).contiguous()
+    _native.check(library.taac_masked_mean_head(hidden.contiguous().data_ptr(), lengths.data_ptr(), w_head.data_ptr(),
+                                                b_head.data_ptr(), expected.data_ptr(), batch, tokens, d_model,
+                                                _native.current_stream(device)), "masked_mean_head")
+    torch.testing.assert_close(p, expected, rtol=0, atol=2e-6)
+    assert abs(p[0].item() - torch.sigmoid(torch.tensor(0.25)).item()) < 1e-6    # no valid token: sigmoid(bias)
+    want = oracle.backbone(inputs.emb[1:], inputs.key_lengths[1:], inputs.blocks, inputs.head_weight, inputs.head_bias,
+                           num_heads=heads)
+    torch.testing.assert_close(p.cpu()[1:], want, rtol=0, atol=2e-2)
