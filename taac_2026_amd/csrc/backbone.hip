@@ -596,10 +596,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
   // the attention output as stacks of per-head planes [3 * heads][M][dh] / [heads][M][dh] instead of [M][3 * D] / [M][D]
   // rows: a head's rows are then contiguous for the attention kernel (64-byte pieces of 1 536-byte rows otherwise), and the
   // dense kernels on either side address the planes directly. TAAC_BACKBONE_ROW_MAJOR_QKV keeps the rows (same results).
-  bool planes = fused && !fp8 && !split_out_ffn && rope_cos_sin == nullptr && (dh == 32 || dh == 64) &&
-                !(flags & TAAC_BACKBONE_ROW_MAJOR_QKV);
-  for (int i = 0; i < n_blocks && planes; ++i)
-    planes = blocks[i].query_norm_weight == nullptr && blocks[i].key_norm_weight == nullptr;
+  const bool planes = fused && !fp8 && !split_out_ffn && (dh == 32 || dh == 64) && !(flags & TAAC_BACKBONE_ROW_MAJOR_QKV);
   const int64_t plane_elems = M * dh;
   const int64_t plane_strides[4] = {static_cast<int64_t>(T) * dh, plane_elems, dh, 1};
   // The last block's kernel (out projection + feed-forward in one) also leaves every token's dot product with the head
@@ -671,11 +668,16 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
                            as_stream(stream)) != hipSuccess)
           return set_error(TAAC_ERR_LAUNCH, "%s: copy of the query / key norm weights failed", name);
       }
-      if ((rc = taac_norm_linear_qk_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, qkv, 3 * D, M, D,
-                                        heads, T, weights_in_epilogue ? qk_weight : nullptr, rope_cos_sin,
-                                        qk_norm ? qk_sumsq : nullptr, rows, n_rows, nullptr,
-                                        w.attn_norm_weight != nullptr, stream)) != TAAC_OK)
-        return rc;
+      if (planes)
+        rc = norm_linear_qk_heads(cur, D, w.attn_norm_weight, eps, w.qkv_bias, pk_qkv, qkv, M, D, heads, T,
+                                  weights_in_epilogue ? qk_weight : nullptr, rope_cos_sin, qk_norm ? qk_sumsq : nullptr,
+                                  rows, n_rows, w.attn_norm_weight != nullptr, stream);
+      else
+        rc = taac_norm_linear_qk_fwd(cur, D, w.attn_norm_weight, eps, nullptr, w.qkv_bias, pk_qkv, qkv, 3 * D, M, D, heads,
+                                     T, weights_in_epilogue ? qk_weight : nullptr, rope_cos_sin,
+                                     qk_norm ? qk_sumsq : nullptr, rows, n_rows, nullptr, w.attn_norm_weight != nullptr,
+                                     stream);
+      if (rc != TAAC_OK) return rc;
       if (qk_norm) {
         if ((rc = taac_row_rstd(qk_sumsq, M, D, eps, qk_rstd, rows, n_rows, stream)) != TAAC_OK) return rc;
         q_scale = qk_rstd;
@@ -704,7 +706,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
     }
     if (planes) {
       if ((rc = taac_flash_attn_scaled_fwd(qkv, qkv + heads * plane_elems, qkv + 2 * heads * plane_elems, key_lengths,
-                                           nullptr, nullptr, nullptr, h, B, heads, T, T, dh, plane_strides, plane_strides,
+                                           q_scale, k_scale, q_col_scale, h, B, heads, T, T, dh, plane_strides, plane_strides,
                                            plane_strides, plane_strides, 0, rows ? 2 : 1, TAAC_BF16, stream)) != TAAC_OK)
         return rc;
       if ((rc = attn_out_ffn_readout(h, D, dh, w.out_bias, pk_out, cur, D, w.ffn_norm_weight, eps, w.up_bias, w.down_bias,

@@ -36,6 +36,12 @@ bool test_fp8_tiled();
 // Packs the qkv / out / feed-forward weights (gate first) of n backbone blocks into fragment order (ffn.hip).
 int pack_backbone_blocks(const taac_block_weights* blocks, int n, int32_t D, int32_t F, void* const* packed_qkv,
                          void* const* packed_out, void* const* packed_ffn, hipStream_t s, const char* name);
+// RMSNorm + q | k | v projection with the query / key epilogue (ffn.hip; the arguments of taac_norm_linear_qk_fwd with
+// packed weights) whose output is a stack of per-head planes [3 * num_heads][M][head_dim], head_dim 32 or 64.
+int norm_linear_qk_heads(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* bias,
+                         const void* packed_weights, void* out, int64_t M, int32_t d_model, int32_t num_heads,
+                         int32_t tokens_per_sample, const void* qk_weight, const void* cos_sin, float* qk_sumsq,
+                         const int32_t* rows, const int32_t* n_rows, int norm_folded, void* stream);
 // Out projection + feed-forward half of a block (ffn.hip; attn_plane: 0 = rows of ld_attn elements, 32 / 64 = per-head
 // planes) that also writes the dot product of every stored output row with head_w to token_dots[row].
 int attn_out_ffn_readout(const void* attn, int64_t ld_attn, int attn_plane, const void* out_bias,

@@ -1273,7 +1273,12 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
 #pragma unroll
               for (int e = 0; e < 8; ++e) v[e] = static_cast<bf16_t>(f[e]);
             }
-            __builtin_nontemporal_store(v, reinterpret_cast<bf16x8*>(p.out + static_cast<int64_t>(info[j].x) * p.ldo + col8));
+            // feature planes: column col8 lies in plane col8 >> shift, at col8 % 2^shift of the row
+            const int64_t at = p.out_plane_shift > 0
+                                   ? (((static_cast<int64_t>(col8 >> p.out_plane_shift) * p.M + info[j].x) << p.out_plane_shift) +
+                                      (col8 & ((1 << p.out_plane_shift) - 1)))
+                                   : static_cast<int64_t>(info[j].x) * p.ldo + col8;
+            __builtin_nontemporal_store(v, reinterpret_cast<bf16x8*>(p.out + at));
           }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -1652,8 +1657,9 @@ int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void*
                        const void* bias, const void* packed_weights, const void* residual, int64_t ldr, void* out,
                        int64_t ldo, int64_t M, int32_t N, int32_t K, const int32_t* rows, const int32_t* n_rows,
                        const int32_t* x_rows, const QkExtras& qk, int norm_folded, void* stream, int out_plane = 0) {
-  if (out_plane != 0 && (residual || qk.enabled || (out_plane != 32 && out_plane != 64) || static_cast<int64_t>(8) * M + 8 > 0xffffffffLL))
-    return set_error(TAAC_ERR_UNSUPPORTED, "%s: output planes are 32 or 64 features wide, without residual or query / key epilogue", name);
+  if (out_plane != 0 && (residual || (out_plane != 32 && out_plane != 64) || static_cast<int64_t>(8) * M + 8 > 0xffffffffLL ||
+                         (qk.enabled && qk.head_dim != out_plane)))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: output planes are 32 or 64 features wide (the head width under a query / key epilogue), without residual", name);
   if (norm_folded && (!norm_weight || !packed_weights))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: norm_folded needs the norm weight and the packed weights it was folded into", name);
   if (M < 0 || N <= 0 || K <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, N and K > 0", name);
@@ -1786,6 +1792,24 @@ extern "C" int taac_attn_out_ffn_heads_fwd(const void* attn, int32_t head_dim, c
 }
 
 namespace taac {
+// taac_norm_linear_qk_fwd (packed weights) writing q | k | v as per-head planes like taac_norm_linear_heads_fwd.
+int norm_linear_qk_heads(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* bias,
+                         const void* packed_weights, void* out, int64_t M, int32_t d_model, int32_t num_heads,
+                         int32_t tokens_per_sample, const void* qk_weight, const void* cos_sin, float* qk_sumsq,
+                         const int32_t* rows, const int32_t* n_rows, int norm_folded, void* stream) {
+  QkExtras qk;
+  qk.enabled = true;
+  qk.qk_weight = qk_weight;
+  qk.cos_sin = cos_sin;
+  qk.qk_sumsq = qk_sumsq;
+  qk.qk_chunks = 2 * d_model / kNC;
+  qk.head_dim = d_model / num_heads;
+  qk.tokens_per_sample = tokens_per_sample;
+  return norm_linear_launch("taac_backbone_fwd", x, ldx, norm_weight, eps, nullptr, bias, packed_weights, nullptr, 0, out,
+                            3 * d_model, M, 3 * d_model, d_model, rows, n_rows, nullptr, qk, norm_folded, stream,
+                            d_model / num_heads);
+}
+
 // taac_attn_out_ffn_fwd (attn_plane = 0) / taac_attn_out_ffn_heads_fwd (attn_plane = head_dim) that also leaves, for every
 // token it stores, the dot product of the output row with head_w in token_dots[row] (see TsParams::head_w).
 int attn_out_ffn_readout(const void* attn, int64_t ld_attn, int attn_plane, const void* out_bias,

@@ -163,6 +163,31 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
                                           None, 1, None)
     assert status == invalid and b"norm_folded needs" in library.taac_last_error()
 
+    # the same two layers on per-head planes: packed weights only, head_dim 32 or 64, model width 128 / 256
+    def plane_projection(**kw):
+        a = dict(packed=fake, head_dim=32, m=8, n=768, k=256)
+        a.update(kw)
+        return library.taac_norm_linear_heads_fwd(fake, a["k"], None, 1e-6, None, a["packed"], fake, a["head_dim"], a["m"],
+                                                  a["n"], a["k"], None, None, 0, None)
+
+    assert plane_projection(packed=None) == invalid and b"packed" in library.taac_last_error()
+    assert plane_projection(head_dim=16) == unsupported and b"head_dim" in library.taac_last_error()
+    assert plane_projection(k=192) == unsupported
+    assert plane_projection(m=0) == ok
+
+    def plane_tail(**kw):
+        a = dict(packed_out=fake, residual=fake, packed_ffn=fake, head_dim=64, d=256, f=64, m=8)
+        a.update(kw)
+        return library.taac_attn_out_ffn_heads_fwd(fake, a["head_dim"], None, a["packed_out"], a["residual"], a["d"], None,
+                                                   1e-6, None, None, a["packed_ffn"], fake, a["d"], a["m"], a["d"], a["f"],
+                                                   None, None, 0, None)
+
+    assert plane_tail(packed_out=None) == invalid and b"packed" in library.taac_last_error()
+    assert plane_tail(head_dim=48) == unsupported and b"head_dim" in library.taac_last_error()
+    assert plane_tail(residual=None) == invalid and b"block input" in library.taac_last_error()
+    assert plane_tail(d=192) == unsupported
+    assert plane_tail(m=0) == ok
+
     # readout: indices inside the sequence, one kind of validity, a complete classifier, something to write
     def readout(**kw):
         a = dict(lengths=None, bits=None, t=16, d=64, cls=0, cand=3, fc1=fake, fc2=fake, hidden=32, actions=1, emb=None,

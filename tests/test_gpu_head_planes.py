@@ -122,10 +122,20 @@ def test_one_block_in_planes_matches_the_oracle(device, d_model, heads):
 
 @pytest.mark.parametrize("d_model,heads,d_ff", [(256, 8, 1024), (256, 4, 512), (128, 4, 256), (128, 2, 512)])
 @pytest.mark.parametrize("dense_tokens", [False, True])
-def test_backbone_plane_route_equals_its_row_major_route(device, d_model, heads, d_ff, dense_tokens):
+@pytest.mark.parametrize("qk_norm,rope_base", [(False, None), (True, None), (True, 10000.0), (False, 10000.0)])
+def test_backbone_plane_route_equals_its_row_major_route(device, d_model, heads, d_ff, dense_tokens, qk_norm, rope_base):
+    """Also with the query / key norms and the rotary embedding of the reference's attention layers, whose projection
+    epilogue (statistic, weight, rotation) then stores into the planes."""
     inputs = workloads.backbone_inputs(batch=7, n_feature_tokens=16, n_sequence_tokens=240, d_model=d_model,
-                                       num_heads=heads, d_ff=d_ff, n_blocks=3, min_sequence_len=3, seed=d_model + heads)
-    model = PCVRBackbone(d_model=d_model, num_heads=heads, d_ff=d_ff, n_blocks=3)
+                                       num_heads=heads, d_ff=d_ff, n_blocks=3, min_sequence_len=3, seed=d_model + heads,
+                                       qk_norm=qk_norm)
+    g = torch.Generator().manual_seed(9)
+    for weights in inputs.blocks:
+        weights["qkv.bias"] = (0.05 * torch.randn(3 * d_model, generator=g)).to(torch.bfloat16)
+        if qk_norm:
+            weights["query_norm.weight"] = (1.0 + 0.1 * torch.randn(d_model, generator=g)).to(torch.bfloat16)
+            weights["key_norm.weight"] = (1.0 + 0.1 * torch.randn(d_model, generator=g)).to(torch.bfloat16)
+    model = PCVRBackbone(d_model=d_model, num_heads=heads, d_ff=d_ff, n_blocks=3, qk_norm=qk_norm, rope_base=rope_base)
     workloads.load_backbone_state(model, inputs)
     model = model.to(device=device, dtype=torch.bfloat16).eval()
     emb, lengths = inputs.emb.to(device), inputs.key_lengths.to(device)
