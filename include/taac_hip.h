@@ -150,8 +150,8 @@ int taac_flash_attn_fwd(const void* q, const void* k, const void* v, const int32
  * taac_flash_attn_fwd with one positive factor per query row and per key row, shared by the heads, and one factor
  * per query feature:
  *   scores = (q_row_scale[b, i] * q[b, h, i, :] * q_col_scale[h, :]) . (k_row_scale[b, j] * k[b, h, j, :]) / sqrt(d).
- * q_row_scale: fp32 [B, Tq] contiguous or NULL (all ones); k_row_scale: fp32 [B, Tk] or NULL; q_col_scale: fp32 [H, d]
- * or NULL. The query row factor joins the softmax scale (no rounding); the query features and the key rows are
+ * q_row_scale: fp32 [B, Tq] contiguous or NULL (all ones); k_row_scale: fp32 [B, Tk] or NULL; q_col_scale: fp32 [H, d],
+ * 16-byte aligned, or NULL. The query row factor joins the softmax scale (no rounding); the query features and the key rows are
  * multiplied in fp32 and rounded once to the storage dtype on their way to the MFMA. Factors of rows in the padding
  * are not read. Everything else as taac_flash_attn_fwd. (The weights of a query norm and of a key norm act on a score
  * only through their product, so q_col_scale = query weight * key weight applies both without touching the keys.)

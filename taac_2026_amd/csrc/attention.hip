@@ -147,6 +147,33 @@ __device__ __forceinline__ uint32_t keep_bytes4(const uint8_t* row, int key0, in
   return w;
 }
 
+// The lane's feature factors of the query (q_col_scale, fp32, 16-byte aligned rows): features 16 * s + 0..7 of k-step s,
+// counted from `offset`; fetched with two 16-byte loads per k-step, all requested before the first is used. Without
+// factors (or in kernels without them) the product is the scale alone.
+template <bool SCALED, int KSTEPS>
+struct QueryFeatureFactors {
+  f32x4 v[SCALED ? KSTEPS : 1][2];
+  bool present = false;
+  __device__ __forceinline__ void load(const float* q_col_scale, int offset) {
+    if constexpr (SCALED) {
+      present = q_col_scale != nullptr;  // uniform over the launch
+      if (present) {
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+          v[s][0] = *reinterpret_cast<const f32x4*>(q_col_scale + offset + 16 * s);
+          v[s][1] = *reinterpret_cast<const f32x4*>(q_col_scale + offset + 16 * s + 4);
+        }
+      }
+    }
+  }
+  __device__ __forceinline__ float times(int s, int e, float c) const {
+    if constexpr (SCALED) {
+      if (present) return v[s][e / 4][e % 4] * c;
+    }
+    return c;
+  }
+};
+
 template <typename T, int DP, bool CAUSAL, bool SCALED, bool MASKED, bool DROPOUT = false>
 __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnParams p) {
   static_assert(!(DROPOUT && SCALED && !MASKED), "dropout comes with the masks of the training path, not with row factors");
@@ -652,19 +679,23 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   if (CAUSAL) kv_end = kv_end < q_begin + kQB ? kv_end : q_begin + kQB;
 
   const int qi = q_begin + wave * 32 + l32;
-  float c = p.scale_log2;  // SCALED: the query's row factor joins the lane's softmax scale
-  if (SCALED && p.q_row_scale != nullptr && qi < q_valid) c *= p.q_row_scale[static_cast<int64_t>(b) * p.Tq + qi];
   // The query enters the products already multiplied by the softmax scale (and log2 e), rounded once more to the storage
-  // type: the score tiles then come out of the matrix unit in the exponent's units.
+  // type: the score tiles then come out of the matrix unit in the exponent's units. SCALED: the query's row factor joins
+  // the lane's softmax scale, the feature factors multiply it per feature. Every load is requested before the first
+  // value is used (one memory latency for the row factor, the query rows and the feature factors together).
+  float q_row_factor = 1.0f;
+  if (SCALED && p.q_row_scale != nullptr && qi < q_valid) q_row_factor = p.q_row_scale[static_cast<int64_t>(b) * p.Tq + qi];
   vec_t qf[KSTEPS];
 #pragma unroll
-  for (int s = 0; s < KSTEPS; ++s) {
+  for (int s = 0; s < KSTEPS; ++s)
     qf[s] = qi < q_valid ? *reinterpret_cast<const vec_t*>(qb + qi * p.qs[2] + 16 * s + 8 * hh) : zero_vec;
-    const float* cf = (SCALED && p.q_col_scale != nullptr) ? p.q_col_scale + h * p.d + 16 * s + 8 * hh : nullptr;
+  QueryFeatureFactors<SCALED, KSTEPS> feature_factors;
+  feature_factors.load(p.q_col_scale, h * p.d + 8 * hh);
+  const float c = (SCALED && p.q_row_scale != nullptr) ? p.scale_log2 * q_row_factor : p.scale_log2;
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
-      qf[s][e] = static_cast<T>(static_cast<float>(qf[s][e]) * (cf != nullptr ? cf[e] * c : c));
-  }
+  for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<T>(static_cast<float>(qf[s][e]) * feature_factors.times(s, e, c));
 
   f32x16 oacc[MB];
 #pragma unroll
@@ -1104,16 +1135,19 @@ __global__ __launch_bounds__(kSparseWaves * kWave) void flash_attn_fwd_sparse_ke
 
   // The query enters the products already multiplied by the softmax scale, log2 e and its row / feature factors, rounded
   // once more to the storage type: the score tiles come out of the matrix unit in the exponent's units.
-  float c = p.scale_log2;
-  if (SCALED && p.q_row_scale != nullptr && qi < q_valid) c *= p.q_row_scale[static_cast<int64_t>(b) * p.Tq + qi];
+  float q_row_factor = 1.0f;
+  if (SCALED && p.q_row_scale != nullptr && qi < q_valid) q_row_factor = p.q_row_scale[static_cast<int64_t>(b) * p.Tq + qi];
   vec_t qf[KSTEPS];
 #pragma unroll
-  for (int s = 0; s < KSTEPS; ++s) {
+  for (int s = 0; s < KSTEPS; ++s)
     qf[s] = qi < q_valid ? *reinterpret_cast<const vec_t*>(qb + qi * p.qs[2] + 16 * s + 8 * hh) : zero_vec;
-    const float* cf = (SCALED && p.q_col_scale != nullptr) ? p.q_col_scale + h * p.d + 16 * s + 8 * hh : nullptr;
+  QueryFeatureFactors<SCALED, KSTEPS> feature_factors;
+  feature_factors.load(p.q_col_scale, h * p.d + 8 * hh);
+  const float c = (SCALED && p.q_row_scale != nullptr) ? p.scale_log2 * q_row_factor : p.scale_log2;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<T>(static_cast<float>(qf[s][e]) * (cf != nullptr ? cf[e] * c : c));
-  }
+  for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<T>(static_cast<float>(qf[s][e]) * feature_factors.times(s, e, c));
   // ---- the tiles this wavefront visits: bit kt of `tiles` (none when every row is in the padding or self-only) -------
   const uint64_t words_with_valid_keys = __builtin_amdgcn_ballot_w64(valid_lane != 0u);
   uint64_t tiles = __builtin_amdgcn_ballot_w64((words_of_tile & words_with_valid_keys) != 0ull);
@@ -1455,8 +1489,8 @@ int attention_entry(const char* name, const void* q, const void* k, const void* 
   if (!strides_ok(q_strides) || !strides_ok(k_strides) || !strides_ok(v_strides) || !strides_ok(o_strides))
     return set_error(TAAC_ERR_UNSUPPORTED,
                      "%s: strides must be non-negative multiples of 8 elements with a unit last stride", name);
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
-    return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(q_col_scale))
+    return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers (and q_col_scale) must be 16-byte aligned", name);
   if (zero_padded_queries && Tq != Tk)
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: zero_padded_queries requires Tq == Tk", name);
 
