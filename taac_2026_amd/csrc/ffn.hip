@@ -226,25 +226,49 @@ __device__ __forceinline__ int64_t input_row(const TsParams& p, int64_t count, i
   return static_cast<int64_t>(p.x_rows[tok]);
 }
 
+// Rows of N tokens at once (token i = tok_of(i)): with an index its N entries are read inside ONE branch, all requested
+// before the first is used - token_row() per token puts every load behind its own test of the index pointer, and a wait
+// behind every load.
+template <int N, typename F>
+__device__ __forceinline__ void token_rows_batch(const int32_t* index, int64_t count, F tok_of, int64_t (&row)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    const int64_t tok = tok_of(i);
+    row[i] = tok < count ? tok : count - 1;
+  }
+  if (index != nullptr) {
+    int32_t v[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = index[row[i]];
+#pragma unroll
+    for (int i = 0; i < N; ++i) row[i] = static_cast<int64_t>(v[i]);
+  }
+}
+
 // Loads the wavefront's token rows as B-operand fragments: lane (l32, hh) holds features 16*ks + 8*hh .. +7 of token
 // l32 of each 32-token tile.
 template <int D, int TT>
 __device__ __forceinline__ void load_token_rows(const TsParams& p, int64_t count, int64_t tok0, int l32, int hh,
                                                 bf16x8 (&xf)[TT][D / 16]) {
   constexpr int KS = D / 16;
+  // the row numbers of all tiles first: one memory latency in front of the row loads, not one per tile
+  int64_t r[TT];
+  token_rows_batch<TT>(p.x_rows != nullptr ? p.x_rows : p.rows, count, [&](int t) { return tok0 + t * 32 + l32; }, r);
+  if (p.x_plane_shift > 0) {  // feature planes: k-step ks lies in plane (16 * ks) >> shift
+    const int sh = p.x_plane_shift;
+    const int64_t plane_elems = p.M << sh;
 #pragma unroll
-  for (int t = 0; t < TT; ++t) {
-    const int64_t r = input_row(p, count, tok0 + t * 32 + l32);
-    if (p.x_plane_shift > 0) {  // feature planes: k-step ks lies in plane (16 * ks) >> shift
-      const int sh = p.x_plane_shift;
-      const bf16_t* row = p.x + (r << sh) + hh * 8;
-      const int64_t plane_elems = p.M << sh;
+    for (int t = 0; t < TT; ++t) {
+      const bf16_t* row = p.x + (r[t] << sh) + hh * 8;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
         xf[t][ks] = *reinterpret_cast<const bf16x8*>(row + ((ks * 16) >> sh) * plane_elems + ((ks * 16) & ((1 << sh) - 1)));
-      continue;
     }
-    const bf16_t* row = p.x + r * p.ldx + hh * 8;
+    return;
+  }
+#pragma unroll
+  for (int t = 0; t < TT; ++t) {
+    const bf16_t* row = p.x + r[t] * p.ldx + hh * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) xf[t][ks] = *reinterpret_cast<const bf16x8*>(row + ks * 16);
   }
@@ -1056,20 +1080,28 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
   // multiply-add for its address instead of a 64-bit row * stride product per piece and step.
   const uint32_t ld16 = static_cast<uint32_t>(p.ldo >> 3);
   auto rows_of_tile = [&](int64_t tok_base, int32_t (&prow)[NST]) {
+    // all row numbers are requested before the first is used (one memory latency for the tile, not one per piece): the
+    // layout branch below must not sit between the loads
+    int64_t row64[NST];
+    token_rows_batch<NST>(p.rows, count, [&](int i) { return tok_base + (i / 4) * 32 + (i % 4) * 8 + lane / 8; }, row64);
 #pragma unroll
-    for (int i = 0; i < NST; ++i) {
-      const int32_t row = static_cast<int32_t>(token_row(p, count, tok_base + (i / 4) * 32 + (i % 4) * 8 + lane / 8));
-      if (!RES && p.out_plane_shift > 0) {
-        // feature planes: the lane's piece j = lane % 8 of a 64-feature chunk lies in plane (8 * j) >> shift of the chunk's
-        // planes, at 16-byte piece j % (plane width / 8) of the row
-        const int psh = p.out_plane_shift - 3;  // log2 of the 16-byte pieces per plane row
-        const uint32_t j = static_cast<uint32_t>(lane % 8);
-        prow[i] = static_cast<int32_t>((((j >> psh) * static_cast<uint32_t>(p.M) + static_cast<uint32_t>(row)) << psh) +
-                                       (j & ((1u << psh) - 1u)));
-        continue;
-      }
-      prow[i] = RES ? row : static_cast<int32_t>(static_cast<uint32_t>(row) * ld16 + static_cast<uint32_t>(lane % 8));
+    for (int i = 0; i < NST; ++i) prow[i] = static_cast<int32_t>(row64[i]);
+    if (RES) return;
+    if (p.out_plane_shift > 0) {
+      // feature planes: the lane's piece j = lane % 8 of a 64-feature chunk lies in plane (8 * j) >> shift of the chunk's
+      // planes, at 16-byte piece j % (plane width / 8) of the row
+      const int psh = p.out_plane_shift - 3;  // log2 of the 16-byte pieces per plane row
+      const uint32_t j = static_cast<uint32_t>(lane % 8);
+      const uint32_t plane_base = (j >> psh) * static_cast<uint32_t>(p.M);
+      const uint32_t piece = j & ((1u << psh) - 1u);
+#pragma unroll
+      for (int i = 0; i < NST; ++i)
+        prow[i] = static_cast<int32_t>(((plane_base + static_cast<uint32_t>(prow[i])) << psh) + piece);
+      return;
     }
+#pragma unroll
+    for (int i = 0; i < NST; ++i)
+      prow[i] = static_cast<int32_t>(static_cast<uint32_t>(prow[i]) * ld16 + static_cast<uint32_t>(lane % 8));
   };
   // bytes between the 64-feature chunks of the output: 128 in a row, 64 features of M rows in the plane layout
   const int64_t chunk_bytes = (!RES && p.out_plane_shift > 0) ? static_cast<int64_t>(kNC) * 2 * p.M : kNC * 2;
