@@ -226,34 +226,51 @@ __device__ __forceinline__ int64_t input_row(const TsParams& p, int64_t count, i
   return static_cast<int64_t>(p.x_rows[tok]);
 }
 
-// Rows of N tokens at once (token i = tok_of(i)): with an index its N entries are read inside ONE branch, all requested
-// before the first is used - token_row() per token puts every load behind its own test of the index pointer, and a wait
-// behind every load.
+// Rows of N tokens at once (token i = tok_of(i)), in two phases: request() issues the N index loads inside ONE test of
+// the index pointer and touches none of the loaded values, row() turns entry i into a row number. Whatever the caller
+// requests between the two is in flight together with the index (token_row() per token puts every load behind its own
+// test of the pointer and a wait behind every load).
+template <int N>
+struct TokenRows {
+  int64_t tok[N];
+  int32_t loaded[N];
+  bool indexed;
+  template <typename F>
+  __device__ __forceinline__ void request(const int32_t* index, int64_t count, F tok_of) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int64_t t = tok_of(i);
+      tok[i] = t < count ? t : count - 1;
+      loaded[i] = 0;
+    }
+    indexed = index != nullptr;
+    if (indexed) {
+#pragma unroll
+      for (int i = 0; i < N; ++i) loaded[i] = index[tok[i]];
+    }
+  }
+  // Marks the point up to which the loaded entries stay untouched (the compiler would otherwise widen them right behind
+  // their loads, with a wait in front).
+  __device__ __forceinline__ void arrive() {
+#pragma unroll
+    for (int i = 0; i < N; ++i) asm volatile("" : "+v"(loaded[i]));
+  }
+  __device__ __forceinline__ int64_t row(int i) const { return indexed ? static_cast<int64_t>(loaded[i]) : tok[i]; }
+};
 template <int N, typename F>
 __device__ __forceinline__ void token_rows_batch(const int32_t* index, int64_t count, F tok_of, int64_t (&row)[N]) {
+  TokenRows<N> rows;
+  rows.request(index, count, tok_of);
 #pragma unroll
-  for (int i = 0; i < N; ++i) {
-    const int64_t tok = tok_of(i);
-    row[i] = tok < count ? tok : count - 1;
-  }
-  if (index != nullptr) {
-    int32_t v[N];
-#pragma unroll
-    for (int i = 0; i < N; ++i) v[i] = index[row[i]];
-#pragma unroll
-    for (int i = 0; i < N; ++i) row[i] = static_cast<int64_t>(v[i]);
-  }
+  for (int i = 0; i < N; ++i) row[i] = rows.row(i);
 }
 
 // Loads the wavefront's token rows as B-operand fragments: lane (l32, hh) holds features 16*ks + 8*hh .. +7 of token
 // l32 of each 32-token tile.
+// The same from row numbers the caller already holds (r[t]: memory row of token l32 of tile t).
 template <int D, int TT>
-__device__ __forceinline__ void load_token_rows(const TsParams& p, int64_t count, int64_t tok0, int l32, int hh,
-                                                bf16x8 (&xf)[TT][D / 16]) {
+__device__ __forceinline__ void load_token_rows_at(const TsParams& p, const int64_t (&r)[TT], int hh, bf16x8 (&xf)[TT][D / 16]) {
   constexpr int KS = D / 16;
-  // the row numbers of all tiles first: one memory latency in front of the row loads, not one per tile
-  int64_t r[TT];
-  token_rows_batch<TT>(p.x_rows != nullptr ? p.x_rows : p.rows, count, [&](int t) { return tok0 + t * 32 + l32; }, r);
   if (p.x_plane_shift > 0) {  // feature planes: k-step ks lies in plane (16 * ks) >> shift
     const int sh = p.x_plane_shift;
     const int64_t plane_elems = p.M << sh;
@@ -272,6 +289,15 @@ __device__ __forceinline__ void load_token_rows(const TsParams& p, int64_t count
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) xf[t][ks] = *reinterpret_cast<const bf16x8*>(row + ks * 16);
   }
+}
+
+template <int D, int TT>
+__device__ __forceinline__ void load_token_rows(const TsParams& p, int64_t count, int64_t tok0, int l32, int hh,
+                                                bf16x8 (&xf)[TT][D / 16]) {
+  // the row numbers of all tiles first: one memory latency in front of the row loads, not one per tile
+  int64_t r[TT];
+  token_rows_batch<TT>(p.x_rows != nullptr ? p.x_rows : p.rows, count, [&](int t) { return tok0 + t * 32 + l32; }, r);
+  load_token_rows_at<D, TT>(p, r, hh, xf);
 }
 
 // RMS-normalises the loaded rows in place: y = bf16( x * rsqrt(mean(x^2) + eps) * w ), w read from its LDS copy.
@@ -342,25 +368,6 @@ __device__ __forceinline__ void token_rstd(float eps, const bf16x8 (&xf)[TT][D /
       }
     ss += __shfl_xor(ss, 32, kWave);
     rstd[t] = rsqrtf(ss * (1.0f / D) + eps);
-  }
-}
-
-// Up-projection bias in fragment row order: entry chunk * 32 + m belongs to row slot m of the chunk's up fragment
-// (slots 0..15 the gated half, 16..31 the other half), so lane l32 of a wavefront finds the bias of its fragment row at
-// chunk * 32 + l32. Zeros when there is no bias.
-__device__ __forceinline__ void stage_up_bias(const bf16_t* b_up, bf16_t* dst, int F, int gate_first, int tid,
-                                              int nthreads) {
-  for (int i = tid; i < 2 * F; i += nthreads) {
-    const int m = i % 32;
-    const int src = ((m < 16) == (gate_first != 0) ? 0 : F) + (i / 32) * kHU + up_unit_of_slot(m % 16);
-    dst[i] = b_up != nullptr ? b_up[src] : static_cast<bf16_t>(0.f);
-  }
-}
-// The same for the plain MLP: a chunk's fragment has 32 hidden units, slots 0..15 the first 16, slots 16..31 the others.
-__device__ __forceinline__ void stage_mlp_bias(const bf16_t* b1, bf16_t* dst, int F, int tid, int nthreads) {
-  for (int i = tid; i < F; i += nthreads) {
-    const int m = i % 32;
-    dst[i] = b1 != nullptr ? b1[(i / 32) * 32 + 16 * (m / 16) + up_unit_of_slot(m % 16)] : static_cast<bf16_t>(0.f);
   }
 }
 
@@ -586,20 +593,67 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
   if constexpr (OUTP) stage_proj(0, 1);
   // The token rows (a row-index load, then the rows) are requested before the bias vectors are staged, so that the two
   // chains of memory latencies run side by side; OUTP: so is the row number of the block input read by the projection.
-  bf16x8 xf[TT][KS];
-  if (active) load_token_rows<D, TT>(p, count, tok0, l32, hh, xf);
-  [[maybe_unused]] int64_t hrow_index[TT];
-  if constexpr (OUTP) {
+  // The workgroup's start is a chain of memory latencies with nothing to hide them behind (it owns the compute unit), so
+  // everything that does not depend on something else is requested at once: the row numbers of the wavefront's tokens and
+  // the bias vectors first (their values stay in registers), then - one latency later - the token rows, and only then
+  // are the bias vectors written to LDS. Two latencies instead of one per vector.
+  TokenRows<TT> out_rows, x_rows;  // rows of the wavefront's tokens in residual / out, and in x when x has an index of its own
+  out_rows.request(p.rows, count, [&](int t) { return tok0 + t * 32 + l32; });
+  x_rows.request(p.x_rows, count, [&](int t) { return tok0 + t * 32 + l32; });
+  constexpr int kThreadsWg = NWAVES * kWave;
+  constexpr int UB = 4;  // first-layer bias entries per thread held in registers (F <= UB * threads / 2 needs no second round)
+  // First-layer bias in fragment row order: entry chunk * 32 + m belongs to row slot m of the chunk's up fragment (GLU: slots
+  // 0..15 the gated half, 16..31 the other half; plain MLP: slots 0..15 the chunk's first 16 units, 16..31 the others), so
+  // lane l32 of a wavefront finds the bias of its fragment row at chunk * 32 + l32. Zeros when there is no bias.
+  auto up_bias_src = [&](int i) -> int {  // index into b1 of staged entry i
+    const int m = i % 32;
+    if constexpr (GLU)
+      return ((m < 16) == (p.gate_first != 0) ? 0 : F) + (i / 32) * kHU + up_unit_of_slot(m % 16);
+    else
+      return (i / 32) * 32 + 16 * (m / 16) + up_unit_of_slot(m % 16);
+  };
+  bf16_t up_bias_regs[UB];
 #pragma unroll
-    for (int t = 0; t < TT; ++t) hrow_index[t] = token_row(p, count, tok0 + t * 32 + l32);
+  for (int u = 0; u < UB; ++u) up_bias_regs[u] = static_cast<bf16_t>(0.f);
+  if (p.b1 != nullptr) {
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+      const int i = tid + u * kThreadsWg;
+      up_bias_regs[u] = p.b1[up_bias_src(i < UPB ? i : UPB - 1)];
+    }
   }
-  if constexpr (GLU)
-    stage_up_bias(p.b1, bias_lds, F, p.gate_first, tid, NWAVES * kWave);
-  else
-    stage_mlp_bias(p.b1, bias_lds, F, tid, NWAVES * kWave);
-  stage_bias(p.b2, bias_lds + UPB, D, tid, NWAVES * kWave);
-  if (p.norm_w != nullptr) stage_bias(p.norm_w, bias_lds + UPB + D, D, tid, NWAVES * kWave);
-  if constexpr (OUTP) stage_bias(p.b0, bias_lds + UPB + 2 * D, D, tid, NWAVES * kWave);
+  const int vec_at = tid * 8 < D ? tid * 8 : D - 8;  // the D-wide vectors: 16 bytes per thread, the first D / 8 threads store
+  bf16x8 b2_regs, normw_regs, b0_regs;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) b2_regs[e] = normw_regs[e] = b0_regs[e] = static_cast<bf16_t>(0.f);
+  if (p.b2 != nullptr) b2_regs = *reinterpret_cast<const bf16x8*>(p.b2 + vec_at);
+  if (p.norm_w != nullptr) normw_regs = *reinterpret_cast<const bf16x8*>(p.norm_w + vec_at);
+  if constexpr (OUTP) {
+    if (p.b0 != nullptr) b0_regs = *reinterpret_cast<const bf16x8*>(p.b0 + vec_at);
+  }
+  out_rows.arrive();
+  x_rows.arrive();
+  int64_t hrow_index[TT];  // OUTP: where the projection reads the block input
+  int64_t xrow_index[TT];
+#pragma unroll
+  for (int t = 0; t < TT; ++t) {
+    hrow_index[t] = out_rows.row(t);
+    xrow_index[t] = p.x_rows != nullptr ? x_rows.row(t) : hrow_index[t];
+  }
+  bf16x8 xf[TT][KS];
+  if (active) load_token_rows_at<D, TT>(p, xrow_index, hh, xf);
+#pragma unroll
+  for (int u = 0; u < UB; ++u) {
+    const int i = tid + u * kThreadsWg;
+    if (i < UPB) bias_lds[i] = up_bias_regs[u];
+  }
+  for (int i = tid + UB * kThreadsWg; i < UPB; i += kThreadsWg)  // wider hidden layers: the rest, one entry at a time
+    bias_lds[i] = p.b1 != nullptr ? p.b1[up_bias_src(i)] : static_cast<bf16_t>(0.f);
+  if (tid * 8 < D) {
+    *reinterpret_cast<bf16x8*>(bias_lds + UPB + vec_at) = b2_regs;
+    if (p.norm_w != nullptr) *reinterpret_cast<bf16x8*>(bias_lds + UPB + D + vec_at) = normw_regs;
+    if constexpr (OUTP) *reinterpret_cast<bf16x8*>(bias_lds + UPB + 2 * D + vec_at) = b0_regs;
+  }
 
   f32x16 oacc[TT][MB];
 #pragma unroll
