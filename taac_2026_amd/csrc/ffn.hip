@@ -1798,7 +1798,7 @@ int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void*
   p.tokens_per_sample = qk.tokens_per_sample;
   hipStream_t s = as_stream(stream);
   // Without a residual two token tiles per wavefront fit the register file: every weight fragment read from LDS then
-  // feeds two MFMAs, which halves the LDS traffic that otherwise caps the kernel.
+  // feeds two MFMAs, which halves the LDS reads (and their share of the power budget) per token.
   const int tt = residual ? 1 : 2;
   const int64_t tiles64 = (M + 256 * tt - 1) / (256 * tt);
   if (tiles64 > 0x3fffffffLL) return set_error(TAAC_ERR_UNSUPPORTED, "%s: too many token tiles", name);
