@@ -149,7 +149,7 @@ def test_backbone_plane_route_equals_its_row_major_route(device, d_model, heads,
         assert torch.equal(hidden, hidden_rows)
 
 
-@pytest.mark.parametrize("d_model,heads,d_ff", [(256, 8, 1024), (128, 2, 256)])
+@pytest.mark.parametrize("d_model,heads,d_ff", [(256, 8, 1024), (128, 2, 256), (128, 8, 256)])  # head widths 32, 64, 16 (rows)
 @pytest.mark.parametrize("dense_tokens", [False, True])
 def test_readout_riding_on_the_last_block_equals_the_readout_kernel(device, d_model, heads, d_ff, dense_tokens):
     """The last block's kernel leaves every token's dot product with the head weight behind and the readout adds those;
