@@ -377,9 +377,16 @@ __device__ __forceinline__ void read_chunk_bias(const bf16_t* bias_lds, int hh, 
   for (int q = 0; q < 8; ++q) bv[q] = *reinterpret_cast<const bf16x4*>(bias_lds + (q / 4) * 32 + (q % 4) * 8 + hh * 4);
 }
 
+// The same from a float32 copy of the bias (no widening per value in the epilogue).
+__device__ __forceinline__ void read_chunk_bias(const float* bias_lds, int hh, f32x4 (&bv)[8]) {
+#pragma unroll
+  for (int q = 0; q < 8; ++q) bv[q] = *reinterpret_cast<const f32x4*>(bias_lds + (q / 4) * 32 + (q % 4) * 8 + hh * 4);
+}
+
 // Writes two 32-feature accumulator blocks (64 features) of one 32-token tile into the wavefront's epilogue tile,
 // adding the bias and rounding to bf16. Accumulator register jq*4 + e of lane (l32, hh) is feature jq*8 + hh*4 + e.
-__device__ __forceinline__ void tile_to_lds(uint8_t* tile, const f32x16& a0, const f32x16& a1, const bf16x4 (&bv)[8],
+template <typename BiasVec>  // bf16x4 or f32x4 pieces
+__device__ __forceinline__ void tile_to_lds(uint8_t* tile, const f32x16& a0, const f32x16& a1, const BiasVec (&bv)[8],
                                             int l32, int hh, float scale = 1.0f) {
 #pragma unroll
   for (int rb = 0; rb < 2; ++rb) {
@@ -1080,6 +1087,9 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
   // QK: (memory row, position in the sample) of the wavefront's tokens, kept in LDS behind the bias and norm weights
   // (written and read by the same wavefront only), instead of in registers.
   int2* rowinfo = reinterpret_cast<int2*>(reinterpret_cast<uint8_t*>(bias_lds) + ((p.N + D) * 2 + 15) / 16 * 16) + wave * kWave;
+  // QK == 0: a float32 copy of the bias in the same place (the epilogue adds it in float32: read as it is needed, the
+  // widening of 64 values per step and wavefront is done once per workgroup instead)
+  float* bias_f32 = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(bias_lds) + ((p.N + D) * 2 + 15) / 16 * 16);
   const int nchunks = p.N / kNC;
   const int64_t count = token_count(p);
   const int num_tiles = static_cast<int>((count + kTokPerWg - 1) / kTokPerWg);
@@ -1201,7 +1211,23 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
   stage(chunk_of(0), 0);
   if (total > 1) stage(chunk_of(1), 1);
   if (RES) request_residual(prow, chunk_of(0), res_cur);
-  stage_bias(p.b1, bias_lds, p.N, tid, NWAVES * kWave);
+  if constexpr (QK == 0) {
+    for (int i = tid * 8; i < p.N; i += NWAVES * kWave * 8) {
+      f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+      if (p.b1 != nullptr) {
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(p.b1 + i);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          lo[e] = static_cast<float>(v[e]);
+          hi[e] = static_cast<float>(v[4 + e]);
+        }
+      }
+      *reinterpret_cast<f32x4*>(bias_f32 + i) = lo;
+      *reinterpret_cast<f32x4*>(bias_f32 + i + 4) = hi;
+    }
+  } else {
+    stage_bias(p.b1, bias_lds, p.N, tid, NWAVES * kWave);
+  }
   if (p.norm_w != nullptr) stage_bias(p.norm_w, bias_lds + p.N, D, tid, NWAVES * kWave);
   load_tile(tok_wave);
   vm_wait<0>();
@@ -1269,12 +1295,14 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     TAAC_READ_PAIR(1);
     TAAC_READ_PAIR(2);
     TAAC_READ_PAIR(3);
-#pragma unroll
-    for (int k4 = 0; k4 < KS; k4 += 4) {
-      const bool last = k4 + 4 >= KS;
+    // (compile-time k-steps: the fragment offsets of the reads go into the instructions' offset fields instead of a vector
+    // add per read)
+    static_for<KS / 4>([&](auto kc) {
+      constexpr int k4 = 4 * decltype(kc)::value;
+      constexpr bool last = k4 + 4 >= KS;
       // pair k4 + i: pairs up to k4 + i + 3 (or KS - 1) have been requested after it
 #define TAAC_STEP(I_)                                                                                   \
-  if (last)                                                                                             \
+  if constexpr (last)                                                                                   \
     lds_wait_pair<2 * (3 - (I_))>(fa[I_], fb[I_]);                                                       \
   else                                                                                                  \
     lds_wait_pair<6>(fa[I_], fb[I_]);                                                                    \
@@ -1283,22 +1311,29 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     acc1[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[I_], xf[t][k4 + (I_)], acc1[t], 0, 0, 0);      \
   }                                                                                                     \
   __builtin_amdgcn_sched_barrier(0)
+#define TAAC_NEXT_PAIR(I_)                                           \
+  if constexpr (!last) {                                             \
+    lds_read_frag<(k4 + 4 + (I_)) * kFrag>(fa[I_], wb);              \
+    lds_read_frag<(KS + k4 + 4 + (I_)) * kFrag>(fb[I_], wb);         \
+  }
       // The read of pair k4 + 4 + i reuses the registers of pair k4 + i right after its two MFMAs were issued.
       TAAC_STEP(0);
-      if (!last) { lds_read_frag<0>(fa[0], wb + (k4 + 4) * kFrag); lds_read_frag<0>(fb[0], wb + (KS + k4 + 4) * kFrag); }
+      TAAC_NEXT_PAIR(0)
       TAAC_STEP(1);
-      if (!last) { lds_read_frag<0>(fa[1], wb + (k4 + 5) * kFrag); lds_read_frag<0>(fb[1], wb + (KS + k4 + 5) * kFrag); }
+      TAAC_NEXT_PAIR(1)
       TAAC_STEP(2);
-      if (!last) { lds_read_frag<0>(fa[2], wb + (k4 + 6) * kFrag); lds_read_frag<0>(fb[2], wb + (KS + k4 + 6) * kFrag); }
+      TAAC_NEXT_PAIR(2)
       TAAC_STEP(3);
-      if (!last) { lds_read_frag<0>(fa[3], wb + (k4 + 7) * kFrag); lds_read_frag<0>(fb[3], wb + (KS + k4 + 7) * kFrag); }
+      TAAC_NEXT_PAIR(3)
+#undef TAAC_NEXT_PAIR
 #undef TAAC_STEP
-    }
+    });
 #undef TAAC_READ_PAIR
 
     // ---- epilogue of this chunk: bias, rounding, transpose through LDS, residual, 4 stores ---------------------------
-    bf16x4 bv[8];
-    if constexpr (QK == 0) read_chunk_bias(bias_lds + chunk * kNC, hh, bv);
+    [[maybe_unused]] bf16x4 bv[8];
+    [[maybe_unused]] f32x4 bvf[8];
+    if constexpr (QK == 0) read_chunk_bias(bias_f32 + chunk * kNC, hh, bvf);
     if constexpr (QK != 0) {
       // Query and key chunks: the sum of squares of the rounded projection goes to qk_sumsq (one value per token and
       // chunk; the statistic of the norm over the model width is their sum). QK == 2 also multiplies the features by
@@ -1372,7 +1407,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void norm_linear_kernel(const TsParam
     }
 #pragma unroll
     for (int t = 0; t < (QK != 0 ? 0 : TT); ++t) {
-      tile_to_lds(tile_lds, acc0[t], acc1[t], bv, l32, hh, rstd[t]);
+      tile_to_lds(tile_lds, acc0[t], acc1[t], bvf, l32, hh, rstd[t]);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -1766,7 +1801,8 @@ int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void*
       !ptr_ok(bias, 15) || !ptr_ok(packed_weights, 15) || !ptr_ok(qk.qk_weight, 15) || !ptr_ok(qk.cos_sin, 15) ||
       !ptr_ok(qk.qk_sumsq, 3))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: tensor base pointers must be 16-byte aligned", name);
-  const size_t rowinfo_bytes = qk.enabled ? 16 + 8 * static_cast<size_t>(kWave) * sizeof(int2) : 0;
+  // behind the 16-bit bias and norm weight: the query / key epilogue's row table, or the float32 copy of the bias
+  const size_t rowinfo_bytes = qk.enabled ? 16 + 8 * static_cast<size_t>(kWave) * sizeof(int2) : 16 + static_cast<size_t>(N) * 4;
   const size_t lds_bytes = static_cast<size_t>(3 * 2 * (K / 16)) * kFrag + 8 * static_cast<size_t>(kStageWave) +
                            static_cast<size_t>(N + K) * 2 + rowinfo_bytes;
   if (lds_bytes > kMaxLdsBytes)
