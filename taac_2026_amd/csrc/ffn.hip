@@ -261,6 +261,9 @@ template <int N, typename F>
 __device__ __forceinline__ void token_rows_batch(const int32_t* index, int64_t count, F tok_of, int64_t (&row)[N]) {
   TokenRows<N> rows;
   rows.request(index, count, tok_of);
+  // the entries are awaited here, on this path: left pending, the compiler protects their registers with waits for ALL
+  // vector-memory operations wherever the paths of the caller meet again (in front of the MFMAs of every step)
+  rows.arrive();
 #pragma unroll
   for (int i = 0; i < N; ++i) row[i] = rows.row(i);
 }
