@@ -443,7 +443,12 @@ __device__ __forceinline__ void tile_to_global(const uint8_t* tile, bf16_t* out,
                                                const bool (&live)[4], int col0, const bf16x8 (&res)[4], int lane,
                                                const bf16_t* head_w, float (&hdot)[4]) {
   bf16x8 hw;
-  if (head_w != nullptr) hw = *reinterpret_cast<const bf16x8*>(head_w + col0 + (lane % 8) * 8);
+  if (head_w != nullptr) {
+    hw = *reinterpret_cast<const bf16x8*>(head_w + col0 + (lane % 8) * 8);
+    // awaited here, on the path that loads it: otherwise the wait (for every vector-memory operation, the stores of the
+    // tile included) lands where the paths meet again, in front of the next piece of every launch
+    asm volatile("" : "+v"(hw));
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int row = i * 8 + lane / 8;
@@ -1010,11 +1015,9 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
     const int64_t tok_base = tok0 + t * 32;
     int64_t prow[4];
     bool live[4];
+    token_rows_batch<4>(p.rows, count, [&](int i) { return tok_base + i * 8 + lane / 8; }, prow);  // one memory latency, not four
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      prow[i] = token_row(p, count, tok_base + i * 8 + lane / 8);
-      live[i] = tok_base + i * 8 + lane / 8 < wg_tok0 + wg_ntok;
-    }
+    for (int i = 0; i < 4; ++i) live[i] = tok_base + i * 8 + lane / 8 < wg_tok0 + wg_ntok;
     float hdot[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int pr = 0; pr < MB / 2; ++pr) {  // 64 features at a time
