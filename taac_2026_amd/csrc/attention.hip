@@ -685,10 +685,13 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   // value is used (one memory latency for the row factor, the query rows and the feature factors together).
   float q_row_factor = 1.0f;
   if (SCALED && p.q_row_scale != nullptr && qi < q_valid) q_row_factor = p.q_row_scale[static_cast<int64_t>(b) * p.Tq + qi];
+  // A lane whose query lies in the padding reads the block's first row instead (valid here: the block holds a valid query):
+  // finite values whose results are never used (the lane's output factor is zero and its row is not stored) - and a load
+  // without a branch around it, so that its wait can sink below the requests for the first K / V chunks.
+  const int q_row_read = qi < q_valid ? qi : q_begin;
   vec_t qf[KSTEPS];
 #pragma unroll
-  for (int s = 0; s < KSTEPS; ++s)
-    qf[s] = qi < q_valid ? *reinterpret_cast<const vec_t*>(qb + qi * p.qs[2] + 16 * s + 8 * hh) : zero_vec;
+  for (int s = 0; s < KSTEPS; ++s) qf[s] = *reinterpret_cast<const vec_t*>(qb + q_row_read * p.qs[2] + 16 * s + 8 * hh);
   QueryFeatureFactors<SCALED, KSTEPS> feature_factors;
   feature_factors.load(p.q_col_scale, h * p.d + 8 * hh);
   const float c = (SCALED && p.q_row_scale != nullptr) ? p.scale_log2 * q_row_factor : p.scale_log2;
