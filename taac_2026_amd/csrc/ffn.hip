@@ -655,8 +655,10 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
     hrow_index[t] = out_rows.row(t);
     xrow_index[t] = p.x_rows != nullptr ? x_rows.row(t) : hrow_index[t];
   }
+  // (wavefronts without tokens load as well - their row numbers are clamped to the last token: a load behind a branch leaves
+  // its registers pending where the paths meet, and the compiler then waits for them again in every later block of code)
   bf16x8 xf[TT][KS];
-  if (active) load_token_rows_at<D, TT>(p, xrow_index, hh, xf);
+  load_token_rows_at<D, TT>(p, xrow_index, hh, xf);
 #pragma unroll
   for (int u = 0; u < UB; ++u) {
     const int i = tid + u * kThreadsWg;
@@ -679,6 +681,13 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
       for (int j = 0; j < 16; ++j) oacc[t][mb][j] = 0.f;
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // The token rows have landed; the compiler is told so here, on the one path every wavefront takes: used for the first
+  // time inside the `if (active)` blocks below, they would count as pending again wherever such a block ends, and every
+  // later block would wait for them anew (with counts that also cover the transfers and loads issued by hand).
+#pragma unroll
+  for (int t = 0; t < TT; ++t)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(xf[t][ks]));
   __syncthreads();
   if (!OUTP && active && p.norm_w != nullptr) normalize_tokens<D, TT>(p.eps, bias_lds + UPB + D, hh, xf, p.norm_folded != 0);
 
@@ -745,7 +754,11 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
               hv[t][q] = *reinterpret_cast<const bf16x4*>(hrow[t] + c * kNC + (q / 4) * 32 + (q % 4) * 8);
           } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) hf[t][j] = *reinterpret_cast<const bf16x8*>(hrow[t] + c * kNC + j * 16);
+            for (int j = 0; j < 4; ++j)  // requested by hand: the wait behind the chunk's MFMAs is counted by hand as well
+              asm volatile("global_load_dwordx4 %0, %1, off offset:%2"
+                           : "=v"(hf[t][j])
+                           : "v"(hrow[t]), "n"((c * kNC + j * 16) * 2)
+                           : "memory");
           }
         }
         if constexpr (!GATE) {
@@ -770,6 +783,19 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
           __builtin_amdgcn_sched_barrier(0);
           if constexpr (i + P < CF) lds_read_frag<(i + P) * kFrag>(pring[i % P], wb0);
         });
+        if constexpr (!GATE) {
+          // The block input of this chunk, requested in front of the next chunk's weight transfers: awaited by hand, with
+          // those transfers left in flight. (The compiler's own count does not know the transfers, so its wait for these
+          // registers - placed at their first use - would be a wait for the transfers as well, with the epilogue
+          // arithmetic of this chunk still to come.)
+          constexpr int kNewer = c + 1 < NCH ? CF / NWAVES : 0;  // transfers of stage_proj(c + 1) per wavefront
+#pragma unroll
+          for (int t = 0; t < TT; ++t)  // the pieces are tied to the wait so that their consumers cannot move above it
+            asm volatile("s_waitcnt vmcnt(%4)"
+                         : "+v"(hf[t][0]), "+v"(hf[t][1]), "+v"(hf[t][2]), "+v"(hf[t][3])
+                         : "n"(kNewer)
+                         : "memory");
+        }
         if constexpr (GATE) {
           // x1 = bf16( bf16(sigmoid(g)) * bf16(projection + b0) + h ), kept in the accumulators; sum of squares for the
           // norm that follows
