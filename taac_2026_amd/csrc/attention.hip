@@ -538,7 +538,7 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_kernel(const AttnPara
   }
 
   // ---- finalise: O / l (0 for rows in the padding), transpose through a wavefront-private LDS tile, 16-byte stores --
-  const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+  const float inv = l_run > 0.f ? __builtin_amdgcn_rcpf(l_run) : 0.f;  // 1 ulp; the products are rounded to 16 bits
   const float fin = (qi < q_valid) ? inv : 0.f;
   if (p.lse != nullptr && hh == 0 && qi < p.Tq)
     p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Tq + qi] =
@@ -689,9 +689,12 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   // finite values whose results are never used (the lane's output factor is zero and its row is not stored) - and a load
   // without a branch around it, so that its wait can sink below the requests for the first K / V chunks.
   const int q_row_read = qi < q_valid ? qi : q_begin;
+  // (rows of q and of the output are addressed like the K / V sources: a 24-bit multiply into a 32-bit byte offset)
+  const uint8_t* q_row_ptr = reinterpret_cast<const uint8_t*>(qb) +
+                             (__umul24(static_cast<uint32_t>(q_row_read), static_cast<uint32_t>(p.qs[2]) * 2u) + 16u * hh);
   vec_t qf[KSTEPS];
 #pragma unroll
-  for (int s = 0; s < KSTEPS; ++s) qf[s] = *reinterpret_cast<const vec_t*>(qb + q_row_read * p.qs[2] + 16 * s + 8 * hh);
+  for (int s = 0; s < KSTEPS; ++s) qf[s] = *reinterpret_cast<const vec_t*>(q_row_ptr + 32 * s);
   QueryFeatureFactors<SCALED, KSTEPS> feature_factors;
   feature_factors.load(p.q_col_scale, h * p.d + 8 * hh);
   const float c = (SCALED && p.q_row_scale != nullptr) ? p.scale_log2 * q_row_factor : p.scale_log2;
@@ -910,18 +913,22 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
         const float mxp = pair_max(mx);
         const bool move = mxp > thr;
         const float shift = move ? mxp : 0.f;
-        const float alpha = (move && m_set) ? __builtin_amdgcn_exp2f(-mxp) : 1.f;
 #pragma unroll
         for (int kt = 0; kt < NT; ++kt)
 #pragma unroll
           for (int j = 0; j < 16; ++j) sacc[kt][j] -= shift;
 #pragma unroll
         for (int j = 0; j < 16; ++j) negm[j] -= shift;
-        l_lane *= alpha;
+        // what a query has accumulated is rescaled only if some query of the wavefront has accumulated anything: not at
+        // a query block's first visible tile, which is where the reference almost always moves
+        if (__builtin_amdgcn_ballot_w64(move && m_set) != 0) {
+          const float alpha = (move && m_set) ? __builtin_amdgcn_exp2f(-mxp) : 1.f;
+          l_lane *= alpha;
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
+          for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-          for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;
+            for (int j = 0; j < 16; ++j) oacc[mb][j] *= alpha;
+        }
         if (move) {
           m_set = true;
           thr = kLazyBits;
@@ -985,7 +992,7 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
   for (; chunk < nchunks; ++chunk) step(chunk, std::integral_constant<int, 0>{});
 
   const float l_run = pair_sum(l_lane);
-  const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+  const float inv = l_run > 0.f ? __builtin_amdgcn_rcpf(l_run) : 0.f;  // 1 ulp; the products are rounded to 16 bits
   const float fin = (qi < q_valid) ? inv : 0.f;
   if (p.lse != nullptr && hh == 0 && qi < p.Tq)
     p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Tq + qi] =
@@ -1023,7 +1030,9 @@ __global__ __launch_bounds__(kThreads) void flash_attn_fwd_dma_kernel(const Attn
     const int row = pass * RPP + lane / C8;
     const int q_row = q_begin + wave * 32 + row;
     const vec_t v = *reinterpret_cast<const vec_t*>(tile + row * OROW + c8 * 16);
-    if (q_row < q_store_end) *reinterpret_cast<vec_t*>(ob + q_row * p.os[2] + c8 * 8) = v;
+    if (q_row < q_store_end)
+      *reinterpret_cast<vec_t*>(reinterpret_cast<uint8_t*>(ob) +
+                                (__umul24(static_cast<uint32_t>(q_row), static_cast<uint32_t>(p.os[2]) * 2u) + c8 * 16u)) = v;
   }
   };
   block(qc_a, std::false_type{});
@@ -1314,7 +1323,7 @@ __global__ __launch_bounds__(kSparseWaves * kWave) void flash_attn_fwd_sparse_ke
 
   // ---- finalise: O / l, transpose through the wavefront's LDS tile, self rows, 16-byte stores -------------------------
   const float l_run = pair_sum(l_lane);
-  const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+  const float inv = l_run > 0.f ? __builtin_amdgcn_rcpf(l_run) : 0.f;  // 1 ulp; the products are rounded to 16 bits
   const float fin = (qi < q_valid) ? inv : 0.f;
   uint8_t* tile = smem;
 #pragma unroll
@@ -1345,9 +1354,13 @@ void launch(const AttnParams& p, bool causal, bool register_staging, hipStream_t
   // TAAC_ATTN_REGISTER_STAGING keeps the general kernel for full head dims too (comparison route of the caller).
   const bool dma_staging = !register_staging;
   // 32-bit source offsets with a 24-bit row multiply: row strides below 8 M elements, sequences below 2^31 bytes
+  // (the same for the query and output rows)
   const bool small_offsets = p.ks[2] < (1 << 22) && p.vs[2] < (1 << 22) && p.Tk < (1 << 22) &&
                              static_cast<int64_t>(p.Tk) * p.ks[2] * 2 < (1ll << 31) &&
-                             static_cast<int64_t>(p.Tk) * p.vs[2] * 2 < (1ll << 31);
+                             static_cast<int64_t>(p.Tk) * p.vs[2] * 2 < (1ll << 31) &&
+                             p.qs[2] >= 0 && p.os[2] >= 0 && p.qs[2] < (1 << 22) && p.os[2] < (1 << 22) && p.Tq < (1 << 22) &&
+                             static_cast<int64_t>(p.Tq) * p.qs[2] * 2 < (1ll << 31) &&
+                             static_cast<int64_t>(p.Tq) * p.os[2] * 2 < (1ll << 31);
   if constexpr (DP == 32 || DP == 64) {
     if (p.compact_keys != nullptr) {  // the entry point has checked the shape
       const int64_t groups = static_cast<int64_t>((p.Tq + 31) / 32) * ((static_cast<int64_t>(p.B) * p.H + kSparseWaves - 1) / kSparseWaves);
