@@ -834,19 +834,24 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
               const u32x4 bias_bits = {b0row[rb], 0u, 0u, 0u};
               acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, bias_bits), ones, acc, 0, 0, 0);
 #pragma unroll
-              for (int j = 0; j < 16; j += 2) {
+              for (int j = 0; j < 16; j += 2) {  // one packed conversion per pair, widened back from the packed word
                 const bf16x2 pair = {static_cast<bf16_t>(acc[j]), static_cast<bf16_t>(acc[j + 1])};
-                acc[j] = static_cast<float>(pair[0]);
-                acc[j + 1] = static_cast<float>(pair[1]);
+                uint32_t bits = __builtin_bit_cast(uint32_t, pair);
+                asm("" : "+v"(bits));  // opaque: the optimiser otherwise splits the pair into two conversions again
+                acc[j] = __builtin_bit_cast(float, bits << 16);
+                acc[j + 1] = __builtin_bit_cast(float, bits & 0xffff0000u);
               }
               acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ident[0], hf[t][2 * rb], acc, 0, 0, 0);
               acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ident[1], hf[t][2 * rb + 1], acc, 0, 0, 0);
 #pragma unroll
               for (int j = 0; j < 16; j += 2) {
                 const bf16x2 pair = {static_cast<bf16_t>(acc[j]), static_cast<bf16_t>(acc[j + 1])};
-                acc[j] = static_cast<float>(pair[0]);
-                acc[j + 1] = static_cast<float>(pair[1]);
-                ss[t] = __builtin_amdgcn_fdot2_f32_bf16(pair, pair, ss[t], false);
+                uint32_t bits = __builtin_bit_cast(uint32_t, pair);
+                asm("" : "+v"(bits));  // opaque: the optimiser otherwise splits the pair into two conversions again
+                acc[j] = __builtin_bit_cast(float, bits << 16);
+                acc[j + 1] = __builtin_bit_cast(float, bits & 0xffff0000u);
+                const bf16x2 rounded = __builtin_bit_cast(bf16x2, bits);
+                ss[t] = __builtin_amdgcn_fdot2_f32_bf16(rounded, rounded, ss[t], false);
               }
             }
         }
