@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define TAAC_ABI_VERSION 8
+#define TAAC_ABI_VERSION 9
 
 enum taac_status {
   TAAC_OK = 0,
@@ -407,8 +407,12 @@ int taac_swiglu_ffn_bwd_hidden(const void* h, int64_t ldh, const void* dy, int64
  * rows / n_rows: both NULL (every row 0..M-1 is a token), or a row index as written by taac_valid_rows: the tokens are
  * rows[0 .. *n_rows) of x / residual / out (*n_rows <= M, read on the device), all other rows are neither read nor
  * written - this is how the layers skip the padded positions of a padded [B, T, D] batch.
- * norm_folded != 0 (needs norm_weight and packed_weights): the blob is that of taac_ffn_pack_weights_norm, i.e. the norm's
- * weight is already part of the up projection, and the kernel multiplies the rows by rsqrt(mean(x^2) + eps) only.
+ * norm_folded: 0, or what the packed blob already holds - TAAC_FOLDED_NORM (needs norm_weight and packed_weights; 1, as
+ * before the second flag existed): the blob is that of taac_ffn_pack_weights_norm / _folded, i.e. the norm's weight is
+ * already part of the up projection, and the kernel multiplies the rows by rsqrt(mean(x^2) + eps) only;
+ * TAAC_FOLDED_ACTIVATION (taac_swiglu_ffn_fwd, taac_attn_out_ffn_fwd and taac_attn_out_ffn_heads_fwd on packed weights):
+ * the blob is that of taac_ffn_pack_weights_folded with fold_activation, whose up projection carries the constants of
+ * silu(g) * u (see there).
  * Replaces: ffn_norm + SwiGLUFeedForward.forward + residual add of UnifiedInteractionBlock.forward
  * (experiments/symbiosis/backbone.py:19-21, 66-67).
  */
@@ -701,6 +705,18 @@ int taac_ffn_pack_weights(const void* w_up, const void* w_down, void* packed, in
  * (w_up[n, k] * norm_weight[k], rounded once), for the feed-forward entry points with norm_folded = 1. */
 int taac_ffn_pack_weights_norm(const void* w_up, const void* w_down, const void* norm_weight, void* packed, int32_t D,
                                int32_t F, int gate_first, void* stream);
+/* The same blob (norm_weight: NULL, or folded as above) which, with fold_activation != 0, also carries the constants of
+ * the gate's activation: the gated half of the up projection is multiplied by -log2(e) and the other half by -ln(2)
+ * inside the same single rounding of each weight, so that silu(g) * u = g' * u' / (1 + 2^g') with g', u' as the matrix
+ * unit delivers them - one multiplication less per hidden unit and token in the kernels, which are then called with
+ * TAAC_FOLDED_ACTIVATION in norm_folded (they scale b_up the same way when they stage it).
+ * taac_ffn_activation_fold_supported: 1 where the kernels take such a blob (D 128 / 256, F a multiple of 32 that leaves
+ * room for three weight buffers), else 0. No counterpart in the reference. */
+#define TAAC_FOLDED_NORM 1
+#define TAAC_FOLDED_ACTIVATION 2
+int taac_ffn_activation_fold_supported(int32_t D, int32_t F);
+int taac_ffn_pack_weights_folded(const void* w_up, const void* w_down, const void* norm_weight, void* packed, int32_t D,
+                                 int32_t F, int gate_first, int fold_activation, void* stream);
 int64_t taac_linear_packed_bytes(int32_t N, int32_t K);
 int taac_linear_pack_weights(const void* w, void* packed, int32_t N, int32_t K, void* stream);
 /* The same blob with the weight of an RMSNorm in front of the layer folded in (packed[n, k] = bf16(w[n, k] *

@@ -23,8 +23,9 @@ TAAC_F32, TAAC_BF16, TAAC_F16 = 0, 1, 2
 EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
 ATTN_CAUSAL, ATTN_REGISTER_STAGING = 1, 2
 BACKBONE_DENSE_TOKENS, BACKBONE_SPLIT_OUT_FFN, BACKBONE_FP8, BACKBONE_ROW_MAJOR_QKV = 1, 2, 4, 8
+FOLDED_NORM, FOLDED_ACTIVATION = 1, 2
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _DTYPE_CODES = {torch.float32: TAAC_F32, torch.bfloat16: TAAC_BF16, torch.float16: TAAC_F16}
 
@@ -237,6 +238,8 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "taac_ffn_packed_bytes": (c_int64, [c_int32, c_int32]),
     "taac_ffn_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int, c_void_p]),
     "taac_ffn_pack_weights_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int, c_void_p]),
+    "taac_ffn_activation_fold_supported": (c_int, [c_int32, c_int32]),
+    "taac_ffn_pack_weights_folded": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int, c_int, c_void_p]),
     "taac_linear_packed_bytes": (c_int64, [c_int32, c_int32]),
     "taac_linear_pack_weights": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
     "taac_linear_pack_weights_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),

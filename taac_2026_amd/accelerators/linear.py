@@ -426,13 +426,21 @@ def clear_packed_weight_cache() -> None:
     _packed_cache.clear()
 
 
+def ffn_activation_fold_supported(d_model: int, hidden_size: int) -> bool:
+    """Whether the fused feed-forward kernels take the constants of ``silu(g) * u`` from the packed up projection at
+    this shape (``pack_ffn_weights(fold_activation=True)``)."""
+    return bool(_native.load_library().taac_ffn_activation_fold_supported(int(d_model), int(hidden_size)))
+
+
 def pack_ffn_weights(up_weight: torch.Tensor, down_weight: torch.Tensor, *, gate_first: bool = True,
-                     norm_weight: torch.Tensor | None = None) -> torch.Tensor:
+                     norm_weight: torch.Tensor | None = None, fold_activation: bool = False) -> torch.Tensor:
     """Fragment-ordered blob of ``(up_weight [2F, D], down_weight [D, F])`` for ``swiglu_ffn`` (uint8 tensor).
 
     The blob depends on ``gate_first`` (which half of ``up_weight`` goes through SiLU): pass the same value to
     ``swiglu_ffn``. ``norm_weight`` ``[D]``: the weight of the RMSNorm in front of the up projection, folded into the
-    blob (``taac_ffn_pack_weights_norm``; the kernels are then called with ``norm_folded = 1``)."""
+    blob (``taac_ffn_pack_weights_norm``; the kernels are then called with ``TAAC_FOLDED_NORM``). ``fold_activation``:
+    the up projection also carries the constants of the gate's activation (``taac_ffn_pack_weights_folded``; the
+    kernels are then called with ``TAAC_FOLDED_ACTIVATION``)."""
     library = _native.load_library()
     d_model, hidden = down_weight.shape
     nbytes = library.taac_ffn_packed_bytes(d_model, hidden)
@@ -440,9 +448,14 @@ def pack_ffn_weights(up_weight: torch.Tensor, down_weight: torch.Tensor, *, gate
         raise RuntimeError(f"pack_ffn_weights: unsupported shape D={d_model}, F={hidden}")
     up_weight, down_weight = up_weight.contiguous(), down_weight.contiguous()
     packed = torch.empty(nbytes, dtype=torch.uint8, device=up_weight.device)
-    if norm_weight is not None:
-        if norm_weight.shape != (d_model,):
-            raise ValueError("rms_norm weight must be 1D and match the normalized dimension")
+    if norm_weight is not None and norm_weight.shape != (d_model,):
+        raise ValueError("rms_norm weight must be 1D and match the normalized dimension")
+    if fold_activation:
+        norm = norm_weight.contiguous() if norm_weight is not None else None
+        status = library.taac_ffn_pack_weights_folded(up_weight.data_ptr(), down_weight.data_ptr(), _native.ptr(norm),
+                                                      packed.data_ptr(), d_model, hidden, int(bool(gate_first)), 1,
+                                                      _native.current_stream(up_weight.device))
+    elif norm_weight is not None:
         status = library.taac_ffn_pack_weights_norm(up_weight.data_ptr(), down_weight.data_ptr(),
                                                     norm_weight.contiguous().data_ptr(), packed.data_ptr(), d_model, hidden,
                                                     int(bool(gate_first)), _native.current_stream(up_weight.device))
@@ -454,15 +467,32 @@ def pack_ffn_weights(up_weight: torch.Tensor, down_weight: torch.Tensor, *, gate
     return packed
 
 
-def _packed_ffn(up_weight: torch.Tensor, down_weight: torch.Tensor, gate_first: bool, norm_weight: torch.Tensor | None):
-    """Cached feed-forward blob, with the weight of the norm in front of it folded in when there is one."""
+def _packed_ffn(up_weight: torch.Tensor, down_weight: torch.Tensor, gate_first: bool, norm_weight: torch.Tensor | None,
+                fold_activation: bool = False):
+    """Cached feed-forward blob, with the weight of the norm in front of it folded in when there is one (and, with
+    ``fold_activation``, the constants of the gate's activation)."""
+    variant = int(bool(gate_first)) + (8 if fold_activation else 0)
     if norm_weight is None:
         return _packed_cache.get((up_weight, down_weight),
-                                 lambda: pack_ffn_weights(up_weight, down_weight, gate_first=gate_first),
-                                 variant=int(bool(gate_first)))
+                                 lambda: pack_ffn_weights(up_weight, down_weight, gate_first=gate_first,
+                                                          fold_activation=fold_activation),
+                                 variant=variant)
     return _packed_cache.get((up_weight, down_weight, norm_weight),
-                             lambda: pack_ffn_weights(up_weight, down_weight, gate_first=gate_first, norm_weight=norm_weight),
-                             variant=4 + int(bool(gate_first)))
+                             lambda: pack_ffn_weights(up_weight, down_weight, gate_first=gate_first, norm_weight=norm_weight,
+                                                      fold_activation=fold_activation),
+                             variant=4 + variant)
+
+
+def _fold_choice(name: str, fold_activation: bool | None, d_model: int, hidden: int) -> bool:
+    """``fold_activation`` of the fused feed-forward wrappers: None takes the folded blob wherever the kernels accept it."""
+    supported = ffn_activation_fold_supported(d_model, hidden)
+    if fold_activation and not supported:
+        raise RuntimeError(f"{name}: the kernels do not take the activation's constants from the blob at D={d_model}, F={hidden}")
+    return supported if fold_activation is None else bool(fold_activation)
+
+
+def _folded_flags(norm_weight: torch.Tensor | None, fold_activation: bool) -> int:
+    return (_native.FOLDED_NORM if norm_weight is not None else 0) | (_native.FOLDED_ACTIVATION if fold_activation else 0)
 
 
 def pack_linear_weight(weight: torch.Tensor, norm_weight: torch.Tensor | None = None) -> torch.Tensor:
@@ -598,8 +628,12 @@ def swiglu_ffn(
     eps: float = 1e-6,
     token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
     out: torch.Tensor | None = None,
+    fold_activation: bool | None = None,
 ) -> torch.Tensor:
     """``residual + down(silu(gate) * value)`` with ``gate, value = up(rmsnorm(x)).chunk(2, -1)``.
+
+    ``fold_activation``: whether the packed up projection carries the constants of the gate's activation (one multiplication less per
+    hidden unit in the kernel; each weight is still rounded once); None takes that form wherever the kernels accept it.
 
     ``norm_weight`` (optional) fuses the pre-FFN RMSNorm; ``residual`` (optional) the residual add. For model widths
     128 / 256 with a hidden size that is a multiple of 32 the whole expression is ONE kernel
@@ -639,7 +673,8 @@ def swiglu_ffn(
         gated = swiglu_linear(h, up_weight, up_bias, gate_first=gate_first)
         res_rows = residual.reshape(-1, d_model) if residual is not None else None
         return linear(gated, down_weight, down_bias, residual=res_rows).reshape(shape)
-    packed = _packed_ffn(up_weight, down_weight, gate_first, norm_weight)
+    fold = _fold_choice(name, fold_activation, d_model, hidden)
+    packed = _packed_ffn(up_weight, down_weight, gate_first, norm_weight, fold)
     res_rows = None
     if residual is not None:
         res_rows = residual.reshape(-1, d_model)
@@ -652,7 +687,7 @@ def swiglu_ffn(
         rows.data_ptr(), rows.stride(0), _native.ptr(norm_weight), float(eps), None,
         _native.ptr(up_bias), None, _native.ptr(down_bias), packed.data_ptr(), _native.ptr(res_rows),
         res_rows.stride(0) if res_rows is not None else d_model, out.data_ptr(), d_model, rows.shape[0], d_model,
-        hidden, int(bool(gate_first)), _native.ptr(index), _native.ptr(count), int(norm_weight is not None),
+        hidden, int(bool(gate_first)), _native.ptr(index), _native.ptr(count), _folded_flags(norm_weight, fold),
         _native.current_stream(x.device),
     )
     _native.check(status, "swiglu_ffn")
@@ -747,6 +782,7 @@ def attention_out_ffn(
     input_rows: torch.Tensor | None = None,
     out: torch.Tensor | None = None,
     update_gate: torch.Tensor | None = None,
+    fold_activation: bool | None = None,
 ) -> torch.Tensor:
     """Second half of a ``UnifiedInteractionBlock`` (experiments/symbiosis/backbone.py:47, 64-67) as ONE kernel:
     ``x1 = residual + F.linear(attn, out_weight, out_bias)`` then ``x1 + down(silu(gate) * value)`` with
@@ -757,7 +793,8 @@ def attention_out_ffn(
 
     ``update_gate`` (shape of ``residual``): the second half of a ``TokenFormerBlock`` (experiments/tokenformer/
     model.py:209-214) instead - ``x1 = residual + sigmoid(update_gate) * F.linear(attn, out_weight, out_bias)``, with
-    ``update_gate`` the output of the block's ``nlir_gate`` layer before the sigmoid (``taac_attn_out_gate_ffn_fwd``)."""
+    ``update_gate`` the output of the block's ``nlir_gate`` layer before the sigmoid (``taac_attn_out_gate_ffn_fwd``).
+    ``fold_activation`` as in :func:`swiglu_ffn` (the kernel with an update gate takes the plain blob)."""
     name = "hip attention_out_ffn"
     tensors = (attn, out_weight, out_bias, residual, up_weight, up_bias, down_weight, down_bias, norm_weight, update_gate)
     require_cuda_tensors(name, *tensors)
@@ -774,7 +811,10 @@ def attention_out_ffn(
     if not (_fused_width(d_model) and hidden % 32 == 0):
         raise RuntimeError("attention_out_ffn: needs model width 128 / 256 and a hidden size that is a multiple of 32")
     packed_out = _packed_cache.get((out_weight,), lambda: pack_linear_weight(out_weight))
-    packed_ffn = _packed_ffn(up_weight, down_weight, True, norm_weight)
+    if update_gate is not None and fold_activation:
+        raise RuntimeError("attention_out_ffn: the kernel with an update gate takes the plain blob (fold_activation=False)")
+    fold = update_gate is None and _fold_choice("attention_out_ffn", fold_activation, d_model, hidden)
+    packed_ffn = _packed_ffn(up_weight, down_weight, True, norm_weight, fold)
     res_rows = residual.reshape(-1, d_model)
     if res_rows.stride(-1) != 1 or res_rows.stride(0) % 8 != 0:
         res_rows = res_rows.contiguous()
@@ -801,7 +841,7 @@ def attention_out_ffn(
         rows.data_ptr(), rows.stride(0), _native.ptr(out_bias), packed_out.data_ptr(), res_rows.data_ptr(),
         res_rows.stride(0), _native.ptr(norm_weight), float(eps), _native.ptr(up_bias), _native.ptr(down_bias),
         packed_ffn.data_ptr(), out.data_ptr(), d_model, rows.shape[0], d_model, hidden, _native.ptr(index),
-        _native.ptr(count), _native.ptr(_input_rows(name, input_rows, index, rows)), int(norm_weight is not None),
+        _native.ptr(count), _native.ptr(_input_rows(name, input_rows, index, rows)), _folded_flags(norm_weight, fold),
         _native.current_stream(attn.device),
     )
     _native.check(status, "attention_out_ffn")
@@ -925,10 +965,12 @@ def attention_out_ffn_heads(
     eps: float = 1e-6,
     token_rows: tuple[torch.Tensor, torch.Tensor] | None = None,
     out: torch.Tensor | None = None,
+    fold_activation: bool | None = None,
 ) -> torch.Tensor:
     """:func:`attention_out_ffn` whose attention output is a contiguous stack of per-head planes ``[H, rows, head_dim]``
     (``taac_attn_out_ffn_heads_fwd``; the layout :func:`flash_attention` leaves behind for queries taken from
-    :func:`norm_linear_heads`). ``residual`` / ``out`` are ``[.., D]`` rows as usual. Same values, bit for bit."""
+    :func:`norm_linear_heads`). ``residual`` / ``out`` are ``[.., D]`` rows as usual. Same values, bit for bit (for the
+    same ``fold_activation``)."""
     name = "hip attention_out_ffn_heads"
     tensors = (attn, out_weight, out_bias, residual, up_weight, up_bias, down_weight, down_bias, norm_weight)
     require_cuda_tensors(name, *tensors)
@@ -946,7 +988,8 @@ def attention_out_ffn_heads(
     if not (_fused_width(d_model) and hidden % 32 == 0):
         raise RuntimeError(f"{name}: needs model width 128 / 256 and a hidden size that is a multiple of 32")
     packed_out = _packed_cache.get((out_weight,), lambda: pack_linear_weight(out_weight))
-    packed_ffn = _packed_ffn(up_weight, down_weight, True, norm_weight)
+    fold = _fold_choice(name, fold_activation, d_model, hidden)
+    packed_ffn = _packed_ffn(up_weight, down_weight, True, norm_weight, fold)
     if res_rows.stride(-1) != 1 or res_rows.stride(0) % 8 != 0:
         res_rows = res_rows.contiguous()
     index, count = _token_rows(name, token_rows, res_rows)
@@ -956,7 +999,7 @@ def attention_out_ffn_heads(
         attn.data_ptr(), int(head_dim), _native.ptr(out_bias), packed_out.data_ptr(), res_rows.data_ptr(), res_rows.stride(0),
         _native.ptr(norm_weight), float(eps), _native.ptr(up_bias), _native.ptr(down_bias), packed_ffn.data_ptr(),
         out.data_ptr(), d_model, row_count, d_model, hidden, _native.ptr(index), _native.ptr(count),
-        int(norm_weight is not None), _native.current_stream(attn.device))
+        _folded_flags(norm_weight, fold), _native.current_stream(attn.device))
     _native.check(status, "attention_out_ffn_heads")
     return out.reshape(shape)
 

@@ -524,6 +524,8 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
   bf16_t* g = reinterpret_cast<bf16_t*>(ws);  // unfused path: gated hidden state; fused path: packed weights
   char* packed = ws;
   const bool fused = fused_shape(D, F);
+  // the packed up projection carries the constants of the gate's activation where the kernels take them from there
+  const bool fold_act = fused && ffn_act_fold_supported(D, F);
   // Fused path: the dense layers walk the valid tokens only (row index built from key_lengths on the device); the
   // padded positions of the residual stream are never read or written. TAAC_BACKBONE_DENSE_TOKENS switches this off.
   int32_t* rows = nullptr;
@@ -562,7 +564,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
       pk[2 * n_blocks + i] = base + align256(static_cast<int64_t>(3) * D * D * 2) + align256(static_cast<int64_t>(D) * D * 2);
     }
     if ((rc = pack_backbone_blocks(blocks, n_blocks, D, F, pk.data(), pk.data() + n_blocks, pk.data() + 2 * n_blocks,
-                                   as_stream(stream), name)) != TAAC_OK)
+                                   fold_act, as_stream(stream), name)) != TAAC_OK)
       return rc;
   }
   // FP8 mode: scales and e4m3 weights of all blocks (three launches), then the scale of the first block's input
@@ -639,6 +641,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
     char* pk_qkv = packed + static_cast<int64_t>(i) * packed_block_bytes(D, F);
     char* pk_out = pk_qkv + align256(static_cast<int64_t>(3) * D * D * 2);
     char* pk_ffn = pk_out + align256(static_cast<int64_t>(D) * D * 2);
+    const int ffn_folded = (w.ffn_norm_weight != nullptr ? TAAC_FOLDED_NORM : 0) | (fold_act ? TAAC_FOLDED_ACTIVATION : 0);
     // attention half
     if ((w.query_norm_weight == nullptr) != (w.key_norm_weight == nullptr))
       return set_error(TAAC_ERR_INVALID_VALUE, "%s: block %d: query and key norm weights come together", name, i);
@@ -710,7 +713,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
                                            plane_strides, plane_strides, 0, rows ? 2 : 1, TAAC_BF16, stream)) != TAAC_OK)
         return rc;
       if ((rc = attn_out_ffn_readout(h, D, dh, w.out_bias, pk_out, cur, D, w.ffn_norm_weight, eps, w.up_bias, w.down_bias,
-                                     pk_ffn, x_out, D, M, D, F, rows, n_rows, w.ffn_norm_weight != nullptr,
+                                     pk_ffn, x_out, D, M, D, F, rows, n_rows, ffn_folded,
                                      ride ? w_head : nullptr, ride ? token_dots : nullptr, stream)) != TAAC_OK)
         return rc;
       dots_ready = ride;
@@ -724,7 +727,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
     if (fused && !split_out_ffn) {
       // out projection + residual and the whole feed-forward half in one kernel; the stream between them stays on chip
       if ((rc = attn_out_ffn_readout(h, D, 0, w.out_bias, pk_out, cur, D, w.ffn_norm_weight, eps, w.up_bias, w.down_bias,
-                                     pk_ffn, x_out, D, M, D, F, rows, n_rows, w.ffn_norm_weight != nullptr,
+                                     pk_ffn, x_out, D, M, D, F, rows, n_rows, ffn_folded,
                                      ride ? w_head : nullptr, ride ? token_dots : nullptr, stream)) != TAAC_OK)
         return rc;
       dots_ready = ride;
@@ -734,7 +737,7 @@ extern "C" int taac_backbone_fwd(const void* emb, const int32_t* key_lengths, co
         return rc;
       // feed-forward half: RMSNorm -> up -> SiLU-gate -> down -> + residual in one kernel
       if ((rc = taac_swiglu_ffn_fwd(x, D, w.ffn_norm_weight, eps, nullptr, w.up_bias, nullptr, w.down_bias, pk_ffn, x,
-                                    D, x_out, D, M, D, F, 1, rows, n_rows, w.ffn_norm_weight != nullptr, stream)) != TAAC_OK)
+                                    D, x_out, D, M, D, F, 1, rows, n_rows, ffn_folded, stream)) != TAAC_OK)
         return rc;
     } else {
       if ((rc = taac_linear_bf16(h, D, w.out_weight, w.out_bias, cur, x, D, M, D, D, TAAC_EPI_RESIDUAL, 1, stream)) !=

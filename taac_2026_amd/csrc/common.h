@@ -34,8 +34,11 @@ int compute_units();
 int test_max_workgroups();
 bool test_fp8_tiled();
 // Packs the qkv / out / feed-forward weights (gate first) of n backbone blocks into fragment order (ffn.hip).
+// fold_act: the up projection also takes the constants of the gate's activation (the kernels are then called with
+// TAAC_FOLDED_ACTIVATION; allowed where ffn_act_fold_supported says so).
 int pack_backbone_blocks(const taac_block_weights* blocks, int n, int32_t D, int32_t F, void* const* packed_qkv,
-                         void* const* packed_out, void* const* packed_ffn, hipStream_t s, const char* name);
+                         void* const* packed_out, void* const* packed_ffn, bool fold_act, hipStream_t s, const char* name);
+bool ffn_act_fold_supported(int32_t D, int32_t F);
 // RMSNorm + q | k | v projection with the query / key epilogue (ffn.hip; the arguments of taac_norm_linear_qk_fwd with
 // packed weights) whose output is a stack of per-head planes [3 * num_heads][M][head_dim], head_dim 32 or 64.
 int norm_linear_qk_heads(const void* x, int64_t ldx, const void* norm_weight, float eps, const void* bias,

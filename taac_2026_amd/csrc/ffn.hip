@@ -95,9 +95,13 @@ __host__ __device__ __forceinline__ int up_unit_of_slot(int m16) {
 // (row block r - KS); exactly the image one barrier step needs in LDS. A fragment is 64 lanes x 16 bytes.
 // col_scale (optional, [D]): weight of the RMSNorm in front of the up projection, folded into its fragments (see
 // linear_pack_piece).
+// fold_act: the constants of the gate's activation join the same rounding - the gated half is multiplied by -log2(e), the
+// other half by -ln 2, so that silu(g) * u = g' * u' / (1 + 2^g') with g' and u' as they leave the matrix unit (the
+// kernel's FOLD form: one multiplication less per hidden unit and token; the first-layer bias is scaled when it is staged).
+constexpr float kFoldGate = -1.4426950408889634f, kFoldValue = -0.6931471805599453f;
 __device__ __forceinline__ void ffn_pack_piece(const bf16_t* __restrict__ w_up, const bf16_t* __restrict__ w_down,
                                                bf16x8* __restrict__ packed, int D, int F, int gate_first, int64_t gid,
-                                               const bf16_t* __restrict__ col_scale = nullptr) {
+                                               const bf16_t* __restrict__ col_scale = nullptr, bool fold_act = false) {
   const int KS = D / 16, MB = D / 32, CFRAG = KS + MB, NFRAG = kCPB * CFRAG;
   const int lane = static_cast<int>(gid % 64);
   const int f = static_cast<int>((gid / 64) % NFRAG);
@@ -111,20 +115,27 @@ __device__ __forceinline__ void ffn_pack_piece(const bf16_t* __restrict__ w_up, 
   else
     src = w_down + static_cast<int64_t>((r - KS) * 32 + l32) * F + unit0 + hh * 8;
   bf16x8 v = *reinterpret_cast<const bf16x8*>(src);
-  if (col_scale != nullptr && r < KS) {
-    const bf16x8 g = *reinterpret_cast<const bf16x8*>(col_scale + r * 16 + hh * 8);
+  if ((col_scale != nullptr || fold_act) && r < KS) {
+    bf16x8 g;
+    if (col_scale != nullptr) {
+      g = *reinterpret_cast<const bf16x8*>(col_scale + r * 16 + hh * 8);
+    } else {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = static_cast<bf16_t>(static_cast<float>(v[e]) * static_cast<float>(g[e]));
+      for (int e = 0; e < 8; ++e) g[e] = static_cast<bf16_t>(1.0f);
+    }
+    const float c = fold_act ? (l32 < 16 ? kFoldGate : kFoldValue) : 1.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = static_cast<bf16_t>(static_cast<float>(v[e]) * static_cast<float>(g[e]) * c);
   }
   packed[gid] = v;
 }
 
 __global__ void ffn_pack_kernel(const bf16_t* __restrict__ w_up, const bf16_t* __restrict__ w_down,
                                 bf16x8* __restrict__ packed, int D, int F, int gate_first,
-                                const bf16_t* __restrict__ col_scale) {
+                                const bf16_t* __restrict__ col_scale, bool fold_act) {
   const int64_t total = static_cast<int64_t>(3) * D * F / 8;
   const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (gid < total) ffn_pack_piece(w_up, w_down, packed, D, F, gate_first, gid, col_scale);
+  if (gid < total) ffn_pack_piece(w_up, w_down, packed, D, F, gate_first, gid, col_scale, fold_act);
 }
 
 // Plain SiLU MLP blob (fc1 [F, D], fc2 [D, F]): chunk c (32 hidden units) holds KS fc1 fragments (k-step r; row slots
@@ -190,7 +201,7 @@ struct PackBatch {
   bf16x8* packed_out[kPackBatch];
   bf16x8* packed_ffn[kPackBatch];
 };
-__global__ void pack_blocks_kernel(const PackBatch batch, int D, int F) {
+__global__ void pack_blocks_kernel(const PackBatch batch, int D, int F, bool fold_act) {
   const int blk = blockIdx.y;
   const int64_t n_qkv = static_cast<int64_t>(3) * D * D / 8, n_out = static_cast<int64_t>(D) * D / 8;
   const int64_t n_ffn = static_cast<int64_t>(3) * D * F / 8;
@@ -199,7 +210,8 @@ __global__ void pack_blocks_kernel(const PackBatch batch, int D, int F) {
   gid -= n_qkv;
   if (gid < n_out) return linear_pack_piece(batch.out[blk], batch.packed_out[blk], D, gid);
   gid -= n_out;
-  if (gid < n_ffn) ffn_pack_piece(batch.up[blk], batch.down[blk], batch.packed_ffn[blk], D, F, 1, gid, batch.ffn_norm[blk]);
+  if (gid < n_ffn)
+    ffn_pack_piece(batch.up[blk], batch.down[blk], batch.packed_ffn[blk], D, F, 1, gid, batch.ffn_norm[blk], fold_act);
 }
 
 // ---- shared pieces ---------------------------------------------------------------------------------------------------
@@ -502,9 +514,10 @@ __device__ __forceinline__ void load_residual(const bf16_t* residual, int64_t ld
 // it arrives as a tensor). Its pieces of a chunk are requested behind the chunk's MFMAs, into the registers the weight
 // fragments have left, so the variant takes no registers of its own.
 // ------------------------------------------------------------------------------------------------------------------
-template <int D, int TT, int NWAVES, int CPB, bool DEFER, bool OUTP, bool GATE = false, bool GLU = true>
+template <int D, int TT, int NWAVES, int CPB, bool DEFER, bool OUTP, bool GATE = false, bool GLU = true, bool FOLD = false>
 __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_kernel(const TsParams p) {
   static_assert(!GATE || OUTP, "the gate belongs to the projection in front");
+  static_assert(!FOLD || GLU, "the folded constants belong to the gated form");
   constexpr int kTokPerWg = NWAVES * 32 * TT;  // TT token tiles of 32 per wavefront
   constexpr int KS = D / 16;             // k-steps of the up projection = up fragments per chunk
   constexpr int MB = D / 32;             // 32-feature row blocks of the down projection
@@ -635,6 +648,8 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
     for (int u = 0; u < UB; ++u) {
       const int i = tid + u * kThreadsWg;
       up_bias_regs[u] = p.b1[up_bias_src(i < UPB ? i : UPB - 1)];
+      if constexpr (FOLD)  // the packed layer's constants (see ffn_pack_piece), one more rounding of the bias
+        up_bias_regs[u] = static_cast<bf16_t>(static_cast<float>(up_bias_regs[u]) * (i % 32 < 16 ? kFoldGate : kFoldValue));
     }
   }
   const int vec_at = tid * 8 < D ? tid * 8 : D - 8;  // the D-wide vectors: 16 bytes per thread, the first D / 8 threads store
@@ -664,8 +679,11 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
     const int i = tid + u * kThreadsWg;
     if (i < UPB) bias_lds[i] = up_bias_regs[u];
   }
-  for (int i = tid + UB * kThreadsWg; i < UPB; i += kThreadsWg)  // wider hidden layers: the rest, one entry at a time
-    bias_lds[i] = p.b1 != nullptr ? p.b1[up_bias_src(i)] : static_cast<bf16_t>(0.f);
+  for (int i = tid + UB * kThreadsWg; i < UPB; i += kThreadsWg) {  // wider hidden layers: the rest, one entry at a time
+    bf16_t b = p.b1 != nullptr ? p.b1[up_bias_src(i)] : static_cast<bf16_t>(0.f);
+    if constexpr (FOLD) b = static_cast<bf16_t>(static_cast<float>(b) * (i % 32 < 16 ? kFoldGate : kFoldValue));
+    bias_lds[i] = b;
+  }
   if (tid * 8 < D) {
     *reinterpret_cast<bf16x8*>(bias_lds + UPB + vec_at) = b2_regs;
     if (p.norm_w != nullptr) *reinterpret_cast<bf16x8*>(bias_lds + UPB + D + vec_at) = normw_regs;
@@ -918,6 +936,8 @@ __global__ __launch_bounds__(NWAVES * kWave, TT == 1 ? 2 : 1) void swiglu_ffn_ke
       for (int e = 0; e < 8; ++e) hb[t][k][e] = static_cast<bf16_t>(0.f);
   // Activation of accumulator register e of a chunk (e < 8 * DK): the B-operand element it becomes.
   auto activate = [](const f32x16& gu, int e) -> bf16_t {
+    if constexpr (FOLD)  // gu[e] = -log2(e) g, gu[8 + e] = -ln(2) u: their product is g u
+      return static_cast<bf16_t>(gu[e] * gu[8 + e] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(gu[e])));
     return static_cast<bf16_t>(GLU ? silu_f(gu[e]) * gu[8 + e] : silu_f(gu[e]));
   };
   int buf = 0;
@@ -1508,7 +1528,7 @@ constexpr int kMaxLdsBytes = 160 * 1024;
 namespace taac {
 // Packs the qkv / out / feed-forward weights (gate first) of n backbone blocks with as few launches as possible.
 int pack_backbone_blocks(const taac_block_weights* blocks, int n, int32_t D, int32_t F, void* const* packed_qkv,
-                         void* const* packed_out, void* const* packed_ffn, hipStream_t s, const char* name) {
+                         void* const* packed_out, void* const* packed_ffn, bool fold_act, hipStream_t s, const char* name) {
   for (int base = 0; base < n; base += kPackBatch) {
     PackBatch batch{};
     const int m = n - base < kPackBatch ? n - base : kPackBatch;
@@ -1529,7 +1549,7 @@ int pack_backbone_blocks(const taac_block_weights* blocks, int n, int32_t D, int
     }
     const int64_t pieces = (static_cast<int64_t>(4) * D * D + static_cast<int64_t>(3) * D * F) / 8;
     hipLaunchKernelGGL(pack_blocks_kernel, dim3(static_cast<uint32_t>((pieces + 255) / 256), m), dim3(256), 0, s, batch,
-                       D, F);
+                       D, F, fold_act);
     const int rc = check_launch(name);
     if (rc != TAAC_OK) return rc;
   }
@@ -1545,9 +1565,20 @@ extern "C" int64_t taac_ffn_packed_bytes(int32_t D, int32_t F) {
 namespace taac {
 namespace {
 int ffn_pack(const char* name, const void* w_up, const void* w_down, const void* norm_weight, void* packed, int32_t D,
-             int32_t F, int gate_first, void* stream);
+             int32_t F, int gate_first, void* stream, bool fold_act = false);
 }
 }  // namespace taac
+
+extern "C" int taac_ffn_activation_fold_supported(int32_t D, int32_t F) { return taac::ffn_act_fold_supported(D, F) ? 1 : 0; }
+
+extern "C" int taac_ffn_pack_weights_folded(const void* w_up, const void* w_down, const void* norm_weight, void* packed,
+                                            int32_t D, int32_t F, int gate_first, int fold_activation, void* stream) {
+  const char* name = "taac_ffn_pack_weights_folded";
+  if (fold_activation && !taac::ffn_act_fold_supported(D, F))
+    return taac::set_error(TAAC_ERR_UNSUPPORTED, "%s: the kernels do not take the activation's constants from the blob at D=%d, F=%d",
+                           name, D, F);
+  return taac::ffn_pack(name, w_up, w_down, norm_weight, packed, D, F, gate_first, stream, fold_activation != 0);
+}
 
 extern "C" int taac_ffn_pack_weights(const void* w_up, const void* w_down, void* packed, int32_t D, int32_t F,
                                      int gate_first, void* stream) {
@@ -1564,7 +1595,7 @@ extern "C" int taac_ffn_pack_weights_norm(const void* w_up, const void* w_down, 
 namespace taac {
 namespace {
 int ffn_pack(const char* name, const void* w_up, const void* w_down, const void* norm_weight, void* packed, int32_t D,
-             int32_t F, int gate_first, void* stream) {
+             int32_t F, int gate_first, void* stream, bool fold_act) {
   if (taac_ffn_packed_bytes(D, F) < 0)
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: D must be 128 or 256 and F a positive multiple of 32", name);
   if (!w_up || !w_down || !packed) return set_error(TAAC_ERR_INVALID_VALUE, "%s: null pointer", name);
@@ -1573,7 +1604,7 @@ int ffn_pack(const char* name, const void* w_up, const void* w_down, const void*
   const int64_t pieces = static_cast<int64_t>(3) * D * F / 8;
   hipLaunchKernelGGL(ffn_pack_kernel, dim3(static_cast<uint32_t>((pieces + 255) / 256)), dim3(256), 0,
                      as_stream(stream), static_cast<const bf16_t*>(w_up), static_cast<const bf16_t*>(w_down),
-                     static_cast<bf16x8*>(packed), D, F, gate_first ? 1 : 0, static_cast<const bf16_t*>(norm_weight));
+                     static_cast<bf16x8*>(packed), D, F, gate_first ? 1 : 0, static_cast<const bf16_t*>(norm_weight), fold_act);
   return check_launch(name);
 }
 }  // namespace
@@ -1625,6 +1656,14 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
               const int32_t* x_rows, int norm_folded, void* stream, const void* update_gate = nullptr, int64_t ldg = 0,
               bool glu = true, int x_plane = 0, const void* head_w = nullptr, float* token_dots = nullptr) {
   const bool with_proj = out_packed != nullptr;
+  if (norm_folded < 0 || norm_folded > (TAAC_FOLDED_NORM | TAAC_FOLDED_ACTIVATION))
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: norm_folded holds TAAC_FOLDED_NORM and / or TAAC_FOLDED_ACTIVATION", name);
+  const bool act_folded = (norm_folded & TAAC_FOLDED_ACTIVATION) != 0;
+  norm_folded &= TAAC_FOLDED_NORM;
+  if (act_folded && (!glu || update_gate != nullptr || packed_weights == nullptr || !ffn_act_fold_supported(D, F)))
+    return set_error(TAAC_ERR_INVALID_VALUE,
+                     "%s: TAAC_FOLDED_ACTIVATION needs the blob of taac_ffn_pack_weights_folded (gated form without an update "
+                     "gate, a shape taac_ffn_activation_fold_supported accepts)", name);
   if ((head_w == nullptr) != (token_dots == nullptr) || !ptr_ok(head_w, 15))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: the readout needs a 16-byte aligned head weight and a buffer of token dots", name);
   if (x_plane != 0 && ((x_plane != 32 && x_plane != 64) || D % x_plane != 0))
@@ -1709,9 +1748,17 @@ int ffn_entry(const char* name, const void* x, int64_t ldx, const void* out_bias
     if (D == 256) TAAC_FFN_LAUNCH(256, 1, 8, 2, true, true, true);
     TAAC_FFN_LAUNCH(128, 1, 8, 2, true, true, true);
   }
+  if (with_proj && act_folded) {
+    if (D == 256) TAAC_FFN_LAUNCH(256, 1, 8, 2, true, true, false, true, true);
+    TAAC_FFN_LAUNCH(128, 1, 8, 2, true, true, false, true, true);
+  }
   if (with_proj) {
     if (D == 256) TAAC_FFN_LAUNCH(256, 1, 8, 2, true, true);
     TAAC_FFN_LAUNCH(128, 1, 8, 2, true, true);
+  }
+  if (act_folded) {  // three buffers fit (ffn_act_fold_supported)
+    if (D == 256) TAAC_FFN_LAUNCH(256, 1, 8, 2, true, false, false, true, true);
+    TAAC_FFN_LAUNCH(128, 1, 8, 2, true, false, false, true, true);
   }
   // Schedule: the down projection of a chunk is deferred by one chunk and interleaved with the next activation (three
   // weight buffers); when a large F leaves no room for the third buffer next to the biases it follows its activation
@@ -1818,6 +1865,8 @@ int norm_linear_launch(const char* name, const void* x, int64_t ldx, const void*
   if (out_plane != 0 && (residual || (out_plane != 32 && out_plane != 64) || static_cast<int64_t>(8) * M + 8 > 0xffffffffLL ||
                          (qk.enabled && qk.head_dim != out_plane)))
     return set_error(TAAC_ERR_UNSUPPORTED, "%s: output planes are 32 or 64 features wide (the head width under a query / key epilogue), without residual", name);
+  if (norm_folded != 0 && norm_folded != TAAC_FOLDED_NORM)
+    return set_error(TAAC_ERR_INVALID_VALUE, "%s: norm_folded is 0 or TAAC_FOLDED_NORM for a linear layer", name);
   if (norm_folded && (!norm_weight || !packed_weights))
     return set_error(TAAC_ERR_INVALID_VALUE, "%s: norm_folded needs the norm weight and the packed weights it was folded into", name);
   if (M < 0 || N <= 0 || K <= 0) return set_error(TAAC_ERR_INVALID_VALUE, "%s: M must be >= 0, N and K > 0", name);
@@ -1979,6 +2028,14 @@ int attn_out_ffn_readout(const void* attn, int64_t ld_attn, int attn_plane, cons
   return ffn_entry("taac_backbone_fwd", attn, ld_attn, out_bias, packed_out_weights, norm_weight, eps, nullptr, b_up, nullptr,
                    b_down, packed_ffn_weights, residual, ldr, out, ldo, M, D, F, 1, rows, n_rows, nullptr, norm_folded,
                    stream, nullptr, 0, true, attn_plane, head_w, token_dots);
+}
+
+// Whether the kernels take the activation's constants from the packed weights at this shape: the gated form with the
+// deferred down projection (three weight buffers next to the biases; the out projection's bias counted in).
+bool ffn_act_fold_supported(int32_t D, int32_t F) {
+  if ((D != 128 && D != 256) || F <= 0 || F % (kHU * kCPB) != 0) return false;
+  const size_t buffer_bytes = static_cast<size_t>(kCPB * (D / 16 + D / 32)) * kFrag;
+  return 3 * buffer_bytes + static_cast<size_t>(2 * F + 3 * D) * 2 <= static_cast<size_t>(kMaxLdsBytes);
 }
 }  // namespace taac
 

@@ -188,6 +188,28 @@ def test_host_side_validation_of_the_widened_entry_points_without_gpu():
     assert plane_tail(d=192) == unsupported
     assert plane_tail(m=0) == ok
 
+    # the flags of norm_folded: the activation's constants come with a packed gated blob at a supported shape, a linear
+    # layer knows the norm flag only
+    def folded_ffn(flags, **kw):
+        a = dict(packed=fake, norm=fake, d=256, f=64, m=0)
+        a.update(kw)
+        return library.taac_swiglu_ffn_fwd(fake, a["d"], a["norm"], 1e-6, fake, None, fake, None, a["packed"], None, a["d"], fake,
+                                           a["d"], a["m"], a["d"], a["f"], 1, None, None, flags, None)
+
+    both = _native.FOLDED_NORM | _native.FOLDED_ACTIVATION
+    assert folded_ffn(both) == ok and folded_ffn(_native.FOLDED_ACTIVATION, norm=None) == ok
+    assert folded_ffn(4) == invalid and b"TAAC_FOLDED" in library.taac_last_error()
+    assert folded_ffn(_native.FOLDED_ACTIVATION, packed=None) == invalid and b"taac_ffn_pack_weights_folded" in library.taac_last_error()
+    assert folded_ffn(both, f=36864) == invalid  # no room for three weight buffers: such a blob cannot exist
+    assert library.taac_ffn_activation_fold_supported(256, 1024) == 1 and library.taac_ffn_activation_fold_supported(128, 512) == 1
+    assert library.taac_ffn_activation_fold_supported(256, 36864) == 0 and library.taac_ffn_activation_fold_supported(64, 128) == 0
+    assert library.taac_ffn_pack_weights_folded(fake, fake, None, fake, 256, 36864, 1, 1, None) == unsupported
+    assert library.taac_ffn_pack_weights_folded(fake, None, None, fake, 256, 64, 1, 1, None) == invalid
+    assert library.taac_attn_out_gate_ffn_fwd(fake, 256, None, fake, fake, 256, fake, 256, None, 1e-6, None, None, fake, fake, 256,
+                                              0, 256, 64, None, None, None, _native.FOLDED_ACTIVATION, None) == invalid
+    assert library.taac_norm_linear_fwd(fake, 256, fake, 1e-6, None, None, fake, None, 256, fake, 256, 0, 256, 256, None, None,
+                                        None, 2, None) == invalid
+
     # readout: indices inside the sequence, one kind of validity, a complete classifier, something to write
     def readout(**kw):
         a = dict(lengths=None, bits=None, t=16, d=64, cls=0, cand=3, fc1=fake, fc2=fake, hidden=32, actions=1, emb=None,

@@ -247,6 +247,60 @@ def test_fused_swiglu_ffn(device, m, d, f, gate_first):
     torch.testing.assert_close(got.cpu().float(), ref_bf16.float(), rtol=4e-2, atol=4e-2)
 
 
+@pytest.mark.parametrize("m,d,f", [(300, 256, 1024), (65, 128, 96)])
+@pytest.mark.parametrize("gate_first", [True, False])
+@pytest.mark.parametrize("with_norm", [True, False])
+def test_fused_ffn_with_the_activation_constants_in_the_packed_weights(device, m, d, f, gate_first, with_norm):
+    """``fold_activation``: the packed up projection carries -log2(e) (gated half) and -ln(2) (other half), the kernel
+    evaluates ``g' * u' / (1 + 2^g')``. Both forms against the oracle's fp32 evaluation, with biases, either gate order,
+    with and without the norm in front (whose weight shares the rounding); the two forms differ by rounding only. The
+    block tail (rows and per-head planes) likewise. A hidden size that leaves no room for the kernels' third weight
+    buffer takes the plain blob."""
+    from taac_2026_amd.api import attention_out_ffn, swiglu_ffn
+    from taac_2026_amd.accelerators.linear import attention_out_ffn_heads, ffn_activation_fold_supported
+
+    assert ffn_activation_fold_supported(d, f) and not ffn_activation_fold_supported(256, 4096)
+    attn, h, nw, wo, bo, wu, bu, wd, bd = _block_tail_inputs(m, d, f, seed=m + f + int(gate_first))
+    norm = nw if with_norm else None
+    x = h
+    xin = oracle.rms_norm_fp32(x, nw).float() if with_norm else x.float()
+    expected = x.float() + oracle.swiglu_ffn(xin, wu.float(), bu.float(), wd.float(), bd.float(), gate_first=gate_first)
+    dev = lambda t: None if t is None else t.to(device)
+    results = {}
+    with torch.no_grad():
+        for fold in (False, True, None):
+            results[fold] = swiglu_ffn(dev(x), dev(wu), dev(bu), dev(wd), dev(bd), residual=dev(x), norm_weight=dev(norm),
+                                       gate_first=gate_first, fold_activation=fold).cpu().float()
+            torch.testing.assert_close(results[fold], expected, **BF16_TOL)
+    assert torch.equal(results[None], results[True])
+    step = 2.0 ** -7
+    assert (results[True] - results[False]).abs().max().item() <= 4 * step * max(1.0, expected.abs().max().item())
+    assert (results[True] - expected).abs().mean().item() <= 1.25 * (results[False] - expected).abs().mean().item() + 1e-4
+    if gate_first:
+        heads = d // 32
+        planes = attn.view(m, heads, 32).transpose(0, 1).contiguous()
+        with torch.no_grad():
+            tails = {fold: attention_out_ffn(dev(attn), dev(wo), dev(bo), dev(h), dev(wu), dev(bu), dev(wd), dev(bd),
+                                             norm_weight=dev(norm), fold_activation=fold).cpu().float() for fold in (False, True)}
+            from_planes = attention_out_ffn_heads(dev(planes), dev(wo), dev(bo), dev(h), dev(wu), dev(bu), dev(wd), dev(bd),
+                                                  norm_weight=dev(norm), fold_activation=True).cpu().float()
+        assert torch.equal(from_planes, tails[True])
+        x1 = (h.float() + (attn.float() @ wo.float().t() + bo.float()).to(torch.bfloat16).float()).to(torch.bfloat16)
+        x1n = oracle.rms_norm_fp32(x1, nw).float() if with_norm else x1.float()
+        tail_expected = x1.float() + oracle.swiglu_ffn(x1n, wu.float(), bu.float(), wd.float(), bd.float())
+        for fold in (False, True):
+            torch.testing.assert_close(tails[fold], tail_expected, **BF16_TOL)
+    # no room for three weight buffers: the wrappers fall back to the plain blob, an explicit request is refused
+    wide_up = (torch.randn(2 * 4096, 256, generator=torch.Generator().manual_seed(1)) * 0.02).to(torch.bfloat16)
+    wide_down = (torch.randn(256, 4096, generator=torch.Generator().manual_seed(2)) * 0.02).to(torch.bfloat16)
+    xs = torch.randn(8, 256, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    with torch.no_grad():
+        wide = swiglu_ffn(dev(xs), dev(wide_up), None, dev(wide_down), None).cpu().float()
+        torch.testing.assert_close(wide, oracle.swiglu_ffn(xs.float(), wide_up.float(), None, wide_down.float(), None), **BF16_TOL)
+        with pytest.raises(RuntimeError):
+            swiglu_ffn(dev(xs), dev(wide_up), None, dev(wide_down), None, fold_activation=True)
+
+
 def _block_tail_inputs(m, d, f, seed):
     g = torch.Generator().manual_seed(seed)
     attn = torch.randn(m, d, generator=g).to(torch.bfloat16)
