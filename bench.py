@@ -62,7 +62,9 @@ class _CallRecorder:
 
     def __getattr__(self, name):
         function = getattr(self._library, name)
-        if not name.startswith("taac_") or name in ("taac_last_error", "taac_abi_version") or name.endswith("_bytes"):
+        # queries (sizes, offsets, what a shape supports) return a value, not a status, and launch nothing
+        if (not name.startswith("taac_") or name in ("taac_last_error", "taac_abi_version")
+                or name.endswith(("_bytes", "_floats", "_offset", "_supported"))):
             return function
 
         def recorded(*args):
