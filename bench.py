@@ -33,12 +33,26 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 
 
+SETTLE_MS = 50.0  # work in front of a timed region: see _event_ms
+
+
 def _event_ms(fn, iters: int, warmup: int) -> float:
     """Duration of ``fn`` in ms per call, HIP events on the current stream (the stream the kernels are launched on):
     the launches are timed in up to five groups and the median group is reported, so that a single stall on a shared
-    host (seen as one group several times slower than the others) does not end up in a kernel figure."""
+    host (seen as one group several times slower than the others) does not end up in a kernel figure.
+
+    The warm-up is ``warmup`` calls and at least ``SETTLE_MS`` of them: a chip that has idled (while the host checked a
+    result against the CPU formulas, say) takes tens of milliseconds of work to bring its clocks back up, and twenty
+    launches of a 0.15 ms kernel are over before that (configuration 3's attention read 0.160 ms that way and 0.147 ms
+    behind 30 ms of its own launches or behind any other GPU work)."""
+    started = time.perf_counter()
     for _ in range(warmup):
         fn()
+    torch.cuda.synchronize()
+    while (time.perf_counter() - started) * 1e3 < SETTLE_MS:
+        for _ in range(max(1, warmup)):
+            fn()
+        torch.cuda.synchronize()
     groups = max(1, min(5, iters // 2))
     per_group = max(1, iters // groups)
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(groups + 1)]
